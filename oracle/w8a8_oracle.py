@@ -1,0 +1,595 @@
+"""NumPy restatement of the reference's W8A8 LoRA linear forward semantics.
+
+TEST INFRASTRUCTURE ONLY (see ``oracle/__init__.py``).  Every function cites the
+reference file:line (relative to the reference checkout) whose arithmetic it
+follows.  bf16 values are carried as float32 arrays whose low 16 mantissa bits
+are zero; ``bf16_round`` is the only place a bf16 rounding happens.
+
+How each function is pinned (the tests that do it live in ``tests/test_oracle_*.py``):
+
+* ``bf16_round``/``bf16_bits``, ``quantize_frozen_weight``, ``dynamic_group_quantize``,
+  ``quantized_frozen_linear_f32``, ``quantized_lora_linear``: the reference's
+  SHA-256-pinned deterministic host case (rocm/probe_w8a8_lora_forward.py:210-218)
+  plus the hand-coded int4 / W4A4 vectors of tests/tx/kernels/test_quantized_lora.py:30-74.
+* ``int_matmul``: brute force in Python integers and the int32 ``numpy.matmul``.
+* ``lora_delta_multi``/``quantized_lora_linear_multi``: the arange closed forms of
+  tests/tx/layers/test_lora_fast_path.py:21-49 and per-row brute force.
+* ``fuse``/``split``: brute force and round trip (skyrl/tx/layers/lora.py:325-351).
+* ``ragged_dot``: the six-row table of tests/tx/layers/test_ragged_dot.py:8-33.
+* ``swiglu_from_interleaved``: the pairing constant 1.9296875 derived from
+  tests/tx/kernels/rocm/test_bf16_rms_gate_up_lora_swiglu.py:335-364.
+* ``rms_norm``: closed forms (constant rows, power-of-two rows).  PARITY UNPINNED
+  in the last f32 bit against XLA-CPU: the reference's ``jnp.mean`` reduction order
+  and ``lax.rsqrt`` rounding live in jaxlib, which is not available; this oracle
+  fixes mean = f32(sum_f64(x*x)/K) and rsqrt = 1/sqrt with IEEE f32 ops.
+* ``silu``: exp/logistic rounding of XLA-CPU is likewise unavailable; PARITY
+  UNPINNED in the last f32 bit, pinned to 1 ulp by the closed-form constant above
+  and by ``scipy.special.expit``.
+* ``moe_route``/``moe_expert_mlp``: ``torch.topk``/``scipy.special.softmax`` special
+  cases and the merged-weight invariant of tests/tx/models/test_qwen3.py:123-180.
+"""
+
+from __future__ import annotations
+
+import hashlib
+from dataclasses import dataclass
+
+import numpy as np
+
+F32 = np.float32
+
+
+# ---------------------------------------------------------------------------
+# bf16 helpers
+# ---------------------------------------------------------------------------
+
+def bf16_bits(a) -> np.ndarray:
+    """float32 -> uint16 bf16 bit pattern, round-to-nearest-even (NaN kept quiet)."""
+    a = np.ascontiguousarray(np.asarray(a, dtype=F32))
+    u = a.view(np.uint32)
+    rounded = (u + np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))) >> np.uint32(16)
+    nan = np.isnan(a)
+    if np.any(nan):
+        rounded = np.where(nan, (u >> np.uint32(16)) | np.uint32(0x40), rounded)
+    return rounded.astype(np.uint16)
+
+
+def bf16_from_bits(bits) -> np.ndarray:
+    bits = np.asarray(bits, dtype=np.uint16)
+    return (bits.astype(np.uint32) << np.uint32(16)).view(F32)
+
+
+def bf16_round(a) -> np.ndarray:
+    """Round float32 values to the nearest bf16 (ties to even), returned as float32."""
+    return bf16_from_bits(bf16_bits(a))
+
+
+def is_bf16_exact(a) -> bool:
+    a = np.ascontiguousarray(np.asarray(a, dtype=F32))
+    return bool(np.all((a.view(np.uint32) & np.uint32(0xFFFF)) == 0))
+
+
+def sha256_bf16(a) -> str:
+    return hashlib.sha256(bf16_bits(a).tobytes(order="C")).hexdigest()
+
+
+# ---------------------------------------------------------------------------
+# storage format (skyrl/tx/kernels/quantized_lora.py:20-91)
+# ---------------------------------------------------------------------------
+
+@dataclass(frozen=True)
+class GroupQuantizedWeight:
+    """K x N weight grouped along K; skyrl/tx/kernels/quantized_lora.py:20-41."""
+
+    codes: np.ndarray
+    scales: np.ndarray
+    original_in_features: int
+    padded_in_features: int
+    bits: int
+    group_size: int
+
+
+def _validate_bits(bits: int) -> None:
+    if bits not in (4, 8):
+        raise ValueError(f"bits must be 4 or 8, got {bits}")
+
+
+def _validate_group_size(group_size: int) -> None:
+    if group_size <= 0 or group_size % 2:
+        raise ValueError(f"group_size must be a positive even integer, got {group_size}")
+
+
+def validate_quantized_weight(weight: GroupQuantizedWeight) -> None:
+    """skyrl/tx/kernels/quantized_lora.py:56-91."""
+    _validate_bits(weight.bits)
+    _validate_group_size(weight.group_size)
+    if weight.original_in_features <= 0 or weight.padded_in_features <= 0:
+        raise ValueError("quantized weight input dimensions must be positive")
+    if weight.padded_in_features < weight.original_in_features:
+        raise ValueError("padded_in_features must be at least original_in_features")
+    if weight.padded_in_features % weight.group_size:
+        raise ValueError("padded_in_features must be divisible by group_size")
+    if weight.codes.ndim != 2 or weight.scales.ndim != 2:
+        raise ValueError("quantized weight codes and scales must both be rank-two")
+    rows = weight.padded_in_features // (2 if weight.bits == 4 else 1)
+    scale_shape = (weight.padded_in_features // weight.group_size, weight.codes.shape[1])
+    if weight.codes.shape[0] != rows:
+        raise ValueError(f"code rows {weight.codes.shape[0]} do not match expected {rows}")
+    if weight.scales.shape != scale_shape:
+        raise ValueError(f"scale shape {weight.scales.shape} does not match expected {scale_shape}")
+    if weight.codes.shape[1] <= 0:
+        raise ValueError("quantized weight output dimension must be positive")
+    want = np.uint8 if weight.bits == 4 else np.int8
+    if weight.codes.dtype != want:
+        raise TypeError(f"W{weight.bits} codes must have dtype {want}, got {weight.codes.dtype}")
+    if not np.issubdtype(weight.scales.dtype, np.floating):
+        raise TypeError(f"quantized weight scales must be floating point, got {weight.scales.dtype}")
+
+
+def pack_signed_int4(values) -> np.ndarray:
+    """skyrl/tx/kernels/quantized_lora.py:94-109 (low nibble = even row, high = odd row)."""
+    values = np.asarray(values)
+    if values.ndim < 1 or values.shape[0] == 0 or values.shape[0] % 2:
+        raise ValueError("signed INT4 packing requires an even, nonempty axis zero")
+    if not np.issubdtype(values.dtype, np.integer):
+        raise TypeError(f"signed INT4 values must be integral, got {values.dtype}")
+    low = (values[0::2].astype(np.int16) & 0xF).astype(np.uint8)
+    high = (values[1::2].astype(np.int16) & 0xF).astype(np.uint8)
+    return low | (high << np.uint8(4))
+
+
+def unpack_signed_int4(packed) -> np.ndarray:
+    """skyrl/tx/kernels/quantized_lora.py:112-125."""
+    packed = np.asarray(packed)
+    if packed.ndim < 1 or packed.shape[0] == 0:
+        raise ValueError("signed INT4 input must have a nonempty axis zero")
+    if packed.dtype != np.uint8:
+        raise TypeError(f"packed signed INT4 values must be uint8, got {packed.dtype}")
+    low = (packed & np.uint8(0xF)).astype(np.int16)
+    high = (packed >> np.uint8(4)).astype(np.int16)
+    low = np.where(low >= 8, low - 16, low).astype(np.int8)
+    high = np.where(high >= 8, high - 16, high).astype(np.int8)
+    inter = np.stack((low, high), axis=1)
+    return inter.reshape((packed.shape[0] * 2, *packed.shape[1:]))
+
+
+def quantize_frozen_weight(weight, *, bits: int = 8, group_size: int = 64,
+                           scale_dtype: str = "bf16") -> GroupQuantizedWeight:
+    """Symmetric per-(group, output) weight quantizer; quantized_lora.py:128-171.
+
+    ``scale_dtype`` is "bf16" (the reference default: scales are *stored* rounded
+    to bf16 while the codes were computed with the f32 scale) or "f32".
+    """
+    _validate_bits(bits)
+    _validate_group_size(group_size)
+    weight = np.asarray(weight)
+    if weight.ndim != 2:
+        raise ValueError(f"weight must have shape [K, N], got {weight.shape}")
+    if weight.shape[0] <= 0 or weight.shape[1] <= 0:
+        raise ValueError(f"weight dimensions must be positive, got {weight.shape}")
+    if not np.issubdtype(weight.dtype, np.floating):
+        raise TypeError(f"weight must be floating point, got {weight.dtype}")
+    if scale_dtype not in ("bf16", "f32"):
+        raise TypeError(f"scale_dtype must be 'bf16' or 'f32', got {scale_dtype}")
+    k, n = weight.shape
+    k_pad = ((k + group_size - 1) // group_size) * group_size
+    padded = np.zeros((k_pad, n), dtype=F32)
+    padded[:k] = weight.astype(F32)
+    grouped = padded.reshape((-1, group_size, n))
+    qmax = (1 << (bits - 1)) - 1
+    amax = np.max(np.abs(grouped), axis=1)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        scales = np.where(amax > 0, amax / F32(qmax), F32(1.0)).astype(F32)
+        q = np.clip(np.rint(grouped / scales[:, None, :]), -qmax, qmax).astype(np.int8)
+    q = q.reshape((k_pad, n))
+    codes = q if bits == 8 else pack_signed_int4(q)
+    stored = bf16_round(scales) if scale_dtype == "bf16" else scales
+    return GroupQuantizedWeight(codes=codes, scales=stored, original_in_features=k,
+                                padded_in_features=k_pad, bits=bits, group_size=group_size)
+
+
+def unpacked_codes(weight: GroupQuantizedWeight) -> np.ndarray:
+    """quantized_lora.py:174-177."""
+    validate_quantized_weight(weight)
+    codes = weight.codes if weight.bits == 8 else unpack_signed_int4(weight.codes)
+    return codes[: weight.padded_in_features].astype(np.int8)
+
+
+def dequantize_frozen_weight(weight: GroupQuantizedWeight) -> np.ndarray:
+    """quantized_lora.py:180-196 (float32 result)."""
+    codes = unpacked_codes(weight)
+    n = codes.shape[1]
+    grouped = codes.reshape((-1, weight.group_size, n)).astype(F32)
+    deq = grouped * weight.scales.astype(F32)[:, None, :]
+    return deq.reshape((weight.padded_in_features, n))[: weight.original_in_features]
+
+
+# ---------------------------------------------------------------------------
+# activation quantizer and integer GEMM
+# ---------------------------------------------------------------------------
+
+def dynamic_group_quantize(x, bits: int = 8, group_size: int | None = None):
+    """Per-(row, group) symmetric dynamic quantizer; quantized_lora.py:199-212.
+
+    Both divisions are IEEE float32 divisions and ``rint`` rounds half to even.
+    Returns (codes int8 [M, G, group_size], scales float32 [M, G]).
+    """
+    x = np.asarray(x, dtype=F32)
+    if group_size is None:
+        group_size = x.shape[1]
+    qmax = (1 << (bits - 1)) - 1
+    grouped = x.reshape((x.shape[0], x.shape[1] // group_size, group_size))
+    amax = np.max(np.abs(grouped), axis=-1)
+    scales = np.where(amax > 0, amax / F32(qmax), F32(1.0)).astype(F32)
+    codes = np.clip(np.rint(grouped / scales[..., None]), -qmax, qmax).astype(np.int8)
+    return codes, scales
+
+
+def quantize_rows(x):
+    """Per-token (group = whole row) A8 quantizer: (codes int8 [M,K], scales f32 [M])."""
+    codes, scales = dynamic_group_quantize(x, 8, None)
+    return codes[:, 0, :], scales[:, 0]
+
+
+def int_matmul(a_codes, b_codes) -> np.ndarray:
+    """Exact int8 x int8 -> int32 matrix product (quantized_lora.py:240-245).
+
+    Small problems use numpy's int32 matmul.  Large ones go through float64 BLAS,
+    which is exact here: |sum| <= K * 127^2 < 2^53 for any K below 5.5e11.
+    """
+    a = np.asarray(a_codes)
+    b = np.asarray(b_codes)
+    if a.shape[0] * a.shape[1] * b.shape[1] <= (1 << 24):
+        return np.matmul(a.astype(np.int32), b.astype(np.int32), dtype=np.int32)
+    out = np.empty((a.shape[0], b.shape[1]), dtype=np.int32)
+    b64 = b.astype(np.float64)
+    step = max(1, (1 << 27) // max(1, a.shape[1]))
+    for r0 in range(0, a.shape[0], step):
+        out[r0:r0 + step] = np.rint(a[r0:r0 + step].astype(np.float64) @ b64).astype(np.int32)
+    return out
+
+
+def quantized_frozen_linear_f32(x, weight: GroupQuantizedWeight, *, activation_bits: int = 8,
+                                return_parts: bool = False):
+    """FP32 epilogue input of the grouped quantized linear; quantized_lora.py:215-254.
+
+    ``scaled = f32(acc) * x_scale * w_scale`` is evaluated left to right and the
+    groups are summed in float32 in group order.
+    """
+    _validate_bits(activation_bits)
+    validate_quantized_weight(weight)
+    x = np.asarray(x)
+    if x.ndim < 1:
+        raise ValueError(f"activations must have at least one dimension, got {x.shape}")
+    if not np.issubdtype(x.dtype, np.floating):
+        raise TypeError(f"activations must be floating point, got {x.dtype}")
+    if x.shape[-1] != weight.original_in_features:
+        raise ValueError(
+            f"activation K={x.shape[-1]} does not match weight K={weight.original_in_features}")
+    flat = x.reshape((-1, x.shape[-1])).astype(F32)
+    padded = np.zeros((flat.shape[0], weight.padded_in_features), dtype=F32)
+    padded[:, : flat.shape[1]] = flat
+    g = weight.group_size
+    x_codes, x_scales = dynamic_group_quantize(padded, activation_bits, g)
+    w_codes = unpacked_codes(weight).reshape((-1, g, weight.codes.shape[-1]))
+    w_scales = weight.scales.astype(F32)
+    n_groups = w_codes.shape[0]
+    out = None
+    accs = []
+    for gi in range(n_groups):
+        acc = int_matmul(x_codes[:, gi, :], w_codes[gi])
+        scaled = acc.astype(F32) * x_scales[:, gi, None] * w_scales[gi][None, :]
+        out = scaled if out is None else (out + scaled).astype(F32)
+        if return_parts:
+            accs.append(acc)
+    out = out.reshape((*x.shape[:-1], w_codes.shape[-1])).astype(F32)
+    if return_parts:
+        return out, x_codes, x_scales, np.stack(accs, axis=1)
+    return out
+
+
+def quantized_frozen_linear(x, weight: GroupQuantizedWeight, *, activation_bits: int = 8):
+    """quantized_lora.py:257-272 with a bf16 activation dtype."""
+    return bf16_round(quantized_frozen_linear_f32(x, weight, activation_bits=activation_bits))
+
+
+def quantized_lora_linear_f32(x, weight: GroupQuantizedWeight, lora_a, lora_b, lora_scaling,
+                              *, activation_bits: int = 8):
+    """Pre-cast value of quantized_lora.py:275-304: base + ((x@A)@B) * s, all float32."""
+    validate_quantized_weight(weight)
+    x = np.asarray(x)
+    lora_a = np.asarray(lora_a)
+    lora_b = np.asarray(lora_b)
+    if lora_a.ndim != 2 or lora_b.ndim != 2:
+        raise ValueError("lora_a and lora_b must both be rank-two")
+    if lora_a.shape != (weight.original_in_features, lora_b.shape[0]):
+        raise ValueError(
+            f"incompatible LoRA shapes: A={lora_a.shape}, B={lora_b.shape}, "
+            f"weight K={weight.original_in_features}")
+    if lora_b.shape[1] != weight.codes.shape[-1]:
+        raise ValueError(
+            f"LoRA output N={lora_b.shape[1]} does not match weight N={weight.codes.shape[-1]}")
+    scaling = np.asarray(lora_scaling, dtype=F32)
+    if scaling.ndim != 0:
+        raise ValueError(f"lora_scaling must be scalar, got {scaling.shape}")
+    base = quantized_frozen_linear_f32(x, weight, activation_bits=activation_bits)
+    flat = x.reshape((-1, x.shape[-1])).astype(F32)
+    z = np.matmul(flat, lora_a.astype(F32), dtype=F32)
+    low = np.matmul(z, lora_b.astype(F32), dtype=F32).reshape(base.shape)
+    return (base + low * scaling).astype(F32)
+
+
+def quantized_lora_linear(x, weight, lora_a, lora_b, lora_scaling, *, activation_bits: int = 8):
+    """quantized_lora.py:400-453: exactly one bf16 cast after the float32 epilogue."""
+    return bf16_round(quantized_lora_linear_f32(x, weight, lora_a, lora_b, lora_scaling,
+                                                activation_bits=activation_bits))
+
+
+# ---------------------------------------------------------------------------
+# multi-adapter LoRA (skyrl/tx/layers/lora.py:118-157) in the float32-epilogue rule
+# ---------------------------------------------------------------------------
+
+def lora_delta_multi(x, lora_a, lora_b, lora_scaling, adapter_indices) -> np.ndarray:
+    """Per-row adapter LoRA delta ((x @ A[i]) @ B[i]) * s[i] in float32.
+
+    Routing follows lora.py:142-157 (rows grouped by adapter, two ragged products,
+    scaling gathered per row); arithmetic follows the float32 rule of
+    quantized_lora.py:300-304.  ``adapter_indices`` is one int per *row*.
+    """
+    x = np.asarray(x, dtype=F32)
+    a = np.asarray(lora_a, dtype=F32)
+    b = np.asarray(lora_b, dtype=F32)
+    s = np.asarray(lora_scaling, dtype=F32)
+    idx = np.asarray(adapter_indices)
+    if a.ndim != 3 or b.ndim != 3:
+        raise ValueError("multi-adapter lora_a/lora_b must be rank-three")
+    if idx.shape != (x.shape[0],):
+        raise ValueError("adapter_indices must hold one entry per row")
+    if idx.size and (idx.min() < 0 or idx.max() >= a.shape[0]):
+        raise ValueError("adapter index out of range")
+    out = np.zeros((x.shape[0], b.shape[2]), dtype=F32)
+    for adapter in np.unique(idx):
+        rows = np.nonzero(idx == adapter)[0]
+        z = np.matmul(x[rows], a[adapter], dtype=F32)
+        out[rows] = np.matmul(z, b[adapter], dtype=F32) * s[adapter]
+    return out
+
+
+def quantized_lora_linear_multi_f32(x, weight, lora_a, lora_b, lora_scaling, adapter_indices,
+                                    residual=None):
+    """base + per-row LoRA delta (+ residual) in one float32 epilogue."""
+    base = quantized_frozen_linear_f32(x, weight)
+    out = (base + lora_delta_multi(x, lora_a, lora_b, lora_scaling, adapter_indices)).astype(F32)
+    if residual is not None:
+        out = (out + np.asarray(residual, dtype=F32)).astype(F32)
+    return out
+
+
+def quantized_lora_linear_multi(x, weight, lora_a, lora_b, lora_scaling, adapter_indices,
+                                residual=None):
+    """Single bf16 cast of ``quantized_lora_linear_multi_f32``.
+
+    With ``residual`` this is the down-projection variant: the order follows the
+    scalar HIP specification rocm/compile_probes/down_lora_residual_gfx1100.hip:120-123
+    (float32 accumulate, += s*lora, += residual, one bf16 store).
+    """
+    return bf16_round(quantized_lora_linear_multi_f32(x, weight, lora_a, lora_b, lora_scaling,
+                                                      adapter_indices, residual))
+
+
+# ---------------------------------------------------------------------------
+# RMSNorm -> gate/up -> SwiGLU (bf16_rms_gate_up_lora_swiglu.py:277-330)
+# ---------------------------------------------------------------------------
+
+def rms_norm(x, gamma, eps: float = 1e-6) -> np.ndarray:
+    """bf16(x * rsqrt(mean(x^2) + eps) * gamma); bf16_rms_gate_up_lora_swiglu.py:299-303.
+
+    ``gamma`` is the float32 multiplier: ``1 + delta`` for the Qwen3.5 flavour
+    (qwen3_5.py:269-278) or the plain weight for Qwen3 (layers/layernorm.py:22-24).
+    mean = float32(sum in float64 / K); rsqrt = 1 / sqrt, both IEEE float32.
+    """
+    x = np.asarray(x, dtype=F32)
+    gamma = np.asarray(gamma, dtype=F32)
+    k = x.shape[-1]
+    ssq = np.sum(x.astype(np.float64) * x.astype(np.float64), axis=-1, keepdims=True)
+    var = (ssq / np.float64(k)).astype(F32)
+    inv = (F32(1.0) / np.sqrt((var + F32(eps)).astype(F32))).astype(F32)
+    normalized = (x * inv).astype(F32)
+    return bf16_round((normalized * gamma).astype(F32))
+
+
+def silu(v) -> np.ndarray:
+    """x * logistic(x) in float32 (jax.nn.silu on an f32 operand)."""
+    v = np.asarray(v, dtype=F32)
+    with np.errstate(over="ignore"):
+        sig = (F32(1.0) / (F32(1.0) + np.exp(-v).astype(F32))).astype(F32)
+    return (v * sig).astype(F32)
+
+
+def swiglu_from_interleaved(fused_bf16) -> np.ndarray:
+    """bf16(silu(gate.f32) * up.f32) with gate = even, up = odd columns.
+
+    Kernel rule of bf16_rms_gate_up_lora_swiglu.py:277-292 and
+    bf16_rms_gate_up_lora_swiglu_contiguous.py:535-538.
+    """
+    fused = np.asarray(fused_bf16, dtype=F32)
+    gate = fused[..., 0::2]
+    up = fused[..., 1::2]
+    return bf16_round((silu(gate) * up).astype(F32))
+
+
+def w8a8_rms_gate_up_lora_swiglu(x, gamma, weight: GroupQuantizedWeight, lora_a, lora_b,
+                                 lora_scaling, adapter_indices, eps: float = 1e-6,
+                                 return_stages: bool = False):
+    """Composite oracle for the fused W8A8 MLP-up stage.
+
+    n = rms_norm(x) (bf16) -> per-token A8 quantization of n -> int GEMM + f32
+    dequant -> + s[idx] * ((n @ A[idx]) @ B[idx]) in f32 -> one bf16 cast (fused)
+    -> adjacent (gate, up) pairs -> bf16(silu(gate) * up).
+    """
+    n = rms_norm(x, gamma, eps)
+    fused_f32 = quantized_lora_linear_multi_f32(n, weight, lora_a, lora_b, lora_scaling,
+                                                adapter_indices)
+    fused = bf16_round(fused_f32)
+    product = swiglu_from_interleaved(fused)
+    if return_stages:
+        return product, {"normalized": n, "fused_f32": fused_f32, "fused": fused}
+    return product
+
+
+# ---------------------------------------------------------------------------
+# fused-projection interleave (skyrl/tx/layers/lora.py:325-351)
+# ---------------------------------------------------------------------------
+
+def fuse(*arrays, group_sizes) -> np.ndarray:
+    assert len(arrays) == len(group_sizes)
+    batch = arrays[0].shape[:-1]
+    num_groups = arrays[0].shape[-1] // group_sizes[0]
+    parts = []
+    for arr, g in zip(arrays, group_sizes):
+        assert arr.shape[-1] == num_groups * g
+        parts.append(np.asarray(arr).reshape(*batch, num_groups, g))
+    return np.concatenate(parts, axis=-1).reshape(*batch, -1)
+
+
+def split(fused, group_sizes):
+    fused = np.asarray(fused)
+    batch, total = fused.shape[:-1], fused.shape[-1]
+    gs = sum(group_sizes)
+    assert total % gs == 0
+    num_groups = total // gs
+    view = fused.reshape(*batch, num_groups, gs)
+    out, offset = [], 0
+    for g in group_sizes:
+        out.append(view[..., offset:offset + g].reshape(*batch, num_groups * g))
+        offset += g
+    return tuple(out)
+
+
+# ---------------------------------------------------------------------------
+# routing helpers (skyrl/tx/layers/util.py:8-87)
+# ---------------------------------------------------------------------------
+
+def prepare_routing(tokens, indices, num_groups: int, adapter_indices=None):
+    """util.py:66-87: stable argsort by group, bincount, inverse permutation."""
+    indices = np.asarray(indices)
+    sort_indices = np.argsort(indices, kind="stable")
+    sorted_tokens = np.asarray(tokens)[sort_indices]
+    sorted_adapters = None if adapter_indices is None else np.asarray(adapter_indices)[sort_indices]
+    group_sizes = np.bincount(indices, minlength=num_groups)[:num_groups]
+    unsort = np.argsort(sort_indices, kind="stable")
+    return sorted_tokens, group_sizes, unsort, sorted_adapters
+
+
+def ragged_dot(lhs, rhs, group_sizes, group_offset=None) -> np.ndarray:
+    """util.py:8-59: rows of group g are multiplied by rhs[g]; with ``group_offset``
+    rhs holds groups [offset, offset + g_local) and rows of other groups give zero.
+    Rows beyond sum(group_sizes) give zero (lax.ragged_dot semantics)."""
+    lhs = np.asarray(lhs, dtype=F32)
+    rhs = np.asarray(rhs, dtype=F32)
+    group_sizes = np.asarray(group_sizes)
+    offset = 0 if group_offset is None else int(np.asarray(group_offset).reshape(-1)[0])
+    out = np.zeros((lhs.shape[0], rhs.shape[2]), dtype=F32)
+    starts = np.concatenate(([0], np.cumsum(group_sizes)))
+    for local in range(rhs.shape[0]):
+        g = local + offset
+        if g >= len(group_sizes):
+            break
+        r0, r1 = int(starts[g]), int(starts[g + 1])
+        if r1 > r0:
+            out[r0:r1] = np.matmul(lhs[r0:r1], rhs[local], dtype=F32)
+    return out
+
+
+# ---------------------------------------------------------------------------
+# MoE expert MLP (skyrl/tx/models/qwen3.py:172-210, layers/lora.py:394-444)
+# ---------------------------------------------------------------------------
+
+def moe_route(router_logits, top_k: int, norm_topk_prob: bool = True):
+    """softmax -> top_k -> renormalise; qwen3.py:175-178.  Ties pick the lower index."""
+    logits = np.asarray(router_logits, dtype=F32)
+    shifted = logits - np.max(logits, axis=-1, keepdims=True)
+    e = np.exp(shifted).astype(F32)
+    probs = (e / np.sum(e, axis=-1, keepdims=True, dtype=F32)).astype(F32)
+    order = np.argsort(-probs, axis=-1, kind="stable")[:, :top_k]
+    weights = np.take_along_axis(probs, order, axis=-1)
+    if norm_topk_prob:
+        weights = (weights / np.sum(weights, axis=-1, keepdims=True, dtype=F32)).astype(F32)
+    return weights.astype(F32), order.astype(np.int32)
+
+
+def grouped_quantized_lora_linear_f32(x_sorted, group_sizes, weights, lora_a, lora_b, scaling):
+    """Per-expert quantized LoRA linear over contiguous row groups, float32 pre-cast.
+
+    ``weights`` is a list of per-expert GroupQuantizedWeight; ``lora_a``/``lora_b``
+    are [E, K, r] / [E, r, N]; ``scaling`` a float32 scalar (lora.py:433-444 with a
+    single adapter; expert e's rows use A[e], B[e]).
+    """
+    x_sorted = np.asarray(x_sorted, dtype=F32)
+    n_out = weights[0].codes.shape[1]
+    out = np.zeros((x_sorted.shape[0], n_out), dtype=F32)
+    starts = np.concatenate(([0], np.cumsum(np.asarray(group_sizes))))
+    for e, w in enumerate(weights):
+        r0, r1 = int(starts[e]), int(starts[e + 1])
+        if r1 > r0:
+            out[r0:r1] = quantized_lora_linear_f32(x_sorted[r0:r1], w, lora_a[e], lora_b[e], scaling)
+    return out
+
+
+def moe_expert_mlp(hidden, router_logits, top_k, gate_up_weights, down_weights,
+                   gate_up_a, gate_up_b, down_a, down_b, scaling, return_stages: bool = False):
+    """Composite oracle for the grouped W8A8 + LoRA expert MLP.
+
+    Routing as in qwen3.py:172-210; gate/up are fused per expert in the adjacent
+    (gate, up) column interleave; every stage boundary is one bf16 cast; the
+    combine ``sum_k down * w_k`` is evaluated in float32 and cast once.
+    """
+    hidden = np.asarray(hidden, dtype=F32)
+    n_experts = len(gate_up_weights)
+    weights, selected = moe_route(router_logits, top_k)
+    expanded = np.repeat(hidden, top_k, axis=0)
+    x_sorted, group_sizes, unsort, _ = prepare_routing(expanded, selected.ravel(), n_experts)
+    fused = bf16_round(grouped_quantized_lora_linear_f32(
+        x_sorted, group_sizes, gate_up_weights, gate_up_a, gate_up_b, scaling))
+    act = swiglu_from_interleaved(fused)
+    down = bf16_round(grouped_quantized_lora_linear_f32(
+        act, group_sizes, down_weights, down_a, down_b, scaling))
+    per_tok = down[unsort].reshape(hidden.shape[0], top_k, -1)
+    out = bf16_round(np.sum(per_tok * weights[..., None], axis=1, dtype=F32))
+    if return_stages:
+        return out, {"group_sizes": group_sizes, "unsort": unsort, "x_sorted": x_sorted,
+                     "fused": fused, "act": act, "down": down, "weights": weights,
+                     "selected": selected}
+    return out
+
+
+# ---------------------------------------------------------------------------
+# numerical gate (rocm/probe_w8a8_lora_forward.py:186-189, 1291-1369)
+# ---------------------------------------------------------------------------
+
+MAX_RELATIVE_L2_ERROR = 0.01
+MIN_COSINE_SIMILARITY = 0.9999
+MAX_ABSOLUTE_ERROR = 0.25
+
+
+def numerical_gate(candidate, expected) -> dict:
+    c = np.asarray(candidate, dtype=np.float64).ravel()
+    e = np.asarray(expected, dtype=np.float64).ravel()
+    diff = c - e
+    den = max(float(np.linalg.norm(e)), 1e-12)
+    rel_l2 = float(np.linalg.norm(diff)) / den
+    cos_den = float(np.linalg.norm(c)) * float(np.linalg.norm(e))
+    cosine = float(np.dot(c, e)) / cos_den if cos_den > 0 else (1.0 if not diff.any() else 0.0)
+    max_abs = float(np.max(np.abs(diff))) if diff.size else 0.0
+    finite = bool(np.all(np.isfinite(c)))
+    passed = finite and rel_l2 < MAX_RELATIVE_L2_ERROR and cosine >= MIN_COSINE_SIMILARITY \
+        and max_abs <= MAX_ABSOLUTE_ERROR
+    return {"relative_l2": rel_l2, "cosine": cosine, "max_abs": max_abs, "finite": finite,
+            "passed": passed}
+
+
+def within_tolerance(candidate, expected, atol: float = 2e-2, rtol: float = 1e-2) -> np.ndarray:
+    """Elementwise |a - b| <= atol + rtol * |b| (the bf16 output criterion)."""
+    c = np.asarray(candidate, dtype=np.float64)
+    e = np.asarray(expected, dtype=np.float64)
+    return np.abs(c - e) <= atol + rtol * np.abs(e)
