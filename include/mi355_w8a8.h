@@ -1,0 +1,156 @@
+/*
+ * mi355_w8a8.h -- plain C ABI of the MI355X (gfx950) W8A8 LoRA linear forward path.
+ *
+ * Every entry point enqueues work on the caller's HIP stream and returns; none
+ * synchronises, allocates or frees device memory, or keeps a pointer after it
+ * returns.  All pointers are device pointers unless marked "host".  A stream is
+ * passed as void* (a hipStream_t; NULL = the default stream).  Return value:
+ * MI355_W8A8_OK or a negative mi355_w8a8_status.
+ *
+ * What each entry point replaces in the reference (paths relative to its root):
+ *   - mi355_w8a8_quantize_rows_v1      skyrl/tx/kernels/quantized_lora.py:199-212
+ *                                      (= skyrl/tx/kernels/rocm/w8a8_lora.py:179-187)
+ *   - mi355_w8a8_pack_weight_v1        the load-time permutation sanctioned by
+ *                                      rocm/QUANTIZED_FFI.md:71-74 of the storage format
+ *                                      skyrl/tx/kernels/quantized_lora.py:20-41
+ *   - mi355_w8a8_lora_linear_v1        skyrl/tx/kernels/quantized_lora.py:400-453 and
+ *                                      skyrl/tx/kernels/rocm/w8a8_lora.py:827-920 (forward),
+ *                                      with the per-row adapter routing of
+ *                                      skyrl/tx/layers/lora.py:118-157
+ *   - mi355_w8a8_rms_gateup_swiglu_v1  skyrl/tx/kernels/rocm/bf16_rms_gate_up_lora_swiglu_contiguous.py:698-712
+ *                                      (forward) on W8A8 weights
+ *   - mi355_w8a8_lora_residual_v1      skyrl/tx/kernels/rocm/bf16_lora_residual.py:507-522 (forward)
+ *                                      on W8A8 weights
+ *   - mi355_w8a8_grouped_v1            skyrl/tx/layers/lora.py:394-444 (LoRAExpert.__call__) with
+ *                                      the ragged_dot of skyrl/tx/layers/util.py:8-59
+ * The typed-FFI handler shape these sit behind is rocm/QUANTIZED_FFI.md:589-599 and
+ * skyrl/tx/kernels/rocm/ffi/gdn_ffi_smoke.hip:43-82.
+ */
+#ifndef MI355_W8A8_H_
+#define MI355_W8A8_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355_W8A8_ABI_VERSION 1
+
+typedef enum mi355_w8a8_status {
+  MI355_W8A8_OK = 0,
+  MI355_W8A8_ERR_NULL = -1,        /* a required pointer is NULL */
+  MI355_W8A8_ERR_SHAPE = -2,       /* a dimension is zero, too large or inconsistent */
+  MI355_W8A8_ERR_ALIGN = -3,       /* a pointer is not 16-byte aligned */
+  MI355_W8A8_ERR_ALIAS = -4,       /* the output overlaps an input */
+  MI355_W8A8_ERR_WORKSPACE = -5,   /* workspace missing or too small */
+  MI355_W8A8_ERR_LAUNCH = -6,      /* the HIP runtime refused a launch */
+  MI355_W8A8_ERR_UNSUPPORTED = -7, /* valid request outside this build's geometry */
+  MI355_W8A8_ERR_STRUCT = -8       /* struct_size does not match this header */
+} mi355_w8a8_status;
+
+/* Flags of mi355_w8a8_problem.flags */
+#define MI355_W8A8_FLAG_SWIGLU 1u      /* out[m, j] = bf16(silu(y[m,2j]) * y[m,2j+1]); out is [M, N/2] */
+#define MI355_W8A8_FLAG_FORCE_TILED 2u /* never take the skinny-M (split-K) kernel */
+#define MI355_W8A8_FLAG_FORCE_SKINNY 4u/* always take the skinny-M kernel (M <= 32) */
+#define MI355_W8A8_FLAG_LORA_SPLIT2 8u /* carry x@A as 2 bf16 terms instead of 3 in the LoRA-B product */
+
+/*
+ * One forward call.  y = dequant(quant(n) @ W) + s[idx] * ((n @ A[idx]) @ B[idx]) (+ residual),
+ * n = x or rmsnorm(x).  The float32 epilogue is cast to bf16 exactly once.
+ */
+typedef struct mi355_w8a8_problem {
+  uint32_t struct_size;     /* sizeof(mi355_w8a8_problem) */
+  uint32_t flags;
+  uint32_t m;               /* rows of x */
+  uint32_t k;               /* in features; multiple of 8 */
+  uint32_t n;               /* out features of W (before SwiGLU halving) */
+  uint32_t n_adapters;      /* leading dim of lora_a/lora_b/lora_scaling; 0 = no LoRA */
+  uint32_t rank;            /* LoRA rank r (<= 64) */
+  float rms_eps;            /* used when rms_gamma != NULL */
+  const void* x;            /* bf16 [m, k] */
+  const void* w_packed;     /* from mi355_w8a8_pack_weight_v1 for the same (k, n) */
+  const float* w_scales;    /* f32 [n], one per output channel */
+  const void* lora_a;       /* bf16 [n_adapters, k, rank] or NULL */
+  const void* lora_b;       /* bf16 [n_adapters, rank, n] or NULL */
+  const float* lora_scaling;/* f32 [n_adapters] (alpha / rank) or NULL */
+  const int32_t* adapter_indices; /* int32 [m], one adapter per row; NULL = adapter 0 for every row */
+  const float* rms_gamma;   /* f32 [k] multiplier of the fused RMSNorm prologue, or NULL */
+  const void* residual;     /* bf16 [m, n_out] added in the f32 epilogue, or NULL */
+  void* out;                /* bf16 [m, n_out]; n_out = n, or n/2 with FLAG_SWIGLU */
+  void* workspace;          /* >= mi355_w8a8_workspace_bytes(...) bytes, 256-byte aligned */
+  uint64_t workspace_bytes;
+  /* Optional auxiliary outputs (NULL to skip); they exist for parity checks. */
+  int8_t* aux_x_codes;      /* int8 [m, k] row-major activation codes */
+  float* aux_x_scales;      /* f32 [m] activation scales */
+  int32_t* aux_acc;         /* int32 [m, n] raw integer accumulators */
+  void* aux_normalized;     /* bf16 [m, k] RMSNorm output (only with rms_gamma) */
+} mi355_w8a8_problem;
+
+/*
+ * Grouped (ragged) call: rows of x are already sorted by group (expert); group g owns
+ * group_sizes[g] consecutive rows, its own packed weight, scales and LoRA pair.
+ */
+typedef struct mi355_w8a8_grouped_problem {
+  uint32_t struct_size;     /* sizeof(mi355_w8a8_grouped_problem) */
+  uint32_t flags;           /* MI355_W8A8_FLAG_SWIGLU allowed */
+  uint32_t m;               /* total rows */
+  uint32_t k;
+  uint32_t n;
+  uint32_t n_groups;
+  uint32_t rank;            /* 0 = no LoRA */
+  uint32_t reserved;
+  const void* x;            /* bf16 [m, k] */
+  const void* w_packed;     /* n_groups packed weights back to back, each mi355_w8a8_packed_weight_bytes(k, n) */
+  const float* w_scales;    /* f32 [n_groups, n] */
+  const void* lora_a;       /* bf16 [n_groups, k, rank] or NULL */
+  const void* lora_b;       /* bf16 [n_groups, rank, n] or NULL */
+  const float* lora_scaling;/* f32 [n_groups] or NULL */
+  const int32_t* group_sizes; /* int32 [n_groups]; rows beyond sum(group_sizes) produce zeros */
+  void* out;                /* bf16 [m, n_out] */
+  void* workspace;
+  uint64_t workspace_bytes;
+  int8_t* aux_x_codes;
+  float* aux_x_scales;
+  int32_t* aux_acc;
+} mi355_w8a8_grouped_problem;
+
+int mi355_w8a8_abi_version(void);
+const char* mi355_w8a8_status_string(int status);
+
+/* Bytes of the packed form of a [k, n] int8 weight (0 when k or n is 0). */
+uint64_t mi355_w8a8_packed_weight_bytes(uint32_t k, uint32_t n);
+
+/* One-time re-layout of row-major int8 codes [k, n] into the MFMA fragment order. */
+int mi355_w8a8_pack_weight_v1(const int8_t* codes_kn, void* packed, uint32_t k, uint32_t n,
+                              void* stream);
+/* Inverse of the above (packed -> row-major [k, n]); used by tests and exporters. */
+int mi355_w8a8_unpack_weight_v1(const void* packed, int8_t* codes_kn, uint32_t k, uint32_t n,
+                                void* stream);
+
+/* Per-token dynamic symmetric int8 quantization: codes int8 [m, k], scales f32 [m]. */
+int mi355_w8a8_quantize_rows_v1(const void* x_bf16, int8_t* codes, float* scales, uint32_t m,
+                                uint32_t k, void* stream);
+
+/* Workspace requirement of the three dense entry points below. */
+uint64_t mi355_w8a8_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t n_adapters,
+                                    uint32_t rank, uint32_t flags);
+uint64_t mi355_w8a8_grouped_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups,
+                                            uint32_t rank, uint32_t flags);
+
+/* W8A8 linear + (multi-adapter) LoRA; rms_gamma, residual and FLAG_SWIGLU must be unset. */
+int mi355_w8a8_lora_linear_v1(const mi355_w8a8_problem* problem, void* stream);
+/* RMSNorm -> W8A8 gate/up + LoRA -> SwiGLU; requires rms_gamma and FLAG_SWIGLU, even n. */
+int mi355_w8a8_rms_gateup_swiglu_v1(const mi355_w8a8_problem* problem, void* stream);
+/* W8A8 down projection + LoRA + residual; requires residual. */
+int mi355_w8a8_lora_residual_v1(const mi355_w8a8_problem* problem, void* stream);
+/* Any combination of the optional stages (superset of the three above). */
+int mi355_w8a8_forward_v1(const mi355_w8a8_problem* problem, void* stream);
+/* Grouped / ragged per-expert variant. */
+int mi355_w8a8_grouped_v1(const mi355_w8a8_grouped_problem* problem, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_W8A8_H_ */

@@ -1,0 +1,12 @@
+"""MI355X-native W8A8 LoRA linear forward path (gfx950 HIP kernels behind a C ABI).
+
+The directory name carries a hyphen, so the package is imported through
+``__graft_entry__.load_package()`` (or any ``importlib`` spec loader) under the
+module name ``skyrl_tx_rocm_amd``.
+"""
+
+from . import _native  # noqa: F401
+from .kernels import quantized_lora  # noqa: F401
+from .kernels.rocm import w8a8_lora  # noqa: F401
+
+__all__ = ["_native", "quantized_lora", "w8a8_lora"]

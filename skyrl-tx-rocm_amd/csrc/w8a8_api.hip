@@ -1,0 +1,350 @@
+// C ABI of the MI355X W8A8 LoRA linear forward path: argument validation, workspace
+// carving and kernel launches.  Nothing here synchronises, allocates or keeps state.
+#include "../../include/mi355_w8a8.h"
+
+#include <hip/hip_runtime.h>
+
+#include "w8a8_device.h"
+#include "w8a8_gemm.h"
+#include "w8a8_prologue.h"
+#include "w8a8_skinny.h"
+
+using namespace w8a8;
+
+namespace {
+
+constexpr uint32_t kMaxK = 16384;
+constexpr uint32_t kMaxRows = 1u << 20;
+constexpr uint32_t kMaxN = 1u << 20;
+constexpr uint32_t kGemmLdsBytes = 131072;
+
+inline uint64_t align256(uint64_t v) { return (v + 255u) & ~uint64_t(255); }
+
+struct WsLayout {
+  uint64_t xq, sx, xn, z, src_row, dst_pos, blk_group, meta, skinny, total;
+  uint32_t slots, ksplit, r_pad, K_pad, KB, n_steps, steps_per_wave;
+};
+
+WsLayout make_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint32_t rank, bool routed) {
+  WsLayout w{};
+  w.K_pad = k_padded(k);
+  w.KB = w.K_pad / 32u;
+  w.slots = routed ? round_up(m + 32u * n_groups, kTileM) : round_up(m, kTileM);
+  w.r_pad = rank ? round_up(rank, 16u) : 0u;
+  w.n_steps = (k + 63u) / 64u;
+  const uint32_t n_pblk = w.slots / 32u;
+  uint32_t ks = 512u / n_pblk;
+  if (ks < 1u) ks = 1u;
+  if (ks > (uint32_t)kMaxKSplit) ks = kMaxKSplit;
+  const uint32_t by_steps = w.n_steps / 4u ? w.n_steps / 4u : 1u;
+  if (ks > by_steps) ks = by_steps;
+  w.ksplit = ks;
+  w.steps_per_wave = (w.n_steps + ks * 4u - 1u) / (ks * 4u);
+  uint64_t off = 0;
+  w.meta = off; off += 256;
+  w.xq = off; off += align256((uint64_t)w.slots * w.K_pad);
+  w.sx = off; off += align256((uint64_t)w.slots * 4u);
+  w.src_row = off; off += align256((uint64_t)w.slots * 4u);
+  w.dst_pos = off; off += align256((uint64_t)m * 4u);
+  w.blk_group = off; off += align256((uint64_t)(w.slots / 32u) * 4u + 2u * (n_groups + 1u) * 4u);
+  w.xn = off; off += rank ? align256((uint64_t)m * k * 2u) : 0u;
+  w.z = off; off += rank ? align256((uint64_t)kMaxKSplit * w.slots * w.r_pad * 4u) : 0u;
+  w.skinny = off; off += align256(skinny_workspace_bytes(m, n));
+  w.total = off;
+  return w;
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline bool overlaps(const void* a, uint64_t an, const void* b, uint64_t bn) {
+  if (!a || !b || an == 0 || bn == 0) return false;
+  const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
+  return a0 < b0 + bn && b0 < a0 + an;
+}
+
+inline int launch_status() { return hipGetLastError() == hipSuccess ? MI355_W8A8_OK : MI355_W8A8_ERR_LAUNCH; }
+
+template <bool RMS>
+int launch_quant(const QuantArgs& a, hipStream_t s) {
+  const uint32_t need = (a.K_pad + 511u) / 512u;
+  const dim3 grid((a.M + 3u) / 4u), block(256);
+#define W8A8_Q(NCH)                                                              \
+  if (need <= NCH) {                                                             \
+    hipLaunchKernelGGL((quant_rows_kernel<NCH, RMS>), grid, block, 0, s, a);     \
+    return launch_status();                                                      \
+  }
+  W8A8_Q(1) W8A8_Q(2) W8A8_Q(4) W8A8_Q(8) W8A8_Q(16) W8A8_Q(24) W8A8_Q(32)
+#undef W8A8_Q
+  return MI355_W8A8_ERR_UNSUPPORTED;
+}
+
+int validate_common(uint32_t m, uint32_t k, uint32_t n) {
+  if (m == 0 || k == 0 || n == 0) return MI355_W8A8_ERR_SHAPE;
+  if (m > kMaxRows || n > kMaxN) return MI355_W8A8_ERR_UNSUPPORTED;
+  if (k % 8u) return MI355_W8A8_ERR_UNSUPPORTED;
+  if (k_padded(k) > kMaxK) return MI355_W8A8_ERR_UNSUPPORTED;
+  return MI355_W8A8_OK;
+}
+
+enum Required { kReqNone = 0, kReqLinear = 1, kReqGateUp = 2, kReqResidual = 3 };
+
+int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
+  if (!p) return MI355_W8A8_ERR_NULL;
+  if (p->struct_size != sizeof(mi355_w8a8_problem)) return MI355_W8A8_ERR_STRUCT;
+  int st = validate_common(p->m, p->k, p->n);
+  if (st) return st;
+  if (!p->x || !p->w_packed || !p->w_scales || !p->out) return MI355_W8A8_ERR_NULL;
+  const bool swiglu = (p->flags & MI355_W8A8_FLAG_SWIGLU) != 0;
+  const bool rms = p->rms_gamma != nullptr;
+  const bool lora = p->n_adapters > 0;
+  if (req == kReqLinear && (swiglu || rms || p->residual)) return MI355_W8A8_ERR_SHAPE;
+  if (req == kReqGateUp && (!swiglu || !rms)) return MI355_W8A8_ERR_SHAPE;
+  if (req == kReqResidual && (!p->residual || swiglu)) return MI355_W8A8_ERR_SHAPE;
+  if (swiglu && (p->n & 1u)) return MI355_W8A8_ERR_SHAPE;
+  if ((p->flags & MI355_W8A8_FLAG_FORCE_TILED) && (p->flags & MI355_W8A8_FLAG_FORCE_SKINNY))
+    return MI355_W8A8_ERR_SHAPE;
+  if (lora) {
+    if (!p->lora_a || !p->lora_b || !p->lora_scaling) return MI355_W8A8_ERR_NULL;
+    if (p->rank == 0 || p->rank > (uint32_t)kMaxRank) return MI355_W8A8_ERR_UNSUPPORTED;
+    if (p->n_adapters > (uint32_t)kMaxAdapters) return MI355_W8A8_ERR_UNSUPPORTED;
+  } else if (p->adapter_indices) {
+    return MI355_W8A8_ERR_SHAPE;
+  }
+  if (p->aux_normalized && !rms) return MI355_W8A8_ERR_SHAPE;
+  const uint32_t n_out = swiglu ? p->n / 2u : p->n;
+  const uint64_t out_bytes = (uint64_t)p->m * n_out * 2u;
+  const uint64_t x_bytes = (uint64_t)p->m * p->k * 2u;
+  if (!aligned16(p->x) || !aligned16(p->w_packed) || !aligned16(p->out) || !aligned16(p->w_scales) ||
+      !aligned16(p->lora_a) || !aligned16(p->lora_b) || !aligned16(p->residual) ||
+      !aligned16(p->rms_gamma) || !aligned16(p->adapter_indices))
+    return MI355_W8A8_ERR_ALIGN;
+  if (overlaps(p->out, out_bytes, p->x, x_bytes) || overlaps(p->out, out_bytes, p->residual, out_bytes) ||
+      overlaps(p->out, out_bytes, p->w_packed, mi355_w8a8_packed_weight_bytes(p->k, p->n)) ||
+      overlaps(p->out, out_bytes, p->lora_b, (uint64_t)p->n_adapters * p->rank * p->n * 2u) ||
+      overlaps(p->out, out_bytes, p->lora_a, (uint64_t)p->n_adapters * p->rank * p->k * 2u) ||
+      overlaps(p->out, out_bytes, p->workspace, p->workspace_bytes))
+    return MI355_W8A8_ERR_ALIAS;
+
+  const bool routed = lora && p->adapter_indices && p->n_adapters > 1;
+  // The workspace is always sized for the routed layout so one allocation serves every call.
+  const uint64_t need = mi355_w8a8_workspace_bytes(p->m, p->k, p->n, p->n_adapters, p->rank, p->flags);
+  if (!p->workspace) return MI355_W8A8_ERR_WORKSPACE;
+  if (p->workspace_bytes < need) return MI355_W8A8_ERR_WORKSPACE;
+  if (reinterpret_cast<uintptr_t>(p->workspace) & 255u) return MI355_W8A8_ERR_ALIGN;
+  const WsLayout w = make_layout(p->m, p->k, p->n, p->n_adapters, lora ? p->rank : 0u, routed);
+  unsigned char* ws = static_cast<unsigned char*>(p->workspace);
+  int32_t* meta = reinterpret_cast<int32_t*>(ws + w.meta);
+  int32_t* src_row = reinterpret_cast<int32_t*>(ws + w.src_row);
+  int32_t* dst_pos = reinterpret_cast<int32_t*>(ws + w.dst_pos);
+  int32_t* blk_group = reinterpret_cast<int32_t*>(ws + w.blk_group);
+
+  (void)hipGetLastError();  // drop a stale error so it is not blamed on these launches
+
+  bool skinny = p->m <= (uint32_t)kSkinnyMaxRows && !(p->flags & MI355_W8A8_FLAG_FORCE_TILED) && !swiglu;
+  if ((p->flags & MI355_W8A8_FLAG_FORCE_SKINNY)) {
+    if (p->m > (uint32_t)kSkinnyMaxRows || swiglu) return MI355_W8A8_ERR_UNSUPPORTED;
+    skinny = true;
+  }
+  if (!skinny_supported()) skinny = false;
+
+  if (skinny) {
+    return launch_skinny(p, ws + w.xq, reinterpret_cast<float*>(ws + w.sx),
+                         reinterpret_cast<uint16_t*>(ws + w.xn), ws + w.skinny, w.K_pad, w.KB, s);
+  }
+
+  if (routed) {
+    hipLaunchKernelGGL(route_rows_kernel, dim3(1), dim3(1024), 0, s, p->adapter_indices, p->m,
+                       p->n_adapters, w.slots, meta, src_row, dst_pos, blk_group);
+    if ((st = launch_status())) return st;
+  }
+
+  QuantArgs q{};
+  q.x = static_cast<const uint16_t*>(p->x);
+  q.gamma = p->rms_gamma;
+  q.eps = p->rms_eps;
+  q.M = p->m; q.K = p->k; q.K_pad = w.K_pad; q.KB = w.KB;
+  q.dst_pos = routed ? dst_pos : nullptr;
+  q.xq_packed = ws + w.xq;
+  q.sx_slots = reinterpret_cast<float*>(ws + w.sx);
+  q.codes_rm = p->aux_x_codes;
+  q.scales_rm = p->aux_x_scales;
+  q.xn = (rms && lora) ? reinterpret_cast<uint16_t*>(ws + w.xn) : nullptr;
+  q.xn_aux = static_cast<uint16_t*>(p->aux_normalized);
+  st = rms ? launch_quant<true>(q, s) : launch_quant<false>(q, s);
+  if (st) return st;
+
+  if (lora) {
+    LoraAArgs la{};
+    la.xsrc = rms ? reinterpret_cast<const uint16_t*>(ws + w.xn) : static_cast<const uint16_t*>(p->x);
+    la.lora_a = static_cast<const uint16_t*>(p->lora_a);
+    la.src_row = routed ? src_row : nullptr;
+    la.blk_group = routed ? blk_group : nullptr;
+    la.meta = routed ? meta : nullptr;
+    la.z_part = reinterpret_cast<float*>(ws + w.z);
+    la.M = p->m; la.K = p->k; la.r = p->rank; la.r_pad = w.r_pad; la.slots = w.slots;
+    la.rows_static = round_up(p->m, 32u);
+    la.steps_per_wave = w.steps_per_wave; la.n_steps = w.n_steps;
+    const dim3 grid(w.slots / 32u, w.ksplit), block(256);
+    if (w.r_pad > 32u) hipLaunchKernelGGL((lora_a_kernel<2>), grid, block, 0, s, la);
+    else hipLaunchKernelGGL((lora_a_kernel<1>), grid, block, 0, s, la);
+    if ((st = launch_status())) return st;
+  }
+
+  GemmArgs g{};
+  g.xq = ws + w.xq;
+  g.wp = static_cast<const unsigned char*>(p->w_packed);
+  g.sx = reinterpret_cast<const float*>(ws + w.sx);
+  g.sw = p->w_scales;
+  g.z_part = lora ? reinterpret_cast<const float*>(ws + w.z) : nullptr;
+  g.lora_b = static_cast<const uint16_t*>(p->lora_b);
+  g.lora_scaling = p->lora_scaling;
+  g.src_row = routed ? src_row : nullptr;
+  g.blk_group = routed ? blk_group : nullptr;
+  g.meta = routed ? meta : nullptr;
+  g.residual = static_cast<const uint16_t*>(p->residual);
+  g.out = p->out;
+  g.w_group_stride = 0;
+  g.M = p->m; g.N = p->n; g.K_pad = w.K_pad; g.KB = w.KB; g.slots = w.slots;
+  g.rows_static = round_up(p->m, 32u);
+  g.tiles_m = w.slots / kTileM;
+  g.tiles_n = n_padded(p->n) / kTileN;
+  g.rank = lora ? p->rank : 0u;
+  g.r_pad = w.r_pad;
+  g.ksplit = w.ksplit;
+  g.nsplit_terms = (p->flags & MI355_W8A8_FLAG_LORA_SPLIT2) ? 2u : 3u;
+  g.grouped = 0;
+  const uint32_t ntile = g.tiles_m * g.tiles_n;
+  const dim3 grid(((ntile + 7u) / 8u) * 8u), block(256);
+  if (p->aux_acc) {
+    GemmArgs ga = g;
+    ga.out = p->aux_acc;
+    ga.residual = nullptr;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm_kernel<kEpiAcc>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes) != hipSuccess)
+      return MI355_W8A8_ERR_LAUNCH;
+    hipLaunchKernelGGL((w8a8_gemm_kernel<kEpiAcc>), grid, block, kGemmLdsBytes, s, ga);
+    if ((st = launch_status())) return st;
+  }
+  if (swiglu) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm_kernel<kEpiSwiglu>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes) != hipSuccess)
+      return MI355_W8A8_ERR_LAUNCH;
+    hipLaunchKernelGGL((w8a8_gemm_kernel<kEpiSwiglu>), grid, block, kGemmLdsBytes, s, g);
+  } else {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm_kernel<kEpiPlain>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes) != hipSuccess)
+      return MI355_W8A8_ERR_LAUNCH;
+    hipLaunchKernelGGL((w8a8_gemm_kernel<kEpiPlain>), grid, block, kGemmLdsBytes, s, g);
+  }
+  return launch_status();
+}
+
+}  // namespace
+
+extern "C" {
+
+int mi355_w8a8_abi_version(void) { return MI355_W8A8_ABI_VERSION; }
+
+const char* mi355_w8a8_status_string(int status) {
+  switch (status) {
+    case MI355_W8A8_OK: return "ok";
+    case MI355_W8A8_ERR_NULL: return "a required pointer is NULL";
+    case MI355_W8A8_ERR_SHAPE: return "a dimension or flag combination is invalid";
+    case MI355_W8A8_ERR_ALIGN: return "a pointer is not sufficiently aligned";
+    case MI355_W8A8_ERR_ALIAS: return "the output overlaps an input or the workspace";
+    case MI355_W8A8_ERR_WORKSPACE: return "workspace missing or too small";
+    case MI355_W8A8_ERR_LAUNCH: return "the HIP runtime refused a launch";
+    case MI355_W8A8_ERR_UNSUPPORTED: return "request outside the supported geometry";
+    case MI355_W8A8_ERR_STRUCT: return "struct_size does not match this library";
+    default: return "unknown status";
+  }
+}
+
+uint64_t mi355_w8a8_packed_weight_bytes(uint32_t k, uint32_t n) {
+  if (k == 0 || n == 0) return 0;
+  return (uint64_t)k_padded(k) * n_padded(n);
+}
+
+int mi355_w8a8_pack_weight_v1(const int8_t* codes_kn, void* packed, uint32_t k, uint32_t n, void* stream) {
+  if (!codes_kn || !packed) return MI355_W8A8_ERR_NULL;
+  if (k == 0 || n == 0) return MI355_W8A8_ERR_SHAPE;
+  if (n > kMaxN || k > (1u << 20)) return MI355_W8A8_ERR_UNSUPPORTED;
+  if (!aligned16(packed)) return MI355_W8A8_ERR_ALIGN;
+  const uint64_t bytes = mi355_w8a8_packed_weight_bytes(k, n);
+  if (overlaps(codes_kn, (uint64_t)k * n, packed, bytes)) return MI355_W8A8_ERR_ALIAS;
+  const uint64_t chunks = bytes / 16u;
+  (void)hipGetLastError();
+  hipLaunchKernelGGL(pack_weight_kernel, dim3((uint32_t)((chunks + 255u) / 256u)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), codes_kn, static_cast<unsigned char*>(packed), k, n,
+                     k_padded(k) / 32u, chunks);
+  return launch_status();
+}
+
+int mi355_w8a8_unpack_weight_v1(const void* packed, int8_t* codes_kn, uint32_t k, uint32_t n, void* stream) {
+  if (!codes_kn || !packed) return MI355_W8A8_ERR_NULL;
+  if (k == 0 || n == 0) return MI355_W8A8_ERR_SHAPE;
+  if (n > kMaxN || k > (1u << 20)) return MI355_W8A8_ERR_UNSUPPORTED;
+  if (overlaps(codes_kn, (uint64_t)k * n, packed, mi355_w8a8_packed_weight_bytes(k, n)))
+    return MI355_W8A8_ERR_ALIAS;
+  const uint64_t total = (uint64_t)k * n;
+  (void)hipGetLastError();
+  hipLaunchKernelGGL(unpack_weight_kernel, dim3((uint32_t)((total + 255u) / 256u)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const unsigned char*>(packed), codes_kn, k, n,
+                     k_padded(k) / 32u);
+  return launch_status();
+}
+
+int mi355_w8a8_quantize_rows_v1(const void* x_bf16, int8_t* codes, float* scales, uint32_t m, uint32_t k,
+                                void* stream) {
+  if (!x_bf16 || !codes || !scales) return MI355_W8A8_ERR_NULL;
+  int st = validate_common(m, k, 1);
+  if (st) return st;
+  if (!aligned16(x_bf16) || (reinterpret_cast<uintptr_t>(codes) & 7u) || (reinterpret_cast<uintptr_t>(scales) & 3u))
+    return MI355_W8A8_ERR_ALIGN;
+  if (overlaps(x_bf16, (uint64_t)m * k * 2u, codes, (uint64_t)m * k) ||
+      overlaps(x_bf16, (uint64_t)m * k * 2u, scales, (uint64_t)m * 4u) ||
+      overlaps(codes, (uint64_t)m * k, scales, (uint64_t)m * 4u))
+    return MI355_W8A8_ERR_ALIAS;
+  QuantArgs q{};
+  q.x = static_cast<const uint16_t*>(x_bf16);
+  q.M = m; q.K = k; q.K_pad = k_padded(k); q.KB = q.K_pad / 32u;
+  q.codes_rm = codes;
+  q.scales_rm = scales;
+  (void)hipGetLastError();
+  return launch_quant<false>(q, static_cast<hipStream_t>(stream));
+}
+
+uint64_t mi355_w8a8_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t n_adapters, uint32_t rank,
+                                    uint32_t flags) {
+  (void)flags;
+  if (validate_common(m, k, n)) return 0;
+  if (n_adapters > (uint32_t)kMaxAdapters || rank > (uint32_t)kMaxRank) return 0;
+  return make_layout(m, k, n, n_adapters, n_adapters ? rank : 0u, n_adapters > 1).total;
+}
+
+int mi355_w8a8_lora_linear_v1(const mi355_w8a8_problem* p, void* stream) {
+  return run_forward(p, static_cast<hipStream_t>(stream), kReqLinear);
+}
+int mi355_w8a8_rms_gateup_swiglu_v1(const mi355_w8a8_problem* p, void* stream) {
+  return run_forward(p, static_cast<hipStream_t>(stream), kReqGateUp);
+}
+int mi355_w8a8_lora_residual_v1(const mi355_w8a8_problem* p, void* stream) {
+  return run_forward(p, static_cast<hipStream_t>(stream), kReqResidual);
+}
+int mi355_w8a8_forward_v1(const mi355_w8a8_problem* p, void* stream) {
+  return run_forward(p, static_cast<hipStream_t>(stream), kReqNone);
+}
+
+uint64_t mi355_w8a8_grouped_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint32_t rank,
+                                            uint32_t flags) {
+  (void)m; (void)k; (void)n; (void)n_groups; (void)rank; (void)flags;
+  return 0;
+}
+
+int mi355_w8a8_grouped_v1(const mi355_w8a8_grouped_problem* p, void* stream) {
+  (void)stream;
+  if (!p) return MI355_W8A8_ERR_NULL;
+  if (p->struct_size != sizeof(mi355_w8a8_grouped_problem)) return MI355_W8A8_ERR_STRUCT;
+  return MI355_W8A8_ERR_UNSUPPORTED;
+}
+
+}  // extern "C"

@@ -1,0 +1,338 @@
+// Prologue kernels: weight (un)packing, adapter routing, per-token quantization with the
+// optional fused RMSNorm, and the LoRA-A projection z = n @ A[adapter].
+#pragma once
+#include "w8a8_device.h"
+
+namespace w8a8 {
+
+// ---------------------------------------------------------------------------------------
+// Weight pack / unpack (one time per weight)
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void pack_weight_kernel(const int8_t* __restrict__ codes,
+                                                          unsigned char* __restrict__ packed, uint32_t K,
+                                                          uint32_t N, uint32_t KB, uint64_t n_chunks) {
+  uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;  // one 16-byte chunk per thread
+  if (idx >= n_chunks) return;
+  uint32_t lane = idx & 63u;
+  uint64_t blk = idx >> 6;
+  uint32_t kb = (uint32_t)(blk % KB);
+  uint32_t nb = (uint32_t)(blk / KB);
+  uint32_t c = nb * 32u + (lane & 31u);
+  uint32_t n = packed_to_orig_col(c);
+  uint32_t k0 = kb * 32u + 16u * (lane >> 5);
+  uint32_t w[4] = {0, 0, 0, 0};
+  if (n < N) {
+#pragma unroll
+    for (int b = 0; b < 16; ++b) {
+      uint32_t k = k0 + b;
+      uint32_t v = (k < K) ? (uint32_t)(uint8_t)codes[(size_t)k * N + n] : 0u;
+      w[b >> 2] |= v << (8 * (b & 3));
+    }
+  }
+  uint4 o = make_uint4(w[0], w[1], w[2], w[3]);
+  *reinterpret_cast<uint4*>(packed + idx * 16) = o;
+}
+
+__global__ __launch_bounds__(256) void unpack_weight_kernel(const unsigned char* __restrict__ packed,
+                                                            int8_t* __restrict__ codes, uint32_t K, uint32_t N,
+                                                            uint32_t KB) {
+  uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (uint64_t)K * N) return;
+  uint32_t k = (uint32_t)(idx / N), n = (uint32_t)(idx % N);
+  // packed column of original column n
+  uint32_t c = (n & ~63u) + 32u * (n & 1u) + ((n & 63u) >> 1);
+  codes[idx] = (int8_t)packed[packed_offset(c, k, KB)];
+}
+
+// ---------------------------------------------------------------------------------------
+// Adapter routing: group rows by adapter, every group padded to a multiple of 32 rows
+// (the counterpart of prepare_routing, skyrl/tx/layers/util.py:66-87).
+//   meta[0]       = number of grouped row slots in use (multiple of 32)
+//   src_row[p]    = original row of grouped slot p, or -1 for padding
+//   dst_pos[m]    = grouped slot of original row m
+//   blk_group[b]  = adapter of the 32-row block b
+// Out-of-range adapter indices are clamped into range (XLA gather semantics).
+// One workgroup; the order of rows inside a group does not influence any result.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void route_rows_kernel(const int32_t* __restrict__ idx, uint32_t M,
+                                                          uint32_t n_groups, uint32_t slots,
+                                                          int32_t* __restrict__ meta, int32_t* __restrict__ src_row,
+                                                          int32_t* __restrict__ dst_pos,
+                                                          int32_t* __restrict__ blk_group) {
+  __shared__ int cnt[kMaxAdapters];
+  __shared__ int start[kMaxAdapters + 1];
+  __shared__ int cursor[kMaxAdapters];
+  const uint32_t tid = threadIdx.x;
+  if (tid < kMaxAdapters) { cnt[tid] = 0; cursor[tid] = 0; }
+  __syncthreads();
+  for (uint32_t i = tid; i < M; i += 1024) {
+    int a = idx[i];
+    a = a < 0 ? 0 : (a >= (int)n_groups ? (int)n_groups - 1 : a);
+    atomicAdd(&cnt[a], 1);
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int pos = 0;
+    for (uint32_t a = 0; a < n_groups; ++a) {
+      start[a] = pos;
+      pos += (cnt[a] + 31) & ~31;
+    }
+    start[n_groups] = pos;
+    meta[0] = pos;
+  }
+  __syncthreads();
+  for (uint32_t p = tid; p < slots; p += 1024) src_row[p] = -1;
+  const int total = start[n_groups];
+  for (uint32_t b = tid; b < slots / 32; b += 1024) {
+    int g = 0;
+    int row = (int)b * 32;
+    if (row < total) {
+      for (uint32_t a = 0; a < n_groups; ++a)
+        if (row >= start[a] && row < start[a + 1]) g = (int)a;
+    }
+    blk_group[b] = g;
+  }
+  __syncthreads();
+  for (uint32_t i = tid; i < M; i += 1024) {
+    int a = idx[i];
+    a = a < 0 ? 0 : (a >= (int)n_groups ? (int)n_groups - 1 : a);
+    int p = start[a] + atomicAdd(&cursor[a], 1);
+    src_row[p] = (int)i;
+    dst_pos[i] = p;
+  }
+}
+
+// Same tables for rows that arrive already grouped (ragged groups of an expert layer,
+// skyrl/tx/layers/util.py:8-59): group g owns group_sizes[g] consecutive rows; rows past
+// sum(group_sizes) get dst_pos = -1 and the caller's output rows are zero-filled.
+__global__ __launch_bounds__(1024) void route_groups_kernel(const int32_t* __restrict__ group_sizes, uint32_t M,
+                                                            uint32_t n_groups, uint32_t slots,
+                                                            int32_t* __restrict__ meta, int32_t* __restrict__ src_row,
+                                                            int32_t* __restrict__ dst_pos,
+                                                            int32_t* __restrict__ blk_group,
+                                                            int32_t* __restrict__ row_start /* [n_groups+1] scratch */,
+                                                            int32_t* __restrict__ slot_start /* [n_groups+1] scratch */) {
+  const uint32_t tid = threadIdx.x;
+  if (tid == 0) {
+    int r = 0, p = 0;
+    for (uint32_t g = 0; g < n_groups; ++g) {
+      int sz = group_sizes[g];
+      if (sz < 0) sz = 0;
+      if (r + sz > (int)M) sz = (int)M - r;
+      row_start[g] = r;
+      slot_start[g] = p;
+      r += sz;
+      p += (sz + 31) & ~31;
+    }
+    row_start[n_groups] = r;
+    slot_start[n_groups] = p;
+    meta[0] = p;
+  }
+  __syncthreads();
+  __threadfence_block();
+  for (uint32_t p = tid; p < slots; p += 1024) src_row[p] = -1;
+  for (uint32_t i = tid; i < M; i += 1024) dst_pos[i] = -1;
+  for (uint32_t b = tid; b < slots / 32; b += 1024) blk_group[b] = 0;
+  __syncthreads();
+  // one wave per group walks its rows
+  const uint32_t wave = tid >> 6, lane = tid & 63;
+  for (uint32_t g = wave; g < n_groups; g += 16) {
+    int r0 = row_start[g], r1 = row_start[g + 1], p0 = slot_start[g], p1 = slot_start[g + 1];
+    for (int i = (int)lane; i < r1 - r0; i += 64) {
+      src_row[p0 + i] = r0 + i;
+      dst_pos[r0 + i] = p0 + i;
+    }
+    for (int b = p0 / 32 + (int)lane; b < p1 / 32; b += 64) blk_group[b] = (int)g;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Per-token dynamic int8 quantization (skyrl/tx/kernels/quantized_lora.py:199-212 with one
+// group per row), optionally preceded by RMSNorm
+// (skyrl/tx/kernels/rocm/bf16_rms_gate_up_lora_swiglu.py:299-303).  One wave per row; the
+// row lives in registers (NCH chunks of 8 bf16 per lane).  Bit-exact rules:
+//   scale = amax > 0 ? amax / 127 : 1         IEEE float32 division
+//   code  = clamp(rint(v / scale), -127, 127) IEEE division, round half to even
+//   RMSNorm: mean = float(sum_f64(x*x) / K), inv = 1 / sqrt(mean + eps) (IEEE), and
+//            n = bf16((x * inv) * gamma) with two separate float32 multiplications.
+// ---------------------------------------------------------------------------------------
+struct QuantArgs {
+  const uint16_t* x;       // bf16 [M, K]
+  const float* gamma;      // f32 [K] or null
+  float eps;
+  uint32_t M, K, K_pad, KB;
+  const int32_t* dst_pos;  // grouped slot per row or null (identity)
+  unsigned char* xq_packed;// packed codes or null
+  float* sx_slots;         // f32 per grouped slot or null
+  int8_t* codes_rm;        // row-major codes [M, K] or null
+  float* scales_rm;        // f32 [M] or null
+  uint16_t* xn;            // bf16 [M, K] normalized rows or null
+  uint16_t* xn_aux;        // second copy for the caller or null
+};
+
+template <int NCH, bool RMS>
+__global__ __launch_bounds__(256) void quant_rows_kernel(QuantArgs a) {
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t m = blockIdx.x * 4u + (threadIdx.x >> 6);
+  if (m >= a.M) return;
+  const uint16_t* xr = a.x + (size_t)m * a.K;
+  float v[NCH][8];
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) {
+    uint32_t k0 = (j * 64u + lane) * 8u;
+    uint4 raw = make_uint4(0, 0, 0, 0);
+    if (k0 < a.K) raw = *reinterpret_cast<const uint4*>(xr + k0);
+    uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      v[j][2 * e] = __uint_as_float(w[e] << 16);
+      v[j][2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+    }
+  }
+  if (RMS) {
+    double ss = 0.0;
+#pragma unroll
+    for (int j = 0; j < NCH; ++j)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += (double)v[j][e] * (double)v[j][e];
+    ss = wave_sum(ss);
+    float var = (float)(ss / (double)a.K);
+    float inv = 1.0f / sqrtf(var + a.eps);
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      uint32_t k0 = (j * 64u + lane) * 8u;
+      if (k0 < a.K) {
+        float4 g0 = *reinterpret_cast<const float4*>(a.gamma + k0);
+        float4 g1 = *reinterpret_cast<const float4*>(a.gamma + k0 + 4);
+        float g[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+        uint32_t packed[4];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          float t = v[j][e] * inv;
+          t = t * g[e];
+          uint32_t b = f32_to_bf16_bits(t);
+          v[j][e] = __uint_as_float(b << 16);
+          if (e & 1) packed[e >> 1] |= b << 16; else packed[e >> 1] = b;
+        }
+        uint4 o = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+        if (a.xn) *reinterpret_cast<uint4*>(a.xn + (size_t)m * a.K + k0) = o;
+        if (a.xn_aux) *reinterpret_cast<uint4*>(a.xn_aux + (size_t)m * a.K + k0) = o;
+      }
+    }
+  }
+  float amax = 0.0f;
+#pragma unroll
+  for (int j = 0; j < NCH; ++j)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(v[j][e]));
+  amax = wave_max(amax);
+  const float scale = amax > 0.0f ? amax / 127.0f : 1.0f;
+  const int p = a.dst_pos ? a.dst_pos[m] : (int)m;
+  if (lane == 0) {
+    if (a.sx_slots && p >= 0) a.sx_slots[p] = scale;
+    if (a.scales_rm) a.scales_rm[m] = scale;
+  }
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) {
+    uint32_t c = j * 64u + lane;
+    uint32_t k0 = c * 8u;
+    if (k0 >= a.K_pad) continue;
+    uint32_t lo = 0, hi = 0;
+    if (k0 < a.K) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float q = rintf(v[j][e] / scale);
+        q = fminf(fmaxf(q, -127.0f), 127.0f);
+        uint32_t b = (uint32_t)(int)q & 0xffu;
+        if (e < 4) lo |= b << (8 * e); else hi |= b << (8 * (e - 4));
+      }
+      if (a.codes_rm) *reinterpret_cast<uint2*>(a.codes_rm + (size_t)m * a.K + k0) = make_uint2(lo, hi);
+    }
+    if (a.xq_packed && p >= 0)
+      *reinterpret_cast<uint2*>(a.xq_packed + packed_offset((uint32_t)p, k0, a.KB)) = make_uint2(lo, hi);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// LoRA-A projection on bf16 MFMA: z[p, :] = n[src_row[p], :] @ A[group(p)]  (float32
+// accumulation of exact bf16 products; skyrl/tx/kernels/quantized_lora.py:300-301 and
+// skyrl/tx/layers/lora.py:150).  Grid (32-row blocks, ksplit); the four waves of a
+// workgroup take disjoint K ranges and are reduced through LDS in wave order, K splits
+// are written as separate partials that the GEMM epilogue adds in split order.
+// ---------------------------------------------------------------------------------------
+struct LoraAArgs {
+  const uint16_t* xsrc;     // bf16 [M, K] (x, or the normalized rows)
+  const uint16_t* lora_a;   // bf16 [n_groups, K, r]
+  const int32_t* src_row;   // or null (identity)
+  const int32_t* blk_group; // or null (group 0)
+  const int32_t* meta;      // or null
+  float* z_part;            // f32 [ksplit, slots, r_pad]
+  uint32_t M, K, r, r_pad, slots, rows_static, steps_per_wave, n_steps;
+};
+
+template <int RB>  // number of 32-wide rank blocks (1 or 2)
+__global__ __launch_bounds__(256) void lora_a_kernel(LoraAArgs a) {
+  __shared__ float red[4][RB][16][64];
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  const uint32_t pb = blockIdx.x, ks = blockIdx.y;
+  const uint32_t total = a.meta ? (uint32_t)a.meta[0] : a.rows_static;
+  if (pb * 32u >= total) return;
+  const uint32_t grp = a.blk_group ? (uint32_t)a.blk_group[pb] : 0u;
+  const uint32_t i = lane & 31u, h = lane >> 5;
+  const uint32_t p = pb * 32u + i;
+  int src = a.src_row ? a.src_row[p] : (int)p;
+  if (src >= (int)a.M) src = -1;
+  const uint16_t* xr = a.xsrc + (size_t)(src < 0 ? 0 : src) * a.K;
+  const uint16_t* Ag = a.lora_a + (size_t)grp * a.K * a.r;
+  v16f acc[RB];
+#pragma unroll
+  for (int b = 0; b < RB; ++b)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[b][e] = 0.0f;
+  const uint32_t wg = ks * 4u + wave;
+  uint32_t s0 = wg * a.steps_per_wave, s1 = s0 + a.steps_per_wave;
+  if (s1 > a.n_steps) s1 = a.n_steps;
+  for (uint32_t s = s0; s < s1; ++s) {
+    const uint32_t kbase = s * 64u + 32u * h;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const uint32_t k0 = kbase + 8u * t;
+      v8us xa = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (src >= 0 && k0 < a.K) xa = *reinterpret_cast<const v8us*>(xr + k0);
+#pragma unroll
+      for (int b = 0; b < RB; ++b) {
+        const uint32_t col = b * 32u + i;
+        v8us wb = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (col < a.r && k0 < a.K) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) wb[e] = Ag[(size_t)(k0 + e) * a.r + col];
+        }
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, xa),
+                                                         __builtin_bit_cast(v8bf, wb), acc[b], 0, 0, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int b = 0; b < RB; ++b)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) red[wave][b][e][lane] = acc[b][e];
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int b = 0; b < RB; ++b) {
+      const uint32_t col = b * 32u + i;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        float sum = red[0][b][e][lane];
+        sum += red[1][b][e][lane];
+        sum += red[2][b][e][lane];
+        sum += red[3][b][e][lane];
+        const uint32_t row = 8u * (e >> 2) + 4u * h + (e & 3u);
+        if (col < a.r_pad)
+          a.z_part[((size_t)ks * a.slots + pb * 32u + row) * a.r_pad + col] = sum;
+      }
+    }
+  }
+}
+
+}  // namespace w8a8

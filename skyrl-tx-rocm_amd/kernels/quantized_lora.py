@@ -1,0 +1,171 @@
+"""Storage format and public entry points of the grouped-quantized LoRA linear.
+
+Mirrors the interface of the reference's ``skyrl/tx/kernels/quantized_lora.py``
+(``GroupQuantizedWeight`` :20-41, ``quantize_frozen_weight`` :128-171,
+``dequantize_frozen_weight`` :180-196, ``quantized_frozen_linear`` :257-272,
+``quantized_lora_linear`` :400-453) on torch tensors.  The forward functions run the
+gfx950 HIP kernels; they accept the per-token / per-channel geometry
+(``bits == 8``, ``group_size == K``, ``activation_bits == 8``) and raise
+``ValueError`` for anything else so a caller can keep its own path for those.
+The weight quantizer is an offline, one-time torch computation.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+
+@dataclass(frozen=True)
+class GroupQuantizedWeight:
+    """K x N weight grouped along K with one scale per (group, output)."""
+
+    codes: torch.Tensor
+    scales: torch.Tensor
+    original_in_features: int
+    padded_in_features: int
+    bits: int
+    group_size: int
+
+
+def _validate_bits(bits: int) -> None:
+    if bits not in (4, 8):
+        raise ValueError(f"bits must be 4 or 8, got {bits}")
+
+
+def _validate_group_size(group_size: int) -> None:
+    if group_size <= 0 or group_size % 2:
+        raise ValueError(f"group_size must be a positive even integer, got {group_size}")
+
+
+def validate_quantized_weight(weight: GroupQuantizedWeight) -> None:
+    _validate_bits(weight.bits)
+    _validate_group_size(weight.group_size)
+    if weight.original_in_features <= 0 or weight.padded_in_features <= 0:
+        raise ValueError("quantized weight input dimensions must be positive")
+    if weight.padded_in_features < weight.original_in_features:
+        raise ValueError("padded_in_features must be at least original_in_features")
+    if weight.padded_in_features % weight.group_size:
+        raise ValueError("padded_in_features must be divisible by group_size")
+    if weight.codes.ndim != 2 or weight.scales.ndim != 2:
+        raise ValueError("quantized weight codes and scales must both be rank-two")
+    rows = weight.padded_in_features // (2 if weight.bits == 4 else 1)
+    scale_shape = (weight.padded_in_features // weight.group_size, weight.codes.shape[1])
+    if weight.codes.shape[0] != rows:
+        raise ValueError(f"code rows {weight.codes.shape[0]} do not match expected {rows}")
+    if tuple(weight.scales.shape) != scale_shape:
+        raise ValueError(f"scale shape {tuple(weight.scales.shape)} does not match expected {scale_shape}")
+    if weight.codes.shape[1] <= 0:
+        raise ValueError("quantized weight output dimension must be positive")
+    want = torch.uint8 if weight.bits == 4 else torch.int8
+    if weight.codes.dtype != want:
+        raise TypeError(f"W{weight.bits} codes must have dtype {want}, got {weight.codes.dtype}")
+    if not weight.scales.dtype.is_floating_point:
+        raise TypeError(f"quantized weight scales must be floating point, got {weight.scales.dtype}")
+
+
+def pack_signed_int4(values: torch.Tensor) -> torch.Tensor:
+    if values.ndim < 1 or values.shape[0] == 0 or values.shape[0] % 2:
+        raise ValueError("signed INT4 packing requires an even, nonempty axis zero")
+    if values.dtype.is_floating_point or values.dtype == torch.bool:
+        raise TypeError(f"signed INT4 values must be integral, got {values.dtype}")
+    low = (values[0::2].to(torch.int16) & 0xF).to(torch.uint8)
+    high = (values[1::2].to(torch.int16) & 0xF).to(torch.uint8)
+    return low | (high << 4)
+
+
+def unpack_signed_int4(packed: torch.Tensor) -> torch.Tensor:
+    if packed.ndim < 1 or packed.shape[0] == 0:
+        raise ValueError("signed INT4 input must have a nonempty axis zero")
+    if packed.dtype != torch.uint8:
+        raise TypeError(f"packed signed INT4 values must be uint8, got {packed.dtype}")
+    low = (packed & 0xF).to(torch.int16)
+    high = (packed >> 4).to(torch.int16)
+    low = torch.where(low >= 8, low - 16, low).to(torch.int8)
+    high = torch.where(high >= 8, high - 16, high).to(torch.int8)
+    return torch.stack((low, high), dim=1).reshape((packed.shape[0] * 2, *packed.shape[1:]))
+
+
+def quantize_frozen_weight(weight: torch.Tensor, *, bits: int = 8, group_size: int = 64,
+                           scale_dtype: torch.dtype = torch.bfloat16) -> GroupQuantizedWeight:
+    """Symmetric per-(group, output) quantizer (offline, once per weight)."""
+    _validate_bits(bits)
+    _validate_group_size(group_size)
+    if weight.ndim != 2:
+        raise ValueError(f"weight must have shape [K, N], got {tuple(weight.shape)}")
+    if weight.shape[0] <= 0 or weight.shape[1] <= 0:
+        raise ValueError(f"weight dimensions must be positive, got {tuple(weight.shape)}")
+    if not weight.dtype.is_floating_point:
+        raise TypeError(f"weight must be floating point, got {weight.dtype}")
+    if not scale_dtype.is_floating_point:
+        raise TypeError(f"scale_dtype must be floating point, got {scale_dtype}")
+    k, n = weight.shape
+    k_pad = ((k + group_size - 1) // group_size) * group_size
+    padded = torch.zeros((k_pad, n), dtype=torch.float32, device=weight.device)
+    padded[:k] = weight.to(torch.float32)
+    grouped = padded.reshape(-1, group_size, n)
+    qmax = (1 << (bits - 1)) - 1
+    amax = grouped.abs().amax(dim=1)
+    scales = torch.where(amax > 0, amax / qmax, torch.ones_like(amax))
+    q = torch.clamp(torch.round(grouped / scales[:, None, :]), -qmax, qmax).to(torch.int8)
+    q = q.reshape(k_pad, n)
+    codes = q if bits == 8 else pack_signed_int4(q)
+    return GroupQuantizedWeight(codes=codes, scales=scales.to(scale_dtype), original_in_features=k,
+                                padded_in_features=k_pad, bits=bits, group_size=group_size)
+
+
+def dequantize_frozen_weight(weight: GroupQuantizedWeight, *, dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    validate_quantized_weight(weight)
+    if not dtype.is_floating_point:
+        raise TypeError(f"dequantized weight dtype must be floating point, got {dtype}")
+    codes = weight.codes if weight.bits == 8 else unpack_signed_int4(weight.codes)
+    codes = codes[: weight.padded_in_features]
+    n = codes.shape[1]
+    grouped = codes.reshape(-1, weight.group_size, n).to(torch.float32)
+    deq = grouped * weight.scales.to(torch.float32)[:, None, :]
+    return deq.reshape(weight.padded_in_features, n)[: weight.original_in_features].to(dtype)
+
+
+def _require_native_geometry(weight: GroupQuantizedWeight, activation_bits: int) -> None:
+    _validate_bits(activation_bits)
+    validate_quantized_weight(weight)
+    if weight.bits != 8 or activation_bits != 8:
+        raise ValueError("the MI355X path implements W8A8 only")
+    if weight.group_size != weight.padded_in_features or weight.padded_in_features != weight.original_in_features:
+        raise ValueError("the MI355X path implements per-token / per-channel scales (group_size == K) only")
+
+
+def quantized_frozen_linear(x: torch.Tensor, weight: GroupQuantizedWeight, *, activation_bits: int = 8):
+    from .rocm import w8a8_lora
+
+    _require_native_geometry(weight, activation_bits)
+    if not x.dtype.is_floating_point:
+        raise TypeError(f"activations must be floating point, got {x.dtype}")
+    return w8a8_lora.w8a8_frozen_linear(x, weight, enabled=True)
+
+
+def quantized_lora_linear(x: torch.Tensor, weight: GroupQuantizedWeight, lora_a: torch.Tensor,
+                          lora_b: torch.Tensor, lora_scaling, *, activation_bits: int = 8) -> torch.Tensor:
+    """Frozen W8A8 linear plus LoRA: bf16(base_f32 + ((x @ A) @ B) * s), one cast."""
+    from .rocm import w8a8_lora
+
+    _require_native_geometry(weight, activation_bits)
+    if x.ndim < 1:
+        raise ValueError(f"activations must have at least one dimension, got {tuple(x.shape)}")
+    if not x.dtype.is_floating_point:
+        raise TypeError(f"activations must be floating point, got {x.dtype}")
+    if lora_a.ndim != 2 or lora_b.ndim != 2:
+        raise ValueError("lora_a and lora_b must both be rank-two")
+    if not lora_a.dtype.is_floating_point or not lora_b.dtype.is_floating_point:
+        raise TypeError(f"LoRA parameters must be floating point, got {lora_a.dtype} and {lora_b.dtype}")
+    if tuple(lora_a.shape) != (weight.original_in_features, lora_b.shape[0]):
+        raise ValueError(
+            f"incompatible LoRA shapes: A={tuple(lora_a.shape)}, B={tuple(lora_b.shape)}, "
+            f"weight K={weight.original_in_features}")
+    if lora_b.shape[1] != weight.codes.shape[-1]:
+        raise ValueError(f"LoRA output N={lora_b.shape[1]} does not match weight N={weight.codes.shape[-1]}")
+    scaling = torch.as_tensor(lora_scaling, dtype=torch.float32)
+    if scaling.ndim != 0:
+        raise ValueError(f"lora_scaling must be scalar, got {tuple(scaling.shape)}")
+    return w8a8_lora.w8a8_lora_linear(x, weight, lora_a, lora_b, scaling, enabled=True)

@@ -1,0 +1,369 @@
+"""W8A8 + LoRA forward entry points on the gfx950 HIP kernels.
+
+Keeps the call surface of the reference's ``skyrl/tx/kernels/rocm/w8a8_lora.py``
+(``w8a8_frozen_linear`` :827-867, ``w8a8_lora_linear`` :870-920): explicit opt-in
+with an exact ``bool``, ``TypeError`` for dtype problems, ``ValueError`` for
+geometry problems, tile keywords accepted (tuning is internal, they are validated
+and otherwise ignored).  Differences, all widenings: per-token / per-channel scales
+(``group_size == K``) instead of group 64, any rank up to 64, float32 or bf16
+scales, and an optional per-row ``adapter_indices`` with stacked adapters
+(``skyrl/tx/layers/lora.py:118-157``).  ``w8a8_rms_gate_up_lora_swiglu`` and
+``w8a8_lora_residual`` are the W8A8 forms of
+``bf16_rms_gate_up_lora_swiglu_contiguous`` (…_contiguous.py:698-712) and
+``bf16_lora_residual`` (bf16_lora_residual.py:507-522).
+
+Tensors are torch CUDA (ROCm) tensors; kernels are enqueued on torch's current
+stream.  There is no CPU or eager fallback.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import math
+import threading
+import weakref
+from dataclasses import dataclass
+
+import torch
+
+from .. import quantized_lora as ql
+from ... import _native
+
+DEFAULT_BLOCK_M = 32
+DEFAULT_BLOCK_N = 64
+DEFAULT_ROW_SUPERBLOCK = 512
+MAX_BLOCK_M = 64
+MAX_BLOCK_N = 128
+MAX_ROW_SUPERBLOCK = 2048
+MAX_IN_FEATURES = 16384
+MAX_OUT_FEATURES = 1 << 20
+MAX_LORA_RANK = 64
+MAX_ADAPTERS = 64
+_SUPPORTED_BLOCK_SIZES = frozenset((16, 32, 64, 128))
+
+
+@dataclass(frozen=True)
+class PackedW8Weight:
+    """A [K, N] int8 weight in MFMA fragment order plus float32 per-channel scales."""
+
+    packed: torch.Tensor   # uint8, mi355_w8a8_packed_weight_bytes(K, N)
+    scales: torch.Tensor   # float32 [N]
+    in_features: int
+    out_features: int
+
+
+def _validate_exact_bool(name: str, value) -> None:
+    if type(value) is not bool:
+        raise TypeError(f"{name} must be an exact bool")
+
+
+def _validate_block_size(name: str, value, maximum: int) -> None:
+    if isinstance(value, bool) or not isinstance(value, int):
+        raise TypeError(f"{name} must be an integer")
+    if value not in _SUPPORTED_BLOCK_SIZES or value > maximum:
+        allowed = sorted(s for s in _SUPPORTED_BLOCK_SIZES if s <= maximum)
+        raise ValueError(f"{name} must be one of {allowed}, got {value}")
+
+
+def _validate_row_superblock(value, block_m: int) -> None:
+    if isinstance(value, bool) or not isinstance(value, int):
+        raise TypeError("row_superblock must be an integer")
+    if not block_m <= value <= MAX_ROW_SUPERBLOCK:
+        raise ValueError(f"row_superblock must be in [{block_m}, {MAX_ROW_SUPERBLOCK}], got {value}")
+    if value % block_m:
+        raise ValueError("row_superblock must be divisible by block_m")
+
+
+def _stream_ptr(device) -> int:
+    return int(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _require_cuda(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on the GPU (there is no CPU path); got device {t.device}")
+
+
+# ---------------------------------------------------------------------------------------
+# weight preparation (one time per weight)
+# ---------------------------------------------------------------------------------------
+_pack_cache: dict = {}
+_pack_lock = threading.Lock()
+
+
+def prepare_weight(weight) -> PackedW8Weight:
+    """Re-layout a per-channel W8 ``GroupQuantizedWeight`` for the kernels (cached).
+
+    This is the load-time permutation; it must not run per forward, so the result
+    is cached on the identity of the codes tensor.
+    """
+    if isinstance(weight, PackedW8Weight):
+        return weight
+    ql.validate_quantized_weight(weight)
+    if weight.bits != 8:
+        raise ValueError(f"the native path requires W8 codes, got W{weight.bits}")
+    if weight.original_in_features != weight.padded_in_features:
+        raise ValueError("the native path does not accept padded K dimensions")
+    if weight.group_size != weight.original_in_features:
+        raise ValueError(
+            f"the native path requires per-channel scales (group size {weight.original_in_features}), "
+            f"got {weight.group_size}")
+    k, n = weight.codes.shape
+    if k % 8:
+        raise ValueError("K must be a positive multiple of 8")
+    if k > MAX_IN_FEATURES:
+        raise ValueError(f"K must not exceed {MAX_IN_FEATURES}")
+    if n > MAX_OUT_FEATURES:
+        raise ValueError(f"N must not exceed {MAX_OUT_FEATURES}")
+    _require_cuda(weight.codes, "weight codes")
+    key = (weight.codes.data_ptr(), weight.scales.data_ptr(), k, n, weight.codes._version, weight.scales._version)
+    with _pack_lock:
+        hit = _pack_cache.get(key)
+        if hit is not None and hit[0]() is weight.codes:
+            return hit[1]
+    lib = _native.load()
+    codes = weight.codes.contiguous()
+    nbytes = int(lib.mi355_w8a8_packed_weight_bytes(k, n))
+    packed = torch.empty(nbytes, dtype=torch.uint8, device=codes.device)
+    with torch.cuda.device(codes.device):
+        _native.check("mi355_w8a8_pack_weight_v1",
+                      lib.mi355_w8a8_pack_weight_v1(codes.data_ptr(), packed.data_ptr(), k, n,
+                                                    _stream_ptr(codes.device)))
+    scales = weight.scales.to(torch.float32).reshape(n).contiguous()
+    out = PackedW8Weight(packed=packed, scales=scales, in_features=k, out_features=n)
+    with _pack_lock:
+        if len(_pack_cache) > 4096:
+            _pack_cache.clear()
+        _pack_cache[key] = (weakref.ref(weight.codes), out)
+    return out
+
+
+def unpack_weight(packed: PackedW8Weight) -> torch.Tensor:
+    """Inverse of the fragment-order packing: int8 [K, N] row-major."""
+    lib = _native.load()
+    out = torch.empty((packed.in_features, packed.out_features), dtype=torch.int8, device=packed.packed.device)
+    with torch.cuda.device(out.device):
+        _native.check("mi355_w8a8_unpack_weight_v1",
+                      lib.mi355_w8a8_unpack_weight_v1(packed.packed.data_ptr(), out.data_ptr(),
+                                                      packed.in_features, packed.out_features,
+                                                      _stream_ptr(out.device)))
+    return out
+
+
+def dynamic_quantize_rows(x: torch.Tensor):
+    """Per-token symmetric int8 quantization: (codes int8 [..., K], scales float32 [...])."""
+    if x.dtype != torch.bfloat16:
+        raise TypeError(f"x must be BF16, got {x.dtype}")
+    if x.ndim < 2 or math.prod(x.shape[:-1]) <= 0:
+        raise ValueError(f"x must have a nonempty row domain and final K axis, got {tuple(x.shape)}")
+    _require_cuda(x, "x")
+    lib = _native.load()
+    flat = x.reshape(-1, x.shape[-1]).contiguous()
+    m, k = flat.shape
+    if k % 8 or k > MAX_IN_FEATURES:
+        raise ValueError(f"K must be a multiple of 8 not exceeding {MAX_IN_FEATURES}, got {k}")
+    codes = torch.empty((m, k), dtype=torch.int8, device=x.device)
+    scales = torch.empty((m,), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        _native.check("mi355_w8a8_quantize_rows_v1",
+                      lib.mi355_w8a8_quantize_rows_v1(flat.data_ptr(), codes.data_ptr(), scales.data_ptr(),
+                                                      m, k, _stream_ptr(x.device)))
+    return codes.reshape(x.shape), scales.reshape(x.shape[:-1])
+
+
+# ---------------------------------------------------------------------------------------
+# the forward call
+# ---------------------------------------------------------------------------------------
+
+def _normalize_lora(lora_a, lora_b, lora_scaling, k: int, n: int, device):
+    """Return stacked (A [n_ad,K,r], B [n_ad,r,N], s [n_ad]) bf16/bf16/f32 tensors."""
+    if lora_a is None and lora_b is None:
+        return None, None, None, 0, 0
+    if lora_a is None or lora_b is None:
+        raise ValueError("lora_a and lora_b must be given together")
+    if lora_a.dtype != torch.bfloat16 or lora_b.dtype != torch.bfloat16:
+        raise TypeError("LoRA A and B must both be BF16")
+    if lora_a.ndim != lora_b.ndim or lora_a.ndim not in (2, 3):
+        raise ValueError("lora_a and lora_b must both be rank-two, or both rank-three (stacked adapters)")
+    a3 = lora_a if lora_a.ndim == 3 else lora_a[None]
+    b3 = lora_b if lora_b.ndim == 3 else lora_b[None]
+    n_ad, ka, r = a3.shape
+    if ka != k or tuple(b3.shape) != (n_ad, r, n):
+        raise ValueError(
+            f"incompatible LoRA shapes: A={tuple(lora_a.shape)}, B={tuple(lora_b.shape)}, weight [K={k}, N={n}]")
+    if r < 1 or r > MAX_LORA_RANK:
+        raise ValueError(f"LoRA rank must be in [1, {MAX_LORA_RANK}], got {r}")
+    if n_ad > MAX_ADAPTERS:
+        raise ValueError(f"at most {MAX_ADAPTERS} adapters are supported, got {n_ad}")
+    s = torch.as_tensor(lora_scaling, dtype=torch.float32, device=device)
+    if s.ndim == 0:
+        s = s.reshape(1).expand(n_ad)
+    if tuple(s.shape) != (n_ad,):
+        raise ValueError(f"lora_scaling must be a scalar or have shape ({n_ad},), got {tuple(s.shape)}")
+    return a3.contiguous(), b3.contiguous(), s.contiguous(), n_ad, r
+
+
+def forward(x: torch.Tensor, weight, lora_a=None, lora_b=None, lora_scaling=None, *,
+            adapter_indices: torch.Tensor | None = None, rms_gamma: torch.Tensor | None = None,
+            eps: float = 1e-6, residual: torch.Tensor | None = None, swiglu: bool = False,
+            flags: int = 0, return_aux: bool = False, entry: str = "forward"):
+    """One W8A8 forward through the C ABI.  Returns bf16 [..., n_out] (and aux tensors)."""
+    if x.dtype != torch.bfloat16:
+        raise TypeError(f"x must be BF16, got {x.dtype}")
+    if x.ndim < 2 or math.prod(x.shape[:-1]) <= 0:
+        raise ValueError(f"x must have a nonempty row domain and final K axis, got {tuple(x.shape)}")
+    _require_cuda(x, "x")
+    pw = prepare_weight(weight)
+    k, n = pw.in_features, pw.out_features
+    if x.shape[-1] != k:
+        raise ValueError(f"x K={x.shape[-1]} does not match W8 K={k}")
+    dev = x.device
+    flat = x.reshape(-1, k).contiguous()
+    m = flat.shape[0]
+    a3, b3, s1, n_ad, r = _normalize_lora(lora_a, lora_b, lora_scaling, k, n, dev)
+    idx = None
+    if adapter_indices is not None:
+        if n_ad == 0:
+            raise ValueError("adapter_indices given without LoRA parameters")
+        idx = adapter_indices.reshape(-1)
+        if idx.shape[0] != m:
+            if idx.shape[0] == 0 or m % idx.shape[0]:
+                raise ValueError(f"adapter_indices of length {idx.shape[0]} do not divide {m} rows")
+            idx = idx.repeat_interleave(m // idx.shape[0])  # one entry per example (lora.py:142)
+        idx = idx.to(device=dev, dtype=torch.int32).contiguous()
+    gamma = None
+    if rms_gamma is not None:
+        if tuple(rms_gamma.shape) != (k,):
+            raise ValueError(f"rms weight must have shape ({k},), got {tuple(rms_gamma.shape)}")
+        gamma = rms_gamma.to(device=dev, dtype=torch.float32).contiguous()
+    if swiglu and n % 2:
+        raise ValueError("SwiGLU needs an even number of fused gate/up columns")
+    n_out = n // 2 if swiglu else n
+    res = None
+    if residual is not None:
+        if residual.dtype != torch.bfloat16:
+            raise TypeError("residual must be BF16")
+        if tuple(residual.shape) != (*x.shape[:-1], n_out):
+            raise ValueError(f"residual must have shape {(*x.shape[:-1], n_out)}, got {tuple(residual.shape)}")
+        res = residual.reshape(m, n_out).contiguous()
+
+    lib = _native.load()
+    if swiglu:
+        flags |= _native.FLAG_SWIGLU
+    out = torch.empty((m, n_out), dtype=torch.bfloat16, device=dev)
+    ws_bytes = int(lib.mi355_w8a8_workspace_bytes(m, k, n, n_ad, r, flags))
+    if ws_bytes == 0:
+        raise ValueError(f"geometry M={m}, K={k}, N={n}, rank={r}, adapters={n_ad} is outside the native path")
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    aux = {}
+    if return_aux:
+        aux["x_codes"] = torch.empty((m, k), dtype=torch.int8, device=dev)
+        aux["x_scales"] = torch.empty((m,), dtype=torch.float32, device=dev)
+        aux["acc"] = torch.empty((m, n), dtype=torch.int32, device=dev)
+        if gamma is not None:
+            aux["normalized"] = torch.empty((m, k), dtype=torch.bfloat16, device=dev)
+
+    p = _native.Problem()
+    p.struct_size = ctypes.sizeof(_native.Problem)
+    p.flags = flags
+    p.m, p.k, p.n, p.n_adapters, p.rank = m, k, n, n_ad, r
+    p.rms_eps = float(eps)
+    p.x = flat.data_ptr()
+    p.w_packed = pw.packed.data_ptr()
+    p.w_scales = pw.scales.data_ptr()
+    p.lora_a = a3.data_ptr() if n_ad else None
+    p.lora_b = b3.data_ptr() if n_ad else None
+    p.lora_scaling = s1.data_ptr() if n_ad else None
+    p.adapter_indices = idx.data_ptr() if idx is not None else None
+    p.rms_gamma = gamma.data_ptr() if gamma is not None else None
+    p.residual = res.data_ptr() if res is not None else None
+    p.out = out.data_ptr()
+    p.workspace = ws.data_ptr()
+    p.workspace_bytes = ws_bytes
+    p.aux_x_codes = aux["x_codes"].data_ptr() if return_aux else None
+    p.aux_x_scales = aux["x_scales"].data_ptr() if return_aux else None
+    p.aux_acc = aux["acc"].data_ptr() if return_aux else None
+    p.aux_normalized = aux["normalized"].data_ptr() if "normalized" in aux else None
+    fn = {"forward": lib.mi355_w8a8_forward_v1, "linear": lib.mi355_w8a8_lora_linear_v1,
+          "gateup": lib.mi355_w8a8_rms_gateup_swiglu_v1, "residual": lib.mi355_w8a8_lora_residual_v1}[entry]
+    with torch.cuda.device(dev):
+        _native.check(f"mi355_w8a8_{entry}", fn(ctypes.byref(p), _stream_ptr(dev)))
+    # ws and the staged copies were allocated for torch's current stream, the one the kernels
+    # were enqueued on, so the caching allocator already orders their reuse after the kernels.
+    result = out.reshape(*x.shape[:-1], n_out)
+    return (result, aux) if return_aux else result
+
+
+def _check_enabled(enabled, interpret, what: str) -> None:
+    _validate_exact_bool("enabled", enabled)
+    _validate_exact_bool("interpret", interpret)
+    if not enabled:
+        raise RuntimeError(f"the W8A8 {what} path is disabled by default")
+    if interpret:
+        raise RuntimeError("interpret=True is not available: the HIP build has no interpreter or CPU path")
+
+
+def _check_tiles(block_m, block_n, row_superblock) -> None:
+    _validate_block_size("block_m", block_m, MAX_BLOCK_M)
+    _validate_block_size("block_n", block_n, MAX_BLOCK_N)
+    _validate_row_superblock(row_superblock, block_m)
+
+
+def w8a8_frozen_linear(x, weight, *, enabled: bool = False, interpret: bool = False,
+                       block_m: int = DEFAULT_BLOCK_M, block_n: int = DEFAULT_BLOCK_N,
+                       row_superblock: int = DEFAULT_ROW_SUPERBLOCK):
+    """Frozen W8A8 base only: bf16(dequant(quant(x) @ Wq))."""
+    _check_enabled(enabled, interpret, "frozen-linear")
+    _check_tiles(block_m, block_n, row_superblock)
+    return forward(x, weight, entry="linear")
+
+
+def w8a8_lora_linear(x, weight, lora_a, lora_b, lora_scaling, *, enabled: bool = False,
+                     interpret: bool = False, block_m: int = DEFAULT_BLOCK_M,
+                     block_n: int = DEFAULT_BLOCK_N, row_superblock: int = DEFAULT_ROW_SUPERBLOCK,
+                     adapter_indices=None):
+    """Frozen W8A8 base + LoRA in one float32 epilogue and one bf16 cast.
+
+    ``lora_a``/``lora_b`` are [K, r]/[r, N] with a scalar ``lora_scaling``, or stacked
+    [n, K, r]/[n, r, N] with ``lora_scaling`` [n] and ``adapter_indices`` selecting
+    an adapter per row (or per example).
+    """
+    _check_enabled(enabled, interpret, "LoRA")
+    _check_tiles(block_m, block_n, row_superblock)
+    if lora_a.ndim == 2:
+        scaling = torch.as_tensor(lora_scaling, dtype=torch.float32)
+        if scaling.ndim != 0:
+            raise TypeError("lora_scaling must be an FP32 scalar")
+    return forward(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices, entry="linear")
+
+
+def w8a8_rms_gate_up_lora_swiglu(x, rms_weight, weight, lora_a, lora_b, lora_scaling, *,
+                                 enabled: bool = False, eps: float = 1e-6, interpret: bool = False,
+                                 rms_is_delta: bool = False, adapter_indices=None):
+    """RMSNorm -> W8A8 gate/up (+LoRA) -> SwiGLU; fused columns are (gate, up) interleaved.
+
+    ``rms_weight`` multiplies the normalized rows (Qwen3); with ``rms_is_delta`` it is
+    the Qwen3.5 delta and the multiplier is ``1 + delta`` evaluated in float32.
+    """
+    _check_enabled(enabled, interpret, "RMSNorm gate/up SwiGLU")
+    _validate_exact_bool("rms_is_delta", rms_is_delta)
+    gamma = rms_weight.to(torch.float32)
+    if rms_is_delta:
+        gamma = 1.0 + gamma
+    return forward(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices,
+                   rms_gamma=gamma, eps=eps, swiglu=True, entry="gateup")
+
+
+def w8a8_lora_residual(x, weight, lora_a, lora_b, lora_scaling, residual, *, enabled: bool = False,
+                       interpret: bool = False, adapter_indices=None):
+    """W8A8 down projection + LoRA + residual, summed in float32 and cast once."""
+    _check_enabled(enabled, interpret, "LoRA residual")
+    return forward(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices,
+                   residual=residual, entry="residual")
+
+
+__all__ = (
+    "DEFAULT_BLOCK_M", "DEFAULT_BLOCK_N", "DEFAULT_ROW_SUPERBLOCK", "MAX_BLOCK_M", "MAX_BLOCK_N",
+    "MAX_IN_FEATURES", "MAX_OUT_FEATURES", "MAX_ROW_SUPERBLOCK", "MAX_LORA_RANK", "PackedW8Weight",
+    "prepare_weight", "unpack_weight", "dynamic_quantize_rows", "forward", "w8a8_frozen_linear",
+    "w8a8_lora_linear", "w8a8_rms_gate_up_lora_swiglu", "w8a8_lora_residual",
+)

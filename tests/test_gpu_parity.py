@@ -1,0 +1,247 @@
+"""GPU parity of the HIP path (through the C ABI) against the CPU oracle.
+
+Bar: int8 activation codes, float32 activation scales and int32 accumulators are
+bit-exact; bf16 outputs satisfy |a - b| <= 2e-2 + 1e-2 * |b| elementwise.
+"""
+
+import hashlib
+
+import numpy as np
+import pytest
+
+from golden import host_case
+from oracle import w8a8_oracle as o
+import w8a8_cases as wc
+
+pytestmark = pytest.mark.gpu
+F32 = np.float32
+ATOL, RTOL = 2e-2, 1e-2
+
+
+@pytest.fixture(scope="module")
+def dev():
+    torch = pytest.importorskip("torch")
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return torch.device("cuda:0")
+
+
+@pytest.fixture(scope="module")
+def pkg():
+    from __graft_entry__ import load_package
+
+    p = load_package()
+    p._native.load()  # fail loudly if the HIP library is missing
+    return p
+
+
+def _assert_integer_stages(aux, st):
+    np.testing.assert_array_equal(aux["x_codes"], st["x_codes"])
+    np.testing.assert_array_equal(aux["x_scales"].view(np.uint32), st["x_scales"].view(np.uint32))
+    np.testing.assert_array_equal(aux["acc"], st["acc"])
+
+
+def _assert_close(got, want, what=""):
+    rep = wc.compare(got, want)
+    print(f"[parity]{what} {rep}", flush=True)
+    assert rep["violations"] == 0, rep
+    assert rep["passed"], rep
+    return rep
+
+
+def test_host_case_bitwise(dev, pkg):
+    """The reference's SHA-256-pinned case through the reference's own call signature."""
+    import torch
+
+    c = host_case.build()
+    ql = pkg.quantized_lora
+    w = ql.GroupQuantizedWeight(torch.from_numpy(c["weight_codes"]).to(dev),
+                                torch.from_numpy(c["weight_scales"]).to(dev).to(torch.bfloat16),
+                                64, 64, 8, 64)
+    bf = lambda a: torch.from_numpy(a).to(dev).to(torch.bfloat16)
+    out = ql.quantized_lora_linear(bf(c["x"]), w, bf(c["lora_a"]), bf(c["lora_b"]), float(c["lora_scaling"]))
+    torch.cuda.synchronize()
+    got = out.to(torch.float32).cpu().numpy()
+    assert got.shape == (3, 32)
+    digest = o.sha256_bf16(np.ascontiguousarray(got[:, :17]))
+    assert digest == host_case.SPEC["sha256"]["expected"]
+    assert np.all(got[:, 17:] == 0)
+
+
+@pytest.mark.parametrize("m,k,student", [(3, 64, False), (128, 1024, False), (33, 4096, False),
+                                         (16, 12288, False), (65, 2560, True), (5, 16384, True), (7, 72, False)])
+def test_quantize_rows_bit_exact(dev, pkg, m, k, student):
+    import torch
+
+    rng = np.random.default_rng(m * 1000 + k)
+    x = rng.standard_t(3, (m, k)) if student else rng.standard_normal((m, k))
+    x = o.bf16_round(x.astype(F32))
+    x[m // 2] = 0.0                      # an all-zero row: scale 1, codes 0
+    if m > 2:
+        x[1, :] = o.bf16_round(F32(1e-30))  # tiny but non-zero row
+    want_c, want_s = o.quantize_rows(x)
+    codes, scales = pkg.w8a8_lora.dynamic_quantize_rows(torch.from_numpy(x).to(dev).to(torch.bfloat16))
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(codes.cpu().numpy(), want_c)
+    np.testing.assert_array_equal(scales.cpu().numpy().view(np.uint32), want_s.view(np.uint32))
+
+
+@pytest.mark.parametrize("k,n", [(64, 17), (128, 256), (1024, 3072), (2560, 520)])
+def test_pack_unpack_roundtrip(dev, pkg, k, n):
+    import torch
+
+    rng = np.random.default_rng(k + n)
+    codes = rng.integers(-128, 128, (k, n), dtype=np.int8)
+    w = pkg.quantized_lora.GroupQuantizedWeight(torch.from_numpy(codes).to(dev),
+                                                torch.ones((1, n), device=dev), k, k, 8, k)
+    packed = pkg.w8a8_lora.prepare_weight(w)
+    assert packed.packed.numel() == ((k + 127) // 128 * 128) * ((n + 255) // 256 * 256)
+    back = pkg.w8a8_lora.unpack_weight(packed)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(back.cpu().numpy(), codes)
+    assert pkg.w8a8_lora.prepare_weight(w) is packed  # cached: the permutation is load-time only
+
+
+def test_config1_single_adapter(dev):
+    """BASELINE config 1: M128 K1024 N3072, one adapter rank 16 alpha 16."""
+    case = wc.make_case(128, 1024, 3072, n_adapters=1, rank=16, seed=1, idx_mode="zero")
+    st = wc.oracle_forward(case, return_stages=True)
+    got, aux = wc.gpu_forward(case)
+    _assert_integer_stages(aux, st)
+    _assert_close(got, st["out"], " cfg1")
+
+
+def test_base_only_no_lora(dev):
+    case = wc.make_case(70, 256, 300, n_adapters=0, seed=2)
+    st = wc.oracle_forward(case, return_stages=True)
+    got, aux = wc.gpu_forward(case)
+    _assert_integer_stages(aux, st)
+    # without LoRA the float32 epilogue has no summation freedom: bit-exact bf16
+    np.testing.assert_array_equal(o.bf16_bits(got), o.bf16_bits(st["out"]))
+
+
+@pytest.mark.parametrize("m,k,n,n_ad,rank", [(512, 512, 1024, 8, 32), (300, 256, 512, 5, 8),
+                                             (1000, 384, 768, 64, 16), (64, 128, 256, 3, 64)])
+def test_multi_adapter_routing(dev, m, k, n, n_ad, rank):
+    case = wc.make_case(m, k, n, n_adapters=n_ad, rank=rank, seed=3 + n_ad)
+    case["s"] = np.linspace(0.25, 2.0, n_ad).astype(F32)
+    st = wc.oracle_forward(case, return_stages=True)
+    got, aux = wc.gpu_forward(case)
+    _assert_integer_stages(aux, st)
+    _assert_close(got, st["out"], f" multi {m}x{k}x{n} a{n_ad} r{rank}")
+
+
+@pytest.mark.parametrize("n", [17, 19, 31, 33])
+@pytest.mark.parametrize("k", [64, 128])
+def test_n_tails_and_row_tail(dev, n, k):
+    """Output tails 17/19/31/33 and M = 33 (tests/tx/kernels/rocm/test_w8a8_lora.py:95-124)."""
+    case = wc.make_case(33, k, n, n_adapters=1, rank=8, seed=n + k, idx_mode="zero")
+    st = wc.oracle_forward(case, return_stages=True)
+    got, aux = wc.gpu_forward(case)
+    _assert_integer_stages(aux, st)
+    _assert_close(got, st["out"], f" tails n{n} k{k}")
+
+
+def test_rms_gate_up_swiglu_reduced(dev):
+    """Config 2 at reduced size: RMSNorm -> gate/up + 8 adapters rank 32 -> SwiGLU."""
+    case = wc.make_case(512, 1024, 2048, n_adapters=8, rank=32, seed=5, rms=True, swiglu=True)
+    st = wc.oracle_forward(case, return_stages=True)
+    got, aux = wc.gpu_forward(case)
+    np.testing.assert_array_equal(o.bf16_bits(aux["normalized"]), o.bf16_bits(st["normalized"]))
+    _assert_integer_stages(aux, st)
+    _assert_close(got, st["out"], " cfg2-reduced")
+    # stage-wise: SwiGLU of the GPU's own pre-activation equals the oracle's SwiGLU to 1 bf16 ulp
+    case2 = dict(case, swiglu=False)
+    fused_gpu, _ = wc.gpu_forward(case2)
+    prod_from_gpu_fused = o.swiglu_from_interleaved(fused_gpu)
+    d = np.abs(o.bf16_bits(got).astype(np.int32) - o.bf16_bits(prod_from_gpu_fused).astype(np.int32))
+    assert d.max() <= 1
+    _assert_close(fused_gpu, st["fused"], " cfg2-reduced pre-activation")
+
+
+def test_swiglu_pairing_closed_form(dev):
+    """gate = even column, up = odd column: every output is 1.9296875 (swapped gives ~2.15)."""
+    k, pairs = 64, 40
+    dense = np.zeros((k, 2 * pairs), F32)
+    dense[:, 0::2] = o.bf16_round(F32(0.02))
+    dense[:, 1::2] = o.bf16_round(F32(0.03))
+    w = o.quantize_frozen_weight(dense, group_size=k, scale_dtype="f32")
+    case = {"m": 9, "k": k, "n": 2 * pairs, "x": np.ones((9, k), F32), "codes": w.codes, "scales": w.scales,
+            "weight": w, "gamma": np.ones(k, F32), "swiglu": True}
+    got, _ = wc.gpu_forward(case)
+    assert np.all(got == F32(1.9296875))
+
+
+def test_down_residual_decode_shape(dev):
+    """Config 3: M16 K12288 N4096, 16 rank-32 adapters (one per row), residual."""
+    case = wc.make_case(16, 12288, 4096, n_adapters=16, rank=32, seed=7, residual=True, idx_mode="arange")
+    st = wc.oracle_forward(case, return_stages=True)
+    got, aux = wc.gpu_forward(case)
+    _assert_integer_stages(aux, st)
+    _assert_close(got, st["out"], " cfg3")
+
+
+@pytest.mark.parametrize("m", [1, 64, 512])
+@pytest.mark.parametrize("k,n", [(2560, 6144), (4096, 2560)])
+def test_config4_student_t(dev, m, k, n):
+    """Config 4: heavy-tailed activations, 4 adapters rank 64 alpha 128 (s = 2)."""
+    case = wc.make_case(m, k, n, n_adapters=4, rank=64, alpha=128, seed=11 + m, student_t=True)
+    st = wc.oracle_forward(case, return_stages=True)
+    got, aux = wc.gpu_forward(case)
+    _assert_integer_stages(aux, st)
+    _assert_close(got, st["out"], f" cfg4 m{m} {k}x{n}")
+
+
+def test_zero_inputs_finite(dev):
+    case = wc.make_case(8, 64, 32, n_adapters=1, rank=8, seed=9, idx_mode="zero")
+    case["x"][:] = 0
+    got, aux = wc.gpu_forward(case)
+    assert np.all(aux["x_codes"] == 0) and np.all(aux["x_scales"] == 1.0)
+    assert np.all(got == 0) and np.all(np.isfinite(got))
+
+
+def test_run_to_run_determinism(dev):
+    case = wc.make_case(300, 512, 768, n_adapters=4, rank=16, seed=13, rms=True, swiglu=True)
+    a = wc.gpu_forward(case, return_aux=False)
+    b = wc.gpu_forward(case, return_aux=False)
+    assert hashlib.sha256(a.tobytes()).hexdigest() == hashlib.sha256(b.tobytes()).hexdigest()
+
+
+def test_split2_flag_stays_in_tolerance(dev, pkg):
+    case = wc.make_case(256, 512, 512, n_adapters=2, rank=32, seed=15)
+    want = wc.oracle_forward(case)
+    got = wc.gpu_forward(case, flags=pkg._native.FLAG_LORA_SPLIT2, return_aux=False)
+    _assert_close(got, want, " split2")
+
+
+def test_reference_call_surface(dev, pkg):
+    """Opt-in and error conventions of skyrl/tx/kernels/rocm/w8a8_lora.py:57-59,844-849."""
+    import torch
+
+    w8 = pkg.w8a8_lora
+    case = wc.make_case(4, 64, 32, n_adapters=1, rank=8, seed=17, idx_mode="zero")
+    t = wc.to_torch(case, dev)
+    with pytest.raises(RuntimeError, match="disabled by default"):
+        w8.w8a8_lora_linear(t["x"], t["weight"], t["a"][0], t["b"][0], 1.0)
+    with pytest.raises(TypeError, match="exact bool"):
+        w8.w8a8_lora_linear(t["x"], t["weight"], t["a"][0], t["b"][0], 1.0, enabled=1)
+    with pytest.raises(TypeError, match="BF16"):
+        w8.w8a8_lora_linear(t["x"].float(), t["weight"], t["a"][0], t["b"][0], 1.0, enabled=True)
+    with pytest.raises(ValueError):
+        w8.w8a8_lora_linear(t["x"][:, :32], t["weight"], t["a"][0], t["b"][0], 1.0, enabled=True)
+    with pytest.raises(ValueError):
+        w8.w8a8_lora_linear(t["x"], t["weight"], t["a"][0][:, :4], t["b"][0], 1.0, enabled=True)
+    with pytest.raises(ValueError):
+        w8.w8a8_lora_linear(t["x"], t["weight"], t["a"][0], t["b"][0], 1.0, enabled=True, block_m=48)
+    out = w8.w8a8_lora_linear(t["x"], t["weight"], t["a"][0], t["b"][0], 1.0, enabled=True)
+    base = w8.w8a8_frozen_linear(t["x"], t["weight"], enabled=True)
+    torch.cuda.synchronize()
+    assert out.shape == (4, 32) and out.dtype == torch.bfloat16 and base.shape == (4, 32)
+    want = o.quantized_lora_linear(case["x"], case["weight"], case["a"][0], case["b"][0], F32(1.0))
+    assert o.within_tolerance(out.float().cpu().numpy(), want).all()
+    # leading batch dimensions are flattened and restored
+    x3 = t["x"].reshape(2, 2, 64)
+    out3 = w8.w8a8_lora_linear(x3, t["weight"], t["a"][0], t["b"][0], 1.0, enabled=True)
+    torch.cuda.synchronize()
+    assert out3.shape == (2, 2, 32)
+    assert torch.equal(out3.reshape(4, 32), out)
