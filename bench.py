@@ -1,0 +1,219 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X W8A8 LoRA linear forward path.
+
+One step = one pass of the hot path over one batch of synthetic input.  The
+default workload is the Qwen3-8B gate/up projection at M = 4096 (RMSNorm ->
+W8A8 [4096 x 4096] x [4096 x 24576] + 8 rank-32 adapters routed per row ->
+SwiGLU).  Inputs are resident in HBM before the timed region.  Prints ONE JSON
+line; ``value`` is int8 TOPS of the whole step (2*M*K*N per step, every kernel of
+the step included); ``roofline`` prices the dominant kernel (the int8 MFMA GEMM)
+from HIP events around that kernel alone; ``cpu_baseline`` times the NumPy oracle
+on a bounded row sample of the same workload on the host cores.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+sys.path.insert(0, str(ROOT / "tests"))
+
+INT8_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA, published (5.0 POP/s)
+HBM_PEAK_GBS = 8000.0     # MI355X HBM3E, published
+
+WORKLOADS = {
+    # name: (m, k, n, adapters, rank, alpha, rms, swiglu, residual, idx_mode, seed)
+    "qwen3-8b-gate_up-m4096": dict(m=4096, k=4096, n=24576, n_adapters=8, rank=32, rms=True, swiglu=True,
+                                   idx_mode="uniform", seed=2),
+    "qwen3-8b-down-m16-decode": dict(m=16, k=12288, n=4096, n_adapters=16, rank=32, residual=True,
+                                     idx_mode="arange", seed=3),
+    "single-linear-m128": dict(m=128, k=1024, n=3072, n_adapters=1, rank=16, idx_mode="zero", seed=1),
+}
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# (see profiles/); None until measured for the workload.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def algorithmic_bytes(c):
+    m, k, n = c["m"], c["k"], c["n"]
+    n_out = n // 2 if c.get("swiglu") else n
+    total = 2 * m * k + k * n + 4 * n + 2 * m * n_out + 4 * m
+    if c.get("n_adapters"):
+        used = min(c["n_adapters"], m)
+        total += 2 * used * c["rank"] * (k + n)
+    if c.get("rms"):
+        total += 4 * k
+    if c.get("residual"):
+        total += 2 * m * n_out
+    return total
+
+
+def gemm_kernel_bytes(c):
+    """Algorithmic bytes of the GEMM kernel alone: int8 codes in, weights, LoRA B, output."""
+    m, k, n = c["m"], c["k"], c["n"]
+    n_out = n // 2 if c.get("swiglu") else n
+    total = m * k + k * n + 4 * n + 4 * m + 2 * m * n_out
+    if c.get("n_adapters"):
+        used = min(c["n_adapters"], m)
+        total += 2 * used * c["rank"] * n + 4 * m * c["rank"]
+    if c.get("residual"):
+        total += 2 * m * n_out
+    return total
+
+
+def cpu_baseline(case, cfg, sample_rows):
+    """Time the NumPy oracle on the first ``sample_rows`` rows of the workload."""
+    import w8a8_cases as wc
+
+    sub = dict(case)
+    sub["m"] = sample_rows
+    sub["x"] = case["x"][:sample_rows]
+    if "idx" in case:
+        sub["idx"] = case["idx"][:sample_rows]
+    if "residual" in case:
+        sub["residual"] = case["residual"][:sample_rows]
+    wc.oracle_forward(sub)  # warm-up (BLAS thread pool, page faults)
+    best = float("inf")
+    out = None
+    for _ in range(2):
+        t0 = time.perf_counter()
+        out = wc.oracle_forward(sub)
+        best = min(best, time.perf_counter() - t0)
+    ops = 2.0 * sample_rows * cfg["k"] * cfg["n"]
+    try:
+        cores = len(os.sched_getaffinity(0))
+    except AttributeError:
+        cores = os.cpu_count() or 1
+    threads = int(os.environ.get("OMP_NUM_THREADS", cores))
+    return out, {"value": ops / best / 1e12, "unit": "TOPS", "cores": min(cores, threads), "kind": "port",
+                 "sample": f"first {sample_rows} of {cfg['m']} rows, full K and N, NumPy oracle "
+                           f"(float64 BLAS for the exact integer GEMM), best of 2, {best:.3f} s",
+                 "seconds": best}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="qwen3-8b-gate_up-m4096", choices=sorted(WORKLOADS))
+    ap.add_argument("--cpu-rows", type=int, default=None, help="rows of the CPU-baseline sample")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--flags", type=int, default=0, help="extra mi355_w8a8_problem.flags")
+    ap.add_argument("--override", default="", help="comma list key=int overriding workload fields (m,k,n,...)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path has no collectives); use --gpus 1",
+              file=sys.stderr)
+        return 2
+
+    import torch
+
+    import w8a8_cases as wc
+    from __graft_entry__ import load_package
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 3
+    pkg = load_package()
+    native = pkg._native
+    native.load()
+    w8 = pkg.w8a8_lora
+    dev = torch.device("cuda:0")
+    cfg = dict(WORKLOADS[args.workload])
+    for item in filter(None, args.override.split(",")):
+        key, val = item.split("=")
+        cfg[key] = int(val)
+    case = wc.make_case(cfg["m"], cfg["k"], cfg["n"], n_adapters=cfg.get("n_adapters", 0),
+                        rank=cfg.get("rank", 16), seed=cfg["seed"], rms=cfg.get("rms", False),
+                        residual=cfg.get("residual", False), swiglu=cfg.get("swiglu", False),
+                        idx_mode=cfg.get("idx_mode", "uniform"))
+    t = wc.to_torch(case, dev)
+    plan = w8.ForwardPlan(t["x"], t["weight"], t.get("a"), t.get("b"), t.get("s"),
+                          adapter_indices=t.get("idx"), rms_gamma=t.get("gamma"), eps=1e-6,
+                          residual=t.get("residual"), swiglu=bool(cfg.get("swiglu")), flags=args.flags)
+    torch.cuda.synchronize()
+
+    for _ in range(args.warmup):
+        plan.run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        plan.run()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    ops = 2.0 * cfg["m"] * cfg["k"] * cfg["n"]
+    tops = ops / (ms_per_step * 1e-3) / 1e12
+
+    # dominant kernel alone: HIP events (torch's current stream is the launch stream) around
+    # GEMM-only launches; the workspace still holds the prologue's results.
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+          for _ in range(args.steps)]
+    for a, b in ev:
+        a.record()
+        plan.run(native.FLAG_SKIP_PROLOGUE)
+        b.record()
+    torch.cuda.synchronize()
+    gemm_ms = np.asarray([a.elapsed_time(b) for a, b in ev])
+    gemm_avg_ms = float(gemm_ms.mean())
+    # prologue alone (routing + quantization + LoRA-A)
+    pa, pb = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    pa.record()
+    for _ in range(args.steps):
+        plan.run(native.FLAG_SKIP_GEMM)
+    pb.record()
+    torch.cuda.synchronize()
+    prologue_ms = pa.elapsed_time(pb) / args.steps
+    out_gpu = plan.run()
+    torch.cuda.synchronize()
+
+    skinny = cfg["m"] <= 32
+    if skinny:
+        bytes_alg = algorithmic_bytes(cfg)
+        achieved = bytes_alg / (gemm_avg_ms * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                    "kernel": "skinny", "kernel_avg_ms": gemm_avg_ms, "algorithmic_bytes": bytes_alg}
+    else:
+        achieved = ops / (gemm_avg_ms * 1e-3) / 1e12
+        roofline = {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                    "frac": achieved / INT8_PEAK_TOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                    "kernel": "w8a8_gemm_kernel", "kernel_avg_ms": gemm_avg_ms,
+                    "kernel_min_ms": float(gemm_ms.min()), "algorithmic_ops": ops,
+                    "algorithmic_bytes": gemm_kernel_bytes(cfg)}
+
+    result = {
+        "metric": "W8A8-LoRA GEMM TOPS & % int8 MFMA peak (Qwen3-8B MLP, M=4096); decode GB/s",
+        "value": tops, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8", "data": "synthetic",
+        "config": {"workload": args.workload, **{k: v for k, v in cfg.items() if k != "seed"}},
+        "frac_of_int8_peak_whole_step": tops / INT8_PEAK_TOPS,
+        "whole_step_gbs": algorithmic_bytes(cfg) / (ms_per_step * 1e-3) / 1e9,
+        "prologue_ms": prologue_ms,
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        rows = args.cpu_rows or min(cfg["m"], 256)
+        want, base = cpu_baseline(case, cfg, rows)
+        result["cpu_baseline"] = base
+        got = out_gpu[:rows].to(torch.float32).cpu().numpy()
+        rep = wc.compare(got, want)
+        result["parity_sample"] = {"rows": rows, "violations": rep["violations"], "size": rep["size"],
+                                   "max_abs": rep["max_abs"], "bitwise_fraction": rep["bitwise_fraction"]}
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -55,6 +55,10 @@ typedef enum mi355_w8a8_status {
 #define MI355_W8A8_FLAG_FORCE_TILED 2u /* never take the skinny-M (split-K) kernel */
 #define MI355_W8A8_FLAG_FORCE_SKINNY 4u/* always take the skinny-M kernel (M <= 32) */
 #define MI355_W8A8_FLAG_LORA_SPLIT2 8u /* carry x@A as 2 bf16 terms instead of 3 in the LoRA-B product */
+/* Stage selection for measurement: the workspace keeps the prologue's results between calls, so a
+ * call with SKIP_PROLOGUE after a full call with the same arguments re-runs only the GEMM kernel. */
+#define MI355_W8A8_FLAG_SKIP_PROLOGUE 16u /* do not run routing / quantization / LoRA-A */
+#define MI355_W8A8_FLAG_SKIP_GEMM 32u     /* run only routing / quantization / LoRA-A */
 
 /*
  * One forward call.  y = dequant(quant(n) @ W) + s[idx] * ((n @ A[idx]) @ B[idx]) (+ residual),

@@ -17,6 +17,8 @@ FLAG_SWIGLU = 1
 FLAG_FORCE_TILED = 2
 FLAG_FORCE_SKINNY = 4
 FLAG_LORA_SPLIT2 = 8
+FLAG_SKIP_PROLOGUE = 16
+FLAG_SKIP_GEMM = 32
 
 STATUS = {
     0: "OK", -1: "ERR_NULL", -2: "ERR_SHAPE", -3: "ERR_ALIGN", -4: "ERR_ALIAS",

@@ -3,6 +3,7 @@
 #include "../../include/mi355_w8a8.h"
 
 #include <hip/hip_runtime.h>
+#include <stdlib.h>
 
 #include "w8a8_device.h"
 #include "w8a8_gemm.h"
@@ -16,39 +17,36 @@ namespace {
 constexpr uint32_t kMaxK = 16384;
 constexpr uint32_t kMaxRows = 1u << 20;
 constexpr uint32_t kMaxN = 1u << 20;
-constexpr uint32_t kGemmLdsBytes = 131072;
 
 inline uint64_t align256(uint64_t v) { return (v + 255u) & ~uint64_t(255); }
 
 struct WsLayout {
-  uint64_t xq, sx, xn, z, src_row, dst_pos, blk_group, meta, skinny, total;
-  uint32_t slots, ksplit, r_pad, K_pad, KB, n_steps, steps_per_wave;
+  uint64_t xq, sx, xn, zp, at, src_row, dst_pos, slot_group, blk_range, skinny, total;
+  uint32_t slots, nkk, K_pad, KB, n_steps, steps_per_wave;
 };
+
+// number of 16-wide rank chunks the kernels are instantiated for (rank padded with zeros)
+inline uint32_t rank_chunks(uint32_t rank) { return rank == 0 ? 0u : (rank <= 16u ? 1u : (rank <= 32u ? 2u : 4u)); }
 
 WsLayout make_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint32_t rank, bool routed) {
   WsLayout w{};
   w.K_pad = k_padded(k);
   w.KB = w.K_pad / 32u;
-  w.slots = routed ? round_up(m + 32u * n_groups, kTileM) : round_up(m, kTileM);
-  w.r_pad = rank ? round_up(rank, 16u) : 0u;
+  w.slots = round_up(m, kTileM);
+  (void)routed;
+  w.nkk = rank_chunks(rank);
   w.n_steps = (k + 63u) / 64u;
-  const uint32_t n_pblk = w.slots / 32u;
-  uint32_t ks = 512u / n_pblk;
-  if (ks < 1u) ks = 1u;
-  if (ks > (uint32_t)kMaxKSplit) ks = kMaxKSplit;
-  const uint32_t by_steps = w.n_steps / 4u ? w.n_steps / 4u : 1u;
-  if (ks > by_steps) ks = by_steps;
-  w.ksplit = ks;
-  w.steps_per_wave = (w.n_steps + ks * 4u - 1u) / (ks * 4u);
+  w.steps_per_wave = (w.n_steps + 7u) / 8u;
   uint64_t off = 0;
-  w.meta = off; off += 256;
   w.xq = off; off += align256((uint64_t)w.slots * w.K_pad);
   w.sx = off; off += align256((uint64_t)w.slots * 4u);
   w.src_row = off; off += align256((uint64_t)w.slots * 4u);
   w.dst_pos = off; off += align256((uint64_t)m * 4u);
-  w.blk_group = off; off += align256((uint64_t)(w.slots / 32u) * 4u + 2u * (n_groups + 1u) * 4u);
+  w.slot_group = off; off += align256((uint64_t)w.slots * 4u);
+  w.blk_range = off; off += align256((uint64_t)(w.slots / 32u) * 4u);
   w.xn = off; off += rank ? align256((uint64_t)m * k * 2u) : 0u;
-  w.z = off; off += rank ? align256((uint64_t)kMaxKSplit * w.slots * w.r_pad * 4u) : 0u;
+  w.zp = off; off += rank ? align256((uint64_t)(w.slots / 32u) * w.nkk * 3u * kBlockBytes) : 0u;
+  w.at = off; off += rank ? align256((uint64_t)n_groups * rank * k * 2u) : 0u;
   w.skinny = off; off += align256(skinny_workspace_bytes(m, n));
   w.total = off;
   return w;
@@ -77,11 +75,47 @@ int launch_quant(const QuantArgs& a, hipStream_t s) {
   return MI355_W8A8_ERR_UNSUPPORTED;
 }
 
+template <int EPI, int NKK>
+int launch_gemm_one(const GemmArgs& g, hipStream_t s) {
+  const uint32_t ntile = g.tiles_m * g.tiles_n;
+  const dim3 grid(((ntile + 7u) / 8u) * 8u), block(256);
+#ifdef W8A8_DEBUG_VARIANTS
+  if constexpr (EPI == kEpiSwiglu && NKK == 2) {
+#define W8A8_DBG(D)                                                                              \
+  if (g.map_mode == 100 + D) {                                                                   \
+    hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm_kernel<EPI, NKK, D>),          \
+                        hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes);              \
+    hipLaunchKernelGGL((w8a8_gemm_kernel<EPI, NKK, D>), grid, block, kGemmLdsBytes, s, g);       \
+    return launch_status();                                                                      \
+  }
+    W8A8_DBG(1) W8A8_DBG(2) W8A8_DBG(3) W8A8_DBG(4)
+#undef W8A8_DBG
+  }
+#endif
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm_kernel<EPI, NKK>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes) != hipSuccess)
+    return MI355_W8A8_ERR_LAUNCH;
+  hipLaunchKernelGGL((w8a8_gemm_kernel<EPI, NKK>), grid, block, kGemmLdsBytes, s, g);
+  return launch_status();
+}
+
+template <int EPI>
+int launch_gemm(const GemmArgs& g, uint32_t nkk, hipStream_t s) {
+  switch (nkk) {
+    case 0: return launch_gemm_one<EPI, 0>(g, s);
+    case 1: return launch_gemm_one<EPI, 1>(g, s);
+    case 2: return launch_gemm_one<EPI, 2>(g, s);
+    case 4: return launch_gemm_one<EPI, 4>(g, s);
+    default: return MI355_W8A8_ERR_UNSUPPORTED;
+  }
+}
+
 int validate_common(uint32_t m, uint32_t k, uint32_t n) {
   if (m == 0 || k == 0 || n == 0) return MI355_W8A8_ERR_SHAPE;
   if (m > kMaxRows || n > kMaxN) return MI355_W8A8_ERR_UNSUPPORTED;
   if (k % 8u) return MI355_W8A8_ERR_UNSUPPORTED;
   if (k_padded(k) > kMaxK) return MI355_W8A8_ERR_UNSUPPORTED;
+  if ((uint64_t)m * n >= (1ull << 32) - (1ull << 20)) return MI355_W8A8_ERR_UNSUPPORTED;  // 32-bit offsets
   return MI355_W8A8_OK;
 }
 
@@ -100,6 +134,7 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   if (req == kReqGateUp && (!swiglu || !rms)) return MI355_W8A8_ERR_SHAPE;
   if (req == kReqResidual && (!p->residual || swiglu)) return MI355_W8A8_ERR_SHAPE;
   if (swiglu && (p->n & 1u)) return MI355_W8A8_ERR_SHAPE;
+  if (swiglu && p->residual) return MI355_W8A8_ERR_UNSUPPORTED;
   if ((p->flags & MI355_W8A8_FLAG_FORCE_TILED) && (p->flags & MI355_W8A8_FLAG_FORCE_SKINNY))
     return MI355_W8A8_ERR_SHAPE;
   if (lora) {
@@ -132,10 +167,10 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   if (reinterpret_cast<uintptr_t>(p->workspace) & 255u) return MI355_W8A8_ERR_ALIGN;
   const WsLayout w = make_layout(p->m, p->k, p->n, p->n_adapters, lora ? p->rank : 0u, routed);
   unsigned char* ws = static_cast<unsigned char*>(p->workspace);
-  int32_t* meta = reinterpret_cast<int32_t*>(ws + w.meta);
   int32_t* src_row = reinterpret_cast<int32_t*>(ws + w.src_row);
   int32_t* dst_pos = reinterpret_cast<int32_t*>(ws + w.dst_pos);
-  int32_t* blk_group = reinterpret_cast<int32_t*>(ws + w.blk_group);
+  int32_t* slot_group = reinterpret_cast<int32_t*>(ws + w.slot_group);
+  int32_t* blk_range = reinterpret_cast<int32_t*>(ws + w.blk_range);
 
   (void)hipGetLastError();  // drop a stale error so it is not blamed on these launches
 
@@ -151,9 +186,11 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
                          reinterpret_cast<uint16_t*>(ws + w.xn), ws + w.skinny, w.K_pad, w.KB, s);
   }
 
-  if (routed) {
+  const bool skip_prologue = (p->flags & MI355_W8A8_FLAG_SKIP_PROLOGUE) != 0;
+  const bool skip_gemm = (p->flags & MI355_W8A8_FLAG_SKIP_GEMM) != 0;
+  if (routed && !skip_prologue) {
     hipLaunchKernelGGL(route_rows_kernel, dim3(1), dim3(1024), 0, s, p->adapter_indices, p->m,
-                       p->n_adapters, w.slots, meta, src_row, dst_pos, blk_group);
+                       p->n_adapters, w.slots, src_row, dst_pos, slot_group, blk_range);
     if ((st = launch_status())) return st;
   }
 
@@ -169,73 +206,59 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   q.scales_rm = p->aux_x_scales;
   q.xn = (rms && lora) ? reinterpret_cast<uint16_t*>(ws + w.xn) : nullptr;
   q.xn_aux = static_cast<uint16_t*>(p->aux_normalized);
-  st = rms ? launch_quant<true>(q, s) : launch_quant<false>(q, s);
-  if (st) return st;
+  if (!skip_prologue) {
+    st = rms ? launch_quant<true>(q, s) : launch_quant<false>(q, s);
+    if (st) return st;
+  }
 
-  if (lora) {
+  if (lora && !skip_prologue) {
+    uint16_t* at = reinterpret_cast<uint16_t*>(ws + w.at);
+    const uint64_t chunks = (uint64_t)p->n_adapters * p->k * ((p->rank + 7u) / 8u);
+    hipLaunchKernelGGL(lora_a_transpose_kernel, dim3((uint32_t)((chunks + 255u) / 256u)), dim3(256), 0, s,
+                       static_cast<const uint16_t*>(p->lora_a), at, p->n_adapters, p->k, p->rank);
+    if ((st = launch_status())) return st;
     LoraAArgs la{};
     la.xsrc = rms ? reinterpret_cast<const uint16_t*>(ws + w.xn) : static_cast<const uint16_t*>(p->x);
-    la.lora_a = static_cast<const uint16_t*>(p->lora_a);
+    la.at = at;
     la.src_row = routed ? src_row : nullptr;
-    la.blk_group = routed ? blk_group : nullptr;
-    la.meta = routed ? meta : nullptr;
-    la.z_part = reinterpret_cast<float*>(ws + w.z);
-    la.M = p->m; la.K = p->k; la.r = p->rank; la.r_pad = w.r_pad; la.slots = w.slots;
-    la.rows_static = round_up(p->m, 32u);
+    la.slot_group = routed ? slot_group : nullptr;
+    la.blk_range = routed ? blk_range : nullptr;
+    la.zp = ws + w.zp;
+    la.M = p->m; la.K = p->k; la.r = p->rank; la.nkk = w.nkk;
     la.steps_per_wave = w.steps_per_wave; la.n_steps = w.n_steps;
-    const dim3 grid(w.slots / 32u, w.ksplit), block(256);
-    if (w.r_pad > 32u) hipLaunchKernelGGL((lora_a_kernel<2>), grid, block, 0, s, la);
+    const dim3 grid(w.slots / 32u), block(512);
+    if (w.nkk > 2u) hipLaunchKernelGGL((lora_a_kernel<2>), grid, block, 0, s, la);
     else hipLaunchKernelGGL((lora_a_kernel<1>), grid, block, 0, s, la);
     if ((st = launch_status())) return st;
   }
 
+  if (skip_gemm) return MI355_W8A8_OK;
   GemmArgs g{};
   g.xq = ws + w.xq;
   g.wp = static_cast<const unsigned char*>(p->w_packed);
   g.sx = reinterpret_cast<const float*>(ws + w.sx);
   g.sw = p->w_scales;
-  g.z_part = lora ? reinterpret_cast<const float*>(ws + w.z) : nullptr;
+  g.zp = lora ? ws + w.zp : nullptr;
   g.lora_b = static_cast<const uint16_t*>(p->lora_b);
   g.lora_scaling = p->lora_scaling;
   g.src_row = routed ? src_row : nullptr;
-  g.blk_group = routed ? blk_group : nullptr;
-  g.meta = routed ? meta : nullptr;
+  g.slot_group = routed ? slot_group : nullptr;
+  g.blk_range = routed ? blk_range : nullptr;
   g.residual = static_cast<const uint16_t*>(p->residual);
   g.out = p->out;
-  g.w_group_stride = 0;
   g.M = p->m; g.N = p->n; g.K_pad = w.K_pad; g.KB = w.KB; g.slots = w.slots;
-  g.rows_static = round_up(p->m, 32u);
   g.tiles_m = w.slots / kTileM;
-  g.tiles_n = n_padded(p->n) / kTileN;
+  g.tiles_n = n_padded(p->n) / kGemmTileN;
   g.rank = lora ? p->rank : 0u;
-  g.r_pad = w.r_pad;
-  g.ksplit = w.ksplit;
   g.nsplit_terms = (p->flags & MI355_W8A8_FLAG_LORA_SPLIT2) ? 2u : 3u;
-  g.grouped = 0;
-  const uint32_t ntile = g.tiles_m * g.tiles_n;
-  const dim3 grid(((ntile + 7u) / 8u) * 8u), block(256);
+  { const char* e = getenv("MI355_W8A8_TILE_MAP"); g.map_mode = e ? (uint32_t)atoi(e) : 0u; }
   if (p->aux_acc) {
     GemmArgs ga = g;
     ga.out = p->aux_acc;
     ga.residual = nullptr;
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm_kernel<kEpiAcc>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes) != hipSuccess)
-      return MI355_W8A8_ERR_LAUNCH;
-    hipLaunchKernelGGL((w8a8_gemm_kernel<kEpiAcc>), grid, block, kGemmLdsBytes, s, ga);
-    if ((st = launch_status())) return st;
+    if ((st = launch_gemm<kEpiAcc>(ga, 0u, s))) return st;
   }
-  if (swiglu) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm_kernel<kEpiSwiglu>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes) != hipSuccess)
-      return MI355_W8A8_ERR_LAUNCH;
-    hipLaunchKernelGGL((w8a8_gemm_kernel<kEpiSwiglu>), grid, block, kGemmLdsBytes, s, g);
-  } else {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm_kernel<kEpiPlain>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes) != hipSuccess)
-      return MI355_W8A8_ERR_LAUNCH;
-    hipLaunchKernelGGL((w8a8_gemm_kernel<kEpiPlain>), grid, block, kGemmLdsBytes, s, g);
-  }
-  return launch_status();
+  return swiglu ? launch_gemm<kEpiSwiglu>(g, w.nkk, s) : launch_gemm<kEpiPlain>(g, w.nkk, s);
 }
 
 }  // namespace

@@ -8,9 +8,9 @@
 // which is exactly one v_mfma_i32_32x32x32_i8 A or B operand, so a wave fetches an
 // operand with a single 16-byte-per-lane load of a contiguous 1 KiB chunk.  Blocks are
 // ordered [row_block][k_block].  Weight columns are additionally permuted inside every
-// group of 64: packed column 64g + 32h + j holds original column 64g + 2j + h, so the
-// (even, odd) = (gate, up) neighbours of a fused gate/up projection land in the same
-// lane of two adjacent blocks.
+// group of 128: packed column 128g + 32j + c holds original column 128g + 4c + j, so a lane
+// of the MFMA output owns four consecutive original columns (two (gate, up) pairs of a fused
+// gate/up projection) in the four adjacent 32-column blocks of its wave.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -39,7 +39,11 @@ __host__ __device__ inline uint32_t n_padded(uint32_t n) { return round_up(n, kT
 
 // original weight column of packed column c
 __host__ __device__ inline uint32_t packed_to_orig_col(uint32_t c) {
-  return (c & ~63u) + 2u * (c & 31u) + ((c >> 5) & 1u);
+  return (c & ~127u) + 4u * (c & 31u) + ((c >> 5) & 3u);
+}
+// packed column of original column n (inverse of the above)
+__host__ __device__ inline uint32_t orig_to_packed_col(uint32_t n) {
+  return (n & ~127u) + 32u * (n & 3u) + ((n & 127u) >> 2);
 }
 // byte offset of element (row r, k) of a packed operand with kb k-blocks per row block
 __host__ __device__ inline size_t packed_offset(uint32_t r, uint32_t k, uint32_t kb) {
@@ -68,8 +72,19 @@ __device__ inline double wave_sum(double v) {
   return v;
 }
 
-// s_waitcnt vmcnt(0) only (gfx9 encoding: vmcnt[3:0]|[15:14], expcnt[6:4], lgkmcnt[11:8])
-__device__ inline void wait_vmcnt0() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+// s_waitcnt vmcnt(N) only (gfx9 encoding: vmcnt[3:0]|[15:14], expcnt[6:4], lgkmcnt[11:8])
+template <int N>
+__device__ inline void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
+__device__ inline void wait_vmcnt0() { wait_vmcnt<0>(); }
+
+// Workgroup barrier for LDS hand-over that does not wait for outstanding global loads: the
+// caller decides with wait_vmcnt<N>() how many direct-to-LDS loads may stay in flight.  The
+// wave first drains its own LDS operations, so data it read is in registers and data it wrote
+// is visible once every wave has passed.
+__device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;

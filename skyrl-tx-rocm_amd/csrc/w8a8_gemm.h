@@ -2,10 +2,13 @@
 //   acc[p, n]  = sum_k xq[p, k] * wq[k, n]                         (v_mfma_i32_32x32x32_i8, exact)
 //   base       = (float(acc) * sx[p]) * sw[n]                      (skyrl/tx/kernels/quantized_lora.py:248-252)
 //   y          = base + low * s[group(p)] (+ residual)             (quantized_lora.py:300-304)
-//   low        = z[p, :] @ B[group(p)]                             (bf16 MFMA, z carried as 2-3 bf16 terms)
+//   low        = z[p, :] @ B[group(p)]                             (bf16 MFMA, z carried as 3 (or 2) bf16 terms)
 //   out        = bf16(y)   or   bf16(silu(bf16(y_gate)) * bf16(y_up))
-// Workgroup = 256 threads = 4 waves, tile 256 x 256, K step 128, two LDS stages of 64 KiB
-// filled by 16-byte direct-to-LDS loads of contiguous 1 KiB fragment blocks.
+// Workgroup = 256 threads = 4 waves stacked along M (64 x 128 each), tile 256 x 128, 128
+// accumulator registers per lane and 72 KiB of LDS, so two workgroups share a CU: while one is
+// in its VALU/store epilogue the other keeps the MFMA pipe busy.  K is consumed in steps of 64
+// through a ring of three 24 KiB LDS stages filled by 16-byte direct-to-LDS loads of contiguous
+// 1 KiB fragment blocks, two tiles ahead of the MFMAs.
 #pragma once
 #include <type_traits>
 
@@ -17,36 +20,55 @@ enum { kEpiPlain = 0, kEpiSwiglu = 1, kEpiAcc = 2 };
 
 struct GemmArgs {
   const unsigned char* xq;   // packed activation codes [slots, K_pad]
-  const unsigned char* wp;   // packed weight [N_pad, K_pad] (per group: + group * w_group_stride)
+  const unsigned char* wp;   // packed weight [N_pad, K_pad]
   const float* sx;           // f32 [slots]
-  const float* sw;           // f32 [N] (per group: + group * N)
-  const float* z_part;       // f32 [ksplit, slots, r_pad] or null
+  const float* sw;           // f32 [N]
+  const unsigned char* zp;   // packed z fragments [slots/32][NKK][3][64 lanes][8 bf16] or null
   const uint16_t* lora_b;    // bf16 [n_groups, rank, N] or null
   const float* lora_scaling; // f32 [n_groups]
-  const int32_t* src_row;    // or null
-  const int32_t* blk_group;  // or null
-  const int32_t* meta;       // or null
+  const int32_t* src_row;    // original row of every grouped slot, or null (identity)
+  const int32_t* slot_group; // LoRA group (adapter) of every grouped slot, or null (group 0)
+  const int32_t* blk_range;  // per 32-row block: first group | last group << 16, or null
   const uint16_t* residual;  // bf16 [M, n_out] or null
   void* out;                 // bf16 [M, n_out] or int32 [M, N]
-  uint64_t w_group_stride;   // bytes between per-group packed weights (0 = shared weight)
-  uint32_t M, N, K_pad, KB, slots, rows_static;
-  uint32_t tiles_m, tiles_n, rank, r_pad, ksplit, nsplit_terms, grouped;
+  uint32_t M, N, K_pad, KB, slots;
+  uint32_t tiles_m, tiles_n, rank, nsplit_terms, map_mode;
 };
 
-template <int EPI>
-__global__ __launch_bounds__(256, 1) void w8a8_gemm_kernel(GemmArgs g) {
+// float32 pair -> packed bf16x2 (round to nearest even, v_cvt_pk_bf16_f32)
+__device__ inline uint32_t pack_bf16x2(float lo, float hi) {
+  typedef float v2f __attribute__((ext_vector_type(2)));
+  typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+  v2f v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, v2bf));
+}
+
+// silu(g) * u with g, u already rounded to bf16 (x * logistic(x), exp and reciprocal in
+// hardware precision: 1 ulp each)
+__device__ inline float swiglu_f32(float g, float u) {
+  const float sig = __builtin_amdgcn_rcpf(1.0f + __expf(-g));
+  return (g * sig) * u;
+}
+
+constexpr int kGemmTileM = 256;
+constexpr int kGemmTileN = 128;
+constexpr int kGemmStages = 3;
+constexpr int kGemmStageBytes = 24576;  // A: 8 row blocks x 2 k blocks, B: 4 column blocks x 2 k blocks
+constexpr int kGemmLdsBytes = kGemmStages * kGemmStageBytes;
+
+template <int EPI, int NKK, int DBG = 0>
+__global__ __launch_bounds__(256, 2) void w8a8_gemm_kernel(GemmArgs g) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 1, wn = wave & 1;
 
   // ---- XCD-aware tile mapping: consecutive workgroup ids land on different XCDs, so each
   // XCD gets a contiguous range of a band-major tile order (4 row tiles x all column tiles).
-  const uint32_t total_rows = g.meta ? (uint32_t)g.meta[0] : g.rows_static;
+  const uint32_t total_rows = round_up(g.M, 32u);
   const uint32_t ntile = g.tiles_m * g.tiles_n;
   const uint32_t per_xcd = (ntile + 7u) / 8u;
-  const uint32_t t = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+  const uint32_t t = g.map_mode == 1 ? blockIdx.x : (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
   if (t >= ntile) return;
   constexpr uint32_t GM = 4;
   const uint32_t band = t / (GM * g.tiles_n);
@@ -54,229 +76,300 @@ __global__ __launch_bounds__(256, 1) void w8a8_gemm_kernel(GemmArgs g) {
   const uint32_t in_band = t - band * GM * g.tiles_n;
   const uint32_t tm = band * GM + in_band % band_rows;
   const uint32_t tn = in_band / band_rows;
-  if (tm * 256u >= total_rows) return;
-
-  // grouped (ragged) mode: a whole row tile may span several groups; weights are per group,
-  // so a tile is processed once per 32-row block run with one weight.  To keep the main loop
-  // simple the grouped launcher guarantees one group per row tile (tile rows = 32-row blocks
-  // of a single group); see launch code.  Dense mode shares one weight.
-  const uint32_t tile_group = (g.grouped && g.blk_group) ? (uint32_t)g.blk_group[tm * 8u] : 0u;
 
   const unsigned char* Ag = g.xq + (size_t)tm * 8u * g.KB * kBlockBytes;
-  const unsigned char* Bg = g.wp + (size_t)tile_group * g.w_group_stride + (size_t)tn * 8u * g.KB * kBlockBytes;
-  const float* swg = g.sw + (size_t)tile_group * (g.grouped ? g.N : 0u);
+  const unsigned char* Bg = g.wp + (size_t)tn * 4u * g.KB * kBlockBytes;
 
-  v16i acc[4][4];
+  v16i acc[2][4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
-  const int KT = (int)(g.K_pad / kTileK);
-  auto issue = [&](int kt, int stage) {
-    unsigned char* As = lds + stage * 65536;
-    unsigned char* Bs = As + 32768;
+  // ---- main loop
+  constexpr int kStages = kGemmStages;
+  constexpr int kLoadsPerTile = 6;  // direct-to-LDS loads each wave issues per tile
+  const int KT = (int)(g.K_pad / 64u);
+  auto issue = [&](int kt) {
+    unsigned char* St = lds + (kt % kStages) * kGemmStageBytes;
 #pragma unroll
-    for (int q = 0; q < 8; ++q) {
-      const int c = wave * 8 + q;  // chunk: row block c / 4 (0..7), k block c % 4
-      const size_t goff = ((size_t)(c >> 2) * g.KB + (size_t)kt * 4 + (c & 3)) * kBlockBytes + lane * 16;
-      load_1k_to_lds(Ag + goff, As + c * kBlockBytes);
-      load_1k_to_lds(Bg + goff, Bs + c * kBlockBytes);
+    for (int q = 0; q < 6; ++q) {
+      const int c = wave * 6 + q;  // chunks 0..15: A (row block c/2, k block c%2); 16..23: B
+      const unsigned char* base = c < 16 ? Ag : Bg;
+      const int rb = c < 16 ? (c >> 1) : ((c - 16) >> 1);
+      const size_t goff = ((size_t)rb * g.KB + (size_t)kt * 2 + (c & 1)) * kBlockBytes + lane * 16;
+      load_1k_to_lds(base + goff, St + c * kBlockBytes);
+    }
+  };
+  auto read_frags = [&](int kt, int ks, v4i (&af)[2], v4i (&bf)[4]) {
+    const unsigned char* As = lds + (kt % kStages) * kGemmStageBytes;
+    const unsigned char* Bs = As + 16384;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      af[i] = *reinterpret_cast<const v4i*>(As + ((wave * 2 + i) * 2 + ks) * kBlockBytes + lane * 16);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      bf[j] = *reinterpret_cast<const v4i*>(Bs + (j * 2 + ks) * kBlockBytes + lane * 16);
+  };
+  auto mfma8 = [&](const v4i (&af)[2], const v4i (&bf)[4]) {
+    if constexpr (DBG == 1) {  // measurement only: no MFMA work, keep the operands alive
+#pragma unroll
+      for (int i = 0; i < 2; ++i) asm volatile("" ::"v"(af[i]), "v"(bf[i]), "v"(bf[i + 2]));
+      return;
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
+  };
+
+  v4i fa0[2], fb0[4], fa1[2], fb1[4];
+#pragma unroll
+  for (int st = 0; st < kStages - 1; ++st)
+    if (st < KT) issue(st);
+  if (KT > kStages - 2) wait_vmcnt<(kStages - 2) * kLoadsPerTile>(); else wait_vmcnt<0>();
+  lds_barrier();
+  read_frags(0, 0, fa0, fb0);
+  const int KT_main = KT - (kStages - 1);  // tiles that still have a tile to prefetch
+  int kt = 0;
+  for (; kt < KT_main; ++kt) {
+    // ---- k-step 0 of tile kt: prefetch the k-step 1 fragments and the tile kStages-1 ahead.
+    // The MFMAs lead so that the wait for their operands does not cover the new LDS reads.
+    read_frags(kt, 1, fa1, fb1);
+    if constexpr (DBG < 2) issue(kt + kStages - 1);
+    mfma8(fa0, fb0);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+#pragma unroll
+    for (int q = 0; q < 6; ++q) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // 1 VMEM read
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- k-step 1: tile kt+1 must have landed before its first fragments are fetched
+    if constexpr (DBG < 2) wait_vmcnt<(kStages - 2) * kLoadsPerTile>();
+    lds_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(kt + 1, 0, fa0, fb0);
+    mfma8(fa1, fb1);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+#pragma unroll
+    for (int q = 0; q < 6; ++q) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  for (; kt < KT; ++kt) {  // drain: nothing left to prefetch
+    read_frags(kt, 1, fa1, fb1);
+    mfma8(fa0, fb0);
+    wait_vmcnt<0>();
+    lds_barrier();
+    if (kt + 1 < KT) read_frags(kt + 1, 0, fa0, fb0);
+    mfma8(fa1, fb1);
+  }
+  lds_barrier();  // every wave is done with the stage buffers; the epilogue reuses the LDS
+
+  // ------------------------------------------------------------------ epilogue
+  // Lane (c = lane % 32, h = lane / 32) owns, in each of its wave's two 32 x 128 strips, the four
+  // consecutive original columns ncol .. ncol+3 (accumulator blocks j = 0..3) of the 16 rows
+  // 8*(v/4) + 4*h + v%4.
+  constexpr bool kLora = (NKK > 0) && (EPI != kEpiAcc);
+  constexpr int kZ = NKK > 0 ? NKK : 1;
+  const int c = lane & 31, h = lane >> 5;
+  const uint32_t m0 = tm * 256u + wave * 64u;
+  const uint32_t ncol = tn * 128u + 4u * c;
+  const uint32_t n_out = (EPI == kEpiSwiglu) ? g.N / 2u : g.N;
+  const bool full_n = (tn * 128u + 128u <= g.N) && ((g.N & 3u) == 0);  // uniform
+  float sw[4] = {0.f, 0.f, 0.f, 0.f};
+  if (EPI != kEpiAcc) {
+    if (full_n) {
+      const float4 s4 = *reinterpret_cast<const float4*>(g.sw + ncol);
+      sw[0] = s4.x; sw[1] = s4.y; sw[2] = s4.z; sw[3] = s4.w;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (ncol + j < g.N) sw[j] = g.sw[ncol + j];
+    }
+  }
+  // LoRA-B staging, private to the wave: bf16 [16*NKK][128] at lds + wave * 16 KiB
+  uint16_t* Bl = reinterpret_cast<uint16_t*>(lds + wave * 16384);
+  int staged = -1;
+
+  auto load_zfrags = [&](uint32_t blk, v8us (&zf)[kZ][3]) {
+    if constexpr (kLora) {
+      const unsigned char* zb = g.zp + (size_t)blk * NKK * 3u * kBlockBytes + lane * 16;
+#pragma unroll
+      for (int kk = 0; kk < NKK; ++kk)
+#pragma unroll
+        for (int s = 0; s < 3; ++s)
+          zf[kk][s] = *reinterpret_cast<const v8us*>(zb + (kk * 3 + s) * kBlockBytes);
     }
   };
 
-  issue(0, 0);
-  wait_vmcnt0();
-  __syncthreads();
-  for (int kt = 0; kt < KT; ++kt) {
-    if (kt + 1 < KT) issue(kt + 1, (kt + 1) & 1);
-    const unsigned char* As = lds + (kt & 1) * 65536;
-    const unsigned char* Bs = As + 32768;
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      v4i af[4], bf[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        af[i] = *reinterpret_cast<const v4i*>(As + ((wm * 4 + i) * 4 + ks) * kBlockBytes + lane * 16);
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        bf[j] = *reinterpret_cast<const v4i*>(Bs + ((wn * 4 + j) * 4 + ks) * kBlockBytes + lane * 16);
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
-    }
-    wait_vmcnt0();
-    __syncthreads();
-  }
-
-  // ------------------------------------------------------------------ epilogue
-  const int c = lane & 31, h = lane >> 5;
-  const uint32_t m0 = tm * 256u + wm * 128u;           // first grouped slot of this wave
-  const uint32_t n0 = tn * 256u + wn * 128u;           // first packed column of this wave
-  const uint32_t n_out = (EPI == kEpiSwiglu) ? g.N / 2u : g.N;
-  // LoRA-B staging, one buffer per wave row (wm): bf16 [r_pad][256] at lds + wm * 32 KiB
-  uint16_t* Bl = reinterpret_cast<uint16_t*>(lds + wm * 32768);
-  int staged0 = -1, staged1 = -1;
-  const bool has_lora = (EPI != kEpiAcc) && g.r_pad > 0 && g.z_part != nullptr;
-
   auto epilogue_block = [&](auto BI) {
     constexpr int bi = decltype(BI)::value;
-    const uint32_t blk0 = tm * 8u + bi, blk1 = blk0 + 4u;
-    const bool act0 = blk0 * 32u < total_rows, act1 = blk1 * 32u < total_rows;
-    const int grp0 = act0 ? (g.blk_group ? g.blk_group[blk0] : 0) : staged0;
-    const int grp1 = act1 ? (g.blk_group ? g.blk_group[blk1] : 0) : staged1;
-    const bool active = wm ? act1 : act0;
-    const int grp = wm ? grp1 : grp0;
-    if (has_lora && (grp0 != staged0 || grp1 != staged1)) {  // uniform over the workgroup
-      __syncthreads();
-      const int mine = wm ? staged1 : staged0;
-      if (grp != mine && grp >= 0) {
-        const uint16_t* Bsrc = g.lora_b + (size_t)grp * g.rank * g.N;
-        const uint32_t ncol0 = tn * 256u;
-        const uint32_t t128 = (uint32_t)(tid & 127);
-        for (uint32_t q = t128; q < g.r_pad * 32u; q += 128) {
-          const uint32_t r = q >> 5, cc = (q & 31u) * 8u;
-          v8us val = {0, 0, 0, 0, 0, 0, 0, 0};
-          if (r < g.rank) {
-            const size_t off = (size_t)r * g.N + ncol0 + cc;
-            if ((g.N & 7u) == 0 && ncol0 + cc + 8u <= g.N) {
-              val = *reinterpret_cast<const v8us*>(Bsrc + off);
-            } else {
-#pragma unroll
-              for (int e = 0; e < 8; ++e)
-                if (ncol0 + cc + e < g.N) val[e] = Bsrc[off + e];
-            }
-          }
-          *reinterpret_cast<v8us*>(Bl + r * 256u + cc) = val;
-        }
-      }
-      __syncthreads();
-      staged0 = grp0;
-      staged1 = grp1;
-    }
-    if (!active) return;
     const uint32_t pbase = m0 + bi * 32u;
+    if (pbase >= total_rows) return;  // wave-uniform
+    const uint32_t blk = pbase / 32u;
+    v8us zf[kZ][3];
+    load_zfrags(blk, zf);
 
-    // rows this lane owns in the block: 8*gq + 4*h + e, gq = 0..3, e = 0..3
+    // rows this lane owns in the block: 8*gq + 4*h + e
     float sxv[16];
-    int srcv[16];
+    uint32_t rowoff[16];  // element offset of the output row, or 0xffffffff for padding rows
+    bool all_rows = true;
 #pragma unroll
     for (int gq = 0; gq < 4; ++gq) {
       const uint32_t p4 = pbase + 8u * gq + 4u * h;
-      const float4 s4 = *reinterpret_cast<const float4*>(g.sx + p4);
-      sxv[4 * gq + 0] = s4.x; sxv[4 * gq + 1] = s4.y; sxv[4 * gq + 2] = s4.z; sxv[4 * gq + 3] = s4.w;
+      if (EPI != kEpiAcc) {
+        const float4 s4 = *reinterpret_cast<const float4*>(g.sx + p4);
+        sxv[4 * gq + 0] = s4.x; sxv[4 * gq + 1] = s4.y; sxv[4 * gq + 2] = s4.z; sxv[4 * gq + 3] = s4.w;
+      }
+      int src[4];
       if (g.src_row) {
         const int4 r4 = *reinterpret_cast<const int4*>(g.src_row + p4);
-        srcv[4 * gq + 0] = r4.x; srcv[4 * gq + 1] = r4.y; srcv[4 * gq + 2] = r4.z; srcv[4 * gq + 3] = r4.w;
+        src[0] = r4.x; src[1] = r4.y; src[2] = r4.z; src[3] = r4.w;
       } else {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) srcv[4 * gq + e] = (int)(p4 + e);
+        for (int e = 0; e < 4; ++e) src[e] = (int)(p4 + e);
       }
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        if (srcv[4 * gq + e] >= (int)g.M) srcv[4 * gq + e] = -1;
+      for (int e = 0; e < 4; ++e) {
+        const bool ok = src[e] >= 0 && src[e] < (int)g.M;
+        all_rows = all_rows && ok;
+        rowoff[4 * gq + e] = ok ? (uint32_t)src[e] * ((EPI == kEpiAcc) ? g.N : n_out) : 0xffffffffu;
+      }
     }
+    const bool fast = full_n && (__builtin_amdgcn_ballot_w64(!all_rows) == 0);  // uniform
 
-    const float sgrp = has_lora ? g.lora_scaling[grp] : 0.0f;
-#pragma unroll
-    for (int jp = 0; jp < 2; ++jp) {
-      const uint32_t ne = n0 + 64u * jp + 2u * c;  // original even column; the odd one is ne + 1
-      v16f low[2];
-      if (has_lora) {
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) low[j][e] = 0.0f;
-        const uint32_t prow = pbase + c;  // A-operand row of this lane
-        const int nkk = (int)(g.r_pad / 16u);
-        for (int kk = 0; kk < nkk; ++kk) {
-          float zf[8];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) zf[e] = 0.0f;
-          for (uint32_t ks = 0; ks < g.ksplit; ++ks) {
-            const float* zp = g.z_part + ((size_t)ks * g.slots + prow) * g.r_pad + 16u * kk + 8u * h;
-            const float4 a0 = *reinterpret_cast<const float4*>(zp);
-            const float4 a1 = *reinterpret_cast<const float4*>(zp + 4);
-            zf[0] += a0.x; zf[1] += a0.y; zf[2] += a0.z; zf[3] += a0.w;
-            zf[4] += a1.x; zf[5] += a1.y; zf[6] += a1.z; zf[7] += a1.w;
-          }
-          v8us zt[3];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const uint32_t b0 = f32_to_bf16_bits(zf[e]);
-            const float r1 = zf[e] - bf16_bits_to_f32(b0);
-            const uint32_t b1 = f32_to_bf16_bits(r1);
-            const float r2 = r1 - bf16_bits_to_f32(b1);
-            const uint32_t b2 = f32_to_bf16_bits(r2);
-            zt[0][e] = (unsigned short)b0; zt[1][e] = (unsigned short)b1; zt[2][e] = (unsigned short)b2;
-          }
-#pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            v8us bfr;
-            const uint32_t col = wn * 128u + 64u * jp + 2u * c + j;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) bfr[e] = Bl[(16u * kk + 8u * h + e) * 256u + col];
-            const v8bf bb = __builtin_bit_cast(v8bf, bfr);
-            if (g.nsplit_terms >= 3)
-              low[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, zt[2]), bb, low[j], 0, 0, 0);
-            low[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, zt[1]), bb, low[j], 0, 0, 0);
-            low[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, zt[0]), bb, low[j], 0, 0, 0);
-          }
-        }
-      }
-      float sw0 = 0.0f, sw1 = 0.0f;
-      if (EPI != kEpiAcc) {
-        if (ne < g.N) sw0 = swg[ne];
-        if (ne + 1u < g.N) sw1 = swg[ne + 1u];
-      }
+    if (EPI == kEpiAcc) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int src = srcv[v];
-        if (src < 0) continue;
-        const int a0 = acc[bi][2 * jp][v], a1 = acc[bi][2 * jp + 1][v];
-        if (EPI == kEpiAcc) {
-          int32_t* o = reinterpret_cast<int32_t*>(g.out) + (size_t)src * g.N;
-          if (ne < g.N) o[ne] = a0;
-          if (ne + 1u < g.N) o[ne + 1u] = a1;
-          continue;
-        }
-        float y0 = ((float)a0 * sxv[v]) * sw0;
-        float y1 = ((float)a1 * sxv[v]) * sw1;
-        if (has_lora) {
-          const float l0 = low[0][v] * sgrp;
-          const float l1 = low[1][v] * sgrp;
-          y0 = y0 + l0;
-          y1 = y1 + l1;
-        }
-        if (EPI == kEpiSwiglu) {
-          const uint32_t pc = ne >> 1;
-          if (pc < n_out) {
-            const float gate = bf16_round_f32(y0), up = bf16_round_f32(y1);
-            const float sig = 1.0f / (1.0f + __expf(-gate));
-            const float prod = (gate * sig) * up;
-            reinterpret_cast<uint16_t*>(g.out)[(size_t)src * n_out + pc] = (uint16_t)f32_to_bf16_bits(prod);
-          }
+        if (!fast && rowoff[v] == 0xffffffffu) continue;
+        int32_t* o = reinterpret_cast<int32_t*>(g.out) + rowoff[v] + ncol;
+        if (fast) {
+          *reinterpret_cast<int4*>(o) = make_int4(acc[bi][0][v], acc[bi][1][v], acc[bi][2][v], acc[bi][3][v]);
         } else {
-          uint16_t* o = reinterpret_cast<uint16_t*>(g.out) + (size_t)src * g.N;
-          if (ne + 1u < g.N && (g.N & 1u) == 0) {
-            if (g.residual) {
-              const uint32_t rr = *reinterpret_cast<const uint32_t*>(g.residual + (size_t)src * g.N + ne);
-              y0 = y0 + bf16_bits_to_f32(rr & 0xffffu);
-              y1 = y1 + __uint_as_float(rr & 0xffff0000u);
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (ncol + j < g.N) o[j] = acc[bi][j][v];
+        }
+      }
+      return;
+    }
+
+    float y[16][4];
+#pragma unroll
+    for (int v = 0; v < 16; ++v)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) y[v][j] = ((float)acc[bi][j][v] * sxv[v]) * sw[j];
+
+    if constexpr (kLora) {
+      // groups (adapters) present in this 32-row block: usually one, two at a group boundary
+      const uint32_t range = g.blk_range ? (uint32_t)g.blk_range[blk] : 0u;
+      const int glo = (int)(range & 0xffffu), ghi = (int)(range >> 16);
+      const int rowgrp = (g.slot_group && ghi > glo) ? g.slot_group[pbase + c] : glo;
+      for (int gi = glo; gi <= ghi; ++gi) {  // wave-uniform
+        if (gi != staged) {
+          // stage B[gi][0:16*NKK][tile columns] as bf16 [16*NKK][128]; LDS operations of one
+          // wave execute in order, so no barrier is needed around this wave-private buffer
+          const uint16_t* Bsrc = g.lora_b + (size_t)gi * g.rank * g.N;
+          const uint32_t tcol0 = tn * 128u;
+          for (uint32_t q = (uint32_t)lane; q < NKK * 16u * 16u; q += 64u) {
+            const uint32_t r = q >> 4, cc = (q & 15u) * 8u;
+            v8us val = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (r < g.rank) {
+              const size_t off = (size_t)r * g.N + tcol0 + cc;
+              if ((g.N & 7u) == 0 && tcol0 + cc + 8u <= g.N) {
+                val = *reinterpret_cast<const v8us*>(Bsrc + off);
+              } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                  if (tcol0 + cc + e < g.N) val[e] = Bsrc[off + e];
+              }
             }
-            *reinterpret_cast<uint32_t*>(o + ne) = f32_to_bf16_bits(y0) | (f32_to_bf16_bits(y1) << 16);
-          } else {
-            if (ne < g.N) {
-              if (g.residual) y0 = y0 + bf16_bits_to_f32(g.residual[(size_t)src * g.N + ne]);
-              o[ne] = (uint16_t)f32_to_bf16_bits(y0);
+            *reinterpret_cast<v8us*>(Bl + r * 128u + cc) = val;
+          }
+          staged = gi;
+        }
+        const bool mine = (ghi == glo) || (rowgrp == gi);
+        const float sgrp = g.lora_scaling[gi];
+#pragma unroll
+        for (int jp = 0; jp < 2; ++jp) {
+          v16f low[2];
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) low[j][e] = 0.0f;
+#pragma unroll
+          for (int kk = 0; kk < NKK; ++kk) {
+            const v8us zero = {0, 0, 0, 0, 0, 0, 0, 0};
+            const v8us z0 = mine ? zf[kk][0] : zero, z1 = mine ? zf[kk][1] : zero, z2 = mine ? zf[kk][2] : zero;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              v8us bfr;
+              const uint32_t col = 4u * c + 2u * jp + j;
+#pragma unroll
+              for (int e = 0; e < 8; ++e) bfr[e] = Bl[(16u * kk + 8u * h + e) * 128u + col];
+              const v8bf bb = __builtin_bit_cast(v8bf, bfr);
+              if (g.nsplit_terms >= 3)
+                low[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, z2), bb, low[j], 0, 0, 0);
+              low[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, z1), bb, low[j], 0, 0, 0);
+              low[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, z0), bb, low[j], 0, 0, 0);
             }
-            if (ne + 1u < g.N) {
-              if (g.residual) y1 = y1 + bf16_bits_to_f32(g.residual[(size_t)src * g.N + ne + 1u]);
-              o[ne + 1u] = (uint16_t)f32_to_bf16_bits(y1);
+          }
+#pragma unroll
+          for (int v = 0; v < 16; ++v)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              const float l = low[j][v] * sgrp;
+              y[v][2 * jp + j] = y[v][2 * jp + j] + l;
+            }
+        }
+      }
+    }
+
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      if (!fast && rowoff[v] == 0xffffffffu) continue;
+      if (EPI == kEpiSwiglu) {
+        // (y0, y1) and (y2, y3) are (gate, up) of the product columns ncol/2 and ncol/2 + 1
+        const uint32_t f01 = pack_bf16x2(y[v][0], y[v][1]), f23 = pack_bf16x2(y[v][2], y[v][3]);
+        const float p0 = swiglu_f32(__uint_as_float(f01 << 16), __uint_as_float(f01 & 0xffff0000u));
+        const float p1 = swiglu_f32(__uint_as_float(f23 << 16), __uint_as_float(f23 & 0xffff0000u));
+        uint16_t* o = reinterpret_cast<uint16_t*>(g.out) + rowoff[v] + (ncol >> 1);
+        const uint32_t pk = pack_bf16x2(p0, p1);
+        if (fast) {
+          *reinterpret_cast<uint32_t*>(o) = pk;
+        } else {
+          if ((ncol >> 1) < n_out) o[0] = (uint16_t)(pk & 0xffffu);
+          if ((ncol >> 1) + 1u < n_out) o[1] = (uint16_t)(pk >> 16);
+        }
+      } else {
+        uint16_t* o = reinterpret_cast<uint16_t*>(g.out) + rowoff[v] + ncol;
+        if (fast) {
+          float r0 = y[v][0], r1 = y[v][1], r2 = y[v][2], r3 = y[v][3];
+          if (g.residual) {
+            const uint2 rr = *reinterpret_cast<const uint2*>(g.residual + rowoff[v] + ncol);
+            r0 = r0 + __uint_as_float(rr.x << 16);
+            r1 = r1 + __uint_as_float(rr.x & 0xffff0000u);
+            r2 = r2 + __uint_as_float(rr.y << 16);
+            r3 = r3 + __uint_as_float(rr.y & 0xffff0000u);
+          }
+          *reinterpret_cast<uint2*>(o) = make_uint2(pack_bf16x2(r0, r1), pack_bf16x2(r2, r3));
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            if (ncol + j < g.N) {
+              float yy = y[v][j];
+              if (g.residual) yy = yy + bf16_bits_to_f32(g.residual[rowoff[v] + ncol + j]);
+              o[j] = (uint16_t)(pack_bf16x2(yy, 0.0f) & 0xffffu);
             }
           }
         }
@@ -285,8 +378,6 @@ __global__ __launch_bounds__(256, 1) void w8a8_gemm_kernel(GemmArgs g) {
   };
   epilogue_block(std::integral_constant<int, 0>{});
   epilogue_block(std::integral_constant<int, 1>{});
-  epilogue_block(std::integral_constant<int, 2>{});
-  epilogue_block(std::integral_constant<int, 3>{});
 }
 
 }  // namespace w8a8

@@ -39,26 +39,24 @@ __global__ __launch_bounds__(256) void unpack_weight_kernel(const unsigned char*
   uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= (uint64_t)K * N) return;
   uint32_t k = (uint32_t)(idx / N), n = (uint32_t)(idx % N);
-  // packed column of original column n
-  uint32_t c = (n & ~63u) + 32u * (n & 1u) + ((n & 63u) >> 1);
-  codes[idx] = (int8_t)packed[packed_offset(c, k, KB)];
+  codes[idx] = (int8_t)packed[packed_offset(orig_to_packed_col(n), k, KB)];
 }
 
 // ---------------------------------------------------------------------------------------
-// Adapter routing: group rows by adapter, every group padded to a multiple of 32 rows
-// (the counterpart of prepare_routing, skyrl/tx/layers/util.py:66-87).
-//   meta[0]       = number of grouped row slots in use (multiple of 32)
-//   src_row[p]    = original row of grouped slot p, or -1 for padding
+// Adapter routing: rows are grouped by adapter with no padding between groups (the
+// counterpart of prepare_routing, skyrl/tx/layers/util.py:66-87).
+//   src_row[p]    = original row of grouped slot p (p < M), -1 for the slots beyond M
 //   dst_pos[m]    = grouped slot of original row m
-//   blk_group[b]  = adapter of the 32-row block b
+//   slot_group[p] = adapter of grouped slot p
+//   blk_range[b]  = first adapter | last adapter << 16 of the 32-row block b
 // Out-of-range adapter indices are clamped into range (XLA gather semantics).
 // One workgroup; the order of rows inside a group does not influence any result.
 // ---------------------------------------------------------------------------------------
 __global__ __launch_bounds__(1024) void route_rows_kernel(const int32_t* __restrict__ idx, uint32_t M,
                                                           uint32_t n_groups, uint32_t slots,
-                                                          int32_t* __restrict__ meta, int32_t* __restrict__ src_row,
-                                                          int32_t* __restrict__ dst_pos,
-                                                          int32_t* __restrict__ blk_group) {
+                                                          int32_t* __restrict__ src_row, int32_t* __restrict__ dst_pos,
+                                                          int32_t* __restrict__ slot_group,
+                                                          int32_t* __restrict__ blk_range) {
   __shared__ int cnt[kMaxAdapters];
   __shared__ int start[kMaxAdapters + 1];
   __shared__ int cursor[kMaxAdapters];
@@ -75,74 +73,40 @@ __global__ __launch_bounds__(1024) void route_rows_kernel(const int32_t* __restr
     int pos = 0;
     for (uint32_t a = 0; a < n_groups; ++a) {
       start[a] = pos;
-      pos += (cnt[a] + 31) & ~31;
+      pos += cnt[a];
     }
     start[n_groups] = pos;
-    meta[0] = pos;
-  }
-  __syncthreads();
-  for (uint32_t p = tid; p < slots; p += 1024) src_row[p] = -1;
-  const int total = start[n_groups];
-  for (uint32_t b = tid; b < slots / 32; b += 1024) {
-    int g = 0;
-    int row = (int)b * 32;
-    if (row < total) {
-      for (uint32_t a = 0; a < n_groups; ++a)
-        if (row >= start[a] && row < start[a + 1]) g = (int)a;
-    }
-    blk_group[b] = g;
   }
   __syncthreads();
   for (uint32_t i = tid; i < M; i += 1024) {
     int a = idx[i];
     a = a < 0 ? 0 : (a >= (int)n_groups ? (int)n_groups - 1 : a);
-    int p = start[a] + atomicAdd(&cursor[a], 1);
+    const int p = start[a] + atomicAdd(&cursor[a], 1);
     src_row[p] = (int)i;
     dst_pos[i] = p;
   }
-}
-
-// Same tables for rows that arrive already grouped (ragged groups of an expert layer,
-// skyrl/tx/layers/util.py:8-59): group g owns group_sizes[g] consecutive rows; rows past
-// sum(group_sizes) get dst_pos = -1 and the caller's output rows are zero-filled.
-__global__ __launch_bounds__(1024) void route_groups_kernel(const int32_t* __restrict__ group_sizes, uint32_t M,
-                                                            uint32_t n_groups, uint32_t slots,
-                                                            int32_t* __restrict__ meta, int32_t* __restrict__ src_row,
-                                                            int32_t* __restrict__ dst_pos,
-                                                            int32_t* __restrict__ blk_group,
-                                                            int32_t* __restrict__ row_start /* [n_groups+1] scratch */,
-                                                            int32_t* __restrict__ slot_start /* [n_groups+1] scratch */) {
-  const uint32_t tid = threadIdx.x;
-  if (tid == 0) {
-    int r = 0, p = 0;
-    for (uint32_t g = 0; g < n_groups; ++g) {
-      int sz = group_sizes[g];
-      if (sz < 0) sz = 0;
-      if (r + sz > (int)M) sz = (int)M - r;
-      row_start[g] = r;
-      slot_start[g] = p;
-      r += sz;
-      p += (sz + 31) & ~31;
+  // group of a slot = the group whose [start, start+count) range holds it
+  for (uint32_t p = tid; p < slots; p += 1024) {
+    int g = 0;
+    if (p < M) {
+      for (uint32_t a = 0; a < n_groups; ++a)
+        if ((int)p >= start[a] && (int)p < start[a + 1]) g = (int)a;
+    } else {
+      src_row[p] = -1;
+      for (uint32_t a = 0; a < n_groups; ++a)
+        if (cnt[a] > 0) g = (int)a;  // padding slots follow the last non-empty group
     }
-    row_start[n_groups] = r;
-    slot_start[n_groups] = p;
-    meta[0] = p;
+    slot_group[p] = g;
   }
-  __syncthreads();
-  __threadfence_block();
-  for (uint32_t p = tid; p < slots; p += 1024) src_row[p] = -1;
-  for (uint32_t i = tid; i < M; i += 1024) dst_pos[i] = -1;
-  for (uint32_t b = tid; b < slots / 32; b += 1024) blk_group[b] = 0;
-  __syncthreads();
-  // one wave per group walks its rows
-  const uint32_t wave = tid >> 6, lane = tid & 63;
-  for (uint32_t g = wave; g < n_groups; g += 16) {
-    int r0 = row_start[g], r1 = row_start[g + 1], p0 = slot_start[g], p1 = slot_start[g + 1];
-    for (int i = (int)lane; i < r1 - r0; i += 64) {
-      src_row[p0 + i] = r0 + i;
-      dst_pos[r0 + i] = p0 + i;
+  for (uint32_t b = tid; b < slots / 32u; b += 1024) {
+    const int p0 = (int)b * 32, p1 = (p0 + 31 < (int)M) ? p0 + 31 : (int)M - 1;
+    int g0 = 0, g1 = 0;
+    for (uint32_t a = 0; a < n_groups; ++a) {
+      if (p0 >= start[a] && p0 < start[a + 1]) g0 = (int)a;
+      if (p1 >= start[a] && p1 < start[a + 1]) g1 = (int)a;
     }
-    for (int b = p0 / 32 + (int)lane; b < p1 / 32; b += 64) blk_group[b] = (int)g;
+    if (p0 >= (int)M) { g0 = 0; g1 = 0; }
+    blk_range[b] = g0 | (g1 << 16);
   }
 }
 
@@ -254,84 +218,144 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(QuantArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------
+// LoRA A re-layout: A [n, K, r] (rank contiguous) -> At [n, r, K] (K contiguous), so that an
+// MFMA operand (8 consecutive k of one rank column) is one 16-byte load.  LoRA parameters
+// are trainable and may change between calls, so this runs per call; it moves n*K*r*2 bytes.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void lora_a_transpose_kernel(const uint16_t* __restrict__ a,
+                                                               uint16_t* __restrict__ at, uint32_t n_groups,
+                                                               uint32_t K, uint32_t r) {
+  const uint32_t rc = (r + 7u) / 8u;  // 8-wide rank chunks per k
+  const uint64_t total = (uint64_t)n_groups * K * rc;
+  const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const uint32_t ch = (uint32_t)(idx % rc);
+  const uint64_t gk = idx / rc;  // group * K + k
+  const uint32_t k = (uint32_t)(gk % K);
+  const uint32_t grp = (uint32_t)(gk / K);
+  const uint16_t* src = a + gk * r + ch * 8u;
+  uint16_t v[8];
+  if ((r & 7u) == 0) {
+    const v8us w = *reinterpret_cast<const v8us*>(src);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = w[e];
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = (ch * 8u + e < r) ? src[e] : (uint16_t)0;
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const uint32_t col = ch * 8u + e;
+    if (col < r) at[((size_t)grp * r + col) * K + k] = v[e];
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // LoRA-A projection on bf16 MFMA: z[p, :] = n[src_row[p], :] @ A[group(p)]  (float32
 // accumulation of exact bf16 products; skyrl/tx/kernels/quantized_lora.py:300-301 and
-// skyrl/tx/layers/lora.py:150).  Grid (32-row blocks, ksplit); the four waves of a
-// workgroup take disjoint K ranges and are reduced through LDS in wave order, K splits
-// are written as separate partials that the GEMM epilogue adds in split order.
+// skyrl/tx/layers/lora.py:150).  One workgroup of 8 waves per 32-row block; the waves take
+// disjoint K ranges and are reduced through LDS in wave order.  The float32 result is split
+// into three bf16 terms (z = hi + mid + lo exactly) and stored in the MFMA operand order the
+// GEMM epilogue consumes: zp[block][kk][term][lane][8], lane = row % 32 + 32 * h holding the
+// rank columns 16 kk + 8 h + 0..7.
 // ---------------------------------------------------------------------------------------
 struct LoraAArgs {
   const uint16_t* xsrc;     // bf16 [M, K] (x, or the normalized rows)
-  const uint16_t* lora_a;   // bf16 [n_groups, K, r]
+  const uint16_t* at;       // bf16 [n_groups, r, K]
   const int32_t* src_row;   // or null (identity)
-  const int32_t* blk_group; // or null (group 0)
-  const int32_t* meta;      // or null
-  float* z_part;            // f32 [ksplit, slots, r_pad]
-  uint32_t M, K, r, r_pad, slots, rows_static, steps_per_wave, n_steps;
+  const int32_t* slot_group;// or null (group 0)
+  const int32_t* blk_range; // or null
+  unsigned char* zp;        // packed z fragments
+  uint32_t M, K, r, nkk, steps_per_wave, n_steps;
 };
 
 template <int RB>  // number of 32-wide rank blocks (1 or 2)
-__global__ __launch_bounds__(256) void lora_a_kernel(LoraAArgs a) {
+__global__ __launch_bounds__(512) void lora_a_kernel(LoraAArgs a) {
   __shared__ float red[4][RB][16][64];
+  __shared__ float zs[32][RB * 32 + 1];
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-  const uint32_t pb = blockIdx.x, ks = blockIdx.y;
-  const uint32_t total = a.meta ? (uint32_t)a.meta[0] : a.rows_static;
-  if (pb * 32u >= total) return;
-  const uint32_t grp = a.blk_group ? (uint32_t)a.blk_group[pb] : 0u;
+  const uint32_t pb = blockIdx.x;
+  if (pb * 32u >= round_up(a.M, 32u)) return;
+  const uint32_t range = a.blk_range ? (uint32_t)a.blk_range[pb] : 0u;
+  const uint32_t glo = range & 0xffffu, ghi = range >> 16;
   const uint32_t i = lane & 31u, h = lane >> 5;
   const uint32_t p = pb * 32u + i;
   int src = a.src_row ? a.src_row[p] : (int)p;
   if (src >= (int)a.M) src = -1;
+  const uint32_t rowgrp = (a.slot_group && ghi > glo) ? (uint32_t)a.slot_group[p] : glo;
   const uint16_t* xr = a.xsrc + (size_t)(src < 0 ? 0 : src) * a.K;
-  const uint16_t* Ag = a.lora_a + (size_t)grp * a.K * a.r;
   v16f acc[RB];
 #pragma unroll
   for (int b = 0; b < RB; ++b)
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[b][e] = 0.0f;
-  const uint32_t wg = ks * 4u + wave;
-  uint32_t s0 = wg * a.steps_per_wave, s1 = s0 + a.steps_per_wave;
+  uint32_t s0 = wave * a.steps_per_wave, s1 = s0 + a.steps_per_wave;
   if (s1 > a.n_steps) s1 = a.n_steps;
-  for (uint32_t s = s0; s < s1; ++s) {
-    const uint32_t kbase = s * 64u + 32u * h;
+  // A block at a group boundary runs once per group with the other groups' rows zeroed.
+  for (uint32_t grp = glo; grp <= ghi; ++grp) {
+    const bool mine = src >= 0 && rowgrp == grp;
+    for (uint32_t s = s0; s < s1; ++s) {
+      const uint32_t kbase = s * 64u + 32u * h;
+      v8us xa[4], wb[RB][4];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const uint32_t k0 = kbase + 8u * t;
-      v8us xa = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (src >= 0 && k0 < a.K) xa = *reinterpret_cast<const v8us*>(xr + k0);
+      for (int t = 0; t < 4; ++t) {
+        const uint32_t k0 = kbase + 8u * t;
+        const v8us zero = {0, 0, 0, 0, 0, 0, 0, 0};
+        xa[t] = (mine && k0 < a.K) ? *reinterpret_cast<const v8us*>(xr + k0) : zero;
 #pragma unroll
-      for (int b = 0; b < RB; ++b) {
-        const uint32_t col = b * 32u + i;
-        v8us wb = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (col < a.r && k0 < a.K) {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) wb[e] = Ag[(size_t)(k0 + e) * a.r + col];
+        for (int b = 0; b < RB; ++b) {
+          const uint32_t col = b * 32u + i;
+          wb[b][t] = (col < a.r && k0 < a.K)
+                         ? *reinterpret_cast<const v8us*>(a.at + ((size_t)grp * a.r + col) * a.K + k0)
+                         : zero;
         }
-        acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, xa),
-                                                         __builtin_bit_cast(v8bf, wb), acc[b], 0, 0, 0);
       }
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int b = 0; b < RB; ++b)
+          acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, xa[t]),
+                                                           __builtin_bit_cast(v8bf, wb[b][t]), acc[b], 0, 0, 0);
     }
   }
+  // fixed-order reduction over the 8 waves: (w + w+4) pairwise, then 0..3 in order
+  if (wave >= 4) {
 #pragma unroll
-  for (int b = 0; b < RB; ++b)
+    for (int b = 0; b < RB; ++b)
 #pragma unroll
-    for (int e = 0; e < 16; ++e) red[wave][b][e][lane] = acc[b][e];
+      for (int e = 0; e < 16; ++e) red[wave - 4][b][e][lane] = acc[b][e];
+  }
   __syncthreads();
-  if (wave == 0) {
+  if (wave < 4) {
 #pragma unroll
-    for (int b = 0; b < RB; ++b) {
-      const uint32_t col = b * 32u + i;
+    for (int b = 0; b < RB; ++b)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        float sum = red[0][b][e][lane];
-        sum += red[1][b][e][lane];
-        sum += red[2][b][e][lane];
-        sum += red[3][b][e][lane];
-        const uint32_t row = 8u * (e >> 2) + 4u * h + (e & 3u);
-        if (col < a.r_pad)
-          a.z_part[((size_t)ks * a.slots + pb * 32u + row) * a.r_pad + col] = sum;
-      }
+      for (int e = 0; e < 16; ++e) red[wave][b][e][lane] = acc[b][e] + red[wave][b][e][lane];
+  }
+  __syncthreads();
+  for (uint32_t q = threadIdx.x; q < RB * 1024u; q += 512u) {
+    const uint32_t l = q & 63u, e = (q >> 6) & 15u, b = q >> 10;
+    float sum = red[0][b][e][l];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) sum += red[w][b][e][l];
+    zs[8u * (e >> 2) + 4u * (l >> 5) + (e & 3u)][b * 32u + (l & 31u)] = sum;
+  }
+  __syncthreads();
+  for (uint32_t q = threadIdx.x; q < a.nkk * 3u * 64u; q += 512u) {
+    const uint32_t l = q & 63u, term = (q >> 6) % 3u, kk = q / 192u;
+    const uint32_t row = l & 31u, hh = l >> 5;
+    v8us o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float z = zs[row][16u * kk + 8u * hh + e];
+      const uint32_t b0 = f32_to_bf16_bits(z);
+      const float r1 = z - bf16_bits_to_f32(b0);
+      const uint32_t b1 = f32_to_bf16_bits(r1);
+      const float r2 = r1 - bf16_bits_to_f32(b1);
+      const uint32_t b2 = f32_to_bf16_bits(r2);
+      o[e] = (unsigned short)(term == 0 ? b0 : (term == 1 ? b1 : b2));
     }
+    *reinterpret_cast<v8us*>(a.zp + (((size_t)pb * a.nkk + kk) * 3u + term) * kBlockBytes + l * 16u) = o;
   }
 }
 

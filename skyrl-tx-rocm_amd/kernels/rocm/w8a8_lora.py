@@ -202,95 +202,132 @@ def _normalize_lora(lora_a, lora_b, lora_scaling, k: int, n: int, device):
     return a3.contiguous(), b3.contiguous(), s.contiguous(), n_ad, r
 
 
+class ForwardPlan:
+    """Validated arguments, output, workspace and the C struct of one forward call.
+
+    Building the plan does all host-side checks and allocations once; ``run()`` is a
+    single C call that enqueues the kernels on torch's current stream, so a caller
+    that repeats the same call (a decode loop, a benchmark) pays no per-call Python
+    or allocator work.  The plan keeps every tensor it points at alive.
+    """
+
+    def __init__(self, x: torch.Tensor, weight, lora_a=None, lora_b=None, lora_scaling=None, *,
+                 adapter_indices: torch.Tensor | None = None, rms_gamma: torch.Tensor | None = None,
+                 eps: float = 1e-6, residual: torch.Tensor | None = None, swiglu: bool = False,
+                 flags: int = 0, return_aux: bool = False, entry: str = "forward"):
+        if x.dtype != torch.bfloat16:
+            raise TypeError(f"x must be BF16, got {x.dtype}")
+        if x.ndim < 2 or math.prod(x.shape[:-1]) <= 0:
+            raise ValueError(f"x must have a nonempty row domain and final K axis, got {tuple(x.shape)}")
+        _require_cuda(x, "x")
+        pw = prepare_weight(weight)
+        k, n = pw.in_features, pw.out_features
+        if x.shape[-1] != k:
+            raise ValueError(f"x K={x.shape[-1]} does not match W8 K={k}")
+        dev = x.device
+        flat = x.reshape(-1, k).contiguous()
+        m = flat.shape[0]
+        a3, b3, s1, n_ad, r = _normalize_lora(lora_a, lora_b, lora_scaling, k, n, dev)
+        idx = None
+        if adapter_indices is not None:
+            if n_ad == 0:
+                raise ValueError("adapter_indices given without LoRA parameters")
+            idx = adapter_indices.reshape(-1)
+            if idx.shape[0] != m:
+                if idx.shape[0] == 0 or m % idx.shape[0]:
+                    raise ValueError(f"adapter_indices of length {idx.shape[0]} do not divide {m} rows")
+                idx = idx.repeat_interleave(m // idx.shape[0])  # one entry per example (lora.py:142)
+            idx = idx.to(device=dev, dtype=torch.int32).contiguous()
+        gamma = None
+        if rms_gamma is not None:
+            if tuple(rms_gamma.shape) != (k,):
+                raise ValueError(f"rms weight must have shape ({k},), got {tuple(rms_gamma.shape)}")
+            gamma = rms_gamma.to(device=dev, dtype=torch.float32).contiguous()
+        if swiglu and n % 2:
+            raise ValueError("SwiGLU needs an even number of fused gate/up columns")
+        n_out = n // 2 if swiglu else n
+        res = None
+        if residual is not None:
+            if residual.dtype != torch.bfloat16:
+                raise TypeError("residual must be BF16")
+            if tuple(residual.shape) != (*x.shape[:-1], n_out):
+                raise ValueError(
+                    f"residual must have shape {(*x.shape[:-1], n_out)}, got {tuple(residual.shape)}")
+            res = residual.reshape(m, n_out).contiguous()
+
+        lib = _native.load()
+        if swiglu:
+            flags |= _native.FLAG_SWIGLU
+        out = torch.empty((m, n_out), dtype=torch.bfloat16, device=dev)
+        ws_bytes = int(lib.mi355_w8a8_workspace_bytes(m, k, n, n_ad, r, flags))
+        if ws_bytes == 0:
+            raise ValueError(
+                f"geometry M={m}, K={k}, N={n}, rank={r}, adapters={n_ad} is outside the native path")
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        aux = {}
+        if return_aux:
+            aux["x_codes"] = torch.empty((m, k), dtype=torch.int8, device=dev)
+            aux["x_scales"] = torch.empty((m,), dtype=torch.float32, device=dev)
+            aux["acc"] = torch.empty((m, n), dtype=torch.int32, device=dev)
+            if gamma is not None:
+                aux["normalized"] = torch.empty((m, k), dtype=torch.bfloat16, device=dev)
+
+        p = _native.Problem()
+        p.struct_size = ctypes.sizeof(_native.Problem)
+        p.flags = flags
+        p.m, p.k, p.n, p.n_adapters, p.rank = m, k, n, n_ad, r
+        p.rms_eps = float(eps)
+        p.x = flat.data_ptr()
+        p.w_packed = pw.packed.data_ptr()
+        p.w_scales = pw.scales.data_ptr()
+        p.lora_a = a3.data_ptr() if n_ad else None
+        p.lora_b = b3.data_ptr() if n_ad else None
+        p.lora_scaling = s1.data_ptr() if n_ad else None
+        p.adapter_indices = idx.data_ptr() if idx is not None else None
+        p.rms_gamma = gamma.data_ptr() if gamma is not None else None
+        p.residual = res.data_ptr() if res is not None else None
+        p.out = out.data_ptr()
+        p.workspace = ws.data_ptr()
+        p.workspace_bytes = ws_bytes
+        p.aux_x_codes = aux["x_codes"].data_ptr() if return_aux else None
+        p.aux_x_scales = aux["x_scales"].data_ptr() if return_aux else None
+        p.aux_acc = aux["acc"].data_ptr() if return_aux else None
+        p.aux_normalized = aux["normalized"].data_ptr() if "normalized" in aux else None
+        self.problem = p
+        self.device = dev
+        self.entry = entry
+        self.flags = flags
+        self.aux = aux
+        self.out = out
+        self.out_shape = (*x.shape[:-1], n_out)
+        self.dims = {"m": m, "k": k, "n": n, "n_out": n_out, "n_adapters": n_ad, "rank": r}
+        self._fn = {"forward": lib.mi355_w8a8_forward_v1, "linear": lib.mi355_w8a8_lora_linear_v1,
+                    "gateup": lib.mi355_w8a8_rms_gateup_swiglu_v1,
+                    "residual": lib.mi355_w8a8_lora_residual_v1}[entry]
+        self._keep = (flat, pw, a3, b3, s1, idx, gamma, res, ws)
+
+    def run(self, extra_flags: int = 0) -> torch.Tensor:
+        """Enqueue the call on torch's current stream; returns the (reused) output tensor."""
+        self.problem.flags = self.flags | extra_flags
+        with torch.cuda.device(self.device):
+            status = self._fn(ctypes.byref(self.problem), _stream_ptr(self.device))
+        self.problem.flags = self.flags
+        _native.check(f"mi355_w8a8_{self.entry}", status)
+        return self.out.reshape(self.out_shape)
+
+
 def forward(x: torch.Tensor, weight, lora_a=None, lora_b=None, lora_scaling=None, *,
             adapter_indices: torch.Tensor | None = None, rms_gamma: torch.Tensor | None = None,
             eps: float = 1e-6, residual: torch.Tensor | None = None, swiglu: bool = False,
             flags: int = 0, return_aux: bool = False, entry: str = "forward"):
     """One W8A8 forward through the C ABI.  Returns bf16 [..., n_out] (and aux tensors)."""
-    if x.dtype != torch.bfloat16:
-        raise TypeError(f"x must be BF16, got {x.dtype}")
-    if x.ndim < 2 or math.prod(x.shape[:-1]) <= 0:
-        raise ValueError(f"x must have a nonempty row domain and final K axis, got {tuple(x.shape)}")
-    _require_cuda(x, "x")
-    pw = prepare_weight(weight)
-    k, n = pw.in_features, pw.out_features
-    if x.shape[-1] != k:
-        raise ValueError(f"x K={x.shape[-1]} does not match W8 K={k}")
-    dev = x.device
-    flat = x.reshape(-1, k).contiguous()
-    m = flat.shape[0]
-    a3, b3, s1, n_ad, r = _normalize_lora(lora_a, lora_b, lora_scaling, k, n, dev)
-    idx = None
-    if adapter_indices is not None:
-        if n_ad == 0:
-            raise ValueError("adapter_indices given without LoRA parameters")
-        idx = adapter_indices.reshape(-1)
-        if idx.shape[0] != m:
-            if idx.shape[0] == 0 or m % idx.shape[0]:
-                raise ValueError(f"adapter_indices of length {idx.shape[0]} do not divide {m} rows")
-            idx = idx.repeat_interleave(m // idx.shape[0])  # one entry per example (lora.py:142)
-        idx = idx.to(device=dev, dtype=torch.int32).contiguous()
-    gamma = None
-    if rms_gamma is not None:
-        if tuple(rms_gamma.shape) != (k,):
-            raise ValueError(f"rms weight must have shape ({k},), got {tuple(rms_gamma.shape)}")
-        gamma = rms_gamma.to(device=dev, dtype=torch.float32).contiguous()
-    if swiglu and n % 2:
-        raise ValueError("SwiGLU needs an even number of fused gate/up columns")
-    n_out = n // 2 if swiglu else n
-    res = None
-    if residual is not None:
-        if residual.dtype != torch.bfloat16:
-            raise TypeError("residual must be BF16")
-        if tuple(residual.shape) != (*x.shape[:-1], n_out):
-            raise ValueError(f"residual must have shape {(*x.shape[:-1], n_out)}, got {tuple(residual.shape)}")
-        res = residual.reshape(m, n_out).contiguous()
-
-    lib = _native.load()
-    if swiglu:
-        flags |= _native.FLAG_SWIGLU
-    out = torch.empty((m, n_out), dtype=torch.bfloat16, device=dev)
-    ws_bytes = int(lib.mi355_w8a8_workspace_bytes(m, k, n, n_ad, r, flags))
-    if ws_bytes == 0:
-        raise ValueError(f"geometry M={m}, K={k}, N={n}, rank={r}, adapters={n_ad} is outside the native path")
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-    aux = {}
-    if return_aux:
-        aux["x_codes"] = torch.empty((m, k), dtype=torch.int8, device=dev)
-        aux["x_scales"] = torch.empty((m,), dtype=torch.float32, device=dev)
-        aux["acc"] = torch.empty((m, n), dtype=torch.int32, device=dev)
-        if gamma is not None:
-            aux["normalized"] = torch.empty((m, k), dtype=torch.bfloat16, device=dev)
-
-    p = _native.Problem()
-    p.struct_size = ctypes.sizeof(_native.Problem)
-    p.flags = flags
-    p.m, p.k, p.n, p.n_adapters, p.rank = m, k, n, n_ad, r
-    p.rms_eps = float(eps)
-    p.x = flat.data_ptr()
-    p.w_packed = pw.packed.data_ptr()
-    p.w_scales = pw.scales.data_ptr()
-    p.lora_a = a3.data_ptr() if n_ad else None
-    p.lora_b = b3.data_ptr() if n_ad else None
-    p.lora_scaling = s1.data_ptr() if n_ad else None
-    p.adapter_indices = idx.data_ptr() if idx is not None else None
-    p.rms_gamma = gamma.data_ptr() if gamma is not None else None
-    p.residual = res.data_ptr() if res is not None else None
-    p.out = out.data_ptr()
-    p.workspace = ws.data_ptr()
-    p.workspace_bytes = ws_bytes
-    p.aux_x_codes = aux["x_codes"].data_ptr() if return_aux else None
-    p.aux_x_scales = aux["x_scales"].data_ptr() if return_aux else None
-    p.aux_acc = aux["acc"].data_ptr() if return_aux else None
-    p.aux_normalized = aux["normalized"].data_ptr() if "normalized" in aux else None
-    fn = {"forward": lib.mi355_w8a8_forward_v1, "linear": lib.mi355_w8a8_lora_linear_v1,
-          "gateup": lib.mi355_w8a8_rms_gateup_swiglu_v1, "residual": lib.mi355_w8a8_lora_residual_v1}[entry]
-    with torch.cuda.device(dev):
-        _native.check(f"mi355_w8a8_{entry}", fn(ctypes.byref(p), _stream_ptr(dev)))
-    # ws and the staged copies were allocated for torch's current stream, the one the kernels
-    # were enqueued on, so the caching allocator already orders their reuse after the kernels.
-    result = out.reshape(*x.shape[:-1], n_out)
-    return (result, aux) if return_aux else result
+    plan = ForwardPlan(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices,
+                       rms_gamma=rms_gamma, eps=eps, residual=residual, swiglu=swiglu, flags=flags,
+                       return_aux=return_aux, entry=entry)
+    result = plan.run()
+    # Everything the kernels touch was allocated for torch's current stream, the one they were
+    # enqueued on, so the caching allocator orders any reuse after them.
+    return (result, plan.aux) if return_aux else result
 
 
 def _check_enabled(enabled, interpret, what: str) -> None:
@@ -364,6 +401,6 @@ def w8a8_lora_residual(x, weight, lora_a, lora_b, lora_scaling, residual, *, ena
 __all__ = (
     "DEFAULT_BLOCK_M", "DEFAULT_BLOCK_N", "DEFAULT_ROW_SUPERBLOCK", "MAX_BLOCK_M", "MAX_BLOCK_N",
     "MAX_IN_FEATURES", "MAX_OUT_FEATURES", "MAX_ROW_SUPERBLOCK", "MAX_LORA_RANK", "PackedW8Weight",
-    "prepare_weight", "unpack_weight", "dynamic_quantize_rows", "forward", "w8a8_frozen_linear",
+    "prepare_weight", "unpack_weight", "dynamic_quantize_rows", "ForwardPlan", "forward", "w8a8_frozen_linear",
     "w8a8_lora_linear", "w8a8_rms_gate_up_lora_swiglu", "w8a8_lora_residual",
 )
