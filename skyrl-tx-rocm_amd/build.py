@@ -34,6 +34,41 @@ def find_hipcc() -> str:
     raise RuntimeError("hipcc not found; a ROCm toolchain is required to build the gfx950 library")
 
 
+def jaxlib_include_dir() -> Path | None:
+    """Directory holding xla/ffi/api/ffi.h (ships inside jaxlib), or None."""
+    env = os.environ.get("JAXLIB_INCLUDE_DIR")
+    if env and (Path(env) / "xla" / "ffi" / "api" / "ffi.h").exists():
+        return Path(env)
+    try:
+        import importlib.util
+
+        spec = importlib.util.find_spec("jaxlib")
+    except (ImportError, ValueError):
+        spec = None
+    if spec and spec.submodule_search_locations:
+        cand = Path(list(spec.submodule_search_locations)[0]) / "include"
+        if (cand / "xla" / "ffi" / "api" / "ffi.h").exists():
+            return cand
+    return None
+
+
+def build_ffi(verbose: bool = False) -> Path | None:
+    """Build the XLA typed-FFI shim next to the C ABI library where jaxlib's headers exist."""
+    inc = jaxlib_include_dir()
+    if inc is None:
+        return None
+    out = LIB_DIR / "libmi355_w8a8_ffi.so"
+    cmd = [find_hipcc(), "-x", "hip", "--offload-arch=gfx950", "-O2", "-std=c++17", "-fPIC", "-shared",
+           "-isystem", str(inc), str(CSRC / "w8a8_xla_ffi.cc"), f"-L{LIB_DIR}", "-lmi355_w8a8",
+           "-Wl,-rpath,$ORIGIN", "-Wl,-z,defs", "-o", str(out)]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed on the FFI shim ({proc.returncode}):\n{proc.stderr}")
+    if verbose and proc.stderr.strip():
+        print(proc.stderr, file=sys.stderr)
+    return out
+
+
 def build(verbose: bool = False) -> Path:
     LIB_DIR.mkdir(parents=True, exist_ok=True)
     tmp = LIB_DIR / "libmi355_w8a8.so.tmp"
@@ -46,6 +81,7 @@ def build(verbose: bool = False) -> Path:
     if verbose and err.strip():
         print(err, file=sys.stderr)
     os.replace(tmp, LIB_PATH)
+    build_ffi(verbose)
     return LIB_PATH
 
 

@@ -119,6 +119,62 @@ int validate_common(uint32_t m, uint32_t k, uint32_t n) {
   return MI355_W8A8_OK;
 }
 
+// Skinny-M path: quantize -> stream (weight + LoRA-A units) -> epilogue.
+int launch_skinny(const mi355_w8a8_problem* p, unsigned char* xq, float* sx, uint16_t* xn, unsigned char* sws,
+                  uint32_t K_pad, uint32_t KB, hipStream_t s) {
+  const bool rms = p->rms_gamma != nullptr;
+  const bool lora = p->n_adapters > 0;
+  const SkinnyLayout L = skinny_layout(p->m, p->k, p->n);
+  int st;
+  if (!(p->flags & MI355_W8A8_FLAG_SKIP_PROLOGUE)) {
+    SkinnyQuantArgs q{};
+    q.x = static_cast<const uint16_t*>(p->x);
+    q.gamma = p->rms_gamma;
+    q.eps = p->rms_eps;
+    q.M = p->m; q.K = p->k; q.K_pad = K_pad; q.KB = KB;
+    q.xq = xq; q.sx = sx;
+    q.codes_rm = p->aux_x_codes; q.scales_rm = p->aux_x_scales;
+    q.xn = (rms && lora) ? xn : nullptr;
+    q.xn_aux = static_cast<uint16_t*>(p->aux_normalized);
+    // without RMSNorm the LoRA-A units depend on x only and ride along with the quantizer
+    q.lora_a = static_cast<const uint16_t*>(p->lora_a);
+    q.idx = p->adapter_indices;
+    q.z_part = reinterpret_cast<float*>(sws + L.z_part);
+    q.n_adapters = p->n_adapters; q.r = p->rank; q.z_chunks = L.z_chunks; q.z_chunk_k = L.z_chunk_k;
+    q.n_z_units = (lora && !rms) ? p->m * L.z_chunks : 0u;
+    if (rms) hipLaunchKernelGGL((skinny_quant_kernel<true>), dim3(p->m), dim3(1024), 0, s, q);
+    else hipLaunchKernelGGL((skinny_quant_kernel<false>), dim3(p->m + q.n_z_units), dim3(1024), 0, s, q);
+    if ((st = launch_status())) return st;
+  }
+  if (p->flags & MI355_W8A8_FLAG_SKIP_GEMM) return MI355_W8A8_OK;
+  SkinnyStreamArgs a{};
+  a.xq = xq;
+  a.wp = static_cast<const unsigned char*>(p->w_packed);
+  a.acc_part = reinterpret_cast<int32_t*>(sws + L.acc_part);
+  a.xsrc = rms ? xn : static_cast<const uint16_t*>(p->x);
+  a.lora_a = static_cast<const uint16_t*>(p->lora_a);
+  a.idx = p->adapter_indices;
+  a.z_part = reinterpret_cast<float*>(sws + L.z_part);
+  a.M = p->m; a.K = p->k; a.KB = KB; a.NB = n_padded(p->n) / 32u;
+  a.ksplit = L.ksplit; a.kb_per_wave = L.kb_per_wave;
+  a.n_adapters = p->n_adapters; a.r = p->rank;
+  a.z_chunks = L.z_chunks; a.z_chunk_k = L.z_chunk_k;
+  a.n_z_units = (lora && rms) ? p->m * L.z_chunks : 0u;
+  hipLaunchKernelGGL(skinny_stream_kernel, dim3(a.n_z_units + a.NB * a.ksplit), dim3(256), 0, s, a);
+  if ((st = launch_status())) return st;
+  SkinnyEpilogueArgs e{};
+  e.acc_part = a.acc_part; e.z_part = a.z_part; e.sx = sx; e.sw = p->w_scales;
+  e.lora_b = lora ? static_cast<const uint16_t*>(p->lora_b) : nullptr;
+  e.lora_scaling = p->lora_scaling; e.idx = p->adapter_indices;
+  e.residual = static_cast<const uint16_t*>(p->residual);
+  e.out = static_cast<uint16_t*>(p->out);
+  e.aux_acc = p->aux_acc;
+  e.M = p->m; e.N = p->n; e.NB = a.NB; e.ksplit = L.ksplit;
+  e.n_adapters = p->n_adapters; e.r = p->rank; e.z_chunks = L.z_chunks;
+  hipLaunchKernelGGL(skinny_epilogue_kernel, dim3((p->n + 255u) / 256u, p->m), dim3(256), 0, s, e);
+  return launch_status();
+}
+
 enum Required { kReqNone = 0, kReqLinear = 1, kReqGateUp = 2, kReqResidual = 3 };
 
 int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {

@@ -1,0 +1,156 @@
+// XLA typed-FFI handlers over the plain C ABI (include/mi355_w8a8.h).
+//
+// Built only where jaxlib's headers exist (xla/ffi/api/ffi.h ships inside jaxlib/include);
+// the build script skips this file otherwise.  Handler shape follows the reference's
+// skyrl/tx/kernels/rocm/ffi/gdn_ffi_smoke.hip:43-82 and its W8A8 design note
+// rocm/QUANTIZED_FFI.md:589-614: typed buffers in, result buffers out (the workspace is an
+// explicit result so XLA owns its stream-ordered lifetime), the platform stream from the call
+// context, validation -> InvalidArgument, launch failure -> Internal, no synchronisation.
+#if __has_include("xla/ffi/api/ffi.h")
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "../../include/mi355_w8a8.h"
+#include "xla/ffi/api/ffi.h"
+
+namespace ffi = xla::ffi;
+
+namespace {
+
+ffi::Error ToError(int status, const char* what) {
+  if (status == MI355_W8A8_OK) return ffi::Error::Success();
+  if (status == MI355_W8A8_ERR_LAUNCH) return ffi::Error::Internal(what);
+  return ffi::Error::InvalidArgument(mi355_w8a8_status_string(status));
+}
+
+bool RowsAndK(ffi::Span<const int64_t> dims, uint32_t* m, uint32_t* k) {
+  if (dims.size() < 2) return false;
+  int64_t rows = 1;
+  for (size_t i = 0; i + 1 < dims.size(); ++i) rows *= dims[i];
+  if (rows <= 0 || rows > (1 << 20) || dims.back() <= 0 || dims.back() > 16384) return false;
+  *m = static_cast<uint32_t>(rows);
+  *k = static_cast<uint32_t>(dims.back());
+  return true;
+}
+
+// x [.., K] bf16, packed weight u8 [bytes], scales f32 [N], A bf16 [n, K, r], B bf16 [n, r, N],
+// scaling f32 [n], adapter index s32 [M]; optional stage inputs are passed as size-0 buffers
+// when unused.  Results: y bf16 [.., n_out], workspace u8 [mi355_w8a8_workspace_bytes].
+ffi::Error Forward(hipStream_t stream, ffi::Buffer<ffi::BF16> x, ffi::Buffer<ffi::U8> w_packed,
+                   ffi::Buffer<ffi::F32> w_scales, ffi::Buffer<ffi::BF16> lora_a,
+                   ffi::Buffer<ffi::BF16> lora_b, ffi::Buffer<ffi::F32> lora_scaling,
+                   ffi::Buffer<ffi::S32> adapter_indices, ffi::Buffer<ffi::F32> rms_gamma,
+                   ffi::Buffer<ffi::BF16> residual, ffi::ResultBuffer<ffi::BF16> y,
+                   ffi::ResultBuffer<ffi::U8> workspace, int32_t swiglu, float rms_eps, int32_t entry) {
+  mi355_w8a8_problem p{};
+  p.struct_size = sizeof(p);
+  if (!RowsAndK(x.dimensions(), &p.m, &p.k))
+    return ffi::Error::InvalidArgument("x must be bf16 [..., K] with a non-empty row domain");
+  if (w_scales.dimensions().size() != 1) return ffi::Error::InvalidArgument("w_scales must be f32 [N]");
+  p.n = static_cast<uint32_t>(w_scales.dimensions()[0]);
+  if (w_packed.size_bytes() != mi355_w8a8_packed_weight_bytes(p.k, p.n))
+    return ffi::Error::InvalidArgument("packed weight size does not match (K, N)");
+  const bool lora = lora_a.element_count() > 0;
+  if (lora) {
+    auto da = lora_a.dimensions();
+    auto db = lora_b.dimensions();
+    if (da.size() != 3 || db.size() != 3 || da[1] != p.k || db[0] != da[0] || db[1] != da[2] ||
+        db[2] != p.n || lora_scaling.element_count() != static_cast<size_t>(da[0]))
+      return ffi::Error::InvalidArgument("LoRA A/B/scaling must be [n,K,r], [n,r,N], [n]");
+    p.n_adapters = static_cast<uint32_t>(da[0]);
+    p.rank = static_cast<uint32_t>(da[2]);
+    p.lora_a = lora_a.untyped_data();
+    p.lora_b = lora_b.untyped_data();
+    p.lora_scaling = lora_scaling.typed_data();
+    if (adapter_indices.element_count() > 0) {
+      if (adapter_indices.element_count() != p.m)
+        return ffi::Error::InvalidArgument("adapter_indices must hold one entry per row");
+      p.adapter_indices = adapter_indices.typed_data();
+    }
+  }
+  if (rms_gamma.element_count() > 0) {
+    if (rms_gamma.element_count() != p.k) return ffi::Error::InvalidArgument("rms_gamma must be f32 [K]");
+    p.rms_gamma = rms_gamma.typed_data();
+    p.rms_eps = rms_eps;
+  }
+  const uint32_t n_out = swiglu ? p.n / 2 : p.n;
+  if (y->element_count() != static_cast<size_t>(p.m) * n_out)
+    return ffi::Error::InvalidArgument("result must be bf16 [..., n_out]");
+  if (residual.element_count() > 0) {
+    if (residual.element_count() != y->element_count())
+      return ffi::Error::InvalidArgument("residual must match the result shape");
+    p.residual = residual.untyped_data();
+  }
+  p.flags = swiglu ? MI355_W8A8_FLAG_SWIGLU : 0u;
+  p.x = x.untyped_data();
+  p.w_packed = w_packed.untyped_data();
+  p.w_scales = w_scales.typed_data();
+  p.out = y->untyped_data();
+  p.workspace = workspace->untyped_data();
+  p.workspace_bytes = workspace->size_bytes();
+  int status;
+  switch (entry) {
+    case 1: status = mi355_w8a8_lora_linear_v1(&p, stream); break;
+    case 2: status = mi355_w8a8_rms_gateup_swiglu_v1(&p, stream); break;
+    case 3: status = mi355_w8a8_lora_residual_v1(&p, stream); break;
+    default: status = mi355_w8a8_forward_v1(&p, stream); break;
+  }
+  return ToError(status, "mi355_w8a8 forward launch submission failed");
+}
+
+ffi::Error QuantizeRows(hipStream_t stream, ffi::Buffer<ffi::BF16> x, ffi::ResultBuffer<ffi::S8> codes,
+                        ffi::ResultBuffer<ffi::F32> scales) {
+  uint32_t m = 0, k = 0;
+  if (!RowsAndK(x.dimensions(), &m, &k))
+    return ffi::Error::InvalidArgument("x must be bf16 [..., K] with a non-empty row domain");
+  if (codes->element_count() != x.element_count() || scales->element_count() != m)
+    return ffi::Error::InvalidArgument("codes must match x and scales must hold one value per row");
+  return ToError(mi355_w8a8_quantize_rows_v1(x.untyped_data(), codes->typed_data(), scales->typed_data(), m, k,
+                                             stream),
+                 "mi355_w8a8 quantize launch submission failed");
+}
+
+ffi::Error PackWeight(hipStream_t stream, ffi::Buffer<ffi::S8> codes, ffi::ResultBuffer<ffi::U8> packed) {
+  auto d = codes.dimensions();
+  if (d.size() != 2 || d[0] <= 0 || d[1] <= 0) return ffi::Error::InvalidArgument("codes must be s8 [K, N]");
+  const uint32_t k = static_cast<uint32_t>(d[0]), n = static_cast<uint32_t>(d[1]);
+  if (packed->size_bytes() != mi355_w8a8_packed_weight_bytes(k, n))
+    return ffi::Error::InvalidArgument("packed buffer size does not match (K, N)");
+  return ToError(mi355_w8a8_pack_weight_v1(codes.typed_data(), packed->untyped_data(), k, n, stream),
+                 "mi355_w8a8 pack launch submission failed");
+}
+
+}  // namespace
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_forward_v1, Forward,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::U8>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::U8>>()
+                                  .Attr<int32_t>("swiglu")
+                                  .Attr<float>("rms_eps")
+                                  .Attr<int32_t>("entry"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_quantize_rows_v1, QuantizeRows,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::S8>>()
+                                  .Ret<ffi::Buffer<ffi::F32>>());
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_pack_weight_v1, PackWeight,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::Buffer<ffi::S8>>()
+                                  .Ret<ffi::Buffer<ffi::U8>>());
+#endif  // __has_include("xla/ffi/api/ffi.h")

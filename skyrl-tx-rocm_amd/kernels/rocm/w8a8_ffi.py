@@ -1,0 +1,136 @@
+"""jax.ffi registration and call wrappers for the W8A8 kernels (XLA typed FFI).
+
+The JAX side of the drop-in: the same function names as the torch host mirror in
+``w8a8_lora.py`` but taking/returning ``jax.Array``.  Registration follows the
+reference's ``skyrl/tx/kernels/rocm/gdn_ffi_smoke.py:281-353``: ``ctypes.CDLL`` on the
+shim library, ``handler.restype = c_void_p``, ``jax.ffi.pycapsule``,
+``jax.ffi.register_ffi_target(name, capsule, platform="ROCM", api_version=1)``, the
+library kept alive for the life of the process, one registration per process under a
+lock.  Calls use ``jax.ffi.ffi_call(..., vmap_method="sequential",
+custom_call_api_version=4)`` with row-major layouts (gdn_ffi_smoke.py:401-414).
+
+JAX and jaxlib are imported lazily: this module imports everywhere, the functions
+raise ``RuntimeError`` where JAX or the shim library (``libmi355_w8a8_ffi.so``, built
+only where jaxlib's headers exist) is missing.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import threading
+from pathlib import Path
+
+from ... import _native
+
+FFI_LIB_PATH = Path(_native.LIB_PATH).with_name("libmi355_w8a8_ffi.so")
+TARGETS = ("mi355_w8a8_ffi_forward_v1", "mi355_w8a8_ffi_quantize_rows_v1", "mi355_w8a8_ffi_pack_weight_v1")
+_ROCM_PLATFORM = "ROCM"
+_REGISTRATION_API_VERSION = 1
+_CUSTOM_CALL_API_VERSION = 4
+
+_lock = threading.Lock()
+_registered = False
+_lifetime_handles: list = []
+
+
+def _import_jax():
+    try:
+        import jax  # noqa: PLC0415
+    except ImportError as error:  # pragma: no cover - depends on the environment
+        raise RuntimeError("the XLA FFI route needs jax/jaxlib, which is not installed") from error
+    return jax
+
+
+def _load_cdll(path: Path):
+    return ctypes.CDLL(str(path), mode=ctypes.RTLD_LOCAL)
+
+
+def register(jax_module=None) -> tuple[str, ...]:
+    """Register the FFI targets once per process; returns the target names."""
+    global _registered
+    jax = jax_module or _import_jax()
+    ffi = getattr(jax, "ffi", None)
+    if ffi is None or not all(callable(getattr(ffi, n, None)) for n in ("pycapsule", "register_ffi_target", "ffi_call")):
+        raise RuntimeError("installed JAX does not expose the required typed-FFI API")
+    with _lock:
+        if _registered:
+            return TARGETS
+        if not FFI_LIB_PATH.exists():
+            raise RuntimeError(f"{FFI_LIB_PATH} is missing: build it where jaxlib's xla/ffi headers are installed")
+        # the C ABI library must be resident first: the shim links against it
+        _lifetime_handles.append(ctypes.CDLL(str(_native.LIB_PATH), mode=ctypes.RTLD_GLOBAL))
+        library = _load_cdll(FFI_LIB_PATH)
+        _lifetime_handles.append(library)  # a capsule is a bare function pointer: never unload
+        for name in TARGETS:
+            try:
+                handler = getattr(library, name)
+            except AttributeError as error:
+                raise RuntimeError(f"FFI library is missing its handler symbol {name}") from error
+            handler.restype = ctypes.c_void_p
+            handler.argtypes = (ctypes.c_void_p,)
+            ffi.register_ffi_target(name, ffi.pycapsule(handler), platform=_ROCM_PLATFORM,
+                                    api_version=_REGISTRATION_API_VERSION)
+        _registered = True
+        return TARGETS
+
+
+def _row_major(ndim: int) -> tuple[int, ...]:
+    return tuple(range(ndim - 1, -1, -1))
+
+
+def _call(jax, name, result_specs, *operands, **attrs):
+    call = jax.ffi.ffi_call(
+        name, result_specs, has_side_effect=False, vmap_method="sequential",
+        input_layouts=tuple(_row_major(o.ndim) for o in operands),
+        output_layouts=tuple(_row_major(len(s.shape)) for s in result_specs),
+        input_output_aliases=None, custom_call_api_version=_CUSTOM_CALL_API_VERSION)
+    return call(*operands, **attrs)
+
+
+def pack_weight(codes):
+    """int8 [K, N] codes -> opaque uint8 packed weight (run once per weight, not per forward)."""
+    jax = _import_jax()
+    register(jax)
+    jnp = jax.numpy
+    k, n = codes.shape
+    nbytes = int(_native.load().mi355_w8a8_packed_weight_bytes(k, n))
+    (packed,) = _call(jax, TARGETS[2], (jax.ShapeDtypeStruct((nbytes,), jnp.uint8),), codes)
+    return packed
+
+
+def quantize_rows(x):
+    jax = _import_jax()
+    register(jax)
+    jnp = jax.numpy
+    return _call(jax, TARGETS[1], (jax.ShapeDtypeStruct(x.shape, jnp.int8),
+                                   jax.ShapeDtypeStruct(x.shape[:-1], jnp.float32)), x)
+
+
+def forward(x, packed_weight, w_scales, lora_a=None, lora_b=None, lora_scaling=None, adapter_indices=None,
+            rms_gamma=None, residual=None, *, swiglu: bool = False, eps: float = 1e-6, entry: int = 0):
+    """W8A8 (+LoRA, +RMSNorm, +SwiGLU, +residual) forward as one XLA custom call."""
+    jax = _import_jax()
+    register(jax)
+    jnp = jax.numpy
+    k = x.shape[-1]
+    n = w_scales.shape[-1]
+    m = 1
+    for d in x.shape[:-1]:
+        m *= d
+    empty = lambda dt, nd: jnp.zeros((0,) * nd, dt)
+    a3 = empty(jnp.bfloat16, 3) if lora_a is None else (lora_a if lora_a.ndim == 3 else lora_a[None])
+    b3 = empty(jnp.bfloat16, 3) if lora_b is None else (lora_b if lora_b.ndim == 3 else lora_b[None])
+    n_ad = a3.shape[0]
+    s1 = empty(jnp.float32, 1) if lora_a is None else jnp.broadcast_to(jnp.asarray(lora_scaling, jnp.float32), (n_ad,))
+    idx = empty(jnp.int32, 1) if adapter_indices is None else adapter_indices.astype(jnp.int32).reshape(-1)
+    gamma = empty(jnp.float32, 1) if rms_gamma is None else rms_gamma.astype(jnp.float32)
+    res = empty(jnp.bfloat16, 2) if residual is None else residual.reshape(m, -1)
+    n_out = n // 2 if swiglu else n
+    ws = int(_native.load().mi355_w8a8_workspace_bytes(m, k, n, n_ad, a3.shape[2] if n_ad else 0, 1 if swiglu else 0))
+    if ws == 0:
+        raise ValueError(f"geometry M={m}, K={k}, N={n} is outside the native path")
+    y, _ = _call(jax, TARGETS[0],
+                 (jax.ShapeDtypeStruct((*x.shape[:-1], n_out), jnp.bfloat16), jax.ShapeDtypeStruct((ws,), jnp.uint8)),
+                 x, packed_weight, w_scales.reshape(n).astype(jnp.float32), a3, b3, s1, idx, gamma, res,
+                 swiglu=int(swiglu), rms_eps=float(eps), entry=int(entry))
+    return y

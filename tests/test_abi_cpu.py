@@ -1,0 +1,144 @@
+"""CPU-only checks of the C ABI: the library loads, exports every symbol the header
+declares, and rejects invalid requests before touching a GPU."""
+
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+from __graft_entry__ import load_package
+
+ROOT = Path(__file__).resolve().parents[1]
+HEADER = ROOT / "include" / "mi355_w8a8.h"
+
+
+@pytest.fixture(scope="module")
+def native():
+    pkg = load_package()
+    if not pkg._native.LIB_PATH.exists():
+        pytest.skip("libmi355_w8a8.so not built (run __graft_entry__.build())")
+    return pkg._native
+
+
+def _declared_functions():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(mi355_w8a8_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(native):
+    lib = native.load()
+    declared = _declared_functions()
+    assert len(declared) >= 13
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert sorted(native.EXPORTS) == declared
+    assert lib.mi355_w8a8_abi_version() == 1
+    assert lib.mi355_w8a8_status_string(0) == b"ok"
+    assert b"workspace" in lib.mi355_w8a8_status_string(-5)
+
+
+def test_struct_sizes_match_header_layout(native):
+    # 8 x 4-byte scalars, 11 pointers, u64, 4 pointers
+    assert ctypes.sizeof(native.Problem) == 8 * 4 + 11 * 8 + 8 + 4 * 8
+    assert ctypes.sizeof(native.GroupedProblem) == 8 * 4 + 9 * 8 + 8 + 3 * 8
+
+
+def test_size_queries(native):
+    lib = native.load()
+    assert lib.mi355_w8a8_packed_weight_bytes(0, 5) == 0
+    assert lib.mi355_w8a8_packed_weight_bytes(64, 17) == 128 * 256
+    assert lib.mi355_w8a8_packed_weight_bytes(4096, 24576) == 4096 * 24576
+    ws = lib.mi355_w8a8_workspace_bytes(4096, 4096, 24576, 8, 32, 0)
+    assert ws >= 4096 * 4096 and ws % 256 == 0
+    assert lib.mi355_w8a8_workspace_bytes(16, 12288, 4096, 16, 32, 0) > 0
+    assert lib.mi355_w8a8_workspace_bytes(0, 64, 64, 0, 0, 0) == 0          # no rows
+    assert lib.mi355_w8a8_workspace_bytes(8, 60, 64, 0, 0, 0) == 0          # K not a multiple of 8
+    assert lib.mi355_w8a8_workspace_bytes(8, 32768, 64, 0, 0, 0) == 0       # K too large
+    assert lib.mi355_w8a8_workspace_bytes(8, 64, 64, 65, 8, 0) == 0         # too many adapters
+    assert lib.mi355_w8a8_workspace_bytes(8, 64, 64, 2, 65, 0) == 0         # rank too large
+
+
+def _problem(native, **kw):
+    p = native.Problem()
+    p.struct_size = ctypes.sizeof(native.Problem)
+    p.m, p.k, p.n = 8, 64, 32
+    fake = 0x10000  # never dereferenced: validation fails first
+    p.x, p.w_packed, p.w_scales, p.out, p.workspace = fake, fake + 0x100000, fake + 0x200000, fake + 0x300000, fake + 0x400000
+    p.workspace_bytes = 1 << 30
+    for k, v in kw.items():
+        setattr(p, k, v)
+    return p
+
+
+def test_validation_errors_without_a_gpu(native):
+    lib = native.load()
+    call = lambda p, fn=lib.mi355_w8a8_forward_v1: fn(ctypes.byref(p), None)
+    assert lib.mi355_w8a8_forward_v1(None, None) == -1
+    assert call(_problem(native, struct_size=12)) == -8
+    assert call(_problem(native, m=0)) == -2
+    assert call(_problem(native, k=60)) == -7
+    assert call(_problem(native, x=None)) == -1
+    assert call(_problem(native, out=None)) == -1
+    assert call(_problem(native, x=0x10008)) == -3                       # misaligned
+    assert call(_problem(native, out=0x10000)) == -4                     # output aliases x
+    assert call(_problem(native, workspace=None)) == -5
+    assert call(_problem(native, workspace_bytes=16)) == -5
+    assert call(_problem(native, n_adapters=1, rank=8)) == -1            # LoRA pointers missing
+    assert call(_problem(native, adapter_indices=0x500000)) == -2        # indices without LoRA
+    assert call(_problem(native, flags=native.FLAG_SWIGLU, n=31)) == -2
+    assert call(_problem(native, flags=native.FLAG_FORCE_TILED | native.FLAG_FORCE_SKINNY)) == -2
+    # entry points insist on their own stage combination
+    assert call(_problem(native), lib.mi355_w8a8_rms_gateup_swiglu_v1) == -2
+    assert call(_problem(native), lib.mi355_w8a8_lora_residual_v1) == -2
+    assert call(_problem(native, rms_gamma=0x600000), lib.mi355_w8a8_lora_linear_v1) == -2
+    assert lib.mi355_w8a8_quantize_rows_v1(None, None, None, 4, 64, None) == -1
+    assert lib.mi355_w8a8_quantize_rows_v1(0x10000, 0x20000, 0x30000, 4, 60, None) == -7
+    assert lib.mi355_w8a8_pack_weight_v1(None, 0x10000, 64, 32, None) == -1
+    assert lib.mi355_w8a8_pack_weight_v1(0x10000, 0x10010, 64, 32, None) == -4
+
+
+def test_python_surface_fails_loudly_on_cpu(native):
+    """There is no CPU fallback: CPU tensors are refused, as is a missing opt-in."""
+    import torch
+
+    pkg = load_package()
+    w8, ql = pkg.w8a8_lora, pkg.quantized_lora
+    w = ql.quantize_frozen_weight(torch.randn(64, 16), bits=8, group_size=64)
+    assert w.codes.dtype == torch.int8 and w.scales.dtype == torch.bfloat16 and tuple(w.scales.shape) == (1, 16)
+    deq = ql.dequantize_frozen_weight(w)
+    assert deq.shape == (64, 16)
+    x = torch.zeros(2, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="disabled by default"):
+        w8.w8a8_frozen_linear(x, w)
+    with pytest.raises(RuntimeError, match="GPU"):
+        w8.w8a8_frozen_linear(x, w, enabled=True)
+    with pytest.raises(TypeError, match="exact bool"):
+        w8.w8a8_frozen_linear(x, w, enabled="yes")
+    with pytest.raises(RuntimeError, match="interpret"):
+        w8.w8a8_frozen_linear(x, w, enabled=True, interpret=True)
+    w64 = ql.quantize_frozen_weight(torch.randn(128, 16), bits=8, group_size=64)
+    with pytest.raises(ValueError, match="per-channel"):
+        w8.prepare_weight(w64)
+    with pytest.raises(ValueError, match="W8A8 only"):
+        ql.quantized_lora_linear(x, ql.quantize_frozen_weight(torch.randn(64, 16), bits=4, group_size=64),
+                                 torch.zeros(64, 4), torch.zeros(4, 16), 1.0)
+
+
+def test_host_quantizer_matches_oracle():
+    import numpy as np
+    import torch
+
+    from oracle import w8a8_oracle as o
+
+    pkg = load_package()
+    rng = np.random.default_rng(3)
+    wd = rng.standard_normal((70, 13)).astype(np.float32)
+    for bits, g in ((8, 10), (4, 14), (8, 70)):
+        got = pkg.quantized_lora.quantize_frozen_weight(torch.from_numpy(wd), bits=bits, group_size=g,
+                                                        scale_dtype=torch.float32)
+        want = o.quantize_frozen_weight(wd, bits=bits, group_size=g, scale_dtype="f32")
+        np.testing.assert_array_equal(got.codes.numpy(), want.codes)
+        np.testing.assert_array_equal(got.scales.numpy(), want.scales)
+        np.testing.assert_array_equal(pkg.quantized_lora.dequantize_frozen_weight(got).numpy(),
+                                      o.dequantize_frozen_weight(want))

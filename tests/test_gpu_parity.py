@@ -172,13 +172,33 @@ def test_swiglu_pairing_closed_form(dev):
     assert np.all(got == F32(1.9296875))
 
 
-def test_down_residual_decode_shape(dev):
-    """Config 3: M16 K12288 N4096, 16 rank-32 adapters (one per row), residual."""
+@pytest.mark.parametrize("path", ["skinny", "tiled"])
+def test_down_residual_decode_shape(dev, pkg, path):
+    """Config 3: M16 K12288 N4096, 16 rank-32 adapters (one per row), residual; both kernels."""
+    flags = pkg._native.FLAG_FORCE_SKINNY if path == "skinny" else pkg._native.FLAG_FORCE_TILED
     case = wc.make_case(16, 12288, 4096, n_adapters=16, rank=32, seed=7, residual=True, idx_mode="arange")
     st = wc.oracle_forward(case, return_stages=True)
-    got, aux = wc.gpu_forward(case)
+    got, aux = wc.gpu_forward(case, flags=flags)
     _assert_integer_stages(aux, st)
-    _assert_close(got, st["out"], " cfg3")
+    _assert_close(got, st["out"], f" cfg3 {path}")
+
+
+@pytest.mark.parametrize("m,k,n,n_ad,rank,rms", [(1, 64, 17, 1, 8, False), (32, 2560, 6144, 4, 64, False),
+                                                 (7, 1024, 520, 3, 24, True), (20, 4096, 2560, 0, 0, True),
+                                                 (31, 384, 96, 2, 5, False)])
+def test_skinny_path_shapes(dev, pkg, m, k, n, n_ad, rank, rms):
+    """The split-K streaming kernel on ragged shapes, ranks and with the RMSNorm prologue."""
+    case = wc.make_case(m, k, n, n_adapters=n_ad, rank=max(rank, 1), seed=m + k, rms=rms, residual=(m % 2 == 0))
+    if n_ad:
+        case["s"] = np.linspace(0.5, 2.0, n_ad).astype(F32)
+    st = wc.oracle_forward(case, return_stages=True)
+    got, aux = wc.gpu_forward(case, flags=pkg._native.FLAG_FORCE_SKINNY)
+    if rms:
+        np.testing.assert_array_equal(o.bf16_bits(aux["normalized"]), o.bf16_bits(st["normalized"]))
+    _assert_integer_stages(aux, st)
+    _assert_close(got, st["out"], f" skinny {m}x{k}x{n}")
+    tiled, _ = wc.gpu_forward(case, flags=pkg._native.FLAG_FORCE_TILED)
+    _assert_close(tiled, st["out"], f" tiled {m}x{k}x{n}")
 
 
 @pytest.mark.parametrize("m", [1, 64, 512])
