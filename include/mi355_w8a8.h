@@ -104,10 +104,11 @@ typedef struct mi355_w8a8_grouped_problem {
   uint32_t n;
   uint32_t n_groups;
   uint32_t rank;            /* 0 = no LoRA */
-  uint32_t reserved;
+  uint32_t groups_per_weight; /* weight / scale index = group / groups_per_weight (0 or 1: one per group) */
   const void* x;            /* bf16 [m, k] */
-  const void* w_packed;     /* n_groups packed weights back to back, each mi355_w8a8_packed_weight_bytes(k, n) */
-  const float* w_scales;    /* f32 [n_groups, n] */
+  const void* w_packed;     /* n_groups / groups_per_weight packed weights back to back, each
+                               mi355_w8a8_packed_weight_bytes(k, n) */
+  const float* w_scales;    /* f32 [n_groups / groups_per_weight, n] */
   const void* lora_a;       /* bf16 [n_groups, k, rank] or NULL */
   const void* lora_b;       /* bf16 [n_groups, rank, n] or NULL */
   const float* lora_scaling;/* f32 [n_groups] or NULL */
@@ -117,7 +118,7 @@ typedef struct mi355_w8a8_grouped_problem {
   uint64_t workspace_bytes;
   int8_t* aux_x_codes;
   float* aux_x_scales;
-  int32_t* aux_acc;
+  int32_t* aux_acc;         /* int32 [m, n]; rows beyond sum(group_sizes) are not written */
 } mi355_w8a8_grouped_problem;
 
 int mi355_w8a8_abi_version(void);

@@ -54,7 +54,7 @@ class GroupedProblem(ctypes.Structure):
 
     _fields_ = [
         ("struct_size", _u32), ("flags", _u32), ("m", _u32), ("k", _u32), ("n", _u32),
-        ("n_groups", _u32), ("rank", _u32), ("reserved", _u32),
+        ("n_groups", _u32), ("rank", _u32), ("groups_per_weight", _u32),
         ("x", _vp), ("w_packed", _vp), ("w_scales", _vp), ("lora_a", _vp), ("lora_b", _vp),
         ("lora_scaling", _vp), ("group_sizes", _vp), ("out", _vp), ("workspace", _vp),
         ("workspace_bytes", _u64), ("aux_x_codes", _vp), ("aux_x_scales", _vp), ("aux_acc", _vp),

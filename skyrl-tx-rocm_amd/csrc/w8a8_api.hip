@@ -75,37 +75,38 @@ int launch_quant(const QuantArgs& a, hipStream_t s) {
   return MI355_W8A8_ERR_UNSUPPORTED;
 }
 
-template <int EPI, int NKK>
+template <int EPI, int NKK, bool GROUPED>
 int launch_gemm_one(const GemmArgs& g, hipStream_t s) {
   const uint32_t ntile = g.tiles_m * g.tiles_n;
   const dim3 grid(((ntile + 7u) / 8u) * 8u), block(256);
+  constexpr uint32_t lds_bytes = GROUPED ? kGroupedLdsBytes : kGemmLdsBytes;
 #ifdef W8A8_DEBUG_VARIANTS
-  if constexpr (EPI == kEpiSwiglu && NKK == 2) {
+  if constexpr (EPI == kEpiSwiglu && NKK == 2 && !GROUPED) {
 #define W8A8_DBG(D)                                                                              \
   if (g.map_mode == 100 + D) {                                                                   \
-    hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm_kernel<EPI, NKK, D>),          \
-                        hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes);              \
-    hipLaunchKernelGGL((w8a8_gemm_kernel<EPI, NKK, D>), grid, block, kGemmLdsBytes, s, g);       \
+    hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm_kernel<EPI, NKK, D, false>),   \
+                        hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);                  \
+    hipLaunchKernelGGL((w8a8_gemm_kernel<EPI, NKK, D, false>), grid, block, lds_bytes, s, g);    \
     return launch_status();                                                                      \
   }
     W8A8_DBG(1) W8A8_DBG(2) W8A8_DBG(3) W8A8_DBG(4)
 #undef W8A8_DBG
   }
 #endif
-  if (hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm_kernel<EPI, NKK>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes) != hipSuccess)
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm_kernel<EPI, NKK, 0, GROUPED>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
     return MI355_W8A8_ERR_LAUNCH;
-  hipLaunchKernelGGL((w8a8_gemm_kernel<EPI, NKK>), grid, block, kGemmLdsBytes, s, g);
+  hipLaunchKernelGGL((w8a8_gemm_kernel<EPI, NKK, 0, GROUPED>), grid, block, lds_bytes, s, g);
   return launch_status();
 }
 
-template <int EPI>
+template <int EPI, bool GROUPED = false>
 int launch_gemm(const GemmArgs& g, uint32_t nkk, hipStream_t s) {
   switch (nkk) {
-    case 0: return launch_gemm_one<EPI, 0>(g, s);
-    case 1: return launch_gemm_one<EPI, 1>(g, s);
-    case 2: return launch_gemm_one<EPI, 2>(g, s);
-    case 4: return launch_gemm_one<EPI, 4>(g, s);
+    case 0: return launch_gemm_one<EPI, 0, GROUPED>(g, s);
+    case 1: return launch_gemm_one<EPI, 1, GROUPED>(g, s);
+    case 2: return launch_gemm_one<EPI, 2, GROUPED>(g, s);
+    case 4: return launch_gemm_one<EPI, 4, GROUPED>(g, s);
     default: return MI355_W8A8_ERR_UNSUPPORTED;
   }
 }
@@ -282,6 +283,7 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
     la.zp = ws + w.zp;
     la.M = p->m; la.K = p->k; la.r = p->rank; la.nkk = w.nkk;
     la.steps_per_wave = w.steps_per_wave; la.n_steps = w.n_steps;
+    la.n_blocks = round_up(p->m, 32u) / 32u;
     const dim3 grid(w.slots / 32u), block(512);
     if (w.nkk > 2u) hipLaunchKernelGGL((lora_a_kernel<2>), grid, block, 0, s, la);
     else hipLaunchKernelGGL((lora_a_kernel<1>), grid, block, 0, s, la);
@@ -303,6 +305,8 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   g.residual = static_cast<const uint16_t*>(p->residual);
   g.out = p->out;
   g.M = p->m; g.N = p->n; g.K_pad = w.K_pad; g.KB = w.KB; g.slots = w.slots;
+  g.total_rows = round_up(p->m, 32u);
+  g.groups_per_weight = 1;
   g.tiles_m = w.slots / kTileM;
   g.tiles_n = n_padded(p->n) / kGemmTileN;
   g.rank = lora ? p->rank : 0u;
@@ -315,6 +319,135 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
     if ((st = launch_gemm<kEpiAcc>(ga, 0u, s))) return st;
   }
   return swiglu ? launch_gemm<kEpiSwiglu>(g, w.nkk, s) : launch_gemm<kEpiPlain>(g, w.nkk, s);
+}
+
+struct GroupedLayout {
+  uint64_t xq, sx, zp, at, src_row, dst_pos, blk_range, total;
+  uint32_t slots, nkk, K_pad, KB, n_steps, steps_per_wave;
+};
+
+GroupedLayout make_grouped_layout(uint32_t m, uint32_t k, uint32_t n_groups, uint32_t rank) {
+  GroupedLayout w{};
+  w.K_pad = k_padded(k);
+  w.KB = w.K_pad / 32u;
+  // every group is padded to 64 slots: at most 63 padding slots per group
+  const uint64_t worst = (uint64_t)m + 63ull * n_groups;
+  w.slots = (uint32_t)((worst + 63ull) / 64ull * 64ull);
+  w.nkk = rank_chunks(rank);
+  w.n_steps = (k + 63u) / 64u;
+  w.steps_per_wave = (w.n_steps + 7u) / 8u;
+  uint64_t off = 0;
+  w.xq = off; off += align256((uint64_t)w.slots * w.K_pad);
+  w.sx = off; off += align256((uint64_t)w.slots * 4u);
+  w.src_row = off; off += align256((uint64_t)w.slots * 4u);
+  w.dst_pos = off; off += align256((uint64_t)m * 4u);
+  w.blk_range = off; off += align256((uint64_t)(w.slots / 32u) * 4u);
+  w.zp = off; off += rank ? align256((uint64_t)(w.slots / 32u) * w.nkk * 3u * kBlockBytes) : 0u;
+  w.at = off; off += rank ? align256((uint64_t)n_groups * rank * k * 2u) : 0u;
+  w.total = off;
+  return w;
+}
+
+int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
+  if (!p) return MI355_W8A8_ERR_NULL;
+  if (p->struct_size != sizeof(mi355_w8a8_grouped_problem)) return MI355_W8A8_ERR_STRUCT;
+  int st = validate_common(p->m, p->k, p->n);
+  if (st) return st;
+  if (p->n_groups == 0) return MI355_W8A8_ERR_SHAPE;
+  if (p->n_groups > (uint32_t)kMaxGroups) return MI355_W8A8_ERR_UNSUPPORTED;
+  if (!p->x || !p->w_packed || !p->w_scales || !p->out || !p->group_sizes) return MI355_W8A8_ERR_NULL;
+  const bool swiglu = (p->flags & MI355_W8A8_FLAG_SWIGLU) != 0;
+  if (swiglu && (p->n & 1u)) return MI355_W8A8_ERR_SHAPE;
+  const bool lora = p->rank > 0;
+  if (lora) {
+    if (!p->lora_a || !p->lora_b || !p->lora_scaling) return MI355_W8A8_ERR_NULL;
+    if (p->rank > (uint32_t)kMaxRank) return MI355_W8A8_ERR_UNSUPPORTED;
+  }
+  const uint32_t gpw = p->groups_per_weight ? p->groups_per_weight : 1u;
+  if (p->n_groups % gpw) return MI355_W8A8_ERR_SHAPE;
+  const uint32_t n_out = swiglu ? p->n / 2u : p->n;
+  const uint64_t out_bytes = (uint64_t)p->m * n_out * 2u;
+  if (!aligned16(p->x) || !aligned16(p->w_packed) || !aligned16(p->out) || !aligned16(p->w_scales) ||
+      !aligned16(p->lora_a) || !aligned16(p->lora_b) || (reinterpret_cast<uintptr_t>(p->group_sizes) & 3u))
+    return MI355_W8A8_ERR_ALIGN;
+  if (overlaps(p->out, out_bytes, p->x, (uint64_t)p->m * p->k * 2u) ||
+      overlaps(p->out, out_bytes, p->workspace, p->workspace_bytes))
+    return MI355_W8A8_ERR_ALIAS;
+  const GroupedLayout w = make_grouped_layout(p->m, p->k, p->n_groups, p->rank);
+  if (!p->workspace || p->workspace_bytes < w.total) return MI355_W8A8_ERR_WORKSPACE;
+  if (reinterpret_cast<uintptr_t>(p->workspace) & 255u) return MI355_W8A8_ERR_ALIGN;
+  unsigned char* ws = static_cast<unsigned char*>(p->workspace);
+  int32_t* src_row = reinterpret_cast<int32_t*>(ws + w.src_row);
+  int32_t* dst_pos = reinterpret_cast<int32_t*>(ws + w.dst_pos);
+  int32_t* blk_range = reinterpret_cast<int32_t*>(ws + w.blk_range);
+  (void)hipGetLastError();
+
+  hipLaunchKernelGGL(route_groups_kernel, dim3(1), dim3(1024), 0, s, p->group_sizes, p->m, p->n_groups, w.slots,
+                     src_row, dst_pos, blk_range);
+  if ((st = launch_status())) return st;
+
+  QuantArgs q{};
+  q.x = static_cast<const uint16_t*>(p->x);
+  q.M = p->m; q.K = p->k; q.K_pad = w.K_pad; q.KB = w.KB;
+  q.dst_pos = dst_pos;
+  q.xq_packed = ws + w.xq;
+  q.sx_slots = reinterpret_cast<float*>(ws + w.sx);
+  q.codes_rm = p->aux_x_codes;
+  q.scales_rm = p->aux_x_scales;
+  q.zero_out = static_cast<uint16_t*>(p->out);
+  q.zero_cols = n_out;
+  if ((st = launch_quant<false>(q, s))) return st;
+
+  if (lora) {
+    uint16_t* at = reinterpret_cast<uint16_t*>(ws + w.at);
+    const uint64_t chunks = (uint64_t)p->n_groups * p->k * ((p->rank + 7u) / 8u);
+    hipLaunchKernelGGL(lora_a_transpose_kernel, dim3((uint32_t)((chunks + 255u) / 256u)), dim3(256), 0, s,
+                       static_cast<const uint16_t*>(p->lora_a), at, p->n_groups, p->k, p->rank);
+    if ((st = launch_status())) return st;
+    LoraAArgs la{};
+    la.xsrc = static_cast<const uint16_t*>(p->x);
+    la.at = at;
+    la.src_row = src_row;
+    la.slot_group = nullptr;
+    la.blk_range = blk_range;
+    la.zp = ws + w.zp;
+    la.M = p->m; la.K = p->k; la.r = p->rank; la.nkk = w.nkk;
+    la.steps_per_wave = w.steps_per_wave; la.n_steps = w.n_steps;
+    la.n_blocks = w.slots / 32u;
+    const dim3 grid(w.slots / 32u), block(512);
+    if (w.nkk > 2u) hipLaunchKernelGGL((lora_a_kernel<2>), grid, block, 0, s, la);
+    else hipLaunchKernelGGL((lora_a_kernel<1>), grid, block, 0, s, la);
+    if ((st = launch_status())) return st;
+  }
+
+  GemmArgs g{};
+  g.xq = ws + w.xq;
+  g.wp = static_cast<const unsigned char*>(p->w_packed);
+  g.sx = reinterpret_cast<const float*>(ws + w.sx);
+  g.sw = p->w_scales;
+  g.zp = lora ? ws + w.zp : nullptr;
+  g.lora_b = static_cast<const uint16_t*>(p->lora_b);
+  g.lora_scaling = p->lora_scaling;
+  g.src_row = src_row;
+  g.slot_group = nullptr;
+  g.blk_range = blk_range;
+  g.residual = nullptr;
+  g.out = p->out;
+  g.w_group_stride = mi355_w8a8_packed_weight_bytes(p->k, p->n);
+  g.M = p->m; g.N = p->n; g.K_pad = w.K_pad; g.KB = w.KB; g.slots = w.slots;
+  g.total_rows = w.slots;
+  g.tiles_m = w.slots / kGroupedTileM;
+  g.tiles_n = (n_padded(p->n) + kGroupedTileN - 1u) / kGroupedTileN;
+  g.rank = p->rank;
+  g.nsplit_terms = (p->flags & MI355_W8A8_FLAG_LORA_SPLIT2) ? 2u : 3u;
+  g.map_mode = 1;  // row-tile-major order: column tiles of one expert run back to back
+  g.groups_per_weight = gpw;
+  if (p->aux_acc) {
+    GemmArgs ga = g;
+    ga.out = p->aux_acc;
+    if ((st = launch_gemm<kEpiAcc, true>(ga, 0u, s))) return st;
+  }
+  return swiglu ? launch_gemm<kEpiSwiglu, true>(g, w.nkk, s) : launch_gemm<kEpiPlain, true>(g, w.nkk, s);
 }
 
 }  // namespace
@@ -415,15 +548,14 @@ int mi355_w8a8_forward_v1(const mi355_w8a8_problem* p, void* stream) {
 
 uint64_t mi355_w8a8_grouped_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint32_t rank,
                                             uint32_t flags) {
-  (void)m; (void)k; (void)n; (void)n_groups; (void)rank; (void)flags;
-  return 0;
+  (void)flags;
+  if (validate_common(m, k, n)) return 0;
+  if (n_groups == 0 || n_groups > (uint32_t)kMaxGroups || rank > (uint32_t)kMaxRank) return 0;
+  return make_grouped_layout(m, k, n_groups, rank).total;
 }
 
 int mi355_w8a8_grouped_v1(const mi355_w8a8_grouped_problem* p, void* stream) {
-  (void)stream;
-  if (!p) return MI355_W8A8_ERR_NULL;
-  if (p->struct_size != sizeof(mi355_w8a8_grouped_problem)) return MI355_W8A8_ERR_STRUCT;
-  return MI355_W8A8_ERR_UNSUPPORTED;
+  return run_grouped(p, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

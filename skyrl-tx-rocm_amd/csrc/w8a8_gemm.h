@@ -31,8 +31,10 @@ struct GemmArgs {
   const int32_t* blk_range;  // per 32-row block: first group | last group << 16, or null
   const uint16_t* residual;  // bf16 [M, n_out] or null
   void* out;                 // bf16 [M, n_out] or int32 [M, N]
-  uint32_t M, N, K_pad, KB, slots;
+  uint64_t w_group_stride;   // grouped mode: bytes between the packed weights of two experts
+  uint32_t M, N, K_pad, KB, slots, total_rows;
   uint32_t tiles_m, tiles_n, rank, nsplit_terms, map_mode;
+  uint32_t groups_per_weight; // grouped mode: weight index = group / groups_per_weight
 };
 
 // float32 pair -> packed bf16x2 (round to nearest even, v_cvt_pk_bf16_f32)
@@ -55,30 +57,48 @@ constexpr int kGemmTileN = 128;
 constexpr int kGemmStages = 3;
 constexpr int kGemmStageBytes = 24576;  // A: 8 row blocks x 2 k blocks, B: 4 column blocks x 2 k blocks
 constexpr int kGemmLdsBytes = kGemmStages * kGemmStageBytes;
+// Grouped (ragged, per-expert weight) mode: tile 64 x 512, the four waves sit side by side along
+// N (64 x 128 each) and share the 64-row activation panel; every 64-row tile belongs to one group.
+constexpr int kGroupedTileM = 64;
+constexpr int kGroupedTileN = 512;
+constexpr int kGroupedStages = 4;
+constexpr int kGroupedStageBytes = 36864;  // A: 2 row blocks x 2 k blocks, B: 16 column blocks x 2 k blocks
+constexpr int kGroupedLdsBytes = kGroupedStages * kGroupedStageBytes;
 
-template <int EPI, int NKK, int DBG = 0>
-__global__ __launch_bounds__(256, 2) void w8a8_gemm_kernel(GemmArgs g) {
+template <int EPI, int NKK, int DBG = 0, bool GROUPED = false>
+__global__ __launch_bounds__(256, GROUPED ? 1 : 2) void w8a8_gemm_kernel(GemmArgs g) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
   // ---- XCD-aware tile mapping: consecutive workgroup ids land on different XCDs, so each
-  // XCD gets a contiguous range of a band-major tile order (4 row tiles x all column tiles).
-  const uint32_t total_rows = round_up(g.M, 32u);
+  // XCD gets a contiguous range of a band-major tile order (GM row tiles x all column tiles).
+  const uint32_t total_rows = g.total_rows;
   const uint32_t ntile = g.tiles_m * g.tiles_n;
   const uint32_t per_xcd = (ntile + 7u) / 8u;
   const uint32_t t = g.map_mode == 1 ? blockIdx.x : (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
   if (t >= ntile) return;
-  constexpr uint32_t GM = 4;
+  constexpr uint32_t GM = GROUPED ? 1 : 4;
   const uint32_t band = t / (GM * g.tiles_n);
   const uint32_t band_rows = (g.tiles_m - band * GM) < GM ? (g.tiles_m - band * GM) : GM;
   const uint32_t in_band = t - band * GM * g.tiles_n;
   const uint32_t tm = band * GM + in_band % band_rows;
   const uint32_t tn = in_band / band_rows;
 
-  const unsigned char* Ag = g.xq + (size_t)tm * 8u * g.KB * kBlockBytes;
-  const unsigned char* Bg = g.wp + (size_t)tn * 4u * g.KB * kBlockBytes;
+  constexpr uint32_t kRowBlocks = GROUPED ? 2 : 8;   // 32-row blocks of the activation panel
+  constexpr uint32_t kColBlocks = GROUPED ? 16 : 4;  // 32-column blocks of the weight panel
+  uint32_t tile_group = 0;
+  if (GROUPED) {
+    const int32_t range = g.blk_range[tm * 2u];
+    if (range < 0) return;  // tile beyond the rows in use
+    tile_group = (uint32_t)range & 0xffffu;
+  }
+  const uint32_t widx = GROUPED ? tile_group / g.groups_per_weight : 0u;
+  const uint32_t ncb_total = n_padded(g.N) / 32u;  // column blocks of the packed weight
+  const unsigned char* Ag = g.xq + (size_t)tm * kRowBlocks * g.KB * kBlockBytes;
+  const unsigned char* Bg = g.wp + (size_t)widx * g.w_group_stride;
+  const float* swp = g.sw + (size_t)widx * (GROUPED ? g.N : 0u);
 
   v16i acc[2][4];
 #pragma unroll
@@ -89,29 +109,33 @@ __global__ __launch_bounds__(256, 2) void w8a8_gemm_kernel(GemmArgs g) {
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
   // ---- main loop
-  constexpr int kStages = kGemmStages;
-  constexpr int kLoadsPerTile = 6;  // direct-to-LDS loads each wave issues per tile
+  constexpr int kStages = GROUPED ? kGroupedStages : kGemmStages;
+  constexpr int kStageBytes = GROUPED ? kGroupedStageBytes : kGemmStageBytes;
+  constexpr int kAChunks = kRowBlocks * 2;                    // 1 KiB chunks of A per stage
+  constexpr int kLoadsPerTile = (kAChunks + kColBlocks * 2) / 4;  // direct-to-LDS loads per wave per tile
   const int KT = (int)(g.K_pad / 64u);
   auto issue = [&](int kt) {
-    unsigned char* St = lds + (kt % kStages) * kGemmStageBytes;
+    unsigned char* St = lds + (kt % kStages) * kStageBytes;
 #pragma unroll
-    for (int q = 0; q < 6; ++q) {
-      const int c = wave * 6 + q;  // chunks 0..15: A (row block c/2, k block c%2); 16..23: B
-      const unsigned char* base = c < 16 ? Ag : Bg;
-      const int rb = c < 16 ? (c >> 1) : ((c - 16) >> 1);
+    for (int q = 0; q < kLoadsPerTile; ++q) {
+      const int c = wave * kLoadsPerTile + q;  // chunks < kAChunks: A (row block c/2, k block c%2); then B
+      const bool isA = c < kAChunks;
+      uint32_t rb = isA ? (uint32_t)(c >> 1) : tn * kColBlocks + (uint32_t)((c - kAChunks) >> 1);
+      if (!isA && rb >= ncb_total) rb = ncb_total - 1u;  // keep every wave's load count equal
+      const unsigned char* base = isA ? Ag : Bg;
       const size_t goff = ((size_t)rb * g.KB + (size_t)kt * 2 + (c & 1)) * kBlockBytes + lane * 16;
       load_1k_to_lds(base + goff, St + c * kBlockBytes);
     }
   };
   auto read_frags = [&](int kt, int ks, v4i (&af)[2], v4i (&bf)[4]) {
-    const unsigned char* As = lds + (kt % kStages) * kGemmStageBytes;
-    const unsigned char* Bs = As + 16384;
+    const unsigned char* As = lds + (kt % kStages) * kStageBytes;
+    const unsigned char* Bs = As + kAChunks * kBlockBytes;
 #pragma unroll
     for (int i = 0; i < 2; ++i)
-      af[i] = *reinterpret_cast<const v4i*>(As + ((wave * 2 + i) * 2 + ks) * kBlockBytes + lane * 16);
+      af[i] = *reinterpret_cast<const v4i*>(As + (((GROUPED ? 0 : wave * 2) + i) * 2 + ks) * kBlockBytes + lane * 16);
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      bf[j] = *reinterpret_cast<const v4i*>(Bs + (j * 2 + ks) * kBlockBytes + lane * 16);
+      bf[j] = *reinterpret_cast<const v4i*>(Bs + (((GROUPED ? wave * 4 : 0) + j) * 2 + ks) * kBlockBytes + lane * 16);
   };
   auto mfma8 = [&](const v4i (&af)[2], const v4i (&bf)[4]) {
     if constexpr (DBG == 1) {  // measurement only: no MFMA work, keep the operands alive
@@ -182,19 +206,21 @@ __global__ __launch_bounds__(256, 2) void w8a8_gemm_kernel(GemmArgs g) {
   constexpr bool kLora = (NKK > 0) && (EPI != kEpiAcc);
   constexpr int kZ = NKK > 0 ? NKK : 1;
   const int c = lane & 31, h = lane >> 5;
-  const uint32_t m0 = tm * 256u + wave * 64u;
-  const uint32_t ncol = tn * 128u + 4u * c;
+  const uint32_t m0 = GROUPED ? tm * 64u : tm * 256u + wave * 64u;
+  const uint32_t tcol0 = GROUPED ? tn * 512u + wave * 128u : tn * 128u;  // first column of the wave
+  const uint32_t ncol = tcol0 + 4u * c;
   const uint32_t n_out = (EPI == kEpiSwiglu) ? g.N / 2u : g.N;
-  const bool full_n = (tn * 128u + 128u <= g.N) && ((g.N & 3u) == 0);  // uniform
+  const bool full_n = (tcol0 + 128u <= g.N) && ((g.N & 3u) == 0);  // wave-uniform
+  if (GROUPED && tcol0 >= g.N) return;  // wave beyond the last column (after the last barrier)
   float sw[4] = {0.f, 0.f, 0.f, 0.f};
   if (EPI != kEpiAcc) {
     if (full_n) {
-      const float4 s4 = *reinterpret_cast<const float4*>(g.sw + ncol);
+      const float4 s4 = *reinterpret_cast<const float4*>(swp + ncol);
       sw[0] = s4.x; sw[1] = s4.y; sw[2] = s4.z; sw[3] = s4.w;
     } else {
 #pragma unroll
       for (int j = 0; j < 4; ++j)
-        if (ncol + j < g.N) sw[j] = g.sw[ncol + j];
+        if (ncol + j < g.N) sw[j] = swp[ncol + j];
     }
   }
   // LoRA-B staging, private to the wave: bf16 [16*NKK][128] at lds + wave * 16 KiB
@@ -217,6 +243,7 @@ __global__ __launch_bounds__(256, 2) void w8a8_gemm_kernel(GemmArgs g) {
     const uint32_t pbase = m0 + bi * 32u;
     if (pbase >= total_rows) return;  // wave-uniform
     const uint32_t blk = pbase / 32u;
+    if (GROUPED && g.blk_range[blk] < 0) return;  // block beyond the rows in use
     v8us zf[kZ][3];
     load_zfrags(blk, zf);
 
@@ -280,7 +307,6 @@ __global__ __launch_bounds__(256, 2) void w8a8_gemm_kernel(GemmArgs g) {
           // stage B[gi][0:16*NKK][tile columns] as bf16 [16*NKK][128]; LDS operations of one
           // wave execute in order, so no barrier is needed around this wave-private buffer
           const uint16_t* Bsrc = g.lora_b + (size_t)gi * g.rank * g.N;
-          const uint32_t tcol0 = tn * 128u;
           for (uint32_t q = (uint32_t)lane; q < NKK * 16u * 16u; q += 64u) {
             const uint32_t r = q >> 4, cc = (q & 15u) * 8u;
             v8us val = {0, 0, 0, 0, 0, 0, 0, 0};

@@ -111,6 +111,52 @@ __global__ __launch_bounds__(1024) void route_rows_kernel(const int32_t* __restr
 }
 
 // ---------------------------------------------------------------------------------------
+// Tables for rows that arrive already grouped (ragged groups of an expert layer,
+// skyrl/tx/layers/util.py:8-59): group g owns group_sizes[g] consecutive rows and is padded
+// to a multiple of 64 grouped slots so that a 64-row GEMM tile never mixes two weights.
+//   src_row[p]   = original row of slot p, -1 for padding
+//   dst_pos[m]   = slot of row m, -1 for rows beyond sum(group_sizes) (their output is zero)
+//   blk_range[b] = g | g << 16 for the 32-row blocks in use, -1 beyond
+// ---------------------------------------------------------------------------------------
+constexpr int kMaxGroups = 1024;
+__global__ __launch_bounds__(1024) void route_groups_kernel(const int32_t* __restrict__ group_sizes, uint32_t M,
+                                                            uint32_t n_groups, uint32_t slots,
+                                                            int32_t* __restrict__ src_row,
+                                                            int32_t* __restrict__ dst_pos,
+                                                            int32_t* __restrict__ blk_range) {
+  __shared__ int row_start[kMaxGroups + 1];
+  __shared__ int slot_start[kMaxGroups + 1];
+  const uint32_t tid = threadIdx.x;
+  if (tid == 0) {
+    int r = 0, p = 0;
+    for (uint32_t g = 0; g < n_groups; ++g) {
+      int sz = group_sizes[g];
+      if (sz < 0) sz = 0;
+      if (r + sz > (int)M) sz = (int)M - r;
+      row_start[g] = r;
+      slot_start[g] = p;
+      r += sz;
+      p += (sz + 63) & ~63;
+    }
+    row_start[n_groups] = r;
+    slot_start[n_groups] = p;
+  }
+  for (uint32_t p = tid; p < slots; p += 1024) src_row[p] = -1;
+  for (uint32_t i = tid; i < M; i += 1024) dst_pos[i] = -1;
+  for (uint32_t b = tid; b < slots / 32u; b += 1024) blk_range[b] = -1;
+  __syncthreads();
+  const uint32_t wave = tid >> 6, lane = tid & 63;
+  for (uint32_t g = wave; g < n_groups; g += 16) {
+    const int r0 = row_start[g], r1 = row_start[g + 1], p0 = slot_start[g], p1 = slot_start[g + 1];
+    for (int i = (int)lane; i < r1 - r0; i += 64) {
+      src_row[p0 + i] = r0 + i;
+      dst_pos[r0 + i] = p0 + i;
+    }
+    for (int b = p0 / 32 + (int)lane; b < p1 / 32; b += 64) blk_range[b] = (int)(g | (g << 16));
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // Per-token dynamic int8 quantization (skyrl/tx/kernels/quantized_lora.py:199-212 with one
 // group per row), optionally preceded by RMSNorm
 // (skyrl/tx/kernels/rocm/bf16_rms_gate_up_lora_swiglu.py:299-303).  One wave per row; the
@@ -132,6 +178,8 @@ struct QuantArgs {
   float* scales_rm;        // f32 [M] or null
   uint16_t* xn;            // bf16 [M, K] normalized rows or null
   uint16_t* xn_aux;        // second copy for the caller or null
+  uint16_t* zero_out;      // bf16 [M, zero_cols]: rows without a slot (dst_pos < 0) are zero-filled
+  uint32_t zero_cols;
 };
 
 template <int NCH, bool RMS>
@@ -192,6 +240,9 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(QuantArgs a) {
   amax = wave_max(amax);
   const float scale = amax > 0.0f ? amax / 127.0f : 1.0f;
   const int p = a.dst_pos ? a.dst_pos[m] : (int)m;
+  if (p < 0 && a.zero_out) {
+    for (uint32_t cidx = lane; cidx < a.zero_cols; cidx += 64u) a.zero_out[(size_t)m * a.zero_cols + cidx] = 0;
+  }
   if (lane == 0) {
     if (a.sx_slots && p >= 0) a.sx_slots[p] = scale;
     if (a.scales_rm) a.scales_rm[m] = scale;
@@ -266,7 +317,7 @@ struct LoraAArgs {
   const int32_t* slot_group;// or null (group 0)
   const int32_t* blk_range; // or null
   unsigned char* zp;        // packed z fragments
-  uint32_t M, K, r, nkk, steps_per_wave, n_steps;
+  uint32_t M, K, r, nkk, steps_per_wave, n_steps, n_blocks;
 };
 
 template <int RB>  // number of 32-wide rank blocks (1 or 2)
@@ -275,7 +326,8 @@ __global__ __launch_bounds__(512) void lora_a_kernel(LoraAArgs a) {
   __shared__ float zs[32][RB * 32 + 1];
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
   const uint32_t pb = blockIdx.x;
-  if (pb * 32u >= round_up(a.M, 32u)) return;
+  if (pb >= a.n_blocks) return;
+  if (a.blk_range && a.blk_range[pb] < 0) return;  // block beyond the rows in use
   const uint32_t range = a.blk_range ? (uint32_t)a.blk_range[pb] : 0u;
   const uint32_t glo = range & 0xffffu, ghi = range >> 16;
   const uint32_t i = lane & 31u, h = lane >> 5;

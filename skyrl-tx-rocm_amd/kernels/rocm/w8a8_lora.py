@@ -330,6 +330,153 @@ def forward(x: torch.Tensor, weight, lora_a=None, lora_b=None, lora_scaling=None
     return (result, plan.aux) if return_aux else result
 
 
+# ---------------------------------------------------------------------------------------
+# grouped (ragged, per-expert) variant
+# ---------------------------------------------------------------------------------------
+@dataclass(frozen=True)
+class PackedGroupedW8Weight:
+    """E stacked [K, N] int8 weights in MFMA fragment order plus float32 scales [E, N]."""
+
+    packed: torch.Tensor
+    scales: torch.Tensor
+    n_weights: int
+    in_features: int
+    out_features: int
+
+
+def prepare_grouped_weight(codes: torch.Tensor, scales: torch.Tensor) -> PackedGroupedW8Weight:
+    """Pack per-expert int8 codes [E, K, N] with per-channel scales [E, N] (or [E, 1, N]) once."""
+    if codes.ndim != 3 or codes.dtype != torch.int8:
+        raise TypeError("grouped W8 codes must be a rank-three INT8 array [E, K, N]")
+    _require_cuda(codes, "weight codes")
+    e, k, n = codes.shape
+    if k % 8 or k > MAX_IN_FEATURES:
+        raise ValueError(f"K must be a multiple of 8 not exceeding {MAX_IN_FEATURES}, got {k}")
+    if scales.numel() != e * n or not scales.dtype.is_floating_point:
+        raise ValueError(f"scales must be floating point with {e * n} elements, got {tuple(scales.shape)}")
+    lib = _native.load()
+    each = int(lib.mi355_w8a8_packed_weight_bytes(k, n))
+    packed = torch.empty(e * each, dtype=torch.uint8, device=codes.device)
+    codes = codes.contiguous()
+    with torch.cuda.device(codes.device):
+        for i in range(e):
+            _native.check("mi355_w8a8_pack_weight_v1",
+                          lib.mi355_w8a8_pack_weight_v1(codes[i].data_ptr(), packed.data_ptr() + i * each, k, n,
+                                                        _stream_ptr(codes.device)))
+    return PackedGroupedW8Weight(packed=packed, scales=scales.to(torch.float32).reshape(e, n).contiguous(),
+                                 n_weights=e, in_features=k, out_features=n)
+
+
+def grouped_forward(x: torch.Tensor, group_sizes: torch.Tensor, weight: PackedGroupedW8Weight, lora_a=None,
+                    lora_b=None, lora_scaling=None, *, swiglu: bool = False, groups_per_weight: int = 1,
+                    flags: int = 0, return_aux: bool = False):
+    """Ragged W8A8 (+LoRA) linear: rows of ``x`` are sorted by group; group g owns
+    ``group_sizes[g]`` consecutive rows and uses weight ``g // groups_per_weight`` and LoRA pair g.
+    Rows beyond ``sum(group_sizes)`` give zeros (``lax.ragged_dot`` semantics)."""
+    if x.dtype != torch.bfloat16:
+        raise TypeError(f"x must be BF16, got {x.dtype}")
+    if x.ndim != 2 or x.shape[0] <= 0:
+        raise ValueError(f"x must be [rows, K] with at least one row, got {tuple(x.shape)}")
+    _require_cuda(x, "x")
+    k, n = weight.in_features, weight.out_features
+    if x.shape[1] != k:
+        raise ValueError(f"x K={x.shape[1]} does not match W8 K={k}")
+    dev = x.device
+    flat = x.contiguous()
+    m = flat.shape[0]
+    gs = group_sizes.to(device=dev, dtype=torch.int32).contiguous()
+    n_groups = gs.numel()
+    if n_groups != weight.n_weights * groups_per_weight:
+        raise ValueError(f"{n_groups} groups do not match {weight.n_weights} weights x {groups_per_weight}")
+    a3 = b3 = s1 = None
+    r = 0
+    if lora_a is not None:
+        if lora_a.dtype != torch.bfloat16 or lora_b.dtype != torch.bfloat16:
+            raise TypeError("LoRA A and B must both be BF16")
+        if lora_a.ndim != 3 or lora_b.ndim != 3 or lora_a.shape[0] != n_groups or lora_a.shape[1] != k:
+            raise ValueError(f"grouped lora_a must be [{n_groups}, {k}, r], got {tuple(lora_a.shape)}")
+        r = lora_a.shape[2]
+        if tuple(lora_b.shape) != (n_groups, r, n):
+            raise ValueError(f"grouped lora_b must be [{n_groups}, {r}, {n}], got {tuple(lora_b.shape)}")
+        if r < 1 or r > MAX_LORA_RANK:
+            raise ValueError(f"LoRA rank must be in [1, {MAX_LORA_RANK}], got {r}")
+        a3, b3 = lora_a.contiguous(), lora_b.contiguous()
+        s1 = torch.as_tensor(lora_scaling, dtype=torch.float32, device=dev)
+        s1 = (s1.reshape(1).expand(n_groups) if s1.ndim == 0 else s1).contiguous()
+        if tuple(s1.shape) != (n_groups,):
+            raise ValueError(f"lora_scaling must be a scalar or have shape ({n_groups},)")
+    if swiglu and n % 2:
+        raise ValueError("SwiGLU needs an even number of fused gate/up columns")
+    n_out = n // 2 if swiglu else n
+    lib = _native.load()
+    if swiglu:
+        flags |= _native.FLAG_SWIGLU
+    ws_bytes = int(lib.mi355_w8a8_grouped_workspace_bytes(m, k, n, n_groups, r, flags))
+    if ws_bytes == 0:
+        raise ValueError(f"geometry M={m}, K={k}, N={n}, groups={n_groups}, rank={r} is outside the native path")
+    out = torch.empty((m, n_out), dtype=torch.bfloat16, device=dev)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    aux = {}
+    if return_aux:
+        aux["x_codes"] = torch.empty((m, k), dtype=torch.int8, device=dev)
+        aux["x_scales"] = torch.empty((m,), dtype=torch.float32, device=dev)
+        aux["acc"] = torch.zeros((m, n), dtype=torch.int32, device=dev)
+    p = _native.GroupedProblem()
+    p.struct_size = ctypes.sizeof(_native.GroupedProblem)
+    p.flags = flags
+    p.m, p.k, p.n, p.n_groups, p.rank, p.groups_per_weight = m, k, n, n_groups, r, groups_per_weight
+    p.x = flat.data_ptr()
+    p.w_packed = weight.packed.data_ptr()
+    p.w_scales = weight.scales.data_ptr()
+    p.lora_a = a3.data_ptr() if r else None
+    p.lora_b = b3.data_ptr() if r else None
+    p.lora_scaling = s1.data_ptr() if r else None
+    p.group_sizes = gs.data_ptr()
+    p.out = out.data_ptr()
+    p.workspace = ws.data_ptr()
+    p.workspace_bytes = ws_bytes
+    p.aux_x_codes = aux["x_codes"].data_ptr() if return_aux else None
+    p.aux_x_scales = aux["x_scales"].data_ptr() if return_aux else None
+    p.aux_acc = aux["acc"].data_ptr() if return_aux else None
+    with torch.cuda.device(dev):
+        _native.check("mi355_w8a8_grouped_v1", lib.mi355_w8a8_grouped_v1(ctypes.byref(p), _stream_ptr(dev)))
+    return (out, aux) if return_aux else out
+
+
+def w8a8_grouped_lora_linear(x, group_sizes, weight, lora_a=None, lora_b=None, lora_scaling=None, *,
+                             enabled: bool = False, interpret: bool = False, swiglu: bool = False,
+                             groups_per_weight: int = 1):
+    """W8A8 form of ``LoRAExpert.__call__`` (skyrl/tx/layers/lora.py:394-444): per-group frozen
+    weight plus per-group LoRA over rows that are already sorted by group."""
+    _check_enabled(enabled, interpret, "grouped LoRA")
+    return grouped_forward(x, group_sizes, weight, lora_a, lora_b, lora_scaling, swiglu=swiglu,
+                           groups_per_weight=groups_per_weight)
+
+
+def w8a8_moe_expert_mlp(hidden, router_logits, top_k: int, gate_up_weight, down_weight, gate_up_a, gate_up_b,
+                        down_a, down_b, lora_scaling, *, enabled: bool = False, norm_topk_prob: bool = True):
+    """Expert MLP of ``Qwen3Experts.__call__`` (skyrl/tx/models/qwen3.py:172-210) on W8A8 weights:
+    softmax -> top-k -> renormalise -> sort rows by expert -> grouped gate/up + SwiGLU -> grouped
+    down -> unsort -> weighted sum.  Routing and the final combine are torch glue; the two
+    grouped GEMMs are the HIP kernels."""
+    _check_enabled(enabled, False, "MoE expert MLP")
+    n_experts = gate_up_weight.n_weights
+    probs = torch.softmax(router_logits.to(torch.float32), dim=-1)
+    weights, selected = torch.topk(probs, top_k, dim=-1)
+    if norm_topk_prob:
+        weights = weights / weights.sum(dim=-1, keepdim=True)
+    flat_experts = selected.reshape(-1)
+    order = torch.sort(flat_experts, stable=True).indices
+    x_sorted = hidden.repeat_interleave(top_k, dim=0)[order]
+    group_sizes = torch.bincount(flat_experts, minlength=n_experts).to(torch.int32)
+    act = grouped_forward(x_sorted, group_sizes, gate_up_weight, gate_up_a, gate_up_b, lora_scaling, swiglu=True)
+    down = grouped_forward(act, group_sizes, down_weight, down_a, down_b, lora_scaling)
+    unsort = torch.empty_like(order)
+    unsort[order] = torch.arange(order.numel(), device=order.device)
+    per_tok = down[unsort].reshape(hidden.shape[0], top_k, -1).to(torch.float32)
+    return (per_tok * weights[..., None]).sum(dim=1).to(torch.bfloat16)
+
+
 def _check_enabled(enabled, interpret, what: str) -> None:
     _validate_exact_bool("enabled", enabled)
     _validate_exact_bool("interpret", interpret)
@@ -402,5 +549,6 @@ __all__ = (
     "DEFAULT_BLOCK_M", "DEFAULT_BLOCK_N", "DEFAULT_ROW_SUPERBLOCK", "MAX_BLOCK_M", "MAX_BLOCK_N",
     "MAX_IN_FEATURES", "MAX_OUT_FEATURES", "MAX_ROW_SUPERBLOCK", "MAX_LORA_RANK", "PackedW8Weight",
     "prepare_weight", "unpack_weight", "dynamic_quantize_rows", "ForwardPlan", "forward", "w8a8_frozen_linear",
-    "w8a8_lora_linear", "w8a8_rms_gate_up_lora_swiglu", "w8a8_lora_residual",
+    "w8a8_lora_linear", "w8a8_rms_gate_up_lora_swiglu", "w8a8_lora_residual", "PackedGroupedW8Weight",
+    "prepare_grouped_weight", "grouped_forward", "w8a8_grouped_lora_linear", "w8a8_moe_expert_mlp",
 )

@@ -265,3 +265,86 @@ def test_reference_call_surface(dev, pkg):
     torch.cuda.synchronize()
     assert out3.shape == (2, 2, 32)
     assert torch.equal(out3.reshape(4, 32), out)
+
+
+# ---------------------------------------------------------------------------------------
+# grouped (per-expert) variant and the MoE composite
+# ---------------------------------------------------------------------------------------
+def _grouped_case(rng, sizes, k, n, rank, extra_rows=0):
+    e = len(sizes)
+    m = int(sum(sizes)) + extra_rows
+    x = o.bf16_round(rng.standard_normal((m, k)).astype(F32))
+    codes = rng.integers(-127, 128, (e, k, n), dtype=np.int8)
+    scales = rng.uniform(0.001, 0.01, (e, n)).astype(F32)
+    a = o.bf16_round((rng.standard_normal((e, k, rank)) * 0.02).astype(F32)) if rank else None
+    b = o.bf16_round((rng.standard_normal((e, rank, n)) * 0.02).astype(F32)) if rank else None
+    return m, x, codes, scales, a, b
+
+
+@pytest.mark.parametrize("sizes,k,n,rank,swiglu,extra", [
+    ([5, 0, 70, 33, 1, 64, 0, 129], 256, 512, 16, False, 0),
+    ([40, 3, 0, 0, 200], 384, 1536, 16, True, 0),
+    ([17, 90], 128, 96, 8, False, 9),
+    ([64, 64, 64], 2048, 768, 0, False, 0),
+])
+def test_grouped_ragged_linear(dev, pkg, sizes, k, n, rank, swiglu, extra):
+    import torch
+
+    rng = np.random.default_rng(len(sizes) * 100 + k)
+    m, x, codes, scales, a, b = _grouped_case(rng, sizes, k, n, rank, extra)
+    s = F32(1.5)
+    weights = [o.GroupQuantizedWeight(codes[e], scales[e:e + 1], k, k, 8, k) for e in range(len(sizes))]
+    st = np.concatenate(([0], np.cumsum(sizes)))
+    want_pre = np.zeros((m, n), F32)
+    want_acc = np.zeros((m, n), np.int32)
+    xc, xs = o.quantize_rows(x)
+    for e, w in enumerate(weights):
+        r0, r1 = int(st[e]), int(st[e + 1])
+        if r1 > r0:
+            if rank:
+                want_pre[r0:r1] = o.quantized_lora_linear_f32(x[r0:r1], w, a[e], b[e], s)
+            else:
+                want_pre[r0:r1] = o.quantized_frozen_linear_f32(x[r0:r1], w)
+            want_acc[r0:r1] = o.int_matmul(xc[r0:r1], codes[e])
+    fused = o.bf16_round(want_pre)
+    want = o.swiglu_from_interleaved(fused) if swiglu else fused
+    w8 = pkg.w8a8_lora
+    bf = lambda t: torch.from_numpy(np.ascontiguousarray(t)).to(dev).to(torch.bfloat16)
+    gw = w8.prepare_grouped_weight(torch.from_numpy(codes).to(dev), torch.from_numpy(scales).to(dev))
+    out, aux = w8.grouped_forward(bf(x), torch.tensor(sizes, dtype=torch.int32), gw,
+                                  bf(a) if rank else None, bf(b) if rank else None, float(s) if rank else None,
+                                  swiglu=swiglu, return_aux=True)
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy()
+    np.testing.assert_array_equal(aux["x_codes"].cpu().numpy(), xc)
+    np.testing.assert_array_equal(aux["x_scales"].cpu().numpy().view(np.uint32), xs.view(np.uint32))
+    np.testing.assert_array_equal(aux["acc"].cpu().numpy(), want_acc)
+    assert np.all(got[int(st[-1]):] == 0)          # rows beyond the groups give zeros
+    _assert_close(got, want, f" grouped {sizes} {k}x{n}")
+
+
+def test_moe_expert_mlp_reduced(dev, pkg):
+    """Config 5 at reduced size: top-4 of 16 experts, hidden 256, intermediate 128, rank 16."""
+    import torch
+
+    rng = np.random.default_rng(55)
+    t, h, inter, e, topk, r = 192, 256, 128, 16, 4, 16
+    hidden = o.bf16_round(rng.standard_normal((t, h)).astype(F32))
+    logits = rng.standard_normal((t, e)).astype(F32)
+    gu_codes = rng.integers(-127, 128, (e, h, 2 * inter), dtype=np.int8)
+    gu_scales = rng.uniform(0.001, 0.01, (e, 2 * inter)).astype(F32)
+    dn_codes = rng.integers(-127, 128, (e, inter, h), dtype=np.int8)
+    dn_scales = rng.uniform(0.001, 0.01, (e, h)).astype(F32)
+    mk = lambda shape: o.bf16_round((rng.standard_normal(shape) * 0.02).astype(F32))
+    gua, gub, da, db = mk((e, h, r)), mk((e, r, 2 * inter)), mk((e, inter, r)), mk((e, r, h))
+    gu = [o.GroupQuantizedWeight(gu_codes[i], gu_scales[i:i + 1], h, h, 8, h) for i in range(e)]
+    dn = [o.GroupQuantizedWeight(dn_codes[i], dn_scales[i:i + 1], inter, inter, 8, inter) for i in range(e)]
+    want = o.moe_expert_mlp(hidden, logits, topk, gu, dn, gua, gub, da, db, F32(1.0))
+    w8 = pkg.w8a8_lora
+    bf = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev).to(torch.bfloat16)
+    guw = w8.prepare_grouped_weight(torch.from_numpy(gu_codes).to(dev), torch.from_numpy(gu_scales).to(dev))
+    dnw = w8.prepare_grouped_weight(torch.from_numpy(dn_codes).to(dev), torch.from_numpy(dn_scales).to(dev))
+    got = w8.w8a8_moe_expert_mlp(bf(hidden), torch.from_numpy(logits).to(dev), topk, guw, dnw, bf(gua), bf(gub),
+                                 bf(da), bf(db), 1.0, enabled=True)
+    torch.cuda.synchronize()
+    _assert_close(got.float().cpu().numpy(), want, " moe reduced")
