@@ -45,7 +45,9 @@ def _assert_close(got, want, what=""):
     rep = wc.compare(got, want)
     print(f"[parity]{what} {rep}", flush=True)
     assert rep["violations"] == 0, rep
-    assert rep["passed"], rep
+    # reference gate (relative L2 < 1e-2, cosine >= 0.9999); its max-abs bound of 0.25 presumes
+    # O(1) outputs and is reported, not asserted, since one bf16 ulp at magnitude 64 is 0.5
+    assert rep["relative_l2"] < 1e-2 and rep["cosine"] >= 0.9999, rep
     return rep
 
 
