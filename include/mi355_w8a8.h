@@ -59,6 +59,9 @@ typedef enum mi355_w8a8_status {
  * call with SKIP_PROLOGUE after a full call with the same arguments re-runs only the GEMM kernel. */
 #define MI355_W8A8_FLAG_SKIP_PROLOGUE 16u /* do not run routing / quantization / LoRA-A */
 #define MI355_W8A8_FLAG_SKIP_GEMM 32u     /* run only routing / quantization / LoRA-A */
+/* tile geometry of the tiled GEMM; default: 256 x 256 once such tiles fill the chip, else 256 x 128 */
+#define MI355_W8A8_FLAG_TILE_256X128 64u
+#define MI355_W8A8_FLAG_TILE_256X256 128u
 
 /*
  * One forward call.  y = dequant(quant(n) @ W) + s[idx] * ((n @ A[idx]) @ B[idx]) (+ residual),

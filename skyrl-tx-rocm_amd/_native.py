@@ -19,6 +19,8 @@ FLAG_FORCE_SKINNY = 4
 FLAG_LORA_SPLIT2 = 8
 FLAG_SKIP_PROLOGUE = 16
 FLAG_SKIP_GEMM = 32
+FLAG_TILE_256X128 = 64
+FLAG_TILE_256X256 = 128
 
 STATUS = {
     0: "OK", -1: "ERR_NULL", -2: "ERR_SHAPE", -3: "ERR_ALIGN", -4: "ERR_ALIAS",

@@ -21,7 +21,7 @@ constexpr uint32_t kMaxN = 1u << 20;
 inline uint64_t align256(uint64_t v) { return (v + 255u) & ~uint64_t(255); }
 
 struct WsLayout {
-  uint64_t xq, sx, xn, zp, at, src_row, dst_pos, slot_group, blk_range, skinny, total;
+  uint64_t xq, sx, xn, zp, at, bp, src_row, dst_pos, slot_group, blk_range, skinny, total;
   uint32_t slots, nkk, K_pad, KB, n_steps, steps_per_wave;
 };
 
@@ -36,7 +36,7 @@ WsLayout make_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint
   (void)routed;
   w.nkk = rank_chunks(rank);
   w.n_steps = (k + 63u) / 64u;
-  w.steps_per_wave = (w.n_steps + 7u) / 8u;
+  w.steps_per_wave = (w.n_steps + 15u) / 16u;
   uint64_t off = 0;
   w.xq = off; off += align256((uint64_t)w.slots * w.K_pad);
   w.sx = off; off += align256((uint64_t)w.slots * 4u);
@@ -47,6 +47,7 @@ WsLayout make_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint
   w.xn = off; off += rank ? align256((uint64_t)m * k * 2u) : 0u;
   w.zp = off; off += rank ? align256((uint64_t)(w.slots / 32u) * w.nkk * 3u * kBlockBytes) : 0u;
   w.at = off; off += rank ? align256((uint64_t)n_groups * rank * k * 2u) : 0u;
+  w.bp = off; off += rank ? align256((uint64_t)n_groups * (n_padded(n) / 32u) * w.nkk * kBlockBytes) : 0u;
   w.skinny = off; off += align256(skinny_workspace_bytes(m, n));
   w.total = off;
   return w;
@@ -75,38 +76,45 @@ int launch_quant(const QuantArgs& a, hipStream_t s) {
   return MI355_W8A8_ERR_UNSUPPORTED;
 }
 
-template <int EPI, int NKK, bool GROUPED>
+template <int EPI, int NKK, int MODE>
 int launch_gemm_one(const GemmArgs& g, hipStream_t s) {
+  // persistent grid: one workgroup slot per CU (two in the 256 x 128 geometry), a multiple of 8
   const uint32_t ntile = g.tiles_m * g.tiles_n;
-  const dim3 grid(((ntile + 7u) / 8u) * 8u), block(256);
-  constexpr uint32_t lds_bytes = GROUPED ? kGroupedLdsBytes : kGemmLdsBytes;
+  uint32_t slots = MODE == kModeDense ? 512u : 256u;
 #ifdef W8A8_DEBUG_VARIANTS
-  if constexpr (EPI == kEpiSwiglu && NKK == 2 && !GROUPED) {
+  { const char* e = getenv("MI355_W8A8_GRID"); if (e && atoi(e) > 0) slots = ((uint32_t)atoi(e) + 7u) / 8u * 8u; }
+#endif
+  const uint32_t want = ((ntile + 7u) / 8u) * 8u;
+  const dim3 grid(want < slots ? want : slots), block(MODE == kModeWide ? 512 : 256);
+  constexpr uint32_t lds_bytes =
+      MODE == kModeGrouped ? kGroupedLdsBytes : (MODE == kModeWide ? kWideLdsBytes : kGemmLdsBytes);
+#ifdef W8A8_DEBUG_VARIANTS
+  if constexpr (EPI == kEpiSwiglu && NKK == 2 && MODE != kModeGrouped) {
 #define W8A8_DBG(D)                                                                              \
   if (g.map_mode == 100 + D) {                                                                   \
-    hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm_kernel<EPI, NKK, D, false>),   \
+    hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm_kernel<EPI, NKK, D, MODE>),    \
                         hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);                  \
-    hipLaunchKernelGGL((w8a8_gemm_kernel<EPI, NKK, D, false>), grid, block, lds_bytes, s, g);    \
+    hipLaunchKernelGGL((w8a8_gemm_kernel<EPI, NKK, D, MODE>), grid, block, lds_bytes, s, g);     \
     return launch_status();                                                                      \
   }
-    W8A8_DBG(1) W8A8_DBG(2) W8A8_DBG(3) W8A8_DBG(4)
+    W8A8_DBG(1) W8A8_DBG(3)
 #undef W8A8_DBG
   }
 #endif
-  if (hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm_kernel<EPI, NKK, 0, GROUPED>),
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm_kernel<EPI, NKK, 0, MODE>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
     return MI355_W8A8_ERR_LAUNCH;
-  hipLaunchKernelGGL((w8a8_gemm_kernel<EPI, NKK, 0, GROUPED>), grid, block, lds_bytes, s, g);
+  hipLaunchKernelGGL((w8a8_gemm_kernel<EPI, NKK, 0, MODE>), grid, block, lds_bytes, s, g);
   return launch_status();
 }
 
-template <int EPI, bool GROUPED = false>
+template <int EPI, int MODE = kModeDense>
 int launch_gemm(const GemmArgs& g, uint32_t nkk, hipStream_t s) {
   switch (nkk) {
-    case 0: return launch_gemm_one<EPI, 0, GROUPED>(g, s);
-    case 1: return launch_gemm_one<EPI, 1, GROUPED>(g, s);
-    case 2: return launch_gemm_one<EPI, 2, GROUPED>(g, s);
-    case 4: return launch_gemm_one<EPI, 4, GROUPED>(g, s);
+    case 0: return launch_gemm_one<EPI, 0, MODE>(g, s);
+    case 1: return launch_gemm_one<EPI, 1, MODE>(g, s);
+    case 2: return launch_gemm_one<EPI, 2, MODE>(g, s);
+    case 4: return launch_gemm_one<EPI, 4, MODE>(g, s);
     default: return MI355_W8A8_ERR_UNSUPPORTED;
   }
 }
@@ -245,9 +253,22 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
 
   const bool skip_prologue = (p->flags & MI355_W8A8_FLAG_SKIP_PROLOGUE) != 0;
   const bool skip_gemm = (p->flags & MI355_W8A8_FLAG_SKIP_GEMM) != 0;
-  if (routed && !skip_prologue) {
-    hipLaunchKernelGGL(route_rows_kernel, dim3(1), dim3(1024), 0, s, p->adapter_indices, p->m,
-                       p->n_adapters, w.slots, src_row, dst_pos, slot_group, blk_range);
+  if ((routed || lora) && !skip_prologue) {
+    LoraPrepArgs pa{};
+    pa.idx = routed ? p->adapter_indices : nullptr;
+    pa.src_row = src_row; pa.dst_pos = dst_pos; pa.slot_group = slot_group; pa.blk_range = blk_range;
+    pa.lora_a = static_cast<const uint16_t*>(p->lora_a);
+    pa.lora_b = static_cast<const uint16_t*>(p->lora_b);
+    pa.at = reinterpret_cast<uint16_t*>(ws + w.at);
+    pa.bp = ws + w.bp;
+    pa.M = p->m; pa.K = p->k; pa.N = p->n; pa.n_groups = p->n_adapters; pa.r = p->rank; pa.nkk = w.nkk;
+    pa.ncb = n_padded(p->n) / 32u; pa.slots = w.slots;
+    pa.route_blocks = routed ? 1u : 0u;
+    const uint64_t a_items = (uint64_t)p->n_adapters * p->k * ((p->rank + 7u) / 8u);
+    const uint64_t b_items = (uint64_t)p->n_adapters * pa.ncb * w.nkk * 64u;
+    pa.a_blocks = (uint32_t)((a_items + 1023u) / 1024u);
+    const uint32_t b_blocks = (uint32_t)((b_items + 1023u) / 1024u);
+    hipLaunchKernelGGL(lora_prep_kernel, dim3(pa.route_blocks + pa.a_blocks + b_blocks), dim3(1024), 0, s, pa);
     if ((st = launch_status())) return st;
   }
 
@@ -270,10 +291,6 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
 
   if (lora && !skip_prologue) {
     uint16_t* at = reinterpret_cast<uint16_t*>(ws + w.at);
-    const uint64_t chunks = (uint64_t)p->n_adapters * p->k * ((p->rank + 7u) / 8u);
-    hipLaunchKernelGGL(lora_a_transpose_kernel, dim3((uint32_t)((chunks + 255u) / 256u)), dim3(256), 0, s,
-                       static_cast<const uint16_t*>(p->lora_a), at, p->n_adapters, p->k, p->rank);
-    if ((st = launch_status())) return st;
     LoraAArgs la{};
     la.xsrc = rms ? reinterpret_cast<const uint16_t*>(ws + w.xn) : static_cast<const uint16_t*>(p->x);
     la.at = at;
@@ -284,7 +301,7 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
     la.M = p->m; la.K = p->k; la.r = p->rank; la.nkk = w.nkk;
     la.steps_per_wave = w.steps_per_wave; la.n_steps = w.n_steps;
     la.n_blocks = round_up(p->m, 32u) / 32u;
-    const dim3 grid(w.slots / 32u), block(512);
+    const dim3 grid(w.slots / 32u), block(1024);
     if (w.nkk > 2u) hipLaunchKernelGGL((lora_a_kernel<2>), grid, block, 0, s, la);
     else hipLaunchKernelGGL((lora_a_kernel<1>), grid, block, 0, s, la);
     if ((st = launch_status())) return st;
@@ -297,7 +314,7 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   g.sx = reinterpret_cast<const float*>(ws + w.sx);
   g.sw = p->w_scales;
   g.zp = lora ? ws + w.zp : nullptr;
-  g.lora_b = static_cast<const uint16_t*>(p->lora_b);
+  g.bp = lora ? ws + w.bp : nullptr;
   g.lora_scaling = p->lora_scaling;
   g.src_row = routed ? src_row : nullptr;
   g.slot_group = routed ? slot_group : nullptr;
@@ -311,22 +328,34 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   g.tiles_n = n_padded(p->n) / kGemmTileN;
   g.rank = lora ? p->rank : 0u;
   g.nsplit_terms = (p->flags & MI355_W8A8_FLAG_LORA_SPLIT2) ? 2u : 3u;
-  { const char* e = getenv("MI355_W8A8_TILE_MAP"); g.map_mode = e ? (uint32_t)atoi(e) : 0u; }
+  g.map_mode = 0u;
+#ifdef W8A8_DEBUG_VARIANTS
+  { const char* e = getenv("MI355_W8A8_TILE_MAP"); if (e) g.map_mode = (uint32_t)atoi(e); }
+#endif
   if (p->aux_acc) {
     GemmArgs ga = g;
     ga.out = p->aux_acc;
     ga.residual = nullptr;
     if ((st = launch_gemm<kEpiAcc>(ga, 0u, s))) return st;
   }
+  // 256 x 256 tiles (one 8-wave workgroup per CU) once they can fill every CU; below that the
+  // 256 x 128 geometry (two 4-wave workgroups per CU) has twice the tiles to spread.
+  bool wide = (uint64_t)g.tiles_m * (n_padded(p->n) / kWideTileN) >= 256u;
+  if (p->flags & MI355_W8A8_FLAG_TILE_256X128) wide = false;
+  if (p->flags & MI355_W8A8_FLAG_TILE_256X256) wide = true;
+  if (wide) {
+    g.tiles_n = n_padded(p->n) / kWideTileN;
+    return swiglu ? launch_gemm<kEpiSwiglu, kModeWide>(g, w.nkk, s) : launch_gemm<kEpiPlain, kModeWide>(g, w.nkk, s);
+  }
   return swiglu ? launch_gemm<kEpiSwiglu>(g, w.nkk, s) : launch_gemm<kEpiPlain>(g, w.nkk, s);
 }
 
 struct GroupedLayout {
-  uint64_t xq, sx, zp, at, src_row, dst_pos, blk_range, total;
+  uint64_t xq, sx, zp, at, bp, src_row, dst_pos, blk_range, total;
   uint32_t slots, nkk, K_pad, KB, n_steps, steps_per_wave;
 };
 
-GroupedLayout make_grouped_layout(uint32_t m, uint32_t k, uint32_t n_groups, uint32_t rank) {
+GroupedLayout make_grouped_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint32_t rank) {
   GroupedLayout w{};
   w.K_pad = k_padded(k);
   w.KB = w.K_pad / 32u;
@@ -335,7 +364,7 @@ GroupedLayout make_grouped_layout(uint32_t m, uint32_t k, uint32_t n_groups, uin
   w.slots = (uint32_t)((worst + 63ull) / 64ull * 64ull);
   w.nkk = rank_chunks(rank);
   w.n_steps = (k + 63u) / 64u;
-  w.steps_per_wave = (w.n_steps + 7u) / 8u;
+  w.steps_per_wave = (w.n_steps + 15u) / 16u;
   uint64_t off = 0;
   w.xq = off; off += align256((uint64_t)w.slots * w.K_pad);
   w.sx = off; off += align256((uint64_t)w.slots * 4u);
@@ -344,6 +373,7 @@ GroupedLayout make_grouped_layout(uint32_t m, uint32_t k, uint32_t n_groups, uin
   w.blk_range = off; off += align256((uint64_t)(w.slots / 32u) * 4u);
   w.zp = off; off += rank ? align256((uint64_t)(w.slots / 32u) * w.nkk * 3u * kBlockBytes) : 0u;
   w.at = off; off += rank ? align256((uint64_t)n_groups * rank * k * 2u) : 0u;
+  w.bp = off; off += rank ? align256((uint64_t)n_groups * (n_padded(n) / 32u) * w.nkk * kBlockBytes) : 0u;
   w.total = off;
   return w;
 }
@@ -373,7 +403,7 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
   if (overlaps(p->out, out_bytes, p->x, (uint64_t)p->m * p->k * 2u) ||
       overlaps(p->out, out_bytes, p->workspace, p->workspace_bytes))
     return MI355_W8A8_ERR_ALIAS;
-  const GroupedLayout w = make_grouped_layout(p->m, p->k, p->n_groups, p->rank);
+  const GroupedLayout w = make_grouped_layout(p->m, p->k, p->n, p->n_groups, p->rank);
   if (!p->workspace || p->workspace_bytes < w.total) return MI355_W8A8_ERR_WORKSPACE;
   if (reinterpret_cast<uintptr_t>(p->workspace) & 255u) return MI355_W8A8_ERR_ALIGN;
   unsigned char* ws = static_cast<unsigned char*>(p->workspace);
@@ -400,10 +430,22 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
 
   if (lora) {
     uint16_t* at = reinterpret_cast<uint16_t*>(ws + w.at);
-    const uint64_t chunks = (uint64_t)p->n_groups * p->k * ((p->rank + 7u) / 8u);
-    hipLaunchKernelGGL(lora_a_transpose_kernel, dim3((uint32_t)((chunks + 255u) / 256u)), dim3(256), 0, s,
-                       static_cast<const uint16_t*>(p->lora_a), at, p->n_groups, p->k, p->rank);
-    if ((st = launch_status())) return st;
+    {
+      LoraPrepArgs pa{};
+      pa.lora_a = static_cast<const uint16_t*>(p->lora_a);
+      pa.lora_b = static_cast<const uint16_t*>(p->lora_b);
+      pa.at = at;
+      pa.bp = ws + w.bp;
+      pa.M = p->m; pa.K = p->k; pa.N = p->n; pa.n_groups = p->n_groups; pa.r = p->rank; pa.nkk = w.nkk;
+      pa.ncb = n_padded(p->n) / 32u; pa.slots = w.slots;
+      pa.route_blocks = 0;
+      const uint64_t a_items = (uint64_t)p->n_groups * p->k * ((p->rank + 7u) / 8u);
+      const uint64_t b_items = (uint64_t)p->n_groups * pa.ncb * w.nkk * 64u;
+      pa.a_blocks = (uint32_t)((a_items + 1023u) / 1024u);
+      const uint32_t b_blocks = (uint32_t)((b_items + 1023u) / 1024u);
+      hipLaunchKernelGGL(lora_prep_kernel, dim3(pa.a_blocks + b_blocks), dim3(1024), 0, s, pa);
+      if ((st = launch_status())) return st;
+    }
     LoraAArgs la{};
     la.xsrc = static_cast<const uint16_t*>(p->x);
     la.at = at;
@@ -414,7 +456,7 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
     la.M = p->m; la.K = p->k; la.r = p->rank; la.nkk = w.nkk;
     la.steps_per_wave = w.steps_per_wave; la.n_steps = w.n_steps;
     la.n_blocks = w.slots / 32u;
-    const dim3 grid(w.slots / 32u), block(512);
+    const dim3 grid(w.slots / 32u), block(1024);
     if (w.nkk > 2u) hipLaunchKernelGGL((lora_a_kernel<2>), grid, block, 0, s, la);
     else hipLaunchKernelGGL((lora_a_kernel<1>), grid, block, 0, s, la);
     if ((st = launch_status())) return st;
@@ -426,7 +468,7 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
   g.sx = reinterpret_cast<const float*>(ws + w.sx);
   g.sw = p->w_scales;
   g.zp = lora ? ws + w.zp : nullptr;
-  g.lora_b = static_cast<const uint16_t*>(p->lora_b);
+  g.bp = lora ? ws + w.bp : nullptr;
   g.lora_scaling = p->lora_scaling;
   g.src_row = src_row;
   g.slot_group = nullptr;
@@ -445,9 +487,9 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
   if (p->aux_acc) {
     GemmArgs ga = g;
     ga.out = p->aux_acc;
-    if ((st = launch_gemm<kEpiAcc, true>(ga, 0u, s))) return st;
+    if ((st = launch_gemm<kEpiAcc, kModeGrouped>(ga, 0u, s))) return st;
   }
-  return swiglu ? launch_gemm<kEpiSwiglu, true>(g, w.nkk, s) : launch_gemm<kEpiPlain, true>(g, w.nkk, s);
+  return swiglu ? launch_gemm<kEpiSwiglu, kModeGrouped>(g, w.nkk, s) : launch_gemm<kEpiPlain, kModeGrouped>(g, w.nkk, s);
 }
 
 }  // namespace
@@ -551,7 +593,7 @@ uint64_t mi355_w8a8_grouped_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, 
   (void)flags;
   if (validate_common(m, k, n)) return 0;
   if (n_groups == 0 || n_groups > (uint32_t)kMaxGroups || rank > (uint32_t)kMaxRank) return 0;
-  return make_grouped_layout(m, k, n_groups, rank).total;
+  return make_grouped_layout(m, k, n, n_groups, rank).total;
 }
 
 int mi355_w8a8_grouped_v1(const mi355_w8a8_grouped_problem* p, void* stream) {

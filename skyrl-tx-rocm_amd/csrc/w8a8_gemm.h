@@ -24,7 +24,7 @@ struct GemmArgs {
   const float* sx;           // f32 [slots]
   const float* sw;           // f32 [N]
   const unsigned char* zp;   // packed z fragments [slots/32][NKK][3][64 lanes][8 bf16] or null
-  const uint16_t* lora_b;    // bf16 [n_groups, rank, N] or null
+  const unsigned char* bp;   // LoRA B in MFMA operand order [n_groups][N_pad/32][NKK][64 lanes][8 bf16] or null
   const float* lora_scaling; // f32 [n_groups]
   const int32_t* src_row;    // original row of every grouped slot, or null (identity)
   const int32_t* slot_group; // LoRA group (adapter) of every grouped slot, or null (group 0)
@@ -65,66 +65,103 @@ constexpr int kGroupedStages = 4;
 constexpr int kGroupedStageBytes = 36864;  // A: 2 row blocks x 2 k blocks, B: 16 column blocks x 2 k blocks
 constexpr int kGroupedLdsBytes = kGroupedStages * kGroupedStageBytes;
 
-template <int EPI, int NKK, int DBG = 0, bool GROUPED = false>
-__global__ __launch_bounds__(256, GROUPED ? 1 : 2) void w8a8_gemm_kernel(GemmArgs g) {
+// Third geometry, "wide": tile 256 x 256, eight waves (4 x 2, 64 x 128 each, two per SIMD), one
+// workgroup per CU, four 32 KiB stages.  It moves a third less L2 -> LDS traffic per MAC than
+// the 256 x 128 geometry at the price of an epilogue that is not hidden behind a second workgroup.
+constexpr int kWideTileN = 256;
+constexpr int kWideStages = 4;
+constexpr int kWideStageBytes = 32768;
+constexpr int kWideLdsBytes = kWideStages * kWideStageBytes;
+
+enum { kModeDense = 0, kModeGrouped = 1, kModeWide = 2 };
+
+// One tile of the persistent loop.
+struct GemmTile {
+  const unsigned char* Ag;  // packed activation panel of the tile
+  const unsigned char* Bg;  // packed weight of the tile's group
+  const float* swp;         // per-channel scales of the tile's group
+  uint32_t tm, tn;
+  bool valid;
+};
+
+template <int EPI, int NKK, int DBG = 0, int MODE = kModeDense>
+__global__ __launch_bounds__(MODE == kModeWide ? 512 : 256, MODE == kModeDense ? 2 : 1)
+void w8a8_gemm_kernel(GemmArgs g) {
+  constexpr bool GROUPED = MODE == kModeGrouped;
+  constexpr bool WIDE = MODE == kModeWide;
+  constexpr int kWaves = WIDE ? 8 : 4;
+  constexpr uint32_t kRowBlocks = GROUPED ? 2 : 8;                 // 32-row blocks of the activation panel
+  constexpr uint32_t kColBlocks = GROUPED ? 16 : (WIDE ? 8 : 4);   // 32-column blocks of the weight panel
+  constexpr int kStages = GROUPED ? kGroupedStages : (WIDE ? kWideStages : kGemmStages);
+  constexpr int kStageBytes = GROUPED ? kGroupedStageBytes : (WIDE ? kWideStageBytes : kGemmStageBytes);
+  constexpr int kAChunks = kRowBlocks * 2;                              // 1 KiB chunks of A per stage
+  constexpr int kLoadsPerTile = (kAChunks + kColBlocks * 2) / kWaves;   // direct-to-LDS loads per wave per k-tile
+  constexpr bool kLora = (NKK > 0) && (EPI != kEpiAcc);
+  constexpr int kZ = NKK > 0 ? NKK : 1;
+
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wrow = GROUPED ? 0 : (WIDE ? (wave >> 1) : wave);  // wave position along M (64 rows each)
+  const int wcol = GROUPED ? wave : (WIDE ? (wave & 1) : 0);   // wave position along N (128 columns each)
+  const int c = lane & 31, h = lane >> 5;
 
-  // ---- XCD-aware tile mapping: consecutive workgroup ids land on different XCDs, so each
-  // XCD gets a contiguous range of a band-major tile order (GM row tiles x all column tiles).
   const uint32_t total_rows = g.total_rows;
   const uint32_t ntile = g.tiles_m * g.tiles_n;
-  const uint32_t per_xcd = (ntile + 7u) / 8u;
-  const uint32_t t = g.map_mode == 1 ? blockIdx.x : (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
-  if (t >= ntile) return;
-  constexpr uint32_t GM = GROUPED ? 1 : 4;
-  const uint32_t band = t / (GM * g.tiles_n);
-  const uint32_t band_rows = (g.tiles_m - band * GM) < GM ? (g.tiles_m - band * GM) : GM;
-  const uint32_t in_band = t - band * GM * g.tiles_n;
-  const uint32_t tm = band * GM + in_band % band_rows;
-  const uint32_t tn = in_band / band_rows;
-
-  constexpr uint32_t kRowBlocks = GROUPED ? 2 : 8;   // 32-row blocks of the activation panel
-  constexpr uint32_t kColBlocks = GROUPED ? 16 : 4;  // 32-column blocks of the weight panel
-  uint32_t tile_group = 0;
-  if (GROUPED) {
-    const int32_t range = g.blk_range[tm * 2u];
-    if (range < 0) return;  // tile beyond the rows in use
-    tile_group = (uint32_t)range & 0xffffu;
-  }
-  const uint32_t widx = GROUPED ? tile_group / g.groups_per_weight : 0u;
   const uint32_t ncb_total = n_padded(g.N) / 32u;  // column blocks of the packed weight
-  const unsigned char* Ag = g.xq + (size_t)tm * kRowBlocks * g.KB * kBlockBytes;
-  const unsigned char* Bg = g.wp + (size_t)widx * g.w_group_stride;
-  const float* swp = g.sw + (size_t)widx * (GROUPED ? g.N : 0u);
-
-  v16i acc[2][4];
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
-
-  // ---- main loop
-  constexpr int kStages = GROUPED ? kGroupedStages : kGemmStages;
-  constexpr int kStageBytes = GROUPED ? kGroupedStageBytes : kGemmStageBytes;
-  constexpr int kAChunks = kRowBlocks * 2;                    // 1 KiB chunks of A per stage
-  constexpr int kLoadsPerTile = (kAChunks + kColBlocks * 2) / 4;  // direct-to-LDS loads per wave per tile
+  const uint32_t n_out = (EPI == kEpiSwiglu) ? g.N / 2u : g.N;
   const int KT = (int)(g.K_pad / 64u);
-  auto issue = [&](int kt) {
+
+  // ---- persistent tile schedule.  Consecutive workgroup ids land on different XCDs, so each XCD
+  // walks a contiguous range of a band-major tile order (GM row tiles x all column tiles) and the
+  // workgroups of an XCD work on neighbouring tiles at any time (shared panels hit in its L2).
+  const uint32_t per_xcd = (ntile + 7u) / 8u;
+  const uint32_t wgs_per_xcd = gridDim.x >> 3;
+  auto tile_of = [&](uint32_t step) -> GemmTile {
+    GemmTile T{};
+    uint32_t t;
+    if (g.map_mode == 1) {
+      t = blockIdx.x + step * gridDim.x;
+    } else {
+      const uint32_t i = (blockIdx.x >> 3) + step * wgs_per_xcd;
+      t = i < per_xcd ? (blockIdx.x & 7u) * per_xcd + i : ntile;
+    }
+    if (t >= ntile) return T;
+    constexpr uint32_t GM = GROUPED ? 1 : 4;
+    const uint32_t band = t / (GM * g.tiles_n);
+    const uint32_t band_rows = (g.tiles_m - band * GM) < GM ? (g.tiles_m - band * GM) : GM;
+    const uint32_t in_band = t - band * GM * g.tiles_n;
+    T.tm = band * GM + in_band % band_rows;
+    T.tn = in_band / band_rows;
+    uint32_t widx = 0;
+    if (GROUPED) {
+      const int32_t range = g.blk_range[T.tm * 2u];
+      if (range < 0) return T;  // tile beyond the rows in use: nothing to do, but later tiles may exist
+      widx = ((uint32_t)range & 0xffffu) / g.groups_per_weight;
+    }
+    T.Ag = g.xq + (size_t)T.tm * kRowBlocks * g.KB * kBlockBytes;
+    T.Bg = g.wp + (size_t)widx * g.w_group_stride;
+    T.swp = g.sw + (size_t)widx * (GROUPED ? g.N : 0u);
+    T.valid = true;
+    return T;
+  };
+  // number of schedule steps of this workgroup (a grouped schedule may contain empty tiles)
+  uint32_t n_steps;
+  if (g.map_mode == 1) n_steps = blockIdx.x < ntile ? (ntile - blockIdx.x + gridDim.x - 1u) / gridDim.x : 0u;
+  else n_steps = (blockIdx.x >> 3) < per_xcd ? (per_xcd - (blockIdx.x >> 3) + wgs_per_xcd - 1u) / wgs_per_xcd : 0u;
+
+  auto issue = [&](const GemmTile& T, int kt) {
     unsigned char* St = lds + (kt % kStages) * kStageBytes;
 #pragma unroll
     for (int q = 0; q < kLoadsPerTile; ++q) {
-      const int c = wave * kLoadsPerTile + q;  // chunks < kAChunks: A (row block c/2, k block c%2); then B
-      const bool isA = c < kAChunks;
-      uint32_t rb = isA ? (uint32_t)(c >> 1) : tn * kColBlocks + (uint32_t)((c - kAChunks) >> 1);
+      const int ch = wave * kLoadsPerTile + q;  // chunks < kAChunks: A (row block ch/2, k block ch%2); then B
+      const bool isA = ch < kAChunks;
+      uint32_t rb = isA ? (uint32_t)(ch >> 1) : T.tn * kColBlocks + (uint32_t)((ch - kAChunks) >> 1);
       if (!isA && rb >= ncb_total) rb = ncb_total - 1u;  // keep every wave's load count equal
-      const unsigned char* base = isA ? Ag : Bg;
-      const size_t goff = ((size_t)rb * g.KB + (size_t)kt * 2 + (c & 1)) * kBlockBytes + lane * 16;
-      load_1k_to_lds(base + goff, St + c * kBlockBytes);
+      const unsigned char* base = isA ? T.Ag : T.Bg;
+      const size_t goff = ((size_t)rb * g.KB + (size_t)kt * 2 + (ch & 1)) * kBlockBytes + lane * 16;
+      load_1k_to_lds(base + goff, St + ch * kBlockBytes);
     }
   };
   auto read_frags = [&](int kt, int ks, v4i (&af)[2], v4i (&bf)[4]) {
@@ -132,278 +169,282 @@ __global__ __launch_bounds__(256, GROUPED ? 1 : 2) void w8a8_gemm_kernel(GemmArg
     const unsigned char* Bs = As + kAChunks * kBlockBytes;
 #pragma unroll
     for (int i = 0; i < 2; ++i)
-      af[i] = *reinterpret_cast<const v4i*>(As + (((GROUPED ? 0 : wave * 2) + i) * 2 + ks) * kBlockBytes + lane * 16);
+      af[i] = *reinterpret_cast<const v4i*>(As + ((wrow * 2 + i) * 2 + ks) * kBlockBytes + lane * 16);
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      bf[j] = *reinterpret_cast<const v4i*>(Bs + (((GROUPED ? wave * 4 : 0) + j) * 2 + ks) * kBlockBytes + lane * 16);
+      bf[j] = *reinterpret_cast<const v4i*>(Bs + ((wcol * 4 + j) * 2 + ks) * kBlockBytes + lane * 16);
   };
-  auto mfma8 = [&](const v4i (&af)[2], const v4i (&bf)[4]) {
-    if constexpr (DBG == 1) {  // measurement only: no MFMA work, keep the operands alive
-#pragma unroll
-      for (int i = 0; i < 2; ++i) asm volatile("" ::"v"(af[i]), "v"(bf[i]), "v"(bf[i + 2]));
-      return;
-    }
+
+  bool prefetched = false;  // the first kStages-1 k-tiles of the current tile are already in flight
+  for (uint32_t step = 0; step < n_steps; ++step) {
+    const GemmTile T = tile_of(step);
+    if (!T.valid) { prefetched = false; continue; }
+
+    v16i acc[2][4];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
-  };
-
-  v4i fa0[2], fb0[4], fa1[2], fb1[4];
 #pragma unroll
-  for (int st = 0; st < kStages - 1; ++st)
-    if (st < KT) issue(st);
-  if (KT > kStages - 2) wait_vmcnt<(kStages - 2) * kLoadsPerTile>(); else wait_vmcnt<0>();
-  lds_barrier();
-  read_frags(0, 0, fa0, fb0);
-  const int KT_main = KT - (kStages - 1);  // tiles that still have a tile to prefetch
-  int kt = 0;
-  for (; kt < KT_main; ++kt) {
-    // ---- k-step 0 of tile kt: prefetch the k-step 1 fragments and the tile kStages-1 ahead.
-    // The MFMAs lead so that the wait for their operands does not cover the new LDS reads.
-    read_frags(kt, 1, fa1, fb1);
-    if constexpr (DBG < 2) issue(kt + kStages - 1);
-    mfma8(fa0, fb0);
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+    auto mfma8 = [&](const v4i (&af)[2], const v4i (&bf)[4]) {
+      if constexpr (DBG == 1) {  // measurement only: no MFMA work, keep the operands alive
 #pragma unroll
-    for (int q = 0; q < 6; ++q) {
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
-      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // 1 VMEM read
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    // ---- k-step 1: tile kt+1 must have landed before its first fragments are fetched
-    if constexpr (DBG < 2) wait_vmcnt<(kStages - 2) * kLoadsPerTile>();
-    lds_barrier();
-    __builtin_amdgcn_sched_barrier(0);
-    read_frags(kt + 1, 0, fa0, fb0);
-    mfma8(fa1, fb1);
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-#pragma unroll
-    for (int q = 0; q < 6; ++q) {
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    __builtin_amdgcn_sched_barrier(0);
-  }
-  for (; kt < KT; ++kt) {  // drain: nothing left to prefetch
-    read_frags(kt, 1, fa1, fb1);
-    mfma8(fa0, fb0);
-    wait_vmcnt<0>();
-    lds_barrier();
-    if (kt + 1 < KT) read_frags(kt + 1, 0, fa0, fb0);
-    mfma8(fa1, fb1);
-  }
-  lds_barrier();  // every wave is done with the stage buffers; the epilogue reuses the LDS
-
-  // ------------------------------------------------------------------ epilogue
-  // Lane (c = lane % 32, h = lane / 32) owns, in each of its wave's two 32 x 128 strips, the four
-  // consecutive original columns ncol .. ncol+3 (accumulator blocks j = 0..3) of the 16 rows
-  // 8*(v/4) + 4*h + v%4.
-  constexpr bool kLora = (NKK > 0) && (EPI != kEpiAcc);
-  constexpr int kZ = NKK > 0 ? NKK : 1;
-  const int c = lane & 31, h = lane >> 5;
-  const uint32_t m0 = GROUPED ? tm * 64u : tm * 256u + wave * 64u;
-  const uint32_t tcol0 = GROUPED ? tn * 512u + wave * 128u : tn * 128u;  // first column of the wave
-  const uint32_t ncol = tcol0 + 4u * c;
-  const uint32_t n_out = (EPI == kEpiSwiglu) ? g.N / 2u : g.N;
-  const bool full_n = (tcol0 + 128u <= g.N) && ((g.N & 3u) == 0);  // wave-uniform
-  if (GROUPED && tcol0 >= g.N) return;  // wave beyond the last column (after the last barrier)
-  float sw[4] = {0.f, 0.f, 0.f, 0.f};
-  if (EPI != kEpiAcc) {
-    if (full_n) {
-      const float4 s4 = *reinterpret_cast<const float4*>(swp + ncol);
-      sw[0] = s4.x; sw[1] = s4.y; sw[2] = s4.z; sw[3] = s4.w;
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (ncol + j < g.N) sw[j] = swp[ncol + j];
-    }
-  }
-  // LoRA-B staging, private to the wave: bf16 [16*NKK][128] at lds + wave * 16 KiB
-  uint16_t* Bl = reinterpret_cast<uint16_t*>(lds + wave * 16384);
-  int staged = -1;
-
-  auto load_zfrags = [&](uint32_t blk, v8us (&zf)[kZ][3]) {
-    if constexpr (kLora) {
-      const unsigned char* zb = g.zp + (size_t)blk * NKK * 3u * kBlockBytes + lane * 16;
-#pragma unroll
-      for (int kk = 0; kk < NKK; ++kk)
-#pragma unroll
-        for (int s = 0; s < 3; ++s)
-          zf[kk][s] = *reinterpret_cast<const v8us*>(zb + (kk * 3 + s) * kBlockBytes);
-    }
-  };
-
-  auto epilogue_block = [&](auto BI) {
-    constexpr int bi = decltype(BI)::value;
-    const uint32_t pbase = m0 + bi * 32u;
-    if (pbase >= total_rows) return;  // wave-uniform
-    const uint32_t blk = pbase / 32u;
-    if (GROUPED && g.blk_range[blk] < 0) return;  // block beyond the rows in use
-    v8us zf[kZ][3];
-    load_zfrags(blk, zf);
-
-    // rows this lane owns in the block: 8*gq + 4*h + e
-    float sxv[16];
-    uint32_t rowoff[16];  // element offset of the output row, or 0xffffffff for padding rows
-    bool all_rows = true;
-#pragma unroll
-    for (int gq = 0; gq < 4; ++gq) {
-      const uint32_t p4 = pbase + 8u * gq + 4u * h;
-      if (EPI != kEpiAcc) {
-        const float4 s4 = *reinterpret_cast<const float4*>(g.sx + p4);
-        sxv[4 * gq + 0] = s4.x; sxv[4 * gq + 1] = s4.y; sxv[4 * gq + 2] = s4.z; sxv[4 * gq + 3] = s4.w;
+        for (int i = 0; i < 2; ++i) asm volatile("" ::"v"(af[i]), "v"(bf[i]), "v"(bf[i + 2]));
+        return;
       }
-      int src[4];
-      if (g.src_row) {
-        const int4 r4 = *reinterpret_cast<const int4*>(g.src_row + p4);
-        src[0] = r4.x; src[1] = r4.y; src[2] = r4.z; src[3] = r4.w;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
+    };
+
+    // ---- main loop
+    v4i fa0[2], fb0[4], fa1[2], fb1[4];
+    if (!prefetched) {
+#pragma unroll
+      for (int st = 0; st < kStages - 1; ++st)
+        if (st < KT) issue(T, st);
+      if (KT > kStages - 2) wait_vmcnt<(kStages - 2) * kLoadsPerTile>(); else wait_vmcnt<0>();
+    } else {
+      wait_vmcnt<0>();  // prefetch of this tile and the previous tile's stores
+    }
+    lds_barrier();
+    read_frags(0, 0, fa0, fb0);
+    const int KT_main = KT - (kStages - 1);  // k-tiles that still have a k-tile to prefetch
+    int kt = 0;
+    for (; kt < KT_main; ++kt) {
+      // ---- k-step 0 of k-tile kt: prefetch the k-step 1 fragments and the k-tile kStages-1 ahead.
+      // The MFMAs lead so that the wait for their operands does not cover the new LDS reads.
+      read_frags(kt, 1, fa1, fb1);
+      if constexpr (DBG < 2) issue(T, kt + kStages - 1);
+      mfma8(fa0, fb0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+#pragma unroll
+      for (int q = 0; q < 6; ++q) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // 1 VMEM read
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      // ---- k-step 1: k-tile kt+1 must have landed before its first fragments are fetched
+      if constexpr (DBG < 2) wait_vmcnt<(kStages - 2) * kLoadsPerTile>();
+      if constexpr (DBG != 4) lds_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (DBG != 3) read_frags(kt + 1, 0, fa0, fb0);
+      mfma8(fa1, fb1);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+#pragma unroll
+      for (int q = 0; q < 6; ++q) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    for (; kt < KT; ++kt) {  // drain: nothing left to prefetch
+      read_frags(kt, 1, fa1, fb1);
+      mfma8(fa0, fb0);
+      wait_vmcnt<0>();
+      lds_barrier();
+      if (kt + 1 < KT) read_frags(kt + 1, 0, fa0, fb0);
+      mfma8(fa1, fb1);
+    }
+    lds_barrier();  // every wave is done with the stage buffers
+
+    // ---- the next tile's first k-tiles travel while this tile's epilogue runs (no LDS below)
+    prefetched = false;
+    if (step + 1 < n_steps) {
+      const GemmTile Tn = tile_of(step + 1);
+      if (Tn.valid) {
+#pragma unroll
+        for (int st = 0; st < kStages - 1; ++st)
+          if (st < KT) issue(Tn, st);
+        prefetched = true;
+      }
+    }
+
+    // ---------------------------------------------------------------- epilogue
+    // Lane (c = lane % 32, h = lane / 32) owns, in each of its wave's two 32 x 128 strips, the four
+    // consecutive original columns ncol .. ncol+3 (accumulator blocks j = 0..3) of the 16 rows
+    // 8*(v/4) + 4*h + v%4.
+    const uint32_t m0 = GROUPED ? T.tm * 64u : T.tm * 256u + wrow * 64u;
+    const uint32_t tcol0 = T.tn * (kColBlocks * 32u) + wcol * 128u;  // first column of the wave
+    const uint32_t ncol = tcol0 + 4u * c;
+    const bool full_n = (tcol0 + 128u <= g.N) && ((g.N & 3u) == 0);  // wave-uniform
+    if (tcol0 >= g.N) continue;  // wave beyond the last column; it still takes part in the next tile
+    float sw[4] = {0.f, 0.f, 0.f, 0.f};
+    if (EPI != kEpiAcc) {
+      if (full_n) {
+        const float4 s4 = *reinterpret_cast<const float4*>(T.swp + ncol);
+        sw[0] = s4.x; sw[1] = s4.y; sw[2] = s4.z; sw[3] = s4.w;
       } else {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) src[e] = (int)(p4 + e);
-      }
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const bool ok = src[e] >= 0 && src[e] < (int)g.M;
-        all_rows = all_rows && ok;
-        rowoff[4 * gq + e] = ok ? (uint32_t)src[e] * ((EPI == kEpiAcc) ? g.N : n_out) : 0xffffffffu;
+        for (int j = 0; j < 4; ++j)
+          if (ncol + j < g.N) sw[j] = T.swp[ncol + j];
       }
     }
-    const bool fast = full_n && (__builtin_amdgcn_ballot_w64(!all_rows) == 0);  // uniform
 
-    if (EPI == kEpiAcc) {
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        if (!fast && rowoff[v] == 0xffffffffu) continue;
-        int32_t* o = reinterpret_cast<int32_t*>(g.out) + rowoff[v] + ncol;
-        if (fast) {
-          *reinterpret_cast<int4*>(o) = make_int4(acc[bi][0][v], acc[bi][1][v], acc[bi][2][v], acc[bi][3][v]);
-        } else {
-#pragma unroll
-          for (int j = 0; j < 4; ++j)
-            if (ncol + j < g.N) o[j] = acc[bi][j][v];
-        }
-      }
-      return;
-    }
+    auto epilogue_block = [&](auto BI) {
+      constexpr int bi = decltype(BI)::value;
+      const uint32_t pbase = m0 + bi * 32u;
+      if (pbase >= total_rows) return;  // wave-uniform
+      const uint32_t blk = pbase / 32u;
+      if (GROUPED && g.blk_range[blk] < 0) return;  // block beyond the rows in use
+      __builtin_amdgcn_sched_barrier(0);  // keep the blocks' register lifetimes apart
 
-    float y[16][4];
-#pragma unroll
-    for (int v = 0; v < 16; ++v)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) y[v][j] = ((float)acc[bi][j][v] * sxv[v]) * sw[j];
+      // Per-row scale and output offset of the block's 32 rows live in one register each (lane l
+      // holds row l % 32); a lane's 16 rows 8*(v/4) + 4*h + v%4 are fetched with readlane below.
+      const float sx_lane = (EPI != kEpiAcc) ? g.sx[pbase + c] : 0.0f;
+      const int src_lane = g.src_row ? g.src_row[pbase + c] : (int)(pbase + c);
+      const bool row_ok = src_lane >= 0 && src_lane < (int)g.M;
+      const uint32_t off_lane = row_ok ? (uint32_t)src_lane * ((EPI == kEpiAcc) ? g.N : n_out) : 0xffffffffu;
+      const bool fast = full_n && (__builtin_amdgcn_ballot_w64(!row_ok) == 0);  // wave-uniform
 
-    if constexpr (kLora) {
-      // groups (adapters) present in this 32-row block: usually one, two at a group boundary
-      const uint32_t range = g.blk_range ? (uint32_t)g.blk_range[blk] : 0u;
-      const int glo = (int)(range & 0xffffu), ghi = (int)(range >> 16);
-      const int rowgrp = (g.slot_group && ghi > glo) ? g.slot_group[pbase + c] : glo;
-      for (int gi = glo; gi <= ghi; ++gi) {  // wave-uniform
-        if (gi != staged) {
-          // stage B[gi][0:16*NKK][tile columns] as bf16 [16*NKK][128]; LDS operations of one
-          // wave execute in order, so no barrier is needed around this wave-private buffer
-          const uint16_t* Bsrc = g.lora_b + (size_t)gi * g.rank * g.N;
-          for (uint32_t q = (uint32_t)lane; q < NKK * 16u * 16u; q += 64u) {
-            const uint32_t r = q >> 4, cc = (q & 15u) * 8u;
-            v8us val = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (r < g.rank) {
-              const size_t off = (size_t)r * g.N + tcol0 + cc;
-              if ((g.N & 7u) == 0 && tcol0 + cc + 8u <= g.N) {
-                val = *reinterpret_cast<const v8us*>(Bsrc + off);
-              } else {
+      if (EPI == kEpiAcc) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e)
-                  if (tcol0 + cc + e < g.N) val[e] = Bsrc[off + e];
-              }
-            }
-            *reinterpret_cast<v8us*>(Bl + r * 128u + cc) = val;
+        for (int v = 0; v < 16; ++v) {
+          const int r_lo = 8 * (v >> 2) + (v & 3), r_hi = r_lo + 4;
+          const uint32_t off_lo = (uint32_t)__builtin_amdgcn_readlane((int)off_lane, r_lo);
+          const uint32_t off_hi = (uint32_t)__builtin_amdgcn_readlane((int)off_lane, r_hi);
+          const uint32_t rowoff = h ? off_hi : off_lo;
+          if (!fast && rowoff == 0xffffffffu) continue;
+          int32_t* o = reinterpret_cast<int32_t*>(g.out) + rowoff + ncol;
+          if (fast) {
+            *reinterpret_cast<int4*>(o) = make_int4(acc[bi][0][v], acc[bi][1][v], acc[bi][2][v], acc[bi][3][v]);
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              if (ncol + j < g.N) o[j] = acc[bi][j][v];
           }
-          staged = gi;
         }
-        const bool mine = (ghi == glo) || (rowgrp == gi);
-        const float sgrp = g.lora_scaling[gi];
+        return;
+      }
+
+      // Groups (adapters) present in this 32-row block: one, except at a group boundary.  A
+      // boundary block is simply processed once per group; each pass stores only its own rows.
+      const uint32_t range = (kLora && g.blk_range) ? (uint32_t)g.blk_range[blk] : 0u;
+      const int glo = (int)(range & 0xffffu), ghi = (int)(range >> 16);
+      const int grp_lane = (kLora && g.slot_group && ghi > glo) ? g.slot_group[pbase + c] : glo;
+      for (int gi = glo; gi <= ghi; ++gi) {  // wave-uniform
+      // The lane's four columns are processed as two pairs (jp): LoRA MFMAs of the pair (section A),
+      // then dequantize + add + activate per row (section B).  The first pair's packed result waits
+      // in `hold` so that every row is written with one 4- or 8-byte store.
+      uint32_t hold[16];
 #pragma unroll
-        for (int jp = 0; jp < 2; ++jp) {
-          v16f low[2];
+      for (int jp = 0; jp < 2; ++jp) {
+        // ---- section A: lowS[j][v] = s_g * (z @ B_g) for the column pair
+        v16f lowS[2];
+        if constexpr (kLora) {
+          const unsigned char* zb = g.zp + (size_t)blk * NKK * 3u * kBlockBytes + lane * 16;
+          // operand of packed column block cb = tcol0/32 + j: rows 16kk + 8h + 0..7 of column 4c + j
+          const unsigned char* bb0 =
+              g.bp + ((size_t)gi * ncb_total + tcol0 / 32u + 2u * jp) * NKK * kBlockBytes + lane * 16;
+#pragma unroll
+          for (int kk = 0; kk < NKK; ++kk) {
+            v8us zf[3];
+#pragma unroll
+            for (int t3 = 0; t3 < 3; ++t3) zf[t3] = *reinterpret_cast<const v8us*>(zb + (kk * 3 + t3) * kBlockBytes);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              const v8bf bb = __builtin_bit_cast(
+                  v8bf, *reinterpret_cast<const v8us*>(bb0 + ((size_t)j * NKK + kk) * kBlockBytes));
+              v16f cur;
+              if (kk == 0) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) cur[e] = 0.0f;
+              } else {
+                cur = lowS[j];
+              }
+              if (g.nsplit_terms >= 3)
+                cur = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, zf[2]), bb, cur, 0, 0, 0);
+              cur = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, zf[1]), bb, cur, 0, 0, 0);
+              cur = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, zf[0]), bb, cur, 0, 0, 0);
+              lowS[j] = cur;
+            }
+          }
+          const float sgrp = g.lora_scaling[gi];
 #pragma unroll
           for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) low[j][e] = 0.0f;
-#pragma unroll
-          for (int kk = 0; kk < NKK; ++kk) {
-            const v8us zero = {0, 0, 0, 0, 0, 0, 0, 0};
-            const v8us z0 = mine ? zf[kk][0] : zero, z1 = mine ? zf[kk][1] : zero, z2 = mine ? zf[kk][2] : zero;
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-              v8us bfr;
-              const uint32_t col = 4u * c + 2u * jp + j;
-#pragma unroll
-              for (int e = 0; e < 8; ++e) bfr[e] = Bl[(16u * kk + 8u * h + e) * 128u + col];
-              const v8bf bb = __builtin_bit_cast(v8bf, bfr);
-              if (g.nsplit_terms >= 3)
-                low[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, z2), bb, low[j], 0, 0, 0);
-              low[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, z1), bb, low[j], 0, 0, 0);
-              low[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, z0), bb, low[j], 0, 0, 0);
-            }
-          }
-#pragma unroll
-          for (int v = 0; v < 16; ++v)
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-              const float l = low[j][v] * sgrp;
-              y[v][2 * jp + j] = y[v][2 * jp + j] + l;
-            }
+            for (int e = 0; e < 16; ++e) lowS[j][e] = lowS[j][e] * sgrp;
         }
-      }
-    }
 
+        // ---- section B
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      if (!fast && rowoff[v] == 0xffffffffu) continue;
-      if (EPI == kEpiSwiglu) {
-        // (y0, y1) and (y2, y3) are (gate, up) of the product columns ncol/2 and ncol/2 + 1
-        const uint32_t f01 = pack_bf16x2(y[v][0], y[v][1]), f23 = pack_bf16x2(y[v][2], y[v][3]);
-        const float p0 = swiglu_f32(__uint_as_float(f01 << 16), __uint_as_float(f01 & 0xffff0000u));
-        const float p1 = swiglu_f32(__uint_as_float(f23 << 16), __uint_as_float(f23 & 0xffff0000u));
-        uint16_t* o = reinterpret_cast<uint16_t*>(g.out) + rowoff[v] + (ncol >> 1);
-        const uint32_t pk = pack_bf16x2(p0, p1);
-        if (fast) {
-          *reinterpret_cast<uint32_t*>(o) = pk;
-        } else {
-          if ((ncol >> 1) < n_out) o[0] = (uint16_t)(pk & 0xffffu);
-          if ((ncol >> 1) + 1u < n_out) o[1] = (uint16_t)(pk >> 16);
-        }
-      } else {
-        uint16_t* o = reinterpret_cast<uint16_t*>(g.out) + rowoff[v] + ncol;
-        if (fast) {
-          float r0 = y[v][0], r1 = y[v][1], r2 = y[v][2], r3 = y[v][3];
-          if (g.residual) {
-            const uint2 rr = *reinterpret_cast<const uint2*>(g.residual + rowoff[v] + ncol);
-            r0 = r0 + __uint_as_float(rr.x << 16);
-            r1 = r1 + __uint_as_float(rr.x & 0xffff0000u);
-            r2 = r2 + __uint_as_float(rr.y << 16);
-            r3 = r3 + __uint_as_float(rr.y & 0xffff0000u);
+        for (int v = 0; v < 16; ++v) {
+          const int r_lo = 8 * (v >> 2) + (v & 3), r_hi = r_lo + 4;
+          const uint32_t off_lo = (uint32_t)__builtin_amdgcn_readlane((int)off_lane, r_lo);
+          const uint32_t off_hi = (uint32_t)__builtin_amdgcn_readlane((int)off_lane, r_hi);
+          const uint32_t rowoff = h ? off_hi : off_lo;
+          const float sx_lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sx_lane), r_lo));
+          const float sx_hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sx_lane), r_hi));
+          const float sxv = h ? sx_hi : sx_lo;
+          float y0 = ((float)acc[bi][2 * jp][v] * sxv) * sw[2 * jp];
+          float y1 = ((float)acc[bi][2 * jp + 1][v] * sxv) * sw[2 * jp + 1];
+          if constexpr (kLora) {
+            y0 = y0 + lowS[0][v];
+            y1 = y1 + lowS[1][v];
           }
-          *reinterpret_cast<uint2*>(o) = make_uint2(pack_bf16x2(r0, r1), pack_bf16x2(r2, r3));
-        } else {
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            if (ncol + j < g.N) {
-              float yy = y[v][j];
-              if (g.residual) yy = yy + bf16_bits_to_f32(g.residual[rowoff[v] + ncol + j]);
-              o[j] = (uint16_t)(pack_bf16x2(yy, 0.0f) & 0xffffu);
+          bool row_valid = fast || rowoff != 0xffffffffu;
+          if (kLora && ghi > glo) {  // boundary block: this pass owns only the rows of group gi
+            const int g_lo = __builtin_amdgcn_readlane(grp_lane, r_lo), g_hi = __builtin_amdgcn_readlane(grp_lane, r_hi);
+            row_valid = row_valid && ((h ? g_hi : g_lo) == gi);
+          }
+          uint32_t mine_bits;
+          if (EPI == kEpiSwiglu) {
+            // (y0, y1) = (gate, up) of the product column ncol/2 + jp
+            const uint32_t f = pack_bf16x2(y0, y1);
+            mine_bits = __float_as_uint(swiglu_f32(__uint_as_float(f << 16), __uint_as_float(f & 0xffff0000u)));
+          } else {
+            if (g.residual && row_valid) {
+              uint32_t rr;
+              if (fast) {
+                rr = *reinterpret_cast<const uint32_t*>(g.residual + rowoff + ncol + 2u * jp);
+              } else {
+                rr = 0;
+                if (ncol + 2u * jp < g.N) rr |= (uint32_t)g.residual[rowoff + ncol + 2u * jp];
+                if (ncol + 2u * jp + 1u < g.N) rr |= (uint32_t)g.residual[rowoff + ncol + 2u * jp + 1u] << 16;
+              }
+              y0 = y0 + __uint_as_float(rr << 16);
+              y1 = y1 + __uint_as_float(rr & 0xffff0000u);
+            }
+            mine_bits = pack_bf16x2(y0, y1);
+          }
+          if (jp == 0) {
+            hold[v] = mine_bits;
+            continue;
+          }
+          if (!row_valid) continue;
+          if (EPI == kEpiSwiglu) {
+            const uint32_t pk = pack_bf16x2(__uint_as_float(hold[v]), __uint_as_float(mine_bits));
+            uint16_t* o = reinterpret_cast<uint16_t*>(g.out) + rowoff + (ncol >> 1);
+            if (fast) {
+              *reinterpret_cast<uint32_t*>(o) = pk;
+            } else {
+              if ((ncol >> 1) < n_out) o[0] = (uint16_t)(pk & 0xffffu);
+              if ((ncol >> 1) + 1u < n_out) o[1] = (uint16_t)(pk >> 16);
+            }
+          } else {
+            uint16_t* o = reinterpret_cast<uint16_t*>(g.out) + rowoff + ncol;
+            if (fast) {
+              *reinterpret_cast<uint2*>(o) = make_uint2(hold[v], mine_bits);
+            } else {
+              if (ncol + 0u < g.N) o[0] = (uint16_t)(hold[v] & 0xffffu);
+              if (ncol + 1u < g.N) o[1] = (uint16_t)(hold[v] >> 16);
+              if (ncol + 2u < g.N) o[2] = (uint16_t)(mine_bits & 0xffffu);
+              if (ncol + 3u < g.N) o[3] = (uint16_t)(mine_bits >> 16);
             }
           }
         }
       }
-    }
-  };
-  epilogue_block(std::integral_constant<int, 0>{});
-  epilogue_block(std::integral_constant<int, 1>{});
+      }  // groups of the block
+    };
+    epilogue_block(std::integral_constant<int, 0>{});
+    epilogue_block(std::integral_constant<int, 1>{});
+  }
 }
 
 }  // namespace w8a8

@@ -52,11 +52,10 @@ __global__ __launch_bounds__(256) void unpack_weight_kernel(const unsigned char*
 // Out-of-range adapter indices are clamped into range (XLA gather semantics).
 // One workgroup; the order of rows inside a group does not influence any result.
 // ---------------------------------------------------------------------------------------
-__global__ __launch_bounds__(1024) void route_rows_kernel(const int32_t* __restrict__ idx, uint32_t M,
-                                                          uint32_t n_groups, uint32_t slots,
-                                                          int32_t* __restrict__ src_row, int32_t* __restrict__ dst_pos,
-                                                          int32_t* __restrict__ slot_group,
-                                                          int32_t* __restrict__ blk_range) {
+__device__ inline void route_rows_block(const int32_t* __restrict__ idx, uint32_t M, uint32_t n_groups,
+                                        uint32_t slots, int32_t* __restrict__ src_row,
+                                        int32_t* __restrict__ dst_pos, int32_t* __restrict__ slot_group,
+                                        int32_t* __restrict__ blk_range) {
   __shared__ int cnt[kMaxAdapters];
   __shared__ int start[kMaxAdapters + 1];
   __shared__ int cursor[kMaxAdapters];
@@ -273,12 +272,10 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(QuantArgs a) {
 // MFMA operand (8 consecutive k of one rank column) is one 16-byte load.  LoRA parameters
 // are trainable and may change between calls, so this runs per call; it moves n*K*r*2 bytes.
 // ---------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void lora_a_transpose_kernel(const uint16_t* __restrict__ a,
-                                                               uint16_t* __restrict__ at, uint32_t n_groups,
-                                                               uint32_t K, uint32_t r) {
+__device__ inline void lora_a_transpose_item(const uint16_t* __restrict__ a, uint16_t* __restrict__ at,
+                                             uint32_t n_groups, uint32_t K, uint32_t r, uint64_t idx) {
   const uint32_t rc = (r + 7u) / 8u;  // 8-wide rank chunks per k
   const uint64_t total = (uint64_t)n_groups * K * rc;
-  const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= total) return;
   const uint32_t ch = (uint32_t)(idx % rc);
   const uint64_t gk = idx / rc;  // group * K + k
@@ -302,6 +299,63 @@ __global__ __launch_bounds__(256) void lora_a_transpose_kernel(const uint16_t* _
 }
 
 // ---------------------------------------------------------------------------------------
+// LoRA B re-layout: B [n, r, N] -> MFMA B-operand order bp[n][N_pad/32][nkk][64 lanes][8]:
+// lane (c = l % 32, h = l / 32) of packed column block cb holds rows 16 kk + 8 h + 0..7 (zero
+// beyond the rank) of the original column packed_to_orig_col(32 cb + c) (zero beyond N).
+// Like A^T this runs per call because LoRA parameters are trainable.
+// ---------------------------------------------------------------------------------------
+__device__ inline void lora_b_pack_item(const uint16_t* __restrict__ b, unsigned char* __restrict__ bp,
+                                        uint32_t n_groups, uint32_t r, uint32_t N, uint32_t ncb, uint32_t nkk,
+                                        uint64_t idx) {
+  const uint64_t total = (uint64_t)n_groups * ncb * nkk * 64u;  // one 16-byte operand per thread
+  if (idx >= total) return;
+  const uint32_t l = (uint32_t)(idx & 63u);
+  const uint64_t rest = idx >> 6;
+  const uint32_t kk = (uint32_t)(rest % nkk);
+  const uint64_t gc = rest / nkk;
+  const uint32_t cb = (uint32_t)(gc % ncb), grp = (uint32_t)(gc / ncb);
+  const uint32_t col = packed_to_orig_col(cb * 32u + (l & 31u));
+  v8us o = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (col < N) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint32_t row = 16u * kk + 8u * (l >> 5) + e;
+      if (row < r) o[e] = b[((size_t)grp * r + row) * N + col];
+    }
+  }
+  *reinterpret_cast<v8us*>(bp + idx * 16u) = o;
+}
+
+// ---------------------------------------------------------------------------------------
+// One launch for the three independent preparation jobs of a call: adapter routing (block 0
+// when `idx` is given), LoRA A transposition and LoRA B operand packing (the other blocks).
+// ---------------------------------------------------------------------------------------
+struct LoraPrepArgs {
+  const int32_t* idx;        // adapter per row, or null (no routing block)
+  int32_t* src_row; int32_t* dst_pos; int32_t* slot_group; int32_t* blk_range;
+  const uint16_t* lora_a;    // bf16 [n_groups, K, r]
+  const uint16_t* lora_b;    // bf16 [n_groups, r, N]
+  uint16_t* at;              // bf16 [n_groups, r, K]
+  unsigned char* bp;         // packed B operands
+  uint32_t M, K, N, n_groups, r, nkk, ncb, slots, route_blocks, a_blocks;
+};
+
+__global__ __launch_bounds__(1024) void lora_prep_kernel(LoraPrepArgs p) {
+  uint32_t b = blockIdx.x;
+  if (b < p.route_blocks) {
+    route_rows_block(p.idx, p.M, p.n_groups, p.slots, p.src_row, p.dst_pos, p.slot_group, p.blk_range);
+    return;
+  }
+  b -= p.route_blocks;
+  if (b < p.a_blocks) {
+    lora_a_transpose_item(p.lora_a, p.at, p.n_groups, p.K, p.r, (uint64_t)b * 1024u + threadIdx.x);
+    return;
+  }
+  b -= p.a_blocks;
+  lora_b_pack_item(p.lora_b, p.bp, p.n_groups, p.r, p.N, p.ncb, p.nkk, (uint64_t)b * 1024u + threadIdx.x);
+}
+
+// ---------------------------------------------------------------------------------------
 // LoRA-A projection on bf16 MFMA: z[p, :] = n[src_row[p], :] @ A[group(p)]  (float32
 // accumulation of exact bf16 products; skyrl/tx/kernels/quantized_lora.py:300-301 and
 // skyrl/tx/layers/lora.py:150).  One workgroup of 8 waves per 32-row block; the waves take
@@ -321,7 +375,7 @@ struct LoraAArgs {
 };
 
 template <int RB>  // number of 32-wide rank blocks (1 or 2)
-__global__ __launch_bounds__(512) void lora_a_kernel(LoraAArgs a) {
+__global__ __launch_bounds__(1024) void lora_a_kernel(LoraAArgs a) {
   __shared__ float red[4][RB][16][64];
   __shared__ float zs[32][RB * 32 + 1];
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
@@ -346,46 +400,64 @@ __global__ __launch_bounds__(512) void lora_a_kernel(LoraAArgs a) {
   // A block at a group boundary runs once per group with the other groups' rows zeroed.
   for (uint32_t grp = glo; grp <= ghi; ++grp) {
     const bool mine = src >= 0 && rowgrp == grp;
-    for (uint32_t s = s0; s < s1; ++s) {
-      const uint32_t kbase = s * 64u + 32u * h;
-      v8us xa[4], wb[RB][4];
+    const uint16_t* atg = a.at + (size_t)grp * a.r * a.K;
+    // U 64-wide k steps per iteration: all their operand loads go out before the MFMAs
+    constexpr int U = RB == 1 ? 2 : 1;  // 1024 threads leave 128 registers per lane
+    for (uint32_t s = s0; s < s1; s += U) {
+      v8us xa[U][4], wb[U][RB][4];
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const uint32_t k0 = kbase + 8u * t;
-        const v8us zero = {0, 0, 0, 0, 0, 0, 0, 0};
-        xa[t] = (mine && k0 < a.K) ? *reinterpret_cast<const v8us*>(xr + k0) : zero;
+      for (int u = 0; u < U; ++u) {
+        const uint32_t kbase = (s + u) * 64u + 32u * h;
+        const bool step_ok = (s + u) < s1;
 #pragma unroll
-        for (int b = 0; b < RB; ++b) {
-          const uint32_t col = b * 32u + i;
-          wb[b][t] = (col < a.r && k0 < a.K)
-                         ? *reinterpret_cast<const v8us*>(a.at + ((size_t)grp * a.r + col) * a.K + k0)
-                         : zero;
+        for (int t = 0; t < 4; ++t) {
+          const uint32_t k0 = kbase + 8u * t;
+          const v8us zero = {0, 0, 0, 0, 0, 0, 0, 0};
+          const bool ok = step_ok && k0 < a.K;
+          xa[u][t] = (mine && ok) ? *reinterpret_cast<const v8us*>(xr + k0) : zero;
+#pragma unroll
+          for (int b = 0; b < RB; ++b) {
+            const uint32_t col = b * 32u + i;
+            wb[u][b][t] = (col < a.r && ok) ? *reinterpret_cast<const v8us*>(atg + (size_t)col * a.K + k0) : zero;
+          }
         }
       }
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
+      for (int u = 0; u < U; ++u)
 #pragma unroll
-        for (int b = 0; b < RB; ++b)
-          acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, xa[t]),
-                                                           __builtin_bit_cast(v8bf, wb[b][t]), acc[b], 0, 0, 0);
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int b = 0; b < RB; ++b)
+            acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, xa[u][t]),
+                                                             __builtin_bit_cast(v8bf, wb[u][b][t]), acc[b], 0, 0, 0);
     }
   }
-  // fixed-order reduction over the 8 waves: (w + w+4) pairwise, then 0..3 in order
-  if (wave >= 4) {
+  // fixed-order reduction over the 16 waves: waves 4..7, 8..11, 12..15 are added, in that order,
+  // onto waves 0..3, whose four partial sums are then added in wave order
+  for (uint32_t round = 1; round < 4; ++round) {
+    if ((wave >> 2) == round) {
 #pragma unroll
-    for (int b = 0; b < RB; ++b)
+      for (int b = 0; b < RB; ++b)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) red[wave - 4][b][e][lane] = acc[b][e];
+        for (int e = 0; e < 16; ++e) red[wave & 3u][b][e][lane] = acc[b][e];
+    }
+    __syncthreads();
+    if (wave < 4) {
+#pragma unroll
+      for (int b = 0; b < RB; ++b)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[b][e] = acc[b][e] + red[wave][b][e][lane];
+    }
+    __syncthreads();
   }
-  __syncthreads();
   if (wave < 4) {
 #pragma unroll
     for (int b = 0; b < RB; ++b)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) red[wave][b][e][lane] = acc[b][e] + red[wave][b][e][lane];
+      for (int e = 0; e < 16; ++e) red[wave][b][e][lane] = acc[b][e];
   }
   __syncthreads();
-  for (uint32_t q = threadIdx.x; q < RB * 1024u; q += 512u) {
+  for (uint32_t q = threadIdx.x; q < RB * 1024u; q += 1024u) {
     const uint32_t l = q & 63u, e = (q >> 6) & 15u, b = q >> 10;
     float sum = red[0][b][e][l];
 #pragma unroll
@@ -393,7 +465,7 @@ __global__ __launch_bounds__(512) void lora_a_kernel(LoraAArgs a) {
     zs[8u * (e >> 2) + 4u * (l >> 5) + (e & 3u)][b * 32u + (l & 31u)] = sum;
   }
   __syncthreads();
-  for (uint32_t q = threadIdx.x; q < a.nkk * 3u * 64u; q += 512u) {
+  for (uint32_t q = threadIdx.x; q < a.nkk * 3u * 64u; q += 1024u) {
     const uint32_t l = q & 63u, term = (q >> 6) % 3u, kk = q / 192u;
     const uint32_t row = l & 31u, hh = l >> 5;
     v8us o;

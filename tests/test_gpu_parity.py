@@ -229,6 +229,26 @@ def test_run_to_run_determinism(dev):
     assert hashlib.sha256(a.tobytes()).hexdigest() == hashlib.sha256(b.tobytes()).hexdigest()
 
 
+@pytest.mark.parametrize("shape", [
+    dict(m=300, k=512, n=768, n_adapters=4, rank=16, rms=True, swiglu=True),
+    dict(m=515, k=384, n=1000, n_adapters=5, rank=32),
+    dict(m=100, k=256, n=520, n_adapters=3, rank=64, residual=True),
+    dict(m=64, k=128, n=256, n_adapters=0),
+])
+def test_tile_geometries_agree_bitwise(dev, pkg, shape):
+    """The 256 x 128 and 256 x 256 tile geometries compute every element the same way."""
+    shape = dict(shape)
+    m, k, n = shape.pop("m"), shape.pop("k"), shape.pop("n")
+    case = wc.make_case(m, k, n, seed=29, **shape)
+    want = wc.oracle_forward(case)
+    narrow = wc.gpu_forward(case, flags=pkg._native.FLAG_FORCE_TILED | pkg._native.FLAG_TILE_256X128,
+                            return_aux=False)
+    wide = wc.gpu_forward(case, flags=pkg._native.FLAG_FORCE_TILED | pkg._native.FLAG_TILE_256X256,
+                          return_aux=False)
+    assert np.array_equal(narrow.view(np.uint32), wide.view(np.uint32))
+    _assert_close(wide, want, f" wide {m}x{k}x{n}")
+
+
 def test_split2_flag_stays_in_tolerance(dev, pkg):
     case = wc.make_case(256, 512, 512, n_adapters=2, rank=32, seed=15)
     want = wc.oracle_forward(case)
