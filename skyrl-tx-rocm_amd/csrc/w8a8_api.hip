@@ -21,7 +21,7 @@ constexpr uint32_t kMaxN = 1u << 20;
 inline uint64_t align256(uint64_t v) { return (v + 255u) & ~uint64_t(255); }
 
 struct WsLayout {
-  uint64_t xq, sx, xn, zp, at, bp, src_row, dst_pos, slot_group, blk_range, skinny, total;
+  uint64_t xq, sx, xn, zp, at, bp, src_row, dst_pos, slot_group, blk_range, tile_ctr, skinny, total;
   uint32_t slots, nkk, K_pad, KB, n_steps, steps_per_wave;
 };
 
@@ -44,6 +44,7 @@ WsLayout make_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint
   w.dst_pos = off; off += align256((uint64_t)m * 4u);
   w.slot_group = off; off += align256((uint64_t)w.slots * 4u);
   w.blk_range = off; off += align256((uint64_t)(w.slots / 32u) * 4u);
+  w.tile_ctr = off; off += 1024u;  // two sets of eight counters, 64 bytes apart
   w.xn = off; off += rank ? align256((uint64_t)m * k * 2u) : 0u;
   w.zp = off; off += rank ? align256((uint64_t)(w.slots / 32u) * w.nkk * 3u * kBlockBytes) : 0u;
   w.at = off; off += rank ? align256((uint64_t)n_groups * rank * k * 2u) : 0u;
@@ -97,7 +98,7 @@ int launch_gemm_one(const GemmArgs& g, hipStream_t s) {
     hipLaunchKernelGGL((w8a8_gemm_kernel<EPI, NKK, D, MODE>), grid, block, lds_bytes, s, g);     \
     return launch_status();                                                                      \
   }
-    W8A8_DBG(1) W8A8_DBG(3)
+    W8A8_DBG(1) W8A8_DBG(3) W8A8_DBG(5) W8A8_DBG(6)
 #undef W8A8_DBG
   }
 #endif
@@ -284,9 +285,13 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   q.scales_rm = p->aux_x_scales;
   q.xn = (rms && lora) ? reinterpret_cast<uint16_t*>(ws + w.xn) : nullptr;
   q.xn_aux = static_cast<uint16_t*>(p->aux_normalized);
+  q.tile_ctr = reinterpret_cast<uint32_t*>(ws + w.tile_ctr);
   if (!skip_prologue) {
     st = rms ? launch_quant<true>(q, s) : launch_quant<false>(q, s);
     if (st) return st;
+  } else if (!skip_gemm) {  // measurement calls: the tile counters still have to start at zero
+    hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(256), 0, s, q.tile_ctr, 256u);
+    if ((st = launch_status())) return st;
   }
 
   if (lora && !skip_prologue) {
@@ -300,6 +305,7 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
     la.zp = ws + w.zp;
     la.M = p->m; la.K = p->k; la.r = p->rank; la.nkk = w.nkk;
     la.steps_per_wave = w.steps_per_wave; la.n_steps = w.n_steps;
+    la.nterms = (p->flags & MI355_W8A8_FLAG_LORA_SPLIT2) ? 2u : 3u;
     la.n_blocks = round_up(p->m, 32u) / 32u;
     const dim3 grid(w.slots / 32u), block(1024);
     if (w.nkk > 2u) hipLaunchKernelGGL((lora_a_kernel<2>), grid, block, 0, s, la);
@@ -327,16 +333,17 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   g.tiles_m = w.slots / kTileM;
   g.tiles_n = n_padded(p->n) / kGemmTileN;
   g.rank = lora ? p->rank : 0u;
-  g.nsplit_terms = (p->flags & MI355_W8A8_FLAG_LORA_SPLIT2) ? 2u : 3u;
   g.map_mode = 0u;
 #ifdef W8A8_DEBUG_VARIANTS
   { const char* e = getenv("MI355_W8A8_TILE_MAP"); if (e) g.map_mode = (uint32_t)atoi(e); }
 #endif
+  g.tile_ctr = reinterpret_cast<uint32_t*>(ws + w.tile_ctr);
   if (p->aux_acc) {
     GemmArgs ga = g;
     ga.out = p->aux_acc;
     ga.residual = nullptr;
     if ((st = launch_gemm<kEpiAcc>(ga, 0u, s))) return st;
+    g.tile_ctr += 128;  // the second counter set
   }
   // 256 x 256 tiles (one 8-wave workgroup per CU) once they can fill every CU; below that the
   // 256 x 128 geometry (two 4-wave workgroups per CU) has twice the tiles to spread.
@@ -455,6 +462,7 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
     la.zp = ws + w.zp;
     la.M = p->m; la.K = p->k; la.r = p->rank; la.nkk = w.nkk;
     la.steps_per_wave = w.steps_per_wave; la.n_steps = w.n_steps;
+    la.nterms = (p->flags & MI355_W8A8_FLAG_LORA_SPLIT2) ? 2u : 3u;
     la.n_blocks = w.slots / 32u;
     const dim3 grid(w.slots / 32u), block(1024);
     if (w.nkk > 2u) hipLaunchKernelGGL((lora_a_kernel<2>), grid, block, 0, s, la);
@@ -481,7 +489,6 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
   g.tiles_m = w.slots / kGroupedTileM;
   g.tiles_n = (n_padded(p->n) + kGroupedTileN - 1u) / kGroupedTileN;
   g.rank = p->rank;
-  g.nsplit_terms = (p->flags & MI355_W8A8_FLAG_LORA_SPLIT2) ? 2u : 3u;
   g.map_mode = 1;  // row-tile-major order: column tiles of one expert run back to back
   g.groups_per_weight = gpw;
   if (p->aux_acc) {

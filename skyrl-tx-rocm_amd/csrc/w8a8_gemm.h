@@ -24,8 +24,8 @@ struct GemmArgs {
   const float* sx;           // f32 [slots]
   const float* sw;           // f32 [N]
   const unsigned char* zp;   // packed z fragments [slots/32][NKK][3][64 lanes][8 bf16] or null
-  const unsigned char* bp;   // LoRA B in MFMA operand order [n_groups][N_pad/32][NKK][64 lanes][8 bf16] or null
   const float* lora_scaling; // f32 [n_groups]
+  const unsigned char* bp;   // LoRA B in MFMA operand order [n_groups][N_pad/32][NKK][64 lanes][8 bf16] or null
   const int32_t* src_row;    // original row of every grouped slot, or null (identity)
   const int32_t* slot_group; // LoRA group (adapter) of every grouped slot, or null (group 0)
   const int32_t* blk_range;  // per 32-row block: first group | last group << 16, or null
@@ -33,8 +33,9 @@ struct GemmArgs {
   void* out;                 // bf16 [M, n_out] or int32 [M, N]
   uint64_t w_group_stride;   // grouped mode: bytes between the packed weights of two experts
   uint32_t M, N, K_pad, KB, slots, total_rows;
-  uint32_t tiles_m, tiles_n, rank, nsplit_terms, map_mode;
+  uint32_t tiles_m, tiles_n, rank, map_mode;
   uint32_t groups_per_weight; // grouped mode: weight index = group / groups_per_weight
+  uint32_t* tile_ctr;         // 8 zeroed counters, 64 bytes apart (one per XCD), or null: static schedule
 };
 
 // float32 pair -> packed bf16x2 (round to nearest even, v_cvt_pk_bf16_f32)
@@ -118,15 +119,10 @@ void w8a8_gemm_kernel(GemmArgs g) {
   // workgroups of an XCD work on neighbouring tiles at any time (shared panels hit in its L2).
   const uint32_t per_xcd = (ntile + 7u) / 8u;
   const uint32_t wgs_per_xcd = gridDim.x >> 3;
-  auto tile_of = [&](uint32_t step) -> GemmTile {
+  // `i` is a position inside the XCD's range of the tile order.
+  auto tile_at = [&](uint32_t i) -> GemmTile {
     GemmTile T{};
-    uint32_t t;
-    if (g.map_mode == 1) {
-      t = blockIdx.x + step * gridDim.x;
-    } else {
-      const uint32_t i = (blockIdx.x >> 3) + step * wgs_per_xcd;
-      t = i < per_xcd ? (blockIdx.x & 7u) * per_xcd + i : ntile;
-    }
+    const uint32_t t = i < per_xcd ? (blockIdx.x & 7u) * per_xcd + i : ntile;
     if (t >= ntile) return T;
     constexpr uint32_t GM = GROUPED ? 1 : 4;
     const uint32_t band = t / (GM * g.tiles_n);
@@ -146,10 +142,19 @@ void w8a8_gemm_kernel(GemmArgs g) {
     T.valid = true;
     return T;
   };
-  // number of schedule steps of this workgroup (a grouped schedule may contain empty tiles)
-  uint32_t n_steps;
-  if (g.map_mode == 1) n_steps = blockIdx.x < ntile ? (ntile - blockIdx.x + gridDim.x - 1u) / gridDim.x : 0u;
-  else n_steps = (blockIdx.x >> 3) < per_xcd ? (per_xcd - (blockIdx.x >> 3) + wgs_per_xcd - 1u) / wgs_per_xcd : 0u;
+  // Static schedule: position (workgroup index inside the XCD) + step * (workgroups per XCD).
+  // Dynamic schedule (two workgroups per CU): positions come from the XCD's counter, because the
+  // hardware favours the older workgroup of a CU and a static split would leave the younger one
+  // to finish alone.  The result does not depend on which workgroup computes which tile.
+  const bool dyn = MODE == kModeDense && g.tile_ctr != nullptr;
+  uint32_t* const ctr = g.tile_ctr + (blockIdx.x & 7u) * 16u;
+  __shared__ uint32_t dyn_slot[2];
+  uint32_t cur_i = blockIdx.x >> 3, nxt_i = 0;
+  if (dyn) {
+    if (tid == 0) dyn_slot[0] = atomicAdd(ctr, 1u);
+    __syncthreads();
+    cur_i = dyn_slot[0];
+  }
 
   auto issue = [&](const GemmTile& T, int kt) {
     unsigned char* St = lds + (kt % kStages) * kStageBytes;
@@ -176,9 +181,10 @@ void w8a8_gemm_kernel(GemmArgs g) {
   };
 
   bool prefetched = false;  // the first kStages-1 k-tiles of the current tile are already in flight
-  for (uint32_t step = 0; step < n_steps; ++step) {
-    const GemmTile T = tile_of(step);
-    if (!T.valid) { prefetched = false; continue; }
+  for (uint32_t step = 0; cur_i < per_xcd; ++step, cur_i = nxt_i) {
+    const GemmTile T = tile_at(cur_i);
+    nxt_i = cur_i + wgs_per_xcd;
+    if (!T.valid) { prefetched = false; continue; }  // static schedules only (empty grouped tile, range end)
 
     v16i acc[2][4];
 #pragma unroll
@@ -211,6 +217,8 @@ void w8a8_gemm_kernel(GemmArgs g) {
       wait_vmcnt<0>();  // prefetch of this tile and the previous tile's stores
     }
     lds_barrier();
+    uint32_t grabbed = 0;  // next position of a dynamic schedule; it arrives during the main loop
+    if (dyn && tid == 0) grabbed = atomicAdd(ctr, 1u);
     read_frags(0, 0, fa0, fb0);
     const int KT_main = KT - (kStages - 1);  // k-tiles that still have a k-tile to prefetch
     int kt = 0;
@@ -252,12 +260,14 @@ void w8a8_gemm_kernel(GemmArgs g) {
       if (kt + 1 < KT) read_frags(kt + 1, 0, fa0, fb0);
       mfma8(fa1, fb1);
     }
+    if (dyn && tid == 0) dyn_slot[(step + 1u) & 1u] = grabbed;  // the drain loop has waited for it
     lds_barrier();  // every wave is done with the stage buffers
+    if (dyn) nxt_i = dyn_slot[(step + 1u) & 1u];
 
     // ---- the next tile's first k-tiles travel while this tile's epilogue runs (no LDS below)
     prefetched = false;
-    if (step + 1 < n_steps) {
-      const GemmTile Tn = tile_of(step + 1);
+    if (nxt_i < per_xcd) {
+      const GemmTile Tn = tile_at(nxt_i);
       if (Tn.valid) {
 #pragma unroll
         for (int st = 0; st < kStages - 1; ++st)
@@ -286,9 +296,13 @@ void w8a8_gemm_kernel(GemmArgs g) {
           if (ncol + j < g.N) sw[j] = T.swp[ncol + j];
       }
     }
-
     auto epilogue_block = [&](auto BI) {
       constexpr int bi = decltype(BI)::value;
+      if constexpr (DBG == 6) {  // measurement only: no epilogue, keep the accumulators alive
+#pragma unroll
+        for (int j = 0; j < 4; ++j) asm volatile("" ::"v"(acc[bi][j]));
+        return;
+      }
       const uint32_t pbase = m0 + bi * 32u;
       if (pbase >= total_rows) return;  // wave-uniform
       const uint32_t blk = pbase / 32u;
@@ -296,20 +310,19 @@ void w8a8_gemm_kernel(GemmArgs g) {
       __builtin_amdgcn_sched_barrier(0);  // keep the blocks' register lifetimes apart
 
       // Per-row scale and output offset of the block's 32 rows live in one register each (lane l
-      // holds row l % 32); a lane's 16 rows 8*(v/4) + 4*h + v%4 are fetched with readlane below.
+      // holds row l % 32); a lane's 16 rows 8*(v/4) + 4*h + v%4 are fetched across lanes below.
       const float sx_lane = (EPI != kEpiAcc) ? g.sx[pbase + c] : 0.0f;
       const int src_lane = g.src_row ? g.src_row[pbase + c] : (int)(pbase + c);
       const bool row_ok = src_lane >= 0 && src_lane < (int)g.M;
       const uint32_t off_lane = row_ok ? (uint32_t)src_lane * ((EPI == kEpiAcc) ? g.N : n_out) : 0xffffffffu;
       const bool fast = full_n && (__builtin_amdgcn_ballot_w64(!row_ok) == 0);  // wave-uniform
+      const int row_addr = 16 * h;  // byte address (4 * lane) of the lane holding row 4*h
 
       if (EPI == kEpiAcc) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const int r_lo = 8 * (v >> 2) + (v & 3), r_hi = r_lo + 4;
-          const uint32_t off_lo = (uint32_t)__builtin_amdgcn_readlane((int)off_lane, r_lo);
-          const uint32_t off_hi = (uint32_t)__builtin_amdgcn_readlane((int)off_lane, r_hi);
-          const uint32_t rowoff = h ? off_hi : off_lo;
+          const uint32_t rowoff =
+              (uint32_t)__builtin_amdgcn_ds_bpermute(row_addr + 4 * (8 * (v >> 2) + (v & 3)), (int)off_lane);
           if (!fast && rowoff == 0xffffffffu) continue;
           int32_t* o = reinterpret_cast<int32_t*>(g.out) + rowoff + ncol;
           if (fast) {
@@ -358,8 +371,7 @@ void w8a8_gemm_kernel(GemmArgs g) {
               } else {
                 cur = lowS[j];
               }
-              if (g.nsplit_terms >= 3)
-                cur = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, zf[2]), bb, cur, 0, 0, 0);
+              cur = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, zf[2]), bb, cur, 0, 0, 0);
               cur = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, zf[1]), bb, cur, 0, 0, 0);
               cur = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, zf[0]), bb, cur, 0, 0, 0);
               lowS[j] = cur;
@@ -375,24 +387,25 @@ void w8a8_gemm_kernel(GemmArgs g) {
         // ---- section B
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const int r_lo = 8 * (v >> 2) + (v & 3), r_hi = r_lo + 4;
-          const uint32_t off_lo = (uint32_t)__builtin_amdgcn_readlane((int)off_lane, r_lo);
-          const uint32_t off_hi = (uint32_t)__builtin_amdgcn_readlane((int)off_lane, r_hi);
-          const uint32_t rowoff = h ? off_hi : off_lo;
-          const float sx_lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sx_lane), r_lo));
-          const float sx_hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sx_lane), r_hi));
-          const float sxv = h ? sx_hi : sx_lo;
-          float y0 = ((float)acc[bi][2 * jp][v] * sxv) * sw[2 * jp];
-          float y1 = ((float)acc[bi][2 * jp + 1][v] * sxv) * sw[2 * jp + 1];
+          // row 8*(v/4) + 4*h + v%4 of the block: its data sits in that lane (cross-lane read on
+          // the LDS crossbar, which is idle here; no vector-ALU work)
+          const int src_lane_addr = row_addr + 4 * (8 * (v >> 2) + (v & 3));
+          const uint32_t rowoff = (uint32_t)__builtin_amdgcn_ds_bpermute(src_lane_addr, (int)off_lane);
+          const float sxv =
+              __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src_lane_addr, __builtin_bit_cast(int, sx_lane)));
+          const float t0 = (float)acc[bi][2 * jp][v] * sxv;
+          const float t1 = (float)acc[bi][2 * jp + 1][v] * sxv;
+          // same f32 operations, in the same order, as the reference epilogue: a fused
+          // multiply-add here would flip rare bf16 roundings that SwiGLU then amplifies
+          float y0 = t0 * sw[2 * jp];
+          float y1 = t1 * sw[2 * jp + 1];
           if constexpr (kLora) {
             y0 = y0 + lowS[0][v];
             y1 = y1 + lowS[1][v];
           }
           bool row_valid = fast || rowoff != 0xffffffffu;
-          if (kLora && ghi > glo) {  // boundary block: this pass owns only the rows of group gi
-            const int g_lo = __builtin_amdgcn_readlane(grp_lane, r_lo), g_hi = __builtin_amdgcn_readlane(grp_lane, r_hi);
-            row_valid = row_valid && ((h ? g_hi : g_lo) == gi);
-          }
+          if (kLora && ghi > glo)  // boundary block: this pass owns only the rows of group gi
+            row_valid = row_valid && (__builtin_amdgcn_ds_bpermute(src_lane_addr, grp_lane) == gi);
           uint32_t mine_bits;
           if (EPI == kEpiSwiglu) {
             // (y0, y1) = (gate, up) of the product column ncol/2 + jp
@@ -422,7 +435,8 @@ void w8a8_gemm_kernel(GemmArgs g) {
             const uint32_t pk = pack_bf16x2(__uint_as_float(hold[v]), __uint_as_float(mine_bits));
             uint16_t* o = reinterpret_cast<uint16_t*>(g.out) + rowoff + (ncol >> 1);
             if (fast) {
-              *reinterpret_cast<uint32_t*>(o) = pk;
+              if constexpr (DBG == 5) asm volatile("" ::"v"(pk), "v"(o));  // measurement only: no stores
+              else *reinterpret_cast<uint32_t*>(o) = pk;
             } else {
               if ((ncol >> 1) < n_out) o[0] = (uint16_t)(pk & 0xffffu);
               if ((ncol >> 1) + 1u < n_out) o[1] = (uint16_t)(pk >> 16);

@@ -179,12 +179,14 @@ struct QuantArgs {
   uint16_t* xn_aux;        // second copy for the caller or null
   uint16_t* zero_out;      // bf16 [M, zero_cols]: rows without a slot (dst_pos < 0) are zero-filled
   uint32_t zero_cols;
+  uint32_t* tile_ctr;      // 256 words cleared for the GEMM launches' tile counters, or null
 };
 
 template <int NCH, bool RMS>
 __global__ __launch_bounds__(256) void quant_rows_kernel(QuantArgs a) {
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t m = blockIdx.x * 4u + (threadIdx.x >> 6);
+  if (a.tile_ctr && blockIdx.x == 0) a.tile_ctr[threadIdx.x] = 0u;
   if (m >= a.M) return;
   const uint16_t* xr = a.x + (size_t)m * a.K;
   float v[NCH][8];
@@ -326,6 +328,11 @@ __device__ inline void lora_b_pack_item(const uint16_t* __restrict__ b, unsigned
   *reinterpret_cast<v8us*>(bp + idx * 16u) = o;
 }
 
+// Clears `count` 32-bit words (one workgroup).
+__global__ __launch_bounds__(256) void zero_words_kernel(uint32_t* p, uint32_t count) {
+  for (uint32_t i = threadIdx.x; i < count; i += 256u) p[i] = 0u;
+}
+
 // ---------------------------------------------------------------------------------------
 // One launch for the three independent preparation jobs of a call: adapter routing (block 0
 // when `idx` is given), LoRA A transposition and LoRA B operand packing (the other blocks).
@@ -372,6 +379,7 @@ struct LoraAArgs {
   const int32_t* blk_range; // or null
   unsigned char* zp;        // packed z fragments
   uint32_t M, K, r, nkk, steps_per_wave, n_steps, n_blocks;
+  uint32_t nterms;          // bf16 terms carried per value: 3 (exact split of the f32 value) or 2
 };
 
 template <int RB>  // number of 32-wide rank blocks (1 or 2)
@@ -477,7 +485,7 @@ __global__ __launch_bounds__(1024) void lora_a_kernel(LoraAArgs a) {
       const uint32_t b1 = f32_to_bf16_bits(r1);
       const float r2 = r1 - bf16_bits_to_f32(b1);
       const uint32_t b2 = f32_to_bf16_bits(r2);
-      o[e] = (unsigned short)(term == 0 ? b0 : (term == 1 ? b1 : b2));
+      o[e] = (unsigned short)(term == 0 ? b0 : (term == 1 ? b1 : (a.nterms >= 3u ? b2 : 0u)));
     }
     *reinterpret_cast<v8us*>(a.zp + (((size_t)pb * a.nkk + kk) * 3u + term) * kBlockBytes + l * 16u) = o;
   }
