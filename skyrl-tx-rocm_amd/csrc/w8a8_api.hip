@@ -155,33 +155,34 @@ int launch_skinny(const mi355_w8a8_problem* p, unsigned char* xq, float* sx, uin
     if (rms) hipLaunchKernelGGL((skinny_quant_kernel<true>), dim3(p->m), dim3(1024), 0, s, q);
     else hipLaunchKernelGGL((skinny_quant_kernel<false>), dim3(p->m + q.n_z_units), dim3(1024), 0, s, q);
     if ((st = launch_status())) return st;
+    if (lora && rms) {  // the LoRA-A units read the normalized rows the quantizer has just written
+      SkinnyLoraAArgs la{};
+      la.xsrc = xn; la.lora_a = static_cast<const uint16_t*>(p->lora_a); la.idx = p->adapter_indices;
+      la.z_part = q.z_part; la.K = p->k; la.n_adapters = p->n_adapters; la.r = p->rank;
+      la.z_chunks = L.z_chunks; la.z_chunk_k = L.z_chunk_k;
+      hipLaunchKernelGGL(skinny_lora_a_kernel, dim3(p->m * L.z_chunks), dim3(1024), 0, s, la);
+      if ((st = launch_status())) return st;
+    }
   }
   if (p->flags & MI355_W8A8_FLAG_SKIP_GEMM) return MI355_W8A8_OK;
   SkinnyStreamArgs a{};
   a.xq = xq;
   a.wp = static_cast<const unsigned char*>(p->w_packed);
-  a.acc_part = reinterpret_cast<int32_t*>(sws + L.acc_part);
-  a.xsrc = rms ? xn : static_cast<const uint16_t*>(p->x);
-  a.lora_a = static_cast<const uint16_t*>(p->lora_a);
-  a.idx = p->adapter_indices;
-  a.z_part = reinterpret_cast<float*>(sws + L.z_part);
-  a.M = p->m; a.K = p->k; a.KB = KB; a.NB = n_padded(p->n) / 32u;
-  a.ksplit = L.ksplit; a.kb_per_wave = L.kb_per_wave;
-  a.n_adapters = p->n_adapters; a.r = p->rank;
-  a.z_chunks = L.z_chunks; a.z_chunk_k = L.z_chunk_k;
-  a.n_z_units = (lora && rms) ? p->m * L.z_chunks : 0u;
-  hipLaunchKernelGGL(skinny_stream_kernel, dim3(a.n_z_units + a.NB * a.ksplit), dim3(256), 0, s, a);
-  if ((st = launch_status())) return st;
-  SkinnyEpilogueArgs e{};
-  e.acc_part = a.acc_part; e.z_part = a.z_part; e.sx = sx; e.sw = p->w_scales;
-  e.lora_b = lora ? static_cast<const uint16_t*>(p->lora_b) : nullptr;
-  e.lora_scaling = p->lora_scaling; e.idx = p->adapter_indices;
-  e.residual = static_cast<const uint16_t*>(p->residual);
-  e.out = static_cast<uint16_t*>(p->out);
-  e.aux_acc = p->aux_acc;
-  e.M = p->m; e.N = p->n; e.NB = a.NB; e.ksplit = L.ksplit;
-  e.n_adapters = p->n_adapters; e.r = p->rank; e.z_chunks = L.z_chunks;
-  hipLaunchKernelGGL(skinny_epilogue_kernel, dim3((p->n + 255u) / 256u, p->m), dim3(256), 0, s, e);
+  a.z_part = reinterpret_cast<const float*>(sws + L.z_part);
+  a.sx = sx; a.sw = p->w_scales;
+  a.lora_b = lora ? static_cast<const uint16_t*>(p->lora_b) : nullptr;
+  a.lora_scaling = p->lora_scaling; a.idx = p->adapter_indices;
+  a.residual = static_cast<const uint16_t*>(p->residual);
+  a.out = static_cast<uint16_t*>(p->out);
+  a.aux_acc = p->aux_acc;
+  a.M = p->m; a.N = p->n; a.N_pad = n_padded(p->n); a.K = p->k; a.KB = KB;
+  a.pairs_per_wave = L.pairs_per_wave;
+  a.n_adapters = p->n_adapters; a.r = p->rank; a.z_chunks = L.z_chunks;
+  a.n_groups = a.N_pad / 128u;
+  // eight units per 128-column group; groups are dealt to the eight XCD residues of the block index
+  const dim3 grid(((a.n_groups + 7u) / 8u) * 64u), block(kSkinnyStreamThreads);
+  if (p->m > 16u) hipLaunchKernelGGL((skinny_stream_kernel<true>), grid, block, 0, s, a);
+  else hipLaunchKernelGGL((skinny_stream_kernel<false>), grid, block, 0, s, a);
   return launch_status();
 }
 

@@ -98,7 +98,6 @@ void w8a8_gemm_kernel(GemmArgs g) {
   constexpr int kAChunks = kRowBlocks * 2;                              // 1 KiB chunks of A per stage
   constexpr int kLoadsPerTile = (kAChunks + kColBlocks * 2) / kWaves;   // direct-to-LDS loads per wave per k-tile
   constexpr bool kLora = (NKK > 0) && (EPI != kEpiAcc);
-  constexpr int kZ = NKK > 0 ? NKK : 1;
 
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int tid = threadIdx.x;

@@ -1,15 +1,16 @@
 // Skinny-M (decode) path, M <= 32 rows: the weight is streamed exactly once from HBM.
 //   1. skinny_quant_kernel   one workgroup per row: (RMSNorm,) absmax, scale, int8 codes in
 //                            MFMA operand order.
-//   2. skinny_stream_kernel  work units of two kinds share one launch:
-//        - weight units: a wave owns 32 output columns x a K range, loads 1 KiB weight blocks
-//          straight from HBM into MFMA operands (no LDS: every block is used once), the four
-//          waves of a workgroup are reduced through LDS and stored as an int32 partial;
-//        - LoRA-A units: z_part[chunk][m][:] = x[m, chunk] @ A[idx[m]][chunk, :] in float32.
-//   3. skinny_epilogue_kernel  sums the int32 partials (exact, order-free) and the float32 z
-//                            partials (fixed order), applies (float(acc) * sx) * sw
-//                            + s * (z @ B[idx[m]]) + residual and casts to bf16 once.
-// No atomics: results are bit-identical from run to run.
+//                            LoRA-A units ride along: z_part[chunk][m][:] = x[m, chunk] @
+//                            A[idx[m]][chunk, :] in float32 (a launch of their own when they
+//                            need the normalized rows).
+//   2. skinny_stream_kernel  every workgroup owns 16 weight columns for all of K: its eight waves
+//                            stream the weight once from HBM straight into MFMA operands (no LDS:
+//                            every byte is used once), are reduced through LDS, and the workgroup
+//                            finishes its columns: (float(acc) * sx) * sw + s * (z @ B[idx[m]])
+//                            + residual, one bf16 cast.
+// Integer sums are exact and the float32 sums have a fixed order: results are bit-identical
+// from run to run.  No atomics, no data crosses workgroups inside a launch.
 #pragma once
 #include "../../include/mi355_w8a8.h"
 #include "w8a8_device.h"
@@ -17,45 +18,30 @@
 namespace w8a8 {
 
 constexpr int kSkinnyMaxRows = 32;
-constexpr uint32_t kSkinnyMaxKSplit = 8;
-constexpr uint32_t kSkinnyMaxZChunks = 64;
-constexpr uint32_t kSkinnyZChunkK = 512;  // K elements per LoRA-A work unit (per row)
+constexpr uint32_t kSkinnyMaxZChunks = 16;
+constexpr uint32_t kSkinnyZChunkK = 1024;  // K elements per LoRA-A work unit (per row)
 
 struct SkinnyLayout {
-  uint64_t acc_part, z_part, total;
-  uint32_t ksplit, kb_per_wave, z_chunks, z_chunk_k;
+  uint64_t z_part, total;
+  uint32_t pairs_per_wave, z_chunks, z_chunk_k;
 };
 
 inline SkinnyLayout skinny_layout(uint32_t m, uint32_t k, uint32_t n) {
-  (void)m;
+  (void)m; (void)n;
   SkinnyLayout L{};
-  const uint32_t KB = k_padded(k) / 32u;
-  const uint32_t nb = (n + 31u) / 32u;
-  // enough workgroups for ~3 per CU, at least 4 k-blocks per wave
-  uint32_t ks = (768u + nb - 1u) / nb;
-  if (ks < 1u) ks = 1u;
-  if (ks > kSkinnyMaxKSplit) ks = kSkinnyMaxKSplit;
-  while (ks > 1u && KB / (ks * 4u) < 4u) --ks;
-  L.ksplit = ks;
-  L.kb_per_wave = (KB + ks * 4u - 1u) / (ks * 4u);
+  const uint32_t n_pairs = k_padded(k) / 64u;
+  L.pairs_per_wave = (n_pairs + 7u) / 8u;
   uint32_t zc = (k + kSkinnyZChunkK - 1u) / kSkinnyZChunkK;
   uint32_t zk = kSkinnyZChunkK;
   while (zc > kSkinnyMaxZChunks) { zk *= 2u; zc = (k + zk - 1u) / zk; }
   L.z_chunks = zc;
   L.z_chunk_k = zk;
-  L.acc_part = 0;
-  uint64_t off = (uint64_t)kSkinnyMaxKSplit * kSkinnyMaxRows * n_padded(n) * 4u;
-  L.z_part = off;
-  off += (uint64_t)kSkinnyMaxZChunks * kSkinnyMaxRows * kMaxRank * 4u;
-  L.total = off;
+  L.z_part = 0;
+  L.total = (uint64_t)kSkinnyMaxZChunks * kSkinnyMaxRows * kMaxRank * 4u;
   return L;
 }
 
-inline uint64_t skinny_workspace_bytes(uint32_t m, uint32_t n) {
-  (void)m;
-  return (uint64_t)kSkinnyMaxKSplit * kSkinnyMaxRows * n_padded(n) * 4u +
-         (uint64_t)kSkinnyMaxZChunks * kSkinnyMaxRows * kMaxRank * 4u;
-}
+inline uint64_t skinny_workspace_bytes(uint32_t m, uint32_t n) { return skinny_layout(m, 128u, n).total; }
 inline bool skinny_supported() { return true; }
 
 // ---------------------------------------------------------------------------------------
@@ -71,7 +57,7 @@ struct SkinnyQuantArgs {
   uint16_t* xn;          // bf16 [M, K] normalized rows (RMSNorm only) or null
   uint16_t* xn_aux;      // optional copy for the caller
   // LoRA-A work units that share the launch (they need only x, not the codes); with RMSNorm they
-  // would need the normalized rows, so then they run in the stream kernel instead
+  // need the normalized rows and run as a launch of their own
   const uint16_t* lora_a;  // bf16 [n_adapters, K, r] or null
   const int32_t* idx;      // adapter per row or null
   float* z_part;           // f32 [z_chunks][32][kMaxRank]
@@ -139,8 +125,9 @@ __global__ __launch_bounds__(1024) void skinny_quant_kernel(SkinnyQuantArgs a) {
   __shared__ double red_sum[16];
   __shared__ float zw[16][64];
   if (blockIdx.x >= a.M) {
-    skinny_lora_a_unit<1024>(a.x, a.lora_a, a.idx, a.z_part, blockIdx.x - a.M, a.K, a.n_adapters, a.r,
-                             a.z_chunks, a.z_chunk_k, zw);
+    const uint32_t unit = blockIdx.x - a.M;
+    skinny_lora_a_unit<1024>(a.x, a.lora_a, a.idx, a.z_part, unit, a.K, a.n_adapters, a.r, a.z_chunks,
+                             a.z_chunk_k, zw);
     return;
   }
   const uint32_t m = blockIdx.x;
@@ -231,130 +218,168 @@ __global__ __launch_bounds__(1024) void skinny_quant_kernel(SkinnyQuantArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------
-struct SkinnyStreamArgs {
-  const unsigned char* xq;   // packed codes of the single 32-row block
-  const unsigned char* wp;   // packed weight
-  int32_t* acc_part;         // int32 [ksplit][32][Nb*32]
-  const uint16_t* xsrc;      // bf16 [M, K] rows for LoRA-A (x or normalized rows) or null
-  const uint16_t* lora_a;    // bf16 [n_adapters, K, r]
-  const int32_t* idx;        // adapter per row or null
-  float* z_part;             // f32 [z_chunks][32][kMaxRank]
-  uint32_t M, K, KB, NB, ksplit, kb_per_wave, n_adapters, r, z_chunks, z_chunk_k, n_z_units;
+// LoRA-A units as a launch of their own (only when they need the normalized rows of the
+// quantizer launch; otherwise they ride along with it).
+struct SkinnyLoraAArgs {
+  const uint16_t* xsrc; const uint16_t* lora_a; const int32_t* idx; float* z_part;
+  uint32_t K, n_adapters, r, z_chunks, z_chunk_k;
 };
-
-__global__ __launch_bounds__(256) void skinny_stream_kernel(SkinnyStreamArgs a) {
-  __shared__ __attribute__((aligned(16))) int red[3][16][64];
-  __shared__ float zw[4][64];
-  const uint32_t tid = threadIdx.x, lane = tid & 63u;
-  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  if (blockIdx.x < a.n_z_units) {
-    skinny_lora_a_unit<256>(a.xsrc, a.lora_a, a.idx, a.z_part, blockIdx.x, a.K, a.n_adapters, a.r,
-                            a.z_chunks, a.z_chunk_k, zw);
-    return;
-  }
-  // ---- weight unit: column block nb, K split ks; wave w takes k-blocks [kb0, kb1)
-  const uint32_t u = blockIdx.x - a.n_z_units;
-  const uint32_t nb = u % a.NB, ks = u / a.NB;
-  uint32_t kb0 = (ks * 4u + wave) * a.kb_per_wave, kb1 = kb0 + a.kb_per_wave;
-  if (kb1 > a.KB) kb1 = a.KB;
-  const unsigned char* wsrc = a.wp + (size_t)nb * a.KB * kBlockBytes + lane * 16u;
-  const unsigned char* xsrc = a.xq + lane * 16u;
-  v16i acc;
-#pragma unroll
-  for (int e = 0; e < 16; ++e) acc[e] = 0;
-  uint32_t kb = kb0;
-  for (; kb + 8u <= kb1; kb += 8u) {
-    v4i wf[8], xf[8];
-#pragma unroll
-    for (int t = 0; t < 8; ++t) {
-      wf[t] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wsrc + (size_t)(kb + t) * kBlockBytes));
-      xf[t] = *reinterpret_cast<const v4i*>(xsrc + (size_t)(kb + t) * kBlockBytes);
-    }
-#pragma unroll
-    for (int t = 0; t < 8; ++t) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(xf[t], wf[t], acc, 0, 0, 0);
-  }
-  for (; kb < kb1; ++kb) {
-    const v4i wf = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wsrc + (size_t)kb * kBlockBytes));
-    const v4i xf = *reinterpret_cast<const v4i*>(xsrc + (size_t)kb * kBlockBytes);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(xf, wf, acc, 0, 0, 0);
-  }
-  if (wave > 0) {
-#pragma unroll
-    for (int e = 0; e < 16; ++e) red[wave - 1][e][lane] = acc[e];
-  }
-  __syncthreads();
-  if (wave == 0) {
-    const uint32_t c = lane & 31u, h = lane >> 5;
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const int s = acc[e] + red[0][e][lane] + red[1][e][lane] + red[2][e][lane];
-      const uint32_t row = 8u * (e >> 2) + 4u * h + (e & 3u);
-      if (row < a.M) a.acc_part[((size_t)ks * kSkinnyMaxRows + row) * (a.NB * 32u) + nb * 32u + c] = s;
-    }
-  }
+__global__ __launch_bounds__(1024) void skinny_lora_a_kernel(SkinnyLoraAArgs a) {
+  __shared__ float zw[16][64];
+  skinny_lora_a_unit<1024>(a.xsrc, a.lora_a, a.idx, a.z_part, blockIdx.x, a.K, a.n_adapters, a.r, a.z_chunks,
+                           a.z_chunk_k, zw);
 }
 
 // ---------------------------------------------------------------------------------------
-struct SkinnyEpilogueArgs {
-  const int32_t* acc_part;   // int32 [ksplit][32][NB*32], columns in packed order
+constexpr uint32_t kSkinnyStreamWaves = 8;   // waves of a stream workgroup; they split K
+constexpr uint32_t kSkinnyStreamThreads = kSkinnyStreamWaves * 64u;
+
+struct SkinnyStreamArgs {
+  const unsigned char* xq;   // packed codes of the single 32-row block
+  const unsigned char* wp;   // packed weight
   const float* z_part;       // f32 [z_chunks][32][kMaxRank]
   const float* sx;           // f32 [32]
   const float* sw;           // f32 [N]
   const uint16_t* lora_b;    // bf16 [n_adapters, r, N] or null
   const float* lora_scaling;
-  const int32_t* idx;
+  const int32_t* idx;        // adapter per row or null
   const uint16_t* residual;  // bf16 [M, N] or null
   uint16_t* out;             // bf16 [M, N]
   int32_t* aux_acc;          // int32 [M, N] or null
-  uint32_t M, N, NB, ksplit, n_adapters, r, z_chunks;
+  uint32_t M, N, N_pad, K, KB, pairs_per_wave, n_adapters, r, z_chunks, n_groups;
 };
 
-__global__ __launch_bounds__(256) void skinny_epilogue_kernel(SkinnyEpilogueArgs a) {
-  __shared__ float zs[4][kMaxRank];
-  __shared__ float z[kMaxRank];
-  const uint32_t m = blockIdx.y;
-  const uint32_t tid = threadIdx.x;
-  int ad = 0;
-  float sgrp = 0.f;
-  if (a.lora_b) {
-    ad = a.idx ? a.idx[m] : 0;
-    ad = ad < 0 ? 0 : (ad >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad);
-    sgrp = a.lora_scaling[ad];
-    // z[r] = sum over chunks, four interleaved partial sums combined in a fixed order
-    const uint32_t r = tid & 63u, cg = tid >> 6;
-    float s = 0.f;
-#pragma unroll 4
-    for (uint32_t ch = cg; ch < a.z_chunks; ch += 4u) s += a.z_part[((size_t)ch * kSkinnyMaxRows + m) * kMaxRank + r];
-    zs[cg][r] = s;
+// Every workgroup owns 16 packed weight columns for all of K and finishes them itself; nothing
+// crosses workgroups.
+//  * Its eight waves each stream a K range of the weight from HBM straight into
+//    v_mfma_i32_16x16x64_i8 operands (a lane loads its 16 bytes from the 1 KiB fragment blocks:
+//    column c of a block pair's four 16-wide k chunks) and are reduced through LDS.
+//  * Finish: (float(acc) * sx) * sw + s * (z @ B) + residual, one bf16 cast.  z[m][r] is the
+//    fixed-order sum of the LoRA-A partials; the rank sum runs in two fixed halves.
+// Packed column pc of block nb is original column 128*(nb/4) + 4*pc + nb%4, so the eight units of
+// a 128-column group read the same stretches of B; they are given workgroup ids that land on one
+// XCD (ids are dealt round-robin to the XCDs) so that those stretches come from HBM once.
+template <bool ROWS2>  // more than 16 rows: a second MFMA per step for rows 16..31
+__global__ __launch_bounds__(kSkinnyStreamThreads) void skinny_stream_kernel(SkinnyStreamArgs a) {
+  // 64-wide k steps a wave keeps in flight (1 KiB of weight each): 192 KiB per workgroup, one
+  // workgroup per CU
+  constexpr uint32_t kInFlight = ROWS2 ? 16 : 24;
+  constexpr uint32_t kRankSplit = ROWS2 ? 1 : 2;  // threads per output in the finish step
+  __shared__ __attribute__((aligned(16))) int red[kSkinnyStreamWaves][2][4][64];  // 16 KiB
+  __shared__ float zl[kSkinnyMaxRows][kMaxRank];                                 // 8 KiB
+  __shared__ float low_odd[256];
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t slot = blockIdx.x >> 3;
+  const uint32_t grp = (slot >> 3) * 8u + (blockIdx.x & 7u);
+  if (grp >= a.n_groups) return;
+  const uint32_t nb = grp * 4u + ((slot & 7u) >> 1), chalf = slot & 1u;
+  const uint32_t c16 = lane & 15u, q = lane >> 4;        // MFMA operand: column / row c16, k chunk q
+  const uint32_t pc = 16u * chalf + c16;                 // packed column inside block nb
+  // byte offsets inside a pair of 1 KiB blocks: chunk q sits in block q/2, k half q%2
+  const uint32_t w_lane_off = (q >> 1) * kBlockBytes + (pc + 32u * (q & 1u)) * 16u;
+  const uint32_t x_lane_off = (q >> 1) * kBlockBytes + (c16 + 32u * (q & 1u)) * 16u;
+  const unsigned char* wsrc = a.wp + (size_t)nb * a.KB * kBlockBytes + w_lane_off;
+  const unsigned char* xsrc = a.xq + x_lane_off;
+  const uint32_t n_pairs = a.KB >> 1;
+  uint32_t p0 = wave * a.pairs_per_wave, p1 = p0 + a.pairs_per_wave;
+  if (p0 > n_pairs) p0 = n_pairs;
+  if (p1 > n_pairs) p1 = n_pairs;
+
+  // ---- finish step mapping: thread -> output (row frow, packed column pc) and a rank share
+  const uint32_t fe = (tid >> 6) & 3u;
+  const uint32_t frow = (ROWS2 ? 16u * (tid >> 8) : 0u) + 4u * q + fe;
+  const uint32_t rsel = ROWS2 ? 0u : (tid >> 8);  // ranks rsel, rsel + kRankSplit, ...
+  const uint32_t fn = 128u * (nb >> 2) + 4u * pc + (nb & 3u);
+  const bool fvalid = frow < a.M && fn < a.N;
+  const bool lora = a.lora_b != nullptr;
+  const float f_sx = fvalid ? a.sx[frow] : 0.f;
+  const float f_sw = fvalid ? a.sw[fn] : 0.f;
+  const float f_res = (fvalid && a.residual) ? bf16_bits_to_f32(a.residual[(size_t)frow * a.N + fn]) : 0.f;
+  int ad = (fvalid && lora && a.idx) ? a.idx[frow] : 0;
+  ad = ad < 0 ? 0 : (ad >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad);
+  const float f_s = (fvalid && lora) ? a.lora_scaling[ad] : 0.f;
+  const uint16_t* Bp = a.lora_b + ((size_t)ad * a.r + rsel) * a.N + fn;
+  // z[m][r] share of this thread: value index tid (and tid + 512, ...) of the M x rpad values
+  const uint32_t rpad = (a.r + 7u) & ~7u;
+  const uint32_t n_zval = lora ? a.M * rpad : 0u;
+  v4i acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
+  uint32_t base = p0;
+  do {
+    v4i wf[kInFlight], xf[kInFlight], xg[ROWS2 ? kInFlight : 1];
+#pragma unroll
+    for (uint32_t t = 0; t < kInFlight; ++t) {
+      const uint32_t pr = base + t < p1 ? base + t : (p1 ? p1 - 1u : 0u);  // clamped: repeats are skipped below
+      wf[t] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wsrc + (size_t)pr * 2u * kBlockBytes));
+    }
+#pragma unroll
+    for (uint32_t t = 0; t < kInFlight; ++t) {
+      const uint32_t pr = base + t < p1 ? base + t : (p1 ? p1 - 1u : 0u);
+      xf[t] = *reinterpret_cast<const v4i*>(xsrc + (size_t)pr * 2u * kBlockBytes);
+      if constexpr (ROWS2) xg[t] = *reinterpret_cast<const v4i*>(xsrc + (size_t)pr * 2u * kBlockBytes + 256u);
+    }
+#pragma unroll
+    for (uint32_t t = 0; t < kInFlight; ++t) {
+      if (base + t < p1) {  // wave-uniform
+        acc0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[t], wf[t], acc0, 0, 0, 0);
+        if constexpr (ROWS2) acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(xg[t], wf[t], acc1, 0, 0, 0);
+      }
+    }
+    base += kInFlight;
+  } while (base < p1);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    red[wave][0][e][lane] = acc0[e];
+    red[wave][1][e][lane] = acc1[e];
+  }
+  // The low-rank term's loads start only now: issued while the weight stream is in flight they
+  // would be served after it anyway, and here they cost one trip to an idle memory.
+  uint16_t bq[16];
+#pragma unroll
+  for (uint32_t t = 0; t < 16; ++t)
+    bq[t] = (fvalid && lora && rsel + kRankSplit * t < a.r) ? Bp[(size_t)(kRankSplit * t) * a.N] : (uint16_t)0;
+  for (uint32_t zi = tid; zi < n_zval; zi += kSkinnyStreamThreads) {
+    const float* zp = a.z_part + (size_t)(zi / rpad) * kMaxRank + zi % rpad;
+    float zv[kSkinnyMaxZChunks];
+#pragma unroll
+    for (uint32_t ch = 0; ch < kSkinnyMaxZChunks; ++ch)
+      zv[ch] = ch < a.z_chunks ? zp[(size_t)ch * kSkinnyMaxRows * kMaxRank] : 0.f;
+    float s4[4] = {0.f, 0.f, 0.f, 0.f};  // four interleaved partial sums, combined in a fixed order
+#pragma unroll
+    for (uint32_t ch = 0; ch < kSkinnyMaxZChunks; ++ch) s4[ch & 3u] += zv[ch];
+    zl[zi / rpad][zi % rpad] = ((s4[0] + s4[1]) + s4[2]) + s4[3];
   }
   __syncthreads();
-  if (a.lora_b && tid < (uint32_t)kMaxRank) z[tid] = ((zs[0][tid] + zs[1][tid]) + zs[2][tid]) + zs[3][tid];
-  __syncthreads();
-  const uint32_t n = blockIdx.x * 256u + tid;
-  if (n >= a.N) return;
-  const uint32_t pc = orig_to_packed_col(n);
-  int acc = 0;
-#pragma unroll 8
-  for (uint32_t ks = 0; ks < a.ksplit; ++ks) acc += a.acc_part[((size_t)ks * kSkinnyMaxRows + m) * (a.NB * 32u) + pc];
-  if (a.aux_acc) a.aux_acc[(size_t)m * a.N + n] = acc;
-  float y = ((float)acc * a.sx[m]) * a.sw[n];
-  if (a.lora_b) {
-    const uint16_t* Bp = a.lora_b + (size_t)ad * a.r * a.N + n;
-    float low = 0.f;
-    uint32_t r = 0;
-    for (; r + 8u <= a.r; r += 8u) {
-      float bv[8];
+  // ---- finish
+  float low = 0.f;
+  if (fvalid && lora) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) bv[e] = bf16_bits_to_f32(Bp[(size_t)(r + e) * a.N]);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) low = fmaf(z[r + e], bv[e], low);
+    for (uint32_t t = 0; t < 16; ++t) {
+      const uint32_t r = rsel + kRankSplit * t;
+      if (r < a.r) low = fmaf(zl[frow][r], bf16_bits_to_f32(bq[t]), low);
     }
-    for (; r < a.r; ++r) low = fmaf(z[r], bf16_bits_to_f32(Bp[(size_t)r * a.N]), low);
-    const float l = low * sgrp;
+    for (uint32_t r = rsel + kRankSplit * 16u; r < a.r; r += kRankSplit)
+      low = fmaf(zl[frow][r], bf16_bits_to_f32(Bp[(size_t)(r - rsel) * a.N]), low);
+  }
+  if (!ROWS2) {
+    if (rsel == 1u) low_odd[tid & 255u] = low;
+    __syncthreads();
+    if (rsel == 1u) return;
+    low = low + low_odd[tid];
+  }
+  if (!fvalid) return;
+  int sum = 0;
+#pragma unroll
+  for (uint32_t w = 0; w < kSkinnyStreamWaves; ++w) sum += red[w][ROWS2 ? (tid >> 8) : 0u][fe][lane];
+  float y = ((float)sum * f_sx) * f_sw;
+  if (lora) {
+    const float l = low * f_s;
     y = y + l;
   }
-  if (a.residual) y = y + bf16_bits_to_f32(a.residual[(size_t)m * a.N + n]);
-  a.out[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(y);
+  const size_t o = (size_t)frow * a.N + fn;
+  if (a.residual) y = y + f_res;
+  a.out[o] = (uint16_t)f32_to_bf16_bits(y);
+  if (a.aux_acc) a.aux_acc[o] = sum;
 }
 
 }  // namespace w8a8
