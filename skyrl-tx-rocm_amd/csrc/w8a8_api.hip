@@ -274,43 +274,41 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
     if ((st = launch_status())) return st;
   }
 
-  QuantArgs q{};
+  // quantizer and LoRA-A projection: one pass over x
+  QuantLoraArgs q{};
   q.x = static_cast<const uint16_t*>(p->x);
   q.gamma = p->rms_gamma;
   q.eps = p->rms_eps;
   q.M = p->m; q.K = p->k; q.K_pad = w.K_pad; q.KB = w.KB;
-  q.dst_pos = routed ? dst_pos : nullptr;
+  q.n_half_blocks = round_up(p->m, 32u) / 16u;
+  q.src_row = routed ? src_row : nullptr;
+  q.slot_group = routed ? slot_group : nullptr;
+  q.blk_range = routed ? blk_range : nullptr;
   q.xq_packed = ws + w.xq;
   q.sx_slots = reinterpret_cast<float*>(ws + w.sx);
   q.codes_rm = p->aux_x_codes;
   q.scales_rm = p->aux_x_scales;
-  q.xn = (rms && lora) ? reinterpret_cast<uint16_t*>(ws + w.xn) : nullptr;
   q.xn_aux = static_cast<uint16_t*>(p->aux_normalized);
+  q.at = lora ? reinterpret_cast<const uint16_t*>(ws + w.at) : nullptr;
+  q.zp = ws + w.zp;
+  q.r = p->rank; q.nkk = w.nkk;
+  q.nterms = (p->flags & MI355_W8A8_FLAG_LORA_SPLIT2) ? 2u : 3u;
   q.tile_ctr = reinterpret_cast<uint32_t*>(ws + w.tile_ctr);
   if (!skip_prologue) {
-    st = rms ? launch_quant<true>(q, s) : launch_quant<false>(q, s);
-    if (st) return st;
+    const dim3 grid(q.n_half_blocks), block(1024);
+#define W8A8_QL(CB)                                                                   \
+  if (rms) hipLaunchKernelGGL((quant_lora_kernel<CB, true>), grid, block, 0, s, q);   \
+  else hipLaunchKernelGGL((quant_lora_kernel<CB, false>), grid, block, 0, s, q)
+    switch (lora ? w.nkk : 0u) {
+      case 0: W8A8_QL(0); break;
+      case 1: W8A8_QL(1); break;
+      case 2: W8A8_QL(2); break;
+      default: W8A8_QL(4); break;
+    }
+#undef W8A8_QL
+    if ((st = launch_status())) return st;
   } else if (!skip_gemm) {  // measurement calls: the tile counters still have to start at zero
     hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(256), 0, s, q.tile_ctr, 256u);
-    if ((st = launch_status())) return st;
-  }
-
-  if (lora && !skip_prologue) {
-    uint16_t* at = reinterpret_cast<uint16_t*>(ws + w.at);
-    LoraAArgs la{};
-    la.xsrc = rms ? reinterpret_cast<const uint16_t*>(ws + w.xn) : static_cast<const uint16_t*>(p->x);
-    la.at = at;
-    la.src_row = routed ? src_row : nullptr;
-    la.slot_group = routed ? slot_group : nullptr;
-    la.blk_range = routed ? blk_range : nullptr;
-    la.zp = ws + w.zp;
-    la.M = p->m; la.K = p->k; la.r = p->rank; la.nkk = w.nkk;
-    la.steps_per_wave = w.steps_per_wave; la.n_steps = w.n_steps;
-    la.nterms = (p->flags & MI355_W8A8_FLAG_LORA_SPLIT2) ? 2u : 3u;
-    la.n_blocks = round_up(p->m, 32u) / 32u;
-    const dim3 grid(w.slots / 32u), block(1024);
-    if (w.nkk > 2u) hipLaunchKernelGGL((lora_a_kernel<2>), grid, block, 0, s, la);
-    else hipLaunchKernelGGL((lora_a_kernel<1>), grid, block, 0, s, la);
     if ((st = launch_status())) return st;
   }
 

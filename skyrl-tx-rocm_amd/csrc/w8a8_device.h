@@ -53,12 +53,15 @@ __host__ __device__ inline size_t packed_offset(uint32_t r, uint32_t k, uint32_t
 
 __device__ inline float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
 
-// float -> bf16 bits, round to nearest even (finite inputs; NaN stays NaN)
-__device__ inline uint32_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
-  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+// float pair -> packed bf16x2, round to nearest even (one v_cvt_pk_bf16_f32; NaN stays NaN)
+__device__ inline uint32_t pack_bf16x2(float lo, float hi) {
+  typedef float v2f __attribute__((ext_vector_type(2)));
+  typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+  const v2f v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, v2bf));
 }
+// float -> bf16 bits, round to nearest even
+__device__ inline uint32_t f32_to_bf16_bits(float f) { return pack_bf16x2(f, 0.0f) & 0xffffu; }
 __device__ inline float bf16_round_f32(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
 
 __device__ inline float wave_max(float v) {

@@ -38,14 +38,6 @@ struct GemmArgs {
   uint32_t* tile_ctr;         // 8 zeroed counters, 64 bytes apart (one per XCD), or null: static schedule
 };
 
-// float32 pair -> packed bf16x2 (round to nearest even, v_cvt_pk_bf16_f32)
-__device__ inline uint32_t pack_bf16x2(float lo, float hi) {
-  typedef float v2f __attribute__((ext_vector_type(2)));
-  typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
-  v2f v = {lo, hi};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, v2bf));
-}
-
 // silu(g) * u with g, u already rounded to bf16 (x * logistic(x), exp and reciprocal in
 // hardware precision: 1 ulp each)
 __device__ inline float swiglu_f32(float g, float u) {

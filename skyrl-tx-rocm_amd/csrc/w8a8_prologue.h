@@ -491,4 +491,303 @@ __global__ __launch_bounds__(1024) void lora_a_kernel(LoraAArgs a) {
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Quantizer and LoRA-A projection in one pass over x (the dense path's prologue).
+// One workgroup of 16 waves per 16 grouped slots (half a 32-row block):
+//   1. wave w owns slot row w: (RMSNorm statistics,) absmax of the (normalized) row -> scale;
+//   2. the waves split K in 32-wide blocks; lane (i = lane % 16, q = lane / 16) takes the 8 values
+//      k = 32 kb + 8 q .. +7 of row i, normalizes them exactly as step 1 did, and uses them twice:
+//      as int8 codes written into the activation's 1 KiB fragment block, and as the A operand of
+//      v_mfma_f32_16x16x32_bf16 against the transposed LoRA A of the row's group, so the
+//      normalized rows never travel through memory;
+//   3. the waves' z tiles are added in a fixed order, split exactly into three bf16 terms and
+//      stored in the operand order the GEMM epilogue reads (see lora_a_kernel).
+// Arithmetic follows quant_rows_kernel (skyrl/tx/kernels/quantized_lora.py:199-212 and the
+// RMSNorm of bf16_rms_gate_up_lora_swiglu.py:299-303) operation for operation.
+// ---------------------------------------------------------------------------------------
+struct QuantLoraArgs {
+  const uint16_t* x;        // bf16 [M, K]
+  const float* gamma;       // f32 [K] (RMS only)
+  float eps;
+  uint32_t M, K, K_pad, KB, n_half_blocks;  // n_half_blocks = ceil(M / 16)
+  const int32_t* src_row;   // original row of a slot, or null (identity)
+  const int32_t* slot_group;// or null
+  const int32_t* blk_range; // per 32-slot block, or null (group 0)
+  unsigned char* xq_packed; // packed codes [slots/32][KB][1 KiB]
+  float* sx_slots;          // f32 [slots]
+  int8_t* codes_rm;         // row-major codes [M, K] or null
+  float* scales_rm;         // f32 [M] or null
+  uint16_t* xn_aux;         // bf16 [M, K] normalized rows for the caller, or null
+  const uint16_t* at;       // bf16 [n_groups, r, K] or null (CB == 0)
+  unsigned char* zp;        // packed z fragments
+  uint32_t r, nkk, nterms;
+  uint32_t* tile_ctr;       // 256 words cleared for the GEMM launches' tile counters, or null
+};
+
+template <int CB, bool RMS>  // CB: 16-wide rank blocks (0 = no LoRA, 1, 2, 4)
+__global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
+  constexpr int kCB = CB > 0 ? CB : 1;
+  __shared__ float row_inv[16], row_scale[16];
+  __shared__ int row_src[16];
+  __shared__ float red[8][kCB][4][64];     // wave tiles on their way to waves 0..7, then 0..3
+  __shared__ float zs[16][kCB * 16 + 1];
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t hb = blockIdx.x;  // half block: slots 16 hb .. 16 hb + 15
+  if (a.tile_ctr && hb == 0 && tid < 256u) a.tile_ctr[tid] = 0u;
+  if (hb >= a.n_half_blocks) return;
+  const uint32_t pb = hb >> 1, half16 = hb & 1u;
+
+  // ---- 1. row statistics: wave w, slot row w
+  {
+    const uint32_t p = hb * 16u + wave;
+    int src = a.src_row ? a.src_row[p] : (int)p;
+    if (src < 0 || src >= (int)a.M) src = -1;
+    float inv = 1.0f, amax = 0.0f;
+    if (src >= 0) {
+      const uint16_t* xr = a.x + (size_t)src * a.K;
+      // eight 16-byte loads of the row are in flight at a time
+      if (RMS) {
+        double ss = 0.0;
+        for (uint32_t kbase = 0; kbase < a.K; kbase += 4096u) {
+          uint4 raw[8];
+#pragma unroll
+          for (uint32_t u = 0; u < 8; ++u) {
+            const uint32_t k0 = kbase + (u * 64u + lane) * 8u;
+            raw[u] = k0 < a.K ? *reinterpret_cast<const uint4*>(xr + k0) : make_uint4(0, 0, 0, 0);
+          }
+#pragma unroll
+          for (uint32_t u = 0; u < 8; ++u) {
+            const uint32_t w[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              // the square of a bf16 value is exact in double, so the fused form rounds like mul + add
+              const double lo = (double)__uint_as_float(w[e] << 16), hi = (double)__uint_as_float(w[e] & 0xffff0000u);
+              ss = __builtin_fma(lo, lo, ss);
+              ss = __builtin_fma(hi, hi, ss);
+            }
+          }
+        }
+        ss = wave_sum(ss);
+        const float var = (float)(ss / (double)a.K);
+        inv = 1.0f / sqrtf(var + a.eps);
+      }
+      for (uint32_t kbase = 0; kbase < a.K; kbase += 4096u) {
+        uint4 raw[8];
+#pragma unroll
+        for (uint32_t u = 0; u < 8; ++u) {
+          const uint32_t k0 = kbase + (u * 64u + lane) * 8u;
+          raw[u] = k0 < a.K ? *reinterpret_cast<const uint4*>(xr + k0) : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 8; ++u) {
+          const uint32_t k0 = kbase + (u * 64u + lane) * 8u;
+          const uint32_t w[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
+          float g[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f};
+          if (RMS && k0 < a.K) {
+            const float4 g0 = *reinterpret_cast<const float4*>(a.gamma + k0);
+            const float4 g1 = *reinterpret_cast<const float4*>(a.gamma + k0 + 4);
+            g[0] = g0.x; g[1] = g0.y; g[2] = g0.z; g[3] = g0.w; g[4] = g1.x; g[5] = g1.y; g[6] = g1.z; g[7] = g1.w;
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float v0 = __uint_as_float(w[e] << 16), v1 = __uint_as_float(w[e] & 0xffff0000u);
+            if (RMS) {
+              float t0 = v0 * inv, t1 = v1 * inv;
+              t0 = t0 * g[2 * e];
+              t1 = t1 * g[2 * e + 1];
+              const uint32_t pk = pack_bf16x2(t0, t1);
+              v0 = __uint_as_float(pk << 16);
+              v1 = __uint_as_float(pk & 0xffff0000u);
+            }
+            amax = fmaxf(amax, fmaxf(fabsf(v0), fabsf(v1)));
+          }
+        }
+      }
+      amax = wave_max(amax);
+    }
+    const float scale = amax > 0.0f ? amax / 127.0f : 1.0f;
+    if (lane == 0) {
+      row_inv[wave] = inv;
+      row_scale[wave] = scale;
+      row_src[wave] = src;
+      a.sx_slots[p] = scale;
+      if (a.scales_rm && src >= 0) a.scales_rm[src] = scale;
+    }
+  }
+  __syncthreads();
+
+  // ---- 2. codes and z
+  const uint32_t i = lane & 15u, q = lane >> 4;
+  const int src = row_src[i];
+  const float inv = row_inv[i], scale = row_scale[i];
+  const float rscale = __builtin_amdgcn_rcpf(scale);
+  const uint16_t* xr = a.x + (size_t)(src < 0 ? 0 : src) * a.K;
+  const uint32_t range = (CB > 0 && a.blk_range) ? (uint32_t)a.blk_range[pb] : 0u;
+  const uint32_t glo = range & 0xffffu, ghi = range >> 16;
+  const uint32_t rowgrp = (CB > 0 && a.slot_group && ghi > glo) ? (uint32_t)a.slot_group[hb * 16u + i] : glo;
+  v4f acc[kCB];
+#pragma unroll
+  for (int b = 0; b < kCB; ++b) acc[b] = v4f{0.f, 0.f, 0.f, 0.f};
+  // fragment block byte offset of this lane's 8 codes: row 16*half16 + i, k half q/2, byte 8*(q%2)
+  const uint32_t code_off = (16u * half16 + i + 32u * (q >> 1)) * 16u + 8u * (q & 1u);
+  for (uint32_t kb0 = wave; kb0 < a.KB; kb0 += 32u) {  // two k-blocks per round, all loads first
+    uint4 raw2[2];
+    float4 gm[2][2];
+    v4i wpre[2][kCB];
+#pragma unroll
+    for (uint32_t u = 0; u < 2; ++u) {
+      const uint32_t kb = kb0 + 16u * u;
+      const uint32_t k0 = kb * 32u + q * 8u;
+      const bool inK = kb < a.KB && k0 < a.K;
+      raw2[u] = (inK && src >= 0) ? *reinterpret_cast<const uint4*>(xr + k0) : make_uint4(0, 0, 0, 0);
+      if (RMS) {
+        gm[u][0] = inK ? *reinterpret_cast<const float4*>(a.gamma + k0) : make_float4(0.f, 0.f, 0.f, 0.f);
+        gm[u][1] = inK ? *reinterpret_cast<const float4*>(a.gamma + k0 + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+      if constexpr (CB > 0) {
+        const uint16_t* atg = a.at + (size_t)glo * a.r * a.K + k0;
+#pragma unroll
+        for (int b = 0; b < CB; ++b) {
+          const uint32_t col = b * 16u + i;
+          wpre[u][b] = (inK && col < a.r) ? *reinterpret_cast<const v4i*>(atg + (size_t)col * a.K) : v4i{0, 0, 0, 0};
+        }
+      }
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < 2; ++u) {
+      const uint32_t kb = kb0 + 16u * u;
+      if (kb >= a.KB) break;  // wave-uniform
+      const uint32_t k0 = kb * 32u + q * 8u;
+      const bool live = src >= 0 && k0 < a.K;  // K is a multiple of 8
+      uint32_t nb[4] = {raw2[u].x, raw2[u].y, raw2[u].z, raw2[u].w};  // the (normalized) values as bf16 pairs
+      float v[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        v[e] = (e & 1) ? __uint_as_float(nb[e >> 1] & 0xffff0000u) : __uint_as_float(nb[e >> 1] << 16);
+      if (RMS && live) {
+        const float g[8] = {gm[u][0].x, gm[u][0].y, gm[u][0].z, gm[u][0].w, gm[u][1].x, gm[u][1].y, gm[u][1].z, gm[u][1].w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float t0 = v[2 * e] * inv, t1 = v[2 * e + 1] * inv;
+          t0 = t0 * g[2 * e];
+          t1 = t1 * g[2 * e + 1];
+          nb[e] = pack_bf16x2(t0, t1);
+          v[2 * e] = __uint_as_float(nb[e] << 16);
+          v[2 * e + 1] = __uint_as_float(nb[e] & 0xffff0000u);
+        }
+        if (a.xn_aux)
+          *reinterpret_cast<uint4*>(a.xn_aux + (size_t)src * a.K + k0) = make_uint4(nb[0], nb[1], nb[2], nb[3]);
+      }
+      // codes = rint(v / scale) with the correctly rounded quotient.  v * (1 / scale) with the
+      // hardware reciprocal is within 3 * 2^-24 * 128 < 2.3e-5 of it, so both round to the same
+      // integer unless the product lies that close to a tie; those cases (and scales outside the
+      // reciprocal's safe range) are redone with the division.
+      float c[8];
+      bool redo = !(scale > 1e-30f && scale < 1e30f);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float t = v[e] * rscale;
+        c[e] = rintf(t);
+        redo = redo || (fabsf(t - c[e]) > 0.4999f);
+      }
+      if (__builtin_amdgcn_ballot_w64(redo) != 0) {  // wave-uniform
+#pragma unroll
+        for (int e = 0; e < 8; ++e) c[e] = rintf(v[e] / scale);
+      }
+      uint32_t lo = 0, hi = 0;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float cc = fminf(fmaxf(c[e], -127.0f), 127.0f);
+        const uint32_t b = (uint32_t)(int)cc & 0xffu;
+        if (e < 4) lo |= b << (8 * e); else hi |= b << (8 * (e - 4));
+      }
+      if (!live) { lo = 0; hi = 0; }
+      if (live && a.codes_rm) *reinterpret_cast<uint2*>(a.codes_rm + (size_t)src * a.K + k0) = make_uint2(lo, hi);
+      *reinterpret_cast<uint2*>(a.xq_packed + ((size_t)pb * a.KB + kb) * kBlockBytes + code_off) = make_uint2(lo, hi);
+      if constexpr (CB > 0) {
+        // A block at a group boundary runs once per group with the other groups' rows zeroed.
+        for (uint32_t grp = glo; grp <= ghi; ++grp) {
+          v4i xa = {0, 0, 0, 0};
+          if (live && rowgrp == grp) xa = v4i{(int)nb[0], (int)nb[1], (int)nb[2], (int)nb[3]};
+          const uint16_t* atg = a.at + (size_t)grp * a.r * a.K + k0;
+#pragma unroll
+          for (int b = 0; b < CB; ++b) {
+            v4i wb = wpre[u][b];
+            if (grp != glo) {  // wave-uniform, boundary blocks only
+              const uint32_t col = b * 16u + i;
+              wb = (col < a.r && k0 < a.K) ? *reinterpret_cast<const v4i*>(atg + (size_t)col * a.K) : v4i{0, 0, 0, 0};
+            }
+            acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, xa),
+                                                             __builtin_bit_cast(v8bf, wb), acc[b], 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+  if constexpr (CB == 0) return;
+
+  // ---- 3. fixed-order sum of the 16 wave tiles: 8..15 onto 0..7, 4..7 onto 0..3, then 0+1+2+3
+  if (wave >= 8u) {
+#pragma unroll
+    for (int b = 0; b < kCB; ++b)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) red[wave - 8u][b][e][lane] = acc[b][e];
+  }
+  __syncthreads();
+  if (wave < 8u) {
+#pragma unroll
+    for (int b = 0; b < kCB; ++b)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[b][e] = acc[b][e] + red[wave][b][e][lane];
+  }
+  __syncthreads();
+  if (wave >= 4u && wave < 8u) {
+#pragma unroll
+    for (int b = 0; b < kCB; ++b)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) red[wave - 4u][b][e][lane] = acc[b][e];
+  }
+  __syncthreads();
+  if (wave < 4u) {
+#pragma unroll
+    for (int b = 0; b < kCB; ++b)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[b][e] = acc[b][e] + red[wave][b][e][lane];
+  }
+  __syncthreads();
+  if (wave < 4u) {
+#pragma unroll
+    for (int b = 0; b < kCB; ++b)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) red[wave][b][e][lane] = acc[b][e];
+  }
+  __syncthreads();
+  // MFMA result layout: lane l holds column l % 16 and rows 4 * (l / 16) + e
+  for (uint32_t t = tid; t < (uint32_t)kCB * 256u; t += 1024u) {
+    const uint32_t l = t & 63u, e = (t >> 6) & 3u, b = t >> 8;
+    const float sum = ((red[0][b][e][l] + red[1][b][e][l]) + red[2][b][e][l]) + red[3][b][e][l];
+    zs[4u * (l >> 4) + e][b * 16u + (l & 15u)] = sum;
+  }
+  __syncthreads();
+  // zp[pb][kk][term][lane64][8]: lane = row % 32 + 32 * hh holds rank columns 16 kk + 8 hh + 0..7
+  for (uint32_t t = tid; t < a.nkk * 3u * 32u; t += 1024u) {
+    const uint32_t row = t & 15u, hh = (t >> 4) & 1u, term = (t >> 5) % 3u, kk = t / 96u;
+    v8us o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint32_t col = 16u * kk + 8u * hh + e;
+      const float z = col < (uint32_t)kCB * 16u ? zs[row][col] : 0.0f;
+      const uint32_t b0 = f32_to_bf16_bits(z);
+      const float r1 = z - bf16_bits_to_f32(b0);
+      const uint32_t b1 = f32_to_bf16_bits(r1);
+      const float r2 = r1 - bf16_bits_to_f32(b1);
+      const uint32_t b2 = f32_to_bf16_bits(r2);
+      o[e] = (unsigned short)(term == 0 ? b0 : (term == 1 ? b1 : (a.nterms >= 3u ? b2 : 0u)));
+    }
+    const uint32_t l64 = 16u * half16 + row + 32u * hh;
+    *reinterpret_cast<v8us*>(a.zp + (((size_t)pb * a.nkk + kk) * 3u + term) * kBlockBytes + l64 * 16u) = o;
+  }
+}
+
 }  // namespace w8a8
