@@ -88,14 +88,31 @@ __device__ inline void skinny_lora_a_unit(const uint16_t* __restrict__ xsrc, con
   uint32_t k_end = k_begin + z_chunk_k;
   if (k_end > K) k_end = K;
   if (q < rch) {
-    for (uint32_t k = k_begin + kl; k < k_end; k += kpt) {
-      const float xv = bf16_bits_to_f32(xr[k]);
-      const uint16_t* src = Ar + (size_t)k * r + q * 8u;
-      if ((r & 7u) == 0) {
-        const v8us w = *reinterpret_cast<const v8us*>(src);
+    if ((r & 7u) == 0) {
+      // four rows of A per round, their loads issued together (same order of additions as a plain loop)
+      for (uint32_t k = k_begin + kl; k < k_end; k += 4u * kpt) {
+        v8us w[4];
+        float xv[4];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) accz[e] = fmaf(xv, bf16_bits_to_f32(w[e]), accz[e]);
-      } else {
+        for (uint32_t u = 0; u < 4; ++u) {
+          const uint32_t ku = k + u * kpt;
+          const bool in = ku < k_end;
+          const v8us zero = {0, 0, 0, 0, 0, 0, 0, 0};
+          w[u] = in ? *reinterpret_cast<const v8us*>(Ar + (size_t)ku * r + q * 8u) : zero;
+          xv[u] = in ? bf16_bits_to_f32(xr[ku]) : 0.f;
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+          if (k + u * kpt < k_end) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) accz[e] = fmaf(xv[u], bf16_bits_to_f32(w[u][e]), accz[e]);
+          }
+        }
+      }
+    } else {
+      for (uint32_t k = k_begin + kl; k < k_end; k += kpt) {
+        const float xv = bf16_bits_to_f32(xr[k]);
+        const uint16_t* src = Ar + (size_t)k * r + q * 8u;
 #pragma unroll
         for (int e = 0; e < 8; ++e)
           if (q * 8u + e < r) accz[e] = fmaf(xv, bf16_bits_to_f32(src[e]), accz[e]);
@@ -293,13 +310,14 @@ __global__ __launch_bounds__(kSkinnyStreamThreads) void skinny_stream_kernel(Ski
   const uint32_t fn = 128u * (nb >> 2) + 4u * pc + (nb & 3u);
   const bool fvalid = frow < a.M && fn < a.N;
   const bool lora = a.lora_b != nullptr;
-  const float f_sx = fvalid ? a.sx[frow] : 0.f;
-  const float f_sw = fvalid ? a.sw[fn] : 0.f;
-  const float f_res = (fvalid && a.residual) ? bf16_bits_to_f32(a.residual[(size_t)frow * a.N + fn]) : 0.f;
-  int ad = (fvalid && lora && a.idx) ? a.idx[frow] : 0;
-  ad = ad < 0 ? 0 : (ad >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad);
-  const float f_s = (fvalid && lora) ? a.lora_scaling[ad] : 0.f;
-  const uint16_t* Bp = a.lora_b + ((size_t)ad * a.r + rsel) * a.N + fn;
+  // The finish step's operands are requested now and used after the stream.  Lanes without an
+  // output read element 0 instead of selecting on the loaded value: a select would make the wave
+  // wait for memory before its first weight load.
+  const uint32_t srow = fvalid ? frow : 0u, scol = fvalid ? fn : 0u;
+  const float f_sx = a.sx[srow];
+  const float f_sw = a.sw[scol];
+  int ad_raw = 0;
+  if (lora && a.idx) ad_raw = a.idx[srow];
   // z[m][r] share of this thread: value index tid (and tid + 512, ...) of the M x rpad values
   const uint32_t rpad = (a.r + 7u) & ~7u;
   const uint32_t n_zval = lora ? a.M * rpad : 0u;
@@ -334,6 +352,11 @@ __global__ __launch_bounds__(kSkinnyStreamThreads) void skinny_stream_kernel(Ski
   }
   // The low-rank term's loads start only now: issued while the weight stream is in flight they
   // would be served after it anyway, and here they cost one trip to an idle memory.
+  uint16_t res_raw = 0;  // travels with the low-rank term's loads
+  if (a.residual) res_raw = a.residual[(size_t)srow * a.N + scol];
+  const int ad = ad_raw < 0 ? 0 : (ad_raw >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad_raw);
+  const float f_s = (fvalid && lora) ? a.lora_scaling[ad] : 0.f;
+  const uint16_t* Bp = a.lora_b + ((size_t)ad * a.r + rsel) * a.N + fn;
   uint16_t bq[16];
 #pragma unroll
   for (uint32_t t = 0; t < 16; ++t)
@@ -377,7 +400,7 @@ __global__ __launch_bounds__(kSkinnyStreamThreads) void skinny_stream_kernel(Ski
     y = y + l;
   }
   const size_t o = (size_t)frow * a.N + fn;
-  if (a.residual) y = y + f_res;
+  if (a.residual) y = y + bf16_bits_to_f32(res_raw);
   a.out[o] = (uint16_t)f32_to_bf16_bits(y);
   if (a.aux_acc) a.aux_acc[o] = sum;
 }
