@@ -45,7 +45,8 @@ WsLayout make_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint
   w.slot_group = off; off += align256((uint64_t)w.slots * 4u);
   w.blk_range = off; off += align256((uint64_t)(w.slots / 32u) * 4u);
   w.tile_ctr = off; off += 1024u;  // two sets of eight counters, 64 bytes apart
-  w.xn = off; off += rank ? align256((uint64_t)m * k * 2u) : 0u;
+  // normalized rows: only the decode path keeps them in memory (RMSNorm + LoRA, M <= 32)
+  w.xn = off; off += (rank && m <= (uint32_t)kSkinnyMaxRows) ? align256((uint64_t)m * k * 2u) : 0u;
   w.zp = off; off += rank ? align256((uint64_t)(w.slots / 32u) * w.nkk * 3u * kBlockBytes) : 0u;
   w.at = off; off += rank ? align256((uint64_t)n_groups * rank * k * 2u) : 0u;
   w.bp = off; off += rank ? align256((uint64_t)n_groups * (n_padded(n) / 32u) * w.nkk * kBlockBytes) : 0u;

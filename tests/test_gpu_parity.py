@@ -377,3 +377,92 @@ def test_moe_expert_mlp_reduced(dev, pkg):
     print(f"[parity] moe reduced {rep}", flush=True)
     assert rep["finite"] and rep["relative_l2"] < 1e-3 and rep["cosine"] >= 0.9999, rep
     assert rep["violations"] < 1e-3 * rep["size"], rep
+
+
+@pytest.mark.parametrize("what", ["x_row", "x_elem", "w_col", "w_scale", "a_rank", "b_col", "scaling", "residual",
+                                  "gamma", "index"])
+def test_every_operand_matters(dev, what):
+    """Operand sensitivity in the spirit of the reference's mutation list
+    (rocm/probe_w8a8_lora_forward.py:1127-1190): changing any one operand changes the output, and
+    the changed output still agrees with the oracle."""
+    base = wc.make_case(40, 128, 96, n_adapters=3, rank=16, seed=41, rms=True, residual=True)
+    got0 = wc.gpu_forward(base, return_aux=False)
+    case = {k: (v.copy() if isinstance(v, np.ndarray) else v) for k, v in base.items()}
+    if what == "x_row":
+        case["x"][7] = o.bf16_round(case["x"][7] * F32(-1.5))
+    elif what == "x_elem":
+        case["x"][3, 17] = o.bf16_round(case["x"][3, 17] + F32(4.0))
+    elif what == "w_col":
+        case["codes"][:, 5] = -case["codes"][:, 5]
+    elif what == "w_scale":
+        case["scales"][0, 11] *= F32(2.0)
+    elif what == "a_rank":
+        case["a"][1, :, 15] = o.bf16_round(case["a"][1, :, 15] + F32(0.25))
+    elif what == "b_col":
+        case["b"][2, :, 95] = o.bf16_round(case["b"][2, :, 95] + F32(0.5))
+    elif what == "scaling":
+        case["s"][0] *= F32(3.0)
+    elif what == "residual":
+        case["residual"][39, 0] = o.bf16_round(case["residual"][39, 0] + F32(1.0))
+    elif what == "gamma":
+        case["gamma"][64] *= F32(1.5)
+    elif what == "index":
+        case["idx"][0] = (case["idx"][0] + 1) % 3
+    case["weight"] = o.GroupQuantizedWeight(case["codes"], case["scales"], case["k"], case["k"], 8, case["k"])
+    got1 = wc.gpu_forward(case, return_aux=False)
+    assert np.any(got0 != got1), f"mutating {what} left the output unchanged"
+    _assert_close(got1, wc.oracle_forward(case), f" mutated {what}")
+
+
+def test_one_cast_after_the_f32_epilogue(dev):
+    """The output is bf16(base_f32 + s * low_f32), not the sum of two early bf16 casts
+    (skyrl/tx/kernels/quantized_lora.py:298-299, tests/tx/kernels/test_quantized_lora.py:178-199)."""
+    case = wc.make_case(64, 256, 128, n_adapters=1, rank=16, seed=43, idx_mode="zero")
+    got = wc.gpu_forward(case, return_aux=False)
+    base = o.quantized_frozen_linear_f32(case["x"], case["weight"])
+    low = (case["x"].astype(F32) @ case["a"][0].astype(F32)) @ case["b"][0].astype(F32)
+    single = o.bf16_round(base + low * case["s"][0])
+    early = o.bf16_round(o.bf16_round(base) + o.bf16_round(low * case["s"][0]))
+    assert np.any(single != early)  # the inputs can tell the two apart
+    differ = single != early
+    agree_single = np.mean(o.bf16_bits(got)[differ] == o.bf16_bits(single)[differ])
+    agree_early = np.mean(o.bf16_bits(got)[differ] == o.bf16_bits(early)[differ])
+    assert agree_single > 0.95 and agree_early < 0.05, (agree_single, agree_early)
+
+
+def test_quantizer_ties_round_to_even(dev, pkg):
+    """Exact ties and near-ties of x / scale: rint is half-to-even on the correctly rounded
+    quotient (skyrl/tx/kernels/quantized_lora.py:207-211)."""
+    import torch
+
+    k = 256
+    rows = []
+    half = (np.arange(k, dtype=F32) % 127) + F32(0.5)            # k + 0.5: exact ties when scale == 1
+    half[0] = F32(127.0)                                         # absmax 127 -> scale exactly 1.0
+    rows.append(half)
+    rows.append(-half)
+    third = (np.arange(k, dtype=F32) % 97) * F32(1.5)            # scale = 144/127: quotients near ties
+    third[0] = F32(144.0)
+    rows.append(third)
+    tiny = ((np.arange(k, dtype=F32) % 63) - 31) * F32(2.0 ** -20)  # small magnitudes, scale far from 1
+    rows.append(tiny)
+    x = o.bf16_round(np.stack(rows))
+    want_codes, want_scales = o.quantize_rows(x)
+    case = wc.make_case(4, k, 64, n_adapters=0, seed=47)
+    case["x"] = x
+    for flags in (pkg._native.FLAG_FORCE_TILED, pkg._native.FLAG_FORCE_SKINNY):
+        _, aux = wc.gpu_forward(case, flags=flags)
+        np.testing.assert_array_equal(aux["x_codes"], want_codes)
+        np.testing.assert_array_equal(aux["x_scales"].view(np.uint32), want_scales.reshape(-1).view(np.uint32))
+    codes, scales = pkg.w8a8_lora.dynamic_quantize_rows(torch.from_numpy(x).to(dev).to(torch.bfloat16))
+    np.testing.assert_array_equal(codes.cpu().numpy(), want_codes)
+
+
+@pytest.mark.parametrize("m", [4, 80])
+def test_largest_k(dev, m):
+    """K = 16384 is the largest K the library accepts (both the decode and the tiled path)."""
+    case = wc.make_case(m, 16384, 256, n_adapters=2, rank=8, seed=53, residual=True)
+    st = wc.oracle_forward(case, return_stages=True)
+    got, aux = wc.gpu_forward(case)
+    _assert_integer_stages(aux, st)
+    _assert_close(got, st["out"], f" K=16384 m={m}")
