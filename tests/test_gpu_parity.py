@@ -391,7 +391,7 @@ def test_every_operand_matters(dev, what):
     if what == "x_row":
         case["x"][7] = o.bf16_round(case["x"][7] * F32(-1.5))
     elif what == "x_elem":
-        case["x"][3, 17] = o.bf16_round(case["x"][3, 17] + F32(4.0))
+        case["x"][3, 17:18] = o.bf16_round(case["x"][3, 17:18] + F32(4.0))
     elif what == "w_col":
         case["codes"][:, 5] = -case["codes"][:, 5]
     elif what == "w_scale":
@@ -403,7 +403,7 @@ def test_every_operand_matters(dev, what):
     elif what == "scaling":
         case["s"][0] *= F32(3.0)
     elif what == "residual":
-        case["residual"][39, 0] = o.bf16_round(case["residual"][39, 0] + F32(1.0))
+        case["residual"][39, 0:1] = o.bf16_round(case["residual"][39, 0:1] + F32(1.0))
     elif what == "gamma":
         case["gamma"][64] *= F32(1.5)
     elif what == "index":
