@@ -50,7 +50,7 @@ WsLayout make_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint
   w.zp = off; off += rank ? align256((uint64_t)(w.slots / 32u) * w.nkk * 3u * kBlockBytes) : 0u;
   w.at = off; off += rank ? align256((uint64_t)n_groups * rank * k * 2u) : 0u;
   w.bp = off; off += rank ? align256((uint64_t)n_groups * (n_padded(n) / 32u) * w.nkk * kBlockBytes) : 0u;
-  w.skinny = off; off += align256(skinny_workspace_bytes(m, n));
+  w.skinny = off; off += align256(skinny_workspace_bytes(m, n, rank));
   w.total = off;
   return w;
 }
@@ -135,7 +135,7 @@ int launch_skinny(const mi355_w8a8_problem* p, unsigned char* xq, float* sx, uin
                   uint32_t K_pad, uint32_t KB, hipStream_t s) {
   const bool rms = p->rms_gamma != nullptr;
   const bool lora = p->n_adapters > 0;
-  const SkinnyLayout L = skinny_layout(p->m, p->k, p->n);
+  const SkinnyLayout L = skinny_layout(p->m, p->k, p->n, p->rank);
   int st;
   if (!(p->flags & MI355_W8A8_FLAG_SKIP_PROLOGUE)) {
     SkinnyQuantArgs q{};
@@ -153,8 +153,15 @@ int launch_skinny(const mi355_w8a8_problem* p, unsigned char* xq, float* sx, uin
     q.z_part = reinterpret_cast<float*>(sws + L.z_part);
     q.n_adapters = p->n_adapters; q.r = p->rank; q.z_chunks = L.z_chunks; q.z_chunk_k = L.z_chunk_k;
     q.n_z_units = (lora && !rms) ? p->m * L.z_chunks : 0u;
-    if (rms) hipLaunchKernelGGL((skinny_quant_kernel<true>), dim3(p->m), dim3(1024), 0, s, q);
-    else hipLaunchKernelGGL((skinny_quant_kernel<false>), dim3(p->m + q.n_z_units), dim3(1024), 0, s, q);
+    const bool regroup = lora && p->rank <= 32u && p->m <= 16u && (p->n % 8u) == 0;
+    q.lora_b = regroup ? static_cast<const uint16_t*>(p->lora_b) : nullptr;
+    q.bsel = reinterpret_cast<uint16_t*>(sws + L.bsel);
+    q.N = p->n; q.n_groups = n_padded(p->n) / 128u;
+    q.lora_scaling = lora ? p->lora_scaling : nullptr;
+    q.row_scaling = reinterpret_cast<float*>(sws + L.row_scaling);
+    const uint32_t n_regroup = regroup ? (p->m * q.n_groups + 3u) / 4u : 0u;
+    if (rms) hipLaunchKernelGGL((skinny_quant_kernel<true>), dim3(p->m + n_regroup), dim3(1024), 0, s, q);
+    else hipLaunchKernelGGL((skinny_quant_kernel<false>), dim3(p->m + q.n_z_units + n_regroup), dim3(1024), 0, s, q);
     if ((st = launch_status())) return st;
     if (lora && rms) {  // the LoRA-A units read the normalized rows the quantizer has just written
       SkinnyLoraAArgs la{};
@@ -172,7 +179,9 @@ int launch_skinny(const mi355_w8a8_problem* p, unsigned char* xq, float* sx, uin
   a.z_part = reinterpret_cast<const float*>(sws + L.z_part);
   a.sx = sx; a.sw = p->w_scales;
   a.lora_b = lora ? static_cast<const uint16_t*>(p->lora_b) : nullptr;
+  a.bsel = (lora && p->rank <= 32u && p->m <= 16u && (p->n % 8u) == 0) ? reinterpret_cast<const uint16_t*>(sws + L.bsel) : nullptr;
   a.lora_scaling = p->lora_scaling; a.idx = p->adapter_indices;
+  a.row_scaling = reinterpret_cast<const float*>(sws + L.row_scaling);
   a.residual = static_cast<const uint16_t*>(p->residual);
   a.out = static_cast<uint16_t*>(p->out);
   a.aux_acc = p->aux_acc;

@@ -22,12 +22,11 @@ constexpr uint32_t kSkinnyMaxZChunks = 16;
 constexpr uint32_t kSkinnyZChunkK = 1024;  // K elements per LoRA-A work unit (per row)
 
 struct SkinnyLayout {
-  uint64_t z_part, total;
+  uint64_t z_part, row_scaling, bsel, total;
   uint32_t pairs_per_wave, z_chunks, z_chunk_k;
 };
 
-inline SkinnyLayout skinny_layout(uint32_t m, uint32_t k, uint32_t n) {
-  (void)m; (void)n;
+inline SkinnyLayout skinny_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t rank) {
   SkinnyLayout L{};
   const uint32_t n_pairs = k_padded(k) / 64u;
   L.pairs_per_wave = (n_pairs + 7u) / 8u;
@@ -37,11 +36,18 @@ inline SkinnyLayout skinny_layout(uint32_t m, uint32_t k, uint32_t n) {
   L.z_chunks = zc;
   L.z_chunk_k = zk;
   L.z_part = 0;
-  L.total = (uint64_t)kSkinnyMaxZChunks * kSkinnyMaxRows * kMaxRank * 4u;
+  L.row_scaling = (uint64_t)kSkinnyMaxZChunks * kSkinnyMaxRows * kMaxRank * 4u;
+  L.bsel = L.row_scaling + 256u;
+  // LoRA B regrouped for the stream kernel's finish step (skinny_regroup_b): [unit][row][rank half]
+  // [column][16 ranks] bf16, for M <= 16 and rank <= 32
+  const bool regroup = rank > 0 && rank <= 32u && m <= 16u;
+  L.total = L.bsel + (regroup ? (uint64_t)(n_padded(n) / 16u) * m * 2u * 16u * 32u : 0u);
   return L;
 }
 
-inline uint64_t skinny_workspace_bytes(uint32_t m, uint32_t n) { return skinny_layout(m, 128u, n).total; }
+inline uint64_t skinny_workspace_bytes(uint32_t m, uint32_t n, uint32_t rank) {
+  return skinny_layout(m, 128u, n, rank).total;
+}
 inline bool skinny_supported() { return true; }
 
 // ---------------------------------------------------------------------------------------
@@ -62,7 +68,48 @@ struct SkinnyQuantArgs {
   const int32_t* idx;      // adapter per row or null
   float* z_part;           // f32 [z_chunks][32][kMaxRank]
   uint32_t n_adapters, r, z_chunks, z_chunk_k, n_z_units;
+  // LoRA-B regrouping items that share the launch (M <= 16, rank <= 32, N % 8 == 0), four per block
+  const uint16_t* lora_b;  // bf16 [n_adapters, r, N] or null
+  uint16_t* bsel;          // bf16 [N_pad/16 units][M][2][16][16]
+  uint32_t N, n_groups;    // n_groups = N_pad / 128
+  const float* lora_scaling;  // f32 [n_adapters] or null
+  float* row_scaling;      // f32 [32]: lora_scaling[idx[m]], written here for the stream kernel
 };
+
+// The stream kernel's unit u = 8 G + 2 j + h owns the original columns 128 G + 4 (16 h + c) + j,
+// c = 0..15, and its finish step needs, per row m and column c, the ranks of one parity:
+//   bsel[u][m][p][c][t] = B[idx[m]][p + 2 t][128 G + 4 (16 h + c) + j],  t = 0..15
+// so that a thread reads its 16 values as one 32-byte piece instead of 16 two-byte values that each
+// cost a 128-byte line.  One item = (row m, column group G): its r x 128 tile of B goes through LDS.
+__device__ inline void skinny_regroup_b(const SkinnyQuantArgs& a, uint32_t block, uint16_t (*tile)[32][128]) {
+  const uint32_t team = threadIdx.x >> 8, t256 = threadIdx.x & 255u;
+  const uint32_t item = block * 4u + team;
+  const bool live = item < a.M * a.n_groups;
+  const uint32_t m = live ? item / a.n_groups : 0u, G = live ? item % a.n_groups : 0u;
+  int ad = a.idx ? a.idx[m] : 0;
+  ad = ad < 0 ? 0 : (ad >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad);
+  const uint16_t* Bsrc = a.lora_b + (size_t)ad * a.r * a.N + G * 128u;
+#pragma unroll
+  for (uint32_t u = 0; u < 2; ++u) {  // 32 ranks x 16 pieces of 8 columns
+    const uint32_t piece = t256 + 256u * u, rr = piece >> 4, c8 = (piece & 15u) * 8u;
+    v8us v = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (live && rr < a.r && G * 128u + c8 < a.N) v = *reinterpret_cast<const v8us*>(Bsrc + (size_t)rr * a.N + c8);
+    *reinterpret_cast<v8us*>(&tile[team][rr][c8]) = v;
+  }
+  __syncthreads();
+  if (!live) return;
+  const uint32_t u8 = t256 >> 5, par = (t256 >> 4) & 1u, c = t256 & 15u;
+  const uint32_t col = 4u * (16u * (u8 & 1u) + c) + (u8 >> 1);
+  v8us lo, hi;
+#pragma unroll
+  for (uint32_t t = 0; t < 8; ++t) {
+    lo[t] = tile[team][par + 2u * t][col];
+    hi[t] = tile[team][par + 2u * (t + 8u)][col];
+  }
+  uint16_t* dst = a.bsel + (((((size_t)G * 8u + u8) * a.M + m) * 2u + par) * 16u + c) * 16u;
+  *reinterpret_cast<v8us*>(dst) = lo;
+  *reinterpret_cast<v8us*>(dst + 8) = hi;
+}
 
 // z_part[ch][m][:] = x[m, chunk ch] @ A[idx[m]][chunk ch, :] in float32.  Thread (kl, q)
 // accumulates rank columns 8q..8q+7 over the rows k = k_begin + kl + kpt*j; lanes with equal q are
@@ -141,6 +188,11 @@ __global__ __launch_bounds__(1024) void skinny_quant_kernel(SkinnyQuantArgs a) {
   __shared__ float red_max[16];
   __shared__ double red_sum[16];
   __shared__ float zw[16][64];
+  if (blockIdx.x >= a.M + a.n_z_units) {
+    __shared__ __attribute__((aligned(16))) uint16_t tile[4][32][128];  // 32 KiB
+    skinny_regroup_b(a, blockIdx.x - a.M - a.n_z_units, tile);
+    return;
+  }
   if (blockIdx.x >= a.M) {
     const uint32_t unit = blockIdx.x - a.M;
     skinny_lora_a_unit<1024>(a.x, a.lora_a, a.idx, a.z_part, unit, a.K, a.n_adapters, a.r, a.z_chunks,
@@ -214,6 +266,11 @@ __global__ __launch_bounds__(1024) void skinny_quant_kernel(SkinnyQuantArgs a) {
   if (tid == 0) {
     a.sx[m] = scale;
     if (a.scales_rm) a.scales_rm[m] = scale;
+    if (a.lora_scaling) {
+      int ad = a.idx ? a.idx[m] : 0;
+      ad = ad < 0 ? 0 : (ad >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad);
+      a.row_scaling[m] = a.lora_scaling[ad];
+    }
   }
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
@@ -258,7 +315,9 @@ struct SkinnyStreamArgs {
   const float* sx;           // f32 [32]
   const float* sw;           // f32 [N]
   const uint16_t* lora_b;    // bf16 [n_adapters, r, N] or null
+  const uint16_t* bsel;      // B regrouped per unit (skinny_regroup_b) or null: then B is gathered directly
   const float* lora_scaling;
+  const float* row_scaling;  // f32 [32]: lora_scaling[idx[m]] (from the quantizer launch)
   const int32_t* idx;        // adapter per row or null
   const uint16_t* residual;  // bf16 [M, N] or null
   uint16_t* out;             // bf16 [M, N]
@@ -321,6 +380,29 @@ __global__ __launch_bounds__(kSkinnyStreamThreads) void skinny_stream_kernel(Ski
   // z[m][r] share of this thread: value index tid (and tid + 512, ...) of the M x rpad values
   const uint32_t rpad = (a.r + 7u) & ~7u;
   const uint32_t n_zval = lora ? a.M * rpad : 0u;
+  // With B regrouped per unit the low-rank term needs three independent, coalesced requests per
+  // thread (its 16 ranks of B, its z partials, its row's scaling).  They go out ahead of the weight
+  // loads: a wave's loads return in order, so they are back while the weight is still streaming,
+  // and the term is computed under the stream.  (Issued later they would wait for the stream.)
+  const bool early = !ROWS2 && lora && a.bsel != nullptr && n_zval <= kSkinnyStreamThreads;  // workgroup-uniform
+  float low = 0.f, f_s = 0.f;
+  uint16_t res_raw = 0;
+  v8us blo = {0, 0, 0, 0, 0, 0, 0, 0}, bhi = {0, 0, 0, 0, 0, 0, 0, 0};
+  float zv[kSkinnyMaxZChunks];
+  if (early) {
+    if (a.residual) res_raw = a.residual[(size_t)srow * a.N + scol];
+    f_s = a.row_scaling[srow];
+    const uint32_t unit = grp * 8u + (slot & 7u);
+    const uint16_t* bs = a.bsel + (((((size_t)unit * a.M + srow) * 2u + rsel) * 16u + c16) * 16u);
+    blo = *reinterpret_cast<const v8us*>(bs);
+    bhi = *reinterpret_cast<const v8us*>(bs + 8);
+    const uint32_t zi = tid < n_zval ? tid : 0u;
+    const float* zp = a.z_part + (size_t)(zi / rpad) * kMaxRank + zi % rpad;
+#pragma unroll
+    for (uint32_t ch = 0; ch < kSkinnyMaxZChunks; ++ch)
+      zv[ch] = ch < a.z_chunks ? zp[(size_t)ch * kSkinnyMaxRows * kMaxRank] : 0.f;
+  }
+  __builtin_amdgcn_sched_barrier(0);  // the weight loads below are issued after the requests above
   v4i acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
   uint32_t base = p0;
   do {
@@ -336,6 +418,26 @@ __global__ __launch_bounds__(kSkinnyStreamThreads) void skinny_stream_kernel(Ski
       xf[t] = *reinterpret_cast<const v4i*>(xsrc + (size_t)pr * 2u * kBlockBytes);
       if constexpr (ROWS2) xg[t] = *reinterpret_cast<const v4i*>(xsrc + (size_t)pr * 2u * kBlockBytes + 256u);
     }
+    if (early && base == p0) {  // workgroup-uniform: the low-rank term, under the first round's loads
+      __builtin_amdgcn_sched_barrier(0);
+      if (tid < n_zval) {  // z[m][r]: four interleaved partial sums, combined in a fixed order
+        float s4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (uint32_t ch = 0; ch < kSkinnyMaxZChunks; ++ch) s4[ch & 3u] += zv[ch];
+        zl[tid / rpad][tid % rpad] = ((s4[0] + s4[1]) + s4[2]) + s4[3];
+      }
+      __syncthreads();
+#pragma unroll
+      for (uint32_t t = 0; t < 16; ++t) {
+        const uint32_t r = rsel + kRankSplit * t;
+        const uint16_t bv = t < 8u ? blo[t & 7u] : bhi[t & 7u];
+        if (r < a.r) low = fmaf(zl[srow][r], bf16_bits_to_f32(bv), low);
+      }
+      if (rsel == 1u) low_odd[tid & 255u] = low;  // the two rank halves of an output, added in a fixed order
+      __syncthreads();
+      if (rsel == 0u) low = low + low_odd[tid];
+      __builtin_amdgcn_sched_barrier(0);
+    }
 #pragma unroll
     for (uint32_t t = 0; t < kInFlight; ++t) {
       if (base + t < p1) {  // wave-uniform
@@ -350,46 +452,47 @@ __global__ __launch_bounds__(kSkinnyStreamThreads) void skinny_stream_kernel(Ski
     red[wave][0][e][lane] = acc0[e];
     red[wave][1][e][lane] = acc1[e];
   }
-  // The low-rank term's loads start only now: issued while the weight stream is in flight they
-  // would be served after it anyway, and here they cost one trip to an idle memory.
-  uint16_t res_raw = 0;  // travels with the low-rank term's loads
-  if (a.residual) res_raw = a.residual[(size_t)srow * a.N + scol];
-  const int ad = ad_raw < 0 ? 0 : (ad_raw >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad_raw);
-  const float f_s = (fvalid && lora) ? a.lora_scaling[ad] : 0.f;
-  const uint16_t* Bp = a.lora_b + ((size_t)ad * a.r + rsel) * a.N + fn;
-  uint16_t bq[16];
+  if (!early) {
+    // Without the regrouped B the term's loads start only now: issued while the weight stream is in
+    // flight they would be served after it anyway, and here they cost one trip to an idle memory.
+    if (a.residual) res_raw = a.residual[(size_t)srow * a.N + scol];
+    const int ad = ad_raw < 0 ? 0 : (ad_raw >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad_raw);
+    f_s = (fvalid && lora) ? a.lora_scaling[ad] : 0.f;
+    const uint16_t* Bp = a.lora_b + ((size_t)ad * a.r + rsel) * a.N + fn;
+    uint16_t bq[16];
 #pragma unroll
-  for (uint32_t t = 0; t < 16; ++t)
-    bq[t] = (fvalid && lora && rsel + kRankSplit * t < a.r) ? Bp[(size_t)(kRankSplit * t) * a.N] : (uint16_t)0;
-  for (uint32_t zi = tid; zi < n_zval; zi += kSkinnyStreamThreads) {
-    const float* zp = a.z_part + (size_t)(zi / rpad) * kMaxRank + zi % rpad;
-    float zv[kSkinnyMaxZChunks];
+    for (uint32_t t = 0; t < 16; ++t)
+      bq[t] = (fvalid && lora && rsel + kRankSplit * t < a.r) ? Bp[(size_t)(kRankSplit * t) * a.N] : (uint16_t)0;
+    for (uint32_t zi = tid; zi < n_zval; zi += kSkinnyStreamThreads) {
+      const float* zp = a.z_part + (size_t)(zi / rpad) * kMaxRank + zi % rpad;
+      float zw4[kSkinnyMaxZChunks];
 #pragma unroll
-    for (uint32_t ch = 0; ch < kSkinnyMaxZChunks; ++ch)
-      zv[ch] = ch < a.z_chunks ? zp[(size_t)ch * kSkinnyMaxRows * kMaxRank] : 0.f;
-    float s4[4] = {0.f, 0.f, 0.f, 0.f};  // four interleaved partial sums, combined in a fixed order
+      for (uint32_t ch = 0; ch < kSkinnyMaxZChunks; ++ch)
+        zw4[ch] = ch < a.z_chunks ? zp[(size_t)ch * kSkinnyMaxRows * kMaxRank] : 0.f;
+      float s4[4] = {0.f, 0.f, 0.f, 0.f};  // four interleaved partial sums, combined in a fixed order
 #pragma unroll
-    for (uint32_t ch = 0; ch < kSkinnyMaxZChunks; ++ch) s4[ch & 3u] += zv[ch];
-    zl[zi / rpad][zi % rpad] = ((s4[0] + s4[1]) + s4[2]) + s4[3];
-  }
-  __syncthreads();
-  // ---- finish
-  float low = 0.f;
-  if (fvalid && lora) {
-#pragma unroll
-    for (uint32_t t = 0; t < 16; ++t) {
-      const uint32_t r = rsel + kRankSplit * t;
-      if (r < a.r) low = fmaf(zl[frow][r], bf16_bits_to_f32(bq[t]), low);
+      for (uint32_t ch = 0; ch < kSkinnyMaxZChunks; ++ch) s4[ch & 3u] += zw4[ch];
+      zl[zi / rpad][zi % rpad] = ((s4[0] + s4[1]) + s4[2]) + s4[3];
     }
-    for (uint32_t r = rsel + kRankSplit * 16u; r < a.r; r += kRankSplit)
-      low = fmaf(zl[frow][r], bf16_bits_to_f32(Bp[(size_t)(r - rsel) * a.N]), low);
-  }
-  if (!ROWS2) {
-    if (rsel == 1u) low_odd[tid & 255u] = low;
     __syncthreads();
-    if (rsel == 1u) return;
-    low = low + low_odd[tid];
+    if (fvalid && lora) {
+#pragma unroll
+      for (uint32_t t = 0; t < 16; ++t) {
+        const uint32_t r = rsel + kRankSplit * t;
+        if (r < a.r) low = fmaf(zl[frow][r], bf16_bits_to_f32(bq[t]), low);
+      }
+      for (uint32_t r = rsel + kRankSplit * 16u; r < a.r; r += kRankSplit)
+        low = fmaf(zl[frow][r], bf16_bits_to_f32(Bp[(size_t)(r - rsel) * a.N]), low);
+    }
+    if (!ROWS2) {
+      if (rsel == 1u) low_odd[tid & 255u] = low;
+      __syncthreads();
+      if (rsel == 0u) low = low + low_odd[tid];
+    }
+  } else {
+    __syncthreads();  // the accumulators in `red`
   }
+  if (!ROWS2 && rsel == 1u) return;
   if (!fvalid) return;
   int sum = 0;
 #pragma unroll
