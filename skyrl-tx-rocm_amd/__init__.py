@@ -8,5 +8,6 @@ module name ``skyrl_tx_rocm_amd``.
 from . import _native  # noqa: F401
 from .kernels import quantized_lora  # noqa: F401
 from .kernels.rocm import w8a8_lora  # noqa: F401
+from .layers import lora  # noqa: F401
 
-__all__ = ["_native", "quantized_lora", "w8a8_lora"]
+__all__ = ["_native", "quantized_lora", "w8a8_lora", "lora"]
