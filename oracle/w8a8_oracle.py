@@ -25,6 +25,10 @@ How each function is pinned (the tests that do it live in ``tests/test_oracle_*.
 * ``silu``: exp/logistic rounding of XLA-CPU is likewise unavailable; PARITY
   UNPINNED in the last f32 bit, pinned to 1 ulp by the closed-form constant above
   and by ``scipy.special.expit``.
+* ``quantized_lora_linear_bwd*``: ``torch.autograd`` (float64, CPU) through the straight-through
+  function ``x @ dequant(W) + s * (x @ A) @ B``, central finite differences of the LoRA
+  terms, and the zero/linearity identities of the equations.  PARITY UNPINNED in the float32
+  summation order of XLA (float64 accumulation here).
 * ``moe_route``/``moe_expert_mlp``: ``torch.topk``/``scipy.special.softmax`` special
   cases and the merged-weight invariant of tests/tx/models/test_qwen3.py:123-180.
 """
@@ -375,6 +379,94 @@ def quantized_lora_linear_multi(x, weight, lora_a, lora_b, lora_scaling, adapter
     """
     return bf16_round(quantized_lora_linear_multi_f32(x, weight, lora_a, lora_b, lora_scaling,
                                                       adapter_indices, residual))
+
+
+# ---------------------------------------------------------------------------
+# backward of the quantized LoRA linear (quantized_lora.py:337-394)
+# ---------------------------------------------------------------------------
+
+def _mm64(a, b) -> np.ndarray:
+    """float32 matrix product evaluated with float64 accumulation and rounded once.
+
+    The reference contracts in float32 through XLA, whose summation order is not
+    available here; the float64 sum is the order-free value every float32 order
+    approximates (PARITY UNPINNED in the last float32 bits, far inside the bf16 gate).
+    """
+    return np.matmul(np.asarray(a, dtype=np.float64), np.asarray(b, dtype=np.float64)).astype(F32)
+
+
+def quantized_lora_linear_bwd_f32(x, weight: GroupQuantizedWeight, lora_a, lora_b, lora_scaling, dy):
+    """Float32 cotangents (dx, dA, dB, dscaling) of quantized_lora.py:337-394.
+
+    Straight-through base: ``dx_base = dy @ (codes * scales).T`` (:361-378), the
+    activation quantizer has no derivative of its own.  ``r = (dy @ B.T) * s`` (:352),
+    ``dx = dx_base + r @ A.T`` (:379), ``dA = x.T @ r`` (:380), ``dB = ((x @ A).T @ dy) * s``
+    (:381), ``dscaling = sum(dy * ((x @ A) @ B))`` (:382-383).
+    """
+    validate_quantized_weight(weight)
+    x = np.asarray(x, dtype=F32)
+    dy = np.asarray(dy, dtype=F32)
+    a = np.asarray(lora_a, dtype=F32)
+    b = np.asarray(lora_b, dtype=F32)
+    s = F32(np.asarray(lora_scaling, dtype=F32).reshape(()))
+    flat = x.reshape((-1, x.shape[-1]))
+    dyf = dy.reshape((-1, dy.shape[-1]))
+    if flat.shape[0] != dyf.shape[0]:
+        raise ValueError("x and dy must have the same row domain")
+    z = _mm64(flat, a)
+    r = (_mm64(dyf, b.T) * s).astype(F32)
+    wdeq = dequantize_frozen_weight(weight)[: weight.original_in_features]
+    dx = (_mm64(dyf, wdeq.T) + _mm64(r, a.T)).astype(F32)
+    da = _mm64(flat.T, r)
+    db = (_mm64(z.T, dyf) * s).astype(F32)
+    dscaling = F32(np.sum(dyf.astype(np.float64) * np.matmul(z.astype(np.float64), b.astype(np.float64))))
+    return dx.reshape(x.shape), da, db, dscaling
+
+
+def quantized_lora_linear_bwd(x, weight, lora_a, lora_b, lora_scaling, dy):
+    """Cotangents cast as the reference casts them (quantized_lora.py:384-391): dx to the
+    activation dtype, dA/dB to the LoRA dtype (both bf16 here), dscaling to float32."""
+    dx, da, db, ds = quantized_lora_linear_bwd_f32(x, weight, lora_a, lora_b, lora_scaling, dy)
+    return bf16_round(dx), bf16_round(da), bf16_round(db), ds
+
+
+def quantized_lora_linear_multi_bwd_f32(x, weight, lora_a, lora_b, lora_scaling, adapter_indices, dy):
+    """Per-row adapters: the cotangent of ``quantized_lora_linear_multi_f32``.
+
+    Rows of adapter ``g`` contribute to ``dA[g]``, ``dB[g]``, ``dscaling[g]`` only (the
+    derivative of the grouped products of skyrl/tx/layers/lora.py:142-157); adapters no row
+    names get zeros.  The base term is shared.
+    """
+    x = np.asarray(x, dtype=F32)
+    dy = np.asarray(dy, dtype=F32)
+    a = np.asarray(lora_a, dtype=F32)
+    b = np.asarray(lora_b, dtype=F32)
+    s = np.asarray(lora_scaling, dtype=F32)
+    idx = np.asarray(adapter_indices)
+    if a.ndim != 3 or b.ndim != 3 or s.shape != (a.shape[0],):
+        raise ValueError("multi-adapter lora_a/lora_b must be rank-three with one scaling each")
+    if x.ndim != 2 or idx.shape != (x.shape[0],) or dy.shape[0] != x.shape[0]:
+        raise ValueError("x, dy are [rows, .] with one adapter index per row")
+    wdeq = dequantize_frozen_weight(weight)[: weight.original_in_features]
+    dx = _mm64(dy, wdeq.T)
+    da = np.zeros_like(a)
+    db = np.zeros_like(b)
+    ds = np.zeros_like(s)
+    for g in np.unique(idx):
+        rows = np.nonzero(idx == g)[0]
+        z = _mm64(x[rows], a[g])
+        r = (_mm64(dy[rows], b[g].T) * s[g]).astype(F32)
+        dx[rows] = (dx[rows] + _mm64(r, a[g].T)).astype(F32)
+        da[g] = _mm64(x[rows].T, r)
+        db[g] = (_mm64(z.T, dy[rows]) * s[g]).astype(F32)
+        ds[g] = F32(np.sum(dy[rows].astype(np.float64) * np.matmul(z.astype(np.float64), b[g].astype(np.float64))))
+    return dx, da, db, ds
+
+
+def quantized_lora_linear_multi_bwd(x, weight, lora_a, lora_b, lora_scaling, adapter_indices, dy):
+    dx, da, db, ds = quantized_lora_linear_multi_bwd_f32(x, weight, lora_a, lora_b, lora_scaling,
+                                                         adapter_indices, dy)
+    return bf16_round(dx), bf16_round(da), bf16_round(db), ds
 
 
 # ---------------------------------------------------------------------------
