@@ -124,6 +124,38 @@ typedef struct mi355_w8a8_grouped_problem {
   int32_t* aux_acc;         /* int32 [m, n]; rows beyond sum(group_sizes) are not written */
 } mi355_w8a8_grouped_problem;
 
+/*
+ * Backward of the plain W8A8 LoRA linear (no RMSNorm / SwiGLU / residual stage):
+ *   dx  = dy @ bf16(codes * scales).T + ((dy @ B[idx].T) * s[idx]) @ A[idx].T
+ *   dA[g] = x_g.T @ ((dy_g @ B[g].T) * s[g])     dB[g] = ((x_g @ A[g]).T @ dy_g) * s[g]
+ *   ds[g] = sum(dy_g * ((x_g @ A[g]) @ B[g]))    (rows of adapter g; zero for adapters without rows)
+ * The activation quantizer is treated as the identity (straight-through), as the reference does.
+ */
+typedef struct mi355_w8a8_bwd_problem {
+  uint32_t struct_size;     /* sizeof(mi355_w8a8_bwd_problem) */
+  uint32_t flags;           /* reserved, 0 */
+  uint32_t m;               /* rows */
+  uint32_t k;               /* in features (columns of dx); multiple of 8 */
+  uint32_t n;               /* out features (columns of dy); multiple of 8 */
+  uint32_t n_adapters;      /* 0 = no LoRA */
+  uint32_t rank;
+  uint32_t reserved;
+  const void* x;            /* bf16 [m, k]; needed only when a LoRA cotangent is requested */
+  const void* dy;           /* bf16 [m, n] output cotangent */
+  const void* w_packed;     /* the forward's packed weight */
+  const float* w_scales;    /* f32 [n] */
+  const void* lora_a;       /* bf16 [n_adapters, k, rank] or NULL */
+  const void* lora_b;       /* bf16 [n_adapters, rank, n] or NULL */
+  const float* lora_scaling;/* f32 [n_adapters] or NULL */
+  const int32_t* adapter_indices; /* int32 [m] or NULL (adapter 0 for every row) */
+  void* dx;                 /* bf16 [m, k] */
+  void* d_lora_a;           /* bf16 [n_adapters, k, rank] or NULL (not wanted) */
+  void* d_lora_b;           /* bf16 [n_adapters, rank, n] or NULL */
+  float* d_lora_scaling;    /* f32 [n_adapters] or NULL */
+  void* workspace;          /* >= mi355_w8a8_bwd_workspace_bytes(...) bytes, 256-byte aligned */
+  uint64_t workspace_bytes;
+} mi355_w8a8_bwd_problem;
+
 int mi355_w8a8_abi_version(void);
 const char* mi355_w8a8_status_string(int status);
 
@@ -157,6 +189,15 @@ int mi355_w8a8_lora_residual_v1(const mi355_w8a8_problem* problem, void* stream)
 int mi355_w8a8_forward_v1(const mi355_w8a8_problem* problem, void* stream);
 /* Grouped / ragged per-expert variant. */
 int mi355_w8a8_grouped_v1(const mi355_w8a8_grouped_problem* problem, void* stream);
+
+/*
+ * Backward (VJP) of mi355_w8a8_lora_linear_v1: replaces the custom_vjp rule
+ * _quantized_lora_linear_bwd (skyrl/tx/kernels/quantized_lora.py:337-394) with the bf16 weight
+ * policy of the ROCm prototype's pull-back (skyrl/tx/kernels/rocm/w8a8_lora.py:298-339,722-821).
+ */
+uint64_t mi355_w8a8_bwd_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t n_adapters,
+                                        uint32_t rank, uint32_t flags);
+int mi355_w8a8_lora_linear_bwd_v1(const mi355_w8a8_bwd_problem* problem, void* stream);
 
 #ifdef __cplusplus
 }

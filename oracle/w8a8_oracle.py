@@ -395,7 +395,16 @@ def _mm64(a, b) -> np.ndarray:
     return np.matmul(np.asarray(a, dtype=np.float64), np.asarray(b, dtype=np.float64)).astype(F32)
 
 
-def quantized_lora_linear_bwd_f32(x, weight: GroupQuantizedWeight, lora_a, lora_b, lora_scaling, dy):
+def pullback_weight(weight: GroupQuantizedWeight, relaxed: bool) -> np.ndarray:
+    """[K, N] weight the input pull-back contracts with: float32 ``codes * scales``
+    (quantized_lora.py:370) or, relaxed, that product rounded to bf16 per element, the policy of
+    the ROCm kernel's W8A16 pull-back (skyrl/tx/kernels/rocm/w8a8_lora.py:326-330)."""
+    wdeq = dequantize_frozen_weight(weight)[: weight.original_in_features]
+    return bf16_round(wdeq) if relaxed else wdeq
+
+
+def quantized_lora_linear_bwd_f32(x, weight: GroupQuantizedWeight, lora_a, lora_b, lora_scaling, dy,
+                                  relaxed_weight: bool = False):
     """Float32 cotangents (dx, dA, dB, dscaling) of quantized_lora.py:337-394.
 
     Straight-through base: ``dx_base = dy @ (codes * scales).T`` (:361-378), the
@@ -415,7 +424,7 @@ def quantized_lora_linear_bwd_f32(x, weight: GroupQuantizedWeight, lora_a, lora_
         raise ValueError("x and dy must have the same row domain")
     z = _mm64(flat, a)
     r = (_mm64(dyf, b.T) * s).astype(F32)
-    wdeq = dequantize_frozen_weight(weight)[: weight.original_in_features]
+    wdeq = pullback_weight(weight, relaxed_weight)
     dx = (_mm64(dyf, wdeq.T) + _mm64(r, a.T)).astype(F32)
     da = _mm64(flat.T, r)
     db = (_mm64(z.T, dyf) * s).astype(F32)
@@ -423,14 +432,15 @@ def quantized_lora_linear_bwd_f32(x, weight: GroupQuantizedWeight, lora_a, lora_
     return dx.reshape(x.shape), da, db, dscaling
 
 
-def quantized_lora_linear_bwd(x, weight, lora_a, lora_b, lora_scaling, dy):
+def quantized_lora_linear_bwd(x, weight, lora_a, lora_b, lora_scaling, dy, relaxed_weight: bool = False):
     """Cotangents cast as the reference casts them (quantized_lora.py:384-391): dx to the
     activation dtype, dA/dB to the LoRA dtype (both bf16 here), dscaling to float32."""
-    dx, da, db, ds = quantized_lora_linear_bwd_f32(x, weight, lora_a, lora_b, lora_scaling, dy)
+    dx, da, db, ds = quantized_lora_linear_bwd_f32(x, weight, lora_a, lora_b, lora_scaling, dy, relaxed_weight)
     return bf16_round(dx), bf16_round(da), bf16_round(db), ds
 
 
-def quantized_lora_linear_multi_bwd_f32(x, weight, lora_a, lora_b, lora_scaling, adapter_indices, dy):
+def quantized_lora_linear_multi_bwd_f32(x, weight, lora_a, lora_b, lora_scaling, adapter_indices, dy,
+                                        relaxed_weight: bool = False):
     """Per-row adapters: the cotangent of ``quantized_lora_linear_multi_f32``.
 
     Rows of adapter ``g`` contribute to ``dA[g]``, ``dB[g]``, ``dscaling[g]`` only (the
@@ -447,7 +457,7 @@ def quantized_lora_linear_multi_bwd_f32(x, weight, lora_a, lora_b, lora_scaling,
         raise ValueError("multi-adapter lora_a/lora_b must be rank-three with one scaling each")
     if x.ndim != 2 or idx.shape != (x.shape[0],) or dy.shape[0] != x.shape[0]:
         raise ValueError("x, dy are [rows, .] with one adapter index per row")
-    wdeq = dequantize_frozen_weight(weight)[: weight.original_in_features]
+    wdeq = pullback_weight(weight, relaxed_weight)
     dx = _mm64(dy, wdeq.T)
     da = np.zeros_like(a)
     db = np.zeros_like(b)
@@ -463,9 +473,10 @@ def quantized_lora_linear_multi_bwd_f32(x, weight, lora_a, lora_b, lora_scaling,
     return dx, da, db, ds
 
 
-def quantized_lora_linear_multi_bwd(x, weight, lora_a, lora_b, lora_scaling, adapter_indices, dy):
+def quantized_lora_linear_multi_bwd(x, weight, lora_a, lora_b, lora_scaling, adapter_indices, dy,
+                                    relaxed_weight: bool = False):
     dx, da, db, ds = quantized_lora_linear_multi_bwd_f32(x, weight, lora_a, lora_b, lora_scaling,
-                                                         adapter_indices, dy)
+                                                         adapter_indices, dy, relaxed_weight)
     return bf16_round(dx), bf16_round(da), bf16_round(db), ds
 
 

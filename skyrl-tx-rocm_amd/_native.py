@@ -33,6 +33,7 @@ EXPORTS = (
     "mi355_w8a8_workspace_bytes", "mi355_w8a8_grouped_workspace_bytes",
     "mi355_w8a8_lora_linear_v1", "mi355_w8a8_rms_gateup_swiglu_v1", "mi355_w8a8_lora_residual_v1",
     "mi355_w8a8_forward_v1", "mi355_w8a8_grouped_v1",
+    "mi355_w8a8_bwd_workspace_bytes", "mi355_w8a8_lora_linear_bwd_v1",
 )
 
 _u32, _u64, _vp, _f32 = ctypes.c_uint32, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_float
@@ -63,6 +64,18 @@ class GroupedProblem(ctypes.Structure):
     ]
 
 
+class BwdProblem(ctypes.Structure):
+    """struct mi355_w8a8_bwd_problem"""
+
+    _fields_ = [
+        ("struct_size", _u32), ("flags", _u32), ("m", _u32), ("k", _u32), ("n", _u32),
+        ("n_adapters", _u32), ("rank", _u32), ("reserved", _u32),
+        ("x", _vp), ("dy", _vp), ("w_packed", _vp), ("w_scales", _vp), ("lora_a", _vp), ("lora_b", _vp),
+        ("lora_scaling", _vp), ("adapter_indices", _vp), ("dx", _vp), ("d_lora_a", _vp), ("d_lora_b", _vp),
+        ("d_lora_scaling", _vp), ("workspace", _vp), ("workspace_bytes", _u64),
+    ]
+
+
 class NativeError(RuntimeError):
     def __init__(self, fn: str, status: int, detail: str):
         super().__init__(f"{fn} failed: {STATUS.get(status, status)} ({detail})")
@@ -86,7 +99,8 @@ def _bind(lib: ctypes.CDLL) -> None:
         fn.argtypes = (_vp, _vp, _u32, _u32, _vp)
     lib.mi355_w8a8_quantize_rows_v1.restype = ctypes.c_int
     lib.mi355_w8a8_quantize_rows_v1.argtypes = (_vp, _vp, _vp, _u32, _u32, _vp)
-    for name in ("mi355_w8a8_workspace_bytes", "mi355_w8a8_grouped_workspace_bytes"):
+    for name in ("mi355_w8a8_workspace_bytes", "mi355_w8a8_grouped_workspace_bytes",
+                 "mi355_w8a8_bwd_workspace_bytes"):
         fn = getattr(lib, name)
         fn.restype = _u64
         fn.argtypes = (_u32, _u32, _u32, _u32, _u32, _u32)
@@ -97,6 +111,8 @@ def _bind(lib: ctypes.CDLL) -> None:
         fn.argtypes = (ctypes.POINTER(Problem), _vp)
     lib.mi355_w8a8_grouped_v1.restype = ctypes.c_int
     lib.mi355_w8a8_grouped_v1.argtypes = (ctypes.POINTER(GroupedProblem), _vp)
+    lib.mi355_w8a8_lora_linear_bwd_v1.restype = ctypes.c_int
+    lib.mi355_w8a8_lora_linear_bwd_v1.argtypes = (ctypes.POINTER(BwdProblem), _vp)
 
 
 def load() -> ctypes.CDLL:

@@ -9,6 +9,7 @@
 #include "w8a8_gemm.h"
 #include "w8a8_prologue.h"
 #include "w8a8_skinny.h"
+#include "w8a8_backward.h"
 
 using namespace w8a8;
 
@@ -508,6 +509,229 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
   return swiglu ? launch_gemm<kEpiSwiglu, kModeGrouped>(g, w.nkk, s) : launch_gemm<kEpiPlain, kModeGrouped>(g, w.nkk, s);
 }
 
+// ---------------------------------------------------------------------------------------
+// backward
+// ---------------------------------------------------------------------------------------
+struct BwdLayout {
+  uint64_t dyp, swp, at, ap, rp, z, r_raw, rs, src_row, dst_pos, slot_group, blk_range, group_off, partA, partB, total;
+  uint32_t slots, nkk, K_pad, KB, N_pad, NB, tiles_m, tiles_k, max_chunks, R;
+};
+
+BwdLayout make_bwd_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint32_t rank) {
+  BwdLayout w{};
+  w.K_pad = k_padded(k); w.KB = w.K_pad / 32u;
+  w.N_pad = n_padded(n); w.NB = w.N_pad / 32u;
+  w.slots = round_up(m, kTileM);
+  w.tiles_m = w.slots / 256u;
+  w.tiles_k = (w.K_pad + 255u) / 256u;
+  w.nkk = rank_chunks(rank);
+  w.R = w.nkk * 16u;
+  w.max_chunks = (m + kBwdChunkRows - 1u) / kBwdChunkRows + n_groups;
+  uint64_t off = 0;
+  w.dyp = off; off += align256((uint64_t)w.slots * w.N_pad * 2u);
+  w.swp = off; off += align256((uint64_t)(w.N_pad + kBwdScalePad) * 4u);  // a stage fetches 1 KiB of scales starting at its own 32
+  w.src_row = off; off += align256((uint64_t)w.slots * 4u);
+  w.dst_pos = off; off += align256((uint64_t)m * 4u);
+  w.slot_group = off; off += align256((uint64_t)w.slots * 4u);
+  w.blk_range = off; off += align256((uint64_t)(w.slots / 32u) * 4u);
+  w.group_off = off; off += align256((uint64_t)(kMaxAdapters + 1) * 4u);
+  if (rank) {
+    w.at = off; off += align256((uint64_t)n_groups * rank * k * 2u);
+    w.ap = off; off += align256((uint64_t)n_groups * w.KB * w.nkk * kBlockBytes);
+    w.rp = off; off += align256((uint64_t)(w.slots / 32u) * w.nkk * 3u * kBlockBytes);
+    w.z = off; off += align256((uint64_t)w.slots * kBwdRankStride * 4u);
+    w.r_raw = off; off += align256((uint64_t)w.slots * kBwdRankStride * 4u);
+    w.rs = off; off += align256((uint64_t)w.slots * kBwdRankStride * 4u);
+    w.partA = off; off += align256((uint64_t)w.max_chunks * w.R * k * 4u);
+    w.partB = off; off += align256((uint64_t)w.max_chunks * w.R * n * 4u);
+  }
+  w.total = off;
+  return w;
+}
+
+int validate_bwd_dims(uint32_t m, uint32_t k, uint32_t n, uint32_t n_adapters, uint32_t rank) {
+  int st = validate_common(m, k, n);
+  if (st) return st;
+  if (n % 8u) return MI355_W8A8_ERR_UNSUPPORTED;
+  if ((uint64_t)m * k >= (1ull << 32) - (1ull << 20)) return MI355_W8A8_ERR_UNSUPPORTED;  // 32-bit offsets
+  if (n_adapters > (uint32_t)kMaxAdapters || rank > (uint32_t)kMaxRank) return MI355_W8A8_ERR_UNSUPPORTED;
+  if (n_adapters && rank == 0) return MI355_W8A8_ERR_UNSUPPORTED;
+  return MI355_W8A8_OK;
+}
+
+template <int NKK>
+int launch_bwd_dx(const BwdDxArgs& g, hipStream_t s) {
+  const uint32_t ntile = g.tiles_m * g.tiles_k;
+  const uint32_t want = ((ntile + 7u) / 8u) * 8u;
+  const dim3 grid(want < 256u ? want : 256u), block(512);
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_dx_kernel<NKK>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLdsBytes) != hipSuccess)
+    return MI355_W8A8_ERR_LAUNCH;
+  hipLaunchKernelGGL((bwd_dx_kernel<NKK>), grid, block, kBwdLdsBytes, s, g);
+  return launch_status();
+}
+
+int run_backward(const mi355_w8a8_bwd_problem* p, hipStream_t s) {
+  if (!p) return MI355_W8A8_ERR_NULL;
+  if (p->struct_size != sizeof(mi355_w8a8_bwd_problem)) return MI355_W8A8_ERR_STRUCT;
+  int st = validate_bwd_dims(p->m, p->k, p->n, p->n_adapters, p->rank);
+  if (st) return st;
+  if (p->flags) return MI355_W8A8_ERR_SHAPE;
+  if (!p->dy || !p->w_packed || !p->w_scales || !p->dx) return MI355_W8A8_ERR_NULL;
+  const bool lora = p->n_adapters > 0;
+  const bool want_grads = p->d_lora_a || p->d_lora_b || p->d_lora_scaling;
+  if (lora) {
+    if (!p->lora_a || !p->lora_b || !p->lora_scaling) return MI355_W8A8_ERR_NULL;
+    if (want_grads && !p->x) return MI355_W8A8_ERR_NULL;
+  } else if (p->adapter_indices || want_grads) {
+    return MI355_W8A8_ERR_SHAPE;
+  }
+  if (!aligned16(p->x) || !aligned16(p->dy) || !aligned16(p->w_packed) || !aligned16(p->w_scales) ||
+      !aligned16(p->lora_a) || !aligned16(p->lora_b) || !aligned16(p->dx) || !aligned16(p->d_lora_a) ||
+      !aligned16(p->d_lora_b) || !aligned16(p->adapter_indices))
+    return MI355_W8A8_ERR_ALIGN;
+  const uint64_t dx_bytes = (uint64_t)p->m * p->k * 2u, dy_bytes = (uint64_t)p->m * p->n * 2u;
+  const uint64_t a_bytes = (uint64_t)p->n_adapters * p->rank * p->k * 2u, b_bytes = (uint64_t)p->n_adapters * p->rank * p->n * 2u;
+  if (overlaps(p->dx, dx_bytes, p->dy, dy_bytes) || overlaps(p->dx, dx_bytes, p->x, dx_bytes) ||
+      overlaps(p->dx, dx_bytes, p->workspace, p->workspace_bytes) ||
+      overlaps(p->d_lora_a, a_bytes, p->lora_a, a_bytes) || overlaps(p->d_lora_b, b_bytes, p->lora_b, b_bytes) ||
+      overlaps(p->d_lora_a, a_bytes, p->workspace, p->workspace_bytes) ||
+      overlaps(p->d_lora_b, b_bytes, p->workspace, p->workspace_bytes) ||
+      overlaps(p->d_lora_a, a_bytes, p->dx, dx_bytes) || overlaps(p->d_lora_b, b_bytes, p->dx, dx_bytes))
+    return MI355_W8A8_ERR_ALIAS;
+  const BwdLayout w = make_bwd_layout(p->m, p->k, p->n, p->n_adapters, lora ? p->rank : 0u);
+  if (!p->workspace || p->workspace_bytes < w.total) return MI355_W8A8_ERR_WORKSPACE;
+  if (reinterpret_cast<uintptr_t>(p->workspace) & 255u) return MI355_W8A8_ERR_ALIGN;
+  unsigned char* ws = static_cast<unsigned char*>(p->workspace);
+  const bool routed = lora && p->adapter_indices && p->n_adapters > 1;
+  int32_t* src_row = reinterpret_cast<int32_t*>(ws + w.src_row);
+  int32_t* slot_group = reinterpret_cast<int32_t*>(ws + w.slot_group);
+  int32_t* blk_range = reinterpret_cast<int32_t*>(ws + w.blk_range);
+  int32_t* group_off = reinterpret_cast<int32_t*>(ws + w.group_off);
+  (void)hipGetLastError();
+
+  {  // tables: routing, A transposed / in operand order, scales in packed column order
+    BwdPrepArgs pa{};
+    pa.idx = routed ? p->adapter_indices : nullptr;
+    pa.src_row = src_row; pa.dst_pos = reinterpret_cast<int32_t*>(ws + w.dst_pos);
+    pa.slot_group = slot_group; pa.blk_range = blk_range; pa.group_off = group_off;
+    pa.lora_a = static_cast<const uint16_t*>(p->lora_a);
+    pa.at = lora ? reinterpret_cast<uint16_t*>(ws + w.at) : nullptr;
+    pa.ap = lora ? ws + w.ap : nullptr;
+    pa.sw = p->w_scales; pa.swp = reinterpret_cast<float*>(ws + w.swp);
+    pa.M = p->m; pa.K = p->k; pa.N = p->n; pa.N_pad = w.N_pad; pa.n_groups = p->n_adapters; pa.r = p->rank;
+    pa.nkk = w.nkk; pa.kb32 = w.KB; pa.slots = w.slots;
+    pa.route_blocks = lora ? 1u : 0u;
+    pa.a_blocks = lora ? (uint32_t)(((uint64_t)p->n_adapters * p->k * ((p->rank + 7u) / 8u) + 1023u) / 1024u) : 0u;
+    pa.ap_blocks = lora ? (uint32_t)(((uint64_t)p->n_adapters * w.KB * w.nkk * 64u + 1023u) / 1024u) : 0u;
+    const uint32_t sw_blocks = (w.N_pad + 1023u) / 1024u;
+    hipLaunchKernelGGL(bwd_prep_kernel, dim3(pa.route_blocks + pa.a_blocks + pa.ap_blocks + sw_blocks), dim3(1024), 0, s, pa);
+    if ((st = launch_status())) return st;
+  }
+  {  // dy into operand order
+    BwdPackDyArgs d{};
+    d.dy = static_cast<const uint16_t*>(p->dy);
+    d.src_row = routed ? src_row : nullptr;
+    d.dyp = ws + w.dyp;
+    d.M = p->m; d.N = p->n; d.NB = w.NB; d.n_row_blocks = w.slots / 32u; d.n_col_groups = w.N_pad / 128u;
+    const uint64_t waves = (uint64_t)d.n_row_blocks * d.n_col_groups * 2u;
+    hipLaunchKernelGGL(bwd_pack_dy_kernel, dim3((uint32_t)((waves + 3u) / 4u)), dim3(256), 0, s, d);
+    if ((st = launch_status())) return st;
+  }
+  if (lora) {
+    // r = dy @ B.T (raw, scaled, and the scaled value split into bf16 terms for the pull-back epilogue)
+    LoraAArgs la{};
+    la.xsrc = static_cast<const uint16_t*>(p->dy);
+    la.at = static_cast<const uint16_t*>(p->lora_b);  // [n_adapters, rank, n]: already contraction-contiguous
+    la.src_row = routed ? src_row : nullptr;
+    la.slot_group = routed ? slot_group : nullptr;
+    la.blk_range = routed ? blk_range : nullptr;
+    la.zp = ws + w.rp;
+    la.M = p->m; la.K = p->n; la.r = p->rank; la.nkk = w.nkk;
+    la.n_steps = (p->n + 63u) / 64u; la.steps_per_wave = (la.n_steps + 15u) / 16u;
+    la.nterms = 3u;
+    la.n_blocks = w.slots / 32u;
+    la.zf = reinterpret_cast<float*>(ws + w.r_raw);
+    la.zsf = reinterpret_cast<float*>(ws + w.rs);
+    la.group_scale = p->lora_scaling;
+    la.zf_stride = kBwdRankStride;
+    const dim3 grid(la.n_blocks), block(1024);
+    if (w.nkk > 2u) hipLaunchKernelGGL((lora_a_kernel<2>), grid, block, 0, s, la);
+    else hipLaunchKernelGGL((lora_a_kernel<1>), grid, block, 0, s, la);
+    if ((st = launch_status())) return st;
+    if (p->d_lora_b || p->d_lora_scaling) {  // z = x @ A, recomputed rather than saved by the forward
+      LoraAArgs lz = la;
+      lz.xsrc = static_cast<const uint16_t*>(p->x);
+      lz.at = reinterpret_cast<const uint16_t*>(ws + w.at);
+      lz.zp = nullptr;
+      lz.K = p->k;
+      lz.n_steps = (p->k + 63u) / 64u; lz.steps_per_wave = (lz.n_steps + 15u) / 16u;
+      lz.zf = reinterpret_cast<float*>(ws + w.z);
+      lz.zsf = nullptr; lz.group_scale = nullptr;
+      if (w.nkk > 2u) hipLaunchKernelGGL((lora_a_kernel<2>), grid, block, 0, s, lz);
+      else hipLaunchKernelGGL((lora_a_kernel<1>), grid, block, 0, s, lz);
+      if ((st = launch_status())) return st;
+    }
+  }
+  {
+    BwdDxArgs g{};
+    g.dyp = ws + w.dyp;
+    g.wp = static_cast<const unsigned char*>(p->w_packed);
+    g.swp = reinterpret_cast<const float*>(ws + w.swp);
+    g.rp = lora ? ws + w.rp : nullptr;
+    g.ap = lora ? ws + w.ap : nullptr;
+    g.src_row = routed ? src_row : nullptr;
+    g.slot_group = routed ? slot_group : nullptr;
+    g.blk_range = routed ? blk_range : nullptr;
+    g.dx = static_cast<uint16_t*>(p->dx);
+    g.M = p->m; g.K = p->k; g.KB = w.KB; g.NB = w.NB; g.tiles_m = w.tiles_m; g.tiles_k = w.tiles_k;
+    switch (lora ? w.nkk : 0u) {
+      case 0: st = launch_bwd_dx<0>(g, s); break;
+      case 1: st = launch_bwd_dx<1>(g, s); break;
+      case 2: st = launch_bwd_dx<2>(g, s); break;
+      default: st = launch_bwd_dx<4>(g, s); break;
+    }
+    if (st) return st;
+  }
+  if (lora && want_grads) {
+    BwdDloraArgs d{};
+    d.x = static_cast<const uint16_t*>(p->x);
+    d.dy = static_cast<const uint16_t*>(p->dy);
+    d.rs = reinterpret_cast<const float*>(ws + w.rs);
+    d.z = reinterpret_cast<const float*>(ws + w.z);
+    d.src_row = routed ? src_row : nullptr;
+    d.group_off = group_off;
+    d.partA = reinterpret_cast<float*>(ws + w.partA);
+    d.partB = reinterpret_cast<float*>(ws + w.partB);
+    d.M = p->m; d.K = p->k; d.N = p->n; d.n_groups = p->n_adapters; d.max_chunks = w.max_chunks;
+    d.col_tiles_a = p->d_lora_a ? (p->k + 511u) / 512u : 0u;
+    d.col_tiles_b = p->d_lora_b ? (p->n + 511u) / 512u : 0u;
+    if (d.col_tiles_a + d.col_tiles_b) {
+      const dim3 grid(w.max_chunks * (d.col_tiles_a + d.col_tiles_b)), block(256);
+      if (w.R == 16u) hipLaunchKernelGGL((bwd_dlora_kernel<16>), grid, block, 0, s, d);
+      else if (w.R == 32u) hipLaunchKernelGGL((bwd_dlora_kernel<32>), grid, block, 0, s, d);
+      else hipLaunchKernelGGL((bwd_dlora_kernel<64>), grid, block, 0, s, d);
+      if ((st = launch_status())) return st;
+    }
+    BwdReduceArgs r{};
+    r.partA = d.partA; r.partB = d.partB;
+    r.r_raw = reinterpret_cast<const float*>(ws + w.r_raw);
+    r.z = d.z;
+    r.lora_scaling = p->lora_scaling;
+    r.group_off = group_off;
+    r.d_a = static_cast<uint16_t*>(p->d_lora_a);
+    r.d_b = static_cast<uint16_t*>(p->d_lora_b);
+    r.d_s = p->d_lora_scaling;
+    r.K = p->k; r.N = p->n; r.r = p->rank; r.R = w.R; r.n_groups = p->n_adapters;
+    r.blocks_a = p->d_lora_a ? (uint32_t)(((uint64_t)p->n_adapters * p->rank * p->k + 255u) / 256u) : 0u;
+    r.blocks_b = p->d_lora_b ? (uint32_t)(((uint64_t)p->n_adapters * p->rank * p->n + 255u) / 256u) : 0u;
+    const uint32_t s_blocks = p->d_lora_scaling ? p->n_adapters : 0u;
+    hipLaunchKernelGGL(bwd_dlora_reduce_kernel, dim3(r.blocks_a + r.blocks_b + s_blocks), dim3(256), 0, s, r);
+    if ((st = launch_status())) return st;
+  }
+  return MI355_W8A8_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -614,6 +838,17 @@ uint64_t mi355_w8a8_grouped_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, 
 
 int mi355_w8a8_grouped_v1(const mi355_w8a8_grouped_problem* p, void* stream) {
   return run_grouped(p, static_cast<hipStream_t>(stream));
+}
+
+uint64_t mi355_w8a8_bwd_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t n_adapters, uint32_t rank,
+                                        uint32_t flags) {
+  (void)flags;
+  if (validate_bwd_dims(m, k, n, n_adapters, rank)) return 0;
+  return make_bwd_layout(m, k, n, n_adapters, n_adapters ? rank : 0u).total;
+}
+
+int mi355_w8a8_lora_linear_bwd_v1(const mi355_w8a8_bwd_problem* p, void* stream) {
+  return run_backward(p, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

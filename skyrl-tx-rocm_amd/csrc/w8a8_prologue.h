@@ -49,13 +49,16 @@ __global__ __launch_bounds__(256) void unpack_weight_kernel(const unsigned char*
 //   dst_pos[m]    = grouped slot of original row m
 //   slot_group[p] = adapter of grouped slot p
 //   blk_range[b]  = first adapter | last adapter << 16 of the 32-row block b
+//   group_off[a]  = first grouped slot of adapter a (optional; entry n_groups = M)
 // Out-of-range adapter indices are clamped into range (XLA gather semantics).
-// One workgroup; the order of rows inside a group does not influence any result.
+// One workgroup.  The order of rows inside a group does not influence any forward result; the
+// backward asks for the stable order because it sums over a group's rows.
 // ---------------------------------------------------------------------------------------
 __device__ inline void route_rows_block(const int32_t* __restrict__ idx, uint32_t M, uint32_t n_groups,
                                         uint32_t slots, int32_t* __restrict__ src_row,
                                         int32_t* __restrict__ dst_pos, int32_t* __restrict__ slot_group,
-                                        int32_t* __restrict__ blk_range) {
+                                        int32_t* __restrict__ blk_range, int32_t* __restrict__ group_off = nullptr,
+                                        bool stable = false) {
   __shared__ int cnt[kMaxAdapters];
   __shared__ int start[kMaxAdapters + 1];
   __shared__ int cursor[kMaxAdapters];
@@ -77,12 +80,50 @@ __device__ inline void route_rows_block(const int32_t* __restrict__ idx, uint32_
     start[n_groups] = pos;
   }
   __syncthreads();
-  for (uint32_t i = tid; i < M; i += 1024) {
-    int a = idx[i];
-    a = a < 0 ? 0 : (a >= (int)n_groups ? (int)n_groups - 1 : a);
-    const int p = start[a] + atomicAdd(&cursor[a], 1);
-    src_row[p] = (int)i;
-    dst_pos[i] = p;
+  if (group_off && tid <= n_groups) group_off[tid] = start[tid];  // first slot of every group, then M
+  if (stable) {
+    // rows keep their order inside a group (reductions over a group's rows then have a fixed order):
+    // rank = rows of the same group before this one, counted per wave with ballots, per 1024-row
+    // chunk with the waves' counts, and across chunks with the running count in cursor[]
+    __shared__ int wave_cnt[16][kMaxAdapters];
+    const uint32_t lane = tid & 63u, wave = tid >> 6;
+    for (uint32_t base = 0; base < M; base += 1024) {
+      const uint32_t i = base + tid;
+      int a = -1;
+      if (i < M) {
+        a = idx[i];
+        a = a < 0 ? 0 : (a >= (int)n_groups ? (int)n_groups - 1 : a);
+      }
+      int rank = 0;
+      for (uint32_t g = 0; g < n_groups; ++g) {
+        const unsigned long long mask = __builtin_amdgcn_ballot_w64(a == (int)g);
+        if (a == (int)g) rank = __builtin_popcountll(mask & ((1ull << lane) - 1ull));
+        if (lane == 0) wave_cnt[wave][g] = __builtin_popcountll(mask);
+      }
+      __syncthreads();
+      if (a >= 0) {
+        int off = cursor[a];
+        for (uint32_t w = 0; w < wave; ++w) off += wave_cnt[w][a];
+        const int p = start[a] + off + rank;
+        src_row[p] = (int)i;
+        dst_pos[i] = p;
+      }
+      __syncthreads();
+      if (tid < n_groups) {
+        int t = 0;
+        for (uint32_t w = 0; w < 16; ++w) t += wave_cnt[w][tid];
+        cursor[tid] += t;
+      }
+      __syncthreads();
+    }
+  } else {
+    for (uint32_t i = tid; i < M; i += 1024) {
+      int a = idx[i];
+      a = a < 0 ? 0 : (a >= (int)n_groups ? (int)n_groups - 1 : a);
+      const int p = start[a] + atomicAdd(&cursor[a], 1);
+      src_row[p] = (int)i;
+      dst_pos[i] = p;
+    }
   }
   // group of a slot = the group whose [start, start+count) range holds it
   for (uint32_t p = tid; p < slots; p += 1024) {
@@ -380,6 +421,9 @@ struct LoraAArgs {
   unsigned char* zp;        // packed z fragments
   uint32_t M, K, r, nkk, steps_per_wave, n_steps, n_blocks;
   uint32_t nterms;          // bf16 terms carried per value: 3 (exact split of the f32 value) or 2
+  // Optional float32 copies (backward): zf = the raw projection, zsf = the projection times the
+  // row's group scale; with group_scale the packed fragments carry the scaled value.  [slot][zf_stride]
+  float* zf; float* zsf; const float* group_scale; uint32_t zf_stride;
 };
 
 template <int RB>  // number of 32-wide rank blocks (1 or 2)
@@ -473,6 +517,21 @@ __global__ __launch_bounds__(1024) void lora_a_kernel(LoraAArgs a) {
     zs[8u * (e >> 2) + 4u * (l >> 5) + (e & 3u)][b * 32u + (l & 31u)] = sum;
   }
   __syncthreads();
+  if (a.zf || a.group_scale) {
+    for (uint32_t q = threadIdx.x; q < 32u * RB * 32u; q += 1024u) {
+      const uint32_t row = q / (RB * 32u), col = q % (RB * 32u);
+      const float raw = zs[row][col];
+      if (a.zf) a.zf[(size_t)(pb * 32u + row) * a.zf_stride + col] = raw;
+      if (a.group_scale) {
+        const uint32_t gr = (a.slot_group && ghi > glo) ? (uint32_t)a.slot_group[pb * 32u + row] : glo;
+        const float scaled = raw * a.group_scale[gr];
+        zs[row][col] = scaled;
+        if (a.zsf) a.zsf[(size_t)(pb * 32u + row) * a.zf_stride + col] = scaled;
+      }
+    }
+    __syncthreads();
+  }
+  if (!a.zp) return;
   for (uint32_t q = threadIdx.x; q < a.nkk * 3u * 64u; q += 1024u) {
     const uint32_t l = q & 63u, term = (q >> 6) % 3u, kk = q / 192u;
     const uint32_t row = l & 31u, hh = l >> 5;

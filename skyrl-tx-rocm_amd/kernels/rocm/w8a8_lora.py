@@ -331,6 +331,83 @@ def forward(x: torch.Tensor, weight, lora_a=None, lora_b=None, lora_scaling=None
 
 
 # ---------------------------------------------------------------------------------------
+# backward of the plain linear (skyrl/tx/kernels/quantized_lora.py:337-394)
+# ---------------------------------------------------------------------------------------
+
+def backward(x: torch.Tensor | None, dy: torch.Tensor, weight, lora_a=None, lora_b=None, lora_scaling=None, *,
+             adapter_indices: torch.Tensor | None = None, need_lora_grads: bool = True):
+    """Cotangents of ``forward(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=...)``.
+
+    Returns ``(dx, d_lora_a, d_lora_b, d_lora_scaling)``; the LoRA entries are ``None`` without
+    LoRA or with ``need_lora_grads=False``.  The activation quantizer is straight-through; the
+    frozen weight enters as ``bf16(codes * scales)`` (skyrl/tx/kernels/rocm/w8a8_lora.py:298-339).
+    """
+    if dy.dtype != torch.bfloat16:
+        raise TypeError(f"dy must be BF16, got {dy.dtype}")
+    if dy.ndim < 2 or math.prod(dy.shape[:-1]) <= 0:
+        raise ValueError(f"dy must have a nonempty row domain and final N axis, got {tuple(dy.shape)}")
+    _require_cuda(dy, "dy")
+    pw = prepare_weight(weight)
+    k, n = pw.in_features, pw.out_features
+    if dy.shape[-1] != n:
+        raise ValueError(f"dy N={dy.shape[-1]} does not match W8 N={n}")
+    dev = dy.device
+    dyf = dy.reshape(-1, n).contiguous()
+    m = dyf.shape[0]
+    a3, b3, s1, n_ad, r = _normalize_lora(lora_a, lora_b, lora_scaling, k, n, dev)
+    want = bool(n_ad) and need_lora_grads
+    xf = None
+    if want:
+        if x is None:
+            raise ValueError("x is needed for the LoRA cotangents")
+        if x.dtype != torch.bfloat16:
+            raise TypeError(f"x must be BF16, got {x.dtype}")
+        _require_cuda(x, "x")
+        if tuple(x.shape) != (*dy.shape[:-1], k):
+            raise ValueError(f"x must have shape {(*dy.shape[:-1], k)}, got {tuple(x.shape)}")
+        xf = x.reshape(m, k).contiguous()
+    idx = None
+    if adapter_indices is not None:
+        if n_ad == 0:
+            raise ValueError("adapter_indices given without LoRA parameters")
+        idx = adapter_indices.reshape(-1)
+        if idx.shape[0] != m:
+            if idx.shape[0] == 0 or m % idx.shape[0]:
+                raise ValueError(f"adapter_indices of length {idx.shape[0]} do not divide {m} rows")
+            idx = idx.repeat_interleave(m // idx.shape[0])
+        idx = idx.to(device=dev, dtype=torch.int32).contiguous()
+    lib = _native.load()
+    ws_bytes = int(lib.mi355_w8a8_bwd_workspace_bytes(m, k, n, n_ad, r, 0))
+    if ws_bytes == 0:
+        raise ValueError(f"geometry M={m}, K={k}, N={n}, rank={r}, adapters={n_ad} is outside the native backward")
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    dx = torch.empty((m, k), dtype=torch.bfloat16, device=dev)
+    da = torch.empty((n_ad, k, r), dtype=torch.bfloat16, device=dev) if want else None
+    db = torch.empty((n_ad, r, n), dtype=torch.bfloat16, device=dev) if want else None
+    ds = torch.empty((n_ad,), dtype=torch.float32, device=dev) if want else None
+    p = _native.BwdProblem()
+    p.struct_size = ctypes.sizeof(_native.BwdProblem)
+    p.m, p.k, p.n, p.n_adapters, p.rank = m, k, n, n_ad, r
+    p.x = xf.data_ptr() if xf is not None else None
+    p.dy = dyf.data_ptr()
+    p.w_packed = pw.packed.data_ptr()
+    p.w_scales = pw.scales.data_ptr()
+    p.lora_a = a3.data_ptr() if n_ad else None
+    p.lora_b = b3.data_ptr() if n_ad else None
+    p.lora_scaling = s1.data_ptr() if n_ad else None
+    p.adapter_indices = idx.data_ptr() if idx is not None else None
+    p.dx = dx.data_ptr()
+    p.d_lora_a = da.data_ptr() if want else None
+    p.d_lora_b = db.data_ptr() if want else None
+    p.d_lora_scaling = ds.data_ptr() if want else None
+    p.workspace = ws.data_ptr()
+    p.workspace_bytes = ws_bytes
+    with torch.cuda.device(dev):
+        _native.check("mi355_w8a8_lora_linear_bwd_v1", lib.mi355_w8a8_lora_linear_bwd_v1(ctypes.byref(p), _stream_ptr(dev)))
+    return dx.reshape(*dy.shape[:-1], k), da, db, ds
+
+
+# ---------------------------------------------------------------------------------------
 # grouped (ragged, per-expert) variant
 # ---------------------------------------------------------------------------------------
 @dataclass(frozen=True)

@@ -96,3 +96,21 @@ def test_backward_identities():
     np.testing.assert_array_equal(cast[0], o.bf16_round(dx))
     np.testing.assert_array_equal(cast[1], o.bf16_round(da))
     assert cast[3].dtype == F32
+
+
+def test_relaxed_weight_policy_rounds_each_weight_once():
+    """The ROCm pull-back contracts bf16(codes * scales) (rocm/w8a8_lora.py:326-330): dx moves by at
+    most the rounding of the weights, the LoRA cotangents do not move at all."""
+    x, w, a, b, s, dy, idx = _case(21, m=8, k=16, n=24, r=2, n_ad=2)
+    exact = o.quantized_lora_linear_multi_bwd_f32(x, w, a, b, s, idx, dy)
+    relaxed = o.quantized_lora_linear_multi_bwd_f32(x, w, a, b, s, idx, dy, relaxed_weight=True)
+    wdeq = o.dequantize_frozen_weight(w)
+    np.testing.assert_array_equal(o.pullback_weight(w, True), o.bf16_round(wdeq))
+    np.testing.assert_array_equal(o.pullback_weight(w, False), wdeq)
+    bound = np.abs(dy) @ np.abs(o.bf16_round(wdeq) - wdeq).T + 1e-5
+    assert np.all(np.abs(relaxed[0] - exact[0]) <= bound) and np.any(relaxed[0] != exact[0])
+    for i in (1, 2, 3):
+        np.testing.assert_array_equal(relaxed[i], exact[i])
+    base_only = o.quantized_lora_linear_multi_bwd_f32(x, w, a, np.zeros_like(b), s, idx, dy, relaxed_weight=True)[0]
+    np.testing.assert_allclose(base_only, dy.astype(np.float64) @ o.bf16_round(wdeq).T.astype(np.float64),
+                               rtol=1e-6, atol=1e-5)
