@@ -148,3 +148,43 @@ def test_backward_rejects_bad_requests(dev, pkg):
     assert lib.mi355_w8a8_bwd_workspace_bytes(16, 64, 252, 0, 0, 0) == 0   # N not a multiple of 8
     assert lib.mi355_w8a8_bwd_workspace_bytes(16, 60, 256, 0, 0, 0) == 0
     assert lib.mi355_w8a8_bwd_workspace_bytes(16, 64, 256, 2, 0, 0) == 0   # adapters without a rank
+
+
+@pytest.mark.parametrize("m,k,n,r,n_ad", [(4096, 4096, 24576, 32, 8), (4096, 12288, 4096, 32, 8)])
+def test_backward_full_size(dev, pkg, m, k, n, r, n_ad):
+    """The gate/up and down projections of Qwen3-8B at M = 4096: dx on sampled rows (rows are
+    independent in dx), dA / dB / dscaling complete, and the exact properties that do not depend on
+    the size: row permutation permutes dx bitwise, doubling dy doubles everything bitwise."""
+    x, w, a, b, s, idx, dy = _make(20260714 + k, m, k, n, r, n_ad)
+    print(f"[case] backward full size m={m} k={k} n={n}", flush=True)
+    got = _run(pkg, dev, x, w, a, b, s, idx, dy)
+    rng = np.random.default_rng(1)
+    rows = np.sort(rng.choice(m, 48, replace=False))
+    wr = o.pullback_weight(w, True)
+    want_dx = np.empty((len(rows), k), dtype=F32)
+    for j, row in enumerate(rows):
+        g = idx[row]
+        rs = (o._mm64(dy[row:row + 1], b[g].T) * s[g]).astype(F32)
+        want_dx[j] = (o._mm64(dy[row:row + 1], wr.T) + o._mm64(rs, a[g].T))[0]
+    rep = wc.compare(got[0][rows], o.bf16_round(want_dx))
+    print(f"[backward parity full] dx {rep}", flush=True)
+    assert rep["violations"] == 0, rep
+    da = np.zeros_like(a); db = np.zeros_like(b); ds = np.zeros_like(s)
+    for g in range(n_ad):
+        sel = np.nonzero(idx == g)[0]
+        z = o._mm64(x[sel], a[g])
+        rr = o._mm64(dy[sel], b[g].T)
+        da[g] = o._mm64(x[sel].T, (rr * s[g]).astype(F32))
+        db[g] = (o._mm64(z.T, dy[sel]) * s[g]).astype(F32)
+        ds[g] = F32(np.sum(rr.astype(np.float64) * z))
+    for name, u, v in (("dA", got[1], da), ("dB", got[2], db)):
+        rep = wc.compare(u, o.bf16_round(v))
+        print(f"[backward parity full] {name} {rep}", flush=True)
+        assert rep["violations"] == 0, (name, rep)
+    np.testing.assert_allclose(got[3], ds, rtol=1e-3, atol=1e-2)
+    perm = rng.permutation(m)
+    moved = _run(pkg, dev, x[perm], w, a, b, s, idx[perm], dy[perm], need_lora_grads=False)
+    np.testing.assert_array_equal(moved[0], got[0][perm])
+    twice = _run(pkg, dev, x, w, a, b, s, idx, dy * F32(2))
+    for u, v in zip(twice, got):
+        np.testing.assert_array_equal(u, v * F32(2))
