@@ -407,6 +407,45 @@ def backward(x: torch.Tensor | None, dy: torch.Tensor, weight, lora_a=None, lora
     return dx.reshape(*dy.shape[:-1], k), da, db, ds
 
 
+class _LoraLinearFunction(torch.autograd.Function):
+    """``forward`` with the custom derivative of the reference (``_quantized_lora_linear.defvjp``,
+    skyrl/tx/kernels/quantized_lora.py:397): cotangents for x, A, B and the scaling; the frozen
+    codes and scales get none."""
+
+    @staticmethod
+    def forward(ctx, x, lora_a, lora_b, lora_scaling, weight, adapter_indices):
+        out = forward(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices, entry="linear")
+        ctx.save_for_backward(x, lora_a, lora_b, lora_scaling)
+        ctx.weight = weight
+        ctx.adapter_indices = adapter_indices
+        return out
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, lora_a, lora_b, lora_scaling = ctx.saved_tensors
+        need = lora_a is not None and any(ctx.needs_input_grad[1:4])
+        dx, da, db, ds = backward(x, dy.contiguous(), ctx.weight, lora_a, lora_b, lora_scaling,
+                                  adapter_indices=ctx.adapter_indices, need_lora_grads=need)
+        if need:
+            if lora_a.ndim == 2:
+                da, db = da[0], db[0]
+            ds = ds.reshape(lora_scaling.shape).to(lora_scaling.dtype)
+        return dx, da, db, ds, None, None
+
+
+def lora_linear(x: torch.Tensor, weight, lora_a=None, lora_b=None, lora_scaling=None, *,
+                adapter_indices: torch.Tensor | None = None) -> torch.Tensor:
+    """Plain W8A8 (+LoRA) linear that autograd can differentiate: the forward kernels, and the
+    backward kernels when x or a LoRA parameter requires a gradient."""
+    tensors = [t for t in (x, lora_a, lora_b, lora_scaling) if isinstance(t, torch.Tensor)]
+    if not (torch.is_grad_enabled() and any(t.requires_grad for t in tensors)):
+        return forward(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices, entry="linear")
+    scaling = lora_scaling
+    if lora_a is not None and not isinstance(scaling, torch.Tensor):
+        scaling = torch.as_tensor(scaling, dtype=torch.float32, device=x.device)
+    return _LoraLinearFunction.apply(x, lora_a, lora_b, scaling, weight, adapter_indices)
+
+
 # ---------------------------------------------------------------------------------------
 # grouped (ragged, per-expert) variant
 # ---------------------------------------------------------------------------------------
@@ -575,7 +614,7 @@ def w8a8_frozen_linear(x, weight, *, enabled: bool = False, interpret: bool = Fa
     """Frozen W8A8 base only: bf16(dequant(quant(x) @ Wq))."""
     _check_enabled(enabled, interpret, "frozen-linear")
     _check_tiles(block_m, block_n, row_superblock)
-    return forward(x, weight, entry="linear")
+    return lora_linear(x, weight)
 
 
 def w8a8_lora_linear(x, weight, lora_a, lora_b, lora_scaling, *, enabled: bool = False,
@@ -594,7 +633,7 @@ def w8a8_lora_linear(x, weight, lora_a, lora_b, lora_scaling, *, enabled: bool =
         scaling = torch.as_tensor(lora_scaling, dtype=torch.float32)
         if scaling.ndim != 0:
             raise TypeError("lora_scaling must be an FP32 scalar")
-    return forward(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices, entry="linear")
+    return lora_linear(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices)
 
 
 def w8a8_rms_gate_up_lora_swiglu(x, rms_weight, weight, lora_a, lora_b, lora_scaling, *,
@@ -625,7 +664,8 @@ def w8a8_lora_residual(x, weight, lora_a, lora_b, lora_scaling, residual, *, ena
 __all__ = (
     "DEFAULT_BLOCK_M", "DEFAULT_BLOCK_N", "DEFAULT_ROW_SUPERBLOCK", "MAX_BLOCK_M", "MAX_BLOCK_N",
     "MAX_IN_FEATURES", "MAX_OUT_FEATURES", "MAX_ROW_SUPERBLOCK", "MAX_LORA_RANK", "PackedW8Weight",
-    "prepare_weight", "unpack_weight", "dynamic_quantize_rows", "ForwardPlan", "forward", "w8a8_frozen_linear",
+    "prepare_weight", "unpack_weight", "dynamic_quantize_rows", "ForwardPlan", "forward", "backward", "lora_linear",
+    "w8a8_frozen_linear",
     "w8a8_lora_linear", "w8a8_rms_gate_up_lora_swiglu", "w8a8_lora_residual", "PackedGroupedW8Weight",
     "prepare_grouped_weight", "grouped_forward", "w8a8_grouped_lora_linear", "w8a8_moe_expert_mlp",
 )

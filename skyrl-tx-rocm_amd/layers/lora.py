@@ -50,7 +50,9 @@ class LoRALinear(LoRAMixin):
     ``adapter_indices`` holds one adapter per example (leading dimension of ``x``) and is repeated
     per token, as in ``LoRAMixin.apply_lora`` (lora.py:118-157); rows are sorted and un-sorted
     inside the native call.  ``out = bf16(W8A8(x) + s[idx] * (x @ A[idx]) @ B[idx])`` with one
-    cast (skyrl/tx/kernels/quantized_lora.py:298-299).
+    cast (skyrl/tx/kernels/quantized_lora.py:298-299).  When ``x`` or a LoRA tensor requires a
+    gradient the call is differentiable through the native backward (the reference's custom VJP,
+    quantized_lora.py:337-394).
     """
 
     def __init__(self, in_features: int, out_features: int, *, weight: ql.GroupQuantizedWeight | None = None,
@@ -86,10 +88,10 @@ class LoRALinear(LoRAMixin):
         if self._lora_active(adapter_indices):
             if adapter_indices.shape[0] != x.shape[0]:
                 raise ValueError("adapter_indices must hold one entry per example (leading axis of x)")
-            out = w8.forward(x, self.weight, self.lora_A, self.lora_B, self.lora_scaling,
-                             adapter_indices=adapter_indices)
+            out = w8.lora_linear(x, self.weight, self.lora_A, self.lora_B, self.lora_scaling,
+                                 adapter_indices=adapter_indices)
         else:
-            out = w8.forward(x, self.weight)
+            out = w8.lora_linear(x, self.weight)
         return out if self.bias is None else out + self.bias
 
 

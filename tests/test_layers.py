@@ -138,15 +138,16 @@ def test_layers_fail_loudly_without_a_gpu_path(pkg):
 K_IN, N_OUT, RANK, N_AD = 40, 7, 3, 3
 
 
-def _closed_form_layer(pkg, dev, cls=None, **kw):
+def _closed_form_layer(pkg, dev, cls=None, n_out=None, **kw):
     import torch
 
     L = pkg.lora
     cls = cls or L.LoRALinear
-    layer = cls(K_IN, N_OUT, max_lora_adapters=N_AD, max_lora_rank=RANK, device=dev, **kw)
-    kernel = o.bf16_round((np.arange(K_IN * N_OUT, dtype=F32).reshape(K_IN, N_OUT) / 53.0) % 3.0 - 1.5)
+    n_out = n_out or N_OUT
+    layer = cls(K_IN, n_out, max_lora_adapters=N_AD, max_lora_rank=RANK, device=dev, **kw)
+    kernel = o.bf16_round((np.arange(K_IN * n_out, dtype=F32).reshape(K_IN, n_out) / 53.0) % 3.0 - 1.5)
     a = o.bf16_round(np.arange(N_AD * K_IN * RANK, dtype=F32).reshape(N_AD, K_IN, RANK) / 97.0 / 8.0)
-    b = o.bf16_round(np.arange(N_AD * RANK * N_OUT, dtype=F32).reshape(N_AD, RANK, N_OUT) / 89.0)
+    b = o.bf16_round(np.arange(N_AD * RANK * n_out, dtype=F32).reshape(N_AD, RANK, n_out) / 89.0)
     s = np.asarray([0.25, 0.75, 1.25], dtype=F32)
     layer.load_dense(torch.from_numpy(kernel))
     layer.lora_A = torch.from_numpy(a).to(dev).to(torch.bfloat16)
@@ -281,3 +282,47 @@ def test_expert_layer_uses_expert_major_adapter_pairs(pkg, dev):
     np.testing.assert_array_equal(again, got)
     with pytest.raises(NotImplementedError):
         layer(xt, torch.from_numpy(group_sizes).to(dev), group_offset=torch.ones(1, dtype=torch.int32))
+
+
+@pytest.mark.gpu
+def test_linear_gradients_match_oracle_and_generic_routing(pkg, dev):
+    """The reference's gradient test (tests/tx/layers/test_lora_fast_path.py:103-133): the loss on the
+    first example must give the same gradients whether the batch holds that example alone or a
+    second one behind it; here the values are also checked against the oracle's backward."""
+    import torch
+
+    n_out = 8  # the native backward takes output widths that are multiples of 8
+    layer, kernel, w, a, b, s = _closed_form_layer(pkg, dev, n_out=n_out)
+    x = o.bf16_round(np.arange(4 * K_IN, dtype=F32).reshape(1, 4, K_IN) / 17.0 / 8.0)
+    cot = o.bf16_round(np.arange(4 * n_out, dtype=F32).reshape(4, n_out) / 31.0)
+    cot_t = torch.from_numpy(cot).to(dev)
+
+    def grads(duplicate):
+        for name in ("lora_A", "lora_B", "lora_scaling"):
+            setattr(layer, name, getattr(layer, name).detach().clone().requires_grad_(True))
+        xt = torch.from_numpy(x).to(dev).to(torch.bfloat16).requires_grad_(True)
+        inp, indices = xt, torch.tensor([1], dtype=torch.int32, device=dev)
+        if duplicate:
+            inp = torch.cat([xt, (xt * 0.5 + 0.25).detach()], dim=0)
+            indices = torch.tensor([1, 1], dtype=torch.int32, device=dev)
+        out = layer(inp, adapter_indices=indices)[0]
+        loss = (out.float() * cot_t).sum()
+        loss.backward()
+        torch.cuda.synchronize()
+        f = lambda t: t.grad.detach().float().cpu().numpy()
+        return float(loss.detach()), f(xt), f(layer.lora_A), f(layer.lora_B), f(layer.lora_scaling)
+
+    fast, generic = grads(False), grads(True)
+    assert abs(fast[0] - generic[0]) <= 2e-2 * max(1.0, abs(fast[0]))
+    np.testing.assert_array_equal(fast[1], generic[1])           # dx of the first example: same rows, same kernels
+    want = o.quantized_lora_linear_bwd(x[0], w, a[1], b[1], s[1], cot, relaxed_weight=True)
+    assert wc.compare(fast[1][0], want[0])["violations"] == 0
+    assert wc.compare(fast[2][1], want[1])["violations"] == 0
+    assert wc.compare(fast[3][1], want[2])["violations"] == 0
+    np.testing.assert_allclose(fast[4][1], want[3], rtol=1e-3)
+    # adapters no row names receive zero gradients
+    assert not fast[2][[0, 2]].any() and not fast[3][[0, 2]].any() and not fast[4][[0, 2]].any()
+    # the duplicated batch adds the second example's rows to the LoRA gradients only through the
+    # loss, which ignores them: same values up to the summation order
+    for i in (2, 3):
+        assert wc.compare(generic[i], fast[i])["violations"] == 0
