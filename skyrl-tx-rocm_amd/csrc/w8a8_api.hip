@@ -513,8 +513,8 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
 // backward
 // ---------------------------------------------------------------------------------------
 struct BwdLayout {
-  uint64_t dyp, swp, at, ap, rp, z, r_raw, rs, src_row, dst_pos, slot_group, blk_range, group_off, partA, partB, total;
-  uint32_t slots, nkk, K_pad, KB, N_pad, NB, tiles_m, tiles_k, max_chunks, R;
+  uint64_t dyp, swp, at, ap, rp, z, r_raw, rs, rpart, src_row, dst_pos, slot_group, blk_range, group_off, partA, partB, total;
+  uint32_t slots, nkk, K_pad, KB, N_pad, NB, tiles_m, tiles_k, max_chunks, R, n_slices, groups_per_slice;
 };
 
 BwdLayout make_bwd_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint32_t rank) {
@@ -525,8 +525,13 @@ BwdLayout make_bwd_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups,
   w.tiles_m = w.slots / 256u;
   w.tiles_k = (w.K_pad + 255u) / 256u;
   w.nkk = rank_chunks(rank);
-  w.R = w.nkk * 16u;
+  w.R = w.nkk > 2u ? 64u : 32u;  // rank rows of a partial (32-wide rank blocks)
   w.max_chunks = (m + kBwdChunkRows - 1u) / kBwdChunkRows + n_groups;
+  {  // dy is packed (and r accumulated) by workgroups that own a slice of the 128-column groups
+    const uint32_t ng = w.N_pad / 128u;
+    w.n_slices = (ng + 3u) / 4u < 8u ? (ng + 3u) / 4u : 8u;
+    w.groups_per_slice = (ng + w.n_slices - 1u) / w.n_slices;
+  }
   uint64_t off = 0;
   w.dyp = off; off += align256((uint64_t)w.slots * w.N_pad * 2u);
   w.swp = off; off += align256((uint64_t)(w.N_pad + kBwdScalePad) * 4u);  // a stage fetches 1 KiB of scales starting at its own 32
@@ -542,6 +547,7 @@ BwdLayout make_bwd_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups,
     w.z = off; off += align256((uint64_t)w.slots * kBwdRankStride * 4u);
     w.r_raw = off; off += align256((uint64_t)w.slots * kBwdRankStride * 4u);
     w.rs = off; off += align256((uint64_t)w.slots * kBwdRankStride * 4u);
+    w.rpart = off; off += align256((uint64_t)w.n_slices * w.slots * kBwdRankStride * 4u);  // also the K slices of z
     w.partA = off; off += align256((uint64_t)w.max_chunks * w.R * k * 4u);
     w.partB = off; off += align256((uint64_t)w.max_chunks * w.R * n * 4u);
   }
@@ -628,48 +634,65 @@ int run_backward(const mi355_w8a8_bwd_problem* p, hipStream_t s) {
     hipLaunchKernelGGL(bwd_prep_kernel, dim3(pa.route_blocks + pa.a_blocks + pa.ap_blocks + sw_blocks), dim3(1024), 0, s, pa);
     if ((st = launch_status())) return st;
   }
-  {  // dy into operand order
+  {  // dy into operand order; the same pass leaves the partial sums of r = dy @ B.T
     BwdPackDyArgs d{};
     d.dy = static_cast<const uint16_t*>(p->dy);
     d.src_row = routed ? src_row : nullptr;
+    d.slot_group = routed ? slot_group : nullptr;
+    d.blk_range = routed ? blk_range : nullptr;
     d.dyp = ws + w.dyp;
+    d.lora_b = static_cast<const uint16_t*>(p->lora_b);
+    d.rpart = lora ? reinterpret_cast<float*>(ws + w.rpart) : nullptr;
     d.M = p->m; d.N = p->n; d.NB = w.NB; d.n_row_blocks = w.slots / 32u; d.n_col_groups = w.N_pad / 128u;
-    const uint64_t waves = (uint64_t)d.n_row_blocks * d.n_col_groups * 2u;
-    hipLaunchKernelGGL(bwd_pack_dy_kernel, dim3((uint32_t)((waves + 3u) / 4u)), dim3(256), 0, s, d);
+    d.n_slices = w.n_slices; d.groups_per_slice = w.groups_per_slice; d.r = p->rank; d.slots = w.slots;
+    const dim3 grid(d.n_row_blocks * d.n_slices), block(256);
+    if (!lora) hipLaunchKernelGGL((bwd_pack_dy_kernel<0>), grid, block, 0, s, d);
+    else if (w.nkk > 2u) hipLaunchKernelGGL((bwd_pack_dy_kernel<2>), grid, block, 0, s, d);
+    else hipLaunchKernelGGL((bwd_pack_dy_kernel<1>), grid, block, 0, s, d);
     if ((st = launch_status())) return st;
   }
   if (lora) {
-    // r = dy @ B.T (raw, scaled, and the scaled value split into bf16 terms for the pull-back epilogue)
-    LoraAArgs la{};
-    la.xsrc = static_cast<const uint16_t*>(p->dy);
-    la.at = static_cast<const uint16_t*>(p->lora_b);  // [n_adapters, rank, n]: already contraction-contiguous
-    la.src_row = routed ? src_row : nullptr;
-    la.slot_group = routed ? slot_group : nullptr;
-    la.blk_range = routed ? blk_range : nullptr;
-    la.zp = ws + w.rp;
-    la.M = p->m; la.K = p->n; la.r = p->rank; la.nkk = w.nkk;
-    la.n_steps = (p->n + 63u) / 64u; la.steps_per_wave = (la.n_steps + 15u) / 16u;
-    la.nterms = 3u;
-    la.n_blocks = w.slots / 32u;
-    la.zf = reinterpret_cast<float*>(ws + w.r_raw);
-    la.zsf = reinterpret_cast<float*>(ws + w.rs);
-    la.group_scale = p->lora_scaling;
-    la.zf_stride = kBwdRankStride;
-    const dim3 grid(la.n_blocks), block(1024);
-    if (w.nkk > 2u) hipLaunchKernelGGL((lora_a_kernel<2>), grid, block, 0, s, la);
-    else hipLaunchKernelGGL((lora_a_kernel<1>), grid, block, 0, s, la);
-    if ((st = launch_status())) return st;
+    {
+      BwdRFinishArgs f{};
+      f.rpart = reinterpret_cast<const float*>(ws + w.rpart);
+      f.slot_group = routed ? slot_group : nullptr;
+      f.lora_scaling = p->lora_scaling;
+      f.r_raw = reinterpret_cast<float*>(ws + w.r_raw);
+      f.rs = reinterpret_cast<float*>(ws + w.rs);
+      f.rp = ws + w.rp;
+      f.n_slices = w.n_slices; f.slots = w.slots; f.nkk = w.nkk; f.cols = w.nkk > 2u ? 64u : 32u;
+      hipLaunchKernelGGL(bwd_r_finish_kernel, dim3(w.slots / 32u), dim3(256), 0, s, f);
+      if ((st = launch_status())) return st;
+    }
     if (p->d_lora_b || p->d_lora_scaling) {  // z = x @ A, recomputed rather than saved by the forward
-      LoraAArgs lz = la;
+      LoraAArgs lz{};
       lz.xsrc = static_cast<const uint16_t*>(p->x);
       lz.at = reinterpret_cast<const uint16_t*>(ws + w.at);
+      lz.src_row = routed ? src_row : nullptr;
+      lz.slot_group = routed ? slot_group : nullptr;
+      lz.blk_range = routed ? blk_range : nullptr;
       lz.zp = nullptr;
-      lz.K = p->k;
+      lz.M = p->m; lz.K = p->k; lz.r = p->rank; lz.nkk = w.nkk;
       lz.n_steps = (p->k + 63u) / 64u; lz.steps_per_wave = (lz.n_steps + 15u) / 16u;
-      lz.zf = reinterpret_cast<float*>(ws + w.z);
-      lz.zsf = nullptr; lz.group_scale = nullptr;
+      lz.nterms = 3u;
+      lz.n_blocks = w.slots / 32u;
+      // K is cut into slices so that the launch fills the chip; the slices land in the partial
+      // table (r's partials have been consumed) and are added in slice order
+      const uint32_t nks = w.n_slices;
+      lz.n_ksplit = nks;
+      lz.steps_per_wave = ((lz.n_steps + nks - 1u) / nks + 15u) / 16u;
+      lz.zf = reinterpret_cast<float*>(ws + w.rpart);
+      lz.zf_stride = kBwdRankStride;
+      lz.zf_slice = w.slots * kBwdRankStride;
+      const dim3 grid(lz.n_blocks * nks), block(1024);
       if (w.nkk > 2u) hipLaunchKernelGGL((lora_a_kernel<2>), grid, block, 0, s, lz);
       else hipLaunchKernelGGL((lora_a_kernel<1>), grid, block, 0, s, lz);
+      if ((st = launch_status())) return st;
+      BwdRFinishArgs f{};
+      f.rpart = reinterpret_cast<const float*>(ws + w.rpart);
+      f.r_raw = reinterpret_cast<float*>(ws + w.z);
+      f.n_slices = nks; f.slots = w.slots; f.nkk = w.nkk; f.cols = w.nkk > 2u ? 64u : 32u;
+      hipLaunchKernelGGL(bwd_r_finish_kernel, dim3(w.slots / 32u), dim3(256), 0, s, f);
       if ((st = launch_status())) return st;
     }
   }
@@ -704,13 +727,19 @@ int run_backward(const mi355_w8a8_bwd_problem* p, hipStream_t s) {
     d.partA = reinterpret_cast<float*>(ws + w.partA);
     d.partB = reinterpret_cast<float*>(ws + w.partB);
     d.M = p->m; d.K = p->k; d.N = p->n; d.n_groups = p->n_adapters; d.max_chunks = w.max_chunks;
-    d.col_tiles_a = p->d_lora_a ? (p->k + 511u) / 512u : 0u;
-    d.col_tiles_b = p->d_lora_b ? (p->n + 511u) / 512u : 0u;
+    d.col_tiles_a = p->d_lora_a ? (p->k + 255u) / 256u : 0u;
+    d.col_tiles_b = p->d_lora_b ? (p->n + 255u) / 256u : 0u;
     if (d.col_tiles_a + d.col_tiles_b) {
       const dim3 grid(w.max_chunks * (d.col_tiles_a + d.col_tiles_b)), block(256);
-      if (w.R == 16u) hipLaunchKernelGGL((bwd_dlora_kernel<16>), grid, block, 0, s, d);
-      else if (w.R == 32u) hipLaunchKernelGGL((bwd_dlora_kernel<32>), grid, block, 0, s, d);
-      else hipLaunchKernelGGL((bwd_dlora_kernel<64>), grid, block, 0, s, d);
+      const uint32_t lds_bytes = (kBwdStageRows / 32u) * (w.R / 32u) * 6u * kBlockBytes;
+      if (w.R == 32u) {
+        hipLaunchKernelGGL((bwd_dlora_kernel<1>), grid, block, lds_bytes, s, d);
+      } else {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_dlora_kernel<2>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
+          return MI355_W8A8_ERR_LAUNCH;
+        hipLaunchKernelGGL((bwd_dlora_kernel<2>), grid, block, lds_bytes, s, d);
+      }
       if ((st = launch_status())) return st;
     }
     BwdReduceArgs r{};
@@ -724,7 +753,7 @@ int run_backward(const mi355_w8a8_bwd_problem* p, hipStream_t s) {
     r.d_s = p->d_lora_scaling;
     r.K = p->k; r.N = p->n; r.r = p->rank; r.R = w.R; r.n_groups = p->n_adapters;
     r.blocks_a = p->d_lora_a ? (uint32_t)(((uint64_t)p->n_adapters * p->rank * p->k + 255u) / 256u) : 0u;
-    r.blocks_b = p->d_lora_b ? (uint32_t)(((uint64_t)p->n_adapters * p->rank * p->n + 255u) / 256u) : 0u;
+    r.blocks_b = p->d_lora_b ? (uint32_t)(((uint64_t)p->n_adapters * p->rank * p->n / 4u + 255u) / 256u) : 0u;
     const uint32_t s_blocks = p->d_lora_scaling ? p->n_adapters : 0u;
     hipLaunchKernelGGL(bwd_dlora_reduce_kernel, dim3(r.blocks_a + r.blocks_b + s_blocks), dim3(256), 0, s, r);
     if ((st = launch_status())) return st;

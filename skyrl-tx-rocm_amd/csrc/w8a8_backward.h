@@ -23,51 +23,157 @@ namespace w8a8 {
 //   32 nb + 16 q + 8 (e / 4) + 4 h + e % 4,
 // the n that the transposing MFMA leaves in contraction slot 8 h + e of its q-th half.  Rows are
 // in grouped (adapter-sorted) slot order; slots without a row and columns beyond N are zero.
-// One wave per (row block, 128-column group, q): a lane reads 2 x 16 consecutive original columns
-// of its row and owns the four packed blocks (j = column % 4) that interleave them.
+// A wave takes a row block and a 128-column group at a time: a lane reads 4 x 16 consecutive
+// original columns of its row and owns the pieces of the eight packed blocks (q, j = column % 4)
+// that interleave them.
+// The same pass computes r = dy @ B[group].T on bf16 MFMAs (the 8-value pieces a lane has loaded
+// are A operands as they are; the matching pieces of B are 16-byte loads), so dy is read once:
+// a workgroup of four waves owns one 32-row block and one slice of the 128-column groups, and
+// leaves its partial sum in rpart[slice][slot][64]; bwd_r_finish_kernel adds the slices.
 // ---------------------------------------------------------------------------------------
+constexpr uint32_t kBwdRankStride = 64;  // floats per slot in the z / r tables
+
 struct BwdPackDyArgs {
-  const uint16_t* dy;      // bf16 [M, N]
-  const int32_t* src_row;  // original row of a slot or null (identity)
+  const uint16_t* dy;        // bf16 [M, N]
+  const int32_t* src_row;    // original row of a slot or null (identity)
+  const int32_t* slot_group; // or null (group 0)
+  const int32_t* blk_range;  // or null
   unsigned char* dyp;
-  uint32_t M, N, NB, n_row_blocks, n_col_groups;
+  const uint16_t* lora_b;    // bf16 [n_groups, r, N] or null (no LoRA: packing only)
+  float* rpart;              // f32 [n_slices][slots][64]
+  uint32_t M, N, NB, n_row_blocks, n_col_groups, n_slices, groups_per_slice, r, slots;
 };
 
+template <int RB>  // 32-wide rank blocks (0 = packing only)
 __global__ __launch_bounds__(256) void bwd_pack_dy_kernel(BwdPackDyArgs a) {
-  const uint32_t lane = threadIdx.x & 63u;
-  const uint64_t gid = (uint64_t)blockIdx.x * 4u + (threadIdx.x >> 6);
-  const uint32_t q = (uint32_t)(gid & 1u);
-  const uint64_t rest = gid >> 1;
-  const uint32_t G = (uint32_t)(rest % a.n_col_groups);
-  const uint32_t mb = (uint32_t)(rest / a.n_col_groups);
+  constexpr int kRB = RB > 0 ? RB : 1;
+  __shared__ float red[4][kRB][16][64];
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  const uint32_t mb = blockIdx.x / a.n_slices, sl = blockIdx.x % a.n_slices;
   if (mb >= a.n_row_blocks) return;
   const uint32_t i = lane & 31u, h = lane >> 5;
   const uint32_t p = mb * 32u + i;
   int src = -1;
   if (a.src_row) src = a.src_row[p]; else if (p < a.M) src = (int)p;
   if (src >= (int)a.M) src = -1;
-  const uint32_t c0 = 128u * G + 64u * q + 16u * h;
-  uint16_t v[2][16];
+  const uint32_t range = (RB > 0 && a.blk_range) ? (uint32_t)a.blk_range[mb] : 0u;
+  const uint32_t glo = range & 0xffffu, ghi = range >> 16;
+  const uint32_t rowgrp = (RB > 0 && a.slot_group && ghi > glo) ? (uint32_t)a.slot_group[p] : glo;
+  const bool vec = (a.N & 7u) == 0;
+  v16f acc[kRB];
 #pragma unroll
-  for (int ch = 0; ch < 2; ++ch) {
-    const uint32_t col = c0 + 32u * ch;
-    if (src >= 0 && col + 16u <= a.N && (a.N & 7u) == 0) {
-      const v8us lo = *reinterpret_cast<const v8us*>(a.dy + (size_t)src * a.N + col);
-      const v8us hi = *reinterpret_cast<const v8us*>(a.dy + (size_t)src * a.N + col + 8u);
+  for (int b = 0; b < kRB; ++b)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) { v[ch][e] = lo[e]; v[ch][8 + e] = hi[e]; }
-    } else {
+    for (int e = 0; e < 16; ++e) acc[b][e] = 0.0f;
+  const uint32_t g_end = (sl + 1u) * a.groups_per_slice < a.n_col_groups ? (sl + 1u) * a.groups_per_slice : a.n_col_groups;
+  for (uint32_t G = sl * a.groups_per_slice + wave; G < g_end; G += 4u) {
+    // piece t = 4 q + 2 ch + part: the 8 columns 128 G + 64 q + 32 ch + 16 h + 8 part .. + 7 of the lane's row
+    v8us pc[8];
 #pragma unroll
-      for (int e = 0; e < 16; ++e) v[ch][e] = (src >= 0 && col + e < a.N) ? a.dy[(size_t)src * a.N + col + e] : (uint16_t)0;
+    for (int t = 0; t < 8; ++t) {
+      const uint32_t col = 128u * G + 64u * (t >> 2) + 32u * ((t >> 1) & 1) + 16u * h + 8u * (t & 1);
+      if (src >= 0 && vec && col + 8u <= a.N) {
+        pc[t] = *reinterpret_cast<const v8us*>(a.dy + (size_t)src * a.N + col);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) pc[t][e] = (src >= 0 && col + e < a.N) ? a.dy[(size_t)src * a.N + col + e] : (uint16_t)0;
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        // element e < 4 of packed block j: column 4 e + j of the first 16, e >= 4: of the second 16
+        v8us o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          o[e] = pc[4 * q + ((4 * e + j) >> 3)][(4 * e + j) & 7];
+          o[4 + e] = pc[4 * q + 2 + ((4 * e + j) >> 3)][(4 * e + j) & 7];
+        }
+        const size_t off = ((((size_t)mb * a.NB + 4u * G + j) * 2u + q) * 64u + lane) * 16u;
+        *reinterpret_cast<v8us*>(a.dyp + off) = o;
+      }
+    if constexpr (RB > 0) {
+      // a block at a group boundary runs once per group with the other groups' rows zeroed
+      for (uint32_t grp = glo; grp <= ghi; ++grp) {
+        const bool mine = src >= 0 && rowgrp == grp;
+        const uint16_t* bg = a.lora_b + (size_t)grp * a.r * a.N;
+        v8us wb[RB][8];
+#pragma unroll
+        for (int b = 0; b < RB; ++b)
+#pragma unroll
+          for (int t = 0; t < 8; ++t) {
+            const uint32_t col = 128u * G + 64u * (t >> 2) + 32u * ((t >> 1) & 1) + 16u * h + 8u * (t & 1);
+            const uint32_t j = b * 32u + i;
+            const v8us zero = {0, 0, 0, 0, 0, 0, 0, 0};
+            wb[b][t] = (j < a.r && col + 8u <= a.N) ? *reinterpret_cast<const v8us*>(bg + (size_t)j * a.N + col) : zero;
+          }
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+          const v8us zero = {0, 0, 0, 0, 0, 0, 0, 0};
+          const v8bf xa = __builtin_bit_cast(v8bf, mine ? pc[t] : zero);
+#pragma unroll
+          for (int b = 0; b < RB; ++b)
+            acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa, __builtin_bit_cast(v8bf, wb[b][t]), acc[b], 0, 0, 0);
+        }
+      }
     }
   }
+  if constexpr (RB > 0) {
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
+    for (int b = 0; b < RB; ++b)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) red[wave][b][e][lane] = acc[b][e];
+    __syncthreads();
+    for (uint32_t q = threadIdx.x; q < RB * 1024u; q += 256u) {
+      const uint32_t l = q & 63u, e = (q >> 6) & 15u, b = q >> 10;
+      const float sum = ((red[0][b][e][l] + red[1][b][e][l]) + red[2][b][e][l]) + red[3][b][e][l];
+      const uint32_t row = 8u * (e >> 2) + 4u * (l >> 5) + (e & 3u), col = b * 32u + (l & 31u);
+      a.rpart[((size_t)sl * a.slots + mb * 32u + row) * kBwdRankStride + col] = sum;
+    }
+  }
+}
+
+// r of a 32-row block: the slices' partial sums added in slice order; written raw (for dscaling),
+// scaled by the row's group (for dA), and the scaled value split exactly into three bf16 terms in
+// the operand order of the pull-back epilogue, rp[block][kk][term][lane][8].
+struct BwdRFinishArgs {
+  const float* rpart; const int32_t* slot_group; const float* lora_scaling;
+  float* r_raw; float* rs; unsigned char* rp;
+  uint32_t n_slices, slots, nkk, cols;  // cols = 16 * nkk rounded up to 32
+};
+
+__global__ __launch_bounds__(256) void bwd_r_finish_kernel(BwdRFinishArgs a) {
+  __shared__ float zs[32][kBwdRankStride + 1];
+  const uint32_t pb = blockIdx.x;
+  for (uint32_t q = threadIdx.x; q < 32u * a.cols; q += 256u) {
+    const uint32_t row = q / a.cols, col = q % a.cols, slot = pb * 32u + row;
+    float raw = 0.0f;
+    for (uint32_t sl = 0; sl < a.n_slices; ++sl) raw += a.rpart[((size_t)sl * a.slots + slot) * kBwdRankStride + col];
+    a.r_raw[(size_t)slot * kBwdRankStride + col] = raw;
+    if (!a.rp) continue;  // plain sum of the slices (the z table)
+    const uint32_t gr = a.slot_group ? (uint32_t)a.slot_group[slot] : 0u;
+    const float scaled = raw * a.lora_scaling[gr];
+    a.rs[(size_t)slot * kBwdRankStride + col] = scaled;
+    zs[row][col] = scaled;
+  }
+  if (!a.rp) return;
+  __syncthreads();
+  for (uint32_t q = threadIdx.x; q < a.nkk * 3u * 64u; q += 256u) {
+    const uint32_t l = q & 63u, term = (q >> 6) % 3u, kk = q / 192u;
+    const uint32_t row = l & 31u, hh = l >> 5;
     v8us o;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) { o[e] = v[0][4 * e + j]; o[4 + e] = v[1][4 * e + j]; }
-    const size_t off = ((((size_t)mb * a.NB + 4u * G + j) * 2u + q) * 64u + lane) * 16u;
-    *reinterpret_cast<v8us*>(a.dyp + off) = o;
+    for (int e = 0; e < 8; ++e) {
+      const float z = zs[row][16u * kk + 8u * hh + e];
+      const uint32_t b0 = f32_to_bf16_bits(z);
+      const float r1 = z - bf16_bits_to_f32(b0);
+      const uint32_t b1 = f32_to_bf16_bits(r1);
+      const float r2 = r1 - bf16_bits_to_f32(b1);
+      const uint32_t b2 = f32_to_bf16_bits(r2);
+      o[e] = (unsigned short)(term == 0 ? b0 : (term == 1 ? b1 : b2));
+    }
+    *reinterpret_cast<v8us*>(a.rp + (((size_t)pb * a.nkk + kk) * 3u + term) * kBlockBytes + l * 16u) = o;
   }
 }
 
@@ -414,15 +520,15 @@ __global__ __launch_bounds__(512, 1) void bwd_dx_kernel(BwdDxArgs g) {
 
 // ---------------------------------------------------------------------------------------
 // LoRA cotangents.  Rows are in grouped order; group g owns slots group_off[g] .. group_off[g+1].
-// Every group is cut into chunks of 256 rows; chunk c of the call computes, for its rows,
+// Every group is cut into chunks of 512 rows; chunk c of the call computes, for its rows,
 //   partA[c][j][k] = sum_m rs[m][j] * x[m][k]        partB[c][j][n] = sum_m z[m][j] * dy[m][n]
-// in float32 (a thread owns two adjacent columns and the whole rank), and a second kernel adds a
+// with float32 accumulation, and a second kernel adds a
 // group's chunks in chunk order, scales dB, casts and writes dA [g][K][r], dB [g][r][N], plus
 // ds[g] = sum_m sum_j r[m][j] * z[m][j] with r the unscaled dy @ B.T.  Fixed orders: results are
 // deterministic.
 // ---------------------------------------------------------------------------------------
-constexpr uint32_t kBwdChunkRows = 256;
-constexpr uint32_t kBwdRankStride = 64;  // floats per slot in the z / r tables
+constexpr uint32_t kBwdChunkRows = 512;  // rows of a chunk
+constexpr uint32_t kBwdStageRows = 256;  // rows whose skinny operand sits in LDS at a time
 
 struct BwdDloraArgs {
   const uint16_t* x;        // bf16 [M, K]
@@ -454,13 +560,21 @@ __device__ inline bool bwd_find_chunk(const int32_t* group_off, uint32_t n_group
   return false;
 }
 
-template <int R>  // rank padded to 16, 32 or 64
+// Matrix-core version.  out[j][c] = sum_m P[m][j] * Q[m][c] contracts over rows, so both operands
+// need the row index inside a lane.  P (float32, 32 or 64 rank columns) is split exactly into three
+// bf16 terms and staged in LDS in A-operand order.  Q (bf16 rows of x or dy) is read as ordinary
+// row fragments and transposed by the matrix core: two v_mfma_f32_32x32x16_bf16 against identity
+// halves return Q[m][c] with lane = c and sixteen rows per lane (exact: the values are bf16), which
+// packs into the B operands of the contraction over m.  A wave owns 64 columns (two 32-column
+// strips) and walks the chunk's 32-row blocks, eight per staging pass of P; a workgroup of four
+// waves owns 256 columns.
+template <int RB>  // 32-wide rank blocks
 __global__ __launch_bounds__(256) void bwd_dlora_kernel(BwdDloraArgs a) {
-  constexpr uint32_t kStageRows = 128;  // rows of the skinny operand staged in LDS at a time
-  __shared__ float P[kStageRows][R];
-  __shared__ int rowsrc[kStageRows];
+  // P operands: [row block 8][rank block RB][q 2][term 3][64 lanes][8 bf16]
+  extern __shared__ __attribute__((aligned(1024))) unsigned char pop[];
+  __shared__ int rowsrc[kBwdStageRows];
   __shared__ uint32_t info[3];
-  const uint32_t tid = threadIdx.x;
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const uint32_t per_chunk = a.col_tiles_a + a.col_tiles_b;
   const uint32_t cid = blockIdx.x / per_chunk, ct = blockIdx.x % per_chunk;
   if (tid == 0) {
@@ -476,52 +590,112 @@ __global__ __launch_bounds__(256) void bwd_dlora_kernel(BwdDloraArgs a) {
   const uint16_t* Q = job_a ? a.x : a.dy;
   const uint32_t C = job_a ? a.K : a.N;
   float* part = job_a ? a.partA : a.partB;
-  const uint32_t col = ((job_a ? ct : ct - a.col_tiles_a) * 256u + tid) * 2u;
-  const bool active = col < C;  // C is even
-  const uint16_t* qcol = Q + (active ? col : 0u);
-  float acc0[R], acc1[R];
+  const uint32_t c = lane & 31u, h = lane >> 5;
+  const uint32_t col0 = ((job_a ? ct : ct - a.col_tiles_a) * 4u + wave) * 64u;  // first column of the wave
+  const bool active = col0 < C;
+  // identity halves: lane (column c, half h) element e is 1 where the contraction slot 8 h + e is column c
+  v8us id0 = {0, 0, 0, 0, 0, 0, 0, 0}, id1 = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-  for (int j = 0; j < R; ++j) { acc0[j] = 0.0f; acc1[j] = 0.0f; }
-  for (uint32_t base = 0; base < rows; base += kStageRows) {
-    const uint32_t cnt = rows - base < kStageRows ? rows - base : kStageRows;
-    __syncthreads();
-    for (uint32_t i = tid; i < cnt * R; i += 256u)
-      P[i / R][i % R] = psrc[(size_t)(slot0 + base + i / R) * kBwdRankStride + i % R];
-    for (uint32_t i = tid; i < cnt; i += 256u)
-      rowsrc[i] = a.src_row ? a.src_row[slot0 + base + i] : (int)(slot0 + base + i);
+  for (int e = 0; e < 8; ++e) {
+    id0[e] = (c == 8u * h + e) ? (unsigned short)0x3f80 : (unsigned short)0;
+    id1[e] = (c == 16u + 8u * h + e) ? (unsigned short)0x3f80 : (unsigned short)0;
+  }
+  v16f acc[2][RB];
+#pragma unroll
+  for (int st = 0; st < 2; ++st)
+#pragma unroll
+    for (int b = 0; b < RB; ++b)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[st][b][e] = 0.0f;
+  const v8us zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  auto load_q = [&](uint32_t bi, v8us (&dst)[2][2]) {  // [strip][column half]: row c of the block, 8 columns
+    const int srow = rowsrc[bi * 32u + c];
+#pragma unroll
+    for (int st = 0; st < 2; ++st)
+#pragma unroll
+      for (int hc = 0; hc < 2; ++hc) {
+        const uint32_t col = col0 + 32u * st + 16u * hc + 8u * h;
+        dst[st][hc] = (srow >= 0 && col + 8u <= C) ? *reinterpret_cast<const v8us*>(Q + (size_t)srow * C + col) : zero8;
+      }
+  };
+  for (uint32_t base = 0; base < rows; base += kBwdStageRows) {
+    const uint32_t cnt = rows - base < kBwdStageRows ? rows - base : kBwdStageRows;
+    const uint32_t n_blocks = (cnt + 31u) / 32u;
+    __syncthreads();  // the previous pass's operands are no longer read
+    // stage P: item = (row block, rank block, q, lane); element e is row 16 q + 8 (e / 4) + 4 h + e % 4
+    for (uint32_t it = tid; it < n_blocks * RB * 2u * 64u; it += 256u) {
+      const uint32_t l = it & 63u, q = (it >> 6) & 1u, jb = (it >> 7) % RB, bi = (it >> 7) / RB;
+      const uint32_t j = jb * 32u + (l & 31u), hh = l >> 5;
+      v8us t0, t1, t2;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const uint32_t m = bi * 32u + 16u * q + 8u * (e >> 2) + 4u * hh + (e & 3);
+        const float v = m < cnt ? psrc[(size_t)(slot0 + base + m) * kBwdRankStride + j] : 0.0f;
+        const uint32_t b0 = f32_to_bf16_bits(v);
+        const float r1 = v - bf16_bits_to_f32(b0);
+        const uint32_t b1 = f32_to_bf16_bits(r1);
+        const float r2 = r1 - bf16_bits_to_f32(b1);
+        t0[e] = (unsigned short)b0; t1[e] = (unsigned short)b1; t2[e] = (unsigned short)f32_to_bf16_bits(r2);
+      }
+      unsigned char* dst = pop + ((((size_t)bi * RB + jb) * 2u + q) * 3u) * kBlockBytes + l * 16u;
+      *reinterpret_cast<v8us*>(dst) = t0;
+      *reinterpret_cast<v8us*>(dst + kBlockBytes) = t1;
+      *reinterpret_cast<v8us*>(dst + 2 * kBlockBytes) = t2;
+    }
+    for (uint32_t i = tid; i < kBwdStageRows; i += 256u)
+      rowsrc[i] = i < cnt ? (a.src_row ? a.src_row[slot0 + base + i] : (int)(slot0 + base + i)) : -1;
     __syncthreads();
     if (!active) continue;
-    uint32_t m = 0;
-    for (; m + 4u <= cnt; m += 4u) {
-      uint32_t w[4];
+    v8us qf[2][2];
+    load_q(0, qf);
+    for (uint32_t bi = 0; bi < n_blocks; ++bi) {
+      v8us qn[2][2];
+      if (bi + 1u < n_blocks) load_q(bi + 1u, qn);
 #pragma unroll
-      for (int u = 0; u < 4; ++u) w[u] = *reinterpret_cast<const uint32_t*>(qcol + (size_t)rowsrc[m + u] * C);
+      for (int st = 0; st < 2; ++st) {
+        v16f tr;
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const float q0 = __uint_as_float(w[u] << 16), q1 = __uint_as_float(w[u] & 0xffff0000u);
+        for (int e = 0; e < 16; ++e) tr[e] = 0.0f;
+        tr = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, qf[st][0]), __builtin_bit_cast(v8bf, id0), tr, 0, 0, 0);
+        tr = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, qf[st][1]), __builtin_bit_cast(v8bf, id1), tr, 0, 0, 0);
+        v4i bq[2];
 #pragma unroll
-        for (int j = 0; j < R; ++j) {
-          const float pv = P[m + u][j];
-          acc0[j] = __builtin_fmaf(pv, q0, acc0[j]);
-          acc1[j] = __builtin_fmaf(pv, q1, acc1[j]);
-        }
+        for (int q = 0; q < 2; ++q)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) bq[q][e] = (int)pack_bf16x2(tr[8 * q + 2 * e], tr[8 * q + 2 * e + 1]);
+#pragma unroll
+        for (int b = 0; b < RB; ++b)
+#pragma unroll
+          for (int q = 0; q < 2; ++q)
+#pragma unroll
+            for (int t3 = 2; t3 >= 0; --t3) {
+              const v8bf pf = __builtin_bit_cast(
+                  v8bf, *reinterpret_cast<const v8us*>(pop + ((((size_t)bi * RB + b) * 2u + q) * 3u + t3) * kBlockBytes + lane * 16u));
+              acc[st][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf, __builtin_bit_cast(v8bf, bq[q]), acc[st][b], 0, 0, 0);
+            }
       }
-    }
-    for (; m < cnt; ++m) {
-      const uint32_t w = *reinterpret_cast<const uint32_t*>(qcol + (size_t)rowsrc[m] * C);
-      const float q0 = __uint_as_float(w << 16), q1 = __uint_as_float(w & 0xffff0000u);
+      if (bi + 1u < n_blocks) {
 #pragma unroll
-      for (int j = 0; j < R; ++j) {
-        const float pv = P[m][j];
-        acc0[j] = __builtin_fmaf(pv, q0, acc0[j]);
-        acc1[j] = __builtin_fmaf(pv, q1, acc1[j]);
+        for (int st = 0; st < 2; ++st)
+#pragma unroll
+          for (int hc = 0; hc < 2; ++hc) qf[st][hc] = qn[st][hc];
       }
     }
   }
   if (!active) return;
+  // lane (c, h) holds column col0 + 32 st + c, rank rows 32 b + 8 (v / 4) + 4 h + v % 4
 #pragma unroll
-  for (int j = 0; j < R; ++j)
-    *reinterpret_cast<float2*>(part + ((size_t)cid * R + j) * C + col) = make_float2(acc0[j], acc1[j]);
+  for (int st = 0; st < 2; ++st) {
+    const uint32_t col = col0 + 32u * st + c;
+    if (col >= C) continue;
+#pragma unroll
+    for (int b = 0; b < RB; ++b)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const uint32_t j = b * 32u + 8u * (v >> 2) + 4u * h + (v & 3);
+        part[((size_t)cid * (RB * 32u) + j) * C + col] = acc[st][b][v];
+      }
+  }
 }
 
 struct BwdReduceArgs {
@@ -550,21 +724,28 @@ __global__ __launch_bounds__(256) void bwd_dlora_reduce_kernel(BwdReduceArgs a) 
   }
   __syncthreads();
   uint32_t b = blockIdx.x;
-  if (b < a.blocks_a + a.blocks_b) {
-    const bool job_a = b < a.blocks_a;
-    const uint32_t C = job_a ? a.K : a.N;
-    const uint64_t e = (uint64_t)(job_a ? b : b - a.blocks_a) * 256u + tid;  // (group, j, column), column fastest
-    if (e >= (uint64_t)a.n_groups * a.r * C) return;
-    const uint32_t col = (uint32_t)(e % C);
-    const uint32_t j = (uint32_t)((e / C) % a.r), grp = (uint32_t)(e / ((uint64_t)C * a.r));
-    const float* part = job_a ? a.partA : a.partB;
+  if (b < a.blocks_a) {
+    // dA [group][k][j]: a thread per output element, j fastest, so that the stores are contiguous
+    const uint64_t e = (uint64_t)b * 256u + tid;
+    if (e >= (uint64_t)a.n_groups * a.K * a.r || !a.d_a) return;
+    const uint32_t j = (uint32_t)(e % a.r), col = (uint32_t)((e / a.r) % a.K), grp = (uint32_t)(e / ((uint64_t)a.r * a.K));
     float sum = 0.0f;
-    for (uint32_t ch = chunk0[grp]; ch < chunk0[grp + 1]; ++ch) sum += part[((size_t)ch * a.R + j) * C + col];
-    if (job_a) {
-      if (a.d_a) a.d_a[((size_t)grp * a.K + col) * a.r + j] = (uint16_t)f32_to_bf16_bits(sum);
-    } else {
-      if (a.d_b) a.d_b[((size_t)grp * a.r + j) * a.N + col] = (uint16_t)f32_to_bf16_bits(sum * a.lora_scaling[grp]);
+    for (uint32_t ch = chunk0[grp]; ch < chunk0[grp + 1]; ++ch) sum += a.partA[((size_t)ch * a.R + j) * a.K + col];
+    a.d_a[e] = (uint16_t)f32_to_bf16_bits(sum);
+    return;
+  }
+  if (b < a.blocks_a + a.blocks_b) {
+    // dB [group][j][n]: a thread per four adjacent columns (N is a multiple of 8)
+    const uint64_t e = ((uint64_t)(b - a.blocks_a) * 256u + tid) * 4u;
+    if (e >= (uint64_t)a.n_groups * a.r * a.N || !a.d_b) return;
+    const uint32_t col = (uint32_t)(e % a.N), j = (uint32_t)((e / a.N) % a.r), grp = (uint32_t)(e / ((uint64_t)a.N * a.r));
+    float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (uint32_t ch = chunk0[grp]; ch < chunk0[grp + 1]; ++ch) {
+      const float4 v = *reinterpret_cast<const float4*>(a.partB + ((size_t)ch * a.R + j) * a.N + col);
+      sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
     }
+    const float sc = a.lora_scaling[grp];
+    *reinterpret_cast<uint2*>(a.d_b + e) = make_uint2(pack_bf16x2(sum.x * sc, sum.y * sc), pack_bf16x2(sum.z * sc, sum.w * sc));
     return;
   }
   b -= a.blocks_a + a.blocks_b;  // one block per group: ds

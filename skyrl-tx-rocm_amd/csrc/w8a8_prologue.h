@@ -424,6 +424,10 @@ struct LoraAArgs {
   // Optional float32 copies (backward): zf = the raw projection, zsf = the projection times the
   // row's group scale; with group_scale the packed fragments carry the scaled value.  [slot][zf_stride]
   float* zf; float* zsf; const float* group_scale; uint32_t zf_stride;
+  // K split (backward): with n_ksplit > 1 the grid holds n_ksplit workgroups per row block, each
+  // sums its own range of k steps and writes zf + ksplit_index * zf_slice (floats); the caller adds
+  // the slices.  0 or 1: one workgroup per row block.
+  uint32_t n_ksplit, zf_slice;
 };
 
 template <int RB>  // number of 32-wide rank blocks (1 or 2)
@@ -431,7 +435,8 @@ __global__ __launch_bounds__(1024) void lora_a_kernel(LoraAArgs a) {
   __shared__ float red[4][RB][16][64];
   __shared__ float zs[32][RB * 32 + 1];
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-  const uint32_t pb = blockIdx.x;
+  const uint32_t nks = a.n_ksplit > 1u ? a.n_ksplit : 1u;
+  const uint32_t pb = blockIdx.x / nks, ks = blockIdx.x % nks;
   if (pb >= a.n_blocks) return;
   if (a.blk_range && a.blk_range[pb] < 0) return;  // block beyond the rows in use
   const uint32_t range = a.blk_range ? (uint32_t)a.blk_range[pb] : 0u;
@@ -447,8 +452,10 @@ __global__ __launch_bounds__(1024) void lora_a_kernel(LoraAArgs a) {
   for (int b = 0; b < RB; ++b)
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[b][e] = 0.0f;
-  uint32_t s0 = wave * a.steps_per_wave, s1 = s0 + a.steps_per_wave;
-  if (s1 > a.n_steps) s1 = a.n_steps;
+  const uint32_t slice_steps = (a.n_steps + nks - 1u) / nks;
+  const uint32_t slice_end = (ks + 1u) * slice_steps < a.n_steps ? (ks + 1u) * slice_steps : a.n_steps;
+  uint32_t s0 = ks * slice_steps + wave * a.steps_per_wave, s1 = s0 + a.steps_per_wave;
+  if (s1 > slice_end) s1 = slice_end;
   // A block at a group boundary runs once per group with the other groups' rows zeroed.
   for (uint32_t grp = glo; grp <= ghi; ++grp) {
     const bool mine = src >= 0 && rowgrp == grp;
@@ -521,7 +528,7 @@ __global__ __launch_bounds__(1024) void lora_a_kernel(LoraAArgs a) {
     for (uint32_t q = threadIdx.x; q < 32u * RB * 32u; q += 1024u) {
       const uint32_t row = q / (RB * 32u), col = q % (RB * 32u);
       const float raw = zs[row][col];
-      if (a.zf) a.zf[(size_t)(pb * 32u + row) * a.zf_stride + col] = raw;
+      if (a.zf) a.zf[(size_t)ks * a.zf_slice + (size_t)(pb * 32u + row) * a.zf_stride + col] = raw;
       if (a.group_scale) {
         const uint32_t gr = (a.slot_group && ghi > glo) ? (uint32_t)a.slot_group[pb * 32u + row] : glo;
         const float scaled = raw * a.group_scale[gr];
