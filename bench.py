@@ -27,6 +27,7 @@ sys.path.insert(0, str(ROOT))
 sys.path.insert(0, str(ROOT / "tests"))
 
 INT8_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA, published (5.0 POP/s)
+BF16_PEAK_TFLOPS = 2500.0 # MI355X dense bf16 MFMA, published (2.5 PFLOP/s)
 HBM_PEAK_GBS = 8000.0     # MI355X HBM3E, published
 
 WORKLOADS = {
@@ -36,14 +37,20 @@ WORKLOADS = {
     "qwen3-8b-down-m16-decode": dict(m=16, k=12288, n=4096, n_adapters=16, rank=32, residual=True,
                                      idx_mode="arange", seed=3),
     "single-linear-m128": dict(m=128, k=1024, n=3072, n_adapters=1, rank=16, idx_mode="zero", seed=1),
+    # backward (dx pull-back + LoRA cotangents) of the plain linear at the gate/up and down shapes
+    "qwen3-8b-gate_up-m4096-backward": dict(m=4096, k=4096, n=24576, n_adapters=8, rank=32, idx_mode="uniform",
+                                            seed=2, backward=True),
+    "qwen3-8b-down-m4096-backward": dict(m=4096, k=12288, n=4096, n_adapters=8, rank=32, idx_mode="uniform",
+                                         seed=4, backward=True),
 }
 
 # HBM bytes per launch of the dominant kernel(s) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # (summaries under profiles/): (FETCH_SIZE * 2.0 + WRITE_SIZE * 1.0) KiB, the factors being what the
 # same counters read for a 256 MiB device copy with 16-byte loads.  None where not measured.
 MEASURED_TRAFFIC_BYTES = {
-    "qwen3-8b-gate_up-m4096": int((390574 * 2.0 + 129536) * 1024),                 # w8a8_gemm_kernel
-    "qwen3-8b-down-m16-decode": int(((6550 + 27627) * 2.0 + 432 + 128) * 1024),   # both decode kernels
+    "qwen3-8b-gate_up-m4096": int((389417 * 2.0 + 129536) * 1024),                      # w8a8_gemm_kernel
+    "qwen3-8b-down-m16-decode": int(((8614 + 27632) * 2.0 + 4529 + 128) * 1024),       # both decode kernels
+    "qwen3-8b-gate_up-m4096-backward": int((400599 * 2.0 + 44726) * 1024),             # bwd_dx_kernel
 }
 
 
@@ -109,6 +116,85 @@ def cpu_baseline(case, cfg, sample_rows):
                  "seconds": best}
 
 
+def bench_backward(args, cfg, pkg, dev):
+    """One step = one backward call (tables, dy packing + r, z, dx pull-back, dA / dB / dscaling).
+    ``value`` counts the pull-back's 2*M*K*N only; the roofline prices bwd_dx_kernel alone
+    (bf16 MFMA) from HIP events around launches of that kernel."""
+    import torch
+
+    import w8a8_cases as wc
+    from oracle import w8a8_oracle as o
+
+    native, w8 = pkg._native, pkg.w8a8_lora
+    case = wc.make_case(cfg["m"], cfg["k"], cfg["n"], n_adapters=cfg["n_adapters"], rank=cfg["rank"],
+                        seed=cfg["seed"], idx_mode=cfg.get("idx_mode", "uniform"))
+    rng = np.random.default_rng(cfg["seed"] + 1000)
+    dy = o.bf16_round(rng.standard_normal((cfg["m"], cfg["n"])).astype(np.float32))
+    t = wc.to_torch(case, dev)
+    dy_t = torch.from_numpy(dy).to(dev).to(torch.bfloat16)
+    plan = w8.BackwardPlan(t["x"], dy_t, t["weight"], t.get("a"), t.get("b"), t.get("s"),
+                           adapter_indices=t.get("idx"))
+    dx_only = w8.BackwardPlan(None, dy_t, t["weight"], t.get("a"), t.get("b"), t.get("s"),
+                              adapter_indices=t.get("idx"), need_lora_grads=False)
+    torch.cuda.synchronize()
+    for _ in range(args.warmup):
+        plan.run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        plan.run()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    flops = 2.0 * cfg["m"] * cfg["k"] * cfg["n"]
+    dx_only.run()  # fills its workspace; the kernel-only launches below reuse it
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for a, b in ev:
+        a.record()
+        dx_only.run(native.FLAG_SKIP_PROLOGUE)
+        b.record()
+    torch.cuda.synchronize()
+    k_ms = np.asarray([a.elapsed_time(b) for a, b in ev])
+    achieved = flops / (float(k_ms.mean()) * 1e-3) / 1e12
+    got = [None if v is None else v.to(torch.float32).cpu().numpy() for v in plan.run()]
+    torch.cuda.synchronize()
+    m, k, n = cfg["m"], cfg["k"], cfg["n"]
+    result = {
+        "metric": "W8A8-LoRA linear backward (W8A16 pull-back + LoRA cotangents), TFLOP/s of 2*M*K*N per call",
+        "value": flops / (ms_per_step * 1e-3) / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / BF16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "kernel": "bwd_dx_kernel",
+                     "kernel_avg_ms": float(k_ms.mean()), "kernel_min_ms": float(k_ms.min()),
+                     "algorithmic_flops": flops,
+                     # dy once, int8 weight once, dx once (the kernel reads dy re-laid-out by the packing pass)
+                     "algorithmic_bytes": 2 * m * n + k * n + 2 * m * k},
+    }
+    if not args.no_cpu_baseline:
+        rows = args.cpu_rows or 256
+        sel = slice(0, rows)
+        t1 = time.perf_counter()
+        want = o.quantized_lora_linear_multi_bwd(case["x"][sel], case["weight"], case["a"], case["b"], case["s"],
+                                                 case["idx"][sel], dy[sel], relaxed_weight=True)
+        secs = time.perf_counter() - t1
+        try:
+            cores = len(os.sched_getaffinity(0))
+        except AttributeError:
+            cores = os.cpu_count() or 1
+        threads = int(os.environ.get("OMP_NUM_THREADS", cores))
+        result["cpu_baseline"] = {"value": 2.0 * rows * k * n / secs / 1e12, "unit": "TFLOP/s",
+                                  "cores": min(cores, threads), "kind": "port",
+                                  "sample": f"first {rows} of {m} rows, full K and N, NumPy oracle backward "
+                                            f"(float64 BLAS), one run, {secs:.3f} s", "seconds": secs}
+        rep = wc.compare(got[0][sel], want[0])  # dx rows are independent of the other rows
+        result["parity_sample"] = {"rows": rows, "violations": rep["violations"], "size": rep["size"],
+                                   "max_abs": rep["max_abs"], "bitwise_fraction": rep["bitwise_fraction"]}
+    print(json.dumps(result))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -149,6 +235,8 @@ def main() -> int:
     for item in filter(None, args.override.split(",")):
         key, val = item.split("=")
         cfg[key] = int(val)
+    if cfg.pop("backward", False):
+        return bench_backward(args, cfg, pkg, dev)
     case = wc.make_case(cfg["m"], cfg["k"], cfg["n"], n_adapters=cfg.get("n_adapters", 0),
                         rank=cfg.get("rank", 16), seed=cfg["seed"], rms=cfg.get("rms", False),
                         residual=cfg.get("residual", False), swiglu=cfg.get("swiglu", False),

@@ -133,7 +133,7 @@ typedef struct mi355_w8a8_grouped_problem {
  */
 typedef struct mi355_w8a8_bwd_problem {
   uint32_t struct_size;     /* sizeof(mi355_w8a8_bwd_problem) */
-  uint32_t flags;           /* reserved, 0 */
+  uint32_t flags;           /* 0, or MI355_W8A8_FLAG_SKIP_PROLOGUE / _SKIP_GEMM (measurement only) */
   uint32_t m;               /* rows */
   uint32_t k;               /* in features (columns of dx); multiple of 8 */
   uint32_t n;               /* out features (columns of dy); multiple of 8 */

@@ -582,7 +582,9 @@ int run_backward(const mi355_w8a8_bwd_problem* p, hipStream_t s) {
   if (p->struct_size != sizeof(mi355_w8a8_bwd_problem)) return MI355_W8A8_ERR_STRUCT;
   int st = validate_bwd_dims(p->m, p->k, p->n, p->n_adapters, p->rank);
   if (st) return st;
-  if (p->flags) return MI355_W8A8_ERR_SHAPE;
+  if (p->flags & ~(MI355_W8A8_FLAG_SKIP_PROLOGUE | MI355_W8A8_FLAG_SKIP_GEMM)) return MI355_W8A8_ERR_SHAPE;
+  const bool skip_prologue = (p->flags & MI355_W8A8_FLAG_SKIP_PROLOGUE) != 0;  // measurement: the workspace holds a previous call's tables
+  const bool skip_gemm = (p->flags & MI355_W8A8_FLAG_SKIP_GEMM) != 0;
   if (!p->dy || !p->w_packed || !p->w_scales || !p->dx) return MI355_W8A8_ERR_NULL;
   const bool lora = p->n_adapters > 0;
   const bool want_grads = p->d_lora_a || p->d_lora_b || p->d_lora_scaling;
@@ -616,7 +618,7 @@ int run_backward(const mi355_w8a8_bwd_problem* p, hipStream_t s) {
   int32_t* group_off = reinterpret_cast<int32_t*>(ws + w.group_off);
   (void)hipGetLastError();
 
-  {  // tables: routing, A transposed / in operand order, scales in packed column order
+  if (!skip_prologue) {  // tables: routing, A transposed / in operand order, scales in packed column order
     BwdPrepArgs pa{};
     pa.idx = routed ? p->adapter_indices : nullptr;
     pa.src_row = src_row; pa.dst_pos = reinterpret_cast<int32_t*>(ws + w.dst_pos);
@@ -634,7 +636,7 @@ int run_backward(const mi355_w8a8_bwd_problem* p, hipStream_t s) {
     hipLaunchKernelGGL(bwd_prep_kernel, dim3(pa.route_blocks + pa.a_blocks + pa.ap_blocks + sw_blocks), dim3(1024), 0, s, pa);
     if ((st = launch_status())) return st;
   }
-  {  // dy into operand order; the same pass leaves the partial sums of r = dy @ B.T
+  if (!skip_prologue) {  // dy into operand order; the same pass leaves the partial sums of r = dy @ B.T
     BwdPackDyArgs d{};
     d.dy = static_cast<const uint16_t*>(p->dy);
     d.src_row = routed ? src_row : nullptr;
@@ -651,7 +653,7 @@ int run_backward(const mi355_w8a8_bwd_problem* p, hipStream_t s) {
     else hipLaunchKernelGGL((bwd_pack_dy_kernel<1>), grid, block, 0, s, d);
     if ((st = launch_status())) return st;
   }
-  if (lora) {
+  if (lora && !skip_prologue) {
     {
       BwdRFinishArgs f{};
       f.rpart = reinterpret_cast<const float*>(ws + w.rpart);
@@ -696,7 +698,7 @@ int run_backward(const mi355_w8a8_bwd_problem* p, hipStream_t s) {
       if ((st = launch_status())) return st;
     }
   }
-  {
+  if (!skip_gemm) {
     BwdDxArgs g{};
     g.dyp = ws + w.dyp;
     g.wp = static_cast<const unsigned char*>(p->w_packed);

@@ -334,6 +334,90 @@ def forward(x: torch.Tensor, weight, lora_a=None, lora_b=None, lora_scaling=None
 # backward of the plain linear (skyrl/tx/kernels/quantized_lora.py:337-394)
 # ---------------------------------------------------------------------------------------
 
+class BackwardPlan:
+    """Validated arguments, outputs, workspace and the C struct of one backward call; ``run()`` is
+    a single C call on torch's current stream (see ``ForwardPlan``)."""
+
+    def __init__(self, x: torch.Tensor | None, dy: torch.Tensor, weight, lora_a=None, lora_b=None,
+                 lora_scaling=None, *, adapter_indices: torch.Tensor | None = None, need_lora_grads: bool = True):
+        if dy.dtype != torch.bfloat16:
+            raise TypeError(f"dy must be BF16, got {dy.dtype}")
+        if dy.ndim < 2 or math.prod(dy.shape[:-1]) <= 0:
+            raise ValueError(f"dy must have a nonempty row domain and final N axis, got {tuple(dy.shape)}")
+        _require_cuda(dy, "dy")
+        pw = prepare_weight(weight)
+        k, n = pw.in_features, pw.out_features
+        if dy.shape[-1] != n:
+            raise ValueError(f"dy N={dy.shape[-1]} does not match W8 N={n}")
+        dev = dy.device
+        dyf = dy.reshape(-1, n).contiguous()
+        m = dyf.shape[0]
+        a3, b3, s1, n_ad, r = _normalize_lora(lora_a, lora_b, lora_scaling, k, n, dev)
+        want = bool(n_ad) and need_lora_grads
+        xf = None
+        if want:
+            if x is None:
+                raise ValueError("x is needed for the LoRA cotangents")
+            if x.dtype != torch.bfloat16:
+                raise TypeError(f"x must be BF16, got {x.dtype}")
+            _require_cuda(x, "x")
+            if tuple(x.shape) != (*dy.shape[:-1], k):
+                raise ValueError(f"x must have shape {(*dy.shape[:-1], k)}, got {tuple(x.shape)}")
+            xf = x.reshape(m, k).contiguous()
+        idx = None
+        if adapter_indices is not None:
+            if n_ad == 0:
+                raise ValueError("adapter_indices given without LoRA parameters")
+            idx = adapter_indices.reshape(-1)
+            if idx.shape[0] != m:
+                if idx.shape[0] == 0 or m % idx.shape[0]:
+                    raise ValueError(f"adapter_indices of length {idx.shape[0]} do not divide {m} rows")
+                idx = idx.repeat_interleave(m // idx.shape[0])
+            idx = idx.to(device=dev, dtype=torch.int32).contiguous()
+        lib = _native.load()
+        ws_bytes = int(lib.mi355_w8a8_bwd_workspace_bytes(m, k, n, n_ad, r, 0))
+        if ws_bytes == 0:
+            raise ValueError(
+                f"geometry M={m}, K={k}, N={n}, rank={r}, adapters={n_ad} is outside the native backward")
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        self.dx = torch.empty((m, k), dtype=torch.bfloat16, device=dev)
+        self.d_lora_a = torch.empty((n_ad, k, r), dtype=torch.bfloat16, device=dev) if want else None
+        self.d_lora_b = torch.empty((n_ad, r, n), dtype=torch.bfloat16, device=dev) if want else None
+        self.d_lora_scaling = torch.empty((n_ad,), dtype=torch.float32, device=dev) if want else None
+        p = _native.BwdProblem()
+        p.struct_size = ctypes.sizeof(_native.BwdProblem)
+        p.m, p.k, p.n, p.n_adapters, p.rank = m, k, n, n_ad, r
+        p.x = xf.data_ptr() if xf is not None else None
+        p.dy = dyf.data_ptr()
+        p.w_packed = pw.packed.data_ptr()
+        p.w_scales = pw.scales.data_ptr()
+        p.lora_a = a3.data_ptr() if n_ad else None
+        p.lora_b = b3.data_ptr() if n_ad else None
+        p.lora_scaling = s1.data_ptr() if n_ad else None
+        p.adapter_indices = idx.data_ptr() if idx is not None else None
+        p.dx = self.dx.data_ptr()
+        p.d_lora_a = self.d_lora_a.data_ptr() if want else None
+        p.d_lora_b = self.d_lora_b.data_ptr() if want else None
+        p.d_lora_scaling = self.d_lora_scaling.data_ptr() if want else None
+        p.workspace = ws.data_ptr()
+        p.workspace_bytes = ws_bytes
+        self.problem = p
+        self.device = dev
+        self.dx_shape = (*dy.shape[:-1], k)
+        self.dims = {"m": m, "k": k, "n": n, "n_adapters": n_ad, "rank": r}
+        self._fn = lib.mi355_w8a8_lora_linear_bwd_v1
+        self._keep = (xf, dyf, pw, a3, b3, s1, idx, ws)
+
+    def run(self, flags: int = 0):
+        """Enqueue the call; returns ``(dx, d_lora_a, d_lora_b, d_lora_scaling)`` (reused tensors)."""
+        self.problem.flags = flags
+        with torch.cuda.device(self.device):
+            status = self._fn(ctypes.byref(self.problem), _stream_ptr(self.device))
+        self.problem.flags = 0
+        _native.check("mi355_w8a8_lora_linear_bwd_v1", status)
+        return self.dx.reshape(self.dx_shape), self.d_lora_a, self.d_lora_b, self.d_lora_scaling
+
+
 def backward(x: torch.Tensor | None, dy: torch.Tensor, weight, lora_a=None, lora_b=None, lora_scaling=None, *,
              adapter_indices: torch.Tensor | None = None, need_lora_grads: bool = True):
     """Cotangents of ``forward(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=...)``.
@@ -342,69 +426,8 @@ def backward(x: torch.Tensor | None, dy: torch.Tensor, weight, lora_a=None, lora
     LoRA or with ``need_lora_grads=False``.  The activation quantizer is straight-through; the
     frozen weight enters as ``bf16(codes * scales)`` (skyrl/tx/kernels/rocm/w8a8_lora.py:298-339).
     """
-    if dy.dtype != torch.bfloat16:
-        raise TypeError(f"dy must be BF16, got {dy.dtype}")
-    if dy.ndim < 2 or math.prod(dy.shape[:-1]) <= 0:
-        raise ValueError(f"dy must have a nonempty row domain and final N axis, got {tuple(dy.shape)}")
-    _require_cuda(dy, "dy")
-    pw = prepare_weight(weight)
-    k, n = pw.in_features, pw.out_features
-    if dy.shape[-1] != n:
-        raise ValueError(f"dy N={dy.shape[-1]} does not match W8 N={n}")
-    dev = dy.device
-    dyf = dy.reshape(-1, n).contiguous()
-    m = dyf.shape[0]
-    a3, b3, s1, n_ad, r = _normalize_lora(lora_a, lora_b, lora_scaling, k, n, dev)
-    want = bool(n_ad) and need_lora_grads
-    xf = None
-    if want:
-        if x is None:
-            raise ValueError("x is needed for the LoRA cotangents")
-        if x.dtype != torch.bfloat16:
-            raise TypeError(f"x must be BF16, got {x.dtype}")
-        _require_cuda(x, "x")
-        if tuple(x.shape) != (*dy.shape[:-1], k):
-            raise ValueError(f"x must have shape {(*dy.shape[:-1], k)}, got {tuple(x.shape)}")
-        xf = x.reshape(m, k).contiguous()
-    idx = None
-    if adapter_indices is not None:
-        if n_ad == 0:
-            raise ValueError("adapter_indices given without LoRA parameters")
-        idx = adapter_indices.reshape(-1)
-        if idx.shape[0] != m:
-            if idx.shape[0] == 0 or m % idx.shape[0]:
-                raise ValueError(f"adapter_indices of length {idx.shape[0]} do not divide {m} rows")
-            idx = idx.repeat_interleave(m // idx.shape[0])
-        idx = idx.to(device=dev, dtype=torch.int32).contiguous()
-    lib = _native.load()
-    ws_bytes = int(lib.mi355_w8a8_bwd_workspace_bytes(m, k, n, n_ad, r, 0))
-    if ws_bytes == 0:
-        raise ValueError(f"geometry M={m}, K={k}, N={n}, rank={r}, adapters={n_ad} is outside the native backward")
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-    dx = torch.empty((m, k), dtype=torch.bfloat16, device=dev)
-    da = torch.empty((n_ad, k, r), dtype=torch.bfloat16, device=dev) if want else None
-    db = torch.empty((n_ad, r, n), dtype=torch.bfloat16, device=dev) if want else None
-    ds = torch.empty((n_ad,), dtype=torch.float32, device=dev) if want else None
-    p = _native.BwdProblem()
-    p.struct_size = ctypes.sizeof(_native.BwdProblem)
-    p.m, p.k, p.n, p.n_adapters, p.rank = m, k, n, n_ad, r
-    p.x = xf.data_ptr() if xf is not None else None
-    p.dy = dyf.data_ptr()
-    p.w_packed = pw.packed.data_ptr()
-    p.w_scales = pw.scales.data_ptr()
-    p.lora_a = a3.data_ptr() if n_ad else None
-    p.lora_b = b3.data_ptr() if n_ad else None
-    p.lora_scaling = s1.data_ptr() if n_ad else None
-    p.adapter_indices = idx.data_ptr() if idx is not None else None
-    p.dx = dx.data_ptr()
-    p.d_lora_a = da.data_ptr() if want else None
-    p.d_lora_b = db.data_ptr() if want else None
-    p.d_lora_scaling = ds.data_ptr() if want else None
-    p.workspace = ws.data_ptr()
-    p.workspace_bytes = ws_bytes
-    with torch.cuda.device(dev):
-        _native.check("mi355_w8a8_lora_linear_bwd_v1", lib.mi355_w8a8_lora_linear_bwd_v1(ctypes.byref(p), _stream_ptr(dev)))
-    return dx.reshape(*dy.shape[:-1], k), da, db, ds
+    return BackwardPlan(x, dy, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices,
+                        need_lora_grads=need_lora_grads).run()
 
 
 class _LoraLinearFunction(torch.autograd.Function):
@@ -664,7 +687,7 @@ def w8a8_lora_residual(x, weight, lora_a, lora_b, lora_scaling, residual, *, ena
 __all__ = (
     "DEFAULT_BLOCK_M", "DEFAULT_BLOCK_N", "DEFAULT_ROW_SUPERBLOCK", "MAX_BLOCK_M", "MAX_BLOCK_N",
     "MAX_IN_FEATURES", "MAX_OUT_FEATURES", "MAX_ROW_SUPERBLOCK", "MAX_LORA_RANK", "PackedW8Weight",
-    "prepare_weight", "unpack_weight", "dynamic_quantize_rows", "ForwardPlan", "forward", "backward", "lora_linear",
+    "prepare_weight", "unpack_weight", "dynamic_quantize_rows", "ForwardPlan", "forward", "BackwardPlan", "backward", "lora_linear",
     "w8a8_frozen_linear",
     "w8a8_lora_linear", "w8a8_rms_gate_up_lora_swiglu", "w8a8_lora_residual", "PackedGroupedW8Weight",
     "prepare_grouped_weight", "grouped_forward", "w8a8_grouped_lora_linear", "w8a8_moe_expert_mlp",
