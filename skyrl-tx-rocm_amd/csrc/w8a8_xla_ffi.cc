@@ -99,6 +99,62 @@ ffi::Error Forward(hipStream_t stream, ffi::Buffer<ffi::BF16> x, ffi::Buffer<ffi
   return ToError(status, "mi355_w8a8 forward launch submission failed");
 }
 
+// Backward of the plain linear.  x [.., K] bf16, dy [.., N] bf16, packed weight, scales, A, B,
+// scaling and adapter index as in Forward (size-0 buffers when there is no LoRA).  Results:
+// dx bf16 [.., K], dA bf16 [n, K, r], dB bf16 [n, r, N], dscaling f32 [n] (size-0 without LoRA),
+// workspace u8 [mi355_w8a8_bwd_workspace_bytes].
+ffi::Error Backward(hipStream_t stream, ffi::Buffer<ffi::BF16> x, ffi::Buffer<ffi::BF16> dy,
+                    ffi::Buffer<ffi::U8> w_packed, ffi::Buffer<ffi::F32> w_scales,
+                    ffi::Buffer<ffi::BF16> lora_a, ffi::Buffer<ffi::BF16> lora_b,
+                    ffi::Buffer<ffi::F32> lora_scaling, ffi::Buffer<ffi::S32> adapter_indices,
+                    ffi::ResultBuffer<ffi::BF16> dx, ffi::ResultBuffer<ffi::BF16> d_lora_a,
+                    ffi::ResultBuffer<ffi::BF16> d_lora_b, ffi::ResultBuffer<ffi::F32> d_lora_scaling,
+                    ffi::ResultBuffer<ffi::U8> workspace) {
+  mi355_w8a8_bwd_problem p{};
+  p.struct_size = sizeof(p);
+  if (!RowsAndK(x.dimensions(), &p.m, &p.k))
+    return ffi::Error::InvalidArgument("x must be bf16 [..., K] with a non-empty row domain");
+  if (w_scales.dimensions().size() != 1) return ffi::Error::InvalidArgument("w_scales must be f32 [N]");
+  p.n = static_cast<uint32_t>(w_scales.dimensions()[0]);
+  auto ddy = dy.dimensions();
+  if (ddy.size() < 2 || ddy.back() != p.n || dy.element_count() != static_cast<size_t>(p.m) * p.n)
+    return ffi::Error::InvalidArgument("dy must be bf16 [..., N] over the rows of x");
+  if (w_packed.size_bytes() != mi355_w8a8_packed_weight_bytes(p.k, p.n))
+    return ffi::Error::InvalidArgument("packed weight size does not match (K, N)");
+  if (dx->element_count() != x.element_count()) return ffi::Error::InvalidArgument("dx must match x");
+  if (lora_a.element_count() > 0) {
+    auto da = lora_a.dimensions();
+    auto db = lora_b.dimensions();
+    if (da.size() != 3 || db.size() != 3 || da[1] != p.k || db[0] != da[0] || db[1] != da[2] ||
+        db[2] != p.n || lora_scaling.element_count() != static_cast<size_t>(da[0]))
+      return ffi::Error::InvalidArgument("LoRA A/B/scaling must be [n,K,r], [n,r,N], [n]");
+    if (d_lora_a->element_count() != lora_a.element_count() || d_lora_b->element_count() != lora_b.element_count() ||
+        d_lora_scaling->element_count() != lora_scaling.element_count())
+      return ffi::Error::InvalidArgument("the LoRA cotangents must match the LoRA parameters");
+    p.n_adapters = static_cast<uint32_t>(da[0]);
+    p.rank = static_cast<uint32_t>(da[2]);
+    p.lora_a = lora_a.untyped_data();
+    p.lora_b = lora_b.untyped_data();
+    p.lora_scaling = lora_scaling.typed_data();
+    p.d_lora_a = d_lora_a->untyped_data();
+    p.d_lora_b = d_lora_b->untyped_data();
+    p.d_lora_scaling = d_lora_scaling->typed_data();
+    if (adapter_indices.element_count() > 0) {
+      if (adapter_indices.element_count() != p.m)
+        return ffi::Error::InvalidArgument("adapter_indices must hold one entry per row");
+      p.adapter_indices = adapter_indices.typed_data();
+    }
+  }
+  p.x = x.untyped_data();
+  p.dy = dy.untyped_data();
+  p.w_packed = w_packed.untyped_data();
+  p.w_scales = w_scales.typed_data();
+  p.dx = dx->untyped_data();
+  p.workspace = workspace->untyped_data();
+  p.workspace_bytes = workspace->size_bytes();
+  return ToError(mi355_w8a8_lora_linear_bwd_v1(&p, stream), "mi355_w8a8 backward launch submission failed");
+}
+
 ffi::Error QuantizeRows(hipStream_t stream, ffi::Buffer<ffi::BF16> x, ffi::ResultBuffer<ffi::S8> codes,
                         ffi::ResultBuffer<ffi::F32> scales) {
   uint32_t m = 0, k = 0;
@@ -152,5 +208,22 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_pack_weight_v1, PackWeight,
                               ffi::Ffi::Bind()
                                   .Ctx<ffi::PlatformStream<hipStream_t>>()
                                   .Arg<ffi::Buffer<ffi::S8>>()
+                                  .Ret<ffi::Buffer<ffi::U8>>());
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_backward_v1, Backward,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::U8>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::F32>>()
                                   .Ret<ffi::Buffer<ffi::U8>>());
 #endif  // __has_include("xla/ffi/api/ffi.h")

@@ -23,7 +23,8 @@ from pathlib import Path
 from ... import _native
 
 FFI_LIB_PATH = Path(_native.LIB_PATH).with_name("libmi355_w8a8_ffi.so")
-TARGETS = ("mi355_w8a8_ffi_forward_v1", "mi355_w8a8_ffi_quantize_rows_v1", "mi355_w8a8_ffi_pack_weight_v1")
+TARGETS = ("mi355_w8a8_ffi_forward_v1", "mi355_w8a8_ffi_quantize_rows_v1", "mi355_w8a8_ffi_pack_weight_v1",
+           "mi355_w8a8_ffi_backward_v1")
 _ROCM_PLATFORM = "ROCM"
 _REGISTRATION_API_VERSION = 1
 _CUSTOM_CALL_API_VERSION = 4
@@ -134,3 +135,38 @@ def forward(x, packed_weight, w_scales, lora_a=None, lora_b=None, lora_scaling=N
                  x, packed_weight, w_scales.reshape(n).astype(jnp.float32), a3, b3, s1, idx, gamma, res,
                  swiglu=int(swiglu), rms_eps=float(eps), entry=int(entry))
     return y
+
+
+def backward(x, dy, packed_weight, w_scales, lora_a=None, lora_b=None, lora_scaling=None, adapter_indices=None):
+    """Cotangents of the plain linear as one XLA custom call: ``(dx, dA, dB, dscaling)`` (the LoRA
+    entries are ``None`` without LoRA).  This is the body of the ``custom_vjp`` backward rule that
+    replaces ``_quantized_lora_linear_bwd`` (skyrl/tx/kernels/quantized_lora.py:337-394)."""
+    jax = _import_jax()
+    register(jax)
+    jnp = jax.numpy
+    k = x.shape[-1]
+    n = w_scales.shape[-1]
+    m = 1
+    for d in x.shape[:-1]:
+        m *= d
+    empty = lambda dt, nd: jnp.zeros((0,) * nd, dt)
+    a3 = empty(jnp.bfloat16, 3) if lora_a is None else (lora_a if lora_a.ndim == 3 else lora_a[None])
+    b3 = empty(jnp.bfloat16, 3) if lora_b is None else (lora_b if lora_b.ndim == 3 else lora_b[None])
+    n_ad = a3.shape[0]
+    rank = a3.shape[2] if n_ad else 0
+    s1 = empty(jnp.float32, 1) if lora_a is None else jnp.broadcast_to(jnp.asarray(lora_scaling, jnp.float32), (n_ad,))
+    idx = empty(jnp.int32, 1) if adapter_indices is None else adapter_indices.astype(jnp.int32).reshape(-1)
+    ws = int(_native.load().mi355_w8a8_bwd_workspace_bytes(m, k, n, n_ad, rank, 0))
+    if ws == 0:
+        raise ValueError(f"geometry M={m}, K={k}, N={n} is outside the native backward")
+    dx, da, db, ds, _ = _call(
+        jax, TARGETS[3],
+        (jax.ShapeDtypeStruct(x.shape, jnp.bfloat16), jax.ShapeDtypeStruct(a3.shape, jnp.bfloat16),
+         jax.ShapeDtypeStruct(b3.shape, jnp.bfloat16), jax.ShapeDtypeStruct(s1.shape, jnp.float32),
+         jax.ShapeDtypeStruct((ws,), jnp.uint8)),
+        x, dy, packed_weight, w_scales.reshape(n).astype(jnp.float32), a3, b3, s1, idx)
+    if lora_a is None:
+        return dx, None, None, None
+    if lora_a.ndim == 2:
+        return dx, da[0], db[0], ds[0]
+    return dx, da, db, ds
