@@ -582,6 +582,98 @@ def grouped_forward(x: torch.Tensor, group_sizes: torch.Tensor, weight: PackedGr
     return (out, aux) if return_aux else out
 
 
+def grouped_backward(x: torch.Tensor | None, dy: torch.Tensor, group_sizes: torch.Tensor,
+                     weight: PackedGroupedW8Weight, lora_a=None, lora_b=None, lora_scaling=None, *,
+                     groups_per_weight: int = 1, need_lora_grads: bool = True):
+    """Cotangents of ``grouped_forward`` (plain epilogue): ``(dx, d_lora_a, d_lora_b, d_lora_scaling)``.
+
+    One dense backward call per weight (expert) over its rows, the groups that share the weight
+    taking the role of adapters.  The group sizes are read on the host to cut the rows, which waits
+    for the stream once per call; rows beyond ``sum(group_sizes)`` get a zero ``dx``.
+    """
+    if dy.ndim != 2 or dy.dtype != torch.bfloat16:
+        raise TypeError("dy must be a BF16 matrix [rows, N]")
+    _require_cuda(dy, "dy")
+    k, n = weight.in_features, weight.out_features
+    if dy.shape[1] != n:
+        raise ValueError(f"dy N={dy.shape[1]} does not match W8 N={n}")
+    gpw = int(groups_per_weight)
+    sizes = [max(0, int(v)) for v in group_sizes.detach().to("cpu").reshape(-1).tolist()]
+    if len(sizes) != weight.n_weights * gpw:
+        raise ValueError(f"{len(sizes)} groups do not match {weight.n_weights} weights x {gpw}")
+    lora = lora_a is not None
+    want = lora and need_lora_grads
+    dev = dy.device
+    m = dy.shape[0]
+    dx = torch.zeros((m, k), dtype=torch.bfloat16, device=dev)
+    da = torch.zeros_like(lora_a) if want else None
+    db = torch.zeros_like(lora_b) if want else None
+    s_all = None
+    if lora:
+        s_all = torch.as_tensor(lora_scaling, dtype=torch.float32, device=dev)
+        s_all = s_all.reshape(1).expand(len(sizes)).contiguous() if s_all.ndim == 0 else s_all
+    ds = torch.zeros(len(sizes), dtype=torch.float32, device=dev) if want else None
+    each = weight.packed.numel() // weight.n_weights
+    row = 0
+    for wi in range(weight.n_weights):
+        g0 = wi * gpw
+        counts = sizes[g0:g0 + gpw]
+        rows = min(sum(counts), m - row)
+        if rows <= 0:
+            continue
+        pw = PackedW8Weight(packed=weight.packed[wi * each:(wi + 1) * each], scales=weight.scales[wi],
+                            in_features=k, out_features=n)
+        sl = slice(row, row + rows)
+        idx = None
+        if lora and gpw > 1:
+            idx = torch.repeat_interleave(torch.arange(gpw, dtype=torch.int32, device=dev),
+                                          torch.tensor(counts, device=dev))[:rows]
+        out = backward(x[sl] if want else None, dy[sl], pw,
+                       lora_a[g0:g0 + gpw] if lora else None, lora_b[g0:g0 + gpw] if lora else None,
+                       s_all[g0:g0 + gpw] if lora else None, adapter_indices=idx, need_lora_grads=want)
+        dx[sl] = out[0]
+        if want:
+            da[g0:g0 + gpw], db[g0:g0 + gpw], ds[g0:g0 + gpw] = out[1], out[2], out[3]
+        row += rows
+    return dx, da, db, ds
+
+
+class _GroupedLinearFunction(torch.autograd.Function):
+    """``grouped_forward`` (plain epilogue) with the per-expert backward as its derivative."""
+
+    @staticmethod
+    def forward(ctx, x, lora_a, lora_b, lora_scaling, weight, group_sizes, groups_per_weight):
+        out = grouped_forward(x, group_sizes, weight, lora_a, lora_b, lora_scaling,
+                              groups_per_weight=groups_per_weight)
+        ctx.save_for_backward(x, lora_a, lora_b, lora_scaling, group_sizes)
+        ctx.weight = weight
+        ctx.gpw = groups_per_weight
+        return out
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, lora_a, lora_b, lora_scaling, group_sizes = ctx.saved_tensors
+        need = lora_a is not None and any(ctx.needs_input_grad[1:4])
+        dx, da, db, ds = grouped_backward(x, dy.contiguous(), group_sizes, ctx.weight, lora_a, lora_b,
+                                          lora_scaling, groups_per_weight=ctx.gpw, need_lora_grads=need)
+        if need:
+            ds = ds.reshape(lora_scaling.shape).to(lora_scaling.dtype) if lora_scaling.ndim else ds.sum()
+        return dx, da, db, ds, None, None, None
+
+
+def grouped_lora_linear(x, group_sizes, weight, lora_a=None, lora_b=None, lora_scaling=None, *,
+                        groups_per_weight: int = 1):
+    """Ragged W8A8 (+LoRA) linear that autograd can differentiate (plain epilogue only)."""
+    tensors = [t for t in (x, lora_a, lora_b, lora_scaling) if isinstance(t, torch.Tensor)]
+    if not (torch.is_grad_enabled() and any(t.requires_grad for t in tensors)):
+        return grouped_forward(x, group_sizes, weight, lora_a, lora_b, lora_scaling,
+                               groups_per_weight=groups_per_weight)
+    scaling = lora_scaling
+    if lora_a is not None and not isinstance(scaling, torch.Tensor):
+        scaling = torch.as_tensor(scaling, dtype=torch.float32, device=x.device)
+    return _GroupedLinearFunction.apply(x, lora_a, lora_b, scaling, weight, group_sizes, groups_per_weight)
+
+
 def w8a8_grouped_lora_linear(x, group_sizes, weight, lora_a=None, lora_b=None, lora_scaling=None, *,
                              enabled: bool = False, interpret: bool = False, swiglu: bool = False,
                              groups_per_weight: int = 1):
@@ -690,5 +782,6 @@ __all__ = (
     "prepare_weight", "unpack_weight", "dynamic_quantize_rows", "ForwardPlan", "forward", "BackwardPlan", "backward", "lora_linear",
     "w8a8_frozen_linear",
     "w8a8_lora_linear", "w8a8_rms_gate_up_lora_swiglu", "w8a8_lora_residual", "PackedGroupedW8Weight",
-    "prepare_grouped_weight", "grouped_forward", "w8a8_grouped_lora_linear", "w8a8_moe_expert_mlp",
+    "prepare_grouped_weight", "grouped_forward", "grouped_backward", "grouped_lora_linear",
+    "w8a8_grouped_lora_linear", "w8a8_moe_expert_mlp",
 )

@@ -144,7 +144,8 @@ class LoRAExpert(LoRAMixin):
     Rows of ``x`` arrive sorted by expert; ``group_sizes[e]`` rows belong to expert ``e``.  LoRA
     pairs are indexed ``expert * max_lora_adapters + adapter`` (lora.py:414-431): rows are
     stably re-sorted by that combined index, run through the grouped kernel with
-    ``max_lora_adapters`` LoRA groups per expert weight, and put back.
+    ``max_lora_adapters`` LoRA groups per expert weight, and put back.  Differentiable: the backward
+    runs the dense backward kernels once per expert.
     """
 
     def __init__(self, num_experts: int, in_features: int, out_features: int, *,
@@ -171,7 +172,7 @@ class LoRAExpert(LoRAMixin):
             raise NotImplementedError("expert shards (group_offset != 0) belong to the multi-GPU dispatch, "
                                       "which this one-GPU build leaves out")
         if not self._lora_active(adapter_indices_sorted):
-            return w8.grouped_forward(x, group_sizes, self.weight)
+            return w8.grouped_lora_linear(x, group_sizes, self.weight)
         n_ad, n_exp = self.max_lora_adapters, self.num_experts
         gs = group_sizes.to(device=x.device, dtype=torch.int64)
         expert = torch.repeat_interleave(torch.arange(n_exp, device=x.device), gs, output_size=x.shape[0])
@@ -182,11 +183,9 @@ class LoRAExpert(LoRAMixin):
         a = self.lora_A.transpose(0, 1).reshape(n_exp * n_ad, self.in_features, self.max_lora_rank)
         b = self.lora_B.transpose(0, 1).reshape(n_exp * n_ad, self.max_lora_rank, self.out_features)
         scaling = self.lora_scaling.repeat(n_exp)
-        out_sorted = w8.grouped_forward(x[order], sizes, self.weight, a.contiguous(), b.contiguous(), scaling,
-                                        groups_per_weight=n_ad)
-        out = torch.empty_like(out_sorted)
-        out[order] = out_sorted
-        return out
+        out_sorted = w8.grouped_lora_linear(x[order], sizes, self.weight, a.contiguous(), b.contiguous(), scaling,
+                                            groups_per_weight=n_ad)
+        return torch.zeros_like(out_sorted).index_copy(0, order, out_sorted)
 
 
 def init_lora_adapter(layer: LoRAMixin, adapter_index: int, *, rank: int, alpha: float, seed: int = 0) -> None:

@@ -42,6 +42,8 @@ def test_struct_sizes_match_header_layout(native):
     # 8 x 4-byte scalars, 11 pointers, u64, 4 pointers
     assert ctypes.sizeof(native.Problem) == 8 * 4 + 11 * 8 + 8 + 4 * 8
     assert ctypes.sizeof(native.GroupedProblem) == 8 * 4 + 9 * 8 + 8 + 3 * 8
+    # backward: 8 x 4-byte scalars, 13 pointers, u64
+    assert ctypes.sizeof(native.BwdProblem) == 8 * 4 + 13 * 8 + 8
 
 
 def test_size_queries(native):
@@ -96,6 +98,46 @@ def test_validation_errors_without_a_gpu(native):
     assert lib.mi355_w8a8_quantize_rows_v1(0x10000, 0x20000, 0x30000, 4, 60, None) == -7
     assert lib.mi355_w8a8_pack_weight_v1(None, 0x10000, 64, 32, None) == -1
     assert lib.mi355_w8a8_pack_weight_v1(0x10000, 0x10010, 64, 32, None) == -4
+
+
+def test_backward_validation_errors_without_a_gpu(native):
+    lib = native.load()
+
+    def problem(**kw):
+        p = native.BwdProblem()
+        p.struct_size = ctypes.sizeof(native.BwdProblem)
+        p.m, p.k, p.n = 8, 64, 32
+        fake = 0x10000  # never dereferenced: validation fails first
+        p.dy, p.w_packed, p.w_scales, p.dx, p.workspace = fake, fake + 0x100000, fake + 0x200000, fake + 0x300000, fake + 0x400000
+        p.workspace_bytes = 1 << 30
+        for k, v in kw.items():
+            setattr(p, k, v)
+        return p
+
+    call = lambda p: lib.mi355_w8a8_lora_linear_bwd_v1(ctypes.byref(p), None)
+    assert lib.mi355_w8a8_lora_linear_bwd_v1(None, None) == -1
+    assert call(problem(struct_size=8)) == -8
+    assert call(problem(m=0)) == -2
+    assert call(problem(n=36)) == -7                                   # N not a multiple of 8
+    assert call(problem(k=60)) == -7
+    assert call(problem(flags=1)) == -2                                # SwiGLU has no native backward
+    assert call(problem(dy=None)) == -1
+    assert call(problem(dx=None)) == -1
+    assert call(problem(dx=0x10008)) == -3
+    assert call(problem(dx=0x10000)) == -4                             # dx aliases dy
+    assert call(problem(workspace=None)) == -5
+    assert call(problem(workspace_bytes=64)) == -5
+    assert call(problem(n_adapters=2, rank=8)) == -1                   # LoRA pointers missing
+    assert call(problem(d_lora_a=0x700000)) == -2                      # cotangent wanted without LoRA
+    assert call(problem(adapter_indices=0x500000)) == -2
+    lora = dict(n_adapters=2, rank=8, lora_a=0x800000, lora_b=0x900000, lora_scaling=0xa00000)
+    assert call(problem(**lora, d_lora_a=0xb00000)) == -1              # x is needed for a LoRA cotangent
+    assert call(problem(**lora, x=0xc00000, d_lora_a=0x800000)) == -4  # dA aliases A
+    assert lib.mi355_w8a8_bwd_workspace_bytes(4096, 4096, 24576, 8, 32, 0) % 256 == 0
+    assert lib.mi355_w8a8_bwd_workspace_bytes(4096, 4096, 24576, 8, 32, 0) > 2 * 4096 * 24576
+    assert lib.mi355_w8a8_bwd_workspace_bytes(8, 64, 32, 0, 0, 0) > 0
+    assert lib.mi355_w8a8_bwd_workspace_bytes(8, 64, 36, 0, 0, 0) == 0
+    assert lib.mi355_w8a8_bwd_workspace_bytes(8, 64, 32, 65, 8, 0) == 0
 
 
 def test_python_surface_fails_loudly_on_cpu(native):

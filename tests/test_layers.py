@@ -326,3 +326,50 @@ def test_linear_gradients_match_oracle_and_generic_routing(pkg, dev):
     # loss, which ignores them: same values up to the summation order
     for i in (2, 3):
         assert wc.compare(generic[i], fast[i])["violations"] == 0
+
+
+@pytest.mark.gpu
+def test_expert_layer_gradients_match_oracle(pkg, dev):
+    """Gradients of the expert layer: per expert, the oracle's multi-adapter backward over that
+    expert's rows; the scaling gradient adds up over the experts that share an adapter."""
+    import torch
+
+    L = pkg.lora
+    n_exp, n_ad, k, n, r = 3, 2, 64, 48, 4
+    rng = np.random.default_rng(8)
+    layer = L.LoRAExpert(n_exp, k, n, max_lora_adapters=n_ad, max_lora_rank=r, device=dev)
+    dense = o.bf16_round(rng.standard_normal((n_exp, k, n)).astype(F32) * 0.1)
+    ws = [o.quantize_frozen_weight(dense[e], bits=8, group_size=k, scale_dtype="f32") for e in range(n_exp)]
+    layer.load_quantized(torch.from_numpy(np.stack([w.codes for w in ws])),
+                         torch.from_numpy(np.stack([np.asarray(w.scales, F32).reshape(n) for w in ws])))
+    a = o.bf16_round(rng.standard_normal((n_ad, n_exp, k, r)).astype(F32) * 0.1)
+    b = o.bf16_round(rng.standard_normal((n_ad, n_exp, r, n)).astype(F32) * 0.1)
+    s = np.asarray([0.5, 1.5], dtype=F32)
+    layer.lora_A = torch.from_numpy(a).to(dev).to(torch.bfloat16).requires_grad_(True)
+    layer.lora_B = torch.from_numpy(b).to(dev).to(torch.bfloat16).requires_grad_(True)
+    layer.lora_scaling = torch.from_numpy(s).to(dev).requires_grad_(True)
+    group_sizes = np.asarray([17, 0, 30], dtype=np.int32)
+    rows = int(group_sizes.sum())
+    expert = np.repeat(np.arange(n_exp), group_sizes)
+    adapter = rng.integers(0, n_ad, rows).astype(np.int32)
+    x = o.bf16_round(rng.standard_normal((rows, k)).astype(F32))
+    cot = o.bf16_round(rng.standard_normal((rows, n)).astype(F32))
+    xt = torch.from_numpy(x).to(dev).to(torch.bfloat16).requires_grad_(True)
+    out = layer(xt, torch.from_numpy(group_sizes).to(dev), torch.from_numpy(adapter).to(dev))
+    (out.float() * torch.from_numpy(cot).to(dev)).sum().backward()
+    torch.cuda.synchronize()
+    f = lambda t: t.grad.detach().float().cpu().numpy()
+    dx, da, db, ds = f(xt), f(layer.lora_A), f(layer.lora_B), f(layer.lora_scaling)
+    want_ds = np.zeros(n_ad, dtype=np.float64)
+    for e in range(n_exp):
+        sel = np.nonzero(expert == e)[0]
+        if sel.size == 0:
+            assert not da[:, e].any() and not db[:, e].any()
+            continue
+        want = o.quantized_lora_linear_multi_bwd(x[sel], ws[e], a[:, e], b[:, e], s, adapter[sel], cot[sel],
+                                                 relaxed_weight=True)
+        assert wc.compare(dx[sel], want[0])["violations"] == 0
+        assert wc.compare(da[:, e], want[1])["violations"] == 0
+        assert wc.compare(db[:, e], want[2])["violations"] == 0
+        want_ds += want[3]
+    np.testing.assert_allclose(ds, want_ds, rtol=2e-3, atol=1e-3)
