@@ -109,6 +109,29 @@ class FusedLoRALinear(LoRALinear):
     def __call__(self, x: torch.Tensor, adapter_indices: torch.Tensor | None = None) -> tuple[torch.Tensor, ...]:
         return self.split(super().__call__(x, adapter_indices), self.group_sizes)
 
+    def load_components(self, kernels) -> None:
+        """Checkpoint step for a fused projection (skyrl/tx/utils/models.py:159-191,330-339): the
+        component kernels ``[in, out_i]`` are interleaved group by group on the host, then quantized
+        per output channel and packed once."""
+        kernels = list(kernels)
+        if len(kernels) != len(self.components):
+            raise ValueError(f"expected one kernel per component {self.components}, got {len(kernels)}")
+        self.load_dense(self.fuse(*[k.to(torch.float32) for k in kernels], group_sizes=self.group_sizes))
+
+    def load_split_adapter(self, adapter_index: int, lora_a_parts, lora_b_parts) -> None:
+        """Load an adapter trained on the split projections: the branches must share one ``lora_A``
+        (models.py:149-156); their ``lora_B`` are interleaved like the kernels."""
+        a0 = lora_a_parts[0]
+        if not all(torch.allclose(a0.float(), part.float()) for part in lora_a_parts[1:]):
+            raise RuntimeError("Cannot load split LoRA adapter into fused projection because the source "
+                               "branches do not share the same lora_A matrix.")
+        if not 0 <= adapter_index < self.max_lora_adapters:
+            raise ValueError(f"adapter_index {adapter_index} outside [0, {self.max_lora_adapters})")
+        fused_b = self.fuse(*lora_b_parts, group_sizes=self.group_sizes)
+        with torch.no_grad():
+            self.lora_A[adapter_index] = a0.to(device=self.lora_A.device, dtype=torch.bfloat16)
+            self.lora_B[adapter_index] = fused_b.to(device=self.lora_B.device, dtype=torch.bfloat16)
+
     @staticmethod
     def fuse(*arrays: torch.Tensor, group_sizes: tuple[int, ...]) -> torch.Tensor:
         """Interleave per-component arrays group by group (inverse of ``split``)."""

@@ -373,3 +373,34 @@ def test_expert_layer_gradients_match_oracle(pkg, dev):
         assert wc.compare(db[:, e], want[2])["violations"] == 0
         want_ds += want[3]
     np.testing.assert_allclose(ds, want_ds, rtol=2e-3, atol=1e-3)
+
+
+def test_fused_checkpoint_loading(pkg):
+    """Component kernels and split adapters land in the fused layout of the reference's loader
+    (skyrl/tx/utils/models.py:149-191): interleaved by group, quantized per output channel."""
+    import torch
+
+    L = pkg.lora
+    rng = np.random.default_rng(4)
+    k, heads, hd = 16, 2, 4                       # q has 2 heads per kv head
+    q = rng.standard_normal((k, heads * 2 * hd)).astype(F32)
+    kk = rng.standard_normal((k, heads * hd)).astype(F32)
+    v = rng.standard_normal((k, heads * hd)).astype(F32)
+    sizes = (2 * hd, hd, hd)
+    layer = L.FusedLoRALinear(k, q.shape[1] + kk.shape[1] + v.shape[1], components=("q_proj", "k_proj", "v_proj"),
+                              group_sizes=sizes, max_lora_adapters=2, max_lora_rank=4, device="cpu")
+    layer.load_components([torch.from_numpy(t) for t in (q, kk, v)])
+    want = o.quantize_frozen_weight(o.fuse(q, kk, v, group_sizes=sizes), bits=8, group_size=k, scale_dtype="f32")
+    np.testing.assert_array_equal(layer.weight.codes.numpy(), want.codes)
+    np.testing.assert_array_equal(layer.weight.scales.numpy(), want.scales)
+    a = torch.from_numpy(rng.standard_normal((k, 4)).astype(F32))
+    bs = [torch.from_numpy(rng.standard_normal((4, t.shape[1])).astype(F32)) for t in (q, kk, v)]
+    layer.load_split_adapter(1, [a, a.clone(), a.clone()], bs)
+    np.testing.assert_array_equal(layer.lora_B[1].float().numpy(),
+                                  o.bf16_round(o.fuse(*[b.numpy() for b in bs], group_sizes=sizes)))
+    np.testing.assert_array_equal(layer.lora_A[1].float().numpy(), o.bf16_round(a.numpy()))
+    assert not layer.lora_A[0].any()
+    with pytest.raises(RuntimeError, match="share the same lora_A"):
+        layer.load_split_adapter(0, [a, a + 1, a], bs)
+    with pytest.raises(ValueError):
+        layer.load_components([torch.from_numpy(q)])
