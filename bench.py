@@ -42,6 +42,11 @@ WORKLOADS = {
                                             seed=2, backward=True),
     "qwen3-8b-down-m4096-backward": dict(m=4096, k=12288, n=4096, n_adapters=8, rank=32, idx_mode="uniform",
                                          seed=4, backward=True),
+    # Qwen3.5-4B attention input stage: RMSNorm -> W8A8 QKV [2560 -> 10240] + 4 adapters rank 64 ->
+    # split, Q/K RMSNorm, partial RoPE (16 query heads, 4 kv heads, head_dim 256, 64 rotary dims)
+    "qwen3.5-4b-qkv-m2048": dict(m=2048, k=2560, n=10240, n_adapters=4, rank=64, alpha=128, rms=True,
+                                 idx_mode="uniform", seed=5,
+                                 qkv=dict(num_query_heads=16, num_kv_heads=4, head_dim=256, rotary_dim=64)),
 }
 
 # HBM bytes per launch of the dominant kernel(s) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
@@ -195,6 +200,92 @@ def bench_backward(args, cfg, pkg, dev):
     return 0
 
 
+def bench_qkv(args, cfg, pkg, dev):
+    """One step = the W8A8 QKV projection (RMSNorm prologue, GEMM, LoRA) + the split / Q-K norm /
+    RoPE kernel.  ``value`` is int8 TOPS of the projection over the whole step; the roofline prices
+    qkv_post_kernel (HBM-bound: it reads the fused projection once and writes q, k, v, gate once)."""
+    import torch
+
+    import w8a8_cases as wc
+    from oracle import w8a8_oracle as o
+
+    w8 = pkg.w8a8_lora
+    geo = cfg["qkv"]
+    qcfg = w8.Qwen35QKVStageConfig(geo["num_query_heads"], geo["num_kv_heads"], geo["head_dim"], geo["rotary_dim"],
+                                   10_000_000.0, 1e-6)
+    assert qcfg.fused_width == cfg["n"]
+    case = wc.make_case(cfg["m"], cfg["k"], cfg["n"], n_adapters=cfg["n_adapters"], rank=cfg["rank"],
+                        alpha=cfg.get("alpha"), seed=cfg["seed"], rms=True, idx_mode=cfg["idx_mode"])
+    rng = np.random.default_rng(cfg["seed"] + 77)
+    qw, kw = (rng.standard_normal(geo["head_dim"]).astype(np.float32) * 0.1 for _ in range(2))
+    pos = rng.integers(0, 32768, cfg["m"]).astype(np.int32)
+    t = wc.to_torch(case, dev)
+    qw_t, kw_t, pos_t = (torch.from_numpy(v).to(dev) for v in (qw, kw, pos))
+    plan = w8.ForwardPlan(t["x"], t["weight"], t["a"], t["b"], t["s"], adapter_indices=t["idx"],
+                          rms_gamma=t["gamma"], eps=1e-6)
+
+    post = w8.QkvPostPlan(plan.run(), qw_t, kw_t, pos_t, qcfg)  # reads the forward plan's (reused) output
+
+    def step():
+        plan.run()
+        return post.run()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for a, b in ev:
+        a.record()
+        post.run()
+        b.record()
+    torch.cuda.synchronize()
+    k_ms = np.asarray([a.elapsed_time(b) for a, b in ev])
+    m, k, n = cfg["m"], cfg["k"], cfg["n"]
+    bytes_alg = 4 * m * n + 4 * m + 8 * geo["head_dim"]
+    achieved = bytes_alg / (float(k_ms.mean()) * 1e-3) / 1e9
+    ops = 2.0 * m * k * n
+    result = {
+        "metric": "Qwen3.5 attention input stage on the W8A8 QKV projection, int8 TOPS of 2*M*K*N per step",
+        "value": ops / (ms_per_step * 1e-3) / 1e12, "unit": "TOPS", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": "qkv_post_kernel",
+                     "kernel_avg_ms": float(k_ms.mean()), "kernel_min_ms": float(k_ms.min()),
+                     "algorithmic_bytes": bytes_alg},
+    }
+    if not args.no_cpu_baseline:
+        rows = args.cpu_rows or 256
+        t1 = time.perf_counter()
+        want = o.w8a8_qkv_lora_rope(case["x"][:rows], case["gamma"] - 1.0, qw, kw, case["weight"], case["a"], case["b"],
+                                    case["s"], case["idx"][:rows], pos[:rows], num_query_heads=geo["num_query_heads"],
+                                    num_kv_heads=geo["num_kv_heads"], head_dim=geo["head_dim"],
+                                    rotary_dim=geo["rotary_dim"], rope_theta=10_000_000.0, eps=1e-6)
+        secs = time.perf_counter() - t1
+        try:
+            cores = len(os.sched_getaffinity(0))
+        except AttributeError:
+            cores = os.cpu_count() or 1
+        threads = int(os.environ.get("OMP_NUM_THREADS", cores))
+        result["cpu_baseline"] = {"value": 2.0 * rows * k * n / secs / 1e12, "unit": "TOPS", "cores": min(cores, threads),
+                                  "kind": "port", "sample": f"first {rows} of {m} rows, NumPy oracle of the whole stage, "
+                                                            f"one run, {secs:.3f} s", "seconds": secs}
+        viol = size = 0
+        for u, w_ in zip(out, want):
+            rep = wc.compare(u[:rows].to(torch.float32).cpu().numpy().reshape(w_.shape), w_)
+            viol += rep["violations"]
+            size += rep["size"]
+        result["parity_sample"] = {"rows": rows, "violations": viol, "size": size}
+    print(json.dumps(result))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -237,6 +328,8 @@ def main() -> int:
         cfg[key] = int(val)
     if cfg.pop("backward", False):
         return bench_backward(args, cfg, pkg, dev)
+    if "qkv" in cfg:
+        return bench_qkv(args, cfg, pkg, dev)
     case = wc.make_case(cfg["m"], cfg["k"], cfg["n"], n_adapters=cfg.get("n_adapters", 0),
                         rank=cfg.get("rank", 16), seed=cfg["seed"], rms=cfg.get("rms", False),
                         residual=cfg.get("residual", False), swiglu=cfg.get("swiglu", False),

@@ -156,6 +156,32 @@ typedef struct mi355_w8a8_bwd_problem {
   uint64_t workspace_bytes;
 } mi355_w8a8_bwd_problem;
 
+/*
+ * Qwen3.5 attention input stage behind the fused QKV projection: split of the interleaved
+ * projection (per kv head: queries_per_kv (q, gate) chunk pairs, then k, then v), RMSNorm with
+ * (1 + weight) over every Q and K head, partial RoPE on Q and K.
+ */
+typedef struct mi355_w8a8_qkv_post_problem {
+  uint32_t struct_size;     /* sizeof(mi355_w8a8_qkv_post_problem) */
+  uint32_t flags;           /* 0 */
+  uint32_t m;               /* rows (batch * sequence) */
+  uint32_t num_query_heads;
+  uint32_t num_kv_heads;    /* divides num_query_heads */
+  uint32_t head_dim;        /* even, <= 512 */
+  uint32_t rotary_dim;      /* even, <= head_dim; 0 = no RoPE */
+  float rope_theta;
+  float rms_eps;
+  uint32_t reserved;
+  const void* fused;        /* bf16 [m, num_query_heads * 2 * head_dim + 2 * num_kv_heads * head_dim] */
+  const float* q_norm_weight; /* f32 [head_dim], delta form: the multiplier is 1 + weight */
+  const float* k_norm_weight; /* f32 [head_dim] */
+  const int32_t* positions; /* int32 [m] */
+  void* q;                  /* bf16 [m, num_query_heads, head_dim] */
+  void* k;                  /* bf16 [m, num_kv_heads, head_dim] */
+  void* v;                  /* bf16 [m, num_kv_heads, head_dim] */
+  void* gate;               /* bf16 [m, num_query_heads * head_dim] */
+} mi355_w8a8_qkv_post_problem;
+
 int mi355_w8a8_abi_version(void);
 const char* mi355_w8a8_status_string(int status);
 
@@ -198,6 +224,14 @@ int mi355_w8a8_grouped_v1(const mi355_w8a8_grouped_problem* problem, void* strea
 uint64_t mi355_w8a8_bwd_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t n_adapters,
                                         uint32_t rank, uint32_t flags);
 int mi355_w8a8_lora_linear_bwd_v1(const mi355_w8a8_bwd_problem* problem, void* stream);
+
+/*
+ * The part of qwen35_qkv_lora_rope behind the projection (skyrl/tx/kernels/qwen3_5_qkv_lora.py:
+ * 266-286: _split_interleaved_qkv, the Q/gate split, _delta_rms_norm on Q and K,
+ * _apply_partial_rope).  The projection with its input RMSNorm is mi355_w8a8_forward_v1 with
+ * rms_gamma = 1 + input_norm_weight.
+ */
+int mi355_w8a8_qkv_split_norm_rope_v1(const mi355_w8a8_qkv_post_problem* problem, void* stream);
 
 #ifdef __cplusplus
 }

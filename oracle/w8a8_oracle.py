@@ -29,6 +29,11 @@ How each function is pinned (the tests that do it live in ``tests/test_oracle_*.
   function ``x @ dequant(W) + s * (x @ A) @ B``, central finite differences of the LoRA
   terms, and the zero/linearity identities of the equations.  PARITY UNPINNED in the float32
   summation order of XLA (float64 accumulation here).
+* ``delta_rms_norm``/``apply_partial_rope``/``qkv_split_norm_rope``: ``torch.nn.functional.rms_norm``,
+  the rotation written as a complex product, its group law R(p)R(q) = R(p + q), norm
+  preservation, position 0 and ``rotary_dim`` 0 identities, and an enumerated interleaving
+  (tests/tx/kernels/test_qwen3_5_qkv_lora.py:75-83 states it as ``FusedLoRALinear.split``).
+  sin/cos/pow of XLA-CPU are not available: PARITY UNPINNED in their last float32 bits.
 * ``moe_route``/``moe_expert_mlp``: ``torch.topk``/``scipy.special.softmax`` special
   cases and the merged-weight invariant of tests/tx/models/test_qwen3.py:123-180.
 """
@@ -45,6 +50,75 @@ F32 = np.float32
 
 # ---------------------------------------------------------------------------
 # bf16 helpers
+# ---------------------------------------------------------------------------
+# Qwen3.5 attention input stage after the fused projection
+# (skyrl/tx/kernels/qwen3_5_qkv_lora.py:88-95, 119-145, 216-286)
+# ---------------------------------------------------------------------------
+
+def delta_rms_norm(x, weight, eps: float) -> np.ndarray:
+    """qwen3_5_qkv_lora.py:88-95: float32 statistics, multiplier ``1 + weight``, cast to bf16.
+    mean and rsqrt are fixed as in ``rms_norm`` (PARITY UNPINNED in the last float32 bit)."""
+    return rms_norm(x, (F32(1.0) + np.asarray(weight, dtype=F32)).astype(F32), eps)
+
+
+def rope_sin_cos(positions, rotary_dim: int, rope_theta: float):
+    """qwen3_5_qkv_lora.py:119-127: angle[p, i] = p / theta ** (2 i / rotary_dim), float32."""
+    fraction = (F32(2.0) * np.arange(0, rotary_dim // 2, dtype=F32) / F32(rotary_dim)).astype(F32)
+    timescale = np.power(F32(rope_theta), fraction).astype(F32)
+    angles = (np.asarray(positions).astype(F32)[..., None] / timescale).astype(F32)
+    return np.sin(angles).astype(F32), np.cos(angles).astype(F32)
+
+
+def apply_partial_rope(x, positions, rotary_dim: int, rope_theta: float) -> np.ndarray:
+    """qwen3_5_qkv_lora.py:130-145.  ``x`` is [..., heads, head_dim] (bf16 values), ``positions``
+    [...]: the first ``rotary_dim`` entries of a head are rotated in halves (i, i + rotary_dim / 2),
+    the products are float32, the result is cast to bf16 once; the rest passes through."""
+    x = np.asarray(x, dtype=F32)
+    if rotary_dim == 0:
+        return x.copy()
+    half = rotary_dim // 2
+    first, second = x[..., :half], x[..., half:rotary_dim]
+    sin, cos = rope_sin_cos(positions, rotary_dim, rope_theta)
+    sin, cos = sin[..., None, :], cos[..., None, :]
+    out = x.copy()
+    out[..., :half] = bf16_round((first * cos).astype(F32) - (second * sin).astype(F32))
+    out[..., half:rotary_dim] = bf16_round((first * sin).astype(F32) + (second * cos).astype(F32))
+    return out
+
+
+def qkv_split_norm_rope(fused, q_norm_weight, k_norm_weight, positions, *, num_query_heads: int,
+                        num_kv_heads: int, head_dim: int, rotary_dim: int, rope_theta: float, eps: float):
+    """qwen3_5_qkv_lora.py:266-286 on an interleaved fused projection [rows, width] (bf16 values):
+    per kv head one group of ``queries_per_kv`` (q, gate) chunk pairs, then k, then v.  Returns
+    q [rows, Hq, D], k [rows, Hkv, D], v [rows, Hkv, D], gate [rows, Hq * D]."""
+    fused = np.asarray(fused, dtype=F32)
+    rows = fused.shape[0]
+    qpk = num_query_heads // num_kv_heads
+    q_raw, k_raw, v_raw = split(fused, (qpk * 2 * head_dim, head_dim, head_dim))
+    q_and_gate = q_raw.reshape(rows, num_query_heads, 2 * head_dim)
+    q_raw, gate = q_and_gate[..., :head_dim], q_and_gate[..., head_dim:]
+    k_raw = k_raw.reshape(rows, num_kv_heads, head_dim)
+    v = v_raw.reshape(rows, num_kv_heads, head_dim)
+    q = delta_rms_norm(q_raw.reshape(-1, head_dim), q_norm_weight, eps).reshape(q_raw.shape)
+    k = delta_rms_norm(k_raw.reshape(-1, head_dim), k_norm_weight, eps).reshape(k_raw.shape)
+    q = apply_partial_rope(q, positions, rotary_dim, rope_theta)
+    k = apply_partial_rope(k, positions, rotary_dim, rope_theta)
+    return q, k, v.copy(), gate.reshape(rows, num_query_heads * head_dim).copy()
+
+
+def w8a8_qkv_lora_rope(hidden, input_norm_weight, q_norm_weight, k_norm_weight, weight: GroupQuantizedWeight,
+                       lora_a, lora_b, lora_scaling, adapter_indices, positions, **config):
+    """The stage with the W8A8 projection in the place of the bf16 one: delta RMSNorm -> W8A8 +
+    LoRA (one cast) -> split, Q/K norms, partial RoPE.  ``hidden`` is [rows, K]."""
+    eps = config["eps"]
+    normalized = delta_rms_norm(hidden, input_norm_weight, eps)
+    if lora_a is None:
+        fused = quantized_frozen_linear(normalized, weight)
+    else:
+        fused = quantized_lora_linear_multi(normalized, weight, lora_a, lora_b, lora_scaling, adapter_indices)
+    return qkv_split_norm_rope(fused, q_norm_weight, k_norm_weight, positions, **config)
+
+
 # ---------------------------------------------------------------------------
 
 def bf16_bits(a) -> np.ndarray:

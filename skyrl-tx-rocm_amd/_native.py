@@ -34,6 +34,7 @@ EXPORTS = (
     "mi355_w8a8_lora_linear_v1", "mi355_w8a8_rms_gateup_swiglu_v1", "mi355_w8a8_lora_residual_v1",
     "mi355_w8a8_forward_v1", "mi355_w8a8_grouped_v1",
     "mi355_w8a8_bwd_workspace_bytes", "mi355_w8a8_lora_linear_bwd_v1",
+    "mi355_w8a8_qkv_split_norm_rope_v1",
 )
 
 _u32, _u64, _vp, _f32 = ctypes.c_uint32, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_float
@@ -76,6 +77,17 @@ class BwdProblem(ctypes.Structure):
     ]
 
 
+class QkvPostProblem(ctypes.Structure):
+    """struct mi355_w8a8_qkv_post_problem"""
+
+    _fields_ = [
+        ("struct_size", _u32), ("flags", _u32), ("m", _u32), ("num_query_heads", _u32), ("num_kv_heads", _u32),
+        ("head_dim", _u32), ("rotary_dim", _u32), ("rope_theta", _f32), ("rms_eps", _f32), ("reserved", _u32),
+        ("fused", _vp), ("q_norm_weight", _vp), ("k_norm_weight", _vp), ("positions", _vp),
+        ("q", _vp), ("k", _vp), ("v", _vp), ("gate", _vp),
+    ]
+
+
 class NativeError(RuntimeError):
     def __init__(self, fn: str, status: int, detail: str):
         super().__init__(f"{fn} failed: {STATUS.get(status, status)} ({detail})")
@@ -113,6 +125,8 @@ def _bind(lib: ctypes.CDLL) -> None:
     lib.mi355_w8a8_grouped_v1.argtypes = (ctypes.POINTER(GroupedProblem), _vp)
     lib.mi355_w8a8_lora_linear_bwd_v1.restype = ctypes.c_int
     lib.mi355_w8a8_lora_linear_bwd_v1.argtypes = (ctypes.POINTER(BwdProblem), _vp)
+    lib.mi355_w8a8_qkv_split_norm_rope_v1.restype = ctypes.c_int
+    lib.mi355_w8a8_qkv_split_norm_rope_v1.argtypes = (ctypes.POINTER(QkvPostProblem), _vp)
 
 
 def load() -> ctypes.CDLL:

@@ -10,6 +10,7 @@
 #include "w8a8_prologue.h"
 #include "w8a8_skinny.h"
 #include "w8a8_backward.h"
+#include "w8a8_qkv_post.h"
 
 using namespace w8a8;
 
@@ -763,6 +764,43 @@ int run_backward(const mi355_w8a8_bwd_problem* p, hipStream_t s) {
   return MI355_W8A8_OK;
 }
 
+int run_qkv_post(const mi355_w8a8_qkv_post_problem* p, hipStream_t s) {
+  if (!p) return MI355_W8A8_ERR_NULL;
+  if (p->struct_size != sizeof(mi355_w8a8_qkv_post_problem)) return MI355_W8A8_ERR_STRUCT;
+  if (p->flags) return MI355_W8A8_ERR_SHAPE;
+  if (p->m == 0 || p->num_query_heads == 0 || p->num_kv_heads == 0 || p->head_dim == 0) return MI355_W8A8_ERR_SHAPE;
+  if (p->num_query_heads % p->num_kv_heads) return MI355_W8A8_ERR_SHAPE;
+  if ((p->head_dim & 1u) || (p->rotary_dim & 1u) || p->rotary_dim > p->head_dim) return MI355_W8A8_ERR_SHAPE;
+  if (!(p->rope_theta > 0.0f) || !(p->rms_eps > 0.0f)) return MI355_W8A8_ERR_SHAPE;
+  if (p->head_dim > kQkvMaxHeadDim || p->m > kMaxRows || p->num_query_heads > 1024u) return MI355_W8A8_ERR_UNSUPPORTED;
+  const uint64_t width = ((uint64_t)p->num_query_heads * 2u + 2u * p->num_kv_heads) * p->head_dim;
+  if (width * p->m >= (1ull << 32)) return MI355_W8A8_ERR_UNSUPPORTED;
+  if (!p->fused || !p->q_norm_weight || !p->k_norm_weight || !p->positions || !p->q || !p->k || !p->v || !p->gate)
+    return MI355_W8A8_ERR_NULL;
+  if (!aligned16(p->fused) || !aligned16(p->q) || !aligned16(p->k) || !aligned16(p->v) || !aligned16(p->gate) ||
+      !aligned16(p->q_norm_weight) || !aligned16(p->k_norm_weight) || (reinterpret_cast<uintptr_t>(p->positions) & 3u))
+    return MI355_W8A8_ERR_ALIGN;
+  const uint64_t fused_bytes = width * p->m * 2u;
+  const uint64_t q_bytes = (uint64_t)p->m * p->num_query_heads * p->head_dim * 2u;
+  const uint64_t kv_bytes = (uint64_t)p->m * p->num_kv_heads * p->head_dim * 2u;
+  if (overlaps(p->fused, fused_bytes, p->q, q_bytes) || overlaps(p->fused, fused_bytes, p->gate, q_bytes) ||
+      overlaps(p->fused, fused_bytes, p->k, kv_bytes) || overlaps(p->fused, fused_bytes, p->v, kv_bytes) ||
+      overlaps(p->q, q_bytes, p->gate, q_bytes) || overlaps(p->k, kv_bytes, p->v, kv_bytes) ||
+      overlaps(p->q, q_bytes, p->k, kv_bytes) || overlaps(p->q, q_bytes, p->v, kv_bytes) ||
+      overlaps(p->gate, q_bytes, p->k, kv_bytes) || overlaps(p->gate, q_bytes, p->v, kv_bytes))
+    return MI355_W8A8_ERR_ALIAS;
+  QkvPostArgs a{};
+  a.fused = static_cast<const uint16_t*>(p->fused);
+  a.q_w = p->q_norm_weight; a.k_w = p->k_norm_weight; a.pos = p->positions;
+  a.q = static_cast<uint16_t*>(p->q); a.k = static_cast<uint16_t*>(p->k);
+  a.v = static_cast<uint16_t*>(p->v); a.gate = static_cast<uint16_t*>(p->gate);
+  a.M = p->m; a.Hq = p->num_query_heads; a.Hkv = p->num_kv_heads; a.D = p->head_dim; a.rot = p->rotary_dim;
+  a.width = (uint32_t)width; a.theta = p->rope_theta; a.eps = p->rms_eps;
+  (void)hipGetLastError();
+  hipLaunchKernelGGL(qkv_post_kernel, dim3(p->m), dim3(256), 0, s, a);
+  return launch_status();
+}
+
 }  // namespace
 
 extern "C" {
@@ -880,6 +918,10 @@ uint64_t mi355_w8a8_bwd_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint
 
 int mi355_w8a8_lora_linear_bwd_v1(const mi355_w8a8_bwd_problem* p, void* stream) {
   return run_backward(p, static_cast<hipStream_t>(stream));
+}
+
+int mi355_w8a8_qkv_split_norm_rope_v1(const mi355_w8a8_qkv_post_problem* p, void* stream) {
+  return run_qkv_post(p, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

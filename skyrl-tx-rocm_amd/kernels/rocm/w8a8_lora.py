@@ -776,6 +776,123 @@ def w8a8_lora_residual(x, weight, lora_a, lora_b, lora_scaling, residual, *, ena
                    residual=residual, entry="residual")
 
 
+# ---------------------------------------------------------------------------------------
+# Qwen3.5 attention input stage (skyrl/tx/kernels/qwen3_5_qkv_lora.py)
+# ---------------------------------------------------------------------------------------
+@dataclass(frozen=True)
+class Qwen35QKVStageConfig:
+    """Static geometry of the stage (qwen3_5_qkv_lora.py:36-85, same fields and checks)."""
+
+    num_query_heads: int
+    num_kv_heads: int
+    head_dim: int
+    rotary_dim: int
+    rope_theta: float
+    rms_norm_eps: float
+
+    def __post_init__(self) -> None:
+        if self.num_query_heads <= 0 or self.num_kv_heads <= 0:
+            raise ValueError("num_query_heads and num_kv_heads must be positive")
+        if self.num_query_heads % self.num_kv_heads != 0:
+            raise ValueError("num_query_heads must be divisible by num_kv_heads")
+        if self.head_dim <= 0:
+            raise ValueError("head_dim must be positive")
+        if self.rotary_dim < 0 or self.rotary_dim > self.head_dim or self.rotary_dim % 2:
+            raise ValueError("rotary_dim must be even and lie in [0, head_dim]")
+        if self.rope_theta <= 0:
+            raise ValueError("rope_theta must be positive")
+        if self.rms_norm_eps <= 0:
+            raise ValueError("rms_norm_eps must be positive")
+
+    @property
+    def queries_per_kv(self) -> int:
+        return self.num_query_heads // self.num_kv_heads
+
+    @property
+    def q_projection_width(self) -> int:
+        return self.num_query_heads * 2 * self.head_dim
+
+    @property
+    def kv_projection_width(self) -> int:
+        return self.num_kv_heads * self.head_dim
+
+    @property
+    def fused_width(self) -> int:
+        return self.q_projection_width + 2 * self.kv_projection_width
+
+
+class QkvPostPlan:
+    """Outputs and the C struct of one split / Q-K norm / partial-RoPE call; ``run()`` is a single
+    C call on torch's current stream (see ``ForwardPlan``)."""
+
+    def __init__(self, fused: torch.Tensor, q_norm_weight: torch.Tensor, k_norm_weight: torch.Tensor,
+                 positions: torch.Tensor, config: Qwen35QKVStageConfig):
+        if fused.dtype != torch.bfloat16:
+            raise TypeError(f"fused must be BF16, got {fused.dtype}")
+        _require_cuda(fused, "fused")
+        if fused.shape[-1] != config.fused_width:
+            raise ValueError(f"fused width {fused.shape[-1]} does not match the configuration ({config.fused_width})")
+        lead = tuple(fused.shape[:-1])
+        if tuple(positions.shape) != lead:
+            raise ValueError(f"positions must have shape {lead}, got {tuple(positions.shape)}")
+        d = config.head_dim
+        if tuple(q_norm_weight.shape) != (d,) or tuple(k_norm_weight.shape) != (d,):
+            raise ValueError(f"q_norm_weight and k_norm_weight must have shape ({d},)")
+        dev = fused.device
+        flat = fused.reshape(-1, config.fused_width).contiguous()
+        m = flat.shape[0]
+        qw = q_norm_weight.to(device=dev, dtype=torch.float32).contiguous()
+        kw = k_norm_weight.to(device=dev, dtype=torch.float32).contiguous()
+        pos = positions.reshape(-1).to(device=dev, dtype=torch.int32).contiguous()
+        self.q = torch.empty((m, config.num_query_heads, d), dtype=torch.bfloat16, device=dev)
+        self.k = torch.empty((m, config.num_kv_heads, d), dtype=torch.bfloat16, device=dev)
+        self.v = torch.empty((m, config.num_kv_heads, d), dtype=torch.bfloat16, device=dev)
+        self.gate = torch.empty((m, config.num_query_heads * d), dtype=torch.bfloat16, device=dev)
+        p = _native.QkvPostProblem()
+        p.struct_size = ctypes.sizeof(_native.QkvPostProblem)
+        p.m, p.num_query_heads, p.num_kv_heads = m, config.num_query_heads, config.num_kv_heads
+        p.head_dim, p.rotary_dim = d, config.rotary_dim
+        p.rope_theta, p.rms_eps = float(config.rope_theta), float(config.rms_norm_eps)
+        p.fused, p.q_norm_weight, p.k_norm_weight = flat.data_ptr(), qw.data_ptr(), kw.data_ptr()
+        p.positions = pos.data_ptr()
+        p.q, p.k, p.v, p.gate = self.q.data_ptr(), self.k.data_ptr(), self.v.data_ptr(), self.gate.data_ptr()
+        self.problem = p
+        self.device = dev
+        self.lead = lead
+        self.config = config
+        self._fn = _native.load().mi355_w8a8_qkv_split_norm_rope_v1
+        self._keep = (flat, qw, kw, pos)
+
+    def run(self):
+        with torch.cuda.device(self.device):
+            status = self._fn(ctypes.byref(self.problem), _stream_ptr(self.device))
+        _native.check("mi355_w8a8_qkv_split_norm_rope_v1", status)
+        c, lead = self.config, self.lead
+        return (self.q.reshape(*lead, c.num_query_heads, c.head_dim), self.k.reshape(*lead, c.num_kv_heads, c.head_dim),
+                self.v.reshape(*lead, c.num_kv_heads, c.head_dim), self.gate.reshape(*lead, c.num_query_heads * c.head_dim))
+
+
+def qkv_split_norm_rope(fused: torch.Tensor, q_norm_weight: torch.Tensor, k_norm_weight: torch.Tensor,
+                        positions: torch.Tensor, config: Qwen35QKVStageConfig):
+    """Split of the interleaved projection, Q/K RMSNorm with ``1 + weight``, partial RoPE
+    (qwen3_5_qkv_lora.py:266-286).  ``fused`` is bf16 [..., fused_width], ``positions`` int [...].
+    Returns q [..., Hq, D], k [..., Hkv, D], v [..., Hkv, D], gate [..., Hq * D]."""
+    return QkvPostPlan(fused, q_norm_weight, k_norm_weight, positions, config).run()
+
+
+def w8a8_qkv_lora_rope(hidden, input_norm_weight, q_norm_weight, k_norm_weight, weight, lora_a, lora_b, lora_scaling,
+                       positions, *, config: Qwen35QKVStageConfig, adapter_indices=None, enabled: bool = False,
+                       interpret: bool = False):
+    """``qwen35_qkv_lora_rope`` (qwen3_5_qkv_lora.py:532-…) with the W8A8 projection in the place of
+    the bf16 one: decoder RMSNorm (delta weights) fused into the quantizer, W8A8 QKV + LoRA in one
+    float32 epilogue, then the split / Q-K norm / partial-RoPE kernel.  Forward only."""
+    _check_enabled(enabled, interpret, "QKV input stage")
+    gamma = 1.0 + input_norm_weight.to(torch.float32)
+    fused = forward(hidden, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices,
+                    rms_gamma=gamma, eps=config.rms_norm_eps)
+    return qkv_split_norm_rope(fused, q_norm_weight, k_norm_weight, positions, config)
+
+
 __all__ = (
     "DEFAULT_BLOCK_M", "DEFAULT_BLOCK_N", "DEFAULT_ROW_SUPERBLOCK", "MAX_BLOCK_M", "MAX_BLOCK_N",
     "MAX_IN_FEATURES", "MAX_OUT_FEATURES", "MAX_ROW_SUPERBLOCK", "MAX_LORA_RANK", "PackedW8Weight",
@@ -783,5 +900,6 @@ __all__ = (
     "w8a8_frozen_linear",
     "w8a8_lora_linear", "w8a8_rms_gate_up_lora_swiglu", "w8a8_lora_residual", "PackedGroupedW8Weight",
     "prepare_grouped_weight", "grouped_forward", "grouped_backward", "grouped_lora_linear",
-    "w8a8_grouped_lora_linear", "w8a8_moe_expert_mlp",
+    "w8a8_grouped_lora_linear", "w8a8_moe_expert_mlp", "Qwen35QKVStageConfig", "QkvPostPlan", "qkv_split_norm_rope",
+    "w8a8_qkv_lora_rope",
 )
