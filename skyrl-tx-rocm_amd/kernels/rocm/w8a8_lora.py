@@ -433,14 +433,17 @@ def backward(x: torch.Tensor | None, dy: torch.Tensor, weight, lora_a=None, lora
 class _LoraLinearFunction(torch.autograd.Function):
     """``forward`` with the custom derivative of the reference (``_quantized_lora_linear.defvjp``,
     skyrl/tx/kernels/quantized_lora.py:397): cotangents for x, A, B and the scaling; the frozen
-    codes and scales get none."""
+    codes and scales get none.  With a residual (added in the float32 epilogue) its cotangent is the
+    output cotangent, as in ``_bf16_lora_residual_bwd``."""
 
     @staticmethod
-    def forward(ctx, x, lora_a, lora_b, lora_scaling, weight, adapter_indices):
-        out = forward(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices, entry="linear")
+    def forward(ctx, x, lora_a, lora_b, lora_scaling, weight, adapter_indices, residual):
+        out = forward(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices,
+                      residual=residual, entry="linear" if residual is None else "residual")
         ctx.save_for_backward(x, lora_a, lora_b, lora_scaling)
         ctx.weight = weight
         ctx.adapter_indices = adapter_indices
+        ctx.has_residual = residual is not None
         return out
 
     @staticmethod
@@ -453,20 +456,21 @@ class _LoraLinearFunction(torch.autograd.Function):
             if lora_a.ndim == 2:
                 da, db = da[0], db[0]
             ds = ds.reshape(lora_scaling.shape).to(lora_scaling.dtype)
-        return dx, da, db, ds, None, None
+        return dx, da, db, ds, None, None, (dy if ctx.has_residual else None)
 
 
 def lora_linear(x: torch.Tensor, weight, lora_a=None, lora_b=None, lora_scaling=None, *,
-                adapter_indices: torch.Tensor | None = None) -> torch.Tensor:
-    """Plain W8A8 (+LoRA) linear that autograd can differentiate: the forward kernels, and the
-    backward kernels when x or a LoRA parameter requires a gradient."""
-    tensors = [t for t in (x, lora_a, lora_b, lora_scaling) if isinstance(t, torch.Tensor)]
+                adapter_indices: torch.Tensor | None = None, residual: torch.Tensor | None = None) -> torch.Tensor:
+    """Plain W8A8 (+LoRA, + residual) linear that autograd can differentiate: the forward kernels,
+    and the backward kernels when x, a LoRA parameter or the residual requires a gradient."""
+    tensors = [t for t in (x, lora_a, lora_b, lora_scaling, residual) if isinstance(t, torch.Tensor)]
     if not (torch.is_grad_enabled() and any(t.requires_grad for t in tensors)):
-        return forward(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices, entry="linear")
+        return forward(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices,
+                       residual=residual, entry="linear" if residual is None else "residual")
     scaling = lora_scaling
     if lora_a is not None and not isinstance(scaling, torch.Tensor):
         scaling = torch.as_tensor(scaling, dtype=torch.float32, device=x.device)
-    return _LoraLinearFunction.apply(x, lora_a, lora_b, scaling, weight, adapter_indices)
+    return _LoraLinearFunction.apply(x, lora_a, lora_b, scaling, weight, adapter_indices, residual)
 
 
 # ---------------------------------------------------------------------------------------
@@ -772,8 +776,9 @@ def w8a8_lora_residual(x, weight, lora_a, lora_b, lora_scaling, residual, *, ena
                        interpret: bool = False, adapter_indices=None):
     """W8A8 down projection + LoRA + residual, summed in float32 and cast once."""
     _check_enabled(enabled, interpret, "LoRA residual")
-    return forward(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices,
-                   residual=residual, entry="residual")
+    if residual is None:
+        raise ValueError("w8a8_lora_residual needs a residual")
+    return lora_linear(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices, residual=residual)
 
 
 # ---------------------------------------------------------------------------------------

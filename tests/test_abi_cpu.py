@@ -184,3 +184,44 @@ def test_host_quantizer_matches_oracle():
         np.testing.assert_array_equal(got.scales.numpy(), want.scales)
         np.testing.assert_array_equal(pkg.quantized_lora.dequantize_frozen_weight(got).numpy(),
                                       o.dequantize_frozen_weight(want))
+
+
+def test_same_named_fused_entry_points_validate_like_the_reference(native):
+    """bf16_rms_gate_up_lora_swiglu_contiguous / bf16_lora_residual keep the reference's surface:
+    default off, exact bools, tile keywords checked, a bf16 matrix in the place of the quantized
+    kernel refused."""
+    import torch
+
+    pkg = load_package()
+    gate_up = pkg.bf16_rms_gate_up_lora_swiglu_contiguous.bf16_rms_gate_up_lora_swiglu_contiguous
+    down = pkg.bf16_lora_residual.bf16_lora_residual
+    ql = pkg.quantized_lora
+    x = torch.zeros(2, 64, dtype=torch.bfloat16)
+    w = ql.quantize_frozen_weight(torch.randn(64, 16), bits=8, group_size=64, scale_dtype=torch.float32)
+    a, b, s = torch.zeros(64, 4, dtype=torch.bfloat16), torch.zeros(4, 16, dtype=torch.bfloat16), 1.0
+    delta = torch.zeros(64)
+    with pytest.raises(RuntimeError, match="disabled by default"):
+        gate_up(x, delta, w, a, b, s)
+    with pytest.raises(TypeError, match="exact bool"):
+        gate_up(x, delta, w, a, b, s, enabled=1)
+    with pytest.raises(RuntimeError, match="interpret"):
+        gate_up(x, delta, w, a, b, s, enabled=True, interpret=True)
+    with pytest.raises(ValueError, match="block_k"):
+        gate_up(x, delta, w, a, b, s, enabled=True, block_k=0)
+    with pytest.raises(ValueError, match="eps"):
+        gate_up(x, delta, w, a, b, s, enabled=True, eps=0.0)
+    with pytest.raises(TypeError, match="GroupQuantizedWeight"):
+        gate_up(x, delta, torch.zeros(64, 16, dtype=torch.bfloat16), a, b, s, enabled=True)
+    with pytest.raises(RuntimeError, match="GPU"):
+        gate_up(x, delta, w, a, b, s, enabled=True)                  # CPU tensors: no CPU path
+    res = torch.zeros(2, 16, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="disabled by default"):
+        down(x, w, a, b, s, res)
+    with pytest.raises(TypeError, match="exact bool"):
+        down(x, w, a, b, s, res, enabled=True, pallas_input_vjp="no")
+    with pytest.raises(ValueError, match="row_superblock"):
+        down(x, w, a, b, s, res, enabled=True, row_superblock=-1)
+    with pytest.raises(TypeError, match="GroupQuantizedWeight"):
+        down(x, torch.zeros(64, 16, dtype=torch.bfloat16), a, b, s, res, enabled=True)
+    with pytest.raises(RuntimeError, match="GPU"):
+        down(x, w, a, b, s, res, enabled=True)

@@ -466,3 +466,37 @@ def test_largest_k(dev, m):
     got, aux = wc.gpu_forward(case)
     _assert_integer_stages(aux, st)
     _assert_close(got, st["out"], f" K=16384 m={m}")
+
+
+def test_same_named_fused_entry_points(dev, pkg):
+    """``bf16_rms_gate_up_lora_swiglu_contiguous`` (delta RMSNorm weights) and ``bf16_lora_residual``
+    in the reference's argument order on a quantized kernel; the residual form is differentiable with
+    respect to x, A, B and the residual like the reference's custom VJP."""
+    import torch
+
+    gate_up = pkg.bf16_rms_gate_up_lora_swiglu_contiguous.bf16_rms_gate_up_lora_swiglu_contiguous
+    down = pkg.bf16_lora_residual.bf16_lora_residual
+    case = wc.make_case(48, 128, 96, n_adapters=1, rank=8, seed=31, rms=True, swiglu=True, idx_mode="zero")
+    t = wc.to_torch(case, dev)
+    delta = t["gamma"] - 1.0                                   # the reference stores the delta
+    out = gate_up(t["x"], delta, t["weight"], t["a"][0], t["b"][0], 1.0, enabled=True, eps=1e-6)
+    torch.cuda.synchronize()
+    case_delta = dict(case, gamma=(F32(1.0) + (case["gamma"] - F32(1.0)).astype(F32)).astype(F32))
+    assert wc.compare(out.float().cpu().numpy(), wc.oracle_forward(case_delta))["violations"] == 0
+
+    case = wc.make_case(40, 128, 64, n_adapters=1, rank=8, seed=32, residual=True, idx_mode="zero")
+    t = wc.to_torch(case, dev)
+    x = t["x"].clone().requires_grad_(True)
+    a = t["a"][0].clone().requires_grad_(True)
+    b = t["b"][0].clone().requires_grad_(True)
+    res = t["residual"].clone().requires_grad_(True)
+    out = down(x, t["weight"], a, b, 1.0, res, enabled=True)
+    assert wc.compare(out.detach().float().cpu().numpy(), wc.oracle_forward(case))["violations"] == 0
+    cot = o.bf16_round(np.random.default_rng(5).standard_normal((40, 64)).astype(F32))
+    (out.float() * torch.from_numpy(cot).to(dev)).sum().backward()
+    torch.cuda.synchronize()
+    want = o.quantized_lora_linear_bwd(case["x"], case["weight"], case["a"][0], case["b"][0], F32(1.0), cot,
+                                       relaxed_weight=True)
+    for got, ref in ((x.grad, want[0]), (a.grad, want[1]), (b.grad, want[2])):
+        assert wc.compare(got.float().cpu().numpy(), ref)["violations"] == 0
+    np.testing.assert_array_equal(res.grad.float().cpu().numpy(), cot)     # the residual's cotangent is dy
