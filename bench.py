@@ -42,6 +42,10 @@ WORKLOADS = {
                                             seed=2, backward=True),
     "qwen3-8b-down-m4096-backward": dict(m=4096, k=12288, n=4096, n_adapters=8, rank=32, idx_mode="uniform",
                                          seed=4, backward=True),
+    # backward of the fused RMSNorm -> gate/up -> SwiGLU call: forward recomputation, SwiGLU pull-back,
+    # linear backward, RMSNorm pull-back
+    "qwen3-8b-gate_up-m4096-fused-backward": dict(m=4096, k=4096, n=24576, n_adapters=8, rank=32, rms=True,
+                                                  swiglu=True, idx_mode="uniform", seed=2, backward=True),
     # Qwen3.5-4B attention input stage: RMSNorm -> W8A8 QKV [2560 -> 10240] + 4 adapters rank 64 ->
     # split, Q/K RMSNorm, partial RoPE (16 query heads, 4 kv heads, head_dim 256, 64 rotary dims)
     "qwen3.5-4b-qkv-m2048": dict(m=2048, k=2560, n=10240, n_adapters=4, rank=64, alpha=128, rms=True,
@@ -200,6 +204,114 @@ def bench_backward(args, cfg, pkg, dev):
     return 0
 
 
+def bench_fused_backward(args, cfg, pkg, dev):
+    """One step = one backward of the fused RMSNorm -> gate/up -> SwiGLU call: the forward
+    recomputation (projection + normalized rows), the SwiGLU pull-back, the linear backward and the
+    RMSNorm pull-back.  ``value`` counts the pull-back's 2*M*K*N only; the roofline prices
+    bwd_dx_kernel (bf16 MFMA) as in the plain backward, and ``stages`` gives the two memory-bound
+    pull-back kernels against HBM."""
+    import torch
+
+    import w8a8_cases as wc
+    from oracle import w8a8_oracle as o
+
+    native, w8 = pkg._native, pkg.w8a8_lora
+    m, k, n = cfg["m"], cfg["k"], cfg["n"]
+    case = wc.make_case(m, k, n, n_adapters=cfg["n_adapters"], rank=cfg["rank"], seed=cfg["seed"],
+                        idx_mode=cfg.get("idx_mode", "uniform"), rms=True)
+    rng = np.random.default_rng(cfg["seed"] + 2000)
+    c = o.bf16_round(rng.standard_normal((m, n // 2)).astype(np.float32))
+    t = wc.to_torch(case, dev)
+    c_t = torch.from_numpy(c).to(dev).to(torch.bfloat16)
+    plan = w8.FusedBackwardPlan(t["x"], t["gamma"], t["weight"], t["a"], t["b"], t["s"], c_t,
+                                adapter_indices=t["idx"])
+    torch.cuda.synchronize()
+    for _ in range(args.warmup):
+        plan.run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        plan.run()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    got = [v.to(torch.float32).cpu().numpy() for v in plan.run()]
+    torch.cuda.synchronize()
+    flops = 2.0 * m * k * n
+
+    def timed(fn):
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        for a, b in ev:
+            a.record()
+            fn()
+            b.record()
+        torch.cuda.synchronize()
+        return np.asarray([a.elapsed_time(b) for a, b in ev])
+
+    # the stages on their own, on the buffers of a complete run; the two in-place stages write to
+    # scratch outputs here so that every repetition sees the same operands
+    lib = native.load()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    fwd_ms = timed(plan.fwd.run)
+    scratch_n = torch.empty_like(plan.fwd.out)
+    swiglu_ms = timed(lambda: native.check("swiglu_bwd", lib.mi355_w8a8_swiglu_bwd_v1(
+        plan.fwd.out.data_ptr(), plan.d_product.data_ptr(), scratch_n.data_ptr(), m, n, stream)))
+    plan.run_swiglu_stage()
+    linear_ms = timed(plan.bwd.run)
+    scratch_k = torch.empty_like(plan.bwd.dx)
+    rms_ms = timed(lambda: native.check("rms_norm_bwd", lib.mi355_w8a8_rms_norm_bwd_v1(
+        plan.x.data_ptr(), plan.gamma.data_ptr(), plan.bwd.dx.data_ptr(), scratch_k.data_ptr(), m, k, plan.eps,
+        stream)))
+    dx_only = w8.BackwardPlan(None, plan.fwd.out, t["weight"], t["a"], t["b"], t["s"], adapter_indices=t["idx"],
+                              need_lora_grads=False)
+    dx_only.run()
+    k_ms = timed(lambda: dx_only.run(native.FLAG_SKIP_PROLOGUE))
+    achieved = flops / (float(k_ms.mean()) * 1e-3) / 1e12
+    swiglu_bytes = 5 * m * n          # projection in and out (bf16 [M, N]) + cotangent in (bf16 [M, N/2])
+    rms_bytes = 6 * m * k + 4 * k     # x, d_normalized in, d_x out (bf16 [M, K]) + gamma
+    result = {
+        "metric": "fused RMSNorm/gate-up/SwiGLU backward (recompute + pull-backs + LoRA cotangents), "
+                  "TFLOP/s of 2*M*K*N per call",
+        "value": flops / (ms_per_step * 1e-3) / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / BF16_PEAK_TFLOPS, "traffic": None, "kernel": "bwd_dx_kernel",
+                     "kernel_avg_ms": float(k_ms.mean()), "kernel_min_ms": float(k_ms.min()),
+                     "algorithmic_flops": flops, "algorithmic_bytes": 2 * m * n + k * n + 2 * m * k},
+        "stages": {
+            "forward_recompute_ms": float(fwd_ms.mean()), "linear_backward_ms": float(linear_ms.mean()),
+            "swiglu_bwd_kernel": {"avg_ms": float(swiglu_ms.mean()), "algorithmic_bytes": swiglu_bytes,
+                                  "achieved_gbs": swiglu_bytes / (float(swiglu_ms.mean()) * 1e-3) / 1e9,
+                                  "frac_of_hbm": swiglu_bytes / (float(swiglu_ms.mean()) * 1e-3) / 1e9 / HBM_PEAK_GBS},
+            "rms_norm_bwd_kernel": {"avg_ms": float(rms_ms.mean()), "algorithmic_bytes": rms_bytes,
+                                    "achieved_gbs": rms_bytes / (float(rms_ms.mean()) * 1e-3) / 1e9,
+                                    "frac_of_hbm": rms_bytes / (float(rms_ms.mean()) * 1e-3) / 1e9 / HBM_PEAK_GBS},
+        },
+    }
+    if not args.no_cpu_baseline:
+        rows = args.cpu_rows or 256
+        sel = slice(0, rows)
+        t1 = time.perf_counter()
+        want = o.w8a8_rms_gate_up_lora_swiglu_bwd(case["x"][sel], case["gamma"], case["weight"], case["a"], case["b"],
+                                                  case["s"], case["idx"][sel], c[sel])
+        secs = time.perf_counter() - t1
+        try:
+            cores = len(os.sched_getaffinity(0))
+        except AttributeError:
+            cores = os.cpu_count() or 1
+        threads = int(os.environ.get("OMP_NUM_THREADS", cores))
+        result["cpu_baseline"] = {"value": 2.0 * rows * k * n / secs / 1e12, "unit": "TFLOP/s",
+                                  "cores": min(cores, threads), "kind": "port",
+                                  "sample": f"first {rows} of {m} rows, full K and N, NumPy oracle of the fused "
+                                            f"backward (forward stages + pull-backs, float64 BLAS), one run, "
+                                            f"{secs:.3f} s", "seconds": secs}
+        gate = o.numerical_gate(got[0][sel], want[0])  # dx rows are independent of the other rows
+        result["parity_sample"] = {"rows": rows, "relative_l2": gate["relative_l2"], "cosine": gate["cosine"]}
+    print(json.dumps(result))
+    return 0
+
+
 def bench_qkv(args, cfg, pkg, dev):
     """One step = the W8A8 QKV projection (RMSNorm prologue, GEMM, LoRA) + the split / Q-K norm /
     RoPE kernel.  ``value`` is int8 TOPS of the projection over the whole step; the roofline prices
@@ -327,6 +439,8 @@ def main() -> int:
         key, val = item.split("=")
         cfg[key] = int(val)
     if cfg.pop("backward", False):
+        if cfg.get("swiglu"):
+            return bench_fused_backward(args, cfg, pkg, dev)
         return bench_backward(args, cfg, pkg, dev)
     if "qkv" in cfg:
         return bench_qkv(args, cfg, pkg, dev)

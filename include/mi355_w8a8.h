@@ -233,6 +233,29 @@ int mi355_w8a8_lora_linear_bwd_v1(const mi355_w8a8_bwd_problem* problem, void* s
  */
 int mi355_w8a8_qkv_split_norm_rope_v1(const mi355_w8a8_qkv_post_problem* problem, void* stream);
 
+/*
+ * The two stages around the projection in the pull-back of the fused RMSNorm -> gate/up + LoRA ->
+ * SwiGLU call (skyrl/tx/kernels/rocm/bf16_rms_gate_up_lora_swiglu_contiguous.py:643-689).  With
+ * fused = the bf16 projection (mi355_w8a8_forward_v1 with rms_gamma, without FLAG_SWIGLU, which
+ * also returns the normalized activations in aux_normalized), the whole rule is
+ *   d_fused = swiglu_bwd(fused, d_product)
+ *   d_normalized, d_lora_a, d_lora_b, d_lora_scaling = mi355_w8a8_lora_linear_bwd_v1(normalized, d_fused)
+ *   d_x = rms_norm_bwd(x, gamma, d_normalized)
+ *
+ * mi355_w8a8_swiglu_bwd_v1 replaces _fp32_swiglu_pullback_interleaved (:541-553): fused bf16 [m, n]
+ * with columns (gate_0, up_0, gate_1, up_1, ...), d_product bf16 [m, n / 2], d_fused bf16 [m, n];
+ * n % 8 == 0; d_fused may be the fused buffer itself.
+ *
+ * mi355_w8a8_rms_norm_bwd_v1 replaces _rms_norm_pullback (:556-574): x, d_normalized, d_x bf16
+ * [m, k]; gamma f32 [k] is the multiplier itself (1 + rms_delta); the row statistics are recomputed
+ * from x with the forward's rule; d_x may be the d_normalized buffer itself.  gamma gets no
+ * cotangent, as in the reference.
+ */
+int mi355_w8a8_swiglu_bwd_v1(const void* fused, const void* d_product, void* d_fused, uint32_t m, uint32_t n,
+                             void* stream);
+int mi355_w8a8_rms_norm_bwd_v1(const void* x, const float* gamma, const void* d_normalized, void* d_x, uint32_t m,
+                               uint32_t k, float eps, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

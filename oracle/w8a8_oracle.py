@@ -29,6 +29,12 @@ How each function is pinned (the tests that do it live in ``tests/test_oracle_*.
   function ``x @ dequant(W) + s * (x @ A) @ B``, central finite differences of the LoRA
   terms, and the zero/linearity identities of the equations.  PARITY UNPINNED in the float32
   summation order of XLA (float64 accumulation here).
+* ``swiglu_pullback_interleaved``/``rms_norm_pullback``/``w8a8_rms_gate_up_lora_swiglu_bwd``:
+  ``torch.autograd`` (float64, CPU) through ``silu(g) * u`` and through the smooth RMSNorm, the
+  closed forms at g = 0 (d_gate = c u / 2, d_up = 0) and for a constant row (dx = 0 when dn * gamma
+  is parallel to x), and the orthogonality sum(x * dx) ~ eps-term; the composite against autograd
+  through the whole smooth function on bf16-exact inputs.  exp, the float32 reduction order and
+  rsqrt of XLA are not available: PARITY UNPINNED in their last float32 bits.
 * ``delta_rms_norm``/``apply_partial_rope``/``qkv_split_norm_rope``: ``torch.nn.functional.rms_norm``,
   the rotation written as a complex product, its group law R(p)R(q) = R(p + q), norm
   preservation, position 0 and ``rotary_dim`` 0 identities, and an enumerated interleaving
@@ -612,6 +618,77 @@ def w8a8_rms_gate_up_lora_swiglu(x, gamma, weight: GroupQuantizedWeight, lora_a,
     if return_stages:
         return product, {"normalized": n, "fused_f32": fused_f32, "fused": fused}
     return product
+
+
+# ---------------------------------------------------------------------------
+# backward of RMSNorm -> gate/up -> SwiGLU
+# (rocm/bf16_rms_gate_up_lora_swiglu_contiguous.py:541-574, 643-689)
+# ---------------------------------------------------------------------------
+
+def swiglu_pullback_interleaved(fused_bf16, d_product) -> np.ndarray:
+    """bf16 cotangent of the interleaved projection; float32 operations in the order of
+    bf16_rms_gate_up_lora_swiglu_contiguous.py:541-553:
+    d_up = c * (g * sig), d_gate = (c * u) * sig + (g * (c * u)) * (sig * (1 - sig)).
+    """
+    fused = np.asarray(fused_bf16, dtype=F32)
+    gate = fused[..., 0::2]
+    up = fused[..., 1::2]
+    c = np.asarray(d_product, dtype=F32).reshape(gate.shape)
+    with np.errstate(over="ignore"):
+        sig = (F32(1.0) / (F32(1.0) + np.exp(-gate).astype(F32))).astype(F32)
+    d_up = (c * (gate * sig).astype(F32)).astype(F32)
+    wc = (c * up).astype(F32)
+    sprime = (sig * (F32(1.0) - sig).astype(F32)).astype(F32)
+    d_gate = ((wc * sig).astype(F32) + ((gate * wc).astype(F32) * sprime).astype(F32)).astype(F32)
+    out = np.empty(fused.shape, dtype=F32)
+    out[..., 0::2] = d_gate
+    out[..., 1::2] = d_up
+    return bf16_round(out)
+
+
+def rms_norm_pullback(x, gamma, d_normalized, eps: float = 1e-6) -> np.ndarray:
+    """bf16 cotangent of x through ``rms_norm``; bf16_rms_gate_up_lora_swiglu_contiguous.py:556-574.
+
+    p = dn * gamma; den = mean(x^2) + eps and inv = 1 / sqrt(den) as in ``rms_norm``;
+    t = (sum_k x p) * (-0.5 * (inv / den)) / K; dx = bf16((p * inv + x * t) + t * x).
+    The row sum is taken in float64 and rounded once (the reference's float32 reduction order is
+    XLA's: PARITY UNPINNED in its last bits).
+    """
+    x = np.asarray(x, dtype=F32)
+    gamma = np.asarray(gamma, dtype=F32)
+    dn = np.asarray(d_normalized, dtype=F32)
+    k = x.shape[-1]
+    ssq = np.sum(x.astype(np.float64) * x.astype(np.float64), axis=-1, keepdims=True)
+    den = ((ssq / np.float64(k)).astype(F32) + F32(eps)).astype(F32)
+    inv = (F32(1.0) / np.sqrt(den)).astype(F32)
+    p = (dn * gamma).astype(F32)
+    ic = np.sum(x.astype(np.float64) * p.astype(np.float64), axis=-1, keepdims=True).astype(F32)
+    dc = (ic * (F32(-0.5) * (inv / den).astype(F32)).astype(F32)).astype(F32)
+    t = (dc / F32(k)).astype(F32)
+    xt = (x * t).astype(F32)
+    return bf16_round((((p * inv).astype(F32) + xt).astype(F32) + xt).astype(F32))
+
+
+def w8a8_rms_gate_up_lora_swiglu_bwd(x, gamma, weight: GroupQuantizedWeight, lora_a, lora_b, lora_scaling,
+                                     adapter_indices, d_product, eps: float = 1e-6,
+                                     relaxed_weight: bool = True, return_stages: bool = False):
+    """Cotangents (dx, dA, dB, dscaling) of ``w8a8_rms_gate_up_lora_swiglu``.
+
+    The structure of bf16_rms_gate_up_lora_swiglu_contiguous.py:643-689 (SwiGLU pull-back on the
+    saved bf16 projection, the projection's pull-back on the bf16 normalized rows, the RMSNorm
+    pull-back) with the quantized projection's own rule in the middle
+    (``quantized_lora_linear_multi_bwd``: straight-through quantizer, LoRA terms in float32, one
+    cast per cotangent).
+    """
+    product, stages = w8a8_rms_gate_up_lora_swiglu(x, gamma, weight, lora_a, lora_b, lora_scaling,
+                                                   adapter_indices, eps, return_stages=True)
+    d_fused = swiglu_pullback_interleaved(stages["fused"], d_product)
+    dn, da, db, ds = quantized_lora_linear_multi_bwd(stages["normalized"], weight, lora_a, lora_b, lora_scaling,
+                                                     adapter_indices, d_fused, relaxed_weight)
+    dx = rms_norm_pullback(x, gamma, dn, eps)
+    if return_stages:
+        return (dx, da, db, ds), {"d_fused": d_fused, "d_normalized": dn, **stages}
+    return dx, da, db, ds
 
 
 # ---------------------------------------------------------------------------

@@ -35,6 +35,7 @@ EXPORTS = (
     "mi355_w8a8_forward_v1", "mi355_w8a8_grouped_v1",
     "mi355_w8a8_bwd_workspace_bytes", "mi355_w8a8_lora_linear_bwd_v1",
     "mi355_w8a8_qkv_split_norm_rope_v1",
+    "mi355_w8a8_swiglu_bwd_v1", "mi355_w8a8_rms_norm_bwd_v1",
 )
 
 _u32, _u64, _vp, _f32 = ctypes.c_uint32, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_float
@@ -127,6 +128,10 @@ def _bind(lib: ctypes.CDLL) -> None:
     lib.mi355_w8a8_lora_linear_bwd_v1.argtypes = (ctypes.POINTER(BwdProblem), _vp)
     lib.mi355_w8a8_qkv_split_norm_rope_v1.restype = ctypes.c_int
     lib.mi355_w8a8_qkv_split_norm_rope_v1.argtypes = (ctypes.POINTER(QkvPostProblem), _vp)
+    lib.mi355_w8a8_swiglu_bwd_v1.restype = ctypes.c_int
+    lib.mi355_w8a8_swiglu_bwd_v1.argtypes = (_vp, _vp, _vp, _u32, _u32, _vp)
+    lib.mi355_w8a8_rms_norm_bwd_v1.restype = ctypes.c_int
+    lib.mi355_w8a8_rms_norm_bwd_v1.argtypes = (_vp, _vp, _vp, _vp, _u32, _u32, _f32, _vp)
 
 
 def load() -> ctypes.CDLL:

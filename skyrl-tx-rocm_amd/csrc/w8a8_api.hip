@@ -11,6 +11,7 @@
 #include "w8a8_skinny.h"
 #include "w8a8_backward.h"
 #include "w8a8_qkv_post.h"
+#include "w8a8_fused_bwd.h"
 
 using namespace w8a8;
 
@@ -801,6 +802,51 @@ int run_qkv_post(const mi355_w8a8_qkv_post_problem* p, hipStream_t s) {
   return launch_status();
 }
 
+int run_swiglu_bwd(const void* fused, const void* d_product, void* d_fused, uint32_t m, uint32_t n, hipStream_t s) {
+  if (!fused || !d_product || !d_fused) return MI355_W8A8_ERR_NULL;
+  if (m == 0 || n == 0 || (n & 7u)) return MI355_W8A8_ERR_SHAPE;
+  if (m > kMaxRows) return MI355_W8A8_ERR_UNSUPPORTED;
+  if (!aligned16(fused) || !aligned16(d_fused) || (reinterpret_cast<uintptr_t>(d_product) & 7u))
+    return MI355_W8A8_ERR_ALIGN;
+  const uint64_t fused_bytes = (uint64_t)m * n * 2u;
+  // d_fused may be fused itself (element i is read and written by the same thread), nothing else
+  if (d_fused != fused && overlaps(d_fused, fused_bytes, fused, fused_bytes)) return MI355_W8A8_ERR_ALIAS;
+  if (overlaps(d_fused, fused_bytes, d_product, fused_bytes / 2u)) return MI355_W8A8_ERR_ALIAS;
+  SwigluBwdArgs a{};
+  a.fused = static_cast<const uint16_t*>(fused);
+  a.dprod = static_cast<const uint16_t*>(d_product);
+  a.dfused = static_cast<uint16_t*>(d_fused);
+  a.n_chunks = (uint64_t)m * n / 8u;
+  const uint64_t blocks = (a.n_chunks + 255u) / 256u;
+  (void)hipGetLastError();
+  hipLaunchKernelGGL(swiglu_bwd_kernel, dim3((uint32_t)(blocks < 16384u ? blocks : 16384u)), dim3(256), 0, s, a);
+  return launch_status();
+}
+
+int run_rms_norm_bwd(const void* x, const float* gamma, const void* d_normalized, void* d_x, uint32_t m, uint32_t k,
+                     float eps, hipStream_t s) {
+  if (!x || !gamma || !d_normalized || !d_x) return MI355_W8A8_ERR_NULL;
+  if (m == 0 || k == 0 || !(eps > 0.0f)) return MI355_W8A8_ERR_SHAPE;
+  if (m > kMaxRows) return MI355_W8A8_ERR_UNSUPPORTED;
+  if (!aligned16(x) || !aligned16(d_normalized) || !aligned16(d_x) || !aligned16(gamma)) return MI355_W8A8_ERR_ALIGN;
+  const uint64_t bytes = (uint64_t)m * k * 2u;
+  // d_x may be d_normalized itself (a row is reduced before any of it is rewritten, element i by
+  // the thread that reads it), nothing else
+  if (d_x != d_normalized && overlaps(d_x, bytes, d_normalized, bytes)) return MI355_W8A8_ERR_ALIAS;
+  if (overlaps(d_x, bytes, x, bytes) || overlaps(d_x, bytes, gamma, (uint64_t)k * 4u)) return MI355_W8A8_ERR_ALIAS;
+  RmsNormBwdArgs a{};
+  a.x = static_cast<const uint16_t*>(x);
+  a.gamma = gamma;
+  a.dn = static_cast<const uint16_t*>(d_normalized);
+  a.dx = static_cast<uint16_t*>(d_x);
+  a.M = m; a.K = k; a.eps = eps;
+  (void)hipGetLastError();
+  if ((k & 7u) == 0) hipLaunchKernelGGL((rms_norm_bwd_kernel<true>), dim3(m), dim3(256), 0, s, a);
+  else hipLaunchKernelGGL((rms_norm_bwd_kernel<false>), dim3(m), dim3(256), 0, s, a);
+  return launch_status();
+}
+
+
 }  // namespace
 
 extern "C" {
@@ -922,6 +968,16 @@ int mi355_w8a8_lora_linear_bwd_v1(const mi355_w8a8_bwd_problem* p, void* stream)
 
 int mi355_w8a8_qkv_split_norm_rope_v1(const mi355_w8a8_qkv_post_problem* p, void* stream) {
   return run_qkv_post(p, static_cast<hipStream_t>(stream));
+}
+
+int mi355_w8a8_swiglu_bwd_v1(const void* fused, const void* d_product, void* d_fused, uint32_t m, uint32_t n,
+                             void* stream) {
+  return run_swiglu_bwd(fused, d_product, d_fused, m, n, static_cast<hipStream_t>(stream));
+}
+
+int mi355_w8a8_rms_norm_bwd_v1(const void* x, const float* gamma, const void* d_normalized, void* d_x, uint32_t m,
+                               uint32_t k, float eps, void* stream) {
+  return run_rms_norm_bwd(x, gamma, d_normalized, d_x, m, k, eps, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

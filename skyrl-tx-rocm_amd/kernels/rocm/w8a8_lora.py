@@ -214,7 +214,8 @@ class ForwardPlan:
     def __init__(self, x: torch.Tensor, weight, lora_a=None, lora_b=None, lora_scaling=None, *,
                  adapter_indices: torch.Tensor | None = None, rms_gamma: torch.Tensor | None = None,
                  eps: float = 1e-6, residual: torch.Tensor | None = None, swiglu: bool = False,
-                 flags: int = 0, return_aux: bool = False, entry: str = "forward"):
+                 flags: int = 0, return_aux: bool = False, entry: str = "forward",
+                 want_normalized: bool = False):
         if x.dtype != torch.bfloat16:
             raise TypeError(f"x must be BF16, got {x.dtype}")
         if x.ndim < 2 or math.prod(x.shape[:-1]) <= 0:
@@ -269,8 +270,8 @@ class ForwardPlan:
             aux["x_codes"] = torch.empty((m, k), dtype=torch.int8, device=dev)
             aux["x_scales"] = torch.empty((m,), dtype=torch.float32, device=dev)
             aux["acc"] = torch.empty((m, n), dtype=torch.int32, device=dev)
-            if gamma is not None:
-                aux["normalized"] = torch.empty((m, k), dtype=torch.bfloat16, device=dev)
+        if (return_aux or want_normalized) and gamma is not None:
+            aux["normalized"] = torch.empty((m, k), dtype=torch.bfloat16, device=dev)
 
         p = _native.Problem()
         p.struct_size = ctypes.sizeof(_native.Problem)
@@ -304,6 +305,7 @@ class ForwardPlan:
         self._fn = {"forward": lib.mi355_w8a8_forward_v1, "linear": lib.mi355_w8a8_lora_linear_v1,
                     "gateup": lib.mi355_w8a8_rms_gateup_swiglu_v1,
                     "residual": lib.mi355_w8a8_lora_residual_v1}[entry]
+        self.x_flat, self.gamma, self.adapter_indices = flat, gamma, idx
         self._keep = (flat, pw, a3, b3, s1, idx, gamma, res, ws)
 
     def run(self, extra_flags: int = 0) -> torch.Tensor:
@@ -471,6 +473,178 @@ def lora_linear(x: torch.Tensor, weight, lora_a=None, lora_b=None, lora_scaling=
     if lora_a is not None and not isinstance(scaling, torch.Tensor):
         scaling = torch.as_tensor(scaling, dtype=torch.float32, device=x.device)
     return _LoraLinearFunction.apply(x, lora_a, lora_b, scaling, weight, adapter_indices, residual)
+
+
+# ---------------------------------------------------------------------------------------
+# backward of the fused RMSNorm -> gate/up -> SwiGLU call
+# (skyrl/tx/kernels/rocm/bf16_rms_gate_up_lora_swiglu_contiguous.py:643-689)
+# ---------------------------------------------------------------------------------------
+def swiglu_backward(fused: torch.Tensor, d_product: torch.Tensor, *, in_place: bool = False) -> torch.Tensor:
+    """Cotangent of the interleaved projection from the cotangent of ``silu(gate) * up``
+    (``_fp32_swiglu_pullback_interleaved``, :541-553).  ``fused`` bf16 [..., N], ``d_product``
+    bf16 [..., N / 2]; with ``in_place`` the result overwrites ``fused``."""
+    if fused.dtype != torch.bfloat16 or d_product.dtype != torch.bfloat16:
+        raise TypeError("fused and d_product must be BF16")
+    _require_cuda(fused, "fused")
+    _require_cuda(d_product, "d_product")
+    n = fused.shape[-1]
+    if fused.ndim < 2 or n % 8 or tuple(d_product.shape) != (*fused.shape[:-1], n // 2):
+        raise ValueError(f"need fused [..., N] with N % 8 == 0 and d_product [..., N / 2], got "
+                         f"{tuple(fused.shape)} and {tuple(d_product.shape)}")
+    if in_place and not fused.is_contiguous():
+        raise ValueError("in_place needs a contiguous fused tensor")
+    f2 = fused.reshape(-1, n).contiguous()
+    d2 = d_product.reshape(-1, n // 2).contiguous()
+    out = f2 if in_place else torch.empty_like(f2)
+    with torch.cuda.device(fused.device):
+        status = _native.load().mi355_w8a8_swiglu_bwd_v1(f2.data_ptr(), d2.data_ptr(), out.data_ptr(), f2.shape[0], n,
+                                                         _stream_ptr(fused.device))
+    _native.check("mi355_w8a8_swiglu_bwd_v1", status)
+    return out.reshape(fused.shape)
+
+
+def rms_norm_backward(x: torch.Tensor, gamma: torch.Tensor, d_normalized: torch.Tensor, *, eps: float = 1e-6,
+                      in_place: bool = False) -> torch.Tensor:
+    """Cotangent of x through ``bf16(x * rsqrt(mean(x^2) + eps) * gamma)`` (``_rms_norm_pullback``,
+    :556-574); ``gamma`` float32 [K] is the multiplier itself.  With ``in_place`` the result
+    overwrites ``d_normalized``."""
+    if x.dtype != torch.bfloat16 or d_normalized.dtype != torch.bfloat16:
+        raise TypeError("x and d_normalized must be BF16")
+    _require_cuda(x, "x")
+    _require_cuda(d_normalized, "d_normalized")
+    k = x.shape[-1]
+    if x.ndim < 2 or tuple(d_normalized.shape) != tuple(x.shape) or tuple(gamma.shape) != (k,):
+        raise ValueError(f"need x and d_normalized [..., K] and gamma [K], got {tuple(x.shape)}, "
+                         f"{tuple(d_normalized.shape)} and {tuple(gamma.shape)}")
+    if not isinstance(eps, float) or not eps > 0.0:
+        raise ValueError(f"eps must be a positive float, got {eps!r}")
+    if in_place and not d_normalized.is_contiguous():
+        raise ValueError("in_place needs a contiguous d_normalized tensor")
+    x2 = x.reshape(-1, k).contiguous()
+    d2 = d_normalized.reshape(-1, k).contiguous()
+    g = gamma.to(device=x.device, dtype=torch.float32).contiguous()
+    out = d2 if in_place else torch.empty_like(d2)
+    with torch.cuda.device(x.device):
+        status = _native.load().mi355_w8a8_rms_norm_bwd_v1(x2.data_ptr(), g.data_ptr(), d2.data_ptr(), out.data_ptr(),
+                                                           x2.shape[0], k, eps, _stream_ptr(x.device))
+    _native.check("mi355_w8a8_rms_norm_bwd_v1", status)
+    return out.reshape(x.shape)
+
+
+class FusedBackwardPlan:
+    """Buffers and C structs of one backward of the fused RMSNorm -> gate/up -> SwiGLU call.
+
+    The forward keeps neither the projection nor the normalized rows, so ``run()`` recomputes both
+    with one forward call (no SwiGLU, normalized rows as the auxiliary output) and then runs three
+    native stages: the SwiGLU pull-back in place on the projection, the linear backward on the
+    normalized rows, and the RMSNorm pull-back in place on that call's dx.
+    """
+
+    def __init__(self, x: torch.Tensor, gamma: torch.Tensor, weight, lora_a, lora_b, lora_scaling,
+                 d_product: torch.Tensor, *, adapter_indices: torch.Tensor | None = None, eps: float = 1e-6,
+                 need_lora_grads: bool = True):
+        if not isinstance(eps, float) or not eps > 0.0:
+            raise ValueError(f"eps must be a positive float, got {eps!r}")
+        self.fwd = ForwardPlan(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices,
+                               rms_gamma=gamma, eps=eps, want_normalized=True)
+        d = self.fwd.dims
+        m, k, n = d["m"], d["k"], d["n"]
+        if n % 8:
+            raise ValueError(f"the fused backward needs N % 8 == 0, got N={n}")
+        if d_product.dtype != torch.bfloat16:
+            raise TypeError(f"d_product must be BF16, got {d_product.dtype}")
+        _require_cuda(d_product, "d_product")
+        if tuple(d_product.shape) != (*x.shape[:-1], n // 2):
+            raise ValueError(f"d_product must have shape {(*x.shape[:-1], n // 2)}, got {tuple(d_product.shape)}")
+        self.d_product = d_product.reshape(m, n // 2).contiguous()
+        self.x = self.fwd.x_flat
+        self.gamma = self.fwd.gamma
+        self.eps = eps
+        idx = self.fwd.adapter_indices
+        # fwd.out doubles as the projection and, after the in-place pull-back, as its cotangent
+        self.bwd = BackwardPlan(self.fwd.aux["normalized"], self.fwd.out, weight, lora_a, lora_b, lora_scaling,
+                                adapter_indices=idx, need_lora_grads=need_lora_grads)
+        self.device = x.device
+        self.dx_shape = tuple(x.shape)
+        self.dims = d
+        self._lib = _native.load()
+
+    def run_swiglu_stage(self) -> None:
+        d = self.dims
+        with torch.cuda.device(self.device):
+            status = self._lib.mi355_w8a8_swiglu_bwd_v1(self.fwd.out.data_ptr(), self.d_product.data_ptr(),
+                                                        self.fwd.out.data_ptr(), d["m"], d["n"],
+                                                        _stream_ptr(self.device))
+        _native.check("mi355_w8a8_swiglu_bwd_v1", status)
+
+    def run_rms_stage(self) -> None:
+        d = self.dims
+        with torch.cuda.device(self.device):
+            status = self._lib.mi355_w8a8_rms_norm_bwd_v1(self.x.data_ptr(), self.gamma.data_ptr(),
+                                                          self.bwd.dx.data_ptr(), self.bwd.dx.data_ptr(), d["m"],
+                                                          d["k"], self.eps, _stream_ptr(self.device))
+        _native.check("mi355_w8a8_rms_norm_bwd_v1", status)
+
+    def run(self):
+        """Enqueue the four calls; returns ``(dx, d_lora_a, d_lora_b, d_lora_scaling)`` (reused tensors)."""
+        self.fwd.run()
+        self.run_swiglu_stage()
+        dn, da, db, ds = self.bwd.run()
+        self.run_rms_stage()
+        return dn.reshape(self.dx_shape), da, db, ds
+
+
+def rms_gate_up_swiglu_backward(x: torch.Tensor, gamma: torch.Tensor, weight, lora_a, lora_b, lora_scaling,
+                                d_product: torch.Tensor, *, adapter_indices: torch.Tensor | None = None,
+                                eps: float = 1e-6, need_lora_grads: bool = True):
+    """Cotangents ``(dx, d_lora_a, d_lora_b, d_lora_scaling)`` of the fused call
+    (bf16_rms_gate_up_lora_swiglu_contiguous.py:643-689 around the quantized projection's own rule)."""
+    return FusedBackwardPlan(x, gamma, weight, lora_a, lora_b, lora_scaling, d_product,
+                             adapter_indices=adapter_indices, eps=eps, need_lora_grads=need_lora_grads).run()
+
+
+class _RmsGateUpFunction(torch.autograd.Function):
+    """The fused forward with the derivative rule of ``_bf16_rms_gate_up_lora_swiglu_contiguous``
+    (bf16_rms_gate_up_lora_swiglu_contiguous.py:577-695): cotangents for x, A, B (and the scaling);
+    none for the norm weight and the frozen kernel."""
+
+    @staticmethod
+    def forward(ctx, x, lora_a, lora_b, lora_scaling, gamma, weight, adapter_indices, eps):
+        out = forward(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices,
+                      rms_gamma=gamma, eps=eps, swiglu=True, entry="gateup")
+        ctx.save_for_backward(x, lora_a, lora_b, lora_scaling, gamma)
+        ctx.weight = weight
+        ctx.adapter_indices = adapter_indices
+        ctx.eps = eps
+        return out
+
+    @staticmethod
+    def backward(ctx, d_product):
+        x, lora_a, lora_b, lora_scaling, gamma = ctx.saved_tensors
+        need = lora_a is not None and any(ctx.needs_input_grad[1:4])
+        dx, da, db, ds = rms_gate_up_swiglu_backward(x, gamma, ctx.weight, lora_a, lora_b, lora_scaling,
+                                                     d_product.contiguous(), adapter_indices=ctx.adapter_indices,
+                                                     eps=ctx.eps, need_lora_grads=need)
+        if need:
+            if lora_a.ndim == 2:
+                da, db = da[0], db[0]
+            ds = ds.reshape(lora_scaling.shape).to(lora_scaling.dtype)
+        return dx, da, db, ds, None, None, None, None
+
+
+def rms_gate_up_lora_swiglu(x: torch.Tensor, gamma: torch.Tensor, weight, lora_a=None, lora_b=None,
+                            lora_scaling=None, *, adapter_indices: torch.Tensor | None = None,
+                            eps: float = 1e-6) -> torch.Tensor:
+    """RMSNorm (multiplier ``gamma``, float32) -> W8A8 gate/up (+LoRA) -> SwiGLU that autograd can
+    differentiate in x and the LoRA parameters."""
+    tensors = [t for t in (x, lora_a, lora_b, lora_scaling) if isinstance(t, torch.Tensor)]
+    if not (torch.is_grad_enabled() and any(t.requires_grad for t in tensors)):
+        return forward(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices,
+                       rms_gamma=gamma, eps=eps, swiglu=True, entry="gateup")
+    scaling = lora_scaling
+    if lora_a is not None and not isinstance(scaling, torch.Tensor):
+        scaling = torch.as_tensor(scaling, dtype=torch.float32, device=x.device)
+    return _RmsGateUpFunction.apply(x, lora_a, lora_b, scaling, gamma, weight, adapter_indices, eps)
 
 
 # ---------------------------------------------------------------------------------------
@@ -761,15 +935,16 @@ def w8a8_rms_gate_up_lora_swiglu(x, rms_weight, weight, lora_a, lora_b, lora_sca
     """RMSNorm -> W8A8 gate/up (+LoRA) -> SwiGLU; fused columns are (gate, up) interleaved.
 
     ``rms_weight`` multiplies the normalized rows (Qwen3); with ``rms_is_delta`` it is
-    the Qwen3.5 delta and the multiplier is ``1 + delta`` evaluated in float32.
+    the Qwen3.5 delta and the multiplier is ``1 + delta`` evaluated in float32.  Differentiable in
+    x and the LoRA parameters; the norm weight and the frozen kernel are constants.
     """
     _check_enabled(enabled, interpret, "RMSNorm gate/up SwiGLU")
     _validate_exact_bool("rms_is_delta", rms_is_delta)
-    gamma = rms_weight.to(torch.float32)
+    gamma = rms_weight.detach().to(torch.float32)
     if rms_is_delta:
         gamma = 1.0 + gamma
-    return forward(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices,
-                   rms_gamma=gamma, eps=eps, swiglu=True, entry="gateup")
+    return rms_gate_up_lora_swiglu(x, gamma, weight, lora_a, lora_b, lora_scaling,
+                                   adapter_indices=adapter_indices, eps=eps)
 
 
 def w8a8_lora_residual(x, weight, lora_a, lora_b, lora_scaling, residual, *, enabled: bool = False,
