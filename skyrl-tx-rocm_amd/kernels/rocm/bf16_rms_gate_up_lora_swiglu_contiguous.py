@@ -6,7 +6,9 @@ Same name, positional order and keywords as the reference's entry point
 shape; ``frozen_weight`` is a ``GroupQuantizedWeight`` (int8 codes, one scale per output channel,
 columns interleaved gate0, up0, gate1, up1, ...) instead of a bf16 matrix.  RMSNorm with
 ``1 + rms_delta``, the W8A8 gate/up projection, LoRA and SwiGLU run as one native forward call.
-Tile keywords are validated as exact integers and otherwise ignored; forward only.
+Tile keywords are validated as exact integers and otherwise ignored.  Under autograd the call has
+the reference's derivative rule (:643-689): cotangents for ``x``, ``lora_a``, ``lora_b``; none for
+``rms_delta`` and the frozen kernel.
 """
 
 from __future__ import annotations
