@@ -46,6 +46,9 @@ WORKLOADS = {
     # linear backward, RMSNorm pull-back
     "qwen3-8b-gate_up-m4096-fused-backward": dict(m=4096, k=4096, n=24576, n_adapters=8, rank=32, rms=True,
                                                   swiglu=True, idx_mode="uniform", seed=2, backward=True),
+    # token routing around the expert GEMMs at the Qwen3-30B-A3B geometry: softmax / top-8 of 128 experts,
+    # stable sort of the 32768 (token, choice) pairs with the gather of their rows, weighted combine
+    "qwen3-30b-a3b-moe-routing-t4096": dict(m=4096, n_experts=128, top_k=8, hidden=2048, seed=6, moe_routing=True),
     # Qwen3.5-4B attention input stage: RMSNorm -> W8A8 QKV [2560 -> 10240] + 4 adapters rank 64 ->
     # split, Q/K RMSNorm, partial RoPE (16 query heads, 4 kv heads, head_dim 256, 64 rotary dims)
     "qwen3.5-4b-qkv-m2048": dict(m=2048, k=2560, n=10240, n_adapters=4, rank=64, alpha=128, rms=True,
@@ -312,6 +315,94 @@ def bench_fused_backward(args, cfg, pkg, dev):
     return 0
 
 
+def bench_moe_routing(args, cfg, pkg, dev):
+    """One step = route + dispatch + combine (the expert GEMMs between dispatch and combine are the
+    grouped workloads' business; here the sorted rows stand in for the expert output).  ``value`` and
+    the roofline are HBM bytes per second: the roofline prices the dispatch call (histogram, scan,
+    scatter and gather kernels), which moves the most bytes."""
+    import torch
+
+    from oracle import w8a8_oracle as o
+
+    w8 = pkg.w8a8_lora
+    t, e, k, h = cfg["m"], cfg["n_experts"], cfg["top_k"], cfg["hidden"]
+    rng = np.random.default_rng(cfg["seed"])
+    logits = (rng.standard_normal((t, e)) * 2.0).astype(np.float32)
+    hidden = o.bf16_round(rng.standard_normal((t, h)).astype(np.float32))
+    logits_t = torch.from_numpy(logits).to(dev)
+    hidden_t = torch.from_numpy(hidden).to(dev).to(torch.bfloat16)
+
+    def step():
+        weights, selected = w8.moe_route(logits_t, k)
+        xs, sizes, _, unsort, _ = w8.moe_dispatch(hidden_t, selected, e, repeat=k)
+        return w8.moe_combine(xs, unsort, weights), weights, selected, xs, sizes, unsort
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    combined, weights, selected, xs, sizes, unsort = out
+
+    def timed(fn):
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        for a, b in ev:
+            a.record()
+            fn()
+            b.record()
+        torch.cuda.synchronize()
+        return float(np.mean([a.elapsed_time(b) for a, b in ev]))
+
+    route_ms = timed(lambda: w8.moe_route(logits_t, k))
+    dispatch_ms = timed(lambda: w8.moe_dispatch(hidden_t, selected, e, repeat=k))
+    combine_ms = timed(lambda: w8.moe_combine(xs, unsort, weights))
+    p = t * k
+    route_bytes = 4 * t * e + 8 * p
+    dispatch_bytes = 2 * t * h + 2 * p * h + 4 * p * 3 + 4 * e   # rows in once, rows out, indices in, two index arrays out
+    combine_bytes = 2 * p * h + 2 * t * h + 8 * p
+    total_bytes = route_bytes + dispatch_bytes + combine_bytes
+    achieved = dispatch_bytes / (dispatch_ms * 1e-3) / 1e9
+    result = {
+        "metric": "MoE token routing (route + dispatch + combine), GB/s of algorithmic HBM bytes per call",
+        "value": total_bytes / (ms_per_step * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "moe_hist_kernel + moe_scan_kernel + moe_scatter_kernel + moe_gather_kernel (one dispatch call)",
+                     "kernel_avg_ms": dispatch_ms, "algorithmic_bytes": dispatch_bytes},
+        "stages": {"route_ms": route_ms, "route_bytes": route_bytes, "dispatch_ms": dispatch_ms,
+                   "combine_ms": combine_ms, "combine_bytes": combine_bytes,
+                   "combine_gbs": combine_bytes / (combine_ms * 1e-3) / 1e9},
+    }
+    if not args.no_cpu_baseline:
+        t1 = time.perf_counter()
+        want_w, want_sel = o.moe_route(logits, k)
+        want_xs, want_sizes, want_unsort, _ = o.prepare_routing(np.repeat(hidden, k, axis=0), want_sel.ravel(), e)
+        want_out = o.moe_combine(want_xs, want_unsort, want_w)
+        secs = time.perf_counter() - t1
+        try:
+            cores = len(os.sched_getaffinity(0))
+        except AttributeError:
+            cores = os.cpu_count() or 1
+        result["cpu_baseline"] = {"value": total_bytes / secs / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                                  "sample": f"the whole workload ({t} tokens), NumPy oracle route + prepare_routing + "
+                                            f"combine, one run, {secs:.3f} s", "seconds": secs}
+        sel = selected.cpu().numpy()
+        rows_same = (sel == want_sel).all(axis=1)
+        got_out = combined.to(torch.float32).cpu().numpy()
+        result["parity_sample"] = {
+            "tokens": t, "tokens_with_equal_selection": int(rows_same.sum()),
+            "group_sizes_equal": bool((sizes.cpu().numpy() == want_sizes).all()),
+            "combine_violations": int(np.count_nonzero(~o.within_tolerance(got_out[rows_same], want_out[rows_same])))}
+    print(json.dumps(result))
+    return 0
+
+
 def bench_qkv(args, cfg, pkg, dev):
     """One step = the W8A8 QKV projection (RMSNorm prologue, GEMM, LoRA) + the split / Q-K norm /
     RoPE kernel.  ``value`` is int8 TOPS of the projection over the whole step; the roofline prices
@@ -442,6 +533,8 @@ def main() -> int:
         if cfg.get("swiglu"):
             return bench_fused_backward(args, cfg, pkg, dev)
         return bench_backward(args, cfg, pkg, dev)
+    if cfg.pop("moe_routing", False):
+        return bench_moe_routing(args, cfg, pkg, dev)
     if "qkv" in cfg:
         return bench_qkv(args, cfg, pkg, dev)
     case = wc.make_case(cfg["m"], cfg["k"], cfg["n"], n_adapters=cfg.get("n_adapters", 0),

@@ -23,6 +23,12 @@
  *                                      on W8A8 weights
  *   - mi355_w8a8_grouped_v1            skyrl/tx/layers/lora.py:394-444 (LoRAExpert.__call__) with
  *                                      the ragged_dot of skyrl/tx/layers/util.py:8-59
+ *   - mi355_w8a8_lora_linear_bwd_v1    skyrl/tx/kernels/quantized_lora.py:337-394 (the VJP)
+ *   - mi355_w8a8_swiglu_bwd_v1 / mi355_w8a8_rms_norm_bwd_v1
+ *                                      skyrl/tx/kernels/rocm/bf16_rms_gate_up_lora_swiglu_contiguous.py:541-574
+ *   - mi355_w8a8_qkv_split_norm_rope_v1 skyrl/tx/kernels/qwen3_5_qkv_lora.py:266-286
+ *   - mi355_w8a8_moe_route_v1 / _moe_dispatch_v1 / _moe_combine_v1
+ *                                      skyrl/tx/models/qwen3.py:172-210, skyrl/tx/layers/util.py:66-87
  * The typed-FFI handler shape these sit behind is rocm/QUANTIZED_FFI.md:589-599 and
  * skyrl/tx/kernels/rocm/ffi/gdn_ffi_smoke.hip:43-82.
  */
@@ -255,6 +261,56 @@ int mi355_w8a8_swiglu_bwd_v1(const void* fused, const void* d_product, void* d_f
                              void* stream);
 int mi355_w8a8_rms_norm_bwd_v1(const void* x, const float* gamma, const void* d_normalized, void* d_x, uint32_t m,
                                uint32_t k, float eps, void* stream);
+
+/*
+ * Token routing around the grouped expert GEMMs (Qwen3Experts.__call__, skyrl/tx/models/qwen3.py:
+ * 172-210).  Index outputs are exact; nothing here synchronizes or allocates.
+ *
+ * mi355_w8a8_moe_route_v1 replaces qwen3.py:175-178: probabilities = softmax(router_logits) in
+ * float32, top_k largest per token in descending order (ties: the lower expert, as lax.top_k),
+ * weights divided by their sum when norm_topk_prob.  router_logits f32 [n_tokens, n_experts],
+ * weights f32 and selected int32 [n_tokens, top_k]; n_experts <= 1024, top_k <= min(64, n_experts).
+ */
+int mi355_w8a8_moe_route_v1(const float* router_logits, uint32_t n_tokens, uint32_t n_experts, uint32_t top_k,
+                            uint32_t norm_topk_prob, float* weights, int32_t* selected, void* stream);
+
+/*
+ * mi355_w8a8_moe_dispatch_v1 replaces prepare_routing (skyrl/tx/layers/util.py:66-87) together with
+ * the jnp.repeat in front of it (qwen3.py:189-190): pair p = (token p / repeat, choice p % repeat)
+ * belongs to group indices[p]; the pairs are sorted by group, stably, and every pair's token row is
+ * copied to its sorted position.  repeat = top_k for the expert MLP, 1 for a plain prepare_routing.
+ * Group indices outside [0, n_groups) are clamped into range.
+ */
+typedef struct mi355_w8a8_moe_dispatch_problem {
+  uint32_t struct_size;     /* sizeof(mi355_w8a8_moe_dispatch_problem) */
+  uint32_t flags;           /* 0 */
+  uint32_t n_pairs;         /* rows to sort = tokens * repeat */
+  uint32_t repeat;          /* >= 1, divides n_pairs */
+  uint32_t width;           /* bf16 columns of a token row, multiple of 8 (ignored without tokens) */
+  uint32_t n_groups;        /* <= 1024 */
+  const void* tokens;       /* bf16 [n_pairs / repeat, width], or NULL: index outputs only */
+  const int32_t* indices;   /* int32 [n_pairs] */
+  const int32_t* adapter_indices; /* optional int32 [n_pairs / repeat], sorted along with the rows */
+  void* sorted_tokens;      /* bf16 [n_pairs, width] (with tokens) */
+  int32_t* group_sizes;     /* int32 [n_groups] */
+  int32_t* sort_indices;    /* int32 [n_pairs]: the pair at every sorted position (argsort) */
+  int32_t* unsort_indices;  /* int32 [n_pairs]: the sorted position of every pair (its inverse) */
+  int32_t* sorted_adapters; /* int32 [n_pairs], with adapter_indices */
+  void* workspace;          /* 256-byte aligned device scratch */
+  uint64_t workspace_bytes; /* >= mi355_w8a8_moe_dispatch_workspace_bytes(n_pairs, n_groups) */
+} mi355_w8a8_moe_dispatch_problem;
+
+uint64_t mi355_w8a8_moe_dispatch_workspace_bytes(uint32_t n_pairs, uint32_t n_groups);
+int mi355_w8a8_moe_dispatch_v1(const mi355_w8a8_moe_dispatch_problem* problem, void* stream);
+
+/*
+ * mi355_w8a8_moe_combine_v1 replaces the unsort and weighted sum of qwen3.py:205-207:
+ * out[t] = bf16(sum_j f32(expert_out[unsort_indices[t * top_k + j]]) * weights[t, j]), products and
+ * the sum in float32 in choice order.  expert_out bf16 [n_tokens * top_k, width] in sorted order,
+ * out bf16 [n_tokens, width]; width a multiple of 8, top_k <= 64.
+ */
+int mi355_w8a8_moe_combine_v1(const void* expert_out, const int32_t* unsort_indices, const float* weights, void* out,
+                              uint32_t n_tokens, uint32_t top_k, uint32_t width, void* stream);
 
 #ifdef __cplusplus
 }

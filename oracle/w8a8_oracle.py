@@ -790,6 +790,15 @@ def grouped_quantized_lora_linear_f32(x_sorted, group_sizes, weights, lora_a, lo
     return out
 
 
+def moe_combine(expert_out, unsort, weights) -> np.ndarray:
+    """bf16(sum_j f32(expert_out[unsort[t k + j]]) * weights[t, j]); qwen3.py:205-207 with the products
+    and the sum over the choices in float32, choice order, one cast."""
+    weights = np.asarray(weights, dtype=F32)
+    t, top_k = weights.shape
+    per_tok = np.asarray(expert_out, dtype=F32)[np.asarray(unsort)].reshape(t, top_k, -1)
+    return bf16_round(np.sum(per_tok * weights[..., None], axis=1, dtype=F32))
+
+
 def moe_expert_mlp(hidden, router_logits, top_k, gate_up_weights, down_weights,
                    gate_up_a, gate_up_b, down_a, down_b, scaling, return_stages: bool = False):
     """Composite oracle for the grouped W8A8 + LoRA expert MLP.
@@ -808,8 +817,7 @@ def moe_expert_mlp(hidden, router_logits, top_k, gate_up_weights, down_weights,
     act = swiglu_from_interleaved(fused)
     down = bf16_round(grouped_quantized_lora_linear_f32(
         act, group_sizes, down_weights, down_a, down_b, scaling))
-    per_tok = down[unsort].reshape(hidden.shape[0], top_k, -1)
-    out = bf16_round(np.sum(per_tok * weights[..., None], axis=1, dtype=F32))
+    out = moe_combine(down, unsort, weights)
     if return_stages:
         return out, {"group_sizes": group_sizes, "unsort": unsort, "x_sorted": x_sorted,
                      "fused": fused, "act": act, "down": down, "weights": weights,

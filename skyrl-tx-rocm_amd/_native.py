@@ -36,6 +36,8 @@ EXPORTS = (
     "mi355_w8a8_bwd_workspace_bytes", "mi355_w8a8_lora_linear_bwd_v1",
     "mi355_w8a8_qkv_split_norm_rope_v1",
     "mi355_w8a8_swiglu_bwd_v1", "mi355_w8a8_rms_norm_bwd_v1",
+    "mi355_w8a8_moe_route_v1", "mi355_w8a8_moe_dispatch_workspace_bytes", "mi355_w8a8_moe_dispatch_v1",
+    "mi355_w8a8_moe_combine_v1",
 )
 
 _u32, _u64, _vp, _f32 = ctypes.c_uint32, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_float
@@ -89,6 +91,18 @@ class QkvPostProblem(ctypes.Structure):
     ]
 
 
+class MoeDispatchProblem(ctypes.Structure):
+    """struct mi355_w8a8_moe_dispatch_problem"""
+
+    _fields_ = [
+        ("struct_size", _u32), ("flags", _u32), ("n_pairs", _u32), ("repeat", _u32), ("width", _u32),
+        ("n_groups", _u32),
+        ("tokens", _vp), ("indices", _vp), ("adapter_indices", _vp), ("sorted_tokens", _vp), ("group_sizes", _vp),
+        ("sort_indices", _vp), ("unsort_indices", _vp), ("sorted_adapters", _vp), ("workspace", _vp),
+        ("workspace_bytes", _u64),
+    ]
+
+
 class NativeError(RuntimeError):
     def __init__(self, fn: str, status: int, detail: str):
         super().__init__(f"{fn} failed: {STATUS.get(status, status)} ({detail})")
@@ -128,6 +142,14 @@ def _bind(lib: ctypes.CDLL) -> None:
     lib.mi355_w8a8_lora_linear_bwd_v1.argtypes = (ctypes.POINTER(BwdProblem), _vp)
     lib.mi355_w8a8_qkv_split_norm_rope_v1.restype = ctypes.c_int
     lib.mi355_w8a8_qkv_split_norm_rope_v1.argtypes = (ctypes.POINTER(QkvPostProblem), _vp)
+    lib.mi355_w8a8_moe_route_v1.restype = ctypes.c_int
+    lib.mi355_w8a8_moe_route_v1.argtypes = (_vp, _u32, _u32, _u32, _u32, _vp, _vp, _vp)
+    lib.mi355_w8a8_moe_dispatch_workspace_bytes.restype = _u64
+    lib.mi355_w8a8_moe_dispatch_workspace_bytes.argtypes = (_u32, _u32)
+    lib.mi355_w8a8_moe_dispatch_v1.restype = ctypes.c_int
+    lib.mi355_w8a8_moe_dispatch_v1.argtypes = (ctypes.POINTER(MoeDispatchProblem), _vp)
+    lib.mi355_w8a8_moe_combine_v1.restype = ctypes.c_int
+    lib.mi355_w8a8_moe_combine_v1.argtypes = (_vp, _vp, _vp, _vp, _u32, _u32, _u32, _vp)
     lib.mi355_w8a8_swiglu_bwd_v1.restype = ctypes.c_int
     lib.mi355_w8a8_swiglu_bwd_v1.argtypes = (_vp, _vp, _vp, _u32, _u32, _vp)
     lib.mi355_w8a8_rms_norm_bwd_v1.restype = ctypes.c_int

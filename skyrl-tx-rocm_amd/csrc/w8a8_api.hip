@@ -12,6 +12,7 @@
 #include "w8a8_backward.h"
 #include "w8a8_qkv_post.h"
 #include "w8a8_fused_bwd.h"
+#include "w8a8_moe.h"
 
 using namespace w8a8;
 
@@ -847,6 +848,125 @@ int run_rms_norm_bwd(const void* x, const float* gamma, const void* d_normalized
 }
 
 
+int run_moe_route(const float* logits, uint32_t t, uint32_t e, uint32_t top_k, uint32_t norm, float* weights,
+                  int32_t* selected, hipStream_t s) {
+  if (!logits || !weights || !selected) return MI355_W8A8_ERR_NULL;
+  if (t == 0 || e == 0 || top_k == 0 || top_k > e || norm > 1u) return MI355_W8A8_ERR_SHAPE;
+  if (e > kMoeMaxExperts || top_k > kMoeMaxTopK || t > kMaxRows) return MI355_W8A8_ERR_UNSUPPORTED;
+  if ((reinterpret_cast<uintptr_t>(logits) | reinterpret_cast<uintptr_t>(weights) |
+       reinterpret_cast<uintptr_t>(selected)) & 3u)
+    return MI355_W8A8_ERR_ALIGN;
+  const uint64_t out_bytes = (uint64_t)t * top_k * 4u;
+  if (overlaps(weights, out_bytes, logits, (uint64_t)t * e * 4u) ||
+      overlaps(selected, out_bytes, logits, (uint64_t)t * e * 4u) || overlaps(weights, out_bytes, selected, out_bytes))
+    return MI355_W8A8_ERR_ALIAS;
+  MoeRouteArgs a{};
+  a.logits = logits; a.weights = weights; a.selected = selected;
+  a.T = t; a.E = e; a.top_k = top_k; a.norm = norm;
+  (void)hipGetLastError();
+  const dim3 grid((t + 3u) / 4u), block(256);
+  if (e <= 64u) hipLaunchKernelGGL((moe_route_kernel<1>), grid, block, 0, s, a);
+  else if (e <= 128u) hipLaunchKernelGGL((moe_route_kernel<2>), grid, block, 0, s, a);
+  else if (e <= 256u) hipLaunchKernelGGL((moe_route_kernel<4>), grid, block, 0, s, a);
+  else if (e <= 512u) hipLaunchKernelGGL((moe_route_kernel<8>), grid, block, 0, s, a);
+  else hipLaunchKernelGGL((moe_route_kernel<16>), grid, block, 0, s, a);
+  return launch_status();
+}
+
+struct MoeSortLayout { uint64_t chunk_cnt, group_start, total; uint32_t n_chunks; };
+
+MoeSortLayout make_moe_sort_layout(uint32_t n_pairs, uint32_t n_groups) {
+  MoeSortLayout L{};
+  L.n_chunks = (n_pairs + kMoeChunk - 1u) / kMoeChunk;
+  L.chunk_cnt = 0;
+  L.group_start = ((uint64_t)L.n_chunks * n_groups * 4u + 255u) & ~255ull;
+  L.total = L.group_start + (((uint64_t)n_groups * 4u + 255u) & ~255ull);
+  return L;
+}
+
+int validate_moe_sort_dims(uint32_t n_pairs, uint32_t n_groups) {
+  if (n_pairs == 0 || n_groups == 0) return MI355_W8A8_ERR_SHAPE;
+  if (n_groups > kMoeMaxExperts || n_pairs > (1u << 30)) return MI355_W8A8_ERR_UNSUPPORTED;
+  return MI355_W8A8_OK;
+}
+
+int run_moe_dispatch(const mi355_w8a8_moe_dispatch_problem* p, hipStream_t s) {
+  if (!p) return MI355_W8A8_ERR_NULL;
+  if (p->struct_size != sizeof(mi355_w8a8_moe_dispatch_problem)) return MI355_W8A8_ERR_STRUCT;
+  if (p->flags) return MI355_W8A8_ERR_SHAPE;
+  int st = validate_moe_sort_dims(p->n_pairs, p->n_groups);
+  if (st) return st;
+  if (p->repeat == 0 || p->n_pairs % p->repeat) return MI355_W8A8_ERR_SHAPE;
+  if (!p->indices || !p->group_sizes || !p->sort_indices || !p->unsort_indices) return MI355_W8A8_ERR_NULL;
+  if ((p->adapter_indices != nullptr) != (p->sorted_adapters != nullptr)) return MI355_W8A8_ERR_NULL;
+  if ((p->tokens != nullptr) != (p->sorted_tokens != nullptr)) return MI355_W8A8_ERR_NULL;
+  if (p->tokens && (p->width == 0 || (p->width & 7u))) return MI355_W8A8_ERR_SHAPE;
+  if (!aligned16(p->tokens) || !aligned16(p->sorted_tokens)) return MI355_W8A8_ERR_ALIGN;
+  if ((reinterpret_cast<uintptr_t>(p->indices) | reinterpret_cast<uintptr_t>(p->group_sizes) |
+       reinterpret_cast<uintptr_t>(p->sort_indices) | reinterpret_cast<uintptr_t>(p->unsort_indices) |
+       reinterpret_cast<uintptr_t>(p->adapter_indices) | reinterpret_cast<uintptr_t>(p->sorted_adapters)) & 3u)
+    return MI355_W8A8_ERR_ALIGN;
+  const uint64_t idx_bytes = (uint64_t)p->n_pairs * 4u;
+  if (p->tokens) {
+    const uint64_t out_bytes = (uint64_t)p->n_pairs * p->width * 2u;
+    if (overlaps(p->sorted_tokens, out_bytes, p->tokens, out_bytes / p->repeat) ||
+        overlaps(p->sorted_tokens, out_bytes, p->indices, idx_bytes) ||
+        overlaps(p->sorted_tokens, out_bytes, p->sort_indices, idx_bytes) ||
+        overlaps(p->sorted_tokens, out_bytes, p->unsort_indices, idx_bytes))
+      return MI355_W8A8_ERR_ALIAS;
+  }
+  if (overlaps(p->sort_indices, idx_bytes, p->indices, idx_bytes) ||
+      overlaps(p->unsort_indices, idx_bytes, p->indices, idx_bytes) ||
+      overlaps(p->sort_indices, idx_bytes, p->unsort_indices, idx_bytes))
+    return MI355_W8A8_ERR_ALIAS;
+  const MoeSortLayout L = make_moe_sort_layout(p->n_pairs, p->n_groups);
+  if (!p->workspace || p->workspace_bytes < L.total) return MI355_W8A8_ERR_WORKSPACE;
+  if (reinterpret_cast<uintptr_t>(p->workspace) & 255u) return MI355_W8A8_ERR_ALIGN;
+  unsigned char* ws = static_cast<unsigned char*>(p->workspace);
+  MoeSortArgs a{};
+  a.indices = p->indices;
+  a.tokens = static_cast<const uint16_t*>(p->tokens);
+  a.adapters = p->adapter_indices;
+  a.sorted_tokens = static_cast<uint16_t*>(p->sorted_tokens);
+  a.group_sizes = p->group_sizes;
+  a.sort_indices = p->sort_indices;
+  a.unsort_indices = p->unsort_indices;
+  a.sorted_adapters = p->sorted_adapters;
+  a.chunk_cnt = reinterpret_cast<int32_t*>(ws + L.chunk_cnt);
+  a.group_start = reinterpret_cast<int32_t*>(ws + L.group_start);
+  a.P = p->n_pairs; a.G = p->n_groups; a.repeat = p->repeat; a.width = p->width; a.n_chunks = L.n_chunks;
+  (void)hipGetLastError();
+  hipLaunchKernelGGL(moe_hist_kernel, dim3(L.n_chunks), dim3(1024), 0, s, a);
+  if ((st = launch_status())) return st;
+  hipLaunchKernelGGL(moe_scan_kernel, dim3(1), dim3(1024), 0, s, a);
+  if ((st = launch_status())) return st;
+  hipLaunchKernelGGL(moe_scatter_kernel, dim3(L.n_chunks), dim3(1024), 0, s, a);
+  if ((st = launch_status()) || !a.tokens) return st;
+  hipLaunchKernelGGL(moe_gather_kernel, dim3((p->n_pairs + 7u) / 8u), dim3(256), 0, s, a);
+  return launch_status();
+}
+
+int run_moe_combine(const void* expert_out, const int32_t* unsort, const float* weights, void* out, uint32_t t,
+                    uint32_t top_k, uint32_t width, hipStream_t s) {
+  if (!expert_out || !unsort || !weights || !out) return MI355_W8A8_ERR_NULL;
+  if (t == 0 || top_k == 0 || width == 0 || (width & 7u)) return MI355_W8A8_ERR_SHAPE;
+  if (top_k > kMoeMaxTopK || t > kMaxRows || (uint64_t)t * top_k > (1ull << 30)) return MI355_W8A8_ERR_UNSUPPORTED;
+  if (!aligned16(expert_out) || !aligned16(out)) return MI355_W8A8_ERR_ALIGN;
+  if ((reinterpret_cast<uintptr_t>(unsort) | reinterpret_cast<uintptr_t>(weights)) & 3u) return MI355_W8A8_ERR_ALIGN;
+  const uint64_t out_bytes = (uint64_t)t * width * 2u;
+  if (overlaps(out, out_bytes, expert_out, out_bytes * top_k) || overlaps(out, out_bytes, unsort, (uint64_t)t * top_k * 4u) ||
+      overlaps(out, out_bytes, weights, (uint64_t)t * top_k * 4u))
+    return MI355_W8A8_ERR_ALIAS;
+  MoeCombineArgs a{};
+  a.expert_out = static_cast<const uint16_t*>(expert_out);
+  a.unsort = unsort; a.weights = weights;
+  a.out = static_cast<uint16_t*>(out);
+  a.T = t; a.top_k = top_k; a.width = width;
+  (void)hipGetLastError();
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(t), dim3(256), 0, s, a);
+  return launch_status();
+}
+
 }  // namespace
 
 extern "C" {
@@ -978,6 +1098,27 @@ int mi355_w8a8_swiglu_bwd_v1(const void* fused, const void* d_product, void* d_f
 int mi355_w8a8_rms_norm_bwd_v1(const void* x, const float* gamma, const void* d_normalized, void* d_x, uint32_t m,
                                uint32_t k, float eps, void* stream) {
   return run_rms_norm_bwd(x, gamma, d_normalized, d_x, m, k, eps, static_cast<hipStream_t>(stream));
+}
+
+int mi355_w8a8_moe_route_v1(const float* router_logits, uint32_t n_tokens, uint32_t n_experts, uint32_t top_k,
+                            uint32_t norm_topk_prob, float* weights, int32_t* selected, void* stream) {
+  return run_moe_route(router_logits, n_tokens, n_experts, top_k, norm_topk_prob, weights, selected,
+                       static_cast<hipStream_t>(stream));
+}
+
+uint64_t mi355_w8a8_moe_dispatch_workspace_bytes(uint32_t n_pairs, uint32_t n_groups) {
+  if (validate_moe_sort_dims(n_pairs, n_groups)) return 0;
+  return make_moe_sort_layout(n_pairs, n_groups).total;
+}
+
+int mi355_w8a8_moe_dispatch_v1(const mi355_w8a8_moe_dispatch_problem* p, void* stream) {
+  return run_moe_dispatch(p, static_cast<hipStream_t>(stream));
+}
+
+int mi355_w8a8_moe_combine_v1(const void* expert_out, const int32_t* unsort_indices, const float* weights, void* out,
+                              uint32_t n_tokens, uint32_t top_k, uint32_t width, void* stream) {
+  return run_moe_combine(expert_out, unsort_indices, weights, out, n_tokens, top_k, width,
+                         static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

@@ -862,28 +862,134 @@ def w8a8_grouped_lora_linear(x, group_sizes, weight, lora_a=None, lora_b=None, l
                            groups_per_weight=groups_per_weight)
 
 
+def moe_route(router_logits: torch.Tensor, top_k: int, norm_topk_prob: bool = True):
+    """softmax -> top-k -> renormalise (skyrl/tx/models/qwen3.py:175-178) in float32.  Returns
+    ``(weights f32 [T, top_k], selected int32 [T, top_k])``; ties pick the lower expert."""
+    _require_cuda(router_logits, "router_logits")
+    if router_logits.ndim != 2 or router_logits.shape[0] <= 0:
+        raise ValueError(f"router_logits must be [tokens, experts], got {tuple(router_logits.shape)}")
+    if isinstance(top_k, bool) or not isinstance(top_k, int) or not 1 <= top_k <= router_logits.shape[1]:
+        raise ValueError(f"top_k must be an integer in [1, {router_logits.shape[1]}], got {top_k!r}")
+    _validate_exact_bool("norm_topk_prob", norm_topk_prob)
+    logits = router_logits.detach().to(torch.float32).contiguous()
+    t, e = logits.shape
+    dev = logits.device
+    weights = torch.empty((t, top_k), dtype=torch.float32, device=dev)
+    selected = torch.empty((t, top_k), dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        status = _native.load().mi355_w8a8_moe_route_v1(logits.data_ptr(), t, e, top_k, int(norm_topk_prob),
+                                                        weights.data_ptr(), selected.data_ptr(), _stream_ptr(dev))
+    _native.check("mi355_w8a8_moe_route_v1", status)
+    return weights, selected
+
+
+def moe_dispatch(tokens: torch.Tensor | None, indices: torch.Tensor, num_groups: int, *, repeat: int = 1,
+                 adapter_indices: torch.Tensor | None = None):
+    """Stable sort of rows by group with the gather of their token rows, on the device and without a
+    host round trip.  Pair ``p`` reads token ``p // repeat`` (and its adapter index).  Returns
+    ``(sorted_tokens, group_sizes, sort_indices, unsort_indices, sorted_adapters)``."""
+    _require_cuda(indices, "indices")
+    dev = indices.device
+    idx = indices.reshape(-1).to(torch.int32).contiguous()
+    n_pairs = idx.numel()
+    if n_pairs <= 0:
+        raise ValueError("indices must not be empty")
+    if isinstance(repeat, bool) or not isinstance(repeat, int) or repeat < 1 or n_pairs % repeat:
+        raise ValueError(f"repeat must be a positive integer dividing {n_pairs} rows, got {repeat!r}")
+    if isinstance(num_groups, bool) or not isinstance(num_groups, int) or num_groups < 1:
+        raise ValueError(f"num_groups must be a positive integer, got {num_groups!r}")
+    lib = _native.load()
+    ws_bytes = int(lib.mi355_w8a8_moe_dispatch_workspace_bytes(n_pairs, num_groups))
+    if ws_bytes == 0:
+        raise ValueError(f"{n_pairs} rows in {num_groups} groups are outside the native dispatch")
+    tok = sorted_tokens = None
+    width = 0
+    if tokens is not None:
+        if tokens.dtype != torch.bfloat16:
+            raise TypeError(f"tokens must be BF16, got {tokens.dtype}")
+        _require_cuda(tokens, "tokens")
+        if tokens.ndim != 2 or tokens.shape[0] * repeat != n_pairs or tokens.shape[1] % 8:
+            raise ValueError(f"tokens must be [{n_pairs // repeat}, width] with width % 8 == 0, got "
+                             f"{tuple(tokens.shape)}")
+        tok = tokens.contiguous()
+        width = tok.shape[1]
+        sorted_tokens = torch.empty((n_pairs, width), dtype=torch.bfloat16, device=dev)
+    ad = sorted_adapters = None
+    if adapter_indices is not None:
+        ad = adapter_indices.reshape(-1).to(device=dev, dtype=torch.int32).contiguous()
+        if ad.numel() * repeat != n_pairs:
+            raise ValueError(f"adapter_indices must have {n_pairs // repeat} entries, got {ad.numel()}")
+        sorted_adapters = torch.empty(n_pairs, dtype=torch.int32, device=dev)
+    group_sizes = torch.empty(num_groups, dtype=torch.int32, device=dev)
+    sort_indices = torch.empty(n_pairs, dtype=torch.int32, device=dev)
+    unsort_indices = torch.empty(n_pairs, dtype=torch.int32, device=dev)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    p = _native.MoeDispatchProblem()
+    p.struct_size = ctypes.sizeof(_native.MoeDispatchProblem)
+    p.n_pairs, p.repeat, p.width, p.n_groups = n_pairs, repeat, width, num_groups
+    p.tokens = tok.data_ptr() if tok is not None else None
+    p.indices = idx.data_ptr()
+    p.adapter_indices = ad.data_ptr() if ad is not None else None
+    p.sorted_tokens = sorted_tokens.data_ptr() if tok is not None else None
+    p.group_sizes = group_sizes.data_ptr()
+    p.sort_indices = sort_indices.data_ptr()
+    p.unsort_indices = unsort_indices.data_ptr()
+    p.sorted_adapters = sorted_adapters.data_ptr() if ad is not None else None
+    p.workspace = ws.data_ptr()
+    p.workspace_bytes = ws_bytes
+    with torch.cuda.device(dev):
+        status = lib.mi355_w8a8_moe_dispatch_v1(ctypes.byref(p), _stream_ptr(dev))
+    _native.check("mi355_w8a8_moe_dispatch_v1", status)
+    return sorted_tokens, group_sizes, sort_indices, unsort_indices, sorted_adapters
+
+
+def prepare_routing(tokens: torch.Tensor, indices: torch.Tensor, num_groups: int,
+                    adapter_indices: torch.Tensor | None = None):
+    """``prepare_routing`` of skyrl/tx/layers/util.py:66-87, same arguments and results
+    ``(sorted_tokens, group_sizes, unsort_indices, sorted_adapter_indices)``, on the native sort."""
+    sorted_tokens, group_sizes, _, unsort, sorted_adapters = moe_dispatch(tokens, indices, num_groups,
+                                                                          adapter_indices=adapter_indices)
+    return sorted_tokens, group_sizes, unsort, sorted_adapters
+
+
+def moe_combine(expert_out: torch.Tensor, unsort_indices: torch.Tensor, weights: torch.Tensor) -> torch.Tensor:
+    """``sum_j expert_out[unsort[t * top_k + j]] * weights[t, j]`` in float32, one bf16 cast
+    (qwen3.py:205-207).  ``expert_out`` bf16 [T * top_k, H], ``weights`` f32 [T, top_k]."""
+    if expert_out.dtype != torch.bfloat16:
+        raise TypeError(f"expert_out must be BF16, got {expert_out.dtype}")
+    _require_cuda(expert_out, "expert_out")
+    if weights.ndim != 2 or expert_out.ndim != 2 or expert_out.shape[0] != weights.numel() or expert_out.shape[1] % 8:
+        raise ValueError(f"need expert_out [T * top_k, H] with H % 8 == 0 and weights [T, top_k], got "
+                         f"{tuple(expert_out.shape)} and {tuple(weights.shape)}")
+    if unsort_indices.numel() != weights.numel():
+        raise ValueError("unsort_indices must have one entry per (token, choice)")
+    dev = expert_out.device
+    t, top_k = weights.shape
+    eo = expert_out.contiguous()
+    un = unsort_indices.reshape(-1).to(device=dev, dtype=torch.int32).contiguous()
+    w = weights.detach().to(device=dev, dtype=torch.float32).contiguous()
+    out = torch.empty((t, eo.shape[1]), dtype=torch.bfloat16, device=dev)
+    with torch.cuda.device(dev):
+        status = _native.load().mi355_w8a8_moe_combine_v1(eo.data_ptr(), un.data_ptr(), w.data_ptr(), out.data_ptr(),
+                                                          t, top_k, eo.shape[1], _stream_ptr(dev))
+    _native.check("mi355_w8a8_moe_combine_v1", status)
+    return out
+
+
 def w8a8_moe_expert_mlp(hidden, router_logits, top_k: int, gate_up_weight, down_weight, gate_up_a, gate_up_b,
                         down_a, down_b, lora_scaling, *, enabled: bool = False, norm_topk_prob: bool = True):
     """Expert MLP of ``Qwen3Experts.__call__`` (skyrl/tx/models/qwen3.py:172-210) on W8A8 weights:
     softmax -> top-k -> renormalise -> sort rows by expert -> grouped gate/up + SwiGLU -> grouped
-    down -> unsort -> weighted sum.  Routing and the final combine are torch glue; the two
-    grouped GEMMs are the HIP kernels."""
+    down -> unsort -> weighted sum.  Five native calls on one stream, no host round trip: route,
+    dispatch, the two grouped GEMMs, combine."""
     _check_enabled(enabled, False, "MoE expert MLP")
     n_experts = gate_up_weight.n_weights
-    probs = torch.softmax(router_logits.to(torch.float32), dim=-1)
-    weights, selected = torch.topk(probs, top_k, dim=-1)
-    if norm_topk_prob:
-        weights = weights / weights.sum(dim=-1, keepdim=True)
-    flat_experts = selected.reshape(-1)
-    order = torch.sort(flat_experts, stable=True).indices
-    x_sorted = hidden.repeat_interleave(top_k, dim=0)[order]
-    group_sizes = torch.bincount(flat_experts, minlength=n_experts).to(torch.int32)
+    weights, selected = moe_route(router_logits, top_k, norm_topk_prob)
+    x_sorted, group_sizes, _, unsort, _ = moe_dispatch(hidden.reshape(-1, hidden.shape[-1]), selected, n_experts,
+                                                       repeat=top_k)
     act = grouped_forward(x_sorted, group_sizes, gate_up_weight, gate_up_a, gate_up_b, lora_scaling, swiglu=True)
     down = grouped_forward(act, group_sizes, down_weight, down_a, down_b, lora_scaling)
-    unsort = torch.empty_like(order)
-    unsort[order] = torch.arange(order.numel(), device=order.device)
-    per_tok = down[unsort].reshape(hidden.shape[0], top_k, -1).to(torch.float32)
-    return (per_tok * weights[..., None]).sum(dim=1).to(torch.bfloat16)
+    return moe_combine(down, unsort, weights)
 
 
 def _check_enabled(enabled, interpret, what: str) -> None:
