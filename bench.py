@@ -49,6 +49,10 @@ WORKLOADS = {
     # token routing around the expert GEMMs at the Qwen3-30B-A3B geometry: softmax / top-8 of 128 experts,
     # stable sort of the 32768 (token, choice) pairs with the gather of their rows, weighted combine
     "qwen3-30b-a3b-moe-routing-t4096": dict(m=4096, n_experts=128, top_k=8, hidden=2048, seed=6, moe_routing=True),
+    # the whole expert MLP of BASELINE config 5 (T = 2048): route, dispatch, grouped gate/up + SwiGLU, grouped down,
+    # combine; rank-16 LoRA on every expert
+    "qwen3-30b-a3b-moe-mlp-t2048": dict(m=2048, n_experts=128, top_k=8, hidden=2048, intermediate=768, rank=16,
+                                        seed=5, moe_mlp=True),
     # Qwen3.5-4B attention input stage: RMSNorm -> W8A8 QKV [2560 -> 10240] + 4 adapters rank 64 ->
     # split, Q/K RMSNorm, partial RoPE (16 query heads, 4 kv heads, head_dim 256, 64 rotary dims)
     "qwen3.5-4b-qkv-m2048": dict(m=2048, k=2560, n=10240, n_adapters=4, rank=64, alpha=128, rms=True,
@@ -403,6 +407,98 @@ def bench_moe_routing(args, cfg, pkg, dev):
     return 0
 
 
+def bench_moe_mlp(args, cfg, pkg, dev):
+    """One step = the whole expert MLP: route, dispatch (indices only), grouped gate/up + SwiGLU
+    (reading the hidden rows through the sort order), grouped down, combine.  ``value`` counts the
+    integer GEMM work 2 * T * top_k * (H * 2I + I * H); the roofline prices the grouped gate/up call
+    (its GEMM kernel dominates) against int8 MFMA peak from HIP events around that call."""
+    import torch
+
+    from oracle import w8a8_oracle as o
+
+    w8 = pkg.w8a8_lora
+    t, e, k, h, inter, r = cfg["m"], cfg["n_experts"], cfg["top_k"], cfg["hidden"], cfg["intermediate"], cfg["rank"]
+    rng = np.random.default_rng(cfg["seed"])
+    hidden = o.bf16_round(rng.standard_normal((t, h)).astype(np.float32))
+    logits = rng.standard_normal((t, e)).astype(np.float32)
+    gu_codes = rng.integers(-127, 128, (e, h, 2 * inter), dtype=np.int8)
+    gu_scales = rng.uniform(0.001, 0.01, (e, 2 * inter)).astype(np.float32)
+    dn_codes = rng.integers(-127, 128, (e, inter, h), dtype=np.int8)
+    dn_scales = rng.uniform(0.001, 0.01, (e, h)).astype(np.float32)
+    mk = lambda shape: o.bf16_round((rng.standard_normal(shape) * 0.02).astype(np.float32))
+    gua, gub, da, db = mk((e, h, r)), mk((e, r, 2 * inter)), mk((e, inter, r)), mk((e, r, h))
+    bf = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev).to(torch.bfloat16)
+    guw = w8.prepare_grouped_weight(torch.from_numpy(gu_codes).to(dev), torch.from_numpy(gu_scales).to(dev))
+    dnw = w8.prepare_grouped_weight(torch.from_numpy(dn_codes).to(dev), torch.from_numpy(dn_scales).to(dev))
+    hidden_t, logits_t = bf(hidden), torch.from_numpy(logits).to(dev)
+    gua_t, gub_t, da_t, db_t = bf(gua), bf(gub), bf(da), bf(db)
+
+    def step():
+        return w8.w8a8_moe_expert_mlp(hidden_t, logits_t, k, guw, dnw, gua_t, gub_t, da_t, db_t, 1.0, enabled=True)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        got = step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    p = t * k
+    ops = 2.0 * p * (h * 2 * inter + inter * h)
+
+    def timed(fn):
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        for a, b in ev:
+            a.record()
+            fn()
+            b.record()
+        torch.cuda.synchronize()
+        return float(np.mean([a.elapsed_time(b) for a, b in ev]))
+
+    weights, selected = w8.moe_route(logits_t, k)
+    _, sizes, sort_i, unsort, _ = w8.moe_dispatch(None, selected, e, repeat=k)
+    act = w8.grouped_forward(hidden_t, sizes, guw, gua_t, gub_t, 1.0, swiglu=True, row_map=sort_i, row_repeat=k)
+    down = w8.grouped_forward(act, sizes, dnw, da_t, db_t, 1.0)
+    stages = {
+        "route_ms": timed(lambda: w8.moe_route(logits_t, k)),
+        "dispatch_ms": timed(lambda: w8.moe_dispatch(None, selected, e, repeat=k)),
+        "gate_up_ms": timed(lambda: w8.grouped_forward(hidden_t, sizes, guw, gua_t, gub_t, 1.0, swiglu=True,
+                                                       row_map=sort_i, row_repeat=k)),
+        "down_ms": timed(lambda: w8.grouped_forward(act, sizes, dnw, da_t, db_t, 1.0)),
+        "combine_ms": timed(lambda: w8.moe_combine(down, unsort, weights)),
+    }
+    gu_ops = 2.0 * p * h * 2 * inter
+    achieved = gu_ops / (stages["gate_up_ms"] * 1e-3) / 1e12
+    result = {
+        "metric": "grouped W8A8-LoRA expert MLP (route, dispatch, gate/up + SwiGLU, down, combine), TOPS of the integer GEMM work",
+        "value": ops / (ms_per_step * 1e-3) / 1e12, "unit": "TOPS", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                     "frac": achieved / INT8_PEAK_TOPS, "traffic": None,
+                     "kernel": "the grouped gate/up call (route_groups, quant_rows, lora_prep, lora_a, w8a8_gemm_kernel "
+                               "in grouped mode)",
+                     "kernel_avg_ms": stages["gate_up_ms"], "algorithmic_ops": gu_ops},
+        "stages": stages,
+    }
+    if not args.no_cpu_baseline:
+        rows = args.cpu_rows or 64
+        gu = [o.GroupQuantizedWeight(gu_codes[i], gu_scales[i:i + 1], h, h, 8, h) for i in range(e)]
+        dn = [o.GroupQuantizedWeight(dn_codes[i], dn_scales[i:i + 1], inter, inter, 8, inter) for i in range(e)]
+        t1 = time.perf_counter()
+        want = o.moe_expert_mlp(hidden[:rows], logits[:rows], k, gu, dn, gua, gub, da, db, np.float32(1.0))
+        secs = time.perf_counter() - t1
+        result["cpu_baseline"] = {"value": ops * rows / t / secs / 1e12, "unit": "TOPS", "cores": 1, "kind": "port",
+                                  "sample": f"first {rows} of {t} tokens (tokens are independent), all experts, NumPy "
+                                            f"oracle expert MLP, one run, {secs:.3f} s", "seconds": secs}
+        gate = o.numerical_gate(got[:rows].to(torch.float32).cpu().numpy(), want)
+        result["parity_sample"] = {"tokens": rows, "relative_l2": gate["relative_l2"], "cosine": gate["cosine"]}
+    print(json.dumps(result))
+    return 0
+
+
 def bench_qkv(args, cfg, pkg, dev):
     """One step = the W8A8 QKV projection (RMSNorm prologue, GEMM, LoRA) + the split / Q-K norm /
     RoPE kernel.  ``value`` is int8 TOPS of the projection over the whole step; the roofline prices
@@ -533,6 +629,8 @@ def main() -> int:
         if cfg.get("swiglu"):
             return bench_fused_backward(args, cfg, pkg, dev)
         return bench_backward(args, cfg, pkg, dev)
+    if cfg.pop("moe_mlp", False):
+        return bench_moe_mlp(args, cfg, pkg, dev)
     if cfg.pop("moe_routing", False):
         return bench_moe_routing(args, cfg, pkg, dev)
     if "qkv" in cfg:

@@ -68,6 +68,10 @@ typedef enum mi355_w8a8_status {
 /* tile geometry of the tiled GEMM; default: 256 x 256 once such tiles fill the chip, else 256 x 128 */
 #define MI355_W8A8_FLAG_TILE_256X128 64u
 #define MI355_W8A8_FLAG_TILE_256X256 128u
+/* tile rows of the grouped call (and the slots every group is padded to); default: 128 once the
+ * groups average at least 96 rows, else 64.  Pass the same flags to the workspace query. */
+#define MI355_W8A8_FLAG_GROUPED_TILE64 256u
+#define MI355_W8A8_FLAG_GROUPED_TILE128 512u
 
 /*
  * One forward call.  y = dequant(quant(n) @ W) + s[idx] * ((n @ A[idx]) @ B[idx]) (+ residual),
@@ -107,7 +111,7 @@ typedef struct mi355_w8a8_problem {
  */
 typedef struct mi355_w8a8_grouped_problem {
   uint32_t struct_size;     /* sizeof(mi355_w8a8_grouped_problem) */
-  uint32_t flags;           /* MI355_W8A8_FLAG_SWIGLU allowed */
+  uint32_t flags;           /* MI355_W8A8_FLAG_SWIGLU, _GROUPED_TILE64 / _GROUPED_TILE128 allowed */
   uint32_t m;               /* total rows */
   uint32_t k;
   uint32_t n;
@@ -128,6 +132,14 @@ typedef struct mi355_w8a8_grouped_problem {
   int8_t* aux_x_codes;
   float* aux_x_scales;
   int32_t* aux_acc;         /* int32 [m, n]; rows beyond sum(group_sizes) are not written */
+  /* Optional gather on the way in (NULL: row i of the call is row i of x).  With a map, row i is
+   * read from x[x_row_map[i] / x_row_repeat] and x holds one row per token: passing the
+   * sort_indices of mi355_w8a8_moe_dispatch_v1 and repeat = top_k lets the first expert projection
+   * read the unsorted hidden states, and the dispatch can skip the row copies.  Map values must lie
+   * in [0, rows of x * x_row_repeat); they are not checked. */
+  const int32_t* x_row_map; /* int32 [m] or NULL */
+  uint32_t x_row_repeat;    /* >= 1 with a map */
+  uint32_t reserved;
 } mi355_w8a8_grouped_problem;
 
 /*

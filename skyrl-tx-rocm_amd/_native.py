@@ -21,6 +21,8 @@ FLAG_SKIP_PROLOGUE = 16
 FLAG_SKIP_GEMM = 32
 FLAG_TILE_256X128 = 64
 FLAG_TILE_256X256 = 128
+FLAG_GROUPED_TILE64 = 256
+FLAG_GROUPED_TILE128 = 512
 
 STATUS = {
     0: "OK", -1: "ERR_NULL", -2: "ERR_SHAPE", -3: "ERR_ALIGN", -4: "ERR_ALIAS",
@@ -65,6 +67,7 @@ class GroupedProblem(ctypes.Structure):
         ("x", _vp), ("w_packed", _vp), ("w_scales", _vp), ("lora_a", _vp), ("lora_b", _vp),
         ("lora_scaling", _vp), ("group_sizes", _vp), ("out", _vp), ("workspace", _vp),
         ("workspace_bytes", _u64), ("aux_x_codes", _vp), ("aux_x_scales", _vp), ("aux_acc", _vp),
+        ("x_row_map", _vp), ("x_row_repeat", _u32), ("reserved", _u32),
     ]
 
 

@@ -32,6 +32,17 @@ struct WsLayout {
 // number of 16-wide rank chunks the kernels are instantiated for (rank padded with zeros)
 inline uint32_t rank_chunks(uint32_t rank) { return rank == 0 ? 0u : (rank <= 16u ? 1u : (rank <= 32u ? 2u : 4u)); }
 
+// Between the skinny-M limit and this many rows a call without SwiGLU may run the skinny-M kernels
+// on chunks of 32 rows: the weight is streamed once per chunk (the later passes from the last-level
+// cache), which beats the handful of 256-row tiles such a call would give the tiled kernel.
+// Measured on 2560 x 6144, 4096 x 2560, 12288 x 4096 and 4096 x 24576 weights: two chunks always
+// win while the weight stays in the caches (<= 64 MB), four chunks win from K = 4096 on.
+constexpr uint32_t kSkinnyChunkedMaxRows = 128;
+inline bool skinny_chunked_pays(uint32_t m, uint32_t k, uint32_t n) {
+  if (m > kSkinnyChunkedMaxRows || (uint64_t)k_padded(k) * n_padded(n) > (64ull << 20)) return false;
+  return m <= 64u || k >= 4096u;
+}
+
 WsLayout make_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint32_t rank, bool routed) {
   WsLayout w{};
   w.K_pad = k_padded(k);
@@ -50,7 +61,8 @@ WsLayout make_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint
   w.blk_range = off; off += align256((uint64_t)(w.slots / 32u) * 4u);
   w.tile_ctr = off; off += 1024u;  // two sets of eight counters, 64 bytes apart
   // normalized rows: only the decode path keeps them in memory (RMSNorm + LoRA, M <= 32)
-  w.xn = off; off += (rank && m <= (uint32_t)kSkinnyMaxRows) ? align256((uint64_t)m * k * 2u) : 0u;
+  w.xn = off;
+  off += (rank && m <= kSkinnyChunkedMaxRows) ? align256((uint64_t)(m < 32u ? m : 32u) * k * 2u) : 0u;
   w.zp = off; off += rank ? align256((uint64_t)(w.slots / 32u) * w.nkk * 3u * kBlockBytes) : 0u;
   w.at = off; off += rank ? align256((uint64_t)n_groups * rank * k * 2u) : 0u;
   w.bp = off; off += rank ? align256((uint64_t)n_groups * (n_padded(n) / 32u) * w.nkk * kBlockBytes) : 0u;
@@ -91,11 +103,12 @@ int launch_gemm_one(const GemmArgs& g, hipStream_t s) {
   { const char* e = getenv("MI355_W8A8_GRID"); if (e && atoi(e) > 0) slots = ((uint32_t)atoi(e) + 7u) / 8u * 8u; }
 #endif
   const uint32_t want = ((ntile + 7u) / 8u) * 8u;
-  const dim3 grid(want < slots ? want : slots), block(MODE == kModeWide ? 512 : 256);
+  const dim3 grid(want < slots ? want : slots), block((MODE == kModeWide || MODE == kModeGrouped128) ? 512 : 256);
   constexpr uint32_t lds_bytes =
-      MODE == kModeGrouped ? kGroupedLdsBytes : (MODE == kModeWide ? kWideLdsBytes : kGemmLdsBytes);
+      MODE == kModeGrouped128 ? kGrouped128LdsBytes
+                              : (MODE == kModeGrouped ? kGroupedLdsBytes : (MODE == kModeWide ? kWideLdsBytes : kGemmLdsBytes));
 #ifdef W8A8_DEBUG_VARIANTS
-  if constexpr (EPI == kEpiSwiglu && NKK == 2 && MODE != kModeGrouped) {
+  if constexpr (EPI == kEpiSwiglu && NKK == 2 && MODE != kModeGrouped && MODE != kModeGrouped128) {
 #define W8A8_DBG(D)                                                                              \
   if (g.map_mode == 100 + D) {                                                                   \
     hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm_kernel<EPI, NKK, D, MODE>),    \
@@ -136,7 +149,7 @@ int validate_common(uint32_t m, uint32_t k, uint32_t n) {
 
 // Skinny-M path: quantize -> stream (weight + LoRA-A units) -> epilogue.
 int launch_skinny(const mi355_w8a8_problem* p, unsigned char* xq, float* sx, uint16_t* xn, unsigned char* sws,
-                  uint32_t K_pad, uint32_t KB, hipStream_t s) {
+                  uint32_t K_pad, uint32_t KB, hipStream_t s, bool allow_regroup = true) {
   const bool rms = p->rms_gamma != nullptr;
   const bool lora = p->n_adapters > 0;
   const SkinnyLayout L = skinny_layout(p->m, p->k, p->n, p->rank);
@@ -157,7 +170,7 @@ int launch_skinny(const mi355_w8a8_problem* p, unsigned char* xq, float* sx, uin
     q.z_part = reinterpret_cast<float*>(sws + L.z_part);
     q.n_adapters = p->n_adapters; q.r = p->rank; q.z_chunks = L.z_chunks; q.z_chunk_k = L.z_chunk_k;
     q.n_z_units = (lora && !rms) ? p->m * L.z_chunks : 0u;
-    const bool regroup = lora && p->rank <= 32u && p->m <= 16u && (p->n % 8u) == 0;
+    const bool regroup = allow_regroup && lora && p->rank <= 32u && p->m <= 16u && (p->n % 8u) == 0;
     q.lora_b = regroup ? static_cast<const uint16_t*>(p->lora_b) : nullptr;
     q.bsel = reinterpret_cast<uint16_t*>(sws + L.bsel);
     q.N = p->n; q.n_groups = n_padded(p->n) / 128u;
@@ -183,7 +196,8 @@ int launch_skinny(const mi355_w8a8_problem* p, unsigned char* xq, float* sx, uin
   a.z_part = reinterpret_cast<const float*>(sws + L.z_part);
   a.sx = sx; a.sw = p->w_scales;
   a.lora_b = lora ? static_cast<const uint16_t*>(p->lora_b) : nullptr;
-  a.bsel = (lora && p->rank <= 32u && p->m <= 16u && (p->n % 8u) == 0) ? reinterpret_cast<const uint16_t*>(sws + L.bsel) : nullptr;
+  a.bsel = (allow_regroup && lora && p->rank <= 32u && p->m <= 16u && (p->n % 8u) == 0)
+               ? reinterpret_cast<const uint16_t*>(sws + L.bsel) : nullptr;
   a.lora_scaling = p->lora_scaling; a.idx = p->adapter_indices;
   a.row_scaling = reinterpret_cast<const float*>(sws + L.row_scaling);
   a.residual = static_cast<const uint16_t*>(p->residual);
@@ -265,6 +279,28 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   if (skinny) {
     return launch_skinny(p, ws + w.xq, reinterpret_cast<float*>(ws + w.sx),
                          reinterpret_cast<uint16_t*>(ws + w.xn), ws + w.skinny, w.K_pad, w.KB, s);
+  }
+  if (skinny_supported() && !swiglu && skinny_chunked_pays(p->m, p->k, p->n) &&
+      !(p->flags & (MI355_W8A8_FLAG_FORCE_TILED | MI355_W8A8_FLAG_SKIP_PROLOGUE | MI355_W8A8_FLAG_SKIP_GEMM |
+                    MI355_W8A8_FLAG_TILE_256X128 | MI355_W8A8_FLAG_TILE_256X256))) {
+    for (uint32_t row0 = 0; row0 < p->m; row0 += (uint32_t)kSkinnyMaxRows) {
+      mi355_w8a8_problem sub = *p;
+      sub.m = p->m - row0 < (uint32_t)kSkinnyMaxRows ? p->m - row0 : (uint32_t)kSkinnyMaxRows;
+      sub.x = static_cast<const unsigned char*>(p->x) + (size_t)row0 * p->k * 2u;
+      sub.out = static_cast<unsigned char*>(p->out) + (size_t)row0 * p->n * 2u;
+      if (p->residual) sub.residual = static_cast<const unsigned char*>(p->residual) + (size_t)row0 * p->n * 2u;
+      if (p->adapter_indices) sub.adapter_indices = p->adapter_indices + row0;
+      if (p->aux_x_codes) sub.aux_x_codes = p->aux_x_codes + (size_t)row0 * p->k;
+      if (p->aux_x_scales) sub.aux_x_scales = p->aux_x_scales + row0;
+      if (p->aux_acc) sub.aux_acc = p->aux_acc + (size_t)row0 * p->n;
+      if (p->aux_normalized)
+        sub.aux_normalized = static_cast<unsigned char*>(p->aux_normalized) + (size_t)row0 * p->k * 2u;
+      // the chunks share the workspace: they run one after the other on the stream
+      if ((st = launch_skinny(&sub, ws + w.xq, reinterpret_cast<float*>(ws + w.sx),
+                              reinterpret_cast<uint16_t*>(ws + w.xn), ws + w.skinny, w.K_pad, w.KB, s, false)))
+        return st;
+    }
+    return MI355_W8A8_OK;
   }
 
   const bool skip_prologue = (p->flags & MI355_W8A8_FLAG_SKIP_PROLOGUE) != 0;
@@ -372,16 +408,26 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
 
 struct GroupedLayout {
   uint64_t xq, sx, zp, at, bp, src_row, dst_pos, blk_range, total;
-  uint32_t slots, nkk, K_pad, KB, n_steps, steps_per_wave;
+  uint32_t slots, nkk, K_pad, KB, n_steps, steps_per_wave, pad;
 };
 
-GroupedLayout make_grouped_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint32_t rank) {
+// Rows of padding per group = rows of a GEMM tile: 128 once the groups average at least 96 rows (the
+// weight panel then travels L2 -> LDS once per 128 rows), else 64; the flags force either.
+uint32_t grouped_pad(uint32_t m, uint32_t n_groups, uint32_t flags) {
+  if (flags & MI355_W8A8_FLAG_GROUPED_TILE64) return 64u;
+  if (flags & MI355_W8A8_FLAG_GROUPED_TILE128) return 128u;
+  return (uint64_t)m >= 96ull * n_groups ? 128u : 64u;
+}
+
+GroupedLayout make_grouped_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint32_t rank,
+                                  uint32_t flags) {
   GroupedLayout w{};
   w.K_pad = k_padded(k);
   w.KB = w.K_pad / 32u;
-  // every group is padded to 64 slots: at most 63 padding slots per group
-  const uint64_t worst = (uint64_t)m + 63ull * n_groups;
-  w.slots = (uint32_t)((worst + 63ull) / 64ull * 64ull);
+  w.pad = grouped_pad(m, n_groups, flags);
+  // every group is padded to a multiple of pad slots: at most pad - 1 padding slots per group
+  const uint64_t worst = (uint64_t)m + (uint64_t)(w.pad - 1u) * n_groups;
+  w.slots = (uint32_t)((worst + w.pad - 1u) / w.pad * w.pad);
   w.nkk = rank_chunks(rank);
   w.n_steps = (k + 63u) / 64u;
   w.steps_per_wave = (w.n_steps + 15u) / 16u;
@@ -420,10 +466,18 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
   if (!aligned16(p->x) || !aligned16(p->w_packed) || !aligned16(p->out) || !aligned16(p->w_scales) ||
       !aligned16(p->lora_a) || !aligned16(p->lora_b) || (reinterpret_cast<uintptr_t>(p->group_sizes) & 3u))
     return MI355_W8A8_ERR_ALIGN;
-  if (overlaps(p->out, out_bytes, p->x, (uint64_t)p->m * p->k * 2u) ||
+  const uint32_t x_repeat = p->x_row_map ? p->x_row_repeat : 1u;
+  if (p->x_row_map && (x_repeat == 0 || (reinterpret_cast<uintptr_t>(p->x_row_map) & 3u)))
+    return x_repeat == 0 ? MI355_W8A8_ERR_SHAPE : MI355_W8A8_ERR_ALIGN;
+  // with a row map x holds one row per token: at least ceil(m / repeat) of them
+  const uint64_t x_rows = ((uint64_t)p->m + x_repeat - 1u) / x_repeat;
+  if (overlaps(p->out, out_bytes, p->x, x_rows * p->k * 2u) ||
+      overlaps(p->out, out_bytes, p->x_row_map, (uint64_t)p->m * 4u) ||
       overlaps(p->out, out_bytes, p->workspace, p->workspace_bytes))
     return MI355_W8A8_ERR_ALIAS;
-  const GroupedLayout w = make_grouped_layout(p->m, p->k, p->n, p->n_groups, p->rank);
+  if ((p->flags & MI355_W8A8_FLAG_GROUPED_TILE64) && (p->flags & MI355_W8A8_FLAG_GROUPED_TILE128))
+    return MI355_W8A8_ERR_SHAPE;
+  const GroupedLayout w = make_grouped_layout(p->m, p->k, p->n, p->n_groups, p->rank, p->flags);
   if (!p->workspace || p->workspace_bytes < w.total) return MI355_W8A8_ERR_WORKSPACE;
   if (reinterpret_cast<uintptr_t>(p->workspace) & 255u) return MI355_W8A8_ERR_ALIGN;
   unsigned char* ws = static_cast<unsigned char*>(p->workspace);
@@ -432,10 +486,31 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
   int32_t* blk_range = reinterpret_cast<int32_t*>(ws + w.blk_range);
   (void)hipGetLastError();
 
-  hipLaunchKernelGGL(route_groups_kernel, dim3(1), dim3(1024), 0, s, p->group_sizes, p->m, p->n_groups, w.slots,
-                     src_row, dst_pos, blk_range);
-  if ((st = launch_status())) return st;
+  // launch 1: the slot layout of the groups (one block) next to the LoRA operand re-layouts
+  {
+    LoraPrepArgs pa{};
+    pa.src_row = src_row; pa.dst_pos = dst_pos; pa.blk_range = blk_range;
+    pa.group_sizes = p->group_sizes; pa.group_pad = w.pad;
+    pa.lora_a = static_cast<const uint16_t*>(p->lora_a);
+    pa.lora_b = static_cast<const uint16_t*>(p->lora_b);
+    pa.at = reinterpret_cast<uint16_t*>(ws + w.at);
+    pa.bp = ws + w.bp;
+    pa.M = p->m; pa.K = p->k; pa.N = p->n; pa.n_groups = p->n_groups; pa.r = p->rank; pa.nkk = w.nkk;
+    pa.ncb = n_padded(p->n) / 32u; pa.slots = w.slots;
+    pa.route_blocks = 1;
+    uint32_t b_blocks = 0;
+    if (lora) {
+      const uint64_t a_items = (uint64_t)p->n_groups * p->k * ((p->rank + 7u) / 8u);
+      const uint64_t b_items = (uint64_t)p->n_groups * pa.ncb * w.nkk * 64u;
+      pa.a_blocks = (uint32_t)((a_items + 1023u) / 1024u);
+      b_blocks = (uint32_t)((b_items + 1023u) / 1024u);
+    }
+    hipLaunchKernelGGL(lora_prep_kernel, dim3(1u + pa.a_blocks + b_blocks), dim3(1024), 0, s, pa);
+    if ((st = launch_status())) return st;
+  }
 
+  // launch 2: the quantizer, a wave per row (measured faster here than the fused quantizer + LoRA-A
+  // kernel of the dense path, whose 16-slot workgroups are sized for longer rows)
   QuantArgs q{};
   q.x = static_cast<const uint16_t*>(p->x);
   q.M = p->m; q.K = p->k; q.K_pad = w.K_pad; q.KB = w.KB;
@@ -446,32 +521,18 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
   q.scales_rm = p->aux_x_scales;
   q.zero_out = static_cast<uint16_t*>(p->out);
   q.zero_cols = n_out;
+  q.row_map = p->x_row_map; q.row_div = x_repeat;
   if ((st = launch_quant<false>(q, s))) return st;
 
+  // launch 3: LoRA-A projection per 32-slot block
   if (lora) {
-    uint16_t* at = reinterpret_cast<uint16_t*>(ws + w.at);
-    {
-      LoraPrepArgs pa{};
-      pa.lora_a = static_cast<const uint16_t*>(p->lora_a);
-      pa.lora_b = static_cast<const uint16_t*>(p->lora_b);
-      pa.at = at;
-      pa.bp = ws + w.bp;
-      pa.M = p->m; pa.K = p->k; pa.N = p->n; pa.n_groups = p->n_groups; pa.r = p->rank; pa.nkk = w.nkk;
-      pa.ncb = n_padded(p->n) / 32u; pa.slots = w.slots;
-      pa.route_blocks = 0;
-      const uint64_t a_items = (uint64_t)p->n_groups * p->k * ((p->rank + 7u) / 8u);
-      const uint64_t b_items = (uint64_t)p->n_groups * pa.ncb * w.nkk * 64u;
-      pa.a_blocks = (uint32_t)((a_items + 1023u) / 1024u);
-      const uint32_t b_blocks = (uint32_t)((b_items + 1023u) / 1024u);
-      hipLaunchKernelGGL(lora_prep_kernel, dim3(pa.a_blocks + b_blocks), dim3(1024), 0, s, pa);
-      if ((st = launch_status())) return st;
-    }
     LoraAArgs la{};
     la.xsrc = static_cast<const uint16_t*>(p->x);
-    la.at = at;
+    la.at = reinterpret_cast<const uint16_t*>(ws + w.at);
     la.src_row = src_row;
     la.slot_group = nullptr;
     la.blk_range = blk_range;
+    la.row_map = p->x_row_map; la.row_div = x_repeat;
     la.zp = ws + w.zp;
     la.M = p->m; la.K = p->k; la.r = p->rank; la.nkk = w.nkk;
     la.steps_per_wave = w.steps_per_wave; la.n_steps = w.n_steps;
@@ -499,7 +560,7 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
   g.w_group_stride = mi355_w8a8_packed_weight_bytes(p->k, p->n);
   g.M = p->m; g.N = p->n; g.K_pad = w.K_pad; g.KB = w.KB; g.slots = w.slots;
   g.total_rows = w.slots;
-  g.tiles_m = w.slots / kGroupedTileM;
+  g.tiles_m = w.slots / w.pad;
   g.tiles_n = (n_padded(p->n) + kGroupedTileN - 1u) / kGroupedTileN;
   g.rank = p->rank;
   g.map_mode = 1;  // row-tile-major order: column tiles of one expert run back to back
@@ -507,8 +568,13 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
   if (p->aux_acc) {
     GemmArgs ga = g;
     ga.out = p->aux_acc;
-    if ((st = launch_gemm<kEpiAcc, kModeGrouped>(ga, 0u, s))) return st;
+    if ((st = w.pad == 128u ? launch_gemm<kEpiAcc, kModeGrouped128>(ga, 0u, s)
+                            : launch_gemm<kEpiAcc, kModeGrouped>(ga, 0u, s)))
+      return st;
   }
+  if (w.pad == 128u)
+    return swiglu ? launch_gemm<kEpiSwiglu, kModeGrouped128>(g, w.nkk, s)
+                  : launch_gemm<kEpiPlain, kModeGrouped128>(g, w.nkk, s);
   return swiglu ? launch_gemm<kEpiSwiglu, kModeGrouped>(g, w.nkk, s) : launch_gemm<kEpiPlain, kModeGrouped>(g, w.nkk, s);
 }
 
@@ -1065,10 +1131,9 @@ int mi355_w8a8_forward_v1(const mi355_w8a8_problem* p, void* stream) {
 
 uint64_t mi355_w8a8_grouped_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint32_t rank,
                                             uint32_t flags) {
-  (void)flags;
   if (validate_common(m, k, n)) return 0;
   if (n_groups == 0 || n_groups > (uint32_t)kMaxGroups || rank > (uint32_t)kMaxRank) return 0;
-  return make_grouped_layout(m, k, n, n_groups, rank).total;
+  return make_grouped_layout(m, k, n, n_groups, rank, flags).total;
 }
 
 int mi355_w8a8_grouped_v1(const mi355_w8a8_grouped_problem* p, void* stream) {

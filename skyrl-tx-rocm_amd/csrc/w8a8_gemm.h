@@ -57,6 +57,12 @@ constexpr int kGroupedTileN = 512;
 constexpr int kGroupedStages = 4;
 constexpr int kGroupedStageBytes = 36864;  // A: 2 row blocks x 2 k blocks, B: 16 column blocks x 2 k blocks
 constexpr int kGroupedLdsBytes = kGroupedStages * kGroupedStageBytes;
+// grouped geometry for experts with many rows: 128 x 512 tile, 8 waves (2 x 4), the weight panel
+// travels L2 -> LDS once per 128 rows instead of once per 64
+constexpr int kGrouped128TileM = 128;
+constexpr int kGrouped128Stages = 3;
+constexpr int kGrouped128StageBytes = 40960;  // A: 4 row blocks x 2 k blocks, B: 16 column blocks x 2 k blocks
+constexpr int kGrouped128LdsBytes = kGrouped128Stages * kGrouped128StageBytes;
 
 // Third geometry, "wide": tile 256 x 256, eight waves (4 x 2, 64 x 128 each, two per SIMD), one
 // workgroup per CU, four 32 KiB stages.  It moves a third less L2 -> LDS traffic per MAC than
@@ -66,7 +72,7 @@ constexpr int kWideStages = 4;
 constexpr int kWideStageBytes = 32768;
 constexpr int kWideLdsBytes = kWideStages * kWideStageBytes;
 
-enum { kModeDense = 0, kModeGrouped = 1, kModeWide = 2 };
+enum { kModeDense = 0, kModeGrouped = 1, kModeWide = 2, kModeGrouped128 = 3 };
 
 // One tile of the persistent loop.
 struct GemmTile {
@@ -78,15 +84,17 @@ struct GemmTile {
 };
 
 template <int EPI, int NKK, int DBG = 0, int MODE = kModeDense>
-__global__ __launch_bounds__(MODE == kModeWide ? 512 : 256, MODE == kModeDense ? 2 : 1)
+__global__ __launch_bounds__((MODE == kModeWide || MODE == kModeGrouped128) ? 512 : 256, MODE == kModeDense ? 2 : 1)
 void w8a8_gemm_kernel(GemmArgs g) {
-  constexpr bool GROUPED = MODE == kModeGrouped;
+  constexpr bool G128 = MODE == kModeGrouped128;
+  constexpr bool GROUPED = MODE == kModeGrouped || G128;
   constexpr bool WIDE = MODE == kModeWide;
-  constexpr int kWaves = WIDE ? 8 : 4;
-  constexpr uint32_t kRowBlocks = GROUPED ? 2 : 8;                 // 32-row blocks of the activation panel
+  constexpr int kWaves = (WIDE || G128) ? 8 : 4;
+  constexpr uint32_t kRowBlocks = G128 ? 4 : (GROUPED ? 2 : 8);    // 32-row blocks of the activation panel
   constexpr uint32_t kColBlocks = GROUPED ? 16 : (WIDE ? 8 : 4);   // 32-column blocks of the weight panel
-  constexpr int kStages = GROUPED ? kGroupedStages : (WIDE ? kWideStages : kGemmStages);
-  constexpr int kStageBytes = GROUPED ? kGroupedStageBytes : (WIDE ? kWideStageBytes : kGemmStageBytes);
+  constexpr int kStages = G128 ? kGrouped128Stages : (GROUPED ? kGroupedStages : (WIDE ? kWideStages : kGemmStages));
+  constexpr int kStageBytes =
+      G128 ? kGrouped128StageBytes : (GROUPED ? kGroupedStageBytes : (WIDE ? kWideStageBytes : kGemmStageBytes));
   constexpr int kAChunks = kRowBlocks * 2;                              // 1 KiB chunks of A per stage
   constexpr int kLoadsPerTile = (kAChunks + kColBlocks * 2) / kWaves;   // direct-to-LDS loads per wave per k-tile
   constexpr bool kLora = (NKK > 0) && (EPI != kEpiAcc);
@@ -95,8 +103,8 @@ void w8a8_gemm_kernel(GemmArgs g) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wrow = GROUPED ? 0 : (WIDE ? (wave >> 1) : wave);  // wave position along M (64 rows each)
-  const int wcol = GROUPED ? wave : (WIDE ? (wave & 1) : 0);   // wave position along N (128 columns each)
+  const int wrow = G128 ? (wave >> 2) : (GROUPED ? 0 : (WIDE ? (wave >> 1) : wave));  // wave position along M (64 rows each)
+  const int wcol = G128 ? (wave & 3) : (GROUPED ? wave : (WIDE ? (wave & 1) : 0));    // wave position along N (128 columns each)
   const int c = lane & 31, h = lane >> 5;
 
   const uint32_t total_rows = g.total_rows;
@@ -123,7 +131,7 @@ void w8a8_gemm_kernel(GemmArgs g) {
     T.tn = in_band / band_rows;
     uint32_t widx = 0;
     if (GROUPED) {
-      const int32_t range = g.blk_range[T.tm * 2u];
+      const int32_t range = g.blk_range[T.tm * kRowBlocks];
       if (range < 0) return T;  // tile beyond the rows in use: nothing to do, but later tiles may exist
       widx = ((uint32_t)range & 0xffffu) / g.groups_per_weight;
     }
@@ -271,7 +279,7 @@ void w8a8_gemm_kernel(GemmArgs g) {
     // Lane (c = lane % 32, h = lane / 32) owns, in each of its wave's two 32 x 128 strips, the four
     // consecutive original columns ncol .. ncol+3 (accumulator blocks j = 0..3) of the 16 rows
     // 8*(v/4) + 4*h + v%4.
-    const uint32_t m0 = GROUPED ? T.tm * 64u : T.tm * 256u + wrow * 64u;
+    const uint32_t m0 = T.tm * (kRowBlocks * 32u) + wrow * 64u;
     const uint32_t tcol0 = T.tn * (kColBlocks * 32u) + wcol * 128u;  // first column of the wave
     const uint32_t ncol = tcol0 + 4u * c;
     const bool full_n = (tcol0 + 128u <= g.N) && ((g.N & 3u) == 0);  // wave-uniform

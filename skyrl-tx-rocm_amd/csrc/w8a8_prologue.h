@@ -153,30 +153,33 @@ __device__ inline void route_rows_block(const int32_t* __restrict__ idx, uint32_
 // ---------------------------------------------------------------------------------------
 // Tables for rows that arrive already grouped (ragged groups of an expert layer,
 // skyrl/tx/layers/util.py:8-59): group g owns group_sizes[g] consecutive rows and is padded
-// to a multiple of 64 grouped slots so that a 64-row GEMM tile never mixes two weights.
+// to a multiple of `pad` (64 or 128) grouped slots so that a GEMM tile never mixes two weights.
 //   src_row[p]   = original row of slot p, -1 for padding
 //   dst_pos[m]   = slot of row m, -1 for rows beyond sum(group_sizes) (their output is zero)
 //   blk_range[b] = g | g << 16 for the 32-row blocks in use, -1 beyond
 // ---------------------------------------------------------------------------------------
 constexpr int kMaxGroups = 1024;
-__global__ __launch_bounds__(1024) void route_groups_kernel(const int32_t* __restrict__ group_sizes, uint32_t M,
-                                                            uint32_t n_groups, uint32_t slots,
-                                                            int32_t* __restrict__ src_row,
-                                                            int32_t* __restrict__ dst_pos,
-                                                            int32_t* __restrict__ blk_range) {
+// One workgroup of 1024 threads.  Rows beyond sum(group_sizes) get no slot; their output rows
+// (zero_out, bf16 [M, zero_cols], optional) are cleared here.
+__device__ inline void route_groups_block(const int32_t* __restrict__ group_sizes, uint32_t M, uint32_t n_groups,
+                                          uint32_t slots, int32_t* __restrict__ src_row,
+                                          int32_t* __restrict__ dst_pos, int32_t* __restrict__ blk_range,
+                                          uint32_t pad, uint16_t* __restrict__ zero_out, uint32_t zero_cols) {
   __shared__ int row_start[kMaxGroups + 1];
   __shared__ int slot_start[kMaxGroups + 1];
   const uint32_t tid = threadIdx.x;
+  if (tid < n_groups) row_start[tid] = group_sizes[tid];  // sizes first, starts below
+  __syncthreads();
   if (tid == 0) {
     int r = 0, p = 0;
     for (uint32_t g = 0; g < n_groups; ++g) {
-      int sz = group_sizes[g];
+      int sz = row_start[g];
       if (sz < 0) sz = 0;
       if (r + sz > (int)M) sz = (int)M - r;
       row_start[g] = r;
       slot_start[g] = p;
       r += sz;
-      p += (sz + 63) & ~63;
+      p += (sz + (int)pad - 1) & ~((int)pad - 1);
     }
     row_start[n_groups] = r;
     slot_start[n_groups] = p;
@@ -194,6 +197,18 @@ __global__ __launch_bounds__(1024) void route_groups_kernel(const int32_t* __res
     }
     for (int b = p0 / 32 + (int)lane; b < p1 / 32; b += 64) blk_range[b] = (int)(g | (g << 16));
   }
+  if (zero_out) {
+    const size_t begin = (size_t)row_start[n_groups] * zero_cols, end = (size_t)M * zero_cols;
+    for (size_t i = begin + tid; i < end; i += 1024) zero_out[i] = 0;
+  }
+}
+
+__global__ __launch_bounds__(1024) void route_groups_kernel(const int32_t* __restrict__ group_sizes, uint32_t M,
+                                                            uint32_t n_groups, uint32_t slots,
+                                                            int32_t* __restrict__ src_row,
+                                                            int32_t* __restrict__ dst_pos,
+                                                            int32_t* __restrict__ blk_range, uint32_t pad) {
+  route_groups_block(group_sizes, M, n_groups, slots, src_row, dst_pos, blk_range, pad, nullptr, 0u);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -221,6 +236,10 @@ struct QuantArgs {
   uint16_t* zero_out;      // bf16 [M, zero_cols]: rows without a slot (dst_pos < 0) are zero-filled
   uint32_t zero_cols;
   uint32_t* tile_ctr;      // 256 words cleared for the GEMM launches' tile counters, or null
+  // Optional gather on the way in: row m is read from x[row_map[m] / row_div] (the sorted (token,
+  // choice) pairs of an expert layer read their token's row; x then has the tokens' row count)
+  const int32_t* row_map;
+  uint32_t row_div;
 };
 
 template <int NCH, bool RMS>
@@ -229,7 +248,8 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(QuantArgs a) {
   const uint32_t m = blockIdx.x * 4u + (threadIdx.x >> 6);
   if (a.tile_ctr && blockIdx.x == 0) a.tile_ctr[threadIdx.x] = 0u;
   if (m >= a.M) return;
-  const uint16_t* xr = a.x + (size_t)m * a.K;
+  const uint32_t xrow = a.row_map ? (uint32_t)a.row_map[m] / a.row_div : m;
+  const uint16_t* xr = a.x + (size_t)xrow * a.K;
   float v[NCH][8];
 #pragma unroll
   for (int j = 0; j < NCH; ++j) {
@@ -386,12 +406,21 @@ struct LoraPrepArgs {
   uint16_t* at;              // bf16 [n_groups, r, K]
   unsigned char* bp;         // packed B operands
   uint32_t M, K, N, n_groups, r, nkk, ncb, slots, route_blocks, a_blocks;
+  // grouped (ragged) call: the routing block lays the groups out from their sizes instead
+  const int32_t* group_sizes;  // int32 [n_groups] or null
+  uint32_t group_pad;          // slots every group is padded to
+  uint16_t* zero_out;          // bf16 [M, zero_cols]: rows beyond the groups are cleared, or null
+  uint32_t zero_cols;
 };
 
 __global__ __launch_bounds__(1024) void lora_prep_kernel(LoraPrepArgs p) {
   uint32_t b = blockIdx.x;
   if (b < p.route_blocks) {
-    route_rows_block(p.idx, p.M, p.n_groups, p.slots, p.src_row, p.dst_pos, p.slot_group, p.blk_range);
+    if (p.group_sizes)
+      route_groups_block(p.group_sizes, p.M, p.n_groups, p.slots, p.src_row, p.dst_pos, p.blk_range, p.group_pad,
+                         p.zero_out, p.zero_cols);
+    else
+      route_rows_block(p.idx, p.M, p.n_groups, p.slots, p.src_row, p.dst_pos, p.slot_group, p.blk_range);
     return;
   }
   b -= p.route_blocks;
@@ -428,6 +457,9 @@ struct LoraAArgs {
   // sums its own range of k steps and writes zf + ksplit_index * zf_slice (floats); the caller adds
   // the slices.  0 or 1: one workgroup per row block.
   uint32_t n_ksplit, zf_slice;
+  // Optional gather on the way in (see QuantArgs): source row = row_map[row] / row_div
+  const int32_t* row_map;
+  uint32_t row_div;
 };
 
 template <int RB>  // number of 32-wide rank blocks (1 or 2)
@@ -445,6 +477,7 @@ __global__ __launch_bounds__(1024) void lora_a_kernel(LoraAArgs a) {
   const uint32_t p = pb * 32u + i;
   int src = a.src_row ? a.src_row[p] : (int)p;
   if (src >= (int)a.M) src = -1;
+  if (a.row_map && src >= 0) src = (int)((uint32_t)a.row_map[src] / a.row_div);
   const uint32_t rowgrp = (a.slot_group && ghi > glo) ? (uint32_t)a.slot_group[p] : glo;
   const uint16_t* xr = a.xsrc + (size_t)(src < 0 ? 0 : src) * a.K;
   v16f acc[RB];
@@ -588,7 +621,15 @@ struct QuantLoraArgs {
   unsigned char* zp;        // packed z fragments
   uint32_t r, nkk, nterms;
   uint32_t* tile_ctr;       // 256 words cleared for the GEMM launches' tile counters, or null
+  // Optional gather on the way in (see QuantArgs): row `src` is read from x[row_map[src] / row_div];
+  // the auxiliary outputs keep the index `src`
+  const int32_t* row_map;
+  uint32_t row_div;
 };
+
+__device__ inline size_t quant_lora_x_row(const QuantLoraArgs& a, int src) {
+  return a.row_map ? (size_t)((uint32_t)a.row_map[src] / a.row_div) : (size_t)src;
+}
 
 template <int CB, bool RMS>  // CB: 16-wide rank blocks (0 = no LoRA, 1, 2, 4)
 __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
@@ -603,6 +644,7 @@ __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
   if (a.tile_ctr && hb == 0 && tid < 256u) a.tile_ctr[tid] = 0u;
   if (hb >= a.n_half_blocks) return;
   const uint32_t pb = hb >> 1, half16 = hb & 1u;
+  if (a.blk_range && a.blk_range[pb] < 0) return;  // grouped layout: block beyond the slots in use
 
   // ---- 1. row statistics: wave w, slot row w
   {
@@ -611,7 +653,7 @@ __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
     if (src < 0 || src >= (int)a.M) src = -1;
     float inv = 1.0f, amax = 0.0f;
     if (src >= 0) {
-      const uint16_t* xr = a.x + (size_t)src * a.K;
+      const uint16_t* xr = a.x + quant_lora_x_row(a, src) * a.K;
       // eight 16-byte loads of the row are in flight at a time
       if (RMS) {
         double ss = 0.0;
@@ -688,7 +730,7 @@ __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
   const int src = row_src[i];
   const float inv = row_inv[i], scale = row_scale[i];
   const float rscale = __builtin_amdgcn_rcpf(scale);
-  const uint16_t* xr = a.x + (size_t)(src < 0 ? 0 : src) * a.K;
+  const uint16_t* xr = a.x + (src < 0 ? (size_t)0 : quant_lora_x_row(a, src)) * a.K;
   const uint32_t range = (CB > 0 && a.blk_range) ? (uint32_t)a.blk_range[pb] : 0u;
   const uint32_t glo = range & 0xffffu, ghi = range >> 16;
   const uint32_t rowgrp = (CB > 0 && a.slot_group && ghi > glo) ? (uint32_t)a.slot_group[hb * 16u + i] : glo;

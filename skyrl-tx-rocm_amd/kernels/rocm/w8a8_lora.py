@@ -686,10 +686,15 @@ def prepare_grouped_weight(codes: torch.Tensor, scales: torch.Tensor) -> PackedG
 
 def grouped_forward(x: torch.Tensor, group_sizes: torch.Tensor, weight: PackedGroupedW8Weight, lora_a=None,
                     lora_b=None, lora_scaling=None, *, swiglu: bool = False, groups_per_weight: int = 1,
-                    flags: int = 0, return_aux: bool = False):
+                    flags: int = 0, return_aux: bool = False, row_map: torch.Tensor | None = None,
+                    row_repeat: int = 1):
     """Ragged W8A8 (+LoRA) linear: rows of ``x`` are sorted by group; group g owns
     ``group_sizes[g]`` consecutive rows and uses weight ``g // groups_per_weight`` and LoRA pair g.
-    Rows beyond ``sum(group_sizes)`` give zeros (``lax.ragged_dot`` semantics)."""
+    Rows beyond ``sum(group_sizes)`` give zeros (``lax.ragged_dot`` semantics).
+
+    With ``row_map`` (int32 [rows]) the call has ``row_map.numel()`` rows and row i is read from
+    ``x[row_map[i] // row_repeat]``: the sorted (token, choice) pairs of an expert layer read the
+    unsorted hidden states, and no sorted copy of them is ever written."""
     if x.dtype != torch.bfloat16:
         raise TypeError(f"x must be BF16, got {x.dtype}")
     if x.ndim != 2 or x.shape[0] <= 0:
@@ -701,6 +706,14 @@ def grouped_forward(x: torch.Tensor, group_sizes: torch.Tensor, weight: PackedGr
     dev = x.device
     flat = x.contiguous()
     m = flat.shape[0]
+    rmap = None
+    if row_map is not None:
+        if isinstance(row_repeat, bool) or not isinstance(row_repeat, int) or row_repeat < 1:
+            raise ValueError(f"row_repeat must be a positive integer, got {row_repeat!r}")
+        rmap = row_map.reshape(-1).to(device=dev, dtype=torch.int32).contiguous()
+        m = rmap.numel()
+        if m <= 0 or m > flat.shape[0] * row_repeat:
+            raise ValueError(f"row_map with {m} entries does not fit {flat.shape[0]} rows x {row_repeat}")
     gs = group_sizes.to(device=dev, dtype=torch.int32).contiguous()
     n_groups = gs.numel()
     if n_groups != weight.n_weights * groups_per_weight:
@@ -755,6 +768,8 @@ def grouped_forward(x: torch.Tensor, group_sizes: torch.Tensor, weight: PackedGr
     p.aux_x_codes = aux["x_codes"].data_ptr() if return_aux else None
     p.aux_x_scales = aux["x_scales"].data_ptr() if return_aux else None
     p.aux_acc = aux["acc"].data_ptr() if return_aux else None
+    p.x_row_map = rmap.data_ptr() if rmap is not None else None
+    p.x_row_repeat = row_repeat if rmap is not None else 0
     with torch.cuda.device(dev):
         _native.check("mi355_w8a8_grouped_v1", lib.mi355_w8a8_grouped_v1(ctypes.byref(p), _stream_ptr(dev)))
     return (out, aux) if return_aux else out
@@ -981,13 +996,15 @@ def w8a8_moe_expert_mlp(hidden, router_logits, top_k: int, gate_up_weight, down_
     """Expert MLP of ``Qwen3Experts.__call__`` (skyrl/tx/models/qwen3.py:172-210) on W8A8 weights:
     softmax -> top-k -> renormalise -> sort rows by expert -> grouped gate/up + SwiGLU -> grouped
     down -> unsort -> weighted sum.  Five native calls on one stream, no host round trip: route,
-    dispatch, the two grouped GEMMs, combine."""
+    dispatch (indices only), the two grouped GEMMs (the first reads the hidden rows through the sort
+    order), combine."""
     _check_enabled(enabled, False, "MoE expert MLP")
     n_experts = gate_up_weight.n_weights
     weights, selected = moe_route(router_logits, top_k, norm_topk_prob)
-    x_sorted, group_sizes, _, unsort, _ = moe_dispatch(hidden.reshape(-1, hidden.shape[-1]), selected, n_experts,
-                                                       repeat=top_k)
-    act = grouped_forward(x_sorted, group_sizes, gate_up_weight, gate_up_a, gate_up_b, lora_scaling, swiglu=True)
+    # indices only: the first projection gathers the hidden rows itself through the sort order
+    _, group_sizes, sort_indices, unsort, _ = moe_dispatch(None, selected, n_experts, repeat=top_k)
+    act = grouped_forward(hidden.reshape(-1, hidden.shape[-1]), group_sizes, gate_up_weight, gate_up_a, gate_up_b,
+                          lora_scaling, swiglu=True, row_map=sort_indices, row_repeat=top_k)
     down = grouped_forward(act, group_sizes, down_weight, down_a, down_b, lora_scaling)
     return moe_combine(down, unsort, weights)
 

@@ -41,7 +41,7 @@ def test_library_exports_every_declared_symbol(native):
 def test_struct_sizes_match_header_layout(native):
     # 8 x 4-byte scalars, 11 pointers, u64, 4 pointers
     assert ctypes.sizeof(native.Problem) == 8 * 4 + 11 * 8 + 8 + 4 * 8
-    assert ctypes.sizeof(native.GroupedProblem) == 8 * 4 + 9 * 8 + 8 + 3 * 8
+    assert ctypes.sizeof(native.GroupedProblem) == 8 * 4 + 9 * 8 + 8 + 3 * 8 + 8 + 2 * 4
     # backward: 8 x 4-byte scalars, 13 pointers, u64
     assert ctypes.sizeof(native.BwdProblem) == 8 * 4 + 13 * 8 + 8
 

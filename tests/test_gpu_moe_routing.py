@@ -187,3 +187,38 @@ def test_routing_rejects_bad_arguments(dev, pkg):
     assert pkg._native.STATUS[st] == "ERR_ALIAS"
     st = lib.mi355_w8a8_moe_route_v1(logits.data_ptr(), 4, 8, 2, 1, logits.data_ptr(), idx.data_ptr(), None)
     assert pkg._native.STATUS[st] == "ERR_ALIAS"
+
+
+@pytest.mark.parametrize("swiglu,rank", [(True, 16), (False, 0)])
+def test_grouped_call_reads_rows_through_the_sort_order(dev, pkg, swiglu, rank):
+    """The grouped projection with a row map gives bit for bit what it gives on the gathered copy
+    (codes, scales, integer accumulators, output), so the dispatch can skip the row copies."""
+    import torch
+
+    rng = np.random.default_rng(17)
+    t, h, n, e, topk = 150, 256, 384, 12, 3
+    print(f"[case] grouped row map swiglu={swiglu} rank={rank}", flush=True)
+    w8 = pkg.w8a8_lora
+    hidden = _bf(dev, o.bf16_round(rng.standard_normal((t, h)).astype(F32)))
+    selected = torch.from_numpy(np.stack([rng.permutation(e)[:topk] for _ in range(t)]).astype(np.int32)).to(dev)
+    codes = torch.from_numpy(rng.integers(-127, 128, (e, h, n), dtype=np.int8)).to(dev)
+    scales = torch.from_numpy(rng.uniform(0.001, 0.01, (e, n)).astype(F32)).to(dev)
+    weight = w8.prepare_grouped_weight(codes, scales)
+    a = b = s = None
+    if rank:
+        a = _bf(dev, o.bf16_round((rng.standard_normal((e, h, rank)) * 0.05).astype(F32)))
+        b = _bf(dev, o.bf16_round((rng.standard_normal((e, rank, n)) * 0.05).astype(F32)))
+        s = 1.5
+    xs, sizes, sort_i, unsort, _ = w8.moe_dispatch(hidden, selected, e, repeat=topk)
+    want, want_aux = w8.grouped_forward(xs, sizes, weight, a, b, s, swiglu=swiglu, return_aux=True)
+    got, got_aux = w8.grouped_forward(hidden, sizes, weight, a, b, s, swiglu=swiglu, return_aux=True,
+                                      row_map=sort_i, row_repeat=topk)
+    torch.cuda.synchronize()
+    assert tuple(got.shape) == tuple(want.shape) == (t * topk, n // 2 if swiglu else n)
+    assert torch.equal(got, want)
+    for key in ("x_codes", "x_scales", "acc"):
+        assert torch.equal(got_aux[key], want_aux[key]), key
+    with pytest.raises(ValueError):
+        w8.grouped_forward(hidden, sizes, weight, a, b, s, row_map=sort_i, row_repeat=0)
+    with pytest.raises(ValueError):
+        w8.grouped_forward(hidden[:10], sizes, weight, a, b, s, row_map=sort_i, row_repeat=topk)

@@ -203,6 +203,26 @@ def test_skinny_path_shapes(dev, pkg, m, k, n, n_ad, rank, rms):
     _assert_close(tiled, st["out"], f" tiled {m}x{k}x{n}")
 
 
+@pytest.mark.parametrize("m,k,n,n_ad,rank,rms", [(33, 512, 264, 3, 16, True), (47, 1024, 520, 2, 40, False),
+                                                 (64, 2560, 1024, 0, 0, True), (100, 4096, 512, 5, 8, True),
+                                                 (128, 4096, 776, 4, 64, False)])
+def test_chunked_skinny_path(dev, pkg, m, k, n, n_ad, rank, rms):
+    """Between 33 and 128 rows a call without SwiGLU whose weight fits the caches runs the streaming
+    kernels on 32-row chunks: every stage against the oracle, ragged last chunks, and the tiled kernel on
+    the same case (integer stages bit-equal between the two paths)."""
+    case = wc.make_case(m, k, n, n_adapters=n_ad, rank=max(rank, 1), seed=3 * m + k, rms=rms, residual=(m % 2 == 1))
+    st = wc.oracle_forward(case, return_stages=True)
+    got, aux = wc.gpu_forward(case)
+    if rms:
+        np.testing.assert_array_equal(o.bf16_bits(aux["normalized"]), o.bf16_bits(st["normalized"]))
+    _assert_integer_stages(aux, st)
+    _assert_close(got, st["out"], f" chunked {m}x{k}x{n}")
+    tiled, aux_t = wc.gpu_forward(case, flags=pkg._native.FLAG_FORCE_TILED)
+    _assert_close(tiled, st["out"], f" tiled {m}x{k}x{n}")
+    for key in ("x_codes", "x_scales", "acc"):
+        np.testing.assert_array_equal(aux[key], aux_t[key])
+
+
 @pytest.mark.parametrize("m", [1, 64, 512])
 @pytest.mark.parametrize("k,n", [(2560, 6144), (4096, 2560)])
 def test_config4_student_t(dev, m, k, n):
@@ -303,14 +323,18 @@ def _grouped_case(rng, sizes, k, n, rank, extra_rows=0):
     return m, x, codes, scales, a, b
 
 
+@pytest.mark.parametrize("tile_rows", [64, 128])
 @pytest.mark.parametrize("sizes,k,n,rank,swiglu,extra", [
     ([5, 0, 70, 33, 1, 64, 0, 129], 256, 512, 16, False, 0),
     ([40, 3, 0, 0, 200], 384, 1536, 16, True, 0),
     ([17, 90], 128, 96, 8, False, 9),
     ([64, 64, 64], 2048, 768, 0, False, 0),
+    ([128, 300, 127, 129], 320, 1032, 32, True, 3),
 ])
-def test_grouped_ragged_linear(dev, pkg, sizes, k, n, rank, swiglu, extra):
+def test_grouped_ragged_linear(dev, pkg, sizes, k, n, rank, swiglu, extra, tile_rows):
     import torch
+
+    tile_flag = pkg._native.FLAG_GROUPED_TILE64 if tile_rows == 64 else pkg._native.FLAG_GROUPED_TILE128
 
     rng = np.random.default_rng(len(sizes) * 100 + k)
     m, x, codes, scales, a, b = _grouped_case(rng, sizes, k, n, rank, extra)
@@ -335,7 +359,7 @@ def test_grouped_ragged_linear(dev, pkg, sizes, k, n, rank, swiglu, extra):
     gw = w8.prepare_grouped_weight(torch.from_numpy(codes).to(dev), torch.from_numpy(scales).to(dev))
     out, aux = w8.grouped_forward(bf(x), torch.tensor(sizes, dtype=torch.int32), gw,
                                   bf(a) if rank else None, bf(b) if rank else None, float(s) if rank else None,
-                                  swiglu=swiglu, return_aux=True)
+                                  swiglu=swiglu, return_aux=True, flags=tile_flag)
     torch.cuda.synchronize()
     got = out.float().cpu().numpy()
     np.testing.assert_array_equal(aux["x_codes"].cpu().numpy(), xc)
