@@ -671,11 +671,21 @@ def main() -> int:
 
     # dominant kernel alone: HIP events (torch's current stream is the launch stream) around
     # GEMM-only launches; the workspace still holds the prologue's results.
+    # (a call of 33..128 rows that runs as 32-row chunks of the streaming kernels keeps no stage to
+    # rerun: the library says so, and the figures below are then taken around whole calls)
+    try:
+        plans[0].run(native.FLAG_SKIP_PROLOGUE)
+        stage_flags = (native.FLAG_SKIP_PROLOGUE, native.FLAG_SKIP_GEMM)
+    except native.NativeError as err:
+        if err.status != -7:
+            raise
+        stage_flags = (0, 0)
+        skinny = True
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
           for _ in range(args.steps)]
     for i, (a, b) in enumerate(ev):
         a.record()
-        plans[i % rotate].run(native.FLAG_SKIP_PROLOGUE)
+        plans[i % rotate].run(stage_flags[0])
         b.record()
     torch.cuda.synchronize()
     gemm_ms = np.asarray([a.elapsed_time(b) for a, b in ev])
@@ -684,10 +694,10 @@ def main() -> int:
     pa, pb = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     pa.record()
     for i in range(args.steps):
-        plans[i % rotate].run(native.FLAG_SKIP_GEMM)
+        plans[i % rotate].run(stage_flags[1])
     pb.record()
     torch.cuda.synchronize()
-    prologue_ms = pa.elapsed_time(pb) / args.steps
+    prologue_ms = pa.elapsed_time(pb) / args.steps if stage_flags[1] else None
     out_gpu = plan.run()
     torch.cuda.synchronize()
 

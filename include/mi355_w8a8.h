@@ -58,11 +58,13 @@ typedef enum mi355_w8a8_status {
 
 /* Flags of mi355_w8a8_problem.flags */
 #define MI355_W8A8_FLAG_SWIGLU 1u      /* out[m, j] = bf16(silu(y[m,2j]) * y[m,2j+1]); out is [M, N/2] */
-#define MI355_W8A8_FLAG_FORCE_TILED 2u /* never take the skinny-M (split-K) kernel */
+#define MI355_W8A8_FLAG_FORCE_TILED 2u /* never take the skinny-M (split-K) kernel, whole or in 32-row chunks */
 #define MI355_W8A8_FLAG_FORCE_SKINNY 4u/* always take the skinny-M kernel (M <= 32) */
 #define MI355_W8A8_FLAG_LORA_SPLIT2 8u /* carry x@A as 2 bf16 terms instead of 3 in the LoRA-B product */
 /* Stage selection for measurement: the workspace keeps the prologue's results between calls, so a
  * call with SKIP_PROLOGUE after a full call with the same arguments re-runs only the GEMM kernel. */
+/* Calls of 33..128 rows that run as 32-row chunks of the skinny-M kernels (see FORCE_TILED) keep no
+ * prologue results and answer these two flags with MI355_W8A8_ERR_UNSUPPORTED. */
 #define MI355_W8A8_FLAG_SKIP_PROLOGUE 16u /* do not run routing / quantization / LoRA-A */
 #define MI355_W8A8_FLAG_SKIP_GEMM 32u     /* run only routing / quantization / LoRA-A */
 /* tile geometry of the tiled GEMM; default: 256 x 256 once such tiles fill the chip, else 256 x 128 */

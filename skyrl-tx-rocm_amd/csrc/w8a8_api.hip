@@ -281,8 +281,11 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
                          reinterpret_cast<uint16_t*>(ws + w.xn), ws + w.skinny, w.K_pad, w.KB, s);
   }
   if (skinny_supported() && !swiglu && skinny_chunked_pays(p->m, p->k, p->n) &&
-      !(p->flags & (MI355_W8A8_FLAG_FORCE_TILED | MI355_W8A8_FLAG_SKIP_PROLOGUE | MI355_W8A8_FLAG_SKIP_GEMM |
-                    MI355_W8A8_FLAG_TILE_256X128 | MI355_W8A8_FLAG_TILE_256X256))) {
+      !(p->flags & (MI355_W8A8_FLAG_FORCE_TILED | MI355_W8A8_FLAG_TILE_256X128 | MI355_W8A8_FLAG_TILE_256X256))) {
+    // The chunks overwrite each other's prologue results, so there is no GEMM-only or prologue-only
+    // rerun of such a call; the choice of path must not depend on those flags either (a GEMM-only
+    // tiled call would read tables no tiled prologue has written).
+    if (p->flags & (MI355_W8A8_FLAG_SKIP_PROLOGUE | MI355_W8A8_FLAG_SKIP_GEMM)) return MI355_W8A8_ERR_UNSUPPORTED;
     for (uint32_t row0 = 0; row0 < p->m; row0 += (uint32_t)kSkinnyMaxRows) {
       mi355_w8a8_problem sub = *p;
       sub.m = p->m - row0 < (uint32_t)kSkinnyMaxRows ? p->m - row0 : (uint32_t)kSkinnyMaxRows;
