@@ -177,6 +177,103 @@ ffi::Error PackWeight(hipStream_t stream, ffi::Buffer<ffi::S8> codes, ffi::Resul
                  "mi355_w8a8 pack launch submission failed");
 }
 
+// d_fused = swiglu pull-back(fused, d_product); fused bf16 [.., N], d_product bf16 [.., N / 2].
+ffi::Error SwigluBwd(hipStream_t stream, ffi::Buffer<ffi::BF16> fused, ffi::Buffer<ffi::BF16> d_product,
+                     ffi::ResultBuffer<ffi::BF16> d_fused) {
+  uint32_t m = 0, n = 0;
+  if (!RowsAndK(fused.dimensions(), &m, &n))
+    return ffi::Error::InvalidArgument("fused must be bf16 [..., N] with a non-empty row domain");
+  if (d_product.element_count() * 2 != fused.element_count() || d_fused->element_count() != fused.element_count())
+    return ffi::Error::InvalidArgument("d_product must be [..., N / 2] and d_fused must match fused");
+  return ToError(mi355_w8a8_swiglu_bwd_v1(fused.untyped_data(), d_product.untyped_data(), d_fused->untyped_data(), m, n,
+                                          stream),
+                 "mi355_w8a8 swiglu pull-back launch submission failed");
+}
+
+// d_x = RMSNorm pull-back(x, gamma, d_normalized); x and d_normalized bf16 [.., K], gamma f32 [K].
+ffi::Error RmsNormBwd(hipStream_t stream, ffi::Buffer<ffi::BF16> x, ffi::Buffer<ffi::F32> gamma,
+                      ffi::Buffer<ffi::BF16> d_normalized, ffi::ResultBuffer<ffi::BF16> d_x, float eps) {
+  uint32_t m = 0, k = 0;
+  if (!RowsAndK(x.dimensions(), &m, &k))
+    return ffi::Error::InvalidArgument("x must be bf16 [..., K] with a non-empty row domain");
+  if (gamma.element_count() != k || d_normalized.element_count() != x.element_count() ||
+      d_x->element_count() != x.element_count())
+    return ffi::Error::InvalidArgument("gamma must be f32 [K]; d_normalized and d_x must match x");
+  return ToError(mi355_w8a8_rms_norm_bwd_v1(x.untyped_data(), gamma.typed_data(), d_normalized.untyped_data(),
+                                            d_x->untyped_data(), m, k, eps, stream),
+                 "mi355_w8a8 rms norm pull-back launch submission failed");
+}
+
+// router_logits f32 [T, E] -> weights f32 [T, top_k], selected s32 [T, top_k].
+ffi::Error MoeRoute(hipStream_t stream, ffi::Buffer<ffi::F32> router_logits, ffi::ResultBuffer<ffi::F32> weights,
+                    ffi::ResultBuffer<ffi::S32> selected, int32_t norm_topk_prob) {
+  auto d = router_logits.dimensions();
+  auto dw = weights->dimensions();
+  if (d.size() != 2 || dw.size() != 2 || d[0] <= 0 || dw[0] != d[0] || dw[1] <= 0 ||
+      selected->element_count() != weights->element_count())
+    return ffi::Error::InvalidArgument("router_logits must be f32 [T, E]; weights and selected [T, top_k]");
+  return ToError(mi355_w8a8_moe_route_v1(router_logits.typed_data(), static_cast<uint32_t>(d[0]),
+                                         static_cast<uint32_t>(d[1]), static_cast<uint32_t>(dw[1]),
+                                         norm_topk_prob ? 1u : 0u, weights->typed_data(), selected->typed_data(), stream),
+                 "mi355_w8a8 moe route launch submission failed");
+}
+
+// Stable sort of the pairs by group.  tokens bf16 [P / repeat, H] (size 0: indices only), indices s32
+// [P], adapter_indices s32 [P / repeat] (size 0: none).  Results: sorted_tokens bf16 [P, H] (size 0
+// without tokens), group_sizes s32 [G], sort_indices and unsort_indices s32 [P], sorted_adapters s32
+// [P] (size 0 without adapter indices), workspace u8 [mi355_w8a8_moe_dispatch_workspace_bytes].
+ffi::Error MoeDispatch(hipStream_t stream, ffi::Buffer<ffi::BF16> tokens, ffi::Buffer<ffi::S32> indices,
+                       ffi::Buffer<ffi::S32> adapter_indices, ffi::ResultBuffer<ffi::BF16> sorted_tokens,
+                       ffi::ResultBuffer<ffi::S32> group_sizes, ffi::ResultBuffer<ffi::S32> sort_indices,
+                       ffi::ResultBuffer<ffi::S32> unsort_indices, ffi::ResultBuffer<ffi::S32> sorted_adapters,
+                       ffi::ResultBuffer<ffi::U8> workspace, int32_t repeat) {
+  mi355_w8a8_moe_dispatch_problem p{};
+  p.struct_size = sizeof(p);
+  p.n_pairs = static_cast<uint32_t>(indices.element_count());
+  p.n_groups = static_cast<uint32_t>(group_sizes->element_count());
+  p.repeat = repeat > 0 ? static_cast<uint32_t>(repeat) : 0u;
+  if (p.n_pairs == 0 || p.repeat == 0 || sort_indices->element_count() != p.n_pairs ||
+      unsort_indices->element_count() != p.n_pairs)
+    return ffi::Error::InvalidArgument("indices, sort_indices and unsort_indices must hold one entry per pair");
+  if (tokens.element_count() > 0) {
+    auto d = tokens.dimensions();
+    if (d.size() != 2 || static_cast<uint64_t>(d[0]) * p.repeat != p.n_pairs ||
+        sorted_tokens->element_count() != static_cast<size_t>(p.n_pairs) * d[1])
+      return ffi::Error::InvalidArgument("tokens must be bf16 [P / repeat, H] and sorted_tokens [P, H]");
+    p.width = static_cast<uint32_t>(d[1]);
+    p.tokens = tokens.untyped_data();
+    p.sorted_tokens = sorted_tokens->untyped_data();
+  }
+  if (adapter_indices.element_count() > 0) {
+    if (adapter_indices.element_count() * p.repeat != p.n_pairs || sorted_adapters->element_count() != p.n_pairs)
+      return ffi::Error::InvalidArgument("adapter_indices must be [P / repeat] and sorted_adapters [P]");
+    p.adapter_indices = adapter_indices.typed_data();
+    p.sorted_adapters = sorted_adapters->typed_data();
+  }
+  p.indices = indices.typed_data();
+  p.group_sizes = group_sizes->typed_data();
+  p.sort_indices = sort_indices->typed_data();
+  p.unsort_indices = unsort_indices->typed_data();
+  p.workspace = workspace->untyped_data();
+  p.workspace_bytes = workspace->size_bytes();
+  return ToError(mi355_w8a8_moe_dispatch_v1(&p, stream), "mi355_w8a8 moe dispatch launch submission failed");
+}
+
+// out[t] = sum_j expert_out[unsort[t k + j]] * weights[t, j]; expert_out bf16 [T k, H], out bf16 [T, H].
+ffi::Error MoeCombine(hipStream_t stream, ffi::Buffer<ffi::BF16> expert_out, ffi::Buffer<ffi::S32> unsort_indices,
+                      ffi::Buffer<ffi::F32> weights, ffi::ResultBuffer<ffi::BF16> out) {
+  auto de = expert_out.dimensions();
+  auto dw = weights.dimensions();
+  if (de.size() != 2 || dw.size() != 2 || dw[0] <= 0 || dw[1] <= 0 || de[0] != dw[0] * dw[1] ||
+      unsort_indices.element_count() != static_cast<size_t>(de[0]) ||
+      out->element_count() != static_cast<size_t>(dw[0]) * de[1])
+    return ffi::Error::InvalidArgument("expert_out must be [T * top_k, H], weights [T, top_k], out [T, H]");
+  return ToError(mi355_w8a8_moe_combine_v1(expert_out.untyped_data(), unsort_indices.typed_data(), weights.typed_data(),
+                                           out->untyped_data(), static_cast<uint32_t>(dw[0]),
+                                           static_cast<uint32_t>(dw[1]), static_cast<uint32_t>(de[1]), stream),
+                 "mi355_w8a8 moe combine launch submission failed");
+}
+
 }  // namespace
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_forward_v1, Forward,
@@ -226,4 +323,49 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_backward_v1, Backward,
                                   .Ret<ffi::Buffer<ffi::BF16>>()
                                   .Ret<ffi::Buffer<ffi::F32>>()
                                   .Ret<ffi::Buffer<ffi::U8>>());
+XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_swiglu_bwd_v1, SwigluBwd,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>());
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_rms_norm_bwd_v1, RmsNormBwd,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Attr<float>("eps"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_moe_route_v1, MoeRoute,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Ret<ffi::Buffer<ffi::F32>>()
+                                  .Ret<ffi::Buffer<ffi::S32>>()
+                                  .Attr<int32_t>("norm_topk_prob"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_moe_dispatch_v1, MoeDispatch,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::S32>>()
+                                  .Ret<ffi::Buffer<ffi::S32>>()
+                                  .Ret<ffi::Buffer<ffi::S32>>()
+                                  .Ret<ffi::Buffer<ffi::S32>>()
+                                  .Ret<ffi::Buffer<ffi::U8>>()
+                                  .Attr<int32_t>("repeat"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_moe_combine_v1, MoeCombine,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>());
 #endif  // __has_include("xla/ffi/api/ffi.h")

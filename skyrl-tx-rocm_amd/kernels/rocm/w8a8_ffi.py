@@ -24,7 +24,8 @@ from ... import _native
 
 FFI_LIB_PATH = Path(_native.LIB_PATH).with_name("libmi355_w8a8_ffi.so")
 TARGETS = ("mi355_w8a8_ffi_forward_v1", "mi355_w8a8_ffi_quantize_rows_v1", "mi355_w8a8_ffi_pack_weight_v1",
-           "mi355_w8a8_ffi_backward_v1")
+           "mi355_w8a8_ffi_backward_v1", "mi355_w8a8_ffi_swiglu_bwd_v1", "mi355_w8a8_ffi_rms_norm_bwd_v1",
+           "mi355_w8a8_ffi_moe_route_v1", "mi355_w8a8_ffi_moe_dispatch_v1", "mi355_w8a8_ffi_moe_combine_v1")
 _ROCM_PLATFORM = "ROCM"
 _REGISTRATION_API_VERSION = 1
 _CUSTOM_CALL_API_VERSION = 4

@@ -89,5 +89,5 @@ def test_shim_source_obeys_the_handler_rules():
                        "-ffast-math"):
             assert banned not in text, (src.name, banned)
     shim = (root / "w8a8_xla_ffi.cc").read_text()
-    assert shim.count("XLA_FFI_DEFINE_HANDLER_SYMBOL") == 4
+    assert shim.count("XLA_FFI_DEFINE_HANDLER_SYMBOL") == 9
     assert "PlatformStream<hipStream_t>" in shim
