@@ -29,6 +29,8 @@
  *   - mi355_w8a8_qkv_split_norm_rope_v1 skyrl/tx/kernels/qwen3_5_qkv_lora.py:266-286
  *   - mi355_w8a8_moe_route_v1 / _moe_dispatch_v1 / _moe_combine_v1
  *                                      skyrl/tx/models/qwen3.py:172-210, skyrl/tx/layers/util.py:66-87
+ *   - mi355_w8a8_gq_linear_v1          skyrl/tx/kernels/quantized_lora.py:215-304 in its general form
+ *                                      (W4 / W8 codes, A4 / A8 activations, scales per K group)
  * The typed-FFI handler shape these sit behind is rocm/QUANTIZED_FFI.md:589-599 and
  * skyrl/tx/kernels/rocm/ffi/gdn_ffi_smoke.hip:43-82.
  */
@@ -325,6 +327,53 @@ int mi355_w8a8_moe_dispatch_v1(const mi355_w8a8_moe_dispatch_problem* problem, v
  */
 int mi355_w8a8_moe_combine_v1(const void* expert_out, const int32_t* unsort_indices, const float* weights, void* out,
                               uint32_t n_tokens, uint32_t top_k, uint32_t width, void* stream);
+
+/*
+ * Group-scaled quantized linear: the general form of quantized_frozen_linear / quantized_lora_linear
+ * (skyrl/tx/kernels/quantized_lora.py:215-304) -- W4 or W8 codes with one scale per (K group, output),
+ * A4 or A8 activations quantized per (row, K group):
+ *   out = bf16( sum_g ((f32(acc_g) * x_scale[m, g]) * w_scale[g, n])  +  s[idx] * ((x @ A[idx]) @ B[idx]) )
+ * with the groups added in float32 in group order, as the reference does (the float32 base is
+ * reproduced bit for bit; aux_base returns it).  group_size must be a multiple of 32 and divide
+ * k_pad; k <= k_pad (the reference pads K with zeros).  The per-channel W8A8 case
+ * (group_size == k) is better served by mi355_w8a8_forward_v1.
+ *
+ * mi355_w8a8_gq_pack_weight_v1 re-lays the reference's codes (bits 8: int8 [k_pad, n]; bits 4: uint8
+ * [k_pad / 2, n] with the even k in the low nibble, quantized_lora.py:94-125) into matrix-core
+ * fragments once at load time; 4-bit codes stay 4-bit (half a byte per weight in HBM).
+ */
+uint64_t mi355_w8a8_gq_packed_weight_bytes(uint32_t k_pad, uint32_t n, uint32_t weight_bits);
+int mi355_w8a8_gq_pack_weight_v1(const void* codes, void* packed, uint32_t k_pad, uint32_t n, uint32_t weight_bits,
+                                 void* stream);
+
+typedef struct mi355_w8a8_gq_problem {
+  uint32_t struct_size;      /* sizeof(mi355_w8a8_gq_problem) */
+  uint32_t flags;            /* 0 */
+  uint32_t m, k, k_pad, n;
+  uint32_t group_size;       /* multiple of 32, divides k_pad */
+  uint32_t weight_bits;      /* 4 or 8 */
+  uint32_t activation_bits;  /* 4 or 8 */
+  uint32_t n_adapters;       /* 0 = no LoRA */
+  uint32_t rank;             /* <= 64 */
+  uint32_t reserved;
+  const void* x;             /* bf16 [m, k] */
+  const void* w_packed;      /* from mi355_w8a8_gq_pack_weight_v1 */
+  const float* w_scales;     /* f32 [k_pad / group_size, n] */
+  const void* lora_a;        /* bf16 [n_adapters, k, rank] or NULL */
+  const void* lora_b;        /* bf16 [n_adapters, rank, n] or NULL */
+  const float* lora_scaling; /* f32 [n_adapters] or NULL */
+  const int32_t* adapter_indices; /* int32 [m] or NULL (adapter 0) */
+  void* out;                 /* bf16 [m, n] */
+  void* workspace;           /* >= mi355_w8a8_gq_workspace_bytes(...), 256-byte aligned */
+  uint64_t workspace_bytes;
+  /* Optional auxiliary outputs for parity checks (NULL to skip) */
+  int8_t* aux_x_codes;       /* int8 [m, k_pad] */
+  float* aux_x_scales;       /* f32 [m, k_pad / group_size] */
+  float* aux_base;           /* f32 [m, n]: the float32 base before the LoRA term */
+} mi355_w8a8_gq_problem;
+
+uint64_t mi355_w8a8_gq_workspace_bytes(uint32_t m, uint32_t k_pad, uint32_t group_size, uint32_t rank);
+int mi355_w8a8_gq_linear_v1(const mi355_w8a8_gq_problem* problem, void* stream);
 
 #ifdef __cplusplus
 }

@@ -40,6 +40,8 @@ EXPORTS = (
     "mi355_w8a8_swiglu_bwd_v1", "mi355_w8a8_rms_norm_bwd_v1",
     "mi355_w8a8_moe_route_v1", "mi355_w8a8_moe_dispatch_workspace_bytes", "mi355_w8a8_moe_dispatch_v1",
     "mi355_w8a8_moe_combine_v1",
+    "mi355_w8a8_gq_packed_weight_bytes", "mi355_w8a8_gq_pack_weight_v1", "mi355_w8a8_gq_workspace_bytes",
+    "mi355_w8a8_gq_linear_v1",
 )
 
 _u32, _u64, _vp, _f32 = ctypes.c_uint32, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_float
@@ -106,6 +108,19 @@ class MoeDispatchProblem(ctypes.Structure):
     ]
 
 
+class GqProblem(ctypes.Structure):
+    """struct mi355_w8a8_gq_problem"""
+
+    _fields_ = [
+        ("struct_size", _u32), ("flags", _u32), ("m", _u32), ("k", _u32), ("k_pad", _u32), ("n", _u32),
+        ("group_size", _u32), ("weight_bits", _u32), ("activation_bits", _u32), ("n_adapters", _u32),
+        ("rank", _u32), ("reserved", _u32),
+        ("x", _vp), ("w_packed", _vp), ("w_scales", _vp), ("lora_a", _vp), ("lora_b", _vp), ("lora_scaling", _vp),
+        ("adapter_indices", _vp), ("out", _vp), ("workspace", _vp), ("workspace_bytes", _u64),
+        ("aux_x_codes", _vp), ("aux_x_scales", _vp), ("aux_base", _vp),
+    ]
+
+
 class NativeError(RuntimeError):
     def __init__(self, fn: str, status: int, detail: str):
         super().__init__(f"{fn} failed: {STATUS.get(status, status)} ({detail})")
@@ -153,6 +168,14 @@ def _bind(lib: ctypes.CDLL) -> None:
     lib.mi355_w8a8_moe_dispatch_v1.argtypes = (ctypes.POINTER(MoeDispatchProblem), _vp)
     lib.mi355_w8a8_moe_combine_v1.restype = ctypes.c_int
     lib.mi355_w8a8_moe_combine_v1.argtypes = (_vp, _vp, _vp, _vp, _u32, _u32, _u32, _vp)
+    lib.mi355_w8a8_gq_packed_weight_bytes.restype = _u64
+    lib.mi355_w8a8_gq_packed_weight_bytes.argtypes = (_u32, _u32, _u32)
+    lib.mi355_w8a8_gq_pack_weight_v1.restype = ctypes.c_int
+    lib.mi355_w8a8_gq_pack_weight_v1.argtypes = (_vp, _vp, _u32, _u32, _u32, _vp)
+    lib.mi355_w8a8_gq_workspace_bytes.restype = _u64
+    lib.mi355_w8a8_gq_workspace_bytes.argtypes = (_u32, _u32, _u32, _u32)
+    lib.mi355_w8a8_gq_linear_v1.restype = ctypes.c_int
+    lib.mi355_w8a8_gq_linear_v1.argtypes = (ctypes.POINTER(GqProblem), _vp)
     lib.mi355_w8a8_swiglu_bwd_v1.restype = ctypes.c_int
     lib.mi355_w8a8_swiglu_bwd_v1.argtypes = (_vp, _vp, _vp, _u32, _u32, _vp)
     lib.mi355_w8a8_rms_norm_bwd_v1.restype = ctypes.c_int

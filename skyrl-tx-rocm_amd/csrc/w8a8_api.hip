@@ -13,6 +13,7 @@
 #include "w8a8_qkv_post.h"
 #include "w8a8_fused_bwd.h"
 #include "w8a8_moe.h"
+#include "w8a8_gq.h"
 
 using namespace w8a8;
 
@@ -1036,6 +1037,119 @@ int run_moe_combine(const void* expert_out, const int32_t* unsort, const float* 
   return launch_status();
 }
 
+struct GqLayout { uint64_t codes, scales, z, total; uint32_t m_pad, G; };
+
+GqLayout make_gq_layout(uint32_t m, uint32_t k_pad, uint32_t group, uint32_t rank) {
+  GqLayout L{};
+  L.m_pad = round_up(m, 32u);
+  L.G = k_pad / group;
+  uint64_t off = 0;
+  L.codes = off; off += align256((uint64_t)L.m_pad * k_pad);
+  L.scales = off; off += align256((uint64_t)L.m_pad * L.G * 4u);
+  L.z = off; off += rank ? align256((uint64_t)m * 64u * 4u) : 0u;
+  L.total = off;
+  return L;
+}
+
+int validate_gq_dims(uint32_t m, uint32_t k_pad, uint32_t group, uint32_t rank) {
+  if (m == 0 || k_pad == 0 || group == 0) return MI355_W8A8_ERR_SHAPE;
+  if ((group & 31u) || k_pad % group) return MI355_W8A8_ERR_UNSUPPORTED;
+  if (m > kMaxRows || k_pad > kMaxK || rank > (uint32_t)kMaxRank) return MI355_W8A8_ERR_UNSUPPORTED;
+  return MI355_W8A8_OK;
+}
+
+int run_gq_pack(const void* codes, void* packed, uint32_t k_pad, uint32_t n, uint32_t bits, hipStream_t s) {
+  if (!codes || !packed) return MI355_W8A8_ERR_NULL;
+  if (k_pad == 0 || n == 0 || (bits != 4u && bits != 8u)) return MI355_W8A8_ERR_SHAPE;
+  if ((k_pad & 31u) || k_pad > kMaxK || n > kMaxN) return MI355_W8A8_ERR_UNSUPPORTED;
+  if (!aligned16(packed)) return MI355_W8A8_ERR_ALIGN;
+  const uint64_t src_bytes = (uint64_t)k_pad * n / (bits == 4u ? 2u : 1u);
+  if (overlaps(packed, gq_packed_bytes(k_pad, n, bits), codes, src_bytes)) return MI355_W8A8_ERR_ALIAS;
+  GqPackArgs a{};
+  a.codes = static_cast<const unsigned char*>(codes);
+  a.packed = static_cast<unsigned char*>(packed);
+  a.k_pad = k_pad; a.n = n; a.bits = bits;
+  a.n_items = (uint64_t)((n + 31u) / 32u) * (k_pad / 32u) * 64u;
+  (void)hipGetLastError();
+  hipLaunchKernelGGL(gq_pack_weight_kernel, dim3((uint32_t)((a.n_items + 255u) / 256u)), dim3(256), 0, s, a);
+  return launch_status();
+}
+
+int run_gq_linear(const mi355_w8a8_gq_problem* p, hipStream_t s) {
+  if (!p) return MI355_W8A8_ERR_NULL;
+  if (p->struct_size != sizeof(mi355_w8a8_gq_problem)) return MI355_W8A8_ERR_STRUCT;
+  if (p->flags) return MI355_W8A8_ERR_SHAPE;
+  int st = validate_gq_dims(p->m, p->k_pad, p->group_size, p->rank);
+  if (st) return st;
+  if (p->n == 0 || p->k == 0 || p->k > p->k_pad) return MI355_W8A8_ERR_SHAPE;
+  if ((p->weight_bits != 4u && p->weight_bits != 8u) || (p->activation_bits != 4u && p->activation_bits != 8u))
+    return MI355_W8A8_ERR_SHAPE;
+  if (p->n > kMaxN || (uint64_t)p->m * p->n >= (1ull << 32)) return MI355_W8A8_ERR_UNSUPPORTED;
+  if (!p->x || !p->w_packed || !p->w_scales || !p->out) return MI355_W8A8_ERR_NULL;
+  const bool lora = p->n_adapters > 0;
+  if (lora) {
+    if (!p->lora_a || !p->lora_b || !p->lora_scaling) return MI355_W8A8_ERR_NULL;
+    if (p->rank == 0 || p->n_adapters > (uint32_t)kMaxGroups) return MI355_W8A8_ERR_UNSUPPORTED;
+  } else if (p->adapter_indices) {
+    return MI355_W8A8_ERR_SHAPE;
+  }
+  if (!aligned16(p->w_packed) || (reinterpret_cast<uintptr_t>(p->x) & 1u) || (reinterpret_cast<uintptr_t>(p->out) & 1u) ||
+      (reinterpret_cast<uintptr_t>(p->w_scales) & 3u) || (reinterpret_cast<uintptr_t>(p->adapter_indices) & 3u))
+    return MI355_W8A8_ERR_ALIGN;
+  const uint64_t out_bytes = (uint64_t)p->m * p->n * 2u;
+  if (overlaps(p->out, out_bytes, p->x, (uint64_t)p->m * p->k * 2u) ||
+      overlaps(p->out, out_bytes, p->w_packed, gq_packed_bytes(p->k_pad, p->n, p->weight_bits)) ||
+      overlaps(p->out, out_bytes, p->workspace, p->workspace_bytes))
+    return MI355_W8A8_ERR_ALIAS;
+  const GqLayout L = make_gq_layout(p->m, p->k_pad, p->group_size, lora ? p->rank : 0u);
+  if (!p->workspace || p->workspace_bytes < L.total) return MI355_W8A8_ERR_WORKSPACE;
+  if (reinterpret_cast<uintptr_t>(p->workspace) & 255u) return MI355_W8A8_ERR_ALIGN;
+  unsigned char* ws = static_cast<unsigned char*>(p->workspace);
+  (void)hipGetLastError();
+
+  GqQuantArgs q{};
+  q.x = static_cast<const uint16_t*>(p->x);
+  q.codes = reinterpret_cast<int8_t*>(ws + L.codes);
+  q.scales = reinterpret_cast<float*>(ws + L.scales);
+  q.M = p->m; q.M_pad = L.m_pad; q.K = p->k; q.K_pad = p->k_pad; q.group = p->group_size; q.G = L.G;
+  q.qmax = p->activation_bits == 4u ? 7.0f : 127.0f;
+  hipLaunchKernelGGL(gq_quant_kernel, dim3(L.m_pad / 4u), dim3(256), 0, s, q);
+  if ((st = launch_status())) return st;
+  if (p->aux_x_codes &&
+      hipMemcpyAsync(p->aux_x_codes, q.codes, (size_t)p->m * p->k_pad, hipMemcpyDeviceToDevice, s) != hipSuccess)
+    return MI355_W8A8_ERR_LAUNCH;
+  if (p->aux_x_scales &&
+      hipMemcpyAsync(p->aux_x_scales, q.scales, (size_t)p->m * L.G * 4u, hipMemcpyDeviceToDevice, s) != hipSuccess)
+    return MI355_W8A8_ERR_LAUNCH;
+
+  if (lora) {
+    GqLoraZArgs z{};
+    z.x = q.x;
+    z.lora_a = static_cast<const uint16_t*>(p->lora_a);
+    z.idx = p->adapter_indices;
+    z.z = reinterpret_cast<float*>(ws + L.z);
+    z.M = p->m; z.K = p->k; z.r = p->rank; z.n_adapters = p->n_adapters;
+    hipLaunchKernelGGL(gq_lora_z_kernel, dim3((p->m + 3u) / 4u), dim3(256), 0, s, z);
+    if ((st = launch_status())) return st;
+  }
+
+  GqGemmArgs g{};
+  g.codes = q.codes; g.xs = q.scales;
+  g.wp = static_cast<const unsigned char*>(p->w_packed);
+  g.ws = p->w_scales;
+  g.z = lora ? reinterpret_cast<const float*>(ws + L.z) : nullptr;
+  g.lora_b = static_cast<const uint16_t*>(p->lora_b);
+  g.lora_scaling = p->lora_scaling;
+  g.idx = p->adapter_indices;
+  g.out = static_cast<uint16_t*>(p->out);
+  g.aux_base = p->aux_base;
+  g.M = p->m; g.N = p->n; g.K_pad = p->k_pad; g.group = p->group_size; g.G = L.G; g.bits = p->weight_bits;
+  g.r = p->rank; g.n_adapters = p->n_adapters;
+  g.n_col_blocks = (p->n + 31u) / 32u;
+  hipLaunchKernelGGL(gq_gemm_kernel, dim3((g.n_col_blocks + 3u) / 4u, L.m_pad / 32u), dim3(256), 0, s, g);
+  return launch_status();
+}
+
 }  // namespace
 
 extern "C" {
@@ -1187,6 +1301,25 @@ int mi355_w8a8_moe_combine_v1(const void* expert_out, const int32_t* unsort_indi
                               uint32_t n_tokens, uint32_t top_k, uint32_t width, void* stream) {
   return run_moe_combine(expert_out, unsort_indices, weights, out, n_tokens, top_k, width,
                          static_cast<hipStream_t>(stream));
+}
+
+uint64_t mi355_w8a8_gq_packed_weight_bytes(uint32_t k_pad, uint32_t n, uint32_t weight_bits) {
+  if (k_pad == 0 || (k_pad & 31u) || n == 0 || (weight_bits != 4u && weight_bits != 8u)) return 0;
+  return gq_packed_bytes(k_pad, n, weight_bits);
+}
+
+int mi355_w8a8_gq_pack_weight_v1(const void* codes, void* packed, uint32_t k_pad, uint32_t n, uint32_t weight_bits,
+                                 void* stream) {
+  return run_gq_pack(codes, packed, k_pad, n, weight_bits, static_cast<hipStream_t>(stream));
+}
+
+uint64_t mi355_w8a8_gq_workspace_bytes(uint32_t m, uint32_t k_pad, uint32_t group_size, uint32_t rank) {
+  if (validate_gq_dims(m, k_pad, group_size, rank)) return 0;
+  return make_gq_layout(m, k_pad, group_size, rank).total;
+}
+
+int mi355_w8a8_gq_linear_v1(const mi355_w8a8_gq_problem* p, void* stream) {
+  return run_gq_linear(p, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

@@ -4,9 +4,10 @@ Mirrors the interface of the reference's ``skyrl/tx/kernels/quantized_lora.py``
 (``GroupQuantizedWeight`` :20-41, ``quantize_frozen_weight`` :128-171,
 ``dequantize_frozen_weight`` :180-196, ``quantized_frozen_linear`` :257-272,
 ``quantized_lora_linear`` :400-453) on torch tensors.  The forward functions run the
-gfx950 HIP kernels; they accept the per-token / per-channel geometry
-(``bits == 8``, ``group_size == K``, ``activation_bits == 8``) and raise
-``ValueError`` for anything else so a caller can keep its own path for those.
+gfx950 HIP kernels: the per-token / per-channel geometry (``bits == 8``,
+``group_size == K``, ``activation_bits == 8``) takes the tiled / streaming W8A8
+kernels, every other geometry of the format with ``group_size % 32 == 0`` (W4 codes,
+scales per K group, A4 activations) the group-scaled kernels of ``rocm/gq_linear.py``.
 The weight quantizer is an offline, one-time torch computation.
 """
 
@@ -127,30 +128,31 @@ def dequantize_frozen_weight(weight: GroupQuantizedWeight, *, dtype: torch.dtype
     return deq.reshape(weight.padded_in_features, n)[: weight.original_in_features].to(dtype)
 
 
-def _require_native_geometry(weight: GroupQuantizedWeight, activation_bits: int) -> None:
+def _is_per_channel_w8a8(weight: GroupQuantizedWeight, activation_bits: int) -> bool:
+    """True for the geometry of the fast W8A8 kernels; validates the arguments either way."""
     _validate_bits(activation_bits)
     validate_quantized_weight(weight)
-    if weight.bits != 8 or activation_bits != 8:
-        raise ValueError("the MI355X path implements W8A8 only")
-    if weight.group_size != weight.padded_in_features or weight.padded_in_features != weight.original_in_features:
-        raise ValueError("the MI355X path implements per-token / per-channel scales (group_size == K) only")
+    return (weight.bits == 8 and activation_bits == 8 and weight.group_size == weight.padded_in_features
+            and weight.padded_in_features == weight.original_in_features)
 
 
 def quantized_frozen_linear(x: torch.Tensor, weight: GroupQuantizedWeight, *, activation_bits: int = 8):
-    from .rocm import w8a8_lora
+    from .rocm import gq_linear, w8a8_lora
 
-    _require_native_geometry(weight, activation_bits)
+    per_channel = _is_per_channel_w8a8(weight, activation_bits)
     if not x.dtype.is_floating_point:
         raise TypeError(f"activations must be floating point, got {x.dtype}")
-    return w8a8_lora.w8a8_frozen_linear(x, weight, enabled=True)
+    if per_channel:
+        return w8a8_lora.w8a8_frozen_linear(x, weight, enabled=True)
+    return gq_linear.forward(x, weight, activation_bits=activation_bits)
 
 
 def quantized_lora_linear(x: torch.Tensor, weight: GroupQuantizedWeight, lora_a: torch.Tensor,
                           lora_b: torch.Tensor, lora_scaling, *, activation_bits: int = 8) -> torch.Tensor:
     """Frozen W8A8 linear plus LoRA: bf16(base_f32 + ((x @ A) @ B) * s), one cast."""
-    from .rocm import w8a8_lora
+    from .rocm import gq_linear, w8a8_lora
 
-    _require_native_geometry(weight, activation_bits)
+    per_channel = _is_per_channel_w8a8(weight, activation_bits)
     if x.ndim < 1:
         raise ValueError(f"activations must have at least one dimension, got {tuple(x.shape)}")
     if not x.dtype.is_floating_point:
@@ -168,4 +170,6 @@ def quantized_lora_linear(x: torch.Tensor, weight: GroupQuantizedWeight, lora_a:
     scaling = torch.as_tensor(lora_scaling, dtype=torch.float32)
     if scaling.ndim != 0:
         raise ValueError(f"lora_scaling must be scalar, got {tuple(scaling.shape)}")
-    return w8a8_lora.w8a8_lora_linear(x, weight, lora_a, lora_b, scaling, enabled=True)
+    if per_channel:
+        return w8a8_lora.w8a8_lora_linear(x, weight, lora_a, lora_b, scaling, enabled=True)
+    return gq_linear.forward(x, weight, lora_a, lora_b, scaling, activation_bits=activation_bits)

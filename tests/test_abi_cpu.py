@@ -165,9 +165,16 @@ def test_python_surface_fails_loudly_on_cpu(native):
     w64 = ql.quantize_frozen_weight(torch.randn(128, 16), bits=8, group_size=64)
     with pytest.raises(ValueError, match="per-channel"):
         w8.prepare_weight(w64)
-    with pytest.raises(ValueError, match="W8A8 only"):
-        ql.quantized_lora_linear(x, ql.quantize_frozen_weight(torch.randn(64, 16), bits=4, group_size=64),
-                                 torch.zeros(64, 4), torch.zeros(4, 16), 1.0)
+    # W4 / grouped scales go to the group-scaled kernels, which refuse CPU tensors just the same
+    w4 = ql.quantize_frozen_weight(torch.randn(64, 16), bits=4, group_size=64)
+    with pytest.raises(RuntimeError, match="GPU"):
+        ql.quantized_lora_linear(x, w4, torch.zeros(64, 4, dtype=torch.bfloat16),
+                                 torch.zeros(4, 16, dtype=torch.bfloat16), 1.0)
+    with pytest.raises(RuntimeError, match="GPU"):
+        ql.quantized_frozen_linear(x, ql.quantize_frozen_weight(torch.randn(64, 16), bits=8, group_size=32),
+                                   activation_bits=4)
+    with pytest.raises(ValueError, match="bits must be 4 or 8"):
+        ql.quantized_frozen_linear(x, w4, activation_bits=5)
 
 
 def test_host_quantizer_matches_oracle():

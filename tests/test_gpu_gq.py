@@ -1,0 +1,162 @@
+"""GPU parity of the group-scaled quantized linear (W4 / W8 codes, A4 / A8 activations, scales per K
+group) through the C ABI, against the CPU oracle and the reference's hand-coded W4A4 case.
+
+Bar: activation codes, activation scales and the float32 base (the sum over the groups before the
+LoRA term) bit for bit; the bf16 output bit for bit without LoRA and to |a - b| <= 2e-2 + 1e-2 |b|
+with it (the float32 summation order of the two small LoRA products differs).
+"""
+
+import numpy as np
+import pytest
+
+from oracle import w8a8_oracle as o
+import w8a8_cases as wc
+
+pytestmark = pytest.mark.gpu
+F32 = np.float32
+
+
+@pytest.fixture(scope="module")
+def dev():
+    torch = pytest.importorskip("torch")
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return torch.device("cuda:0")
+
+
+@pytest.fixture(scope="module")
+def pkg():
+    from __graft_entry__ import load_package
+
+    p = load_package()
+    p._native.load()
+    return p
+
+
+def _to_dev(pkg, dev, w):
+    import torch
+
+    return pkg.quantized_lora.GroupQuantizedWeight(torch.from_numpy(w.codes).to(dev), torch.from_numpy(w.scales).to(dev),
+                                                   w.original_in_features, w.padded_in_features, w.bits, w.group_size)
+
+
+def _bf(dev, v):
+    import torch
+
+    return torch.from_numpy(np.ascontiguousarray(v)).to(dev).to(torch.bfloat16)
+
+
+def test_reference_hand_coded_w4a4_case(dev, pkg):
+    """tests/tx/kernels/test_quantized_lora.py:58-74 (groups of 2) embedded in groups of 32: every
+    group is followed by 30 zero weights and zero activations, which changes no amax, code or sum."""
+    import torch
+
+    small = o.GroupQuantizedWeight(codes=np.asarray([[0x31, 0x4E], [0x0B, 0x96]], dtype=np.uint8),
+                                   scales=np.asarray([[0.5, 2.0], [1.5, 0.25]], dtype=F32), original_in_features=3,
+                                   padded_in_features=4, bits=4, group_size=2)
+    x_small = np.asarray([[7.0, -3.0, -7.0], [0.0, 0.0, 3.0]], dtype=F32)
+    expected = np.asarray([[51.5, -62.5], [-22.5, 4.5]], dtype=F32)
+    np.testing.assert_allclose(o.quantized_frozen_linear_f32(x_small, small, activation_bits=4), expected, rtol=1e-6)
+    codes = np.zeros((64, 2), dtype=np.int8)
+    codes[[0, 1, 32, 33]] = o.unpack_signed_int4(small.codes)
+    x = np.zeros((2, 64), dtype=F32)
+    x[:, [0, 1, 32]] = x_small
+    big = o.GroupQuantizedWeight(codes=o.pack_signed_int4(codes), scales=small.scales, original_in_features=64,
+                                 padded_in_features=64, bits=4, group_size=32)
+    got, aux = pkg.gq_linear.forward(_bf(dev, x), _to_dev(pkg, dev, big), activation_bits=4, return_aux=True)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(aux["base"].cpu().numpy(), expected)
+    np.testing.assert_array_equal(got.to(torch.float32).cpu().numpy(), expected)
+    via_api = pkg.quantized_lora.quantized_frozen_linear(_bf(dev, x), _to_dev(pkg, dev, big), activation_bits=4)
+    assert torch.equal(via_api, got)
+
+
+CASES = [
+    # m, k, n, weight bits, activation bits, group, rank, adapters
+    (5, 64, 17, 4, 8, 32, 0, 0),
+    (33, 200, 96, 4, 4, 64, 8, 1),        # K padded to 256
+    (70, 512, 264, 8, 8, 128, 16, 3),     # W8 with grouped scales, three adapters
+    (16, 1024, 520, 4, 8, 64, 32, 4),
+    (128, 384, 130, 8, 4, 96, 0, 0),      # group of three k blocks, A4
+    (300, 2048, 256, 4, 8, 2048, 64, 2),  # one group: per-channel W4
+]
+
+
+@pytest.mark.parametrize("m,k,n,wb,ab,group,rank,n_ad", CASES)
+def test_gq_linear_matches_oracle(dev, pkg, m, k, n, wb, ab, group, rank, n_ad):
+    import torch
+
+    rng = np.random.default_rng(m * 7 + k + n)
+    x = o.bf16_round(rng.standard_t(4, (m, k)).astype(F32))
+    w = o.quantize_frozen_weight((rng.standard_normal((k, n)) * 0.05).astype(F32), bits=wb, group_size=group,
+                                 scale_dtype="f32")
+    print(f"[case] gq linear m={m} k={k} n={n} W{wb}A{ab} group={group} rank={rank} adapters={n_ad}", flush=True)
+    base, x_codes, x_scales, _ = o.quantized_frozen_linear_f32(x, w, activation_bits=ab, return_parts=True)
+    a = b = s = idx = None
+    want_f32 = base
+    if n_ad:
+        a = o.bf16_round((rng.standard_normal((n_ad, k, rank)) * 0.05).astype(F32))
+        b = o.bf16_round((rng.standard_normal((n_ad, rank, n)) * 0.05).astype(F32))
+        s = rng.uniform(0.5, 2.0, n_ad).astype(F32)
+        idx = rng.integers(0, n_ad, m).astype(np.int32)
+        want_f32 = (base + o.lora_delta_multi(x, a, b, s, idx)).astype(F32)
+    got, aux = pkg.gq_linear.forward(_bf(dev, x), _to_dev(pkg, dev, w), None if a is None else _bf(dev, a),
+                                     None if b is None else _bf(dev, b),
+                                     None if s is None else torch.from_numpy(s).to(dev), activation_bits=ab,
+                                     adapter_indices=None if idx is None else torch.from_numpy(idx).to(dev),
+                                     return_aux=True)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(aux["x_codes"].cpu().numpy(), x_codes.reshape(m, -1))
+    np.testing.assert_array_equal(aux["x_scales"].cpu().numpy().view(np.uint32), x_scales.view(np.uint32))
+    np.testing.assert_array_equal(aux["base"].cpu().numpy().view(np.uint32), base.view(np.uint32))
+    got_np = got.to(torch.float32).cpu().numpy()
+    want = o.bf16_round(want_f32)
+    if not n_ad:
+        np.testing.assert_array_equal(o.bf16_bits(got_np), o.bf16_bits(want))
+    rep = wc.compare(got_np, want)
+    print(f"[gq parity] m{m}k{k}n{n} W{wb}A{ab} {rep}", flush=True)
+    assert rep["violations"] == 0, rep
+
+
+def test_gq_single_adapter_through_the_reference_entry_point(dev, pkg):
+    import torch
+
+    rng = np.random.default_rng(9)
+    m, k, n, r = 24, 256, 64, 8
+    x = o.bf16_round(rng.standard_normal((2, m // 2, k)).astype(F32))
+    w = o.quantize_frozen_weight(rng.standard_normal((k, n)).astype(F32) * 0.1, bits=4, group_size=64)   # bf16 scales
+    a = o.bf16_round((rng.standard_normal((k, r)) * 0.1).astype(F32))
+    b = o.bf16_round((rng.standard_normal((r, n)) * 0.1).astype(F32))
+    want = o.quantized_lora_linear(x, w, a, b, F32(0.75), activation_bits=8)
+    import torch as _t
+    wt = pkg.quantized_lora.GroupQuantizedWeight(_t.from_numpy(w.codes).to(dev),
+                                                 _t.from_numpy(w.scales).to(dev).to(_t.bfloat16), k, k, 4, 64)
+    got = pkg.quantized_lora.quantized_lora_linear(_bf(dev, x), wt, _bf(dev, a), _bf(dev, b), 0.75)
+    torch.cuda.synchronize()
+    assert tuple(got.shape) == (2, m // 2, n)
+    rep = wc.compare(got.to(torch.float32).cpu().numpy(), want)
+    assert rep["violations"] == 0, rep
+
+
+def test_gq_pack_keeps_four_bits_and_rejects_bad_geometry(dev, pkg):
+    import torch
+
+    lib = pkg._native.load()
+    assert lib.mi355_w8a8_gq_packed_weight_bytes(64, 32, 4) == 2 * 512
+    assert lib.mi355_w8a8_gq_packed_weight_bytes(64, 33, 8) == 2 * 2 * 1024
+    assert lib.mi355_w8a8_gq_packed_weight_bytes(48, 32, 4) == 0
+    assert lib.mi355_w8a8_gq_workspace_bytes(4, 64, 10, 0) == 0
+    w = o.quantize_frozen_weight(np.ones((70, 8), F32), bits=4, group_size=14, scale_dtype="f32")
+    with pytest.raises(ValueError, match="group_size % 32"):
+        pkg.gq_linear.forward(torch.zeros(2, 70, dtype=torch.bfloat16, device=dev), _to_dev(pkg, dev, w))
+    w = o.quantize_frozen_weight(np.ones((64, 8), F32), bits=4, group_size=32, scale_dtype="f32")
+    wt = _to_dev(pkg, dev, w)
+    with pytest.raises(ValueError):
+        pkg.gq_linear.forward(torch.zeros(2, 60, dtype=torch.bfloat16, device=dev), wt)
+    with pytest.raises(TypeError):
+        pkg.gq_linear.forward(torch.zeros(2, 64, dtype=torch.float32, device=dev), wt)
+    with pytest.raises(ValueError):
+        pkg.gq_linear.forward(torch.zeros(2, 64, dtype=torch.bfloat16, device=dev), wt, activation_bits=5)
+    with pytest.raises(ValueError):
+        pkg.gq_linear.forward(torch.zeros(2, 64, dtype=torch.bfloat16, device=dev), wt,
+                              adapter_indices=torch.zeros(2, dtype=torch.int32, device=dev))
