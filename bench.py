@@ -53,6 +53,10 @@ WORKLOADS = {
     # combine; rank-16 LoRA on every expert
     "qwen3-30b-a3b-moe-mlp-t2048": dict(m=2048, n_experts=128, top_k=8, hidden=2048, intermediate=768, rank=16,
                                         seed=5, moe_mlp=True),
+    # group-scaled W4A8 (int4 codes, one scale per 128 k and output, activations quantized per row and group)
+    # at the Qwen3-8B down-projection shape, 8 adapters rank 32
+    "qwen3-8b-down-m4096-w4a8-g128": dict(m=4096, k=12288, n=4096, n_adapters=8, rank=32, weight_bits=4,
+                                          activation_bits=8, group_size=128, seed=8, gq=True),
     # Qwen3.5-4B attention input stage: RMSNorm -> W8A8 QKV [2560 -> 10240] + 4 adapters rank 64 ->
     # split, Q/K RMSNorm, partial RoPE (16 query heads, 4 kv heads, head_dim 256, 64 rotary dims)
     "qwen3.5-4b-qkv-m2048": dict(m=2048, k=2560, n=10240, n_adapters=4, rank=64, alpha=128, rms=True,
@@ -499,6 +503,79 @@ def bench_moe_mlp(args, cfg, pkg, dev):
     return 0
 
 
+def bench_gq(args, cfg, pkg, dev):
+    """One step = one group-scaled quantized linear call (quantizer, LoRA z, GEMM with the group
+    epilogue).  ``value`` counts 2*M*K*N; the roofline prices gq_gemm_kernel against int8 MFMA peak from
+    HIP events around whole calls minus nothing -- the call is that kernel plus two short ones, so the
+    figure is a lower bound for the kernel."""
+    import torch
+
+    import w8a8_cases as wc
+    from oracle import w8a8_oracle as o
+
+    gq, ql = pkg.gq_linear, pkg.quantized_lora
+    m, k, n, r, n_ad = cfg["m"], cfg["k"], cfg["n"], cfg["rank"], cfg["n_adapters"]
+    wb, ab, group = cfg["weight_bits"], cfg["activation_bits"], cfg["group_size"]
+    rng = np.random.default_rng(cfg["seed"])
+    x = o.bf16_round(rng.standard_normal((m, k)).astype(np.float32))
+    dense = (rng.standard_normal((k, n)) * 0.05).astype(np.float32)
+    w = o.quantize_frozen_weight(dense, bits=wb, group_size=group, scale_dtype="f32")
+    a = o.bf16_round((rng.standard_normal((n_ad, k, r)) * 0.02).astype(np.float32))
+    b = o.bf16_round((rng.standard_normal((n_ad, r, n)) * 0.02).astype(np.float32))
+    s = np.ones(n_ad, np.float32)
+    idx = rng.integers(0, n_ad, m).astype(np.int32)
+    bf = lambda t: torch.from_numpy(np.ascontiguousarray(t)).to(dev).to(torch.bfloat16)
+    wt = gq.prepare_group_weight(ql.GroupQuantizedWeight(torch.from_numpy(w.codes).to(dev),
+                                                         torch.from_numpy(w.scales).to(dev), k, w.padded_in_features,
+                                                         wb, group))
+    x_t, a_t, b_t = bf(x), bf(a), bf(b)
+    s_t, idx_t = torch.from_numpy(s).to(dev), torch.from_numpy(idx).to(dev)
+    step = lambda: gq.forward(x_t, wt, a_t, b_t, s_t, activation_bits=ab, adapter_indices=idx_t)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        got = step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for e0, e1 in ev:
+        e0.record()
+        step()
+        e1.record()
+    torch.cuda.synchronize()
+    call_ms = float(np.mean([e0.elapsed_time(e1) for e0, e1 in ev]))
+    ops = 2.0 * m * k * n
+    achieved = ops / (call_ms * 1e-3) / 1e12
+    result = {
+        "metric": f"group-scaled W{wb}A{ab} LoRA linear forward (group {group}), TOPS of 2*M*K*N per call",
+        "value": ops / (ms_per_step * 1e-3) / 1e12, "unit": "TOPS", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                     "frac": achieved / INT8_PEAK_TOPS, "traffic": None,
+                     "kernel": "gq_gemm_kernel (timed with gq_quant_kernel and gq_lora_z_kernel: whole calls)",
+                     "kernel_avg_ms": call_ms, "algorithmic_ops": ops,
+                     "algorithmic_bytes": 2 * m * k + k * n * wb // 8 + 4 * (k // group) * n + 2 * m * n},
+    }
+    if not args.no_cpu_baseline:
+        rows = args.cpu_rows or 128
+        t1 = time.perf_counter()
+        want = o.bf16_round(o.quantized_frozen_linear_f32(x[:rows], w, activation_bits=ab)
+                            + o.lora_delta_multi(x[:rows], a, b, s, idx[:rows]))
+        secs = time.perf_counter() - t1
+        result["cpu_baseline"] = {"value": 2.0 * rows * k * n / secs / 1e12, "unit": "TOPS", "cores": 1, "kind": "port",
+                                  "sample": f"first {rows} of {m} rows, full K and N, NumPy oracle (group by group), "
+                                            f"one run, {secs:.3f} s", "seconds": secs}
+        rep = wc.compare(got[:rows].to(torch.float32).cpu().numpy(), want)
+        result["parity_sample"] = {"rows": rows, "violations": rep["violations"], "size": rep["size"],
+                                   "max_abs": rep["max_abs"], "bitwise_fraction": rep["bitwise_fraction"]}
+    print(json.dumps(result))
+    return 0
+
+
 def bench_qkv(args, cfg, pkg, dev):
     """One step = the W8A8 QKV projection (RMSNorm prologue, GEMM, LoRA) + the split / Q-K norm /
     RoPE kernel.  ``value`` is int8 TOPS of the projection over the whole step; the roofline prices
@@ -629,6 +706,8 @@ def main() -> int:
         if cfg.get("swiglu"):
             return bench_fused_backward(args, cfg, pkg, dev)
         return bench_backward(args, cfg, pkg, dev)
+    if cfg.pop("gq", False):
+        return bench_gq(args, cfg, pkg, dev)
     if cfg.pop("moe_mlp", False):
         return bench_moe_mlp(args, cfg, pkg, dev)
     if cfg.pop("moe_routing", False):

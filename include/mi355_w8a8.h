@@ -372,7 +372,8 @@ typedef struct mi355_w8a8_gq_problem {
   float* aux_base;           /* f32 [m, n]: the float32 base before the LoRA term */
 } mi355_w8a8_gq_problem;
 
-uint64_t mi355_w8a8_gq_workspace_bytes(uint32_t m, uint32_t k_pad, uint32_t group_size, uint32_t rank);
+uint64_t mi355_w8a8_gq_workspace_bytes(uint32_t m, uint32_t k_pad, uint32_t group_size, uint32_t n_adapters,
+                                       uint32_t rank);
 int mi355_w8a8_gq_linear_v1(const mi355_w8a8_gq_problem* problem, void* stream);
 
 #ifdef __cplusplus

@@ -173,7 +173,7 @@ def _bind(lib: ctypes.CDLL) -> None:
     lib.mi355_w8a8_gq_pack_weight_v1.restype = ctypes.c_int
     lib.mi355_w8a8_gq_pack_weight_v1.argtypes = (_vp, _vp, _u32, _u32, _u32, _vp)
     lib.mi355_w8a8_gq_workspace_bytes.restype = _u64
-    lib.mi355_w8a8_gq_workspace_bytes.argtypes = (_u32, _u32, _u32, _u32)
+    lib.mi355_w8a8_gq_workspace_bytes.argtypes = (_u32, _u32, _u32, _u32, _u32)
     lib.mi355_w8a8_gq_linear_v1.restype = ctypes.c_int
     lib.mi355_w8a8_gq_linear_v1.argtypes = (ctypes.POINTER(GqProblem), _vp)
     lib.mi355_w8a8_swiglu_bwd_v1.restype = ctypes.c_int

@@ -1037,16 +1037,21 @@ int run_moe_combine(const void* expert_out, const int32_t* unsort, const float* 
   return launch_status();
 }
 
-struct GqLayout { uint64_t codes, scales, z, total; uint32_t m_pad, G; };
+struct GqLayout { uint64_t codes, scales, z, src_row, dst_pos, slot_group, blk_range, at, total; uint32_t m_pad, G; };
 
-GqLayout make_gq_layout(uint32_t m, uint32_t k_pad, uint32_t group, uint32_t rank) {
+GqLayout make_gq_layout(uint32_t m, uint32_t k_pad, uint32_t group, uint32_t n_adapters, uint32_t rank) {
   GqLayout L{};
   L.m_pad = round_up(m, 32u);
   L.G = k_pad / group;
   uint64_t off = 0;
   L.codes = off; off += align256((uint64_t)L.m_pad * k_pad);
   L.scales = off; off += align256((uint64_t)L.m_pad * L.G * 4u);
-  L.z = off; off += rank ? align256((uint64_t)m * 64u * 4u) : 0u;
+  L.z = off; off += rank ? align256((uint64_t)L.m_pad * 64u * 4u) : 0u;
+  L.src_row = off; off += rank ? align256((uint64_t)L.m_pad * 4u) : 0u;
+  L.dst_pos = off; off += rank ? align256((uint64_t)L.m_pad * 4u) : 0u;
+  L.slot_group = off; off += rank ? align256((uint64_t)L.m_pad * 4u) : 0u;
+  L.blk_range = off; off += rank ? align256((uint64_t)(L.m_pad / 32u) * 4u) : 0u;
+  L.at = off; off += (rank && n_adapters <= (uint32_t)kMaxAdapters) ? align256((uint64_t)n_adapters * rank * k_pad * 2u) : 0u;
   L.total = off;
   return L;
 }
@@ -1101,7 +1106,7 @@ int run_gq_linear(const mi355_w8a8_gq_problem* p, hipStream_t s) {
       overlaps(p->out, out_bytes, p->w_packed, gq_packed_bytes(p->k_pad, p->n, p->weight_bits)) ||
       overlaps(p->out, out_bytes, p->workspace, p->workspace_bytes))
     return MI355_W8A8_ERR_ALIAS;
-  const GqLayout L = make_gq_layout(p->m, p->k_pad, p->group_size, lora ? p->rank : 0u);
+  const GqLayout L = make_gq_layout(p->m, p->k_pad, p->group_size, p->n_adapters, lora ? p->rank : 0u);
   if (!p->workspace || p->workspace_bytes < L.total) return MI355_W8A8_ERR_WORKSPACE;
   if (reinterpret_cast<uintptr_t>(p->workspace) & 255u) return MI355_W8A8_ERR_ALIGN;
   unsigned char* ws = static_cast<unsigned char*>(p->workspace);
@@ -1111,25 +1116,64 @@ int run_gq_linear(const mi355_w8a8_gq_problem* p, hipStream_t s) {
   q.x = static_cast<const uint16_t*>(p->x);
   q.codes = reinterpret_cast<int8_t*>(ws + L.codes);
   q.scales = reinterpret_cast<float*>(ws + L.scales);
+  q.codes_rm = p->aux_x_codes; q.scales_rm = p->aux_x_scales;
   q.M = p->m; q.M_pad = L.m_pad; q.K = p->k; q.K_pad = p->k_pad; q.group = p->group_size; q.G = L.G;
   q.qmax = p->activation_bits == 4u ? 7.0f : 127.0f;
   hipLaunchKernelGGL(gq_quant_kernel, dim3(L.m_pad / 4u), dim3(256), 0, s, q);
   if ((st = launch_status())) return st;
-  if (p->aux_x_codes &&
-      hipMemcpyAsync(p->aux_x_codes, q.codes, (size_t)p->m * p->k_pad, hipMemcpyDeviceToDevice, s) != hipSuccess)
-    return MI355_W8A8_ERR_LAUNCH;
-  if (p->aux_x_scales &&
-      hipMemcpyAsync(p->aux_x_scales, q.scales, (size_t)p->m * L.G * 4u, hipMemcpyDeviceToDevice, s) != hipSuccess)
-    return MI355_W8A8_ERR_LAUNCH;
 
-  if (lora) {
+  // z = x @ A[idx]: rows routed by adapter and multiplied on the matrix core (the kernels of the
+  // per-channel path) when the adapter count and K allow it, else one wave per row
+  const bool fast_z = lora && p->n_adapters <= (uint32_t)kMaxAdapters && (p->k & 7u) == 0 && aligned16(p->x) &&
+                      aligned16(p->lora_a);
+  const bool routed = fast_z && p->adapter_indices && p->n_adapters > 1u;
+  int32_t* dst_pos = reinterpret_cast<int32_t*>(ws + L.dst_pos);
+  if (fast_z) {
+    int32_t* src_row = reinterpret_cast<int32_t*>(ws + L.src_row);
+    int32_t* slot_group = reinterpret_cast<int32_t*>(ws + L.slot_group);
+    int32_t* blk_range = reinterpret_cast<int32_t*>(ws + L.blk_range);
+    uint16_t* at = reinterpret_cast<uint16_t*>(ws + L.at);
+    LoraPrepArgs pa{};
+    pa.idx = routed ? p->adapter_indices : nullptr;
+    pa.src_row = src_row; pa.dst_pos = dst_pos; pa.slot_group = slot_group; pa.blk_range = blk_range;
+    pa.lora_a = static_cast<const uint16_t*>(p->lora_a);
+    pa.at = at;
+    pa.M = p->m; pa.K = p->k; pa.N = p->n; pa.n_groups = p->n_adapters; pa.r = p->rank;
+    pa.slots = L.m_pad;
+    pa.route_blocks = routed ? 1u : 0u;
+    const uint64_t a_items = (uint64_t)p->n_adapters * p->k * ((p->rank + 7u) / 8u);
+    pa.a_blocks = (uint32_t)((a_items + 1023u) / 1024u);
+    hipLaunchKernelGGL(lora_prep_kernel, dim3(pa.route_blocks + pa.a_blocks), dim3(1024), 0, s, pa);
+    if ((st = launch_status())) return st;
+    LoraAArgs la{};
+    la.xsrc = q.x;
+    la.at = at;
+    la.src_row = routed ? src_row : nullptr;
+    la.slot_group = routed ? slot_group : nullptr;
+    la.blk_range = routed ? blk_range : nullptr;
+    la.zp = nullptr;
+    la.zf = reinterpret_cast<float*>(ws + L.z);
+    la.zf_stride = 64u;
+    la.M = p->m; la.K = p->k; la.r = p->rank; la.nkk = rank_chunks(p->rank);
+    la.n_steps = (p->k + 63u) / 64u; la.steps_per_wave = (la.n_steps + 15u) / 16u;
+    la.nterms = 3u;
+    la.n_blocks = L.m_pad / 32u;
+    const dim3 zgrid(L.m_pad / 32u), zblock(1024);
+    if (la.nkk > 2u) hipLaunchKernelGGL((lora_a_kernel<2>), zgrid, zblock, 0, s, la);
+    else hipLaunchKernelGGL((lora_a_kernel<1>), zgrid, zblock, 0, s, la);
+    if ((st = launch_status())) return st;
+  } else if (lora) {
     GqLoraZArgs z{};
     z.x = q.x;
     z.lora_a = static_cast<const uint16_t*>(p->lora_a);
     z.idx = p->adapter_indices;
     z.z = reinterpret_cast<float*>(ws + L.z);
     z.M = p->m; z.K = p->k; z.r = p->rank; z.n_adapters = p->n_adapters;
-    hipLaunchKernelGGL(gq_lora_z_kernel, dim3((p->m + 3u) / 4u), dim3(256), 0, s, z);
+    const dim3 zgrid((p->m + 3u) / 4u), zblock(256);
+    if (p->rank <= 8u) hipLaunchKernelGGL((gq_lora_z_kernel<1>), zgrid, zblock, 0, s, z);
+    else if (p->rank <= 16u) hipLaunchKernelGGL((gq_lora_z_kernel<2>), zgrid, zblock, 0, s, z);
+    else if (p->rank <= 32u) hipLaunchKernelGGL((gq_lora_z_kernel<4>), zgrid, zblock, 0, s, z);
+    else hipLaunchKernelGGL((gq_lora_z_kernel<8>), zgrid, zblock, 0, s, z);
     if ((st = launch_status())) return st;
   }
 
@@ -1138,15 +1182,19 @@ int run_gq_linear(const mi355_w8a8_gq_problem* p, hipStream_t s) {
   g.wp = static_cast<const unsigned char*>(p->w_packed);
   g.ws = p->w_scales;
   g.z = lora ? reinterpret_cast<const float*>(ws + L.z) : nullptr;
+  g.z_slot = routed ? dst_pos : nullptr;
   g.lora_b = static_cast<const uint16_t*>(p->lora_b);
   g.lora_scaling = p->lora_scaling;
   g.idx = p->adapter_indices;
   g.out = static_cast<uint16_t*>(p->out);
   g.aux_base = p->aux_base;
-  g.M = p->m; g.N = p->n; g.K_pad = p->k_pad; g.group = p->group_size; g.G = L.G; g.bits = p->weight_bits;
+  g.M = p->m; g.M_pad = L.m_pad; g.N = p->n; g.K_pad = p->k_pad; g.group = p->group_size; g.G = L.G;
+  g.bits = p->weight_bits;
   g.r = p->rank; g.n_adapters = p->n_adapters;
   g.n_col_blocks = (p->n + 31u) / 32u;
-  hipLaunchKernelGGL(gq_gemm_kernel, dim3((g.n_col_blocks + 3u) / 4u, L.m_pad / 32u), dim3(256), 0, s, g);
+  const dim3 grid((g.n_col_blocks + 7u) / 8u, (L.m_pad / 32u + 1u) / 2u), block(256);
+  if (p->weight_bits == 4u) hipLaunchKernelGGL((gq_gemm_kernel<true>), grid, block, 0, s, g);
+  else hipLaunchKernelGGL((gq_gemm_kernel<false>), grid, block, 0, s, g);
   return launch_status();
 }
 
@@ -1313,9 +1361,10 @@ int mi355_w8a8_gq_pack_weight_v1(const void* codes, void* packed, uint32_t k_pad
   return run_gq_pack(codes, packed, k_pad, n, weight_bits, static_cast<hipStream_t>(stream));
 }
 
-uint64_t mi355_w8a8_gq_workspace_bytes(uint32_t m, uint32_t k_pad, uint32_t group_size, uint32_t rank) {
+uint64_t mi355_w8a8_gq_workspace_bytes(uint32_t m, uint32_t k_pad, uint32_t group_size, uint32_t n_adapters,
+                                       uint32_t rank) {
   if (validate_gq_dims(m, k_pad, group_size, rank)) return 0;
-  return make_gq_layout(m, k_pad, group_size, rank).total;
+  return make_gq_layout(m, k_pad, group_size, n_adapters, n_adapters ? rank : 0u).total;
 }
 
 int mi355_w8a8_gq_linear_v1(const mi355_w8a8_gq_problem* p, void* stream) {

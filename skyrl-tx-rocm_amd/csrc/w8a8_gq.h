@@ -13,7 +13,7 @@
 //   gq_pack_weight_kernel  reference layout -> matrix-core fragments, 4-bit codes stay 4-bit
 //   gq_quant_kernel        per (row, group): amax, scale, codes (row-major int8, rows padded to 32)
 //   gq_lora_z_kernel       z = x @ A[idx] in float32
-//   gq_gemm_kernel         one wave per 32 x 32 output block over all groups, epilogue, store
+//   gq_gemm_kernel         one wave per 64 x 64 output tile over all groups, epilogue, store
 #pragma once
 #include "w8a8_device.h"
 
@@ -68,39 +68,77 @@ __global__ __launch_bounds__(256) void gq_pack_weight_kernel(GqPackArgs a) {
 // ---------------------------------------------------------------------------------------
 struct GqQuantArgs {
   const uint16_t* x;   // bf16 [M, K]
-  int8_t* codes;       // int8 [M_pad, K_pad]; rows >= M and columns >= K hold zeros
-  float* scales;       // f32 [M_pad, G]
+  int8_t* codes;       // matrix-core fragments [M_pad / 32][K_pad / 32][1 KiB]: lane l = row l % 32,
+                       // k = 16 (l / 32) + 0..15; rows >= M and columns >= K hold zeros
+  float* scales;       // f32 [G, M_pad]
+  int8_t* codes_rm;    // optional row-major copy int8 [M, K_pad]
+  float* scales_rm;    // optional row-major copy f32 [M, G]
   uint32_t M, M_pad, K, K_pad, group, G;
   float qmax;          // 127 or 7
 };
 
 // scale = amax > 0 ? amax / qmax : 1, code = clip(rint(x / scale), -qmax, qmax), IEEE float32
-// division, round half to even (quantized_lora.py:199-212).  One wave per row, group after group.
+// division, round half to even (quantized_lora.py:199-212).  One wave per row, three passes over
+// pieces of 8 consecutive k: the pieces' maxima go to LDS, every lane then forms the scales of its
+// groups from them, and the pieces are quantized with their group's scale (K_pad <= 16384).
+constexpr uint32_t kGqMaxPieces = 2048, kGqMaxGroups = 512;
+
+__device__ inline void gq_load_piece(const GqQuantArgs& a, const uint16_t* xr, bool live, uint32_t k, float (&v)[8]) {
+  if (live && k + 8u <= a.K && (a.K & 7u) == 0) {  // rows are 16-byte aligned when K % 8 == 0
+    const uint4 raw = *reinterpret_cast<const uint4*>(xr + k);
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = (j & 1) ? __uint_as_float(w[j >> 1] & 0xffff0000u) : __uint_as_float(w[j >> 1] << 16);
+  } else {
+#pragma unroll
+    for (uint32_t j = 0; j < 8; ++j) v[j] = (live && k + j < a.K) ? bf16_bits_to_f32(xr[k + j]) : 0.0f;
+  }
+}
+
 __global__ __launch_bounds__(256) void gq_quant_kernel(GqQuantArgs a) {
-  const uint32_t lane = threadIdx.x & 63u;
-  const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6);
+  __shared__ float piece_max[4][kGqMaxPieces];
+  __shared__ float group_scale[4][kGqMaxGroups];
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  const uint32_t row = blockIdx.x * 4u + wave;
   if (row >= a.M_pad) return;
   const bool live = row < a.M;
   const uint16_t* xr = a.x + (size_t)(live ? row : 0u) * a.K;
-  int8_t* cr = a.codes + (size_t)row * a.K_pad;
-  for (uint32_t g = 0; g < a.G; ++g) {
-    const uint32_t k0 = g * a.group;
+  int8_t* cblk = a.codes + (size_t)(row >> 5) * (a.K_pad / 32u) * 1024u + (row & 31u) * 16u;
+  const uint32_t n_pieces = a.K_pad / 8u, pieces_per_group = a.group / 8u;
+  for (uint32_t p = lane; p < n_pieces; p += 64u) {
+    float v[8];
+    gq_load_piece(a, xr, live, p * 8u, v);
+    float m = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(v[j]));
+    piece_max[wave][p] = m;
+  }
+  __builtin_amdgcn_s_waitcnt(0xc07f);
+  __builtin_amdgcn_wave_barrier();
+  for (uint32_t g = lane; g < a.G; g += 64u) {
     float amax = 0.0f;
-    for (uint32_t e = lane; e < a.group; e += 64u) {
-      const uint32_t k = k0 + e;
-      const float v = (live && k < a.K) ? bf16_bits_to_f32(xr[k]) : 0.0f;
-      amax = fmaxf(amax, fabsf(v));
-    }
-    amax = wave_max(amax);
+    for (uint32_t p = 0; p < pieces_per_group; ++p) amax = fmaxf(amax, piece_max[wave][g * pieces_per_group + p]);
     const float scale = amax > 0.0f ? amax / a.qmax : 1.0f;
-    for (uint32_t e = lane; e < a.group; e += 64u) {
-      const uint32_t k = k0 + e;
-      const float v = (live && k < a.K) ? bf16_bits_to_f32(xr[k]) : 0.0f;
-      float q = __builtin_rintf(v / scale);
+    group_scale[wave][g] = scale;
+    a.scales[(size_t)g * a.M_pad + row] = scale;
+    if (a.scales_rm && live) a.scales_rm[(size_t)row * a.G + g] = scale;
+  }
+  __builtin_amdgcn_s_waitcnt(0xc07f);
+  __builtin_amdgcn_wave_barrier();
+  for (uint32_t p = lane; p < n_pieces; p += 64u) {
+    const uint32_t k = p * 8u;
+    float v[8];
+    gq_load_piece(a, xr, live, k, v);
+    const float scale = group_scale[wave][p / pieces_per_group];
+    uint32_t w[2] = {0, 0};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      float q = __builtin_rintf(v[j] / scale);
       q = fminf(fmaxf(q, -a.qmax), a.qmax);
-      cr[k] = (int8_t)(int)q;
+      w[j >> 2] |= ((uint32_t)(int)q & 0xffu) << (8 * (j & 3));
     }
-    if (lane == 0) a.scales[(size_t)row * a.G + g] = scale;
+    *reinterpret_cast<uint2*>(cblk + (size_t)(k >> 5) * 1024u + ((k >> 4) & 1u) * 512u + (k & 15u)) = make_uint2(w[0], w[1]);
+    if (a.codes_rm && live) *reinterpret_cast<uint2*>(a.codes_rm + (size_t)row * a.K_pad + k) = make_uint2(w[0], w[1]);
   }
 }
 
@@ -113,8 +151,10 @@ struct GqLoraZArgs {
   uint32_t M, K, r, n_adapters;
 };
 
-// z[m, :] = x[m, :] @ A[idx[m]] in float32: a wave per row, lane l sums k = l, l + 64, ... in order,
-// then the lanes are added by a fixed butterfly.
+// z[m, :] = x[m, :] @ A[idx[m]] in float32: a wave per row, lane l sums k = l, l + 64, ... in order
+// for all ranks at once (RB blocks of 8 ranks in registers), then the lanes are added by a fixed
+// butterfly.
+template <uint32_t RB>
 __global__ __launch_bounds__(256) void gq_lora_z_kernel(GqLoraZArgs a) {
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6);
@@ -123,31 +163,49 @@ __global__ __launch_bounds__(256) void gq_lora_z_kernel(GqLoraZArgs a) {
   ad = ad < 0 ? 0 : (ad >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad);
   const uint16_t* xr = a.x + (size_t)row * a.K;
   const uint16_t* ap = a.lora_a + (size_t)ad * a.K * a.r;
-  for (uint32_t r0 = 0; r0 < a.r; r0 += 8u) {
-    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    for (uint32_t k = lane; k < a.K; k += 64u) {
-      const float xv = bf16_bits_to_f32(xr[k]);
+  const bool vec = (a.r & 7u) == 0;  // rows of A are then 16-byte pieces
+  float acc[RB * 8];
 #pragma unroll
-      for (uint32_t j = 0; j < 8; ++j)
-        if (r0 + j < a.r) acc[j] = fmaf(xv, bf16_bits_to_f32(ap[(size_t)k * a.r + r0 + j]), acc[j]);
+  for (uint32_t j = 0; j < RB * 8u; ++j) acc[j] = 0.0f;
+  for (uint32_t k = lane; k < a.K; k += 64u) {
+    const float xv = bf16_bits_to_f32(xr[k]);
+    const uint16_t* ar = ap + (size_t)k * a.r;
+#pragma unroll
+    for (uint32_t b = 0; b < RB; ++b) {
+      if (b * 8u >= a.r) break;
+      if (vec) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(ar + b * 8u);
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) {
+          const float av = (j & 1u) ? __uint_as_float(w[j >> 1] & 0xffff0000u) : __uint_as_float(w[j >> 1] << 16);
+          acc[b * 8u + j] = fmaf(xv, av, acc[b * 8u + j]);
+        }
+      } else {
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j)
+          if (b * 8u + j < a.r) acc[b * 8u + j] = fmaf(xv, bf16_bits_to_f32(ar[b * 8u + j]), acc[b * 8u + j]);
+      }
     }
+  }
 #pragma unroll
-    for (uint32_t j = 0; j < 8; ++j) {
-      float v = acc[j];
+  for (uint32_t j = 0; j < RB * 8u; ++j) {
+    float v = acc[j];
 #pragma unroll
-      for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
-      if (lane == 0 && r0 + j < a.r) a.z[(size_t)row * 64u + r0 + j] = v;
-    }
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    if (lane == 0 && j < a.r) a.z[(size_t)row * 64u + j] = v;
   }
 }
 
 // ---------------------------------------------------------------------------------------
 struct GqGemmArgs {
-  const int8_t* codes;         // int8 [M_pad, K_pad]
-  const float* xs;             // f32 [M_pad, G]
+  const int8_t* codes;         // fragments [M_pad / 32][K_pad / 32][1 KiB]
+  const float* xs;             // f32 [G, M_pad]
+  uint32_t M_pad;
   const unsigned char* wp;     // packed weight
   const float* ws;             // f32 [G, N]
-  const float* z;              // f32 [M, 64] or null
+  const float* z;              // f32 [rows or slots, 64] or null
+  const int32_t* z_slot;       // int32 [M]: where row m's z lives (rows routed by adapter), or null: row m
   const uint16_t* lora_b;      // bf16 [n_adapters, r, N]
   const float* lora_scaling;   // f32 [n_adapters]
   const int32_t* idx;          // int32 [M] or null
@@ -156,67 +214,185 @@ struct GqGemmArgs {
   uint32_t M, N, K_pad, group, G, bits, r, n_adapters, n_col_blocks;
 };
 
-// One wave per 32 x 32 output block.  Lane l of a block holds column l % 32 and the 16 rows
-// 8 (v / 4) + 4 (l / 32) + v % 4, v = 0..15.
-__global__ __launch_bounds__(256) void gq_gemm_kernel(GqGemmArgs a) {
+// One wave per 64 x 64 output tile (2 x 2 blocks of 32 x 32), four waves (128 columns) per workgroup.
+// Lane l of a block holds column l % 32 and the 16 rows 8 (v / 4) + 4 (l / 32) + v % 4, v = 0..15.
+template <bool W4>
+__device__ inline v4i gq_weight_fragment(const unsigned char* p) {
+  if (W4) {
+    const uint2 raw = *reinterpret_cast<const uint2*>(p);
+    v4i f;
+    f[0] = (int)((raw.x << 4) & 0xf0f0f0f0u);
+    f[1] = (int)(raw.x & 0xf0f0f0f0u);
+    f[2] = (int)((raw.y << 4) & 0xf0f0f0f0u);
+    f[3] = (int)(raw.y & 0xf0f0f0f0u);
+    return f;
+  }
+  return *reinterpret_cast<const v4i*>(p);
+}
+
+template <bool W4>
+__global__ __launch_bounds__(256, 2) void gq_gemm_kernel(GqGemmArgs a) {
+  __shared__ float zs[4][64][64];  // per wave: the z rows of its tile (LoRA); reads are broadcasts, no padding needed
+  constexpr uint32_t kBlkBytes = W4 ? 512u : 1024u, kLaneBytes = W4 ? 8u : 16u;
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-  const uint32_t cb = blockIdx.x * 4u + wave;     // column block
-  if (cb >= a.n_col_blocks) return;
-  const uint32_t rb = blockIdx.y;                 // row block
+  const uint32_t cb0 = (blockIdx.x * 4u + wave) * 2u;  // first of the wave's two column blocks
+  const uint32_t rb0 = blockIdx.y * 2u;                // first of its two row blocks
+  const bool active = cb0 < a.n_col_blocks;            // idle waves still reach the barrier-free end
+  if (!active) return;
   const uint32_t c = lane & 31u, h = lane >> 5;
-  const uint32_t col = cb * 32u + c;
   const uint32_t kbs = a.K_pad / 32u, blocks_per_group = a.group / 32u;
-  const int8_t* arow = a.codes + (size_t)(rb * 32u + c) * a.K_pad + 16u * h;
-  const unsigned char* wblk = a.wp + (size_t)cb * kbs * (a.bits == 4u ? 512u : 1024u) + lane * (a.bits == 4u ? 8u : 16u);
-  const bool col_ok = col < a.N;
-  float outv[16];
+  const uint32_t n_rb = (a.M + 31u) / 32u;
+  // a tile that hangs over the edge re-reads its last valid block; those results are never stored
+  const uint32_t rb1 = rb0 + 1u < n_rb ? rb0 + 1u : rb0;
+  const uint32_t cb1 = cb0 + 1u < a.n_col_blocks ? cb0 + 1u : cb0;
+  const int8_t* ar0 = a.codes + (size_t)rb0 * kbs * 1024u + lane * 16u;
+  const int8_t* ar1 = a.codes + (size_t)rb1 * kbs * 1024u + lane * 16u;
+  const unsigned char* w0 = a.wp + (size_t)cb0 * kbs * kBlkBytes + lane * kLaneBytes;
+  const unsigned char* w1 = a.wp + (size_t)cb1 * kbs * kBlkBytes + lane * kLaneBytes;
+  const uint32_t col[2] = {cb0 * 32u + c, cb1 * 32u + c};
+  const uint32_t rbs[2] = {rb0, rb1};
+  float outv[2][2][16];
+  v4i fa0 = *reinterpret_cast<const v4i*>(ar0), fa1 = *reinterpret_cast<const v4i*>(ar1);
+  v4i fb0 = gq_weight_fragment<W4>(w0), fb1 = gq_weight_fragment<W4>(w1);
   for (uint32_t g = 0; g < a.G; ++g) {
-    v16i acc;
+    v16i acc[2][2];
 #pragma unroll
-    for (int e = 0; e < 16; ++e) acc[e] = 0;
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+    // the group's scales are requested before its MFMAs so that they have arrived when those end
+    float sw[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) sw[j] = col[j] < a.N ? a.ws[(size_t)g * a.N + col[j]] : 0.0f;
+    float4 sx4[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)  // rows 8 q + 4 h + 0..3 of the block: four consecutive scales
+        sx4[i][q] = *reinterpret_cast<const float4*>(a.xs + (size_t)g * a.M_pad + rbs[i] * 32u + 8u * q + 4u * h);
     for (uint32_t b = 0; b < blocks_per_group; ++b) {
       const uint32_t kb = g * blocks_per_group + b;
-      const v4i af = *reinterpret_cast<const v4i*>(arow + (size_t)kb * 32u);
-      v4i bf;
-      if (a.bits == 4u) {
-        const uint2 raw = *reinterpret_cast<const uint2*>(wblk + (size_t)kb * 512u);
-        bf[0] = (int)((raw.x << 4) & 0xf0f0f0f0u);
-        bf[1] = (int)(raw.x & 0xf0f0f0f0u);
-        bf[2] = (int)((raw.y << 4) & 0xf0f0f0f0u);
-        bf[3] = (int)(raw.y & 0xf0f0f0f0u);
-      } else {
-        bf = *reinterpret_cast<const v4i*>(wblk + (size_t)kb * 1024u);
+      const uint32_t kn = kb + 1u < kbs ? kb + 1u : kb;  // the next step's fragments travel during the MFMAs
+      const v4i na0 = *reinterpret_cast<const v4i*>(ar0 + (size_t)kn * 1024u);
+      const v4i na1 = *reinterpret_cast<const v4i*>(ar1 + (size_t)kn * 1024u);
+      const v4i nb0 = gq_weight_fragment<W4>(w0 + (size_t)kn * kBlkBytes);
+      const v4i nb1 = gq_weight_fragment<W4>(w1 + (size_t)kn * kBlkBytes);
+      acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa0, fb0, acc[0][0], 0, 0, 0);
+      acc[0][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa0, fb1, acc[0][1], 0, 0, 0);
+      acc[1][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa1, fb0, acc[1][0], 0, 0, 0);
+      acc[1][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa1, fb1, acc[1][1], 0, 0, 0);
+      fa0 = na0; fa1 = na1; fb0 = nb0; fb1 = nb1;
+    }
+    // (f32(acc) * sx) * sw in the reference's order; for 4-bit codes sw carries the exact factor 1/16
+    if (W4) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) sw[j] = sw[j] * 0.0625f;
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float sxq[4] = {sx4[i][q].x, sx4[i][q].y, sx4[i][q].z, sx4[i][q].w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int v = 4 * q + e;
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            float t = (float)acc[i][j][v] * sxq[e];
+            t = t * sw[j];
+            outv[i][j][v] = g == 0 ? t : outv[i][j][v] + t;
+          }
+        }
       }
-      acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf, acc, 0, 0, 0);
-    }
-    const float sw = col_ok ? a.ws[(size_t)g * a.N + col] : 0.0f;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const uint32_t row = rb * 32u + 8u * (v >> 2) + 4u * h + (v & 3);
-      const float sx = a.xs[(size_t)row * a.G + g];
-      float t = (float)acc[v] * sx;
-      t = t * sw;
-      if (a.bits == 4u) t = t * 0.0625f;  // exact: the codes entered as 16 * code
-      outv[v] = g == 0 ? t : outv[v] + t;
-    }
   }
-  if (!col_ok) return;
-#pragma unroll
-  for (int v = 0; v < 16; ++v) {
-    const uint32_t row = rb * 32u + 8u * (v >> 2) + 4u * h + (v & 3);
-    if (row >= a.M) continue;
-    float y = outv[v];
-    if (a.aux_base) a.aux_base[(size_t)row * a.N + col] = y;
-    if (a.z) {
-      int ad = a.idx ? a.idx[row] : 0;
-      ad = ad < 0 ? 0 : (ad >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad);
-      const float* zr = a.z + (size_t)row * 64u;
-      const uint16_t* bp = a.lora_b + (size_t)ad * a.r * a.N + col;
-      float low = 0.0f;
-      for (uint32_t r = 0; r < a.r; ++r) low = fmaf(zr[r], bf16_bits_to_f32(bp[(size_t)r * a.N]), low);
-      y = y + low * a.lora_scaling[ad];
+  // ---- epilogue: LoRA term per adapter present in the tile, store
+  const bool lora = a.z != nullptr;
+  if (lora) {
+    for (uint32_t t = lane; t < 64u * 64u; t += 64u) {
+      const uint32_t rr = t >> 6, r = t & 63u;
+      const uint32_t row = (rr < 32u ? rb0 : rb1) * 32u + (rr & 31u);
+      const bool ok = row < a.M && r < a.r;
+      const uint32_t zrow = (ok && a.z_slot) ? (uint32_t)a.z_slot[row] : row;
+      zs[wave][rr][r] = ok ? a.z[(size_t)zrow * 64u + r] : 0.0f;
     }
-    a.out[(size_t)row * a.N + col] = (uint16_t)f32_to_bf16_bits(y);
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_wave_barrier();
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    if (i == 1 && rb1 == rb0) break;
+    float low[2][16];
+    int ad_row[16];
+    if (lora) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const uint32_t row = rbs[i] * 32u + 8u * (v >> 2) + 4u * h + (v & 3);
+        int ad = (a.idx && row < a.M) ? a.idx[row] : 0;
+        ad_row[v] = ad < 0 ? 0 : (ad >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) low[j][v] = 0.0f;
+      }
+      // adapters present among the wave's rows, smallest first; every round handles one of them
+      int done_below = -1;
+      for (;;) {
+        int cand = 0x7fffffff;
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          if (ad_row[v] > done_below && ad_row[v] < cand) cand = ad_row[v];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+          const int o = __shfl_xor(cand, off);
+          cand = o < cand ? o : cand;
+        }
+        if (cand == 0x7fffffff) break;
+        done_below = cand;
+        const float sg = a.lora_scaling[cand];
+        for (uint32_t r0 = 0; r0 < a.r; r0 += 16u) {  // sixteen ranks of B in flight at a time
+          uint16_t braw[2][16];
+#pragma unroll
+          for (uint32_t t = 0; t < 16; ++t)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+              braw[j][t] = (col[j] < a.N && r0 + t < a.r) ? a.lora_b[((size_t)cand * a.r + r0 + t) * a.N + col[j]]
+                                                           : (uint16_t)0;
+#pragma unroll
+          for (uint32_t t = 0; t < 16; ++t) {
+            if (r0 + t >= a.r) break;
+            const float bv[2] = {bf16_bits_to_f32(braw[0][t]), bf16_bits_to_f32(braw[1][t])};
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+              const float zv = zs[wave][i * 32 + 8 * (v >> 2) + 4 * (int)h + (v & 3)][r0 + t];
+              if (ad_row[v] == cand) {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) low[j][v] = fmaf(zv, bv[j], low[j][v]);
+              }
+            }
+          }
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          if (ad_row[v] == cand) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) low[j][v] = low[j][v] * sg;
+          }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      if (j == 1 && cb1 == cb0) break;
+      if (col[j] >= a.N) continue;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const uint32_t row = rbs[i] * 32u + 8u * (v >> 2) + 4u * h + (v & 3);
+        if (row >= a.M) continue;
+        float y = outv[i][j][v];
+        if (a.aux_base) a.aux_base[(size_t)row * a.N + col[j]] = y;
+        if (lora) y = y + low[j][v];
+        a.out[(size_t)row * a.N + col[j]] = (uint16_t)f32_to_bf16_bits(y);
+      }
+    }
   }
 }
 

@@ -118,7 +118,7 @@ def forward(x: torch.Tensor, weight, lora_a=None, lora_b=None, lora_scaling=None
     elif adapter_indices is not None:
         raise ValueError("adapter_indices given without LoRA parameters")
     lib = _native.load()
-    ws_bytes = int(lib.mi355_w8a8_gq_workspace_bytes(m, pw.padded_in_features, pw.group_size, r))
+    ws_bytes = int(lib.mi355_w8a8_gq_workspace_bytes(m, pw.padded_in_features, pw.group_size, n_ad, r))
     if ws_bytes == 0:
         raise ValueError(f"geometry M={m}, K_pad={pw.padded_in_features}, group={pw.group_size}, rank={r} is outside "
                          "the native path")

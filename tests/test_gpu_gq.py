@@ -79,6 +79,8 @@ CASES = [
     (16, 1024, 520, 4, 8, 64, 32, 4),
     (128, 384, 130, 8, 4, 96, 0, 0),      # group of three k blocks, A4
     (300, 2048, 256, 4, 8, 2048, 64, 2),  # one group: per-channel W4
+    (45, 100, 40, 4, 8, 32, 5, 3),        # K not a multiple of 8: LoRA-A by the wave-per-row kernel
+    (90, 256, 72, 8, 8, 64, 12, 1),       # one adapter without indices
 ]
 
 
@@ -100,6 +102,8 @@ def test_gq_linear_matches_oracle(dev, pkg, m, k, n, wb, ab, group, rank, n_ad):
         s = rng.uniform(0.5, 2.0, n_ad).astype(F32)
         idx = rng.integers(0, n_ad, m).astype(np.int32)
         want_f32 = (base + o.lora_delta_multi(x, a, b, s, idx)).astype(F32)
+        if n_ad == 1:
+            idx = None                # no indices: every row takes adapter 0
     got, aux = pkg.gq_linear.forward(_bf(dev, x), _to_dev(pkg, dev, w), None if a is None else _bf(dev, a),
                                      None if b is None else _bf(dev, b),
                                      None if s is None else torch.from_numpy(s).to(dev), activation_bits=ab,
@@ -145,7 +149,8 @@ def test_gq_pack_keeps_four_bits_and_rejects_bad_geometry(dev, pkg):
     assert lib.mi355_w8a8_gq_packed_weight_bytes(64, 32, 4) == 2 * 512
     assert lib.mi355_w8a8_gq_packed_weight_bytes(64, 33, 8) == 2 * 2 * 1024
     assert lib.mi355_w8a8_gq_packed_weight_bytes(48, 32, 4) == 0
-    assert lib.mi355_w8a8_gq_workspace_bytes(4, 64, 10, 0) == 0
+    assert lib.mi355_w8a8_gq_workspace_bytes(4, 64, 10, 0, 0) == 0
+    assert lib.mi355_w8a8_gq_workspace_bytes(4, 64, 32, 2, 8) > lib.mi355_w8a8_gq_workspace_bytes(4, 64, 32, 0, 0) > 0
     w = o.quantize_frozen_weight(np.ones((70, 8), F32), bits=4, group_size=14, scale_dtype="f32")
     with pytest.raises(ValueError, match="group_size % 32"):
         pkg.gq_linear.forward(torch.zeros(2, 70, dtype=torch.bfloat16, device=dev), _to_dev(pkg, dev, w))
