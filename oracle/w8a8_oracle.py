@@ -40,7 +40,7 @@ How each function is pinned (the tests that do it live in ``tests/test_oracle_*.
   preservation, position 0 and ``rotary_dim`` 0 identities, and an enumerated interleaving
   (tests/tx/kernels/test_qwen3_5_qkv_lora.py:75-83 states it as ``FusedLoRALinear.split``).
   sin/cos/pow of XLA-CPU are not available: PARITY UNPINNED in their last float32 bits.
-* ``moe_route``/``moe_expert_mlp``: ``torch.topk``/``scipy.special.softmax`` special
+* ``moe_route``/``moe_combine``/``moe_expert_mlp``: ``torch.topk``/``scipy.special.softmax`` special
   cases and the merged-weight invariant of tests/tx/models/test_qwen3.py:123-180.
 """
 

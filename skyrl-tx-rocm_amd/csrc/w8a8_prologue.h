@@ -203,14 +203,6 @@ __device__ inline void route_groups_block(const int32_t* __restrict__ group_size
   }
 }
 
-__global__ __launch_bounds__(1024) void route_groups_kernel(const int32_t* __restrict__ group_sizes, uint32_t M,
-                                                            uint32_t n_groups, uint32_t slots,
-                                                            int32_t* __restrict__ src_row,
-                                                            int32_t* __restrict__ dst_pos,
-                                                            int32_t* __restrict__ blk_range, uint32_t pad) {
-  route_groups_block(group_sizes, M, n_groups, slots, src_row, dst_pos, blk_range, pad, nullptr, 0u);
-}
-
 // ---------------------------------------------------------------------------------------
 // Per-token dynamic int8 quantization (skyrl/tx/kernels/quantized_lora.py:199-212 with one
 // group per row), optionally preceded by RMSNorm
@@ -621,15 +613,7 @@ struct QuantLoraArgs {
   unsigned char* zp;        // packed z fragments
   uint32_t r, nkk, nterms;
   uint32_t* tile_ctr;       // 256 words cleared for the GEMM launches' tile counters, or null
-  // Optional gather on the way in (see QuantArgs): row `src` is read from x[row_map[src] / row_div];
-  // the auxiliary outputs keep the index `src`
-  const int32_t* row_map;
-  uint32_t row_div;
 };
-
-__device__ inline size_t quant_lora_x_row(const QuantLoraArgs& a, int src) {
-  return a.row_map ? (size_t)((uint32_t)a.row_map[src] / a.row_div) : (size_t)src;
-}
 
 template <int CB, bool RMS>  // CB: 16-wide rank blocks (0 = no LoRA, 1, 2, 4)
 __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
@@ -644,7 +628,6 @@ __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
   if (a.tile_ctr && hb == 0 && tid < 256u) a.tile_ctr[tid] = 0u;
   if (hb >= a.n_half_blocks) return;
   const uint32_t pb = hb >> 1, half16 = hb & 1u;
-  if (a.blk_range && a.blk_range[pb] < 0) return;  // grouped layout: block beyond the slots in use
 
   // ---- 1. row statistics: wave w, slot row w
   {
@@ -653,7 +636,7 @@ __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
     if (src < 0 || src >= (int)a.M) src = -1;
     float inv = 1.0f, amax = 0.0f;
     if (src >= 0) {
-      const uint16_t* xr = a.x + quant_lora_x_row(a, src) * a.K;
+      const uint16_t* xr = a.x + (size_t)src * a.K;
       // eight 16-byte loads of the row are in flight at a time
       if (RMS) {
         double ss = 0.0;
@@ -730,7 +713,7 @@ __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
   const int src = row_src[i];
   const float inv = row_inv[i], scale = row_scale[i];
   const float rscale = __builtin_amdgcn_rcpf(scale);
-  const uint16_t* xr = a.x + (src < 0 ? (size_t)0 : quant_lora_x_row(a, src)) * a.K;
+  const uint16_t* xr = a.x + (size_t)(src < 0 ? 0 : src) * a.K;
   const uint32_t range = (CB > 0 && a.blk_range) ? (uint32_t)a.blk_range[pb] : 0u;
   const uint32_t glo = range & 0xffffu, ghi = range >> 16;
   const uint32_t rowgrp = (CB > 0 && a.slot_group && ghi > glo) ? (uint32_t)a.slot_group[hb * 16u + i] : glo;

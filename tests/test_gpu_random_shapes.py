@@ -84,3 +84,112 @@ def test_backward_random_geometry(dev, seed):
         rep = wc.compare(got[0], want)
         assert rep["violations"] == 0, rep
         assert got[1] is None
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_grouped_random_geometry(dev, seed):
+    """Ragged groups (empty ones included), both grouped tile geometries, with and without the row
+    map on the way in: integer stages bit-equal to the oracle, outputs within tolerance."""
+    import torch
+
+    from __graft_entry__ import load_package
+
+    pkg = load_package()
+    w8, nat = pkg.w8a8_lora, pkg._native
+    rng = np.random.default_rng(20_000 + seed)
+    e = int(rng.choice([1, 2, 5, 9]))
+    sizes = [int(v) for v in rng.choice([0, 1, 31, 64, 65, 130, 200], e)]
+    if sum(sizes) == 0:
+        sizes[0] = 3
+    k = 8 * int(rng.integers(4, 80))
+    n = 2 * int(rng.integers(4, 400))
+    rank = int(rng.choice([0, 4, 16, 33]))
+    swiglu = bool(seed & 1)
+    extra = int(rng.integers(0, 5))
+    m = sum(sizes) + extra
+    flag = nat.FLAG_GROUPED_TILE64 if seed % 3 == 0 else (nat.FLAG_GROUPED_TILE128 if seed % 3 == 1 else 0)
+    print(f"[case] grouped seed={seed} sizes={sizes} k={k} n={n} rank={rank} swiglu={swiglu} flag={flag}", flush=True)
+    x = o.bf16_round(rng.standard_normal((m, k)).astype(F32))
+    codes = rng.integers(-127, 128, (e, k, n), dtype=np.int8)
+    scales = rng.uniform(0.001, 0.01, (e, n)).astype(F32)
+    a = o.bf16_round((rng.standard_normal((e, k, max(rank, 1))) * 0.02).astype(F32))
+    b = o.bf16_round((rng.standard_normal((e, max(rank, 1), n)) * 0.02).astype(F32))
+    weights = [o.GroupQuantizedWeight(codes[i], scales[i:i + 1], k, k, 8, k) for i in range(e)]
+    st = np.concatenate(([0], np.cumsum(sizes)))
+    pre = np.zeros((m, n), F32)
+    acc = np.zeros((m, n), np.int32)
+    xc, xs = o.quantize_rows(x)
+    for i, w in enumerate(weights):
+        r0, r1 = int(st[i]), int(st[i + 1])
+        if r1 > r0:
+            pre[r0:r1] = (o.quantized_lora_linear_f32(x[r0:r1], w, a[i], b[i], F32(1.25)) if rank
+                          else o.quantized_frozen_linear_f32(x[r0:r1], w))
+            acc[r0:r1] = o.int_matmul(xc[r0:r1], codes[i])
+    fused = o.bf16_round(pre)
+    want = o.swiglu_from_interleaved(fused) if swiglu else fused
+    bf = lambda t: torch.from_numpy(np.ascontiguousarray(t)).to(dev).to(torch.bfloat16)
+    gw = w8.prepare_grouped_weight(torch.from_numpy(codes).to(dev), torch.from_numpy(scales).to(dev))
+    lora = (bf(a), bf(b), 1.25) if rank else (None, None, None)
+    gs = torch.tensor(sizes, dtype=torch.int32)
+    out, aux = w8.grouped_forward(bf(x), gs, gw, *lora, swiglu=swiglu, return_aux=True, flags=flag)
+    # the same call reading its rows through a map: a permuted copy of x with every row twice
+    perm = rng.permutation(m)
+    table = np.empty((m, k), F32)
+    table[perm] = x
+    row_map = torch.from_numpy((2 * perm + rng.integers(0, 2, m)).astype(np.int32)).to(dev)
+    mapped = w8.grouped_forward(bf(table), gs, gw, *lora, swiglu=swiglu, flags=flag, row_map=row_map, row_repeat=2)
+    torch.cuda.synchronize()
+    used = int(st[-1])
+    np.testing.assert_array_equal(aux["x_codes"].cpu().numpy(), xc)
+    np.testing.assert_array_equal(aux["acc"].cpu().numpy()[:used], acc[:used])
+    got = out.float().cpu().numpy()
+    assert not got[used:].any()
+    rep = wc.compare(got, want)
+    assert rep["violations"] == 0, rep
+    assert torch.equal(mapped, out)
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_group_scaled_random_geometry(dev, seed):
+    """W4 / W8 codes with grouped scales, A4 / A8: codes, scales and the float32 base bit-equal."""
+    import torch
+
+    from __graft_entry__ import load_package
+
+    pkg = load_package()
+    rng = np.random.default_rng(30_000 + seed)
+    m = int(rng.choice([1, 16, 31, 33, 64, 100, 257]))
+    group = 32 * int(rng.choice([1, 2, 3, 4, 8]))
+    k = int(rng.integers(1, 6)) * group - int(rng.choice([0, 0, 8, 20]))
+    n = int(rng.integers(1, 300))
+    wb, ab = int(rng.choice([4, 8])), int(rng.choice([4, 8]))
+    n_ad = int(rng.choice([0, 1, 3]))
+    rank = int(rng.choice([2, 8, 24, 64]))
+    print(f"[case] group-scaled seed={seed} m={m} k={k} n={n} W{wb}A{ab} group={group} adapters={n_ad} rank={rank}",
+          flush=True)
+    x = o.bf16_round(rng.standard_t(4, (m, k)).astype(F32))
+    w = o.quantize_frozen_weight((rng.standard_normal((k, n)) * 0.05).astype(F32), bits=wb, group_size=group,
+                                 scale_dtype="f32")
+    base, x_codes, x_scales, _ = o.quantized_frozen_linear_f32(x, w, activation_bits=ab, return_parts=True)
+    want = base
+    args = [None, None, None]
+    idx_t = None
+    if n_ad:
+        a = o.bf16_round((rng.standard_normal((n_ad, k, rank)) * 0.05).astype(F32))
+        b = o.bf16_round((rng.standard_normal((n_ad, rank, n)) * 0.05).astype(F32))
+        s = rng.uniform(0.5, 2.0, n_ad).astype(F32)
+        idx = rng.integers(0, n_ad, m).astype(np.int32)
+        want = (base + o.lora_delta_multi(x, a, b, s, idx)).astype(F32)
+        bf = lambda t: torch.from_numpy(np.ascontiguousarray(t)).to(dev).to(torch.bfloat16)
+        args = [bf(a), bf(b), torch.from_numpy(s).to(dev)]
+        idx_t = torch.from_numpy(idx).to(dev)
+    wt = pkg.quantized_lora.GroupQuantizedWeight(torch.from_numpy(w.codes).to(dev), torch.from_numpy(w.scales).to(dev),
+                                                 k, w.padded_in_features, wb, group)
+    got, aux = pkg.gq_linear.forward(torch.from_numpy(x).to(dev).to(torch.bfloat16), wt, *args, activation_bits=ab,
+                                     adapter_indices=idx_t, return_aux=True)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(aux["x_codes"].cpu().numpy(), x_codes.reshape(m, -1))
+    np.testing.assert_array_equal(aux["x_scales"].cpu().numpy().view(np.uint32), x_scales.view(np.uint32))
+    np.testing.assert_array_equal(aux["base"].cpu().numpy().view(np.uint32), base.view(np.uint32))
+    rep = wc.compare(got.float().cpu().numpy(), o.bf16_round(want))
+    assert rep["violations"] == 0, rep
