@@ -1037,6 +1037,7 @@ int run_moe_combine(const void* expert_out, const int32_t* unsort, const float* 
   return launch_status();
 }
 
+constexpr uint32_t kGqZSlices = 32;
 struct GqLayout { uint64_t codes, scales, z, src_row, dst_pos, slot_group, blk_range, at, total; uint32_t m_pad, G; };
 
 GqLayout make_gq_layout(uint32_t m, uint32_t k_pad, uint32_t group, uint32_t n_adapters, uint32_t rank) {
@@ -1046,7 +1047,8 @@ GqLayout make_gq_layout(uint32_t m, uint32_t k_pad, uint32_t group, uint32_t n_a
   uint64_t off = 0;
   L.codes = off; off += align256((uint64_t)L.m_pad * k_pad);
   L.scales = off; off += align256((uint64_t)L.m_pad * L.G * 4u);
-  L.z = off; off += rank ? align256((uint64_t)L.m_pad * 64u * 4u) : 0u;
+  // decode (one row block): LoRA-A arrives as up to kGqZSlices slices over K
+  L.z = off; off += rank ? align256((uint64_t)L.m_pad * 64u * 4u * (L.m_pad == 32u ? kGqZSlices : 1u)) : 0u;
   L.src_row = off; off += rank ? align256((uint64_t)L.m_pad * 4u) : 0u;
   L.dst_pos = off; off += rank ? align256((uint64_t)L.m_pad * 4u) : 0u;
   L.slot_group = off; off += rank ? align256((uint64_t)L.m_pad * 4u) : 0u;
@@ -1119,15 +1121,21 @@ int run_gq_linear(const mi355_w8a8_gq_problem* p, hipStream_t s) {
   q.codes_rm = p->aux_x_codes; q.scales_rm = p->aux_x_scales;
   q.M = p->m; q.M_pad = L.m_pad; q.K = p->k; q.K_pad = p->k_pad; q.group = p->group_size; q.G = L.G;
   q.qmax = p->activation_bits == 4u ? 7.0f : 127.0f;
-  hipLaunchKernelGGL(gq_quant_kernel, dim3(L.m_pad / 4u), dim3(256), 0, s, q);
+  // few rows: a row's groups are dealt to several waves so that the launch still fills the chip
+  const uint32_t q_slices = L.m_pad >= 1024u ? 1u : (L.G < 16u ? L.G : 16u);
+  q.groups_per_slice = (L.G + q_slices - 1u) / q_slices;
+  hipLaunchKernelGGL(gq_quant_kernel, dim3(L.m_pad / 4u, (L.G + q.groups_per_slice - 1u) / q.groups_per_slice), dim3(256),
+                     0, s, q);
   if ((st = launch_status())) return st;
 
   // z = x @ A[idx]: rows routed by adapter and multiplied on the matrix core (the kernels of the
   // per-channel path) when the adapter count and K allow it, else one wave per row
-  const bool fast_z = lora && p->n_adapters <= (uint32_t)kMaxAdapters && (p->k & 7u) == 0 && aligned16(p->x) &&
-                      aligned16(p->lora_a);
+  const bool decode = L.m_pad == 32u;  // few rows: a wave per (row, k slice) instead of one row block
+  const bool fast_z = lora && !decode && p->n_adapters <= (uint32_t)kMaxAdapters && (p->k & 7u) == 0 &&
+                      aligned16(p->x) && aligned16(p->lora_a);
   const bool routed = fast_z && p->adapter_indices && p->n_adapters > 1u;
   int32_t* dst_pos = reinterpret_cast<int32_t*>(ws + L.dst_pos);
+  uint32_t z_slices = 1u;
   if (fast_z) {
     int32_t* src_row = reinterpret_cast<int32_t*>(ws + L.src_row);
     int32_t* slot_group = reinterpret_cast<int32_t*>(ws + L.slot_group);
@@ -1169,7 +1177,11 @@ int run_gq_linear(const mi355_w8a8_gq_problem* p, hipStream_t s) {
     z.idx = p->adapter_indices;
     z.z = reinterpret_cast<float*>(ws + L.z);
     z.M = p->m; z.K = p->k; z.r = p->rank; z.n_adapters = p->n_adapters;
-    const dim3 zgrid((p->m + 3u) / 4u), zblock(256);
+    z.k_split = decode ? (p->k + 255u) / 256u : 1u;
+    if (z.k_split > kGqZSlices) z.k_split = kGqZSlices;
+    z.k_chunk = round_up((p->k + z.k_split - 1u) / z.k_split, 64u);
+    z_slices = z.k_split;
+    const dim3 zgrid((p->m + 3u) / 4u, z.k_split), zblock(256);
     if (p->rank <= 8u) hipLaunchKernelGGL((gq_lora_z_kernel<1>), zgrid, zblock, 0, s, z);
     else if (p->rank <= 16u) hipLaunchKernelGGL((gq_lora_z_kernel<2>), zgrid, zblock, 0, s, z);
     else if (p->rank <= 32u) hipLaunchKernelGGL((gq_lora_z_kernel<4>), zgrid, zblock, 0, s, z);
@@ -1183,6 +1195,7 @@ int run_gq_linear(const mi355_w8a8_gq_problem* p, hipStream_t s) {
   g.ws = p->w_scales;
   g.z = lora ? reinterpret_cast<const float*>(ws + L.z) : nullptr;
   g.z_slot = routed ? dst_pos : nullptr;
+  g.z_slices = z_slices; g.z_slice_stride = p->m * 64u;
   g.lora_b = static_cast<const uint16_t*>(p->lora_b);
   g.lora_scaling = p->lora_scaling;
   g.idx = p->adapter_indices;
@@ -1192,6 +1205,12 @@ int run_gq_linear(const mi355_w8a8_gq_problem* p, hipStream_t s) {
   g.bits = p->weight_bits;
   g.r = p->rank; g.n_adapters = p->n_adapters;
   g.n_col_blocks = (p->n + 31u) / 32u;
+  if (L.m_pad == 32u) {  // decode: split the groups over the waves of a workgroup per column block
+    const dim3 sgrid(g.n_col_blocks), sblock(kGqSkinnyWaves * 64u);
+    if (p->weight_bits == 4u) hipLaunchKernelGGL((gq_skinny_kernel<true>), sgrid, sblock, 0, s, g);
+    else hipLaunchKernelGGL((gq_skinny_kernel<false>), sgrid, sblock, 0, s, g);
+    return launch_status();
+  }
   const dim3 grid((g.n_col_blocks + 7u) / 8u, (L.m_pad / 32u + 1u) / 2u), block(256);
   if (p->weight_bits == 4u) hipLaunchKernelGGL((gq_gemm_kernel<true>), grid, block, 0, s, g);
   else hipLaunchKernelGGL((gq_gemm_kernel<false>), grid, block, 0, s, g);

@@ -75,6 +75,7 @@ struct GqQuantArgs {
   float* scales_rm;    // optional row-major copy f32 [M, G]
   uint32_t M, M_pad, K, K_pad, group, G;
   float qmax;          // 127 or 7
+  uint32_t groups_per_slice;  // grid y = slices of a row's groups (few rows: more waves per row)
 };
 
 // scale = amax > 0 ? amax / qmax : 1, code = clip(rint(x / scale), -qmax, qmax), IEEE float32
@@ -104,10 +105,14 @@ __global__ __launch_bounds__(256) void gq_quant_kernel(GqQuantArgs a) {
   const bool live = row < a.M;
   const uint16_t* xr = a.x + (size_t)(live ? row : 0u) * a.K;
   int8_t* cblk = a.codes + (size_t)(row >> 5) * (a.K_pad / 32u) * 1024u + (row & 31u) * 16u;
-  const uint32_t n_pieces = a.K_pad / 8u, pieces_per_group = a.group / 8u;
+  const uint32_t pieces_per_group = a.group / 8u;
+  const uint32_t g_lo = blockIdx.y * a.groups_per_slice;
+  const uint32_t g_hi = g_lo + a.groups_per_slice < a.G ? g_lo + a.groups_per_slice : a.G;
+  if (g_lo >= g_hi) return;
+  const uint32_t p_lo = g_lo * pieces_per_group, n_pieces = (g_hi - g_lo) * pieces_per_group;
   for (uint32_t p = lane; p < n_pieces; p += 64u) {
     float v[8];
-    gq_load_piece(a, xr, live, p * 8u, v);
+    gq_load_piece(a, xr, live, (p_lo + p) * 8u, v);
     float m = 0.0f;
 #pragma unroll
     for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(v[j]));
@@ -115,18 +120,19 @@ __global__ __launch_bounds__(256) void gq_quant_kernel(GqQuantArgs a) {
   }
   __builtin_amdgcn_s_waitcnt(0xc07f);
   __builtin_amdgcn_wave_barrier();
-  for (uint32_t g = lane; g < a.G; g += 64u) {
+  for (uint32_t gl = lane; gl < g_hi - g_lo; gl += 64u) {
+    const uint32_t g = g_lo + gl;
     float amax = 0.0f;
-    for (uint32_t p = 0; p < pieces_per_group; ++p) amax = fmaxf(amax, piece_max[wave][g * pieces_per_group + p]);
+    for (uint32_t p = 0; p < pieces_per_group; ++p) amax = fmaxf(amax, piece_max[wave][gl * pieces_per_group + p]);
     const float scale = amax > 0.0f ? amax / a.qmax : 1.0f;
-    group_scale[wave][g] = scale;
+    group_scale[wave][gl] = scale;
     a.scales[(size_t)g * a.M_pad + row] = scale;
     if (a.scales_rm && live) a.scales_rm[(size_t)row * a.G + g] = scale;
   }
   __builtin_amdgcn_s_waitcnt(0xc07f);
   __builtin_amdgcn_wave_barrier();
   for (uint32_t p = lane; p < n_pieces; p += 64u) {
-    const uint32_t k = p * 8u;
+    const uint32_t k = (p_lo + p) * 8u;
     float v[8];
     gq_load_piece(a, xr, live, k, v);
     const float scale = group_scale[wave][p / pieces_per_group];
@@ -147,13 +153,14 @@ struct GqLoraZArgs {
   const uint16_t* x;       // bf16 [M, K]
   const uint16_t* lora_a;  // bf16 [n_adapters, K, r]
   const int32_t* idx;      // int32 [M] or null (adapter 0)
-  float* z;                // f32 [M, 64]
+  float* z;                // f32 [k_split][M][64]: slice s holds the sum over its range of k
   uint32_t M, K, r, n_adapters;
+  uint32_t k_split, k_chunk;  // slices (grid y) and k per slice (a multiple of 64)
 };
 
-// z[m, :] = x[m, :] @ A[idx[m]] in float32: a wave per row, lane l sums k = l, l + 64, ... in order
-// for all ranks at once (RB blocks of 8 ranks in registers), then the lanes are added by a fixed
-// butterfly.
+// z[m, :] = x[m, :] @ A[idx[m]] in float32: a wave per (row, k slice), lane l sums k = l, l + 64, ...
+// of the slice in order for all ranks at once (RB blocks of 8 ranks in registers), then the lanes are
+// added by a fixed butterfly; the consumer adds the slices in order.
 template <uint32_t RB>
 __global__ __launch_bounds__(256) void gq_lora_z_kernel(GqLoraZArgs a) {
   const uint32_t lane = threadIdx.x & 63u;
@@ -167,7 +174,10 @@ __global__ __launch_bounds__(256) void gq_lora_z_kernel(GqLoraZArgs a) {
   float acc[RB * 8];
 #pragma unroll
   for (uint32_t j = 0; j < RB * 8u; ++j) acc[j] = 0.0f;
-  for (uint32_t k = lane; k < a.K; k += 64u) {
+  const uint32_t k_lo = blockIdx.y * a.k_chunk;
+  const uint32_t k_hi = k_lo + a.k_chunk < a.K ? k_lo + a.k_chunk : a.K;
+  float* zout = a.z + ((size_t)blockIdx.y * a.M + row) * 64u;
+  for (uint32_t k = k_lo + lane; k < k_hi; k += 64u) {
     const float xv = bf16_bits_to_f32(xr[k]);
     const uint16_t* ar = ap + (size_t)k * a.r;
 #pragma unroll
@@ -193,7 +203,7 @@ __global__ __launch_bounds__(256) void gq_lora_z_kernel(GqLoraZArgs a) {
     float v = acc[j];
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
-    if (lane == 0 && j < a.r) a.z[(size_t)row * 64u + j] = v;
+    if (lane == 0 && j < a.r) zout[j] = v;
   }
 }
 
@@ -206,6 +216,8 @@ struct GqGemmArgs {
   const float* ws;             // f32 [G, N]
   const float* z;              // f32 [rows or slots, 64] or null
   const int32_t* z_slot;       // int32 [M]: where row m's z lives (rows routed by adapter), or null: row m
+  uint32_t z_slices;           // decode kernel: z arrives as this many slices to add, z_slice_stride floats apart
+  uint32_t z_slice_stride;
   const uint16_t* lora_b;      // bf16 [n_adapters, r, N]
   const float* lora_scaling;   // f32 [n_adapters]
   const int32_t* idx;          // int32 [M] or null
@@ -393,6 +405,130 @@ __global__ __launch_bounds__(256, 2) void gq_gemm_kernel(GqGemmArgs a) {
         a.out[(size_t)row * a.N + col[j]] = (uint16_t)f32_to_bf16_bits(y);
       }
     }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Up to 32 rows (decode): a workgroup of eight waves owns one 32-column block for all of K.  Wave w
+// takes a contiguous range of groups, streams its weight fragments eight k blocks ahead, forms its
+// groups' float32 terms in group order, and the eight partial sums are added in wave order through
+// LDS -- the groups are summed in order inside a wave and the waves in order, which differs from
+// the strictly sequential float32 sum of the reference only in rounding (inside the bf16 tolerance;
+// the result is the same from run to run).
+constexpr uint32_t kGqSkinnyWaves = 8;
+
+template <bool W4>
+__global__ __launch_bounds__(512) void gq_skinny_kernel(GqGemmArgs a) {
+  __shared__ float red[kGqSkinnyWaves][16][64];
+  constexpr uint32_t kBlkBytes = W4 ? 512u : 1024u, kLaneBytes = W4 ? 8u : 16u, U = 8u;
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t cb = blockIdx.x;
+  const uint32_t c = lane & 31u, h = lane >> 5;
+  const uint32_t col = cb * 32u + c;
+  const uint32_t kbs = a.K_pad / 32u, bpg = a.group / 32u;
+  const uint32_t g_lo = (wave * a.G) / kGqSkinnyWaves, g_hi = ((wave + 1u) * a.G) / kGqSkinnyWaves;
+  const int8_t* ap = a.codes + lane * 16u;  // row block 0
+  const unsigned char* wp = a.wp + (size_t)cb * kbs * kBlkBytes + lane * kLaneBytes;
+  float part[16];
+#pragma unroll
+  for (int v = 0; v < 16; ++v) part[v] = 0.0f;
+  v16i acc;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[e] = 0;
+  const uint32_t kb_lo = g_lo * bpg, kb_hi = g_hi * bpg;
+  // the scales of the group in progress, requested a group ahead
+  auto load_scales = [&](uint32_t g, float& sw, float4 (&sx)[4]) {
+    const uint32_t gg = g < a.G ? g : a.G - 1u;
+    sw = col < a.N ? a.ws[(size_t)gg * a.N + col] : 0.0f;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) sx[q] = *reinterpret_cast<const float4*>(a.xs + (size_t)gg * a.M_pad + 8u * q + 4u * h);
+  };
+  float sw_cur;
+  float4 sx_cur[4];
+  load_scales(g_lo, sw_cur, sx_cur);
+  bool first = true;
+  for (uint32_t base = kb_lo; base < kb_hi; base += U) {
+    v4i fa[U], fb[U];
+#pragma unroll
+    for (uint32_t u = 0; u < U; ++u) {
+      const uint32_t kb = base + u < kb_hi ? base + u : kb_hi - 1u;  // the tail repeats a block, unused
+      fa[u] = *reinterpret_cast<const v4i*>(ap + (size_t)kb * 1024u);
+      fb[u] = gq_weight_fragment<W4>(wp + (size_t)kb * kBlkBytes);
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < U; ++u) {
+      const uint32_t kb = base + u;
+      if (kb < kb_hi) {  // wave-uniform
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[u], fb[u], acc, 0, 0, 0);
+        if ((kb + 1u) % bpg == 0) {  // the group is complete
+          float sw = sw_cur;
+          if (W4) sw = sw * 0.0625f;
+          float4 sx[4] = {sx_cur[0], sx_cur[1], sx_cur[2], sx_cur[3]};
+          load_scales((kb + 1u) / bpg, sw_cur, sx_cur);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const float sxq[4] = {sx[q].x, sx[q].y, sx[q].z, sx[q].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int v = 4 * q + e;
+              float t = (float)acc[v] * sxq[e];
+              t = t * sw;
+              part[v] = first ? t : part[v] + t;
+              acc[v] = 0;
+            }
+          }
+          first = false;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < 16; ++v) red[wave][v][lane] = part[v];
+  __shared__ float zsum[32][64];
+  if (a.z) {
+    for (uint32_t q = tid; q < 32u * 64u; q += 512u) {
+      const uint32_t row = q >> 6, r = q & 63u;
+      float zv = 0.0f;
+      if (row < a.M && r < a.r) {
+        const float* zp = a.z + (size_t)(a.z_slot ? (uint32_t)a.z_slot[row] : row) * 64u + r;
+        for (uint32_t sl = 0; sl < a.z_slices; ++sl) zv = sl == 0 ? zp[0] : zv + zp[(size_t)sl * a.z_slice_stride];
+      }
+      zsum[row][r] = zv;
+    }
+  }
+  __syncthreads();
+  for (uint32_t o = tid; o < 1024u; o += 512u) {
+    const uint32_t v = o >> 6, l = o & 63u;
+    const uint32_t row = 8u * (v >> 2) + 4u * (l >> 5) + (v & 3u), ocol = cb * 32u + (l & 31u);
+    if (row >= a.M || ocol >= a.N) continue;
+    float y = 0.0f;
+    bool any = false;
+#pragma unroll
+    for (uint32_t w = 0; w < kGqSkinnyWaves; ++w) {
+      const bool has = (w * a.G) / kGqSkinnyWaves < ((w + 1u) * a.G) / kGqSkinnyWaves;  // the wave had groups
+      if (has) {
+        y = any ? y + red[w][v][l] : red[w][v][l];
+        any = true;
+      }
+    }
+    if (a.aux_base) a.aux_base[(size_t)row * a.N + ocol] = y;
+    if (a.z) {
+      int ad = a.idx ? a.idx[row] : 0;
+      ad = ad < 0 ? 0 : (ad >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad);
+      const float* zr = zsum[row];
+      const uint16_t* bp = a.lora_b + (size_t)ad * a.r * a.N + ocol;
+      float low = 0.0f;
+      for (uint32_t r0 = 0; r0 < a.r; r0 += 8u) {
+        uint16_t braw[8];
+#pragma unroll
+        for (uint32_t t = 0; t < 8; ++t) braw[t] = r0 + t < a.r ? bp[(size_t)(r0 + t) * a.N] : (uint16_t)0;
+#pragma unroll
+        for (uint32_t t = 0; t < 8; ++t)
+          if (r0 + t < a.r) low = fmaf(zr[r0 + t], bf16_bits_to_f32(braw[t]), low);
+      }
+      y = y + low * a.lora_scaling[ad];
+    }
+    a.out[(size_t)row * a.N + ocol] = (uint16_t)f32_to_bf16_bits(y);
   }
 }
 

@@ -1,9 +1,10 @@
 """GPU parity of the group-scaled quantized linear (W4 / W8 codes, A4 / A8 activations, scales per K
 group) through the C ABI, against the CPU oracle and the reference's hand-coded W4A4 case.
 
-Bar: activation codes, activation scales and the float32 base (the sum over the groups before the
-LoRA term) bit for bit; the bf16 output bit for bit without LoRA and to |a - b| <= 2e-2 + 1e-2 |b|
-with it (the float32 summation order of the two small LoRA products differs).
+Bar: activation codes and scales bit for bit; above 32 rows also the float32 base (the sum over
+the groups before the LoRA term) and, without LoRA, the bf16 output; otherwise |a - b| <= 2e-2 +
+1e-2 |b| (the float32 summation order of the LoRA products differs, and the decode kernel for up to
+32 rows adds the groups per wave before it adds the waves).
 """
 
 import numpy as np
@@ -112,10 +113,13 @@ def test_gq_linear_matches_oracle(dev, pkg, m, k, n, wb, ab, group, rank, n_ad):
     torch.cuda.synchronize()
     np.testing.assert_array_equal(aux["x_codes"].cpu().numpy(), x_codes.reshape(m, -1))
     np.testing.assert_array_equal(aux["x_scales"].cpu().numpy().view(np.uint32), x_scales.view(np.uint32))
-    np.testing.assert_array_equal(aux["base"].cpu().numpy().view(np.uint32), base.view(np.uint32))
+    if m > 32:
+        np.testing.assert_array_equal(aux["base"].cpu().numpy().view(np.uint32), base.view(np.uint32))
+    else:   # decode kernel: the groups are summed per wave, then the waves (same terms, other order)
+        np.testing.assert_allclose(aux["base"].cpu().numpy(), base, rtol=2e-6, atol=1e-6 * float(np.abs(base).max()))
     got_np = got.to(torch.float32).cpu().numpy()
     want = o.bf16_round(want_f32)
-    if not n_ad:
+    if not n_ad and m > 32:
         np.testing.assert_array_equal(o.bf16_bits(got_np), o.bf16_bits(want))
     rep = wc.compare(got_np, want)
     print(f"[gq parity] m{m}k{k}n{n} W{wb}A{ab} {rep}", flush=True)

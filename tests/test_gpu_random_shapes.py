@@ -190,6 +190,9 @@ def test_group_scaled_random_geometry(dev, seed):
     torch.cuda.synchronize()
     np.testing.assert_array_equal(aux["x_codes"].cpu().numpy(), x_codes.reshape(m, -1))
     np.testing.assert_array_equal(aux["x_scales"].cpu().numpy().view(np.uint32), x_scales.view(np.uint32))
-    np.testing.assert_array_equal(aux["base"].cpu().numpy().view(np.uint32), base.view(np.uint32))
+    if m > 32:
+        np.testing.assert_array_equal(aux["base"].cpu().numpy().view(np.uint32), base.view(np.uint32))
+    else:   # decode kernel: the groups are summed per wave, then the waves (same terms, other order)
+        np.testing.assert_allclose(aux["base"].cpu().numpy(), base, rtol=2e-6, atol=1e-6 * float(np.abs(base).max()))
     rep = wc.compare(got.float().cpu().numpy(), o.bf16_round(want))
     assert rep["violations"] == 0, rep
