@@ -272,6 +272,13 @@ def bench_fused_backward(args, cfg, pkg, dev):
     rms_ms = timed(lambda: native.check("rms_norm_bwd", lib.mi355_w8a8_rms_norm_bwd_v1(
         plan.x.data_ptr(), plan.gamma.data_ptr(), plan.bwd.dx.data_ptr(), scratch_k.data_ptr(), m, k, plan.eps,
         stream)))
+    # the backward of a training forward that kept the projection and the normalized rows: no recomputation
+    def saved_projection_backward():
+        native.check("swiglu_bwd", lib.mi355_w8a8_swiglu_bwd_v1(
+            plan.fwd.out.data_ptr(), plan.d_product.data_ptr(), scratch_n.data_ptr(), m, n, stream))
+        plan.bwd.run()
+        plan.run_rms_stage()
+    saved_ms = timed(saved_projection_backward)
     dx_only = w8.BackwardPlan(None, plan.fwd.out, t["weight"], t["a"], t["b"], t["s"], adapter_indices=t["idx"],
                               need_lora_grads=False)
     dx_only.run()
@@ -292,6 +299,7 @@ def bench_fused_backward(args, cfg, pkg, dev):
                      "algorithmic_flops": flops, "algorithmic_bytes": 2 * m * n + k * n + 2 * m * k},
         "stages": {
             "forward_recompute_ms": float(fwd_ms.mean()), "linear_backward_ms": float(linear_ms.mean()),
+            "backward_with_saved_projection_ms": float(saved_ms.mean()),
             "swiglu_bwd_kernel": {"avg_ms": float(swiglu_ms.mean()), "algorithmic_bytes": swiglu_bytes,
                                   "achieved_gbs": swiglu_bytes / (float(swiglu_ms.mean()) * 1e-3) / 1e9,
                                   "frac_of_hbm": swiglu_bytes / (float(swiglu_ms.mean()) * 1e-3) / 1e9 / HBM_PEAK_GBS},

@@ -275,6 +275,13 @@ int mi355_w8a8_qkv_split_norm_rope_v1(const mi355_w8a8_qkv_post_problem* problem
  */
 int mi355_w8a8_swiglu_bwd_v1(const void* fused, const void* d_product, void* d_fused, uint32_t m, uint32_t n,
                              void* stream);
+/*
+ * The SwiGLU stage on its own (_fp32_swiglu_from_interleaved, :535-538): product bf16 [m, n / 2] from the
+ * bf16 projection [m, n], bit for bit what FLAG_SWIGLU produces.  A training forward that keeps the
+ * projection for the pull-back (as the reference's _forward_with_residuals does, :489-532) runs the
+ * projection without the flag and then this call, and its backward skips the recomputation.
+ */
+int mi355_w8a8_swiglu_v1(const void* fused, void* product, uint32_t m, uint32_t n, void* stream);
 int mi355_w8a8_rms_norm_bwd_v1(const void* x, const float* gamma, const void* d_normalized, void* d_x, uint32_t m,
                                uint32_t k, float eps, void* stream);
 

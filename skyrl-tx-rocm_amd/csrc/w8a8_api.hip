@@ -894,6 +894,22 @@ int run_swiglu_bwd(const void* fused, const void* d_product, void* d_fused, uint
   return launch_status();
 }
 
+int run_swiglu_fwd(const void* fused, void* product, uint32_t m, uint32_t n, hipStream_t s) {
+  if (!fused || !product) return MI355_W8A8_ERR_NULL;
+  if (m == 0 || n == 0 || (n & 7u)) return MI355_W8A8_ERR_SHAPE;
+  if (m > kMaxRows) return MI355_W8A8_ERR_UNSUPPORTED;
+  if (!aligned16(fused) || (reinterpret_cast<uintptr_t>(product) & 7u)) return MI355_W8A8_ERR_ALIGN;
+  if (overlaps(product, (uint64_t)m * n, fused, (uint64_t)m * n * 2u)) return MI355_W8A8_ERR_ALIAS;
+  SwigluFwdArgs a{};
+  a.fused = static_cast<const uint16_t*>(fused);
+  a.product = static_cast<uint16_t*>(product);
+  a.n_chunks = (uint64_t)m * n / 8u;
+  const uint64_t blocks = (a.n_chunks + 255u) / 256u;
+  (void)hipGetLastError();
+  hipLaunchKernelGGL(swiglu_fwd_kernel, dim3((uint32_t)(blocks < 16384u ? blocks : 16384u)), dim3(256), 0, s, a);
+  return launch_status();
+}
+
 int run_rms_norm_bwd(const void* x, const float* gamma, const void* d_normalized, void* d_x, uint32_t m, uint32_t k,
                      float eps, hipStream_t s) {
   if (!x || !gamma || !d_normalized || !d_x) return MI355_W8A8_ERR_NULL;
@@ -1337,6 +1353,10 @@ int mi355_w8a8_lora_linear_bwd_v1(const mi355_w8a8_bwd_problem* p, void* stream)
 
 int mi355_w8a8_qkv_split_norm_rope_v1(const mi355_w8a8_qkv_post_problem* p, void* stream) {
   return run_qkv_post(p, static_cast<hipStream_t>(stream));
+}
+
+int mi355_w8a8_swiglu_v1(const void* fused, void* product, uint32_t m, uint32_t n, void* stream) {
+  return run_swiglu_fwd(fused, product, m, n, static_cast<hipStream_t>(stream));
 }
 
 int mi355_w8a8_swiglu_bwd_v1(const void* fused, const void* d_product, void* d_fused, uint32_t m, uint32_t n,

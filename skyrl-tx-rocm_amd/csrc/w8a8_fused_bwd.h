@@ -49,6 +49,31 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(SwigluBwdArgs a) {
   }
 }
 
+// The SwiGLU stage on its own: product[m, j] = bf16(silu(gate) * up) of the bf16 projection, the same
+// arithmetic as the GEMM epilogue (bf16_rms_gate_up_lora_swiglu_contiguous.py:535-538).  A training
+// forward stores the projection for the pull-back and forms the product with this kernel.
+struct SwigluFwdArgs {
+  const uint16_t* fused;  // bf16 [M, N]
+  uint16_t* product;      // bf16 [M, N / 2]
+  uint64_t n_chunks;      // M * N / 8
+};
+
+__global__ __launch_bounds__(256) void swiglu_fwd_kernel(SwigluFwdArgs a) {
+  const uint64_t stride = (uint64_t)gridDim.x * 256u;
+  for (uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x; i < a.n_chunks; i += stride) {
+    const uint4 f = *reinterpret_cast<const uint4*>(a.fused + 8u * i);
+    const uint32_t w[4] = {f.x, f.y, f.z, f.w};
+    float p[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float g = __uint_as_float(w[j] << 16), u = __uint_as_float(w[j] & 0xffff0000u);
+      const float sig = __builtin_amdgcn_rcpf(1.0f + __expf(-g));
+      p[j] = (g * sig) * u;
+    }
+    *reinterpret_cast<uint2*>(a.product + 4u * i) = make_uint2(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]));
+  }
+}
+
 struct RmsNormBwdArgs {
   const uint16_t* x;    // bf16 [M, K]
   const float* gamma;   // f32 [K]: the multiplier itself (1 + delta for the Qwen3.5 flavour)

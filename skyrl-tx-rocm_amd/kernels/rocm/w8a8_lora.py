@@ -603,40 +603,85 @@ def rms_gate_up_swiglu_backward(x: torch.Tensor, gamma: torch.Tensor, weight, lo
                              adapter_indices=adapter_indices, eps=eps, need_lora_grads=need_lora_grads).run()
 
 
+def swiglu(fused: torch.Tensor) -> torch.Tensor:
+    """``bf16(silu(gate) * up)`` of an interleaved bf16 projection [..., N] -> [..., N / 2], bit for bit
+    what the fused forward produces (``_fp32_swiglu_from_interleaved``, :535-538)."""
+    if fused.dtype != torch.bfloat16:
+        raise TypeError(f"fused must be BF16, got {fused.dtype}")
+    _require_cuda(fused, "fused")
+    n = fused.shape[-1]
+    if fused.ndim < 2 or n % 8:
+        raise ValueError(f"need fused [..., N] with N % 8 == 0, got {tuple(fused.shape)}")
+    f2 = fused.reshape(-1, n).contiguous()
+    out = torch.empty((f2.shape[0], n // 2), dtype=torch.bfloat16, device=fused.device)
+    with torch.cuda.device(fused.device):
+        status = _native.load().mi355_w8a8_swiglu_v1(f2.data_ptr(), out.data_ptr(), f2.shape[0], n,
+                                                     _stream_ptr(fused.device))
+    _native.check("mi355_w8a8_swiglu_v1", status)
+    return out.reshape(*fused.shape[:-1], n // 2)
+
+
 class _RmsGateUpFunction(torch.autograd.Function):
     """The fused forward with the derivative rule of ``_bf16_rms_gate_up_lora_swiglu_contiguous``
     (bf16_rms_gate_up_lora_swiglu_contiguous.py:577-695): cotangents for x, A, B (and the scaling);
-    none for the norm weight and the frozen kernel."""
+    none for the norm weight and the frozen kernel.
+
+    With ``save_projection`` the forward keeps the bf16 projection and the normalized rows for the
+    backward, as the reference's training forward does (``_forward_with_residuals``, :489-532): the
+    projection runs without the SwiGLU flag and a separate kernel forms the product (bit-identical
+    output).  Without it the forward keeps nothing and the backward recomputes both.
+    """
 
     @staticmethod
-    def forward(ctx, x, lora_a, lora_b, lora_scaling, gamma, weight, adapter_indices, eps):
-        out = forward(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices,
-                      rms_gamma=gamma, eps=eps, swiglu=True, entry="gateup")
-        ctx.save_for_backward(x, lora_a, lora_b, lora_scaling, gamma)
+    def forward(ctx, x, lora_a, lora_b, lora_scaling, gamma, weight, adapter_indices, eps, save_projection):
         ctx.weight = weight
         ctx.adapter_indices = adapter_indices
         ctx.eps = eps
-        return out
+        ctx.saved_projection = bool(save_projection) and prepare_weight(weight).out_features % 8 == 0
+        if ctx.saved_projection:
+            # the tiled kernel, as the fused call takes it (the streaming kernels for few rows have no
+            # SwiGLU epilogue and add the LoRA term in another order): the product is then bit-identical
+            plan = ForwardPlan(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices,
+                               rms_gamma=gamma, eps=eps, want_normalized=True, flags=_native.FLAG_FORCE_TILED)
+            fused = plan.run()
+            ctx.save_for_backward(x, lora_a, lora_b, lora_scaling, gamma, fused, plan.aux["normalized"])
+            return swiglu(fused)
+        ctx.save_for_backward(x, lora_a, lora_b, lora_scaling, gamma)
+        return forward(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices,
+                       rms_gamma=gamma, eps=eps, swiglu=True, entry="gateup")
 
     @staticmethod
     def backward(ctx, d_product):
-        x, lora_a, lora_b, lora_scaling, gamma = ctx.saved_tensors
+        x, lora_a, lora_b, lora_scaling, gamma = ctx.saved_tensors[:5]
         need = lora_a is not None and any(ctx.needs_input_grad[1:4])
-        dx, da, db, ds = rms_gate_up_swiglu_backward(x, gamma, ctx.weight, lora_a, lora_b, lora_scaling,
-                                                     d_product.contiguous(), adapter_indices=ctx.adapter_indices,
-                                                     eps=ctx.eps, need_lora_grads=need)
+        if ctx.saved_projection:
+            fused, normalized = ctx.saved_tensors[5:]
+            d_fused = swiglu_backward(fused, d_product.contiguous().reshape(*fused.shape[:-1], -1))
+            idx = ctx.adapter_indices
+            rows = normalized.shape[0]
+            if idx is not None and idx.numel() != rows:
+                idx = idx.reshape(-1).repeat_interleave(rows // idx.numel())
+            dn, da, db, ds = backward(normalized, d_fused.reshape(rows, -1), ctx.weight, lora_a, lora_b, lora_scaling,
+                                      adapter_indices=idx, need_lora_grads=need)
+            dx = rms_norm_backward(x.reshape(rows, -1), gamma, dn, eps=ctx.eps, in_place=True).reshape(x.shape)
+        else:
+            dx, da, db, ds = rms_gate_up_swiglu_backward(x, gamma, ctx.weight, lora_a, lora_b, lora_scaling,
+                                                         d_product.contiguous(),
+                                                         adapter_indices=ctx.adapter_indices, eps=ctx.eps,
+                                                         need_lora_grads=need)
         if need:
             if lora_a.ndim == 2:
                 da, db = da[0], db[0]
             ds = ds.reshape(lora_scaling.shape).to(lora_scaling.dtype)
-        return dx, da, db, ds, None, None, None, None
+        return dx, da, db, ds, None, None, None, None, None
 
 
 def rms_gate_up_lora_swiglu(x: torch.Tensor, gamma: torch.Tensor, weight, lora_a=None, lora_b=None,
                             lora_scaling=None, *, adapter_indices: torch.Tensor | None = None,
-                            eps: float = 1e-6) -> torch.Tensor:
+                            eps: float = 1e-6, save_projection: bool = True) -> torch.Tensor:
     """RMSNorm (multiplier ``gamma``, float32) -> W8A8 gate/up (+LoRA) -> SwiGLU that autograd can
-    differentiate in x and the LoRA parameters."""
+    differentiate in x and the LoRA parameters.  ``save_projection`` (default, the reference's
+    choice) trades 2 * M * (N + K) bytes kept until the backward for not recomputing the projection."""
     tensors = [t for t in (x, lora_a, lora_b, lora_scaling) if isinstance(t, torch.Tensor)]
     if not (torch.is_grad_enabled() and any(t.requires_grad for t in tensors)):
         return forward(x, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices,
@@ -644,7 +689,7 @@ def rms_gate_up_lora_swiglu(x: torch.Tensor, gamma: torch.Tensor, weight, lora_a
     scaling = lora_scaling
     if lora_a is not None and not isinstance(scaling, torch.Tensor):
         scaling = torch.as_tensor(scaling, dtype=torch.float32, device=x.device)
-    return _RmsGateUpFunction.apply(x, lora_a, lora_b, scaling, gamma, weight, adapter_indices, eps)
+    return _RmsGateUpFunction.apply(x, lora_a, lora_b, scaling, gamma, weight, adapter_indices, eps, save_projection)
 
 
 # ---------------------------------------------------------------------------------------

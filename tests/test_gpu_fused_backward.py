@@ -276,3 +276,37 @@ def test_fused_backward_full_size_properties(dev, pkg):
         assert torch.equal(g2.float(), g1.float() * 2)
         assert not g0.any()
     assert float(one[0].float().abs().mean()) > 0
+
+
+def test_saved_projection_and_recomputation_agree(dev, pkg):
+    """The training forward that keeps the projection (the reference's choice) and the one that keeps
+    nothing give bit-identical outputs and cotangents; the stand-alone SwiGLU kernel reproduces the
+    fused epilogue bit for bit."""
+    import torch
+
+    m, k, n, r, n_ad = 150, 512, 1032, 16, 3
+    x, delta, w, a, b, s, idx, c = _fused_case(31, m, k, n, r, n_ad)
+    gamma = _t(dev, (F32(1.0) + delta).astype(F32), torch.float32)
+    ql, w8 = pkg.quantized_lora, pkg.w8a8_lora
+    wt = ql.GroupQuantizedWeight(torch.from_numpy(w.codes).to(dev), torch.from_numpy(w.scales).to(dev), k, k, 8, k)
+    it = _t(dev, idx, torch.int32)
+    results = []
+    for keep in (True, False):
+        xt = _t(dev, x).requires_grad_(True)
+        at = _t(dev, a).requires_grad_(True)
+        bt = _t(dev, b).requires_grad_(True)
+        st = _t(dev, s, torch.float32).requires_grad_(True)
+        out = w8.rms_gate_up_lora_swiglu(xt, gamma, wt, at, bt, st, adapter_indices=it, save_projection=keep)
+        out.backward(_t(dev, c))
+        torch.cuda.synchronize()
+        results.append((out.detach(), xt.grad, at.grad, bt.grad, st.grad))
+    for kept, recomputed in zip(*results):
+        assert torch.equal(kept, recomputed)
+    plain = w8.forward(_t(dev, x), wt, _t(dev, a), _t(dev, b), _t(dev, s, torch.float32), adapter_indices=it,
+                       rms_gamma=gamma)
+    assert torch.equal(w8.swiglu(plain), results[0][0])
+    with pytest.raises(ValueError):
+        w8.swiglu(plain[:, :12])
+    lib = pkg._native.load()
+    st_ = lib.mi355_w8a8_swiglu_v1(plain.data_ptr(), plain.data_ptr() + 16, m, n, None)
+    assert pkg._native.STATUS[st_] == "ERR_ALIAS"
