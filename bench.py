@@ -49,7 +49,7 @@ WORKLOADS = {
     # token routing around the expert GEMMs at the Qwen3-30B-A3B geometry: softmax / top-8 of 128 experts,
     # stable sort of the 32768 (token, choice) pairs with the gather of their rows, weighted combine
     "qwen3-30b-a3b-moe-routing-t4096": dict(m=4096, n_experts=128, top_k=8, hidden=2048, seed=6, moe_routing=True),
-    # the whole expert MLP of BASELINE config 5 (T = 2048): route, dispatch, grouped gate/up + SwiGLU, grouped down,
+    # the whole expert MLP of benchmark configuration 5 (T = 2048): route, dispatch, grouped gate/up + SwiGLU, grouped down,
     # combine; rank-16 LoRA on every expert
     "qwen3-30b-a3b-moe-mlp-t2048": dict(m=2048, n_experts=128, top_k=8, hidden=2048, intermediate=768, rank=16,
                                         seed=5, moe_mlp=True),

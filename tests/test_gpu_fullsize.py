@@ -1,4 +1,4 @@
-"""BASELINE configurations at full size: oracle comparison on row samples (rows are
+"""The benchmark configurations at full size: oracle comparison on row samples (rows are
 independent units of this path) plus size-independent exact properties."""
 
 import hashlib

@@ -105,7 +105,7 @@ def test_pack_unpack_roundtrip(dev, pkg, k, n):
 
 
 def test_config1_single_adapter(dev):
-    """BASELINE config 1: M128 K1024 N3072, one adapter rank 16 alpha 16."""
+    """benchmark configuration 1: M128 K1024 N3072, one adapter rank 16 alpha 16."""
     case = wc.make_case(128, 1024, 3072, n_adapters=1, rank=16, seed=1, idx_mode="zero")
     st = wc.oracle_forward(case, return_stages=True)
     got, aux = wc.gpu_forward(case)
