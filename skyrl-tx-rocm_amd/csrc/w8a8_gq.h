@@ -14,6 +14,7 @@
 //   gq_quant_kernel        per (row, group): amax, scale, codes (row-major int8, rows padded to 32)
 //   gq_lora_z_kernel       z = x @ A[idx] in float32
 //   gq_gemm_kernel         one wave per 64 x 64 output tile over all groups, epilogue, store
+//   gq_skinny_kernel       up to 32 rows: the groups dealt to the eight waves of a column block
 #pragma once
 #include "w8a8_device.h"
 
@@ -228,6 +229,38 @@ struct GqGemmArgs {
 
 // One wave per 64 x 64 output tile (2 x 2 blocks of 32 x 32), four waves (128 columns) per workgroup.
 // Lane l of a block holds column l % 32 and the 16 rows 8 (v / 4) + 4 (l / 32) + v % 4, v = 0..15.
+// A weight fragment as it sits in memory (8 or 16 bytes per lane) and its expansion to the int8
+// operand; kept apart so that a fragment loaded one step ahead is only expanded when it is used
+// (expanding at load time would make the load's latency part of the step).
+template <bool W4>
+struct GqRawFragment { uint4 v; };
+
+template <bool W4>
+__device__ inline GqRawFragment<W4> gq_load_raw(const unsigned char* p) {
+  GqRawFragment<W4> r;
+  if (W4) {
+    const uint2 t = *reinterpret_cast<const uint2*>(p);
+    r.v = make_uint4(t.x, t.y, 0u, 0u);
+  } else {
+    r.v = *reinterpret_cast<const uint4*>(p);
+  }
+  return r;
+}
+
+template <bool W4>
+__device__ inline v4i gq_expand(const GqRawFragment<W4>& r) {
+  v4i f;
+  if (W4) {
+    f[0] = (int)((r.v.x << 4) & 0xf0f0f0f0u);
+    f[1] = (int)(r.v.x & 0xf0f0f0f0u);
+    f[2] = (int)((r.v.y << 4) & 0xf0f0f0f0u);
+    f[3] = (int)(r.v.y & 0xf0f0f0f0u);
+  } else {
+    f[0] = (int)r.v.x; f[1] = (int)r.v.y; f[2] = (int)r.v.z; f[3] = (int)r.v.w;
+  }
+  return f;
+}
+
 template <bool W4>
 __device__ inline v4i gq_weight_fragment(const unsigned char* p) {
   if (W4) {
@@ -242,9 +275,98 @@ __device__ inline v4i gq_weight_fragment(const unsigned char* p) {
   return *reinterpret_cast<const v4i*>(p);
 }
 
+// Epilogue of one 32-row block of a wave's tile: the LoRA term per adapter present among the block's
+// rows (their z rows staged in the wave's LDS buffer), the add, the cast, the store.  outv[j][v] is the
+// float32 base of column block j, row 8 (v / 4) + 4 (lane / 32) + v % 4.
+__device__ inline void gq_store_row_block(const GqGemmArgs& a, const float (&outv)[2][16], uint32_t rb,
+                                          const uint32_t (&col)[2], bool two_cols, float (*zbuf)[64], uint32_t lane) {
+  const uint32_t h = lane >> 5;
+  const bool lora = a.z != nullptr;
+  float low[2][16];
+  if (lora) {
+    __builtin_amdgcn_wave_barrier();  // the buffer's previous use by this wave is over
+    for (uint32_t t = lane; t < 32u * 64u; t += 64u) {
+      const uint32_t rr = t >> 6, r = t & 63u;
+      const uint32_t row = rb * 32u + rr;
+      const bool ok = row < a.M && r < a.r;
+      const uint32_t zrow = (ok && a.z_slot) ? (uint32_t)a.z_slot[row] : row;
+      zbuf[rr][r] = ok ? a.z[(size_t)zrow * 64u + r] : 0.0f;
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_wave_barrier();
+    int ad_row[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const uint32_t row = rb * 32u + 8u * (v >> 2) + 4u * h + (v & 3);
+      int ad = (a.idx && row < a.M) ? a.idx[row] : 0;
+      ad_row[v] = ad < 0 ? 0 : (ad >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) low[j][v] = 0.0f;
+    }
+    // adapters present among the wave's rows, smallest first; every round handles one of them
+    int done_below = -1;
+    for (;;) {
+      int cand = 0x7fffffff;
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        if (ad_row[v] > done_below && ad_row[v] < cand) cand = ad_row[v];
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) {
+        const int o = __shfl_xor(cand, off);
+        cand = o < cand ? o : cand;
+      }
+      if (cand == 0x7fffffff) break;
+      done_below = cand;
+      const float sg = a.lora_scaling[cand];
+      for (uint32_t r0 = 0; r0 < a.r; r0 += 16u) {  // sixteen ranks of B in flight at a time
+        uint16_t braw[2][16];
+#pragma unroll
+        for (uint32_t t = 0; t < 16; ++t)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            braw[j][t] = (col[j] < a.N && r0 + t < a.r) ? a.lora_b[((size_t)cand * a.r + r0 + t) * a.N + col[j]]
+                                                         : (uint16_t)0;
+#pragma unroll
+        for (uint32_t t = 0; t < 16; ++t) {
+          if (r0 + t >= a.r) break;
+          const float bv[2] = {bf16_bits_to_f32(braw[0][t]), bf16_bits_to_f32(braw[1][t])};
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const float zv = zbuf[8 * (v >> 2) + 4 * (int)h + (v & 3)][r0 + t];
+            if (ad_row[v] == cand) {
+#pragma unroll
+              for (int j = 0; j < 2; ++j) low[j][v] = fmaf(zv, bv[j], low[j][v]);
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        if (ad_row[v] == cand) {
+#pragma unroll
+          for (int j = 0; j < 2; ++j) low[j][v] = low[j][v] * sg;
+        }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    if (j == 1 && !two_cols) break;
+    if (col[j] >= a.N) continue;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const uint32_t row = rb * 32u + 8u * (v >> 2) + 4u * h + (v & 3);
+      if (row >= a.M) continue;
+      float y = outv[j][v];
+      if (a.aux_base) a.aux_base[(size_t)row * a.N + col[j]] = y;
+      if (lora) y = y + low[j][v];
+      a.out[(size_t)row * a.N + col[j]] = (uint16_t)f32_to_bf16_bits(y);
+    }
+  }
+}
+
 template <bool W4>
 __global__ __launch_bounds__(256, 2) void gq_gemm_kernel(GqGemmArgs a) {
-  __shared__ float zs[4][64][64];  // per wave: the z rows of its tile (LoRA); reads are broadcasts, no padding needed
+  __shared__ float zs[4][32][64];  // per wave: the z rows of a row block (LoRA); reads are broadcasts, no padding needed
   constexpr uint32_t kBlkBytes = W4 ? 512u : 1024u, kLaneBytes = W4 ? 8u : 16u;
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
   const uint32_t cb0 = (blockIdx.x * 4u + wave) * 2u;  // first of the wave's two column blocks
@@ -264,148 +386,98 @@ __global__ __launch_bounds__(256, 2) void gq_gemm_kernel(GqGemmArgs a) {
   const uint32_t col[2] = {cb0 * 32u + c, cb1 * 32u + c};
   const uint32_t rbs[2] = {rb0, rb1};
   float outv[2][2][16];
-  v4i fa0 = *reinterpret_cast<const v4i*>(ar0), fa1 = *reinterpret_cast<const v4i*>(ar1);
-  v4i fb0 = gq_weight_fragment<W4>(w0), fb1 = gq_weight_fragment<W4>(w1);
-  for (uint32_t g = 0; g < a.G; ++g) {
-    v16i acc[2][2];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
-    // the group's scales are requested before its MFMAs so that they have arrived when those end
-    float sw[2];
+      for (int v = 0; v < 16; ++v) outv[i][j][v] = 0.0f;
+  v16i acc[2][2];
+  float sw[2];
+  float4 sx4[2][4];
+  // the group's scales are requested when it starts so that they have arrived when its MFMAs end
+  auto load_scales = [&](uint32_t g) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) sw[j] = col[j] < a.N ? a.ws[(size_t)g * a.N + col[j]] : 0.0f;
-    float4 sx4[2][4];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int q = 0; q < 4; ++q)  // rows 8 q + 4 h + 0..3 of the block: four consecutive scales
         sx4[i][q] = *reinterpret_cast<const float4*>(a.xs + (size_t)g * a.M_pad + rbs[i] * 32u + 8u * q + 4u * h);
-    for (uint32_t b = 0; b < blocks_per_group; ++b) {
-      const uint32_t kb = g * blocks_per_group + b;
-      const uint32_t kn = kb + 1u < kbs ? kb + 1u : kb;  // the next step's fragments travel during the MFMAs
-      const v4i na0 = *reinterpret_cast<const v4i*>(ar0 + (size_t)kn * 1024u);
-      const v4i na1 = *reinterpret_cast<const v4i*>(ar1 + (size_t)kn * 1024u);
-      const v4i nb0 = gq_weight_fragment<W4>(w0 + (size_t)kn * kBlkBytes);
-      const v4i nb1 = gq_weight_fragment<W4>(w1 + (size_t)kn * kBlkBytes);
+  };
+  // one k block: four MFMAs (from zero when the block opens a group) and, when it closes a group,
+  // (f32(acc) * sx) * sw added in group order; for 4-bit codes sw carries the exact factor 1/16
+  auto step = [&](uint32_t kb, const v4i& fa0, const v4i& fa1, const GqRawFragment<W4>& r0, const GqRawFragment<W4>& r1) {
+    const v4i fb0 = gq_expand<W4>(r0), fb1 = gq_expand<W4>(r1);
+    if (kb % blocks_per_group == 0) {
+      const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+      acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa0, fb0, zero, 0, 0, 0);
+      acc[0][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa0, fb1, zero, 0, 0, 0);
+      acc[1][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa1, fb0, zero, 0, 0, 0);
+      acc[1][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa1, fb1, zero, 0, 0, 0);
+    } else {
       acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa0, fb0, acc[0][0], 0, 0, 0);
       acc[0][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa0, fb1, acc[0][1], 0, 0, 0);
       acc[1][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa1, fb0, acc[1][0], 0, 0, 0);
       acc[1][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa1, fb1, acc[1][1], 0, 0, 0);
-      fa0 = na0; fa1 = na1; fb0 = nb0; fb1 = nb1;
     }
-    // (f32(acc) * sx) * sw in the reference's order; for 4-bit codes sw carries the exact factor 1/16
-    if (W4) {
-#pragma unroll
-      for (int j = 0; j < 2; ++j) sw[j] = sw[j] * 0.0625f;
-    }
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const float sxq[4] = {sx4[i][q].x, sx4[i][q].y, sx4[i][q].z, sx4[i][q].w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int v = 4 * q + e;
-#pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            float t = (float)acc[i][j][v] * sxq[e];
-            t = t * sw[j];
-            outv[i][j][v] = g == 0 ? t : outv[i][j][v] + t;
-          }
-        }
+    if ((kb + 1u) % blocks_per_group == 0) {
+      float swl[2] = {sw[0], sw[1]};
+      if (W4) {
+        swl[0] = swl[0] * 0.0625f;
+        swl[1] = swl[1] * 0.0625f;
       }
-  }
-  // ---- epilogue: LoRA term per adapter present in the tile, store
-  const bool lora = a.z != nullptr;
-  if (lora) {
-    for (uint32_t t = lane; t < 64u * 64u; t += 64u) {
-      const uint32_t rr = t >> 6, r = t & 63u;
-      const uint32_t row = (rr < 32u ? rb0 : rb1) * 32u + (rr & 31u);
-      const bool ok = row < a.M && r < a.r;
-      const uint32_t zrow = (ok && a.z_slot) ? (uint32_t)a.z_slot[row] : row;
-      zs[wave][rr][r] = ok ? a.z[(size_t)zrow * 64u + r] : 0.0f;
-    }
-    __builtin_amdgcn_s_waitcnt(0xc07f);
-    __builtin_amdgcn_wave_barrier();
-  }
+      float4 sxl[2][4];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    if (i == 1 && rb1 == rb0) break;
-    float low[2][16];
-    int ad_row[16];
-    if (lora) {
+      for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const uint32_t row = rbs[i] * 32u + 8u * (v >> 2) + 4u * h + (v & 3);
-        int ad = (a.idx && row < a.M) ? a.idx[row] : 0;
-        ad_row[v] = ad < 0 ? 0 : (ad >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad);
+        for (int q = 0; q < 4; ++q) sxl[i][q] = sx4[i][q];
+      const uint32_t gn = (kb + 1u) / blocks_per_group;
+      if (gn < a.G) load_scales(gn);
 #pragma unroll
-        for (int j = 0; j < 2; ++j) low[j][v] = 0.0f;
-      }
-      // adapters present among the wave's rows, smallest first; every round handles one of them
-      int done_below = -1;
-      for (;;) {
-        int cand = 0x7fffffff;
+      for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int v = 0; v < 16; ++v)
-          if (ad_row[v] > done_below && ad_row[v] < cand) cand = ad_row[v];
+        for (int q = 0; q < 4; ++q) {
+          const float sxq[4] = {sxl[i][q].x, sxl[i][q].y, sxl[i][q].z, sxl[i][q].w};
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-          const int o = __shfl_xor(cand, off);
-          cand = o < cand ? o : cand;
-        }
-        if (cand == 0x7fffffff) break;
-        done_below = cand;
-        const float sg = a.lora_scaling[cand];
-        for (uint32_t r0 = 0; r0 < a.r; r0 += 16u) {  // sixteen ranks of B in flight at a time
-          uint16_t braw[2][16];
+          for (int e = 0; e < 4; ++e) {
+            const int v = 4 * q + e;
 #pragma unroll
-          for (uint32_t t = 0; t < 16; ++t)
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-              braw[j][t] = (col[j] < a.N && r0 + t < a.r) ? a.lora_b[((size_t)cand * a.r + r0 + t) * a.N + col[j]]
-                                                           : (uint16_t)0;
-#pragma unroll
-          for (uint32_t t = 0; t < 16; ++t) {
-            if (r0 + t >= a.r) break;
-            const float bv[2] = {bf16_bits_to_f32(braw[0][t]), bf16_bits_to_f32(braw[1][t])};
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-              const float zv = zs[wave][i * 32 + 8 * (v >> 2) + 4 * (int)h + (v & 3)][r0 + t];
-              if (ad_row[v] == cand) {
-#pragma unroll
-                for (int j = 0; j < 2; ++j) low[j][v] = fmaf(zv, bv[j], low[j][v]);
-              }
+            for (int j = 0; j < 2; ++j) {
+              float t = (float)acc[i][j][v] * sxq[e];
+              t = t * swl[j];
+              outv[i][j][v] = outv[i][j][v] + t;  // from +0: the first term as it is (a product is never -0 here)
             }
           }
         }
-#pragma unroll
-        for (int v = 0; v < 16; ++v)
-          if (ad_row[v] == cand) {
-#pragma unroll
-            for (int j = 0; j < 2; ++j) low[j][v] = low[j][v] * sg;
-          }
-      }
     }
+  };
+  // two sets of fragments take turns: one is used while the other travels (no copies between steps:
+  // the loop is unrolled by the number of sets so that every set has its own registers; four sets
+  // were measured slower)
+  constexpr uint32_t kSets = 2;
+  v4i fa[kSets][2];
+  GqRawFragment<W4> fr[kSets][2];
+  auto load_set = [&](uint32_t set, uint32_t kb) {
+    const uint32_t k = kb < kbs ? kb : kbs - 1u;  // beyond the end: a repeated block, unused
+    fa[set][0] = *reinterpret_cast<const v4i*>(ar0 + (size_t)k * 1024u);
+    fa[set][1] = *reinterpret_cast<const v4i*>(ar1 + (size_t)k * 1024u);
+    fr[set][0] = gq_load_raw<W4>(w0 + (size_t)k * kBlkBytes);
+    fr[set][1] = gq_load_raw<W4>(w1 + (size_t)k * kBlkBytes);
+  };
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      if (j == 1 && cb1 == cb0) break;
-      if (col[j] >= a.N) continue;
+  for (uint32_t u = 0; u + 1u < kSets; ++u) load_set(u, u);
+  load_scales(0);
+  for (uint32_t kb = 0; kb < kbs; kb += kSets) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const uint32_t row = rbs[i] * 32u + 8u * (v >> 2) + 4u * h + (v & 3);
-        if (row >= a.M) continue;
-        float y = outv[i][j][v];
-        if (a.aux_base) a.aux_base[(size_t)row * a.N + col[j]] = y;
-        if (lora) y = y + low[j][v];
-        a.out[(size_t)row * a.N + col[j]] = (uint16_t)f32_to_bf16_bits(y);
-      }
+    for (uint32_t u = 0; u < kSets; ++u) {
+      load_set((u + kSets - 1u) % kSets, kb + u + kSets - 1u);
+      if (kb + u < kbs) step(kb + u, fa[u][0], fa[u][1], fr[u][0], fr[u][1]);
     }
   }
+  // ---- epilogue: LoRA term per adapter present in the tile, store
+  gq_store_row_block(a, outv[0], rb0, col, cb1 != cb0, zs[wave], lane);
+  if (rb1 != rb0) gq_store_row_block(a, outv[1], rb1, col, cb1 != cb0, zs[wave], lane);
 }
 
 // ---------------------------------------------------------------------------------------

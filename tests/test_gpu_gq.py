@@ -82,6 +82,9 @@ CASES = [
     (300, 2048, 256, 4, 8, 2048, 64, 2),  # one group: per-channel W4
     (45, 100, 40, 4, 8, 32, 5, 3),        # K not a multiple of 8: LoRA-A by the wave-per-row kernel
     (90, 256, 72, 8, 8, 64, 12, 1),       # one adapter without indices
+    (2050, 200, 2056, 4, 8, 64, 8, 3),    # many tiles, ragged edges, an odd number of k blocks
+    (2048, 384, 2048, 8, 4, 96, 0, 0),    # 8-bit codes, three k blocks a group
+    (1024, 2048, 512, 4, 8, 1024, 40, 5),  # long groups
 ]
 
 
