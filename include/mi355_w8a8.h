@@ -27,6 +27,8 @@
  *   - mi355_w8a8_swiglu_bwd_v1 / mi355_w8a8_rms_norm_bwd_v1
  *                                      skyrl/tx/kernels/rocm/bf16_rms_gate_up_lora_swiglu_contiguous.py:541-574
  *   - mi355_w8a8_qkv_split_norm_rope_v1 skyrl/tx/kernels/qwen3_5_qkv_lora.py:266-286
+ *   - mi355_w8a8_qkv_split_norm_rope_bwd_v1, mi355_w8a8_delta_rms_norm_bwd_v1
+ *                                       skyrl/tx/kernels/qwen3_5_qkv_lora.py:360-451
  *   - mi355_w8a8_moe_route_v1 / _moe_dispatch_v1 / _moe_combine_v1
  *                                      skyrl/tx/models/qwen3.py:172-210, skyrl/tx/layers/util.py:66-87
  *   - mi355_w8a8_gq_linear_v1          skyrl/tx/kernels/quantized_lora.py:215-304 in its general form
@@ -204,6 +206,37 @@ typedef struct mi355_w8a8_qkv_post_problem {
   void* gate;               /* bf16 [m, num_query_heads * head_dim] */
 } mi355_w8a8_qkv_post_problem;
 
+/*
+ * Pull-back of the stage above.  fused is the raw projection the forward consumed; the four output
+ * cotangents come in, the cotangent of the fused projection goes out, optionally with the
+ * cotangents of the two head-norm weights.
+ */
+typedef struct mi355_w8a8_qkv_post_bwd_problem {
+  uint32_t struct_size;     /* sizeof(mi355_w8a8_qkv_post_bwd_problem) */
+  uint32_t flags;           /* 0 */
+  uint32_t m;
+  uint32_t num_query_heads;
+  uint32_t num_kv_heads;
+  uint32_t head_dim;
+  uint32_t rotary_dim;
+  float rope_theta;
+  float rms_eps;
+  uint32_t reserved;
+  const void* fused;        /* bf16 [m, fused width] */
+  const float* q_norm_weight; /* f32 [head_dim], delta form */
+  const float* k_norm_weight; /* f32 [head_dim] */
+  const int32_t* positions; /* int32 [m] */
+  const void* d_q;          /* bf16 [m, num_query_heads, head_dim] */
+  const void* d_k;          /* bf16 [m, num_kv_heads, head_dim] */
+  const void* d_v;          /* bf16 [m, num_kv_heads, head_dim] */
+  const void* d_gate;       /* bf16 [m, num_query_heads * head_dim] */
+  void* d_fused;            /* bf16 [m, fused width] */
+  float* d_q_norm_weight;   /* f32 [head_dim] or NULL; both or neither */
+  float* d_k_norm_weight;   /* f32 [head_dim] or NULL */
+  void* workspace;          /* needed with the weight cotangents only */
+  uint64_t workspace_bytes; /* >= mi355_w8a8_qkv_bwd_workspace_bytes(m, head_dim) */
+} mi355_w8a8_qkv_post_bwd_problem;
+
 int mi355_w8a8_abi_version(void);
 const char* mi355_w8a8_status_string(int status);
 
@@ -254,6 +287,31 @@ int mi355_w8a8_lora_linear_bwd_v1(const mi355_w8a8_bwd_problem* problem, void* s
  * rms_gamma = 1 + input_norm_weight.
  */
 int mi355_w8a8_qkv_split_norm_rope_v1(const mi355_w8a8_qkv_post_problem* problem, void* stream);
+
+/*
+ * Pull-back of qwen35_qkv_lora_rope behind and before the projection
+ * (_qwen35_qkv_lora_rope_bwd, skyrl/tx/kernels/qwen3_5_qkv_lora.py:360-451).  The whole rule, with
+ * fused and normalized = the projection and its normalized input (mi355_w8a8_forward_v1 with
+ * rms_gamma = 1 + input_norm_weight and aux_normalized), is
+ *   d_fused [, d_q_norm_weight, d_k_norm_weight] = qkv_split_norm_rope_bwd(fused, d_q, d_k, d_v, d_gate)
+ *   d_normalized, d_lora_a, d_lora_b, d_lora_scaling = mi355_w8a8_lora_linear_bwd_v1(normalized, d_fused)
+ *   d_hidden [, d_input_norm_weight] = delta_rms_norm_bwd(hidden, 1 + input_norm_weight, d_normalized)
+ *
+ * mi355_w8a8_qkv_split_norm_rope_bwd_v1 replaces :391-425: _apply_partial_rope_transpose (:148-164)
+ * on d_q and d_k, _delta_rms_norm_vjp (:97-116) per Q and K head against the raw projection, and
+ * _fuse_interleaved_qkv (:235-247) of the result with d_gate and d_v.
+ *
+ * mi355_w8a8_delta_rms_norm_bwd_v1 replaces _delta_rms_norm_vjp (:97-116) for the decoder norm: x,
+ * d_normalized, d_x bf16 [m, k]; gamma f32 [k] is the multiplier 1 + weight.  d_gamma f32 [k] is
+ * optional (the cotangent of the weight; 1 + weight has the same one) and then needs the workspace
+ * and a d_x buffer apart from d_normalized; without it d_x may be the d_normalized buffer itself.
+ */
+uint64_t mi355_w8a8_qkv_bwd_workspace_bytes(uint32_t m, uint32_t head_dim);
+int mi355_w8a8_qkv_split_norm_rope_bwd_v1(const mi355_w8a8_qkv_post_bwd_problem* problem, void* stream);
+uint64_t mi355_w8a8_delta_rms_norm_bwd_workspace_bytes(uint32_t m, uint32_t k);
+int mi355_w8a8_delta_rms_norm_bwd_v1(const void* x, const float* gamma, const void* d_normalized, void* d_x,
+                                     float* d_gamma, void* workspace, uint64_t workspace_bytes, uint32_t m,
+                                     uint32_t k, float eps, void* stream);
 
 /*
  * The two stages around the projection in the pull-back of the fused RMSNorm -> gate/up + LoRA ->

@@ -40,6 +40,12 @@ How each function is pinned (the tests that do it live in ``tests/test_oracle_*.
   preservation, position 0 and ``rotary_dim`` 0 identities, and an enumerated interleaving
   (tests/tx/kernels/test_qwen3_5_qkv_lora.py:75-83 states it as ``FusedLoRALinear.split``).
   sin/cos/pow of XLA-CPU are not available: PARITY UNPINNED in their last float32 bits.
+* ``apply_partial_rope_transpose``/``delta_rms_norm_vjp``/``qkv_split_norm_rope_bwd``/
+  ``w8a8_qkv_lora_rope_bwd``: the adjoint identity <R x, y> = <x, R^T y> and R^T R = 1 of the rotation,
+  ``torch.autograd`` (float64, CPU) through the smooth RMSNorm with ``1 + weight`` for dx and dweight,
+  the re-interleave as the exact adjoint of the split (enumerated), and the composite against
+  autograd through the whole smooth stage on bf16-exact inputs.  PARITY UNPINNED in the last
+  float32 bits of XLA's reductions, rsqrt, sin, cos and pow.
 * ``moe_route``/``moe_combine``/``moe_expert_mlp``: ``torch.topk``/``scipy.special.softmax`` special
   cases and the merged-weight invariant of tests/tx/models/test_qwen3.py:123-180.
 """
@@ -123,6 +129,100 @@ def w8a8_qkv_lora_rope(hidden, input_norm_weight, q_norm_weight, k_norm_weight, 
     else:
         fused = quantized_lora_linear_multi(normalized, weight, lora_a, lora_b, lora_scaling, adapter_indices)
     return qkv_split_norm_rope(fused, q_norm_weight, k_norm_weight, positions, **config)
+
+
+# ---------------------------------------------------------------------------
+# pull-back of the Qwen3.5 attention input stage (qwen3_5_qkv_lora.py:97-116, 148-164, 360-451)
+# ---------------------------------------------------------------------------
+
+def apply_partial_rope_transpose(dy, positions, rotary_dim: int, rope_theta: float) -> np.ndarray:
+    """qwen3_5_qkv_lora.py:148-164: the transposed rotation on a bf16 cotangent [..., heads, head_dim]:
+    [first cos + second sin, -first sin + second cos] in float32, one cast; the rest passes through."""
+    dy = np.asarray(dy, dtype=F32)
+    if rotary_dim == 0:
+        return dy.copy()
+    half = rotary_dim // 2
+    first, second = dy[..., :half], dy[..., half:rotary_dim]
+    sin, cos = rope_sin_cos(positions, rotary_dim, rope_theta)
+    sin, cos = sin[..., None, :], cos[..., None, :]
+    out = dy.copy()
+    out[..., :half] = bf16_round((first * cos).astype(F32) + (second * sin).astype(F32))
+    out[..., half:rotary_dim] = bf16_round((-first * sin).astype(F32) + (second * cos).astype(F32))
+    return out
+
+
+def delta_rms_norm_vjp(x, weight, dy, eps: float):
+    """qwen3_5_qkv_lora.py:97-116 on rows [rows, width] (bf16 values): float32 statistics with the
+    forward's mean and rsqrt rule, dx = bf16(inv * (dy (1 + w) - n * mean(dy (1 + w) n))) and the
+    float32 weight cotangent sum_rows(dy * n) (summed in float64, rounded once; the reference's
+    float32 reduction order is XLA's: PARITY UNPINNED in its last bits)."""
+    x = np.asarray(x, dtype=F32)
+    dy = np.asarray(dy, dtype=F32)
+    ew = (F32(1.0) + np.asarray(weight, dtype=F32)).astype(F32)
+    width = x.shape[-1]
+    ssq = np.sum(x.astype(np.float64) * x.astype(np.float64), axis=-1, keepdims=True)
+    inv = (F32(1.0) / np.sqrt(((ssq / np.float64(width)).astype(F32) + F32(eps)).astype(F32))).astype(F32)
+    normalized = (x * inv).astype(F32)
+    weighted = (dy * ew).astype(F32)
+    prod = (weighted * normalized).astype(F32)
+    mu = (np.sum(prod.astype(np.float64), axis=-1, keepdims=True) / np.float64(width)).astype(F32)
+    dx = (inv * (weighted - (normalized * mu).astype(F32)).astype(F32)).astype(F32)
+    dweight = np.sum((dy * normalized).astype(F32).astype(np.float64).reshape(-1, width), axis=0).astype(F32)
+    return bf16_round(dx), dweight
+
+
+def qkv_split_norm_rope_bwd(fused, q_norm_weight, k_norm_weight, positions, dq, dk, dv, dgate, *,
+                            num_query_heads: int, num_kv_heads: int, head_dim: int, rotary_dim: int,
+                            rope_theta: float, eps: float):
+    """qwen3_5_qkv_lora.py:389-425: from the raw projection [rows, width] and the four output
+    cotangents to the cotangent of the projection (bf16 values) and the float32 cotangents of the
+    two head-norm weights."""
+    fused = np.asarray(fused, dtype=F32)
+    rows = fused.shape[0]
+    qpk = num_query_heads // num_kv_heads
+    q_proj, k_proj, _ = split(fused, (qpk * 2 * head_dim, head_dim, head_dim))
+    q_raw = q_proj.reshape(rows, num_query_heads, 2 * head_dim)[..., :head_dim]
+    k_raw = k_proj.reshape(rows, num_kv_heads, head_dim)
+    dq = apply_partial_rope_transpose(np.asarray(dq, dtype=F32).reshape(rows, num_query_heads, head_dim),
+                                      positions, rotary_dim, rope_theta)
+    dk = apply_partial_rope_transpose(np.asarray(dk, dtype=F32).reshape(rows, num_kv_heads, head_dim),
+                                      positions, rotary_dim, rope_theta)
+    dq_raw, dq_w = delta_rms_norm_vjp(q_raw.reshape(-1, head_dim), q_norm_weight, dq.reshape(-1, head_dim), eps)
+    dk_raw, dk_w = delta_rms_norm_vjp(k_raw.reshape(-1, head_dim), k_norm_weight, dk.reshape(-1, head_dim), eps)
+    dq_proj = np.concatenate([dq_raw.reshape(rows, num_query_heads, head_dim),
+                              np.asarray(dgate, dtype=F32).reshape(rows, num_query_heads, head_dim)],
+                             axis=-1).reshape(rows, num_query_heads * 2 * head_dim)
+    dfused = fuse(dq_proj, dk_raw.reshape(rows, num_kv_heads * head_dim),
+                  np.asarray(dv, dtype=F32).reshape(rows, num_kv_heads * head_dim),
+                  group_sizes=(qpk * 2 * head_dim, head_dim, head_dim))
+    return dfused, dq_w, dk_w
+
+
+def w8a8_qkv_lora_rope_bwd(hidden, input_norm_weight, q_norm_weight, k_norm_weight, weight: GroupQuantizedWeight,
+                           lora_a, lora_b, lora_scaling, adapter_indices, positions, dq, dk, dv, dgate,
+                           relaxed_weight: bool = True, **config):
+    """The structure of _qwen35_qkv_lora_rope_bwd (qwen3_5_qkv_lora.py:360-451) with the quantized
+    projection's own rule in the middle (``quantized_lora_linear_multi_bwd``).  Returns a dict with
+    dhidden, d_input_norm_weight, d_q_norm_weight, d_k_norm_weight, d_lora_a, d_lora_b, d_lora_scaling
+    and the intermediate dfused."""
+    eps = config["eps"]
+    normalized = delta_rms_norm(hidden, input_norm_weight, eps)
+    if lora_a is None:
+        fused = quantized_frozen_linear(normalized, weight)
+    else:
+        fused = quantized_lora_linear_multi(normalized, weight, lora_a, lora_b, lora_scaling, adapter_indices)
+    dfused, dq_w, dk_w = qkv_split_norm_rope_bwd(fused, q_norm_weight, k_norm_weight, positions, dq, dk, dv, dgate,
+                                                 **config)
+    if lora_a is None:
+        dn = bf16_round(_mm64(dfused, pullback_weight(weight, relaxed_weight).T))
+        da = db = ds = None
+    else:
+        dn, da, db, ds = quantized_lora_linear_multi_bwd(normalized, weight, lora_a, lora_b, lora_scaling,
+                                                         adapter_indices, dfused, relaxed_weight)
+    dhidden, d_in_w = delta_rms_norm_vjp(hidden, input_norm_weight, dn, eps)
+    return {"dhidden": dhidden, "d_input_norm_weight": d_in_w, "d_q_norm_weight": dq_w, "d_k_norm_weight": dk_w,
+            "d_lora_a": da, "d_lora_b": db, "d_lora_scaling": ds, "dfused": dfused, "fused": fused,
+            "normalized": normalized, "d_normalized": dn}
 
 
 # ---------------------------------------------------------------------------

@@ -37,6 +37,8 @@ EXPORTS = (
     "mi355_w8a8_forward_v1", "mi355_w8a8_grouped_v1",
     "mi355_w8a8_bwd_workspace_bytes", "mi355_w8a8_lora_linear_bwd_v1",
     "mi355_w8a8_qkv_split_norm_rope_v1",
+    "mi355_w8a8_qkv_bwd_workspace_bytes", "mi355_w8a8_qkv_split_norm_rope_bwd_v1",
+    "mi355_w8a8_delta_rms_norm_bwd_workspace_bytes", "mi355_w8a8_delta_rms_norm_bwd_v1",
     "mi355_w8a8_swiglu_v1", "mi355_w8a8_swiglu_bwd_v1", "mi355_w8a8_rms_norm_bwd_v1",
     "mi355_w8a8_moe_route_v1", "mi355_w8a8_moe_dispatch_workspace_bytes", "mi355_w8a8_moe_dispatch_v1",
     "mi355_w8a8_moe_combine_v1",
@@ -93,6 +95,18 @@ class QkvPostProblem(ctypes.Structure):
         ("head_dim", _u32), ("rotary_dim", _u32), ("rope_theta", _f32), ("rms_eps", _f32), ("reserved", _u32),
         ("fused", _vp), ("q_norm_weight", _vp), ("k_norm_weight", _vp), ("positions", _vp),
         ("q", _vp), ("k", _vp), ("v", _vp), ("gate", _vp),
+    ]
+
+
+class QkvPostBwdProblem(ctypes.Structure):
+    """struct mi355_w8a8_qkv_post_bwd_problem"""
+
+    _fields_ = [
+        ("struct_size", _u32), ("flags", _u32), ("m", _u32), ("num_query_heads", _u32), ("num_kv_heads", _u32),
+        ("head_dim", _u32), ("rotary_dim", _u32), ("rope_theta", _f32), ("rms_eps", _f32), ("reserved", _u32),
+        ("fused", _vp), ("q_norm_weight", _vp), ("k_norm_weight", _vp), ("positions", _vp),
+        ("d_q", _vp), ("d_k", _vp), ("d_v", _vp), ("d_gate", _vp), ("d_fused", _vp),
+        ("d_q_norm_weight", _vp), ("d_k_norm_weight", _vp), ("workspace", _vp), ("workspace_bytes", _u64),
     ]
 
 
@@ -160,6 +174,14 @@ def _bind(lib: ctypes.CDLL) -> None:
     lib.mi355_w8a8_lora_linear_bwd_v1.argtypes = (ctypes.POINTER(BwdProblem), _vp)
     lib.mi355_w8a8_qkv_split_norm_rope_v1.restype = ctypes.c_int
     lib.mi355_w8a8_qkv_split_norm_rope_v1.argtypes = (ctypes.POINTER(QkvPostProblem), _vp)
+    lib.mi355_w8a8_qkv_bwd_workspace_bytes.restype = _u64
+    lib.mi355_w8a8_qkv_bwd_workspace_bytes.argtypes = (_u32, _u32)
+    lib.mi355_w8a8_qkv_split_norm_rope_bwd_v1.restype = ctypes.c_int
+    lib.mi355_w8a8_qkv_split_norm_rope_bwd_v1.argtypes = (ctypes.POINTER(QkvPostBwdProblem), _vp)
+    lib.mi355_w8a8_delta_rms_norm_bwd_workspace_bytes.restype = _u64
+    lib.mi355_w8a8_delta_rms_norm_bwd_workspace_bytes.argtypes = (_u32, _u32)
+    lib.mi355_w8a8_delta_rms_norm_bwd_v1.restype = ctypes.c_int
+    lib.mi355_w8a8_delta_rms_norm_bwd_v1.argtypes = (_vp, _vp, _vp, _vp, _vp, _vp, _u64, _u32, _u32, _f32, _vp)
     lib.mi355_w8a8_moe_route_v1.restype = ctypes.c_int
     lib.mi355_w8a8_moe_route_v1.argtypes = (_vp, _u32, _u32, _u32, _u32, _vp, _vp, _vp)
     lib.mi355_w8a8_moe_dispatch_workspace_bytes.restype = _u64

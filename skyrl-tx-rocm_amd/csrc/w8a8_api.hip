@@ -873,6 +873,136 @@ int run_qkv_post(const mi355_w8a8_qkv_post_problem* p, hipStream_t s) {
   return launch_status();
 }
 
+// Workgroups of the QKV pull-back when the head-norm weights get cotangents: each leaves one partial.
+inline uint32_t qkv_bwd_parts(uint32_t m) { return m < 1024u ? m : 1024u; }
+inline uint64_t qkv_bwd_workspace_bytes(uint32_t m, uint32_t head_dim) {
+  return (uint64_t)qkv_bwd_parts(m) * 2u * head_dim * 4u;
+}
+
+int run_qkv_post_bwd(const mi355_w8a8_qkv_post_bwd_problem* p, hipStream_t s) {
+  if (!p) return MI355_W8A8_ERR_NULL;
+  if (p->struct_size != sizeof(mi355_w8a8_qkv_post_bwd_problem)) return MI355_W8A8_ERR_STRUCT;
+  if (p->flags) return MI355_W8A8_ERR_SHAPE;
+  if (p->m == 0 || p->num_query_heads == 0 || p->num_kv_heads == 0 || p->head_dim == 0) return MI355_W8A8_ERR_SHAPE;
+  if (p->num_query_heads % p->num_kv_heads) return MI355_W8A8_ERR_SHAPE;
+  if ((p->head_dim & 1u) || (p->rotary_dim & 1u) || p->rotary_dim > p->head_dim) return MI355_W8A8_ERR_SHAPE;
+  if (!(p->rope_theta > 0.0f) || !(p->rms_eps > 0.0f)) return MI355_W8A8_ERR_SHAPE;
+  if (p->head_dim > kQkvMaxHeadDim || p->m > kMaxRows || p->num_query_heads > 1024u) return MI355_W8A8_ERR_UNSUPPORTED;
+  const uint64_t width = ((uint64_t)p->num_query_heads * 2u + 2u * p->num_kv_heads) * p->head_dim;
+  if (width * p->m >= (1ull << 32)) return MI355_W8A8_ERR_UNSUPPORTED;
+  if (!p->fused || !p->q_norm_weight || !p->k_norm_weight || !p->positions || !p->d_q || !p->d_k || !p->d_v ||
+      !p->d_gate || !p->d_fused)
+    return MI355_W8A8_ERR_NULL;
+  const bool wgrad = p->d_q_norm_weight != nullptr;
+  if (wgrad != (p->d_k_norm_weight != nullptr)) return MI355_W8A8_ERR_NULL;
+  if (!aligned16(p->fused) || !aligned16(p->d_q) || !aligned16(p->d_k) || !aligned16(p->d_v) || !aligned16(p->d_gate) ||
+      !aligned16(p->d_fused) || !aligned16(p->q_norm_weight) || !aligned16(p->k_norm_weight) ||
+      (reinterpret_cast<uintptr_t>(p->positions) & 3u))
+    return MI355_W8A8_ERR_ALIGN;
+  const uint64_t fused_bytes = width * p->m * 2u;
+  const uint64_t q_bytes = (uint64_t)p->m * p->num_query_heads * p->head_dim * 2u;
+  const uint64_t kv_bytes = (uint64_t)p->m * p->num_kv_heads * p->head_dim * 2u;
+  if (overlaps(p->d_fused, fused_bytes, p->fused, fused_bytes) || overlaps(p->d_fused, fused_bytes, p->d_q, q_bytes) ||
+      overlaps(p->d_fused, fused_bytes, p->d_gate, q_bytes) || overlaps(p->d_fused, fused_bytes, p->d_k, kv_bytes) ||
+      overlaps(p->d_fused, fused_bytes, p->d_v, kv_bytes))
+    return MI355_W8A8_ERR_ALIAS;
+  const uint32_t parts = qkv_bwd_parts(p->m);
+  if (wgrad) {
+    const uint64_t need = qkv_bwd_workspace_bytes(p->m, p->head_dim);
+    if (!p->workspace) return MI355_W8A8_ERR_NULL;
+    if (p->workspace_bytes < need) return MI355_W8A8_ERR_WORKSPACE;
+    if (!aligned16(p->workspace) || (reinterpret_cast<uintptr_t>(p->d_q_norm_weight) & 3u) ||
+        (reinterpret_cast<uintptr_t>(p->d_k_norm_weight) & 3u))
+      return MI355_W8A8_ERR_ALIGN;
+    if (overlaps(p->workspace, need, p->d_fused, fused_bytes) || overlaps(p->workspace, need, p->fused, fused_bytes) ||
+        overlaps(p->d_q_norm_weight, p->head_dim * 4ull, p->d_k_norm_weight, p->head_dim * 4ull))
+      return MI355_W8A8_ERR_ALIAS;
+  }
+  QkvPostBwdArgs a{};
+  a.fused = static_cast<const uint16_t*>(p->fused);
+  a.q_w = p->q_norm_weight; a.k_w = p->k_norm_weight; a.pos = p->positions;
+  a.dq = static_cast<const uint16_t*>(p->d_q); a.dk = static_cast<const uint16_t*>(p->d_k);
+  a.dv = static_cast<const uint16_t*>(p->d_v); a.dgate = static_cast<const uint16_t*>(p->d_gate);
+  a.dfused = static_cast<uint16_t*>(p->d_fused);
+  a.partial = wgrad ? static_cast<float*>(p->workspace) : nullptr;
+  a.M = p->m; a.Hq = p->num_query_heads; a.Hkv = p->num_kv_heads; a.D = p->head_dim; a.rot = p->rotary_dim;
+  a.width = (uint32_t)width; a.theta = p->rope_theta; a.eps = p->rms_eps;
+  const bool vec4 = (p->head_dim & 3u) == 0;
+  (void)hipGetLastError();
+  if (wgrad) {
+    if (vec4) hipLaunchKernelGGL((qkv_post_bwd_kernel<4, true>), dim3(parts), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((qkv_post_bwd_kernel<1, true>), dim3(parts), dim3(256), 0, s, a);
+    int st;
+    if ((st = launch_status())) return st;
+    ColumnSumArgs c{};
+    c.partial = a.partial; c.n_parts = parts; c.stride = 2u * p->head_dim; c.cols = p->head_dim;
+    c.out = p->d_q_norm_weight; c.col0 = 0;
+    hipLaunchKernelGGL(column_sum_kernel, dim3((p->head_dim + 255u) / 256u), dim3(256), 0, s, c);
+    c.out = p->d_k_norm_weight; c.col0 = p->head_dim;
+    hipLaunchKernelGGL(column_sum_kernel, dim3((p->head_dim + 255u) / 256u), dim3(256), 0, s, c);
+  } else {
+    if (vec4) hipLaunchKernelGGL((qkv_post_bwd_kernel<4, false>), dim3(p->m), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((qkv_post_bwd_kernel<1, false>), dim3(p->m), dim3(256), 0, s, a);
+  }
+  return launch_status();
+}
+
+// Row slices of the decoder-norm weight cotangent: each leaves one partial row.
+inline uint32_t rms_dgamma_slices(uint32_t m) { return m < 256u ? m : 256u; }
+inline uint64_t delta_rms_bwd_workspace_bytes(uint32_t m, uint32_t k) {
+  return (uint64_t)round_up(m, 64u) * 4u + (uint64_t)rms_dgamma_slices(m) * k * 4u;
+}
+
+int run_delta_rms_norm_bwd(const void* x, const float* gamma, const void* d_normalized, void* d_x, float* d_gamma,
+                           void* workspace, uint64_t workspace_bytes, uint32_t m, uint32_t k, float eps,
+                           hipStream_t s) {
+  if (!x || !gamma || !d_normalized || !d_x) return MI355_W8A8_ERR_NULL;
+  if (m == 0 || k == 0 || !(eps > 0.0f)) return MI355_W8A8_ERR_SHAPE;
+  if (m > kMaxRows) return MI355_W8A8_ERR_UNSUPPORTED;
+  if (!aligned16(x) || !aligned16(d_normalized) || !aligned16(d_x) || !aligned16(gamma)) return MI355_W8A8_ERR_ALIGN;
+  const uint64_t bytes = (uint64_t)m * k * 2u;
+  if (overlaps(d_x, bytes, x, bytes) || overlaps(d_x, bytes, gamma, (uint64_t)k * 4u)) return MI355_W8A8_ERR_ALIAS;
+  const uint64_t need = delta_rms_bwd_workspace_bytes(m, k);
+  if (d_gamma) {
+    // the weight cotangent reads d_normalized after the row pull-back has written d_x
+    if (overlaps(d_x, bytes, d_normalized, bytes)) return MI355_W8A8_ERR_ALIAS;
+    if (!workspace) return MI355_W8A8_ERR_NULL;
+    if (workspace_bytes < need) return MI355_W8A8_ERR_WORKSPACE;
+    if (!aligned16(workspace) || (reinterpret_cast<uintptr_t>(d_gamma) & 3u)) return MI355_W8A8_ERR_ALIGN;
+    if (overlaps(workspace, need, d_x, bytes) || overlaps(workspace, need, x, bytes) ||
+        overlaps(workspace, need, d_normalized, bytes) || overlaps(d_gamma, (uint64_t)k * 4u, d_x, bytes))
+      return MI355_W8A8_ERR_ALIAS;
+  } else if (d_x != d_normalized && overlaps(d_x, bytes, d_normalized, bytes)) {
+    return MI355_W8A8_ERR_ALIAS;
+  }
+  DeltaRmsBwdArgs a{};
+  a.x = static_cast<const uint16_t*>(x);
+  a.gamma = gamma;
+  a.dn = static_cast<const uint16_t*>(d_normalized);
+  a.dx = static_cast<uint16_t*>(d_x);
+  a.inv_out = d_gamma ? static_cast<float*>(workspace) : nullptr;
+  a.M = m; a.K = k; a.eps = eps;
+  (void)hipGetLastError();
+  if ((k & 7u) == 0) hipLaunchKernelGGL((delta_rms_norm_bwd_kernel<true>), dim3(m), dim3(256), 0, s, a);
+  else hipLaunchKernelGGL((delta_rms_norm_bwd_kernel<false>), dim3(m), dim3(256), 0, s, a);
+  int st;
+  if ((st = launch_status())) return st;
+  if (d_gamma) {
+    const uint32_t slices = rms_dgamma_slices(m);
+    RmsDgammaArgs g{};
+    g.x = a.x; g.dn = a.dn; g.inv = a.inv_out;
+    g.partial = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + (uint64_t)round_up(m, 64u) * 4u);
+    g.M = m; g.K = k;
+    hipLaunchKernelGGL(rms_dgamma_partial_kernel, dim3((k + 255u) / 256u, slices), dim3(256), 0, s, g);
+    if ((st = launch_status())) return st;
+    ColumnSumArgs c{};
+    c.partial = g.partial; c.n_parts = slices; c.stride = k; c.cols = k; c.col0 = 0; c.out = d_gamma;
+    hipLaunchKernelGGL(column_sum_kernel, dim3((k + 255u) / 256u), dim3(256), 0, s, c);
+    return launch_status();
+  }
+  return MI355_W8A8_OK;
+}
+
 int run_swiglu_bwd(const void* fused, const void* d_product, void* d_fused, uint32_t m, uint32_t n, hipStream_t s) {
   if (!fused || !d_product || !d_fused) return MI355_W8A8_ERR_NULL;
   if (m == 0 || n == 0 || (n & 7u)) return MI355_W8A8_ERR_SHAPE;
@@ -1353,6 +1483,23 @@ int mi355_w8a8_lora_linear_bwd_v1(const mi355_w8a8_bwd_problem* p, void* stream)
 
 int mi355_w8a8_qkv_split_norm_rope_v1(const mi355_w8a8_qkv_post_problem* p, void* stream) {
   return run_qkv_post(p, static_cast<hipStream_t>(stream));
+}
+
+uint64_t mi355_w8a8_qkv_bwd_workspace_bytes(uint32_t m, uint32_t head_dim) { return qkv_bwd_workspace_bytes(m, head_dim); }
+
+int mi355_w8a8_qkv_split_norm_rope_bwd_v1(const mi355_w8a8_qkv_post_bwd_problem* p, void* stream) {
+  return run_qkv_post_bwd(p, static_cast<hipStream_t>(stream));
+}
+
+uint64_t mi355_w8a8_delta_rms_norm_bwd_workspace_bytes(uint32_t m, uint32_t k) {
+  return delta_rms_bwd_workspace_bytes(m, k);
+}
+
+int mi355_w8a8_delta_rms_norm_bwd_v1(const void* x, const float* gamma, const void* d_normalized, void* d_x,
+                                     float* d_gamma, void* workspace, uint64_t workspace_bytes, uint32_t m,
+                                     uint32_t k, float eps, void* stream) {
+  return run_delta_rms_norm_bwd(x, gamma, d_normalized, d_x, d_gamma, workspace, workspace_bytes, m, k, eps,
+                                static_cast<hipStream_t>(stream));
 }
 
 int mi355_w8a8_swiglu_v1(const void* fused, void* product, uint32_t m, uint32_t n, void* stream) {

@@ -169,4 +169,115 @@ __global__ __launch_bounds__(256) void rms_norm_bwd_kernel(RmsNormBwdArgs a) {
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// The RMSNorm pull-back in the form of the Qwen3.5 attention input stage
+// (_delta_rms_norm_vjp, skyrl/tx/kernels/qwen3_5_qkv_lora.py:97-116), float32:
+//   n = x inv,  p = dn gamma,  mu = mean(p n),  dx = bf16(inv (p - n mu)),  dgamma = sum_rows dn n
+// One workgroup per row, three passes over the row (the later ones from L2).  When inv_out is set
+// the row's inv is stored for the weight-cotangent kernel below.
+struct DeltaRmsBwdArgs {
+  const uint16_t* x;    // bf16 [M, K]
+  const float* gamma;   // f32 [K]: the multiplier 1 + weight
+  const uint16_t* dn;   // bf16 [M, K]
+  uint16_t* dx;         // bf16 [M, K]; may be the same buffer as dn
+  float* inv_out;       // f32 [M] or null
+  uint32_t M, K;
+  float eps;
+};
+
+template <bool VEC>
+__global__ __launch_bounds__(256) void delta_rms_norm_bwd_kernel(DeltaRmsBwdArgs a) {
+  __shared__ double slots[4];
+  const uint32_t row = blockIdx.x, tid = threadIdx.x;
+  if (row >= a.M) return;
+  const uint16_t* xr = a.x + (size_t)row * a.K;
+  const uint16_t* dr = a.dn + (size_t)row * a.K;
+  uint16_t* outr = a.dx + (size_t)row * a.K;
+  constexpr uint32_t W = VEC ? 8u : 1u;
+  double ss = 0.0;
+  for (uint32_t i = W * tid; i < a.K; i += W * 256u) {
+    if (VEC) {
+      const uint4 xv = *reinterpret_cast<const uint4*>(xr + i);
+      const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float x = (e & 1) ? __uint_as_float(xw[e >> 1] & 0xffff0000u) : __uint_as_float(xw[e >> 1] << 16);
+        ss += (double)x * (double)x;
+      }
+    } else {
+      const float x = bf16_bits_to_f32(xr[i]);
+      ss += (double)x * (double)x;
+    }
+  }
+  ss = block_sum_256(ss, slots);
+  const float mean = (float)(ss / (double)a.K);
+  const float inv = 1.0f / sqrtf(mean + a.eps);
+  if (a.inv_out && tid == 0) a.inv_out[row] = inv;
+  double sp = 0.0;
+  for (uint32_t i = W * tid; i < a.K; i += W * 256u) {
+    if (VEC) {
+      const uint4 xv = *reinterpret_cast<const uint4*>(xr + i);
+      const uint4 dv = *reinterpret_cast<const uint4*>(dr + i);
+      const float4 g0 = *reinterpret_cast<const float4*>(a.gamma + i);
+      const float4 g1 = *reinterpret_cast<const float4*>(a.gamma + i + 4u);
+      const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w}, dw[4] = {dv.x, dv.y, dv.z, dv.w};
+      const float gv[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float x = (e & 1) ? __uint_as_float(xw[e >> 1] & 0xffff0000u) : __uint_as_float(xw[e >> 1] << 16);
+        const float d = (e & 1) ? __uint_as_float(dw[e >> 1] & 0xffff0000u) : __uint_as_float(dw[e >> 1] << 16);
+        sp += (double)((d * gv[e]) * (x * inv));
+      }
+    } else {
+      const float x = bf16_bits_to_f32(xr[i]);
+      sp += (double)((bf16_bits_to_f32(dr[i]) * a.gamma[i]) * (x * inv));
+    }
+  }
+  sp = block_sum_256(sp, slots);
+  const float mu = (float)(sp / (double)a.K);
+  for (uint32_t i = W * tid; i < a.K; i += W * 256u) {
+    if (VEC) {
+      const uint4 xv = *reinterpret_cast<const uint4*>(xr + i);
+      const uint4 dv = *reinterpret_cast<const uint4*>(dr + i);
+      const float4 g0 = *reinterpret_cast<const float4*>(a.gamma + i);
+      const float4 g1 = *reinterpret_cast<const float4*>(a.gamma + i + 4u);
+      const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w}, dw[4] = {dv.x, dv.y, dv.z, dv.w};
+      const float gv[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+      float o[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float x = (e & 1) ? __uint_as_float(xw[e >> 1] & 0xffff0000u) : __uint_as_float(xw[e >> 1] << 16);
+        const float d = (e & 1) ? __uint_as_float(dw[e >> 1] & 0xffff0000u) : __uint_as_float(dw[e >> 1] << 16);
+        o[e] = inv * ((d * gv[e]) - (x * inv) * mu);
+      }
+      *reinterpret_cast<uint4*>(outr + i) = make_uint4(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]),
+                                                       pack_bf16x2(o[4], o[5]), pack_bf16x2(o[6], o[7]));
+    } else {
+      const float x = bf16_bits_to_f32(xr[i]);
+      const float p = bf16_bits_to_f32(dr[i]) * a.gamma[i];
+      outr[i] = (uint16_t)f32_to_bf16_bits(inv * (p - (x * inv) * mu));
+    }
+  }
+}
+
+// partial[slice][c] = sum over the rows r = slice, slice + n_slices, ... of dn[r, c] * (x[r, c] * inv[r]);
+// one thread per column, gridDim = (ceil(K / 256), n_slices).  dn is the cotangent the pull-back
+// above received: this kernel runs before a pull-back that overwrites it.
+struct RmsDgammaArgs {
+  const uint16_t* x;    // bf16 [M, K]
+  const uint16_t* dn;   // bf16 [M, K]
+  const float* inv;     // f32 [M]
+  float* partial;       // f32 [n_slices][K]
+  uint32_t M, K;
+};
+
+__global__ __launch_bounds__(256) void rms_dgamma_partial_kernel(RmsDgammaArgs a) {
+  const uint32_t c = blockIdx.x * 256u + threadIdx.x;
+  if (c >= a.K) return;
+  float s = 0.0f;
+  for (uint32_t r = blockIdx.y; r < a.M; r += gridDim.y)
+    s += bf16_bits_to_f32(a.dn[(size_t)r * a.K + c]) * (bf16_bits_to_f32(a.x[(size_t)r * a.K + c]) * a.inv[r]);
+  a.partial[(size_t)blockIdx.y * a.K + c] = s;
+}
+
 }  // namespace w8a8

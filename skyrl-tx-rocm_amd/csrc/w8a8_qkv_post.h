@@ -157,4 +157,183 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostArgs a) {
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Pull-back of the kernel above (qwen3_5_qkv_lora.py:391-425): the transposed partial rotation on
+// the Q and K cotangents, the RMSNorm pull-back of every Q and K head against the raw projection,
+// and the re-interleave with the gate and V cotangents into the cotangent of the fused projection.
+// Optionally the cotangents of the two head-norm weights (sums over rows and heads).
+//
+// Per head, float32 in the order of _apply_partial_rope_transpose (:148-164) and
+// _delta_rms_norm_vjp (:97-116):
+//   u  = bf16([first cos + second sin, second cos - first sin]) on the rotated part of dy
+//   n  = x inv,  p = u (1 + w),  mu = mean(p n),  dx = bf16(inv (p - n mu)),  dw += u n
+struct QkvPostBwdArgs {
+  const uint16_t* fused;   // bf16 [M, width] raw projection
+  const float* q_w;        // f32 [D]
+  const float* k_w;        // f32 [D]
+  const int32_t* pos;      // int32 [M]
+  const uint16_t* dq;      // bf16 [M, Hq, D]
+  const uint16_t* dk;      // bf16 [M, Hkv, D]
+  const uint16_t* dv;      // bf16 [M, Hkv, D]
+  const uint16_t* dgate;   // bf16 [M, Hq * D]
+  uint16_t* dfused;        // bf16 [M, width]
+  float* partial;          // f32 [gridDim.x][2][D] when the weight cotangents are wanted
+  uint32_t M, Hq, Hkv, D, rot, width;
+  float theta, eps;
+};
+
+// V consecutive elements per lane and piece (V = 4: 8-byte accesses; V = 1: any geometry); a head
+// has at most kQkvMaxHeadDim / (64 V) pieces per lane.  Workgroups stride over the rows so that the
+// weight cotangents accumulate in registers; WGRAD = false leaves them out altogether.
+template <int V, bool WGRAD>
+__global__ __launch_bounds__(256) void qkv_post_bwd_kernel(QkvPostBwdArgs a) {
+  constexpr uint32_t NP = kQkvMaxHeadDim / (64u * V);
+  __shared__ float sn[kQkvMaxHeadDim / 2], cs[kQkvMaxHeadDim / 2];
+  __shared__ float buf[4][kQkvMaxHeadDim];
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t half = a.rot / 2u;
+  const uint32_t qpk = a.Hq / a.Hkv;
+  const uint32_t group_width = (qpk * 2u + 2u) * a.D;
+  const uint32_t units = a.Hq + a.Hkv;
+  float wq[NP * V], wk[NP * V];
+#pragma unroll
+  for (uint32_t e = 0; e < NP * V; ++e) wq[e] = wk[e] = 0.0f;
+
+  for (uint32_t row = blockIdx.x; row < a.M; row += gridDim.x) {
+    __syncthreads();  // the tables of the previous row are no longer read
+    const float position = (float)a.pos[row];
+    for (uint32_t i = tid; i < half; i += 256u) {
+      const float fraction = (2.0f * (float)i) / (float)a.rot;
+      const float angle = position / powf(a.theta, fraction);
+      sn[i] = sinf(angle);
+      cs[i] = cosf(angle);
+    }
+    __syncthreads();
+    const uint16_t* frow = a.fused + (size_t)row * a.width;
+    uint16_t* orow = a.dfused + (size_t)row * a.width;
+    for (uint32_t u = wave; u < units; u += 4u) {  // wave-uniform
+      const bool is_q = u < a.Hq;
+      const uint32_t g = is_q ? u / qpk : u - a.Hq;
+      const uint32_t off = g * group_width + (is_q ? (u % qpk) * 2u * a.D : qpk * 2u * a.D);
+      const float* w = is_q ? a.q_w : a.k_w;
+      const uint16_t* dy = is_q ? a.dq + ((size_t)row * a.Hq + u) * a.D : a.dk + ((size_t)row * a.Hkv + g) * a.D;
+      const uint16_t* dcopy = is_q ? a.dgate + ((size_t)row * a.Hq + u) * a.D : a.dv + ((size_t)row * a.Hkv + g) * a.D;
+      float x[NP * V], d[NP * V];
+      double ss = 0.0;
+#pragma unroll
+      for (uint32_t j = 0; j < NP; ++j) {
+        const uint32_t i = V * lane + 64u * V * j;
+        if (i < a.D) {
+          if (V == 4) {
+            *reinterpret_cast<uint2*>(orow + off + a.D + i) = *reinterpret_cast<const uint2*>(dcopy + i);
+            const uint2 xr = *reinterpret_cast<const uint2*>(frow + off + i);
+            const uint2 dr = *reinterpret_cast<const uint2*>(dy + i);
+            x[4 * j + 0] = __uint_as_float(xr.x << 16); x[4 * j + 1] = __uint_as_float(xr.x & 0xffff0000u);
+            x[4 * j + 2] = __uint_as_float(xr.y << 16); x[4 * j + 3] = __uint_as_float(xr.y & 0xffff0000u);
+            d[4 * j + 0] = __uint_as_float(dr.x << 16); d[4 * j + 1] = __uint_as_float(dr.x & 0xffff0000u);
+            d[4 * j + 2] = __uint_as_float(dr.y << 16); d[4 * j + 3] = __uint_as_float(dr.y & 0xffff0000u);
+          } else {
+            orow[off + a.D + i] = dcopy[i];
+            x[j] = bf16_bits_to_f32(frow[off + i]);
+            d[j] = bf16_bits_to_f32(dy[i]);
+          }
+#pragma unroll
+          for (int e = 0; e < V; ++e) {
+            ss += (double)x[V * j + e] * (double)x[V * j + e];
+            buf[wave][i + e] = d[V * j + e];
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < V; ++e) x[V * j + e] = d[V * j + e] = 0.0f;
+        }
+      }
+      ss = wave_sum(ss);
+      const float mean = (float)(ss / (double)a.D);
+      const float inv = 1.0f / sqrtf(mean + a.eps);
+      // the rotation pairs element i with i +- rot / 2, held by another lane of this wave
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+      __builtin_amdgcn_wave_barrier();
+      float n[NP * V], p[NP * V];
+      double sp = 0.0;
+#pragma unroll
+      for (uint32_t j = 0; j < NP; ++j) {
+        const uint32_t i = V * lane + 64u * V * j;
+        if (i < a.D) {
+#pragma unroll
+          for (int e = 0; e < V; ++e) {
+            const uint32_t c = i + e;
+            float uo = d[V * j + e];
+            if (c < a.rot) {
+              if (c < half) uo = uo * cs[c] + buf[wave][c + half] * sn[c];
+              else uo = uo * cs[c - half] - buf[wave][c - half] * sn[c - half];
+              uo = bf16_round_f32(uo);
+            }
+            d[V * j + e] = uo;
+            n[V * j + e] = x[V * j + e] * inv;
+            p[V * j + e] = uo * (1.0f + w[c]);
+            sp += (double)(p[V * j + e] * n[V * j + e]);
+          }
+        }
+      }
+      sp = wave_sum(sp);
+      const float mu = (float)(sp / (double)a.D);
+#pragma unroll
+      for (uint32_t j = 0; j < NP; ++j) {
+        const uint32_t i = V * lane + 64u * V * j;
+        if (i < a.D) {
+          float o[V];
+#pragma unroll
+          for (int e = 0; e < V; ++e) {
+            o[e] = inv * (p[V * j + e] - n[V * j + e] * mu);
+            if (WGRAD) {
+              const float t = d[V * j + e] * n[V * j + e];
+              wq[V * j + e] += is_q ? t : 0.0f;
+              wk[V * j + e] += is_q ? 0.0f : t;
+            }
+          }
+          if (V == 4) {
+            *reinterpret_cast<uint2*>(orow + off + i) = make_uint2(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]));
+          } else {
+            orow[off + i] = (uint16_t)f32_to_bf16_bits(o[0]);
+          }
+        }
+      }
+      __builtin_amdgcn_s_waitcnt(0xc07f);
+      __builtin_amdgcn_wave_barrier();  // buf[wave] is rewritten by the next unit
+    }
+  }
+  if (WGRAD) {
+    // the four waves' sums, wave 0 first; buf is free once every wave is past its rows
+    for (uint32_t which = 0; which < 2; ++which) {
+      __syncthreads();
+#pragma unroll
+      for (uint32_t j = 0; j < NP; ++j) {
+        const uint32_t i = V * lane + 64u * V * j;
+        if (i < a.D) {
+#pragma unroll
+          for (int e = 0; e < V; ++e) buf[wave][i + e] = which == 0 ? wq[V * j + e] : wk[V * j + e];
+        }
+      }
+      __syncthreads();
+      for (uint32_t i = tid; i < a.D; i += 256u)
+        a.partial[((size_t)blockIdx.x * 2u + which) * a.D + i] = ((buf[0][i] + buf[1][i]) + buf[2][i]) + buf[3][i];
+    }
+  }
+}
+
+// out[c] = sum over the first n_parts rows of partial[part][c], in order; one thread per column.
+struct ColumnSumArgs {
+  const float* partial;  // f32 [n_parts][stride]
+  float* out;            // f32 [cols]
+  uint32_t n_parts, stride, cols, col0;
+};
+
+__global__ __launch_bounds__(256) void column_sum_kernel(ColumnSumArgs a) {
+  const uint32_t c = blockIdx.x * 256u + threadIdx.x;
+  if (c >= a.cols) return;
+  float s = 0.0f;
+  for (uint32_t p = 0; p < a.n_parts; ++p) s += a.partial[(size_t)p * a.stride + a.col0 + c];
+  a.out[c] = s;
+}
+
 }  // namespace w8a8

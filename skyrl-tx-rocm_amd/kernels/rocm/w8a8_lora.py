@@ -1228,17 +1228,190 @@ def qkv_split_norm_rope(fused: torch.Tensor, q_norm_weight: torch.Tensor, k_norm
     return QkvPostPlan(fused, q_norm_weight, k_norm_weight, positions, config).run()
 
 
+def qkv_split_norm_rope_backward(fused: torch.Tensor, q_norm_weight: torch.Tensor, k_norm_weight: torch.Tensor,
+                                 positions: torch.Tensor, config: Qwen35QKVStageConfig, d_q, d_k, d_v, d_gate, *,
+                                 need_norm_weight_grads: bool = False):
+    """Pull-back of ``qkv_split_norm_rope`` (qwen3_5_qkv_lora.py:391-425): ``fused`` is the raw bf16
+    projection the forward consumed; a missing output cotangent (None) counts as zero.  Returns
+    ``(d_fused, d_q_norm_weight, d_k_norm_weight)``, the last two float32 [head_dim] or None."""
+    if fused.dtype != torch.bfloat16:
+        raise TypeError(f"fused must be BF16, got {fused.dtype}")
+    _require_cuda(fused, "fused")
+    if fused.shape[-1] != config.fused_width:
+        raise ValueError(f"fused width {fused.shape[-1]} does not match the configuration ({config.fused_width})")
+    lead = tuple(fused.shape[:-1])
+    if tuple(positions.shape) != lead:
+        raise ValueError(f"positions must have shape {lead}, got {tuple(positions.shape)}")
+    d, hq, hkv = config.head_dim, config.num_query_heads, config.num_kv_heads
+    if tuple(q_norm_weight.shape) != (d,) or tuple(k_norm_weight.shape) != (d,):
+        raise ValueError(f"q_norm_weight and k_norm_weight must have shape ({d},)")
+    dev = fused.device
+    flat = fused.reshape(-1, config.fused_width).contiguous()
+    m = flat.shape[0]
+
+    def cot(t, width, name):
+        if t is None:
+            return torch.zeros((m, width), dtype=torch.bfloat16, device=dev)
+        if t.dtype != torch.bfloat16:
+            raise TypeError(f"{name} must be BF16, got {t.dtype}")
+        if t.numel() != m * width:
+            raise ValueError(f"{name} must hold {m} x {width} elements, got {tuple(t.shape)}")
+        return t.reshape(m, width).contiguous()
+
+    dq, dk = cot(d_q, hq * d, "d_q"), cot(d_k, hkv * d, "d_k")
+    dv, dg = cot(d_v, hkv * d, "d_v"), cot(d_gate, hq * d, "d_gate")
+    qw = q_norm_weight.to(device=dev, dtype=torch.float32).contiguous()
+    kw = k_norm_weight.to(device=dev, dtype=torch.float32).contiguous()
+    pos = positions.reshape(-1).to(device=dev, dtype=torch.int32).contiguous()
+    d_fused = torch.empty_like(flat)
+    lib = _native.load()
+    p = _native.QkvPostBwdProblem()
+    p.struct_size = ctypes.sizeof(_native.QkvPostBwdProblem)
+    p.m, p.num_query_heads, p.num_kv_heads, p.head_dim, p.rotary_dim = m, hq, hkv, d, config.rotary_dim
+    p.rope_theta, p.rms_eps = float(config.rope_theta), float(config.rms_norm_eps)
+    p.fused, p.q_norm_weight, p.k_norm_weight, p.positions = flat.data_ptr(), qw.data_ptr(), kw.data_ptr(), pos.data_ptr()
+    p.d_q, p.d_k, p.d_v, p.d_gate, p.d_fused = dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dg.data_ptr(), d_fused.data_ptr()
+    dqw = dkw = ws = None
+    if need_norm_weight_grads:
+        dqw = torch.empty(d, dtype=torch.float32, device=dev)
+        dkw = torch.empty(d, dtype=torch.float32, device=dev)
+        ws = torch.empty(int(lib.mi355_w8a8_qkv_bwd_workspace_bytes(m, d)), dtype=torch.uint8, device=dev)
+        p.d_q_norm_weight, p.d_k_norm_weight = dqw.data_ptr(), dkw.data_ptr()
+        p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
+    with torch.cuda.device(dev):
+        status = lib.mi355_w8a8_qkv_split_norm_rope_bwd_v1(ctypes.byref(p), _stream_ptr(dev))
+    _native.check("mi355_w8a8_qkv_split_norm_rope_bwd_v1", status)
+    return d_fused.reshape(fused.shape), dqw, dkw
+
+
+def delta_rms_norm_backward(x: torch.Tensor, gamma: torch.Tensor, d_normalized: torch.Tensor, *, eps: float = 1e-6,
+                            need_weight_grad: bool = False, in_place: bool = False):
+    """Pull-back of ``bf16(x * rsqrt(mean(x^2) + eps) * gamma)`` in the form of ``_delta_rms_norm_vjp``
+    (qwen3_5_qkv_lora.py:97-116); ``gamma`` float32 [K] is the multiplier ``1 + weight``.  Returns
+    ``(d_x, d_weight)``; ``d_weight`` float32 [K] (None unless asked for) is the cotangent of the
+    weight.  ``in_place`` overwrites ``d_normalized`` and excludes ``need_weight_grad``."""
+    if x.dtype != torch.bfloat16 or d_normalized.dtype != torch.bfloat16:
+        raise TypeError("x and d_normalized must be BF16")
+    _require_cuda(x, "x")
+    _require_cuda(d_normalized, "d_normalized")
+    k = x.shape[-1]
+    if x.ndim < 2 or tuple(d_normalized.shape) != tuple(x.shape) or tuple(gamma.shape) != (k,):
+        raise ValueError(f"need x and d_normalized [..., K] and gamma [K], got {tuple(x.shape)}, "
+                         f"{tuple(d_normalized.shape)} and {tuple(gamma.shape)}")
+    if not isinstance(eps, float) or not eps > 0.0:
+        raise ValueError(f"eps must be a positive float, got {eps!r}")
+    if in_place and need_weight_grad:
+        raise ValueError("the weight cotangent reads d_normalized after d_x is written: not in place")
+    if in_place and not d_normalized.is_contiguous():
+        raise ValueError("in_place needs a contiguous d_normalized tensor")
+    x2 = x.reshape(-1, k).contiguous()
+    d2 = d_normalized.reshape(-1, k).contiguous()
+    g = gamma.to(device=x.device, dtype=torch.float32).contiguous()
+    out = d2 if in_place else torch.empty_like(d2)
+    lib = _native.load()
+    dw = ws = None
+    dw_ptr = ws_ptr = ws_bytes = 0
+    if need_weight_grad:
+        dw = torch.empty(k, dtype=torch.float32, device=x.device)
+        ws = torch.empty(int(lib.mi355_w8a8_delta_rms_norm_bwd_workspace_bytes(x2.shape[0], k)), dtype=torch.uint8,
+                         device=x.device)
+        dw_ptr, ws_ptr, ws_bytes = dw.data_ptr(), ws.data_ptr(), ws.numel()
+    with torch.cuda.device(x.device):
+        status = lib.mi355_w8a8_delta_rms_norm_bwd_v1(x2.data_ptr(), g.data_ptr(), d2.data_ptr(), out.data_ptr(), dw_ptr,
+                                                      ws_ptr, ws_bytes, x2.shape[0], k, eps, _stream_ptr(x.device))
+    _native.check("mi355_w8a8_delta_rms_norm_bwd_v1", status)
+    return out.reshape(x.shape), dw
+
+
+class _QkvStageFunction(torch.autograd.Function):
+    """The stage with the derivative rule of ``_qwen35_qkv_lora_rope`` (qwen3_5_qkv_lora.py:288-454):
+    cotangents for the hidden rows, the three norm weights, A, B and the scaling; none for the frozen
+    kernel and the positions.  The forward keeps the bf16 projection and the normalized rows
+    (``save_projection``) or nothing beyond its inputs, in which case the backward recomputes both
+    with one forward call, as the reference's rule does (:378-388)."""
+
+    @staticmethod
+    def forward(ctx, hidden, input_norm_weight, q_norm_weight, k_norm_weight, lora_a, lora_b, lora_scaling, weight,
+                positions, config, adapter_indices, save_projection):
+        ctx.weight, ctx.config, ctx.adapter_indices = weight, config, adapter_indices
+        ctx.saved_projection = bool(save_projection)
+        gamma = 1.0 + input_norm_weight.detach().to(torch.float32)
+        plan = ForwardPlan(hidden, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices,
+                           rms_gamma=gamma, eps=config.rms_norm_eps, want_normalized=ctx.saved_projection)
+        fused = plan.run()
+        keep = (fused, plan.aux["normalized"]) if ctx.saved_projection else ()
+        ctx.save_for_backward(hidden, input_norm_weight, q_norm_weight, k_norm_weight, lora_a, lora_b, lora_scaling,
+                              positions, *keep)
+        q, k, v, gate = qkv_split_norm_rope(fused, q_norm_weight, k_norm_weight, positions, config)
+        return q, k, v, gate
+
+    @staticmethod
+    def backward(ctx, d_q, d_k, d_v, d_gate):
+        hidden, in_w, q_w, k_w, lora_a, lora_b, lora_scaling, positions = ctx.saved_tensors[:8]
+        config = ctx.config
+        gamma = 1.0 + in_w.detach().to(torch.float32)
+        if ctx.saved_projection:
+            fused, normalized = ctx.saved_tensors[8:]
+        else:
+            plan = ForwardPlan(hidden, ctx.weight, lora_a, lora_b, lora_scaling, adapter_indices=ctx.adapter_indices,
+                               rms_gamma=gamma, eps=config.rms_norm_eps, want_normalized=True)
+            fused = plan.run()
+            normalized = plan.aux["normalized"]
+        need_lora = lora_a is not None and any(ctx.needs_input_grad[4:7])
+        need_head = ctx.needs_input_grad[2] or ctx.needs_input_grad[3]
+        need_in = ctx.needs_input_grad[1]
+        d_fused, dqw, dkw = qkv_split_norm_rope_backward(fused, q_w, k_w, positions, config, d_q, d_k, d_v, d_gate,
+                                                         need_norm_weight_grads=need_head)
+        rows = normalized.shape[0]
+        idx = ctx.adapter_indices
+        if idx is not None and idx.numel() != rows:
+            idx = idx.reshape(-1).repeat_interleave(rows // idx.numel())
+        dn, da, db, ds = backward(normalized, d_fused.reshape(rows, -1), ctx.weight, lora_a, lora_b, lora_scaling,
+                                  adapter_indices=idx, need_lora_grads=need_lora)
+        dh, dinw = delta_rms_norm_backward(hidden.reshape(rows, -1), gamma, dn, eps=config.rms_norm_eps,
+                                           need_weight_grad=need_in, in_place=not need_in)
+        if need_lora:
+            if lora_a.ndim == 2:
+                da, db = da[0], db[0]
+            ds = ds.reshape(lora_scaling.shape).to(lora_scaling.dtype)
+        else:
+            da = db = ds = None
+        dinw = dinw.to(in_w.dtype) if need_in else None
+        dqw = dqw.to(q_w.dtype) if ctx.needs_input_grad[2] else None
+        dkw = dkw.to(k_w.dtype) if ctx.needs_input_grad[3] else None
+        return dh.reshape(hidden.shape), dinw, dqw, dkw, da, db, ds, None, None, None, None, None
+
+
+def qkv_lora_rope(hidden, input_norm_weight, q_norm_weight, k_norm_weight, weight, lora_a, lora_b, lora_scaling,
+                  positions, *, config: Qwen35QKVStageConfig, adapter_indices=None, save_projection: bool = True):
+    """The attention input stage that autograd can differentiate in the hidden rows, the norm weights
+    and the LoRA parameters.  ``save_projection`` keeps 2 * M * (fused width + K) bytes until the
+    backward instead of recomputing the projection there."""
+    tensors = [t for t in (hidden, input_norm_weight, q_norm_weight, k_norm_weight, lora_a, lora_b, lora_scaling)
+               if isinstance(t, torch.Tensor)]
+    if not (torch.is_grad_enabled() and any(t.requires_grad for t in tensors)):
+        gamma = 1.0 + input_norm_weight.to(torch.float32)
+        fused = forward(hidden, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices,
+                        rms_gamma=gamma, eps=config.rms_norm_eps)
+        return qkv_split_norm_rope(fused, q_norm_weight, k_norm_weight, positions, config)
+    scaling = lora_scaling
+    if lora_a is not None and not isinstance(scaling, torch.Tensor):
+        scaling = torch.as_tensor(scaling, dtype=torch.float32, device=hidden.device)
+    return _QkvStageFunction.apply(hidden, input_norm_weight, q_norm_weight, k_norm_weight, lora_a, lora_b, scaling,
+                                   weight, positions, config, adapter_indices, save_projection)
+
+
 def w8a8_qkv_lora_rope(hidden, input_norm_weight, q_norm_weight, k_norm_weight, weight, lora_a, lora_b, lora_scaling,
                        positions, *, config: Qwen35QKVStageConfig, adapter_indices=None, enabled: bool = False,
-                       interpret: bool = False):
+                       interpret: bool = False, save_projection: bool = True):
     """``qwen35_qkv_lora_rope`` (qwen3_5_qkv_lora.py:532-…) with the W8A8 projection in the place of
     the bf16 one: decoder RMSNorm (delta weights) fused into the quantizer, W8A8 QKV + LoRA in one
-    float32 epilogue, then the split / Q-K norm / partial-RoPE kernel.  Forward only."""
+    float32 epilogue, then the split / Q-K norm / partial-RoPE kernel; under autograd with the
+    derivative rule of ``_qwen35_qkv_lora_rope_bwd`` (:360-451)."""
     _check_enabled(enabled, interpret, "QKV input stage")
-    gamma = 1.0 + input_norm_weight.to(torch.float32)
-    fused = forward(hidden, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices,
-                    rms_gamma=gamma, eps=config.rms_norm_eps)
-    return qkv_split_norm_rope(fused, q_norm_weight, k_norm_weight, positions, config)
+    return qkv_lora_rope(hidden, input_norm_weight, q_norm_weight, k_norm_weight, weight, lora_a, lora_b,
+                         lora_scaling, positions, config=config, adapter_indices=adapter_indices,
+                         save_projection=save_projection)
 
 
 __all__ = (
@@ -1249,5 +1422,5 @@ __all__ = (
     "w8a8_lora_linear", "w8a8_rms_gate_up_lora_swiglu", "w8a8_lora_residual", "PackedGroupedW8Weight",
     "prepare_grouped_weight", "grouped_forward", "grouped_backward", "grouped_lora_linear",
     "w8a8_grouped_lora_linear", "w8a8_moe_expert_mlp", "Qwen35QKVStageConfig", "QkvPostPlan", "qkv_split_norm_rope",
-    "w8a8_qkv_lora_rope",
+    "w8a8_qkv_lora_rope", "qkv_lora_rope", "qkv_split_norm_rope_backward", "delta_rms_norm_backward",
 )
