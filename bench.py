@@ -62,6 +62,11 @@ WORKLOADS = {
     "qwen3.5-4b-qkv-m2048": dict(m=2048, k=2560, n=10240, n_adapters=4, rank=64, alpha=128, rms=True,
                                  idx_mode="uniform", seed=5,
                                  qkv=dict(num_query_heads=16, num_kv_heads=4, head_dim=256, rotary_dim=64)),
+    # backward of that stage with frozen norm weights: split / norm / RoPE pull-back, linear backward with
+    # the LoRA cotangents, decoder-norm pull-back (projection and normalized rows kept by the forward)
+    "qwen3.5-4b-qkv-m2048-backward": dict(m=2048, k=2560, n=10240, n_adapters=4, rank=64, alpha=128, rms=True,
+                                          idx_mode="uniform", seed=5, qkv_backward=True,
+                                          qkv=dict(num_query_heads=16, num_kv_heads=4, head_dim=256, rotary_dim=64)),
 }
 
 # HBM bytes per launch of the dominant kernel(s) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
@@ -670,6 +675,125 @@ def bench_qkv(args, cfg, pkg, dev):
     return 0
 
 
+def bench_qkv_backward(args, cfg, pkg, dev):
+    """One step = one backward of the attention input stage whose forward kept the projection and the
+    normalized rows: split / Q-K norm / RoPE pull-back, linear backward (dx + LoRA cotangents), decoder
+    RMSNorm pull-back.  ``value`` counts the pull-back's 2*M*K*N; the roofline prices
+    qkv_post_bwd_kernel (HBM-bound: the projection and the four cotangents in, d_fused out)."""
+    import torch
+
+    import w8a8_cases as wc
+    from oracle import w8a8_oracle as o
+
+    native, w8 = pkg._native, pkg.w8a8_lora
+    geo = cfg["qkv"]
+    theta = 10_000_000.0
+    qcfg = w8.Qwen35QKVStageConfig(geo["num_query_heads"], geo["num_kv_heads"], geo["head_dim"], geo["rotary_dim"],
+                                   theta, 1e-6)
+    m, k, n = cfg["m"], cfg["k"], cfg["n"]
+    hq, hkv, d = geo["num_query_heads"], geo["num_kv_heads"], geo["head_dim"]
+    assert qcfg.fused_width == n
+    case = wc.make_case(m, k, n, n_adapters=cfg["n_adapters"], rank=cfg["rank"], alpha=cfg.get("alpha"),
+                        seed=cfg["seed"], rms=True, idx_mode=cfg["idx_mode"])
+    rng = np.random.default_rng(cfg["seed"] + 78)
+    qw, kw = (rng.standard_normal(d).astype(np.float32) * 0.1 for _ in range(2))
+    pos = rng.integers(0, 32768, m).astype(np.int32)
+    cots = [o.bf16_round(rng.standard_normal(shape).astype(np.float32))
+            for shape in ((m, hq, d), (m, hkv, d), (m, hkv, d), (m, hq * d))]
+    t = wc.to_torch(case, dev)
+    qw_t, kw_t, pos_t = (torch.from_numpy(v).to(dev) for v in (qw, kw, pos))
+    cots_t = [torch.from_numpy(c).to(dev).to(torch.bfloat16) for c in cots]
+    in_w = t["gamma"] - 1.0
+    fwd = w8.ForwardPlan(t["x"], t["weight"], t["a"], t["b"], t["s"], adapter_indices=t["idx"], rms_gamma=t["gamma"],
+                         eps=1e-6, want_normalized=True)
+    fused = fwd.run()
+    plan = w8.QkvStageBackwardPlan(t["x"], in_w, qw_t, kw_t, t["weight"], t["a"], t["b"], t["s"], pos_t, qcfg, *cots_t,
+                                   adapter_indices=t["idx"], fused=fused, normalized=fwd.aux["normalized"])
+    torch.cuda.synchronize()
+    for _ in range(args.warmup):
+        plan.run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        plan.run()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    got = [v.to(torch.float32).cpu().numpy() for v in plan.run()]
+    torch.cuda.synchronize()
+
+    def timed(fn):
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        for a, b in ev:
+            a.record()
+            fn()
+            b.record()
+        torch.cuda.synchronize()
+        return np.asarray([a.elapsed_time(b) for a, b in ev])
+
+    lib = native.load()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    k_ms = timed(plan.run_post_stage)
+    linear_ms = timed(plan.bwd.run)
+    scratch_k = torch.empty_like(plan.bwd.dx)
+    rms_ms = timed(lambda: native.check("delta_rms_norm_bwd", lib.mi355_w8a8_delta_rms_norm_bwd_v1(
+        plan.x.data_ptr(), plan.gamma.data_ptr(), plan.bwd.dx.data_ptr(), scratch_k.data_ptr(), None, None, 0, m, k,
+        plan.eps, stream)))
+    recompute_ms = timed(fwd.run)
+    # with trainable norm weights: the two pull-backs also form the weight cotangents
+    wgrad_post_ms = timed(lambda: w8.qkv_split_norm_rope_backward(fused, qw_t, kw_t, pos_t, qcfg, *cots_t,
+                                                                  need_norm_weight_grads=True))
+    dn_copy = plan.bwd.dx.clone()
+    wgrad_rms_ms = timed(lambda: w8.delta_rms_norm_backward(plan.x, plan.gamma, dn_copy, eps=1e-6,
+                                                            need_weight_grad=True))
+    flops = 2.0 * m * k * n
+    bytes_alg = 6 * m * n + 4 * m + 8 * d   # projection, cotangents (as wide together), d_fused: bf16 [M, N] each
+    achieved = bytes_alg / (float(k_ms.mean()) * 1e-3) / 1e9
+    rms_bytes = 6 * m * k + 4 * k
+    result = {
+        "metric": "Qwen3.5 attention input stage backward (pull-backs + LoRA cotangents, saved projection), "
+                  "TFLOP/s of 2*M*K*N per call",
+        "value": flops / (ms_per_step * 1e-3) / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": "qkv_post_bwd_kernel",
+                     "kernel_avg_ms": float(k_ms.mean()), "kernel_min_ms": float(k_ms.min()),
+                     "algorithmic_bytes": bytes_alg},
+        "stages": {
+            "linear_backward_ms": float(linear_ms.mean()), "forward_recompute_ms": float(recompute_ms.mean()),
+            "delta_rms_norm_bwd_kernel": {"avg_ms": float(rms_ms.mean()), "algorithmic_bytes": rms_bytes,
+                                          "achieved_gbs": rms_bytes / (float(rms_ms.mean()) * 1e-3) / 1e9,
+                                          "frac_of_hbm": rms_bytes / (float(rms_ms.mean()) * 1e-3) / 1e9 / HBM_PEAK_GBS},
+            "with_norm_weight_cotangents": {"post_call_ms": float(wgrad_post_ms.mean()),
+                                            "decoder_norm_call_ms": float(wgrad_rms_ms.mean())},
+        },
+    }
+    if not args.no_cpu_baseline:
+        rows = args.cpu_rows or 256
+        sel = slice(0, rows)
+        t1 = time.perf_counter()
+        want = o.w8a8_qkv_lora_rope_bwd(case["x"][sel], case["gamma"] - 1.0, qw, kw, case["weight"], case["a"],
+                                        case["b"], case["s"], case["idx"][sel], pos[sel], *(c[sel] for c in cots),
+                                        num_query_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                        rotary_dim=geo["rotary_dim"], rope_theta=theta, eps=1e-6)
+        secs = time.perf_counter() - t1
+        try:
+            cores = len(os.sched_getaffinity(0))
+        except AttributeError:
+            cores = os.cpu_count() or 1
+        threads = int(os.environ.get("OMP_NUM_THREADS", cores))
+        result["cpu_baseline"] = {"value": 2.0 * rows * k * n / secs / 1e12, "unit": "TFLOP/s",
+                                  "cores": min(cores, threads), "kind": "port",
+                                  "sample": f"first {rows} of {m} rows, NumPy oracle of the stage's backward "
+                                            f"(forward stages + pull-backs, float64 BLAS), one run, {secs:.3f} s",
+                                  "seconds": secs}
+        gate = o.numerical_gate(got[0][sel], want["dhidden"])  # rows of d_hidden are independent of each other
+        result["parity_sample"] = {"rows": rows, "relative_l2": gate["relative_l2"], "cosine": gate["cosine"]}
+    print(json.dumps(result))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -720,6 +844,8 @@ def main() -> int:
         return bench_moe_mlp(args, cfg, pkg, dev)
     if cfg.pop("moe_routing", False):
         return bench_moe_routing(args, cfg, pkg, dev)
+    if cfg.pop("qkv_backward", False):
+        return bench_qkv_backward(args, cfg, pkg, dev)
     if "qkv" in cfg:
         return bench_qkv(args, cfg, pkg, dev)
     case = wc.make_case(cfg["m"], cfg["k"], cfg["n"], n_adapters=cfg.get("n_adapters", 0),

@@ -937,9 +937,9 @@ int run_qkv_post_bwd(const mi355_w8a8_qkv_post_bwd_problem* p, hipStream_t s) {
     ColumnSumArgs c{};
     c.partial = a.partial; c.n_parts = parts; c.stride = 2u * p->head_dim; c.cols = p->head_dim;
     c.out = p->d_q_norm_weight; c.col0 = 0;
-    hipLaunchKernelGGL(column_sum_kernel, dim3((p->head_dim + 255u) / 256u), dim3(256), 0, s, c);
+    hipLaunchKernelGGL(column_sum_kernel, dim3((p->head_dim + 15u) / 16u), dim3(256), 0, s, c);
     c.out = p->d_k_norm_weight; c.col0 = p->head_dim;
-    hipLaunchKernelGGL(column_sum_kernel, dim3((p->head_dim + 255u) / 256u), dim3(256), 0, s, c);
+    hipLaunchKernelGGL(column_sum_kernel, dim3((p->head_dim + 15u) / 16u), dim3(256), 0, s, c);
   } else {
     if (vec4) hipLaunchKernelGGL((qkv_post_bwd_kernel<4, false>), dim3(p->m), dim3(256), 0, s, a);
     else hipLaunchKernelGGL((qkv_post_bwd_kernel<1, false>), dim3(p->m), dim3(256), 0, s, a);
@@ -997,7 +997,7 @@ int run_delta_rms_norm_bwd(const void* x, const float* gamma, const void* d_norm
     if ((st = launch_status())) return st;
     ColumnSumArgs c{};
     c.partial = g.partial; c.n_parts = slices; c.stride = k; c.cols = k; c.col0 = 0; c.out = d_gamma;
-    hipLaunchKernelGGL(column_sum_kernel, dim3((k + 255u) / 256u), dim3(256), 0, s, c);
+    hipLaunchKernelGGL(column_sum_kernel, dim3((k + 15u) / 16u), dim3(256), 0, s, c);
     return launch_status();
   }
   return MI355_W8A8_OK;

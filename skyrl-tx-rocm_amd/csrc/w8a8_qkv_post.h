@@ -321,7 +321,9 @@ __global__ __launch_bounds__(256) void qkv_post_bwd_kernel(QkvPostBwdArgs a) {
   }
 }
 
-// out[c] = sum over the first n_parts rows of partial[part][c], in order; one thread per column.
+// out[c] = sum over the n_parts rows of partial[part][col0 + c].  A workgroup takes 16 columns; its
+// 16 lanes per column sum every 16th part each (lane l: parts l, l + 16, ...), then lane 0 adds the
+// 16 sums in lane order: a fixed order whatever the launch.
 struct ColumnSumArgs {
   const float* partial;  // f32 [n_parts][stride]
   float* out;            // f32 [cols]
@@ -329,11 +331,22 @@ struct ColumnSumArgs {
 };
 
 __global__ __launch_bounds__(256) void column_sum_kernel(ColumnSumArgs a) {
-  const uint32_t c = blockIdx.x * 256u + threadIdx.x;
-  if (c >= a.cols) return;
+  __shared__ float red[16][17];
+  const uint32_t cl = threadIdx.x & 15u, pl = threadIdx.x >> 4;
+  const uint32_t c = blockIdx.x * 16u + cl;
   float s = 0.0f;
-  for (uint32_t p = 0; p < a.n_parts; ++p) s += a.partial[(size_t)p * a.stride + a.col0 + c];
-  a.out[c] = s;
+  if (c < a.cols) {
+#pragma unroll 4
+    for (uint32_t p = pl; p < a.n_parts; p += 16u) s += a.partial[(size_t)p * a.stride + a.col0 + c];
+  }
+  red[pl][cl] = s;
+  __syncthreads();
+  if (pl == 0 && c < a.cols) {
+    float t = red[0][cl];
+#pragma unroll
+    for (uint32_t l = 1; l < 16; ++l) t += red[l][cl];
+    a.out[c] = t;
+  }
 }
 
 }  // namespace w8a8

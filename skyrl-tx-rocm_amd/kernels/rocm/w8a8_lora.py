@@ -1323,6 +1323,92 @@ def delta_rms_norm_backward(x: torch.Tensor, gamma: torch.Tensor, d_normalized: 
     return out.reshape(x.shape), dw
 
 
+class QkvStageBackwardPlan:
+    """Buffers and C structs of one backward of the attention input stage with frozen norm weights
+    (the LoRA-training case): ``run()`` enqueues the forward recomputation (unless the projection and
+    the normalized rows are handed in), the split / norm / RoPE pull-back, the linear backward and the
+    decoder-norm pull-back in place on that call's dx.  Repeated calls reuse every buffer."""
+
+    def __init__(self, hidden: torch.Tensor, input_norm_weight: torch.Tensor, q_norm_weight: torch.Tensor,
+                 k_norm_weight: torch.Tensor, weight, lora_a, lora_b, lora_scaling, positions: torch.Tensor,
+                 config: Qwen35QKVStageConfig, d_q, d_k, d_v, d_gate, *, adapter_indices=None,
+                 need_lora_grads: bool = True, fused: torch.Tensor | None = None,
+                 normalized: torch.Tensor | None = None):
+        if (fused is None) != (normalized is None):
+            raise ValueError("hand in both the projection and the normalized rows, or neither")
+        dev = hidden.device
+        d, hq, hkv = config.head_dim, config.num_query_heads, config.num_kv_heads
+        k = hidden.shape[-1]
+        gamma = (1.0 + input_norm_weight.detach().to(torch.float32)).to(dev).contiguous()
+        self.fwd = None
+        if fused is None:
+            self.fwd = ForwardPlan(hidden, weight, lora_a, lora_b, lora_scaling, adapter_indices=adapter_indices,
+                                   rms_gamma=gamma, eps=config.rms_norm_eps, want_normalized=True)
+            fused, normalized = self.fwd.out, self.fwd.aux["normalized"]
+        if fused.dtype != torch.bfloat16 or fused.shape[-1] != config.fused_width:
+            raise ValueError("fused must be the bf16 projection of this configuration")
+        flat = fused.reshape(-1, config.fused_width).contiguous()
+        m = flat.shape[0]
+        if hidden.numel() != m * k or normalized.numel() != m * k:
+            raise ValueError("hidden, normalized and fused disagree on the number of rows")
+
+        def cot(t, width, name):
+            if t is None:
+                return torch.zeros((m, width), dtype=torch.bfloat16, device=dev)
+            if t.dtype != torch.bfloat16 or t.numel() != m * width:
+                raise ValueError(f"{name} must be BF16 with {m} x {width} elements")
+            return t.reshape(m, width).contiguous()
+
+        cots = (cot(d_q, hq * d, "d_q"), cot(d_k, hkv * d, "d_k"), cot(d_v, hkv * d, "d_v"), cot(d_gate, hq * d, "d_gate"))
+        qw = q_norm_weight.detach().to(device=dev, dtype=torch.float32).contiguous()
+        kw = k_norm_weight.detach().to(device=dev, dtype=torch.float32).contiguous()
+        pos = positions.reshape(-1).to(device=dev, dtype=torch.int32).contiguous()
+        if pos.numel() != m:
+            raise ValueError(f"positions must name {m} rows, got {tuple(positions.shape)}")
+        self.d_fused = torch.empty_like(flat)
+        p = _native.QkvPostBwdProblem()
+        p.struct_size = ctypes.sizeof(_native.QkvPostBwdProblem)
+        p.m, p.num_query_heads, p.num_kv_heads, p.head_dim, p.rotary_dim = m, hq, hkv, d, config.rotary_dim
+        p.rope_theta, p.rms_eps = float(config.rope_theta), float(config.rms_norm_eps)
+        p.fused, p.q_norm_weight, p.k_norm_weight, p.positions = flat.data_ptr(), qw.data_ptr(), kw.data_ptr(), pos.data_ptr()
+        p.d_q, p.d_k, p.d_v, p.d_gate = (c.data_ptr() for c in cots)
+        p.d_fused = self.d_fused.data_ptr()
+        self.post_problem = p
+        idx = adapter_indices
+        if idx is not None and idx.numel() != m:
+            idx = idx.reshape(-1).repeat_interleave(m // idx.numel())
+        self.bwd = BackwardPlan(normalized.reshape(m, k), self.d_fused, weight, lora_a, lora_b, lora_scaling,
+                                adapter_indices=idx, need_lora_grads=need_lora_grads)
+        self.x = hidden.reshape(m, k).contiguous()
+        self.gamma, self.eps = gamma, float(config.rms_norm_eps)
+        self.device, self.dx_shape, self.m, self.k = dev, tuple(hidden.shape), m, k
+        self._lib = _native.load()
+        self._keep = (flat, normalized, cots, qw, kw, pos)
+
+    def run_post_stage(self) -> None:
+        with torch.cuda.device(self.device):
+            status = self._lib.mi355_w8a8_qkv_split_norm_rope_bwd_v1(ctypes.byref(self.post_problem),
+                                                                     _stream_ptr(self.device))
+        _native.check("mi355_w8a8_qkv_split_norm_rope_bwd_v1", status)
+
+    def run_rms_stage(self) -> None:
+        dx = self.bwd.dx
+        with torch.cuda.device(self.device):
+            status = self._lib.mi355_w8a8_delta_rms_norm_bwd_v1(self.x.data_ptr(), self.gamma.data_ptr(), dx.data_ptr(),
+                                                                dx.data_ptr(), None, None, 0, self.m, self.k, self.eps,
+                                                                _stream_ptr(self.device))
+        _native.check("mi355_w8a8_delta_rms_norm_bwd_v1", status)
+
+    def run(self):
+        """Returns ``(d_hidden, d_lora_a, d_lora_b, d_lora_scaling)`` (reused tensors)."""
+        if self.fwd is not None:
+            self.fwd.run()
+        self.run_post_stage()
+        dn, da, db, ds = self.bwd.run()
+        self.run_rms_stage()
+        return dn.reshape(self.dx_shape), da, db, ds
+
+
 class _QkvStageFunction(torch.autograd.Function):
     """The stage with the derivative rule of ``_qwen35_qkv_lora_rope`` (qwen3_5_qkv_lora.py:288-454):
     cotangents for the hidden rows, the three norm weights, A, B and the scaling; none for the frozen
@@ -1422,5 +1508,5 @@ __all__ = (
     "w8a8_lora_linear", "w8a8_rms_gate_up_lora_swiglu", "w8a8_lora_residual", "PackedGroupedW8Weight",
     "prepare_grouped_weight", "grouped_forward", "grouped_backward", "grouped_lora_linear",
     "w8a8_grouped_lora_linear", "w8a8_moe_expert_mlp", "Qwen35QKVStageConfig", "QkvPostPlan", "qkv_split_norm_rope",
-    "w8a8_qkv_lora_rope", "qkv_lora_rope", "qkv_split_norm_rope_backward", "delta_rms_norm_backward",
+    "w8a8_qkv_lora_rope", "qkv_lora_rope", "qkv_split_norm_rope_backward", "delta_rms_norm_backward", "QkvStageBackwardPlan",
 )
