@@ -51,6 +51,7 @@ __global__ __launch_bounds__(256) void bwd_pack_dy_kernel(BwdPackDyArgs a) {
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
   const uint32_t mb = blockIdx.x / a.n_slices, sl = blockIdx.x % a.n_slices;
   if (mb >= a.n_row_blocks) return;
+  if (a.blk_range && a.blk_range[mb] < 0) return;  // block beyond the slots in use (grouped calls)
   const uint32_t i = lane & 31u, h = lane >> 5;
   const uint32_t p = mb * 32u + i;
   int src = -1;
@@ -243,6 +244,151 @@ __global__ __launch_bounds__(1024) void bwd_prep_kernel(BwdPrepArgs p) {
 }
 
 // ---------------------------------------------------------------------------------------
+// Tables of a grouped (per-expert) backward: the rows arrive sorted by group, group g owning
+// group_sizes[g] consecutive rows, and groups_per_weight consecutive groups share a frozen weight
+// (skyrl/tx/layers/lora.py:394-444).  Every weight's rows start at a multiple of 256 slots, so that
+// a pull-back tile never mixes two weights; inside a weight the groups follow each other without
+// gaps, exactly as the adapters of a dense call over that weight's rows would.
+//   src_row / dst_pos / slot_group / blk_range   as in the dense call (blk_range -1 beyond the slots in use)
+//   group_beg[g], group_end[g]                   slots of group g
+//   tile_weight[t]                               weight of 256-slot tile t, -1 beyond the slots in use
+//   chunk_tab[c] = (group, first slot, rows)     the 512-row chunks of the LoRA cotangents; rows 0 beyond
+//   chunk0[g]                                    first chunk of group g (n_groups + 1 entries)
+// One workgroup of 1024 threads.  Rows beyond sum(group_sizes) get no slot; their dx rows are cleared.
+// ---------------------------------------------------------------------------------------
+struct BwdGroupTables {
+  int32_t* src_row; int32_t* dst_pos; int32_t* slot_group; int32_t* blk_range;
+  int32_t* group_beg; int32_t* group_end; int32_t* tile_weight; int32_t* chunk_tab; int32_t* chunk0;
+};
+
+__device__ inline void route_weight_groups_block(const int32_t* __restrict__ group_sizes, uint32_t M, uint32_t n_groups,
+                                                 uint32_t gpw, uint32_t slots, uint32_t max_chunks, BwdGroupTables t,
+                                                 uint16_t* __restrict__ dx, uint32_t K) {
+  __shared__ int row_start[kMaxGroups + 1];
+  __shared__ int slot_beg[kMaxGroups + 1];
+  __shared__ int slot_end[kMaxGroups];
+  __shared__ int chunk_first[kMaxGroups + 1];
+  __shared__ int used_slots;
+  const uint32_t tid = threadIdx.x;
+  if (tid < n_groups) row_start[tid] = group_sizes[tid];  // sizes first, starts below
+  __syncthreads();
+  if (tid == 0) {
+    int r = 0, p = 0, ch = 0;
+    for (uint32_t g = 0; g < n_groups; ++g) {
+      if (g % gpw == 0) p = (p + 255) & ~255;
+      int sz = row_start[g];
+      if (sz < 0) sz = 0;
+      if (r + sz > (int)M) sz = (int)M - r;
+      row_start[g] = r;
+      slot_beg[g] = p;
+      chunk_first[g] = ch;
+      r += sz;
+      p += sz;
+      slot_end[g] = p;
+      ch += (sz + (int)kBwdChunkRows - 1) / (int)kBwdChunkRows;
+    }
+    row_start[n_groups] = r;
+    slot_beg[n_groups] = p;
+    chunk_first[n_groups] = ch;
+    used_slots = (p + 255) & ~255;
+  }
+  for (uint32_t p = tid; p < slots; p += 1024) { t.src_row[p] = -1; t.slot_group[p] = 0; }
+  for (uint32_t i = tid; i < M; i += 1024) t.dst_pos[i] = -1;
+  for (uint32_t c = tid; c < max_chunks; c += 1024) {
+    t.chunk_tab[3u * c] = 0; t.chunk_tab[3u * c + 1u] = 0; t.chunk_tab[3u * c + 2u] = 0;
+  }
+  __syncthreads();
+  const int used = used_slots;
+  for (uint32_t b = tid; b < slots / 32u; b += 1024) t.blk_range[b] = (int)(b * 32u) < used ? 0 : -1;
+  for (uint32_t tl = tid; tl < slots / 256u; tl += 1024) t.tile_weight[tl] = -1;
+  if (tid <= n_groups) t.chunk0[tid] = chunk_first[tid];
+  if (tid < n_groups) { t.group_beg[tid] = slot_beg[tid]; t.group_end[tid] = slot_end[tid]; }
+  __syncthreads();
+  const uint32_t wave = tid >> 6, lane = tid & 63;
+  for (uint32_t g = wave; g < n_groups; g += 16) {
+    const int r0 = row_start[g], cnt = row_start[g + 1] - r0, p0 = slot_beg[g];
+    for (int i = (int)lane; i < cnt; i += 64) {
+      t.src_row[p0 + i] = r0 + i;
+      t.dst_pos[r0 + i] = p0 + i;
+      t.slot_group[p0 + i] = (int)g;
+    }
+    const int nch = chunk_first[g + 1] - chunk_first[g];
+    for (int c = (int)lane; c < nch; c += 64) {
+      const int s0 = p0 + c * (int)kBwdChunkRows;
+      const int rows = slot_end[g] - s0 < (int)kBwdChunkRows ? slot_end[g] - s0 : (int)kBwdChunkRows;
+      int32_t* e = t.chunk_tab + 3 * (chunk_first[g] + c);
+      e[0] = (int)g; e[1] = s0; e[2] = rows;
+    }
+  }
+  // per weight: its tiles, and for every 32-slot block the groups its rows belong to; blocks and
+  // padding slots without a row name the weight's last group that has rows (or its first group)
+  const uint32_t n_weights = n_groups / gpw;
+  for (uint32_t w = wave; w < n_weights; w += 16) {
+    const uint32_t g0 = w * gpw, g1 = g0 + gpw;  // groups of this weight
+    const int wb = slot_beg[g0], we = slot_end[g1 - 1];
+    if (we == wb) continue;  // no rows: no tile
+    const int wpad = (we + 255) & ~255;
+    int glast = (int)g0;
+    for (uint32_t g = g0; g < g1; ++g)
+      if (slot_end[g] > slot_beg[g]) glast = (int)g;
+    for (int tl = wb / 256 + (int)lane; tl < wpad / 256; tl += 64) t.tile_weight[tl] = (int)w;
+    for (int p = we + (int)lane; p < wpad; p += 64) t.slot_group[p] = glast;
+    for (int b = wb / 32 + (int)lane; b < wpad / 32; b += 64) {
+      const int p0 = b * 32, p1 = p0 + 31 < we ? p0 + 31 : we - 1;
+      int lo = glast, hi = glast;
+      if (p0 < we) {
+        for (uint32_t g = g0; g < g1; ++g) {
+          if (p0 >= slot_beg[g] && p0 < slot_end[g]) lo = (int)g;
+          if (p1 >= slot_beg[g] && p1 < slot_end[g]) hi = (int)g;
+        }
+      }
+      t.blk_range[b] = lo | (hi << 16);
+    }
+  }
+  if (dx) {
+    const size_t begin = (size_t)row_start[n_groups] * K, end = (size_t)M * K;
+    for (size_t i = begin + tid; i < end; i += 1024) dx[i] = 0;
+  }
+}
+
+struct BwdGroupedPrepArgs {
+  const int32_t* group_sizes;
+  BwdGroupTables tab;
+  const uint16_t* lora_a;    // bf16 [n_groups, K, r]
+  uint16_t* at;              // bf16 [n_groups, r, K]
+  unsigned char* ap;
+  const float* sw;           // f32 [n_weights, N]
+  float* swp;                // f32 [n_weights][sw_stride] in packed column order
+  uint16_t* dx;              // rows beyond the groups are cleared
+  uint32_t M, K, N, N_pad, n_groups, gpw, n_weights, r, nkk, kb32, slots, max_chunks, sw_stride;
+  uint32_t a_blocks, ap_blocks, sw_blocks_per_weight;
+};
+
+__global__ __launch_bounds__(1024) void bwd_grouped_prep_kernel(BwdGroupedPrepArgs p) {
+  uint32_t b = blockIdx.x;
+  if (b == 0) {
+    route_weight_groups_block(p.group_sizes, p.M, p.n_groups, p.gpw, p.slots, p.max_chunks, p.tab, p.dx, p.K);
+    return;
+  }
+  b -= 1u;
+  if (b < p.a_blocks) {
+    lora_a_transpose_item(p.lora_a, p.at, p.n_groups, p.K, p.r, (uint64_t)b * 1024u + threadIdx.x);
+    return;
+  }
+  b -= p.a_blocks;
+  if (b < p.ap_blocks) {
+    lora_a_operand_item(p.lora_a, p.ap, p.n_groups, p.K, p.r, p.kb32, p.nkk, (uint64_t)b * 1024u + threadIdx.x);
+    return;
+  }
+  b -= p.ap_blocks;
+  const uint32_t w = b / p.sw_blocks_per_weight, c = (b % p.sw_blocks_per_weight) * 1024u + threadIdx.x;
+  if (w < p.n_weights && c < p.N_pad) {
+    const uint32_t n = packed_to_orig_col(c);
+    p.swp[(size_t)w * p.sw_stride + c] = n < p.N ? p.sw[(size_t)w * p.N + n] : 0.0f;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // dx = dyp @ bf16(W * sw).T (+ rs @ A.T), one bf16 cast.
 // Workgroup = 8 waves (2 along rows x 4 along k), tile 256 rows x 256 k, wave tile 128 x 64
 // (4 x 2 accumulator blocks of v_mfma_f32_32x32x16_bf16).  The contraction runs over n in stages
@@ -269,6 +415,11 @@ struct BwdDxArgs {
   const int32_t* src_row; const int32_t* slot_group; const int32_t* blk_range;
   uint16_t* dx;               // bf16 [M, K]
   uint32_t M, K, KB, NB, tiles_m, tiles_k;
+  // grouped calls: the weight of every 256-slot tile (-1: tile without rows), the bytes between two
+  // packed weights and the floats between two scale tables; null / 0 for one weight
+  const int32_t* tile_weight;
+  size_t w_stride;
+  uint32_t sw_stride;
 };
 
 template <int NKK>
@@ -299,12 +450,18 @@ __global__ __launch_bounds__(512, 1) void bwd_dx_kernel(BwdDxArgs g) {
     const uint32_t band_rows = (g.tiles_m - band * 4u) < 4u ? (g.tiles_m - band * 4u) : 4u;
     const uint32_t in_band = t - band * 4u * g.tiles_k;
     const uint32_t tm = band * 4u + in_band % band_rows, tk = in_band / band_rows;
+    int tw = 0;
+    if (g.tile_weight) {
+      tw = g.tile_weight[tm];
+      if (tw < 0) continue;  // workgroup-uniform: no row lives in this tile
+    }
+    const float* swp_t = g.swp + (size_t)tw * g.sw_stride;
 
     // this wave's two panel chunks of a stage (row block = wave, halves q = 0, 1) and its weight block
     const unsigned char* Ag = g.dyp + ((size_t)(tm * 8u + (uint32_t)wave) * g.NB) * 2048u + lane * 16;
     const uint32_t kbw = tk * 8u + (uint32_t)wcol * 2u;  // first of the two k blocks this wave multiplies
     const uint32_t kbl = tk * 8u + (uint32_t)wave < g.KB ? tk * 8u + (uint32_t)wave : g.KB - 1u;  // the block it loads
-    const unsigned char* Bg = g.wp + (size_t)kbl * kBlockBytes + lane * 16;
+    const unsigned char* Bg = g.wp + (size_t)tw * g.w_stride + (size_t)kbl * kBlockBytes + lane * 16;
     const size_t nb_stride = (size_t)g.KB * kBlockBytes;
 
     auto issue = [&](int nb) {
@@ -314,7 +471,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dx_kernel(BwdDxArgs g) {
       load_1k_to_lds(src + 1024, St + (wave * 2 + 1) * kBlockBytes);
       load_1k_to_lds(Bg + (size_t)nb * nb_stride, St + kBwdStagePanel + wave * kBlockBytes);
       // every wave fetches the same 1 KiB of scales (the stage's 32 lead it) to the same place
-      load_1k_to_lds(reinterpret_cast<const unsigned char*>(g.swp + 32 * nb) + lane * 16,
+      load_1k_to_lds(reinterpret_cast<const unsigned char*>(swp_t + 32 * nb) + lane * 16,
                      St + kBwdStagePanel + kBwdStageWeight);
     };
 
@@ -537,6 +694,7 @@ struct BwdDloraArgs {
   const float* z;           // f32 [slots][64]  x @ A
   const int32_t* src_row;   // or null
   const int32_t* group_off; // [n_groups + 1]
+  const int32_t* chunk_tab; // grouped calls: (group, first slot, rows) per chunk instead of group_off
   float* partA;             // [max_chunks][R][K]
   float* partB;             // [max_chunks][R][N]
   uint32_t M, K, N, n_groups, max_chunks, col_tiles_a, col_tiles_b;
@@ -579,7 +737,12 @@ __global__ __launch_bounds__(256) void bwd_dlora_kernel(BwdDloraArgs a) {
   const uint32_t cid = blockIdx.x / per_chunk, ct = blockIdx.x % per_chunk;
   if (tid == 0) {
     uint32_t grp = 0, slot0 = 0, rows = 0;
-    if (!bwd_find_chunk(a.group_off, a.n_groups, cid, grp, slot0, rows)) rows = 0;
+    if (a.chunk_tab) {
+      grp = (uint32_t)a.chunk_tab[3u * cid]; slot0 = (uint32_t)a.chunk_tab[3u * cid + 1u];
+      rows = (uint32_t)a.chunk_tab[3u * cid + 2u];
+    } else if (!bwd_find_chunk(a.group_off, a.n_groups, cid, grp, slot0, rows)) {
+      rows = 0;
+    }
     info[0] = grp; info[1] = slot0; info[2] = rows;
   }
   __syncthreads();
@@ -704,6 +867,8 @@ struct BwdReduceArgs {
   const float* z;           // f32 [slots][64]
   const float* lora_scaling;
   const int32_t* group_off;
+  // grouped calls: first chunk of every group (n_groups + 1) and the groups' slot ranges, in memory
+  const int32_t* chunk0_tab; const int32_t* group_beg; const int32_t* group_end;
   uint16_t* d_a;            // bf16 [n_groups, K, r] or null
   uint16_t* d_b;            // bf16 [n_groups, r, N] or null
   float* d_s;               // f32 [n_groups] or null
@@ -711,18 +876,19 @@ struct BwdReduceArgs {
 };
 
 __global__ __launch_bounds__(256) void bwd_dlora_reduce_kernel(BwdReduceArgs a) {
-  __shared__ uint32_t chunk0[kMaxAdapters + 1];
+  __shared__ uint32_t chunk0_lds[kMaxAdapters + 1];
   __shared__ double red[256];
   const uint32_t tid = threadIdx.x;
-  if (tid == 0) {
+  if (!a.chunk0_tab && tid == 0) {
     uint32_t run = 0;
     for (uint32_t gq = 0; gq < a.n_groups; ++gq) {
-      chunk0[gq] = run;
+      chunk0_lds[gq] = run;
       run += ((uint32_t)(a.group_off[gq + 1] - a.group_off[gq]) + kBwdChunkRows - 1u) / kBwdChunkRows;
     }
-    chunk0[a.n_groups] = run;
+    chunk0_lds[a.n_groups] = run;
   }
   __syncthreads();
+  auto chunk0 = [&](uint32_t gq) -> uint32_t { return a.chunk0_tab ? (uint32_t)a.chunk0_tab[gq] : chunk0_lds[gq]; };
   uint32_t b = blockIdx.x;
   if (b < a.blocks_a) {
     // dA [group][k][j]: a thread per output element, j fastest, so that the stores are contiguous
@@ -730,7 +896,7 @@ __global__ __launch_bounds__(256) void bwd_dlora_reduce_kernel(BwdReduceArgs a) 
     if (e >= (uint64_t)a.n_groups * a.K * a.r || !a.d_a) return;
     const uint32_t j = (uint32_t)(e % a.r), col = (uint32_t)((e / a.r) % a.K), grp = (uint32_t)(e / ((uint64_t)a.r * a.K));
     float sum = 0.0f;
-    for (uint32_t ch = chunk0[grp]; ch < chunk0[grp + 1]; ++ch) sum += a.partA[((size_t)ch * a.R + j) * a.K + col];
+    for (uint32_t ch = chunk0(grp), ce = chunk0(grp + 1u); ch < ce; ++ch) sum += a.partA[((size_t)ch * a.R + j) * a.K + col];
     a.d_a[e] = (uint16_t)f32_to_bf16_bits(sum);
     return;
   }
@@ -740,7 +906,7 @@ __global__ __launch_bounds__(256) void bwd_dlora_reduce_kernel(BwdReduceArgs a) 
     if (e >= (uint64_t)a.n_groups * a.r * a.N || !a.d_b) return;
     const uint32_t col = (uint32_t)(e % a.N), j = (uint32_t)((e / a.N) % a.r), grp = (uint32_t)(e / ((uint64_t)a.N * a.r));
     float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (uint32_t ch = chunk0[grp]; ch < chunk0[grp + 1]; ++ch) {
+    for (uint32_t ch = chunk0(grp), ce = chunk0(grp + 1u); ch < ce; ++ch) {
       const float4 v = *reinterpret_cast<const float4*>(a.partB + ((size_t)ch * a.R + j) * a.N + col);
       sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
     }
@@ -750,7 +916,8 @@ __global__ __launch_bounds__(256) void bwd_dlora_reduce_kernel(BwdReduceArgs a) 
   }
   b -= a.blocks_a + a.blocks_b;  // one block per group: ds
   if (b >= a.n_groups || !a.d_s) return;
-  const uint32_t o0 = (uint32_t)a.group_off[b], o1 = (uint32_t)a.group_off[b + 1];
+  const uint32_t o0 = (uint32_t)(a.group_beg ? a.group_beg[b] : a.group_off[b]);
+  const uint32_t o1 = (uint32_t)(a.group_end ? a.group_end[b] : a.group_off[b + 1]);
   double sum = 0.0;
   for (uint32_t i = o0 * a.r + tid; i < o1 * a.r; i += 256u) {
     const uint32_t slot = i / a.r, j = i % a.r;
