@@ -24,6 +24,7 @@
  *   - mi355_w8a8_grouped_v1            skyrl/tx/layers/lora.py:394-444 (LoRAExpert.__call__) with
  *                                      the ragged_dot of skyrl/tx/layers/util.py:8-59
  *   - mi355_w8a8_lora_linear_bwd_v1    skyrl/tx/kernels/quantized_lora.py:337-394 (the VJP)
+ *   - mi355_w8a8_grouped_bwd_v1        the same rule over skyrl/tx/layers/lora.py:394-444
  *   - mi355_w8a8_swiglu_bwd_v1 / mi355_w8a8_rms_norm_bwd_v1
  *                                      skyrl/tx/kernels/rocm/bf16_rms_gate_up_lora_swiglu_contiguous.py:541-574
  *   - mi355_w8a8_qkv_split_norm_rope_v1 skyrl/tx/kernels/qwen3_5_qkv_lora.py:266-286
@@ -181,6 +182,37 @@ typedef struct mi355_w8a8_bwd_problem {
 } mi355_w8a8_bwd_problem;
 
 /*
+ * Backward of the grouped call (plain epilogue): rows of x and dy are sorted by group as in the
+ * forward; group g owns group_sizes[g] consecutive rows and its own LoRA pair, groups_per_weight
+ * consecutive groups share a frozen weight.  Cotangents of groups without rows are zero, dx rows
+ * beyond sum(group_sizes) are zero.
+ */
+typedef struct mi355_w8a8_grouped_bwd_problem {
+  uint32_t struct_size;     /* sizeof(mi355_w8a8_grouped_bwd_problem) */
+  uint32_t flags;           /* 0 */
+  uint32_t m;               /* total rows */
+  uint32_t k;               /* multiple of 8 */
+  uint32_t n;               /* multiple of 8 */
+  uint32_t n_groups;        /* <= 1024 */
+  uint32_t rank;            /* 0 = no LoRA */
+  uint32_t groups_per_weight; /* 0 or 1: one weight per group */
+  const void* x;            /* bf16 [m, k]; needed only when a LoRA cotangent is requested */
+  const void* dy;           /* bf16 [m, n] */
+  const void* w_packed;     /* n_groups / groups_per_weight packed weights back to back */
+  const float* w_scales;    /* f32 [n_groups / groups_per_weight, n] */
+  const void* lora_a;       /* bf16 [n_groups, k, rank] or NULL */
+  const void* lora_b;       /* bf16 [n_groups, rank, n] or NULL */
+  const float* lora_scaling;/* f32 [n_groups] or NULL */
+  const int32_t* group_sizes; /* int32 [n_groups] */
+  void* dx;                 /* bf16 [m, k] */
+  void* d_lora_a;           /* bf16 [n_groups, k, rank] or NULL (not wanted) */
+  void* d_lora_b;           /* bf16 [n_groups, rank, n] or NULL */
+  float* d_lora_scaling;    /* f32 [n_groups] or NULL */
+  void* workspace;          /* >= mi355_w8a8_grouped_bwd_workspace_bytes(...), 256-byte aligned */
+  uint64_t workspace_bytes;
+} mi355_w8a8_grouped_bwd_problem;
+
+/*
  * Qwen3.5 attention input stage behind the fused QKV projection: split of the interleaved
  * projection (per kv head: queries_per_kv (q, gate) chunk pairs, then k, then v), RMSNorm with
  * (1 + weight) over every Q and K head, partial RoPE on Q and K.
@@ -279,6 +311,17 @@ int mi355_w8a8_grouped_v1(const mi355_w8a8_grouped_problem* problem, void* strea
 uint64_t mi355_w8a8_bwd_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t n_adapters,
                                         uint32_t rank, uint32_t flags);
 int mi355_w8a8_lora_linear_bwd_v1(const mi355_w8a8_bwd_problem* problem, void* stream);
+
+/*
+ * Backward of mi355_w8a8_grouped_v1 without FLAG_SWIGLU: the derivative of LoRAExpert.__call__
+ * (skyrl/tx/layers/lora.py:394-444, ragged_dot of skyrl/tx/layers/util.py:8-59) under the rule of
+ * mi355_w8a8_lora_linear_bwd_v1, in one call for all groups: every weight's rows form their own
+ * 256-row pull-back tiles, the groups that share a weight take the role of its adapters.  The
+ * results are bit-equal to one mi355_w8a8_lora_linear_bwd_v1 call per weight over its rows.
+ */
+uint64_t mi355_w8a8_grouped_bwd_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups,
+                                                uint32_t rank, uint32_t groups_per_weight);
+int mi355_w8a8_grouped_bwd_v1(const mi355_w8a8_grouped_bwd_problem* problem, void* stream);
 
 /*
  * The part of qwen35_qkv_lora_rope behind the projection (skyrl/tx/kernels/qwen3_5_qkv_lora.py:

@@ -36,6 +36,7 @@ EXPORTS = (
     "mi355_w8a8_lora_linear_v1", "mi355_w8a8_rms_gateup_swiglu_v1", "mi355_w8a8_lora_residual_v1",
     "mi355_w8a8_forward_v1", "mi355_w8a8_grouped_v1",
     "mi355_w8a8_bwd_workspace_bytes", "mi355_w8a8_lora_linear_bwd_v1",
+    "mi355_w8a8_grouped_bwd_workspace_bytes", "mi355_w8a8_grouped_bwd_v1",
     "mi355_w8a8_qkv_split_norm_rope_v1",
     "mi355_w8a8_qkv_bwd_workspace_bytes", "mi355_w8a8_qkv_split_norm_rope_bwd_v1",
     "mi355_w8a8_delta_rms_norm_bwd_workspace_bytes", "mi355_w8a8_delta_rms_norm_bwd_v1",
@@ -83,6 +84,18 @@ class BwdProblem(ctypes.Structure):
         ("n_adapters", _u32), ("rank", _u32), ("reserved", _u32),
         ("x", _vp), ("dy", _vp), ("w_packed", _vp), ("w_scales", _vp), ("lora_a", _vp), ("lora_b", _vp),
         ("lora_scaling", _vp), ("adapter_indices", _vp), ("dx", _vp), ("d_lora_a", _vp), ("d_lora_b", _vp),
+        ("d_lora_scaling", _vp), ("workspace", _vp), ("workspace_bytes", _u64),
+    ]
+
+
+class GroupedBwdProblem(ctypes.Structure):
+    """struct mi355_w8a8_grouped_bwd_problem"""
+
+    _fields_ = [
+        ("struct_size", _u32), ("flags", _u32), ("m", _u32), ("k", _u32), ("n", _u32),
+        ("n_groups", _u32), ("rank", _u32), ("groups_per_weight", _u32),
+        ("x", _vp), ("dy", _vp), ("w_packed", _vp), ("w_scales", _vp), ("lora_a", _vp), ("lora_b", _vp),
+        ("lora_scaling", _vp), ("group_sizes", _vp), ("dx", _vp), ("d_lora_a", _vp), ("d_lora_b", _vp),
         ("d_lora_scaling", _vp), ("workspace", _vp), ("workspace_bytes", _u64),
     ]
 
@@ -172,6 +185,10 @@ def _bind(lib: ctypes.CDLL) -> None:
     lib.mi355_w8a8_grouped_v1.argtypes = (ctypes.POINTER(GroupedProblem), _vp)
     lib.mi355_w8a8_lora_linear_bwd_v1.restype = ctypes.c_int
     lib.mi355_w8a8_lora_linear_bwd_v1.argtypes = (ctypes.POINTER(BwdProblem), _vp)
+    lib.mi355_w8a8_grouped_bwd_workspace_bytes.restype = _u64
+    lib.mi355_w8a8_grouped_bwd_workspace_bytes.argtypes = (_u32, _u32, _u32, _u32, _u32, _u32)
+    lib.mi355_w8a8_grouped_bwd_v1.restype = ctypes.c_int
+    lib.mi355_w8a8_grouped_bwd_v1.argtypes = (ctypes.POINTER(GroupedBwdProblem), _vp)
     lib.mi355_w8a8_qkv_split_norm_rope_v1.restype = ctypes.c_int
     lib.mi355_w8a8_qkv_split_norm_rope_v1.argtypes = (ctypes.POINTER(QkvPostProblem), _vp)
     lib.mi355_w8a8_qkv_bwd_workspace_bytes.restype = _u64

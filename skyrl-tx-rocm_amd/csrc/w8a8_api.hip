@@ -836,6 +836,267 @@ int run_backward(const mi355_w8a8_bwd_problem* p, hipStream_t s) {
   return MI355_W8A8_OK;
 }
 
+// ---------------------------------------------------------------------------------------
+// grouped (per-expert) backward
+// ---------------------------------------------------------------------------------------
+struct BwdGroupedLayout {
+  uint64_t dyp, swp, src_row, dst_pos, slot_group, blk_range, group_beg, group_end, tile_weight, chunk_tab, chunk0,
+      at, ap, rp, z, r_raw, rs, rpart, partA, partB, total;
+  uint32_t slots, nkk, K_pad, KB, N_pad, NB, tiles_m, tiles_k, max_chunks, R, n_slices, groups_per_slice, n_weights,
+      gpw, sw_stride;
+};
+
+BwdGroupedLayout make_bwd_grouped_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint32_t rank,
+                                         uint32_t gpw_in) {
+  BwdGroupedLayout w{};
+  w.gpw = gpw_in ? gpw_in : 1u;
+  w.n_weights = n_groups / w.gpw;
+  w.K_pad = k_padded(k); w.KB = w.K_pad / 32u;
+  w.N_pad = n_padded(n); w.NB = w.N_pad / 32u;
+  // every weight with rows pads its slots to a multiple of 256
+  const uint32_t with_rows = w.n_weights < m ? w.n_weights : m;
+  w.slots = round_up(m + 255u * with_rows, 256u);
+  w.tiles_m = w.slots / 256u;
+  w.tiles_k = (w.K_pad + 255u) / 256u;
+  w.nkk = rank_chunks(rank);
+  w.R = w.nkk > 2u ? 64u : 32u;
+  w.max_chunks = (m + kBwdChunkRows - 1u) / kBwdChunkRows + n_groups;
+  {
+    const uint32_t ng = w.N_pad / 128u;
+    w.n_slices = (ng + 3u) / 4u < 8u ? (ng + 3u) / 4u : 8u;
+    w.groups_per_slice = (ng + w.n_slices - 1u) / w.n_slices;
+  }
+  w.sw_stride = w.N_pad + kBwdScalePad;
+  uint64_t off = 0;
+  w.dyp = off; off += align256((uint64_t)w.slots * w.N_pad * 2u);
+  w.swp = off; off += align256((uint64_t)w.n_weights * w.sw_stride * 4u);
+  w.src_row = off; off += align256((uint64_t)w.slots * 4u);
+  w.dst_pos = off; off += align256((uint64_t)m * 4u);
+  w.slot_group = off; off += align256((uint64_t)w.slots * 4u);
+  w.blk_range = off; off += align256((uint64_t)(w.slots / 32u) * 4u);
+  w.group_beg = off; off += align256((uint64_t)n_groups * 4u);
+  w.group_end = off; off += align256((uint64_t)n_groups * 4u);
+  w.tile_weight = off; off += align256((uint64_t)w.tiles_m * 4u);
+  w.chunk_tab = off; off += align256((uint64_t)w.max_chunks * 12u);
+  w.chunk0 = off; off += align256((uint64_t)(n_groups + 1u) * 4u);
+  if (rank) {
+    w.at = off; off += align256((uint64_t)n_groups * rank * k * 2u);
+    w.ap = off; off += align256((uint64_t)n_groups * w.KB * w.nkk * kBlockBytes);
+    w.rp = off; off += align256((uint64_t)(w.slots / 32u) * w.nkk * 3u * kBlockBytes);
+    w.z = off; off += align256((uint64_t)w.slots * kBwdRankStride * 4u);
+    w.r_raw = off; off += align256((uint64_t)w.slots * kBwdRankStride * 4u);
+    w.rs = off; off += align256((uint64_t)w.slots * kBwdRankStride * 4u);
+    w.rpart = off; off += align256((uint64_t)w.n_slices * w.slots * kBwdRankStride * 4u);
+    w.partA = off; off += align256((uint64_t)w.max_chunks * w.R * k * 4u);
+    w.partB = off; off += align256((uint64_t)w.max_chunks * w.R * n * 4u);
+  }
+  w.total = off;
+  return w;
+}
+
+int validate_bwd_grouped_dims(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint32_t rank, uint32_t gpw) {
+  int st = validate_common(m, k, n);
+  if (st) return st;
+  if (n % 8u) return MI355_W8A8_ERR_UNSUPPORTED;
+  if (n_groups == 0) return MI355_W8A8_ERR_SHAPE;
+  if (gpw == 0) gpw = 1;
+  if (n_groups % gpw) return MI355_W8A8_ERR_SHAPE;
+  if (n_groups > (uint32_t)kMaxGroups || rank > (uint32_t)kMaxRank) return MI355_W8A8_ERR_UNSUPPORTED;
+  // 32-bit element offsets into dx, and slots that stay below the row limit
+  if ((uint64_t)m * k >= (1ull << 32) - (1ull << 20)) return MI355_W8A8_ERR_UNSUPPORTED;
+  if ((uint64_t)m + 255ull * (n_groups / gpw) + 256ull > (uint64_t)kMaxRows) return MI355_W8A8_ERR_UNSUPPORTED;
+  return MI355_W8A8_OK;
+}
+
+int run_grouped_backward(const mi355_w8a8_grouped_bwd_problem* p, hipStream_t s) {
+  if (!p) return MI355_W8A8_ERR_NULL;
+  if (p->struct_size != sizeof(mi355_w8a8_grouped_bwd_problem)) return MI355_W8A8_ERR_STRUCT;
+  if (p->flags) return MI355_W8A8_ERR_SHAPE;
+  int st = validate_bwd_grouped_dims(p->m, p->k, p->n, p->n_groups, p->rank, p->groups_per_weight);
+  if (st) return st;
+  if (!p->dy || !p->w_packed || !p->w_scales || !p->dx || !p->group_sizes) return MI355_W8A8_ERR_NULL;
+  const bool lora = p->rank > 0;
+  const bool want_grads = p->d_lora_a || p->d_lora_b || p->d_lora_scaling;
+  if (lora) {
+    if (!p->lora_a || !p->lora_b || !p->lora_scaling) return MI355_W8A8_ERR_NULL;
+    if (want_grads && !p->x) return MI355_W8A8_ERR_NULL;
+  } else if (p->lora_a || p->lora_b || want_grads) {
+    return MI355_W8A8_ERR_SHAPE;
+  }
+  if (!aligned16(p->x) || !aligned16(p->dy) || !aligned16(p->w_packed) || !aligned16(p->w_scales) ||
+      !aligned16(p->lora_a) || !aligned16(p->lora_b) || !aligned16(p->dx) || !aligned16(p->d_lora_a) ||
+      !aligned16(p->d_lora_b) || (reinterpret_cast<uintptr_t>(p->group_sizes) & 3u))
+    return MI355_W8A8_ERR_ALIGN;
+  const uint64_t dx_bytes = (uint64_t)p->m * p->k * 2u, dy_bytes = (uint64_t)p->m * p->n * 2u;
+  const uint64_t a_bytes = (uint64_t)p->n_groups * p->rank * p->k * 2u, b_bytes = (uint64_t)p->n_groups * p->rank * p->n * 2u;
+  if (overlaps(p->dx, dx_bytes, p->dy, dy_bytes) || overlaps(p->dx, dx_bytes, p->x, dx_bytes) ||
+      overlaps(p->dx, dx_bytes, p->workspace, p->workspace_bytes) ||
+      overlaps(p->d_lora_a, a_bytes, p->lora_a, a_bytes) || overlaps(p->d_lora_b, b_bytes, p->lora_b, b_bytes) ||
+      overlaps(p->d_lora_a, a_bytes, p->workspace, p->workspace_bytes) ||
+      overlaps(p->d_lora_b, b_bytes, p->workspace, p->workspace_bytes) ||
+      overlaps(p->d_lora_a, a_bytes, p->dx, dx_bytes) || overlaps(p->d_lora_b, b_bytes, p->dx, dx_bytes))
+    return MI355_W8A8_ERR_ALIAS;
+  const BwdGroupedLayout w = make_bwd_grouped_layout(p->m, p->k, p->n, p->n_groups, p->rank, p->groups_per_weight);
+  if (!p->workspace || p->workspace_bytes < w.total) return MI355_W8A8_ERR_WORKSPACE;
+  if (reinterpret_cast<uintptr_t>(p->workspace) & 255u) return MI355_W8A8_ERR_ALIGN;
+  unsigned char* ws = static_cast<unsigned char*>(p->workspace);
+  BwdGroupTables tab{};
+  tab.src_row = reinterpret_cast<int32_t*>(ws + w.src_row);
+  tab.dst_pos = reinterpret_cast<int32_t*>(ws + w.dst_pos);
+  tab.slot_group = reinterpret_cast<int32_t*>(ws + w.slot_group);
+  tab.blk_range = reinterpret_cast<int32_t*>(ws + w.blk_range);
+  tab.group_beg = reinterpret_cast<int32_t*>(ws + w.group_beg);
+  tab.group_end = reinterpret_cast<int32_t*>(ws + w.group_end);
+  tab.tile_weight = reinterpret_cast<int32_t*>(ws + w.tile_weight);
+  tab.chunk_tab = reinterpret_cast<int32_t*>(ws + w.chunk_tab);
+  tab.chunk0 = reinterpret_cast<int32_t*>(ws + w.chunk0);
+  (void)hipGetLastError();
+
+  {  // tables: routing, A transposed / in operand order, every weight's scales in packed column order
+    BwdGroupedPrepArgs pa{};
+    pa.group_sizes = p->group_sizes;
+    pa.tab = tab;
+    pa.lora_a = static_cast<const uint16_t*>(p->lora_a);
+    pa.at = lora ? reinterpret_cast<uint16_t*>(ws + w.at) : nullptr;
+    pa.ap = lora ? ws + w.ap : nullptr;
+    pa.sw = p->w_scales; pa.swp = reinterpret_cast<float*>(ws + w.swp);
+    pa.dx = static_cast<uint16_t*>(p->dx);
+    pa.M = p->m; pa.K = p->k; pa.N = p->n; pa.N_pad = w.N_pad; pa.n_groups = p->n_groups; pa.gpw = w.gpw;
+    pa.n_weights = w.n_weights; pa.r = p->rank; pa.nkk = w.nkk; pa.kb32 = w.KB; pa.slots = w.slots;
+    pa.max_chunks = w.max_chunks; pa.sw_stride = w.sw_stride;
+    pa.a_blocks = lora ? (uint32_t)(((uint64_t)p->n_groups * p->k * ((p->rank + 7u) / 8u) + 1023u) / 1024u) : 0u;
+    pa.ap_blocks = lora ? (uint32_t)(((uint64_t)p->n_groups * w.KB * w.nkk * 64u + 1023u) / 1024u) : 0u;
+    pa.sw_blocks_per_weight = (w.N_pad + 1023u) / 1024u;
+    hipLaunchKernelGGL(bwd_grouped_prep_kernel,
+                       dim3(1u + pa.a_blocks + pa.ap_blocks + pa.sw_blocks_per_weight * w.n_weights), dim3(1024), 0, s, pa);
+    if ((st = launch_status())) return st;
+  }
+  {  // dy into operand order; the same pass leaves the partial sums of r = dy @ B.T
+    BwdPackDyArgs d{};
+    d.dy = static_cast<const uint16_t*>(p->dy);
+    d.src_row = tab.src_row; d.slot_group = tab.slot_group; d.blk_range = tab.blk_range;
+    d.dyp = ws + w.dyp;
+    d.lora_b = static_cast<const uint16_t*>(p->lora_b);
+    d.rpart = lora ? reinterpret_cast<float*>(ws + w.rpart) : nullptr;
+    d.M = p->m; d.N = p->n; d.NB = w.NB; d.n_row_blocks = w.slots / 32u; d.n_col_groups = w.N_pad / 128u;
+    d.n_slices = w.n_slices; d.groups_per_slice = w.groups_per_slice; d.r = p->rank; d.slots = w.slots;
+    const dim3 grid(d.n_row_blocks * d.n_slices), block(256);
+    if (!lora) hipLaunchKernelGGL((bwd_pack_dy_kernel<0>), grid, block, 0, s, d);
+    else if (w.nkk > 2u) hipLaunchKernelGGL((bwd_pack_dy_kernel<2>), grid, block, 0, s, d);
+    else hipLaunchKernelGGL((bwd_pack_dy_kernel<1>), grid, block, 0, s, d);
+    if ((st = launch_status())) return st;
+  }
+  if (lora) {
+    {
+      BwdRFinishArgs f{};
+      f.rpart = reinterpret_cast<const float*>(ws + w.rpart);
+      f.slot_group = tab.slot_group;
+      f.blk_range = tab.blk_range;
+      f.lora_scaling = p->lora_scaling;
+      f.r_raw = reinterpret_cast<float*>(ws + w.r_raw);
+      f.rs = reinterpret_cast<float*>(ws + w.rs);
+      f.rp = ws + w.rp;
+      f.n_slices = w.n_slices; f.slots = w.slots; f.nkk = w.nkk; f.cols = w.nkk > 2u ? 64u : 32u;
+      hipLaunchKernelGGL(bwd_r_finish_kernel, dim3(w.slots / 32u), dim3(256), 0, s, f);
+      if ((st = launch_status())) return st;
+    }
+    if (p->d_lora_b || p->d_lora_scaling) {  // z = x @ A
+      LoraAArgs lz{};
+      lz.xsrc = static_cast<const uint16_t*>(p->x);
+      lz.at = reinterpret_cast<const uint16_t*>(ws + w.at);
+      lz.src_row = tab.src_row; lz.slot_group = tab.slot_group; lz.blk_range = tab.blk_range;
+      lz.zp = nullptr;
+      lz.M = p->m; lz.K = p->k; lz.r = p->rank; lz.nkk = w.nkk;
+      lz.n_steps = (p->k + 63u) / 64u;
+      lz.nterms = 3u;
+      lz.n_blocks = w.slots / 32u;
+      const uint32_t nks = w.n_slices;
+      lz.n_ksplit = nks;
+      lz.steps_per_wave = ((lz.n_steps + nks - 1u) / nks + 15u) / 16u;
+      lz.zf = reinterpret_cast<float*>(ws + w.rpart);
+      lz.zf_stride = kBwdRankStride;
+      lz.zf_slice = w.slots * kBwdRankStride;
+      const dim3 grid(lz.n_blocks * nks), block(1024);
+      if (w.nkk > 2u) hipLaunchKernelGGL((lora_a_kernel<2>), grid, block, 0, s, lz);
+      else hipLaunchKernelGGL((lora_a_kernel<1>), grid, block, 0, s, lz);
+      if ((st = launch_status())) return st;
+      BwdRFinishArgs f{};
+      f.rpart = reinterpret_cast<const float*>(ws + w.rpart);
+      f.blk_range = tab.blk_range;
+      f.r_raw = reinterpret_cast<float*>(ws + w.z);
+      f.n_slices = nks; f.slots = w.slots; f.nkk = w.nkk; f.cols = w.nkk > 2u ? 64u : 32u;
+      hipLaunchKernelGGL(bwd_r_finish_kernel, dim3(w.slots / 32u), dim3(256), 0, s, f);
+      if ((st = launch_status())) return st;
+    }
+  }
+  {
+    BwdDxArgs g{};
+    g.dyp = ws + w.dyp;
+    g.wp = static_cast<const unsigned char*>(p->w_packed);
+    g.swp = reinterpret_cast<const float*>(ws + w.swp);
+    g.rp = lora ? ws + w.rp : nullptr;
+    g.ap = lora ? ws + w.ap : nullptr;
+    g.src_row = tab.src_row; g.slot_group = tab.slot_group; g.blk_range = tab.blk_range;
+    g.dx = static_cast<uint16_t*>(p->dx);
+    g.M = p->m; g.K = p->k; g.KB = w.KB; g.NB = w.NB; g.tiles_m = w.tiles_m; g.tiles_k = w.tiles_k;
+    g.tile_weight = tab.tile_weight;
+    g.w_stride = (size_t)mi355_w8a8_packed_weight_bytes(p->k, p->n);
+    g.sw_stride = w.sw_stride;
+    switch (lora ? w.nkk : 0u) {
+      case 0: st = launch_bwd_dx<0>(g, s); break;
+      case 1: st = launch_bwd_dx<1>(g, s); break;
+      case 2: st = launch_bwd_dx<2>(g, s); break;
+      default: st = launch_bwd_dx<4>(g, s); break;
+    }
+    if (st) return st;
+  }
+  if (lora && want_grads) {
+    BwdDloraArgs d{};
+    d.x = static_cast<const uint16_t*>(p->x);
+    d.dy = static_cast<const uint16_t*>(p->dy);
+    d.rs = reinterpret_cast<const float*>(ws + w.rs);
+    d.z = reinterpret_cast<const float*>(ws + w.z);
+    d.src_row = tab.src_row;
+    d.group_off = nullptr;
+    d.chunk_tab = tab.chunk_tab;
+    d.partA = reinterpret_cast<float*>(ws + w.partA);
+    d.partB = reinterpret_cast<float*>(ws + w.partB);
+    d.M = p->m; d.K = p->k; d.N = p->n; d.n_groups = p->n_groups; d.max_chunks = w.max_chunks;
+    d.col_tiles_a = p->d_lora_a ? (p->k + 255u) / 256u : 0u;
+    d.col_tiles_b = p->d_lora_b ? (p->n + 255u) / 256u : 0u;
+    if (d.col_tiles_a + d.col_tiles_b) {
+      const dim3 grid(w.max_chunks * (d.col_tiles_a + d.col_tiles_b)), block(256);
+      const uint32_t lds_bytes = (kBwdStageRows / 32u) * (w.R / 32u) * 6u * kBlockBytes;
+      if (w.R == 32u) {
+        hipLaunchKernelGGL((bwd_dlora_kernel<1>), grid, block, lds_bytes, s, d);
+      } else {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_dlora_kernel<2>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
+          return MI355_W8A8_ERR_LAUNCH;
+        hipLaunchKernelGGL((bwd_dlora_kernel<2>), grid, block, lds_bytes, s, d);
+      }
+      if ((st = launch_status())) return st;
+    }
+    BwdReduceArgs r{};
+    r.partA = d.partA; r.partB = d.partB;
+    r.r_raw = reinterpret_cast<const float*>(ws + w.r_raw);
+    r.z = d.z;
+    r.lora_scaling = p->lora_scaling;
+    r.group_off = nullptr;
+    r.chunk0_tab = tab.chunk0; r.group_beg = tab.group_beg; r.group_end = tab.group_end;
+    r.d_a = static_cast<uint16_t*>(p->d_lora_a);
+    r.d_b = static_cast<uint16_t*>(p->d_lora_b);
+    r.d_s = p->d_lora_scaling;
+    r.K = p->k; r.N = p->n; r.r = p->rank; r.R = w.R; r.n_groups = p->n_groups;
+    r.blocks_a = p->d_lora_a ? (uint32_t)(((uint64_t)p->n_groups * p->rank * p->k + 255u) / 256u) : 0u;
+    r.blocks_b = p->d_lora_b ? (uint32_t)(((uint64_t)p->n_groups * p->rank * p->n / 4u + 255u) / 256u) : 0u;
+    const uint32_t s_blocks = p->d_lora_scaling ? p->n_groups : 0u;
+    hipLaunchKernelGGL(bwd_dlora_reduce_kernel, dim3(r.blocks_a + r.blocks_b + s_blocks), dim3(256), 0, s, r);
+    if ((st = launch_status())) return st;
+  }
+  return MI355_W8A8_OK;
+}
+
 int run_qkv_post(const mi355_w8a8_qkv_post_problem* p, hipStream_t s) {
   if (!p) return MI355_W8A8_ERR_NULL;
   if (p->struct_size != sizeof(mi355_w8a8_qkv_post_problem)) return MI355_W8A8_ERR_STRUCT;
@@ -1479,6 +1740,16 @@ uint64_t mi355_w8a8_bwd_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint
 
 int mi355_w8a8_lora_linear_bwd_v1(const mi355_w8a8_bwd_problem* p, void* stream) {
   return run_backward(p, static_cast<hipStream_t>(stream));
+}
+
+uint64_t mi355_w8a8_grouped_bwd_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint32_t rank,
+                                                uint32_t groups_per_weight) {
+  if (validate_bwd_grouped_dims(m, k, n, n_groups, rank, groups_per_weight)) return 0;
+  return make_bwd_grouped_layout(m, k, n, n_groups, rank, groups_per_weight).total;
+}
+
+int mi355_w8a8_grouped_bwd_v1(const mi355_w8a8_grouped_bwd_problem* p, void* stream) {
+  return run_grouped_backward(p, static_cast<hipStream_t>(stream));
 }
 
 int mi355_w8a8_qkv_split_norm_rope_v1(const mi355_w8a8_qkv_post_problem* p, void* stream) {

@@ -32,6 +32,8 @@ namespace w8a8 {
 // leaves its partial sum in rpart[slice][slot][64]; bwd_r_finish_kernel adds the slices.
 // ---------------------------------------------------------------------------------------
 constexpr uint32_t kBwdRankStride = 64;  // floats per slot in the z / r tables
+constexpr uint32_t kBwdChunkRows = 512;  // rows of a chunk of the LoRA cotangents
+constexpr uint32_t kBwdStageRows = 256;  // rows whose skinny operand sits in LDS at a time
 
 struct BwdPackDyArgs {
   const uint16_t* dy;        // bf16 [M, N]
@@ -139,7 +141,7 @@ __global__ __launch_bounds__(256) void bwd_pack_dy_kernel(BwdPackDyArgs a) {
 // scaled by the row's group (for dA), and the scaled value split exactly into three bf16 terms in
 // the operand order of the pull-back epilogue, rp[block][kk][term][lane][8].
 struct BwdRFinishArgs {
-  const float* rpart; const int32_t* slot_group; const float* lora_scaling;
+  const float* rpart; const int32_t* slot_group; const int32_t* blk_range; const float* lora_scaling;
   float* r_raw; float* rs; unsigned char* rp;
   uint32_t n_slices, slots, nkk, cols;  // cols = 16 * nkk rounded up to 32
 };
@@ -147,6 +149,7 @@ struct BwdRFinishArgs {
 __global__ __launch_bounds__(256) void bwd_r_finish_kernel(BwdRFinishArgs a) {
   __shared__ float zs[32][kBwdRankStride + 1];
   const uint32_t pb = blockIdx.x;
+  if (a.blk_range && a.blk_range[pb] < 0) return;  // block beyond the slots in use (grouped calls)
   for (uint32_t q = threadIdx.x; q < 32u * a.cols; q += 256u) {
     const uint32_t row = q / a.cols, col = q % a.cols, slot = pb * 32u + row;
     float raw = 0.0f;
@@ -301,7 +304,7 @@ __device__ inline void route_weight_groups_block(const int32_t* __restrict__ gro
   const int used = used_slots;
   for (uint32_t b = tid; b < slots / 32u; b += 1024) t.blk_range[b] = (int)(b * 32u) < used ? 0 : -1;
   for (uint32_t tl = tid; tl < slots / 256u; tl += 1024) t.tile_weight[tl] = -1;
-  if (tid <= n_groups) t.chunk0[tid] = chunk_first[tid];
+  for (uint32_t g = tid; g <= n_groups; g += 1024) t.chunk0[g] = chunk_first[g];
   if (tid < n_groups) { t.group_beg[tid] = slot_beg[tid]; t.group_end[tid] = slot_end[tid]; }
   __syncthreads();
   const uint32_t wave = tid >> 6, lane = tid & 63;
@@ -684,8 +687,6 @@ __global__ __launch_bounds__(512, 1) void bwd_dx_kernel(BwdDxArgs g) {
 // ds[g] = sum_m sum_j r[m][j] * z[m][j] with r the unscaled dy @ B.T.  Fixed orders: results are
 // deterministic.
 // ---------------------------------------------------------------------------------------
-constexpr uint32_t kBwdChunkRows = 512;  // rows of a chunk
-constexpr uint32_t kBwdStageRows = 256;  // rows whose skinny operand sits in LDS at a time
 
 struct BwdDloraArgs {
   const uint16_t* x;        // bf16 [M, K]

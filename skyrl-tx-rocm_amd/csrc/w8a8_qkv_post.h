@@ -224,7 +224,7 @@ __global__ __launch_bounds__(256) void qkv_post_bwd_kernel(QkvPostBwdArgs a) {
       for (uint32_t j = 0; j < NP; ++j) {
         const uint32_t i = V * lane + 64u * V * j;
         if (i < a.D) {
-          if (V == 4) {
+          if constexpr (V == 4) {
             *reinterpret_cast<uint2*>(orow + off + a.D + i) = *reinterpret_cast<const uint2*>(dcopy + i);
             const uint2 xr = *reinterpret_cast<const uint2*>(frow + off + i);
             const uint2 dr = *reinterpret_cast<const uint2*>(dy + i);
@@ -291,7 +291,7 @@ __global__ __launch_bounds__(256) void qkv_post_bwd_kernel(QkvPostBwdArgs a) {
               wk[V * j + e] += is_q ? 0.0f : t;
             }
           }
-          if (V == 4) {
+          if constexpr (V == 4) {
             *reinterpret_cast<uint2*>(orow + off + i) = make_uint2(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]));
           } else {
             orow[off + i] = (uint16_t)f32_to_bf16_bits(o[0]);

@@ -820,15 +820,108 @@ def grouped_forward(x: torch.Tensor, group_sizes: torch.Tensor, weight: PackedGr
     return (out, aux) if return_aux else out
 
 
+class GroupedBackwardPlan:
+    """Validated arguments, outputs, workspace and the C struct of one grouped backward call;
+    ``run()`` is a single C call on torch's current stream.  Nothing is read back to the host."""
+
+    def __init__(self, x: torch.Tensor | None, dy: torch.Tensor, group_sizes: torch.Tensor,
+                 weight: PackedGroupedW8Weight, lora_a=None, lora_b=None, lora_scaling=None, *,
+                 groups_per_weight: int = 1, need_lora_grads: bool = True):
+        if dy.ndim != 2 or dy.dtype != torch.bfloat16:
+            raise TypeError("dy must be a BF16 matrix [rows, N]")
+        _require_cuda(dy, "dy")
+        k, n = weight.in_features, weight.out_features
+        if dy.shape[1] != n or dy.shape[0] <= 0:
+            raise ValueError(f"dy must be [rows, {n}] with at least one row, got {tuple(dy.shape)}")
+        dev = dy.device
+        dyf = dy.contiguous()
+        m = dyf.shape[0]
+        gpw = int(groups_per_weight)
+        gs = group_sizes.to(device=dev, dtype=torch.int32).contiguous()
+        n_groups = gs.numel()
+        if gpw < 1 or n_groups != weight.n_weights * gpw:
+            raise ValueError(f"{n_groups} groups do not match {weight.n_weights} weights x {gpw}")
+        a3 = b3 = s1 = xf = None
+        r = 0
+        if lora_a is not None:
+            if lora_a.dtype != torch.bfloat16 or lora_b.dtype != torch.bfloat16:
+                raise TypeError("LoRA A and B must both be BF16")
+            if lora_a.ndim != 3 or lora_a.shape[0] != n_groups or lora_a.shape[1] != k:
+                raise ValueError(f"grouped lora_a must be [{n_groups}, {k}, r], got {tuple(lora_a.shape)}")
+            r = lora_a.shape[2]
+            if tuple(lora_b.shape) != (n_groups, r, n):
+                raise ValueError(f"grouped lora_b must be [{n_groups}, {r}, {n}], got {tuple(lora_b.shape)}")
+            if r < 1 or r > MAX_LORA_RANK:
+                raise ValueError(f"LoRA rank must be in [1, {MAX_LORA_RANK}], got {r}")
+            a3, b3 = lora_a.detach().contiguous(), lora_b.detach().contiguous()
+            s1 = torch.as_tensor(lora_scaling, dtype=torch.float32, device=dev).detach()
+            s1 = (s1.reshape(1).expand(n_groups) if s1.ndim == 0 else s1).contiguous()
+            if tuple(s1.shape) != (n_groups,):
+                raise ValueError(f"lora_scaling must be a scalar or have shape ({n_groups},)")
+        want = bool(r) and need_lora_grads
+        if want:
+            if x is None:
+                raise ValueError("x is needed for the LoRA cotangents")
+            if x.dtype != torch.bfloat16 or tuple(x.shape) != (m, k):
+                raise ValueError(f"x must be BF16 [{m}, {k}], got {x.dtype} {tuple(x.shape)}")
+            _require_cuda(x, "x")
+            xf = x.detach().contiguous()
+        lib = _native.load()
+        ws_bytes = int(lib.mi355_w8a8_grouped_bwd_workspace_bytes(m, k, n, n_groups, r, gpw))
+        if ws_bytes == 0:
+            raise ValueError(f"geometry M={m}, K={k}, N={n}, groups={n_groups}, rank={r} is outside the native backward")
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        self.dx = torch.empty((m, k), dtype=torch.bfloat16, device=dev)
+        self.d_lora_a = torch.empty((n_groups, k, r), dtype=torch.bfloat16, device=dev) if want else None
+        self.d_lora_b = torch.empty((n_groups, r, n), dtype=torch.bfloat16, device=dev) if want else None
+        self.d_lora_scaling = torch.empty((n_groups,), dtype=torch.float32, device=dev) if want else None
+        p = _native.GroupedBwdProblem()
+        p.struct_size = ctypes.sizeof(_native.GroupedBwdProblem)
+        p.m, p.k, p.n, p.n_groups, p.rank, p.groups_per_weight = m, k, n, n_groups, r, gpw
+        p.x = xf.data_ptr() if xf is not None else None
+        p.dy = dyf.data_ptr()
+        p.w_packed, p.w_scales = weight.packed.data_ptr(), weight.scales.data_ptr()
+        p.lora_a = a3.data_ptr() if r else None
+        p.lora_b = b3.data_ptr() if r else None
+        p.lora_scaling = s1.data_ptr() if r else None
+        p.group_sizes = gs.data_ptr()
+        p.dx = self.dx.data_ptr()
+        p.d_lora_a = self.d_lora_a.data_ptr() if want else None
+        p.d_lora_b = self.d_lora_b.data_ptr() if want else None
+        p.d_lora_scaling = self.d_lora_scaling.data_ptr() if want else None
+        p.workspace, p.workspace_bytes = ws.data_ptr(), ws_bytes
+        self.problem = p
+        self.device = dev
+        self.dims = {"m": m, "k": k, "n": n, "n_groups": n_groups, "rank": r}
+        self._fn = lib.mi355_w8a8_grouped_bwd_v1
+        self._keep = (xf, dyf, gs, weight, a3, b3, s1, ws)
+
+    def run(self):
+        """Enqueue the call; returns ``(dx, d_lora_a, d_lora_b, d_lora_scaling)`` (reused tensors)."""
+        with torch.cuda.device(self.device):
+            status = self._fn(ctypes.byref(self.problem), _stream_ptr(self.device))
+        _native.check("mi355_w8a8_grouped_bwd_v1", status)
+        return self.dx, self.d_lora_a, self.d_lora_b, self.d_lora_scaling
+
+
 def grouped_backward(x: torch.Tensor | None, dy: torch.Tensor, group_sizes: torch.Tensor,
                      weight: PackedGroupedW8Weight, lora_a=None, lora_b=None, lora_scaling=None, *,
                      groups_per_weight: int = 1, need_lora_grads: bool = True):
-    """Cotangents of ``grouped_forward`` (plain epilogue): ``(dx, d_lora_a, d_lora_b, d_lora_scaling)``.
+    """Cotangents of ``grouped_forward`` (plain epilogue): ``(dx, d_lora_a, d_lora_b, d_lora_scaling)``,
+    one native call for all groups (the derivative of ``LoRAExpert.__call__``, skyrl/tx/layers/lora.py:
+    394-444, under the rule of ``backward``).  Rows beyond ``sum(group_sizes)`` get a zero ``dx``;
+    groups without rows get zero cotangents."""
+    return GroupedBackwardPlan(x, dy, group_sizes, weight, lora_a, lora_b, lora_scaling,
+                               groups_per_weight=groups_per_weight, need_lora_grads=need_lora_grads).run()
 
-    One dense backward call per weight (expert) over its rows, the groups that share the weight
-    taking the role of adapters.  The group sizes are read on the host to cut the rows, which waits
-    for the stream once per call; rows beyond ``sum(group_sizes)`` get a zero ``dx``.
-    """
+
+def grouped_backward_per_weight(x: torch.Tensor | None, dy: torch.Tensor, group_sizes: torch.Tensor,
+                     weight: PackedGroupedW8Weight, lora_a=None, lora_b=None, lora_scaling=None, *,
+                     groups_per_weight: int = 1, need_lora_grads: bool = True):
+    """The same cotangents as ``grouped_backward`` from one dense backward call per weight (expert)
+    over its rows, the groups that share the weight taking the role of adapters.  The group sizes
+    are read on the host to cut the rows, which waits for the stream; kept as the statement of what
+    the single native call computes (the two agree bit for bit)."""
     if dy.ndim != 2 or dy.dtype != torch.bfloat16:
         raise TypeError("dy must be a BF16 matrix [rows, N]")
     _require_cuda(dy, "dy")
@@ -1506,7 +1599,8 @@ __all__ = (
     "prepare_weight", "unpack_weight", "dynamic_quantize_rows", "ForwardPlan", "forward", "BackwardPlan", "backward", "lora_linear",
     "w8a8_frozen_linear",
     "w8a8_lora_linear", "w8a8_rms_gate_up_lora_swiglu", "w8a8_lora_residual", "PackedGroupedW8Weight",
-    "prepare_grouped_weight", "grouped_forward", "grouped_backward", "grouped_lora_linear",
+    "prepare_grouped_weight", "grouped_forward", "grouped_backward", "grouped_backward_per_weight",
+    "GroupedBackwardPlan", "grouped_lora_linear",
     "w8a8_grouped_lora_linear", "w8a8_moe_expert_mlp", "Qwen35QKVStageConfig", "QkvPostPlan", "qkv_split_norm_rope",
     "w8a8_qkv_lora_rope", "qkv_lora_rope", "qkv_split_norm_rope_backward", "delta_rms_norm_backward", "QkvStageBackwardPlan",
 )
