@@ -53,6 +53,10 @@ WORKLOADS = {
     # combine; rank-16 LoRA on every expert
     "qwen3-30b-a3b-moe-mlp-t2048": dict(m=2048, n_experts=128, top_k=8, hidden=2048, intermediate=768, rank=16,
                                         seed=5, moe_mlp=True),
+    # backward of the two grouped expert projections of that layer (16384 sorted pairs over 128 experts): dx and the
+    # LoRA cotangents of gate/up [2048 -> 1536] and of down [768 -> 2048], one native call each
+    "qwen3-30b-a3b-moe-experts-t2048-backward": dict(m=2048, n_experts=128, top_k=8, hidden=2048, intermediate=768,
+                                                     rank=16, seed=5, moe_backward=True),
     # group-scaled W4A8 (int4 codes, one scale per 128 k and output, activations quantized per row and group)
     # at the Qwen3-8B down-projection shape, 8 adapters rank 32
     "qwen3-8b-down-m4096-w4a8-g128": dict(m=4096, k=12288, n=4096, n_adapters=8, rank=32, weight_bits=4,
@@ -516,6 +520,115 @@ def bench_moe_mlp(args, cfg, pkg, dev):
     return 0
 
 
+def bench_moe_backward(args, cfg, pkg, dev):
+    """One step = the backward of the two grouped expert projections (gate/up without SwiGLU, down) over
+    the sorted (token, choice) pairs: dx and dA, dB, dscaling for every expert, one native call per
+    projection.  ``value`` counts the pull-backs' 2 * P * (H * 2I + I * H); the roofline prices
+    bwd_dx_kernel of the gate/up call against the bf16 MFMA peak on the rows that exist (tiles are
+    padded to 256 slots per expert, which the figure charges to the kernel)."""
+    import torch
+
+    from oracle import w8a8_oracle as o
+
+    native, w8 = pkg._native, pkg.w8a8_lora
+    t, e, topk, h, inter, r = cfg["m"], cfg["n_experts"], cfg["top_k"], cfg["hidden"], cfg["intermediate"], cfg["rank"]
+    p_rows = t * topk
+    rng = np.random.default_rng(cfg["seed"])
+    logits = torch.from_numpy(rng.standard_normal((t, e)).astype(np.float32)).to(dev)
+    _, selected = w8.moe_route(logits, topk)
+    _, sizes, _, _, _ = w8.moe_dispatch(None, selected, e, repeat=topk)
+    gen = torch.Generator(device=dev).manual_seed(cfg["seed"])
+    rnd = lambda *shape, scale=1.0: (torch.randn(*shape, device=dev, generator=gen) * scale).to(torch.bfloat16)
+
+    def weight(k, n):
+        codes = torch.randint(-127, 128, (e, k, n), dtype=torch.int8, device=dev, generator=gen)
+        scales = torch.rand(e, n, device=dev, generator=gen) * 0.009 + 0.001
+        return w8.prepare_grouped_weight(codes, scales), codes, scales
+
+    guw, gu_codes, gu_scales = weight(h, 2 * inter)
+    dnw, _, _ = weight(inter, h)
+    x_gu, dy_gu = rnd(p_rows, h), rnd(p_rows, 2 * inter)
+    x_dn, dy_dn = rnd(p_rows, inter), rnd(p_rows, h)
+    gua, gub = rnd(e, h, r, scale=0.02), rnd(e, r, 2 * inter, scale=0.02)
+    dna, dnb = rnd(e, inter, r, scale=0.02), rnd(e, r, h, scale=0.02)
+    s = torch.ones(e, device=dev)
+    plan_gu = w8.GroupedBackwardPlan(x_gu, dy_gu, sizes, guw, gua, gub, s)
+    plan_dn = w8.GroupedBackwardPlan(x_dn, dy_dn, sizes, dnw, dna, dnb, s)
+
+    def step():
+        plan_gu.run()
+        plan_dn.run()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+
+    def timed(fn, reps=None):
+        reps = reps or args.steps
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+        for a, b in ev:
+            a.record()
+            fn()
+            b.record()
+        torch.cuda.synchronize()
+        return np.asarray([a.elapsed_time(b) for a, b in ev])
+
+    gu_ms, dn_ms = timed(plan_gu.run), timed(plan_dn.run)
+    dx_only = w8.GroupedBackwardPlan(None, dy_gu, sizes, guw, None, None, None)
+    dx_ms = timed(dx_only.run)
+    # the same cotangents from one dense call per expert (what the single call replaces)
+    loop_ms = timed(lambda: w8.grouped_backward_per_weight(x_gu, dy_gu, sizes, guw, gua, gub, s), reps=3)
+    flops = 2.0 * p_rows * (h * 2 * inter + inter * h)
+    gu_flops = 2.0 * p_rows * h * 2 * inter
+    achieved = gu_flops / (float(dx_ms.mean()) * 1e-3) / 1e12
+    result = {
+        "metric": "backward of the grouped W8A8-LoRA expert projections (dx + LoRA cotangents, gate/up and down), "
+                  "TFLOP/s of 2*P*K*N per call",
+        "value": flops / (ms_per_step * 1e-3) / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / BF16_PEAK_TFLOPS, "traffic": None,
+                     "kernel": "the gate/up call without LoRA (tables, bwd_pack_dy_kernel, bwd_dx_kernel)",
+                     "kernel_avg_ms": float(dx_ms.mean()), "kernel_min_ms": float(dx_ms.min()),
+                     "algorithmic_flops": gu_flops},
+        "stages": {"gate_up_call_ms": float(gu_ms.mean()), "down_call_ms": float(dn_ms.mean()),
+                   "gate_up_one_dense_call_per_expert_ms": float(loop_ms.mean())},
+    }
+    if not args.no_cpu_baseline:
+        n_exp = args.cpu_rows or 4     # experts of the sample
+        counts = sizes.cpu().numpy()
+        starts = np.concatenate(([0], np.cumsum(counts)))
+        sel = slice(0, int(starts[n_exp]))
+        xs, dys = (v[sel].to(torch.float32).cpu().numpy() for v in (x_gu, dy_gu))
+        a_np, b_np = (v[:n_exp].to(torch.float32).cpu().numpy() for v in (gua, gub))
+        codes_np, scales_np = gu_codes[:n_exp].cpu().numpy(), gu_scales[:n_exp].cpu().numpy()
+        t1 = time.perf_counter()
+        want = []
+        for i in range(n_exp):
+            w = o.GroupQuantizedWeight(codes_np[i], scales_np[i:i + 1], h, h, 8, h)
+            rows = slice(int(starts[i]), int(starts[i + 1]))
+            want.append(o.quantized_lora_linear_multi_bwd(xs[rows], w, a_np[i:i + 1], b_np[i:i + 1], np.ones(1, np.float32),
+                                                          np.zeros(rows.stop - rows.start, np.int64), dys[rows], True))
+        secs = time.perf_counter() - t1
+        done = int(starts[n_exp])
+        result["cpu_baseline"] = {"value": 2.0 * done * h * 2 * inter / secs / 1e12, "unit": "TFLOP/s", "cores": 1,
+                                  "kind": "port",
+                                  "sample": f"the first {n_exp} experts' {done} rows of the gate/up call, NumPy oracle "
+                                            f"backward per expert (float64 BLAS), one run, {secs:.3f} s", "seconds": secs}
+        got_dx = plan_gu.run()[0][sel].to(torch.float32).cpu().numpy()
+        gate = o.numerical_gate(got_dx, np.concatenate([w_[0] for w_ in want]))
+        result["parity_sample"] = {"rows": done, "relative_l2": gate["relative_l2"], "cosine": gate["cosine"]}
+    print(json.dumps(result))
+    return 0
+
+
 def bench_gq(args, cfg, pkg, dev):
     """One step = one group-scaled quantized linear call (quantizer, LoRA z, GEMM with the group
     epilogue).  ``value`` counts 2*M*K*N; the roofline prices gq_gemm_kernel against int8 MFMA peak from
@@ -840,6 +953,8 @@ def main() -> int:
         return bench_backward(args, cfg, pkg, dev)
     if cfg.pop("gq", False):
         return bench_gq(args, cfg, pkg, dev)
+    if cfg.pop("moe_backward", False):
+        return bench_moe_backward(args, cfg, pkg, dev)
     if cfg.pop("moe_mlp", False):
         return bench_moe_mlp(args, cfg, pkg, dev)
     if cfg.pop("moe_routing", False):

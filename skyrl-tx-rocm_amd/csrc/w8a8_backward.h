@@ -53,7 +53,7 @@ __global__ __launch_bounds__(256) void bwd_pack_dy_kernel(BwdPackDyArgs a) {
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
   const uint32_t mb = blockIdx.x / a.n_slices, sl = blockIdx.x % a.n_slices;
   if (mb >= a.n_row_blocks) return;
-  if (a.blk_range && a.blk_range[mb] < 0) return;  // block beyond the slots in use (grouped calls)
+  if (a.blk_range && a.blk_range[mb] < 0) return;  // block without rows (grouped calls): never consumed
   const uint32_t i = lane & 31u, h = lane >> 5;
   const uint32_t p = mb * 32u + i;
   int src = -1;
@@ -149,7 +149,7 @@ struct BwdRFinishArgs {
 __global__ __launch_bounds__(256) void bwd_r_finish_kernel(BwdRFinishArgs a) {
   __shared__ float zs[32][kBwdRankStride + 1];
   const uint32_t pb = blockIdx.x;
-  if (a.blk_range && a.blk_range[pb] < 0) return;  // block beyond the slots in use (grouped calls)
+  if (a.blk_range && a.blk_range[pb] < 0) return;  // block without rows (grouped calls): never consumed
   for (uint32_t q = threadIdx.x; q < 32u * a.cols; q += 256u) {
     const uint32_t row = q / a.cols, col = q % a.cols, slot = pb * 32u + row;
     float raw = 0.0f;
@@ -252,9 +252,10 @@ __global__ __launch_bounds__(1024) void bwd_prep_kernel(BwdPrepArgs p) {
 // (skyrl/tx/layers/lora.py:394-444).  Every weight's rows start at a multiple of 256 slots, so that
 // a pull-back tile never mixes two weights; inside a weight the groups follow each other without
 // gaps, exactly as the adapters of a dense call over that weight's rows would.
-//   src_row / dst_pos / slot_group / blk_range   as in the dense call (blk_range -1 beyond the slots in use)
+//   src_row / dst_pos / slot_group / blk_range   as in the dense call; blk_range -1 for 32-slot blocks without a
+//                                                row: no kernel prepares or consumes their operands
 //   group_beg[g], group_end[g]                   slots of group g
-//   tile_weight[t]                               weight of 256-slot tile t, -1 beyond the slots in use
+//   tile_weight[t]                               weight of 256-slot tile t | its rows << 16, -1 beyond the slots in use
 //   chunk_tab[c] = (group, first slot, rows)     the 512-row chunks of the LoRA cotangents; rows 0 beyond
 //   chunk0[g]                                    first chunk of group g (n_groups + 1 entries)
 // One workgroup of 1024 threads.  Rows beyond sum(group_sizes) get no slot; their dx rows are cleared.
@@ -271,7 +272,6 @@ __device__ inline void route_weight_groups_block(const int32_t* __restrict__ gro
   __shared__ int slot_beg[kMaxGroups + 1];
   __shared__ int slot_end[kMaxGroups];
   __shared__ int chunk_first[kMaxGroups + 1];
-  __shared__ int used_slots;
   const uint32_t tid = threadIdx.x;
   if (tid < n_groups) row_start[tid] = group_sizes[tid];  // sizes first, starts below
   __syncthreads();
@@ -293,7 +293,6 @@ __device__ inline void route_weight_groups_block(const int32_t* __restrict__ gro
     row_start[n_groups] = r;
     slot_beg[n_groups] = p;
     chunk_first[n_groups] = ch;
-    used_slots = (p + 255) & ~255;
   }
   for (uint32_t p = tid; p < slots; p += 1024) { t.src_row[p] = -1; t.slot_group[p] = 0; }
   for (uint32_t i = tid; i < M; i += 1024) t.dst_pos[i] = -1;
@@ -301,8 +300,7 @@ __device__ inline void route_weight_groups_block(const int32_t* __restrict__ gro
     t.chunk_tab[3u * c] = 0; t.chunk_tab[3u * c + 1u] = 0; t.chunk_tab[3u * c + 2u] = 0;
   }
   __syncthreads();
-  const int used = used_slots;
-  for (uint32_t b = tid; b < slots / 32u; b += 1024) t.blk_range[b] = (int)(b * 32u) < used ? 0 : -1;
+  for (uint32_t b = tid; b < slots / 32u; b += 1024) t.blk_range[b] = -1;
   for (uint32_t tl = tid; tl < slots / 256u; tl += 1024) t.tile_weight[tl] = -1;
   for (uint32_t g = tid; g <= n_groups; g += 1024) t.chunk0[g] = chunk_first[g];
   if (tid < n_groups) { t.group_beg[tid] = slot_beg[tid]; t.group_end[tid] = slot_end[tid]; }
@@ -334,16 +332,17 @@ __device__ inline void route_weight_groups_block(const int32_t* __restrict__ gro
     int glast = (int)g0;
     for (uint32_t g = g0; g < g1; ++g)
       if (slot_end[g] > slot_beg[g]) glast = (int)g;
-    for (int tl = wb / 256 + (int)lane; tl < wpad / 256; tl += 64) t.tile_weight[tl] = (int)w;
+    for (int tl = wb / 256 + (int)lane; tl < wpad / 256; tl += 64) {
+      const int rows = we - tl * 256 < 256 ? we - tl * 256 : 256;
+      t.tile_weight[tl] = (int)w | (rows << 16);
+    }
     for (int p = we + (int)lane; p < wpad; p += 64) t.slot_group[p] = glast;
-    for (int b = wb / 32 + (int)lane; b < wpad / 32; b += 64) {
+    for (int b = wb / 32 + (int)lane; b < (we + 31) / 32; b += 64) {  // blocks without a row stay at -1
       const int p0 = b * 32, p1 = p0 + 31 < we ? p0 + 31 : we - 1;
       int lo = glast, hi = glast;
-      if (p0 < we) {
-        for (uint32_t g = g0; g < g1; ++g) {
-          if (p0 >= slot_beg[g] && p0 < slot_end[g]) lo = (int)g;
-          if (p1 >= slot_beg[g] && p1 < slot_end[g]) hi = (int)g;
-        }
+      for (uint32_t g = g0; g < g1; ++g) {
+        if (p0 >= slot_beg[g] && p0 < slot_end[g]) lo = (int)g;
+        if (p1 >= slot_beg[g] && p1 < slot_end[g]) hi = (int)g;
       }
       t.blk_range[b] = lo | (hi << 16);
     }
@@ -418,8 +417,9 @@ struct BwdDxArgs {
   const int32_t* src_row; const int32_t* slot_group; const int32_t* blk_range;
   uint16_t* dx;               // bf16 [M, K]
   uint32_t M, K, KB, NB, tiles_m, tiles_k;
-  // grouped calls: the weight of every 256-slot tile (-1: tile without rows), the bytes between two
-  // packed weights and the floats between two scale tables; null / 0 for one weight
+  // grouped calls: weight | rows << 16 of every 256-slot tile (-1: tile without rows; the rows fill the
+  // tile from its first slot), the bytes between two packed weights and the floats between two scale
+  // tables; null / 0 for one weight
   const int32_t* tile_weight;
   size_t w_stride;
   uint32_t sw_stride;
@@ -444,20 +444,38 @@ __global__ __launch_bounds__(512, 1) void bwd_dx_kernel(BwdDxArgs g) {
   }
 
   const uint32_t ntile = g.tiles_m * g.tiles_k;
-  const uint32_t per_xcd = (ntile + 7u) / 8u, wgs_per_xcd = gridDim.x >> 3;
+  const uint32_t wgs_per_xcd = gridDim.x >> 3, xcd = blockIdx.x & 7u;
+  // band-major tile order: 4 row tiles x all k tiles, so an XCD's workgroups share panels.  One weight:
+  // every XCD walks a contiguous range of bands.  Grouped calls: the bands are dealt round-robin to the
+  // XCDs, because the slots in use end before the last bands and a contiguous split would leave the
+  // last XCDs without work.
+  const uint32_t band_tiles = 4u * g.tiles_k, n_bands = (g.tiles_m + 3u) / 4u;
+  const uint32_t per_xcd = g.tile_weight ? ((n_bands + 7u) / 8u) * band_tiles : (ntile + 7u) / 8u;
   for (uint32_t ti = blockIdx.x >> 3; ti < per_xcd; ti += wgs_per_xcd) {
-    const uint32_t t = (blockIdx.x & 7u) * per_xcd + ti;
-    if (t >= ntile) break;
-    // band-major tile order: 4 row tiles x all k tiles, so an XCD's workgroups share panels
-    const uint32_t band = t / (4u * g.tiles_k);
+    uint32_t band, in_band;
+    if (g.tile_weight) {
+      band = xcd + 8u * (ti / band_tiles);
+      in_band = ti % band_tiles;
+      if (band >= n_bands) break;
+    } else {
+      const uint32_t t = xcd * per_xcd + ti;
+      if (t >= ntile) break;
+      band = t / band_tiles;
+      in_band = t - band * band_tiles;
+    }
     const uint32_t band_rows = (g.tiles_m - band * 4u) < 4u ? (g.tiles_m - band * 4u) : 4u;
-    const uint32_t in_band = t - band * 4u * g.tiles_k;
+    if (in_band >= band_rows * g.tiles_k) continue;  // a last band with fewer than 4 row tiles (grouped order only)
     const uint32_t tm = band * 4u + in_band % band_rows, tk = in_band / band_rows;
     int tw = 0;
+    int n_act = 4;  // 32-row blocks of this wave that hold rows: the others skip their matrix-core work
     if (g.tile_weight) {
-      tw = g.tile_weight[tm];
-      if (tw < 0) continue;  // workgroup-uniform: no row lives in this tile
+      const int tv = g.tile_weight[tm];
+      if (tv < 0) continue;  // workgroup-uniform: no row lives in this tile
+      tw = tv & 0xffff;
+      const int live = ((tv >> 16) + 31) / 32 - wrow * 4;
+      n_act = live < 0 ? 0 : (live > 4 ? 4 : live);
     }
+    n_act = __builtin_amdgcn_readfirstlane(n_act);
     const float* swp_t = g.swp + (size_t)tw * g.sw_stride;
 
     // this wave's two panel chunks of a stage (row block = wave, halves q = 0, 1) and its weight block
@@ -536,6 +554,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dx_kernel(BwdDxArgs g) {
     // One stage: 16 MFMAs of stage nb against the dy panel in LDS; between them the operands of
     // stage nb + 1 are prepared (vector ALU work under the matrix core's shadow).
     auto stage = [&](int nb, const v8bf (&bqC)[2][2], v8bf (&bqN)[2][2], bool convert_next) {
+      if (n_act == 0) return;  // wave-uniform: a wave without rows only feeds the pipeline
       NextRegs nx;
       v16i tr;
       uint32_t pk[8];
@@ -546,8 +565,10 @@ __global__ __launch_bounds__(512, 1) void bwd_dx_kernel(BwdDxArgs g) {
         const int q = pair >> 2, rb = pair & 3;
         v8bf af_next = af;
         if (pair < 7) af_next = panel_frag(nb, pair + 1);
-        acc[rb][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bqC[0][q], acc[rb][0], 0, 0, 0);
-        acc[rb][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bqC[1][q], acc[rb][1], 0, 0, 0);
+        if (rb < n_act) {
+          acc[rb][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bqC[0][q], acc[rb][0], 0, 0, 0);
+          acc[rb][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bqC[1][q], acc[rb][1], 0, 0, 0);
+        }
         if (convert_next) {
           if (pair == 0) {
             next_wait(nx);
@@ -578,7 +599,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dx_kernel(BwdDxArgs g) {
     for (int i = 0; i < kBwdAhead; ++i) issue(i);  // NB >= 8
     wait_vmcnt<0>();
     lds_barrier();
-    {  // operands of stage 0
+    if (n_act > 0) {  // operands of stage 0
       NextRegs nx;
       next_read(0, nx);
       next_wait(nx);
