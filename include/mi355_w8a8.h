@@ -437,6 +437,19 @@ int mi355_w8a8_moe_combine_v1(const void* expert_out, const int32_t* unsort_indi
                               uint32_t n_tokens, uint32_t top_k, uint32_t width, void* stream);
 
 /*
+ * Pull-back of the combine (the derivative of qwen3.py:205-207 in its two operands): for the sorted
+ * row at position pos with pair = sort_indices[pos],
+ *   d_expert_out[pos] = bf16(f32(d_out[pair / top_k]) * weights[pair])
+ *   d_weights[pair]   = sum_c f32(expert_out[pos, c]) * f32(d_out[pair / top_k, c])   (float32)
+ * d_out bf16 [n_tokens, width]; expert_out, d_expert_out bf16 [n_tokens * top_k, width] in sorted order;
+ * d_weights f32 [n_tokens, top_k] or NULL (then expert_out may be NULL too).  The cotangent of the hidden
+ * rows through the gather of the dispatch is mi355_w8a8_moe_combine_v1 with unit weights.
+ */
+int mi355_w8a8_moe_combine_bwd_v1(const void* d_out, const void* expert_out, const int32_t* sort_indices,
+                                  const float* weights, void* d_expert_out, float* d_weights, uint32_t n_tokens,
+                                  uint32_t top_k, uint32_t width, void* stream);
+
+/*
  * Group-scaled quantized linear: the general form of quantized_frozen_linear / quantized_lora_linear
  * (skyrl/tx/kernels/quantized_lora.py:215-304) -- W4 or W8 codes with one scale per (K group, output),
  * A4 or A8 activations quantized per (row, K group):

@@ -46,6 +46,9 @@ How each function is pinned (the tests that do it live in ``tests/test_oracle_*.
   the re-interleave as the exact adjoint of the split (enumerated), and the composite against
   autograd through the whole smooth stage on bf16-exact inputs.  PARITY UNPINNED in the last
   float32 bits of XLA's reductions, rsqrt, sin, cos and pow.
+* ``moe_combine_bwd``/``moe_route_bwd``/``moe_expert_mlp_bwd``: ``torch.autograd`` (float64, CPU) through
+  the gather-weighted sum, through softmax / gather / renormalise with the selection held fixed, and
+  through the whole smooth expert MLP on bf16-exact inputs; zero and linearity identities.
 * ``moe_route``/``moe_combine``/``moe_expert_mlp``: ``torch.topk``/``scipy.special.softmax`` special
   cases and the merged-weight invariant of tests/tx/models/test_qwen3.py:123-180.
 """
@@ -923,6 +926,84 @@ def moe_expert_mlp(hidden, router_logits, top_k, gate_up_weights, down_weights,
                      "fused": fused, "act": act, "down": down, "weights": weights,
                      "selected": selected}
     return out
+
+
+# ---------------------------------------------------------------------------
+# pull-back of the expert MLP: the derivative of qwen3.py:172-210, written out
+# ---------------------------------------------------------------------------
+
+def moe_combine_bwd(d_out, expert_out, unsort, weights):
+    """Cotangents of ``moe_combine`` in its two operands: d_expert_out[unsort[t k + j]] =
+    bf16(d_out[t] * w[t, j]) and d_w[t, j] = sum_c expert_out[unsort[t k + j], c] * d_out[t, c]
+    (float32 products, summed in float64 and rounded once)."""
+    d_out = np.asarray(d_out, dtype=F32)
+    expert_out = np.asarray(expert_out, dtype=F32)
+    w = np.asarray(weights, dtype=F32)
+    t, k = w.shape
+    rows = np.asarray(unsort).reshape(t, k)
+    d_expert = np.zeros_like(expert_out)
+    d_w = np.zeros_like(w)
+    for j in range(k):
+        d_expert[rows[:, j]] = bf16_round((d_out * w[:, j:j + 1]).astype(F32))
+        d_w[:, j] = np.sum((expert_out[rows[:, j]] * d_out).astype(F32).astype(np.float64), axis=1).astype(F32)
+    return d_expert, d_w
+
+
+def moe_route_bwd(router_logits, selected, d_weights, norm_topk_prob: bool = True) -> np.ndarray:
+    """Cotangent of the router logits through softmax -> (fixed) top-k selection -> renormalisation
+    (qwen3.py:175-178), float64 inside, float32 out."""
+    logits = np.asarray(router_logits, dtype=np.float64)
+    sel = np.asarray(selected)
+    dw = np.asarray(d_weights, dtype=np.float64)
+    z = logits - logits.max(axis=-1, keepdims=True)
+    p = np.exp(z)
+    p /= p.sum(axis=-1, keepdims=True)
+    ps = np.take_along_axis(p, sel, axis=1)
+    if norm_topk_prob:
+        tot = ps.sum(axis=-1, keepdims=True)
+        w = ps / tot
+        dps = (dw - np.sum(dw * w, axis=-1, keepdims=True)) / tot
+    else:
+        dps = dw
+    dp = np.zeros_like(p)
+    np.put_along_axis(dp, sel, dps, axis=1)
+    return (p * (dp - np.sum(p * dp, axis=-1, keepdims=True))).astype(F32)
+
+
+def moe_expert_mlp_bwd(hidden, router_logits, top_k, gate_up_weights, down_weights, gate_up_a, gate_up_b,
+                       down_a, down_b, scaling, d_out, relaxed_weight: bool = True):
+    """Cotangents of ``moe_expert_mlp``: the chain combine -> grouped down -> SwiGLU -> grouped gate/up ->
+    gather written backwards, every grouped projection under ``quantized_lora_linear_bwd`` per expert,
+    every stage boundary one bf16 cast, the scatter-add of the gather summed in float32 in choice
+    order.  ``scaling`` is one float32 scalar shared by all experts and both projections.  Returns a
+    dict: d_hidden, d_router_logits, d_gate_up_a/b, d_down_a/b, d_scaling."""
+    hidden = np.asarray(hidden, dtype=F32)
+    _, st = moe_expert_mlp(hidden, router_logits, top_k, gate_up_weights, down_weights, gate_up_a, gate_up_b,
+                           down_a, down_b, scaling, return_stages=True)
+    sizes, unsort = st["group_sizes"], st["unsort"]
+    d_down, d_w = moe_combine_bwd(d_out, st["down"], unsort, st["weights"])
+    starts = np.concatenate(([0], np.cumsum(sizes)))
+
+    def grouped_bwd(x, dy, weights, a, b):
+        dx = np.zeros_like(x)
+        da, db = np.zeros_like(a), np.zeros_like(b)
+        ds = F32(0.0)
+        for e, w in enumerate(weights):
+            r0, r1 = int(starts[e]), int(starts[e + 1])
+            if r1 > r0:
+                dx[r0:r1], da[e], db[e], dse = quantized_lora_linear_bwd(x[r0:r1], w, a[e], b[e], scaling, dy[r0:r1],
+                                                                         relaxed_weight)
+                ds = F32(ds + F32(dse))
+        return dx, da, db, ds
+
+    d_act, d_da, d_db, ds_dn = grouped_bwd(st["act"], d_down, down_weights, np.asarray(down_a, F32), np.asarray(down_b, F32))
+    d_fused = swiglu_pullback_interleaved(st["fused"], d_act)
+    d_xs, d_ga, d_gb, ds_gu = grouped_bwd(st["x_sorted"], d_fused, gate_up_weights, np.asarray(gate_up_a, F32),
+                                          np.asarray(gate_up_b, F32))
+    d_hidden = moe_combine(d_xs, unsort, np.ones_like(st["weights"]))
+    return {"d_hidden": d_hidden, "d_router_logits": moe_route_bwd(router_logits, st["selected"], d_w),
+            "d_weights": d_w, "d_gate_up_a": d_ga, "d_gate_up_b": d_gb, "d_down_a": d_da, "d_down_b": d_db,
+            "d_scaling": F32(ds_dn + ds_gu), "d_down": d_down, "d_act": d_act, "d_fused": d_fused, "stages": st}
 
 
 # ---------------------------------------------------------------------------

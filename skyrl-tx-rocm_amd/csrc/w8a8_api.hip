@@ -1444,6 +1444,33 @@ int run_moe_combine(const void* expert_out, const int32_t* unsort, const float* 
   return launch_status();
 }
 
+int run_moe_combine_bwd(const void* d_out, const void* expert_out, const int32_t* sort, const float* weights,
+                        void* d_expert_out, float* d_weights, uint32_t t, uint32_t top_k, uint32_t width, hipStream_t s) {
+  if (!d_out || !sort || !weights || !d_expert_out) return MI355_W8A8_ERR_NULL;
+  if (d_weights && !expert_out) return MI355_W8A8_ERR_NULL;
+  if (t == 0 || top_k == 0 || width == 0 || (width & 7u)) return MI355_W8A8_ERR_SHAPE;
+  if (top_k > kMoeMaxTopK || t > kMaxRows || (uint64_t)t * top_k > (1ull << 30)) return MI355_W8A8_ERR_UNSUPPORTED;
+  if (!aligned16(d_out) || !aligned16(expert_out) || !aligned16(d_expert_out)) return MI355_W8A8_ERR_ALIGN;
+  if ((reinterpret_cast<uintptr_t>(sort) | reinterpret_cast<uintptr_t>(weights) | reinterpret_cast<uintptr_t>(d_weights)) & 3u)
+    return MI355_W8A8_ERR_ALIGN;
+  const uint64_t tok_bytes = (uint64_t)t * width * 2u, pair_bytes = tok_bytes * top_k, tab_bytes = (uint64_t)t * top_k * 4u;
+  if (overlaps(d_expert_out, pair_bytes, d_out, tok_bytes) || overlaps(d_expert_out, pair_bytes, expert_out, pair_bytes) ||
+      overlaps(d_expert_out, pair_bytes, sort, tab_bytes) || overlaps(d_expert_out, pair_bytes, weights, tab_bytes) ||
+      overlaps(d_weights, tab_bytes, weights, tab_bytes) || overlaps(d_weights, tab_bytes, d_expert_out, pair_bytes) ||
+      overlaps(d_weights, tab_bytes, sort, tab_bytes))
+    return MI355_W8A8_ERR_ALIAS;
+  MoeCombineBwdArgs a{};
+  a.d_out = static_cast<const uint16_t*>(d_out);
+  a.expert_out = d_weights ? static_cast<const uint16_t*>(expert_out) : nullptr;
+  a.sort = sort; a.weights = weights;
+  a.d_expert_out = static_cast<uint16_t*>(d_expert_out);
+  a.d_weights = d_weights;
+  a.P = t * top_k; a.top_k = top_k; a.width = width;
+  (void)hipGetLastError();
+  hipLaunchKernelGGL(moe_combine_bwd_kernel, dim3((a.P + 7u) / 8u), dim3(256), 0, s, a);
+  return launch_status();
+}
+
 constexpr uint32_t kGqZSlices = 32;
 struct GqLayout { uint64_t codes, scales, z, src_row, dst_pos, slot_group, blk_range, at, total; uint32_t m_pad, G; };
 
@@ -1806,6 +1833,13 @@ int mi355_w8a8_moe_combine_v1(const void* expert_out, const int32_t* unsort_indi
                               uint32_t n_tokens, uint32_t top_k, uint32_t width, void* stream) {
   return run_moe_combine(expert_out, unsort_indices, weights, out, n_tokens, top_k, width,
                          static_cast<hipStream_t>(stream));
+}
+
+int mi355_w8a8_moe_combine_bwd_v1(const void* d_out, const void* expert_out, const int32_t* sort_indices,
+                                  const float* weights, void* d_expert_out, float* d_weights, uint32_t n_tokens,
+                                  uint32_t top_k, uint32_t width, void* stream) {
+  return run_moe_combine_bwd(d_out, expert_out, sort_indices, weights, d_expert_out, d_weights, n_tokens, top_k, width,
+                             static_cast<hipStream_t>(stream));
 }
 
 uint64_t mi355_w8a8_gq_packed_weight_bytes(uint32_t k_pad, uint32_t n, uint32_t weight_bits) {

@@ -9,6 +9,7 @@
 //   moe_scatter_kernel         per chunk: stable position of every pair, the index arrays
 //   moe_gather_kernel          a wave per sorted row: the token rows copied to their positions
 //   moe_combine_kernel         one workgroup per token: sum_j expert_out[unsort[t k + j]] * w[t, j]
+//   moe_combine_bwd_kernel     a wave per sorted row: the cotangents of expert_out and of w
 #pragma once
 #include "w8a8_device.h"
 
@@ -236,6 +237,62 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(MoeCombineArgs a) {
     *reinterpret_cast<uint4*>(a.out + (size_t)t * a.width + c) =
         make_uint4(pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3]), pack_bf16x2(acc[4], acc[5]),
                    pack_bf16x2(acc[6], acc[7]));
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Pull-back of the combine: for the sorted row at position pos, with pair = sort[pos] (token
+// pair / top_k, weight w[pair]):
+//   d_expert_out[pos] = bf16(f32(d_out[token]) * w[pair])
+//   d_weights[pair]   = sum_c f32(expert_out[pos, c]) * f32(d_out[token, c])      (float32)
+// the derivative of out[t] = sum_j expert_out[unsort[t k + j]] * w[t, j] (qwen3.py:205-207).  A wave
+// per sorted row; the dot product is summed per lane, then across the wave.
+struct MoeCombineBwdArgs {
+  const uint16_t* d_out;       // bf16 [T, width]
+  const uint16_t* expert_out;  // bf16 [P, width] in sorted order, or null (no weight cotangent)
+  const int32_t* sort;         // int32 [P]
+  const float* weights;        // f32 [T, top_k]
+  uint16_t* d_expert_out;      // bf16 [P, width]
+  float* d_weights;            // f32 [T, top_k] or null
+  uint32_t P, top_k, width;
+};
+
+__global__ __launch_bounds__(256) void moe_combine_bwd_kernel(MoeCombineBwdArgs a) {
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (uint32_t u = 0; u < 2; ++u) {
+    const uint32_t pos = blockIdx.x * 8u + wave * 2u + u;
+    if (pos >= a.P) return;
+    const uint32_t pair = (uint32_t)a.sort[pos];
+    const float w = a.weights[pair];
+    const uint16_t* src = a.d_out + (size_t)(pair / a.top_k) * a.width;
+    const uint16_t* eo = a.expert_out ? a.expert_out + (size_t)pos * a.width : nullptr;
+    uint16_t* out = a.d_expert_out + (size_t)pos * a.width;
+    float dot = 0.0f;
+    for (uint32_t c = lane * 8u; c < a.width; c += 512u) {
+      const uint4 raw = *reinterpret_cast<const uint4*>(src + c);
+      const uint32_t rw[4] = {raw.x, raw.y, raw.z, raw.w};
+      uint32_t ew[4] = {0, 0, 0, 0};
+      if (eo) {
+        const uint4 er = *reinterpret_cast<const uint4*>(eo + c);
+        ew[0] = er.x; ew[1] = er.y; ew[2] = er.z; ew[3] = er.w;
+      }
+      float o[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float d = (e & 1) ? __uint_as_float(rw[e >> 1] & 0xffff0000u) : __uint_as_float(rw[e >> 1] << 16);
+        const float x = (e & 1) ? __uint_as_float(ew[e >> 1] & 0xffff0000u) : __uint_as_float(ew[e >> 1] << 16);
+        o[e] = d * w;
+        dot += x * d;
+      }
+      *reinterpret_cast<uint4*>(out + c) =
+          make_uint4(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]), pack_bf16x2(o[4], o[5]), pack_bf16x2(o[6], o[7]));
+    }
+    if (a.d_weights) {
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off);
+      if (lane == 0) a.d_weights[pair] = dot;
+    }
   }
 }
 

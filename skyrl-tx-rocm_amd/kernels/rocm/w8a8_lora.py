@@ -1129,22 +1129,134 @@ def moe_combine(expert_out: torch.Tensor, unsort_indices: torch.Tensor, weights:
     return out
 
 
+def moe_combine_backward(d_out: torch.Tensor, expert_out: torch.Tensor | None, sort_indices: torch.Tensor,
+                         weights: torch.Tensor, *, need_weight_grads: bool = True):
+    """Pull-back of ``moe_combine``: ``d_expert_out[pos] = bf16(d_out[pair // top_k] * w[pair])`` and
+    ``d_weights[pair] = <expert_out[pos], d_out[pair // top_k]>`` in float32, with
+    ``pair = sort_indices[pos]`` (the derivative of qwen3.py:205-207).  Returns
+    ``(d_expert_out, d_weights)``; the second is None unless asked for."""
+    if d_out.dtype != torch.bfloat16:
+        raise TypeError(f"d_out must be BF16, got {d_out.dtype}")
+    _require_cuda(d_out, "d_out")
+    if weights.ndim != 2 or d_out.ndim != 2 or d_out.shape[0] != weights.shape[0] or d_out.shape[1] % 8:
+        raise ValueError(f"need d_out [T, H] with H % 8 == 0 and weights [T, top_k], got {tuple(d_out.shape)} and "
+                         f"{tuple(weights.shape)}")
+    t, top_k = weights.shape
+    width = d_out.shape[1]
+    if sort_indices.numel() != t * top_k:
+        raise ValueError("sort_indices must have one entry per (token, choice)")
+    dev = d_out.device
+    do = d_out.contiguous()
+    so = sort_indices.reshape(-1).to(device=dev, dtype=torch.int32).contiguous()
+    w = weights.detach().to(device=dev, dtype=torch.float32).contiguous()
+    eo = None
+    if need_weight_grads:
+        if expert_out is None or expert_out.dtype != torch.bfloat16 or tuple(expert_out.shape) != (t * top_k, width):
+            raise ValueError(f"the weight cotangent needs expert_out BF16 [{t * top_k}, {width}]")
+        eo = expert_out.contiguous()
+    d_eo = torch.empty((t * top_k, width), dtype=torch.bfloat16, device=dev)
+    d_w = torch.empty((t, top_k), dtype=torch.float32, device=dev) if need_weight_grads else None
+    with torch.cuda.device(dev):
+        status = _native.load().mi355_w8a8_moe_combine_bwd_v1(
+            do.data_ptr(), eo.data_ptr() if eo is not None else None, so.data_ptr(), w.data_ptr(), d_eo.data_ptr(),
+            d_w.data_ptr() if d_w is not None else None, t, top_k, width, _stream_ptr(dev))
+    _native.check("mi355_w8a8_moe_combine_bwd_v1", status)
+    return d_eo, d_w
+
+
+class _MoeExpertMlpFunction(torch.autograd.Function):
+    """The expert MLP behind the routing, differentiable in the hidden rows, the routing weights and
+    the four LoRA factors: the chain of the forward written backwards (combine pull-back, grouped
+    backward of the down projection, SwiGLU pull-back, grouped backward of gate/up, scatter-add of the
+    gather as a combine with unit weights).  The forward keeps the gate/up projection, the activated
+    rows and the down projection."""
+
+    @staticmethod
+    def forward(ctx, hidden, weights, gate_up_a, gate_up_b, down_a, down_b, lora_scaling, selected, gate_up_weight,
+                down_weight, top_k):
+        n_experts = gate_up_weight.n_weights
+        _, group_sizes, sort_indices, unsort, _ = moe_dispatch(None, selected, n_experts, repeat=top_k)
+        fused = grouped_forward(hidden, group_sizes, gate_up_weight, gate_up_a, gate_up_b, lora_scaling,
+                                row_map=sort_indices, row_repeat=top_k)
+        act = swiglu(fused)
+        down = grouped_forward(act, group_sizes, down_weight, down_a, down_b, lora_scaling)
+        ctx.save_for_backward(hidden, weights, gate_up_a, gate_up_b, down_a, down_b, lora_scaling, group_sizes,
+                              sort_indices, unsort, fused, act, down)
+        ctx.gate_up_weight, ctx.down_weight, ctx.top_k, ctx.selected = gate_up_weight, down_weight, top_k, selected
+        return moe_combine(down, unsort, weights)
+
+    @staticmethod
+    def backward(ctx, d_out):
+        (hidden, weights, gate_up_a, gate_up_b, down_a, down_b, lora_scaling, group_sizes, sort_indices, unsort, fused,
+         act, down) = ctx.saved_tensors
+        top_k = ctx.top_k
+        lora = gate_up_a is not None
+        need_lora = lora and any(ctx.needs_input_grad[2:7])
+        need_w = ctx.needs_input_grad[1]
+        d_down, d_w = moe_combine_backward(d_out.contiguous(), down if need_w else None, sort_indices, weights,
+                                           need_weight_grads=need_w)
+        d_act, d_da, d_db, ds_dn = grouped_backward(act, d_down, group_sizes, ctx.down_weight, down_a, down_b,
+                                                    lora_scaling, need_lora_grads=need_lora)
+        d_fused = swiglu_backward(fused, d_act)
+        x_sorted = None
+        if need_lora:  # the LoRA cotangents of gate/up contract over the sorted hidden rows
+            x_sorted = moe_dispatch(hidden, ctx.selected, ctx.gate_up_weight.n_weights, repeat=top_k)[0]
+        d_xs, d_ga, d_gb, ds_gu = grouped_backward(x_sorted, d_fused, group_sizes, ctx.gate_up_weight, gate_up_a,
+                                                   gate_up_b, lora_scaling, need_lora_grads=need_lora)
+        d_hidden = None
+        if ctx.needs_input_grad[0]:
+            d_hidden = moe_combine(d_xs, unsort, torch.ones_like(weights))
+        d_s = None
+        if need_lora and ctx.needs_input_grad[6]:
+            d_s = ds_dn + ds_gu
+            d_s = d_s.reshape(lora_scaling.shape).to(lora_scaling.dtype) if lora_scaling.ndim else d_s.sum().to(lora_scaling.dtype)
+        if not need_lora:
+            d_ga = d_gb = d_da = d_db = None
+        return d_hidden, d_w, d_ga, d_gb, d_da, d_db, d_s, None, None, None, None
+
+
+def moe_expert_mlp(hidden, router_logits, top_k: int, gate_up_weight, down_weight, gate_up_a=None, gate_up_b=None,
+                   down_a=None, down_b=None, lora_scaling=None, *, norm_topk_prob: bool = True):
+    """Expert MLP of ``Qwen3Experts.__call__`` (skyrl/tx/models/qwen3.py:172-210) on W8A8 weights.
+    Without gradients: five native calls (route, dispatch of indices, grouped gate/up + SwiGLU reading
+    the hidden rows through the sort order, grouped down, combine).  Under autograd the same values
+    come from the projection without the fused SwiGLU plus the stand-alone SwiGLU kernel, and the call
+    is differentiable in ``hidden``, ``router_logits`` (through the routing weights, the selection
+    held fixed as ``lax.top_k`` does) and the LoRA factors and scaling."""
+    n_experts = gate_up_weight.n_weights
+    h2 = hidden.reshape(-1, hidden.shape[-1])
+    weights, selected = moe_route(router_logits, top_k, norm_topk_prob)
+    tensors = [t for t in (hidden, router_logits, gate_up_a, gate_up_b, down_a, down_b, lora_scaling)
+               if isinstance(t, torch.Tensor)]
+    if not (torch.is_grad_enabled() and any(t.requires_grad for t in tensors)):
+        # indices only: the first projection gathers the hidden rows itself through the sort order
+        _, group_sizes, sort_indices, unsort, _ = moe_dispatch(None, selected, n_experts, repeat=top_k)
+        act = grouped_forward(h2, group_sizes, gate_up_weight, gate_up_a, gate_up_b, lora_scaling, swiglu=True,
+                              row_map=sort_indices, row_repeat=top_k)
+        down = grouped_forward(act, group_sizes, down_weight, down_a, down_b, lora_scaling)
+        return moe_combine(down, unsort, weights).reshape(hidden.shape)
+    if router_logits.requires_grad:
+        # the routing weights as a differentiable function of the logits with the native selection:
+        # the values are the native ones, the derivative that of softmax -> gather -> renormalise
+        probs = torch.softmax(router_logits.reshape(-1, router_logits.shape[-1]).to(torch.float32), dim=-1)
+        picked = probs.gather(1, selected.to(torch.int64))
+        if norm_topk_prob:
+            picked = picked / picked.sum(dim=-1, keepdim=True)
+        weights = picked + (weights - picked).detach()
+    scaling = lora_scaling
+    if gate_up_a is not None and not isinstance(scaling, torch.Tensor):
+        scaling = torch.as_tensor(scaling, dtype=torch.float32, device=hidden.device)
+    out = _MoeExpertMlpFunction.apply(h2, weights, gate_up_a, gate_up_b, down_a, down_b, scaling, selected,
+                                      gate_up_weight, down_weight, top_k)
+    return out.reshape(hidden.shape)
+
+
 def w8a8_moe_expert_mlp(hidden, router_logits, top_k: int, gate_up_weight, down_weight, gate_up_a, gate_up_b,
                         down_a, down_b, lora_scaling, *, enabled: bool = False, norm_topk_prob: bool = True):
-    """Expert MLP of ``Qwen3Experts.__call__`` (skyrl/tx/models/qwen3.py:172-210) on W8A8 weights:
-    softmax -> top-k -> renormalise -> sort rows by expert -> grouped gate/up + SwiGLU -> grouped
-    down -> unsort -> weighted sum.  Five native calls on one stream, no host round trip: route,
-    dispatch (indices only), the two grouped GEMMs (the first reads the hidden rows through the sort
-    order), combine."""
+    """``moe_expert_mlp`` behind the reference's opt-in switch."""
     _check_enabled(enabled, False, "MoE expert MLP")
-    n_experts = gate_up_weight.n_weights
-    weights, selected = moe_route(router_logits, top_k, norm_topk_prob)
-    # indices only: the first projection gathers the hidden rows itself through the sort order
-    _, group_sizes, sort_indices, unsort, _ = moe_dispatch(None, selected, n_experts, repeat=top_k)
-    act = grouped_forward(hidden.reshape(-1, hidden.shape[-1]), group_sizes, gate_up_weight, gate_up_a, gate_up_b,
-                          lora_scaling, swiglu=True, row_map=sort_indices, row_repeat=top_k)
-    down = grouped_forward(act, group_sizes, down_weight, down_a, down_b, lora_scaling)
-    return moe_combine(down, unsort, weights)
+    return moe_expert_mlp(hidden, router_logits, top_k, gate_up_weight, down_weight, gate_up_a, gate_up_b, down_a,
+                          down_b, lora_scaling, norm_topk_prob=norm_topk_prob)
 
 
 def _check_enabled(enabled, interpret, what: str) -> None:
@@ -1601,6 +1713,6 @@ __all__ = (
     "w8a8_lora_linear", "w8a8_rms_gate_up_lora_swiglu", "w8a8_lora_residual", "PackedGroupedW8Weight",
     "prepare_grouped_weight", "grouped_forward", "grouped_backward", "grouped_backward_per_weight",
     "GroupedBackwardPlan", "grouped_lora_linear",
-    "w8a8_grouped_lora_linear", "w8a8_moe_expert_mlp", "Qwen35QKVStageConfig", "QkvPostPlan", "qkv_split_norm_rope",
+    "w8a8_grouped_lora_linear", "w8a8_moe_expert_mlp", "moe_expert_mlp", "moe_combine_backward", "Qwen35QKVStageConfig", "QkvPostPlan", "qkv_split_norm_rope",
     "w8a8_qkv_lora_rope", "qkv_lora_rope", "qkv_split_norm_rope_backward", "delta_rms_norm_backward", "QkvStageBackwardPlan",
 )
