@@ -583,6 +583,23 @@ def bench_moe_backward(args, cfg, pkg, dev):
     dx_ms = timed(dx_only.run)
     # the same cotangents from one dense call per expert (what the single call replaces)
     loop_ms = timed(lambda: w8.grouped_backward_per_weight(x_gu, dy_gu, sizes, guw, gua, gub, s), reps=3)
+    # the whole layer through autograd: training forward (projection kept, separate SwiGLU) and its backward
+    hid = rnd(t, h).requires_grad_(True)
+    params = [v.clone().requires_grad_(True) for v in (gua, gub, dna, dnb)]
+    d_hid = rnd(t, h)
+
+    def train_step():
+        out = w8.moe_expert_mlp(hid, logits, topk, guw, dnw, *params, 1.0)
+        out.backward(d_hid)
+
+    for _ in range(3):
+        train_step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    for _ in range(10):
+        train_step()
+    torch.cuda.synchronize()
+    layer_ms = (time.perf_counter() - t1) / 10 * 1e3
     flops = 2.0 * p_rows * (h * 2 * inter + inter * h)
     gu_flops = 2.0 * p_rows * h * 2 * inter
     achieved = gu_flops / (float(dx_ms.mean()) * 1e-3) / 1e12
@@ -599,7 +616,8 @@ def bench_moe_backward(args, cfg, pkg, dev):
                      "kernel_avg_ms": float(dx_ms.mean()), "kernel_min_ms": float(dx_ms.min()),
                      "algorithmic_flops": gu_flops},
         "stages": {"gate_up_call_ms": float(gu_ms.mean()), "down_call_ms": float(dn_ms.mean()),
-                   "gate_up_one_dense_call_per_expert_ms": float(loop_ms.mean())},
+                   "gate_up_one_dense_call_per_expert_ms": float(loop_ms.mean()),
+                   "expert_mlp_forward_and_backward_through_autograd_ms": layer_ms},
     }
     if not args.no_cpu_baseline:
         n_exp = args.cpu_rows or 4     # experts of the sample
