@@ -893,6 +893,7 @@ class GroupedBackwardPlan:
         self.problem = p
         self.device = dev
         self.dims = {"m": m, "k": k, "n": n, "n_groups": n_groups, "rank": r}
+        self.group_sizes = gs   # the int32 tensor the call reads: rewrite it in place to route the next run differently
         self._fn = lib.mi355_w8a8_grouped_bwd_v1
         self._keep = (xf, dyf, gs, weight, a3, b3, s1, ws)
 

@@ -133,3 +133,31 @@ def test_qkv_stage_backward_plan_replays(dev, pkg):
             c.copy_(torch.randn(c.shape, device=dev, generator=gen).to(torch.bfloat16))
 
     _replays(torch, plan.run, lambda: list(outs), refresh, n=3)
+
+
+def test_grouped_backward_plan_replays(dev, pkg):
+    import torch
+
+    w8 = pkg.w8a8_lora
+    e, k, n, r = 6, 256, 384, 8
+    sizes = [40, 0, 300, 7, 129, 64]
+    m = sum(sizes) + 3
+    print(f"[case] graph grouped backward groups={e} m={m} k={k} n={n}", flush=True)
+    codes = torch.randint(-127, 128, (e, k, n), dtype=torch.int8, device=dev)
+    scales = (torch.rand(e, n, device=dev) * 0.8 + 0.2) / (127.0 * k ** 0.5)
+    gw = w8.prepare_grouped_weight(codes, scales)
+    x = torch.randn(m, k, device=dev).to(torch.bfloat16)
+    dy = torch.randn(m, n, device=dev).to(torch.bfloat16)
+    a = (torch.randn(e, k, r, device=dev) * 0.1).to(torch.bfloat16)
+    b = (torch.randn(e, r, n, device=dev) * 0.1).to(torch.bfloat16)
+    gs = torch.tensor(sizes, dtype=torch.int32, device=dev)
+    plan = w8.GroupedBackwardPlan(x, dy, gs, gw, a, b, torch.ones(e, device=dev))
+    outs = plan.run()
+    gen = torch.Generator(device=dev).manual_seed(8)
+    layouts = [[40, 0, 300, 7, 129, 64], [0, 0, 1, 500, 0, 39], [90, 90, 90, 90, 90, 90], [540, 0, 0, 0, 0, 0]]
+
+    def refresh(i):
+        dy.copy_(torch.randn(dy.shape, device=dev, generator=gen).to(torch.bfloat16))
+        plan.group_sizes.copy_(torch.tensor(layouts[i % len(layouts)], dtype=torch.int32))   # the group sizes too
+
+    _replays(torch, plan.run, lambda: list(outs), refresh)

@@ -149,6 +149,66 @@ def test_grouped_random_geometry(dev, seed):
     assert torch.equal(mapped, out)
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_grouped_backward_random_geometry(dev, seed):
+    """The single grouped backward call on ragged groups (empty ones, several groups per weight, spare
+    rows): bit-equal to one dense backward call per weight, dx within tolerance of the oracle."""
+    import torch
+
+    from __graft_entry__ import load_package
+
+    pkg = load_package()
+    w8 = pkg.w8a8_lora
+    rng = np.random.default_rng(30_000 + seed)
+    gpw = int(rng.choice([1, 1, 2, 3]))
+    n_weights = int(rng.choice([1, 2, 5, 9, 70]))
+    e = gpw * n_weights
+    sizes = [int(v) for v in rng.choice([0, 0, 1, 31, 33, 64, 130, 257, 300] if n_weights < 20 else [0, 1, 7, 40], e)]
+    if sum(sizes) == 0:
+        sizes[-1] = 5
+    k = 8 * int(rng.integers(4, 90))
+    n = 8 * int(rng.integers(2, 120))
+    rank = int(rng.choice([0, 4, 16, 33, 64]))
+    extra = int(rng.integers(0, 4))
+    m = sum(sizes) + extra
+    print(f"[case] grouped backward seed={seed} weights={n_weights} gpw={gpw} rows={m} k={k} n={n} rank={rank}", flush=True)
+    bf = lambda t: torch.from_numpy(np.ascontiguousarray(t)).to(dev).to(torch.bfloat16)
+    x = o.bf16_round(rng.standard_normal((m, k)).astype(F32))
+    dy = o.bf16_round(rng.standard_normal((m, n)).astype(F32))
+    codes = rng.integers(-127, 128, (n_weights, k, n), dtype=np.int8)
+    scales = (rng.uniform(0.2, 1.0, (n_weights, n)) / (127.0 * np.sqrt(k))).astype(F32)
+    gw = w8.prepare_grouped_weight(torch.from_numpy(codes).to(dev), torch.from_numpy(scales).to(dev))
+    gs = torch.tensor(sizes, dtype=torch.int32, device=dev)
+    lora = (None, None, None)
+    if rank:
+        lora = (bf(rng.standard_normal((e, k, rank)).astype(F32) * 0.1), bf(rng.standard_normal((e, rank, n)).astype(F32) * 0.1),
+                torch.from_numpy(rng.uniform(0.5, 2.0, e).astype(F32)).to(dev))
+    got = w8.grouped_backward(bf(x), bf(dy), gs, gw, *lora, groups_per_weight=gpw)
+    ref = w8.grouped_backward_per_weight(bf(x), bf(dy), gs, gw, *lora, groups_per_weight=gpw)
+    torch.cuda.synchronize()
+    for g, r in zip(got, ref):
+        assert (g is None and r is None) or torch.equal(g, r)
+    # dx of the base term against the oracle: per weight dy @ bf16(codes * scales).T (+ the LoRA term)
+    st = np.concatenate(([0], np.cumsum(sizes)))
+    want = np.zeros((m, k), F32)
+    for wi in range(n_weights):
+        r0, r1 = int(st[wi * gpw]), int(st[(wi + 1) * gpw])
+        if r1 == r0:
+            continue
+        w = o.GroupQuantizedWeight(codes[wi], scales[wi:wi + 1], k, k, 8, k)
+        base = o._mm64(dy[r0:r1], o.pullback_weight(w, True).T)
+        if rank:
+            a_np, b_np = (v.float().cpu().numpy() for v in lora[:2])
+            s_np = lora[2].cpu().numpy()
+            for g in range(wi * gpw, (wi + 1) * gpw):
+                q0, q1 = int(st[g]) - r0, int(st[g + 1]) - r0
+                r_ = (o._mm64(dy[r0:r1][q0:q1], b_np[g].T) * s_np[g]).astype(F32)
+                base[q0:q1] = (base[q0:q1] + o._mm64(r_, a_np[g].T)).astype(F32)
+        want[r0:r1] = o.bf16_round(base)
+    rep = wc.compare(got[0].float().cpu().numpy(), want)
+    assert rep["violations"] == 0, rep
+
+
 @pytest.mark.parametrize("seed", range(10))
 def test_group_scaled_random_geometry(dev, seed):
     """W4 / W8 codes with grouped scales, A4 / A8: codes, scales and the float32 base bit-equal."""
