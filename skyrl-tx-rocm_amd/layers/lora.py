@@ -168,7 +168,7 @@ class LoRAExpert(LoRAMixin):
     pairs are indexed ``expert * max_lora_adapters + adapter`` (lora.py:414-431): rows are
     stably re-sorted by that combined index, run through the grouped kernel with
     ``max_lora_adapters`` LoRA groups per expert weight, and put back.  Differentiable: the backward
-    runs the dense backward kernels once per expert.
+    is one native grouped call for all experts and adapters.
     """
 
     def __init__(self, num_experts: int, in_features: int, out_features: int, *,
