@@ -650,6 +650,153 @@ int launch_bwd_dx(const BwdDxArgs& g, hipStream_t s) {
   return launch_status();
 }
 
+// The stages of a backward call behind its routing tables: dy into operand order (with the partial
+// sums of r = dy @ B.T), r and z finished, the pull-back GEMM, the LoRA cotangents.  The dense call
+// and the grouped call differ only in who wrote the tables and in the per-tile weights.
+struct BwdBody {
+  uint32_t m, k, n, n_groups, rank;
+  const void* x; const void* dy; const void* w_packed;
+  const void* lora_b; const float* lora_scaling;
+  void* dx; void* d_lora_a; void* d_lora_b; float* d_lora_scaling;
+  bool lora, want_grads, skip_prologue, skip_gemm;
+  // tables (null: identity routing, everything in group 0)
+  const int32_t* src_row; const int32_t* slot_group; const int32_t* blk_range; const int32_t* group_off;
+  // grouped calls only
+  const int32_t* skip_range;  // blk_range again when blocks without rows are to be skipped
+  const int32_t* tile_weight; const int32_t* chunk_tab; const int32_t* chunk0; const int32_t* group_beg;
+  const int32_t* group_end;
+  size_t w_stride; uint32_t sw_stride;
+};
+
+template <class Layout>
+int launch_bwd_body(const BwdBody& b, const Layout& w, unsigned char* ws, hipStream_t s) {
+  int st;
+  if (!b.skip_prologue) {  // dy into operand order; the same pass leaves the partial sums of r = dy @ B.T
+    BwdPackDyArgs d{};
+    d.dy = static_cast<const uint16_t*>(b.dy);
+    d.src_row = b.src_row; d.slot_group = b.slot_group; d.blk_range = b.blk_range;
+    d.dyp = ws + w.dyp;
+    d.lora_b = static_cast<const uint16_t*>(b.lora_b);
+    d.rpart = b.lora ? reinterpret_cast<float*>(ws + w.rpart) : nullptr;
+    d.M = b.m; d.N = b.n; d.NB = w.NB; d.n_row_blocks = w.slots / 32u; d.n_col_groups = w.N_pad / 128u;
+    d.n_slices = w.n_slices; d.groups_per_slice = w.groups_per_slice; d.r = b.rank; d.slots = w.slots;
+    const dim3 grid(d.n_row_blocks * d.n_slices), block(256);
+    if (!b.lora) hipLaunchKernelGGL((bwd_pack_dy_kernel<0>), grid, block, 0, s, d);
+    else if (w.nkk > 2u) hipLaunchKernelGGL((bwd_pack_dy_kernel<2>), grid, block, 0, s, d);
+    else hipLaunchKernelGGL((bwd_pack_dy_kernel<1>), grid, block, 0, s, d);
+    if ((st = launch_status())) return st;
+  }
+  if (b.lora && !b.skip_prologue) {
+    {
+      BwdRFinishArgs f{};
+      f.rpart = reinterpret_cast<const float*>(ws + w.rpart);
+      f.slot_group = b.slot_group;
+      f.blk_range = b.skip_range;
+      f.lora_scaling = b.lora_scaling;
+      f.r_raw = reinterpret_cast<float*>(ws + w.r_raw);
+      f.rs = reinterpret_cast<float*>(ws + w.rs);
+      f.rp = ws + w.rp;
+      f.n_slices = w.n_slices; f.slots = w.slots; f.nkk = w.nkk; f.cols = w.nkk > 2u ? 64u : 32u;
+      hipLaunchKernelGGL(bwd_r_finish_kernel, dim3(w.slots / 32u), dim3(256), 0, s, f);
+      if ((st = launch_status())) return st;
+    }
+    if (b.d_lora_b || b.d_lora_scaling) {  // z = x @ A, recomputed rather than saved by the forward
+      LoraAArgs lz{};
+      lz.xsrc = static_cast<const uint16_t*>(b.x);
+      lz.at = reinterpret_cast<const uint16_t*>(ws + w.at);
+      lz.src_row = b.src_row; lz.slot_group = b.slot_group; lz.blk_range = b.blk_range;
+      lz.zp = nullptr;
+      lz.M = b.m; lz.K = b.k; lz.r = b.rank; lz.nkk = w.nkk;
+      lz.n_steps = (b.k + 63u) / 64u;
+      lz.nterms = 3u;
+      lz.n_blocks = w.slots / 32u;
+      // K is cut into slices so that the launch fills the chip; the slices land in the partial
+      // table (r's partials have been consumed) and are added in slice order
+      const uint32_t nks = w.n_slices;
+      lz.n_ksplit = nks;
+      lz.steps_per_wave = ((lz.n_steps + nks - 1u) / nks + 15u) / 16u;
+      lz.zf = reinterpret_cast<float*>(ws + w.rpart);
+      lz.zf_stride = kBwdRankStride;
+      lz.zf_slice = w.slots * kBwdRankStride;
+      const dim3 grid(lz.n_blocks * nks), block(1024);
+      if (w.nkk > 2u) hipLaunchKernelGGL((lora_a_kernel<2>), grid, block, 0, s, lz);
+      else hipLaunchKernelGGL((lora_a_kernel<1>), grid, block, 0, s, lz);
+      if ((st = launch_status())) return st;
+      BwdRFinishArgs f{};
+      f.rpart = reinterpret_cast<const float*>(ws + w.rpart);
+      f.blk_range = b.skip_range;
+      f.r_raw = reinterpret_cast<float*>(ws + w.z);
+      f.n_slices = nks; f.slots = w.slots; f.nkk = w.nkk; f.cols = w.nkk > 2u ? 64u : 32u;
+      hipLaunchKernelGGL(bwd_r_finish_kernel, dim3(w.slots / 32u), dim3(256), 0, s, f);
+      if ((st = launch_status())) return st;
+    }
+  }
+  if (!b.skip_gemm) {
+    BwdDxArgs g{};
+    g.dyp = ws + w.dyp;
+    g.wp = static_cast<const unsigned char*>(b.w_packed);
+    g.swp = reinterpret_cast<const float*>(ws + w.swp);
+    g.rp = b.lora ? ws + w.rp : nullptr;
+    g.ap = b.lora ? ws + w.ap : nullptr;
+    g.src_row = b.src_row; g.slot_group = b.slot_group; g.blk_range = b.blk_range;
+    g.dx = static_cast<uint16_t*>(b.dx);
+    g.M = b.m; g.K = b.k; g.KB = w.KB; g.NB = w.NB; g.tiles_m = w.tiles_m; g.tiles_k = w.tiles_k;
+    g.tile_weight = b.tile_weight; g.w_stride = b.w_stride; g.sw_stride = b.sw_stride;
+    switch (b.lora ? w.nkk : 0u) {
+      case 0: st = launch_bwd_dx<0>(g, s); break;
+      case 1: st = launch_bwd_dx<1>(g, s); break;
+      case 2: st = launch_bwd_dx<2>(g, s); break;
+      default: st = launch_bwd_dx<4>(g, s); break;
+    }
+    if (st) return st;
+  }
+  if (b.lora && b.want_grads) {
+    BwdDloraArgs d{};
+    d.x = static_cast<const uint16_t*>(b.x);
+    d.dy = static_cast<const uint16_t*>(b.dy);
+    d.rs = reinterpret_cast<const float*>(ws + w.rs);
+    d.z = reinterpret_cast<const float*>(ws + w.z);
+    d.src_row = b.src_row;
+    d.group_off = b.group_off;
+    d.chunk_tab = b.chunk_tab;
+    d.partA = reinterpret_cast<float*>(ws + w.partA);
+    d.partB = reinterpret_cast<float*>(ws + w.partB);
+    d.M = b.m; d.K = b.k; d.N = b.n; d.n_groups = b.n_groups; d.max_chunks = w.max_chunks;
+    d.col_tiles_a = b.d_lora_a ? (b.k + 255u) / 256u : 0u;
+    d.col_tiles_b = b.d_lora_b ? (b.n + 255u) / 256u : 0u;
+    if (d.col_tiles_a + d.col_tiles_b) {
+      const dim3 grid(w.max_chunks * (d.col_tiles_a + d.col_tiles_b)), block(256);
+      const uint32_t lds_bytes = (kBwdStageRows / 32u) * (w.R / 32u) * 6u * kBlockBytes;
+      if (w.R == 32u) {
+        hipLaunchKernelGGL((bwd_dlora_kernel<1>), grid, block, lds_bytes, s, d);
+      } else {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_dlora_kernel<2>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
+          return MI355_W8A8_ERR_LAUNCH;
+        hipLaunchKernelGGL((bwd_dlora_kernel<2>), grid, block, lds_bytes, s, d);
+      }
+      if ((st = launch_status())) return st;
+    }
+    BwdReduceArgs r{};
+    r.partA = d.partA; r.partB = d.partB;
+    r.r_raw = reinterpret_cast<const float*>(ws + w.r_raw);
+    r.z = d.z;
+    r.lora_scaling = b.lora_scaling;
+    r.group_off = b.group_off;
+    r.chunk0_tab = b.chunk0; r.group_beg = b.group_beg; r.group_end = b.group_end;
+    r.d_a = static_cast<uint16_t*>(b.d_lora_a);
+    r.d_b = static_cast<uint16_t*>(b.d_lora_b);
+    r.d_s = b.d_lora_scaling;
+    r.K = b.k; r.N = b.n; r.r = b.rank; r.R = w.R; r.n_groups = b.n_groups;
+    r.blocks_a = b.d_lora_a ? (uint32_t)(((uint64_t)b.n_groups * b.rank * b.k + 255u) / 256u) : 0u;
+    r.blocks_b = b.d_lora_b ? (uint32_t)(((uint64_t)b.n_groups * b.rank * b.n / 4u + 255u) / 256u) : 0u;
+    const uint32_t s_blocks = b.d_lora_scaling ? b.n_groups : 0u;
+    hipLaunchKernelGGL(bwd_dlora_reduce_kernel, dim3(r.blocks_a + r.blocks_b + s_blocks), dim3(256), 0, s, r);
+    if ((st = launch_status())) return st;
+  }
+  return MI355_W8A8_OK;
+}
+
 int run_backward(const mi355_w8a8_bwd_problem* p, hipStream_t s) {
   if (!p) return MI355_W8A8_ERR_NULL;
   if (p->struct_size != sizeof(mi355_w8a8_bwd_problem)) return MI355_W8A8_ERR_STRUCT;
@@ -709,131 +856,16 @@ int run_backward(const mi355_w8a8_bwd_problem* p, hipStream_t s) {
     hipLaunchKernelGGL(bwd_prep_kernel, dim3(pa.route_blocks + pa.a_blocks + pa.ap_blocks + sw_blocks), dim3(1024), 0, s, pa);
     if ((st = launch_status())) return st;
   }
-  if (!skip_prologue) {  // dy into operand order; the same pass leaves the partial sums of r = dy @ B.T
-    BwdPackDyArgs d{};
-    d.dy = static_cast<const uint16_t*>(p->dy);
-    d.src_row = routed ? src_row : nullptr;
-    d.slot_group = routed ? slot_group : nullptr;
-    d.blk_range = routed ? blk_range : nullptr;
-    d.dyp = ws + w.dyp;
-    d.lora_b = static_cast<const uint16_t*>(p->lora_b);
-    d.rpart = lora ? reinterpret_cast<float*>(ws + w.rpart) : nullptr;
-    d.M = p->m; d.N = p->n; d.NB = w.NB; d.n_row_blocks = w.slots / 32u; d.n_col_groups = w.N_pad / 128u;
-    d.n_slices = w.n_slices; d.groups_per_slice = w.groups_per_slice; d.r = p->rank; d.slots = w.slots;
-    const dim3 grid(d.n_row_blocks * d.n_slices), block(256);
-    if (!lora) hipLaunchKernelGGL((bwd_pack_dy_kernel<0>), grid, block, 0, s, d);
-    else if (w.nkk > 2u) hipLaunchKernelGGL((bwd_pack_dy_kernel<2>), grid, block, 0, s, d);
-    else hipLaunchKernelGGL((bwd_pack_dy_kernel<1>), grid, block, 0, s, d);
-    if ((st = launch_status())) return st;
-  }
-  if (lora && !skip_prologue) {
-    {
-      BwdRFinishArgs f{};
-      f.rpart = reinterpret_cast<const float*>(ws + w.rpart);
-      f.slot_group = routed ? slot_group : nullptr;
-      f.lora_scaling = p->lora_scaling;
-      f.r_raw = reinterpret_cast<float*>(ws + w.r_raw);
-      f.rs = reinterpret_cast<float*>(ws + w.rs);
-      f.rp = ws + w.rp;
-      f.n_slices = w.n_slices; f.slots = w.slots; f.nkk = w.nkk; f.cols = w.nkk > 2u ? 64u : 32u;
-      hipLaunchKernelGGL(bwd_r_finish_kernel, dim3(w.slots / 32u), dim3(256), 0, s, f);
-      if ((st = launch_status())) return st;
-    }
-    if (p->d_lora_b || p->d_lora_scaling) {  // z = x @ A, recomputed rather than saved by the forward
-      LoraAArgs lz{};
-      lz.xsrc = static_cast<const uint16_t*>(p->x);
-      lz.at = reinterpret_cast<const uint16_t*>(ws + w.at);
-      lz.src_row = routed ? src_row : nullptr;
-      lz.slot_group = routed ? slot_group : nullptr;
-      lz.blk_range = routed ? blk_range : nullptr;
-      lz.zp = nullptr;
-      lz.M = p->m; lz.K = p->k; lz.r = p->rank; lz.nkk = w.nkk;
-      lz.n_steps = (p->k + 63u) / 64u; lz.steps_per_wave = (lz.n_steps + 15u) / 16u;
-      lz.nterms = 3u;
-      lz.n_blocks = w.slots / 32u;
-      // K is cut into slices so that the launch fills the chip; the slices land in the partial
-      // table (r's partials have been consumed) and are added in slice order
-      const uint32_t nks = w.n_slices;
-      lz.n_ksplit = nks;
-      lz.steps_per_wave = ((lz.n_steps + nks - 1u) / nks + 15u) / 16u;
-      lz.zf = reinterpret_cast<float*>(ws + w.rpart);
-      lz.zf_stride = kBwdRankStride;
-      lz.zf_slice = w.slots * kBwdRankStride;
-      const dim3 grid(lz.n_blocks * nks), block(1024);
-      if (w.nkk > 2u) hipLaunchKernelGGL((lora_a_kernel<2>), grid, block, 0, s, lz);
-      else hipLaunchKernelGGL((lora_a_kernel<1>), grid, block, 0, s, lz);
-      if ((st = launch_status())) return st;
-      BwdRFinishArgs f{};
-      f.rpart = reinterpret_cast<const float*>(ws + w.rpart);
-      f.r_raw = reinterpret_cast<float*>(ws + w.z);
-      f.n_slices = nks; f.slots = w.slots; f.nkk = w.nkk; f.cols = w.nkk > 2u ? 64u : 32u;
-      hipLaunchKernelGGL(bwd_r_finish_kernel, dim3(w.slots / 32u), dim3(256), 0, s, f);
-      if ((st = launch_status())) return st;
-    }
-  }
-  if (!skip_gemm) {
-    BwdDxArgs g{};
-    g.dyp = ws + w.dyp;
-    g.wp = static_cast<const unsigned char*>(p->w_packed);
-    g.swp = reinterpret_cast<const float*>(ws + w.swp);
-    g.rp = lora ? ws + w.rp : nullptr;
-    g.ap = lora ? ws + w.ap : nullptr;
-    g.src_row = routed ? src_row : nullptr;
-    g.slot_group = routed ? slot_group : nullptr;
-    g.blk_range = routed ? blk_range : nullptr;
-    g.dx = static_cast<uint16_t*>(p->dx);
-    g.M = p->m; g.K = p->k; g.KB = w.KB; g.NB = w.NB; g.tiles_m = w.tiles_m; g.tiles_k = w.tiles_k;
-    switch (lora ? w.nkk : 0u) {
-      case 0: st = launch_bwd_dx<0>(g, s); break;
-      case 1: st = launch_bwd_dx<1>(g, s); break;
-      case 2: st = launch_bwd_dx<2>(g, s); break;
-      default: st = launch_bwd_dx<4>(g, s); break;
-    }
-    if (st) return st;
-  }
-  if (lora && want_grads) {
-    BwdDloraArgs d{};
-    d.x = static_cast<const uint16_t*>(p->x);
-    d.dy = static_cast<const uint16_t*>(p->dy);
-    d.rs = reinterpret_cast<const float*>(ws + w.rs);
-    d.z = reinterpret_cast<const float*>(ws + w.z);
-    d.src_row = routed ? src_row : nullptr;
-    d.group_off = group_off;
-    d.partA = reinterpret_cast<float*>(ws + w.partA);
-    d.partB = reinterpret_cast<float*>(ws + w.partB);
-    d.M = p->m; d.K = p->k; d.N = p->n; d.n_groups = p->n_adapters; d.max_chunks = w.max_chunks;
-    d.col_tiles_a = p->d_lora_a ? (p->k + 255u) / 256u : 0u;
-    d.col_tiles_b = p->d_lora_b ? (p->n + 255u) / 256u : 0u;
-    if (d.col_tiles_a + d.col_tiles_b) {
-      const dim3 grid(w.max_chunks * (d.col_tiles_a + d.col_tiles_b)), block(256);
-      const uint32_t lds_bytes = (kBwdStageRows / 32u) * (w.R / 32u) * 6u * kBlockBytes;
-      if (w.R == 32u) {
-        hipLaunchKernelGGL((bwd_dlora_kernel<1>), grid, block, lds_bytes, s, d);
-      } else {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_dlora_kernel<2>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
-          return MI355_W8A8_ERR_LAUNCH;
-        hipLaunchKernelGGL((bwd_dlora_kernel<2>), grid, block, lds_bytes, s, d);
-      }
-      if ((st = launch_status())) return st;
-    }
-    BwdReduceArgs r{};
-    r.partA = d.partA; r.partB = d.partB;
-    r.r_raw = reinterpret_cast<const float*>(ws + w.r_raw);
-    r.z = d.z;
-    r.lora_scaling = p->lora_scaling;
-    r.group_off = group_off;
-    r.d_a = static_cast<uint16_t*>(p->d_lora_a);
-    r.d_b = static_cast<uint16_t*>(p->d_lora_b);
-    r.d_s = p->d_lora_scaling;
-    r.K = p->k; r.N = p->n; r.r = p->rank; r.R = w.R; r.n_groups = p->n_adapters;
-    r.blocks_a = p->d_lora_a ? (uint32_t)(((uint64_t)p->n_adapters * p->rank * p->k + 255u) / 256u) : 0u;
-    r.blocks_b = p->d_lora_b ? (uint32_t)(((uint64_t)p->n_adapters * p->rank * p->n / 4u + 255u) / 256u) : 0u;
-    const uint32_t s_blocks = p->d_lora_scaling ? p->n_adapters : 0u;
-    hipLaunchKernelGGL(bwd_dlora_reduce_kernel, dim3(r.blocks_a + r.blocks_b + s_blocks), dim3(256), 0, s, r);
-    if ((st = launch_status())) return st;
-  }
-  return MI355_W8A8_OK;
+  BwdBody b{};
+  b.m = p->m; b.k = p->k; b.n = p->n; b.n_groups = p->n_adapters; b.rank = p->rank;
+  b.x = p->x; b.dy = p->dy; b.w_packed = p->w_packed; b.lora_b = p->lora_b; b.lora_scaling = p->lora_scaling;
+  b.dx = p->dx; b.d_lora_a = p->d_lora_a; b.d_lora_b = p->d_lora_b; b.d_lora_scaling = p->d_lora_scaling;
+  b.lora = lora; b.want_grads = want_grads; b.skip_prologue = skip_prologue; b.skip_gemm = skip_gemm;
+  b.src_row = routed ? src_row : nullptr;
+  b.slot_group = routed ? slot_group : nullptr;
+  b.blk_range = routed ? blk_range : nullptr;
+  b.group_off = group_off;
+  return launch_bwd_body(b, w, ws, s);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -971,130 +1003,17 @@ int run_grouped_backward(const mi355_w8a8_grouped_bwd_problem* p, hipStream_t s)
                        dim3(1u + pa.a_blocks + pa.ap_blocks + pa.sw_blocks_per_weight * w.n_weights), dim3(1024), 0, s, pa);
     if ((st = launch_status())) return st;
   }
-  {  // dy into operand order; the same pass leaves the partial sums of r = dy @ B.T
-    BwdPackDyArgs d{};
-    d.dy = static_cast<const uint16_t*>(p->dy);
-    d.src_row = tab.src_row; d.slot_group = tab.slot_group; d.blk_range = tab.blk_range;
-    d.dyp = ws + w.dyp;
-    d.lora_b = static_cast<const uint16_t*>(p->lora_b);
-    d.rpart = lora ? reinterpret_cast<float*>(ws + w.rpart) : nullptr;
-    d.M = p->m; d.N = p->n; d.NB = w.NB; d.n_row_blocks = w.slots / 32u; d.n_col_groups = w.N_pad / 128u;
-    d.n_slices = w.n_slices; d.groups_per_slice = w.groups_per_slice; d.r = p->rank; d.slots = w.slots;
-    const dim3 grid(d.n_row_blocks * d.n_slices), block(256);
-    if (!lora) hipLaunchKernelGGL((bwd_pack_dy_kernel<0>), grid, block, 0, s, d);
-    else if (w.nkk > 2u) hipLaunchKernelGGL((bwd_pack_dy_kernel<2>), grid, block, 0, s, d);
-    else hipLaunchKernelGGL((bwd_pack_dy_kernel<1>), grid, block, 0, s, d);
-    if ((st = launch_status())) return st;
-  }
-  if (lora) {
-    {
-      BwdRFinishArgs f{};
-      f.rpart = reinterpret_cast<const float*>(ws + w.rpart);
-      f.slot_group = tab.slot_group;
-      f.blk_range = tab.blk_range;
-      f.lora_scaling = p->lora_scaling;
-      f.r_raw = reinterpret_cast<float*>(ws + w.r_raw);
-      f.rs = reinterpret_cast<float*>(ws + w.rs);
-      f.rp = ws + w.rp;
-      f.n_slices = w.n_slices; f.slots = w.slots; f.nkk = w.nkk; f.cols = w.nkk > 2u ? 64u : 32u;
-      hipLaunchKernelGGL(bwd_r_finish_kernel, dim3(w.slots / 32u), dim3(256), 0, s, f);
-      if ((st = launch_status())) return st;
-    }
-    if (p->d_lora_b || p->d_lora_scaling) {  // z = x @ A
-      LoraAArgs lz{};
-      lz.xsrc = static_cast<const uint16_t*>(p->x);
-      lz.at = reinterpret_cast<const uint16_t*>(ws + w.at);
-      lz.src_row = tab.src_row; lz.slot_group = tab.slot_group; lz.blk_range = tab.blk_range;
-      lz.zp = nullptr;
-      lz.M = p->m; lz.K = p->k; lz.r = p->rank; lz.nkk = w.nkk;
-      lz.n_steps = (p->k + 63u) / 64u;
-      lz.nterms = 3u;
-      lz.n_blocks = w.slots / 32u;
-      const uint32_t nks = w.n_slices;
-      lz.n_ksplit = nks;
-      lz.steps_per_wave = ((lz.n_steps + nks - 1u) / nks + 15u) / 16u;
-      lz.zf = reinterpret_cast<float*>(ws + w.rpart);
-      lz.zf_stride = kBwdRankStride;
-      lz.zf_slice = w.slots * kBwdRankStride;
-      const dim3 grid(lz.n_blocks * nks), block(1024);
-      if (w.nkk > 2u) hipLaunchKernelGGL((lora_a_kernel<2>), grid, block, 0, s, lz);
-      else hipLaunchKernelGGL((lora_a_kernel<1>), grid, block, 0, s, lz);
-      if ((st = launch_status())) return st;
-      BwdRFinishArgs f{};
-      f.rpart = reinterpret_cast<const float*>(ws + w.rpart);
-      f.blk_range = tab.blk_range;
-      f.r_raw = reinterpret_cast<float*>(ws + w.z);
-      f.n_slices = nks; f.slots = w.slots; f.nkk = w.nkk; f.cols = w.nkk > 2u ? 64u : 32u;
-      hipLaunchKernelGGL(bwd_r_finish_kernel, dim3(w.slots / 32u), dim3(256), 0, s, f);
-      if ((st = launch_status())) return st;
-    }
-  }
-  {
-    BwdDxArgs g{};
-    g.dyp = ws + w.dyp;
-    g.wp = static_cast<const unsigned char*>(p->w_packed);
-    g.swp = reinterpret_cast<const float*>(ws + w.swp);
-    g.rp = lora ? ws + w.rp : nullptr;
-    g.ap = lora ? ws + w.ap : nullptr;
-    g.src_row = tab.src_row; g.slot_group = tab.slot_group; g.blk_range = tab.blk_range;
-    g.dx = static_cast<uint16_t*>(p->dx);
-    g.M = p->m; g.K = p->k; g.KB = w.KB; g.NB = w.NB; g.tiles_m = w.tiles_m; g.tiles_k = w.tiles_k;
-    g.tile_weight = tab.tile_weight;
-    g.w_stride = (size_t)mi355_w8a8_packed_weight_bytes(p->k, p->n);
-    g.sw_stride = w.sw_stride;
-    switch (lora ? w.nkk : 0u) {
-      case 0: st = launch_bwd_dx<0>(g, s); break;
-      case 1: st = launch_bwd_dx<1>(g, s); break;
-      case 2: st = launch_bwd_dx<2>(g, s); break;
-      default: st = launch_bwd_dx<4>(g, s); break;
-    }
-    if (st) return st;
-  }
-  if (lora && want_grads) {
-    BwdDloraArgs d{};
-    d.x = static_cast<const uint16_t*>(p->x);
-    d.dy = static_cast<const uint16_t*>(p->dy);
-    d.rs = reinterpret_cast<const float*>(ws + w.rs);
-    d.z = reinterpret_cast<const float*>(ws + w.z);
-    d.src_row = tab.src_row;
-    d.group_off = nullptr;
-    d.chunk_tab = tab.chunk_tab;
-    d.partA = reinterpret_cast<float*>(ws + w.partA);
-    d.partB = reinterpret_cast<float*>(ws + w.partB);
-    d.M = p->m; d.K = p->k; d.N = p->n; d.n_groups = p->n_groups; d.max_chunks = w.max_chunks;
-    d.col_tiles_a = p->d_lora_a ? (p->k + 255u) / 256u : 0u;
-    d.col_tiles_b = p->d_lora_b ? (p->n + 255u) / 256u : 0u;
-    if (d.col_tiles_a + d.col_tiles_b) {
-      const dim3 grid(w.max_chunks * (d.col_tiles_a + d.col_tiles_b)), block(256);
-      const uint32_t lds_bytes = (kBwdStageRows / 32u) * (w.R / 32u) * 6u * kBlockBytes;
-      if (w.R == 32u) {
-        hipLaunchKernelGGL((bwd_dlora_kernel<1>), grid, block, lds_bytes, s, d);
-      } else {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_dlora_kernel<2>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
-          return MI355_W8A8_ERR_LAUNCH;
-        hipLaunchKernelGGL((bwd_dlora_kernel<2>), grid, block, lds_bytes, s, d);
-      }
-      if ((st = launch_status())) return st;
-    }
-    BwdReduceArgs r{};
-    r.partA = d.partA; r.partB = d.partB;
-    r.r_raw = reinterpret_cast<const float*>(ws + w.r_raw);
-    r.z = d.z;
-    r.lora_scaling = p->lora_scaling;
-    r.group_off = nullptr;
-    r.chunk0_tab = tab.chunk0; r.group_beg = tab.group_beg; r.group_end = tab.group_end;
-    r.d_a = static_cast<uint16_t*>(p->d_lora_a);
-    r.d_b = static_cast<uint16_t*>(p->d_lora_b);
-    r.d_s = p->d_lora_scaling;
-    r.K = p->k; r.N = p->n; r.r = p->rank; r.R = w.R; r.n_groups = p->n_groups;
-    r.blocks_a = p->d_lora_a ? (uint32_t)(((uint64_t)p->n_groups * p->rank * p->k + 255u) / 256u) : 0u;
-    r.blocks_b = p->d_lora_b ? (uint32_t)(((uint64_t)p->n_groups * p->rank * p->n / 4u + 255u) / 256u) : 0u;
-    const uint32_t s_blocks = p->d_lora_scaling ? p->n_groups : 0u;
-    hipLaunchKernelGGL(bwd_dlora_reduce_kernel, dim3(r.blocks_a + r.blocks_b + s_blocks), dim3(256), 0, s, r);
-    if ((st = launch_status())) return st;
-  }
-  return MI355_W8A8_OK;
+  BwdBody b{};
+  b.m = p->m; b.k = p->k; b.n = p->n; b.n_groups = p->n_groups; b.rank = p->rank;
+  b.x = p->x; b.dy = p->dy; b.w_packed = p->w_packed; b.lora_b = p->lora_b; b.lora_scaling = p->lora_scaling;
+  b.dx = p->dx; b.d_lora_a = p->d_lora_a; b.d_lora_b = p->d_lora_b; b.d_lora_scaling = p->d_lora_scaling;
+  b.lora = lora; b.want_grads = want_grads;
+  b.src_row = tab.src_row; b.slot_group = tab.slot_group; b.blk_range = tab.blk_range; b.skip_range = tab.blk_range;
+  b.tile_weight = tab.tile_weight; b.chunk_tab = tab.chunk_tab; b.chunk0 = tab.chunk0;
+  b.group_beg = tab.group_beg; b.group_end = tab.group_end;
+  b.w_stride = (size_t)mi355_w8a8_packed_weight_bytes(p->k, p->n);
+  b.sw_stride = w.sw_stride;
+  return launch_bwd_body(b, w, ws, s);
 }
 
 int run_qkv_post(const mi355_w8a8_qkv_post_problem* p, hipStream_t s) {
