@@ -468,18 +468,23 @@ __global__ __launch_bounds__(512, 1) void bwd_dx_kernel(BwdDxArgs g) {
     const uint32_t tm = band * 4u + in_band % band_rows, tk = in_band / band_rows;
     int tw = 0;
     int n_act = 4;  // 32-row blocks of this wave that hold rows: the others skip their matrix-core work
+    uint32_t load_rb = (uint32_t)wave;  // row block whose dy panel chunks this wave fetches
     if (g.tile_weight) {
       const int tv = g.tile_weight[tm];
       if (tv < 0) continue;  // workgroup-uniform: no row lives in this tile
       tw = tv & 0xffff;
-      const int live = ((tv >> 16) + 31) / 32 - wrow * 4;
+      const int live_blocks = ((tv >> 16) + 31) / 32;
+      const int live = live_blocks - wrow * 4;
       n_act = live < 0 ? 0 : (live > 4 ? 4 : live);
+      // a block without rows is never multiplied: its slot is filled from block 0 of the tile, which
+      // is in the caches anyway, instead of streaming unused memory (the load count stays the same)
+      if (wave >= live_blocks) load_rb = 0u;
     }
     n_act = __builtin_amdgcn_readfirstlane(n_act);
     const float* swp_t = g.swp + (size_t)tw * g.sw_stride;
 
     // this wave's two panel chunks of a stage (row block = wave, halves q = 0, 1) and its weight block
-    const unsigned char* Ag = g.dyp + ((size_t)(tm * 8u + (uint32_t)wave) * g.NB) * 2048u + lane * 16;
+    const unsigned char* Ag = g.dyp + ((size_t)(tm * 8u + load_rb) * g.NB) * 2048u + lane * 16;
     const uint32_t kbw = tk * 8u + (uint32_t)wcol * 2u;  // first of the two k blocks this wave multiplies
     const uint32_t kbl = tk * 8u + (uint32_t)wave < g.KB ? tk * 8u + (uint32_t)wave : g.KB - 1u;  // the block it loads
     const unsigned char* Bg = g.wp + (size_t)tw * g.w_stride + (size_t)kbl * kBlockBytes + lane * 16;
