@@ -399,6 +399,16 @@ int mi355_w8a8_moe_route_v1(const float* router_logits, uint32_t n_tokens, uint3
                             uint32_t norm_topk_prob, float* weights, int32_t* selected, void* stream);
 
 /*
+ * Pull-back of mi355_w8a8_moe_route_v1 to the logits with the selection held fixed, as lax.top_k
+ * differentiates (qwen3.py:175-178): d_router_logits f32 [n_tokens, n_experts] from d_weights f32
+ * [n_tokens, top_k] and the selected int32 [n_tokens, top_k] the forward returned.  d_router_logits
+ * may be the router_logits buffer itself.
+ */
+int mi355_w8a8_moe_route_bwd_v1(const float* router_logits, const int32_t* selected, const float* d_weights,
+                                uint32_t n_tokens, uint32_t n_experts, uint32_t top_k, uint32_t norm_topk_prob,
+                                float* d_router_logits, void* stream);
+
+/*
  * mi355_w8a8_moe_dispatch_v1 replaces prepare_routing (skyrl/tx/layers/util.py:66-87) together with
  * the jnp.repeat in front of it (qwen3.py:189-190): pair p = (token p / repeat, choice p % repeat)
  * belongs to group indices[p]; the pairs are sorted by group, stably, and every pair's token row is

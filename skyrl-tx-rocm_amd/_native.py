@@ -41,7 +41,7 @@ EXPORTS = (
     "mi355_w8a8_qkv_bwd_workspace_bytes", "mi355_w8a8_qkv_split_norm_rope_bwd_v1",
     "mi355_w8a8_delta_rms_norm_bwd_workspace_bytes", "mi355_w8a8_delta_rms_norm_bwd_v1",
     "mi355_w8a8_swiglu_v1", "mi355_w8a8_swiglu_bwd_v1", "mi355_w8a8_rms_norm_bwd_v1",
-    "mi355_w8a8_moe_route_v1", "mi355_w8a8_moe_dispatch_workspace_bytes", "mi355_w8a8_moe_dispatch_v1",
+    "mi355_w8a8_moe_route_v1", "mi355_w8a8_moe_route_bwd_v1", "mi355_w8a8_moe_dispatch_workspace_bytes", "mi355_w8a8_moe_dispatch_v1",
     "mi355_w8a8_moe_combine_v1", "mi355_w8a8_moe_combine_bwd_v1",
     "mi355_w8a8_gq_packed_weight_bytes", "mi355_w8a8_gq_pack_weight_v1", "mi355_w8a8_gq_workspace_bytes",
     "mi355_w8a8_gq_linear_v1",
@@ -201,6 +201,8 @@ def _bind(lib: ctypes.CDLL) -> None:
     lib.mi355_w8a8_delta_rms_norm_bwd_v1.argtypes = (_vp, _vp, _vp, _vp, _vp, _vp, _u64, _u32, _u32, _f32, _vp)
     lib.mi355_w8a8_moe_route_v1.restype = ctypes.c_int
     lib.mi355_w8a8_moe_route_v1.argtypes = (_vp, _u32, _u32, _u32, _u32, _vp, _vp, _vp)
+    lib.mi355_w8a8_moe_route_bwd_v1.restype = ctypes.c_int
+    lib.mi355_w8a8_moe_route_bwd_v1.argtypes = (_vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp, _vp)
     lib.mi355_w8a8_moe_dispatch_workspace_bytes.restype = _u64
     lib.mi355_w8a8_moe_dispatch_workspace_bytes.argtypes = (_u32, _u32)
     lib.mi355_w8a8_moe_dispatch_v1.restype = ctypes.c_int

@@ -1269,6 +1269,32 @@ int run_moe_route(const float* logits, uint32_t t, uint32_t e, uint32_t top_k, u
   return launch_status();
 }
 
+int run_moe_route_bwd(const float* logits, const int32_t* selected, const float* d_weights, uint32_t t, uint32_t e,
+                      uint32_t top_k, uint32_t norm, float* d_logits, hipStream_t s) {
+  if (!logits || !selected || !d_weights || !d_logits) return MI355_W8A8_ERR_NULL;
+  if (t == 0 || e == 0 || top_k == 0 || top_k > e || norm > 1u) return MI355_W8A8_ERR_SHAPE;
+  if (e > kMoeMaxExperts || top_k > kMoeMaxTopK || t > kMaxRows) return MI355_W8A8_ERR_UNSUPPORTED;
+  if ((reinterpret_cast<uintptr_t>(logits) | reinterpret_cast<uintptr_t>(selected) |
+       reinterpret_cast<uintptr_t>(d_weights) | reinterpret_cast<uintptr_t>(d_logits)) & 3u)
+    return MI355_W8A8_ERR_ALIGN;
+  const uint64_t tab_bytes = (uint64_t)t * top_k * 4u, row_bytes = (uint64_t)t * e * 4u;
+  // d_logits may be the logits buffer itself (a token's row is read whole before it is rewritten), nothing else
+  if (d_logits != logits && overlaps(d_logits, row_bytes, logits, row_bytes)) return MI355_W8A8_ERR_ALIAS;
+  if (overlaps(d_logits, row_bytes, selected, tab_bytes) || overlaps(d_logits, row_bytes, d_weights, tab_bytes))
+    return MI355_W8A8_ERR_ALIAS;
+  MoeRouteBwdArgs a{};
+  a.logits = logits; a.selected = selected; a.d_weights = d_weights; a.d_logits = d_logits;
+  a.T = t; a.E = e; a.top_k = top_k; a.norm = norm;
+  (void)hipGetLastError();
+  const dim3 grid((t + 3u) / 4u), block(256);
+  if (e <= 64u) hipLaunchKernelGGL((moe_route_bwd_kernel<1>), grid, block, 0, s, a);
+  else if (e <= 128u) hipLaunchKernelGGL((moe_route_bwd_kernel<2>), grid, block, 0, s, a);
+  else if (e <= 256u) hipLaunchKernelGGL((moe_route_bwd_kernel<4>), grid, block, 0, s, a);
+  else if (e <= 512u) hipLaunchKernelGGL((moe_route_bwd_kernel<8>), grid, block, 0, s, a);
+  else hipLaunchKernelGGL((moe_route_bwd_kernel<16>), grid, block, 0, s, a);
+  return launch_status();
+}
+
 struct MoeSortLayout { uint64_t chunk_cnt, group_start, total; uint32_t n_chunks; };
 
 MoeSortLayout make_moe_sort_layout(uint32_t n_pairs, uint32_t n_groups) {
@@ -1737,6 +1763,13 @@ int mi355_w8a8_moe_route_v1(const float* router_logits, uint32_t n_tokens, uint3
                             uint32_t norm_topk_prob, float* weights, int32_t* selected, void* stream) {
   return run_moe_route(router_logits, n_tokens, n_experts, top_k, norm_topk_prob, weights, selected,
                        static_cast<hipStream_t>(stream));
+}
+
+int mi355_w8a8_moe_route_bwd_v1(const float* router_logits, const int32_t* selected, const float* d_weights,
+                                uint32_t n_tokens, uint32_t n_experts, uint32_t top_k, uint32_t norm_topk_prob,
+                                float* d_router_logits, void* stream) {
+  return run_moe_route_bwd(router_logits, selected, d_weights, n_tokens, n_experts, top_k, norm_topk_prob,
+                           d_router_logits, static_cast<hipStream_t>(stream));
 }
 
 uint64_t mi355_w8a8_moe_dispatch_workspace_bytes(uint32_t n_pairs, uint32_t n_groups) {

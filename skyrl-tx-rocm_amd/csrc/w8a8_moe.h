@@ -4,6 +4,7 @@
 // the expert outputs back to token order.  Index work is exact; everything is memory-bound.
 //
 //   moe_route_kernel           one wave per token: probabilities, top-k (ties: lower expert), weights
+//   moe_route_bwd_kernel       one wave per token: the weights' cotangent back to the logits
 //   moe_hist_kernel            per 1024-pair chunk: pairs per group
 //   moe_scan_kernel            one workgroup: group sizes, group starts, per-chunk offsets
 //   moe_scatter_kernel         per chunk: stable position of every pair, the index arrays
@@ -91,6 +92,88 @@ __global__ __launch_bounds__(256) void moe_route_kernel(MoeRouteArgs a) {
   if (lane < a.top_k) {
     a.weights[(size_t)t * a.top_k + lane] = my_w;
     a.selected[(size_t)t * a.top_k + lane] = my_i;
+  }
+}
+
+// Pull-back of the routing weights to the router logits with the selection held fixed (lax.top_k
+// has no derivative in its indices): p = softmax(l); ps = p[selected]; w = ps / sum(ps) when
+// normalised;  d_ps = (d_w - sum(d_w w)) / sum(ps)  (or d_w);  d_l = p (d_p - sum(p d_p)) with d_p
+// zero outside the selection (qwen3.py:175-178).  One wave per token, float32.
+struct MoeRouteBwdArgs {
+  const float* logits;     // f32 [T, E]
+  const int32_t* selected; // int32 [T, top_k]
+  const float* d_weights;  // f32 [T, top_k]
+  float* d_logits;         // f32 [T, E]
+  uint32_t T, E, top_k, norm;
+};
+
+template <uint32_t NV>
+__global__ __launch_bounds__(256) void moe_route_bwd_kernel(MoeRouteBwdArgs a) {
+  __shared__ float tab[4][kMoeMaxExperts];
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  const uint32_t t = blockIdx.x * 4u + wave;
+  if (t >= a.T) return;
+  const float* row = a.logits + (size_t)t * a.E;
+  float v[NV];
+  float mx = -INFINITY;
+#pragma unroll
+  for (uint32_t j = 0; j < NV; ++j) {
+    const uint32_t e = j * 64u + lane;
+    v[j] = e < a.E ? row[e] : -INFINITY;
+    mx = fmaxf(mx, v[j]);
+  }
+  mx = wave_max(mx);
+  float sum = 0.0f;
+#pragma unroll
+  for (uint32_t j = 0; j < NV; ++j) {
+    const uint32_t e = j * 64u + lane;
+    v[j] = e < a.E ? expf(v[j] - mx) : 0.0f;
+    sum += v[j];
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+#pragma unroll
+  for (uint32_t j = 0; j < NV; ++j) {
+    const uint32_t e = j * 64u + lane;
+    v[j] = v[j] / sum;
+    if (e < a.E) tab[wave][e] = v[j];
+  }
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave reads what its own lanes wrote
+  __builtin_amdgcn_wave_barrier();
+  // lane j < top_k owns choice j
+  const bool own = lane < a.top_k;
+  const int sel = own ? a.selected[(size_t)t * a.top_k + lane] : 0;
+  const uint32_t se = sel < 0 ? 0u : ((uint32_t)sel >= a.E ? a.E - 1u : (uint32_t)sel);
+  const float dw = own ? a.d_weights[(size_t)t * a.top_k + lane] : 0.0f;
+  const float ps = own ? tab[wave][se] : 0.0f;
+  float dps = dw;
+  if (a.norm) {
+    float tot = ps, dot = 0.0f;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) tot += __shfl_xor(tot, off);
+    dot = dw * (ps / tot);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off);
+    dps = (dw - dot) / tot;
+  }
+  float s = own ? ps * dps : 0.0f;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off);
+  __builtin_amdgcn_wave_barrier();  // every lane has read its probability
+#pragma unroll
+  for (uint32_t j = 0; j < NV; ++j) {
+    const uint32_t e = j * 64u + lane;
+    if (e < a.E) tab[wave][e] = 0.0f;
+  }
+  __builtin_amdgcn_s_waitcnt(0xc07f);
+  __builtin_amdgcn_wave_barrier();
+  if (own) tab[wave][se] = dps;  // the selection holds distinct experts
+  __builtin_amdgcn_s_waitcnt(0xc07f);
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (uint32_t j = 0; j < NV; ++j) {
+    const uint32_t e = j * 64u + lane;
+    if (e < a.E) a.d_logits[(size_t)t * a.E + e] = v[j] * (tab[wave][e] - s);
   }
 }
 

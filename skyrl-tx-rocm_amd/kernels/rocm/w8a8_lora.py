@@ -1037,6 +1037,48 @@ def moe_route(router_logits: torch.Tensor, top_k: int, norm_topk_prob: bool = Tr
     return weights, selected
 
 
+def moe_route_backward(router_logits: torch.Tensor, selected: torch.Tensor, d_weights: torch.Tensor,
+                       norm_topk_prob: bool = True) -> torch.Tensor:
+    """Cotangent of the router logits from the cotangent of the routing weights, the selection held
+    fixed as ``lax.top_k`` does (the derivative of qwen3.py:175-178).  float32 [T, E]."""
+    _require_cuda(router_logits, "router_logits")
+    if router_logits.ndim != 2 or tuple(selected.shape) != tuple(d_weights.shape) or selected.ndim != 2 or \
+            selected.shape[0] != router_logits.shape[0]:
+        raise ValueError(f"need router_logits [T, E] and selected, d_weights [T, top_k], got "
+                         f"{tuple(router_logits.shape)}, {tuple(selected.shape)}, {tuple(d_weights.shape)}")
+    _validate_exact_bool("norm_topk_prob", norm_topk_prob)
+    dev = router_logits.device
+    logits = router_logits.detach().to(torch.float32).contiguous()
+    sel = selected.to(device=dev, dtype=torch.int32).contiguous()
+    dw = d_weights.detach().to(device=dev, dtype=torch.float32).contiguous()
+    t, e = logits.shape
+    out = torch.empty_like(logits)
+    with torch.cuda.device(dev):
+        status = _native.load().mi355_w8a8_moe_route_bwd_v1(logits.data_ptr(), sel.data_ptr(), dw.data_ptr(), t, e,
+                                                            sel.shape[1], int(norm_topk_prob), out.data_ptr(),
+                                                            _stream_ptr(dev))
+    _native.check("mi355_w8a8_moe_route_bwd_v1", status)
+    return out
+
+
+class _MoeRouteFunction(torch.autograd.Function):
+    """``moe_route`` whose weights are differentiable in the logits (the indices are not)."""
+
+    @staticmethod
+    def forward(ctx, router_logits, top_k, norm_topk_prob):
+        weights, selected = moe_route(router_logits, top_k, norm_topk_prob)
+        ctx.save_for_backward(router_logits, selected)
+        ctx.norm = norm_topk_prob
+        ctx.mark_non_differentiable(selected)
+        return weights, selected
+
+    @staticmethod
+    def backward(ctx, d_weights, _d_selected):
+        router_logits, selected = ctx.saved_tensors
+        d_logits = moe_route_backward(router_logits, selected, d_weights.contiguous(), ctx.norm)
+        return d_logits.reshape(router_logits.shape).to(router_logits.dtype), None, None
+
+
 def moe_dispatch(tokens: torch.Tensor | None, indices: torch.Tensor, num_groups: int, *, repeat: int = 1,
                  adapter_indices: torch.Tensor | None = None):
     """Stable sort of rows by group with the gather of their token rows, on the device and without a
@@ -1226,24 +1268,21 @@ def moe_expert_mlp(hidden, router_logits, top_k: int, gate_up_weight, down_weigh
     held fixed as ``lax.top_k`` does) and the LoRA factors and scaling."""
     n_experts = gate_up_weight.n_weights
     h2 = hidden.reshape(-1, hidden.shape[-1])
-    weights, selected = moe_route(router_logits, top_k, norm_topk_prob)
     tensors = [t for t in (hidden, router_logits, gate_up_a, gate_up_b, down_a, down_b, lora_scaling)
                if isinstance(t, torch.Tensor)]
-    if not (torch.is_grad_enabled() and any(t.requires_grad for t in tensors)):
+    training = torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
+    logits2 = router_logits.reshape(-1, router_logits.shape[-1])
+    if training and router_logits.requires_grad:
+        weights, selected = _MoeRouteFunction.apply(logits2, top_k, norm_topk_prob)
+    else:
+        weights, selected = moe_route(logits2, top_k, norm_topk_prob)
+    if not training:
         # indices only: the first projection gathers the hidden rows itself through the sort order
         _, group_sizes, sort_indices, unsort, _ = moe_dispatch(None, selected, n_experts, repeat=top_k)
         act = grouped_forward(h2, group_sizes, gate_up_weight, gate_up_a, gate_up_b, lora_scaling, swiglu=True,
                               row_map=sort_indices, row_repeat=top_k)
         down = grouped_forward(act, group_sizes, down_weight, down_a, down_b, lora_scaling)
         return moe_combine(down, unsort, weights).reshape(hidden.shape)
-    if router_logits.requires_grad:
-        # the routing weights as a differentiable function of the logits with the native selection:
-        # the values are the native ones, the derivative that of softmax -> gather -> renormalise
-        probs = torch.softmax(router_logits.reshape(-1, router_logits.shape[-1]).to(torch.float32), dim=-1)
-        picked = probs.gather(1, selected.to(torch.int64))
-        if norm_topk_prob:
-            picked = picked / picked.sum(dim=-1, keepdim=True)
-        weights = picked + (weights - picked).detach()
     scaling = lora_scaling
     if gate_up_a is not None and not isinstance(scaling, torch.Tensor):
         scaling = torch.as_tensor(scaling, dtype=torch.float32, device=hidden.device)
@@ -1714,6 +1753,6 @@ __all__ = (
     "w8a8_lora_linear", "w8a8_rms_gate_up_lora_swiglu", "w8a8_lora_residual", "PackedGroupedW8Weight",
     "prepare_grouped_weight", "grouped_forward", "grouped_backward", "grouped_backward_per_weight",
     "GroupedBackwardPlan", "grouped_lora_linear",
-    "w8a8_grouped_lora_linear", "w8a8_moe_expert_mlp", "moe_expert_mlp", "moe_combine_backward", "Qwen35QKVStageConfig", "QkvPostPlan", "qkv_split_norm_rope",
+    "w8a8_grouped_lora_linear", "w8a8_moe_expert_mlp", "moe_expert_mlp", "moe_combine_backward", "moe_route_backward", "Qwen35QKVStageConfig", "QkvPostPlan", "qkv_split_norm_rope",
     "w8a8_qkv_lora_rope", "qkv_lora_rope", "qkv_split_norm_rope_backward", "delta_rms_norm_backward", "QkvStageBackwardPlan",
 )

@@ -62,6 +62,35 @@ def test_combine_backward_matches_oracle(dev, pkg, t, k, width):
     assert none is None and torch.equal(only, d_e)
 
 
+@pytest.mark.parametrize("t,e,k,norm", [(1, 2, 1, True), (37, 12, 4, True), (300, 128, 8, True), (64, 130, 8, False),
+                                        (9, 1000, 64, True)])
+def test_route_backward_matches_oracle(dev, pkg, t, e, k, norm):
+    import torch
+
+    w8 = pkg.w8a8_lora
+    rng = np.random.default_rng(t + e)
+    logits = (rng.standard_normal((t, e)) * 2.0).astype(F32)
+    dw = rng.standard_normal((t, k)).astype(F32)
+    print(f"[case] route backward t={t} e={e} k={k} norm={norm}", flush=True)
+    lt = torch.from_numpy(logits).to(dev)
+    _, sel = w8.moe_route(lt, k, norm)
+    got = _np(w8.moe_route_backward(lt, sel, torch.from_numpy(dw).to(dev), norm))
+    want = o.moe_route_bwd(logits, sel.cpu().numpy(), dw, norm)
+    scale = max(float(np.abs(want).max()), 1e-6)
+    assert np.abs(got - want).max() <= 2e-5 * scale + 1e-9, float(np.abs(got - want).max()) / scale
+    assert np.abs(got.sum(-1)).max() <= 1e-5 * scale * e ** 0.5     # softmax is shift invariant
+    # through autograd, against torch's own derivative of softmax -> gather -> renormalise
+    la = lt.clone().requires_grad_(True)
+    wts, sel2 = w8._MoeRouteFunction.apply(la, k, norm)
+    assert torch.equal(sel2, sel) and not sel2.requires_grad
+    wts.backward(torch.from_numpy(dw).to(dev))
+    lb = lt.clone().requires_grad_(True)
+    ps = torch.softmax(lb, -1).gather(1, sel.to(torch.int64))
+    (ps / ps.sum(-1, keepdim=True) if norm else ps).backward(torch.from_numpy(dw).to(dev))
+    torch.cuda.synchronize()
+    assert float((la.grad - lb.grad).abs().max()) <= 2e-5 * scale + 1e-9
+
+
 def _mlp_case(seed, t, e, h, inter, r):
     rng = np.random.default_rng(seed)
     hidden = o.bf16_round(rng.standard_normal((t, h)).astype(F32))
