@@ -80,6 +80,14 @@ MEASURED_TRAFFIC_BYTES = {
     "qwen3-8b-gate_up-m4096": int((389417 * 2.0 + 129536) * 1024),                      # w8a8_gemm_kernel
     "qwen3-8b-down-m16-decode": int(((8614 + 27632) * 2.0 + 4529 + 128) * 1024),       # both decode kernels
     "qwen3-8b-gate_up-m4096-backward": int((400599 * 2.0 + 44726) * 1024),             # bwd_dx_kernel
+    "qwen3-30b-a3b-moe-mlp-t2048": int((250936 * 2.0 + 32332) * 1024),                 # grouped gate/up w8a8_gemm_kernel
+    # bwd_pack_dy_kernel + bwd_dx_kernel of the gate/up call without LoRA
+    "qwen3-30b-a3b-moe-experts-t2048-backward": int(((25875 + 225514) * 2.0 + 55008 + 66048) * 1024),
+    "qwen3-8b-gate_up-m4096-fused-backward": int((396251 * 2.0 + 35991) * 1024),       # bwd_dx_kernel
+    "qwen3-8b-down-m4096-w4a8-g128": int((233437 * 2.0 + 32768) * 1024),               # gq_gemm_kernel
+    "qwen3-30b-a3b-moe-routing-t4096": int((8487 * 2.0 + 131472) * 1024),              # the four dispatch kernels
+    "qwen3.5-4b-qkv-m2048": int((20611 * 2.0 + 40960) * 1024),                          # qkv_post_kernel
+    "qwen3.5-4b-qkv-m2048-backward": int((30830 * 2.0 + 40960) * 1024),                 # qkv_post_bwd_kernel
 }
 
 
@@ -303,7 +311,7 @@ def bench_fused_backward(args, cfg, pkg, dev):
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / BF16_PEAK_TFLOPS, "traffic": None, "kernel": "bwd_dx_kernel",
+                     "frac": achieved / BF16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "kernel": "bwd_dx_kernel",
                      "kernel_avg_ms": float(k_ms.mean()), "kernel_min_ms": float(k_ms.min()),
                      "algorithmic_flops": flops, "algorithmic_bytes": 2 * m * n + k * n + 2 * m * k},
         "stages": {
@@ -397,8 +405,8 @@ def bench_moe_routing(args, cfg, pkg, dev):
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": "moe_hist_kernel + moe_scan_kernel + moe_scatter_kernel + moe_gather_kernel (one dispatch call)",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "kernel": "moe_hist_kernel + moe_scan_kernel + moe_scatter_kernel + moe_spread_kernel (one dispatch call)",
                      "kernel_avg_ms": dispatch_ms, "algorithmic_bytes": dispatch_bytes},
         "stages": {"route_ms": route_ms, "route_bytes": route_bytes, "dispatch_ms": dispatch_ms,
                    "combine_ms": combine_ms, "combine_bytes": combine_bytes,
@@ -431,8 +439,10 @@ def bench_moe_routing(args, cfg, pkg, dev):
 def bench_moe_mlp(args, cfg, pkg, dev):
     """One step = the whole expert MLP: route, dispatch (indices only), grouped gate/up + SwiGLU
     (reading the hidden rows through the sort order), grouped down, combine.  ``value`` counts the
-    integer GEMM work 2 * T * top_k * (H * 2I + I * H); the roofline prices the grouped gate/up call
-    (its GEMM kernel dominates) against int8 MFMA peak from HIP events around that call."""
+    integer GEMM work 2 * T * top_k * (H * 2I + I * H); the roofline prices the GEMM kernel
+    of the grouped gate/up call (the dominant kernel) from HIP events around that kernel alone.  With 128
+    rows per expert the kernel is bound by the int8 weights it streams (HBM), not by the matrix cores; the
+    fraction of the int8 MFMA peak is reported next to it."""
     import torch
 
     from oracle import w8a8_oracle as o
@@ -490,18 +500,27 @@ def bench_moe_mlp(args, cfg, pkg, dev):
         "combine_ms": timed(lambda: w8.moe_combine(down, unsort, weights)),
     }
     gu_ops = 2.0 * p * h * 2 * inter
-    achieved = gu_ops / (stages["gate_up_ms"] * 1e-3) / 1e12
+    # the gate/up GEMM kernel alone: the plan's workspace keeps the prologue's tables and codes
+    gu_plan = w8.GroupedForwardPlan(hidden_t, sizes, guw, gua_t, gub_t, 1.0, swiglu=True, row_map=sort_i, row_repeat=k)
+    gu_plan.run()
+    gemm_ms = timed(lambda: gu_plan.run(pkg._native.FLAG_SKIP_PROLOGUE))
+    stages["gate_up_gemm_kernel_ms"] = gemm_ms
+    # every expert's int8 weight once, the codes and row scales, the channel scales, LoRA B and the three bf16
+    # terms of x.A per row, the bf16 product out.  At 128 rows per expert the weights are 87 % of it: 3.4 int8
+    # ops per byte at the two peaks' ratio of 625, so HBM is the roofline that bounds the kernel
+    gemm_bytes = e * h * 2 * inter + p * h + 4 * p + 4 * e * 2 * inter + 2 * e * r * 2 * inter + 6 * p * r + 2 * p * inter
+    achieved = gemm_bytes / (gemm_ms * 1e-3) / 1e9
     result = {
         "metric": "grouped W8A8-LoRA expert MLP (route, dispatch, gate/up + SwiGLU, down, combine), TOPS of the integer GEMM work",
         "value": ops / (ms_per_step * 1e-3) / 1e12, "unit": "TOPS", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
-        "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-                     "frac": achieved / INT8_PEAK_TOPS, "traffic": None,
-                     "kernel": "the grouped gate/up call (route_groups, quant_rows, lora_prep, lora_a, w8a8_gemm_kernel "
-                               "in grouped mode)",
-                     "kernel_avg_ms": stages["gate_up_ms"], "algorithmic_ops": gu_ops},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "kernel": "w8a8_gemm_kernel in grouped mode, gate/up projection with the SwiGLU epilogue",
+                     "kernel_avg_ms": gemm_ms, "algorithmic_bytes": gemm_bytes, "algorithmic_ops": gu_ops,
+                     "frac_of_int8_mfma_peak": gu_ops / (gemm_ms * 1e-3) / 1e12 / INT8_PEAK_TOPS},
         "stages": stages,
     }
     if not args.no_cpu_baseline:
@@ -524,8 +543,9 @@ def bench_moe_backward(args, cfg, pkg, dev):
     """One step = the backward of the two grouped expert projections (gate/up without SwiGLU, down) over
     the sorted (token, choice) pairs: dx and dA, dB, dscaling for every expert, one native call per
     projection.  ``value`` counts the pull-backs' 2 * P * (H * 2I + I * H); the roofline prices
-    bwd_dx_kernel of the gate/up call against the bf16 MFMA peak on the rows that exist (tiles are
-    padded to 256 slots per expert, which the figure charges to the kernel)."""
+    the gate/up call without LoRA (tables, dy packing, bwd_dx_kernel) on the rows that exist.  With 128
+    rows per expert the call is bound by the int8 weights it streams (HBM: 65 us of traffic against 41 us
+    of bf16 MFMA work at the two peaks); the fraction of the bf16 MFMA peak is reported next to it."""
     import torch
 
     from oracle import w8a8_oracle as o
@@ -602,7 +622,10 @@ def bench_moe_backward(args, cfg, pkg, dev):
     layer_ms = (time.perf_counter() - t1) / 10 * 1e3
     flops = 2.0 * p_rows * (h * 2 * inter + inter * h)
     gu_flops = 2.0 * p_rows * h * 2 * inter
-    achieved = gu_flops / (float(dx_ms.mean()) * 1e-3) / 1e12
+    # every expert's int8 weight once, dy in, dx out: at 128 rows per expert 5 ms of HBM time per ms of bf16
+    # MFMA time at the two peaks, so HBM is the roofline that bounds the pull-back
+    dx_bytes = e * h * 2 * inter + 2 * p_rows * 2 * inter + 2 * p_rows * h
+    achieved = dx_bytes / (float(dx_ms.mean()) * 1e-3) / 1e9
     result = {
         "metric": "backward of the grouped W8A8-LoRA expert projections (dx + LoRA cotangents, gate/up and down), "
                   "TFLOP/s of 2*P*K*N per call",
@@ -610,11 +633,12 @@ def bench_moe_backward(args, cfg, pkg, dev):
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
-        "roofline": {"bound": "mfma", "achieved": achieved, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / BF16_PEAK_TFLOPS, "traffic": None,
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
                      "kernel": "the gate/up call without LoRA (tables, bwd_pack_dy_kernel, bwd_dx_kernel)",
                      "kernel_avg_ms": float(dx_ms.mean()), "kernel_min_ms": float(dx_ms.min()),
-                     "algorithmic_flops": gu_flops},
+                     "algorithmic_bytes": dx_bytes, "algorithmic_flops": gu_flops,
+                     "frac_of_bf16_mfma_peak": gu_flops / (float(dx_ms.mean()) * 1e-3) / 1e12 / BF16_PEAK_TFLOPS},
         "stages": {"gate_up_call_ms": float(gu_ms.mean()), "down_call_ms": float(dn_ms.mean()),
                    "gate_up_one_dense_call_per_expert_ms": float(loop_ms.mean()),
                    "expert_mlp_forward_and_backward_through_autograd_ms": layer_ms},
@@ -699,7 +723,7 @@ def bench_gq(args, cfg, pkg, dev):
         "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-                     "frac": achieved / INT8_PEAK_TOPS, "traffic": None,
+                     "frac": achieved / INT8_PEAK_TOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
                      "kernel": "gq_gemm_kernel (timed with gq_quant_kernel and gq_lora_z_kernel: whole calls)",
                      "kernel_avg_ms": call_ms, "algorithmic_ops": ops,
                      "algorithmic_bytes": 2 * m * k + k * n * wb // 8 + 4 * (k // group) * n + 2 * m * n},
@@ -776,7 +800,8 @@ def bench_qkv(args, cfg, pkg, dev):
         "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": "qkv_post_kernel",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "kernel": "qkv_post_kernel",
                      "kernel_avg_ms": float(k_ms.mean()), "kernel_min_ms": float(k_ms.min()),
                      "algorithmic_bytes": bytes_alg},
     }
@@ -888,7 +913,8 @@ def bench_qkv_backward(args, cfg, pkg, dev):
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": "qkv_post_bwd_kernel",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "kernel": "qkv_post_bwd_kernel",
                      "kernel_avg_ms": float(k_ms.mean()), "kernel_min_ms": float(k_ms.min()),
                      "algorithmic_bytes": bytes_alg},
         "stages": {
@@ -965,6 +991,13 @@ def main() -> int:
     for item in filter(None, args.override.split(",")):
         key, val = item.split("=")
         cfg[key] = int(val)
+    if args.calibration_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     if cfg.pop("backward", False):
         if cfg.get("swiglu"):
             return bench_fused_backward(args, cfg, pkg, dev)
@@ -996,13 +1029,6 @@ def main() -> int:
                                     flags=args.flags))
     plan = plans[0]
     torch.cuda.synchronize()
-    if args.calibration_copy:
-        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
-        dst = torch.empty_like(src)
-        torch.cuda.synchronize()
-        dst.copy_(src)
-        torch.cuda.synchronize()
-
     for i in range(args.warmup):
         plans[i % rotate].run()
     torch.cuda.synchronize()

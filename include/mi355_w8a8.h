@@ -118,7 +118,8 @@ typedef struct mi355_w8a8_problem {
  */
 typedef struct mi355_w8a8_grouped_problem {
   uint32_t struct_size;     /* sizeof(mi355_w8a8_grouped_problem) */
-  uint32_t flags;           /* MI355_W8A8_FLAG_SWIGLU, _GROUPED_TILE64 / _GROUPED_TILE128 allowed */
+  uint32_t flags;           /* MI355_W8A8_FLAG_SWIGLU, _GROUPED_TILE64 / _GROUPED_TILE128, and for measurement
+                             * _SKIP_PROLOGUE / _SKIP_GEMM (same arguments and workspace as the full call before) */
   uint32_t m;               /* total rows */
   uint32_t k;
   uint32_t n;

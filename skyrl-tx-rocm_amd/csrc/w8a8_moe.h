@@ -9,6 +9,7 @@
 //   moe_scan_kernel            one workgroup: group sizes, group starts, per-chunk offsets
 //   moe_scatter_kernel         per chunk: stable position of every pair, the index arrays
 //   moe_gather_kernel          a wave per sorted row: the token rows copied to their positions
+//   moe_spread_kernel          the same copy, a wave per token, when a token goes to several groups
 //   moe_combine_kernel         one workgroup per token: sum_j expert_out[unsort[t k + j]] * w[t, j]
 //   moe_combine_bwd_kernel     a wave per sorted row: the cotangents of expert_out and of w
 #pragma once
@@ -280,6 +281,30 @@ __global__ __launch_bounds__(256) void moe_gather_kernel(MoeSortArgs a) {
     uint16_t* out = a.sorted_tokens + (size_t)pos * a.width;
     for (uint32_t c = lane * 8u; c < a.width; c += 512u)
       *reinterpret_cast<uint4*>(out + c) = *reinterpret_cast<const uint4*>(src + c);
+  }
+}
+
+// The same rows written from the token's side when every token goes to several groups
+// (repeat > 1): sorted_tokens[unsort_indices[t * repeat + j]] = tokens[t].  A wave per token
+// reads the row once and stores it `repeat` times; the gather form reads it once per pair,
+// and those reads miss the caches because the copies of a token lie far apart in the sorted order.
+__global__ __launch_bounds__(256) void moe_spread_kernel(MoeSortArgs a) {
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  const uint32_t t = blockIdx.x * 4u + wave;
+  if (t >= a.P / a.repeat) return;
+  const uint16_t* src = a.tokens + (size_t)t * a.width;
+  const int32_t* dst = a.unsort_indices + (size_t)t * a.repeat;
+  for (uint32_t c0 = lane * 8u; c0 < a.width; c0 += 2048u) {  // four 16-byte pieces per lane and round
+    uint4 v[4];
+#pragma unroll
+    for (uint32_t u = 0; u < 4; ++u)
+      if (c0 + u * 512u < a.width) v[u] = *reinterpret_cast<const uint4*>(src + c0 + u * 512u);
+    for (uint32_t j = 0; j < a.repeat; ++j) {
+      uint16_t* out = a.sorted_tokens + (size_t)(uint32_t)dst[j] * a.width;
+#pragma unroll
+      for (uint32_t u = 0; u < 4; ++u)
+        if (c0 + u * 512u < a.width) *reinterpret_cast<uint4*>(out + c0 + u * 512u) = v[u];
+    }
   }
 }
 

@@ -19,6 +19,7 @@ stream.  There is no CPU or eager fallback.
 from __future__ import annotations
 
 import ctypes
+import functools
 import math
 import threading
 import weakref
@@ -174,6 +175,30 @@ def dynamic_quantize_rows(x: torch.Tensor):
 # the forward call
 # ---------------------------------------------------------------------------------------
 
+@functools.lru_cache(maxsize=256)
+def _constant_scaling(value: float, count: int, device: str) -> torch.Tensor:
+    return torch.full((count,), value, dtype=torch.float32, device=torch.device(device))
+
+
+def _scaling_vector(lora_scaling, count: int, device) -> torch.Tensor:
+    """FP32 [count] on ``device``.  A Python number becomes one cached constant vector per (value, count,
+    device): converting it at every call would be a host-to-device copy the host has to wait for, in
+    front of every native call.  The cached vectors are inputs only; nothing writes them."""
+    if isinstance(lora_scaling, (int, float)) and not isinstance(lora_scaling, bool):
+        return _constant_scaling(float(lora_scaling), count, str(device))
+    s = torch.as_tensor(lora_scaling, dtype=torch.float32, device=device)
+    if s.ndim == 0:
+        s = s.reshape(1).expand(count)
+    return s.contiguous()
+
+
+def _scaling_scalar(lora_scaling, device) -> torch.Tensor:
+    """FP32 tensor on ``device`` for the autograd functions; a Python number comes from the constant cache."""
+    if isinstance(lora_scaling, (int, float)) and not isinstance(lora_scaling, bool):
+        return _constant_scaling(float(lora_scaling), 1, str(device)).reshape(())
+    return torch.as_tensor(lora_scaling, dtype=torch.float32, device=device)
+
+
 def _normalize_lora(lora_a, lora_b, lora_scaling, k: int, n: int, device):
     """Return stacked (A [n_ad,K,r], B [n_ad,r,N], s [n_ad]) bf16/bf16/f32 tensors."""
     if lora_a is None and lora_b is None:
@@ -194,12 +219,10 @@ def _normalize_lora(lora_a, lora_b, lora_scaling, k: int, n: int, device):
         raise ValueError(f"LoRA rank must be in [1, {MAX_LORA_RANK}], got {r}")
     if n_ad > MAX_ADAPTERS:
         raise ValueError(f"at most {MAX_ADAPTERS} adapters are supported, got {n_ad}")
-    s = torch.as_tensor(lora_scaling, dtype=torch.float32, device=device)
-    if s.ndim == 0:
-        s = s.reshape(1).expand(n_ad)
+    s = _scaling_vector(lora_scaling, n_ad, device)
     if tuple(s.shape) != (n_ad,):
         raise ValueError(f"lora_scaling must be a scalar or have shape ({n_ad},), got {tuple(s.shape)}")
-    return a3.contiguous(), b3.contiguous(), s.contiguous(), n_ad, r
+    return a3.contiguous(), b3.contiguous(), s, n_ad, r
 
 
 class ForwardPlan:
@@ -471,7 +494,7 @@ def lora_linear(x: torch.Tensor, weight, lora_a=None, lora_b=None, lora_scaling=
                        residual=residual, entry="linear" if residual is None else "residual")
     scaling = lora_scaling
     if lora_a is not None and not isinstance(scaling, torch.Tensor):
-        scaling = torch.as_tensor(scaling, dtype=torch.float32, device=x.device)
+        scaling = _scaling_scalar(scaling, x.device)
     return _LoraLinearFunction.apply(x, lora_a, lora_b, scaling, weight, adapter_indices, residual)
 
 
@@ -688,7 +711,7 @@ def rms_gate_up_lora_swiglu(x: torch.Tensor, gamma: torch.Tensor, weight, lora_a
                        rms_gamma=gamma, eps=eps, swiglu=True, entry="gateup")
     scaling = lora_scaling
     if lora_a is not None and not isinstance(scaling, torch.Tensor):
-        scaling = torch.as_tensor(scaling, dtype=torch.float32, device=x.device)
+        scaling = _scaling_scalar(scaling, x.device)
     return _RmsGateUpFunction.apply(x, lora_a, lora_b, scaling, gamma, weight, adapter_indices, eps, save_projection)
 
 
@@ -729,95 +752,126 @@ def prepare_grouped_weight(codes: torch.Tensor, scales: torch.Tensor) -> PackedG
                                  n_weights=e, in_features=k, out_features=n)
 
 
-def grouped_forward(x: torch.Tensor, group_sizes: torch.Tensor, weight: PackedGroupedW8Weight, lora_a=None,
-                    lora_b=None, lora_scaling=None, *, swiglu: bool = False, groups_per_weight: int = 1,
-                    flags: int = 0, return_aux: bool = False, row_map: torch.Tensor | None = None,
-                    row_repeat: int = 1):
-    """Ragged W8A8 (+LoRA) linear: rows of ``x`` are sorted by group; group g owns
-    ``group_sizes[g]`` consecutive rows and uses weight ``g // groups_per_weight`` and LoRA pair g.
-    Rows beyond ``sum(group_sizes)`` give zeros (``lax.ragged_dot`` semantics).
+class GroupedForwardPlan:
+    """Validated arguments, output, workspace and the C struct of one ragged W8A8 (+LoRA) call;
+    ``run()`` is a single C call on torch's current stream that neither allocates nor synchronizes, so
+    it can be captured in a HIP graph.  ``x``, ``group_sizes`` (``plan.group_sizes``), the LoRA tensors
+    and ``row_map`` (``plan.row_map``) are read at every run: rewrite them in place between runs.
+
+    Rows of ``x`` are sorted by group; group g owns ``group_sizes[g]`` consecutive rows and uses weight
+    ``g // groups_per_weight`` and LoRA pair g.  Rows beyond ``sum(group_sizes)`` give zeros
+    (``lax.ragged_dot`` semantics).
 
     With ``row_map`` (int32 [rows]) the call has ``row_map.numel()`` rows and row i is read from
     ``x[row_map[i] // row_repeat]``: the sorted (token, choice) pairs of an expert layer read the
     unsorted hidden states, and no sorted copy of them is ever written."""
-    if x.dtype != torch.bfloat16:
-        raise TypeError(f"x must be BF16, got {x.dtype}")
-    if x.ndim != 2 or x.shape[0] <= 0:
-        raise ValueError(f"x must be [rows, K] with at least one row, got {tuple(x.shape)}")
-    _require_cuda(x, "x")
-    k, n = weight.in_features, weight.out_features
-    if x.shape[1] != k:
-        raise ValueError(f"x K={x.shape[1]} does not match W8 K={k}")
-    dev = x.device
-    flat = x.contiguous()
-    m = flat.shape[0]
-    rmap = None
-    if row_map is not None:
-        if isinstance(row_repeat, bool) or not isinstance(row_repeat, int) or row_repeat < 1:
-            raise ValueError(f"row_repeat must be a positive integer, got {row_repeat!r}")
-        rmap = row_map.reshape(-1).to(device=dev, dtype=torch.int32).contiguous()
-        m = rmap.numel()
-        if m <= 0 or m > flat.shape[0] * row_repeat:
-            raise ValueError(f"row_map with {m} entries does not fit {flat.shape[0]} rows x {row_repeat}")
-    gs = group_sizes.to(device=dev, dtype=torch.int32).contiguous()
-    n_groups = gs.numel()
-    if n_groups != weight.n_weights * groups_per_weight:
-        raise ValueError(f"{n_groups} groups do not match {weight.n_weights} weights x {groups_per_weight}")
-    a3 = b3 = s1 = None
-    r = 0
-    if lora_a is not None:
-        if lora_a.dtype != torch.bfloat16 or lora_b.dtype != torch.bfloat16:
-            raise TypeError("LoRA A and B must both be BF16")
-        if lora_a.ndim != 3 or lora_b.ndim != 3 or lora_a.shape[0] != n_groups or lora_a.shape[1] != k:
-            raise ValueError(f"grouped lora_a must be [{n_groups}, {k}, r], got {tuple(lora_a.shape)}")
-        r = lora_a.shape[2]
-        if tuple(lora_b.shape) != (n_groups, r, n):
-            raise ValueError(f"grouped lora_b must be [{n_groups}, {r}, {n}], got {tuple(lora_b.shape)}")
-        if r < 1 or r > MAX_LORA_RANK:
-            raise ValueError(f"LoRA rank must be in [1, {MAX_LORA_RANK}], got {r}")
-        a3, b3 = lora_a.contiguous(), lora_b.contiguous()
-        s1 = torch.as_tensor(lora_scaling, dtype=torch.float32, device=dev)
-        s1 = (s1.reshape(1).expand(n_groups) if s1.ndim == 0 else s1).contiguous()
-        if tuple(s1.shape) != (n_groups,):
-            raise ValueError(f"lora_scaling must be a scalar or have shape ({n_groups},)")
-    if swiglu and n % 2:
-        raise ValueError("SwiGLU needs an even number of fused gate/up columns")
-    n_out = n // 2 if swiglu else n
-    lib = _native.load()
-    if swiglu:
-        flags |= _native.FLAG_SWIGLU
-    ws_bytes = int(lib.mi355_w8a8_grouped_workspace_bytes(m, k, n, n_groups, r, flags))
-    if ws_bytes == 0:
-        raise ValueError(f"geometry M={m}, K={k}, N={n}, groups={n_groups}, rank={r} is outside the native path")
-    out = torch.empty((m, n_out), dtype=torch.bfloat16, device=dev)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-    aux = {}
-    if return_aux:
-        aux["x_codes"] = torch.empty((m, k), dtype=torch.int8, device=dev)
-        aux["x_scales"] = torch.empty((m,), dtype=torch.float32, device=dev)
-        aux["acc"] = torch.zeros((m, n), dtype=torch.int32, device=dev)
-    p = _native.GroupedProblem()
-    p.struct_size = ctypes.sizeof(_native.GroupedProblem)
-    p.flags = flags
-    p.m, p.k, p.n, p.n_groups, p.rank, p.groups_per_weight = m, k, n, n_groups, r, groups_per_weight
-    p.x = flat.data_ptr()
-    p.w_packed = weight.packed.data_ptr()
-    p.w_scales = weight.scales.data_ptr()
-    p.lora_a = a3.data_ptr() if r else None
-    p.lora_b = b3.data_ptr() if r else None
-    p.lora_scaling = s1.data_ptr() if r else None
-    p.group_sizes = gs.data_ptr()
-    p.out = out.data_ptr()
-    p.workspace = ws.data_ptr()
-    p.workspace_bytes = ws_bytes
-    p.aux_x_codes = aux["x_codes"].data_ptr() if return_aux else None
-    p.aux_x_scales = aux["x_scales"].data_ptr() if return_aux else None
-    p.aux_acc = aux["acc"].data_ptr() if return_aux else None
-    p.x_row_map = rmap.data_ptr() if rmap is not None else None
-    p.x_row_repeat = row_repeat if rmap is not None else 0
-    with torch.cuda.device(dev):
-        _native.check("mi355_w8a8_grouped_v1", lib.mi355_w8a8_grouped_v1(ctypes.byref(p), _stream_ptr(dev)))
-    return (out, aux) if return_aux else out
+
+    def __init__(self, x: torch.Tensor, group_sizes: torch.Tensor, weight: PackedGroupedW8Weight, lora_a=None,
+                 lora_b=None, lora_scaling=None, *, swiglu: bool = False, groups_per_weight: int = 1,
+                 flags: int = 0, return_aux: bool = False, row_map: torch.Tensor | None = None,
+                 row_repeat: int = 1):
+        if x.dtype != torch.bfloat16:
+            raise TypeError(f"x must be BF16, got {x.dtype}")
+        if x.ndim != 2 or x.shape[0] <= 0:
+            raise ValueError(f"x must be [rows, K] with at least one row, got {tuple(x.shape)}")
+        _require_cuda(x, "x")
+        k, n = weight.in_features, weight.out_features
+        if x.shape[1] != k:
+            raise ValueError(f"x K={x.shape[1]} does not match W8 K={k}")
+        dev = x.device
+        flat = x.contiguous()
+        m = flat.shape[0]
+        rmap = None
+        if row_map is not None:
+            if isinstance(row_repeat, bool) or not isinstance(row_repeat, int) or row_repeat < 1:
+                raise ValueError(f"row_repeat must be a positive integer, got {row_repeat!r}")
+            rmap = row_map.reshape(-1).to(device=dev, dtype=torch.int32).contiguous()
+            m = rmap.numel()
+            if m <= 0 or m > flat.shape[0] * row_repeat:
+                raise ValueError(f"row_map with {m} entries does not fit {flat.shape[0]} rows x {row_repeat}")
+        gs = group_sizes.to(device=dev, dtype=torch.int32).contiguous()
+        n_groups = gs.numel()
+        if n_groups != weight.n_weights * groups_per_weight:
+            raise ValueError(f"{n_groups} groups do not match {weight.n_weights} weights x {groups_per_weight}")
+        a3 = b3 = s1 = None
+        r = 0
+        if lora_a is not None:
+            if lora_a.dtype != torch.bfloat16 or lora_b.dtype != torch.bfloat16:
+                raise TypeError("LoRA A and B must both be BF16")
+            if lora_a.ndim != 3 or lora_b.ndim != 3 or lora_a.shape[0] != n_groups or lora_a.shape[1] != k:
+                raise ValueError(f"grouped lora_a must be [{n_groups}, {k}, r], got {tuple(lora_a.shape)}")
+            r = lora_a.shape[2]
+            if tuple(lora_b.shape) != (n_groups, r, n):
+                raise ValueError(f"grouped lora_b must be [{n_groups}, {r}, {n}], got {tuple(lora_b.shape)}")
+            if r < 1 or r > MAX_LORA_RANK:
+                raise ValueError(f"LoRA rank must be in [1, {MAX_LORA_RANK}], got {r}")
+            a3, b3 = lora_a.contiguous(), lora_b.contiguous()
+            s1 = _scaling_vector(lora_scaling, n_groups, dev)
+            if tuple(s1.shape) != (n_groups,):
+                raise ValueError(f"lora_scaling must be a scalar or have shape ({n_groups},)")
+        if swiglu and n % 2:
+            raise ValueError("SwiGLU needs an even number of fused gate/up columns")
+        n_out = n // 2 if swiglu else n
+        lib = _native.load()
+        if swiglu:
+            flags |= _native.FLAG_SWIGLU
+        ws_bytes = int(lib.mi355_w8a8_grouped_workspace_bytes(m, k, n, n_groups, r, flags))
+        if ws_bytes == 0:
+            raise ValueError(f"geometry M={m}, K={k}, N={n}, groups={n_groups}, rank={r} is outside the native path")
+        self.device = dev
+        self.out = torch.empty((m, n_out), dtype=torch.bfloat16, device=dev)
+        self.workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        self.aux = {}
+        if return_aux:
+            self.aux["x_codes"] = torch.empty((m, k), dtype=torch.int8, device=dev)
+            self.aux["x_scales"] = torch.empty((m,), dtype=torch.float32, device=dev)
+            self.aux["acc"] = torch.zeros((m, n), dtype=torch.int32, device=dev)
+        self.x_flat, self.group_sizes, self.row_map, self.weight = flat, gs, rmap, weight
+        self._keep = (a3, b3, s1)
+        p = _native.GroupedProblem()
+        p.struct_size = ctypes.sizeof(_native.GroupedProblem)
+        p.flags = flags
+        p.m, p.k, p.n, p.n_groups, p.rank, p.groups_per_weight = m, k, n, n_groups, r, groups_per_weight
+        p.x = flat.data_ptr()
+        p.w_packed = weight.packed.data_ptr()
+        p.w_scales = weight.scales.data_ptr()
+        p.lora_a = a3.data_ptr() if r else None
+        p.lora_b = b3.data_ptr() if r else None
+        p.lora_scaling = s1.data_ptr() if r else None
+        p.group_sizes = gs.data_ptr()
+        p.out = self.out.data_ptr()
+        p.workspace = self.workspace.data_ptr()
+        p.workspace_bytes = ws_bytes
+        p.aux_x_codes = self.aux["x_codes"].data_ptr() if return_aux else None
+        p.aux_x_scales = self.aux["x_scales"].data_ptr() if return_aux else None
+        p.aux_acc = self.aux["acc"].data_ptr() if return_aux else None
+        p.x_row_map = rmap.data_ptr() if rmap is not None else None
+        p.x_row_repeat = row_repeat if rmap is not None else 0
+        self.problem = p
+        self.flags = flags
+        self._lib = lib
+
+    def run(self, extra_flags: int = 0) -> torch.Tensor:
+        """Enqueue the call on torch's current stream; returns the (reused) output tensor.  ``extra_flags``
+        adds the measurement flags ``FLAG_SKIP_PROLOGUE`` / ``FLAG_SKIP_GEMM`` for this run."""
+        self.problem.flags = self.flags | extra_flags
+        with torch.cuda.device(self.device):
+            status = self._lib.mi355_w8a8_grouped_v1(ctypes.byref(self.problem), _stream_ptr(self.device))
+        self.problem.flags = self.flags
+        _native.check("mi355_w8a8_grouped_v1", status)
+        return self.out
+
+
+def grouped_forward(x: torch.Tensor, group_sizes: torch.Tensor, weight: PackedGroupedW8Weight, lora_a=None,
+                    lora_b=None, lora_scaling=None, *, swiglu: bool = False, groups_per_weight: int = 1,
+                    flags: int = 0, return_aux: bool = False, row_map: torch.Tensor | None = None,
+                    row_repeat: int = 1):
+    """Ragged W8A8 (+LoRA) linear in one native call: a ``GroupedForwardPlan`` built and run once."""
+    plan = GroupedForwardPlan(x, group_sizes, weight, lora_a, lora_b, lora_scaling, swiglu=swiglu,
+                              groups_per_weight=groups_per_weight, flags=flags, return_aux=return_aux,
+                              row_map=row_map, row_repeat=row_repeat)
+    out = plan.run()
+    return (out, plan.aux) if return_aux else out
 
 
 class GroupedBackwardPlan:
@@ -854,8 +908,7 @@ class GroupedBackwardPlan:
             if r < 1 or r > MAX_LORA_RANK:
                 raise ValueError(f"LoRA rank must be in [1, {MAX_LORA_RANK}], got {r}")
             a3, b3 = lora_a.detach().contiguous(), lora_b.detach().contiguous()
-            s1 = torch.as_tensor(lora_scaling, dtype=torch.float32, device=dev).detach()
-            s1 = (s1.reshape(1).expand(n_groups) if s1.ndim == 0 else s1).contiguous()
+            s1 = _scaling_vector(lora_scaling, n_groups, dev).detach()
             if tuple(s1.shape) != (n_groups,):
                 raise ValueError(f"lora_scaling must be a scalar or have shape ({n_groups},)")
         want = bool(r) and need_lora_grads
@@ -1002,7 +1055,7 @@ def grouped_lora_linear(x, group_sizes, weight, lora_a=None, lora_b=None, lora_s
                                groups_per_weight=groups_per_weight)
     scaling = lora_scaling
     if lora_a is not None and not isinstance(scaling, torch.Tensor):
-        scaling = torch.as_tensor(scaling, dtype=torch.float32, device=x.device)
+        scaling = _scaling_scalar(scaling, x.device)
     return _GroupedLinearFunction.apply(x, lora_a, lora_b, scaling, weight, group_sizes, groups_per_weight)
 
 
@@ -1285,7 +1338,7 @@ def moe_expert_mlp(hidden, router_logits, top_k: int, gate_up_weight, down_weigh
         return moe_combine(down, unsort, weights).reshape(hidden.shape)
     scaling = lora_scaling
     if gate_up_a is not None and not isinstance(scaling, torch.Tensor):
-        scaling = torch.as_tensor(scaling, dtype=torch.float32, device=hidden.device)
+        scaling = _scaling_scalar(scaling, hidden.device)
     out = _MoeExpertMlpFunction.apply(h2, weights, gate_up_a, gate_up_b, down_a, down_b, scaling, selected,
                                       gate_up_weight, down_weight, top_k)
     return out.reshape(hidden.shape)
@@ -1727,7 +1780,7 @@ def qkv_lora_rope(hidden, input_norm_weight, q_norm_weight, k_norm_weight, weigh
         return qkv_split_norm_rope(fused, q_norm_weight, k_norm_weight, positions, config)
     scaling = lora_scaling
     if lora_a is not None and not isinstance(scaling, torch.Tensor):
-        scaling = torch.as_tensor(scaling, dtype=torch.float32, device=hidden.device)
+        scaling = _scaling_scalar(scaling, hidden.device)
     return _QkvStageFunction.apply(hidden, input_norm_weight, q_norm_weight, k_norm_weight, lora_a, lora_b, scaling,
                                    weight, positions, config, adapter_indices, save_projection)
 
@@ -1752,7 +1805,7 @@ __all__ = (
     "w8a8_frozen_linear",
     "w8a8_lora_linear", "w8a8_rms_gate_up_lora_swiglu", "w8a8_lora_residual", "PackedGroupedW8Weight",
     "prepare_grouped_weight", "grouped_forward", "grouped_backward", "grouped_backward_per_weight",
-    "GroupedBackwardPlan", "grouped_lora_linear",
+    "GroupedBackwardPlan", "GroupedForwardPlan", "grouped_lora_linear",
     "w8a8_grouped_lora_linear", "w8a8_moe_expert_mlp", "moe_expert_mlp", "moe_combine_backward", "moe_route_backward", "Qwen35QKVStageConfig", "QkvPostPlan", "qkv_split_norm_rope",
     "w8a8_qkv_lora_rope", "qkv_lora_rope", "qkv_split_norm_rope_backward", "delta_rms_norm_backward", "QkvStageBackwardPlan",
 )

@@ -161,3 +161,46 @@ def test_grouped_backward_plan_replays(dev, pkg):
         plan.group_sizes.copy_(torch.tensor(layouts[i % len(layouts)], dtype=torch.int32))   # the group sizes too
 
     _replays(torch, plan.run, lambda: list(outs), refresh)
+
+
+@pytest.mark.parametrize("swiglu,mapped", [(False, False), (True, True)])
+def test_grouped_forward_plan_replays(dev, pkg, swiglu, mapped):
+    import torch
+
+    w8, native = pkg.w8a8_lora, pkg._native
+    e, k, n, r, rep = 6, 256, 384, 8, 2
+    layouts = [[40, 0, 300, 7, 129, 64], [0, 0, 1, 500, 0, 39], [90, 90, 90, 90, 90, 90], [540, 0, 0, 0, 0, 0]]
+    m = sum(layouts[0]) + 2
+    print(f"[case] graph grouped forward groups={e} m={m} k={k} n={n} swiglu={swiglu} row_map={mapped}", flush=True)
+    codes = torch.randint(-127, 128, (e, k, n), dtype=torch.int8, device=dev)
+    scales = (torch.rand(e, n, device=dev) * 0.8 + 0.2) / (127.0 * k ** 0.5)
+    gw = w8.prepare_grouped_weight(codes, scales)
+    x = torch.randn(m // rep if mapped else m, k, device=dev).to(torch.bfloat16)
+    a = (torch.randn(e, k, r, device=dev) * 0.1).to(torch.bfloat16)
+    b = (torch.randn(e, r, n, device=dev) * 0.1).to(torch.bfloat16)
+    gs = torch.tensor(layouts[0], dtype=torch.int32, device=dev)
+    rmap = torch.randperm(m, device=dev).to(torch.int32) if mapped else None
+    plan = w8.GroupedForwardPlan(x, gs, gw, a, b, torch.ones(e, device=dev), swiglu=swiglu, row_map=rmap,
+                                 row_repeat=rep if mapped else 1)
+    assert plan.x_flat.data_ptr() == x.data_ptr()
+    gen = torch.Generator(device=dev).manual_seed(11)
+
+    def refresh(i):
+        x.copy_(torch.randn(x.shape, device=dev, generator=gen).to(torch.bfloat16) * (1.0 + i))
+        plan.group_sizes.copy_(torch.tensor(layouts[i % len(layouts)], dtype=torch.int32))
+        if mapped:
+            plan.row_map.copy_(torch.randperm(m, device=dev, generator=gen).to(torch.int32))
+
+    _replays(torch, plan.run, lambda: [plan.out], refresh)
+    # the measurement flags: the GEMM kernel alone over the tables the full call left in the workspace
+    rows = sum(layouts[3 % len(layouts)])                # the layout of the last replay
+    want = plan.run().clone()
+    plan.out.fill_(3.0)
+    got = plan.run(native.FLAG_SKIP_PROLOGUE)
+    torch.cuda.synchronize()
+    assert torch.equal(got[:rows], want[:rows])
+    assert bool((got[rows:] == 3.0).all())               # the rows past the groups belong to the prologue
+    plan.out.fill_(3.0)
+    plan.run(native.FLAG_SKIP_GEMM)
+    torch.cuda.synchronize()
+    assert bool((plan.out[:rows] == 3.0).all()) and bool((plan.out[rows:] == 0).all())

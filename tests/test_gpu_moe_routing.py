@@ -78,7 +78,8 @@ def test_route_ties_pick_the_lower_expert(dev, pkg):
 
 
 @pytest.mark.parametrize("t,rep,g,h,with_ad", [(1, 1, 1, 8, False), (50, 2, 8, 64, True), (1000, 8, 128, 256, True),
-                                               (4099, 1, 1024, 16, False), (700, 4, 3, 520, True)])
+                                               (4099, 1, 1024, 16, False), (700, 4, 3, 520, True),
+                                               (33, 3, 5, 2568, False), (257, 8, 16, 4096, False)])
 def test_dispatch_matches_oracle(dev, pkg, t, rep, g, h, with_ad):
     import torch
 
