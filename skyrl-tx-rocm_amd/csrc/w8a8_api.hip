@@ -647,16 +647,21 @@ int validate_bwd_dims(uint32_t m, uint32_t k, uint32_t n, uint32_t n_adapters, u
   return MI355_W8A8_OK;
 }
 
-template <int NKK>
-int launch_bwd_dx(const BwdDxArgs& g, hipStream_t s) {
+template <int NKK, bool ROWS128>
+int launch_bwd_dx_geometry(const BwdDxArgs& g, hipStream_t s) {
   const uint32_t ntile = g.tiles_m * g.tiles_k;
   const uint32_t want = ((ntile + 7u) / 8u) * 8u;
   const dim3 grid(want < 256u ? want : 256u), block(512);
-  if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_dx_kernel<NKK>),
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_dx_kernel<NKK, ROWS128>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLdsBytes) != hipSuccess)
     return MI355_W8A8_ERR_LAUNCH;
-  hipLaunchKernelGGL((bwd_dx_kernel<NKK>), grid, block, kBwdLdsBytes, s, g);
+  hipLaunchKernelGGL((bwd_dx_kernel<NKK, ROWS128>), grid, block, kBwdLdsBytes, s, g);
   return launch_status();
+}
+
+template <int NKK>
+int launch_bwd_dx(const BwdDxArgs& g, bool rows128, hipStream_t s) {
+  return rows128 ? launch_bwd_dx_geometry<NKK, true>(g, s) : launch_bwd_dx_geometry<NKK, false>(g, s);
 }
 
 // The stages of a backward call behind its routing tables: dy into operand order (with the partial
@@ -675,6 +680,7 @@ struct BwdBody {
   const int32_t* tile_weight; const int32_t* chunk_tab; const int32_t* chunk0; const int32_t* group_beg;
   const int32_t* group_end;
   size_t w_stride; uint32_t sw_stride;
+  bool rows128;  // the pull-back runs 128-row x 512-k tiles (the tables are padded to match)
 };
 
 template <class Layout>
@@ -752,10 +758,10 @@ int launch_bwd_body(const BwdBody& b, const Layout& w, unsigned char* ws, hipStr
     g.M = b.m; g.K = b.k; g.KB = w.KB; g.NB = w.NB; g.tiles_m = w.tiles_m; g.tiles_k = w.tiles_k;
     g.tile_weight = b.tile_weight; g.w_stride = b.w_stride; g.sw_stride = b.sw_stride;
     switch (b.lora ? w.nkk : 0u) {
-      case 0: st = launch_bwd_dx<0>(g, s); break;
-      case 1: st = launch_bwd_dx<1>(g, s); break;
-      case 2: st = launch_bwd_dx<2>(g, s); break;
-      default: st = launch_bwd_dx<4>(g, s); break;
+      case 0: st = launch_bwd_dx<0>(g, b.rows128, s); break;
+      case 1: st = launch_bwd_dx<1>(g, b.rows128, s); break;
+      case 2: st = launch_bwd_dx<2>(g, b.rows128, s); break;
+      default: st = launch_bwd_dx<4>(g, b.rows128, s); break;
     }
     if (st) return st;
   }
@@ -884,7 +890,7 @@ struct BwdGroupedLayout {
   uint64_t dyp, swp, src_row, dst_pos, slot_group, blk_range, group_beg, group_end, tile_weight, chunk_tab, chunk0,
       at, ap, rp, z, r_raw, rs, rpart, partA, partB, total;
   uint32_t slots, nkk, K_pad, KB, N_pad, NB, tiles_m, tiles_k, max_chunks, R, n_slices, groups_per_slice, n_weights,
-      gpw, sw_stride;
+      gpw, sw_stride, tile_rows;
 };
 
 BwdGroupedLayout make_bwd_grouped_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint32_t rank,
@@ -894,11 +900,20 @@ BwdGroupedLayout make_bwd_grouped_layout(uint32_t m, uint32_t k, uint32_t n, uin
   w.n_weights = n_groups / w.gpw;
   w.K_pad = k_padded(k); w.KB = w.K_pad / 32u;
   w.N_pad = n_padded(n); w.NB = w.N_pad / 32u;
-  // every weight with rows pads its slots to a multiple of 256
+  // Tile geometry of the pull-back: 256 rows x 256 k, or 128 rows x 512 k (the same area).  The group sizes
+  // live on the device, so the choice goes by the average rows per weight: a weight with r rows takes about
+  // r / rows + 1/2 row tiles, and the geometry with fewer tiles in total wins (ties keep 256 rows).
+  {
+    const double avg = (double)m / (double)w.n_weights;
+    const double t256 = (avg / 256.0 + 0.5) * (double)((w.KB + 7u) / 8u);
+    const double t128 = (avg / 128.0 + 0.5) * (double)((w.KB + 15u) / 16u);
+    w.tile_rows = t128 < t256 ? 128u : 256u;
+  }
+  // every weight with rows pads its slots to a multiple of the tile rows
   const uint32_t with_rows = w.n_weights < m ? w.n_weights : m;
-  w.slots = round_up(m + 255u * with_rows, 256u);
-  w.tiles_m = w.slots / 256u;
-  w.tiles_k = (w.K_pad + 255u) / 256u;
+  w.slots = round_up(m + (w.tile_rows - 1u) * with_rows, 256u);
+  w.tiles_m = w.slots / w.tile_rows;
+  w.tiles_k = w.tile_rows == 128u ? (w.KB + 15u) / 16u : (w.KB + 7u) / 8u;
   w.nkk = rank_chunks(rank);
   w.R = w.nkk > 2u ? 64u : 32u;
   w.max_chunks = (m + kBwdChunkRows - 1u) / kBwdChunkRows + n_groups;
@@ -1004,7 +1019,7 @@ int run_grouped_backward(const mi355_w8a8_grouped_bwd_problem* p, hipStream_t s)
     pa.dx = static_cast<uint16_t*>(p->dx);
     pa.M = p->m; pa.K = p->k; pa.N = p->n; pa.N_pad = w.N_pad; pa.n_groups = p->n_groups; pa.gpw = w.gpw;
     pa.n_weights = w.n_weights; pa.r = p->rank; pa.nkk = w.nkk; pa.kb32 = w.KB; pa.slots = w.slots;
-    pa.max_chunks = w.max_chunks; pa.sw_stride = w.sw_stride;
+    pa.max_chunks = w.max_chunks; pa.sw_stride = w.sw_stride; pa.tile_rows = w.tile_rows;
     pa.a_blocks = lora ? (uint32_t)(((uint64_t)p->n_groups * p->k * ((p->rank + 7u) / 8u) + 1023u) / 1024u) : 0u;
     pa.ap_blocks = lora ? (uint32_t)(((uint64_t)p->n_groups * w.KB * w.nkk * 64u + 1023u) / 1024u) : 0u;
     pa.sw_blocks_per_weight = (w.N_pad + 1023u) / 1024u;
@@ -1022,6 +1037,7 @@ int run_grouped_backward(const mi355_w8a8_grouped_bwd_problem* p, hipStream_t s)
   b.group_beg = tab.group_beg; b.group_end = tab.group_end;
   b.w_stride = (size_t)mi355_w8a8_packed_weight_bytes(p->k, p->n);
   b.sw_stride = w.sw_stride;
+  b.rows128 = w.tile_rows == 128u;
   return launch_bwd_body(b, w, ws, s);
 }
 

@@ -249,13 +249,14 @@ __global__ __launch_bounds__(1024) void bwd_prep_kernel(BwdPrepArgs p) {
 // ---------------------------------------------------------------------------------------
 // Tables of a grouped (per-expert) backward: the rows arrive sorted by group, group g owning
 // group_sizes[g] consecutive rows, and groups_per_weight consecutive groups share a frozen weight
-// (skyrl/tx/layers/lora.py:394-444).  Every weight's rows start at a multiple of 256 slots, so that
+// (skyrl/tx/layers/lora.py:394-444).  Every weight's rows start at a multiple of the pull-back's tile rows
+// (256 slots, or 128 when the weights average few rows), so that
 // a pull-back tile never mixes two weights; inside a weight the groups follow each other without
 // gaps, exactly as the adapters of a dense call over that weight's rows would.
 //   src_row / dst_pos / slot_group / blk_range   as in the dense call; blk_range -1 for 32-slot blocks without a
 //                                                row: no kernel prepares or consumes their operands
 //   group_beg[g], group_end[g]                   slots of group g
-//   tile_weight[t]                               weight of 256-slot tile t | its rows << 16, -1 beyond the slots in use
+//   tile_weight[t]                               weight of tile t | its rows << 16, -1 beyond the slots in use
 //   chunk_tab[c] = (group, first slot, rows)     the 512-row chunks of the LoRA cotangents; rows 0 beyond
 //   chunk0[g]                                    first chunk of group g (n_groups + 1 entries)
 // One workgroup of 1024 threads.  Rows beyond sum(group_sizes) get no slot; their dx rows are cleared.
@@ -267,7 +268,8 @@ struct BwdGroupTables {
 
 __device__ inline void route_weight_groups_block(const int32_t* __restrict__ group_sizes, uint32_t M, uint32_t n_groups,
                                                  uint32_t gpw, uint32_t slots, uint32_t max_chunks, BwdGroupTables t,
-                                                 uint16_t* __restrict__ dx, uint32_t K) {
+                                                 uint16_t* __restrict__ dx, uint32_t K, uint32_t tile_rows) {
+  const int pad = (int)tile_rows;  // 256, or 128 for the pull-back's 128-row tiles
   __shared__ int row_start[kMaxGroups + 1];
   __shared__ int slot_beg[kMaxGroups + 1];
   __shared__ int slot_end[kMaxGroups];
@@ -278,7 +280,7 @@ __device__ inline void route_weight_groups_block(const int32_t* __restrict__ gro
   if (tid == 0) {
     int r = 0, p = 0, ch = 0;
     for (uint32_t g = 0; g < n_groups; ++g) {
-      if (g % gpw == 0) p = (p + 255) & ~255;
+      if (g % gpw == 0) p = (p + pad - 1) & ~(pad - 1);
       int sz = row_start[g];
       if (sz < 0) sz = 0;
       if (r + sz > (int)M) sz = (int)M - r;
@@ -301,7 +303,7 @@ __device__ inline void route_weight_groups_block(const int32_t* __restrict__ gro
   }
   __syncthreads();
   for (uint32_t b = tid; b < slots / 32u; b += 1024) t.blk_range[b] = -1;
-  for (uint32_t tl = tid; tl < slots / 256u; tl += 1024) t.tile_weight[tl] = -1;
+  for (uint32_t tl = tid; tl < slots / tile_rows; tl += 1024) t.tile_weight[tl] = -1;
   for (uint32_t g = tid; g <= n_groups; g += 1024) t.chunk0[g] = chunk_first[g];
   if (tid < n_groups) { t.group_beg[tid] = slot_beg[tid]; t.group_end[tid] = slot_end[tid]; }
   __syncthreads();
@@ -328,12 +330,12 @@ __device__ inline void route_weight_groups_block(const int32_t* __restrict__ gro
     const uint32_t g0 = w * gpw, g1 = g0 + gpw;  // groups of this weight
     const int wb = slot_beg[g0], we = slot_end[g1 - 1];
     if (we == wb) continue;  // no rows: no tile
-    const int wpad = (we + 255) & ~255;
+    const int wpad = (we + pad - 1) & ~(pad - 1);
     int glast = (int)g0;
     for (uint32_t g = g0; g < g1; ++g)
       if (slot_end[g] > slot_beg[g]) glast = (int)g;
-    for (int tl = wb / 256 + (int)lane; tl < wpad / 256; tl += 64) {
-      const int rows = we - tl * 256 < 256 ? we - tl * 256 : 256;
+    for (int tl = wb / pad + (int)lane; tl < wpad / pad; tl += 64) {
+      const int rows = we - tl * pad < pad ? we - tl * pad : pad;
       t.tile_weight[tl] = (int)w | (rows << 16);
     }
     for (int p = we + (int)lane; p < wpad; p += 64) t.slot_group[p] = glast;
@@ -364,12 +366,13 @@ struct BwdGroupedPrepArgs {
   uint16_t* dx;              // rows beyond the groups are cleared
   uint32_t M, K, N, N_pad, n_groups, gpw, n_weights, r, nkk, kb32, slots, max_chunks, sw_stride;
   uint32_t a_blocks, ap_blocks, sw_blocks_per_weight;
+  uint32_t tile_rows;        // slots every weight's rows are padded to: 256 or 128
 };
 
 __global__ __launch_bounds__(1024) void bwd_grouped_prep_kernel(BwdGroupedPrepArgs p) {
   uint32_t b = blockIdx.x;
   if (b == 0) {
-    route_weight_groups_block(p.group_sizes, p.M, p.n_groups, p.gpw, p.slots, p.max_chunks, p.tab, p.dx, p.K);
+    route_weight_groups_block(p.group_sizes, p.M, p.n_groups, p.gpw, p.slots, p.max_chunks, p.tab, p.dx, p.K, p.tile_rows);
     return;
   }
   b -= 1u;
@@ -425,12 +428,19 @@ struct BwdDxArgs {
   uint32_t sw_stride;
 };
 
-template <int NKK>
+// ROWS128: the tile is 128 rows x 512 k (the eight waves side by side along k, the same 128 x 64 wave
+// tile): a stage then holds half the dy panel and twice the weight blocks, the same bytes and the same
+// four loads per wave.  For grouped calls whose weights own few rows each: half the padding per weight,
+// and every wave has rows.
+template <int NKK, bool ROWS128 = false>
 __global__ __launch_bounds__(512, 1) void bwd_dx_kernel(BwdDxArgs g) {
+  constexpr int kRowBlocks = ROWS128 ? 4 : 8, kKBlocks = ROWS128 ? 16 : 8;  // of a tile
+  constexpr int kPanel = kRowBlocks * 2048, kWeight = kKBlocks * kBlockBytes;
+  static_assert(kPanel + kWeight + 1024 == kBwdStageBytes, "a stage keeps its size in both geometries");
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wrow = wave >> 2, wcol = wave & 3;
+  const int wrow = ROWS128 ? 0 : wave >> 2, wcol = ROWS128 ? wave : wave & 3;
   const int c = lane & 31, h = lane >> 5;
   const int NBi = (int)g.NB;  // a multiple of 8
 
@@ -468,7 +478,8 @@ __global__ __launch_bounds__(512, 1) void bwd_dx_kernel(BwdDxArgs g) {
     const uint32_t tm = band * 4u + in_band % band_rows, tk = in_band / band_rows;
     int tw = 0;
     int n_act = 4;  // 32-row blocks of this wave that hold rows: the others skip their matrix-core work
-    uint32_t load_rb = (uint32_t)wave;  // row block whose dy panel chunks this wave fetches
+    // row block whose dy panel this wave fetches: both 1 KiB halves, or one half of it in a 128-row tile
+    uint32_t load_rb = ROWS128 ? (uint32_t)wave >> 1 : (uint32_t)wave;
     if (g.tile_weight) {
       const int tv = g.tile_weight[tm];
       if (tv < 0) continue;  // workgroup-uniform: no row lives in this tile
@@ -478,27 +489,37 @@ __global__ __launch_bounds__(512, 1) void bwd_dx_kernel(BwdDxArgs g) {
       n_act = live < 0 ? 0 : (live > 4 ? 4 : live);
       // a block without rows is never multiplied: its slot is filled from block 0 of the tile, which
       // is in the caches anyway, instead of streaming unused memory (the load count stays the same)
-      if (wave >= live_blocks) load_rb = 0u;
+      if ((int)load_rb >= live_blocks) load_rb = 0u;
     }
     n_act = __builtin_amdgcn_readfirstlane(n_act);
     const float* swp_t = g.swp + (size_t)tw * g.sw_stride;
 
     // this wave's two panel chunks of a stage (row block = wave, halves q = 0, 1) and its weight block
-    const unsigned char* Ag = g.dyp + ((size_t)(tm * 8u + load_rb) * g.NB) * 2048u + lane * 16;
-    const uint32_t kbw = tk * 8u + (uint32_t)wcol * 2u;  // first of the two k blocks this wave multiplies
-    const uint32_t kbl = tk * 8u + (uint32_t)wave < g.KB ? tk * 8u + (uint32_t)wave : g.KB - 1u;  // the block it loads
+    const unsigned char* Ag = g.dyp + ((size_t)(tm * (uint32_t)kRowBlocks + load_rb) * g.NB) * 2048u +
+                              (ROWS128 ? (wave & 1) * 1024 : 0) + lane * 16;
+    const uint32_t kbw = tk * (uint32_t)kKBlocks + (uint32_t)wcol * 2u;  // first of the two k blocks this wave multiplies
+    // the block(s) it loads: one of eight, or its own two of sixteen; blocks past the weight repeat the last
+    const uint32_t kbl0 = tk * (uint32_t)kKBlocks + (ROWS128 ? 2u * (uint32_t)wave : (uint32_t)wave);
+    const uint32_t kbl = kbl0 < g.KB ? kbl0 : g.KB - 1u;
+    const uint32_t kbl1 = kbl0 + 1u < g.KB ? kbl0 + 1u : g.KB - 1u;
     const unsigned char* Bg = g.wp + (size_t)tw * g.w_stride + (size_t)kbl * kBlockBytes + lane * 16;
+    const unsigned char* Bg1 = g.wp + (size_t)tw * g.w_stride + (size_t)kbl1 * kBlockBytes + lane * 16;
     const size_t nb_stride = (size_t)g.KB * kBlockBytes;
 
     auto issue = [&](int nb) {
       unsigned char* St = lds + (nb % kBwdStages) * kBwdStageBytes;
       const unsigned char* src = Ag + (size_t)nb * 2048u;
-      load_1k_to_lds(src, St + (wave * 2) * kBlockBytes);
-      load_1k_to_lds(src + 1024, St + (wave * 2 + 1) * kBlockBytes);
-      load_1k_to_lds(Bg + (size_t)nb * nb_stride, St + kBwdStagePanel + wave * kBlockBytes);
+      if constexpr (ROWS128) {
+        load_1k_to_lds(src, St + wave * kBlockBytes);
+        load_1k_to_lds(Bg + (size_t)nb * nb_stride, St + kPanel + (wave * 2) * kBlockBytes);
+        load_1k_to_lds(Bg1 + (size_t)nb * nb_stride, St + kPanel + (wave * 2 + 1) * kBlockBytes);
+      } else {
+        load_1k_to_lds(src, St + (wave * 2) * kBlockBytes);
+        load_1k_to_lds(src + 1024, St + (wave * 2 + 1) * kBlockBytes);
+        load_1k_to_lds(Bg + (size_t)nb * nb_stride, St + kPanel + wave * kBlockBytes);
+      }
       // every wave fetches the same 1 KiB of scales (the stage's 32 lead it) to the same place
-      load_1k_to_lds(reinterpret_cast<const unsigned char*>(swp_t + 32 * nb) + lane * 16,
-                     St + kBwdStagePanel + kBwdStageWeight);
+      load_1k_to_lds(reinterpret_cast<const unsigned char*>(swp_t + 32 * nb) + lane * 16, St + kPanel + kWeight);
     };
 
     v16f acc[4][2];
@@ -539,9 +560,9 @@ __global__ __launch_bounds__(512, 1) void bwd_dx_kernel(BwdDxArgs g) {
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lptr_t)lds;
     struct NextRegs { v4i raw[2]; v4f s4[4]; };
     auto next_read = [&](int nb1, NextRegs& r) {
-      const uint32_t st = lds_base + (nb1 % kBwdStages) * kBwdStageBytes + kBwdStagePanel;
+      const uint32_t st = lds_base + (nb1 % kBwdStages) * kBwdStageBytes + kPanel;
       const uint32_t wa = st + (wcol * 2) * kBlockBytes + lane * 16;
-      const uint32_t sa = st + kBwdStageWeight + 16 * h;
+      const uint32_t sa = st + kWeight + 16 * h;
       asm volatile("ds_read_b128 %0, %6\n\tds_read_b128 %1, %6 offset:1024\n\t"
                    "ds_read_b128 %2, %7\n\tds_read_b128 %3, %7 offset:32\n\t"
                    "ds_read_b128 %4, %7 offset:64\n\tds_read_b128 %5, %7 offset:96"
@@ -652,7 +673,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dx_kernel(BwdDxArgs g) {
     // ---- epilogue: + rs @ A.T, one cast, rows back to their original positions
 #pragma unroll
     for (int rb = 0; rb < 4; ++rb) {
-      const uint32_t pbase = tm * 256u + (uint32_t)wrow * 128u + rb * 32u;
+      const uint32_t pbase = tm * (uint32_t)(kRowBlocks * 32) + (uint32_t)wrow * 128u + rb * 32u;
       const uint32_t blk = pbase / 32u;
       const int src_lane = g.src_row ? g.src_row[pbase + c] : (int)(pbase + c);
       const bool row_ok = src_lane >= 0 && src_lane < (int)g.M;

@@ -90,6 +90,10 @@ CASES = [
     ([700, 20], 512, 1024, 40, 1, 0),                       # rank over 32, several tiles in a weight
     ([3, 0, 0, 9], 128, 256, 0, 1, 4),                      # no LoRA
     ([(i * 7) % 23 for i in range(130)], 256, 384, 4, 1, 0),  # more groups than a dense call has adapters
+    # wide K and few rows per weight: the pull-back's 128-row x 512-k tiles, rows at the tile boundary, a last
+    # k tile with three of its sixteen blocks
+    ([128, 129, 1, 127, 0, 256], 1096, 264, 16, 1, 0),
+    ([60, 70, 100, 29, 0, 0, 5, 130], 1024, 320, 8, 2, 3),  # the same tiles with two groups per weight
 ]
 
 
