@@ -131,6 +131,23 @@ def test_layers_fail_loudly_without_a_gpu_path(pkg):
         exp.load_quantized(torch.zeros(2, 16, 8, dtype=torch.int8), torch.ones(2, 8))
 
 
+def test_constant_lora_scalings_are_cached_per_value_count_and_device(pkg):
+    """A Python-number ``lora_scaling`` must not become a host-to-device copy at every call."""
+    import torch
+
+    w8 = pkg.w8a8_lora
+    a = w8._scaling_vector(2.5, 4, torch.device("cpu"))
+    assert a.dtype == torch.float32 and a.tolist() == [2.5] * 4
+    assert w8._scaling_vector(2.5, 4, torch.device("cpu")) is a          # the same tensor again
+    assert w8._scaling_vector(2.5, 3, torch.device("cpu")).shape == (3,)
+    assert w8._scaling_vector(2, 4, torch.device("cpu")) is not a
+    t = torch.tensor([1.0, 2.0, 3.0])
+    assert w8._scaling_vector(t, 3, torch.device("cpu")).tolist() == [1.0, 2.0, 3.0]   # tensors pass through
+    assert w8._scaling_vector(torch.tensor(0.5), 2, torch.device("cpu")).tolist() == [0.5, 0.5]
+    s = w8._scaling_scalar(0.25, torch.device("cpu"))
+    assert s.ndim == 0 and float(s) == 0.25 and w8._scaling_scalar(t, torch.device("cpu")) is t
+
+
 # --------------------------------------------------------------------------------------
 # GPU: the layers through the HIP path
 # --------------------------------------------------------------------------------------
