@@ -725,9 +725,13 @@ int launch_bwd_body(const BwdBody& b, const Layout& w, unsigned char* ws, hipStr
       lz.n_steps = (b.k + 63u) / 64u;
       lz.nterms = 3u;
       lz.n_blocks = w.slots / 32u;
-      // K is cut into slices so that the launch fills the chip; the slices land in the partial
-      // table (r's partials have been consumed) and are added in slice order
-      const uint32_t nks = w.n_slices;
+      // K is cut into slices so that a call of few row blocks still fills the chip; the slices land
+      // in the partial table (r's partials have been consumed, it holds n_slices of them) and are
+      // added in slice order.  A slice keeps at least one 64-wide step for each of the 16 waves, and
+      // the count depends on K and N only, so that a grouped call and the dense calls over its
+      // groups add in the same order.
+      const uint32_t by_steps = lz.n_steps / 16u ? lz.n_steps / 16u : 1u;
+      const uint32_t nks = by_steps < w.n_slices ? by_steps : w.n_slices;
       lz.n_ksplit = nks;
       lz.steps_per_wave = ((lz.n_steps + nks - 1u) / nks + 15u) / 16u;
       lz.zf = reinterpret_cast<float*>(ws + w.rpart);
