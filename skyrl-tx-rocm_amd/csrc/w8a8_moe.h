@@ -243,22 +243,16 @@ __global__ __launch_bounds__(1024) void moe_scatter_kernel(MoeSortArgs a) {
   const uint32_t p = chunk * kMoeChunk + tid;
   const bool valid = p < a.P;
   const uint32_t g = valid ? moe_group_of(a, p) : 0u;
-  bool done = !valid;
-  uint32_t rank = 0;
-  // every round settles all lanes that share the group of the first unsettled lane
-  for (;;) {
-    const unsigned long long pending = __builtin_amdgcn_ballot_w64(!done);
-    if (!pending) break;
-    const int leader = __builtin_ctzll(pending);
-    const uint32_t g0 = (uint32_t)__builtin_amdgcn_readlane((int)g, leader);  // leader is wave-uniform
-    const bool mine = !done && g == g0;
-    const unsigned long long mask = __builtin_amdgcn_ballot_w64(mine);
-    if (mine) {
-      rank = (uint32_t)__builtin_popcountll(mask & ((1ull << lane) - 1ull));
-      done = true;
-    }
-    if ((int)lane == leader) wave_cnt[wave][g0] = (uint16_t)__builtin_popcountll(mask);
+  // the lanes of this wave that hold the same group: one ballot per bit of the group index
+  // (at most ten), instead of one round per distinct group
+  unsigned long long same = __builtin_amdgcn_ballot_w64(valid);
+  for (uint32_t bit = 0; (1u << bit) < a.G; ++bit) {  // wave-uniform trip count
+    const bool one = (g >> bit) & 1u;
+    const unsigned long long ones = __builtin_amdgcn_ballot_w64(one);
+    same &= one ? ones : ~ones;
   }
+  const uint32_t rank = (uint32_t)__builtin_popcountll(same & ((1ull << lane) - 1ull));
+  if (valid && rank == 0) wave_cnt[wave][g] = (uint16_t)__builtin_popcountll(same);
   __syncthreads();
   if (valid) {
     uint32_t before = 0;
