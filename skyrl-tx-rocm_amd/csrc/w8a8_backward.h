@@ -927,17 +927,66 @@ __global__ __launch_bounds__(256) void bwd_dlora_reduce_kernel(BwdReduceArgs a) 
   __shared__ uint32_t chunk0_lds[kMaxAdapters + 1];
   __shared__ double red[256];
   const uint32_t tid = threadIdx.x;
-  if (!a.chunk0_tab && tid == 0) {
-    uint32_t run = 0;
-    for (uint32_t gq = 0; gq < a.n_groups; ++gq) {
-      chunk0_lds[gq] = run;
-      run += ((uint32_t)(a.group_off[gq + 1] - a.group_off[gq]) + kBwdChunkRows - 1u) / kBwdChunkRows;
+  if (!a.chunk0_tab && tid < 64u) {
+    // first chunk of every group: the dense tables hold at most 64 groups, so one wave loads all the
+    // offsets at once and scans the chunk counts (a serial loop over dependent loads in front of every
+    // workgroup of this short kernel cost more than the reduction itself)
+    static_assert(kMaxAdapters <= 64, "one wave scans the groups");
+    uint32_t cnt = 0;
+    if (tid < a.n_groups)
+      cnt = ((uint32_t)(a.group_off[tid + 1] - a.group_off[tid]) + kBwdChunkRows - 1u) / kBwdChunkRows;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const uint32_t up = (uint32_t)__shfl_up((int)cnt, o, 64);
+      if ((int)tid >= o) cnt += up;
     }
-    chunk0_lds[a.n_groups] = run;
+    if (tid < a.n_groups) chunk0_lds[tid + 1u] = cnt;  // inclusive sums
+    if (tid == 0) chunk0_lds[0] = 0u;
   }
   __syncthreads();
   auto chunk0 = [&](uint32_t gq) -> uint32_t { return a.chunk0_tab ? (uint32_t)a.chunk0_tab[gq] : chunk0_lds[gq]; };
-  uint32_t b = blockIdx.x;
+  auto reduce_ds = [&](uint32_t b) {  // one block per group
+    const uint32_t o0 = (uint32_t)(a.group_beg ? a.group_beg[b] : a.group_off[b]);
+    const uint32_t o1 = (uint32_t)(a.group_end ? a.group_end[b] : a.group_off[b + 1]);
+    // thread = (rank column j, one of four rows per pass); eight passes of loads are in flight at a time:
+    // one load pair per iteration left this single workgroup per group waiting out a memory latency per
+    // four rows, longer than the rest of the launch takes
+    double sum = 0.0;
+    const uint32_t j = tid & 63u;
+    if (j < a.r) {
+      uint32_t slot = o0 + (tid >> 6);
+      for (; slot + 28u < o1; slot += 32u) {
+        float rv[8], zv[8];
+#pragma unroll
+        for (uint32_t u = 0; u < 8; ++u) {
+          const size_t off = (size_t)(slot + 4u * u) * kBwdRankStride + j;
+          rv[u] = a.r_raw[off];
+          zv[u] = a.z[off];
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 8; ++u) sum += (double)rv[u] * (double)zv[u];
+      }
+      for (; slot < o1; slot += 4u) {
+        const size_t off = (size_t)slot * kBwdRankStride + j;
+        sum += (double)a.r_raw[off] * (double)a.z[off];
+      }
+    }
+    red[tid] = sum;
+    __syncthreads();
+    for (uint32_t o = 128; o > 0; o >>= 1) {
+      if (tid < o) red[tid] += red[tid + o];
+      __syncthreads();
+    }
+    if (tid == 0) a.d_s[b] = (float)red[0];
+  };
+  // The blocks of ds come first in the grid: each walks all rows of its group and takes longest, so it
+  // starts at once and runs beside the short dA / dB blocks instead of after them.
+  const uint32_t blocks_s = a.d_s ? a.n_groups : 0u;
+  if (blockIdx.x < blocks_s) {
+    reduce_ds(blockIdx.x);
+    return;
+  }
+  uint32_t b = blockIdx.x - blocks_s;
   if (b < a.blocks_a) {
     // dA [group][k][j]: a thread per output element, j fastest, so that the stores are contiguous
     const uint64_t e = (uint64_t)b * 256u + tid;
@@ -962,22 +1011,6 @@ __global__ __launch_bounds__(256) void bwd_dlora_reduce_kernel(BwdReduceArgs a) 
     *reinterpret_cast<uint2*>(a.d_b + e) = make_uint2(pack_bf16x2(sum.x * sc, sum.y * sc), pack_bf16x2(sum.z * sc, sum.w * sc));
     return;
   }
-  b -= a.blocks_a + a.blocks_b;  // one block per group: ds
-  if (b >= a.n_groups || !a.d_s) return;
-  const uint32_t o0 = (uint32_t)(a.group_beg ? a.group_beg[b] : a.group_off[b]);
-  const uint32_t o1 = (uint32_t)(a.group_end ? a.group_end[b] : a.group_off[b + 1]);
-  double sum = 0.0;
-  for (uint32_t i = o0 * a.r + tid; i < o1 * a.r; i += 256u) {
-    const uint32_t slot = i / a.r, j = i % a.r;
-    sum += (double)a.r_raw[(size_t)slot * kBwdRankStride + j] * (double)a.z[(size_t)slot * kBwdRankStride + j];
-  }
-  red[tid] = sum;
-  __syncthreads();
-  for (uint32_t o = 128; o > 0; o >>= 1) {
-    if (tid < o) red[tid] += red[tid + o];
-    __syncthreads();
-  }
-  if (tid == 0) a.d_s[b] = (float)red[0];
 }
 
 }  // namespace w8a8
