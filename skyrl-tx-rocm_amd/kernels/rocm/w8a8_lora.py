@@ -175,9 +175,23 @@ def dynamic_quantize_rows(x: torch.Tensor):
 # the forward call
 # ---------------------------------------------------------------------------------------
 
-@functools.lru_cache(maxsize=256)
+def _new_constant(value: float, count: int, device: str) -> torch.Tensor:
+    # An ordinary tensor whatever mode the caller is in: a tensor created under inference_mode could
+    # never be saved for a later backward.
+    with torch.inference_mode(False), torch.no_grad():
+        return torch.full((count,), value, dtype=torch.float32, device=torch.device(device))
+
+
+_cached_constant = functools.lru_cache(maxsize=256)(_new_constant)
+
+
 def _constant_scaling(value: float, count: int, device: str) -> torch.Tensor:
-    return torch.full((count,), value, dtype=torch.float32, device=torch.device(device))
+    """One constant vector per (value, count, device).  During a stream capture the cache is bypassed:
+    a tensor created there lives in the graph's private pool, is only filled at replay and dangles once
+    the graph is gone."""
+    if torch.cuda.is_available() and torch.cuda.is_current_stream_capturing():
+        return _new_constant(value, count, device)
+    return _cached_constant(value, count, device)
 
 
 def _scaling_vector(lora_scaling, count: int, device) -> torch.Tensor:

@@ -92,6 +92,9 @@ class LoRALinear(LoRAMixin):
                                  adapter_indices=adapter_indices)
         else:
             out = w8.lora_linear(x, self.weight)
+        # The bias is a second bf16 addition after the fused call's single cast.  The reference's layer
+        # rounds twice as well (nnx.Linear adds the bias to the base output, apply_lora then adds the
+        # low-rank term, layers/lora.py:262-268), in the other order; Qwen3 projections carry no bias.
         return out if self.bias is None else out + self.bias
 
 
@@ -198,10 +201,18 @@ class LoRAExpert(LoRAMixin):
             return w8.grouped_lora_linear(x, group_sizes, self.weight)
         n_ad, n_exp = self.max_lora_adapters, self.num_experts
         gs = group_sizes.to(device=x.device, dtype=torch.int64)
-        expert = torch.repeat_interleave(torch.arange(n_exp, device=x.device), gs, output_size=x.shape[0])
-        combined = expert * n_ad + adapter_indices_sorted.to(device=x.device, dtype=torch.int64)
+        rows = torch.arange(x.shape[0], device=x.device)
+        ends = torch.cumsum(gs, 0)
+        # Expert of every row.  Rows beyond sum(group_sizes) belong to no expert: they sort behind every
+        # group and come out as zeros, as in the plain path.  (The reference's jnp.repeat with
+        # total_repeat_length, layers/lora.py:411, hands such padding rows to the last expert's adapter
+        # on top of a zero base; callers drop those rows either way.)
+        expert = torch.searchsorted(ends, rows, right=True)
+        spare = expert >= n_exp
+        adapter = adapter_indices_sorted.to(device=x.device, dtype=torch.int64).clamp(0, n_ad - 1)
+        combined = torch.where(spare, n_exp * n_ad, expert * n_ad + adapter)
         order = torch.sort(combined, stable=True).indices
-        sizes = torch.bincount(combined, minlength=n_exp * n_ad).to(torch.int32)
+        sizes = torch.bincount(combined, minlength=n_exp * n_ad + 1)[: n_exp * n_ad].to(torch.int32)
         # expert-first flattening of the LoRA pairs (lora.py:418-431)
         a = self.lora_A.transpose(0, 1).reshape(n_exp * n_ad, self.in_features, self.max_lora_rank)
         b = self.lora_B.transpose(0, 1).reshape(n_exp * n_ad, self.max_lora_rank, self.out_features)
@@ -225,8 +236,10 @@ def init_lora_adapter(layer: LoRAMixin, adapter_index: int, *, rank: int, alpha:
     layer.lora_scaling[adapter_index] = alpha / effective
     layer.lora_ranks[adapter_index] = effective
     shape = layer.lora_A[adapter_index].shape
-    fan_in = shape[-2]
-    bound = math.sqrt(6.0 / fan_in)  # he_uniform
+    # he_uniform as jax.nn.initializers computes it (in_axis = -2, out_axis = -1): leading axes count
+    # as receptive field, so an expert layer's [E, in, r] slice has fan_in = E * in
+    fan_in = math.prod(shape) // shape[-1]
+    bound = math.sqrt(6.0 / fan_in)
     gen = torch.Generator(device="cpu").manual_seed(seed)
     a = (torch.rand(shape, generator=gen, dtype=torch.float32) * 2.0 - 1.0) * bound
     a[..., effective:] = 0.0

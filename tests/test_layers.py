@@ -104,8 +104,41 @@ def test_init_lora_adapter(pkg):
     L.init_lora_adapter(exp, 0, rank=8, alpha=16.0)
     assert exp.lora_ranks.tolist() == [2, 4] and exp.lora_scaling.tolist() == [8, 1]
     assert torch.count_nonzero(exp.lora_A[0, :, :, 2:]) == 0 and torch.count_nonzero(exp.lora_A[0, :, :, :2]) > 0
+    # he_uniform counts the expert axis as receptive field (jax.nn.initializers, in_axis = -2):
+    # fan_in = experts * in_features, so the bound is sqrt(6 / (4 * 16)), not sqrt(6 / 16)
+    bound = (6.0 / (4 * 16)) ** 0.5
+    amax = float(exp.lora_A[0].float().abs().max())
+    assert amax <= bound * (1 + 2 ** -8) and amax > 0.8 * bound
     with pytest.raises(RuntimeError):
         L.init_lora_adapter(L.LoRALinear(16, 8, device="cpu"), 0, rank=2, alpha=1.0)
+
+
+def test_constant_scaling_cache_survives_inference_mode(pkg):
+    """A Python-float scaling first seen under inference_mode must still be usable by a later
+    training call: the cached constant has to be an ordinary tensor that autograd can save."""
+    import torch
+
+    w8 = pkg.w8a8_lora
+    with torch.inference_mode():
+        first = w8._scaling_vector(0.3125, 1, torch.device("cpu"))
+    assert not first.is_inference()
+    s = w8._scaling_scalar(0.3125, torch.device("cpu"))
+    assert s.data_ptr() == first.data_ptr()   # same cached constant on both paths
+
+    class Keep(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, x, scaling):
+            ctx.save_for_backward(x, scaling)
+            return x * scaling
+
+        @staticmethod
+        def backward(ctx, g):
+            x, scaling = ctx.saved_tensors
+            return g * scaling, None
+
+    x = torch.ones(3, requires_grad=True)
+    Keep.apply(x, s).sum().backward()
+    assert x.grad.tolist() == [0.3125] * 3
 
 
 def test_layers_fail_loudly_without_a_gpu_path(pkg):
@@ -297,6 +330,14 @@ def test_expert_layer_uses_expert_major_adapter_pairs(pkg, dev):
     swapped = np.where(adapter == 0, 1, np.where(adapter == 1, 0, adapter)).astype(np.int32)
     again = _to_np(layer(xt, torch.from_numpy(group_sizes).to(dev), torch.from_numpy(swapped).to(dev)))
     np.testing.assert_array_equal(again, got)
+    # rows beyond sum(group_sizes) belong to no expert: zeros, and the rows in use do not move;
+    # an adapter index outside the table is clamped like the kernels clamp it
+    spare = 5
+    x_long = torch.cat([xt, torch.ones(spare, k, dtype=torch.bfloat16, device=dev)])
+    idx_long = torch.cat([torch.from_numpy(swapped), torch.full((spare,), 99, dtype=torch.int32)]).to(dev)
+    longer = _to_np(layer(x_long, torch.from_numpy(group_sizes).to(dev), idx_long))
+    np.testing.assert_array_equal(longer[:rows], got)
+    assert not longer[rows:].any()
     with pytest.raises(NotImplementedError):
         layer(xt, torch.from_numpy(group_sizes).to(dev), group_offset=torch.ones(1, dtype=torch.int32))
 
