@@ -1105,9 +1105,17 @@ def main() -> int:
                     "operand_sets_rotated": rotate}
     else:
         achieved = ops / (gemm_avg_ms * 1e-3) / 1e12
+        # the library's choice of geometry (run_forward in csrc/w8a8_api.hip): the 256 x 256 kernel when its
+        # tiles fill the 256 CUs and K has at least six 64-wide steps, unless a flag forces one
+        pad = lambda v, q: -(-v // q) * q
+        wide = (pad(cfg["m"], 256) // 256) * (pad(cfg["n"], 256) // 256) >= 256 and pad(cfg["k"], 128) >= 384
+        if args.flags & native.FLAG_TILE_256X128:
+            wide = False
+        if args.flags & native.FLAG_TILE_256X256:
+            wide = pad(cfg["k"], 128) >= 384
         roofline = {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
                     "frac": achieved / INT8_PEAK_TOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-                    "kernel": "w8a8_gemm_kernel", "kernel_avg_ms": gemm_avg_ms,
+                    "kernel": "w8a8_gemm16_kernel" if wide else "w8a8_gemm_kernel", "kernel_avg_ms": gemm_avg_ms,
                     "kernel_min_ms": float(gemm_ms.min()), "algorithmic_ops": ops,
                     "algorithmic_bytes": gemm_kernel_bytes(cfg)}
 

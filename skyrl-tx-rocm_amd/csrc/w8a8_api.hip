@@ -3,10 +3,10 @@
 #include "../../include/mi355_w8a8.h"
 
 #include <hip/hip_runtime.h>
-#include <stdlib.h>
 
 #include "w8a8_device.h"
 #include "w8a8_gemm.h"
+#include "w8a8_gemm16.h"
 #include "w8a8_prologue.h"
 #include "w8a8_skinny.h"
 #include "w8a8_backward.h"
@@ -99,32 +99,15 @@ template <int EPI, int NKK, int MODE>
 int launch_gemm_one(const GemmArgs& g, hipStream_t s) {
   // persistent grid: one workgroup slot per CU (two in the 256 x 128 geometry), a multiple of 8
   const uint32_t ntile = g.tiles_m * g.tiles_n;
-  uint32_t slots = MODE == kModeDense ? 512u : 256u;
-#ifdef W8A8_DEBUG_VARIANTS
-  { const char* e = getenv("MI355_W8A8_GRID"); if (e && atoi(e) > 0) slots = ((uint32_t)atoi(e) + 7u) / 8u * 8u; }
-#endif
+  const uint32_t slots = MODE == kModeDense ? 512u : 256u;
   const uint32_t want = ((ntile + 7u) / 8u) * 8u;
-  const dim3 grid(want < slots ? want : slots), block((MODE == kModeWide || MODE == kModeGrouped128) ? 512 : 256);
+  const dim3 grid(want < slots ? want : slots), block(MODE == kModeGrouped128 ? 512 : 256);
   constexpr uint32_t lds_bytes =
-      MODE == kModeGrouped128 ? kGrouped128LdsBytes
-                              : (MODE == kModeGrouped ? kGroupedLdsBytes : (MODE == kModeWide ? kWideLdsBytes : kGemmLdsBytes));
-#ifdef W8A8_DEBUG_VARIANTS
-  if constexpr (EPI == kEpiSwiglu && NKK == 2 && MODE != kModeGrouped && MODE != kModeGrouped128) {
-#define W8A8_DBG(D)                                                                              \
-  if (g.map_mode == 100 + D) {                                                                   \
-    hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm_kernel<EPI, NKK, D, MODE>),    \
-                        hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);                  \
-    hipLaunchKernelGGL((w8a8_gemm_kernel<EPI, NKK, D, MODE>), grid, block, lds_bytes, s, g);     \
-    return launch_status();                                                                      \
-  }
-    W8A8_DBG(1) W8A8_DBG(3) W8A8_DBG(5) W8A8_DBG(6)
-#undef W8A8_DBG
-  }
-#endif
-  if (hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm_kernel<EPI, NKK, 0, MODE>),
+      MODE == kModeGrouped128 ? kGrouped128LdsBytes : (MODE == kModeGrouped ? kGroupedLdsBytes : kGemmLdsBytes);
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm_kernel<EPI, NKK, MODE>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
     return MI355_W8A8_ERR_LAUNCH;
-  hipLaunchKernelGGL((w8a8_gemm_kernel<EPI, NKK, 0, MODE>), grid, block, lds_bytes, s, g);
+  hipLaunchKernelGGL((w8a8_gemm_kernel<EPI, NKK, MODE>), grid, block, lds_bytes, s, g);
   return launch_status();
 }
 
@@ -135,6 +118,30 @@ int launch_gemm(const GemmArgs& g, uint32_t nkk, hipStream_t s) {
     case 1: return launch_gemm_one<EPI, 1, MODE>(g, s);
     case 2: return launch_gemm_one<EPI, 2, MODE>(g, s);
     case 4: return launch_gemm_one<EPI, 4, MODE>(g, s);
+    default: return MI355_W8A8_ERR_UNSUPPORTED;
+  }
+}
+
+template <int EPI, int NKK>
+int launch_gemm16_one(const GemmArgs& g, hipStream_t s) {
+  // persistent grid: one workgroup per CU, a multiple of 8 so that every XCD gets the same share
+  const uint32_t ntile = g.tiles_m * g.tiles_n;
+  const uint32_t want = ((ntile + 7u) / 8u) * 8u;
+  const dim3 grid(want < 256u ? want : 256u), block(512);
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm16_kernel<EPI, NKK>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, kG16LdsBytes) != hipSuccess)
+    return MI355_W8A8_ERR_LAUNCH;
+  hipLaunchKernelGGL((w8a8_gemm16_kernel<EPI, NKK>), grid, block, kG16LdsBytes, s, g);
+  return launch_status();
+}
+
+template <int EPI>
+int launch_gemm16(const GemmArgs& g, uint32_t nkk, hipStream_t s) {
+  switch (nkk) {
+    case 0: return launch_gemm16_one<EPI, 0>(g, s);
+    case 1: return launch_gemm16_one<EPI, 1>(g, s);
+    case 2: return launch_gemm16_one<EPI, 2>(g, s);
+    case 4: return launch_gemm16_one<EPI, 4>(g, s);
     default: return MI355_W8A8_ERR_UNSUPPORTED;
   }
 }
@@ -386,27 +393,22 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   g.tiles_m = w.slots / kTileM;
   g.tiles_n = n_padded(p->n) / kGemmTileN;
   g.rank = lora ? p->rank : 0u;
-  g.map_mode = 0u;
-#ifdef W8A8_DEBUG_VARIANTS
-  { const char* e = getenv("MI355_W8A8_TILE_MAP"); if (e) g.map_mode = (uint32_t)atoi(e); }
-#endif
   g.tile_ctr = reinterpret_cast<uint32_t*>(ws + w.tile_ctr);
+  // 256 x 256 tiles (one 4-wave workgroup per CU, 16 x 16 x 64 MFMAs) once they can fill every CU;
+  // below that the 256 x 128 geometry (two 4-wave workgroups per CU) has twice the tiles to spread.
+  bool wide = (uint64_t)g.tiles_m * (n_padded(p->n) / kG16TileN) >= 256u;
+  if (p->flags & MI355_W8A8_FLAG_TILE_256X128) wide = false;
+  if (p->flags & MI355_W8A8_FLAG_TILE_256X256) wide = true;
+  if (w.K_pad < kG16MinKPad) wide = false;  // its stage schedule needs at least six 64-wide k steps
+  if (wide) g.tiles_n = n_padded(p->n) / kG16TileN;
   if (p->aux_acc) {
     GemmArgs ga = g;
     ga.out = p->aux_acc;
     ga.residual = nullptr;
-    if ((st = launch_gemm<kEpiAcc>(ga, 0u, s))) return st;
+    if ((st = wide ? launch_gemm16_one<kEpiAcc, 0>(ga, s) : launch_gemm<kEpiAcc>(ga, 0u, s))) return st;
     g.tile_ctr += 128;  // the second counter set
   }
-  // 256 x 256 tiles (one 8-wave workgroup per CU) once they can fill every CU; below that the
-  // 256 x 128 geometry (two 4-wave workgroups per CU) has twice the tiles to spread.
-  bool wide = (uint64_t)g.tiles_m * (n_padded(p->n) / kWideTileN) >= 256u;
-  if (p->flags & MI355_W8A8_FLAG_TILE_256X128) wide = false;
-  if (p->flags & MI355_W8A8_FLAG_TILE_256X256) wide = true;
-  if (wide) {
-    g.tiles_n = n_padded(p->n) / kWideTileN;
-    return swiglu ? launch_gemm<kEpiSwiglu, kModeWide>(g, w.nkk, s) : launch_gemm<kEpiPlain, kModeWide>(g, w.nkk, s);
-  }
+  if (wide) return swiglu ? launch_gemm16<kEpiSwiglu>(g, w.nkk, s) : launch_gemm16<kEpiPlain>(g, w.nkk, s);
   return swiglu ? launch_gemm<kEpiSwiglu>(g, w.nkk, s) : launch_gemm<kEpiPlain>(g, w.nkk, s);
 }
 
@@ -576,7 +578,6 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
   g.tiles_m = w.slots / w.pad;
   g.tiles_n = (n_padded(p->n) + kGroupedTileN - 1u) / kGroupedTileN;
   g.rank = p->rank;
-  g.map_mode = 1;  // row-tile-major order: column tiles of one expert run back to back
   g.groups_per_weight = gpw;
   if (p->aux_acc) {
     GemmArgs ga = g;

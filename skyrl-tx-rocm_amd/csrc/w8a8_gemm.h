@@ -33,7 +33,7 @@ struct GemmArgs {
   void* out;                 // bf16 [M, n_out] or int32 [M, N]
   uint64_t w_group_stride;   // grouped mode: bytes between the packed weights of two experts
   uint32_t M, N, K_pad, KB, slots, total_rows;
-  uint32_t tiles_m, tiles_n, rank, map_mode;
+  uint32_t tiles_m, tiles_n, rank;
   uint32_t groups_per_weight; // grouped mode: weight index = group / groups_per_weight
   uint32_t* tile_ctr;         // 8 zeroed counters, 64 bytes apart (one per XCD), or null: static schedule
 };
@@ -64,15 +64,8 @@ constexpr int kGrouped128Stages = 3;
 constexpr int kGrouped128StageBytes = 40960;  // A: 4 row blocks x 2 k blocks, B: 16 column blocks x 2 k blocks
 constexpr int kGrouped128LdsBytes = kGrouped128Stages * kGrouped128StageBytes;
 
-// Third geometry, "wide": tile 256 x 256, eight waves (4 x 2, 64 x 128 each, two per SIMD), one
-// workgroup per CU, four 32 KiB stages.  It moves a third less L2 -> LDS traffic per MAC than
-// the 256 x 128 geometry at the price of an epilogue that is not hidden behind a second workgroup.
-constexpr int kWideTileN = 256;
-constexpr int kWideStages = 4;
-constexpr int kWideStageBytes = 32768;
-constexpr int kWideLdsBytes = kWideStages * kWideStageBytes;
-
-enum { kModeDense = 0, kModeGrouped = 1, kModeWide = 2, kModeGrouped128 = 3 };
+// (The 256 x 256 geometry for large problems is a kernel of its own: w8a8_gemm16.h.)
+enum { kModeDense = 0, kModeGrouped = 1, kModeGrouped128 = 2 };
 
 // One tile of the persistent loop.
 struct GemmTile {
@@ -83,18 +76,16 @@ struct GemmTile {
   bool valid;
 };
 
-template <int EPI, int NKK, int DBG = 0, int MODE = kModeDense>
-__global__ __launch_bounds__((MODE == kModeWide || MODE == kModeGrouped128) ? 512 : 256, MODE == kModeDense ? 2 : 1)
+template <int EPI, int NKK, int MODE = kModeDense>
+__global__ __launch_bounds__(MODE == kModeGrouped128 ? 512 : 256, MODE == kModeDense ? 2 : 1)
 void w8a8_gemm_kernel(GemmArgs g) {
   constexpr bool G128 = MODE == kModeGrouped128;
   constexpr bool GROUPED = MODE == kModeGrouped || G128;
-  constexpr bool WIDE = MODE == kModeWide;
-  constexpr int kWaves = (WIDE || G128) ? 8 : 4;
+  constexpr int kWaves = G128 ? 8 : 4;
   constexpr uint32_t kRowBlocks = G128 ? 4 : (GROUPED ? 2 : 8);    // 32-row blocks of the activation panel
-  constexpr uint32_t kColBlocks = GROUPED ? 16 : (WIDE ? 8 : 4);   // 32-column blocks of the weight panel
-  constexpr int kStages = G128 ? kGrouped128Stages : (GROUPED ? kGroupedStages : (WIDE ? kWideStages : kGemmStages));
-  constexpr int kStageBytes =
-      G128 ? kGrouped128StageBytes : (GROUPED ? kGroupedStageBytes : (WIDE ? kWideStageBytes : kGemmStageBytes));
+  constexpr uint32_t kColBlocks = GROUPED ? 16 : 4;                 // 32-column blocks of the weight panel
+  constexpr int kStages = G128 ? kGrouped128Stages : (GROUPED ? kGroupedStages : kGemmStages);
+  constexpr int kStageBytes = G128 ? kGrouped128StageBytes : (GROUPED ? kGroupedStageBytes : kGemmStageBytes);
   constexpr int kAChunks = kRowBlocks * 2;                              // 1 KiB chunks of A per stage
   constexpr int kLoadsPerTile = (kAChunks + kColBlocks * 2) / kWaves;   // direct-to-LDS loads per wave per k-tile
   constexpr bool kLora = (NKK > 0) && (EPI != kEpiAcc);
@@ -103,8 +94,8 @@ void w8a8_gemm_kernel(GemmArgs g) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wrow = G128 ? (wave >> 2) : (GROUPED ? 0 : (WIDE ? (wave >> 1) : wave));  // wave position along M (64 rows each)
-  const int wcol = G128 ? (wave & 3) : (GROUPED ? wave : (WIDE ? (wave & 1) : 0));    // wave position along N (128 columns each)
+  const int wrow = G128 ? (wave >> 2) : (GROUPED ? 0 : wave);  // wave position along M (64 rows each)
+  const int wcol = G128 ? (wave & 3) : (GROUPED ? wave : 0);    // wave position along N (128 columns each)
   const int c = lane & 31, h = lane >> 5;
 
   const uint32_t total_rows = g.total_rows;
@@ -193,11 +184,6 @@ void w8a8_gemm_kernel(GemmArgs g) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
     auto mfma8 = [&](const v4i (&af)[2], const v4i (&bf)[4]) {
-      if constexpr (DBG == 1) {  // measurement only: no MFMA work, keep the operands alive
-#pragma unroll
-        for (int i = 0; i < 2; ++i) asm volatile("" ::"v"(af[i]), "v"(bf[i]), "v"(bf[i + 2]));
-        return;
-      }
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -225,7 +211,7 @@ void w8a8_gemm_kernel(GemmArgs g) {
       // ---- k-step 0 of k-tile kt: prefetch the k-step 1 fragments and the k-tile kStages-1 ahead.
       // The MFMAs lead so that the wait for their operands does not cover the new LDS reads.
       read_frags(kt, 1, fa1, fb1);
-      if constexpr (DBG < 2) issue(T, kt + kStages - 1);
+      issue(T, kt + kStages - 1);
       mfma8(fa0, fb0);
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
 #pragma unroll
@@ -237,10 +223,10 @@ void w8a8_gemm_kernel(GemmArgs g) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_barrier(0);
       // ---- k-step 1: k-tile kt+1 must have landed before its first fragments are fetched
-      if constexpr (DBG < 2) wait_vmcnt<(kStages - 2) * kLoadsPerTile>();
-      if constexpr (DBG != 4) lds_barrier();
+      wait_vmcnt<(kStages - 2) * kLoadsPerTile>();
+      lds_barrier();
       __builtin_amdgcn_sched_barrier(0);
-      if constexpr (DBG != 3) read_frags(kt + 1, 0, fa0, fb0);
+      read_frags(kt + 1, 0, fa0, fb0);
       mfma8(fa1, fb1);
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
 #pragma unroll
@@ -297,11 +283,6 @@ void w8a8_gemm_kernel(GemmArgs g) {
     }
     auto epilogue_block = [&](auto BI) {
       constexpr int bi = decltype(BI)::value;
-      if constexpr (DBG == 6) {  // measurement only: no epilogue, keep the accumulators alive
-#pragma unroll
-        for (int j = 0; j < 4; ++j) asm volatile("" ::"v"(acc[bi][j]));
-        return;
-      }
       const uint32_t pbase = m0 + bi * 32u;
       if (pbase >= total_rows) return;  // wave-uniform
       const uint32_t blk = pbase / 32u;
@@ -434,8 +415,7 @@ void w8a8_gemm_kernel(GemmArgs g) {
             const uint32_t pk = pack_bf16x2(__uint_as_float(hold[v]), __uint_as_float(mine_bits));
             uint16_t* o = reinterpret_cast<uint16_t*>(g.out) + rowoff + (ncol >> 1);
             if (fast) {
-              if constexpr (DBG == 5) asm volatile("" ::"v"(pk), "v"(o));  // measurement only: no stores
-              else *reinterpret_cast<uint32_t*>(o) = pk;
+              *reinterpret_cast<uint32_t*>(o) = pk;
             } else {
               if ((ncol >> 1) < n_out) o[0] = (uint16_t)(pk & 0xffffu);
               if ((ncol >> 1) + 1u < n_out) o[1] = (uint16_t)(pk >> 16);

@@ -1,0 +1,573 @@
+// Tiled int8 GEMM with the fused float32 epilogue on 16 x 16 x 64 MFMAs:
+//   acc[p, n]  = sum_k xq[p, k] * wq[k, n]                         (v_mfma_i32_16x16x64_i8, exact)
+//   base       = (float(acc) * sx[p]) * sw[n]                      (skyrl/tx/kernels/quantized_lora.py:248-252)
+//   y          = base + low * s[group(p)] (+ residual)             (quantized_lora.py:300-304)
+//   low        = z[p, :] @ B[group(p)]                             (v_mfma_f32_16x16x32_bf16, z carried as 3 (or 2) bf16 terms)
+//   out        = bf16(y)   or   bf16(silu(bf16(y_gate)) * bf16(y_up))
+// Workgroup = 512 threads = 8 waves (2 x 4), tile 256 x 256, wave tile 128 x 64 = 8 x 4 blocks of
+// 16 x 16: 128 accumulator registers per lane, two waves per SIMD, one workgroup per CU (a second
+// wave on the SIMD fills the issue slots that LDS reads, waits, barriers and load issue cost the
+// first; with one wave of 128 x 128 per SIMD the same loop ran at 1300 cycles per stage against the
+// 1024 its MFMAs need).  K is consumed in steps of 64 through a ring of four 32 KiB LDS stages
+// filled by 16-byte direct-to-LDS loads of contiguous 1 KiB fragment blocks, four steps ahead of
+// the MFMAs; the ring runs on across tiles (the last four stages of a tile request the first four
+// of the next), so the epilogue issues no stage loads and none of its own loads queues behind them.
+// The 16 x 16 x 64 instruction is used because it moves a quarter of the accumulator bytes per
+// operation of the 32 x 32 x 32 one: on random operands the part sustains about a fifth more
+// operations per second with it before its power limit sets the clock.
+//
+// Operand mapping.  A 1 KiB fragment block holds 32 rows x 32 k; an MFMA operand is 16 rows x 64 k.
+// Lane l (c16 = l % 16, q = l / 16) reads, from the two consecutive k blocks of a stage, its row
+// c16 (+ 16 for the upper half of the block) in k block q / 2, k half q % 2: 16 consecutive lanes
+// read 256 consecutive bytes, so the reads have no bank conflicts.  Activations are the A operand,
+// weights the B operand: lane (c16, q) ends up with packed weight column c16 of a 16-column
+// fragment and the four rows 4 q + v of a 16-row fragment.  With the column permutation of the
+// packed weight (packed 32 j + c <-> original 4 c + j inside a group of 128) a wave takes, from
+// each of the four 32-column blocks j of a group, the same half `chalf` of the columns: its four
+// fragments give the lane the four consecutive original columns 4 (16 chalf + c16) + j of every
+// one of its rows, and the wave 64 consecutive original columns.
+//
+// The direct-to-LDS loads are inline assembly with hand-counted s_waitcnt vmcnt in front of the
+// barriers.  The compiler treats such a load as a FLAT access that may touch LDS and, while one is
+// outstanding (here: always), turns every wait it inserts into vmcnt(0) / lgkmcnt(0); loads it does
+// not know of can only make its own waits stricter, because the counters retire in order.  Nothing
+// an assembly statement produces is a register value, so the compiler may spill and move freely.
+#pragma once
+#include <type_traits>
+
+#include "w8a8_device.h"
+#include "w8a8_gemm.h"
+
+namespace w8a8 {
+
+typedef float v4f_t __attribute__((ext_vector_type(4)));
+
+constexpr int kG16TileM = 256;
+constexpr int kG16TileN = 256;
+constexpr int kG16Stages = 4;
+constexpr int kG16StageBytes = 32768;  // A: 8 row blocks x 2 k blocks, then B: 8 column blocks x 2 k blocks
+constexpr int kG16RingBytes = kG16Stages * kG16StageBytes;
+constexpr int kG16LdsBytes = kG16RingBytes + 8192;  // + per wave 128 row scales and 128 row positions
+constexpr int kG16Loads = 4;                        // direct-to-LDS loads per wave and stage
+constexpr uint32_t kG16MinKPad = 384;               // at least six stages: the schedule below assumes it
+
+// Four direct-to-LDS loads of 1 KiB each: lane l moves 16 bytes global[base_i + 1024 i + voff] -> LDS[lds_addr +
+// 1024 i + 16 l] (voff = 16 l + ...).  The instruction offset applies to the global and to the LDS address
+// alike, so the four loads share one M0 and the caller passes base_i = chunk address - 1024 i.
+__device__ inline void g16_load_4k(const unsigned char* b0, const unsigned char* b1, const unsigned char* b2,
+                                   const unsigned char* b3, uint32_t voff, uint32_t lds_addr_uniform) {
+  asm volatile("s_mov_b32 m0, %5\n\ts_nop 0\n\t"
+               "global_load_lds_dwordx4 %0, %1\n\t"
+               "global_load_lds_dwordx4 %0, %2 offset:1024\n\t"
+               "global_load_lds_dwordx4 %0, %3 offset:2048\n\t"
+               "global_load_lds_dwordx4 %0, %4 offset:3072"
+               :: "v"(voff), "s"(b0), "s"(b1), "s"(b2), "s"(b3), "s"(lds_addr_uniform) : "memory", "m0");
+}
+__device__ inline void g16_set_m0(uint32_t lds_addr_uniform) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" :: "s"(lds_addr_uniform) : "memory", "m0");
+}
+template <int OFF>
+__device__ inline void g16_load_1k_m0(const unsigned char* base_uniform, uint32_t voff) {  // M0 set before
+  asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" :: "v"(voff), "s"(base_uniform), "n"(OFF) : "memory", "m0");
+}
+// One wave copies 128 dwords: lane l moves global[base + 4 l] and global[base + 256 + 4 l] to the same
+// offsets behind lds_addr.
+__device__ inline void g16_load_128_dwords(const void* base_uniform, uint32_t lane4, uint32_t lds_addr_uniform) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1\n\t"
+               "global_load_lds_dword %0, %1 offset:256"
+               :: "v"(lane4), "s"(base_uniform), "s"(lds_addr_uniform) : "memory", "m0");
+}
+// LDS fragment read.  These are ordinary loads the compiler keeps its books on: it places the waits
+// (precisely, since it never sees the direct-to-LDS loads) and may spill or move the values safely.
+template <int OFF>
+__device__ inline v4i g16_ds_read(uint32_t addr) {
+  typedef __attribute__((address_space(3))) const v4i* lds_v4i_ptr;
+  return *reinterpret_cast<lds_v4i_ptr>((uintptr_t)(addr + OFF));
+}
+template <int N>
+__device__ inline void g16_wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
+template <int J0, int J1, class F>
+__device__ inline void g16_for(F&& f) {  // f(integral_constant<int, J>) for J0 <= J < J1, unrolled at compile time
+  if constexpr (J0 < J1) {
+    f(std::integral_constant<int, J0>{});
+    g16_for<J0 + 1, J1>(f);
+  }
+}
+// The integer MFMAs go through the compiler's builtin: it then knows which instruction produced an
+// accumulator and inserts the wait states the hardware does not interlock (an MFMA result read by the
+// vector ALU or moved between register classes), wherever its register allocation makes them necessary.
+__device__ inline void g16_mfma(v4i& acc, const v4i& a, const v4i& b) {
+  acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc, 0, 0, 0);
+}
+__device__ inline void g16_mfma_first(v4i& acc, const v4i& a, const v4i& b) {
+  const v4i zero = {0, 0, 0, 0};
+  acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, zero, 0, 0, 0);
+}
+constexpr int g16_frag_off(int f) { return (f >> 1) * 2048 + (f & 1) * 256; }  // activation fragment f of a wave's four row blocks
+constexpr int g16_bfrag_off(int j) { return j * 2048; }                        // weight fragment j: the wave's half of column block j
+
+template <int EPI, int NKK>
+__global__ __launch_bounds__(512, 1)
+void w8a8_gemm16_kernel(GemmArgs g) {
+  constexpr bool kLora = (NKK > 0) && (EPI != kEpiAcc);
+  constexpr int kKS = NKK > 2 ? 2 : 1;  // 32-wide rank steps of the LoRA product
+  constexpr uint32_t kNkk = NKK > 0 ? NKK : 1;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wrow = wave >> 2, wcol = wave & 3;  // wave tile: rows 128 wrow, columns 64 wcol of the tile
+  const int cgrp = wcol >> 1, chalf = wcol & 1;  // its 128-column group inside the tile and its half of every block
+  const uint32_t c16 = lane & 15, q = lane >> 4;
+  // byte offset of the lane's 16 bytes inside a pair of k blocks (lower 16 rows of the block)
+  const uint32_t lane_off = (q >> 1) * kBlockBytes + (c16 + 32u * (q & 1u)) * 16u;
+
+  const uint32_t total_rows = g.total_rows;
+  const uint32_t ntile = g.tiles_m * g.tiles_n;
+  const uint32_t ncb_total = n_padded(g.N) / 32u;
+  const uint32_t n_out = (EPI == kEpiSwiglu) ? g.N / 2u : g.N;
+  const int KT = (int)(g.K_pad / 64u);  // even (K is padded to 128) and at least 6
+
+  // ---- persistent schedule: consecutive workgroup ids land on different XCDs, so each XCD walks a
+  // contiguous range of a band-major tile order (4 row tiles x all column tiles) and its workgroups
+  // share panels in its own L2.
+  const uint32_t per_xcd = (ntile + 7u) / 8u;
+  const uint32_t wgs_per_xcd = gridDim.x >> 3;
+  auto tile_at = [&](uint32_t i) -> GemmTile {
+    GemmTile T{};
+    const uint32_t t = i < per_xcd ? (blockIdx.x & 7u) * per_xcd + i : ntile;
+    if (t >= ntile) return T;
+    constexpr uint32_t GM = 4;
+    const uint32_t band = t / (GM * g.tiles_n);
+    const uint32_t band_rows = (g.tiles_m - band * GM) < GM ? (g.tiles_m - band * GM) : GM;
+    const uint32_t in_band = t - band * GM * g.tiles_n;
+    T.tm = band * GM + in_band % band_rows;
+    T.tn = in_band / band_rows;
+    T.Ag = g.xq + (size_t)T.tm * 8u * g.KB * kBlockBytes;
+    T.Bg = g.wp;
+    T.swp = g.sw;
+    T.valid = true;
+    return T;
+  };
+  // chunk ch = 4 wave + i of a stage: 0..15 activations (row block ch / 2, k block ch % 2), 16..31
+  // weights; stage kt of a chunk lies 2 KiB * kt behind its base.  Returned: base - 1024 (i % 4), see
+  // g16_load_4k.
+  auto chunk_base = [&](const GemmTile& Tx, int i) -> const unsigned char* {
+    const int ch = wave * kG16Loads + i;
+    const bool isA = ch < 16;
+    uint32_t rb = isA ? (uint32_t)(ch >> 1) : Tx.tn * 8u + (uint32_t)((ch - 16) >> 1);
+    if (!isA && rb >= ncb_total) rb = ncb_total - 1u;  // keep every wave's load count equal
+    return (isA ? Tx.Ag : Tx.Bg) + ((size_t)rb * g.KB + (uint32_t)(ch & 1)) * kBlockBytes - (size_t)i * 1024u;
+  };
+
+  const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)lds;
+  const uint32_t a0 = lds_addr + (uint32_t)wrow * 8192u + lane_off;           // activation fragments, ring slot 0
+  const uint32_t b0 = lds_addr + 16384u + (uint32_t)cgrp * 8192u + (uint32_t)chalf * 256u + lane_off;  // weight fragments, ring slot 0
+  const uint32_t dma0 = lds_addr + (uint32_t)wave * (kG16Loads * kBlockBytes);  // the wave's chunks, ring slot 0
+  // per wave: f32 sx[128] then int32 src_row[128] of its rows, behind the stage ring
+  unsigned char* const rowdata = lds + kG16RingBytes + wave * 1024;  // (the waves of a row half hold the same data)
+
+  // Raw buffer resources over the LoRA operands: loads through them take a uniform 64-bit base, a uniform
+  // 32-bit offset and a 32-bit lane offset, so no lane holds a 64-bit address.
+  const __amdgpu_buffer_rsrc_t zrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(g.zp), 0, -1, 0x00020000);
+  const __amdgpu_buffer_rsrc_t brsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(g.bp), 0, -1, 0x00020000);
+  uint32_t g0 = 0;          // ring slot of the current tile's stage 0
+  bool prefetched = false;  // the first four stages of the current tile were requested by the previous tile
+  for (uint32_t cur_i = blockIdx.x >> 3; cur_i < per_xcd; cur_i += wgs_per_xcd) {
+    const GemmTile T = tile_at(cur_i);
+    if (!T.valid) { prefetched = false; continue; }
+    const uint32_t nxt_i = cur_i + wgs_per_xcd;
+    GemmTile Tn{};
+    if (nxt_i < per_xcd) Tn = tile_at(nxt_i);
+    const bool has_next = Tn.valid;  // workgroup-uniform
+
+    const unsigned char* cbase[kG16Loads];
+#pragma unroll
+    for (int i = 0; i < kG16Loads; ++i) cbase[i] = chunk_base(T, i);
+
+    v4i acc[8][4];
+    v4i bf[2][4];  // weight fragments of the current / next stage
+    v4i af[4];     // activation fragments, three ahead of the MFMAs
+    if (!prefetched) {
+#pragma unroll
+      for (int st = 0; st < kG16Stages; ++st) {
+        const uint32_t voff = (uint32_t)st * 2048u + (uint32_t)lane * 16u;
+        const uint32_t dst = dma0 + (((uint32_t)st + g0) & 3u) * kG16StageBytes;
+        g16_load_4k(cbase[0], cbase[1], cbase[2], cbase[3], voff, dst);
+      }
+    }
+    // Stage 0 must have landed.  Behind it in the queue: stages 1..3 (12 loads) and, when the previous
+    // tile requested them, that tile's epilogue, which is younger still.
+    g16_wait_vm<3 * kG16Loads>();
+    lds_barrier();
+
+    // LDS reads retire in order; the waits below count the reads issued behind the one they need.
+    // Order here and at the end of every stage: B0..B3, A0, A1, A2.
+    {
+      const uint32_t sa = a0 + ((g0 & 3u) << 15), sb = b0 + ((g0 & 3u) << 15);
+      g16_for<0, 4>([&](auto J) { bf[0][decltype(J)::value] = g16_ds_read<g16_bfrag_off(decltype(J)::value)>(sb); });
+      af[0] = g16_ds_read<g16_frag_off(0)>(sa);
+      af[1] = g16_ds_read<g16_frag_off(1)>(sa);
+      af[2] = g16_ds_read<g16_frag_off(2)>(sa);
+    }
+
+    const unsigned char* nbase[kG16Loads];
+#pragma unroll
+    for (int i = 0; i < kG16Loads; ++i) nbase[i] = has_next ? chunk_base(Tn, i) : cbase[i];
+
+    // One stage: 32 MFMAs per wave.  Activation fragment bi + 3 is fetched under the MFMAs of fragment
+    // bi; before fragment 6 the next stage must have landed (own loads counted, then the barrier), the
+    // buffer of this stage is handed to the loads four stages ahead, and the next stage's first
+    // fragments are fetched under the last 8 MFMAs.  REM = stages of this tile after this one, capped
+    // at 4: a compile-time constant, so that the steady-state loop body has no branches.  With REM < 4
+    // the stage four ahead belongs to the next tile.
+    auto stage = [&](auto PAR, auto FIRST, auto REMC, int kt) {
+      constexpr int P = decltype(PAR)::value;
+      constexpr bool first = decltype(FIRST)::value;
+      constexpr int REM = decltype(REMC)::value;
+      // The stage addresses are formed from values the compiler cannot see through: it would otherwise
+      // compute every stage's addresses once at kernel start and keep them in registers (or spill them).
+      uint32_t a0s = a0, b0s = b0;
+      asm volatile("" : "+v"(a0s), "+v"(b0s));
+      const uint32_t slot = ((uint32_t)kt + g0) & 3u, slot_n = ((uint32_t)kt + 1u + g0) & 3u;
+      const uint32_t sa = a0s + (slot << 15);
+      const uint32_t san = a0s + (slot_n << 15);
+      const uint32_t sbn = b0s + (slot_n << 15);
+      auto mfma_row = [&](auto BI) {
+        constexpr int bi = decltype(BI)::value;
+#pragma unroll
+        for (int bj = 0; bj < 4; ++bj) {
+          if constexpr (first) g16_mfma_first(acc[bi][bj], af[bi & 3], bf[P][bj]);
+          else g16_mfma(acc[bi][bj], af[bi & 3], bf[P][bj]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      using std::integral_constant;
+      // in flight here, oldest first: B0..B3, A0, A1, A2 of this stage
+      af[3] = g16_ds_read<g16_frag_off(3)>(sa);
+      mfma_row(integral_constant<int, 0>{});
+      af[0] = g16_ds_read<g16_frag_off(4)>(sa);
+      mfma_row(integral_constant<int, 1>{});
+      af[1] = g16_ds_read<g16_frag_off(5)>(sa);
+      mfma_row(integral_constant<int, 2>{});
+      af[2] = g16_ds_read<g16_frag_off(6)>(sa);
+      mfma_row(integral_constant<int, 3>{});
+      af[3] = g16_ds_read<g16_frag_off(7)>(sa);
+      mfma_row(integral_constant<int, 4>{});
+      mfma_row(integral_constant<int, 5>{});
+      // The next stage must have landed: own loads first, then everybody's; the barrier also ends every
+      // wave's reads of this stage's buffer.  Three stages are in the queue behind this one as long as
+      // the tile or a next tile provides them.
+      if constexpr (REM >= 3) {
+        g16_wait_vm<2 * kG16Loads>();
+      } else if constexpr (REM >= 1) {
+        if (has_next) g16_wait_vm<2 * kG16Loads>();
+        else if constexpr (REM == 2) g16_wait_vm<kG16Loads>();
+        else g16_wait_vm<0>();
+      }
+      lds_barrier();  // REM == 0: nothing has to land here; the barrier frees this stage's buffer
+      // After the barrier the last 8 MFMAs start at once (their operands are in registers); the next
+      // stage's first fragments (order B0..B3, A0, A1, A2) and the four loads of the stage four ahead
+      // (into the buffer the barrier has just freed) are issued in the gaps between them.  The order is
+      // pinned: bunched in front of the MFMAs, these ten instructions per wave leave the matrix core idle.
+      auto one = [&](auto BI, auto BJ) {
+        constexpr int bi = decltype(BI)::value, bj = decltype(BJ)::value;
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (first) g16_mfma_first(acc[bi][bj], af[bi & 3], bf[P][bj]);
+        else g16_mfma(acc[bi][bj], af[bi & 3], bf[P][bj]);
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      using C6 = integral_constant<int, 6>;
+      using C7 = integral_constant<int, 7>;
+      one(C6{}, integral_constant<int, 0>{});
+      if constexpr (REM >= 1) {
+        bf[1 - P][0] = g16_ds_read<g16_bfrag_off(0)>(sbn);
+        bf[1 - P][1] = g16_ds_read<g16_bfrag_off(1)>(sbn);
+      }
+      one(C6{}, integral_constant<int, 1>{});
+      if constexpr (REM >= 1) {
+        bf[1 - P][2] = g16_ds_read<g16_bfrag_off(2)>(sbn);
+        bf[1 - P][3] = g16_ds_read<g16_bfrag_off(3)>(sbn);
+      }
+      one(C6{}, integral_constant<int, 2>{});
+      if constexpr (REM >= 1) {
+        af[0] = g16_ds_read<g16_frag_off(0)>(san);
+        af[1] = g16_ds_read<g16_frag_off(1)>(san);
+      }
+      one(C6{}, integral_constant<int, 3>{});
+      one(C7{}, integral_constant<int, 0>{});
+      if constexpr (REM >= 1) af[2] = g16_ds_read<g16_frag_off(2)>(san);
+      if (REM >= 4 || (REM >= 1 && has_next)) {  // compile-time facts but has_next; the last stage issues none
+        const uint32_t voff4 = (uint32_t)(REM >= 4 ? kt + kG16Stages : kt + kG16Stages - KT) * 2048u + (uint32_t)lane * 16u;
+        if constexpr (REM >= 4) g16_load_4k(cbase[0], cbase[1], cbase[2], cbase[3], voff4, dma0 + (slot << 15));
+        else g16_load_4k(nbase[0], nbase[1], nbase[2], nbase[3], voff4, dma0 + (slot << 15));
+      }
+      one(C7{}, integral_constant<int, 1>{});
+      one(C7{}, integral_constant<int, 2>{});
+      one(C7{}, integral_constant<int, 3>{});
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    using I3 = std::integral_constant<int, 3>;
+    using I4 = std::integral_constant<int, 4>;
+    using Yes = std::true_type;
+    using No = std::false_type;
+    stage(I0{}, Yes{}, I4{}, 0);
+    stage(I1{}, No{}, I4{}, 1);
+    for (int kt = 2; kt < KT - 4; kt += 2) {
+      stage(I0{}, No{}, I4{}, kt);
+      stage(I1{}, No{}, I4{}, kt + 1);
+    }
+    stage(I0{}, No{}, I3{}, KT - 4);
+    stage(I1{}, No{}, I2{}, KT - 3);
+    stage(I0{}, No{}, I1{}, KT - 2);
+    // adapters present in the wave's four 32-row blocks: one scalar load (the compiler would
+    // fetch them through the vector memory path and wait vmcnt(0))
+    v4i range4 = {0, 0, 0, 0};
+    if (kLora && g.blk_range)
+      asm volatile("s_load_dwordx4 %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)"
+                   : "=s"(range4) : "s"(g.blk_range + (T.tm * 256u + wrow * 128u) / 32u) : "memory");
+    // ---- What the epilogue works with is set up here, behind the main loop's bulk, so that none of it
+    // is live (or spilled) across the loop; preload() requests what it starts from.
+    const uint32_t m0 = T.tm * 256u + wrow * 128u;     // first slot of the wave
+    const uint32_t tgrp0 = T.tn * 256u + cgrp * 128u;  // first column of the wave's group of 128
+    const uint32_t tcol0 = tgrp0 + chalf * 64u;        // first of the wave's 64 columns
+    const bool wave_live = tcol0 < g.N;                // wave-uniform; a dead wave only feeds the loads
+    const bool full_n = (tcol0 + 64u <= g.N) && ((g.N & 3u) == 0);  // wave-uniform
+    const v4i zero4 = {0, 0, 0, 0};
+    v4i swr = zero4;                                   // per-channel scales of the lane's 4 columns
+    const uint32_t range[4] = {(uint32_t)range4.x, (uint32_t)range4.y, (uint32_t)range4.z, (uint32_t)range4.w};
+    v4i zr[2][kKS][3];                                 // z operands: ring of two 16-row fragments
+    v4i br[4][kKS];                                    // LoRA B operands of adapter `bgroup`
+    // (defined on every path: an undefined start would let the last tile's values count as live across the loop)
+#pragma unroll
+    for (int ks = 0; ks < kKS; ++ks) {
+#pragma unroll
+      for (int t3 = 0; t3 < 3; ++t3) zr[0][ks][t3] = zr[1][ks][t3] = zero4;
+#pragma unroll
+      for (int bj = 0; bj < 4; ++bj) br[bj][ks] = zero4;
+    }
+    int bgroup = -1;
+    // operand bytes inside a 1 KiB block of the 32 x 16 layouts the prologue writes: rank octet q sits in
+    // rank chunk q / 2 (16 ranks each), half q % 2.  A rank chunk beyond the rank is read from the last
+    // existing one and zeroed afterwards.
+    uint32_t lora_lane = (c16 + 32u * (q & 1u)) * 16u;
+    asm volatile("" : "+v"(lora_lane));  // per tile: keeps the derived lane offsets out of kernel-long registers
+    const bool lane_has_rank[2] = {(q >> 1) < kNkk, 2u + (q >> 1) < kNkk};
+    // z and B are read through buffer resources: a uniform offset per operand and, per 32-rank step,
+    // one lane offset (rank chunk of the lane, clamped to the last existing one, and lane position).
+    uint32_t zlane[kKS], blane[kKS];
+#pragma unroll
+    for (int ks = 0; ks < kKS; ++ks) {
+      uint32_t kk = 2u * ks + (q >> 1);
+      if (kk >= kNkk) kk = kNkk - 1u;
+      zlane[ks] = kk * 3u * kBlockBytes + lora_lane;
+      blane[ks] = kk * kBlockBytes + lora_lane;
+    }
+    auto z_soff = [&](int bi, int t3) -> uint32_t {
+      return ((m0 / 32u + (uint32_t)(bi >> 1)) * kNkk * 3u + (uint32_t)t3) * kBlockBytes + (uint32_t)(bi & 1) * 256u;
+    };
+    auto b_soff = [&](int gi, int bj) -> uint32_t {
+      return (((uint32_t)gi * ncb_total + tgrp0 / 32u + (uint32_t)bj) * kNkk) * kBlockBytes + (uint32_t)chalf * 256u;
+    };
+    auto load_z = [&](int slot, int bi) {
+#pragma unroll
+      for (int ks = 0; ks < kKS; ++ks)
+#pragma unroll
+        for (int t3 = 0; t3 < 3; ++t3)
+          zr[slot][ks][t3] = lane_has_rank[ks] ? __builtin_amdgcn_raw_buffer_load_b128(zrsrc, zlane[ks], z_soff(bi, t3), 0) : zero4;
+    };
+    auto load_b = [&](int gi) {
+#pragma unroll
+      for (int bj = 0; bj < 4; ++bj)
+#pragma unroll
+        for (int ks = 0; ks < kKS; ++ks)
+          br[bj][ks] = lane_has_rank[ks] ? __builtin_amdgcn_raw_buffer_load_b128(brsrc, blane[ks], b_soff(gi, bj), 0) : zero4;
+      bgroup = gi;
+    };
+    // What the epilogue starts from is requested at the start of the last stage, with loads the compiler
+    // keeps its books on (it places the waits and may move the values as it likes).  No stage load is
+    // issued behind them before they are waited for, so that wait does not stall on a younger load.
+    auto preload = [&]() {
+      if (EPI != kEpiAcc) g16_load_128_dwords(g.sx + m0, (uint32_t)lane * 4u, lds_addr + kG16RingBytes + wave * 1024);
+      if (g.src_row) g16_load_128_dwords(g.src_row + m0, (uint32_t)lane * 4u, lds_addr + kG16RingBytes + wave * 1024 + 512);
+      if (!wave_live) return;
+      if (EPI != kEpiAcc && full_n) swr = *reinterpret_cast<const v4i*>(T.swp + tcol0 + 4u * c16);
+      if constexpr (kLora) {
+        load_z(0, 0);
+        load_z(1, 1);
+        load_b((int)(range[0] & 0xffffu));
+      }
+    };
+
+    preload();
+    stage(I1{}, No{}, I0{}, KT - 1);  // the last stage (KT is even); it also requests the epilogue's operands
+    // The preloads were requested a stage ago and are the youngest loads in the queue.  After the wait
+    // (the builtin, so that the compiler knows its loads are in) the next tile's fourth stage is requested
+    // into the buffer the last barrier has freed.
+    wait_vmcnt<0>();
+    if (has_next) {
+      const uint32_t voff = 3u * 2048u + (uint32_t)lane * 16u;
+      g16_load_4k(nbase[0], nbase[1], nbase[2], nbase[3], voff, dma0 + ((((uint32_t)KT - 1u + g0) & 3u) << 15));
+    }
+    g0 = (g0 + (uint32_t)KT) & 3u;
+    prefetched = has_next;
+
+    // ---------------------------------------------------------------- epilogue
+    // Lane (c16, q) owns, in every 16-row fragment bi, the rows 4 q + v (v = 0..3) and the four
+    // consecutive original columns tcol0 + 4 c16 + j held by the accumulator blocks j.
+    if (!wave_live) continue;  // wave beyond the last column; it still takes part in the next tile
+    const uint32_t ncol = tcol0 + 4u * c16;  // the lane's four consecutive columns
+    float sw[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sw[j] = full_n ? __int_as_float(swr[j]) : 0.0f;  // (a bit_cast of a vector element reads element 0)
+    if (EPI != kEpiAcc && !full_n) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (ncol + j < g.N) sw[j] = T.swp[ncol + j];
+    }
+    g16_for<0, 8>([&](auto BI) {
+      constexpr int bi = decltype(BI)::value;
+      const uint32_t pbase = m0 + bi * 16u;  // first slot of the 16-row fragment
+      if (pbase >= total_rows) return;       // wave-uniform
+      __builtin_amdgcn_sched_barrier(0);     // keep the fragments' register lifetimes apart
+      // the fragment's accumulators leave the accumulation registers here, not earlier
+      asm volatile("" : "+a"(acc[bi][0]), "+a"(acc[bi][1]), "+a"(acc[bi][2]), "+a"(acc[bi][3]));
+      const uint32_t p4 = pbase + 4u * q;
+      float sx[4] = {0.f, 0.f, 0.f, 0.f};
+      if (EPI != kEpiAcc) {
+        const float4 s4 = *reinterpret_cast<const float4*>(rowdata + (16u * bi + 4u * q) * 4u);
+        sx[0] = s4.x; sx[1] = s4.y; sx[2] = s4.z; sx[3] = s4.w;
+      }
+      int src[4] = {(int)p4, (int)p4 + 1, (int)p4 + 2, (int)p4 + 3};
+      if (g.src_row) {
+        const int4 r4 = *reinterpret_cast<const int4*>(rowdata + 512u + (16u * bi + 4u * q) * 4u);
+        src[0] = r4.x; src[1] = r4.y; src[2] = r4.z; src[3] = r4.w;
+      }
+      bool row_ok[4];
+      uint32_t off[4];
+      bool all_ok = true;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        row_ok[v] = src[v] >= 0 && src[v] < (int)g.M;
+        off[v] = row_ok[v] ? (uint32_t)src[v] * ((EPI == kEpiAcc) ? g.N : n_out) : 0u;
+        all_ok = all_ok && row_ok[v];
+      }
+      const bool fast = full_n && (__builtin_amdgcn_ballot_w64(!all_ok) == 0);  // wave-uniform
+
+      if constexpr (EPI == kEpiAcc) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          if (!row_ok[v]) continue;
+          int32_t* o = reinterpret_cast<int32_t*>(g.out) + off[v] + ncol;
+          if (fast) {
+            *reinterpret_cast<int4*>(o) = make_int4(acc[bi][0][v], acc[bi][1][v], acc[bi][2][v], acc[bi][3][v]);
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              if (ncol + j < g.N) o[j] = acc[bi][j][v];
+          }
+        }
+      } else {
+        // Groups (adapters) present in the 32-row block of this fragment: one, except at a group
+        // boundary.  A boundary fragment is processed once per group; each pass stores its own rows.
+        const int glo = (int)(range[bi >> 1] & 0xffffu), ghi = (int)(range[bi >> 1] >> 16);
+        int grp[4] = {glo, glo, glo, glo};
+        if (kLora && g.slot_group && ghi > glo) {
+          const int4 g4 = *reinterpret_cast<const int4*>(g.slot_group + p4);
+          grp[0] = g4.x; grp[1] = g4.y; grp[2] = g4.z; grp[3] = g4.w;
+        }
+        for (int gi = glo; gi <= ghi; ++gi) {  // wave-uniform
+          // ---- low[bj][v] = s_g * (z @ B_g): z rows of this fragment, B columns of fragment bj.  The
+          // three terms of a fragment run as three rounds over the four independent accumulators.
+          v4f_t low[4];
+          if constexpr (kLora) {
+            if (gi != bgroup) load_b(gi);  // wave-uniform: a new adapter begins in this fragment
+            const float sgrp = g.lora_scaling[gi];
+#pragma unroll
+            for (int bj = 0; bj < 4; ++bj) low[bj] = v4f_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < kKS; ++ks)
+#pragma unroll
+              for (int t3 = 2; t3 >= 0; --t3)
+#pragma unroll
+                for (int bj = 0; bj < 4; ++bj)
+                  low[bj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, zr[bi & 1][ks][t3]),
+                                                                    __builtin_bit_cast(v8bf, br[bj][ks]), low[bj], 0, 0, 0);
+            // the low-rank accumulators live in ordinary registers: every accumulation register is taken,
+            // and left to itself the compiler spills one of the integer accumulators to make room
+            asm volatile("" : "+v"(low[0]), "+v"(low[1]), "+v"(low[2]), "+v"(low[3]));
+#pragma unroll
+            for (int bj = 0; bj < 4; ++bj)
+#pragma unroll
+              for (int v = 0; v < 4; ++v) low[bj][v] = low[bj][v] * sgrp;
+          }
+          {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+              bool row_valid = row_ok[v];
+              if (kLora && ghi > glo) row_valid = row_valid && (grp[v] == gi);  // boundary: own rows only
+              float y[4];
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                // same f32 operations, in the same order, as the reference epilogue: a fused
+                // multiply-add here would flip rare bf16 roundings that SwiGLU then amplifies
+                const float t = (float)acc[bi][j][v] * sx[v];
+                y[j] = t * sw[j];
+                if constexpr (kLora) y[j] = y[j] + low[j][v];
+              }
+              if (EPI == kEpiSwiglu) {
+                // (y0, y1) and (y2, y3) are the (gate, up) pairs of product columns ncol/2, ncol/2 + 1
+                const uint32_t f0 = pack_bf16x2(y[0], y[1]), f1 = pack_bf16x2(y[2], y[3]);
+                const float p0 = swiglu_f32(__uint_as_float(f0 << 16), __uint_as_float(f0 & 0xffff0000u));
+                const float p1 = swiglu_f32(__uint_as_float(f1 << 16), __uint_as_float(f1 & 0xffff0000u));
+                if (!row_valid) continue;
+                const uint32_t pk = pack_bf16x2(p0, p1);
+                uint16_t* o = reinterpret_cast<uint16_t*>(g.out) + off[v] + (ncol >> 1);
+                if (fast) {
+                  *reinterpret_cast<uint32_t*>(o) = pk;
+                } else {
+                  if ((ncol >> 1) < n_out) o[0] = (uint16_t)(pk & 0xffffu);
+                  if ((ncol >> 1) + 1u < n_out) o[1] = (uint16_t)(pk >> 16);
+                }
+              } else {
+                if (!row_valid) continue;
+                if (g.residual) {
+                  uint32_t r0 = 0, r1 = 0;
+                  if (fast) {
+                    const uint2 rr = *reinterpret_cast<const uint2*>(g.residual + off[v] + ncol);
+                    r0 = rr.x; r1 = rr.y;
+                  } else {
+                    if (ncol + 0u < g.N) r0 |= (uint32_t)g.residual[off[v] + ncol + 0u];
+                    if (ncol + 1u < g.N) r0 |= (uint32_t)g.residual[off[v] + ncol + 1u] << 16;
+                    if (ncol + 2u < g.N) r1 |= (uint32_t)g.residual[off[v] + ncol + 2u];
+                    if (ncol + 3u < g.N) r1 |= (uint32_t)g.residual[off[v] + ncol + 3u] << 16;
+                  }
+                  y[0] = y[0] + __uint_as_float(r0 << 16);
+                  y[1] = y[1] + __uint_as_float(r0 & 0xffff0000u);
+                  y[2] = y[2] + __uint_as_float(r1 << 16);
+                  y[3] = y[3] + __uint_as_float(r1 & 0xffff0000u);
+                }
+                const uint32_t lo = pack_bf16x2(y[0], y[1]), hi = pack_bf16x2(y[2], y[3]);
+                uint16_t* o = reinterpret_cast<uint16_t*>(g.out) + off[v] + ncol;
+                if (fast) {
+                  *reinterpret_cast<uint2*>(o) = make_uint2(lo, hi);
+                } else {
+                  if (ncol + 0u < g.N) o[0] = (uint16_t)(lo & 0xffffu);
+                  if (ncol + 1u < g.N) o[1] = (uint16_t)(lo >> 16);
+                  if (ncol + 2u < g.N) o[2] = (uint16_t)(hi & 0xffffu);
+                  if (ncol + 3u < g.N) o[3] = (uint16_t)(hi >> 16);
+                }
+              }
+            }
+          }
+        }  // groups of the fragment
+        // this fragment's z operands are spent: their ring slot takes the fragment two ahead
+        if constexpr (kLora && bi + 2 < 8) load_z(bi & 1, bi + 2);
+      }
+    });
+  }
+}
+
+}  // namespace w8a8

@@ -252,21 +252,33 @@ def test_run_to_run_determinism(dev):
 @pytest.mark.parametrize("shape", [
     dict(m=300, k=512, n=768, n_adapters=4, rank=16, rms=True, swiglu=True),
     dict(m=515, k=384, n=1000, n_adapters=5, rank=32),
-    dict(m=100, k=256, n=520, n_adapters=3, rank=64, residual=True),
-    dict(m=64, k=128, n=256, n_adapters=0),
+    dict(m=100, k=448, n=520, n_adapters=3, rank=64, residual=True),
+    dict(m=64, k=392, n=256, n_adapters=0),
+    dict(m=700, k=2048, n=300, n_adapters=0, residual=True),
+    dict(m=257, k=640, n=514, n_adapters=2, rank=8, swiglu=True),
+    dict(m=513, k=1024, n=260, n_adapters=64, rank=16, idx_mode="arange"),
 ])
 def test_tile_geometries_agree_bitwise(dev, pkg, shape):
-    """The 256 x 128 and 256 x 256 tile geometries compute every element the same way."""
+    """The 256 x 128 geometry (32 x 32 x 32 MFMAs, two workgroups per CU) and the 256 x 256 geometry
+    (16 x 16 x 64 MFMAs, one workgroup of eight waves per CU) agree: the int32 accumulators bit for bit, and so does the
+    bf16 output wherever no LoRA term is added.  With LoRA the two low-rank products add their ranks in
+    a different order inside the bf16 MFMAs (16 ranks per instruction against 32), which may move the
+    last bit of an output: both stay inside the tolerance against the oracle and agree on >= 99.9 %."""
     shape = dict(shape)
     m, k, n = shape.pop("m"), shape.pop("k"), shape.pop("n")
     case = wc.make_case(m, k, n, seed=29, **shape)
-    want = wc.oracle_forward(case)
-    narrow = wc.gpu_forward(case, flags=pkg._native.FLAG_FORCE_TILED | pkg._native.FLAG_TILE_256X128,
-                            return_aux=False)
-    wide = wc.gpu_forward(case, flags=pkg._native.FLAG_FORCE_TILED | pkg._native.FLAG_TILE_256X256,
-                          return_aux=False)
-    assert np.array_equal(narrow.view(np.uint32), wide.view(np.uint32))
-    _assert_close(wide, want, f" wide {m}x{k}x{n}")
+    want = wc.oracle_forward(case, return_stages=True)
+    narrow, aux_n = wc.gpu_forward(case, flags=pkg._native.FLAG_FORCE_TILED | pkg._native.FLAG_TILE_256X128)
+    wide, aux_w = wc.gpu_forward(case, flags=pkg._native.FLAG_FORCE_TILED | pkg._native.FLAG_TILE_256X256)
+    for aux in (aux_n, aux_w):
+        assert np.array_equal(aux["acc"], want["acc"])
+        assert np.array_equal(aux["x_codes"], want["x_codes"])
+    if shape.get("n_adapters", 1) == 0:
+        assert np.array_equal(narrow.view(np.uint32), wide.view(np.uint32))
+    else:
+        assert np.mean(narrow.view(np.uint32) == wide.view(np.uint32)) >= 0.999
+    _assert_close(narrow, want["out"], f" narrow {m}x{k}x{n}")
+    _assert_close(wide, want["out"], f" wide {m}x{k}x{n}")
 
 
 def test_split2_flag_stays_in_tolerance(dev, pkg):
