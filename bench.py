@@ -7,8 +7,14 @@ W8A8 [4096 x 4096] x [4096 x 24576] + 8 rank-32 adapters routed per row ->
 SwiGLU).  Inputs are resident in HBM before the timed region.  Prints ONE JSON
 line; ``value`` is int8 TOPS of the whole step (2*M*K*N per step, every kernel of
 the step included); ``roofline`` prices the dominant kernel (the int8 MFMA GEMM)
-from HIP events around that kernel alone; ``cpu_baseline`` times the NumPy oracle
-on a bounded row sample of the same workload on the host cores.
+from HIP events around that kernel alone, against the published peak and against
+the rate the same MFMA instruction sustains on realistic operands in a
+register-only loop; ``decode`` is the roofline block of the decode-shaped call
+(M = 16 down projection, HBM-bound) against the published bandwidth and a measured
+read-only stream; ``cpu_baseline`` times the NumPy oracle on a bounded row sample
+of the same workload on the host cores.  ``--workload calibration`` prints the
+ceilings alone, ``--workload qwen3-4b-attn-mixed-m`` a table over M of the
+attention projections.
 """
 
 from __future__ import annotations
@@ -16,6 +22,7 @@ from __future__ import annotations
 import argparse
 import json
 import os
+import re
 import sys
 import time
 from pathlib import Path
@@ -31,6 +38,11 @@ BF16_PEAK_TFLOPS = 2500.0 # MI355X dense bf16 MFMA, published (2.5 PFLOP/s)
 HBM_PEAK_GBS = 8000.0     # MI355X HBM3E, published
 
 WORKLOADS = {
+    # ceilings of the part: register-only int8 MFMA loops and a read-only stream
+    "calibration": dict(calibration=True),
+    # benchmark configuration 4: Qwen3-4B attention projections over M, 4 adapters rank 64 alpha 128, Student-t(3) rows
+    "qwen3-4b-attn-mixed-m": dict(mixed_m=True, shapes=[("qkv", 2560, 6144), ("o_proj", 4096, 2560)],
+                                  m_values=[1, 64, 512, 2048], n_adapters=4, rank=64, alpha=128, seed=4),
     # name: (m, k, n, adapters, rank, alpha, rms, swiglu, residual, idx_mode, seed)
     "qwen3-8b-gate_up-m4096": dict(m=4096, k=4096, n=24576, n_adapters=8, rank=32, rms=True, swiglu=True,
                                    idx_mode="uniform", seed=2),
@@ -73,22 +85,64 @@ WORKLOADS = {
                                           qkv=dict(num_query_heads=16, num_kv_heads=4, head_dim=256, rotary_dim=64)),
 }
 
-# HBM bytes per launch of the dominant kernel(s) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# (summaries under profiles/): (FETCH_SIZE * 2.0 + WRITE_SIZE * 1.0) KiB, the factors being what the
-# same counters read for a 256 MiB device copy with 16-byte loads.  None where not measured.
-MEASURED_TRAFFIC_BYTES = {
-    "qwen3-8b-gate_up-m4096": int((389417 * 2.0 + 129536) * 1024),                      # w8a8_gemm_kernel
-    "qwen3-8b-down-m16-decode": int(((8614 + 27632) * 2.0 + 4529 + 128) * 1024),       # both decode kernels
-    "qwen3-8b-gate_up-m4096-backward": int((400599 * 2.0 + 44726) * 1024),             # bwd_dx_kernel
-    "qwen3-30b-a3b-moe-mlp-t2048": int((250936 * 2.0 + 32332) * 1024),                 # grouped gate/up w8a8_gemm_kernel
-    # bwd_pack_dy_kernel + bwd_dx_kernel of the gate/up call without LoRA
-    "qwen3-30b-a3b-moe-experts-t2048-backward": int(((25875 + 225514) * 2.0 + 55008 + 66048) * 1024),
-    "qwen3-8b-gate_up-m4096-fused-backward": int((396251 * 2.0 + 35991) * 1024),       # bwd_dx_kernel
-    "qwen3-8b-down-m4096-w4a8-g128": int((233437 * 2.0 + 32768) * 1024),               # gq_gemm_kernel
-    "qwen3-30b-a3b-moe-routing-t4096": int((8487 * 2.0 + 131472) * 1024),              # the four dispatch kernels
-    "qwen3.5-4b-qkv-m2048": int((20611 * 2.0 + 40960) * 1024),                          # qkv_post_kernel
-    "qwen3.5-4b-qkv-m2048-backward": int((30830 * 2.0 + 40960) * 1024),                 # qkv_post_bwd_kernel
+# HBM bytes per launch of the dominant kernel(s): read from the counter lines of the committed rocprofv3
+# --pmc summaries under profiles/ (FETCH_SIZE and WRITE_SIZE in KiB per dispatch), each scaled by what the same
+# counter reads for the 256 MiB device copy of the same run (a kernel of known traffic, 16-byte loads).
+# workload -> (summary file, regular expressions naming the kernels whose traffic is summed)
+PROFILE_TRAFFIC = {
+    "qwen3-8b-gate_up-m4096": ("w8a8_gemm16_kernel__qwen3-8b-gate_up-m4096.txt", [r"w8a8_gemm16_kernel<1, 2>"]),
+    "qwen3-8b-down-m16-decode": ("skinny_stream_kernel__qwen3-8b-down-m16-decode.txt",
+                                 [r"skinny_quant_kernel<", r"skinny_stream_kernel<"]),
+    "qwen3-8b-gate_up-m4096-backward": ("bwd_dx_kernel__qwen3-8b-gate_up-m4096-backward.txt", [r"bwd_dx_kernel<"]),
+    "qwen3-30b-a3b-moe-mlp-t2048": ("w8a8_gemm_kernel_grouped__qwen3-30b-a3b-moe-mlp-t2048.txt",
+                                    [r"w8a8_gemm_kernel<1, 1, "]),  # grouped gate/up with the SwiGLU epilogue
+    "qwen3-30b-a3b-moe-experts-t2048-backward": ("bwd_dx_kernel_grouped__qwen3-30b-a3b-moe-experts-t2048-backward.txt",
+                                                 [r"bwd_pack_dy_kernel<0>", r"bwd_dx_kernel<0, true>"]),
+    "qwen3-8b-gate_up-m4096-fused-backward": ("swiglu_bwd_kernel__qwen3-8b-gate_up-m4096-fused-backward.txt",
+                                              [r"bwd_dx_kernel<"]),
+    "qwen3-8b-down-m4096-w4a8-g128": ("gq_gemm_kernel__qwen3-8b-down-m4096-w4a8-g128.txt", [r"gq_gemm_kernel<"]),
+    "qwen3-30b-a3b-moe-routing-t4096": ("moe_spread_kernel__qwen3-30b-a3b-moe-routing-t4096.txt",
+                                        [r"moe_hist_kernel", r"moe_scan_kernel", r"moe_scatter_kernel",
+                                         r"moe_spread_kernel"]),
+    "qwen3.5-4b-qkv-m2048": ("qkv_post_kernel__qwen3.5-4b-qkv-m2048.txt", [r"qkv_post_kernel\("]),
+    "qwen3.5-4b-qkv-m2048-backward": ("qkv_post_bwd_kernel__qwen3.5-4b-qkv-m2048-backward.txt",
+                                      [r"qkv_post_bwd_kernel<4, false>"]),
 }
+_COUNTER_LINE = re.compile(r"^(?P<name>.+?)\s+grid\s+(?P<grid>\d+)\s+(?P<ctr>FETCH_SIZE|WRITE_SIZE) avg\s+"
+                           r"(?P<kib>[0-9.]+) KiB over (?P<n>\d+) dispatches")
+COPY_KIB = 262144.0  # the calibration copy moves 256 MiB each way
+
+
+def measured_traffic_bytes(workload, profiles_dir=None):
+    """HBM bytes per launch of the workload's dominant kernel(s) from its committed counter summary, or None.
+
+    Every kernel named for the workload must appear once per counter and the summary must hold the
+    calibration copy; anything else (no summary yet, renamed kernel) gives None rather than a stale figure."""
+    entry = PROFILE_TRAFFIC.get(workload)
+    if entry is None:
+        return None
+    path = Path(profiles_dir or ROOT / "profiles") / entry[0]
+    if not path.exists():
+        return None
+    copy = {}
+    rows = []
+    for line in path.read_text().splitlines():
+        hit = _COUNTER_LINE.match(line)
+        if not hit:
+            continue
+        if "cal_copy_kernel" in hit["name"]:
+            copy[hit["ctr"]] = float(hit["kib"])
+        rows.append((hit["name"], hit["ctr"], float(hit["kib"])))
+    if set(copy) != {"FETCH_SIZE", "WRITE_SIZE"} or min(copy.values()) <= 0:
+        return None
+    total = 0.0
+    for pattern in entry[1]:
+        for ctr in ("FETCH_SIZE", "WRITE_SIZE"):
+            vals = [kib for name, c, kib in rows if c == ctr and re.search(pattern, name)]
+            if len(vals) != 1:
+                return None
+            total += vals[0] * (COPY_KIB / copy[ctr])
+    return int(total * 1024)
 
 
 def algorithmic_bytes(c):
@@ -116,6 +170,110 @@ def gemm_kernel_bytes(c):
     if c.get("residual"):
         total += 2 * m * n_out
     return total
+
+
+def _stream_ptr(dev):
+    import torch
+
+    return int(torch.cuda.current_stream(dev).cuda_stream)
+
+
+def calibration_operands(kind, nbytes, seed=1234):
+    """Operand bytes of the register-only MFMA loop.  Per wave 16 fragments of 1 KiB: 8 A then 8 B operands.
+    "zeros"; "random": random bits; "codes": what the path multiplies - activation codes of normal rows
+    quantized by their absolute maximum over 4096 samples (sigma about 127 / 3.9) against uniform weight codes."""
+    rng = np.random.default_rng(seed)
+    if kind == "zeros":
+        return np.zeros(nbytes, np.uint8)
+    if kind == "random":
+        return rng.integers(0, 256, nbytes, dtype=np.uint8)
+    frag = (np.arange(nbytes) >> 10) & 15
+    act = np.clip(np.rint(rng.standard_normal(nbytes) * (127.0 / 3.9)), -127, 127).astype(np.int8)
+    wgt = rng.integers(-127, 128, nbytes, dtype=np.int8)
+    return np.where(frag < 8, act, wgt).astype(np.int8).view(np.uint8)
+
+
+def measure_mfma_ceiling(native, dev, shape, kind, seconds=0.4, iters=2048):
+    """Sustained int8 TOP/s of the register-only MFMA loop and the shader clock it ran at."""
+    import torch
+
+    lib = native.load()
+    nbytes = int(lib.mi355_w8a8_calibrate_operand_bytes())
+    ops = float(lib.mi355_w8a8_calibrate_mfma_ops(shape, iters))
+    src = torch.from_numpy(calibration_operands(kind, nbytes)).to(dev)
+    clocks = torch.zeros(2, dtype=torch.int64, device=dev)
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    stream = _stream_ptr(dev)
+
+    def launch():
+        native.check("mi355_w8a8_calibrate_mfma_v1",
+                     lib.mi355_w8a8_calibrate_mfma_v1(shape, src.data_ptr(), iters, clocks.data_ptr(), sink.data_ptr(),
+                                                      stream))
+
+    launch()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record(); launch(); b.record()
+    torch.cuda.synchronize()
+    n = max(4, int(seconds * 1e3 / max(a.elapsed_time(b), 1e-3)))
+    for _ in range(n):  # the power controller settles over some hundred milliseconds: untimed
+        launch()
+    a.record()
+    for _ in range(n):
+        launch()
+    b.record()
+    torch.cuda.synchronize()
+    ms = a.elapsed_time(b) / n
+    cyc, ticks = (int(v) for v in clocks.cpu())
+    return {"shape": "16x16x64" if shape else "32x32x32", "operands": kind, "tops": ops / (ms * 1e-3) / 1e12,
+            "kernel_avg_ms": ms, "launches": n, "shader_mhz": cyc / max(ticks, 1) * 100.0}
+
+
+def measure_read_ceiling(native, dev, gib=2, launches=20):
+    """Sustained GB/s of a read-only stream over a buffer far beyond the 256 MB last-level cache."""
+    import torch
+
+    lib = native.load()
+    nbytes = gib << 30
+    src = torch.empty(nbytes, dtype=torch.uint8, device=dev).fill_(3)
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    stream = _stream_ptr(dev)
+
+    def launch():
+        native.check("mi355_w8a8_calibrate_read_v1",
+                     lib.mi355_w8a8_calibrate_read_v1(src.data_ptr(), nbytes, sink.data_ptr(), stream))
+
+    for _ in range(3):
+        launch()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(launches):
+        launch()
+    b.record()
+    torch.cuda.synchronize()
+    ms = a.elapsed_time(b) / launches
+    return {"bytes": nbytes, "gbs": nbytes / (ms * 1e-3) / 1e9, "kernel_avg_ms": ms, "launches": launches}
+
+
+def bench_calibration(args, pkg, dev):
+    """What this part sustains: register-only int8 MFMA loops (both instruction shapes; zero, random and
+    realistic operands) and a read-only stream.  The fractions of the other workloads can be read against
+    these as well as against the published peaks."""
+    native = pkg._native
+    mfma = [measure_mfma_ceiling(native, dev, shape, kind, seconds=1.0)
+            for kind in ("zeros", "random", "codes") for shape in (0, 1)]
+    read = measure_read_ceiling(native, dev)
+    best = max(r["tops"] for r in mfma if r["operands"] == "codes")
+    print(json.dumps({
+        "metric": "sustained int8 MFMA TOP/s on realistic operand codes (register-only loop); read stream GB/s",
+        "value": best, "unit": "TOPS", "n_gpus": 1, "steps": sum(r["launches"] for r in mfma), "warmup": 0,
+        "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8",
+        "data": "synthetic", "config": {"workload": args.workload},
+        "mfma": mfma, "read": read,
+        "roofline": {"bound": "mfma", "achieved": best, "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                     "frac": best / INT8_PEAK_TOPS, "traffic": None, "kernel": "cal_mfma_kernel<1>"},
+        "read_frac_of_hbm_peak": read["gbs"] / HBM_PEAK_GBS}))
+    return 0
 
 
 def cpu_baseline(case, cfg, sample_rows):
@@ -202,7 +360,7 @@ def bench_backward(args, cfg, pkg, dev):
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / BF16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "frac": achieved / BF16_PEAK_TFLOPS, "traffic": measured_traffic_bytes(args.workload),
                      "kernel": "bwd_dx_kernel",
                      "kernel_avg_ms": float(k_ms.mean()), "kernel_min_ms": float(k_ms.min()),
                      "algorithmic_flops": flops,
@@ -311,7 +469,7 @@ def bench_fused_backward(args, cfg, pkg, dev):
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / BF16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "kernel": "bwd_dx_kernel",
+                     "frac": achieved / BF16_PEAK_TFLOPS, "traffic": measured_traffic_bytes(args.workload), "kernel": "bwd_dx_kernel",
                      "kernel_avg_ms": float(k_ms.mean()), "kernel_min_ms": float(k_ms.min()),
                      "algorithmic_flops": flops, "algorithmic_bytes": 2 * m * n + k * n + 2 * m * k},
         "stages": {
@@ -405,7 +563,7 @@ def bench_moe_routing(args, cfg, pkg, dev):
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic_bytes(args.workload),
                      "kernel": "moe_hist_kernel + moe_scan_kernel + moe_scatter_kernel + moe_spread_kernel (one dispatch call)",
                      "kernel_avg_ms": dispatch_ms, "algorithmic_bytes": dispatch_bytes},
         "stages": {"route_ms": route_ms, "route_bytes": route_bytes, "dispatch_ms": dispatch_ms,
@@ -517,7 +675,7 @@ def bench_moe_mlp(args, cfg, pkg, dev):
         "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic_bytes(args.workload),
                      "kernel": "w8a8_gemm_kernel in grouped mode, gate/up projection with the SwiGLU epilogue",
                      "kernel_avg_ms": gemm_ms, "algorithmic_bytes": gemm_bytes, "algorithmic_ops": gu_ops,
                      "frac_of_int8_mfma_peak": gu_ops / (gemm_ms * 1e-3) / 1e12 / INT8_PEAK_TOPS},
@@ -634,7 +792,7 @@ def bench_moe_backward(args, cfg, pkg, dev):
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic_bytes(args.workload),
                      "kernel": "the gate/up call without LoRA (tables, bwd_pack_dy_kernel, bwd_dx_kernel)",
                      "kernel_avg_ms": float(dx_ms.mean()), "kernel_min_ms": float(dx_ms.min()),
                      "algorithmic_bytes": dx_bytes, "algorithmic_flops": gu_flops,
@@ -723,7 +881,7 @@ def bench_gq(args, cfg, pkg, dev):
         "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-                     "frac": achieved / INT8_PEAK_TOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "frac": achieved / INT8_PEAK_TOPS, "traffic": measured_traffic_bytes(args.workload),
                      "kernel": "gq_gemm_kernel (timed with gq_quant_kernel and gq_lora_z_kernel: whole calls)",
                      "kernel_avg_ms": call_ms, "algorithmic_ops": ops,
                      "algorithmic_bytes": 2 * m * k + k * n * wb // 8 + 4 * (k // group) * n + 2 * m * n},
@@ -800,7 +958,7 @@ def bench_qkv(args, cfg, pkg, dev):
         "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic_bytes(args.workload),
                      "kernel": "qkv_post_kernel",
                      "kernel_avg_ms": float(k_ms.mean()), "kernel_min_ms": float(k_ms.min()),
                      "algorithmic_bytes": bytes_alg},
@@ -913,7 +1071,7 @@ def bench_qkv_backward(args, cfg, pkg, dev):
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic_bytes(args.workload),
                      "kernel": "qkv_post_bwd_kernel",
                      "kernel_avg_ms": float(k_ms.mean()), "kernel_min_ms": float(k_ms.min()),
                      "algorithmic_bytes": bytes_alg},
@@ -951,6 +1109,166 @@ def bench_qkv_backward(args, cfg, pkg, dev):
     return 0
 
 
+def measure_linear(args, cfg, pkg, dev, steps, warmup, rotate, workload=None, flags=None):
+    """Time one dense forward workload: whole steps (host clock around `steps` back-to-back calls and one HIP
+    event pair per step), the dominant kernel alone, the prologue alone."""
+    import torch
+
+    import w8a8_cases as wc
+
+    native = pkg._native
+    w8 = pkg.w8a8_lora
+    workload = workload or args.workload
+    flags = args.flags if flags is None else flags
+    case = wc.make_case(cfg["m"], cfg["k"], cfg["n"], n_adapters=cfg.get("n_adapters", 0),
+                        rank=cfg.get("rank", 16), seed=cfg["seed"], rms=cfg.get("rms", False),
+                        residual=cfg.get("residual", False), swiglu=cfg.get("swiglu", False),
+                        idx_mode=cfg.get("idx_mode", "uniform"), student_t=cfg.get("x_dist") == "student_t3",
+                        alpha=cfg.get("alpha"))
+    path_flags = flags | (native.FLAG_SWIGLU if cfg.get("swiglu") else 0)
+    path = native.PATH_NAMES.get(native.load().mi355_w8a8_forward_path(cfg["m"], cfg["k"], cfg["n"], path_flags), "?")
+    skinny = path.startswith("skinny")
+    rotate = rotate or (max(1, -(-768_000_000 // algorithmic_bytes(cfg))) if skinny else 1)
+    plans = []
+    for _ in range(rotate):
+        t = wc.to_torch(case, dev)  # a fresh copy of every operand (and its own packed weight)
+        plans.append(w8.ForwardPlan(t["x"], t["weight"], t.get("a"), t.get("b"), t.get("s"),
+                                    adapter_indices=t.get("idx"), rms_gamma=t.get("gamma"), eps=1e-6,
+                                    residual=t.get("residual"), swiglu=bool(cfg.get("swiglu")),
+                                    flags=flags))
+    plan = plans[0]
+    torch.cuda.synchronize()
+    # Spin-up, untimed and before the warm-up steps: the first launches after idle run while clocks and the
+    # power controller settle (up to 20 % slow); the figure quoted is the sustained one.
+    t0 = time.perf_counter()
+    i = 0
+    while time.perf_counter() - t0 < args.spin_up:
+        for _ in range(8):
+            plans[i % rotate].run()
+            i += 1
+        torch.cuda.synchronize()
+    spin_up_s = time.perf_counter() - t0
+    for i in range(warmup):
+        plans[i % rotate].run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        plans[i % rotate].run()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / steps * 1e3
+    ops = 2.0 * cfg["m"] * cfg["k"] * cfg["n"]
+
+    def event_pairs(fn):
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        for i, (a, b) in enumerate(ev):
+            a.record()
+            fn(i)
+            b.record()
+        torch.cuda.synchronize()
+        return np.asarray([a.elapsed_time(b) for a, b in ev])
+
+    # whole steps again, one event pair each: where the step time sits when the host clock is not in it
+    step_ms = event_pairs(lambda i: plans[i % rotate].run())
+    step_event_ms = {"median": float(np.median(step_ms)), "p10": float(np.percentile(step_ms, 10)),
+                     "p90": float(np.percentile(step_ms, 90))}
+
+    # dominant kernel alone: HIP events (torch's current stream is the launch stream) around
+    # GEMM-only launches; the workspace still holds the prologue's results.
+    # (a call that runs as 32-row chunks of the streaming kernels keeps no stage to rerun: the library
+    # says so, and the figures below are then taken around whole calls)
+    try:
+        plans[0].run(native.FLAG_SKIP_PROLOGUE)
+        stage_flags = (native.FLAG_SKIP_PROLOGUE, native.FLAG_SKIP_GEMM)
+    except native.NativeError as err:
+        if err.status != -7:
+            raise
+        stage_flags = (0, 0)
+    gemm_ms = event_pairs(lambda i: plans[i % rotate].run(stage_flags[0]))
+    gemm_avg_ms = float(gemm_ms.mean())
+    # prologue alone (routing + quantization + LoRA-A)
+    pa, pb = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    pa.record()
+    for i in range(steps):
+        plans[i % rotate].run(stage_flags[1])
+    pb.record()
+    torch.cuda.synchronize()
+    prologue_ms = pa.elapsed_time(pb) / steps if stage_flags[1] else None
+    out_gpu = plan.run()
+    torch.cuda.synchronize()
+
+    if skinny:
+        # the decode path is two short kernels per 32 rows; the figure prices them together against the
+        # algorithmic bytes of the whole call.  They last ~20 us together and an event pair around a single
+        # call adds ~2.5 us of its own, so the average launch duration comes from one event pair around all
+        # the steps (back-to-back calls on the launch stream), per call.
+        ra, rb = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ra.record()
+        for i in range(steps):
+            plans[i % rotate].run()
+        rb.record()
+        torch.cuda.synchronize()
+        region_ms = ra.elapsed_time(rb) / steps
+        bytes_alg = algorithmic_bytes(cfg)
+        achieved = bytes_alg / (region_ms * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic_bytes(workload),
+                    "kernel": "skinny_quant_kernel + skinny_stream_kernel",
+                    "kernel_avg_ms": region_ms, "single_call_event_avg_ms": float(step_ms.mean()),
+                    "kernel_min_ms": float(step_ms.min()),
+                    "stream_and_epilogue_avg_ms": gemm_avg_ms, "algorithmic_bytes": bytes_alg,
+                    "operand_sets_rotated": rotate}
+    else:
+        achieved = ops / (gemm_avg_ms * 1e-3) / 1e12
+        roofline = {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                    "frac": achieved / INT8_PEAK_TOPS, "traffic": measured_traffic_bytes(workload),
+                    "kernel": "w8a8_gemm16_kernel" if path == "tiled-256x256" else "w8a8_gemm_kernel",
+                    "kernel_avg_ms": gemm_avg_ms, "kernel_min_ms": float(gemm_ms.min()), "algorithmic_ops": ops,
+                    "algorithmic_bytes": gemm_kernel_bytes(cfg)}
+    return {"ms_per_step": ms_per_step, "ops": ops, "roofline": roofline, "prologue_ms": prologue_ms,
+            "step_event_ms": step_event_ms, "spin_up_s": spin_up_s, "path": path, "case": case,
+            "out_gpu": out_gpu}
+
+
+def bench_mixed_m(args, cfg, pkg, dev):
+    """Benchmark configuration 4: the Qwen3-4B attention projections (QKV [2560 -> 6144] and o_proj
+    [4096 -> 2560]) with 4 adapters of rank 64 on Student-t(3) activations, at M = 1, 64, 512, 2048.  One JSON
+    line with a row per (shape, M); `value` is the int8 TOPS of the largest point."""
+    rows = []
+    for name, k, n in cfg["shapes"]:
+        for m in cfg["m_values"]:
+            c = dict(m=m, k=k, n=n, n_adapters=cfg["n_adapters"], rank=cfg["rank"], alpha=cfg["alpha"],
+                     idx_mode="uniform", x_dist="student_t3", seed=cfg["seed"])
+            r = measure_linear(args, c, pkg, dev, args.steps, args.warmup, 0, workload=f"{args.workload}/{name}/m{m}")
+            roof = r["roofline"]
+            bytes_alg = algorithmic_bytes(c)
+            call_ms = roof["kernel_avg_ms"] if roof["bound"] == "hbm" else r["step_event_ms"]["median"]
+            rows.append({"shape": name, "m": m, "k": k, "n": n, "path": r["path"], "ms_per_step": r["ms_per_step"],
+                         "call_ms": call_ms, "tops": r["ops"] / (call_ms * 1e-3) / 1e12,
+                         "gbs": bytes_alg / (call_ms * 1e-3) / 1e9,
+                         # a point is priced against the bound it is nearer to at its published peak
+                         "bound": "mfma" if r["ops"] / INT8_PEAK_TOPS / 1e12 > bytes_alg / HBM_PEAK_GBS / 1e9 else "hbm",
+                         "frac_of_int8_peak": r["ops"] / (call_ms * 1e-3) / 1e12 / INT8_PEAK_TOPS,
+                         "frac_of_hbm_peak": bytes_alg / (call_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                         "dominant_kernel_ms": roof["kernel_avg_ms"], "prologue_ms": r["prologue_ms"]})
+            del r
+    for row in rows:
+        row["frac"] = row["frac_of_int8_peak"] if row["bound"] == "mfma" else row["frac_of_hbm_peak"]
+    top = max(rows, key=lambda row: row["tops"])
+    print(json.dumps({
+        "metric": "W8A8-LoRA linear TOPS / GB/s over M (Qwen3-4B attention projections, Student-t(3) activations)",
+        "value": top["tops"], "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": top["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8", "data": "synthetic",
+        "config": {"workload": args.workload, "n_adapters": cfg["n_adapters"], "rank": cfg["rank"],
+                   "alpha": cfg["alpha"], "x_dist": "student_t3"},
+        "points": rows,
+        "roofline": {"bound": top["bound"], "achieved": top["tops"], "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                     "frac": top["frac_of_int8_peak"], "traffic": None,
+                     "kernel": f"whole call, {top['shape']} M={top['m']} ({top['path']})"}}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -968,6 +1286,10 @@ def main() -> int:
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 256 MiB device copy (a kernel of known traffic for scaling the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
+    ap.add_argument("--spin-up", type=float, default=0.5,
+                    help="seconds of untimed calls before the warm-up steps (clocks and power controller settle)")
+    ap.add_argument("--no-decode", action="store_true", help="default workload: skip the decode block")
+    ap.add_argument("--no-ceilings", action="store_true", help="default workload: skip the measured ceilings")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path has no collectives); use --gpus 1",
@@ -995,9 +1317,13 @@ def main() -> int:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
         dst = torch.empty_like(src)
         torch.cuda.synchronize()
-        dst.copy_(src)
+        native.check("mi355_w8a8_calibrate_copy_v1",
+                     native.load().mi355_w8a8_calibrate_copy_v1(src.data_ptr(), dst.data_ptr(), 256 << 20,
+                                                                _stream_ptr(dev)))
         torch.cuda.synchronize()
         del src, dst
+    if cfg.pop("calibration", False):
+        return bench_calibration(args, pkg, dev)
     if cfg.pop("backward", False):
         if cfg.get("swiglu"):
             return bench_fused_backward(args, cfg, pkg, dev)
@@ -1014,127 +1340,50 @@ def main() -> int:
         return bench_qkv_backward(args, cfg, pkg, dev)
     if "qkv" in cfg:
         return bench_qkv(args, cfg, pkg, dev)
-    case = wc.make_case(cfg["m"], cfg["k"], cfg["n"], n_adapters=cfg.get("n_adapters", 0),
-                        rank=cfg.get("rank", 16), seed=cfg["seed"], rms=cfg.get("rms", False),
-                        residual=cfg.get("residual", False), swiglu=cfg.get("swiglu", False),
-                        idx_mode=cfg.get("idx_mode", "uniform"))
-    skinny = cfg["m"] <= 32
-    rotate = args.rotate or (max(1, -(-768_000_000 // algorithmic_bytes(cfg))) if skinny else 1)
-    plans = []
-    for _ in range(rotate):
-        t = wc.to_torch(case, dev)  # a fresh copy of every operand (and its own packed weight)
-        plans.append(w8.ForwardPlan(t["x"], t["weight"], t.get("a"), t.get("b"), t.get("s"),
-                                    adapter_indices=t.get("idx"), rms_gamma=t.get("gamma"), eps=1e-6,
-                                    residual=t.get("residual"), swiglu=bool(cfg.get("swiglu")),
-                                    flags=args.flags))
-    plan = plans[0]
-    torch.cuda.synchronize()
-    for i in range(args.warmup):
-        plans[i % rotate].run()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        plans[i % rotate].run()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed / args.steps * 1e3
-    ops = 2.0 * cfg["m"] * cfg["k"] * cfg["n"]
-    tops = ops / (ms_per_step * 1e-3) / 1e12
-
-    # dominant kernel alone: HIP events (torch's current stream is the launch stream) around
-    # GEMM-only launches; the workspace still holds the prologue's results.
-    # (a call of 33..128 rows that runs as 32-row chunks of the streaming kernels keeps no stage to
-    # rerun: the library says so, and the figures below are then taken around whole calls)
-    try:
-        plans[0].run(native.FLAG_SKIP_PROLOGUE)
-        stage_flags = (native.FLAG_SKIP_PROLOGUE, native.FLAG_SKIP_GEMM)
-    except native.NativeError as err:
-        if err.status != -7:
-            raise
-        stage_flags = (0, 0)
-        skinny = True
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-          for _ in range(args.steps)]
-    for i, (a, b) in enumerate(ev):
-        a.record()
-        plans[i % rotate].run(stage_flags[0])
-        b.record()
-    torch.cuda.synchronize()
-    gemm_ms = np.asarray([a.elapsed_time(b) for a, b in ev])
-    gemm_avg_ms = float(gemm_ms.mean())
-    # prologue alone (routing + quantization + LoRA-A)
-    pa, pb = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    pa.record()
-    for i in range(args.steps):
-        plans[i % rotate].run(stage_flags[1])
-    pb.record()
-    torch.cuda.synchronize()
-    prologue_ms = pa.elapsed_time(pb) / args.steps if stage_flags[1] else None
-    out_gpu = plan.run()
-    torch.cuda.synchronize()
-
-    if skinny:
-        # the decode path is two short kernels; the figure prices both together against
-        # the algorithmic bytes of the whole call (events around full calls)
-        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-              for _ in range(args.steps)]
-        for i, (a, b) in enumerate(ev):
-            a.record()
-            plans[i % rotate].run()
-            b.record()
-        torch.cuda.synchronize()
-        call_ms = np.asarray([a.elapsed_time(b) for a, b in ev])
-        # the two kernels of a call last ~23 us together, an event pair around a single call adds
-        # ~2.5 us of its own; the average launch duration is therefore taken from one event pair
-        # around all the steps (back-to-back calls on the launch stream), per call
-        ra, rb = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        ra.record()
-        for i in range(args.steps):
-            plans[i % rotate].run()
-        rb.record()
-        torch.cuda.synchronize()
-        region_ms = ra.elapsed_time(rb) / args.steps
-        bytes_alg = algorithmic_bytes(cfg)
-        achieved = bytes_alg / (region_ms * 1e-3) / 1e9
-        roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-                    "kernel": "skinny_quant_kernel + skinny_stream_kernel",
-                    "kernel_avg_ms": region_ms, "single_call_event_avg_ms": float(call_ms.mean()),
-                    "kernel_min_ms": float(call_ms.min()),
-                    "stream_and_epilogue_avg_ms": gemm_avg_ms, "algorithmic_bytes": bytes_alg,
-                    "operand_sets_rotated": rotate}
-    else:
-        achieved = ops / (gemm_avg_ms * 1e-3) / 1e12
-        # the library's choice of geometry (run_forward in csrc/w8a8_api.hip): the 256 x 256 kernel when its
-        # tiles fill the 256 CUs and K has at least six 64-wide steps, unless a flag forces one
-        pad = lambda v, q: -(-v // q) * q
-        wide = (pad(cfg["m"], 256) // 256) * (pad(cfg["n"], 256) // 256) >= 256 and pad(cfg["k"], 128) >= 384
-        if args.flags & native.FLAG_TILE_256X128:
-            wide = False
-        if args.flags & native.FLAG_TILE_256X256:
-            wide = pad(cfg["k"], 128) >= 384
-        roofline = {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-                    "frac": achieved / INT8_PEAK_TOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-                    "kernel": "w8a8_gemm16_kernel" if wide else "w8a8_gemm_kernel", "kernel_avg_ms": gemm_avg_ms,
-                    "kernel_min_ms": float(gemm_ms.min()), "algorithmic_ops": ops,
-                    "algorithmic_bytes": gemm_kernel_bytes(cfg)}
-
+    if cfg.pop("mixed_m", False):
+        return bench_mixed_m(args, cfg, pkg, dev)
+    r = measure_linear(args, cfg, pkg, dev, args.steps, args.warmup, args.rotate)
+    tops = r["ops"] / (r["ms_per_step"] * 1e-3) / 1e12
     result = {
         "metric": "W8A8-LoRA GEMM TOPS & % int8 MFMA peak (Qwen3-8B MLP, M=4096); decode GB/s",
         "value": tops, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8", "data": "synthetic",
         "config": {"workload": args.workload, **{k: v for k, v in cfg.items() if k != "seed"}},
         "frac_of_int8_peak_whole_step": tops / INT8_PEAK_TOPS,
-        "whole_step_gbs": algorithmic_bytes(cfg) / (ms_per_step * 1e-3) / 1e9,
-        "prologue_ms": prologue_ms,
-        "roofline": roofline,
+        "whole_step_gbs": algorithmic_bytes(cfg) / (r["ms_per_step"] * 1e-3) / 1e9,
+        "step_event_ms": r["step_event_ms"],
+        "spin_up_s": r["spin_up_s"],
+        "prologue_ms": r["prologue_ms"],
+        "path": r["path"],
+        "roofline": r["roofline"],
     }
+    if args.workload == "qwen3-8b-gate_up-m4096" and not args.no_decode:
+        # the second half of the metric: the decode-shaped call (M = 16 down projection with residual),
+        # enough independent operand sets that no call finds its weights in the last-level cache
+        dcfg = dict(WORKLOADS["qwen3-8b-down-m16-decode"])
+        d = measure_linear(args, dcfg, pkg, dev, max(args.steps, 48), max(args.warmup, 12), 0,
+                           workload="qwen3-8b-down-m16-decode")
+        result["decode"] = {"workload": "qwen3-8b-down-m16-decode",
+                            "config": {k: v for k, v in dcfg.items() if k != "seed"},
+                            "ms_per_step": d["ms_per_step"], "path": d["path"], **d["roofline"]}
+        del d
+    if args.workload == "qwen3-8b-gate_up-m4096" and not args.no_ceilings:
+        # what the part sustains on the same instruction with realistic operand codes and nothing else to do,
+        # and on a read-only stream: second denominators beside the published peaks
+        ceil = measure_mfma_ceiling(native, dev, 1, "codes")
+        result["roofline"]["measured_mfma_ceiling_tops"] = ceil["tops"]
+        result["roofline"]["measured_mfma_ceiling_mhz"] = ceil["shader_mhz"]
+        result["roofline"]["frac_of_measured_ceiling"] = result["roofline"]["achieved"] / ceil["tops"]
+        if "decode" in result:
+            rd = measure_read_ceiling(native, dev)
+            result["decode"]["measured_read_ceiling_gbs"] = rd["gbs"]
+            result["decode"]["frac_of_measured_ceiling"] = result["decode"]["achieved"] / rd["gbs"]
     if not args.no_cpu_baseline:
         rows = args.cpu_rows or cfg["m"]
-        want, base = cpu_baseline(case, cfg, rows)
+        want, base = cpu_baseline(r["case"], cfg, rows)
         result["cpu_baseline"] = base
-        got = out_gpu[:rows].to(torch.float32).cpu().numpy()
+        got = r["out_gpu"][:rows].to(torch.float32).cpu().numpy()
         rep = wc.compare(got, want)
         result["parity_sample"] = {"rows": rows, "violations": rep["violations"], "size": rep["size"],
                                    "max_abs": rep["max_abs"], "bitwise_fraction": rep["bitwise_fraction"]}

@@ -508,6 +508,37 @@ uint64_t mi355_w8a8_gq_workspace_bytes(uint32_t m, uint32_t k_pad, uint32_t grou
                                        uint32_t rank);
 int mi355_w8a8_gq_linear_v1(const mi355_w8a8_gq_problem* problem, void* stream);
 
+/*
+ * Which kernels mi355_w8a8_forward_v1 and its three named forms run for these dimensions and flags
+ * (no counterpart in the reference; for benchmarks and logs).  Returns an MI355_W8A8_PATH_* value or
+ * a negative status.
+ */
+#define MI355_W8A8_PATH_SKINNY 1         /* m <= 32: row quantizer + weight-streaming kernel */
+#define MI355_W8A8_PATH_SKINNY_CHUNKS 2  /* 33..128 rows: the same two kernels per chunk of 32 rows */
+#define MI355_W8A8_PATH_TILED_256X128 3  /* prologue + 256 x 128 tiles, two workgroups per CU */
+#define MI355_W8A8_PATH_TILED_256X256 4  /* prologue + 256 x 256 tiles, one workgroup per CU */
+int mi355_w8a8_forward_path(uint32_t m, uint32_t k, uint32_t n, uint32_t flags);
+
+/*
+ * Calibration (no counterpart in the reference: these measure the ceilings the path is priced against,
+ * for bench.py and profiles/).  mi355_w8a8_calibrate_mfma_v1 runs `iters` rounds of int8 MFMAs on
+ * operands that stay in registers: shape 0 = 16 of the 32 x 32 x 32 instruction per wave and round,
+ * shape 1 = 64 of the 16 x 16 x 64 one; 256 workgroups of four waves.  `operands` holds
+ * mi355_w8a8_calibrate_operand_bytes() bytes of codes (zeros, random bits, realistic codes: the rate
+ * the part sustains under its power limit depends on them).  One launch performs
+ * mi355_w8a8_calibrate_mfma_ops(shape, iters) int8 operations.  `clocks` (2 x uint64) receives the
+ * shader cycles and the 100 MHz ticks one workgroup spent in the loop; `sink` is 4 writable bytes.
+ * mi355_w8a8_calibrate_read_v1 streams `bytes` (a multiple of 32768) from `src` and discards them.
+ * mi355_w8a8_calibrate_copy_v1 copies `bytes` (a multiple of 16) with 16-byte loads and stores: a kernel of
+ * known traffic against which hardware traffic counters are scaled.
+ */
+uint64_t mi355_w8a8_calibrate_operand_bytes(void);
+uint64_t mi355_w8a8_calibrate_mfma_ops(uint32_t shape, uint32_t iters);
+int mi355_w8a8_calibrate_mfma_v1(uint32_t shape, const void* operands, uint32_t iters, uint64_t* clocks,
+                                 int32_t* sink, void* stream);
+int mi355_w8a8_calibrate_read_v1(const void* src, uint64_t bytes, uint32_t* sink, void* stream);
+int mi355_w8a8_calibrate_copy_v1(const void* src, void* dst, uint64_t bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -23,6 +23,7 @@ FLAG_TILE_256X128 = 64
 FLAG_TILE_256X256 = 128
 FLAG_GROUPED_TILE64 = 256
 FLAG_GROUPED_TILE128 = 512
+PATH_NAMES = {1: "skinny", 2: "skinny-chunks", 3: "tiled-256x128", 4: "tiled-256x256"}
 
 STATUS = {
     0: "OK", -1: "ERR_NULL", -2: "ERR_SHAPE", -3: "ERR_ALIGN", -4: "ERR_ALIAS",
@@ -45,6 +46,8 @@ EXPORTS = (
     "mi355_w8a8_moe_combine_v1", "mi355_w8a8_moe_combine_bwd_v1",
     "mi355_w8a8_gq_packed_weight_bytes", "mi355_w8a8_gq_pack_weight_v1", "mi355_w8a8_gq_workspace_bytes",
     "mi355_w8a8_gq_linear_v1",
+    "mi355_w8a8_forward_path", "mi355_w8a8_calibrate_operand_bytes", "mi355_w8a8_calibrate_mfma_ops", "mi355_w8a8_calibrate_mfma_v1",
+    "mi355_w8a8_calibrate_read_v1", "mi355_w8a8_calibrate_copy_v1",
 )
 
 _u32, _u64, _vp, _f32 = ctypes.c_uint32, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_float
@@ -219,6 +222,18 @@ def _bind(lib: ctypes.CDLL) -> None:
     lib.mi355_w8a8_gq_workspace_bytes.argtypes = (_u32, _u32, _u32, _u32, _u32)
     lib.mi355_w8a8_gq_linear_v1.restype = ctypes.c_int
     lib.mi355_w8a8_gq_linear_v1.argtypes = (ctypes.POINTER(GqProblem), _vp)
+    lib.mi355_w8a8_forward_path.restype = ctypes.c_int
+    lib.mi355_w8a8_forward_path.argtypes = (_u32, _u32, _u32, _u32)
+    lib.mi355_w8a8_calibrate_operand_bytes.restype = _u64
+    lib.mi355_w8a8_calibrate_operand_bytes.argtypes = ()
+    lib.mi355_w8a8_calibrate_mfma_ops.restype = _u64
+    lib.mi355_w8a8_calibrate_mfma_ops.argtypes = (_u32, _u32)
+    lib.mi355_w8a8_calibrate_mfma_v1.restype = ctypes.c_int
+    lib.mi355_w8a8_calibrate_mfma_v1.argtypes = (_u32, _vp, _u32, _vp, _vp, _vp)
+    lib.mi355_w8a8_calibrate_read_v1.restype = ctypes.c_int
+    lib.mi355_w8a8_calibrate_read_v1.argtypes = (_vp, _u64, _vp, _vp)
+    lib.mi355_w8a8_calibrate_copy_v1.restype = ctypes.c_int
+    lib.mi355_w8a8_calibrate_copy_v1.argtypes = (_vp, _vp, _u64, _vp)
     lib.mi355_w8a8_swiglu_v1.restype = ctypes.c_int
     lib.mi355_w8a8_swiglu_v1.argtypes = (_vp, _vp, _u32, _u32, _vp)
     lib.mi355_w8a8_swiglu_bwd_v1.restype = ctypes.c_int

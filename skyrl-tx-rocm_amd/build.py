@@ -23,7 +23,7 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-ffp-contract=off", "-fno-fast-math",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wall", "-Wextra", "-Wno-unused-parameter", "-Wl,-z,defs", "-Wl,-z,relro", "-Wl,-z,now",
+    "-Wall", "-Wextra", "-Wno-unused-parameter", "-Wno-inline-asm", "-Wl,-z,defs", "-Wl,-z,relro", "-Wl,-z,now",
 ]
 
 

@@ -7,6 +7,7 @@
 #include "w8a8_device.h"
 #include "w8a8_gemm.h"
 #include "w8a8_gemm16.h"
+#include "w8a8_calibration.h"
 #include "w8a8_prologue.h"
 #include "w8a8_skinny.h"
 #include "w8a8_backward.h"
@@ -224,6 +225,29 @@ int launch_skinny(const mi355_w8a8_problem* p, unsigned char* xq, float* sx, uin
 
 enum Required { kReqNone = 0, kReqLinear = 1, kReqGateUp = 2, kReqResidual = 3 };
 
+// Which kernels a forward call of these dimensions runs (an MI355_W8A8_PATH_* value), or a negative
+// status for a contradictory request.  The choice depends on the dimensions and the flags only.
+int choose_forward_path(uint32_t m, uint32_t k, uint32_t n, uint32_t flags) {
+  const bool swiglu = (flags & MI355_W8A8_FLAG_SWIGLU) != 0;
+  bool skinny = m <= (uint32_t)kSkinnyMaxRows && !(flags & MI355_W8A8_FLAG_FORCE_TILED) && !swiglu;
+  if (flags & MI355_W8A8_FLAG_FORCE_SKINNY) {
+    if (m > (uint32_t)kSkinnyMaxRows || swiglu) return MI355_W8A8_ERR_UNSUPPORTED;
+    skinny = true;
+  }
+  if (!skinny_supported()) skinny = false;
+  if (skinny) return MI355_W8A8_PATH_SKINNY;
+  if (skinny_supported() && !swiglu && skinny_chunked_pays(m, k, n) &&
+      !(flags & (MI355_W8A8_FLAG_FORCE_TILED | MI355_W8A8_FLAG_TILE_256X128 | MI355_W8A8_FLAG_TILE_256X256)))
+    return MI355_W8A8_PATH_SKINNY_CHUNKS;
+  // 256 x 256 tiles (one 8-wave workgroup per CU, 16 x 16 x 64 MFMAs) once they can fill every CU;
+  // below that the 256 x 128 geometry (two 4-wave workgroups per CU) has twice the tiles to spread.
+  bool wide = (uint64_t)(round_up(m, kTileM) / kTileM) * (n_padded(n) / kG16TileN) >= 256u;
+  if (flags & MI355_W8A8_FLAG_TILE_256X128) wide = false;
+  if (flags & MI355_W8A8_FLAG_TILE_256X256) wide = true;
+  if (k_padded(k) < kG16MinKPad) wide = false;  // its stage schedule needs at least six 64-wide k steps
+  return wide ? MI355_W8A8_PATH_TILED_256X256 : MI355_W8A8_PATH_TILED_256X128;
+}
+
 int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   if (!p) return MI355_W8A8_ERR_NULL;
   if (p->struct_size != sizeof(mi355_w8a8_problem)) return MI355_W8A8_ERR_STRUCT;
@@ -277,19 +301,14 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
 
   (void)hipGetLastError();  // drop a stale error so it is not blamed on these launches
 
-  bool skinny = p->m <= (uint32_t)kSkinnyMaxRows && !(p->flags & MI355_W8A8_FLAG_FORCE_TILED) && !swiglu;
-  if ((p->flags & MI355_W8A8_FLAG_FORCE_SKINNY)) {
-    if (p->m > (uint32_t)kSkinnyMaxRows || swiglu) return MI355_W8A8_ERR_UNSUPPORTED;
-    skinny = true;
-  }
-  if (!skinny_supported()) skinny = false;
-
+  const int path = choose_forward_path(p->m, p->k, p->n, p->flags);
+  if (path < 0) return path;
+  const bool skinny = path == MI355_W8A8_PATH_SKINNY;
   if (skinny) {
     return launch_skinny(p, ws + w.xq, reinterpret_cast<float*>(ws + w.sx),
                          reinterpret_cast<uint16_t*>(ws + w.xn), ws + w.skinny, w.K_pad, w.KB, s);
   }
-  if (skinny_supported() && !swiglu && skinny_chunked_pays(p->m, p->k, p->n) &&
-      !(p->flags & (MI355_W8A8_FLAG_FORCE_TILED | MI355_W8A8_FLAG_TILE_256X128 | MI355_W8A8_FLAG_TILE_256X256))) {
+  if (path == MI355_W8A8_PATH_SKINNY_CHUNKS) {
     // The chunks overwrite each other's prologue results, so there is no GEMM-only or prologue-only
     // rerun of such a call; the choice of path must not depend on those flags either (a GEMM-only
     // tiled call would read tables no tiled prologue has written).
@@ -394,12 +413,7 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   g.tiles_n = n_padded(p->n) / kGemmTileN;
   g.rank = lora ? p->rank : 0u;
   g.tile_ctr = reinterpret_cast<uint32_t*>(ws + w.tile_ctr);
-  // 256 x 256 tiles (one 4-wave workgroup per CU, 16 x 16 x 64 MFMAs) once they can fill every CU;
-  // below that the 256 x 128 geometry (two 4-wave workgroups per CU) has twice the tiles to spread.
-  bool wide = (uint64_t)g.tiles_m * (n_padded(p->n) / kG16TileN) >= 256u;
-  if (p->flags & MI355_W8A8_FLAG_TILE_256X128) wide = false;
-  if (p->flags & MI355_W8A8_FLAG_TILE_256X256) wide = true;
-  if (w.K_pad < kG16MinKPad) wide = false;  // its stage schedule needs at least six 64-wide k steps
+  const bool wide = path == MI355_W8A8_PATH_TILED_256X256;
   if (wide) g.tiles_n = n_padded(p->n) / kG16TileN;
   if (p->aux_acc) {
     GemmArgs ga = g;
@@ -1845,6 +1859,52 @@ uint64_t mi355_w8a8_gq_workspace_bytes(uint32_t m, uint32_t k_pad, uint32_t grou
 
 int mi355_w8a8_gq_linear_v1(const mi355_w8a8_gq_problem* p, void* stream) {
   return run_gq_linear(p, static_cast<hipStream_t>(stream));
+}
+
+int mi355_w8a8_forward_path(uint32_t m, uint32_t k, uint32_t n, uint32_t flags) {
+  const int st = validate_common(m, k, n);
+  if (st) return st;
+  if ((flags & MI355_W8A8_FLAG_FORCE_TILED) && (flags & MI355_W8A8_FLAG_FORCE_SKINNY)) return MI355_W8A8_ERR_SHAPE;
+  return choose_forward_path(m, k, n, flags);
+}
+
+uint64_t mi355_w8a8_calibrate_operand_bytes(void) { return kCalOperandBytes; }
+
+uint64_t mi355_w8a8_calibrate_mfma_ops(uint32_t shape, uint32_t iters) {
+  // per wave and round: 16 x (2 x 32 x 32 x 32) or 64 x (2 x 16 x 16 x 64) operations; 4 waves x 256 workgroups
+  if (shape > 1u) return 0;
+  return (shape == 1u ? 64ull * 32768ull : 16ull * 65536ull) * 4ull * kCalGrid * iters;
+}
+
+int mi355_w8a8_calibrate_mfma_v1(uint32_t shape, const void* operands, uint32_t iters, uint64_t* clocks,
+                                 int32_t* sink, void* stream) {
+  if (!operands || !clocks || !sink) return MI355_W8A8_ERR_NULL;
+  if (shape > 1u || iters == 0 || iters > (1u << 24)) return MI355_W8A8_ERR_SHAPE;
+  if (reinterpret_cast<uintptr_t>(operands) & 15u) return MI355_W8A8_ERR_ALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const unsigned char* src = static_cast<const unsigned char*>(operands);
+  if (shape == 1u) hipLaunchKernelGGL(cal_mfma_kernel<1>, dim3(kCalGrid), dim3(256), 0, s, src, iters, clocks, sink);
+  else hipLaunchKernelGGL(cal_mfma_kernel<0>, dim3(kCalGrid), dim3(256), 0, s, src, iters, clocks, sink);
+  return launch_status();
+}
+
+int mi355_w8a8_calibrate_read_v1(const void* src, uint64_t bytes, uint32_t* sink, void* stream) {
+  if (!src || !sink) return MI355_W8A8_ERR_NULL;
+  if (bytes == 0 || (bytes & 32767u)) return MI355_W8A8_ERR_SHAPE;
+  if (reinterpret_cast<uintptr_t>(src) & 15u) return MI355_W8A8_ERR_ALIGN;
+  hipLaunchKernelGGL(cal_read_kernel, dim3(2048), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const v4i*>(src), bytes / 16u, sink);
+  return launch_status();
+}
+
+int mi355_w8a8_calibrate_copy_v1(const void* src, void* dst, uint64_t bytes, void* stream) {
+  if (!src || !dst) return MI355_W8A8_ERR_NULL;
+  if (bytes == 0 || (bytes & 15u)) return MI355_W8A8_ERR_SHAPE;
+  if (!aligned16(src) || !aligned16(dst)) return MI355_W8A8_ERR_ALIGN;
+  if (overlaps(src, bytes, dst, bytes)) return MI355_W8A8_ERR_ALIAS;
+  hipLaunchKernelGGL(cal_copy_kernel, dim3(4096), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const v4i*>(src), static_cast<v4i*>(dst), bytes / 16u);
+  return launch_status();
 }
 
 }  // extern "C"
