@@ -143,11 +143,12 @@ typedef struct mi355_w8a8_grouped_problem {
   /* Optional gather on the way in (NULL: row i of the call is row i of x).  With a map, row i is
    * read from x[x_row_map[i] / x_row_repeat] and x holds one row per token: passing the
    * sort_indices of mi355_w8a8_moe_dispatch_v1 and repeat = top_k lets the first expert projection
-   * read the unsorted hidden states, and the dispatch can skip the row copies.  Map values must lie
-   * in [0, rows of x * x_row_repeat); they are not checked. */
+   * read the unsorted hidden states, and the dispatch can skip the row copies.  A map value outside
+   * [0, x_rows * x_row_repeat) reads the nearest row of x (the last one, or row 0 for a negative value)
+   * instead of memory beyond x. */
   const int32_t* x_row_map; /* int32 [m] or NULL */
   uint32_t x_row_repeat;    /* >= 1 with a map */
-  uint32_t reserved;
+  uint32_t x_rows;          /* rows of x with a map; 0 = ceil(m / x_row_repeat), one row per token */
 } mi355_w8a8_grouped_problem;
 
 /*

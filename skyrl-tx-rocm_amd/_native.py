@@ -75,7 +75,7 @@ class GroupedProblem(ctypes.Structure):
         ("x", _vp), ("w_packed", _vp), ("w_scales", _vp), ("lora_a", _vp), ("lora_b", _vp),
         ("lora_scaling", _vp), ("group_sizes", _vp), ("out", _vp), ("workspace", _vp),
         ("workspace_bytes", _u64), ("aux_x_codes", _vp), ("aux_x_scales", _vp), ("aux_acc", _vp),
-        ("x_row_map", _vp), ("x_row_repeat", _u32), ("reserved", _u32),
+        ("x_row_map", _vp), ("x_row_repeat", _u32), ("x_rows", _u32),
     ]
 
 

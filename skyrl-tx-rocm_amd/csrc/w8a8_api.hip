@@ -489,9 +489,10 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
   const uint32_t x_repeat = p->x_row_map ? p->x_row_repeat : 1u;
   if (p->x_row_map && (x_repeat == 0 || (reinterpret_cast<uintptr_t>(p->x_row_map) & 3u)))
     return x_repeat == 0 ? MI355_W8A8_ERR_SHAPE : MI355_W8A8_ERR_ALIGN;
-  // with a row map x holds one row per token: at least ceil(m / repeat) of them
-  const uint64_t x_rows = ((uint64_t)p->m + x_repeat - 1u) / x_repeat;
-  if (overlaps(p->out, out_bytes, p->x, x_rows * p->k * 2u) ||
+  // with a row map x holds one row per token unless the caller says otherwise; gathered reads are
+  // clamped to these rows
+  const uint32_t x_rows = (p->x_row_map && p->x_rows) ? p->x_rows : (p->m + x_repeat - 1u) / x_repeat;
+  if (overlaps(p->out, out_bytes, p->x, (uint64_t)x_rows * p->k * 2u) ||
       overlaps(p->out, out_bytes, p->x_row_map, (uint64_t)p->m * 4u) ||
       overlaps(p->out, out_bytes, p->workspace, p->workspace_bytes))
     return MI355_W8A8_ERR_ALIAS;
@@ -548,7 +549,7 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
   q.scales_rm = p->aux_x_scales;
   q.zero_out = static_cast<uint16_t*>(p->out);
   q.zero_cols = n_out;
-  q.row_map = p->x_row_map; q.row_div = x_repeat;
+  q.row_map = p->x_row_map; q.row_div = x_repeat; q.row_limit = x_rows;
   if ((st = launch_quant<false>(q, s))) return st;
   }
 
@@ -560,7 +561,7 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
     la.src_row = src_row;
     la.slot_group = nullptr;
     la.blk_range = blk_range;
-    la.row_map = p->x_row_map; la.row_div = x_repeat;
+    la.row_map = p->x_row_map; la.row_div = x_repeat; la.row_limit = x_rows;
     la.zp = ws + w.zp;
     la.M = p->m; la.K = p->k; la.r = p->rank; la.nkk = w.nkk;
     la.steps_per_wave = w.steps_per_wave; la.n_steps = w.n_steps;

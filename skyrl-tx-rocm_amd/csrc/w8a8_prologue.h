@@ -229,10 +229,17 @@ struct QuantArgs {
   uint32_t zero_cols;
   uint32_t* tile_ctr;      // 256 words cleared for the GEMM launches' tile counters, or null
   // Optional gather on the way in: row m is read from x[row_map[m] / row_div] (the sorted (token,
-  // choice) pairs of an expert layer read their token's row; x then has the tokens' row count)
+  // choice) pairs of an expert layer read their token's row; x then has the tokens' row count,
+  // row_limit, to which the source row is clamped)
   const int32_t* row_map;
-  uint32_t row_div;
+  uint32_t row_div, row_limit;
 };
+
+// source row of a gathered read: map value / divisor, clamped into [0, limit)
+__device__ inline uint32_t mapped_row(int32_t value, uint32_t div, uint32_t limit) {
+  const uint32_t r = value < 0 ? 0u : (uint32_t)value / div;
+  return r < limit ? r : limit - 1u;
+}
 
 template <int NCH, bool RMS>
 __global__ __launch_bounds__(256) void quant_rows_kernel(QuantArgs a) {
@@ -240,7 +247,7 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(QuantArgs a) {
   const uint32_t m = blockIdx.x * 4u + (threadIdx.x >> 6);
   if (a.tile_ctr && blockIdx.x == 0) a.tile_ctr[threadIdx.x] = 0u;
   if (m >= a.M) return;
-  const uint32_t xrow = a.row_map ? (uint32_t)a.row_map[m] / a.row_div : m;
+  const uint32_t xrow = a.row_map ? mapped_row(a.row_map[m], a.row_div, a.row_limit) : m;
   const uint16_t* xr = a.x + (size_t)xrow * a.K;
   float v[NCH][8];
 #pragma unroll
@@ -449,9 +456,9 @@ struct LoraAArgs {
   // sums its own range of k steps and writes zf + ksplit_index * zf_slice (floats); the caller adds
   // the slices.  0 or 1: one workgroup per row block.
   uint32_t n_ksplit, zf_slice;
-  // Optional gather on the way in (see QuantArgs): source row = row_map[row] / row_div
+  // Optional gather on the way in (see QuantArgs): source row = row_map[row] / row_div, clamped to row_limit
   const int32_t* row_map;
-  uint32_t row_div;
+  uint32_t row_div, row_limit;
 };
 
 template <int RB>  // number of 32-wide rank blocks (1 or 2)
@@ -469,7 +476,7 @@ __global__ __launch_bounds__(1024) void lora_a_kernel(LoraAArgs a) {
   const uint32_t p = pb * 32u + i;
   int src = a.src_row ? a.src_row[p] : (int)p;
   if (src >= (int)a.M) src = -1;
-  if (a.row_map && src >= 0) src = (int)((uint32_t)a.row_map[src] / a.row_div);
+  if (a.row_map && src >= 0) src = (int)mapped_row(a.row_map[src], a.row_div, a.row_limit);
   const uint32_t rowgrp = (a.slot_group && ghi > glo) ? (uint32_t)a.slot_group[p] : glo;
   const uint16_t* xr = a.xsrc + (size_t)(src < 0 ? 0 : src) * a.K;
   v16f acc[RB];

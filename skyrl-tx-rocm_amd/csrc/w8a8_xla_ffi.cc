@@ -274,6 +274,170 @@ ffi::Error MoeCombine(hipStream_t stream, ffi::Buffer<ffi::BF16> expert_out, ffi
                  "mi355_w8a8 moe combine launch submission failed");
 }
 
+// Grouped (ragged) call over rows already sorted by group: x bf16 [M or tokens, K], packed weights u8
+// [n_weights * bytes], scales f32 [n_weights, N], A bf16 [G, K, r], B bf16 [G, r, N], scaling f32 [G]
+// (size-0 buffers without LoRA), group_sizes s32 [G], x_row_map s32 [M] (size 0: row i of the call is
+// row i of x).  Results: y bf16 [M, n_out], workspace u8 [mi355_w8a8_grouped_workspace_bytes].
+ffi::Error Grouped(hipStream_t stream, ffi::Buffer<ffi::BF16> x, ffi::Buffer<ffi::U8> w_packed,
+                   ffi::Buffer<ffi::F32> w_scales, ffi::Buffer<ffi::BF16> lora_a, ffi::Buffer<ffi::BF16> lora_b,
+                   ffi::Buffer<ffi::F32> lora_scaling, ffi::Buffer<ffi::S32> group_sizes,
+                   ffi::Buffer<ffi::S32> x_row_map, ffi::ResultBuffer<ffi::BF16> y,
+                   ffi::ResultBuffer<ffi::U8> workspace, int32_t swiglu, int32_t x_row_repeat) {
+  mi355_w8a8_grouped_problem p{};
+  p.struct_size = sizeof(p);
+  uint32_t x_rows = 0;
+  if (!RowsAndK(x.dimensions(), &x_rows, &p.k))
+    return ffi::Error::InvalidArgument("x must be bf16 [..., K] with a non-empty row domain");
+  auto ds = w_scales.dimensions();
+  if (ds.size() != 2 || ds[0] <= 0 || ds[1] <= 0) return ffi::Error::InvalidArgument("w_scales must be f32 [n_weights, N]");
+  const uint32_t n_weights = static_cast<uint32_t>(ds[0]);
+  p.n = static_cast<uint32_t>(ds[1]);
+  p.n_groups = static_cast<uint32_t>(group_sizes.element_count());
+  if (p.n_groups == 0 || p.n_groups % n_weights != 0)
+    return ffi::Error::InvalidArgument("group_sizes must be s32 [G] with G a multiple of the number of weights");
+  p.groups_per_weight = p.n_groups / n_weights;
+  if (w_packed.size_bytes() != static_cast<size_t>(n_weights) * mi355_w8a8_packed_weight_bytes(p.k, p.n))
+    return ffi::Error::InvalidArgument("packed weights do not match (n_weights, K, N)");
+  if (x_row_map.element_count() > 0) {
+    if (x_row_repeat < 1) return ffi::Error::InvalidArgument("x_row_repeat must be >= 1 with a row map");
+    p.m = static_cast<uint32_t>(x_row_map.element_count());
+    if (static_cast<uint64_t>(x_rows) * static_cast<uint32_t>(x_row_repeat) < p.m)
+      return ffi::Error::InvalidArgument("x_row_map must not name more rows than x holds times x_row_repeat");
+    p.x_row_map = x_row_map.typed_data();
+    p.x_row_repeat = static_cast<uint32_t>(x_row_repeat);
+    p.x_rows = x_rows;
+  } else {
+    p.m = x_rows;
+  }
+  if (lora_a.element_count() > 0) {
+    auto da = lora_a.dimensions();
+    auto db = lora_b.dimensions();
+    if (da.size() != 3 || db.size() != 3 || da[0] != p.n_groups || da[1] != p.k || db[0] != da[0] ||
+        db[1] != da[2] || db[2] != p.n || lora_scaling.element_count() != p.n_groups)
+      return ffi::Error::InvalidArgument("LoRA A/B/scaling must be [G,K,r], [G,r,N], [G]");
+    p.rank = static_cast<uint32_t>(da[2]);
+    p.lora_a = lora_a.untyped_data();
+    p.lora_b = lora_b.untyped_data();
+    p.lora_scaling = lora_scaling.typed_data();
+  }
+  const uint32_t n_out = swiglu ? p.n / 2 : p.n;
+  if (y->element_count() != static_cast<size_t>(p.m) * n_out)
+    return ffi::Error::InvalidArgument("result must be bf16 [M, n_out]");
+  p.flags = swiglu ? MI355_W8A8_FLAG_SWIGLU : 0u;
+  p.x = x.untyped_data();
+  p.w_packed = w_packed.untyped_data();
+  p.w_scales = w_scales.typed_data();
+  p.group_sizes = group_sizes.typed_data();
+  p.out = y->untyped_data();
+  p.workspace = workspace->untyped_data();
+  p.workspace_bytes = workspace->size_bytes();
+  return ToError(mi355_w8a8_grouped_v1(&p, stream), "mi355_w8a8 grouped launch submission failed");
+}
+
+// Attention input stage behind the fused QKV projection: fused bf16 [M, H 2 D + 2 Hkv D], the two
+// head-norm weights f32 [D] (delta form), positions s32 [M].  Results: q bf16 [M, H, D], k and v bf16
+// [M, Hkv, D], gate bf16 [M, H D].
+ffi::Error QkvSplitNormRope(hipStream_t stream, ffi::Buffer<ffi::BF16> fused, ffi::Buffer<ffi::F32> q_norm_weight,
+                            ffi::Buffer<ffi::F32> k_norm_weight, ffi::Buffer<ffi::S32> positions,
+                            ffi::ResultBuffer<ffi::BF16> q, ffi::ResultBuffer<ffi::BF16> k,
+                            ffi::ResultBuffer<ffi::BF16> v, ffi::ResultBuffer<ffi::BF16> gate, int32_t rotary_dim,
+                            float rope_theta, float rms_eps) {
+  mi355_w8a8_qkv_post_problem p{};
+  p.struct_size = sizeof(p);
+  auto dq = q->dimensions();
+  auto dk = k->dimensions();
+  if (dq.size() != 3 || dk.size() != 3 || dq[0] <= 0 || dk[0] != dq[0] || dk[2] != dq[2] || dq[1] <= 0 || dk[1] <= 0)
+    return ffi::Error::InvalidArgument("q must be bf16 [M, H, D] and k bf16 [M, Hkv, D]");
+  p.m = static_cast<uint32_t>(dq[0]);
+  p.num_query_heads = static_cast<uint32_t>(dq[1]);
+  p.num_kv_heads = static_cast<uint32_t>(dk[1]);
+  p.head_dim = static_cast<uint32_t>(dq[2]);
+  const size_t width = static_cast<size_t>(p.num_query_heads) * 2 * p.head_dim + 2 * static_cast<size_t>(p.num_kv_heads) * p.head_dim;
+  if (fused.element_count() != static_cast<size_t>(p.m) * width || v->element_count() != k->element_count() ||
+      gate->element_count() != q->element_count() || positions.element_count() != p.m ||
+      q_norm_weight.element_count() != p.head_dim || k_norm_weight.element_count() != p.head_dim)
+    return ffi::Error::InvalidArgument("fused, v, gate, positions or the norm weights do not match (M, H, Hkv, D)");
+  if (rotary_dim < 0) return ffi::Error::InvalidArgument("rotary_dim must be >= 0");
+  p.rotary_dim = static_cast<uint32_t>(rotary_dim);
+  p.rope_theta = rope_theta;
+  p.rms_eps = rms_eps;
+  p.fused = fused.untyped_data();
+  p.q_norm_weight = q_norm_weight.typed_data();
+  p.k_norm_weight = k_norm_weight.typed_data();
+  p.positions = positions.typed_data();
+  p.q = q->untyped_data();
+  p.k = k->untyped_data();
+  p.v = v->untyped_data();
+  p.gate = gate->untyped_data();
+  return ToError(mi355_w8a8_qkv_split_norm_rope_v1(&p, stream), "mi355_w8a8 qkv stage launch submission failed");
+}
+
+// Group-scaled weight codes into the kernel's operand order: codes s8 [K_pad, N] (4-bit codes one per
+// byte) -> packed u8 [mi355_w8a8_gq_packed_weight_bytes].
+ffi::Error GqPackWeight(hipStream_t stream, ffi::Buffer<ffi::S8> codes, ffi::ResultBuffer<ffi::U8> packed,
+                        int32_t weight_bits) {
+  auto d = codes.dimensions();
+  if (d.size() != 2 || d[0] <= 0 || d[1] <= 0) return ffi::Error::InvalidArgument("codes must be s8 [K_pad, N]");
+  const uint32_t k_pad = static_cast<uint32_t>(d[0]), n = static_cast<uint32_t>(d[1]);
+  const uint64_t need = mi355_w8a8_gq_packed_weight_bytes(k_pad, n, static_cast<uint32_t>(weight_bits));
+  if (need == 0 || packed->size_bytes() != need)
+    return ffi::Error::InvalidArgument("packed buffer size does not match (K_pad, N, weight_bits)");
+  return ToError(mi355_w8a8_gq_pack_weight_v1(codes.typed_data(), packed->untyped_data(), k_pad, n,
+                                              static_cast<uint32_t>(weight_bits), stream),
+                 "mi355_w8a8 gq pack launch submission failed");
+}
+
+// Group-scaled linear (W4 / W8 codes, A4 / A8 activations, one scale per K group): x bf16 [.., K], packed
+// weight, scales f32 [K_pad / group_size, N], LoRA as in Forward.  Results: y bf16 [.., N], workspace u8
+// [mi355_w8a8_gq_workspace_bytes].
+ffi::Error GqLinear(hipStream_t stream, ffi::Buffer<ffi::BF16> x, ffi::Buffer<ffi::U8> w_packed,
+                    ffi::Buffer<ffi::F32> w_scales, ffi::Buffer<ffi::BF16> lora_a, ffi::Buffer<ffi::BF16> lora_b,
+                    ffi::Buffer<ffi::F32> lora_scaling, ffi::Buffer<ffi::S32> adapter_indices,
+                    ffi::ResultBuffer<ffi::BF16> y, ffi::ResultBuffer<ffi::U8> workspace, int32_t group_size,
+                    int32_t weight_bits, int32_t activation_bits) {
+  mi355_w8a8_gq_problem p{};
+  p.struct_size = sizeof(p);
+  if (!RowsAndK(x.dimensions(), &p.m, &p.k))
+    return ffi::Error::InvalidArgument("x must be bf16 [..., K] with a non-empty row domain");
+  auto ds = w_scales.dimensions();
+  if (ds.size() != 2 || ds[0] <= 0 || ds[1] <= 0 || group_size <= 0)
+    return ffi::Error::InvalidArgument("w_scales must be f32 [K_pad / group_size, N] and group_size positive");
+  p.group_size = static_cast<uint32_t>(group_size);
+  p.k_pad = static_cast<uint32_t>(ds[0]) * p.group_size;
+  p.n = static_cast<uint32_t>(ds[1]);
+  p.weight_bits = static_cast<uint32_t>(weight_bits);
+  p.activation_bits = static_cast<uint32_t>(activation_bits);
+  if (p.k_pad < p.k) return ffi::Error::InvalidArgument("the scale groups must cover K");
+  const uint64_t need = mi355_w8a8_gq_packed_weight_bytes(p.k_pad, p.n, p.weight_bits);
+  if (need == 0 || w_packed.size_bytes() != need)
+    return ffi::Error::InvalidArgument("packed weight size does not match (K_pad, N, weight_bits)");
+  if (lora_a.element_count() > 0) {
+    auto da = lora_a.dimensions();
+    auto db = lora_b.dimensions();
+    if (da.size() != 3 || db.size() != 3 || da[1] != p.k || db[0] != da[0] || db[1] != da[2] || db[2] != p.n ||
+        lora_scaling.element_count() != static_cast<size_t>(da[0]))
+      return ffi::Error::InvalidArgument("LoRA A/B/scaling must be [n,K,r], [n,r,N], [n]");
+    p.n_adapters = static_cast<uint32_t>(da[0]);
+    p.rank = static_cast<uint32_t>(da[2]);
+    p.lora_a = lora_a.untyped_data();
+    p.lora_b = lora_b.untyped_data();
+    p.lora_scaling = lora_scaling.typed_data();
+    if (adapter_indices.element_count() > 0) {
+      if (adapter_indices.element_count() != p.m)
+        return ffi::Error::InvalidArgument("adapter_indices must hold one entry per row");
+      p.adapter_indices = adapter_indices.typed_data();
+    }
+  }
+  if (y->element_count() != static_cast<size_t>(p.m) * p.n) return ffi::Error::InvalidArgument("result must be bf16 [..., N]");
+  p.x = x.untyped_data();
+  p.w_packed = w_packed.untyped_data();
+  p.w_scales = w_scales.typed_data();
+  p.out = y->untyped_data();
+  p.workspace = workspace->untyped_data();
+  p.workspace_bytes = workspace->size_bytes();
+  return ToError(mi355_w8a8_gq_linear_v1(&p, stream), "mi355_w8a8 gq linear launch submission failed");
+}
+
 }  // namespace
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_forward_v1, Forward,
@@ -368,4 +532,57 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_moe_combine_v1, MoeCombine,
                                   .Arg<ffi::Buffer<ffi::S32>>()
                                   .Arg<ffi::Buffer<ffi::F32>>()
                                   .Ret<ffi::Buffer<ffi::BF16>>());
+XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_grouped_v1, Grouped,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::U8>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::U8>>()
+                                  .Attr<int32_t>("swiglu")
+                                  .Attr<int32_t>("x_row_repeat"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_qkv_split_norm_rope_v1, QkvSplitNormRope,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Attr<int32_t>("rotary_dim")
+                                  .Attr<float>("rope_theta")
+                                  .Attr<float>("rms_eps"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_gq_pack_weight_v1, GqPackWeight,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::Buffer<ffi::S8>>()
+                                  .Ret<ffi::Buffer<ffi::U8>>()
+                                  .Attr<int32_t>("weight_bits"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_gq_linear_v1, GqLinear,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::U8>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::U8>>()
+                                  .Attr<int32_t>("group_size")
+                                  .Attr<int32_t>("weight_bits")
+                                  .Attr<int32_t>("activation_bits"));
 #endif  // __has_include("xla/ffi/api/ffi.h")

@@ -25,7 +25,9 @@ from ... import _native
 FFI_LIB_PATH = Path(_native.LIB_PATH).with_name("libmi355_w8a8_ffi.so")
 TARGETS = ("mi355_w8a8_ffi_forward_v1", "mi355_w8a8_ffi_quantize_rows_v1", "mi355_w8a8_ffi_pack_weight_v1",
            "mi355_w8a8_ffi_backward_v1", "mi355_w8a8_ffi_swiglu_bwd_v1", "mi355_w8a8_ffi_rms_norm_bwd_v1",
-           "mi355_w8a8_ffi_moe_route_v1", "mi355_w8a8_ffi_moe_dispatch_v1", "mi355_w8a8_ffi_moe_combine_v1")
+           "mi355_w8a8_ffi_moe_route_v1", "mi355_w8a8_ffi_moe_dispatch_v1", "mi355_w8a8_ffi_moe_combine_v1",
+           "mi355_w8a8_ffi_grouped_v1", "mi355_w8a8_ffi_qkv_split_norm_rope_v1", "mi355_w8a8_ffi_gq_pack_weight_v1",
+           "mi355_w8a8_ffi_gq_linear_v1")
 _ROCM_PLATFORM = "ROCM"
 _REGISTRATION_API_VERSION = 1
 _CUSTOM_CALL_API_VERSION = 4
@@ -171,3 +173,176 @@ def backward(x, dy, packed_weight, w_scales, lora_a=None, lora_b=None, lora_scal
     if lora_a.ndim == 2:
         return dx, da[0], db[0], ds[0]
     return dx, da, db, ds
+
+
+def grouped(x, packed_weights, w_scales, group_sizes, lora_a=None, lora_b=None, lora_scaling=None, *,
+            swiglu: bool = False, x_row_map=None, x_row_repeat: int = 1):
+    """Ragged per-group W8A8 (+LoRA, +SwiGLU) linear over rows sorted by group as one XLA custom call: the
+    expert projection of ``LoRAExpert.__call__`` (skyrl/tx/layers/lora.py:394-444).  ``packed_weights`` holds
+    the groups' packed weights back to back, ``w_scales`` is f32 [n_weights, N].  With ``x_row_map`` (the
+    dispatch's sort indices) row i of the call is read from ``x[x_row_map[i] // x_row_repeat]``."""
+    jax = _import_jax()
+    register(jax)
+    jnp = jax.numpy
+    k = x.shape[-1]
+    n = w_scales.shape[-1]
+    n_groups = group_sizes.shape[0]
+    empty = lambda dt, nd: jnp.zeros((0,) * nd, dt)
+    a3 = empty(jnp.bfloat16, 3) if lora_a is None else lora_a
+    b3 = empty(jnp.bfloat16, 3) if lora_b is None else lora_b
+    rank = a3.shape[2] if lora_a is not None else 0
+    s1 = (empty(jnp.float32, 1) if lora_a is None
+          else jnp.broadcast_to(jnp.asarray(lora_scaling, jnp.float32), (n_groups,)))
+    row_map = empty(jnp.int32, 1) if x_row_map is None else x_row_map.astype(jnp.int32).reshape(-1)
+    m = row_map.shape[0] if x_row_map is not None else x.reshape(-1, k).shape[0]
+    if x_row_map is not None and (x_row_repeat < 1 or x.reshape(-1, k).shape[0] * x_row_repeat < m):
+        raise ValueError("x_row_map names more rows than x holds times x_row_repeat")
+    n_out = n // 2 if swiglu else n
+    ws = int(_native.load().mi355_w8a8_grouped_workspace_bytes(m, k, n, n_groups, rank, 1 if swiglu else 0))
+    if ws == 0:
+        raise ValueError(f"geometry M={m}, K={k}, N={n}, groups={n_groups} is outside the native path")
+    y, _ = _call(jax, TARGETS[9],
+                 (jax.ShapeDtypeStruct((m, n_out), jnp.bfloat16), jax.ShapeDtypeStruct((ws,), jnp.uint8)),
+                 x.reshape(-1, k), packed_weights, w_scales.reshape(-1, n).astype(jnp.float32), a3, b3, s1,
+                 group_sizes.astype(jnp.int32), row_map, swiglu=int(swiglu), x_row_repeat=int(x_row_repeat))
+    return y
+
+
+def qkv_split_norm_rope(fused, q_norm_weight, k_norm_weight, positions, *, num_query_heads: int, num_kv_heads: int,
+                        head_dim: int, rotary_dim: int, rope_theta: float, eps: float = 1e-6):
+    """Split / head RMSNorm / partial RoPE behind the fused QKV projection as one XLA custom call
+    (skyrl/tx/kernels/qwen3_5_qkv_lora.py:266-286): returns ``(q, k, v, gate)``."""
+    jax = _import_jax()
+    register(jax)
+    jnp = jax.numpy
+    width = num_query_heads * 2 * head_dim + 2 * num_kv_heads * head_dim
+    if fused.shape[-1] != width:
+        raise ValueError(f"fused projection must be [..., {width}]")
+    lead = fused.shape[:-1]
+    m = 1
+    for d in lead:
+        m *= d
+    q, k, v, gate = _call(
+        jax, TARGETS[10],
+        (jax.ShapeDtypeStruct((m, num_query_heads, head_dim), jnp.bfloat16),
+         jax.ShapeDtypeStruct((m, num_kv_heads, head_dim), jnp.bfloat16),
+         jax.ShapeDtypeStruct((m, num_kv_heads, head_dim), jnp.bfloat16),
+         jax.ShapeDtypeStruct((m, num_query_heads * head_dim), jnp.bfloat16)),
+        fused.reshape(m, width), q_norm_weight.astype(jnp.float32), k_norm_weight.astype(jnp.float32),
+        positions.astype(jnp.int32).reshape(m), rotary_dim=int(rotary_dim), rope_theta=float(rope_theta),
+        rms_eps=float(eps))
+    return (q.reshape(*lead, num_query_heads, head_dim), k.reshape(*lead, num_kv_heads, head_dim),
+            v.reshape(*lead, num_kv_heads, head_dim), gate.reshape(*lead, num_query_heads * head_dim))
+
+
+def gq_pack_weight(codes, weight_bits: int):
+    """int8 [K_pad, N] group-scaled codes (4-bit codes one per byte) -> opaque uint8 packed weight."""
+    jax = _import_jax()
+    register(jax)
+    jnp = jax.numpy
+    k_pad, n = codes.shape
+    nbytes = int(_native.load().mi355_w8a8_gq_packed_weight_bytes(k_pad, n, weight_bits))
+    if nbytes == 0:
+        raise ValueError(f"geometry K_pad={k_pad}, N={n}, W{weight_bits} is outside the native path")
+    (packed,) = _call(jax, TARGETS[11], (jax.ShapeDtypeStruct((nbytes,), jnp.uint8),), codes,
+                      weight_bits=int(weight_bits))
+    return packed
+
+
+def gq_linear(x, packed_weight, w_scales, *, group_size: int, weight_bits: int, activation_bits: int,
+              lora_a=None, lora_b=None, lora_scaling=None, adapter_indices=None):
+    """Group-scaled W4/W8 x A4/A8 (+LoRA) linear as one XLA custom call: the general form of
+    ``_quantized_frozen_linear_f32`` (skyrl/tx/kernels/quantized_lora.py:215-304)."""
+    jax = _import_jax()
+    register(jax)
+    jnp = jax.numpy
+    k = x.shape[-1]
+    n_grp, n = w_scales.shape
+    m = 1
+    for d in x.shape[:-1]:
+        m *= d
+    empty = lambda dt, nd: jnp.zeros((0,) * nd, dt)
+    a3 = empty(jnp.bfloat16, 3) if lora_a is None else (lora_a if lora_a.ndim == 3 else lora_a[None])
+    b3 = empty(jnp.bfloat16, 3) if lora_b is None else (lora_b if lora_b.ndim == 3 else lora_b[None])
+    n_ad = a3.shape[0]
+    s1 = empty(jnp.float32, 1) if lora_a is None else jnp.broadcast_to(jnp.asarray(lora_scaling, jnp.float32), (n_ad,))
+    idx = empty(jnp.int32, 1) if adapter_indices is None else adapter_indices.astype(jnp.int32).reshape(-1)
+    ws = int(_native.load().mi355_w8a8_gq_workspace_bytes(m, n_grp * group_size, group_size, n_ad,
+                                                          a3.shape[2] if n_ad else 0))
+    if ws == 0:
+        raise ValueError(f"geometry M={m}, K_pad={n_grp * group_size}, group {group_size} is outside the native path")
+    y, _ = _call(jax, TARGETS[12],
+                 (jax.ShapeDtypeStruct((*x.shape[:-1], n), jnp.bfloat16), jax.ShapeDtypeStruct((ws,), jnp.uint8)),
+                 x, packed_weight, w_scales.astype(jnp.float32), a3, b3, s1, idx, group_size=int(group_size),
+                 weight_bits=int(weight_bits), activation_bits=int(activation_bits))
+    return y
+
+
+def swiglu_bwd(fused, d_product):
+    """Cotangent of the fused gate/up projection from the cotangent of ``silu(gate) * up``
+    (skyrl/tx/kernels/rocm/bf16_rms_gate_up_lora_swiglu_contiguous.py:541-574)."""
+    jax = _import_jax()
+    register(jax)
+    jnp = jax.numpy
+    (d_fused,) = _call(jax, TARGETS[4], (jax.ShapeDtypeStruct(fused.shape, jnp.bfloat16),), fused, d_product)
+    return d_fused
+
+
+def rms_norm_bwd(x, gamma, d_normalized, *, eps: float = 1e-6):
+    """Cotangent of the rows going into the RMSNorm prologue."""
+    jax = _import_jax()
+    register(jax)
+    jnp = jax.numpy
+    (d_x,) = _call(jax, TARGETS[5], (jax.ShapeDtypeStruct(x.shape, jnp.bfloat16),), x, gamma.astype(jnp.float32),
+                   d_normalized, eps=float(eps))
+    return d_x
+
+
+def moe_route(router_logits, top_k: int, norm_topk_prob: bool):
+    """softmax / top-k (/ renormalisation) of the router logits (skyrl/tx/models/qwen3.py:172-185):
+    ``(weights f32 [T, top_k], selected s32 [T, top_k])``."""
+    jax = _import_jax()
+    register(jax)
+    jnp = jax.numpy
+    t = router_logits.shape[0]
+    return _call(jax, TARGETS[6], (jax.ShapeDtypeStruct((t, top_k), jnp.float32),
+                                   jax.ShapeDtypeStruct((t, top_k), jnp.int32)),
+                 router_logits.astype(jnp.float32), norm_topk_prob=int(bool(norm_topk_prob)))
+
+
+def moe_dispatch(tokens, indices, num_groups: int, *, repeat: int = 1, adapter_indices=None):
+    """Stable sort of the (token, choice) pairs by group (``prepare_routing``, skyrl/tx/layers/util.py:66-87,
+    for ``repeat == 1``): ``(sorted_tokens or None, group_sizes, sort_indices, unsort_indices, sorted_adapters
+    or None)``.  ``tokens=None`` sorts the indices only."""
+    jax = _import_jax()
+    register(jax)
+    jnp = jax.numpy
+    flat = indices.astype(jnp.int32).reshape(-1)
+    pairs = flat.shape[0]
+    empty = lambda dt, nd: jnp.zeros((0,) * nd, dt)
+    tok = empty(jnp.bfloat16, 2) if tokens is None else tokens
+    ad = empty(jnp.int32, 1) if adapter_indices is None else adapter_indices.astype(jnp.int32).reshape(-1)
+    width = 0 if tokens is None else tokens.shape[1]
+    ws = int(_native.load().mi355_w8a8_moe_dispatch_workspace_bytes(pairs, num_groups))
+    if ws == 0:
+        raise ValueError(f"{pairs} pairs over {num_groups} groups is outside the native path")
+    st, gs, si, ui, sa, _ = _call(
+        jax, TARGETS[7],
+        (jax.ShapeDtypeStruct((pairs, width) if tokens is not None else (0, 0), jnp.bfloat16),
+         jax.ShapeDtypeStruct((num_groups,), jnp.int32), jax.ShapeDtypeStruct((pairs,), jnp.int32),
+         jax.ShapeDtypeStruct((pairs,), jnp.int32),
+         jax.ShapeDtypeStruct((pairs,) if adapter_indices is not None else (0,), jnp.int32),
+         jax.ShapeDtypeStruct((ws,), jnp.uint8)),
+        tok, flat, ad, repeat=int(repeat))
+    return (st if tokens is not None else None), gs, si, ui, (sa if adapter_indices is not None else None)
+
+
+def moe_combine(expert_out, unsort_indices, weights):
+    """``out[t] = sum_j expert_out[unsort[t * top_k + j]] * weights[t, j]`` (skyrl/tx/models/qwen3.py:203-210)."""
+    jax = _import_jax()
+    register(jax)
+    jnp = jax.numpy
+    t = weights.shape[0]
+    (out,) = _call(jax, TARGETS[8], (jax.ShapeDtypeStruct((t, expert_out.shape[1]), jnp.bfloat16),), expert_out,
+                   unsort_indices.astype(jnp.int32), weights.astype(jnp.float32))
+    return out

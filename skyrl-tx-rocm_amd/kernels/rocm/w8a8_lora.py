@@ -861,6 +861,7 @@ class GroupedForwardPlan:
         p.aux_acc = self.aux["acc"].data_ptr() if return_aux else None
         p.x_row_map = rmap.data_ptr() if rmap is not None else None
         p.x_row_repeat = row_repeat if rmap is not None else 0
+        p.x_rows = flat.shape[0] if rmap is not None else 0
         self.problem = p
         self.flags = flags
         self._lib = lib

@@ -89,5 +89,84 @@ def test_shim_source_obeys_the_handler_rules():
                        "-ffast-math"):
             assert banned not in text, (src.name, banned)
     shim = (root / "w8a8_xla_ffi.cc").read_text()
-    assert shim.count("XLA_FFI_DEFINE_HANDLER_SYMBOL") == 9
+    assert shim.count("XLA_FFI_DEFINE_HANDLER_SYMBOL") == 13
     assert "PlatformStream<hipStream_t>" in shim
+
+
+def test_every_target_has_a_handler_symbol_and_a_c_entry_point():
+    """One typed-FFI target per variant (the reference's rule, rocm/QUANTIZED_FFI.md:579-599): every name in
+    TARGETS is defined in the shim, and the grouped / attention-stage / group-scaled targets exist."""
+    import re
+    from pathlib import Path
+
+    load_package()
+    from skyrl_tx_rocm_amd.kernels.rocm import w8a8_ffi
+
+    shim = (Path(__file__).resolve().parents[1] / "skyrl-tx-rocm_amd" / "csrc" / "w8a8_xla_ffi.cc").read_text()
+    defined = re.findall(r"XLA_FFI_DEFINE_HANDLER_SYMBOL\((\w+),", shim)
+    assert sorted(defined) == sorted(w8a8_ffi.TARGETS)
+    for name in ("mi355_w8a8_ffi_grouped_v1", "mi355_w8a8_ffi_qkv_split_norm_rope_v1", "mi355_w8a8_ffi_gq_linear_v1"):
+        assert name in w8a8_ffi.TARGETS
+    # each handler ends in a call of the C ABI entry point it is named for
+    for c_entry in ("mi355_w8a8_grouped_v1", "mi355_w8a8_qkv_split_norm_rope_v1", "mi355_w8a8_gq_linear_v1",
+                    "mi355_w8a8_gq_pack_weight_v1"):
+        assert f"{c_entry}(" in shim
+    assert "x_row_map" in shim and "x_row_repeat" in shim
+
+
+class _FakeSpec:
+    def __init__(self, shape, dtype):
+        self.shape, self.dtype = tuple(shape), dtype
+
+
+class _FakeArray:
+    def __init__(self, shape, dtype="bf16"):
+        self.shape, self.dtype, self.ndim = tuple(shape), dtype, len(shape)
+
+    def reshape(self, *shape):
+        shape = shape[0] if len(shape) == 1 and isinstance(shape[0], (tuple, list)) else shape
+        size = 1
+        for d in self.shape:
+            size *= d
+        known = 1
+        for d in shape:
+            if d != -1:
+                known *= d
+        return _FakeArray([size // known if d == -1 else d for d in shape], self.dtype)
+
+    def astype(self, dtype):
+        return _FakeArray(self.shape, dtype)
+
+
+def test_grouped_wrapper_builds_the_call_the_handler_expects(ffi_mod, monkeypatch):
+    """The Python wrapper of the grouped target passes operands, result shapes and attributes in the handler's
+    order (fake JAX: the call is recorded, not run)."""
+    calls = []
+
+    class _CallFfi(_FakeFfi):
+        def ffi_call(self, name, result_specs, **kw):
+            def run(*operands, **attrs):
+                calls.append((name, result_specs, operands, attrs))
+                return tuple(_FakeArray(s.shape, s.dtype) for s in result_specs)
+            return run
+
+    jnp = types.SimpleNamespace(bfloat16="bf16", float32="f32", int32="s32", uint8="u8", int8="s8",
+                                zeros=lambda shape, dt: _FakeArray(shape, dt),
+                                asarray=lambda v, dt: v, broadcast_to=lambda v, shape: _FakeArray(shape, "f32"))
+    jax = types.SimpleNamespace(ffi=_CallFfi(), numpy=jnp, ShapeDtypeStruct=_FakeSpec)
+    monkeypatch.setattr(ffi_mod, "_import_jax", lambda: jax)
+    monkeypatch.setattr(ffi_mod, "register", lambda j=None: ffi_mod.TARGETS)
+    lib = types.SimpleNamespace(mi355_w8a8_grouped_workspace_bytes=lambda *a: 4096)
+    monkeypatch.setattr(ffi_mod._native, "load", lambda: lib)
+    y = ffi_mod.grouped(_FakeArray((100, 64)), _FakeArray((4 * 64 * 256,), "u8"), _FakeArray((4, 256), "f32"),
+                        _FakeArray((4,), "s32"), _FakeArray((4, 64, 8)), _FakeArray((4, 8, 256)), 2.0,
+                        swiglu=True, x_row_map=_FakeArray((800,), "s32"), x_row_repeat=8)
+    assert y.shape == (800, 128)
+    name, specs, operands, attrs = calls[0]
+    assert name == "mi355_w8a8_ffi_grouped_v1"
+    assert [s.shape for s in specs] == [(800, 128), (4096,)]
+    assert [o.shape for o in operands] == [(100, 64), (4 * 64 * 256,), (4, 256), (4, 64, 8), (4, 8, 256), (4,), (4,), (800,)]
+    assert attrs == {"swiglu": 1, "x_row_repeat": 8}
+    with pytest.raises(ValueError, match="x_row_map"):
+        ffi_mod.grouped(_FakeArray((10, 64)), _FakeArray((1,), "u8"), _FakeArray((4, 256), "f32"),
+                        _FakeArray((4,), "s32"), x_row_map=_FakeArray((800,), "s32"), x_row_repeat=8)

@@ -223,3 +223,12 @@ def test_grouped_call_reads_rows_through_the_sort_order(dev, pkg, swiglu, rank):
         w8.grouped_forward(hidden, sizes, weight, a, b, s, row_map=sort_i, row_repeat=0)
     with pytest.raises(ValueError):
         w8.grouped_forward(hidden[:10], sizes, weight, a, b, s, row_map=sort_i, row_repeat=topk)
+    # map values outside the rows of x read the nearest row instead of memory beyond x
+    wild = sort_i.clone()
+    wild[5], wild[77], wild[200] = 2**30, -7, t * topk + 1
+    tame = wild.clone()
+    tame[5], tame[77], tame[200] = t * topk - 1, 0, t * topk - 1
+    got_wild = w8.grouped_forward(hidden, sizes, weight, a, b, s, swiglu=swiglu, row_map=wild, row_repeat=topk)
+    got_tame = w8.grouped_forward(hidden, sizes, weight, a, b, s, swiglu=swiglu, row_map=tame, row_repeat=topk)
+    torch.cuda.synchronize()
+    assert torch.equal(got_wild, got_tame)
