@@ -304,6 +304,19 @@ int mi355_w8a8_lora_residual_v1(const mi355_w8a8_problem* problem, void* stream)
 int mi355_w8a8_forward_v1(const mi355_w8a8_problem* problem, void* stream);
 /* Grouped / ragged per-expert variant. */
 int mi355_w8a8_grouped_v1(const mi355_w8a8_grouped_problem* problem, void* stream);
+/*
+ * mi355_w8a8_forward_v1 on a workspace the library owns.  No counterpart in the reference: it is for
+ * callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid it).  problem->workspace and problem->workspace_bytes are ignored; the call
+ * uses a static device array of MI355_W8A8_STATIC_WORKSPACE_BYTES that every GPU the library runs on
+ * holds until the process ends, and returns MI355_W8A8_ERR_WORKSPACE when
+ * mi355_w8a8_workspace_bytes(...) of the problem exceeds that size.  Inputs and outputs are the
+ * caller's as before.  All calls on one GPU share the array: calls that overlap in time on one GPU
+ * (two streams, two threads) race; calls on one stream are ordered and safe.  The first call on a
+ * device resolves the array's address (a host-side lookup, no allocation).
+ */
+#define MI355_W8A8_STATIC_WORKSPACE_BYTES (32u << 20)
+int mi355_w8a8_forward_static_ws_v1(const mi355_w8a8_problem* problem, void* stream);
 
 /*
  * Backward (VJP) of mi355_w8a8_lora_linear_v1: replaces the custom_vjp rule

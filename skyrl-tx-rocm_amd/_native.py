@@ -23,6 +23,7 @@ FLAG_TILE_256X128 = 64
 FLAG_TILE_256X256 = 128
 FLAG_GROUPED_TILE64 = 256
 FLAG_GROUPED_TILE128 = 512
+STATIC_WORKSPACE_BYTES = 32 << 20
 PATH_NAMES = {1: "skinny", 2: "skinny-chunks", 3: "tiled-256x128", 4: "tiled-256x256"}
 
 STATUS = {
@@ -35,7 +36,7 @@ EXPORTS = (
     "mi355_w8a8_pack_weight_v1", "mi355_w8a8_unpack_weight_v1", "mi355_w8a8_quantize_rows_v1",
     "mi355_w8a8_workspace_bytes", "mi355_w8a8_grouped_workspace_bytes",
     "mi355_w8a8_lora_linear_v1", "mi355_w8a8_rms_gateup_swiglu_v1", "mi355_w8a8_lora_residual_v1",
-    "mi355_w8a8_forward_v1", "mi355_w8a8_grouped_v1",
+    "mi355_w8a8_forward_v1", "mi355_w8a8_forward_static_ws_v1", "mi355_w8a8_grouped_v1",
     "mi355_w8a8_bwd_workspace_bytes", "mi355_w8a8_lora_linear_bwd_v1",
     "mi355_w8a8_grouped_bwd_workspace_bytes", "mi355_w8a8_grouped_bwd_v1",
     "mi355_w8a8_qkv_split_norm_rope_v1",
@@ -180,7 +181,7 @@ def _bind(lib: ctypes.CDLL) -> None:
         fn.restype = _u64
         fn.argtypes = (_u32, _u32, _u32, _u32, _u32, _u32)
     for name in ("mi355_w8a8_lora_linear_v1", "mi355_w8a8_rms_gateup_swiglu_v1",
-                 "mi355_w8a8_lora_residual_v1", "mi355_w8a8_forward_v1"):
+                 "mi355_w8a8_lora_residual_v1", "mi355_w8a8_forward_v1", "mi355_w8a8_forward_static_ws_v1"):
         fn = getattr(lib, name)
         fn.restype = ctypes.c_int
         fn.argtypes = (ctypes.POINTER(Problem), _vp)

@@ -4,6 +4,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
 #include "w8a8_device.h"
 #include "w8a8_gemm.h"
 #include "w8a8_gemm16.h"
@@ -18,7 +20,32 @@
 
 using namespace w8a8;
 
+// Workspace of mi355_w8a8_forward_static_ws_v1: one copy per GPU, held until the process ends.  In host
+// code this name is a stand-in, not a device address: the per-device address comes from
+// hipGetSymbolAddress (static_workspace() below) and only that pointer is handed to kernels.
+static __device__ __align__(256) unsigned char scratch[MI355_W8A8_STATIC_WORKSPACE_BYTES];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device (looked up once per device), or null.
+void* static_workspace() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  return g_scratch_ptr[dev];
+}
 
 constexpr uint32_t kMaxK = 16384;
 constexpr uint32_t kMaxRows = 1u << 20;
@@ -1738,6 +1765,24 @@ int mi355_w8a8_lora_residual_v1(const mi355_w8a8_problem* p, void* stream) {
 }
 int mi355_w8a8_forward_v1(const mi355_w8a8_problem* p, void* stream) {
   return run_forward(p, static_cast<hipStream_t>(stream), kReqNone);
+}
+
+int mi355_w8a8_forward_static_ws_v1(const mi355_w8a8_problem* p, void* stream) {
+  if (!p) return MI355_W8A8_ERR_NULL;
+  if (p->struct_size != sizeof(mi355_w8a8_problem)) return MI355_W8A8_ERR_STRUCT;
+  const int st = validate_common(p->m, p->k, p->n);
+  if (st) return st;
+  const uint64_t need = mi355_w8a8_workspace_bytes(p->m, p->k, p->n, p->n_adapters, p->rank, p->flags);
+  if (need == 0 || need > MI355_W8A8_STATIC_WORKSPACE_BYTES) return MI355_W8A8_ERR_WORKSPACE;
+  void* ws = static_workspace();
+  if (!ws) return MI355_W8A8_ERR_LAUNCH;
+  // Nothing in the workspace has to start at zero: every table a kernel reads is written by an earlier
+  // kernel of the same call (the tile counters are cleared by the quantizer launch), so the contents a
+  // previous call left behind are never read.
+  mi355_w8a8_problem q = *p;
+  q.workspace = ws;
+  q.workspace_bytes = MI355_W8A8_STATIC_WORKSPACE_BYTES;
+  return run_forward(&q, static_cast<hipStream_t>(stream), kReqNone);
 }
 
 uint64_t mi355_w8a8_grouped_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint32_t rank,
