@@ -395,8 +395,8 @@ void w8a8_gemm16_kernel(GemmArgs g) {
       if (!wave_live) return;
       if (EPI != kEpiAcc && full_n) swr = *reinterpret_cast<const v4i*>(T.swp + tcol0 + 4u * c16);
       if constexpr (kLora) {
-        load_z(0, 0);
-        load_z(1, 1);
+        load_z(0, 0);  // (the second fragment's operands are requested when the epilogue starts: during the
+                       // last stage their twelve registers are still needed for its operands)
         load_b((int)(range[0] & 0xffffu));
       }
     };
@@ -418,6 +418,7 @@ void w8a8_gemm16_kernel(GemmArgs g) {
     // Lane (c16, q) owns, in every 16-row fragment bi, the rows 4 q + v (v = 0..3) and the four
     // consecutive original columns tcol0 + 4 c16 + j held by the accumulator blocks j.
     if (!wave_live) continue;  // wave beyond the last column; it still takes part in the next tile
+    if constexpr (kLora) load_z(1, 1);
     const uint32_t ncol = tcol0 + 4u * c16;  // the lane's four consecutive columns
     float sw[4];
 #pragma unroll
