@@ -414,7 +414,9 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
     }
 #undef W8A8_QL
     if ((st = launch_status())) return st;
-  } else if (!skip_gemm) {  // measurement calls: the tile counters still have to start at zero
+  } else if (!skip_gemm && path != MI355_W8A8_PATH_TILED_256X256) {
+    // measurement calls: the tile counters of the 256 x 128 geometry's dynamic schedule still have to
+    // start at zero (the 256 x 256 kernel has a static schedule and no counters)
     hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(256), 0, s, q.tile_ctr, 256u);
     if ((st = launch_status())) return st;
   }
