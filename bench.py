@@ -130,7 +130,10 @@ def measured_traffic_bytes(workload, profiles_dir=None):
         hit = _COUNTER_LINE.match(line)
         if not hit:
             continue
-        if "cal_copy_kernel" in hit["name"]:
+        # the copy of known size: the library's cal_copy_kernel, or in older summaries the runtime's 256 MiB
+        # buffer copy (grid 131072, a single dispatch)
+        if "cal_copy_kernel" in hit["name"] or (hit["name"].startswith("__amd_rocclr_copyBuffer")
+                                               and int(hit["grid"]) == 131072 and int(hit["n"]) == 1):
             copy[hit["ctr"]] = float(hit["kib"])
         rows.append((hit["name"], hit["ctr"], float(hit["kib"])))
     if set(copy) != {"FETCH_SIZE", "WRITE_SIZE"} or min(copy.values()) <= 0:
