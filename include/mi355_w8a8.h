@@ -79,6 +79,11 @@ typedef enum mi355_w8a8_status {
  * groups average at least 96 rows, else 64.  Pass the same flags to the workspace query. */
 #define MI355_W8A8_FLAG_GROUPED_TILE64 256u
 #define MI355_W8A8_FLAG_GROUPED_TILE128 512u
+/* The workspace still holds the transposed LoRA A and the packed LoRA B that an earlier call of the tiled
+ * path wrote there for the same lora_a / lora_b contents and the same (k, n, n_adapters, rank): this call
+ * does not write them again (adapters that do not change between calls, as in serving).  The caller
+ * vouches for it; calls of at most 128 rows keep no such copies and ignore the flag. */
+#define MI355_W8A8_FLAG_LORA_PACK_VALID 1024u
 
 /*
  * One forward call.  y = dequant(quant(n) @ W) + s[idx] * ((n @ A[idx]) @ B[idx]) (+ residual),

@@ -23,6 +23,7 @@ FLAG_TILE_256X128 = 64
 FLAG_TILE_256X256 = 128
 FLAG_GROUPED_TILE64 = 256
 FLAG_GROUPED_TILE128 = 512
+FLAG_LORA_PACK_VALID = 1024
 STATIC_WORKSPACE_BYTES = 32 << 20
 PATH_NAMES = {1: "skinny", 2: "skinny-chunks", 3: "tiled-256x128", 4: "tiled-256x256"}
 

@@ -362,6 +362,8 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
 
   const bool skip_prologue = (p->flags & MI355_W8A8_FLAG_SKIP_PROLOGUE) != 0;
   const bool skip_gemm = (p->flags & MI355_W8A8_FLAG_SKIP_GEMM) != 0;
+  // up to 8192 rows the quantizer's workgroups sort the adapter indices themselves (one launch less)
+  const bool route_inline = routed && p->m <= kInlineRouteMaxRows;
   if ((routed || lora) && !skip_prologue) {
     LoraPrepArgs pa{};
     pa.idx = routed ? p->adapter_indices : nullptr;
@@ -372,13 +374,16 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
     pa.bp = ws + w.bp;
     pa.M = p->m; pa.K = p->k; pa.N = p->n; pa.n_groups = p->n_adapters; pa.r = p->rank; pa.nkk = w.nkk;
     pa.ncb = n_padded(p->n) / 32u; pa.slots = w.slots;
-    pa.route_blocks = routed ? 1u : 0u;
+    pa.route_blocks = (routed && !route_inline) ? 1u : 0u;
     const uint64_t a_items = (uint64_t)p->n_adapters * p->k * ((p->rank + 7u) / 8u);
     const uint64_t b_items = (uint64_t)p->n_adapters * pa.ncb * w.nkk * 64u;
-    pa.a_blocks = (uint32_t)((a_items + 1023u) / 1024u);
-    const uint32_t b_blocks = (uint32_t)((b_items + 1023u) / 1024u);
-    hipLaunchKernelGGL(lora_prep_kernel, dim3(pa.route_blocks + pa.a_blocks + b_blocks), dim3(1024), 0, s, pa);
-    if ((st = launch_status())) return st;
+    const bool pack = !(p->flags & MI355_W8A8_FLAG_LORA_PACK_VALID);  // else the workspace holds both already
+    pa.a_blocks = pack ? (uint32_t)((a_items + 1023u) / 1024u) : 0u;
+    const uint32_t b_blocks = pack ? (uint32_t)((b_items + 1023u) / 1024u) : 0u;
+    if (pa.route_blocks + pa.a_blocks + b_blocks) {
+      hipLaunchKernelGGL(lora_prep_kernel, dim3(pa.route_blocks + pa.a_blocks + b_blocks), dim3(1024), 0, s, pa);
+      if ((st = launch_status())) return st;
+    }
   }
 
   // quantizer and LoRA-A projection: one pass over x
@@ -401,6 +406,10 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   q.r = p->rank; q.nkk = w.nkk;
   q.nterms = (p->flags & MI355_W8A8_FLAG_LORA_SPLIT2) ? 2u : 3u;
   q.tile_ctr = reinterpret_cast<uint32_t*>(ws + w.tile_ctr);
+  if (route_inline) {
+    q.route_idx = p->adapter_indices; q.n_groups = p->n_adapters; q.slots = w.slots;
+    q.src_row = src_row; q.slot_group = slot_group; q.blk_range = blk_range;
+  }
   if (!skip_prologue) {
     const dim3 grid(q.n_half_blocks), block(1024);
 #define W8A8_QL(CB)                                                                   \

@@ -620,7 +620,108 @@ struct QuantLoraArgs {
   unsigned char* zp;        // packed z fragments
   uint32_t r, nkk, nterms;
   uint32_t* tile_ctr;       // 256 words cleared for the GEMM launches' tile counters, or null
+  // Routing inside this launch (route_idx != null; M <= kInlineRouteMaxRows): every workgroup sorts the
+  // adapter indices for itself and WRITES its slots' entries of src_row / slot_group / blk_range
+  // (then non-const outputs, read later by the GEMM) instead of reading them.
+  const int32_t* route_idx; // adapter per row
+  uint32_t n_groups, slots;
 };
+
+constexpr uint32_t kInlineRouteMaxRows = 8192;  // eight rows per thread of a 1024-thread workgroup
+
+// The routing tables of route_rows_block for the 16 slots [16 hb, 16 hb + 16), computed by the
+// workgroup itself: rows keep their order inside a group (slot start[g] + j holds the j-th row of group
+// g), which every workgroup derives alike from the adapter indices alone.  Returns through LDS:
+// out_src[16], out_grp[16], out_range (the group range of the 32-slot block that holds the slots).
+__device__ inline void route_rows_inline(const int32_t* __restrict__ idx, uint32_t M, uint32_t n_groups,
+                                         uint32_t slots, uint32_t hb, int* out_src, int* out_grp, uint32_t* out_range,
+                                         int* out_last_group) {
+  __shared__ int cnt[kMaxAdapters];
+  __shared__ int start[kMaxAdapters + 1];
+  __shared__ int wave_cnt[16];
+  __shared__ int last_nonempty;
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t per = (M + 1023u) / 1024u;  // consecutive rows per thread (<= 8)
+  if (tid < (uint32_t)kMaxAdapters) cnt[tid] = 0;
+  if (tid < 16u) { out_src[tid] = -1; out_grp[tid] = 0; }
+  __syncthreads();
+  int mine[8];
+#pragma unroll
+  for (uint32_t j = 0; j < 8; ++j) {
+    const uint32_t i = tid * per + j;
+    int a = -1;
+    if (j < per && i < M) {
+      a = idx[i];
+      a = a < 0 ? 0 : (a >= (int)n_groups ? (int)n_groups - 1 : a);
+      atomicAdd(&cnt[a], 1);  // integer counts: the order of the additions does not matter
+    }
+    mine[j] = a;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int pos = 0, last = 0;
+    for (uint32_t a = 0; a < n_groups; ++a) {
+      start[a] = pos;
+      pos += cnt[a];
+      if (cnt[a] > 0) last = (int)a;
+    }
+    start[n_groups] = pos;
+    last_nonempty = last;
+    *out_last_group = last;
+  }
+  __syncthreads();
+  // group of a slot: the group whose [start, start + count) holds it; padding slots follow the last
+  // non-empty group
+  auto group_of = [&](uint32_t p) -> int {
+    if (p >= M) return last_nonempty;
+    int g = 0;
+    for (uint32_t a = 0; a < n_groups; ++a)
+      if ((int)p >= start[a] && (int)p < start[a + 1]) g = (int)a;
+    return g;
+  };
+  const uint32_t p0 = hb * 16u;
+  if (tid < 16u) out_grp[tid] = group_of(p0 + tid);
+  if (tid == 16u) {
+    const uint32_t b0 = (p0 / 32u) * 32u;
+    const uint32_t b1 = (b0 + 31u < M) ? b0 + 31u : (M ? M - 1u : 0u);
+    *out_range = b0 >= M ? 0u : ((uint32_t)group_of(b0) | ((uint32_t)group_of(b1) << 16));
+  }
+  // the rows of the slots in use, group by group (a workgroup's 16 slots usually lie in one group)
+  const uint32_t p_end = (p0 + 16u < M) ? p0 + 16u : M;
+  if (p0 < M) {
+    const int g_first = group_of(p0), g_last = group_of(p_end - 1u);
+    for (int g = g_first; g <= g_last; ++g) {  // workgroup-uniform
+      if (cnt[g] == 0) continue;
+      int c = 0;
+#pragma unroll
+      for (uint32_t j = 0; j < 8; ++j) c += (mine[j] == g) ? 1 : 0;
+      // exclusive prefix of c over the threads in thread order: inside the wave, then across waves
+      int incl = c;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const int up = __shfl_up(incl, off, 64);
+        if ((int)lane >= off) incl += up;
+      }
+      __syncthreads();  // wave_cnt is free
+      if (lane == 63u) wave_cnt[wave] = incl;
+      __syncthreads();
+      int before = incl - c;
+      for (uint32_t w = 0; w < wave; ++w) before += wave_cnt[w];
+      // slots of group g among mine: ranks [lo, hi)
+      const int lo = ((int)p0 > start[g] ? (int)p0 : start[g]) - start[g];
+      const int hi = ((int)p_end < start[g + 1] ? (int)p_end : start[g + 1]) - start[g];
+      int rank = before;
+#pragma unroll
+      for (uint32_t j = 0; j < 8; ++j) {
+        if (mine[j] == g) {
+          if (rank >= lo && rank < hi) out_src[start[g] + rank - (int)p0] = (int)(tid * per + j);
+          ++rank;
+        }
+      }
+    }
+  }
+  __syncthreads();
+}
 
 template <int CB, bool RMS>  // CB: 16-wide rank blocks (0 = no LoRA, 1, 2, 4)
 __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
@@ -635,11 +736,30 @@ __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
   if (a.tile_ctr && hb == 0 && tid < 256u) a.tile_ctr[tid] = 0u;
   if (hb >= a.n_half_blocks) return;
   const uint32_t pb = hb >> 1, half16 = hb & 1u;
+  __shared__ int route_src[16], route_grp[16], route_last_group;
+  __shared__ uint32_t route_range;
+  const bool route_here = a.route_idx != nullptr;  // workgroup-uniform
+  if (route_here) {
+    route_rows_inline(a.route_idx, a.M, a.n_groups, a.slots, hb, route_src, route_grp, &route_range, &route_last_group);
+    // the tables the GEMM reads later
+    if (tid < 16u) {
+      const_cast<int32_t*>(a.src_row)[hb * 16u + tid] = route_src[tid];
+      const_cast<int32_t*>(a.slot_group)[hb * 16u + tid] = route_grp[tid];
+    }
+    if (tid == 16u) const_cast<int32_t*>(a.blk_range)[pb] = (int32_t)route_range;  // both halves write the same value
+    if (hb + 1u == a.n_half_blocks) {  // the padding slots behind the last 32-row block, up to the GEMM's tile rows
+      for (uint32_t p = a.n_half_blocks * 16u + tid; p < a.slots; p += 1024u) {
+        const_cast<int32_t*>(a.src_row)[p] = -1;
+        const_cast<int32_t*>(a.slot_group)[p] = route_last_group;
+        if ((p & 31u) == 0) const_cast<int32_t*>(a.blk_range)[p / 32u] = 0;
+      }
+    }
+  }
 
   // ---- 1. row statistics: wave w, slot row w
   {
     const uint32_t p = hb * 16u + wave;
-    int src = a.src_row ? a.src_row[p] : (int)p;
+    int src = route_here ? route_src[wave] : (a.src_row ? a.src_row[p] : (int)p);
     if (src < 0 || src >= (int)a.M) src = -1;
     float inv = 1.0f, amax = 0.0f;
     if (src >= 0) {
@@ -721,9 +841,11 @@ __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
   const float inv = row_inv[i], scale = row_scale[i];
   const float rscale = __builtin_amdgcn_rcpf(scale);
   const uint16_t* xr = a.x + (size_t)(src < 0 ? 0 : src) * a.K;
-  const uint32_t range = (CB > 0 && a.blk_range) ? (uint32_t)a.blk_range[pb] : 0u;
+  const uint32_t range = CB == 0 ? 0u : (route_here ? route_range : (a.blk_range ? (uint32_t)a.blk_range[pb] : 0u));
   const uint32_t glo = range & 0xffffu, ghi = range >> 16;
-  const uint32_t rowgrp = (CB > 0 && a.slot_group && ghi > glo) ? (uint32_t)a.slot_group[hb * 16u + i] : glo;
+  const uint32_t rowgrp = (CB > 0 && ghi > glo)
+                              ? (route_here ? (uint32_t)route_grp[i] : (a.slot_group ? (uint32_t)a.slot_group[hb * 16u + i] : glo))
+                              : glo;
   v4f acc[kCB];
 #pragma unroll
   for (int b = 0; b < kCB; ++b) acc[b] = v4f{0.f, 0.f, 0.f, 0.f};

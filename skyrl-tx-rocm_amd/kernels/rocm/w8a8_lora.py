@@ -344,14 +344,31 @@ class ForwardPlan:
                     "residual": lib.mi355_w8a8_lora_residual_v1}[entry]
         self.x_flat, self.gamma, self.adapter_indices = flat, gamma, idx
         self._keep = (flat, pw, a3, b3, s1, idx, gamma, res, ws)
+        self._lora = (a3, b3) if n_ad else None
+        self._packed_lora_key = None  # versions of A / B whose transposed / packed copies sit in the workspace
 
     def run(self, extra_flags: int = 0) -> torch.Tensor:
-        """Enqueue the call on torch's current stream; returns the (reused) output tensor."""
-        self.problem.flags = self.flags | extra_flags
+        """Enqueue the call on torch's current stream; returns the (reused) output tensor.
+
+        The transposed LoRA A and packed LoRA B live in the plan's workspace: while neither tensor has been
+        written since the last full run (``Tensor._version``), the call is told to keep them
+        (``FLAG_LORA_PACK_VALID``) instead of packing 2 * n * r * (K + N) bytes again.  A training step
+        updates the adapters, so its forward packs once per step as before."""
+        flags = self.flags | extra_flags
+        key = None
+        # (a captured call is replayed later, when the adapters may have changed: it always packs)
+        capturing = torch.cuda.is_current_stream_capturing()
+        if self._lora is not None and not capturing:
+            key = (self._lora[0]._version, self._lora[1]._version)
+            if key == self._packed_lora_key:
+                flags |= _native.FLAG_LORA_PACK_VALID
+        self.problem.flags = flags
         with torch.cuda.device(self.device):
             status = self._fn(ctypes.byref(self.problem), _stream_ptr(self.device))
         self.problem.flags = self.flags
         _native.check(f"mi355_w8a8_{self.entry}", status)
+        if not extra_flags & _native.FLAG_SKIP_PROLOGUE and not capturing:
+            self._packed_lora_key = key
         return self.out.reshape(self.out_shape)
 
 

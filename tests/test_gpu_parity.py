@@ -536,3 +536,42 @@ def test_same_named_fused_entry_points(dev, pkg):
     for got, ref in ((x.grad, want[0]), (a.grad, want[1]), (b.grad, want[2])):
         assert wc.compare(got.float().cpu().numpy(), ref)["violations"] == 0
     np.testing.assert_array_equal(res.grad.float().cpu().numpy(), cot)     # the residual's cotangent is dy
+
+
+def test_lora_pack_is_reused_until_the_adapters_change(dev, pkg):
+    """A plan keeps the transposed A / packed B in its workspace while the adapter tensors are unchanged
+    (the second run is told so and must give the same bits), and packs again after an in-place update."""
+    import torch
+
+    w8 = pkg.w8a8_lora
+    case = wc.make_case(600, 512, 768, n_adapters=3, rank=16, seed=51, rms=True, swiglu=True)
+    t = wc.to_torch(case, dev)
+    plan = w8.ForwardPlan(t["x"], t["weight"], t["a"], t["b"], t["s"], adapter_indices=t["idx"],
+                          rms_gamma=t["gamma"], eps=1e-6, swiglu=True)
+    first = plan.run().clone()
+    assert plan._packed_lora_key is not None
+    second = plan.run().clone()          # FLAG_LORA_PACK_VALID
+    assert torch.equal(first.view(torch.int16), second.view(torch.int16))
+    _assert_close(first.to(torch.float32).cpu().numpy(), wc.oracle_forward(case), " first run")
+    # an in-place update of B bumps its version: the next run packs again and follows the new values
+    t["b"].mul_(2.0)
+    third = plan.run().clone()
+    case2 = dict(case, b=case["b"] * np.float32(2.0))
+    _assert_close(third.to(torch.float32).cpu().numpy(), wc.oracle_forward(case2), " after the update")
+    assert not torch.equal(third.view(torch.int16), first.view(torch.int16))
+
+
+@pytest.mark.parametrize("m", [8192, 8200])
+def test_routing_inside_and_outside_the_quantizer_launch(dev, m):
+    """Up to 8192 rows the quantizer's workgroups sort the adapter indices themselves; beyond, a workgroup
+    of the preparation launch does.  Both sides of the switch, with an empty adapter and out-of-range
+    indices (clamped like an XLA gather), against the oracle."""
+    case = wc.make_case(m, 256, 512, n_adapters=5, rank=8, seed=61)
+    idx = case["idx"].copy()
+    idx[idx == 3] = 1          # adapter 3 has no rows
+    idx[5], idx[77] = -4, 99   # clamped to 0 and 4
+    case["idx"] = idx
+    want = wc.oracle_forward(dict(case, idx=np.clip(idx, 0, 4)), return_stages=True)
+    got, aux = wc.gpu_forward(case, flags=0)
+    _assert_integer_stages(aux, want)
+    _assert_close(got, want["out"], f" routing m={m}")
