@@ -459,10 +459,22 @@ __global__ __launch_bounds__(kSkinnyStreamThreads) void skinny_stream_kernel(Ski
     const int ad = ad_raw < 0 ? 0 : (ad_raw >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad_raw);
     f_s = (fvalid && lora) ? a.lora_scaling[ad] : 0.f;
     const uint16_t* Bp = a.lora_b + ((size_t)ad * a.r + rsel) * a.N + fn;
-    uint16_t bq[16];
+    // Every B value of the thread (ranks rsel, rsel + kRankSplit, ... below 64) is requested before the
+    // first is used: one trip to memory instead of one per value.
+    // The loads are unconditional (a load under a lane condition gets a branch and a wait of its own):
+    // lanes without an output read column 0, ranks beyond the rank read the last one; both are skipped
+    // when the values are used.
+    constexpr uint32_t kBValues = (uint32_t)kMaxRank / kRankSplit;
+    uint32_t bq[kBValues];
+    if (lora) {  // kernel-uniform
+      const uint16_t* Bs = a.lora_b + (size_t)ad * a.r * a.N + scol;
 #pragma unroll
-    for (uint32_t t = 0; t < 16; ++t)
-      bq[t] = (fvalid && lora && rsel + kRankSplit * t < a.r) ? Bp[(size_t)(kRankSplit * t) * a.N] : (uint16_t)0;
+      for (uint32_t t = 0; t < kBValues; ++t) {
+        uint32_t r = rsel + kRankSplit * t;
+        r = r < a.r ? r : a.r - 1u;
+        bq[t] = (uint32_t)Bs[(size_t)r * a.N];
+      }
+    }
     for (uint32_t zi = tid; zi < n_zval; zi += kSkinnyStreamThreads) {
       const float* zp = a.z_part + (size_t)(zi / rpad) * kMaxRank + zi % rpad;
       float zw4[kSkinnyMaxZChunks];
@@ -477,12 +489,10 @@ __global__ __launch_bounds__(kSkinnyStreamThreads) void skinny_stream_kernel(Ski
     __syncthreads();
     if (fvalid && lora) {
 #pragma unroll
-      for (uint32_t t = 0; t < 16; ++t) {
+      for (uint32_t t = 0; t < kBValues; ++t) {
         const uint32_t r = rsel + kRankSplit * t;
         if (r < a.r) low = fmaf(zl[frow][r], bf16_bits_to_f32(bq[t]), low);
       }
-      for (uint32_t r = rsel + kRankSplit * 16u; r < a.r; r += kRankSplit)
-        low = fmaf(zl[frow][r], bf16_bits_to_f32(Bp[(size_t)(r - rsel) * a.N]), low);
     }
     if (!ROWS2) {
       if (rsel == 1u) low_odd[tid & 255u] = low;
