@@ -1140,6 +1140,9 @@ def measure_linear(args, cfg, pkg, dev, steps, warmup, rotate, workload=None, fl
                                     residual=t.get("residual"), swiglu=bool(cfg.get("swiglu")),
                                     flags=flags))
     plan = plans[0]
+    if getattr(args, "repack_lora", False):
+        for pl in plans:
+            pl.keep_lora_pack = False
     torch.cuda.synchronize()
     # Spin-up, untimed and before the warm-up steps: the first launches after idle run while clocks and the
     # power controller settle (up to 20 % slow); the figure quoted is the sustained one.
@@ -1300,6 +1303,9 @@ def main() -> int:
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     ap.add_argument("--spin-up", type=float, default=0.5,
                     help="seconds of untimed calls before the warm-up steps (clocks and power controller settle)")
+    ap.add_argument("--repack-lora", action="store_true",
+                    help="transpose / pack the LoRA factors on every step (a training step's forward) instead of "
+                         "keeping them in the plan's workspace while the adapters are unchanged")
     ap.add_argument("--no-decode", action="store_true", help="default workload: skip the decode block")
     ap.add_argument("--no-ceilings", action="store_true", help="default workload: skip the measured ceilings")
     args = ap.parse_args()
@@ -1368,6 +1374,10 @@ def main() -> int:
         "spin_up_s": r["spin_up_s"],
         "prologue_ms": r["prologue_ms"],
         "path": r["path"],
+        # the steps reuse one plan with unchanged adapters: the transposed / packed LoRA factors stay in its
+        # workspace (MI355_W8A8_FLAG_LORA_PACK_VALID) as they would between the calls of a serving loop;
+        # --repack-lora makes every step pack them again, as a training step does after an adapter update
+        "lora_pack": "repacked every step" if args.repack_lora else "kept in the workspace across steps",
         "roofline": r["roofline"],
     }
     if args.workload == "qwen3-8b-gate_up-m4096" and not args.no_decode:

@@ -438,6 +438,166 @@ ffi::Error GqLinear(hipStream_t stream, ffi::Buffer<ffi::BF16> x, ffi::Buffer<ff
   return ToError(mi355_w8a8_gq_linear_v1(&p, stream), "mi355_w8a8 gq linear launch submission failed");
 }
 
+// Backward of the grouped call (mi355_w8a8_grouped_bwd_v1).  x [M, K] and dy [M, N] bf16 in group order, packed
+// weights, scales f32 [n_weights, N], A [G, K, r], B [G, r, N], scaling [G] (size-0 without LoRA), group_sizes
+// s32 [G].  Results: dx bf16 [M, K], dA, dB bf16 like A, B, dscaling f32 [G] (size 0 without LoRA), workspace u8.
+ffi::Error GroupedBwd(hipStream_t stream, ffi::Buffer<ffi::BF16> x, ffi::Buffer<ffi::BF16> dy,
+                      ffi::Buffer<ffi::U8> w_packed, ffi::Buffer<ffi::F32> w_scales, ffi::Buffer<ffi::BF16> lora_a,
+                      ffi::Buffer<ffi::BF16> lora_b, ffi::Buffer<ffi::F32> lora_scaling,
+                      ffi::Buffer<ffi::S32> group_sizes, ffi::ResultBuffer<ffi::BF16> dx,
+                      ffi::ResultBuffer<ffi::BF16> d_lora_a, ffi::ResultBuffer<ffi::BF16> d_lora_b,
+                      ffi::ResultBuffer<ffi::F32> d_lora_scaling, ffi::ResultBuffer<ffi::U8> workspace) {
+  mi355_w8a8_grouped_bwd_problem p{};
+  p.struct_size = sizeof(p);
+  if (!RowsAndK(x.dimensions(), &p.m, &p.k))
+    return ffi::Error::InvalidArgument("x must be bf16 [M, K] with a non-empty row domain");
+  auto ds = w_scales.dimensions();
+  if (ds.size() != 2 || ds[0] <= 0 || ds[1] <= 0) return ffi::Error::InvalidArgument("w_scales must be f32 [n_weights, N]");
+  const uint32_t n_weights = static_cast<uint32_t>(ds[0]);
+  p.n = static_cast<uint32_t>(ds[1]);
+  p.n_groups = static_cast<uint32_t>(group_sizes.element_count());
+  if (p.n_groups == 0 || p.n_groups % n_weights != 0)
+    return ffi::Error::InvalidArgument("group_sizes must be s32 [G] with G a multiple of the number of weights");
+  p.groups_per_weight = p.n_groups / n_weights;
+  if (dy.element_count() != static_cast<size_t>(p.m) * p.n || dx->element_count() != x.element_count())
+    return ffi::Error::InvalidArgument("dy must be bf16 [M, N] and dx must match x");
+  if (w_packed.size_bytes() != static_cast<size_t>(n_weights) * mi355_w8a8_packed_weight_bytes(p.k, p.n))
+    return ffi::Error::InvalidArgument("packed weights do not match (n_weights, K, N)");
+  if (lora_a.element_count() > 0) {
+    auto da = lora_a.dimensions();
+    auto db = lora_b.dimensions();
+    if (da.size() != 3 || db.size() != 3 || da[0] != p.n_groups || da[1] != p.k || db[0] != da[0] ||
+        db[1] != da[2] || db[2] != p.n || lora_scaling.element_count() != p.n_groups)
+      return ffi::Error::InvalidArgument("LoRA A/B/scaling must be [G,K,r], [G,r,N], [G]");
+    if (d_lora_a->element_count() != lora_a.element_count() || d_lora_b->element_count() != lora_b.element_count() ||
+        d_lora_scaling->element_count() != lora_scaling.element_count())
+      return ffi::Error::InvalidArgument("the LoRA cotangents must match the LoRA parameters");
+    p.rank = static_cast<uint32_t>(da[2]);
+    p.lora_a = lora_a.untyped_data();
+    p.lora_b = lora_b.untyped_data();
+    p.lora_scaling = lora_scaling.typed_data();
+    p.d_lora_a = d_lora_a->untyped_data();
+    p.d_lora_b = d_lora_b->untyped_data();
+    p.d_lora_scaling = d_lora_scaling->typed_data();
+  }
+  p.x = x.untyped_data();
+  p.dy = dy.untyped_data();
+  p.w_packed = w_packed.untyped_data();
+  p.w_scales = w_scales.typed_data();
+  p.group_sizes = group_sizes.typed_data();
+  p.dx = dx->untyped_data();
+  p.workspace = workspace->untyped_data();
+  p.workspace_bytes = workspace->size_bytes();
+  return ToError(mi355_w8a8_grouped_bwd_v1(&p, stream), "mi355_w8a8 grouped backward launch submission failed");
+}
+
+// Pull-back of the attention input stage.  fused bf16 [M, width], the two head-norm weights f32 [D], positions
+// s32 [M], the four output cotangents.  Results: d_fused bf16 [M, width], d_q_norm_weight and d_k_norm_weight
+// f32 [D] (size 0: not wanted, both or neither), workspace u8 (size 0 without the weight cotangents).
+ffi::Error QkvSplitNormRopeBwd(hipStream_t stream, ffi::Buffer<ffi::BF16> fused, ffi::Buffer<ffi::F32> q_norm_weight,
+                               ffi::Buffer<ffi::F32> k_norm_weight, ffi::Buffer<ffi::S32> positions,
+                               ffi::Buffer<ffi::BF16> d_q, ffi::Buffer<ffi::BF16> d_k, ffi::Buffer<ffi::BF16> d_v,
+                               ffi::Buffer<ffi::BF16> d_gate, ffi::ResultBuffer<ffi::BF16> d_fused,
+                               ffi::ResultBuffer<ffi::F32> d_q_norm_weight, ffi::ResultBuffer<ffi::F32> d_k_norm_weight,
+                               ffi::ResultBuffer<ffi::U8> workspace, int32_t rotary_dim, float rope_theta,
+                               float rms_eps) {
+  mi355_w8a8_qkv_post_bwd_problem p{};
+  p.struct_size = sizeof(p);
+  auto dq = d_q.dimensions();
+  auto dk = d_k.dimensions();
+  if (dq.size() != 3 || dk.size() != 3 || dq[0] <= 0 || dk[0] != dq[0] || dk[2] != dq[2] || dq[1] <= 0 || dk[1] <= 0)
+    return ffi::Error::InvalidArgument("d_q must be bf16 [M, H, D] and d_k bf16 [M, Hkv, D]");
+  p.m = static_cast<uint32_t>(dq[0]);
+  p.num_query_heads = static_cast<uint32_t>(dq[1]);
+  p.num_kv_heads = static_cast<uint32_t>(dk[1]);
+  p.head_dim = static_cast<uint32_t>(dq[2]);
+  const size_t width = static_cast<size_t>(p.num_query_heads) * 2 * p.head_dim + 2 * static_cast<size_t>(p.num_kv_heads) * p.head_dim;
+  if (fused.element_count() != static_cast<size_t>(p.m) * width || d_fused->element_count() != fused.element_count() ||
+      d_v.element_count() != d_k.element_count() || d_gate.element_count() != d_q.element_count() ||
+      positions.element_count() != p.m || q_norm_weight.element_count() != p.head_dim ||
+      k_norm_weight.element_count() != p.head_dim)
+    return ffi::Error::InvalidArgument("fused, d_fused, d_v, d_gate, positions or the norm weights do not match (M, H, Hkv, D)");
+  if (rotary_dim < 0) return ffi::Error::InvalidArgument("rotary_dim must be >= 0");
+  const bool want_w = d_q_norm_weight->element_count() > 0 || d_k_norm_weight->element_count() > 0;
+  if (want_w) {
+    if (d_q_norm_weight->element_count() != p.head_dim || d_k_norm_weight->element_count() != p.head_dim)
+      return ffi::Error::InvalidArgument("the norm-weight cotangents must both be f32 [D], or both empty");
+    p.d_q_norm_weight = d_q_norm_weight->typed_data();
+    p.d_k_norm_weight = d_k_norm_weight->typed_data();
+    p.workspace = workspace->untyped_data();
+    p.workspace_bytes = workspace->size_bytes();
+  }
+  p.rotary_dim = static_cast<uint32_t>(rotary_dim);
+  p.rope_theta = rope_theta;
+  p.rms_eps = rms_eps;
+  p.fused = fused.untyped_data();
+  p.q_norm_weight = q_norm_weight.typed_data();
+  p.k_norm_weight = k_norm_weight.typed_data();
+  p.positions = positions.typed_data();
+  p.d_q = d_q.untyped_data();
+  p.d_k = d_k.untyped_data();
+  p.d_v = d_v.untyped_data();
+  p.d_gate = d_gate.untyped_data();
+  p.d_fused = d_fused->untyped_data();
+  return ToError(mi355_w8a8_qkv_split_norm_rope_bwd_v1(&p, stream), "mi355_w8a8 qkv stage backward launch submission failed");
+}
+
+// Pull-back of the decoder norm in delta form: x, d_normalized bf16 [.., K], gamma f32 [K].  Results: d_x bf16
+// [.., K], d_gamma f32 [K] (size 0: not wanted), workspace u8 (size 0 without d_gamma).
+ffi::Error DeltaRmsNormBwd(hipStream_t stream, ffi::Buffer<ffi::BF16> x, ffi::Buffer<ffi::F32> gamma,
+                           ffi::Buffer<ffi::BF16> d_normalized, ffi::ResultBuffer<ffi::BF16> d_x,
+                           ffi::ResultBuffer<ffi::F32> d_gamma, ffi::ResultBuffer<ffi::U8> workspace, float eps) {
+  uint32_t m = 0, k = 0;
+  if (!RowsAndK(x.dimensions(), &m, &k))
+    return ffi::Error::InvalidArgument("x must be bf16 [..., K] with a non-empty row domain");
+  if (gamma.element_count() != k || d_normalized.element_count() != x.element_count() ||
+      d_x->element_count() != x.element_count() || (d_gamma->element_count() != 0 && d_gamma->element_count() != k))
+    return ffi::Error::InvalidArgument("gamma must be f32 [K]; d_normalized and d_x must match x; d_gamma f32 [K] or empty");
+  const bool want_g = d_gamma->element_count() > 0;
+  return ToError(mi355_w8a8_delta_rms_norm_bwd_v1(x.untyped_data(), gamma.typed_data(), d_normalized.untyped_data(),
+                                                  d_x->untyped_data(), want_g ? d_gamma->typed_data() : nullptr,
+                                                  want_g ? workspace->untyped_data() : nullptr,
+                                                  want_g ? workspace->size_bytes() : 0, m, k, eps, stream),
+                 "mi355_w8a8 delta rms norm pull-back launch submission failed");
+}
+
+// Pull-back of the router: logits f32 [T, E], selected s32 [T, top_k], d_weights f32 [T, top_k] -> d_logits f32 [T, E].
+ffi::Error MoeRouteBwd(hipStream_t stream, ffi::Buffer<ffi::F32> router_logits, ffi::Buffer<ffi::S32> selected,
+                       ffi::Buffer<ffi::F32> d_weights, ffi::ResultBuffer<ffi::F32> d_router_logits,
+                       int32_t norm_topk_prob) {
+  auto d = router_logits.dimensions();
+  auto dw = d_weights.dimensions();
+  if (d.size() != 2 || dw.size() != 2 || d[0] <= 0 || dw[0] != d[0] || dw[1] <= 0 ||
+      selected.element_count() != d_weights.element_count() ||
+      d_router_logits->element_count() != router_logits.element_count())
+    return ffi::Error::InvalidArgument("router_logits and d_router_logits must be f32 [T, E]; selected and d_weights [T, top_k]");
+  return ToError(mi355_w8a8_moe_route_bwd_v1(router_logits.typed_data(), selected.typed_data(), d_weights.typed_data(),
+                                             static_cast<uint32_t>(d[0]), static_cast<uint32_t>(d[1]),
+                                             static_cast<uint32_t>(dw[1]), norm_topk_prob ? 1u : 0u,
+                                             d_router_logits->typed_data(), stream),
+                 "mi355_w8a8 moe route pull-back launch submission failed");
+}
+
+// Pull-back of the combine: d_out bf16 [T, H], expert_out bf16 [T top_k, H] in sorted order, sort_indices s32
+// [T top_k], weights f32 [T, top_k].  Results: d_expert_out bf16 [T top_k, H], d_weights f32 [T, top_k].
+ffi::Error MoeCombineBwd(hipStream_t stream, ffi::Buffer<ffi::BF16> d_out, ffi::Buffer<ffi::BF16> expert_out,
+                         ffi::Buffer<ffi::S32> sort_indices, ffi::Buffer<ffi::F32> weights,
+                         ffi::ResultBuffer<ffi::BF16> d_expert_out, ffi::ResultBuffer<ffi::F32> d_weights) {
+  auto dd = d_out.dimensions();
+  auto dw = weights.dimensions();
+  if (dd.size() != 2 || dw.size() != 2 || dw[0] != dd[0] || dw[0] <= 0 || dw[1] <= 0 || dd[1] <= 0)
+    return ffi::Error::InvalidArgument("d_out must be bf16 [T, H] and weights f32 [T, top_k]");
+  const size_t pairs = static_cast<size_t>(dw[0]) * dw[1];
+  if (expert_out.element_count() != pairs * dd[1] || d_expert_out->element_count() != pairs * dd[1] ||
+      sort_indices.element_count() != pairs || d_weights->element_count() != pairs)
+    return ffi::Error::InvalidArgument("expert_out and d_expert_out must be [T * top_k, H]; sort_indices and d_weights hold T * top_k entries");
+  return ToError(mi355_w8a8_moe_combine_bwd_v1(d_out.untyped_data(), expert_out.untyped_data(), sort_indices.typed_data(),
+                                               weights.typed_data(), d_expert_out->untyped_data(), d_weights->typed_data(),
+                                               static_cast<uint32_t>(dw[0]), static_cast<uint32_t>(dw[1]),
+                                               static_cast<uint32_t>(dd[1]), stream),
+                 "mi355_w8a8 moe combine pull-back launch submission failed");
+}
+
 }  // namespace
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_forward_v1, Forward,
@@ -585,4 +745,69 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_gq_linear_v1, GqLinear,
                                   .Attr<int32_t>("group_size")
                                   .Attr<int32_t>("weight_bits")
                                   .Attr<int32_t>("activation_bits"));
+XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_grouped_bwd_v1, GroupedBwd,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::U8>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::F32>>()
+                                  .Ret<ffi::Buffer<ffi::U8>>());
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_qkv_split_norm_rope_bwd_v1, QkvSplitNormRopeBwd,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::F32>>()
+                                  .Ret<ffi::Buffer<ffi::F32>>()
+                                  .Ret<ffi::Buffer<ffi::U8>>()
+                                  .Attr<int32_t>("rotary_dim")
+                                  .Attr<float>("rope_theta")
+                                  .Attr<float>("rms_eps"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_delta_rms_norm_bwd_v1, DeltaRmsNormBwd,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::F32>>()
+                                  .Ret<ffi::Buffer<ffi::U8>>()
+                                  .Attr<float>("eps"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_moe_route_bwd_v1, MoeRouteBwd,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Ret<ffi::Buffer<ffi::F32>>()
+                                  .Attr<int32_t>("norm_topk_prob"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(mi355_w8a8_ffi_moe_combine_bwd_v1, MoeCombineBwd,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::F32>>());
 #endif  // __has_include("xla/ffi/api/ffi.h")

@@ -27,7 +27,8 @@ TARGETS = ("mi355_w8a8_ffi_forward_v1", "mi355_w8a8_ffi_quantize_rows_v1", "mi35
            "mi355_w8a8_ffi_backward_v1", "mi355_w8a8_ffi_swiglu_bwd_v1", "mi355_w8a8_ffi_rms_norm_bwd_v1",
            "mi355_w8a8_ffi_moe_route_v1", "mi355_w8a8_ffi_moe_dispatch_v1", "mi355_w8a8_ffi_moe_combine_v1",
            "mi355_w8a8_ffi_grouped_v1", "mi355_w8a8_ffi_qkv_split_norm_rope_v1", "mi355_w8a8_ffi_gq_pack_weight_v1",
-           "mi355_w8a8_ffi_gq_linear_v1")
+           "mi355_w8a8_ffi_gq_linear_v1", "mi355_w8a8_ffi_grouped_bwd_v1", "mi355_w8a8_ffi_qkv_split_norm_rope_bwd_v1",
+           "mi355_w8a8_ffi_delta_rms_norm_bwd_v1", "mi355_w8a8_ffi_moe_route_bwd_v1", "mi355_w8a8_ffi_moe_combine_bwd_v1")
 _ROCM_PLATFORM = "ROCM"
 _REGISTRATION_API_VERSION = 1
 _CUSTOM_CALL_API_VERSION = 4
@@ -346,3 +347,95 @@ def moe_combine(expert_out, unsort_indices, weights):
     (out,) = _call(jax, TARGETS[8], (jax.ShapeDtypeStruct((t, expert_out.shape[1]), jnp.bfloat16),), expert_out,
                    unsort_indices.astype(jnp.int32), weights.astype(jnp.float32))
     return out
+
+
+def grouped_backward(x, dy, packed_weights, w_scales, group_sizes, lora_a=None, lora_b=None, lora_scaling=None):
+    """Cotangents of the grouped call as one XLA custom call: ``(dx, dA, dB, dscaling)`` (the LoRA entries
+    ``None`` without LoRA) -- the backward rule a ``jax.custom_vjp`` around ``LoRAExpert.__call__``
+    (skyrl/tx/layers/lora.py:394-444) binds."""
+    jax = _import_jax()
+    register(jax)
+    jnp = jax.numpy
+    m, k = x.shape
+    n = w_scales.shape[-1]
+    n_groups = group_sizes.shape[0]
+    n_weights = w_scales.reshape(-1, n).shape[0]
+    empty = lambda dt, nd: jnp.zeros((0,) * nd, dt)
+    a3 = empty(jnp.bfloat16, 3) if lora_a is None else lora_a
+    b3 = empty(jnp.bfloat16, 3) if lora_b is None else lora_b
+    rank = a3.shape[2] if lora_a is not None else 0
+    s1 = (empty(jnp.float32, 1) if lora_a is None
+          else jnp.broadcast_to(jnp.asarray(lora_scaling, jnp.float32), (n_groups,)))
+    ws = int(_native.load().mi355_w8a8_grouped_bwd_workspace_bytes(m, k, n, n_groups, rank, n_groups // n_weights))
+    if ws == 0:
+        raise ValueError(f"geometry M={m}, K={k}, N={n}, groups={n_groups} is outside the native backward")
+    dx, da, db, ds, _ = _call(
+        jax, TARGETS[13],
+        (jax.ShapeDtypeStruct((m, k), jnp.bfloat16), jax.ShapeDtypeStruct(a3.shape, jnp.bfloat16),
+         jax.ShapeDtypeStruct(b3.shape, jnp.bfloat16), jax.ShapeDtypeStruct(s1.shape, jnp.float32),
+         jax.ShapeDtypeStruct((ws,), jnp.uint8)),
+        x, dy, packed_weights, w_scales.reshape(-1, n).astype(jnp.float32), a3, b3, s1, group_sizes.astype(jnp.int32))
+    if lora_a is None:
+        return dx, None, None, None
+    return dx, da, db, ds
+
+
+def qkv_split_norm_rope_backward(fused, q_norm_weight, k_norm_weight, positions, d_q, d_k, d_v, d_gate, *,
+                                 rotary_dim: int, rope_theta: float, eps: float = 1e-6, want_weight_grads: bool = True):
+    """Pull-back of ``qkv_split_norm_rope`` (skyrl/tx/kernels/qwen3_5_qkv_lora.py:391-425):
+    ``(d_fused, d_q_norm_weight, d_k_norm_weight)``; the weight cotangents are ``None`` when not wanted."""
+    jax = _import_jax()
+    register(jax)
+    jnp = jax.numpy
+    m, heads, head_dim = d_q.shape
+    nw = head_dim if want_weight_grads else 0
+    ws = int(_native.load().mi355_w8a8_qkv_bwd_workspace_bytes(m, head_dim)) if want_weight_grads else 0
+    d_fused, dqw, dkw, _ = _call(
+        jax, TARGETS[14],
+        (jax.ShapeDtypeStruct(fused.shape, jnp.bfloat16), jax.ShapeDtypeStruct((nw,), jnp.float32),
+         jax.ShapeDtypeStruct((nw,), jnp.float32), jax.ShapeDtypeStruct((ws,), jnp.uint8)),
+        fused, q_norm_weight.astype(jnp.float32), k_norm_weight.astype(jnp.float32),
+        positions.astype(jnp.int32).reshape(m), d_q, d_k, d_v, d_gate, rotary_dim=int(rotary_dim),
+        rope_theta=float(rope_theta), rms_eps=float(eps))
+    return (d_fused, dqw, dkw) if want_weight_grads else (d_fused, None, None)
+
+
+def delta_rms_norm_backward(x, gamma, d_normalized, *, eps: float = 1e-6, want_gamma_grad: bool = True):
+    """Pull-back of the decoder norm with multiplier ``gamma = 1 + weight``
+    (skyrl/tx/kernels/qwen3_5_qkv_lora.py:97-116): ``(d_x, d_gamma or None)``."""
+    jax = _import_jax()
+    register(jax)
+    jnp = jax.numpy
+    k = x.shape[-1]
+    m = 1
+    for d in x.shape[:-1]:
+        m *= d
+    ng = k if want_gamma_grad else 0
+    ws = int(_native.load().mi355_w8a8_delta_rms_norm_bwd_workspace_bytes(m, k)) if want_gamma_grad else 0
+    d_x, d_gamma, _ = _call(jax, TARGETS[15],
+                            (jax.ShapeDtypeStruct(x.shape, jnp.bfloat16), jax.ShapeDtypeStruct((ng,), jnp.float32),
+                             jax.ShapeDtypeStruct((ws,), jnp.uint8)),
+                            x, gamma.astype(jnp.float32), d_normalized, eps=float(eps))
+    return d_x, (d_gamma if want_gamma_grad else None)
+
+
+def moe_route_backward(router_logits, selected, d_weights, norm_topk_prob: bool):
+    """Cotangent of the router logits with the selection held fixed (skyrl/tx/models/qwen3.py:175-178)."""
+    jax = _import_jax()
+    register(jax)
+    jnp = jax.numpy
+    (d_logits,) = _call(jax, TARGETS[16], (jax.ShapeDtypeStruct(router_logits.shape, jnp.float32),),
+                        router_logits.astype(jnp.float32), selected.astype(jnp.int32), d_weights.astype(jnp.float32),
+                        norm_topk_prob=int(bool(norm_topk_prob)))
+    return d_logits
+
+
+def moe_combine_backward(d_out, expert_out, sort_indices, weights):
+    """Cotangents of the combine in its two operands (skyrl/tx/models/qwen3.py:205-207):
+    ``(d_expert_out bf16 [T * top_k, H], d_weights f32 [T, top_k])``."""
+    jax = _import_jax()
+    register(jax)
+    jnp = jax.numpy
+    return _call(jax, TARGETS[17],
+                 (jax.ShapeDtypeStruct(expert_out.shape, jnp.bfloat16), jax.ShapeDtypeStruct(weights.shape, jnp.float32)),
+                 d_out, expert_out, sort_indices.astype(jnp.int32), weights.astype(jnp.float32))

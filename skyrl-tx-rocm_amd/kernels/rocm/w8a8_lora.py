@@ -346,6 +346,7 @@ class ForwardPlan:
         self._keep = (flat, pw, a3, b3, s1, idx, gamma, res, ws)
         self._lora = (a3, b3) if n_ad else None
         self._packed_lora_key = None  # versions of A / B whose transposed / packed copies sit in the workspace
+        self.keep_lora_pack = True    # False: pack on every run (what a caller that rewrites A / B behind torch's back needs)
 
     def run(self, extra_flags: int = 0) -> torch.Tensor:
         """Enqueue the call on torch's current stream; returns the (reused) output tensor.
@@ -358,7 +359,7 @@ class ForwardPlan:
         key = None
         # (a captured call is replayed later, when the adapters may have changed: it always packs)
         capturing = torch.cuda.is_current_stream_capturing()
-        if self._lora is not None and not capturing:
+        if self._lora is not None and not capturing and self.keep_lora_pack:
             key = (self._lora[0]._version, self._lora[1]._version)
             if key == self._packed_lora_key:
                 flags |= _native.FLAG_LORA_PACK_VALID

@@ -89,7 +89,7 @@ def test_shim_source_obeys_the_handler_rules():
                        "-ffast-math"):
             assert banned not in text, (src.name, banned)
     shim = (root / "w8a8_xla_ffi.cc").read_text()
-    assert shim.count("XLA_FFI_DEFINE_HANDLER_SYMBOL") == 13
+    assert shim.count("XLA_FFI_DEFINE_HANDLER_SYMBOL") == 18
     assert "PlatformStream<hipStream_t>" in shim
 
 
@@ -112,6 +112,18 @@ def test_every_target_has_a_handler_symbol_and_a_c_entry_point():
                     "mi355_w8a8_gq_pack_weight_v1"):
         assert f"{c_entry}(" in shim
     assert "x_row_map" in shim and "x_row_repeat" in shim
+    # every typed-FFI target the integration notes name exists, and every C entry point that launches work
+    # (the *_v1 functions of the header, calibration and measurement helpers aside) sits behind a handler
+    root = Path(__file__).resolve().parents[1]
+    notes = (root / "INTEGRATION.md").read_text()
+    for name in set(re.findall(r"mi355_w8a8_ffi_\w+_v1", notes)):
+        assert name in w8a8_ffi.TARGETS, name
+    header = (root / "include" / "mi355_w8a8.h").read_text()
+    entries = set(re.findall(r"\bint (mi355_w8a8_\w+_v1)\(", header))
+    not_bound = {e for e in entries if f"{e}(" not in shim}
+    assert not_bound <= {"mi355_w8a8_unpack_weight_v1", "mi355_w8a8_forward_static_ws_v1", "mi355_w8a8_swiglu_v1",
+                         "mi355_w8a8_calibrate_mfma_v1", "mi355_w8a8_calibrate_read_v1",
+                         "mi355_w8a8_calibrate_copy_v1"}, not_bound
 
 
 class _FakeSpec:
