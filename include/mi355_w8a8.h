@@ -82,7 +82,9 @@ typedef enum mi355_w8a8_status {
 /* The workspace still holds the transposed LoRA A and the packed LoRA B that an earlier call of the tiled
  * path wrote there for the same lora_a / lora_b contents and the same (k, n, n_adapters, rank): this call
  * does not write them again (adapters that do not change between calls, as in serving).  The caller
- * vouches for it; calls of at most 128 rows keep no such copies and ignore the flag. */
+ * vouches for it; calls of 17..128 rows keep no such copies and ignore the flag. */
+/* For calls of at most 16 rows (rank <= 32) the same flag covers the per-row regrouped copy of B the decode
+ * kernels keep in the workspace: it additionally vouches that adapter_indices has the contents it had then. */
 #define MI355_W8A8_FLAG_LORA_PACK_VALID 1024u
 
 /*

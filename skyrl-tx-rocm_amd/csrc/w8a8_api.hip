@@ -207,12 +207,15 @@ int launch_skinny(const mi355_w8a8_problem* p, unsigned char* xq, float* sx, uin
     q.n_adapters = p->n_adapters; q.r = p->rank; q.z_chunks = L.z_chunks; q.z_chunk_k = L.z_chunk_k;
     q.n_z_units = (lora && !rms) ? p->m * L.z_chunks : 0u;
     const bool regroup = allow_regroup && lora && p->rank <= 32u && p->m <= 16u && (p->n % 8u) == 0;
-    q.lora_b = regroup ? static_cast<const uint16_t*>(p->lora_b) : nullptr;
+    // the caller may vouch that the regrouped B of an earlier call (same B, same adapter per row) is still
+    // in the workspace; a call in 32-row chunks shares one workspace between its chunks and never keeps it
+    const bool keep_regrouped = regroup && (p->flags & MI355_W8A8_FLAG_LORA_PACK_VALID);
+    q.lora_b = (regroup && !keep_regrouped) ? static_cast<const uint16_t*>(p->lora_b) : nullptr;
     q.bsel = reinterpret_cast<uint16_t*>(sws + L.bsel);
     q.N = p->n; q.n_groups = n_padded(p->n) / 128u;
     q.lora_scaling = lora ? p->lora_scaling : nullptr;
     q.row_scaling = reinterpret_cast<float*>(sws + L.row_scaling);
-    const uint32_t n_regroup = regroup ? (p->m * q.n_groups + 3u) / 4u : 0u;
+    const uint32_t n_regroup = (regroup && !keep_regrouped) ? (p->m * q.n_groups + 3u) / 4u : 0u;
     if (rms) hipLaunchKernelGGL((skinny_quant_kernel<true>), dim3(p->m + n_regroup), dim3(1024), 0, s, q);
     else hipLaunchKernelGGL((skinny_quant_kernel<false>), dim3(p->m + q.n_z_units + n_regroup), dim3(1024), 0, s, q);
     if ((st = launch_status())) return st;

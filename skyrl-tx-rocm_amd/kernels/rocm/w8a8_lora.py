@@ -351,7 +351,8 @@ class ForwardPlan:
     def run(self, extra_flags: int = 0) -> torch.Tensor:
         """Enqueue the call on torch's current stream; returns the (reused) output tensor.
 
-        The transposed LoRA A and packed LoRA B live in the plan's workspace: while neither tensor has been
+        The transposed LoRA A and packed LoRA B (for a decode-sized call: B regrouped per row by its adapter)
+        live in the plan's workspace: while neither tensor nor the adapter indices have been
         written since the last full run (``Tensor._version``), the call is told to keep them
         (``FLAG_LORA_PACK_VALID``) instead of packing 2 * n * r * (K + N) bytes again.  A training step
         updates the adapters, so its forward packs once per step as before."""
@@ -360,7 +361,8 @@ class ForwardPlan:
         # (a captured call is replayed later, when the adapters may have changed: it always packs)
         capturing = torch.cuda.is_current_stream_capturing()
         if self._lora is not None and not capturing and self.keep_lora_pack:
-            key = (self._lora[0]._version, self._lora[1]._version)
+            key = (self._lora[0]._version, self._lora[1]._version,
+                   None if self.adapter_indices is None else self.adapter_indices._version)
             if key == self._packed_lora_key:
                 flags |= _native.FLAG_LORA_PACK_VALID
         self.problem.flags = flags

@@ -575,3 +575,27 @@ def test_routing_inside_and_outside_the_quantizer_launch(dev, m):
     got, aux = wc.gpu_forward(case, flags=0)
     _assert_integer_stages(aux, want)
     _assert_close(got, want["out"], f" routing m={m}")
+
+
+def test_decode_regrouped_b_is_reused_until_b_or_the_indices_change(dev, pkg):
+    """The decode kernels keep B regrouped per row in the workspace; a plan reuses it while B and the
+    adapter indices are unchanged and rebuilds it after either is written."""
+    import torch
+
+    w8 = pkg.w8a8_lora
+    case = wc.make_case(12, 1024, 768, n_adapters=5, rank=16, seed=71, residual=True)
+    t = wc.to_torch(case, dev)
+    plan = w8.ForwardPlan(t["x"], t["weight"], t["a"], t["b"], t["s"], adapter_indices=t["idx"], residual=t["residual"])
+    first = plan.run().clone()
+    second = plan.run().clone()          # regrouped B kept
+    assert torch.equal(first.view(torch.int16), second.view(torch.int16))
+    _assert_close(first.to(torch.float32).cpu().numpy(), wc.oracle_forward(case), " decode first run")
+    new_idx = (case["idx"] + 2) % 5
+    plan.adapter_indices.copy_(torch.from_numpy(new_idx.astype(np.int32)).to(dev))
+    third = plan.run().clone()
+    _assert_close(third.to(torch.float32).cpu().numpy(), wc.oracle_forward(dict(case, idx=new_idx.astype(np.int32))),
+                  " decode after new indices")
+    t["b"].mul_(-1.0)
+    fourth = plan.run().clone()
+    _assert_close(fourth.to(torch.float32).cpu().numpy(),
+                  wc.oracle_forward(dict(case, idx=new_idx.astype(np.int32), b=-case["b"])), " decode after new B")
