@@ -72,7 +72,7 @@ typedef enum mi355_w8a8_status {
  * prologue results and answer these two flags with MI355_W8A8_ERR_UNSUPPORTED. */
 #define MI355_W8A8_FLAG_SKIP_PROLOGUE 16u /* do not run routing / quantization / LoRA-A */
 #define MI355_W8A8_FLAG_SKIP_GEMM 32u     /* run only routing / quantization / LoRA-A */
-/* tile geometry of the tiled GEMM; default: 256 x 256 once such tiles fill the chip, else 256 x 128 */
+/* tile geometry of the tiled GEMM; default: 256 x 256 once such tiles fill half the CUs, else 256 x 128 */
 #define MI355_W8A8_FLAG_TILE_256X128 64u
 #define MI355_W8A8_FLAG_TILE_256X256 128u
 /* tile rows of the grouped call (and the slots every group is padded to); default: 128 once the
