@@ -915,13 +915,17 @@ __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) c[e] = rintf(v[e] / scale);
       }
+      // c is an integer in [-127, 127] (|v| <= the row's absmax, so the clip of the reference never
+      // acts): c + 128 converts and lands in its byte with one v_cvt_pk_u8_f32 (which saturates to
+      // 0..255 anyway), and flipping bit 7 of every byte turns the biased value into two's complement
       uint32_t lo = 0, hi = 0;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float cc = fminf(fmaxf(c[e], -127.0f), 127.0f);
-        const uint32_t b = (uint32_t)(int)cc & 0xffu;
-        if (e < 4) lo |= b << (8 * e); else hi |= b << (8 * (e - 4));
+      for (int e = 0; e < 4; ++e) {
+        lo = __builtin_amdgcn_cvt_pk_u8_f32(c[e] + 128.0f, (uint32_t)e, lo);
+        hi = __builtin_amdgcn_cvt_pk_u8_f32(c[e + 4] + 128.0f, (uint32_t)e, hi);
       }
+      lo ^= 0x80808080u;
+      hi ^= 0x80808080u;
       if (!live) { lo = 0; hi = 0; }
       if (live && a.codes_rm) *reinterpret_cast<uint2*>(a.codes_rm + (size_t)src * a.K + k0) = make_uint2(lo, hi);
       *reinterpret_cast<uint2*>(a.xq_packed + ((size_t)pb * a.KB + kb) * kBlockBytes + code_off) = make_uint2(lo, hi);
