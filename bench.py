@@ -116,7 +116,7 @@ COPY_KIB = 262144.0  # the calibration copy moves 256 MiB each way
 def measured_traffic_bytes(workload, profiles_dir=None):
     """HBM bytes per launch of the workload's dominant kernel(s) from its committed counter summary, or None.
 
-    Every kernel named for the workload must appear once per counter and the summary must hold the
+    Every kernel named for the workload must appear for each counter and the summary must hold the
     calibration copy; anything else (no summary yet, renamed kernel) gives None rather than a stale figure."""
     entry = PROFILE_TRAFFIC.get(workload)
     if entry is None:
@@ -135,16 +135,18 @@ def measured_traffic_bytes(workload, profiles_dir=None):
         if "cal_copy_kernel" in hit["name"] or (hit["name"].startswith("__amd_rocclr_copyBuffer")
                                                and int(hit["grid"]) == 131072 and int(hit["n"]) == 1):
             copy[hit["ctr"]] = float(hit["kib"])
-        rows.append((hit["name"], hit["ctr"], float(hit["kib"])))
+        rows.append((hit["name"], hit["ctr"], float(hit["kib"]), int(hit["n"])))
     if set(copy) != {"FETCH_SIZE", "WRITE_SIZE"} or min(copy.values()) <= 0:
         return None
     total = 0.0
     for pattern in entry[1]:
         for ctr in ("FETCH_SIZE", "WRITE_SIZE"):
-            vals = [kib for name, c, kib in rows if c == ctr and re.search(pattern, name)]
-            if len(vals) != 1:
+            # a kernel launched with several grids (a first call that also packs, then the steady calls)
+            # has a line per grid: the one with the most dispatches is the steady call
+            vals = sorted((n, kib) for name, c, kib, n in rows if c == ctr and re.search(pattern, name))
+            if not vals or (len(vals) > 1 and vals[-1][0] == vals[-2][0]):
                 return None
-            total += vals[0] * (COPY_KIB / copy[ctr])
+            total += vals[-1][1] * (COPY_KIB / copy[ctr])
     return int(total * 1024)
 
 
