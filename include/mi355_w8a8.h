@@ -75,6 +75,7 @@ typedef enum mi355_w8a8_status {
 /* tile geometry of the tiled GEMM; default: 256 x 256 once such tiles fill half the CUs, else 256 x 128 */
 #define MI355_W8A8_FLAG_TILE_256X128 64u
 #define MI355_W8A8_FLAG_TILE_256X256 128u
+#define MI355_W8A8_FLAG_TILE_128X128 2048u
 /* tile rows of the grouped call (and the slots every group is padded to); default: 128 once the
  * groups average at least 96 rows, else 64.  Pass the same flags to the workspace query. */
 #define MI355_W8A8_FLAG_GROUPED_TILE64 256u
@@ -538,6 +539,7 @@ int mi355_w8a8_gq_linear_v1(const mi355_w8a8_gq_problem* problem, void* stream);
 #define MI355_W8A8_PATH_SKINNY_CHUNKS 2  /* 33..128 rows: the same two kernels per chunk of 32 rows */
 #define MI355_W8A8_PATH_TILED_256X128 3  /* prologue + 256 x 128 tiles, two workgroups per CU */
 #define MI355_W8A8_PATH_TILED_256X256 4  /* prologue + 256 x 256 tiles, one workgroup per CU */
+#define MI355_W8A8_PATH_TILED_128X128 5  /* prologue + 128 x 128 tiles, two workgroups per CU */
 int mi355_w8a8_forward_path(uint32_t m, uint32_t k, uint32_t n, uint32_t flags);
 
 /*

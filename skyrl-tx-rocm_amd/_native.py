@@ -24,8 +24,9 @@ FLAG_TILE_256X256 = 128
 FLAG_GROUPED_TILE64 = 256
 FLAG_GROUPED_TILE128 = 512
 FLAG_LORA_PACK_VALID = 1024
+FLAG_TILE_128X128 = 2048
 STATIC_WORKSPACE_BYTES = 32 << 20
-PATH_NAMES = {1: "skinny", 2: "skinny-chunks", 3: "tiled-256x128", 4: "tiled-256x256"}
+PATH_NAMES = {1: "skinny", 2: "skinny-chunks", 3: "tiled-256x128", 4: "tiled-256x256", 5: "tiled-128x128"}
 
 STATUS = {
     0: "OK", -1: "ERR_NULL", -2: "ERR_SHAPE", -3: "ERR_ALIGN", -4: "ERR_ALIAS",

@@ -64,12 +64,14 @@ inline uint32_t rank_chunks(uint32_t rank) { return rank == 0 ? 0u : (rank <= 16
 // Between the skinny-M limit and this many rows a call without SwiGLU may run the skinny-M kernels
 // on chunks of 32 rows: the weight is streamed once per chunk (the later passes from the last-level
 // cache), which beats the handful of 256-row tiles such a call would give the tiled kernel.
-// Measured on 2560 x 6144, 4096 x 2560, 12288 x 4096 and 4096 x 24576 weights: two chunks always
-// win while the weight stays in the caches (<= 64 MB), four chunks win from K = 4096 on.
+// Measured on 2560 x 6144, 4096 x 2560, 12288 x 4096 and 4096 x 24576 weights against the 128 x 128
+// tiles: two chunks always win while the weight stays in the caches (<= 64 MB), three from K = 4096
+// on (63 us against 77 at 4096 x 2560), four from K = 8192 on (116 against 139 at 12288 x 4096;
+// at 4096 x 2560 the tiles win, 76 us against 84).
 constexpr uint32_t kSkinnyChunkedMaxRows = 128;
 inline bool skinny_chunked_pays(uint32_t m, uint32_t k, uint32_t n) {
   if (m > kSkinnyChunkedMaxRows || (uint64_t)k_padded(k) * n_padded(n) > (64ull << 20)) return false;
-  return m <= 64u || k >= 4096u;
+  return m <= 64u || (k >= 4096u && (m <= 96u || k >= 8192u));
 }
 
 WsLayout make_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint32_t rank, bool routed) {
@@ -127,11 +129,13 @@ template <int EPI, int NKK, int MODE>
 int launch_gemm_one(const GemmArgs& g, hipStream_t s) {
   // persistent grid: one workgroup slot per CU (two in the 256 x 128 geometry), a multiple of 8
   const uint32_t ntile = g.tiles_m * g.tiles_n;
-  const uint32_t slots = MODE == kModeDense ? 512u : 256u;
+  const uint32_t slots = (MODE == kModeDense || MODE == kModeDense128) ? 512u : 256u;
   const uint32_t want = ((ntile + 7u) / 8u) * 8u;
   const dim3 grid(want < slots ? want : slots), block(MODE == kModeGrouped128 ? 512 : 256);
   constexpr uint32_t lds_bytes =
-      MODE == kModeGrouped128 ? kGrouped128LdsBytes : (MODE == kModeGrouped ? kGroupedLdsBytes : kGemmLdsBytes);
+      MODE == kModeGrouped128 ? kGrouped128LdsBytes
+                              : (MODE == kModeGrouped ? kGroupedLdsBytes
+                                                      : (MODE == kModeDense128 ? kGemmStages * kGemm128StageBytes : kGemmLdsBytes));
   if (hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm_kernel<EPI, NKK, MODE>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
     return MI355_W8A8_ERR_LAUNCH;
@@ -267,7 +271,8 @@ int choose_forward_path(uint32_t m, uint32_t k, uint32_t n, uint32_t flags) {
   if (!skinny_supported()) skinny = false;
   if (skinny) return MI355_W8A8_PATH_SKINNY;
   if (skinny_supported() && !swiglu && skinny_chunked_pays(m, k, n) &&
-      !(flags & (MI355_W8A8_FLAG_FORCE_TILED | MI355_W8A8_FLAG_TILE_256X128 | MI355_W8A8_FLAG_TILE_256X256)))
+      !(flags & (MI355_W8A8_FLAG_FORCE_TILED | MI355_W8A8_FLAG_TILE_256X128 | MI355_W8A8_FLAG_TILE_256X256 |
+                 MI355_W8A8_FLAG_TILE_128X128)))
     return MI355_W8A8_PATH_SKINNY_CHUNKS;
   // 256 x 256 tiles (one 8-wave workgroup per CU, 16 x 16 x 64 MFMAs) once they fill half the CUs;
   // below that the 256 x 128 geometry (two 4-wave workgroups per CU) has twice the tiles to spread.
@@ -277,6 +282,15 @@ int choose_forward_path(uint32_t m, uint32_t k, uint32_t n, uint32_t flags) {
   if (flags & MI355_W8A8_FLAG_TILE_256X128) wide = false;
   if (flags & MI355_W8A8_FLAG_TILE_256X256) wide = true;
   if (k_padded(k) < kG16MinKPad) wide = false;  // its stage schedule needs at least six 64-wide k steps
+  // 128 x 128 tiles (32 x 128 per wave) while all of them are resident at once (two workgroups per
+  // CU): a wave then carries half the MFMAs and half the epilogue of the 256 x 128 geometry and the
+  // call spreads over four times the CUs.  Measured (call, rank-64 adapters): K = 2560, N = 6144 at
+  // M = 512: 62 us against 84; K = 4096, N = 2560 at M = 2048: 88 against 105; beyond 512 tiles the
+  // larger geometries win (K = 2560, N = 6144 at M = 2048: 97 us against 85 on 256 x 256).
+  const bool small = (uint64_t)(round_up(m, (uint32_t)kGemm128TileM) / (uint32_t)kGemm128TileM) * (n_padded(n) / kGemmTileN) <= 512u;
+  const uint32_t forced = flags & (MI355_W8A8_FLAG_TILE_256X128 | MI355_W8A8_FLAG_TILE_256X256 | MI355_W8A8_FLAG_TILE_128X128);
+  if (forced & (forced - 1u)) return MI355_W8A8_ERR_SHAPE;  // two geometries asked for
+  if (forced == MI355_W8A8_FLAG_TILE_128X128 || (!forced && small)) return MI355_W8A8_PATH_TILED_128X128;
   return wide ? MI355_W8A8_PATH_TILED_256X256 : MI355_W8A8_PATH_TILED_256X128;
 }
 
@@ -457,15 +471,21 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   g.rank = lora ? p->rank : 0u;
   g.tile_ctr = reinterpret_cast<uint32_t*>(ws + w.tile_ctr);
   const bool wide = path == MI355_W8A8_PATH_TILED_256X256;
+  const bool small = path == MI355_W8A8_PATH_TILED_128X128;
   if (wide) g.tiles_n = n_padded(p->n) / kG16TileN;
+  if (small) g.tiles_m = round_up(p->m, (uint32_t)kGemm128TileM) / (uint32_t)kGemm128TileM;
   if (p->aux_acc) {
     GemmArgs ga = g;
     ga.out = p->aux_acc;
     ga.residual = nullptr;
-    if ((st = wide ? launch_gemm16_one<kEpiAcc, 0>(ga, s) : launch_gemm<kEpiAcc>(ga, 0u, s))) return st;
+    if ((st = wide ? launch_gemm16_one<kEpiAcc, 0>(ga, s)
+                   : (small ? launch_gemm<kEpiAcc, kModeDense128>(ga, 0u, s) : launch_gemm<kEpiAcc>(ga, 0u, s))))
+      return st;
     g.tile_ctr += 128;  // the second counter set
   }
   if (wide) return swiglu ? launch_gemm16<kEpiSwiglu>(g, w.nkk, s) : launch_gemm16<kEpiPlain>(g, w.nkk, s);
+  if (small)
+    return swiglu ? launch_gemm<kEpiSwiglu, kModeDense128>(g, w.nkk, s) : launch_gemm<kEpiPlain, kModeDense128>(g, w.nkk, s);
   return swiglu ? launch_gemm<kEpiSwiglu>(g, w.nkk, s) : launch_gemm<kEpiPlain>(g, w.nkk, s);
 }
 

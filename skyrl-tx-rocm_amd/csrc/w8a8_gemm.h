@@ -65,7 +65,11 @@ constexpr int kGrouped128StageBytes = 40960;  // A: 4 row blocks x 2 k blocks, B
 constexpr int kGrouped128LdsBytes = kGrouped128Stages * kGrouped128StageBytes;
 
 // (The 256 x 256 geometry for large problems is a kernel of its own: w8a8_gemm16.h.)
-enum { kModeDense = 0, kModeGrouped = 1, kModeGrouped128 = 2 };
+// Dense geometry for calls whose 256 x 128 tiles would leave most CUs idle: 128 x 128 tiles, the four
+// waves stacked along M with 32 x 128 each, so a wave carries half the MFMAs and half the epilogue.
+constexpr int kGemm128TileM = 128;
+constexpr int kGemm128StageBytes = 16384;  // A: 4 row blocks x 2 k blocks, B: 4 column blocks x 2 k blocks
+enum { kModeDense = 0, kModeGrouped = 1, kModeGrouped128 = 2, kModeDense128 = 3 };
 
 // One tile of the persistent loop.
 struct GemmTile {
@@ -77,15 +81,18 @@ struct GemmTile {
 };
 
 template <int EPI, int NKK, int MODE = kModeDense>
-__global__ __launch_bounds__(MODE == kModeGrouped128 ? 512 : 256, MODE == kModeDense ? 2 : 1)
+__global__ __launch_bounds__(MODE == kModeGrouped128 ? 512 : 256, (MODE == kModeDense || MODE == kModeDense128) ? 2 : 1)
 void w8a8_gemm_kernel(GemmArgs g) {
   constexpr bool G128 = MODE == kModeGrouped128;
+  constexpr bool D128 = MODE == kModeDense128;
   constexpr bool GROUPED = MODE == kModeGrouped || G128;
   constexpr int kWaves = G128 ? 8 : 4;
-  constexpr uint32_t kRowBlocks = G128 ? 4 : (GROUPED ? 2 : 8);    // 32-row blocks of the activation panel
+  constexpr int kWR = D128 ? 1 : 2;                                  // 32-row blocks of a wave's tile
+  constexpr uint32_t kRowBlocks = (G128 || D128) ? 4 : (GROUPED ? 2 : 8);  // 32-row blocks of the activation panel
   constexpr uint32_t kColBlocks = GROUPED ? 16 : 4;                 // 32-column blocks of the weight panel
   constexpr int kStages = G128 ? kGrouped128Stages : (GROUPED ? kGroupedStages : kGemmStages);
-  constexpr int kStageBytes = G128 ? kGrouped128StageBytes : (GROUPED ? kGroupedStageBytes : kGemmStageBytes);
+  constexpr int kStageBytes =
+      G128 ? kGrouped128StageBytes : (GROUPED ? kGroupedStageBytes : (D128 ? kGemm128StageBytes : kGemmStageBytes));
   constexpr int kAChunks = kRowBlocks * 2;                              // 1 KiB chunks of A per stage
   constexpr int kLoadsPerTile = (kAChunks + kColBlocks * 2) / kWaves;   // direct-to-LDS loads per wave per k-tile
   constexpr bool kLora = (NKK > 0) && (EPI != kEpiAcc);
@@ -94,7 +101,7 @@ void w8a8_gemm_kernel(GemmArgs g) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wrow = G128 ? (wave >> 2) : (GROUPED ? 0 : wave);  // wave position along M (64 rows each)
+  const int wrow = G128 ? (wave >> 2) : (GROUPED ? 0 : wave);  // wave position along M (32 * kWR rows each)
   const int wcol = G128 ? (wave & 3) : (GROUPED ? wave : 0);    // wave position along N (128 columns each)
   const int c = lane & 31, h = lane >> 5;
 
@@ -136,7 +143,7 @@ void w8a8_gemm_kernel(GemmArgs g) {
   // Dynamic schedule (two workgroups per CU): positions come from the XCD's counter, because the
   // hardware favours the older workgroup of a CU and a static split would leave the younger one
   // to finish alone.  The result does not depend on which workgroup computes which tile.
-  const bool dyn = MODE == kModeDense && g.tile_ctr != nullptr;
+  const bool dyn = !GROUPED && g.tile_ctr != nullptr;
   uint32_t* const ctr = g.tile_ctr + (blockIdx.x & 7u) * 16u;
   __shared__ uint32_t dyn_slot[2];
   uint32_t cur_i = blockIdx.x >> 3, nxt_i = 0;
@@ -159,12 +166,12 @@ void w8a8_gemm_kernel(GemmArgs g) {
       load_1k_to_lds(base + goff, St + ch * kBlockBytes);
     }
   };
-  auto read_frags = [&](int kt, int ks, v4i (&af)[2], v4i (&bf)[4]) {
+  auto read_frags = [&](int kt, int ks, v4i (&af)[kWR], v4i (&bf)[4]) {
     const unsigned char* As = lds + (kt % kStages) * kStageBytes;
     const unsigned char* Bs = As + kAChunks * kBlockBytes;
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
-      af[i] = *reinterpret_cast<const v4i*>(As + ((wrow * 2 + i) * 2 + ks) * kBlockBytes + lane * 16);
+    for (int i = 0; i < kWR; ++i)
+      af[i] = *reinterpret_cast<const v4i*>(As + ((wrow * kWR + i) * 2 + ks) * kBlockBytes + lane * 16);
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       bf[j] = *reinterpret_cast<const v4i*>(Bs + ((wcol * 4 + j) * 2 + ks) * kBlockBytes + lane * 16);
@@ -176,23 +183,23 @@ void w8a8_gemm_kernel(GemmArgs g) {
     nxt_i = cur_i + wgs_per_xcd;
     if (!T.valid) { prefetched = false; continue; }  // static schedules only (empty grouped tile, range end)
 
-    v16i acc[2][4];
+    v16i acc[kWR][4];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < kWR; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
-    auto mfma8 = [&](const v4i (&af)[2], const v4i (&bf)[4]) {
+    auto mfma8 = [&](const v4i (&af)[kWR], const v4i (&bf)[4]) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < kWR; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
     };
 
     // ---- main loop
-    v4i fa0[2], fb0[4], fa1[2], fb1[4];
+    v4i fa0[kWR], fb0[4], fa1[kWR], fb1[4];
     if (!prefetched) {
 #pragma unroll
       for (int st = 0; st < kStages - 1; ++st)
@@ -213,14 +220,24 @@ void w8a8_gemm_kernel(GemmArgs g) {
       read_frags(kt, 1, fa1, fb1);
       issue(T, kt + kStages - 1);
       mfma8(fa0, fb0);
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
-#pragma unroll
-      for (int q = 0; q < 6; ++q) {
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
-        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // 1 VMEM read
+      if constexpr (kWR == 2) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+#pragma unroll
+        for (int q = 0; q < 6; ++q) {
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
+          __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // 1 VMEM read
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      } else {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_barrier(0);
       // ---- k-step 1: k-tile kt+1 must have landed before its first fragments are fetched
       wait_vmcnt<(kStages - 2) * kLoadsPerTile>();
@@ -228,13 +245,22 @@ void w8a8_gemm_kernel(GemmArgs g) {
       __builtin_amdgcn_sched_barrier(0);
       read_frags(kt + 1, 0, fa0, fb0);
       mfma8(fa1, fb1);
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-#pragma unroll
-      for (int q = 0; q < 6; ++q) {
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      if constexpr (kWR == 2) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+#pragma unroll
+        for (int q = 0; q < 6; ++q) {
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      } else {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
     for (; kt < KT; ++kt) {  // drain: nothing left to prefetch
@@ -265,7 +291,7 @@ void w8a8_gemm_kernel(GemmArgs g) {
     // Lane (c = lane % 32, h = lane / 32) owns, in each of its wave's two 32 x 128 strips, the four
     // consecutive original columns ncol .. ncol+3 (accumulator blocks j = 0..3) of the 16 rows
     // 8*(v/4) + 4*h + v%4.
-    const uint32_t m0 = T.tm * (kRowBlocks * 32u) + wrow * 64u;
+    const uint32_t m0 = T.tm * (kRowBlocks * 32u) + wrow * (32u * kWR);
     const uint32_t tcol0 = T.tn * (kColBlocks * 32u) + wcol * 128u;  // first column of the wave
     const uint32_t ncol = tcol0 + 4u * c;
     const bool full_n = (tcol0 + 128u <= g.N) && ((g.N & 3u) == 0);  // wave-uniform
@@ -436,7 +462,7 @@ void w8a8_gemm_kernel(GemmArgs g) {
       }  // groups of the block
     };
     epilogue_block(std::integral_constant<int, 0>{});
-    epilogue_block(std::integral_constant<int, 1>{});
+    if constexpr (kWR == 2) epilogue_block(std::integral_constant<int, 1>{});
   }
 }
 

@@ -270,15 +270,41 @@ def test_tile_geometries_agree_bitwise(dev, pkg, shape):
     want = wc.oracle_forward(case, return_stages=True)
     narrow, aux_n = wc.gpu_forward(case, flags=pkg._native.FLAG_FORCE_TILED | pkg._native.FLAG_TILE_256X128)
     wide, aux_w = wc.gpu_forward(case, flags=pkg._native.FLAG_FORCE_TILED | pkg._native.FLAG_TILE_256X256)
-    for aux in (aux_n, aux_w):
+    small, aux_s = wc.gpu_forward(case, flags=pkg._native.FLAG_FORCE_TILED | pkg._native.FLAG_TILE_128X128)
+    for aux in (aux_n, aux_w, aux_s):
         assert np.array_equal(aux["acc"], want["acc"])
         assert np.array_equal(aux["x_codes"], want["x_codes"])
+    # the 128 x 128 geometry is the 256 x 128 kernel with one 32-row block per wave: the same operations per output
+    assert np.array_equal(narrow.view(np.uint32), small.view(np.uint32))
     if shape.get("n_adapters", 1) == 0:
         assert np.array_equal(narrow.view(np.uint32), wide.view(np.uint32))
     else:
         assert np.mean(narrow.view(np.uint32) == wide.view(np.uint32)) >= 0.999
     _assert_close(narrow, want["out"], f" narrow {m}x{k}x{n}")
     _assert_close(wide, want["out"], f" wide {m}x{k}x{n}")
+
+
+def test_tile_geometry_choice_and_contradictory_flags(dev, pkg):
+    """Which geometry a call takes depends on its dimensions and flags only; asking for two is refused."""
+    nat = pkg._native
+    path = lambda m, k, n, flags=0: nat.PATH_NAMES.get(nat.load().mi355_w8a8_forward_path(m, k, n, flags))
+    assert path(512, 2560, 6144) == "tiled-128x128"       # 4 x 48 tiles: all resident at once
+    assert path(2048, 2560, 6144) == "tiled-256x256"      # 768 small tiles would queue; 192 wide ones fill the CUs
+    assert path(4096, 4096, 24576) == "tiled-256x256"
+    assert path(4096, 256, 4096) == "tiled-256x128"       # too few k steps for the 256 x 256 schedule
+    assert path(16, 12288, 4096) == "skinny"
+    assert path(64, 4096, 2560) == "skinny-chunks"
+    assert path(128, 4096, 2560) == "tiled-128x128"
+    assert path(128, 12288, 4096) == "skinny-chunks"
+    assert path(512, 2560, 6144, nat.FLAG_TILE_256X128) == "tiled-256x128"
+    assert path(4096, 4096, 24576, nat.FLAG_TILE_128X128) == "tiled-128x128"
+    assert nat.load().mi355_w8a8_forward_path(512, 2560, 6144, nat.FLAG_TILE_256X128 | nat.FLAG_TILE_128X128) < 0
+    # a forced geometry on a large call is still exact (1024 tiles of 128 x 128 on 512 workgroup slots)
+    case = wc.make_case(1100, 512, 3000, n_adapters=3, rank=16, seed=41)
+    want = wc.oracle_forward(case, return_stages=True)
+    got, aux = wc.gpu_forward(case, flags=nat.FLAG_TILE_128X128)
+    assert np.array_equal(aux["acc"], want["acc"])
+    _assert_close(got, want["out"], " forced 128x128")
 
 
 def test_split2_flag_stays_in_tolerance(dev, pkg):
