@@ -72,7 +72,9 @@ typedef enum mi355_w8a8_status {
  * prologue results and answer these two flags with MI355_W8A8_ERR_UNSUPPORTED. */
 #define MI355_W8A8_FLAG_SKIP_PROLOGUE 16u /* do not run routing / quantization / LoRA-A */
 #define MI355_W8A8_FLAG_SKIP_GEMM 32u     /* run only routing / quantization / LoRA-A */
-/* tile geometry of the tiled GEMM; default: 256 x 256 once such tiles fill half the CUs, else 256 x 128 */
+/* tile geometry of the tiled GEMM (at most one of the three; two are refused with MI355_W8A8_ERR_SHAPE);
+ * default: 128 x 128 while at most 512 such tiles cover the output, else 256 x 256 (256 x 128 when k is
+ * too short for that kernel's stage schedule) */
 #define MI355_W8A8_FLAG_TILE_256X128 64u
 #define MI355_W8A8_FLAG_TILE_256X256 128u
 #define MI355_W8A8_FLAG_TILE_128X128 2048u
