@@ -56,6 +56,7 @@ inline uint64_t align256(uint64_t v) { return (v + 255u) & ~uint64_t(255); }
 struct WsLayout {
   uint64_t xq, sx, xn, zp, at, bp, src_row, dst_pos, slot_group, blk_range, tile_ctr, skinny, total;
   uint32_t slots, nkk, K_pad, KB, n_steps, steps_per_wave;
+  uint32_t rows_bound;  // the slots that can hold rows (a multiple of 32)
 };
 
 // number of 16-wide rank chunks the kernels are instantiated for (rank padded with zeros)
@@ -63,22 +64,39 @@ inline uint32_t rank_chunks(uint32_t rank) { return rank == 0 ? 0u : (rank <= 16
 
 // Between the skinny-M limit and this many rows a call without SwiGLU may run the skinny-M kernels
 // on chunks of 32 rows: the weight is streamed once per chunk (the later passes from the last-level
-// cache), which beats the handful of 256-row tiles such a call would give the tiled kernel.
-// Measured on 2560 x 6144, 4096 x 2560, 12288 x 4096 and 4096 x 24576 weights against the 128 x 128
-// tiles: two chunks always win while the weight stays in the caches (<= 64 MB), three from K = 4096
-// on (63 us against 77 at 4096 x 2560), four from K = 8192 on (116 against 139 at 12288 x 4096;
-// at 4096 x 2560 the tiles win, 76 us against 84).
+// cache).  A chunk costs 14-29 us, growing with the weight's bytes; the tiled call (128 x 128 tiles,
+// adapters on block boundaries) about 20 us + 7.5 us per 1024 of K whatever the rows.  Measured,
+// chunks against tiles: 4096 x 2560 at 64 rows 43 us / 57, at 96 rows 63 / 57; 12288 x 4096 at
+// 96 rows 88 / 113, at 128 rows 116 / 114; 2560 x 6144 at 33 rows 55 / 42; 1024 x 1024 at 33 rows 27 / 24.
 constexpr uint32_t kSkinnyChunkedMaxRows = 128;
 inline bool skinny_chunked_pays(uint32_t m, uint32_t k, uint32_t n) {
   if (m > kSkinnyChunkedMaxRows || (uint64_t)k_padded(k) * n_padded(n) > (64ull << 20)) return false;
-  return m <= 64u || (k >= 4096u && (m <= 96u || k >= 8192u));
+  if (k < 4096u) return false;
+  if (k >= 8192u) return m <= 96u;
+  return m <= 64u && n_padded(n) <= 4096u;
 }
 
-WsLayout make_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint32_t rank, bool routed) {
+// Grouped slots a call of m rows and n_groups adapters can need when every adapter's rows start on a
+// 32-slot block boundary (sum of the groups' sizes rounded up to 32).
+inline uint32_t padded_rows_bound(uint32_t m, uint32_t n_groups) {
+  return round_up(m + 31u * (n_groups < m ? n_groups : m), 32u);
+}
+// Whether a routed call may lay its groups out that way: the quantizer sorts the rows itself, and the
+// 128 x 128 tiles over the padded slots are still all resident at once (so the empty slots cost no time).
+inline bool padded_groups_fit(uint32_t m, uint32_t n, uint32_t n_groups) {
+  if (n_groups < 2u || m > kInlineRouteMaxRows) return false;
+  const uint64_t tiles = (uint64_t)(round_up(padded_rows_bound(m, n_groups), (uint32_t)kGemm128TileM) / (uint32_t)kGemm128TileM) *
+                         (n_padded(n) / kGemmTileN);
+  return tiles <= 512u;
+}
+
+WsLayout make_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint32_t rank, bool routed,
+                     bool pad_groups = false) {
   WsLayout w{};
   w.K_pad = k_padded(k);
   w.KB = w.K_pad / 32u;
-  w.slots = round_up(m, kTileM);
+  w.rows_bound = pad_groups ? padded_rows_bound(m, n_groups) : round_up(m, 32u);
+  w.slots = round_up(w.rows_bound, kTileM);
   (void)routed;
   w.nkk = rank_chunks(rank);
   w.n_steps = (k + 63u) / 64u;
@@ -338,7 +356,12 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   if (!p->workspace) return MI355_W8A8_ERR_WORKSPACE;
   if (p->workspace_bytes < need) return MI355_W8A8_ERR_WORKSPACE;
   if (reinterpret_cast<uintptr_t>(p->workspace) & 255u) return MI355_W8A8_ERR_ALIGN;
-  const WsLayout w = make_layout(p->m, p->k, p->n, p->n_adapters, lora ? p->rank : 0u, routed);
+  const int path = choose_forward_path(p->m, p->k, p->n, p->flags);
+  if (path < 0) return path;
+  // groups on block boundaries: only where the quantizer sorts the rows itself and the tiles stay resident
+  const bool pad_groups =
+      routed && path == MI355_W8A8_PATH_TILED_128X128 && padded_groups_fit(p->m, p->n, p->n_adapters);
+  const WsLayout w = make_layout(p->m, p->k, p->n, p->n_adapters, lora ? p->rank : 0u, routed, pad_groups);
   unsigned char* ws = static_cast<unsigned char*>(p->workspace);
   int32_t* src_row = reinterpret_cast<int32_t*>(ws + w.src_row);
   int32_t* dst_pos = reinterpret_cast<int32_t*>(ws + w.dst_pos);
@@ -347,8 +370,6 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
 
   (void)hipGetLastError();  // drop a stale error so it is not blamed on these launches
 
-  const int path = choose_forward_path(p->m, p->k, p->n, p->flags);
-  if (path < 0) return path;
   const bool skinny = path == MI355_W8A8_PATH_SKINNY;
   if (skinny) {
     return launch_skinny(p, ws + w.xq, reinterpret_cast<float*>(ws + w.sx),
@@ -411,7 +432,7 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   q.gamma = p->rms_gamma;
   q.eps = p->rms_eps;
   q.M = p->m; q.K = p->k; q.K_pad = w.K_pad; q.KB = w.KB;
-  q.n_half_blocks = round_up(p->m, 32u) / 16u;
+  q.n_half_blocks = w.rows_bound / 16u;
   q.src_row = routed ? src_row : nullptr;
   q.slot_group = routed ? slot_group : nullptr;
   q.blk_range = routed ? blk_range : nullptr;
@@ -427,6 +448,7 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   q.tile_ctr = reinterpret_cast<uint32_t*>(ws + w.tile_ctr);
   if (route_inline) {
     q.route_idx = p->adapter_indices; q.n_groups = p->n_adapters; q.slots = w.slots;
+    q.group_pad = pad_groups ? 32u : 1u;
     q.src_row = src_row; q.slot_group = slot_group; q.blk_range = blk_range;
   }
   if (!skip_prologue) {
@@ -464,7 +486,7 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   g.residual = static_cast<const uint16_t*>(p->residual);
   g.out = p->out;
   g.M = p->m; g.N = p->n; g.K_pad = w.K_pad; g.KB = w.KB; g.slots = w.slots;
-  g.total_rows = round_up(p->m, 32u);
+  g.total_rows = w.rows_bound;
   g.groups_per_weight = 1;
   g.tiles_m = w.slots / kTileM;
   g.tiles_n = n_padded(p->n) / kGemmTileN;
@@ -473,7 +495,7 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   const bool wide = path == MI355_W8A8_PATH_TILED_256X256;
   const bool small = path == MI355_W8A8_PATH_TILED_128X128;
   if (wide) g.tiles_n = n_padded(p->n) / kG16TileN;
-  if (small) g.tiles_m = round_up(p->m, (uint32_t)kGemm128TileM) / (uint32_t)kGemm128TileM;
+  if (small) g.tiles_m = round_up(w.rows_bound, (uint32_t)kGemm128TileM) / (uint32_t)kGemm128TileM;
   if (p->aux_acc) {
     GemmArgs ga = g;
     ga.out = p->aux_acc;
@@ -1787,7 +1809,8 @@ uint64_t mi355_w8a8_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t
   (void)flags;
   if (validate_common(m, k, n)) return 0;
   if (n_adapters > (uint32_t)kMaxAdapters || rank > (uint32_t)kMaxRank) return 0;
-  return make_layout(m, k, n, n_adapters, n_adapters ? rank : 0u, n_adapters > 1).total;
+  // (sized for groups on block boundaries wherever a call of these dimensions may lay them out so)
+  return make_layout(m, k, n, n_adapters, n_adapters ? rank : 0u, n_adapters > 1, padded_groups_fit(m, n, n_adapters)).total;
 }
 
 int mi355_w8a8_lora_linear_v1(const mi355_w8a8_problem* p, void* stream) {

@@ -625,6 +625,7 @@ struct QuantLoraArgs {
   // (then non-const outputs, read later by the GEMM) instead of reading them.
   const int32_t* route_idx; // adapter per row
   uint32_t n_groups, slots;
+  uint32_t group_pad;       // every group's first slot is a multiple of this (1: groups packed; 32: no block holds two groups)
 };
 
 constexpr uint32_t kInlineRouteMaxRows = 8192;  // eight rows per thread of a 1024-thread workgroup
@@ -633,11 +634,16 @@ constexpr uint32_t kInlineRouteMaxRows = 8192;  // eight rows per thread of a 10
 // workgroup itself: rows keep their order inside a group (slot start[g] + j holds the j-th row of group
 // g), which every workgroup derives alike from the adapter indices alone.  Returns through LDS:
 // out_src[16], out_grp[16], out_range (the group range of the 32-slot block that holds the slots).
+// With group_pad = 32 every group starts on a block boundary (the slots between a group's last row and
+// the next group's first stay empty, src -1), so no 32-slot block holds rows of two groups: neither
+// this kernel nor the GEMM's epilogue then runs a block once per group.  The slots in use end at
+// sum(round_up(count, group_pad)) <= M + (group_pad - 1) * min(n_groups, M).
 __device__ inline void route_rows_inline(const int32_t* __restrict__ idx, uint32_t M, uint32_t n_groups,
-                                         uint32_t slots, uint32_t hb, int* out_src, int* out_grp, uint32_t* out_range,
-                                         int* out_last_group) {
+                                         uint32_t slots, uint32_t group_pad, uint32_t hb, int* out_src, int* out_grp,
+                                         uint32_t* out_range, int* out_last_group) {
   __shared__ int cnt[kMaxAdapters];
   __shared__ int start[kMaxAdapters + 1];
+  __shared__ uint32_t used_end;  // first slot behind the last group
   __shared__ int wave_cnt[16];
   __shared__ int last_nonempty;
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
@@ -662,18 +668,20 @@ __device__ inline void route_rows_inline(const int32_t* __restrict__ idx, uint32
     int pos = 0, last = 0;
     for (uint32_t a = 0; a < n_groups; ++a) {
       start[a] = pos;
-      pos += cnt[a];
+      pos += (int)round_up((uint32_t)cnt[a], group_pad);
       if (cnt[a] > 0) last = (int)a;
     }
     start[n_groups] = pos;
+    used_end = (uint32_t)pos;
     last_nonempty = last;
     *out_last_group = last;
   }
   __syncthreads();
+  const uint32_t E = used_end;
   // group of a slot: the group whose [start, start + count) holds it; padding slots follow the last
   // non-empty group
   auto group_of = [&](uint32_t p) -> int {
-    if (p >= M) return last_nonempty;
+    if (p >= E) return last_nonempty;
     int g = 0;
     for (uint32_t a = 0; a < n_groups; ++a)
       if ((int)p >= start[a] && (int)p < start[a + 1]) g = (int)a;
@@ -683,12 +691,12 @@ __device__ inline void route_rows_inline(const int32_t* __restrict__ idx, uint32
   if (tid < 16u) out_grp[tid] = group_of(p0 + tid);
   if (tid == 16u) {
     const uint32_t b0 = (p0 / 32u) * 32u;
-    const uint32_t b1 = (b0 + 31u < M) ? b0 + 31u : (M ? M - 1u : 0u);
-    *out_range = b0 >= M ? 0u : ((uint32_t)group_of(b0) | ((uint32_t)group_of(b1) << 16));
+    const uint32_t b1 = (b0 + 31u < E) ? b0 + 31u : (E ? E - 1u : 0u);
+    *out_range = b0 >= E ? 0u : ((uint32_t)group_of(b0) | ((uint32_t)group_of(b1) << 16));
   }
   // the rows of the slots in use, group by group (a workgroup's 16 slots usually lie in one group)
-  const uint32_t p_end = (p0 + 16u < M) ? p0 + 16u : M;
-  if (p0 < M) {
+  const uint32_t p_end = (p0 + 16u < E) ? p0 + 16u : E;
+  if (p0 < E) {
     const int g_first = group_of(p0), g_last = group_of(p_end - 1u);
     for (int g = g_first; g <= g_last; ++g) {  // workgroup-uniform
       if (cnt[g] == 0) continue;
@@ -709,7 +717,7 @@ __device__ inline void route_rows_inline(const int32_t* __restrict__ idx, uint32
       for (uint32_t w = 0; w < wave; ++w) before += wave_cnt[w];
       // slots of group g among mine: ranks [lo, hi)
       const int lo = ((int)p0 > start[g] ? (int)p0 : start[g]) - start[g];
-      const int hi = ((int)p_end < start[g + 1] ? (int)p_end : start[g + 1]) - start[g];
+      const int hi = ((int)p_end < start[g] + cnt[g] ? (int)p_end : start[g] + cnt[g]) - start[g];
       int rank = before;
 #pragma unroll
       for (uint32_t j = 0; j < 8; ++j) {
@@ -740,7 +748,8 @@ __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
   __shared__ uint32_t route_range;
   const bool route_here = a.route_idx != nullptr;  // workgroup-uniform
   if (route_here) {
-    route_rows_inline(a.route_idx, a.M, a.n_groups, a.slots, hb, route_src, route_grp, &route_range, &route_last_group);
+    route_rows_inline(a.route_idx, a.M, a.n_groups, a.slots, a.group_pad, hb, route_src, route_grp, &route_range,
+                      &route_last_group);
     // the tables the GEMM reads later
     if (tid < 16u) {
       const_cast<int32_t*>(a.src_row)[hb * 16u + tid] = route_src[tid];
@@ -753,6 +762,12 @@ __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
         const_cast<int32_t*>(a.slot_group)[p] = route_last_group;
         if ((p & 31u) == 0) const_cast<int32_t*>(a.blk_range)[p / 32u] = 0;
       }
+    }
+    if (a.group_pad > 1u) {  // padded groups leave whole half blocks empty: nothing reads their codes, scales or z
+      int any = 0;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) any |= (route_src[j] >= 0) ? 1 : 0;
+      if (!any) return;  // workgroup-uniform
     }
   }
 

@@ -90,9 +90,9 @@ def test_validation_errors_without_a_gpu(native):
     assert call(_problem(native, adapter_indices=0x500000)) == -2        # indices without LoRA
     assert call(_problem(native, flags=native.FLAG_SWIGLU, n=31)) == -2
     assert call(_problem(native, flags=native.FLAG_FORCE_TILED | native.FLAG_FORCE_SKINNY)) == -2
-    # 33..128 rows on a cache-resident weight run as 32-row chunks, which keep no stage to rerun
-    assert call(_problem(native, m=64, flags=native.FLAG_SKIP_PROLOGUE)) == -7
-    assert call(_problem(native, m=40, flags=native.FLAG_SKIP_GEMM)) == -7
+    # 33..64 rows over a long K on a cache-resident weight run as 32-row chunks, which keep no stage to rerun
+    assert call(_problem(native, m=64, k=4096, flags=native.FLAG_SKIP_PROLOGUE)) == -7
+    assert call(_problem(native, m=40, k=4096, flags=native.FLAG_SKIP_GEMM)) == -7
     # entry points insist on their own stage combination
     assert call(_problem(native), lib.mi355_w8a8_rms_gateup_swiglu_v1) == -2
     assert call(_problem(native), lib.mi355_w8a8_lora_residual_v1) == -2

@@ -61,7 +61,8 @@ def _replays(torch, run, outputs, refresh, n=4):
 FORWARD_CASES = [
     # m, k, n, adapters, rank, rms, swiglu, residual
     (16, 1024, 768, 4, 16, False, False, True),      # two-kernel streaming path
-    (96, 4096, 1024, 2, 16, True, False, False),     # 32-row chunks of the streaming path
+    (64, 4096, 1024, 2, 16, True, False, False),     # 32-row chunks of the streaming path
+    (96, 4096, 1024, 2, 16, True, False, False),     # 128 x 128 tiles, adapters on block boundaries
     (300, 512, 1024, 3, 32, True, True, False),      # tiled kernel with a persistent schedule
     (1100, 768, 2304, 8, 16, False, False, False),   # several row tiles, per-XCD tile counters
 ]

@@ -203,13 +203,15 @@ def test_skinny_path_shapes(dev, pkg, m, k, n, n_ad, rank, rms):
     _assert_close(tiled, st["out"], f" tiled {m}x{k}x{n}")
 
 
-@pytest.mark.parametrize("m,k,n,n_ad,rank,rms", [(33, 512, 264, 3, 16, True), (47, 1024, 520, 2, 40, False),
-                                                 (64, 2560, 1024, 0, 0, True), (100, 4096, 512, 5, 8, True),
-                                                 (128, 4096, 776, 4, 64, False)])
+@pytest.mark.parametrize("m,k,n,n_ad,rank,rms", [(33, 4096, 264, 3, 16, True), (47, 4096, 520, 2, 40, False),
+                                                 (64, 4096, 1024, 0, 0, True), (96, 8192, 512, 5, 8, True),
+                                                 (81, 12288, 776, 4, 64, False)])
 def test_chunked_skinny_path(dev, pkg, m, k, n, n_ad, rank, rms):
-    """Between 33 and 128 rows a call without SwiGLU whose weight fits the caches runs the streaming
+    """Between 33 and 96 rows a call without SwiGLU over a long K whose weight fits the caches runs the streaming
     kernels on 32-row chunks: every stage against the oracle, ragged last chunks, and the tiled kernel on
     the same case (integer stages bit-equal between the two paths)."""
+    nat = pkg._native
+    assert nat.PATH_NAMES[nat.load().mi355_w8a8_forward_path(m, k, n, 0)] == "skinny-chunks"
     case = wc.make_case(m, k, n, n_adapters=n_ad, rank=max(rank, 1), seed=3 * m + k, rms=rms, residual=(m % 2 == 1))
     st = wc.oracle_forward(case, return_stages=True)
     got, aux = wc.gpu_forward(case)
@@ -295,7 +297,9 @@ def test_tile_geometry_choice_and_contradictory_flags(dev, pkg):
     assert path(16, 12288, 4096) == "skinny"
     assert path(64, 4096, 2560) == "skinny-chunks"
     assert path(128, 4096, 2560) == "tiled-128x128"
-    assert path(128, 12288, 4096) == "skinny-chunks"
+    assert path(96, 12288, 4096) == "skinny-chunks"
+    assert path(128, 12288, 4096) == "tiled-128x128"
+    assert path(64, 2560, 6144) == "tiled-128x128"
     assert path(512, 2560, 6144, nat.FLAG_TILE_256X128) == "tiled-256x128"
     assert path(4096, 4096, 24576, nat.FLAG_TILE_128X128) == "tiled-128x128"
     assert nat.load().mi355_w8a8_forward_path(512, 2560, 6144, nat.FLAG_TILE_256X128 | nat.FLAG_TILE_128X128) < 0
