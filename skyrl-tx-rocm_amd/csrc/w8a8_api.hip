@@ -82,12 +82,14 @@ inline uint32_t padded_rows_bound(uint32_t m, uint32_t n_groups) {
   return round_up(m + 31u * (n_groups < m ? n_groups : m), 32u);
 }
 // Whether a routed call may lay its groups out that way: the quantizer sorts the rows itself, and the
-// 128 x 128 tiles over the padded slots are still all resident at once (so the empty slots cost no time).
-inline bool padded_groups_fit(uint32_t m, uint32_t n, uint32_t n_groups) {
+// tiles over the padded slots are still all resident at once (so the empty slots cost no time): 512
+// tiles of 128 x 128, or 256 of 256 x 256.
+inline bool padded_groups_fit(uint32_t m, uint32_t n, uint32_t n_groups, bool wide_tiles = false) {
   if (n_groups < 2u || m > kInlineRouteMaxRows) return false;
-  const uint64_t tiles = (uint64_t)(round_up(padded_rows_bound(m, n_groups), (uint32_t)kGemm128TileM) / (uint32_t)kGemm128TileM) *
-                         (n_padded(n) / kGemmTileN);
-  return tiles <= 512u;
+  const uint32_t rows = padded_rows_bound(m, n_groups);
+  if (rows > 4096u) return false;  // the quantizer's workgroups (16 slots each) must not outnumber the CUs either
+  if (wide_tiles) return (uint64_t)(round_up(rows, kTileM) / kTileM) * (n_padded(n) / kG16TileN) <= 256u;
+  return (uint64_t)(round_up(rows, (uint32_t)kGemm128TileM) / (uint32_t)kGemm128TileM) * (n_padded(n) / kGemmTileN) <= 512u;
 }
 
 WsLayout make_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint32_t rank, bool routed,
@@ -360,7 +362,8 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   if (path < 0) return path;
   // groups on block boundaries: only where the quantizer sorts the rows itself and the tiles stay resident
   const bool pad_groups =
-      routed && path == MI355_W8A8_PATH_TILED_128X128 && padded_groups_fit(p->m, p->n, p->n_adapters);
+      routed && ((path == MI355_W8A8_PATH_TILED_128X128 && padded_groups_fit(p->m, p->n, p->n_adapters)) ||
+                 (path == MI355_W8A8_PATH_TILED_256X256 && padded_groups_fit(p->m, p->n, p->n_adapters, true)));
   const WsLayout w = make_layout(p->m, p->k, p->n, p->n_adapters, lora ? p->rank : 0u, routed, pad_groups);
   unsigned char* ws = static_cast<unsigned char*>(p->workspace);
   int32_t* src_row = reinterpret_cast<int32_t*>(ws + w.src_row);
@@ -1810,7 +1813,8 @@ uint64_t mi355_w8a8_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t
   if (validate_common(m, k, n)) return 0;
   if (n_adapters > (uint32_t)kMaxAdapters || rank > (uint32_t)kMaxRank) return 0;
   // (sized for groups on block boundaries wherever a call of these dimensions may lay them out so)
-  return make_layout(m, k, n, n_adapters, n_adapters ? rank : 0u, n_adapters > 1, padded_groups_fit(m, n, n_adapters)).total;
+  return make_layout(m, k, n, n_adapters, n_adapters ? rank : 0u, n_adapters > 1,
+                     padded_groups_fit(m, n, n_adapters) || padded_groups_fit(m, n, n_adapters, true)).total;
 }
 
 int mi355_w8a8_lora_linear_v1(const mi355_w8a8_problem* p, void* stream) {
