@@ -115,7 +115,7 @@ WsLayout make_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint
   w.xn = off;
   off += (rank && m <= kSkinnyChunkedMaxRows) ? align256((uint64_t)(m < 32u ? m : 32u) * k * 2u) : 0u;
   w.zp = off; off += rank ? align256((uint64_t)(w.slots / 32u) * w.nkk * 3u * kBlockBytes) : 0u;
-  w.at = off; off += rank ? align256((uint64_t)n_groups * rank * k * 2u) : 0u;
+  w.at = off; off += rank ? align256((uint64_t)n_groups * w.KB * w.nkk * kBlockBytes) : 0u;  // A in operand order
   w.bp = off; off += rank ? align256((uint64_t)n_groups * (n_padded(n) / 32u) * w.nkk * kBlockBytes) : 0u;
   w.skinny = off; off += align256(skinny_workspace_bytes(m, n, rank));
   w.total = off;
@@ -418,7 +418,8 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
     pa.M = p->m; pa.K = p->k; pa.N = p->n; pa.n_groups = p->n_adapters; pa.r = p->rank; pa.nkk = w.nkk;
     pa.ncb = n_padded(p->n) / 32u; pa.slots = w.slots;
     pa.route_blocks = (routed && !route_inline) ? 1u : 0u;
-    const uint64_t a_items = (uint64_t)p->n_adapters * p->k * ((p->rank + 7u) / 8u);
+    pa.a_operand_kb = w.KB;  // the quantizer reads A in MFMA operand order
+    const uint64_t a_items = (uint64_t)p->n_adapters * w.KB * w.nkk * 64u;
     const uint64_t b_items = (uint64_t)p->n_adapters * pa.ncb * w.nkk * 64u;
     const bool pack = !(p->flags & MI355_W8A8_FLAG_LORA_PACK_VALID);  // else the workspace holds both already
     pa.a_blocks = pack ? (uint32_t)((a_items + 1023u) / 1024u) : 0u;

@@ -388,6 +388,36 @@ __device__ inline void lora_b_pack_item(const uint16_t* __restrict__ b, unsigned
   *reinterpret_cast<v8us*>(bp + idx * 16u) = o;
 }
 
+// ---------------------------------------------------------------------------------------
+// LoRA A re-layout for the dense path's quantizer: A [n, K, r] -> the B-operand order of
+// v_mfma_f32_16x16x32_bf16, ap[n][K_pad/32][nkk][64 lanes][8]: lane (i = l % 16, q = l / 16) of
+// k-block kb and rank block b holds k = 32 kb + 8 q + 0..7 (zero beyond K) of rank column
+// 16 b + i (zero beyond the rank).  A wave's operand load is then 1 KiB of consecutive memory
+// (eight cache lines) where the transposed layout gives it sixteen half-used lines, and the
+// quantizer's LoRA-A step is bound by the cache lines its loads touch.
+// ---------------------------------------------------------------------------------------
+__device__ inline void lora_a_pack_item(const uint16_t* __restrict__ a, unsigned char* __restrict__ ap,
+                                        uint32_t n_groups, uint32_t K, uint32_t r, uint32_t KB, uint32_t nkk,
+                                        uint64_t idx) {
+  const uint64_t total = (uint64_t)n_groups * KB * nkk * 64u;  // one 16-byte operand per thread
+  if (idx >= total) return;
+  const uint32_t l = (uint32_t)(idx & 63u);
+  const uint64_t rest = idx >> 6;
+  const uint32_t b = (uint32_t)(rest % nkk);
+  const uint64_t gk = rest / nkk;
+  const uint32_t kb = (uint32_t)(gk % KB), grp = (uint32_t)(gk / KB);
+  const uint32_t col = 16u * b + (l & 15u);
+  v8us o = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (col < r) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint32_t k = 32u * kb + 8u * (l >> 4) + e;
+      if (k < K) o[e] = a[((size_t)grp * K + k) * r + col];
+    }
+  }
+  *reinterpret_cast<v8us*>(ap + idx * 16u) = o;
+}
+
 // Clears `count` 32-bit words (one workgroup).
 __global__ __launch_bounds__(256) void zero_words_kernel(uint32_t* p, uint32_t count) {
   for (uint32_t i = threadIdx.x; i < count; i += 256u) p[i] = 0u;
@@ -405,6 +435,7 @@ struct LoraPrepArgs {
   uint16_t* at;              // bf16 [n_groups, r, K]
   unsigned char* bp;         // packed B operands
   uint32_t M, K, N, n_groups, r, nkk, ncb, slots, route_blocks, a_blocks;
+  uint32_t a_operand_kb;     // 0: `at` is the transposed A; else K_pad / 32 and `at` takes A in MFMA operand order
   // grouped (ragged) call: the routing block lays the groups out from their sizes instead
   const int32_t* group_sizes;  // int32 [n_groups] or null
   uint32_t group_pad;          // slots every group is padded to
@@ -424,7 +455,11 @@ __global__ __launch_bounds__(1024) void lora_prep_kernel(LoraPrepArgs p) {
   }
   b -= p.route_blocks;
   if (b < p.a_blocks) {
-    lora_a_transpose_item(p.lora_a, p.at, p.n_groups, p.K, p.r, (uint64_t)b * 1024u + threadIdx.x);
+    if (p.a_operand_kb)
+      lora_a_pack_item(p.lora_a, reinterpret_cast<unsigned char*>(p.at), p.n_groups, p.K, p.r, p.a_operand_kb, p.nkk,
+                       (uint64_t)b * 1024u + threadIdx.x);
+    else
+      lora_a_transpose_item(p.lora_a, p.at, p.n_groups, p.K, p.r, (uint64_t)b * 1024u + threadIdx.x);
     return;
   }
   b -= p.a_blocks;
@@ -616,7 +651,7 @@ struct QuantLoraArgs {
   int8_t* codes_rm;         // row-major codes [M, K] or null
   float* scales_rm;         // f32 [M] or null
   uint16_t* xn_aux;         // bf16 [M, K] normalized rows for the caller, or null
-  const uint16_t* at;       // bf16 [n_groups, r, K] or null (CB == 0)
+  const uint16_t* at;       // LoRA A in MFMA operand order [n_groups][KB][CB][64 lanes][8 bf16] (lora_a_pack_item) or null (CB == 0)
   unsigned char* zp;        // packed z fragments
   uint32_t r, nkk, nterms;
   uint32_t* tile_ctr;       // 256 words cleared for the GEMM launches' tile counters, or null
@@ -881,12 +916,10 @@ __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
         gm[u][1] = inK ? *reinterpret_cast<const float4*>(a.gamma + k0 + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
       }
       if constexpr (CB > 0) {
-        const uint16_t* atg = a.at + (size_t)glo * a.r * a.K + k0;
+        // operands of group glo, k-block kb: CB consecutive 1 KiB pieces (zero beyond K and the rank)
+        const v4i* ap = reinterpret_cast<const v4i*>(a.at) + (((size_t)glo * a.KB + kb) * CB) * 64u + lane;
 #pragma unroll
-        for (int b = 0; b < CB; ++b) {
-          const uint32_t col = b * 16u + i;
-          wpre[u][b] = (inK && col < a.r) ? *reinterpret_cast<const v4i*>(atg + (size_t)col * a.K) : v4i{0, 0, 0, 0};
-        }
+        for (int b = 0; b < CB; ++b) wpre[u][b] = kb < a.KB ? ap[b * 64] : v4i{0, 0, 0, 0};
       }
     }
 #pragma unroll
@@ -949,14 +982,11 @@ __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
         for (uint32_t grp = glo; grp <= ghi; ++grp) {
           v4i xa = {0, 0, 0, 0};
           if (live && rowgrp == grp) xa = v4i{(int)nb[0], (int)nb[1], (int)nb[2], (int)nb[3]};
-          const uint16_t* atg = a.at + (size_t)grp * a.r * a.K + k0;
+          const v4i* ap = reinterpret_cast<const v4i*>(a.at) + (((size_t)grp * a.KB + kb) * CB) * 64u + lane;
 #pragma unroll
           for (int b = 0; b < CB; ++b) {
             v4i wb = wpre[u][b];
-            if (grp != glo) {  // wave-uniform, boundary blocks only
-              const uint32_t col = b * 16u + i;
-              wb = (col < a.r && k0 < a.K) ? *reinterpret_cast<const v4i*>(atg + (size_t)col * a.K) : v4i{0, 0, 0, 0};
-            }
+            if (grp != glo) wb = ap[b * 64];  // wave-uniform, boundary blocks only
             acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, xa),
                                                              __builtin_bit_cast(v8bf, wb), acc[b], 0, 0, 0);
           }
