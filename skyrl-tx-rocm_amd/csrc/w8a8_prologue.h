@@ -952,13 +952,14 @@ __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
       // integer unless the product lies that close to a tie; those cases (and scales outside the
       // reciprocal's safe range) are redone with the division.
       float c[8];
-      bool redo = !(scale > 1e-30f && scale < 1e30f);
+      float off_integer = 0.0f;  // largest distance of a quotient from its rounded value
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const float t = v[e] * rscale;
         c[e] = rintf(t);
-        redo = redo || (fabsf(t - c[e]) > 0.4999f);
+        off_integer = fmaxf(off_integer, fabsf(t - c[e]));
       }
+      const bool redo = !(scale > 1e-30f && scale < 1e30f) || off_integer > 0.4999f;
       if (__builtin_amdgcn_ballot_w64(redo) != 0) {  // wave-uniform
 #pragma unroll
         for (int e = 0; e < 8; ++e) c[e] = rintf(v[e] / scale);
