@@ -1569,7 +1569,10 @@ GqLayout make_gq_layout(uint32_t m, uint32_t k_pad, uint32_t group, uint32_t n_a
   L.dst_pos = off; off += rank ? align256((uint64_t)L.m_pad * 4u) : 0u;
   L.slot_group = off; off += rank ? align256((uint64_t)L.m_pad * 4u) : 0u;
   L.blk_range = off; off += rank ? align256((uint64_t)(L.m_pad / 32u) * 4u) : 0u;
-  L.at = off; off += (rank && n_adapters <= (uint32_t)kMaxAdapters) ? align256((uint64_t)n_adapters * rank * k_pad * 2u) : 0u;
+  // LoRA A in lora_a_kernel's operand order: per adapter and 64-wide k step 4 KiB per 32 rank columns
+  L.at = off; off += (rank && n_adapters <= (uint32_t)kMaxAdapters)
+                         ? align256((uint64_t)n_adapters * ((k_pad + 63u) / 64u) * (rank_chunks(rank) > 2u ? 2u : 1u) * 4u * kBlockBytes)
+                         : 0u;
   L.total = off;
   return L;
 }
@@ -1665,13 +1668,15 @@ int run_gq_linear(const mi355_w8a8_gq_problem* p, hipStream_t s) {
     pa.M = p->m; pa.K = p->k; pa.N = p->n; pa.n_groups = p->n_adapters; pa.r = p->rank;
     pa.slots = L.m_pad;
     pa.route_blocks = routed ? 1u : 0u;
-    const uint64_t a_items = (uint64_t)p->n_adapters * p->k * ((p->rank + 7u) / 8u);
+    pa.a_operand_steps = (p->k + 63u) / 64u; pa.a_operand_rb = rank_chunks(p->rank) > 2u ? 2u : 1u;  // lora_a_kernel's operand order
+    const uint64_t a_items = (uint64_t)p->n_adapters * pa.a_operand_steps * pa.a_operand_rb * 256u;
     pa.a_blocks = (uint32_t)((a_items + 1023u) / 1024u);
     hipLaunchKernelGGL(lora_prep_kernel, dim3(pa.route_blocks + pa.a_blocks), dim3(1024), 0, s, pa);
     if ((st = launch_status())) return st;
     LoraAArgs la{};
     la.xsrc = q.x;
     la.at = at;
+    la.at_operand = 1u;
     la.src_row = routed ? src_row : nullptr;
     la.slot_group = routed ? slot_group : nullptr;
     la.blk_range = routed ? blk_range : nullptr;

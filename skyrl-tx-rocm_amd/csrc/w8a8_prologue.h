@@ -418,6 +418,33 @@ __device__ inline void lora_a_pack_item(const uint16_t* __restrict__ a, unsigned
   *reinterpret_cast<v8us*>(ap + idx * 16u) = o;
 }
 
+// The same for lora_a_kernel (v_mfma_f32_32x32x16_bf16, 64-wide k steps), whose operand loads of the
+// transposed A touch 32 cache lines each:
+// ap[n][ceil(K / 64)][RB][4][64 lanes][8]: lane (i = l % 32, h = l / 32) of k step s, rank block b and
+// quarter t holds k = 64 s + 32 h + 8 t + 0..7 of rank column 32 b + i.  Pays with few adapters of many
+// rows each; with 128 experts of rank 16 (padded to 32 columns, packed per call) it measured slower.
+__device__ inline void lora_a_pack32_item(const uint16_t* __restrict__ a, unsigned char* __restrict__ ap,
+                                          uint32_t n_groups, uint32_t K, uint32_t r, uint32_t n_steps, uint32_t rb,
+                                          uint64_t idx) {
+  const uint64_t total = (uint64_t)n_groups * n_steps * rb * 256u;  // one 16-byte operand per thread
+  if (idx >= total) return;
+  const uint32_t l = (uint32_t)(idx & 63u), t = (uint32_t)(idx >> 6) & 3u;
+  const uint64_t rest = idx >> 8;
+  const uint32_t b = (uint32_t)(rest % rb);
+  const uint64_t gs = rest / rb;
+  const uint32_t st = (uint32_t)(gs % n_steps), grp = (uint32_t)(gs / n_steps);
+  const uint32_t col = 32u * b + (l & 31u);
+  v8us o = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (col < r) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint32_t k = 64u * st + 32u * (l >> 5) + 8u * t + e;
+      if (k < K) o[e] = a[((size_t)grp * K + k) * r + col];
+    }
+  }
+  *reinterpret_cast<v8us*>(ap + idx * 16u) = o;
+}
+
 // Clears `count` 32-bit words (one workgroup).
 __global__ __launch_bounds__(256) void zero_words_kernel(uint32_t* p, uint32_t count) {
   for (uint32_t i = threadIdx.x; i < count; i += 256u) p[i] = 0u;
@@ -436,6 +463,7 @@ struct LoraPrepArgs {
   unsigned char* bp;         // packed B operands
   uint32_t M, K, N, n_groups, r, nkk, ncb, slots, route_blocks, a_blocks;
   uint32_t a_operand_kb;     // 0: `at` is the transposed A; else K_pad / 32 and `at` takes A in MFMA operand order
+  uint32_t a_operand_steps, a_operand_rb;  // or: ceil(K / 64) and the 32-wide rank blocks of lora_a_kernel's operand order
   // grouped (ragged) call: the routing block lays the groups out from their sizes instead
   const int32_t* group_sizes;  // int32 [n_groups] or null
   uint32_t group_pad;          // slots every group is padded to
@@ -455,7 +483,10 @@ __global__ __launch_bounds__(1024) void lora_prep_kernel(LoraPrepArgs p) {
   }
   b -= p.route_blocks;
   if (b < p.a_blocks) {
-    if (p.a_operand_kb)
+    if (p.a_operand_steps)
+      lora_a_pack32_item(p.lora_a, reinterpret_cast<unsigned char*>(p.at), p.n_groups, p.K, p.r, p.a_operand_steps,
+                         p.a_operand_rb, (uint64_t)b * 1024u + threadIdx.x);
+    else if (p.a_operand_kb)
       lora_a_pack_item(p.lora_a, reinterpret_cast<unsigned char*>(p.at), p.n_groups, p.K, p.r, p.a_operand_kb, p.nkk,
                        (uint64_t)b * 1024u + threadIdx.x);
     else
@@ -477,7 +508,8 @@ __global__ __launch_bounds__(1024) void lora_prep_kernel(LoraPrepArgs p) {
 // ---------------------------------------------------------------------------------------
 struct LoraAArgs {
   const uint16_t* xsrc;     // bf16 [M, K] (x, or the normalized rows)
-  const uint16_t* at;       // bf16 [n_groups, r, K]
+  const uint16_t* at;       // bf16 [n_groups, r, K], or A in operand order (lora_a_pack32_item) when at_operand is set
+  uint32_t at_operand;      // 0 or 1
   const int32_t* src_row;   // or null (identity)
   const int32_t* slot_group;// or null (group 0)
   const int32_t* blk_range; // or null
@@ -544,7 +576,12 @@ __global__ __launch_bounds__(1024) void lora_a_kernel(LoraAArgs a) {
 #pragma unroll
           for (int b = 0; b < RB; ++b) {
             const uint32_t col = b * 32u + i;
-            wb[u][b][t] = (col < a.r && ok) ? *reinterpret_cast<const v8us*>(atg + (size_t)col * a.K + k0) : zero;
+            if (a.at_operand)  // kernel-uniform: 1 KiB of consecutive memory per wave and load (zero beyond K and the rank)
+              wb[u][b][t] = step_ok ? *(reinterpret_cast<const v8us*>(a.at) +
+                                        ((((size_t)grp * a.n_steps + (s + u)) * RB + b) * 4u + t) * 64u + lane)
+                                    : zero;
+            else
+              wb[u][b][t] = (col < a.r && ok) ? *reinterpret_cast<const v8us*>(atg + (size_t)col * a.K + k0) : zero;
           }
         }
       }
