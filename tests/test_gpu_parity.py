@@ -311,6 +311,40 @@ def test_tile_geometry_choice_and_contradictory_flags(dev, pkg):
     _assert_close(got, want["out"], " forced 128x128")
 
 
+@pytest.mark.parametrize("seed", [1, 7])
+def test_randomized_forward_sweep(dev, pkg, seed):
+    """Sixty seeded draws over rows (1..1000), K, N, adapter counts (0..64, some without rows), ranks, RMSNorm,
+    SwiGLU, residual and forced tile geometries: integer stages bit-equal to the oracle, outputs inside the
+    tolerance.  Covers the path switches (decode kernels, 32-row chunks, the three tile geometries, adapters
+    packed or on block boundaries) on shapes nobody picked by hand."""
+    nat = pkg._native
+    rng = np.random.default_rng(seed)
+    for it in range(60):
+        m = int(rng.choice([1, 5, 17, 33, 40, 64, 65, 96, 100, 129, 200, 257, 300, 511, 513, 640, 1000]))
+        k = int(rng.choice([64, 136, 256, 392, 512, 768, 1024, 1536, 2048]))
+        n = int(rng.choice([32, 96, 130, 256, 264, 520, 776, 1024, 1500]))
+        n_ad = int(rng.choice([0, 1, 2, 3, 5, 8, 13, 32, 64]))
+        rank = int(rng.choice([1, 3, 8, 16, 24, 32, 40, 64]))
+        rms = bool(rng.integers(0, 2))
+        swiglu = bool(rng.integers(0, 2)) and n % 2 == 0
+        residual = (not swiglu) and bool(rng.integers(0, 2))
+        idx_mode = str(rng.choice(["uniform", "arange", "zero"]))
+        flags = int(rng.choice([0, 0, 0, nat.FLAG_FORCE_TILED, nat.FLAG_TILE_128X128,
+                                nat.FLAG_FORCE_TILED | nat.FLAG_TILE_256X128, nat.FLAG_FORCE_TILED | nat.FLAG_TILE_256X256]))
+        if (flags & nat.FLAG_TILE_256X256) and k < 384:
+            flags = nat.FLAG_FORCE_TILED
+        what = f" m={m} k={k} n={n} adapters={n_ad} rank={rank} rms={rms} swiglu={swiglu} residual={residual} {idx_mode} flags={flags}"
+        case = wc.make_case(m, k, n, n_adapters=n_ad, rank=rank, seed=1000 * seed + it, rms=rms, swiglu=swiglu,
+                            residual=residual, idx_mode=idx_mode)
+        if n_ad and idx_mode == "uniform" and rng.integers(0, 2):
+            case["idx"] = (case["idx"] // 2 * 2 % n_ad).astype(np.int32)  # adapters without rows
+        st = wc.oracle_forward(case, return_stages=True)
+        got, aux = wc.gpu_forward(case, flags=flags)
+        assert np.array_equal(aux["x_codes"], st["x_codes"]), what
+        assert np.array_equal(aux["acc"], st["acc"]), what
+        _assert_close(got, st["out"], what)
+
+
 def test_split2_flag_stays_in_tolerance(dev, pkg):
     case = wc.make_case(256, 512, 512, n_adapters=2, rank=32, seed=15)
     want = wc.oracle_forward(case)
