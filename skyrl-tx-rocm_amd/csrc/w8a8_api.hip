@@ -82,14 +82,19 @@ inline uint32_t padded_rows_bound(uint32_t m, uint32_t n_groups) {
   return round_up(m + 31u * (n_groups < m ? n_groups : m), 32u);
 }
 // Whether a routed call may lay its groups out that way: the quantizer sorts the rows itself, and the
-// tiles over the padded slots are still all resident at once (so the empty slots cost no time): 512
-// tiles of 128 x 128, or 256 of 256 x 256.
+// empty slots cost no time -- neither the quantizer's workgroups (16 slots each, one resident per CU) nor
+// the GEMM's tiles (512 resident tiles of 128 x 128, 256 of 256 x 256) need another round on the chip
+// than the packed layout does.
 inline bool padded_groups_fit(uint32_t m, uint32_t n, uint32_t n_groups, bool wide_tiles = false) {
   if (n_groups < 2u || m > kInlineRouteMaxRows) return false;
-  const uint32_t rows = padded_rows_bound(m, n_groups);
-  if (rows > 4096u) return false;  // the quantizer's workgroups (16 slots each) must not outnumber the CUs either
-  if (wide_tiles) return (uint64_t)(round_up(rows, kTileM) / kTileM) * (n_padded(n) / kG16TileN) <= 256u;
-  return (uint64_t)(round_up(rows, (uint32_t)kGemm128TileM) / (uint32_t)kGemm128TileM) * (n_padded(n) / kGemmTileN) <= 512u;
+  const uint32_t rows = padded_rows_bound(m, n_groups), base = round_up(m, 32u);
+  auto rounds = [](uint64_t items, uint64_t resident) { return (items + resident - 1u) / resident; };
+  if (rounds(rows / 16u, 256u) != rounds(base / 16u, 256u)) return false;
+  const uint32_t tile_m = wide_tiles ? (uint32_t)kTileM : (uint32_t)kGemm128TileM;
+  const uint64_t per_row = n_padded(n) / (wide_tiles ? (uint32_t)kG16TileN : (uint32_t)kGemmTileN);
+  const uint64_t resident = wide_tiles ? 256u : 512u;
+  return rounds((uint64_t)(round_up(rows, tile_m) / tile_m) * per_row, resident) ==
+         rounds((uint64_t)(round_up(base, tile_m) / tile_m) * per_row, resident);
 }
 
 WsLayout make_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint32_t rank, bool routed,
