@@ -150,6 +150,21 @@ int launch_quant(const QuantArgs& a, hipStream_t s) {
   return MI355_W8A8_ERR_UNSUPPORTED;
 }
 
+// LoRA-A projection on the transposed A.  Up to 32 ranks the operands travel through LDS in whole
+// cache lines (the staged form of the kernel); beyond, two rank blocks per wave leave no room for that.
+int launch_lora_a(const LoraAArgs& la, uint32_t nkk, dim3 grid, hipStream_t s) {
+  if (nkk > 2u || la.at_operand) {
+    if (nkk > 2u) hipLaunchKernelGGL((lora_a_kernel<2>), grid, dim3(1024), 0, s, la);
+    else hipLaunchKernelGGL((lora_a_kernel<1>), grid, dim3(1024), 0, s, la);
+    return launch_status();
+  }
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(&lora_a_kernel<1, true>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, kLoraAStageBytes) != hipSuccess)
+    return MI355_W8A8_ERR_LAUNCH;
+  hipLaunchKernelGGL((lora_a_kernel<1, true>), grid, dim3(1024), kLoraAStageBytes, s, la);
+  return launch_status();
+}
+
 template <int EPI, int NKK, int MODE>
 int launch_gemm_one(const GemmArgs& g, hipStream_t s) {
   // persistent grid: one workgroup slot per CU (two in the 256 x 128 geometry), a multiple of 8
@@ -662,9 +677,7 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
     la.nterms = (p->flags & MI355_W8A8_FLAG_LORA_SPLIT2) ? 2u : 3u;
     la.n_blocks = w.slots / 32u;
     const dim3 grid(w.slots / 32u), block(1024);
-    if (w.nkk > 2u) hipLaunchKernelGGL((lora_a_kernel<2>), grid, block, 0, s, la);
-    else hipLaunchKernelGGL((lora_a_kernel<1>), grid, block, 0, s, la);
-    if ((st = launch_status())) return st;
+    if ((st = launch_lora_a(la, w.nkk, grid, s))) return st;
   }
   if (skip_gemm) return MI355_W8A8_OK;
 
@@ -848,9 +861,8 @@ int launch_bwd_body(const BwdBody& b, const Layout& w, unsigned char* ws, hipStr
       lz.zf_stride = kBwdRankStride;
       lz.zf_slice = w.slots * kBwdRankStride;
       const dim3 grid(lz.n_blocks * nks), block(1024);
-      if (w.nkk > 2u) hipLaunchKernelGGL((lora_a_kernel<2>), grid, block, 0, s, lz);
-      else hipLaunchKernelGGL((lora_a_kernel<1>), grid, block, 0, s, lz);
-      if ((st = launch_status())) return st;
+      (void)block;
+      if ((st = launch_lora_a(lz, w.nkk, grid, s))) return st;
       BwdRFinishArgs f{};
       f.rpart = reinterpret_cast<const float*>(ws + w.rpart);
       f.blk_range = b.skip_range;

@@ -528,8 +528,16 @@ struct LoraAArgs {
   uint32_t row_div, row_limit;
 };
 
-template <int RB>  // number of 32-wide rank blocks (1 or 2)
+// STAGED (RB = 1, the transposed A, no K split): the operands of a k step travel through 8 KiB of LDS
+// per wave.  A register load of an MFMA operand touches 32 cache lines of 32 used bytes, which the
+// vector memory path delivers at a third of the rate of whole lines; a direct-to-LDS load in which
+// eight lanes fetch one 128-byte line (of a row of x, of a rank column of A) moves eight whole lines,
+// and the operands are then read from LDS (line pieces XOR-swizzled by the row, so that eight lanes
+// never share a bank).  Which wave adds which k step, and in which order, does not change.
+constexpr uint32_t kLoraAStageBytes = 16u * 8192u;
+template <int RB, bool STAGED = false>  // RB: number of 32-wide rank blocks (1 or 2)
 __global__ __launch_bounds__(1024) void lora_a_kernel(LoraAArgs a) {
+  static_assert(!STAGED || RB == 1, "the staged form holds one rank block");
   __shared__ float red[4][RB][16][64];
   __shared__ float zs[32][RB * 32 + 1];
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
@@ -555,6 +563,57 @@ __global__ __launch_bounds__(1024) void lora_a_kernel(LoraAArgs a) {
   const uint32_t slice_end = (ks + 1u) * slice_steps < a.n_steps ? (ks + 1u) * slice_steps : a.n_steps;
   uint32_t s0 = ks * slice_steps + wave * a.steps_per_wave, s1 = s0 + a.steps_per_wave;
   if (s1 > slice_end) s1 = slice_end;
+  if constexpr (STAGED) {
+    extern __shared__ __attribute__((aligned(1024))) unsigned char stage_lds[];
+    unsigned char* const my = stage_lds + wave * 8192u;  // x lines at 0, A lines at 4096
+    // lane l fetches, for j = 0..3, piece (l % 8) ^ (l / 8) of the 128-byte line of row / column 8 j + l / 8
+    const uint32_t r8 = lane >> 3, piece = (lane & 7u) ^ r8;
+    const uint16_t* xrow[4];
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j) {
+      const uint32_t pj = pb * 32u + 8u * j + r8;
+      int sj = a.src_row ? a.src_row[pj] : (int)pj;
+      if (sj >= (int)a.M) sj = -1;
+      if (a.row_map && sj >= 0) sj = (int)mapped_row(a.row_map[sj], a.row_div, a.row_limit);
+      xrow[j] = a.xsrc + (size_t)(sj < 0 ? 0 : sj) * a.K;
+    }
+    // where lane (i, h) finds quarter t of its operand: line i, piece 4 h + t
+    const uint32_t rd = (i >> 3) * 1024u + (i & 7u) * 128u;
+    for (uint32_t grp = glo; grp <= ghi; ++grp) {
+      const bool mine = src >= 0 && rowgrp == grp;
+      const uint16_t* atg = a.at + (size_t)grp * a.r * a.K;
+      for (uint32_t s = s0; s < s1; ++s) {
+        uint32_t kp = s * 64u + piece * 8u;
+        if (kp >= a.K) kp = 0;  // a piece beyond K: any address inside the row; it is zeroed where it is used
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+          load_1k_to_lds(reinterpret_cast<const unsigned char*>(xrow[j] + kp), my + j * 1024u);
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+          uint32_t col = 8u * j + r8;
+          if (col >= a.r) col = 0;
+          load_1k_to_lds(reinterpret_cast<const unsigned char*>(atg + (size_t)col * a.K + kp), my + 4096u + j * 1024u);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        v8us xa[4], wb[4];
+#pragma unroll
+        for (uint32_t t = 0; t < 4; ++t) {
+          const uint32_t off = rd + (((4u * h + t) ^ (i & 7u)) * 16u);
+          const v8us zero = {0, 0, 0, 0, 0, 0, 0, 0};
+          const bool ok = s * 64u + 32u * h + 8u * t < a.K;
+          const v8us xv = *reinterpret_cast<const v8us*>(my + off);
+          const v8us wv = *reinterpret_cast<const v8us*>(my + 4096u + off);
+          xa[t] = (mine && ok) ? xv : zero;
+          wb[t] = (i < a.r && ok) ? wv : zero;
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the lines are read before the next step's loads land on them
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+          acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, xa[t]), __builtin_bit_cast(v8bf, wb[t]),
+                                                           acc[0], 0, 0, 0);
+      }
+    }
+  } else
   // A block at a group boundary runs once per group with the other groups' rows zeroed.
   for (uint32_t grp = glo; grp <= ghi; ++grp) {
     const bool mine = src >= 0 && rowgrp == grp;
