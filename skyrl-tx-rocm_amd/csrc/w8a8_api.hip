@@ -153,9 +153,8 @@ int launch_quant(const QuantArgs& a, hipStream_t s) {
 // LoRA-A projection on the transposed A.  Up to 32 ranks the operands travel through LDS in whole
 // cache lines (the staged form of the kernel); beyond, two rank blocks per wave leave no room for that.
 int launch_lora_a(const LoraAArgs& la, uint32_t nkk, dim3 grid, hipStream_t s) {
-  if (nkk > 2u || la.at_operand) {
-    if (nkk > 2u) hipLaunchKernelGGL((lora_a_kernel<2>), grid, dim3(1024), 0, s, la);
-    else hipLaunchKernelGGL((lora_a_kernel<1>), grid, dim3(1024), 0, s, la);
+  if (nkk > 2u) {
+    hipLaunchKernelGGL((lora_a_kernel<2>), grid, dim3(1024), 0, s, la);
     return launch_status();
   }
   if (hipFuncSetAttribute(reinterpret_cast<const void*>(&lora_a_kernel<1, true>),
@@ -1705,9 +1704,8 @@ int run_gq_linear(const mi355_w8a8_gq_problem* p, hipStream_t s) {
     la.nterms = 3u;
     la.n_blocks = L.m_pad / 32u;
     const dim3 zgrid(L.m_pad / 32u), zblock(1024);
-    if (la.nkk > 2u) hipLaunchKernelGGL((lora_a_kernel<2>), zgrid, zblock, 0, s, la);
-    else hipLaunchKernelGGL((lora_a_kernel<1>), zgrid, zblock, 0, s, la);
-    if ((st = launch_status())) return st;
+    (void)zblock;
+    if ((st = launch_lora_a(la, la.nkk, zgrid, s))) return st;
   } else if (lora) {
     GqLoraZArgs z{};
     z.x = q.x;

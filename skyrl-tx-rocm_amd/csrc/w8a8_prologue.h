@@ -588,23 +588,31 @@ __global__ __launch_bounds__(1024) void lora_a_kernel(LoraAArgs a) {
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j)
           load_1k_to_lds(reinterpret_cast<const unsigned char*>(xrow[j] + kp), my + j * 1024u);
+        v8us xa[4], wb[4];
+        if (a.at_operand) {  // kernel-uniform: A already lies in operand order (zero beyond K and the rank)
 #pragma unroll
-        for (uint32_t j = 0; j < 4; ++j) {
-          uint32_t col = 8u * j + r8;
-          if (col >= a.r) col = 0;
-          load_1k_to_lds(reinterpret_cast<const unsigned char*>(atg + (size_t)col * a.K + kp), my + 4096u + j * 1024u);
+          for (uint32_t t = 0; t < 4; ++t)
+            wb[t] = *(reinterpret_cast<const v8us*>(a.at) + (((size_t)grp * a.n_steps + s) * 4u + t) * 64u + lane);
+        } else {
+#pragma unroll
+          for (uint32_t j = 0; j < 4; ++j) {
+            uint32_t col = 8u * j + r8;
+            if (col >= a.r) col = 0;
+            load_1k_to_lds(reinterpret_cast<const unsigned char*>(atg + (size_t)col * a.K + kp), my + 4096u + j * 1024u);
+          }
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        v8us xa[4], wb[4];
 #pragma unroll
         for (uint32_t t = 0; t < 4; ++t) {
           const uint32_t off = rd + (((4u * h + t) ^ (i & 7u)) * 16u);
           const v8us zero = {0, 0, 0, 0, 0, 0, 0, 0};
           const bool ok = s * 64u + 32u * h + 8u * t < a.K;
           const v8us xv = *reinterpret_cast<const v8us*>(my + off);
-          const v8us wv = *reinterpret_cast<const v8us*>(my + 4096u + off);
           xa[t] = (mine && ok) ? xv : zero;
-          wb[t] = (i < a.r && ok) ? wv : zero;
+          if (!a.at_operand) {
+            const v8us wv = *reinterpret_cast<const v8us*>(my + 4096u + off);
+            wb[t] = (i < a.r && ok) ? wv : zero;
+          }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the lines are read before the next step's loads land on them
 #pragma unroll
