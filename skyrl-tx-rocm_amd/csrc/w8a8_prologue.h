@@ -308,6 +308,11 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(QuantArgs a) {
     if (a.sx_slots && p >= 0) a.sx_slots[p] = scale;
     if (a.scales_rm) a.scales_rm[m] = scale;
   }
+  // codes = rint(v / scale) with the correctly rounded quotient, as in quant_lora_kernel: v * (1 / scale)
+  // with the hardware reciprocal rounds to the same integer unless the product lies within 1e-4 of a
+  // tie; those cases (and scales outside the reciprocal's safe range) are redone with the division.
+  const float rscale = __builtin_amdgcn_rcpf(scale);
+  const bool scale_safe = scale > 1e-30f && scale < 1e30f;
 #pragma unroll
   for (int j = 0; j < NCH; ++j) {
     uint32_t c = j * 64u + lane;
@@ -315,13 +320,27 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(QuantArgs a) {
     if (k0 >= a.K_pad) continue;
     uint32_t lo = 0, hi = 0;
     if (k0 < a.K) {
+      float q[8];
+      float off_integer = 0.0f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        float q = rintf(v[j][e] / scale);
-        q = fminf(fmaxf(q, -127.0f), 127.0f);
-        uint32_t b = (uint32_t)(int)q & 0xffu;
-        if (e < 4) lo |= b << (8 * e); else hi |= b << (8 * (e - 4));
+        const float t = v[j][e] * rscale;
+        q[e] = rintf(t);
+        off_integer = fmaxf(off_integer, fabsf(t - q[e]));
       }
+      if (!scale_safe || off_integer > 0.4999f) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) q[e] = rintf(v[j][e] / scale);
+      }
+      // q is an integer in [-127, 127] (|v| <= the row's absmax): q + 128 lands in its byte with one
+      // v_cvt_pk_u8_f32, and flipping bit 7 of every byte turns the biased value into two's complement
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        lo = __builtin_amdgcn_cvt_pk_u8_f32(q[e] + 128.0f, (uint32_t)e, lo);
+        hi = __builtin_amdgcn_cvt_pk_u8_f32(q[e + 4] + 128.0f, (uint32_t)e, hi);
+      }
+      lo ^= 0x80808080u;
+      hi ^= 0x80808080u;
       if (a.codes_rm) *reinterpret_cast<uint2*>(a.codes_rm + (size_t)m * a.K + k0) = make_uint2(lo, hi);
     }
     if (a.xq_packed && p >= 0)
