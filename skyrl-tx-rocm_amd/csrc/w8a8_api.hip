@@ -424,8 +424,12 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
 
   const bool skip_prologue = (p->flags & MI355_W8A8_FLAG_SKIP_PROLOGUE) != 0;
   const bool skip_gemm = (p->flags & MI355_W8A8_FLAG_SKIP_GEMM) != 0;
-  // up to 8192 rows the quantizer's workgroups sort the adapter indices themselves (one launch less)
-  const bool route_inline = routed && p->m <= kInlineRouteMaxRows;
+  // Up to 8192 rows the quantizer's workgroups sort the adapter indices themselves (one launch less) --
+  // unless the launch that lays out the LoRA operands runs anyway (adapters that changed since the last
+  // call, as in every training step): then its first block sorts, beside the others, and the quantizer
+  // reads the tables (4-6 us less in each of its workgroups).
+  const bool pack_launch = lora && !skip_prologue && !(p->flags & MI355_W8A8_FLAG_LORA_PACK_VALID);
+  const bool route_inline = routed && p->m <= kInlineRouteMaxRows && !pack_launch;
   if ((routed || lora) && !skip_prologue) {
     LoraPrepArgs pa{};
     pa.idx = routed ? p->adapter_indices : nullptr;
@@ -437,6 +441,7 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
     pa.M = p->m; pa.K = p->k; pa.N = p->n; pa.n_groups = p->n_adapters; pa.r = p->rank; pa.nkk = w.nkk;
     pa.ncb = n_padded(p->n) / 32u; pa.slots = w.slots;
     pa.route_blocks = (routed && !route_inline) ? 1u : 0u;
+    pa.route_pad = pad_groups ? 32u : 1u;
     pa.a_operand_kb = w.KB;  // the quantizer reads A in MFMA operand order
     const uint64_t a_items = (uint64_t)p->n_adapters * w.KB * w.nkk * 64u;
     const uint64_t b_items = (uint64_t)p->n_adapters * pa.ncb * w.nkk * 64u;
@@ -469,9 +474,9 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   q.r = p->rank; q.nkk = w.nkk;
   q.nterms = (p->flags & MI355_W8A8_FLAG_LORA_SPLIT2) ? 2u : 3u;
   q.tile_ctr = reinterpret_cast<uint32_t*>(ws + w.tile_ctr);
+  q.group_pad = pad_groups ? 32u : 1u;
   if (route_inline) {
     q.route_idx = p->adapter_indices; q.n_groups = p->n_adapters; q.slots = w.slots;
-    q.group_pad = pad_groups ? 32u : 1u;
     q.src_row = src_row; q.slot_group = slot_group; q.blk_range = blk_range;
   }
   if (!skip_prologue) {

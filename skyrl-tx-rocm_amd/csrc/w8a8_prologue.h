@@ -54,11 +54,13 @@ __global__ __launch_bounds__(256) void unpack_weight_kernel(const unsigned char*
 // One workgroup.  The order of rows inside a group does not influence any forward result; the
 // backward asks for the stable order because it sums over a group's rows.
 // ---------------------------------------------------------------------------------------
+// With group_pad = 32 every group starts on a 32-slot boundary (see route_rows_inline): the slots between
+// a group's last row and the next group's first stay empty.
 __device__ inline void route_rows_block(const int32_t* __restrict__ idx, uint32_t M, uint32_t n_groups,
                                         uint32_t slots, int32_t* __restrict__ src_row,
                                         int32_t* __restrict__ dst_pos, int32_t* __restrict__ slot_group,
                                         int32_t* __restrict__ blk_range, int32_t* __restrict__ group_off = nullptr,
-                                        bool stable = false) {
+                                        bool stable = false, uint32_t group_pad = 1u) {
   __shared__ int cnt[kMaxAdapters];
   __shared__ int start[kMaxAdapters + 1];
   __shared__ int cursor[kMaxAdapters];
@@ -75,10 +77,14 @@ __device__ inline void route_rows_block(const int32_t* __restrict__ idx, uint32_
     int pos = 0;
     for (uint32_t a = 0; a < n_groups; ++a) {
       start[a] = pos;
-      pos += cnt[a];
+      pos += (int)round_up((uint32_t)cnt[a], group_pad);
     }
     start[n_groups] = pos;
   }
+  __syncthreads();
+  const uint32_t E = (uint32_t)start[n_groups];  // first slot behind the last group (M when the groups are packed)
+  if (group_pad > 1u)
+    for (uint32_t p = tid; p < E && p < slots; p += 1024) src_row[p] = -1;  // the empty slots between groups
   __syncthreads();
   if (group_off && tid <= n_groups) group_off[tid] = start[tid];  // first slot of every group, then M
   if (stable) {
@@ -125,10 +131,10 @@ __device__ inline void route_rows_block(const int32_t* __restrict__ idx, uint32_
       dst_pos[i] = p;
     }
   }
-  // group of a slot = the group whose [start, start+count) range holds it
+  // group of a slot = the group whose [start, next start) range holds it
   for (uint32_t p = tid; p < slots; p += 1024) {
     int g = 0;
-    if (p < M) {
+    if (p < E) {
       for (uint32_t a = 0; a < n_groups; ++a)
         if ((int)p >= start[a] && (int)p < start[a + 1]) g = (int)a;
     } else {
@@ -139,13 +145,13 @@ __device__ inline void route_rows_block(const int32_t* __restrict__ idx, uint32_
     slot_group[p] = g;
   }
   for (uint32_t b = tid; b < slots / 32u; b += 1024) {
-    const int p0 = (int)b * 32, p1 = (p0 + 31 < (int)M) ? p0 + 31 : (int)M - 1;
+    const int p0 = (int)b * 32, p1 = (p0 + 31 < (int)E) ? p0 + 31 : (int)E - 1;
     int g0 = 0, g1 = 0;
     for (uint32_t a = 0; a < n_groups; ++a) {
       if (p0 >= start[a] && p0 < start[a + 1]) g0 = (int)a;
       if (p1 >= start[a] && p1 < start[a + 1]) g1 = (int)a;
     }
-    if (p0 >= (int)M) { g0 = 0; g1 = 0; }
+    if (p0 >= (int)E) { g0 = 0; g1 = 0; }
     blk_range[b] = g0 | (g1 << 16);
   }
 }
@@ -481,6 +487,7 @@ struct LoraPrepArgs {
   uint16_t* at;              // bf16 [n_groups, r, K]
   unsigned char* bp;         // packed B operands
   uint32_t M, K, N, n_groups, r, nkk, ncb, slots, route_blocks, a_blocks;
+  uint32_t route_pad;        // dense routing block: every group's first slot is a multiple of this (0 or 1: packed)
   uint32_t a_operand_kb;     // 0: `at` is the transposed A; else K_pad / 32 and `at` takes A in MFMA operand order
   uint32_t a_operand_steps, a_operand_rb;  // or: ceil(K / 64) and the 32-wide rank blocks of lora_a_kernel's operand order
   // grouped (ragged) call: the routing block lays the groups out from their sizes instead
@@ -497,7 +504,8 @@ __global__ __launch_bounds__(1024) void lora_prep_kernel(LoraPrepArgs p) {
       route_groups_block(p.group_sizes, p.M, p.n_groups, p.slots, p.src_row, p.dst_pos, p.blk_range, p.group_pad,
                          p.zero_out, p.zero_cols);
     else
-      route_rows_block(p.idx, p.M, p.n_groups, p.slots, p.src_row, p.dst_pos, p.slot_group, p.blk_range);
+      route_rows_block(p.idx, p.M, p.n_groups, p.slots, p.src_row, p.dst_pos, p.slot_group, p.blk_range, nullptr, false,
+                       p.route_pad > 1u ? p.route_pad : 1u);
     return;
   }
   b -= p.route_blocks;
@@ -927,6 +935,13 @@ __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
       for (int j = 0; j < 16; ++j) any |= (route_src[j] >= 0) ? 1 : 0;
       if (!any) return;  // workgroup-uniform
     }
+  }
+
+  if (!route_here && a.group_pad > 1u && a.src_row) {  // the same for tables a routing block has written
+    int any = 0;
+#pragma unroll
+    for (uint32_t j = 0; j < 16; ++j) any |= (a.src_row[hb * 16u + j] >= 0) ? 1 : 0;
+    if (!any) return;  // workgroup-uniform
   }
 
   // ---- 1. row statistics: wave w, slot row w
