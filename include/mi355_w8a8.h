@@ -298,7 +298,9 @@ int mi355_w8a8_unpack_weight_v1(const void* packed, int8_t* codes_kn, uint32_t k
 int mi355_w8a8_quantize_rows_v1(const void* x_bf16, int8_t* codes, float* scales, uint32_t m,
                                 uint32_t k, void* stream);
 
-/* Workspace requirement of the three dense entry points below. */
+/* Workspace requirement of the dense entry points below.  It depends on the dimensions only (never on
+ * the flags or on which rows use which adapter) and covers every layout a call of these dimensions may
+ * choose: adapters packed or each on a 32-slot boundary, any tile geometry, the decode kernels. */
 uint64_t mi355_w8a8_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t n_adapters,
                                     uint32_t rank, uint32_t flags);
 uint64_t mi355_w8a8_grouped_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups,
