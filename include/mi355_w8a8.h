@@ -72,12 +72,14 @@ typedef enum mi355_w8a8_status {
  * prologue results and answer these two flags with MI355_W8A8_ERR_UNSUPPORTED. */
 #define MI355_W8A8_FLAG_SKIP_PROLOGUE 16u /* do not run routing / quantization / LoRA-A */
 #define MI355_W8A8_FLAG_SKIP_GEMM 32u     /* run only routing / quantization / LoRA-A */
-/* tile geometry of the tiled GEMM (at most one of the three; two are refused with MI355_W8A8_ERR_SHAPE);
+/* tile geometry of the tiled GEMM (at most one of the four; two are refused with MI355_W8A8_ERR_SHAPE);
  * default: 128 x 128 while at most 512 such tiles cover the output, else 256 x 256 (256 x 128 when k is
- * too short for that kernel's stage schedule) */
+ * too short for that kernel's stage schedule).  TILE_256X128_PAIR is the 256 x 256 kernel's instruction
+ * (16 x 16 x 64) and schedule in 256 x 128 tiles, two workgroups per CU. */
 #define MI355_W8A8_FLAG_TILE_256X128 64u
 #define MI355_W8A8_FLAG_TILE_256X256 128u
 #define MI355_W8A8_FLAG_TILE_128X128 2048u
+#define MI355_W8A8_FLAG_TILE_256X128_PAIR 4096u
 /* tile rows of the grouped call (and the slots every group is padded to); default: 128 once the
  * groups average at least 96 rows, else 64.  Pass the same flags to the workspace query. */
 #define MI355_W8A8_FLAG_GROUPED_TILE64 256u
@@ -544,6 +546,7 @@ int mi355_w8a8_gq_linear_v1(const mi355_w8a8_gq_problem* problem, void* stream);
 #define MI355_W8A8_PATH_TILED_256X128 3  /* prologue + 256 x 128 tiles, two workgroups per CU */
 #define MI355_W8A8_PATH_TILED_256X256 4  /* prologue + 256 x 256 tiles, one workgroup per CU */
 #define MI355_W8A8_PATH_TILED_128X128 5  /* prologue + 128 x 128 tiles, two workgroups per CU */
+#define MI355_W8A8_PATH_TILED_256X128_PAIR 6  /* prologue + 256 x 128 tiles on 16 x 16 x 64 MFMAs, two workgroups per CU */
 int mi355_w8a8_forward_path(uint32_t m, uint32_t k, uint32_t n, uint32_t flags);
 
 /*

@@ -25,8 +25,10 @@ FLAG_GROUPED_TILE64 = 256
 FLAG_GROUPED_TILE128 = 512
 FLAG_LORA_PACK_VALID = 1024
 FLAG_TILE_128X128 = 2048
+FLAG_TILE_256X128_PAIR = 4096
 STATIC_WORKSPACE_BYTES = 32 << 20
-PATH_NAMES = {1: "skinny", 2: "skinny-chunks", 3: "tiled-256x128", 4: "tiled-256x256", 5: "tiled-128x128"}
+PATH_NAMES = {1: "skinny", 2: "skinny-chunks", 3: "tiled-256x128", 4: "tiled-256x256", 5: "tiled-128x128",
+              6: "tiled-256x128-pair"}
 
 STATUS = {
     0: "OK", -1: "ERR_NULL", -2: "ERR_SHAPE", -3: "ERR_ALIGN", -4: "ERR_ALIAS",

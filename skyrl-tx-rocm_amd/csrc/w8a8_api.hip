@@ -193,26 +193,28 @@ int launch_gemm(const GemmArgs& g, uint32_t nkk, hipStream_t s) {
   }
 }
 
-template <int EPI, int NKK>
+template <int EPI, int NKK, int NW = 4>
 int launch_gemm16_one(const GemmArgs& g, hipStream_t s) {
-  // persistent grid: one workgroup per CU, a multiple of 8 so that every XCD gets the same share
+  // persistent grid: one workgroup per CU (two in the 256 x 128 geometry), a multiple of 8 so that every
+  // XCD gets the same share
+  using Geo = G16Geo<NW>;
   const uint32_t ntile = g.tiles_m * g.tiles_n;
   const uint32_t want = ((ntile + 7u) / 8u) * 8u;
-  const dim3 grid(want < 256u ? want : 256u), block(512);
-  if (hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm16_kernel<EPI, NKK>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, kG16LdsBytes) != hipSuccess)
+  const dim3 grid(want < (uint32_t)Geo::kResident ? want : (uint32_t)Geo::kResident), block(Geo::kThreads);
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemm16_kernel<EPI, NKK, NW>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, Geo::kLdsBytes) != hipSuccess)
     return MI355_W8A8_ERR_LAUNCH;
-  hipLaunchKernelGGL((w8a8_gemm16_kernel<EPI, NKK>), grid, block, kG16LdsBytes, s, g);
+  hipLaunchKernelGGL((w8a8_gemm16_kernel<EPI, NKK, NW>), grid, block, Geo::kLdsBytes, s, g);
   return launch_status();
 }
 
-template <int EPI>
+template <int EPI, int NW = 4>
 int launch_gemm16(const GemmArgs& g, uint32_t nkk, hipStream_t s) {
   switch (nkk) {
-    case 0: return launch_gemm16_one<EPI, 0>(g, s);
-    case 1: return launch_gemm16_one<EPI, 1>(g, s);
-    case 2: return launch_gemm16_one<EPI, 2>(g, s);
-    case 4: return launch_gemm16_one<EPI, 4>(g, s);
+    case 0: return launch_gemm16_one<EPI, 0, NW>(g, s);
+    case 1: return launch_gemm16_one<EPI, 1, NW>(g, s);
+    case 2: return launch_gemm16_one<EPI, 2, NW>(g, s);
+    case 4: return launch_gemm16_one<EPI, 4, NW>(g, s);
     default: return MI355_W8A8_ERR_UNSUPPORTED;
   }
 }
@@ -311,7 +313,7 @@ int choose_forward_path(uint32_t m, uint32_t k, uint32_t n, uint32_t flags) {
   if (skinny) return MI355_W8A8_PATH_SKINNY;
   if (skinny_supported() && !swiglu && skinny_chunked_pays(m, k, n) &&
       !(flags & (MI355_W8A8_FLAG_FORCE_TILED | MI355_W8A8_FLAG_TILE_256X128 | MI355_W8A8_FLAG_TILE_256X256 |
-                 MI355_W8A8_FLAG_TILE_128X128)))
+                 MI355_W8A8_FLAG_TILE_128X128 | MI355_W8A8_FLAG_TILE_256X128_PAIR)))
     return MI355_W8A8_PATH_SKINNY_CHUNKS;
   // 256 x 256 tiles (one 8-wave workgroup per CU, 16 x 16 x 64 MFMAs) once they fill half the CUs;
   // below that the 256 x 128 geometry (two 4-wave workgroups per CU) has twice the tiles to spread.
@@ -327,8 +329,11 @@ int choose_forward_path(uint32_t m, uint32_t k, uint32_t n, uint32_t flags) {
   // M = 512: 62 us against 84; K = 4096, N = 2560 at M = 2048: 88 against 105; beyond 512 tiles the
   // larger geometries win (K = 2560, N = 6144 at M = 2048: 97 us against 85 on 256 x 256).
   const bool small = (uint64_t)(round_up(m, (uint32_t)kGemm128TileM) / (uint32_t)kGemm128TileM) * (n_padded(n) / kGemmTileN) <= 512u;
-  const uint32_t forced = flags & (MI355_W8A8_FLAG_TILE_256X128 | MI355_W8A8_FLAG_TILE_256X256 | MI355_W8A8_FLAG_TILE_128X128);
+  const uint32_t forced = flags & (MI355_W8A8_FLAG_TILE_256X128 | MI355_W8A8_FLAG_TILE_256X256 | MI355_W8A8_FLAG_TILE_128X128 |
+                                   MI355_W8A8_FLAG_TILE_256X128_PAIR);
   if (forced & (forced - 1u)) return MI355_W8A8_ERR_SHAPE;  // two geometries asked for
+  if (forced == MI355_W8A8_FLAG_TILE_256X128_PAIR)  // (its stage schedule needs at least six 64-wide k steps, too)
+    return k_padded(k) < kG16MinKPad ? MI355_W8A8_PATH_TILED_256X128 : MI355_W8A8_PATH_TILED_256X128_PAIR;
   if (forced == MI355_W8A8_FLAG_TILE_128X128 || (!forced && small)) return MI355_W8A8_PATH_TILED_128X128;
   return wide ? MI355_W8A8_PATH_TILED_256X256 : MI355_W8A8_PATH_TILED_256X128;
 }
@@ -475,15 +480,25 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   q.nterms = (p->flags & MI355_W8A8_FLAG_LORA_SPLIT2) ? 2u : 3u;
   q.tile_ctr = reinterpret_cast<uint32_t*>(ws + w.tile_ctr);
   q.group_pad = pad_groups ? 32u : 1u;
+  q.rows_per_wg = quant_lora_rows_per_wg(p->k);
+  q.row_stride = quant_lora_row_stride(p->k);
   if (route_inline) {
     q.route_idx = p->adapter_indices; q.n_groups = p->n_adapters; q.slots = w.slots;
     q.src_row = src_row; q.slot_group = slot_group; q.blk_range = blk_range;
   }
   if (!skip_prologue) {
-    const dim3 grid(q.n_half_blocks), block(1024);
-#define W8A8_QL(CB)                                                                   \
-  if (rms) hipLaunchKernelGGL((quant_lora_kernel<CB, true>), grid, block, 0, s, q);   \
-  else hipLaunchKernelGGL((quant_lora_kernel<CB, false>), grid, block, 0, s, q)
+    const dim3 grid(q.n_half_blocks * (16u / q.rows_per_wg)), block(1024);
+    const uint32_t ql_lds = quant_lora_lds_bytes(p->k, lora ? w.nkk : 0u);
+#define W8A8_QL1(CB, RMS)                                                                                   \
+  {                                                                                                         \
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&quant_lora_kernel<CB, RMS>),                     \
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)ql_lds) != hipSuccess)         \
+      return MI355_W8A8_ERR_LAUNCH;                                                                         \
+    hipLaunchKernelGGL((quant_lora_kernel<CB, RMS>), grid, block, ql_lds, s, q);                            \
+  }
+#define W8A8_QL(CB)                \
+  if (rms) W8A8_QL1(CB, true)      \
+  else W8A8_QL1(CB, false)
     switch (lora ? w.nkk : 0u) {
       case 0: W8A8_QL(0); break;
       case 1: W8A8_QL(1); break;
@@ -491,6 +506,7 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
       default: W8A8_QL(4); break;
     }
 #undef W8A8_QL
+#undef W8A8_QL1
     if ((st = launch_status())) return st;
   } else if (!skip_gemm && path != MI355_W8A8_PATH_TILED_256X256) {
     // measurement calls: the tile counters of the 256 x 128 geometry's dynamic schedule still have to
@@ -521,6 +537,7 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
   g.rank = lora ? p->rank : 0u;
   g.tile_ctr = reinterpret_cast<uint32_t*>(ws + w.tile_ctr);
   const bool wide = path == MI355_W8A8_PATH_TILED_256X256;
+  const bool pair = path == MI355_W8A8_PATH_TILED_256X128_PAIR;
   const bool small = path == MI355_W8A8_PATH_TILED_128X128;
   if (wide) g.tiles_n = n_padded(p->n) / kG16TileN;
   if (small) g.tiles_m = round_up(w.rows_bound, (uint32_t)kGemm128TileM) / (uint32_t)kGemm128TileM;
@@ -529,11 +546,13 @@ int run_forward(const mi355_w8a8_problem* p, hipStream_t s, Required req) {
     ga.out = p->aux_acc;
     ga.residual = nullptr;
     if ((st = wide ? launch_gemm16_one<kEpiAcc, 0>(ga, s)
-                   : (small ? launch_gemm<kEpiAcc, kModeDense128>(ga, 0u, s) : launch_gemm<kEpiAcc>(ga, 0u, s))))
+                   : (pair ? launch_gemm16_one<kEpiAcc, 0, 2>(ga, s)
+                           : (small ? launch_gemm<kEpiAcc, kModeDense128>(ga, 0u, s) : launch_gemm<kEpiAcc>(ga, 0u, s)))))
       return st;
     g.tile_ctr += 128;  // the second counter set
   }
   if (wide) return swiglu ? launch_gemm16<kEpiSwiglu>(g, w.nkk, s) : launch_gemm16<kEpiPlain>(g, w.nkk, s);
+  if (pair) return swiglu ? launch_gemm16<kEpiSwiglu, 2>(g, w.nkk, s) : launch_gemm16<kEpiPlain, 2>(g, w.nkk, s);
   if (small)
     return swiglu ? launch_gemm<kEpiSwiglu, kModeDense128>(g, w.nkk, s) : launch_gemm<kEpiPlain, kModeDense128>(g, w.nkk, s);
   return swiglu ? launch_gemm<kEpiSwiglu>(g, w.nkk, s) : launch_gemm<kEpiPlain>(g, w.nkk, s);

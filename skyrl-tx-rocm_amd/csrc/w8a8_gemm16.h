@@ -44,12 +44,26 @@ typedef float v4f_t __attribute__((ext_vector_type(4)));
 
 constexpr int kG16TileM = 256;
 constexpr int kG16TileN = 256;
-constexpr int kG16Stages = 4;
-constexpr int kG16StageBytes = 32768;  // A: 8 row blocks x 2 k blocks, then B: 8 column blocks x 2 k blocks
-constexpr int kG16RingBytes = kG16Stages * kG16StageBytes;
-constexpr int kG16LdsBytes = kG16RingBytes + 8192;  // + per wave 128 row scales and 128 row positions
-constexpr int kG16Loads = 4;                        // direct-to-LDS loads per wave and stage
 constexpr uint32_t kG16MinKPad = 384;               // at least six stages: the schedule below assumes it
+// Two geometries of the same kernel, told apart by NW, the waves side by side along N (2 rows of them):
+//   NW = 4: tile 256 x 256, 8 waves, one workgroup per CU, ring of four 32 KiB stages;
+//   NW = 2: tile 256 x 128, 4 waves, two independent workgroups per CU (one wave of each per SIMD), ring of
+//           three 24 KiB stages each: while one workgroup runs its epilogue on the vector ALU the other's
+//           main loop has the matrix core to itself.
+// The wave tile (128 x 64), its fragment reads and its epilogue are the same in both.
+template <int NW>
+struct G16Geo {
+  static constexpr int kTileN = 64 * NW;
+  static constexpr int kStages = NW == 4 ? 4 : 3;
+  static constexpr int kStageBytes = 16384 + 4096 * NW;  // A: 8 row blocks x 2 k blocks, then B: 2 NW column blocks x 2 k blocks
+  static constexpr int kRingBytes = kStages * kStageBytes;
+  static constexpr int kWaves = 2 * NW;
+  static constexpr int kLdsBytes = kRingBytes + kWaves * 1024 + (NW == 4 ? 0 : 64);  // + per wave 128 row scales and 128 row positions (+ the next tile's position)
+  static constexpr int kLoads = kStageBytes / 1024 / kWaves;     // direct-to-LDS loads per wave and stage (4 or 6)
+  static constexpr int kThreads = 64 * kWaves;
+  static constexpr int kResident = NW == 4 ? 256 : 512;          // workgroups the chip holds at once
+};
+constexpr int kG16LdsBytes = G16Geo<4>::kLdsBytes;
 
 // Four direct-to-LDS loads of 1 KiB each: lane l moves 16 bytes global[base_i + 1024 i + voff] -> LDS[lds_addr +
 // 1024 i + 16 l] (voff = 16 l + ...).  The instruction offset applies to the global and to the LDS address
@@ -62,6 +76,13 @@ __device__ inline void g16_load_4k(const unsigned char* b0, const unsigned char*
                "global_load_lds_dwordx4 %0, %3 offset:2048\n\t"
                "global_load_lds_dwordx4 %0, %4 offset:3072"
                :: "v"(voff), "s"(b0), "s"(b1), "s"(b2), "s"(b3), "s"(lds_addr_uniform) : "memory", "m0");
+}
+// Two more for the six-load geometry: chunks 4 and 5 of the wave, LDS address and global base 4 KiB on.
+__device__ inline void g16_load_2k(const unsigned char* b4, const unsigned char* b5, uint32_t voff, uint32_t lds_addr_uniform) {
+  asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\t"
+               "global_load_lds_dwordx4 %0, %1\n\t"
+               "global_load_lds_dwordx4 %0, %2 offset:1024"
+               :: "v"(voff), "s"(b4), "s"(b5), "s"(lds_addr_uniform) : "memory", "m0");
 }
 __device__ inline void g16_set_m0(uint32_t lds_addr_uniform) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" :: "s"(lds_addr_uniform) : "memory", "m0");
@@ -106,9 +127,14 @@ __device__ inline void g16_mfma_first(v4i& acc, const v4i& a, const v4i& b) {
 constexpr int g16_frag_off(int f) { return (f >> 1) * 2048 + (f & 1) * 256; }  // activation fragment f of a wave's four row blocks
 constexpr int g16_bfrag_off(int j) { return j * 2048; }                        // weight fragment j: the wave's half of column block j
 
-template <int EPI, int NKK>
-__global__ __launch_bounds__(512, 1)
+template <int EPI, int NKK, int NW = 4>
+__global__ __launch_bounds__(G16Geo<NW>::kThreads, NW == 4 ? 1 : 2)
 void w8a8_gemm16_kernel(GemmArgs g) {
+  using Geo = G16Geo<NW>;
+  constexpr int kS = Geo::kStages;
+  constexpr int kLoads = Geo::kLoads;
+  constexpr uint32_t kSB = Geo::kStageBytes;
+  auto ring = [](uint32_t i) -> uint32_t { return kS == 4 ? (i & 3u) : i % (uint32_t)kS; };
   constexpr bool kLora = (NKK > 0) && (EPI != kEpiAcc);
   constexpr int kKS = NKK > 2 ? 2 : 1;  // 32-wide rank steps of the LoRA product
   constexpr uint32_t kNkk = NKK > 0 ? NKK : 1;
@@ -116,7 +142,7 @@ void w8a8_gemm16_kernel(GemmArgs g) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wrow = wave >> 2, wcol = wave & 3;  // wave tile: rows 128 wrow, columns 64 wcol of the tile
+  const int wrow = wave / NW, wcol = wave % NW;  // wave tile: rows 128 wrow, columns 64 wcol of the tile
   const int cgrp = wcol >> 1, chalf = wcol & 1;  // its 128-column group inside the tile and its half of every block
   const uint32_t c16 = lane & 15, q = lane >> 4;
   // byte offset of the lane's 16 bytes inside a pair of k blocks (lower 16 rows of the block)
@@ -149,71 +175,98 @@ void w8a8_gemm16_kernel(GemmArgs g) {
     T.valid = true;
     return T;
   };
-  // chunk ch = 4 wave + i of a stage: 0..15 activations (row block ch / 2, k block ch % 2), 16..31
+  // chunk ch = kLoads wave + i of a stage: 0..15 activations (row block ch / 2, k block ch % 2), 16..
   // weights; stage kt of a chunk lies 2 KiB * kt behind its base.  Returned: base - 1024 (i % 4), see
   // g16_load_4k.
   auto chunk_base = [&](const GemmTile& Tx, int i) -> const unsigned char* {
-    const int ch = wave * kG16Loads + i;
+    const int ch = wave * kLoads + i;
     const bool isA = ch < 16;
-    uint32_t rb = isA ? (uint32_t)(ch >> 1) : Tx.tn * 8u + (uint32_t)((ch - 16) >> 1);
+    uint32_t rb = isA ? (uint32_t)(ch >> 1) : Tx.tn * (uint32_t)(2 * NW) + (uint32_t)((ch - 16) >> 1);
     if (!isA && rb >= ncb_total) rb = ncb_total - 1u;  // keep every wave's load count equal
-    return (isA ? Tx.Ag : Tx.Bg) + ((size_t)rb * g.KB + (uint32_t)(ch & 1)) * kBlockBytes - (size_t)i * 1024u;
+    return (isA ? Tx.Ag : Tx.Bg) + ((size_t)rb * g.KB + (uint32_t)(ch & 1)) * kBlockBytes - (size_t)(i & 3) * 1024u;
+  };
+  // the wave's loads of one stage: lane offset voff inside the chunks, LDS address of its first chunk
+  auto load_stage = [&](const unsigned char* const* cb, uint32_t voff, uint32_t dst) {
+    if constexpr (kS != 4) dst = __builtin_amdgcn_readfirstlane(dst);  // (the ring position modulo 3 is formed on the vector ALU)
+    g16_load_4k(cb[0], cb[1], cb[2], cb[3], voff, dst);
+    if constexpr (kLoads == 6) g16_load_2k(cb[4], cb[5], voff, dst + 4096u);
   };
 
   const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)lds;
   const uint32_t a0 = lds_addr + (uint32_t)wrow * 8192u + lane_off;           // activation fragments, ring slot 0
   const uint32_t b0 = lds_addr + 16384u + (uint32_t)cgrp * 8192u + (uint32_t)chalf * 256u + lane_off;  // weight fragments, ring slot 0
-  const uint32_t dma0 = lds_addr + (uint32_t)wave * (kG16Loads * kBlockBytes);  // the wave's chunks, ring slot 0
+  const uint32_t dma0 = lds_addr + (uint32_t)wave * (kLoads * kBlockBytes);  // the wave's chunks, ring slot 0
   // per wave: f32 sx[128] then int32 src_row[128] of its rows, behind the stage ring
-  unsigned char* const rowdata = lds + kG16RingBytes + wave * 1024;  // (the waves of a row half hold the same data)
+  unsigned char* const rowdata = lds + Geo::kRingBytes + wave * 1024;  // (the waves of a row half hold the same data)
 
   // Raw buffer resources over the LoRA operands: loads through them take a uniform 64-bit base, a uniform
   // 32-bit offset and a 32-bit lane offset, so no lane holds a 64-bit address.
   const __amdgpu_buffer_rsrc_t zrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(g.zp), 0, -1, 0x00020000);
   const __amdgpu_buffer_rsrc_t brsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(g.bp), 0, -1, 0x00020000);
   uint32_t g0 = 0;          // ring slot of the current tile's stage 0
-  bool prefetched = false;  // the first four stages of the current tile were requested by the previous tile
-  for (uint32_t cur_i = blockIdx.x >> 3; cur_i < per_xcd; cur_i += wgs_per_xcd) {
+  bool prefetched = false;  // the first stages of the current tile were requested by the previous tile
+  // Two workgroups per CU: the one the dispatcher placed first (its LDS allocation starts at 0) runs at a
+  // higher wave priority.  Its main loop then takes every matrix-core slot it can use and the other
+  // workgroup fills the rest -- all of them while the first is in its epilogue -- instead of both running
+  // their main loops and then their epilogues side by side.  Positions beyond the first come from the
+  // XCD's counter, since the two no longer finish their tiles at the same rate.
+  constexpr bool kDyn = NW != 4;
+  uint32_t* const next_slot = reinterpret_cast<uint32_t*>(lds + Geo::kRingBytes + Geo::kWaves * 1024);
+  uint32_t* const ctr = g.tile_ctr + (blockIdx.x & 7u) * 16u;
+  uint32_t cur_i = blockIdx.x >> 3, nxt_i = cur_i + wgs_per_xcd;
+  if constexpr (kDyn) {
+    uint32_t lds_alloc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_LDS_ALLOC, 0, 8)" : "=s"(lds_alloc));
+    if (lds_alloc == 0u) __builtin_amdgcn_s_setprio(2);
+    else __builtin_amdgcn_s_setprio(0);
+    if (tid == 0) *next_slot = wgs_per_xcd + atomicAdd(ctr, 1u);
+    __syncthreads();
+  }
+  auto advance = [&]() {
+    cur_i = nxt_i;
+    if constexpr (!kDyn) nxt_i = cur_i + wgs_per_xcd;
+  };
+  for (; cur_i < per_xcd; advance()) {
     const GemmTile T = tile_at(cur_i);
-    if (!T.valid) { prefetched = false; continue; }
-    const uint32_t nxt_i = cur_i + wgs_per_xcd;
-    GemmTile Tn{};
-    if (nxt_i < per_xcd) Tn = tile_at(nxt_i);
-    const bool has_next = Tn.valid;  // workgroup-uniform
+    if (!T.valid) break;  // positions only grow: nothing valid follows
 
-    const unsigned char* cbase[kG16Loads];
+    const unsigned char* cbase[kLoads];
 #pragma unroll
-    for (int i = 0; i < kG16Loads; ++i) cbase[i] = chunk_base(T, i);
+    for (int i = 0; i < kLoads; ++i) cbase[i] = chunk_base(T, i);
 
     v4i acc[8][4];
     v4i bf[2][4];  // weight fragments of the current / next stage
     v4i af[4];     // activation fragments, three ahead of the MFMAs
     if (!prefetched) {
 #pragma unroll
-      for (int st = 0; st < kG16Stages; ++st) {
+      for (int st = 0; st < kS; ++st) {
         const uint32_t voff = (uint32_t)st * 2048u + (uint32_t)lane * 16u;
-        const uint32_t dst = dma0 + (((uint32_t)st + g0) & 3u) * kG16StageBytes;
-        g16_load_4k(cbase[0], cbase[1], cbase[2], cbase[3], voff, dst);
+        const uint32_t dst = dma0 + ring((uint32_t)st + g0) * kSB;
+        load_stage(cbase, voff, dst);
       }
     }
-    // Stage 0 must have landed.  Behind it in the queue: stages 1..3 (12 loads) and, when the previous
+    // Stage 0 must have landed.  Behind it in the queue: the other stages of the ring and, when the previous
     // tile requested them, that tile's epilogue, which is younger still.
-    g16_wait_vm<3 * kG16Loads>();
+    g16_wait_vm<(kS - 1) * kLoads>();
     lds_barrier();
+    if constexpr (kDyn) nxt_i = __builtin_amdgcn_readfirstlane(*reinterpret_cast<volatile uint32_t*>(next_slot));
+    GemmTile Tn{};
+    if (nxt_i < per_xcd) Tn = tile_at(nxt_i);
+    const bool has_next = Tn.valid;  // workgroup-uniform
 
     // LDS reads retire in order; the waits below count the reads issued behind the one they need.
     // Order here and at the end of every stage: B0..B3, A0, A1, A2.
     {
-      const uint32_t sa = a0 + ((g0 & 3u) << 15), sb = b0 + ((g0 & 3u) << 15);
+      const uint32_t sa = a0 + ring(g0) * kSB, sb = b0 + ring(g0) * kSB;
       g16_for<0, 4>([&](auto J) { bf[0][decltype(J)::value] = g16_ds_read<g16_bfrag_off(decltype(J)::value)>(sb); });
       af[0] = g16_ds_read<g16_frag_off(0)>(sa);
       af[1] = g16_ds_read<g16_frag_off(1)>(sa);
       af[2] = g16_ds_read<g16_frag_off(2)>(sa);
     }
 
-    const unsigned char* nbase[kG16Loads];
+    const unsigned char* nbase[kLoads];
 #pragma unroll
-    for (int i = 0; i < kG16Loads; ++i) nbase[i] = has_next ? chunk_base(Tn, i) : cbase[i];
+    for (int i = 0; i < kLoads; ++i) nbase[i] = has_next ? chunk_base(Tn, i) : cbase[i];
 
     // One stage: 32 MFMAs per wave.  Activation fragment bi + 3 is fetched under the MFMAs of fragment
     // bi; before fragment 6 the next stage must have landed (own loads counted, then the barrier), the
@@ -229,10 +282,10 @@ void w8a8_gemm16_kernel(GemmArgs g) {
       // compute every stage's addresses once at kernel start and keep them in registers (or spill them).
       uint32_t a0s = a0, b0s = b0;
       asm volatile("" : "+v"(a0s), "+v"(b0s));
-      const uint32_t slot = ((uint32_t)kt + g0) & 3u, slot_n = ((uint32_t)kt + 1u + g0) & 3u;
-      const uint32_t sa = a0s + (slot << 15);
-      const uint32_t san = a0s + (slot_n << 15);
-      const uint32_t sbn = b0s + (slot_n << 15);
+      const uint32_t slot = ring((uint32_t)kt + g0), slot_n = ring((uint32_t)kt + 1u + g0);
+      const uint32_t sa = a0s + slot * kSB;
+      const uint32_t san = a0s + slot_n * kSB;
+      const uint32_t sbn = b0s + slot_n * kSB;
       auto mfma_row = [&](auto BI) {
         constexpr int bi = decltype(BI)::value;
 #pragma unroll
@@ -258,12 +311,11 @@ void w8a8_gemm16_kernel(GemmArgs g) {
       // The next stage must have landed: own loads first, then everybody's; the barrier also ends every
       // wave's reads of this stage's buffer.  Three stages are in the queue behind this one as long as
       // the tile or a next tile provides them.
-      if constexpr (REM >= 3) {
-        g16_wait_vm<2 * kG16Loads>();
+      if constexpr (REM >= kS - 1) {
+        g16_wait_vm<(kS - 2) * kLoads>();
       } else if constexpr (REM >= 1) {
-        if (has_next) g16_wait_vm<2 * kG16Loads>();
-        else if constexpr (REM == 2) g16_wait_vm<kG16Loads>();
-        else g16_wait_vm<0>();
+        if (has_next) g16_wait_vm<(kS - 2) * kLoads>();
+        else g16_wait_vm<(REM - 1) * kLoads>();
       }
       lds_barrier();  // REM == 0: nothing has to land here; the barrier frees this stage's buffer
       // After the barrier the last 8 MFMAs start at once (their operands are in registers); the next
@@ -297,10 +349,10 @@ void w8a8_gemm16_kernel(GemmArgs g) {
       one(C6{}, integral_constant<int, 3>{});
       one(C7{}, integral_constant<int, 0>{});
       if constexpr (REM >= 1) af[2] = g16_ds_read<g16_frag_off(2)>(san);
-      if (REM >= 4 || (REM >= 1 && has_next)) {  // compile-time facts but has_next; the last stage issues none
-        const uint32_t voff4 = (uint32_t)(REM >= 4 ? kt + kG16Stages : kt + kG16Stages - KT) * 2048u + (uint32_t)lane * 16u;
-        if constexpr (REM >= 4) g16_load_4k(cbase[0], cbase[1], cbase[2], cbase[3], voff4, dma0 + (slot << 15));
-        else g16_load_4k(nbase[0], nbase[1], nbase[2], nbase[3], voff4, dma0 + (slot << 15));
+      if (REM >= kS || (REM >= 1 && has_next)) {  // compile-time facts but has_next; the last stage issues none
+        const uint32_t voff4 = (uint32_t)(REM >= kS ? kt + kS : kt + kS - KT) * 2048u + (uint32_t)lane * 16u;
+        if constexpr (REM >= kS) load_stage(cbase, voff4, dma0 + slot * kSB);
+        else load_stage(nbase, voff4, dma0 + slot * kSB);
       }
       one(C7{}, integral_constant<int, 1>{});
       one(C7{}, integral_constant<int, 2>{});
@@ -331,7 +383,7 @@ void w8a8_gemm16_kernel(GemmArgs g) {
     // ---- What the epilogue works with is set up here, behind the main loop's bulk, so that none of it
     // is live (or spilled) across the loop; preload() requests what it starts from.
     const uint32_t m0 = T.tm * 256u + wrow * 128u;     // first slot of the wave
-    const uint32_t tgrp0 = T.tn * 256u + cgrp * 128u;  // first column of the wave's group of 128
+    const uint32_t tgrp0 = T.tn * (uint32_t)Geo::kTileN + cgrp * 128u;  // first column of the wave's group of 128
     const uint32_t tcol0 = tgrp0 + chalf * 64u;        // first of the wave's 64 columns
     const bool wave_live = tcol0 < g.N;                // wave-uniform; a dead wave only feeds the loads
     const bool full_n = (tcol0 + 64u <= g.N) && ((g.N & 3u) == 0);  // wave-uniform
@@ -349,6 +401,7 @@ void w8a8_gemm16_kernel(GemmArgs g) {
       for (int bj = 0; bj < 4; ++bj) br[bj][ks] = zero4;
     }
     int bgroup = -1;
+    float bscale = 0.0f;  // lora_scaling[bgroup]
     // operand bytes inside a 1 KiB block of the 32 x 16 layouts the prologue writes: rank octet q sits in
     // rank chunk q / 2 (16 ranks each), half q % 2.  A rank chunk beyond the rank is read from the last
     // existing one and zeroed afterwards.
@@ -385,13 +438,18 @@ void w8a8_gemm16_kernel(GemmArgs g) {
         for (int ks = 0; ks < kKS; ++ks)
           br[bj][ks] = lane_has_rank[ks] ? __builtin_amdgcn_raw_buffer_load_b128(brsrc, blane[ks], b_soff(gi, bj), 0) : zero4;
       bgroup = gi;
+      // the adapter's scaling through the scalar path, once per adapter: a vector load at its use would be
+      // waited for with vmcnt(0), behind the operand loads of the fragments to come and the next tile's stage
+      asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(bscale) : "s"(g.lora_scaling + gi) : "memory");
     };
     // What the epilogue starts from is requested at the start of the last stage, with loads the compiler
     // keeps its books on (it places the waits and may move the values as it likes).  No stage load is
     // issued behind them before they are waited for, so that wait does not stall on a younger load.
+    uint32_t grabbed = 0;  // the position after next of a dynamic schedule, requested with the epilogue's operands
     auto preload = [&]() {
-      if (EPI != kEpiAcc) g16_load_128_dwords(g.sx + m0, (uint32_t)lane * 4u, lds_addr + kG16RingBytes + wave * 1024);
-      if (g.src_row) g16_load_128_dwords(g.src_row + m0, (uint32_t)lane * 4u, lds_addr + kG16RingBytes + wave * 1024 + 512);
+      if (kDyn && tid == 0) grabbed = atomicAdd(ctr, 1u);
+      if (EPI != kEpiAcc) g16_load_128_dwords(g.sx + m0, (uint32_t)lane * 4u, lds_addr + Geo::kRingBytes + wave * 1024);
+      if (g.src_row) g16_load_128_dwords(g.src_row + m0, (uint32_t)lane * 4u, lds_addr + Geo::kRingBytes + wave * 1024 + 512);
       if (!wave_live) return;
       if (EPI != kEpiAcc && full_n) swr = *reinterpret_cast<const v4i*>(T.swp + tcol0 + 4u * c16);
       if constexpr (kLora) {
@@ -407,11 +465,12 @@ void w8a8_gemm16_kernel(GemmArgs g) {
     // (the builtin, so that the compiler knows its loads are in) the next tile's fourth stage is requested
     // into the buffer the last barrier has freed.
     wait_vmcnt<0>();
+    if (kDyn && tid == 0) *next_slot = wgs_per_xcd + grabbed;  // read by every wave behind the next tile's first barrier
     if (has_next) {
-      const uint32_t voff = 3u * 2048u + (uint32_t)lane * 16u;
-      g16_load_4k(nbase[0], nbase[1], nbase[2], nbase[3], voff, dma0 + ((((uint32_t)KT - 1u + g0) & 3u) << 15));
+      const uint32_t voff = (uint32_t)(kS - 1) * 2048u + (uint32_t)lane * 16u;
+      load_stage(nbase, voff, dma0 + ring((uint32_t)KT - 1u + g0) * kSB);
     }
-    g0 = (g0 + (uint32_t)KT) & 3u;
+    g0 = ring(g0 + (uint32_t)KT);
     prefetched = has_next;
 
     // ---------------------------------------------------------------- epilogue
@@ -485,7 +544,7 @@ void w8a8_gemm16_kernel(GemmArgs g) {
           v4f_t low[4];
           if constexpr (kLora) {
             if (gi != bgroup) load_b(gi);  // wave-uniform: a new adapter begins in this fragment
-            const float sgrp = g.lora_scaling[gi];
+            const float sgrp = bscale;
 #pragma unroll
             for (int bj = 0; bj < 4; ++bj) low[bj] = v4f_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -499,10 +558,12 @@ void w8a8_gemm16_kernel(GemmArgs g) {
             // the low-rank accumulators live in ordinary registers: every accumulation register is taken,
             // and left to itself the compiler spills one of the integer accumulators to make room
             asm volatile("" : "+v"(low[0]), "+v"(low[1]), "+v"(low[2]), "+v"(low[3]));
+            if (sgrp != 1.0f) {  // wave-uniform (a product with 1 is exact: leaving it out changes no bit)
 #pragma unroll
-            for (int bj = 0; bj < 4; ++bj)
+              for (int bj = 0; bj < 4; ++bj)
 #pragma unroll
-              for (int v = 0; v < 4; ++v) low[bj][v] = low[bj][v] * sgrp;
+                for (int v = 0; v < 4; ++v) low[bj][v] = low[bj][v] * sgrp;
+            }
           }
           {
 #pragma unroll

@@ -757,13 +757,16 @@ __global__ __launch_bounds__(1024) void lora_a_kernel(LoraAArgs a) {
 
 // ---------------------------------------------------------------------------------------
 // Quantizer and LoRA-A projection in one pass over x (the dense path's prologue).
-// One workgroup of 16 waves per 16 grouped slots (half a 32-row block):
-//   1. wave w owns slot row w: (RMSNorm statistics,) absmax of the (normalized) row -> scale;
-//   2. the waves split K in 32-wide blocks; lane (i = lane % 16, q = lane / 16) takes the 8 values
-//      k = 32 kb + 8 q .. +7 of row i, normalizes them exactly as step 1 did, and uses them twice:
-//      as int8 codes written into the activation's 1 KiB fragment block, and as the A operand of
-//      v_mfma_f32_16x16x32_bf16 against the transposed LoRA A of the row's group, so the
-//      normalized rows never travel through memory;
+// One workgroup of 16 waves per R grouped slots (R = 16, or 8 / 4 / 2 when longer rows would not fit the
+// LDS: half a 32-row block or a part of one):
+//   1. wave w < R copies slot row w from memory into the LDS with direct-to-LDS loads -- the only
+//      time x is read -- and takes its statistics from there: (RMSNorm sum of squares, the row normalized
+//      in place,) absmax -> scale;
+//   2. the waves split K in 32-wide blocks; lane (i = lane % 16, q = lane / 16) takes the 8 (normalized)
+//      values k = 32 kb + 8 q .. +7 of row i from the LDS and uses them twice: as int8 codes written into
+//      the activation's 1 KiB fragment block, and as the A operand of v_mfma_f32_16x16x32_bf16 against the
+//      LoRA A of the row's group in that instruction's operand order, so the normalized rows never travel
+//      through memory;
 //   3. the waves' z tiles are added in a fixed order, split exactly into three bf16 terms and
 //      stored in the operand order the GEMM epilogue reads (see lora_a_kernel).
 // Arithmetic follows quant_rows_kernel (skyrl/tx/kernels/quantized_lora.py:199-212 and the
@@ -792,9 +795,28 @@ struct QuantLoraArgs {
   const int32_t* route_idx; // adapter per row
   uint32_t n_groups, slots;
   uint32_t group_pad;       // every group's first slot is a multiple of this (1: groups packed; 32: no block holds two groups)
+  uint32_t rows_per_wg;     // R: 16, 8, 4 or 2 slots per workgroup (quant_lora_rows_per_wg)
+  uint32_t row_stride;      // bytes between two rows in the LDS (quant_lora_row_stride)
 };
 
 constexpr uint32_t kInlineRouteMaxRows = 8192;  // eight rows per thread of a 1024-thread workgroup
+
+// LDS bytes of a row: its 2 K bytes rounded up to the 1 KiB a wave's direct-to-LDS load moves, plus 16 so
+// that the sixteen rows a wave reads side by side in step 2 (16 bytes each) fall on sixteen different
+// bank groups.
+__host__ __device__ inline uint32_t quant_lora_row_stride(uint32_t k) { return round_up(2u * k, 1024u) + 16u; }
+constexpr uint32_t kQuantLoraLdsBudget = 150u * 1024u;  // rows + reduction tiles; the rest of the 160 KiB is static
+__host__ __device__ inline uint32_t quant_lora_rows_per_wg(uint32_t k) {
+  uint32_t r = 16u;
+  while (r > 2u && r * quant_lora_row_stride(k) > kQuantLoraLdsBudget) r >>= 1;
+  return r;
+}
+// dynamic LDS of a launch: the rows, or the reduction tiles that reuse the same bytes once the rows are spent
+__host__ __device__ inline uint32_t quant_lora_lds_bytes(uint32_t k, uint32_t cb) {
+  const uint32_t rows = quant_lora_rows_per_wg(k) * quant_lora_row_stride(k);
+  const uint32_t red = 8u * (cb ? cb : 1u) * 4u * 64u * 4u;
+  return rows > red ? rows : red;
+}
 
 // The routing tables of route_rows_block for the 16 slots [16 hb, 16 hb + 16), computed by the
 // workgroup itself: rows keep their order inside a group (slot start[g] + j holds the j-th row of group
@@ -804,19 +826,21 @@ constexpr uint32_t kInlineRouteMaxRows = 8192;  // eight rows per thread of a 10
 // the next group's first stay empty, src -1), so no 32-slot block holds rows of two groups: neither
 // this kernel nor the GEMM's epilogue then runs a block once per group.  The slots in use end at
 // sum(round_up(count, group_pad)) <= M + (group_pad - 1) * min(n_groups, M).
+// Steps: every wave counts its rows per group (LDS atomics on its own counters: with 16 waves on a CU
+// the vector ALU's share per wave makes a ballot per group and row several times dearer); wave 0 turns
+// the counts into per-wave prefixes, the groups' first slots and the groups of the sixteen slots; the
+// waves that hold the wanted ranks of a group pick their rows.  Three barriers.
 __device__ inline void route_rows_inline(const int32_t* __restrict__ idx, uint32_t M, uint32_t n_groups,
                                          uint32_t slots, uint32_t group_pad, uint32_t hb, int* out_src, int* out_grp,
                                          uint32_t* out_range, int* out_last_group) {
-  __shared__ int cnt[kMaxAdapters];
+  __shared__ int wcnt[kMaxAdapters][17];  // rows of group g in wave w; then the exclusive prefix over the waves
   __shared__ int start[kMaxAdapters + 1];
+  __shared__ int cnt[kMaxAdapters];
   __shared__ uint32_t used_end;  // first slot behind the last group
-  __shared__ int wave_cnt[16];
-  __shared__ int last_nonempty;
-  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  __shared__ int g_first_s, g_last_s;
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t per = (M + 1023u) / 1024u;  // consecutive rows per thread (<= 8)
-  if (tid < (uint32_t)kMaxAdapters) cnt[tid] = 0;
-  if (tid < 16u) { out_src[tid] = -1; out_grp[tid] = 0; }
-  __syncthreads();
   int mine[8];
 #pragma unroll
   for (uint32_t j = 0; j < 8; ++j) {
@@ -825,89 +849,126 @@ __device__ inline void route_rows_inline(const int32_t* __restrict__ idx, uint32
     if (j < per && i < M) {
       a = idx[i];
       a = a < 0 ? 0 : (a >= (int)n_groups ? (int)n_groups - 1 : a);
-      atomicAdd(&cnt[a], 1);  // integer counts: the order of the additions does not matter
     }
     mine[j] = a;
   }
+  if (lane < n_groups) wcnt[lane][wave] = 0;  // (the loads above are still in flight)
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (uint32_t j = 0; j < 8; ++j)
+    if (j < per && mine[j] >= 0) atomicAdd(&wcnt[mine[j]][wave], 1);  // integer counts of one wave: any order
   __syncthreads();
-  if (tid == 0) {
-    int pos = 0, last = 0;
-    for (uint32_t a = 0; a < n_groups; ++a) {
-      start[a] = pos;
-      pos += (int)round_up((uint32_t)cnt[a], group_pad);
-      if (cnt[a] > 0) last = (int)a;
-    }
-    start[n_groups] = pos;
-    used_end = (uint32_t)pos;
-    last_nonempty = last;
-    *out_last_group = last;
-  }
-  __syncthreads();
-  const uint32_t E = used_end;
-  // group of a slot: the group whose [start, start + count) holds it; padding slots follow the last
-  // non-empty group
-  auto group_of = [&](uint32_t p) -> int {
-    if (p >= E) return last_nonempty;
-    int g = 0;
-    for (uint32_t a = 0; a < n_groups; ++a)
-      if ((int)p >= start[a] && (int)p < start[a + 1]) g = (int)a;
-    return g;
-  };
   const uint32_t p0 = hb * 16u;
-  if (tid < 16u) out_grp[tid] = group_of(p0 + tid);
-  if (tid == 16u) {
+  if (wave == 0) {  // lane g: group g (n_groups <= 64)
+    int total = 0;
+    if (lane < n_groups) {
+      int c[16];
+#pragma unroll
+      for (uint32_t w = 0; w < 16; ++w) c[w] = wcnt[lane][w];  // all reads first: one round trip
+#pragma unroll
+      for (uint32_t w = 0; w < 16; ++w) {
+        wcnt[lane][w] = total;
+        total += c[w];
+      }
+    }
+    const int padded = (int)round_up((uint32_t)total, group_pad);
+    int incl = padded;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int up = __shfl_up(incl, off, 64);
+      if ((int)lane >= off) incl += up;
+    }
+    const int st = incl - padded;  // first slot of group `lane`
+    const uint32_t E = (uint32_t)__shfl(incl, 63, 64);
+    const unsigned long long nonempty = __builtin_amdgcn_ballot_w64(total > 0);
+    const int last_ne = nonempty ? 63 - __builtin_clzll(nonempty) : 0;
+    if (lane < n_groups) { start[lane] = st; cnt[lane] = total; }
+    if (lane == 0) { start[n_groups] = (int)E; used_end = E; *out_last_group = last_ne; }
+    // group of a slot: the last group whose first slot is not behind it (empty groups share their
+    // successor's first slot, so the last one is the one that holds the slot); slots behind the last
+    // group follow the last non-empty one
+    auto group_of = [&](uint32_t p) -> int {
+      if (p >= E) return last_ne;
+      const unsigned long long m = __builtin_amdgcn_ballot_w64(lane < n_groups && (uint32_t)st <= p);
+      return m ? 63 - __builtin_clzll(m) : 0;
+    };
+    const uint32_t p_end = (p0 + 16u < E) ? p0 + 16u : E;
+    const int gf = group_of(p0), gl = group_of(p_end ? p_end - 1u : 0u);
+    int my_grp = group_of(p0 + 15u);  // (the slots behind the last group follow the last non-empty one)
+    if (my_grp != gf) {  // wave-uniform: the sixteen slots hold a group boundary (or the end)
+#pragma unroll
+      for (uint32_t s16 = 0; s16 < 16; ++s16) {
+        const int g = group_of(p0 + s16);
+        if (lane == s16) my_grp = g;
+      }
+    }
+    if (lane < 16u) { out_grp[lane] = my_grp; out_src[lane] = -1; }
     const uint32_t b0 = (p0 / 32u) * 32u;
     const uint32_t b1 = (b0 + 31u < E) ? b0 + 31u : (E ? E - 1u : 0u);
-    *out_range = b0 >= E ? 0u : ((uint32_t)group_of(b0) | ((uint32_t)group_of(b1) << 16));
+    const int gb0 = group_of(b0), gb1 = group_of(b1);
+    if (lane == 0) {
+      *out_range = b0 >= E ? 0u : ((uint32_t)gb0 | ((uint32_t)gb1 << 16));
+      g_first_s = p0 < E ? gf : 1;  // an empty range when the slots lie behind the last group
+      g_last_s = p0 < E ? gl : 0;
+    }
   }
+  __syncthreads();
   // the rows of the slots in use, group by group (a workgroup's 16 slots usually lie in one group)
+  const uint32_t E = used_end;
   const uint32_t p_end = (p0 + 16u < E) ? p0 + 16u : E;
-  if (p0 < E) {
-    const int g_first = group_of(p0), g_last = group_of(p_end - 1u);
-    for (int g = g_first; g <= g_last; ++g) {  // workgroup-uniform
-      if (cnt[g] == 0) continue;
-      int c = 0;
+  const int g_first = g_first_s, g_last = g_last_s;
+  for (int g = g_first; g <= g_last; ++g) {  // workgroup-uniform
+    const int cg = cnt[g], sg = start[g];
+    if (cg == 0) continue;
+    // slots of group g among mine: ranks [lo, hi)
+    const int lo = ((int)p0 > sg ? (int)p0 : sg) - sg;
+    const int hi = ((int)p_end < sg + cg ? (int)p_end : sg + cg) - sg;
+    const int wbefore = wcnt[g][wave];
+    const int wafter = wave < 15u ? wcnt[g][wave + 1u] : cg;
+    if (hi <= lo || wafter <= lo || wbefore >= hi) continue;  // wave-uniform: none of the wanted ranks is in this wave
+    int c = 0;
 #pragma unroll
-      for (uint32_t j = 0; j < 8; ++j) c += (mine[j] == g) ? 1 : 0;
-      // exclusive prefix of c over the threads in thread order: inside the wave, then across waves
-      int incl = c;
+    for (uint32_t j = 0; j < 8; ++j) c += (mine[j] == g) ? 1 : 0;
+    int incl = c;
 #pragma unroll
-      for (int off = 1; off < 64; off <<= 1) {
-        const int up = __shfl_up(incl, off, 64);
-        if ((int)lane >= off) incl += up;
-      }
-      __syncthreads();  // wave_cnt is free
-      if (lane == 63u) wave_cnt[wave] = incl;
-      __syncthreads();
-      int before = incl - c;
-      for (uint32_t w = 0; w < wave; ++w) before += wave_cnt[w];
-      // slots of group g among mine: ranks [lo, hi)
-      const int lo = ((int)p0 > start[g] ? (int)p0 : start[g]) - start[g];
-      const int hi = ((int)p_end < start[g] + cnt[g] ? (int)p_end : start[g] + cnt[g]) - start[g];
-      int rank = before;
+    for (int off = 1; off < 64; off <<= 1) {
+      const int up = __shfl_up(incl, off, 64);
+      if ((int)lane >= off) incl += up;
+    }
+    int rank = wbefore + incl - c;
 #pragma unroll
-      for (uint32_t j = 0; j < 8; ++j) {
-        if (mine[j] == g) {
-          if (rank >= lo && rank < hi) out_src[start[g] + rank - (int)p0] = (int)(tid * per + j);
-          ++rank;
-        }
+    for (uint32_t j = 0; j < 8; ++j) {
+      if (mine[j] == g) {
+        if (rank >= lo && rank < hi) out_src[sg + rank - (int)p0] = (int)(tid * per + j);
+        ++rank;
       }
     }
   }
   __syncthreads();
 }
 
+// One direct-to-LDS load of 1 KiB by a wave: lane l moves global[base + voff] (voff = 1024 u + 16 l) to
+// LDS[lds_addr_uniform + 16 l]; inactive lanes move nothing.
+__device__ inline void ql_load_1k(const unsigned char* base_uniform, uint32_t voff, uint32_t lds_addr_uniform) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :: "v"(voff), "s"(base_uniform), "s"(lds_addr_uniform) : "memory", "m0");
+}
+
 template <int CB, bool RMS>  // CB: 16-wide rank blocks (0 = no LoRA, 1, 2, 4)
 __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
   constexpr int kCB = CB > 0 ? CB : 1;
-  __shared__ float row_inv[16], row_scale[16];
+  extern __shared__ __attribute__((aligned(1024))) unsigned char ql_lds[];  // the rows; later the wave tiles of z
+  __shared__ float row_scale[16];
   __shared__ int row_src[16];
-  __shared__ float red[8][kCB][4][64];     // wave tiles on their way to waves 0..7, then 0..3
   __shared__ float zs[16][kCB * 16 + 1];
+  typedef float red_t[kCB][4][64];  // wave tiles on their way to waves 0..7, then 0..3
+  red_t* const red = reinterpret_cast<red_t*>(ql_lds);
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const uint32_t hb = blockIdx.x;  // half block: slots 16 hb .. 16 hb + 15
-  if (a.tile_ctr && hb == 0 && tid < 256u) a.tile_ctr[tid] = 0u;
+  const uint32_t R = a.rows_per_wg, per_hb = 16u / R;
+  const uint32_t hb = blockIdx.x / per_hb;           // half block: slots 16 hb .. 16 hb + 15
+  const uint32_t r0 = (blockIdx.x % per_hb) * R;     // this workgroup's slots inside it: r0 .. r0 + R - 1
+  if (a.tile_ctr && blockIdx.x == 0 && tid < 256u) a.tile_ctr[tid] = 0u;
   if (hb >= a.n_half_blocks) return;
   const uint32_t pb = hb >> 1, half16 = hb & 1u;
   __shared__ int route_src[16], route_grp[16], route_last_group;
@@ -916,107 +977,120 @@ __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
   if (route_here) {
     route_rows_inline(a.route_idx, a.M, a.n_groups, a.slots, a.group_pad, hb, route_src, route_grp, &route_range,
                       &route_last_group);
-    // the tables the GEMM reads later
-    if (tid < 16u) {
+    // the tables the GEMM reads later (every workgroup of a half block derives the same values)
+    if (tid >= r0 && tid < r0 + R) {
       const_cast<int32_t*>(a.src_row)[hb * 16u + tid] = route_src[tid];
       const_cast<int32_t*>(a.slot_group)[hb * 16u + tid] = route_grp[tid];
     }
-    if (tid == 16u) const_cast<int32_t*>(a.blk_range)[pb] = (int32_t)route_range;  // both halves write the same value
-    if (hb + 1u == a.n_half_blocks) {  // the padding slots behind the last 32-row block, up to the GEMM's tile rows
+    if (tid == 16u) const_cast<int32_t*>(a.blk_range)[pb] = (int32_t)route_range;  // (the same value from each)
+    if (blockIdx.x + 1u == gridDim.x) {  // the padding slots behind the last 32-row block, up to the GEMM's tile rows
       for (uint32_t p = a.n_half_blocks * 16u + tid; p < a.slots; p += 1024u) {
         const_cast<int32_t*>(a.src_row)[p] = -1;
         const_cast<int32_t*>(a.slot_group)[p] = route_last_group;
         if ((p & 31u) == 0) const_cast<int32_t*>(a.blk_range)[p / 32u] = 0;
       }
     }
-    if (a.group_pad > 1u) {  // padded groups leave whole half blocks empty: nothing reads their codes, scales or z
-      int any = 0;
-#pragma unroll
-      for (int j = 0; j < 16; ++j) any |= (route_src[j] >= 0) ? 1 : 0;
-      if (!any) return;  // workgroup-uniform
-    }
   }
-
-  if (!route_here && a.group_pad > 1u && a.src_row) {  // the same for tables a routing block has written
+  if (a.group_pad > 1u && (route_here || a.src_row)) {
+    // padded groups leave whole stretches of slots empty: nothing reads their codes, scales or z
     int any = 0;
-#pragma unroll
-    for (uint32_t j = 0; j < 16; ++j) any |= (a.src_row[hb * 16u + j] >= 0) ? 1 : 0;
+    for (uint32_t j = r0; j < r0 + R; ++j) any |= ((route_here ? route_src[j] : a.src_row[hb * 16u + j]) >= 0) ? 1 : 0;
     if (!any) return;  // workgroup-uniform
   }
-
-  // ---- 1. row statistics: wave w, slot row w
-  {
-    const uint32_t p = hb * 16u + wave;
-    int src = route_here ? route_src[wave] : (a.src_row ? a.src_row[p] : (int)p);
+  // ---- 1. the rows into the LDS and their statistics: wave w, slot row r0 + w
+  const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)ql_lds;
+  const uint32_t row_bytes = 2u * a.K;
+  const uint32_t n_chunks = (row_bytes + 1023u) / 1024u;  // 1 KiB pieces of a row (the last one may be partial)
+  if (wave < R) {
+    const uint32_t sl = r0 + wave;
+    const uint32_t p = hb * 16u + sl;
+    int src = route_here ? route_src[sl] : (a.src_row ? a.src_row[p] : (int)p);
     if (src < 0 || src >= (int)a.M) src = -1;
-    float inv = 1.0f, amax = 0.0f;
+    src = __builtin_amdgcn_readfirstlane(src);
+    unsigned char* const rowl = ql_lds + wave * a.row_stride;
+    float inv = 1.0f;
+    uint32_t amax_bits = 0;  // largest |value| as bf16 bits in both halves
     if (src >= 0) {
-      const uint16_t* xr = a.x + (size_t)src * a.K;
-      // eight 16-byte loads of the row are in flight at a time
+      const unsigned char* xr = reinterpret_cast<const unsigned char*>(a.x) + (size_t)src * row_bytes;
+      const uint32_t row_lds = lds_addr + wave * a.row_stride;
+      for (uint32_t u = 0; u < n_chunks; ++u) {
+        const uint32_t voff = u * 1024u + lane * 16u;
+        if (voff < row_bytes) ql_load_1k(xr, voff, row_lds + u * 1024u);
+      }
+      // (the first chunk's norm weights travel with the row)
+      float4 gn0 = make_float4(0.f, 0.f, 0.f, 0.f), gn1 = gn0;
+      if (RMS && lane * 16u < row_bytes) {
+        gn0 = *reinterpret_cast<const float4*>(a.gamma + lane * 8u);
+        gn1 = *reinterpret_cast<const float4*>(a.gamma + lane * 8u + 4);
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       if (RMS) {
         double ss = 0.0;
-        for (uint32_t kbase = 0; kbase < a.K; kbase += 4096u) {
-          uint4 raw[8];
+        for (uint32_t u = 0; u < n_chunks; ++u) {
+          const uint32_t off = u * 1024u + lane * 16u;
+          const uint4 raw = off < row_bytes ? *reinterpret_cast<const uint4*>(rowl + off) : make_uint4(0, 0, 0, 0);
+          const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
-          for (uint32_t u = 0; u < 8; ++u) {
-            const uint32_t k0 = kbase + (u * 64u + lane) * 8u;
-            raw[u] = k0 < a.K ? *reinterpret_cast<const uint4*>(xr + k0) : make_uint4(0, 0, 0, 0);
-          }
-#pragma unroll
-          for (uint32_t u = 0; u < 8; ++u) {
-            const uint32_t w[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              // the square of a bf16 value is exact in double, so the fused form rounds like mul + add
-              const double lo = (double)__uint_as_float(w[e] << 16), hi = (double)__uint_as_float(w[e] & 0xffff0000u);
-              ss = __builtin_fma(lo, lo, ss);
-              ss = __builtin_fma(hi, hi, ss);
-            }
+          for (int e = 0; e < 4; ++e) {
+            // the square of a bf16 value is exact in double, so the fused form rounds like mul + add
+            const double lo = (double)__uint_as_float(w[e] << 16), hi = (double)__uint_as_float(w[e] & 0xffff0000u);
+            ss = __builtin_fma(lo, lo, ss);
+            ss = __builtin_fma(hi, hi, ss);
           }
         }
         ss = wave_sum(ss);
         const float var = (float)(ss / (double)a.K);
         inv = 1.0f / sqrtf(var + a.eps);
       }
-      for (uint32_t kbase = 0; kbase < a.K; kbase += 4096u) {
-        uint4 raw[8];
-#pragma unroll
-        for (uint32_t u = 0; u < 8; ++u) {
-          const uint32_t k0 = kbase + (u * 64u + lane) * 8u;
-          raw[u] = k0 < a.K ? *reinterpret_cast<const uint4*>(xr + k0) : make_uint4(0, 0, 0, 0);
-        }
-#pragma unroll
-        for (uint32_t u = 0; u < 8; ++u) {
-          const uint32_t k0 = kbase + (u * 64u + lane) * 8u;
-          const uint32_t w[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
-          float g[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f};
-          if (RMS && k0 < a.K) {
-            const float4 g0 = *reinterpret_cast<const float4*>(a.gamma + k0);
-            const float4 g1 = *reinterpret_cast<const float4*>(a.gamma + k0 + 4);
-            g[0] = g0.x; g[1] = g0.y; g[2] = g0.z; g[3] = g0.w; g[4] = g1.x; g[5] = g1.y; g[6] = g1.z; g[7] = g1.w;
+      for (uint32_t u = 0; u < n_chunks; ++u) {
+        const uint32_t off = u * 1024u + lane * 16u;
+        float4 g0 = gn0, g1 = gn1;
+        if (RMS) {  // the norm weights of the next chunk are requested before this one is worked on
+          const uint32_t offn = off + 1024u;
+          if (offn < row_bytes) {
+            gn0 = *reinterpret_cast<const float4*>(a.gamma + (offn >> 1));
+            gn1 = *reinterpret_cast<const float4*>(a.gamma + (offn >> 1) + 4);
           }
+        }
+        if (off >= row_bytes) continue;
+        uint4 raw = *reinterpret_cast<const uint4*>(rowl + off);
+        if (RMS) {
+          const float g[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+          uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            float v0 = __uint_as_float(w[e] << 16), v1 = __uint_as_float(w[e] & 0xffff0000u);
-            if (RMS) {
-              float t0 = v0 * inv, t1 = v1 * inv;
-              t0 = t0 * g[2 * e];
-              t1 = t1 * g[2 * e + 1];
-              const uint32_t pk = pack_bf16x2(t0, t1);
-              v0 = __uint_as_float(pk << 16);
-              v1 = __uint_as_float(pk & 0xffff0000u);
-            }
-            amax = fmaxf(amax, fmaxf(fabsf(v0), fabsf(v1)));
+            float t0 = __uint_as_float(w[e] << 16) * inv, t1 = __uint_as_float(w[e] & 0xffff0000u) * inv;
+            t0 = t0 * g[2 * e];
+            t1 = t1 * g[2 * e + 1];
+            w[e] = pack_bf16x2(t0, t1);
           }
+          raw = make_uint4(w[0], w[1], w[2], w[3]);
+          *reinterpret_cast<uint4*>(rowl + off) = raw;  // the normalized row replaces the row
+          if (a.xn_aux) *reinterpret_cast<uint4*>(reinterpret_cast<unsigned char*>(a.xn_aux) + (size_t)src * row_bytes + off) = raw;
         }
+        // |bf16| compares like its 15 magnitude bits as an integer (a NaN ends above every number and the
+        // scale then falls back to 1, as the reference's comparison amax > 0 does)
+        const uint32_t m0 = raw.x & 0x7fff7fffu, m1 = raw.y & 0x7fff7fffu, m2 = raw.z & 0x7fff7fffu, m3 = raw.w & 0x7fff7fffu;
+        typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+        us2 mx = __builtin_bit_cast(us2, amax_bits);
+        mx = __builtin_elementwise_max(mx, __builtin_bit_cast(us2, m0));
+        mx = __builtin_elementwise_max(mx, __builtin_bit_cast(us2, m1));
+        mx = __builtin_elementwise_max(mx, __builtin_bit_cast(us2, m2));
+        mx = __builtin_elementwise_max(mx, __builtin_bit_cast(us2, m3));
+        amax_bits = __builtin_bit_cast(uint32_t, mx);
       }
-      amax = wave_max(amax);
     }
+    uint32_t top = (amax_bits >> 16) > (amax_bits & 0xffffu) ? (amax_bits >> 16) : (amax_bits & 0xffffu);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const uint32_t other = (uint32_t)__shfl_xor((int)top, o, 64);
+      top = other > top ? other : top;
+    }
+    const float amax = __uint_as_float(top << 16);
     const float scale = amax > 0.0f ? amax / 127.0f : 1.0f;
     if (lane == 0) {
-      row_inv[wave] = inv;
-      row_scale[wave] = scale;
-      row_src[wave] = src;
+      row_scale[sl] = scale;
+      row_src[sl] = src;
       a.sx_slots[p] = scale;
       if (a.scales_rm && src >= 0) a.scales_rm[src] = scale;
     }
@@ -1025,10 +1099,11 @@ __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
 
   // ---- 2. codes and z
   const uint32_t i = lane & 15u, q = lane >> 4;
-  const int src = row_src[i];
-  const float inv = row_inv[i], scale = row_scale[i];
+  const bool mine_row = i >= r0 && i < r0 + R;  // slot row i belongs to this workgroup
+  const int src = mine_row ? row_src[i] : -1;
+  const float scale = mine_row ? row_scale[i] : 1.0f;
   const float rscale = __builtin_amdgcn_rcpf(scale);
-  const uint16_t* xr = a.x + (size_t)(src < 0 ? 0 : src) * a.K;
+  const unsigned char* const rowl = ql_lds + (mine_row ? i - r0 : 0u) * a.row_stride;
   const uint32_t range = CB == 0 ? 0u : (route_here ? route_range : (a.blk_range ? (uint32_t)a.blk_range[pb] : 0u));
   const uint32_t glo = range & 0xffffu, ghi = range >> 16;
   const uint32_t rowgrp = (CB > 0 && ghi > glo)
@@ -1039,131 +1114,110 @@ __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
   for (int b = 0; b < kCB; ++b) acc[b] = v4f{0.f, 0.f, 0.f, 0.f};
   // fragment block byte offset of this lane's 8 codes: row 16*half16 + i, k half q/2, byte 8*(q%2)
   const uint32_t code_off = (16u * half16 + i + 32u * (q >> 1)) * 16u + 8u * (q & 1u);
-  for (uint32_t kb0 = wave; kb0 < a.KB; kb0 += 32u) {  // two k-blocks per round, all loads first
-    uint4 raw2[2];
-    float4 gm[2][2];
-    v4i wpre[2][kCB];
+  // One pass over the k-blocks per group present among the slots (one, except at a group boundary): the
+  // first pass also forms the codes; a later pass only adds the rows of its group to z (the rows are still
+  // in the LDS).  The loop is kept rolled, two k-blocks per trip with their operands requested one trip
+  // ahead and no load inside the work on a k-block, so that the compiler's waits count loads instead of
+  // draining them.
+  auto request = [&](uint32_t grp, uint32_t kb, v4i (&w)[kCB], uint4& raw) {
+    if constexpr (CB > 0) {
+      // operands of group grp, k-block kb: CB consecutive 1 KiB pieces (zero beyond K and the rank)
+      const v4i* ap = reinterpret_cast<const v4i*>(a.at) + (((size_t)grp * a.KB + kb) * CB) * 64u + lane;
 #pragma unroll
-    for (uint32_t u = 0; u < 2; ++u) {
-      const uint32_t kb = kb0 + 16u * u;
-      const uint32_t k0 = kb * 32u + q * 8u;
-      const bool inK = kb < a.KB && k0 < a.K;
-      raw2[u] = (inK && src >= 0) ? *reinterpret_cast<const uint4*>(xr + k0) : make_uint4(0, 0, 0, 0);
-      if (RMS) {
-        gm[u][0] = inK ? *reinterpret_cast<const float4*>(a.gamma + k0) : make_float4(0.f, 0.f, 0.f, 0.f);
-        gm[u][1] = inK ? *reinterpret_cast<const float4*>(a.gamma + k0 + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
-      }
-      if constexpr (CB > 0) {
-        // operands of group glo, k-block kb: CB consecutive 1 KiB pieces (zero beyond K and the rank)
-        const v4i* ap = reinterpret_cast<const v4i*>(a.at) + (((size_t)glo * a.KB + kb) * CB) * 64u + lane;
-#pragma unroll
-        for (int b = 0; b < CB; ++b) wpre[u][b] = kb < a.KB ? ap[b * 64] : v4i{0, 0, 0, 0};
-      }
+      for (int b = 0; b < CB; ++b) w[b] = kb < a.KB ? ap[b * 64] : v4i{0, 0, 0, 0};
     }
-#pragma unroll
-    for (uint32_t u = 0; u < 2; ++u) {
-      const uint32_t kb = kb0 + 16u * u;
-      if (kb >= a.KB) break;  // wave-uniform
+    const uint32_t k0 = kb * 32u + q * 8u;
+    raw = (kb < a.KB && k0 < a.K && src >= 0) ? *reinterpret_cast<const uint4*>(rowl + 2u * k0) : make_uint4(0, 0, 0, 0);
+  };
+  auto work = [&](bool first, bool in_group, uint32_t kb, const v4i (&w)[kCB], const uint4& raw) {
+    if (first) {  // wave-uniform
       const uint32_t k0 = kb * 32u + q * 8u;
       const bool live = src >= 0 && k0 < a.K;  // K is a multiple of 8
-      uint32_t nb[4] = {raw2[u].x, raw2[u].y, raw2[u].z, raw2[u].w};  // the (normalized) values as bf16 pairs
+      const uint32_t nb[4] = {raw.x, raw.y, raw.z, raw.w};  // the (normalized) values as bf16 pairs
       float v[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e)
         v[e] = (e & 1) ? __uint_as_float(nb[e >> 1] & 0xffff0000u) : __uint_as_float(nb[e >> 1] << 16);
-      if (RMS && live) {
-        const float g[8] = {gm[u][0].x, gm[u][0].y, gm[u][0].z, gm[u][0].w, gm[u][1].x, gm[u][1].y, gm[u][1].z, gm[u][1].w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          float t0 = v[2 * e] * inv, t1 = v[2 * e + 1] * inv;
-          t0 = t0 * g[2 * e];
-          t1 = t1 * g[2 * e + 1];
-          nb[e] = pack_bf16x2(t0, t1);
-          v[2 * e] = __uint_as_float(nb[e] << 16);
-          v[2 * e + 1] = __uint_as_float(nb[e] & 0xffff0000u);
-        }
-        if (a.xn_aux)
-          *reinterpret_cast<uint4*>(a.xn_aux + (size_t)src * a.K + k0) = make_uint4(nb[0], nb[1], nb[2], nb[3]);
-      }
       // codes = rint(v / scale) with the correctly rounded quotient.  v * (1 / scale) with the
       // hardware reciprocal is within 3 * 2^-24 * 128 < 2.3e-5 of it, so both round to the same
       // integer unless the product lies that close to a tie; those cases (and scales outside the
       // reciprocal's safe range) are redone with the division.
+      // The codes are formed biased by 128 (the fused v * (1 / scale) + 128 adds at most another 2^-17 to
+      // the distance above, still far inside the tie margin): c is then an integer in [1, 255] (|v| <= the
+      // row's absmax, so the clip of the reference never acts), lands in its byte with one
+      // v_cvt_pk_u8_f32, and flipping bit 7 of every byte turns the biased value into two's complement.
       float c[8];
       float off_integer = 0.0f;  // largest distance of a quotient from its rounded value
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float t = v[e] * rscale;
+        const float t = __builtin_fmaf(v[e], rscale, 128.0f);
         c[e] = rintf(t);
         off_integer = fmaxf(off_integer, fabsf(t - c[e]));
       }
-      const bool redo = !(scale > 1e-30f && scale < 1e30f) || off_integer > 0.4999f;
+      const bool redo = !(scale > 1e-30f && scale < 1e30f) || off_integer > 0.49996f;  // margin 4e-5 > 2.3e-5 + 2^-17
       if (__builtin_amdgcn_ballot_w64(redo) != 0) {  // wave-uniform
 #pragma unroll
-        for (int e = 0; e < 8; ++e) c[e] = rintf(v[e] / scale);
+        for (int e = 0; e < 8; ++e) c[e] = rintf(v[e] / scale) + 128.0f;
       }
-      // c is an integer in [-127, 127] (|v| <= the row's absmax, so the clip of the reference never
-      // acts): c + 128 converts and lands in its byte with one v_cvt_pk_u8_f32 (which saturates to
-      // 0..255 anyway), and flipping bit 7 of every byte turns the biased value into two's complement
       uint32_t lo = 0, hi = 0;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        lo = __builtin_amdgcn_cvt_pk_u8_f32(c[e] + 128.0f, (uint32_t)e, lo);
-        hi = __builtin_amdgcn_cvt_pk_u8_f32(c[e + 4] + 128.0f, (uint32_t)e, hi);
+        lo = __builtin_amdgcn_cvt_pk_u8_f32(c[e], (uint32_t)e, lo);
+        hi = __builtin_amdgcn_cvt_pk_u8_f32(c[e + 4], (uint32_t)e, hi);
       }
-      lo ^= 0x80808080u;
+      lo ^= 0x80808080u;  // (a lane without a value holds zeros: 0 -> 128 -> code 0)
       hi ^= 0x80808080u;
-      if (!live) { lo = 0; hi = 0; }
       if (live && a.codes_rm) *reinterpret_cast<uint2*>(a.codes_rm + (size_t)src * a.K + k0) = make_uint2(lo, hi);
-      *reinterpret_cast<uint2*>(a.xq_packed + ((size_t)pb * a.KB + kb) * kBlockBytes + code_off) = make_uint2(lo, hi);
-      if constexpr (CB > 0) {
-        // A block at a group boundary runs once per group with the other groups' rows zeroed.
-        for (uint32_t grp = glo; grp <= ghi; ++grp) {
-          v4i xa = {0, 0, 0, 0};
-          if (live && rowgrp == grp) xa = v4i{(int)nb[0], (int)nb[1], (int)nb[2], (int)nb[3]};
-          const v4i* ap = reinterpret_cast<const v4i*>(a.at) + (((size_t)grp * a.KB + kb) * CB) * 64u + lane;
-#pragma unroll
-          for (int b = 0; b < CB; ++b) {
-            v4i wb = wpre[u][b];
-            if (grp != glo) wb = ap[b * 64];  // wave-uniform, boundary blocks only
-            acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, xa),
-                                                             __builtin_bit_cast(v8bf, wb), acc[b], 0, 0, 0);
-          }
-        }
-      }
+      if (mine_row) *reinterpret_cast<uint2*>(a.xq_packed + ((size_t)pb * a.KB + kb) * kBlockBytes + code_off) = make_uint2(lo, hi);
     }
+    if constexpr (CB > 0) {
+      // (zeros where the lane has no value; at a group boundary the rows of the other groups are zeroed)
+      const v4i xa = in_group ? v4i{(int)raw.x, (int)raw.y, (int)raw.z, (int)raw.w} : v4i{0, 0, 0, 0};
+#pragma unroll
+      for (int b = 0; b < CB; ++b)
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, xa), __builtin_bit_cast(v8bf, w[b]),
+                                                         acc[b], 0, 0, 0);
+    }
+  };
+#pragma unroll 1
+  for (uint32_t grp = glo; grp <= ghi; ++grp) {  // workgroup-uniform: one trip except at a group boundary
+    const bool first = grp == glo;
+    const bool in_group = ghi == glo || rowgrp == grp;
+    v4i wa[kCB], wb2[kCB];
+    uint4 ra, rb;
+    request(grp, wave, wa, ra);
+    request(grp, wave + 16u, wb2, rb);
+#pragma unroll 1
+    for (uint32_t kb = wave; kb < a.KB; kb += 32u) {
+      work(first, in_group, kb, wa, ra);
+      request(grp, kb + 32u, wa, ra);
+      if (kb + 16u >= a.KB) break;  // wave-uniform
+      work(first, in_group, kb + 16u, wb2, rb);
+      request(grp, kb + 48u, wb2, rb);
+    }
+    if constexpr (CB == 0) break;
   }
   if constexpr (CB == 0) return;
 
   // ---- 3. fixed-order sum of the 16 wave tiles: 8..15 onto 0..7, 4..7 onto 0..3, then 0+1+2+3
-  if (wave >= 8u) {
+  __syncthreads();  // the rows are spent: their bytes take the wave tiles
+#pragma unroll 1
+  for (uint32_t half = 8u; half >= 4u; half >>= 1) {
+    if (wave >= half && wave < 2u * half) {
 #pragma unroll
-    for (int b = 0; b < kCB; ++b)
+      for (int b = 0; b < kCB; ++b)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) red[wave - 8u][b][e][lane] = acc[b][e];
+        for (int e = 0; e < 4; ++e) red[wave - half][b][e][lane] = acc[b][e];
+    }
+    __syncthreads();
+    if (wave < half) {
+#pragma unroll
+      for (int b = 0; b < kCB; ++b)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[b][e] = acc[b][e] + red[wave][b][e][lane];
+    }
+    __syncthreads();
   }
-  __syncthreads();
-  if (wave < 8u) {
-#pragma unroll
-    for (int b = 0; b < kCB; ++b)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) acc[b][e] = acc[b][e] + red[wave][b][e][lane];
-  }
-  __syncthreads();
-  if (wave >= 4u && wave < 8u) {
-#pragma unroll
-    for (int b = 0; b < kCB; ++b)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) red[wave - 4u][b][e][lane] = acc[b][e];
-  }
-  __syncthreads();
-  if (wave < 4u) {
-#pragma unroll
-    for (int b = 0; b < kCB; ++b)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) acc[b][e] = acc[b][e] + red[wave][b][e][lane];
-  }
-  __syncthreads();
   if (wave < 4u) {
 #pragma unroll
     for (int b = 0; b < kCB; ++b)
@@ -1181,6 +1235,7 @@ __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
   // zp[pb][kk][term][lane64][8]: lane = row % 32 + 32 * hh holds rank columns 16 kk + 8 hh + 0..7
   for (uint32_t t = tid; t < a.nkk * 3u * 32u; t += 1024u) {
     const uint32_t row = t & 15u, hh = (t >> 4) & 1u, term = (t >> 5) % 3u, kk = t / 96u;
+    if (row < r0 || row >= r0 + R) continue;
     v8us o;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {

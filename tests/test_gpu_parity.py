@@ -273,9 +273,13 @@ def test_tile_geometries_agree_bitwise(dev, pkg, shape):
     narrow, aux_n = wc.gpu_forward(case, flags=pkg._native.FLAG_FORCE_TILED | pkg._native.FLAG_TILE_256X128)
     wide, aux_w = wc.gpu_forward(case, flags=pkg._native.FLAG_FORCE_TILED | pkg._native.FLAG_TILE_256X256)
     small, aux_s = wc.gpu_forward(case, flags=pkg._native.FLAG_FORCE_TILED | pkg._native.FLAG_TILE_128X128)
-    for aux in (aux_n, aux_w, aux_s):
+    pair, aux_p = wc.gpu_forward(case, flags=pkg._native.FLAG_FORCE_TILED | pkg._native.FLAG_TILE_256X128_PAIR)
+    for aux in (aux_n, aux_w, aux_s, aux_p):
         assert np.array_equal(aux["acc"], want["acc"])
         assert np.array_equal(aux["x_codes"], want["x_codes"])
+    # the 256 x 128 pair geometry is the 256 x 256 kernel with two waves side by side instead of four: the
+    # same wave tile, the same operations per output
+    assert np.array_equal(pair.view(np.uint32), wide.view(np.uint32))
     # the 128 x 128 geometry is the 256 x 128 kernel with one 32-row block per wave: the same operations per output
     assert np.array_equal(narrow.view(np.uint32), small.view(np.uint32))
     if shape.get("n_adapters", 1) == 0:
@@ -330,7 +334,8 @@ def test_randomized_forward_sweep(dev, pkg, seed):
         residual = (not swiglu) and bool(rng.integers(0, 2))
         idx_mode = str(rng.choice(["uniform", "arange", "zero"]))
         flags = int(rng.choice([0, 0, 0, nat.FLAG_FORCE_TILED, nat.FLAG_TILE_128X128,
-                                nat.FLAG_FORCE_TILED | nat.FLAG_TILE_256X128, nat.FLAG_FORCE_TILED | nat.FLAG_TILE_256X256]))
+                                nat.FLAG_FORCE_TILED | nat.FLAG_TILE_256X128, nat.FLAG_FORCE_TILED | nat.FLAG_TILE_256X256,
+                                nat.FLAG_FORCE_TILED | nat.FLAG_TILE_256X128_PAIR]))
         if (flags & nat.FLAG_TILE_256X256) and k < 384:
             flags = nat.FLAG_FORCE_TILED
         what = f" m={m} k={k} n={n} adapters={n_ad} rank={rank} rms={rms} swiglu={swiglu} residual={residual} {idx_mode} flags={flags}"
