@@ -261,8 +261,16 @@ int launch_skinny(const mi355_w8a8_problem* p, unsigned char* xq, float* sx, uin
     q.lora_scaling = lora ? p->lora_scaling : nullptr;
     q.row_scaling = reinterpret_cast<float*>(sws + L.row_scaling);
     const uint32_t n_regroup = (regroup && !keep_regrouped) ? (p->m * q.n_groups + 3u) / 4u : 0u;
-    if (rms) hipLaunchKernelGGL((skinny_quant_kernel<true>), dim3(p->m + n_regroup), dim3(1024), 0, s, q);
-    else hipLaunchKernelGGL((skinny_quant_kernel<false>), dim3(p->m + q.n_z_units + n_regroup), dim3(1024), 0, s, q);
+    // warm-up units over the head of the packed weight (whole units only)
+    {
+      const char* e = getenv("W8A8_WARM_MB");  // EXPERIMENT
+      const uint64_t want = e ? (uint64_t)atoi(e) << 20 : 0u;
+      const uint64_t have = mi355_w8a8_packed_weight_bytes(p->k, p->n);
+      q.warm = static_cast<const unsigned char*>(p->w_packed);
+      q.n_warm_units = (uint32_t)((want < have ? want : have) / kSkinnyWarmBytes);
+    }
+    if (rms) hipLaunchKernelGGL((skinny_quant_kernel<true>), dim3(p->m + n_regroup + q.n_warm_units), dim3(1024), 0, s, q);
+    else hipLaunchKernelGGL((skinny_quant_kernel<false>), dim3(p->m + q.n_z_units + n_regroup + q.n_warm_units), dim3(1024), 0, s, q);
     if ((st = launch_status())) return st;
     if (lora && rms) {  // the LoRA-A units read the normalized rows the quantizer has just written
       SkinnyLoraAArgs la{};

@@ -96,5 +96,19 @@ typedef __attribute__((address_space(3))) void* lptr_t;
 __device__ inline void load_1k_to_lds(const unsigned char* src_lane, unsigned char* lds_dst_uniform) {
   __builtin_amdgcn_global_load_lds((gptr_t)src_lane, (lptr_t)lds_dst_uniform, 16, 0, 0);
 }
+// The same as an assembly statement the compiler keeps no books on (it treats the builtin as an access
+// that may touch the LDS and then drains every counter at its next wait): lane l moves 16 bytes
+// global[base + voff] -> LDS[lds_addr_uniform + 16 l]; inactive lanes move nothing.  The caller waits
+// with s_waitcnt vmcnt and a barrier before the LDS is read.
+// A gather of 64 dwords by one wave: lane l moves 4 bytes global[base + voff] (voff a multiple of 4, any
+// place) -> LDS[lds_addr_uniform + 4 l].
+__device__ inline void lds_gather_dword(const void* base_uniform, uint32_t voff, uint32_t lds_addr_uniform) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+               :: "v"(voff), "s"(base_uniform), "s"(lds_addr_uniform) : "memory", "m0");
+}
+__device__ inline void lds_load_1k(const unsigned char* base_uniform, uint32_t voff, uint32_t lds_addr_uniform) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :: "v"(voff), "s"(base_uniform), "s"(lds_addr_uniform) : "memory", "m0");
+}
 
 }  // namespace w8a8

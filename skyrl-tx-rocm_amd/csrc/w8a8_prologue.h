@@ -947,13 +947,6 @@ __device__ inline void route_rows_inline(const int32_t* __restrict__ idx, uint32
   __syncthreads();
 }
 
-// One direct-to-LDS load of 1 KiB by a wave: lane l moves global[base + voff] (voff = 1024 u + 16 l) to
-// LDS[lds_addr_uniform + 16 l]; inactive lanes move nothing.
-__device__ inline void ql_load_1k(const unsigned char* base_uniform, uint32_t voff, uint32_t lds_addr_uniform) {
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-               :: "v"(voff), "s"(base_uniform), "s"(lds_addr_uniform) : "memory", "m0");
-}
-
 template <int CB, bool RMS>  // CB: 16-wide rank blocks (0 = no LoRA, 1, 2, 4)
 __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
   constexpr int kCB = CB > 0 ? CB : 1;
@@ -1015,7 +1008,7 @@ __global__ __launch_bounds__(1024) void quant_lora_kernel(QuantLoraArgs a) {
       const uint32_t row_lds = lds_addr + wave * a.row_stride;
       for (uint32_t u = 0; u < n_chunks; ++u) {
         const uint32_t voff = u * 1024u + lane * 16u;
-        if (voff < row_bytes) ql_load_1k(xr, voff, row_lds + u * 1024u);
+        if (voff < row_bytes) lds_load_1k(xr, voff, row_lds + u * 1024u);
       }
       // (the first chunk's norm weights travel with the row)
       float4 gn0 = make_float4(0.f, 0.f, 0.f, 0.f), gn1 = gn0;

@@ -74,7 +74,13 @@ struct SkinnyQuantArgs {
   uint32_t N, n_groups;    // n_groups = N_pad / 128
   const float* lora_scaling;  // f32 [n_adapters] or null
   float* row_scaling;      // f32 [32]: lora_scaling[idx[m]], written here for the stream kernel
+  // Weight warm-up units that share the launch: each reads kSkinnyWarmBytes of the packed weight and
+  // discards them.  The launch leaves the memory nearly idle, and what it reads here the stream kernel
+  // finds in the memory-side cache instead of waiting for it behind the rest of its stream.
+  const unsigned char* warm;  // packed weight or null
+  uint32_t n_warm_units;
 };
+constexpr uint32_t kSkinnyWarmBytes = 128u * 1024u;  // per unit: 1024 threads x 8 loads of 16 bytes
 
 // The stream kernel's unit u = 8 G + 2 j + h owns the original columns 128 G + 4 (16 h + c) + j,
 // c = 0..15, and its finish step needs, per row m and column c, the ranks of one parity:
@@ -188,6 +194,16 @@ __global__ __launch_bounds__(1024) void skinny_quant_kernel(SkinnyQuantArgs a) {
   __shared__ float red_max[16];
   __shared__ double red_sum[16];
   __shared__ float zw[16][64];
+  if (blockIdx.x >= gridDim.x - a.n_warm_units) {  // the last blocks of the launch
+    const uint32_t unit = blockIdx.x - (gridDim.x - a.n_warm_units);
+    const v4i* src = reinterpret_cast<const v4i*>(a.warm + (size_t)unit * kSkinnyWarmBytes) + threadIdx.x;
+    v4i got[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) got[j] = src[j * 1024];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) asm volatile("" :: "v"(got[j]));  // arrived; nothing is done with them
+    return;
+  }
   if (blockIdx.x >= a.M + a.n_z_units) {
     __shared__ __attribute__((aligned(16))) uint16_t tile[4][32][128];  // 32 KiB
     skinny_regroup_b(a, blockIdx.x - a.M - a.n_z_units, tile);
@@ -344,6 +360,10 @@ __global__ __launch_bounds__(kSkinnyStreamThreads) void skinny_stream_kernel(Ski
   __shared__ __attribute__((aligned(16))) int red[kSkinnyStreamWaves][2][4][64];  // 16 KiB
   __shared__ float zl[kSkinnyMaxRows][kMaxRank];                                 // 8 KiB
   __shared__ float low_odd[256];
+  // one-round form: the finish step's LoRA operands, staged by direct-to-LDS loads behind the weight stream
+  __shared__ __attribute__((aligned(1024))) float zst[ROWS2 ? 1 : kSkinnyMaxZChunks][16][32];  // z partials [chunk][row][rank], 32 KiB
+  __shared__ __attribute__((aligned(1024))) uint16_t bst[ROWS2 ? 8 : 16 * 2 * 16 * 16];         // the unit's regrouped B, 16 KiB
+  __shared__ __attribute__((aligned(1024))) uint32_t fst[4][256];  // per output thread: sx, sw, the row's LoRA scaling, the residual's dword
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t slot = blockIdx.x >> 3;
@@ -369,24 +389,127 @@ __global__ __launch_bounds__(kSkinnyStreamThreads) void skinny_stream_kernel(Ski
   const uint32_t fn = 128u * (nb >> 2) + 4u * pc + (nb & 3u);
   const bool fvalid = frow < a.M && fn < a.N;
   const bool lora = a.lora_b != nullptr;
-  // The finish step's operands are requested now and used after the stream.  Lanes without an
-  // output read element 0 instead of selecting on the loaded value: a select would make the wave
-  // wait for memory before its first weight load.
+  // Lanes without an output read element 0 instead of selecting on the loaded value.
   const uint32_t srow = fvalid ? frow : 0u, scol = fvalid ? fn : 0u;
-  const float f_sx = a.sx[srow];
-  const float f_sw = a.sw[scol];
-  int ad_raw = 0;
-  if (lora && a.idx) ad_raw = a.idx[srow];
   // z[m][r] share of this thread: value index tid (and tid + 512, ...) of the M x rpad values
   const uint32_t rpad = (a.r + 7u) & ~7u;
   const uint32_t n_zval = lora ? a.M * rpad : 0u;
   // With B regrouped per unit the low-rank term needs three independent, coalesced requests per
-  // thread (its 16 ranks of B, its z partials, its row's scaling).  They go out ahead of the weight
-  // loads: a wave's loads return in order, so they are back while the weight is still streaming,
-  // and the term is computed under the stream.  (Issued later they would wait for the stream.)
+  // thread: its 16 ranks of B, its z partials, its row's scaling.
   const bool early = !ROWS2 && lora && a.bsel != nullptr && n_zval <= kSkinnyStreamThreads;  // workgroup-uniform
-  float low = 0.f, f_s = 0.f;
+  float low = 0.f, f_s = 0.f, f_sx, f_sw;
   uint16_t res_raw = 0;
+  v4i acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
+
+  // ---- One round: every wave's share of K is exactly what it keeps in flight (K = 512 * kInFlight: the
+  // Qwen3-8B down projection), and the low-rank term, if any, has its regrouped B.
+  //  * What the finish step works with (the unit's regrouped B, the z partials of all rows, every output's
+  //    scales and residual) takes no registers -- the operands of the MFMAs take all there are, and a
+  //    value loaded beside them is spilled behind a wait for the whole stream -- the waves copy it into
+  //    the LDS with direct-to-LDS loads, the first loads they issue.
+  //  * Then the weight loads go out, nothing waited for, spilled or converted in front of them.
+  //  * While the weight is on its way the low-rank term is formed from the LDS (a wave's loads return in
+  //    order: a wait that leaves only the weight loads outstanding has the staged pieces).
+  //  * Then the codes are requested, the MFMAs run as their operands arrive, and what is left behind
+  //    them is the sum over the waves and one line of float32 arithmetic per output.
+  const bool one_round = !ROWS2 && n_pairs == kSkinnyStreamWaves * kInFlight && (!lora || early);  // workgroup-uniform
+  if (one_round) {
+    // the staged operands first: a handful of instructions, and their data is then in the LDS long before
+    // the weight is in the registers
+    const uint32_t res_elem = srow * a.N + scol;  // (M * N is below 2^32)
+    if (lora) {  // kernel-uniform
+      const uint32_t unit = grp * 8u + (slot & 7u);
+      const unsigned char* bsrc = reinterpret_cast<const unsigned char*>(a.bsel) + (size_t)unit * a.M * 1024u;  // M KiB, contiguous
+      const uint32_t bst_addr = (uint32_t)(uintptr_t)(lptr_t)bst, zst_addr = (uint32_t)(uintptr_t)(lptr_t)zst;
+      for (uint32_t i = wave; i < a.M; i += kSkinnyStreamWaves) lds_load_1k(bsrc, i * 1024u + lane * 16u, bst_addr + i * 1024u);
+      // z partials: per chunk the first 32 ranks of rows 0..15, two pieces of eight rows x 128 bytes
+      for (uint32_t i = wave; i < 2u * a.z_chunks; i += kSkinnyStreamWaves) {
+        const uint32_t ch = i >> 1, h = i & 1u;
+        const uint32_t voff = ((ch * (uint32_t)kSkinnyMaxRows + 8u * h + (lane >> 3)) * (uint32_t)kMaxRank) * 4u + (lane & 7u) * 16u;
+        lds_load_1k(reinterpret_cast<const unsigned char*>(a.z_part), voff, zst_addr + i * 1024u);
+      }
+      // the chunk slots no unit has written count as zeros, so that the sum below needs no conditions
+      for (uint32_t i = a.z_chunks * 128u + tid; i < kSkinnyMaxZChunks * 128u; i += kSkinnyStreamThreads)
+        reinterpret_cast<float4*>(&zst[0][0][0])[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    if (wave < 4u) {  // the output threads: thread tid finds its four values at fst[.][tid]
+      const uint32_t fst_addr = (uint32_t)(uintptr_t)(lptr_t)fst + wave * 256u;
+      lds_gather_dword(a.sx, srow * 4u, fst_addr);
+      lds_gather_dword(a.sw, scol * 4u, fst_addr + 1024u);
+      if (lora) lds_gather_dword(a.row_scaling, srow * 4u, fst_addr + 2048u);
+      if (a.residual) lds_gather_dword(a.residual, (res_elem * 2u) & ~3u, fst_addr + 3072u);
+    }
+    v4i wf[kInFlight], xf[kInFlight];
+    const unsigned char* wb = wsrc + (size_t)p0 * 2u * kBlockBytes;
+    const unsigned char* xb = xsrc + (size_t)p0 * 2u * kBlockBytes;
+#pragma unroll
+    for (uint32_t t = 0; t < kInFlight; ++t)
+      wf[t] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wb + t * 2u * kBlockBytes));
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- the low-rank term, while the weight is on its way: the staged operands are the wave's oldest
+    // loads, so a wait that leaves the kInFlight weight loads outstanding has them
+    if (lora) {
+      asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kInFlight) : "memory");
+      __syncthreads();  // ... and the other waves' pieces
+      {  // z[m][r] for 16 rows x 32 ranks, one per thread: four interleaved partial sums, combined in a fixed order
+        const uint32_t zr = tid >> 5, zc = tid & 31u;
+        float zv[kSkinnyMaxZChunks];
+#pragma unroll
+        for (uint32_t ch = 0; ch < kSkinnyMaxZChunks; ++ch) zv[ch] = zst[ch][zr][zc];
+        float s4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (uint32_t ch = 0; ch < kSkinnyMaxZChunks; ++ch) s4[ch & 3u] += zv[ch];
+        zl[zr][zc] = ((s4[0] + s4[1]) + s4[2]) + s4[3];
+      }
+      __syncthreads();
+      if (wave < 4u) {  // the output threads
+        // the even and the odd ranks as two chains, added at the end: the order of the two-thread form.
+        // (Ranks beyond the rank are zeros in z and in the regrouped B alike: they add nothing.)
+        float zrow[32];
+#pragma unroll
+        for (uint32_t i = 0; i < 8; ++i) {
+          const float4 z4 = *reinterpret_cast<const float4*>(&zl[srow][4u * i]);
+          zrow[4 * i] = z4.x; zrow[4 * i + 1] = z4.y; zrow[4 * i + 2] = z4.z; zrow[4 * i + 3] = z4.w;
+        }
+        float lo2[2] = {0.f, 0.f};
+#pragma unroll
+        for (uint32_t par = 0; par < 2; ++par) {
+          const uint16_t* bl = bst + ((srow * 2u + par) * 16u + c16) * 16u;
+          const v8us blo = *reinterpret_cast<const v8us*>(bl), bhi = *reinterpret_cast<const v8us*>(bl + 8);
+#pragma unroll
+          for (uint32_t t = 0; t < 16; ++t) {
+            const uint16_t bv = t < 8u ? blo[t & 7u] : bhi[t & 7u];
+            lo2[par] = fmaf(zrow[par + 2u * t], bf16_bits_to_f32(bv), lo2[par]);
+          }
+        }
+        low = lo2[0] + lo2[1];
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (uint32_t t = 0; t < kInFlight; ++t) xf[t] = *reinterpret_cast<const v4i*>(xb + t * 2u * kBlockBytes);
+    __builtin_amdgcn_sched_barrier(0);
+    // four accumulators take turns, so that no MFMA waits for the one before it (integer sums: any order)
+    v4i part[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
+#pragma unroll
+    for (uint32_t t = 0; t < kInFlight; ++t) part[t & 3u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[t], wf[t], part[t & 3u], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) red[wave][0][e][lane] = (part[0][e] + part[1][e]) + (part[2][e] + part[3][e]);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (without LoRA nothing has waited for the staged scales yet)
+    __syncthreads();  // the accumulators of every wave
+    if (wave >= 4u) return;  // one thread per output from here on
+    f_sx = __uint_as_float(fst[0][tid]);
+    f_sw = __uint_as_float(fst[1][tid]);
+    if (a.residual) res_raw = (uint16_t)((res_elem & 1u) ? fst[3][tid] >> 16 : fst[3][tid] & 0xffffu);
+    if (lora) f_s = __uint_as_float(fst[2][tid]);
+  } else {
+  f_sx = a.sx[srow];
+  f_sw = a.sw[scol];
+  int ad_raw = 0;
+  if (lora && a.idx) ad_raw = a.idx[srow];
+  // The low-rank term's requests go out ahead of the weight loads: a wave's loads return in order, so they
+  // are back while the weight is still streaming, and the term is computed under the stream.
   v8us blo = {0, 0, 0, 0, 0, 0, 0, 0}, bhi = {0, 0, 0, 0, 0, 0, 0, 0};
   float zv[kSkinnyMaxZChunks];
   if (early) {
@@ -403,7 +526,6 @@ __global__ __launch_bounds__(kSkinnyStreamThreads) void skinny_stream_kernel(Ski
       zv[ch] = ch < a.z_chunks ? zp[(size_t)ch * kSkinnyMaxRows * kMaxRank] : 0.f;
   }
   __builtin_amdgcn_sched_barrier(0);  // the weight loads below are issued after the requests above
-  v4i acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
   uint32_t base = p0;
   do {
     v4i wf[kInFlight], xf[kInFlight], xg[ROWS2 ? kInFlight : 1];
@@ -458,7 +580,6 @@ __global__ __launch_bounds__(kSkinnyStreamThreads) void skinny_stream_kernel(Ski
     if (a.residual) res_raw = a.residual[(size_t)srow * a.N + scol];
     const int ad = ad_raw < 0 ? 0 : (ad_raw >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad_raw);
     f_s = (fvalid && lora) ? a.lora_scaling[ad] : 0.f;
-    const uint16_t* Bp = a.lora_b + ((size_t)ad * a.r + rsel) * a.N + fn;
     // Every B value of the thread (ranks rsel, rsel + kRankSplit, ... below 64) is requested before the
     // first is used: one trip to memory instead of one per value.
     // The loads are unconditional (a load under a lane condition gets a branch and a wait of its own):
@@ -502,7 +623,8 @@ __global__ __launch_bounds__(kSkinnyStreamThreads) void skinny_stream_kernel(Ski
   } else {
     __syncthreads();  // the accumulators in `red`
   }
-  if (!ROWS2 && rsel == 1u) return;
+  }
+  if (!ROWS2 && rsel == 1u) return;  // (only the multi-round form gets here with rsel == 1)
   if (!fvalid) return;
   int sum = 0;
 #pragma unroll
