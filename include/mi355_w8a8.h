@@ -84,12 +84,16 @@ typedef enum mi355_w8a8_status {
  * groups average at least 96 rows, else 64.  Pass the same flags to the workspace query. */
 #define MI355_W8A8_FLAG_GROUPED_TILE64 256u
 #define MI355_W8A8_FLAG_GROUPED_TILE128 512u
-/* The workspace still holds the transposed LoRA A and the packed LoRA B that an earlier call of the tiled
- * path wrote there for the same lora_a / lora_b contents and the same (k, n, n_adapters, rank): this call
- * does not write them again (adapters that do not change between calls, as in serving).  The caller
- * vouches for it; calls of 17..128 rows keep no such copies and ignore the flag. */
-/* For calls of at most 16 rows (rank <= 32) the same flag covers the per-row regrouped copy of B the decode
- * kernels keep in the workspace: it additionally vouches that adapter_indices has the contents it had then. */
+/* The workspace still holds the LoRA A and B in operand order that an earlier call of the tiled path
+ * (more than 32 rows, not run as 32-row chunks: see mi355_w8a8_forward_path) wrote there for the same
+ * lora_a / lora_b contents and the same (k, n, n_adapters, rank): this call does not write them again
+ * (adapters that do not change between calls, as in serving).  They sit at the start of the workspace, at
+ * places that depend on (k, n, n_adapters, rank) only, so the earlier call may have had another m, other
+ * adapter_indices or another tile geometry.  The caller vouches for it; calls that run as 32-row chunks
+ * keep no such copies and ignore the flag. */
+/* For calls of at most 16 rows (rank <= 32) the flag covers something else: the per-row regrouped copy of B
+ * the decode kernels keep in the workspace.  There it vouches that the earlier call was a decode call with
+ * the same m and that lora_b and adapter_indices have the contents they had then. */
 #define MI355_W8A8_FLAG_LORA_PACK_VALID 1024u
 
 /*
@@ -327,7 +331,10 @@ int mi355_w8a8_grouped_v1(const mi355_w8a8_grouped_problem* problem, void* strea
  * mi355_w8a8_workspace_bytes(...) of the problem exceeds that size.  Inputs and outputs are the
  * caller's as before.  All calls on one GPU share the array: calls that overlap in time on one GPU
  * (two streams, two threads) race; calls on one stream are ordered and safe.  The first call on a
- * device resolves the array's address (a host-side lookup, no allocation).
+ * device resolves the array's address (a host-side lookup, no allocation): make one call on a device
+ * before capturing a graph there.  Because any caller's call in between may have overwritten the array,
+ * MI355_W8A8_FLAG_LORA_PACK_VALID and MI355_W8A8_FLAG_SKIP_PROLOGUE are answered with
+ * MI355_W8A8_ERR_UNSUPPORTED.
  */
 #define MI355_W8A8_STATIC_WORKSPACE_BYTES (32u << 20)
 int mi355_w8a8_forward_static_ws_v1(const mi355_w8a8_problem* problem, void* stream);
@@ -551,7 +558,7 @@ int mi355_w8a8_forward_path(uint32_t m, uint32_t k, uint32_t n, uint32_t flags);
 
 /*
  * Calibration (no counterpart in the reference: these measure the ceilings the path is priced against,
- * for bench.py and profiles/).  mi355_w8a8_calibrate_mfma_v1 runs `iters` rounds of int8 MFMAs on
+ * for bench.py and profiles/).  mi355_w8a8_calibrate_mfma_v1 runs `iters` (at most 2^18) rounds of int8 MFMAs on
  * operands that stay in registers: shape 0 = 16 of the 32 x 32 x 32 instruction per wave and round,
  * shape 1 = 64 of the 16 x 16 x 64 one; 256 workgroups of four waves.  `operands` holds
  * mi355_w8a8_calibrate_operand_bytes() bytes of codes (zeros, random bits, realistic codes: the rate

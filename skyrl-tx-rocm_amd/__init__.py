@@ -7,9 +7,10 @@ module name ``skyrl_tx_rocm_amd``.
 
 from . import _native  # noqa: F401
 from .kernels import quantized_lora  # noqa: F401
+from .kernels import bounded_lora  # noqa: F401
 from .kernels.rocm import w8a8_lora  # noqa: F401
 from .kernels.rocm import bf16_lora_residual, bf16_rms_gate_up_lora_swiglu_contiguous  # noqa: F401
 from .kernels.rocm import gq_linear  # noqa: F401
 from .layers import lora  # noqa: F401
 
-__all__ = ["_native", "quantized_lora", "w8a8_lora", "gq_linear", "lora"]
+__all__ = ["_native", "quantized_lora", "bounded_lora", "w8a8_lora", "gq_linear", "lora"]

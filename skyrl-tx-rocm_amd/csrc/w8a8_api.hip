@@ -109,6 +109,11 @@ WsLayout make_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint
   w.n_steps = (k + 63u) / 64u;
   w.steps_per_wave = (w.n_steps + 15u) / 16u;
   uint64_t off = 0;
+  // The LoRA operands a caller may vouch for (MI355_W8A8_FLAG_LORA_PACK_VALID) come first: their sizes and
+  // so their places depend on (k, n, n_adapters, rank) only -- not on m, the path or the slot layout -- so
+  // calls of different row counts on one workspace find them where an earlier call left them.
+  w.at = off; off += rank ? align256((uint64_t)n_groups * w.KB * w.nkk * kBlockBytes) : 0u;  // A in operand order
+  w.bp = off; off += rank ? align256((uint64_t)n_groups * (n_padded(n) / 32u) * w.nkk * kBlockBytes) : 0u;
   w.xq = off; off += align256((uint64_t)w.slots * w.K_pad);
   w.sx = off; off += align256((uint64_t)w.slots * 4u);
   w.src_row = off; off += align256((uint64_t)w.slots * 4u);
@@ -120,8 +125,6 @@ WsLayout make_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n_groups, uint
   w.xn = off;
   off += (rank && m <= kSkinnyChunkedMaxRows) ? align256((uint64_t)(m < 32u ? m : 32u) * k * 2u) : 0u;
   w.zp = off; off += rank ? align256((uint64_t)(w.slots / 32u) * w.nkk * 3u * kBlockBytes) : 0u;
-  w.at = off; off += rank ? align256((uint64_t)n_groups * w.KB * w.nkk * kBlockBytes) : 0u;  // A in operand order
-  w.bp = off; off += rank ? align256((uint64_t)n_groups * (n_padded(n) / 32u) * w.nkk * kBlockBytes) : 0u;
   w.skinny = off; off += align256(skinny_workspace_bytes(m, n, rank));
   w.total = off;
   return w;
@@ -261,16 +264,8 @@ int launch_skinny(const mi355_w8a8_problem* p, unsigned char* xq, float* sx, uin
     q.lora_scaling = lora ? p->lora_scaling : nullptr;
     q.row_scaling = reinterpret_cast<float*>(sws + L.row_scaling);
     const uint32_t n_regroup = (regroup && !keep_regrouped) ? (p->m * q.n_groups + 3u) / 4u : 0u;
-    // warm-up units over the head of the packed weight (whole units only)
-    {
-      const char* e = getenv("W8A8_WARM_MB");  // EXPERIMENT
-      const uint64_t want = e ? (uint64_t)atoi(e) << 20 : 0u;
-      const uint64_t have = mi355_w8a8_packed_weight_bytes(p->k, p->n);
-      q.warm = static_cast<const unsigned char*>(p->w_packed);
-      q.n_warm_units = (uint32_t)((want < have ? want : have) / kSkinnyWarmBytes);
-    }
-    if (rms) hipLaunchKernelGGL((skinny_quant_kernel<true>), dim3(p->m + n_regroup + q.n_warm_units), dim3(1024), 0, s, q);
-    else hipLaunchKernelGGL((skinny_quant_kernel<false>), dim3(p->m + q.n_z_units + n_regroup + q.n_warm_units), dim3(1024), 0, s, q);
+    if (rms) hipLaunchKernelGGL((skinny_quant_kernel<true>), dim3(p->m + n_regroup), dim3(1024), 0, s, q);
+    else hipLaunchKernelGGL((skinny_quant_kernel<false>), dim3(p->m + q.n_z_units + n_regroup), dim3(1024), 0, s, q);
     if ((st = launch_status())) return st;
     if (lora && rms) {  // the LoRA-A units read the normalized rows the quantizer has just written
       SkinnyLoraAArgs la{};
@@ -707,7 +702,7 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
     la.steps_per_wave = w.steps_per_wave; la.n_steps = w.n_steps;
     la.nterms = (p->flags & MI355_W8A8_FLAG_LORA_SPLIT2) ? 2u : 3u;
     la.n_blocks = w.slots / 32u;
-    const dim3 grid(w.slots / 32u), block(1024);
+    const dim3 grid(w.slots / 32u);
     if ((st = launch_lora_a(la, w.nkk, grid, s))) return st;
   }
   if (skip_gemm) return MI355_W8A8_OK;
@@ -1888,6 +1883,9 @@ int mi355_w8a8_forward_static_ws_v1(const mi355_w8a8_problem* p, void* stream) {
   if (p->struct_size != sizeof(mi355_w8a8_problem)) return MI355_W8A8_ERR_STRUCT;
   const int st = validate_common(p->m, p->k, p->n);
   if (st) return st;
+  // Every caller in the process shares the array: what an earlier call left in it may be another layer's,
+  // so a call must not be told to keep it.
+  if (p->flags & (MI355_W8A8_FLAG_LORA_PACK_VALID | MI355_W8A8_FLAG_SKIP_PROLOGUE)) return MI355_W8A8_ERR_UNSUPPORTED;
   const uint64_t need = mi355_w8a8_workspace_bytes(p->m, p->k, p->n, p->n_adapters, p->rank, p->flags);
   if (need == 0 || need > MI355_W8A8_STATIC_WORKSPACE_BYTES) return MI355_W8A8_ERR_WORKSPACE;
   void* ws = static_workspace();
@@ -2041,7 +2039,7 @@ uint64_t mi355_w8a8_calibrate_mfma_ops(uint32_t shape, uint32_t iters) {
 int mi355_w8a8_calibrate_mfma_v1(uint32_t shape, const void* operands, uint32_t iters, uint64_t* clocks,
                                  int32_t* sink, void* stream) {
   if (!operands || !clocks || !sink) return MI355_W8A8_ERR_NULL;
-  if (shape > 1u || iters == 0 || iters > (1u << 24)) return MI355_W8A8_ERR_SHAPE;
+  if (shape > 1u || iters == 0 || iters > (1u << 18)) return MI355_W8A8_ERR_SHAPE;  // (2^18 rounds keep a launch under half a second)
   if (reinterpret_cast<uintptr_t>(operands) & 15u) return MI355_W8A8_ERR_ALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const unsigned char* src = static_cast<const unsigned char*>(operands);

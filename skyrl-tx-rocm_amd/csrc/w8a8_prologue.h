@@ -555,7 +555,7 @@ struct LoraAArgs {
   uint32_t row_div, row_limit;
 };
 
-// STAGED (RB = 1, the transposed A, no K split): the operands of a k step travel through 8 KiB of LDS
+// STAGED (RB = 1, the transposed A; with or without the K split): the operands of a k step travel through 8 KiB of LDS
 // per wave.  A register load of an MFMA operand touches 32 cache lines of 32 used bytes, which the
 // vector memory path delivers at a third of the rate of whole lines; a direct-to-LDS load in which
 // eight lanes fetch one 128-byte line (of a row of x, of a rank column of A) moves eight whole lines,

@@ -74,13 +74,7 @@ struct SkinnyQuantArgs {
   uint32_t N, n_groups;    // n_groups = N_pad / 128
   const float* lora_scaling;  // f32 [n_adapters] or null
   float* row_scaling;      // f32 [32]: lora_scaling[idx[m]], written here for the stream kernel
-  // Weight warm-up units that share the launch: each reads kSkinnyWarmBytes of the packed weight and
-  // discards them.  The launch leaves the memory nearly idle, and what it reads here the stream kernel
-  // finds in the memory-side cache instead of waiting for it behind the rest of its stream.
-  const unsigned char* warm;  // packed weight or null
-  uint32_t n_warm_units;
 };
-constexpr uint32_t kSkinnyWarmBytes = 128u * 1024u;  // per unit: 1024 threads x 8 loads of 16 bytes
 
 // The stream kernel's unit u = 8 G + 2 j + h owns the original columns 128 G + 4 (16 h + c) + j,
 // c = 0..15, and its finish step needs, per row m and column c, the ranks of one parity:
@@ -194,16 +188,6 @@ __global__ __launch_bounds__(1024) void skinny_quant_kernel(SkinnyQuantArgs a) {
   __shared__ float red_max[16];
   __shared__ double red_sum[16];
   __shared__ float zw[16][64];
-  if (blockIdx.x >= gridDim.x - a.n_warm_units) {  // the last blocks of the launch
-    const uint32_t unit = blockIdx.x - (gridDim.x - a.n_warm_units);
-    const v4i* src = reinterpret_cast<const v4i*>(a.warm + (size_t)unit * kSkinnyWarmBytes) + threadIdx.x;
-    v4i got[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) got[j] = src[j * 1024];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) asm volatile("" :: "v"(got[j]));  // arrived; nothing is done with them
-    return;
-  }
   if (blockIdx.x >= a.M + a.n_z_units) {
     __shared__ __attribute__((aligned(16))) uint16_t tile[4][32][128];  // 32 KiB
     skinny_regroup_b(a, blockIdx.x - a.M - a.n_z_units, tile);
@@ -407,11 +391,12 @@ __global__ __launch_bounds__(kSkinnyStreamThreads) void skinny_stream_kernel(Ski
   //    scales and residual) takes no registers -- the operands of the MFMAs take all there are, and a
   //    value loaded beside them is spilled behind a wait for the whole stream -- the waves copy it into
   //    the LDS with direct-to-LDS loads, the first loads they issue.
-  //  * Then the weight loads go out, nothing waited for, spilled or converted in front of them.
+  //  * Then the code and the weight loads go out, nothing waited for, spilled or converted in front of
+  //    them.
   //  * While the weight is on its way the low-rank term is formed from the LDS (a wave's loads return in
-  //    order: a wait that leaves only the weight loads outstanding has the staged pieces).
-  //  * Then the codes are requested, the MFMAs run as their operands arrive, and what is left behind
-  //    them is the sum over the waves and one line of float32 arithmetic per output.
+  //    order: a wait that leaves only the code and weight loads outstanding has the staged pieces).
+  //  * The MFMAs run as their operands arrive, and what is left behind them is the sum over the waves and
+  //    one line of float32 arithmetic per output.
   const bool one_round = !ROWS2 && n_pairs == kSkinnyStreamWaves * kInFlight && (!lora || early);  // workgroup-uniform
   if (one_round) {
     // the staged operands first: a handful of instructions, and their data is then in the LDS long before
@@ -442,14 +427,19 @@ __global__ __launch_bounds__(kSkinnyStreamThreads) void skinny_stream_kernel(Ski
     v4i wf[kInFlight], xf[kInFlight];
     const unsigned char* wb = wsrc + (size_t)p0 * 2u * kBlockBytes;
     const unsigned char* xb = xsrc + (size_t)p0 * 2u * kBlockBytes;
+    // (the codes first: they come from the L2 and are in the registers long before the weight, whose
+    // requests the memory takes at its own pace)
+#pragma unroll
+    for (uint32_t t = 0; t < kInFlight; ++t) xf[t] = *reinterpret_cast<const v4i*>(xb + t * 2u * kBlockBytes);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (uint32_t t = 0; t < kInFlight; ++t)
       wf[t] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wb + t * 2u * kBlockBytes));
     __builtin_amdgcn_sched_barrier(0);
     // ---- the low-rank term, while the weight is on its way: the staged operands are the wave's oldest
-    // loads, so a wait that leaves the kInFlight weight loads outstanding has them
+    // loads, so a wait that leaves the code and weight loads outstanding has them
     if (lora) {
-      asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kInFlight) : "memory");
+      asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * kInFlight) : "memory");
       __syncthreads();  // ... and the other waves' pieces
       {  // z[m][r] for 16 rows x 32 ranks, one per thread: four interleaved partial sums, combined in a fixed order
         const uint32_t zr = tid >> 5, zc = tid & 31u;
@@ -485,9 +475,6 @@ __global__ __launch_bounds__(kSkinnyStreamThreads) void skinny_stream_kernel(Ski
         low = lo2[0] + lo2[1];
       }
     }
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (uint32_t t = 0; t < kInFlight; ++t) xf[t] = *reinterpret_cast<const v4i*>(xb + t * 2u * kBlockBytes);
     __builtin_amdgcn_sched_barrier(0);
     // four accumulators take turns, so that no MFMA waits for the one before it (integer sums: any order)
     v4i part[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};

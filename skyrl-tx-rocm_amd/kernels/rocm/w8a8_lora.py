@@ -361,8 +361,11 @@ class ForwardPlan:
         # (a captured call is replayed later, when the adapters may have changed: it always packs)
         capturing = torch.cuda.is_current_stream_capturing()
         if self._lora is not None and not capturing and self.keep_lora_pack:
+            # (what the workspace holds also depends on the path the flags choose: decode kernels keep B
+            # regrouped per row, the tiled kernels A and B in operand order)
             key = (self._lora[0]._version, self._lora[1]._version,
-                   None if self.adapter_indices is None else self.adapter_indices._version)
+                   None if self.adapter_indices is None else self.adapter_indices._version,
+                   flags & ~(_native.FLAG_SKIP_PROLOGUE | _native.FLAG_SKIP_GEMM | _native.FLAG_LORA_PACK_VALID))
             if key == self._packed_lora_key:
                 flags |= _native.FLAG_LORA_PACK_VALID
         self.problem.flags = flags

@@ -235,3 +235,37 @@ def test_same_named_fused_entry_points_validate_like_the_reference(native):
         down(x, torch.zeros(64, 16, dtype=torch.bfloat16), a, b, s, res, enabled=True)
     with pytest.raises(RuntimeError, match="GPU"):
         down(x, w, a, b, s, res, enabled=True)
+
+
+def test_bounded_frozen_lora_linear_argument_checks():
+    """The reference's argument checks (skyrl/tx/kernels/bounded_lora.py:31-108) before anything touches a GPU."""
+    import torch
+
+    from __graft_entry__ import load_package
+
+    pkg = load_package()
+    bounded = pkg.bounded_lora.bounded_frozen_lora_linear
+    ql = pkg.quantized_lora
+    x = torch.zeros((2, 5, 16), dtype=torch.bfloat16)
+    w = ql.quantize_frozen_weight(torch.ones((16, 7), dtype=torch.float32), bits=8, group_size=16)
+    a = torch.zeros((16, 8), dtype=torch.bfloat16)
+    b = torch.zeros((8, 7), dtype=torch.bfloat16)
+    with pytest.raises(TypeError, match="token_tile_size must be an integer"):
+        bounded(x, w, a, b, 1.0, token_tile_size=True)
+    with pytest.raises(ValueError, match=r"token_tile_size must be in \[1, 2048\]"):
+        bounded(x, w, a, b, 1.0, token_tile_size=0)
+    with pytest.raises(TypeError, match="GroupQuantizedWeight"):
+        bounded(x, torch.zeros((16, 7), dtype=torch.bfloat16), a, b, 1.0)
+    with pytest.raises(ValueError, match="rank-two"):
+        bounded(x, w, a[None], b, 1.0)
+    with pytest.raises(ValueError, match=r"lora_a must have shape \(16, 8\)"):
+        bounded(x, w, torch.zeros((16, 4), dtype=torch.bfloat16), b, 1.0)
+    with pytest.raises(TypeError, match="floating scalar"):
+        bounded(x, w, a, b, torch.ones(2))
+    with pytest.raises(ValueError, match="residual shape"):
+        bounded(x, w, a, b, 1.0, residual=torch.zeros((2, 5, 8), dtype=torch.bfloat16))
+    with pytest.raises(TypeError, match="residual dtype"):
+        bounded(x, w, a, b, 1.0, residual=torch.zeros((2, 5, 7), dtype=torch.float32))
+    with pytest.raises(TypeError, match="x dtype must be BF16"):
+        bounded(x.float(), w, a, b, 1.0)
+

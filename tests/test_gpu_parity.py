@@ -620,6 +620,34 @@ def test_same_named_fused_entry_points(dev, pkg):
     np.testing.assert_array_equal(res.grad.float().cpu().numpy(), cot)     # the residual's cotangent is dy
 
 
+@pytest.mark.parametrize("token_tile_size", [1, 4, 6, 16])
+def test_bounded_frozen_lora_linear_forward_equation_across_token_tiles(dev, pkg, token_tile_size):
+    """``bounded_frozen_lora_linear`` (skyrl/tx/kernels/bounded_lora.py:121-140, :245-255) on a quantized
+    kernel: ``x @ W8A8 + s * (x @ A) @ B + residual`` for x of shape [2, 5, K] with the rank-8 single adapter,
+    scaling 0.375 and residual of the reference's own test
+    (tests/tx/kernels/test_bounded_lora.py:23-43).  The result is the oracle's, does not depend on
+    ``token_tile_size``, and is what the same rows give when they are passed in pieces of that size."""
+    import torch
+
+    bounded = pkg.bounded_lora.bounded_frozen_lora_linear
+    case = wc.make_case(10, 16, 7, n_adapters=1, rank=8, seed=33, residual=True, idx_mode="zero")
+    case["s"] = np.asarray([0.375], F32)
+    t = wc.to_torch(case, dev)
+    x3, res3 = t["x"].reshape(2, 5, 16), t["residual"].reshape(2, 5, 7)
+    out = bounded(x3, t["weight"], t["a"][0], t["b"][0], 0.375, residual=res3, token_tile_size=token_tile_size)
+    ref_tile = bounded(x3, t["weight"], t["a"][0], t["b"][0], 0.375, residual=res3, token_tile_size=512)
+    torch.cuda.synchronize()
+    assert tuple(out.shape) == (2, 5, 7)
+    assert torch.equal(out.view(torch.int16), ref_tile.view(torch.int16))
+    assert wc.compare(out.float().cpu().numpy().reshape(10, 7), wc.oracle_forward(case))["violations"] == 0
+    # (a piece is copied out: the C ABI wants 16-byte-aligned pointers, and a 7-column row is 14 bytes)
+    pieces = [bounded(t["x"][r0:r0 + token_tile_size].clone(), t["weight"], t["a"][0], t["b"][0], 0.375,
+                      residual=t["residual"][r0:r0 + token_tile_size].clone(), token_tile_size=token_tile_size)
+              for r0 in range(0, 10, token_tile_size)]
+    torch.cuda.synchronize()
+    assert torch.equal(torch.cat(pieces).view(torch.int16), out.reshape(10, 7).view(torch.int16))
+
+
 def test_lora_pack_is_reused_until_the_adapters_change(dev, pkg):
     """A plan keeps the transposed A / packed B in its workspace while the adapter tensors are unchanged
     (the second run is told so and must give the same bits), and packs again after an in-place update."""
@@ -641,6 +669,39 @@ def test_lora_pack_is_reused_until_the_adapters_change(dev, pkg):
     case2 = dict(case, b=case["b"] * np.float32(2.0))
     _assert_close(third.to(torch.float32).cpu().numpy(), wc.oracle_forward(case2), " after the update")
     assert not torch.equal(third.view(torch.int16), first.view(torch.int16))
+
+
+def test_lora_pack_survives_another_row_count_and_geometry(dev, pkg):
+    """The packed LoRA operands sit at the start of the workspace at places that depend on
+    (k, n, n_adapters, rank) only: a call with another m, other adapter indices and another tile geometry
+    on the same workspace may keep them (MI355_W8A8_FLAG_LORA_PACK_VALID) and gives the bits of a call
+    that packs for itself."""
+    import torch
+
+    w8, nat = pkg.w8a8_lora, pkg._native
+    big = wc.make_case(700, 512, 768, n_adapters=3, rank=16, seed=52, residual=True)
+    tb = wc.to_torch(big, dev)
+    plan_big = w8.ForwardPlan(tb["x"], tb["weight"], tb["a"], tb["b"], tb["s"], adapter_indices=tb["idx"],
+                              residual=tb["residual"], flags=nat.FLAG_TILE_256X128)
+    plan_big.run()  # packs A and B into its workspace
+    small = dict(big)
+    rng = np.random.default_rng(5)
+    rows = rng.permutation(700)[:150]
+    small.update(m=150, x=big["x"][rows], residual=big["residual"][rows],
+                 idx=rng.integers(0, 3, 150).astype(np.int32))
+    ts = wc.to_torch(small, dev)
+    ts["a"], ts["b"], ts["s"], ts["weight"] = tb["a"], tb["b"], tb["s"], tb["weight"]
+    plan_small = w8.ForwardPlan(ts["x"], ts["weight"], ts["a"], ts["b"], ts["s"], adapter_indices=ts["idx"],
+                                residual=ts["residual"], flags=nat.FLAG_TILE_128X128)
+    own = plan_small.run().clone()  # packs into its own workspace
+    # the same call on the larger call's workspace, told to keep what is there
+    plan_small.problem.workspace = plan_big.problem.workspace
+    plan_small.problem.workspace_bytes = plan_big.problem.workspace_bytes
+    plan_small.keep_lora_pack = False
+    kept = plan_small.run(nat.FLAG_LORA_PACK_VALID).clone()
+    torch.cuda.synchronize()
+    assert torch.equal(own.view(torch.int16), kept.view(torch.int16))
+    _assert_close(kept.to(torch.float32).cpu().numpy(), wc.oracle_forward(small), " kept pack, other m")
 
 
 @pytest.mark.parametrize("m", [8192, 8200])

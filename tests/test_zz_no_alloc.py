@@ -71,6 +71,67 @@ def test_static_workspace_matches_caller_workspace(pkg, shapes):
         assert rep["violations"] == 0, rep
 
 
+def test_static_workspace_allocates_nothing_and_replays_under_capture(pkg):
+    """After the first call on a device (which looks the array's address up) a call leaves the free device
+    memory as it found it, and a call captured into a HIP graph replays with the eager call's bits."""
+    import torch
+
+    dev = torch.device("cuda:0")
+    w8 = pkg.w8a8_lora
+    case = wc.make_case(260, 512, 520, n_adapters=3, rank=16, seed=47, residual=True)
+    t = wc.to_torch(case, dev)
+    plan = w8.ForwardPlan(t["x"], t["weight"], t["a"], t["b"], t["s"], adapter_indices=t["idx"],
+                          residual=t["residual"])
+    want = plan.run().clone()
+    first = _static_ws_forward(pkg, plan)  # warm-up: resolves the symbol's address
+    torch.cuda.synchronize()
+    native = pkg._native
+    lib = native.load()
+    p = native.Problem()
+    ctypes.memmove(ctypes.byref(p), ctypes.byref(plan.problem), ctypes.sizeof(p))
+    out = torch.full_like(plan.out, float("nan"))
+    p.out = out.data_ptr()
+    p.workspace, p.workspace_bytes = None, 0
+    p.aux_x_codes = p.aux_x_scales = p.aux_acc = p.aux_normalized = None
+    stream = torch.cuda.Stream(device=dev)
+    with torch.cuda.stream(stream):  # (the runtime sets a new stream's own resources up at its first launch)
+        assert lib.mi355_w8a8_forward_static_ws_v1(ctypes.byref(p), int(stream.cuda_stream)) == 0
+    stream.synchronize()
+    free_before = torch.cuda.mem_get_info(dev)[0]
+    with torch.cuda.stream(stream):
+        status = lib.mi355_w8a8_forward_static_ws_v1(ctypes.byref(p), int(stream.cuda_stream))
+    stream.synchronize()
+    assert status == 0
+    assert torch.cuda.mem_get_info(dev)[0] == free_before
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+    # captured: the library records kernel launches only (no allocation, no memset, no synchronisation)
+    graph = torch.cuda.CUDAGraph()
+    out.fill_(float("nan"))
+    with torch.cuda.graph(graph, stream=stream):
+        status = lib.mi355_w8a8_forward_static_ws_v1(ctypes.byref(p), int(torch.cuda.current_stream().cuda_stream))
+    assert status == 0
+    for _ in range(3):
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+    assert torch.equal(first.view(torch.int16), want.view(torch.int16))
+
+
+def test_static_workspace_refuses_to_keep_what_another_caller_may_have_overwritten(pkg):
+    """The array is shared by every caller of the process: flags that tell a call to reuse an earlier call's
+    packed operands or prologue are refused."""
+    native = pkg._native
+    lib = native.load()
+    p = native.Problem()
+    p.struct_size = ctypes.sizeof(p)
+    p.m, p.k, p.n, p.n_adapters, p.rank = 64, 256, 256, 2, 8
+    for flag in (native.FLAG_LORA_PACK_VALID, native.FLAG_SKIP_PROLOGUE):
+        p.flags = flag
+        assert lib.mi355_w8a8_forward_static_ws_v1(ctypes.byref(p), None) == -7  # MI355_W8A8_ERR_UNSUPPORTED
+
+
 def test_static_workspace_rejects_what_does_not_fit(pkg):
     """A problem whose workspace exceeds the static array is refused on the host, before any launch."""
     native = pkg._native
