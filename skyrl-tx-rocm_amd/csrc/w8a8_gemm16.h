@@ -41,6 +41,7 @@
 namespace w8a8 {
 
 typedef float v4f_t __attribute__((ext_vector_type(4)));
+typedef uint32_t v2u_t __attribute__((ext_vector_type(2)));
 
 constexpr int kG16TileM = 256;
 constexpr int kG16TileN = 256;
@@ -203,6 +204,11 @@ void w8a8_gemm16_kernel(GemmArgs g) {
   // 32-bit offset and a 32-bit lane offset, so no lane holds a 64-bit address.
   const __amdgpu_buffer_rsrc_t zrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(g.zp), 0, -1, 0x00020000);
   const __amdgpu_buffer_rsrc_t brsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(g.bp), 0, -1, 0x00020000);
+  // The output through the same kind of resource, for fragments stored without conditions: a lane then
+  // holds a 32-bit byte offset, which an output of less than 4 GiB (and 24-bit row and column counts,
+  // for the one-instruction product) allows.
+  const __amdgpu_buffer_rsrc_t orsrc = __builtin_amdgcn_make_buffer_rsrc(g.out, 0, -1, 0x00020000);
+  const bool out_small = g.M < (1u << 24) && n_out < (1u << 24) && (uint64_t)g.M * n_out < (1ull << 31);
   uint32_t g0 = 0;          // ring slot of the current tile's stage 0
   bool prefetched = false;  // the first stages of the current tile were requested by the previous tile
   // Two workgroups per CU: the one the dispatcher placed first (its LDS allocation starts at 0) runs at a
@@ -478,6 +484,16 @@ void w8a8_gemm16_kernel(GemmArgs g) {
     // consecutive original columns tcol0 + 4 c16 + j held by the accumulator blocks j.
     if (!wave_live) continue;  // wave beyond the last column; it still takes part in the next tile
     if constexpr (kLora) load_z(1, 1);
+    // Does every one of the wave's 128 slots hold a row of the output, and every lane four columns?
+    // (wave-uniform; true for all but the tiles at the end of an adapter's rows or of the matrix)
+    bool tile_plain = out_small && full_n && m0 + 128u <= total_rows;
+    if (g.src_row) {
+      const int2 s2 = *reinterpret_cast<const int2*>(rowdata + 512u + (uint32_t)lane * 8u);
+      const bool both = (uint32_t)s2.x < g.M && (uint32_t)s2.y < g.M;
+      tile_plain = tile_plain && (__builtin_amdgcn_ballot_w64(!both) == 0);
+    } else {
+      tile_plain = tile_plain && m0 + 128u <= g.M;
+    }
     const uint32_t ncol = tcol0 + 4u * c16;  // the lane's four consecutive columns
     float sw[4];
 #pragma unroll
@@ -505,16 +521,28 @@ void w8a8_gemm16_kernel(GemmArgs g) {
         const int4 r4 = *reinterpret_cast<const int4*>(rowdata + 512u + (16u * bi + 4u * q) * 4u);
         src[0] = r4.x; src[1] = r4.y; src[2] = r4.z; src[3] = r4.w;
       }
-      bool row_ok[4];
+      // Groups (adapters) present in the 32-row block of this fragment: one, except at a group
+      // boundary.  A boundary fragment is processed once per group; each pass stores its own rows.
+      const int glo = (int)(range[bi >> 1] & 0xffffu), ghi = (int)(range[bi >> 1] >> 16);
+      // The plain fragment (wave-uniform): every row of the wave's tile exists, all four columns of every
+      // lane exist, one adapter.  It runs without any per-row condition and stores through the buffer path.
+      const bool plain = EPI != kEpiAcc && tile_plain && !(kLora && ghi > glo);
+      bool row_ok[4] = {true, true, true, true};
       uint32_t off[4];
-      bool all_ok = true;
+      bool fast = true;
+      if (plain) {
 #pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        row_ok[v] = src[v] >= 0 && src[v] < (int)g.M;
-        off[v] = row_ok[v] ? (uint32_t)src[v] * ((EPI == kEpiAcc) ? g.N : n_out) : 0u;
-        all_ok = all_ok && row_ok[v];
+        for (int v = 0; v < 4; ++v) off[v] = __umul24((uint32_t)src[v], n_out);
+      } else {
+        bool all_ok = true;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          row_ok[v] = src[v] >= 0 && src[v] < (int)g.M;
+          off[v] = row_ok[v] ? (uint32_t)src[v] * ((EPI == kEpiAcc) ? g.N : n_out) : 0u;
+          all_ok = all_ok && row_ok[v];
+        }
+        fast = full_n && (__builtin_amdgcn_ballot_w64(!all_ok) == 0);  // wave-uniform
       }
-      const bool fast = full_n && (__builtin_amdgcn_ballot_w64(!all_ok) == 0);  // wave-uniform
 
       if constexpr (EPI == kEpiAcc) {
 #pragma unroll
@@ -530,15 +558,12 @@ void w8a8_gemm16_kernel(GemmArgs g) {
           }
         }
       } else {
-        // Groups (adapters) present in the 32-row block of this fragment: one, except at a group
-        // boundary.  A boundary fragment is processed once per group; each pass stores its own rows.
-        const int glo = (int)(range[bi >> 1] & 0xffffu), ghi = (int)(range[bi >> 1] >> 16);
         int grp[4] = {glo, glo, glo, glo};
         if (kLora && g.slot_group && ghi > glo) {
           const int4 g4 = *reinterpret_cast<const int4*>(g.slot_group + p4);
           grp[0] = g4.x; grp[1] = g4.y; grp[2] = g4.z; grp[3] = g4.w;
         }
-        for (int gi = glo; gi <= ghi; ++gi) {  // wave-uniform
+        for (int gi = glo; gi <= ghi; ++gi) {  // wave-uniform (one pass, except at a boundary)
           // ---- low[bj][v] = s_g * (z @ B_g): z rows of this fragment, B columns of fragment bj.  The
           // three terms of a fragment run as three rounds over the four independent accumulators.
           v4f_t low[4];
@@ -565,11 +590,20 @@ void w8a8_gemm16_kernel(GemmArgs g) {
                 for (int v = 0; v < 4; ++v) low[bj][v] = low[bj][v] * sgrp;
             }
           }
-          {
+          // the fragment's rows; PLAIN is the form without per-row conditions
+          auto rows = [&](auto PLAIN) {
+            constexpr bool kPlain = decltype(PLAIN)::value;
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
-              bool row_valid = row_ok[v];
-              if (kLora && ghi > glo) row_valid = row_valid && (grp[v] == gi);  // boundary: own rows only
+              bool row_valid = true;
+              uint32_t offv = off[v], ncolv = ncol;
+              if constexpr (!kPlain) {
+                row_valid = row_ok[v];
+                if (kLora && ghi > glo) row_valid = row_valid && (grp[v] == gi);  // boundary: own rows only
+                // (the addresses and column conditions of this form are formed here, not ahead of the branch
+                // where the plain form would pay for them too)
+                asm volatile("" : "+v"(offv), "+v"(ncolv));
+              }
               float y[4];
 #pragma unroll
               for (int j = 0; j < 4; ++j) {
@@ -584,27 +618,31 @@ void w8a8_gemm16_kernel(GemmArgs g) {
                 const uint32_t f0 = pack_bf16x2(y[0], y[1]), f1 = pack_bf16x2(y[2], y[3]);
                 const float p0 = swiglu_f32(__uint_as_float(f0 << 16), __uint_as_float(f0 & 0xffff0000u));
                 const float p1 = swiglu_f32(__uint_as_float(f1 << 16), __uint_as_float(f1 & 0xffff0000u));
-                if (!row_valid) continue;
+                if (!kPlain && !row_valid) continue;
                 const uint32_t pk = pack_bf16x2(p0, p1);
-                uint16_t* o = reinterpret_cast<uint16_t*>(g.out) + off[v] + (ncol >> 1);
-                if (fast) {
-                  *reinterpret_cast<uint32_t*>(o) = pk;
+                if constexpr (kPlain) {
+                  __builtin_amdgcn_raw_buffer_store_b32(pk, orsrc, 2u * offv + ncolv, 0, 0);
                 } else {
-                  if ((ncol >> 1) < n_out) o[0] = (uint16_t)(pk & 0xffffu);
-                  if ((ncol >> 1) + 1u < n_out) o[1] = (uint16_t)(pk >> 16);
+                  uint16_t* o = reinterpret_cast<uint16_t*>(g.out) + offv + (ncolv >> 1);
+                  if (fast) {
+                    *reinterpret_cast<uint32_t*>(o) = pk;
+                  } else {
+                    if ((ncolv >> 1) < n_out) o[0] = (uint16_t)(pk & 0xffffu);
+                    if ((ncolv >> 1) + 1u < n_out) o[1] = (uint16_t)(pk >> 16);
+                  }
                 }
               } else {
-                if (!row_valid) continue;
+                if (!kPlain && !row_valid) continue;
                 if (g.residual) {
                   uint32_t r0 = 0, r1 = 0;
-                  if (fast) {
-                    const uint2 rr = *reinterpret_cast<const uint2*>(g.residual + off[v] + ncol);
+                  if (kPlain || fast) {
+                    const uint2 rr = *reinterpret_cast<const uint2*>(g.residual + offv + ncolv);
                     r0 = rr.x; r1 = rr.y;
                   } else {
-                    if (ncol + 0u < g.N) r0 |= (uint32_t)g.residual[off[v] + ncol + 0u];
-                    if (ncol + 1u < g.N) r0 |= (uint32_t)g.residual[off[v] + ncol + 1u] << 16;
-                    if (ncol + 2u < g.N) r1 |= (uint32_t)g.residual[off[v] + ncol + 2u];
-                    if (ncol + 3u < g.N) r1 |= (uint32_t)g.residual[off[v] + ncol + 3u] << 16;
+                    if (ncolv + 0u < g.N) r0 |= (uint32_t)g.residual[offv + ncolv + 0u];
+                    if (ncolv + 1u < g.N) r0 |= (uint32_t)g.residual[offv + ncolv + 1u] << 16;
+                    if (ncolv + 2u < g.N) r1 |= (uint32_t)g.residual[offv + ncolv + 2u];
+                    if (ncolv + 3u < g.N) r1 |= (uint32_t)g.residual[offv + ncolv + 3u] << 16;
                   }
                   y[0] = y[0] + __uint_as_float(r0 << 16);
                   y[1] = y[1] + __uint_as_float(r0 & 0xffff0000u);
@@ -612,18 +650,23 @@ void w8a8_gemm16_kernel(GemmArgs g) {
                   y[3] = y[3] + __uint_as_float(r1 & 0xffff0000u);
                 }
                 const uint32_t lo = pack_bf16x2(y[0], y[1]), hi = pack_bf16x2(y[2], y[3]);
-                uint16_t* o = reinterpret_cast<uint16_t*>(g.out) + off[v] + ncol;
-                if (fast) {
-                  *reinterpret_cast<uint2*>(o) = make_uint2(lo, hi);
+                if constexpr (kPlain) {
+                  __builtin_amdgcn_raw_buffer_store_b64(v2u_t{lo, hi}, orsrc, 2u * (offv + ncolv), 0, 0);
                 } else {
-                  if (ncol + 0u < g.N) o[0] = (uint16_t)(lo & 0xffffu);
-                  if (ncol + 1u < g.N) o[1] = (uint16_t)(lo >> 16);
-                  if (ncol + 2u < g.N) o[2] = (uint16_t)(hi & 0xffffu);
-                  if (ncol + 3u < g.N) o[3] = (uint16_t)(hi >> 16);
+                  uint16_t* o = reinterpret_cast<uint16_t*>(g.out) + offv + ncolv;
+                  if (fast) {
+                    *reinterpret_cast<uint2*>(o) = make_uint2(lo, hi);
+                  } else {
+                    if (ncolv + 0u < g.N) o[0] = (uint16_t)(lo & 0xffffu);
+                    if (ncolv + 1u < g.N) o[1] = (uint16_t)(lo >> 16);
+                    if (ncolv + 2u < g.N) o[2] = (uint16_t)(hi & 0xffffu);
+                    if (ncolv + 3u < g.N) o[3] = (uint16_t)(hi >> 16);
+                  }
                 }
               }
             }
-          }
+          };
+          if (plain) rows(std::true_type{}); else rows(std::false_type{});
         }  // groups of the fragment
         // this fragment's z operands are spent: their ring slot takes the fragment two ahead
         if constexpr (kLora && bi + 2 < 8) load_z(bi & 1, bi + 2);
