@@ -524,9 +524,11 @@ void w8a8_gemm16_kernel(GemmArgs g) {
       // Groups (adapters) present in the 32-row block of this fragment: one, except at a group
       // boundary.  A boundary fragment is processed once per group; each pass stores its own rows.
       const int glo = (int)(range[bi >> 1] & 0xffffu), ghi = (int)(range[bi >> 1] >> 16);
-      // The plain fragment (wave-uniform): every row of the wave's tile exists, all four columns of every
-      // lane exist, one adapter.  It runs without any per-row condition and stores through the buffer path.
-      const bool plain = EPI != kEpiAcc && tile_plain && !(kLora && ghi > glo);
+      // The plain fragment (wave-uniform): every row of the wave's tile exists and all four columns of every
+      // lane exist.  It runs without per-row conditions and stores through the buffer path; where two
+      // adapters meet in its 32-row block, each adapter's pass stores the rows that are its own.
+      const bool plain = EPI != kEpiAcc && tile_plain;
+      const bool boundary = kLora && ghi > glo;
       bool row_ok[4] = {true, true, true, true};
       uint32_t off[4];
       bool fast = true;
@@ -590,9 +592,10 @@ void w8a8_gemm16_kernel(GemmArgs g) {
                 for (int v = 0; v < 4; ++v) low[bj][v] = low[bj][v] * sgrp;
             }
           }
-          // the fragment's rows; PLAIN is the form without per-row conditions
-          auto rows = [&](auto PLAIN) {
-            constexpr bool kPlain = decltype(PLAIN)::value;
+          // the fragment's rows; MODE 0 is the general form, 1 the plain one, 2 the plain one of a boundary pass
+          auto rows = [&](auto MODE) {
+            constexpr bool kPlain = decltype(MODE)::value != 0;
+            constexpr bool kOwnRows = decltype(MODE)::value == 2;
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
               bool row_valid = true;
@@ -621,7 +624,7 @@ void w8a8_gemm16_kernel(GemmArgs g) {
                 if (!kPlain && !row_valid) continue;
                 const uint32_t pk = pack_bf16x2(p0, p1);
                 if constexpr (kPlain) {
-                  __builtin_amdgcn_raw_buffer_store_b32(pk, orsrc, 2u * offv + ncolv, 0, 0);
+                  if (!kOwnRows || grp[v] == gi) __builtin_amdgcn_raw_buffer_store_b32(pk, orsrc, 2u * offv + ncolv, 0, 0);
                 } else {
                   uint16_t* o = reinterpret_cast<uint16_t*>(g.out) + offv + (ncolv >> 1);
                   if (fast) {
@@ -651,7 +654,7 @@ void w8a8_gemm16_kernel(GemmArgs g) {
                 }
                 const uint32_t lo = pack_bf16x2(y[0], y[1]), hi = pack_bf16x2(y[2], y[3]);
                 if constexpr (kPlain) {
-                  __builtin_amdgcn_raw_buffer_store_b64(v2u_t{lo, hi}, orsrc, 2u * (offv + ncolv), 0, 0);
+                  if (!kOwnRows || grp[v] == gi) __builtin_amdgcn_raw_buffer_store_b64(v2u_t{lo, hi}, orsrc, 2u * (offv + ncolv), 0, 0);
                 } else {
                   uint16_t* o = reinterpret_cast<uint16_t*>(g.out) + offv + ncolv;
                   if (fast) {
@@ -666,7 +669,9 @@ void w8a8_gemm16_kernel(GemmArgs g) {
               }
             }
           };
-          if (plain) rows(std::true_type{}); else rows(std::false_type{});
+          if (!plain) rows(std::integral_constant<int, 0>{});
+          else if (!boundary) rows(std::integral_constant<int, 1>{});
+          else rows(std::integral_constant<int, 2>{});
         }  // groups of the fragment
         // this fragment's z operands are spent: their ring slot takes the fragment two ahead
         if constexpr (kLora && bi + 2 < 8) load_z(bi & 1, bi + 2);
