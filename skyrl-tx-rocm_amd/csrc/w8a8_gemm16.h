@@ -115,15 +115,18 @@ __device__ inline void g16_for(F&& f) {  // f(integral_constant<int, J>) for J0 
     g16_for<J0 + 1, J1>(f);
   }
 }
-// The integer MFMAs go through the compiler's builtin: it then knows which instruction produced an
-// accumulator and inserts the wait states the hardware does not interlock (an MFMA result read by the
-// vector ALU or moved between register classes), wherever its register allocation makes them necessary.
+// The integer MFMAs are written as assembly with the accumulator tied (one read-write operand).  Through
+// the builtin, destination and accumulator input are separate values, and in the stages ahead of and behind
+// the steady-state loop the register allocator used that freedom: it placed 19 of a tile's 32 accumulator
+// blocks elsewhere and moved them home through the vector registers, with the wait states that takes.
+// What the compiler no longer sees is that an MFMA wrote the accumulator, so it inserts no wait states
+// for a read of it by another unit; none is needed where this kernel reads one: a block is next touched by
+// the MFMA of the following stage (32 MFMAs on), and the epilogue starts behind explicit wait states.
 __device__ inline void g16_mfma(v4i& acc, const v4i& a, const v4i& b) {
-  acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc, 0, 0, 0);
+  asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
 }
 __device__ inline void g16_mfma_first(v4i& acc, const v4i& a, const v4i& b) {
-  const v4i zero = {0, 0, 0, 0};
-  acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, zero, 0, 0, 0);
+  asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, 0" : "=a"(acc) : "v"(a), "v"(b));
 }
 constexpr int g16_frag_off(int f) { return (f >> 1) * 2048 + (f & 1) * 256; }  // activation fragment f of a wave's four row blocks
 constexpr int g16_bfrag_off(int j) { return j * 2048; }                        // weight fragment j: the wave's half of column block j
@@ -467,6 +470,9 @@ void w8a8_gemm16_kernel(GemmArgs g) {
 
     preload();
     stage(I1{}, No{}, I0{}, KT - 1);  // the last stage (KT is even); it also requests the epilogue's operands
+    // (wait states between the last MFMAs and whatever the compiler schedules next: it does not know that the
+    // accumulators were just written, see g16_mfma; sixteen cover this MFMA's result latency)
+    asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");
     // The preloads were requested a stage ago and are the youngest loads in the queue.  After the wait
     // (the builtin, so that the compiler knows its loads are in) the next tile's fourth stage is requested
     // into the buffer the last barrier has freed.
