@@ -90,7 +90,7 @@ WORKLOADS = {
 # counter reads for the 256 MiB device copy of the same run (a kernel of known traffic, 16-byte loads).
 # workload -> (summary file, regular expressions naming the kernels whose traffic is summed)
 PROFILE_TRAFFIC = {
-    "qwen3-8b-gate_up-m4096": ("w8a8_gemm16_kernel__qwen3-8b-gate_up-m4096.txt", [r"w8a8_gemm16_kernel<1, 2>"]),
+    "qwen3-8b-gate_up-m4096": ("w8a8_gemm16_kernel__qwen3-8b-gate_up-m4096.txt", [r"w8a8_gemm16_kernel<1, 2, 4>"]),
     "qwen3-8b-down-m16-decode": ("skinny_stream_kernel__qwen3-8b-down-m16-decode.txt",
                                  [r"skinny_quant_kernel<", r"skinny_stream_kernel<"]),
     "qwen3-8b-gate_up-m4096-backward": ("bwd_dx_kernel__qwen3-8b-gate_up-m4096-backward.txt", [r"bwd_dx_kernel<"]),

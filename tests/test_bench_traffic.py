@@ -28,9 +28,9 @@ def test_parser_scales_by_the_copy_of_known_size(tmp_path):
     name = bench.PROFILE_TRAFFIC["qwen3-8b-gate_up-m4096"][0]
     lines = [
         "w8a8::cal_copy_kernel(int __vector(4) const*, int __vector(4)*, unsigned long)     grid   1048576  FETCH_SIZE avg     131072.0 KiB over 1 dispatches",
-        "void w8a8::w8a8_gemm16_kernel<1, 2>(w8a8::GemmArgs)                                grid    131072  FETCH_SIZE avg       1000.0 KiB over 15 dispatches",
+        "void w8a8::w8a8_gemm16_kernel<1, 2, 4>(w8a8::GemmArgs)                                grid    131072  FETCH_SIZE avg       1000.0 KiB over 15 dispatches",
         "w8a8::cal_copy_kernel(int __vector(4) const*, int __vector(4)*, unsigned long)     grid   1048576  WRITE_SIZE avg     262144.0 KiB over 1 dispatches",
-        "void w8a8::w8a8_gemm16_kernel<1, 2>(w8a8::GemmArgs)                                grid    131072  WRITE_SIZE avg        500.0 KiB over 15 dispatches",
+        "void w8a8::w8a8_gemm16_kernel<1, 2, 4>(w8a8::GemmArgs)                                grid    131072  WRITE_SIZE avg        500.0 KiB over 15 dispatches",
     ]
     (tmp_path / name).write_text("\n".join(lines) + "\n")
     assert bench.measured_traffic_bytes("qwen3-8b-gate_up-m4096", tmp_path) == int((1000.0 * 2.0 + 500.0) * 1024)
