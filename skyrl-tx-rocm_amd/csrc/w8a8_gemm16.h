@@ -578,19 +578,22 @@ void w8a8_gemm16_kernel(GemmArgs g) {
           if constexpr (kLora) {
             if (gi != bgroup) load_b(gi);  // wave-uniform: a new adapter begins in this fragment
             const float sgrp = bscale;
-#pragma unroll
-            for (int bj = 0; bj < 4; ++bj) low[bj] = v4f_t{0.f, 0.f, 0.f, 0.f};
+            // The low-rank accumulators live in ordinary registers (every accumulation register is taken by the
+            // integer accumulators), and the MFMAs write them there: assembly with the accumulator tied, as
+            // g16_mfma.  An accumulator's next MFMA is four MFMAs on; the wait states between the last MFMA
+            // and the first read by the vector ALU, which the compiler would insert for a builtin, are explicit.
 #pragma unroll
             for (int ks = 0; ks < kKS; ++ks)
 #pragma unroll
               for (int t3 = 2; t3 >= 0; --t3)
 #pragma unroll
-                for (int bj = 0; bj < 4; ++bj)
-                  low[bj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, zr[bi & 1][ks][t3]),
-                                                                    __builtin_bit_cast(v8bf, br[bj][ks]), low[bj], 0, 0, 0);
-            // the low-rank accumulators live in ordinary registers: every accumulation register is taken,
-            // and left to itself the compiler spills one of the integer accumulators to make room
-            asm volatile("" : "+v"(low[0]), "+v"(low[1]), "+v"(low[2]), "+v"(low[3]));
+                for (int bj = 0; bj < 4; ++bj) {
+                  if (ks == 0 && t3 == 2)  // (folded once the loops are unrolled)
+                    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=&v"(low[bj]) : "v"(zr[bi & 1][ks][t3]), "v"(br[bj][ks]));
+                  else
+                    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(low[bj]) : "v"(zr[bi & 1][ks][t3]), "v"(br[bj][ks]));
+                }
+            asm volatile("s_nop 7\n\ts_nop 7" : "+v"(low[0]), "+v"(low[1]), "+v"(low[2]), "+v"(low[3]));
             if (sgrp != 1.0f) {  // wave-uniform (a product with 1 is exact: leaving it out changes no bit)
 #pragma unroll
               for (int bj = 0; bj < 4; ++bj)
