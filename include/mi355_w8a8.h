@@ -94,6 +94,9 @@ typedef enum mi355_w8a8_status {
 /* For calls of at most 16 rows (rank <= 32) the flag covers something else: the per-row regrouped copy of B
  * the decode kernels keep in the workspace.  There it vouches that the earlier call was a decode call with
  * the same m and that lora_b and adapter_indices have the contents they had then. */
+/* mi355_w8a8_grouped_v1 takes the flag too: its launch that lays out the slots then leaves the transposed A
+ * and the packed B of an earlier grouped call on the same workspace with the same (k, n, n_groups, rank) as
+ * they are. */
 #define MI355_W8A8_FLAG_LORA_PACK_VALID 1024u
 
 /*

@@ -587,14 +587,16 @@ GroupedLayout make_grouped_layout(uint32_t m, uint32_t k, uint32_t n, uint32_t n
   w.n_steps = (k + 63u) / 64u;
   w.steps_per_wave = (w.n_steps + 15u) / 16u;
   uint64_t off = 0;
+  // (the LoRA operands a caller may vouch for come first, as in make_layout: their places depend on
+  // (k, n, n_groups, rank) only, not on the row count)
+  w.at = off; off += rank ? align256((uint64_t)n_groups * rank * k * 2u) : 0u;
+  w.bp = off; off += rank ? align256((uint64_t)n_groups * (n_padded(n) / 32u) * w.nkk * kBlockBytes) : 0u;
   w.xq = off; off += align256((uint64_t)w.slots * w.K_pad);
   w.sx = off; off += align256((uint64_t)w.slots * 4u);
   w.src_row = off; off += align256((uint64_t)w.slots * 4u);
   w.dst_pos = off; off += align256((uint64_t)m * 4u);
   w.blk_range = off; off += align256((uint64_t)(w.slots / 32u) * 4u);
   w.zp = off; off += rank ? align256((uint64_t)(w.slots / 32u) * w.nkk * 3u * kBlockBytes) : 0u;
-  w.at = off; off += rank ? align256((uint64_t)n_groups * rank * k * 2u) : 0u;
-  w.bp = off; off += rank ? align256((uint64_t)n_groups * (n_padded(n) / 32u) * w.nkk * kBlockBytes) : 0u;
   w.total = off;
   return w;
 }
@@ -661,7 +663,9 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
     pa.ncb = n_padded(p->n) / 32u; pa.slots = w.slots;
     pa.route_blocks = 1;
     uint32_t b_blocks = 0;
-    if (lora) {
+    // (a caller that vouches for the operand packs of an earlier call on this workspace keeps them: the
+    // launch then only lays out the slots)
+    if (lora && !(p->flags & MI355_W8A8_FLAG_LORA_PACK_VALID)) {
       const uint64_t a_items = (uint64_t)p->n_groups * p->k * ((p->rank + 7u) / 8u);
       const uint64_t b_items = (uint64_t)p->n_groups * pa.ncb * w.nkk * 64u;
       pa.a_blocks = (uint32_t)((a_items + 1023u) / 1024u);

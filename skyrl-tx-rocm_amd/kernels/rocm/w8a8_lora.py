@@ -888,15 +888,32 @@ class GroupedForwardPlan:
         self.problem = p
         self.flags = flags
         self._lib = lib
+        self._lora = (a3, b3) if r else None
+        self._packed_lora_key = None  # versions of A and B the workspace holds in operand order
+        self.keep_lora_pack = True    # False: pack on every run
 
     def run(self, extra_flags: int = 0) -> torch.Tensor:
         """Enqueue the call on torch's current stream; returns the (reused) output tensor.  ``extra_flags``
-        adds the measurement flags ``FLAG_SKIP_PROLOGUE`` / ``FLAG_SKIP_GEMM`` for this run."""
-        self.problem.flags = self.flags | extra_flags
+        adds the measurement flags ``FLAG_SKIP_PROLOGUE`` / ``FLAG_SKIP_GEMM`` for this run.
+
+        As in ``ForwardPlan.run``: while neither adapter tensor has been written since the last full run
+        (``Tensor._version``) the call keeps the operand packs in its workspace
+        (``FLAG_LORA_PACK_VALID``); never under graph capture."""
+        flags = self.flags | extra_flags
+        key = None
+        capturing = torch.cuda.is_current_stream_capturing()
+        if self._lora is not None and not capturing and self.keep_lora_pack:
+            key = (self._lora[0]._version, self._lora[1]._version,
+                   flags & ~(_native.FLAG_SKIP_PROLOGUE | _native.FLAG_SKIP_GEMM | _native.FLAG_LORA_PACK_VALID))
+            if key == self._packed_lora_key:
+                flags |= _native.FLAG_LORA_PACK_VALID
+        self.problem.flags = flags
         with torch.cuda.device(self.device):
             status = self._lib.mi355_w8a8_grouped_v1(ctypes.byref(self.problem), _stream_ptr(self.device))
         self.problem.flags = self.flags
         _native.check("mi355_w8a8_grouped_v1", status)
+        if not extra_flags & _native.FLAG_SKIP_PROLOGUE and not capturing:
+            self._packed_lora_key = key
         return self.out
 
 

@@ -463,6 +463,44 @@ def test_grouped_ragged_linear(dev, pkg, sizes, k, n, rank, swiglu, extra, tile_
     _assert_close(got, want, f" grouped {sizes} {k}x{n}")
 
 
+def test_grouped_plan_keeps_the_lora_packs_until_an_adapter_tensor_is_written(dev, pkg):
+    """A grouped plan packs A and B on its first run, keeps the packs while neither tensor is written
+    (the second run is told so and gives the same bits), and packs again after an in-place update."""
+    import torch
+
+    sizes, k, n, rank = [40, 3, 0, 70, 129], 384, 512, 16
+    rng = np.random.default_rng(606)
+    m, x, codes, scales, a, b = _grouped_case(rng, sizes, k, n, rank)
+    s = F32(0.75)
+    weights = [o.GroupQuantizedWeight(codes[e], scales[e:e + 1], k, k, 8, k) for e in range(len(sizes))]
+    st = np.concatenate(([0], np.cumsum(sizes)))
+
+    def oracle(bb):
+        want = np.zeros((m, n), F32)
+        for e, w in enumerate(weights):
+            r0, r1 = int(st[e]), int(st[e + 1])
+            if r1 > r0:
+                want[r0:r1] = o.quantized_lora_linear_f32(x[r0:r1], w, a[e], bb[e], s)
+        return o.bf16_round(want)
+
+    w8 = pkg.w8a8_lora
+    bf = lambda t: torch.from_numpy(np.ascontiguousarray(t)).to(dev).to(torch.bfloat16)
+    gw = w8.prepare_grouped_weight(torch.from_numpy(codes).to(dev), torch.from_numpy(scales).to(dev))
+    ta, tb = bf(a), bf(b)
+    plan = w8.GroupedForwardPlan(bf(x), torch.tensor(sizes, dtype=torch.int32), gw, ta, tb, float(s))
+    first = plan.run().clone()
+    assert plan._packed_lora_key is not None
+    second = plan.run().clone()           # packs kept
+    assert torch.equal(first.view(torch.int16), second.view(torch.int16))
+    _assert_close(first.float().cpu().numpy(), oracle(b), " grouped first run")
+    tb.mul_(-1.0)                         # in place: the version counter moves, the next run packs again
+    third = plan.run().clone()
+    _assert_close(third.float().cpu().numpy(), oracle(-b), " grouped after new B")
+    plan.keep_lora_pack = False
+    fourth = plan.run().clone()
+    assert torch.equal(third.view(torch.int16), fourth.view(torch.int16))
+
+
 def test_moe_expert_mlp_reduced(dev, pkg):
     """Config 5 at reduced size: top-4 of 16 experts, hidden 256, intermediate 128, rank 16."""
     import torch
