@@ -100,7 +100,7 @@ PROFILE_TRAFFIC = {
                                                  [r"bwd_pack_dy_kernel<0>", r"bwd_dx_kernel<0, true>"]),
     "qwen3-8b-gate_up-m4096-fused-backward": ("swiglu_bwd_kernel__qwen3-8b-gate_up-m4096-fused-backward.txt",
                                               [r"bwd_dx_kernel<"]),
-    "qwen3-8b-down-m4096-w4a8-g128": ("gq_gemm_kernel__qwen3-8b-down-m4096-w4a8-g128.txt", [r"gq_gemm_kernel<"]),
+    "qwen3-8b-down-m4096-w4a8-g128": ("gq_gemm_kernel__qwen3-8b-down-m4096-w4a8-g128.txt", [r"gq_gemm_(lds_)?kernel<"]),
     "qwen3-30b-a3b-moe-routing-t4096": ("moe_spread_kernel__qwen3-30b-a3b-moe-routing-t4096.txt",
                                         [r"moe_hist_kernel", r"moe_scan_kernel", r"moe_scatter_kernel",
                                          r"moe_spread_kernel"]),
@@ -887,7 +887,7 @@ def bench_gq(args, cfg, pkg, dev):
         "config": {"workload": args.workload, **{kk: v for kk, v in cfg.items() if kk != "seed"}},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
                      "frac": achieved / INT8_PEAK_TOPS, "traffic": measured_traffic_bytes(args.workload),
-                     "kernel": "gq_gemm_kernel (timed with gq_quant_kernel and gq_lora_z_kernel: whole calls)",
+                     "kernel": "gq_gemm_lds_kernel (timed with gq_quant_kernel and the LoRA-A launches: whole calls)",
                      "kernel_avg_ms": call_ms, "algorithmic_ops": ops,
                      "algorithmic_bytes": 2 * m * k + k * n * wb // 8 + 4 * (k // group) * n + 2 * m * n},
     }

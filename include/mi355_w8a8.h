@@ -516,9 +516,14 @@ uint64_t mi355_w8a8_gq_packed_weight_bytes(uint32_t k_pad, uint32_t n, uint32_t 
 int mi355_w8a8_gq_pack_weight_v1(const void* codes, void* packed, uint32_t k_pad, uint32_t n, uint32_t weight_bits,
                                  void* stream);
 
+/* Calls of more than 32 rows whose groups are multiples of 64 run on 128 x 128 tiles staged through the LDS;
+ * this flag asks for the kernel that feeds its wave tiles straight from the L2 instead (the only one for
+ * other group sizes).  Both give the same bits; the flag exists for that comparison and for measurements. */
+#define MI355_W8A8_FLAG_GQ_DIRECT 1u
+
 typedef struct mi355_w8a8_gq_problem {
   uint32_t struct_size;      /* sizeof(mi355_w8a8_gq_problem) */
-  uint32_t flags;            /* 0 */
+  uint32_t flags;            /* 0 or MI355_W8A8_FLAG_GQ_DIRECT */
   uint32_t m, k, k_pad, n;
   uint32_t group_size;       /* multiple of 32, divides k_pad */
   uint32_t weight_bits;      /* 4 or 8 */

@@ -26,6 +26,7 @@ FLAG_GROUPED_TILE128 = 512
 FLAG_LORA_PACK_VALID = 1024
 FLAG_TILE_128X128 = 2048
 FLAG_TILE_256X128_PAIR = 4096
+FLAG_GQ_DIRECT = 1  # mi355_w8a8_gq_problem.flags
 STATIC_WORKSPACE_BYTES = 32 << 20
 PATH_NAMES = {1: "skinny", 2: "skinny-chunks", 3: "tiled-256x128", 4: "tiled-256x256", 5: "tiled-128x128",
               6: "tiled-256x128-pair"}

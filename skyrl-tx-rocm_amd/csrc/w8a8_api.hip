@@ -1651,7 +1651,7 @@ int run_gq_pack(const void* codes, void* packed, uint32_t k_pad, uint32_t n, uin
 int run_gq_linear(const mi355_w8a8_gq_problem* p, hipStream_t s) {
   if (!p) return MI355_W8A8_ERR_NULL;
   if (p->struct_size != sizeof(mi355_w8a8_gq_problem)) return MI355_W8A8_ERR_STRUCT;
-  if (p->flags) return MI355_W8A8_ERR_SHAPE;
+  if (p->flags & ~MI355_W8A8_FLAG_GQ_DIRECT) return MI355_W8A8_ERR_SHAPE;
   int st = validate_gq_dims(p->m, p->k_pad, p->group_size, p->rank);
   if (st) return st;
   if (p->n == 0 || p->k == 0 || p->k > p->k_pad) return MI355_W8A8_ERR_SHAPE;
@@ -1776,6 +1776,22 @@ int run_gq_linear(const mi355_w8a8_gq_problem* p, hipStream_t s) {
     const dim3 sgrid(g.n_col_blocks), sblock(kGqSkinnyWaves * 64u);
     if (p->weight_bits == 4u) hipLaunchKernelGGL((gq_skinny_kernel<true>), sgrid, sblock, 0, s, g);
     else hipLaunchKernelGGL((gq_skinny_kernel<false>), sgrid, sblock, 0, s, g);
+    return launch_status();
+  }
+  if (p->group_size % 64u == 0 && !(p->flags & MI355_W8A8_FLAG_GQ_DIRECT)) {
+    // groups of whole 64-wide k steps: 128 x 128 tiles staged through the LDS
+    const dim3 grid((g.n_col_blocks + 3u) / 4u, (L.m_pad / 32u + 3u) / 4u), block(256);
+    if (p->weight_bits == 4u) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gq_gemm_lds_kernel<true>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)gq_lds_bytes(true)) != hipSuccess)
+        return MI355_W8A8_ERR_LAUNCH;
+      hipLaunchKernelGGL((gq_gemm_lds_kernel<true>), grid, block, gq_lds_bytes(true), s, g);
+    } else {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gq_gemm_lds_kernel<false>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)gq_lds_bytes(false)) != hipSuccess)
+        return MI355_W8A8_ERR_LAUNCH;
+      hipLaunchKernelGGL((gq_gemm_lds_kernel<false>), grid, block, gq_lds_bytes(false), s, g);
+    }
     return launch_status();
   }
   const dim3 grid((g.n_col_blocks + 7u) / 8u, (L.m_pad / 32u + 1u) / 2u), block(256);

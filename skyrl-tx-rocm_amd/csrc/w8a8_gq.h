@@ -294,58 +294,83 @@ __device__ inline void gq_store_row_block(const GqGemmArgs& a, const float (&out
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);
     __builtin_amdgcn_wave_barrier();
-    int ad_row[16];
+    // The low-rank term on the matrix core: per 16 ranks the lane's eight z values (row lane % 32) are split
+    // exactly into three bf16 terms once; every adapter present among the block's rows then takes one pass
+    // in which the rows of the other adapters are zeroed, against its B values of the lane's column
+    // (v_mfma_f32_32x32x16_bf16: the result lands in the layout of the integer blocks).  A row's sum is
+    // scaled by its adapter's factor afterwards.
+    const uint32_t rowl = lane & 31u, kg = lane >> 5;
+    const uint32_t rowg = rb * 32u + rowl;
+    int my_ad = -1;  // rows beyond M belong to no adapter
+    if (rowg < a.M) {
+      const int ad = a.idx ? a.idx[rowg] : 0;
+      my_ad = ad < 0 ? 0 : (ad >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad);
+    }
+    v16f lacc[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) lacc[j][v] = 0.0f;
+    for (uint32_t r0 = 0; r0 < a.r; r0 += 16u) {
+      uint32_t term[3][4];
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        float hi[2], mid[2], lo[2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          const float z = zbuf[rowl][r0 + 8u * kg + 2u * (uint32_t)d + (uint32_t)e];  // (zeros beyond the rank)
+          hi[e] = bf16_round_f32(z);
+          const float r1 = z - hi[e];
+          mid[e] = bf16_round_f32(r1);
+          lo[e] = bf16_round_f32(r1 - mid[e]);
+        }
+        term[0][d] = pack_bf16x2(hi[0], hi[1]);
+        term[1][d] = pack_bf16x2(mid[0], mid[1]);
+        term[2][d] = pack_bf16x2(lo[0], lo[1]);
+      }
+      int done_below = -1;
+      for (;;) {  // adapters present among the block's rows, smallest first (wave-uniform)
+        int cand = my_ad > done_below ? my_ad : 0x7fffffff;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+          const int o = __shfl_xor(cand, off);
+          cand = o < cand ? o : cand;
+        }
+        if (cand == 0x7fffffff) break;
+        done_below = cand;
+        const bool mine = my_ad == cand;
+        v4i za[3];
+#pragma unroll
+        for (int t = 0; t < 3; ++t)
+#pragma unroll
+          for (int d = 0; d < 4; ++d) za[t][d] = mine ? (int)term[t][d] : 0;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          if (j == 1 && !two_cols) break;
+          uint32_t braw[8];
+#pragma unroll
+          for (uint32_t e = 0; e < 8; ++e) {
+            const uint32_t rank = r0 + 8u * kg + e;
+            braw[e] = (col[j] < a.N && rank < a.r) ? (uint32_t)a.lora_b[((size_t)cand * a.r + rank) * a.N + col[j]] : 0u;
+          }
+          v4i bo;
+#pragma unroll
+          for (int d = 0; d < 4; ++d) bo[d] = (int)(braw[2 * d] | (braw[2 * d + 1] << 16));
+#pragma unroll
+          for (int t = 2; t >= 0; --t)
+            lacc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, za[t]), __builtin_bit_cast(v8bf, bo),
+                                                              lacc[j], 0, 0, 0);
+        }
+      }
+    }
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
       const uint32_t row = rb * 32u + 8u * (v >> 2) + 4u * h + (v & 3);
       int ad = (a.idx && row < a.M) ? a.idx[row] : 0;
-      ad_row[v] = ad < 0 ? 0 : (ad >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad);
+      ad = ad < 0 ? 0 : (ad >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad);
+      const float sg = a.lora_scaling[ad];
 #pragma unroll
-      for (int j = 0; j < 2; ++j) low[j][v] = 0.0f;
-    }
-    // adapters present among the wave's rows, smallest first; every round handles one of them
-    int done_below = -1;
-    for (;;) {
-      int cand = 0x7fffffff;
-#pragma unroll
-      for (int v = 0; v < 16; ++v)
-        if (ad_row[v] > done_below && ad_row[v] < cand) cand = ad_row[v];
-#pragma unroll
-      for (int off = 32; off > 0; off >>= 1) {
-        const int o = __shfl_xor(cand, off);
-        cand = o < cand ? o : cand;
-      }
-      if (cand == 0x7fffffff) break;
-      done_below = cand;
-      const float sg = a.lora_scaling[cand];
-      for (uint32_t r0 = 0; r0 < a.r; r0 += 16u) {  // sixteen ranks of B in flight at a time
-        uint16_t braw[2][16];
-#pragma unroll
-        for (uint32_t t = 0; t < 16; ++t)
-#pragma unroll
-          for (int j = 0; j < 2; ++j)
-            braw[j][t] = (col[j] < a.N && r0 + t < a.r) ? a.lora_b[((size_t)cand * a.r + r0 + t) * a.N + col[j]]
-                                                         : (uint16_t)0;
-#pragma unroll
-        for (uint32_t t = 0; t < 16; ++t) {
-          if (r0 + t >= a.r) break;
-          const float bv[2] = {bf16_bits_to_f32(braw[0][t]), bf16_bits_to_f32(braw[1][t])};
-#pragma unroll
-          for (int v = 0; v < 16; ++v) {
-            const float zv = zbuf[8 * (v >> 2) + 4 * (int)h + (v & 3)][r0 + t];
-            if (ad_row[v] == cand) {
-#pragma unroll
-              for (int j = 0; j < 2; ++j) low[j][v] = fmaf(zv, bv[j], low[j][v]);
-            }
-          }
-        }
-      }
-#pragma unroll
-      for (int v = 0; v < 16; ++v)
-        if (ad_row[v] == cand) {
-#pragma unroll
-          for (int j = 0; j < 2; ++j) low[j][v] = low[j][v] * sg;
-        }
+      for (int j = 0; j < 2; ++j) low[j][v] = lacc[j][v] * sg;
     }
   }
 #pragma unroll
@@ -478,6 +503,169 @@ __global__ __launch_bounds__(256, 2) void gq_gemm_kernel(GqGemmArgs a) {
   // ---- epilogue: LoRA term per adapter present in the tile, store
   gq_store_row_block(a, outv[0], rb0, col, cb1 != cb0, zs[wave], lane);
   if (rb1 != rb0) gq_store_row_block(a, outv[1], rb1, col, cb1 != cb0, zs[wave], lane);
+}
+
+// ---------------------------------------------------------------------------------------
+// The same product for groups that are multiples of 64 k, staged through the LDS: a workgroup of four
+// waves (2 x 2) owns a 128 x 128 output tile; per 64-wide k step its activation fragments (8 KiB), weight
+// fragments (4 or 8 KiB) and the group's scales (128 column and 128 row scales) arrive once per workgroup by
+// direct-to-LDS loads, three steps ahead, and every wave reads the fragments of its 64 x 64 share from
+// there.  Per output the arithmetic and its order are those of gq_gemm_kernel (the step and the epilogue
+// are shared), so the two kernels agree bit for bit; this one asks the L2 for half the bytes and keeps
+// three steps in flight instead of one.
+constexpr uint32_t kGqLdsStages = 4;
+__host__ __device__ constexpr uint32_t gq_lds_stage_bytes(bool w4) { return 8192u + (w4 ? 4096u : 8192u) + 1024u; }
+__host__ __device__ constexpr uint32_t gq_lds_bytes(bool w4) { return kGqLdsStages * gq_lds_stage_bytes(w4); }
+
+template <bool W4>
+__global__ __launch_bounds__(256, 2) void gq_gemm_lds_kernel(GqGemmArgs a) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char gq_lds[];  // the stage ring; the epilogue's z rows afterwards
+  constexpr uint32_t kStage = gq_lds_stage_bytes(W4), kWOff = 8192u, kSOff = 8192u + (W4 ? 4096u : 8192u);
+  constexpr uint32_t kWBlk = W4 ? 512u : 1024u;      // bytes of a weight fragment (one column block, one k block)
+  constexpr uint32_t kLoads = 2u + (W4 ? 1u : 2u) + 1u;  // direct-to-LDS loads per wave and stage
+  constexpr uint32_t NS = kGqLdsStages;
+  typedef __attribute__((address_space(3))) const unsigned char* lds_cptr;
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t wr = wave >> 1, wc = wave & 1u;
+  const uint32_t c = lane & 31u, h = lane >> 5;
+  const uint32_t kbs = a.K_pad / 32u, blocks_per_group = a.group / 32u;  // both even here
+  const uint32_t n_stages = kbs / 2u;
+  const uint32_t n_rb = a.M_pad / 32u;
+  const uint32_t rbase = blockIdx.y * 4u, cbase = blockIdx.x * 4u;
+  // blocks that hang over the edge are read from the last valid one; their results are never stored
+  auto rb_of = [&](uint32_t l) { return rbase + l < n_rb ? rbase + l : n_rb - 1u; };
+  auto cb_of = [&](uint32_t l) { return cbase + l < a.n_col_blocks ? cbase + l : a.n_col_blocks - 1u; };
+  const uint32_t rbs[2] = {rb_of(2u * wr), rb_of(2u * wr + 1u)};
+  const uint32_t cbs[2] = {cb_of(2u * wc), cb_of(2u * wc + 1u)};
+  const uint32_t col[2] = {cbs[0] * 32u + c, cbs[1] * 32u + c};
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(lptr_t)gq_lds;
+  // what this wave brings in per stage: row block `wave` (2 KiB), column block `wave` (1 or 2 KiB), 64 scales
+  const unsigned char* const a_src = reinterpret_cast<const unsigned char*>(a.codes) + (size_t)rb_of(wave) * kbs * 1024u;
+  const unsigned char* const w_src = a.wp + (size_t)cb_of(wave) * kbs * kWBlk;
+  uint32_t s_idx;  // the wave's scale of a group: a column (waves 0, 1) or a row (waves 2, 3), clamped to the last one
+  if (wave < 2u) {
+    const uint32_t cc = cbase * 32u + wave * 64u + lane;
+    s_idx = cc < a.N ? cc : a.N - 1u;
+  } else {
+    const uint32_t rr = rbase * 32u + (wave - 2u) * 64u + lane;
+    s_idx = rr < a.M_pad ? rr : a.M_pad - 1u;
+  }
+  const uint32_t stages_per_group = blocks_per_group / 2u;
+  const float* const s_src = wave < 2u ? a.ws : a.xs;     // the wave's scales: one row of them per group
+  const uint32_t s_stride = wave < 2u ? a.N : a.M_pad;
+  uint32_t ld_sig = 0, ld_group = 0;                      // stage inside its group and group of the next stage requested
+  auto load_stage = [&](uint32_t st) {
+    const uint32_t slot = lds0 + (st % NS) * kStage;
+    lds_load_1k(a_src + (size_t)st * 2048u, lane * 16u, slot + wave * 2048u);
+    lds_load_1k(a_src + (size_t)st * 2048u, 1024u + lane * 16u, slot + wave * 2048u + 1024u);
+    lds_load_1k(w_src + (size_t)st * 2u * kWBlk, lane * 16u, slot + kWOff + wave * 2u * kWBlk);
+    if (!W4) lds_load_1k(w_src + (size_t)st * 2u * kWBlk, 1024u + lane * 16u, slot + kWOff + wave * 2u * kWBlk + 1024u);
+    lds_gather_dword(s_src + (size_t)ld_group * s_stride, s_idx * 4u, slot + kSOff + wave * 256u);
+    if (++ld_sig == stages_per_group) { ld_sig = 0; ++ld_group; }  // (stages are requested in order)
+  };
+
+  float outv[2][2][16];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) outv[i][j][v] = 0.0f;
+  v16i acc[2][2];
+  // one k block, as in gq_gemm_kernel: four MFMAs (from zero when the block opens a group) and, when it
+  // closes a group, (f32(acc) * sx) * sw added in group order; for 4-bit codes sw carries the exact 1/16
+  // (opens / closes: whether the k block is the first / last of its group, workgroup-uniform and kept by
+  // counting: a remainder per k block costs more instructions than the block's four MFMAs leave room for)
+  auto step = [&](bool opens, bool closes, const v4i& fa0, const v4i& fa1, const GqRawFragment<W4>& r0,
+                  const GqRawFragment<W4>& r1, lds_cptr sc) {
+    const v4i fb0 = gq_expand<W4>(r0), fb1 = gq_expand<W4>(r1);
+    if (opens) {
+      const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+      acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa0, fb0, zero, 0, 0, 0);
+      acc[0][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa0, fb1, zero, 0, 0, 0);
+      acc[1][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa1, fb0, zero, 0, 0, 0);
+      acc[1][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa1, fb1, zero, 0, 0, 0);
+    } else {
+      acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa0, fb0, acc[0][0], 0, 0, 0);
+      acc[0][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa0, fb1, acc[0][1], 0, 0, 0);
+      acc[1][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa1, fb0, acc[1][0], 0, 0, 0);
+      acc[1][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa1, fb1, acc[1][1], 0, 0, 0);
+    }
+    if (closes) {
+      typedef __attribute__((address_space(3))) const float* lds_fptr;
+      typedef float gq_f4 __attribute__((ext_vector_type(4)));
+      typedef __attribute__((address_space(3))) const gq_f4* lds_f4ptr;
+      float swl[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        swl[j] = reinterpret_cast<lds_fptr>(sc)[(2u * wc + (uint32_t)j) * 32u + c];
+        if (W4) swl[j] = swl[j] * 0.0625f;
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const gq_f4 s4 = *reinterpret_cast<lds_f4ptr>(sc + 512u + ((2u * wr + (uint32_t)i) * 32u + 8u * q + 4u * h) * 4u);
+          const float sxq[4] = {s4[0], s4[1], s4[2], s4[3]};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int v = 4 * q + e;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              float t = (float)acc[i][j][v] * sxq[e];
+              t = t * swl[j];
+              outv[i][j][v] = outv[i][j][v] + t;
+            }
+          }
+        }
+    }
+  };
+
+  for (uint32_t st = 0; st + 1u < NS && st < n_stages; ++st) load_stage(st);
+  uint32_t sig = 0;  // stage inside its group
+  for (uint32_t st = 0; st < n_stages; ++st) {
+    // stage st has landed once at most the NS - 2 younger stages are outstanding (none are issued near the end)
+    if (st + NS - 2u < n_stages) wait_vmcnt<(NS - 2) * kLoads>();
+    else wait_vmcnt<0>();
+    lds_barrier();  // everybody's pieces of stage st; and every wave is done with stage st - 1
+    if (st + NS - 1u < n_stages) load_stage(st + NS - 1u);  // into the slot of stage st - 1
+    lds_cptr slot = reinterpret_cast<lds_cptr>((uintptr_t)(lds0 + (st % NS) * kStage));
+    v4i fa[2][2];
+    GqRawFragment<W4> fr[2][2];
+#pragma unroll
+    for (uint32_t kl = 0; kl < 2; ++kl) {
+#pragma unroll
+      for (uint32_t i = 0; i < 2; ++i) {
+        typedef __attribute__((address_space(3))) const v4i* lds_v4ptr;
+        fa[kl][i] = *reinterpret_cast<lds_v4ptr>(slot + (2u * wr + i) * 2048u + kl * 1024u + lane * 16u);
+        lds_cptr wp = slot + kWOff + (2u * wc + i) * 2u * kWBlk + kl * kWBlk + lane * (W4 ? 8u : 16u);
+        if (W4) {
+          typedef uint32_t gq_u2 __attribute__((ext_vector_type(2)));
+          typedef __attribute__((address_space(3))) const gq_u2* lds_u2ptr;
+          const gq_u2 t = *reinterpret_cast<lds_u2ptr>(wp);
+          fr[kl][i].v = make_uint4(t[0], t[1], 0u, 0u);
+        } else {
+          typedef uint32_t gq_u4 __attribute__((ext_vector_type(4)));
+          typedef __attribute__((address_space(3))) const gq_u4* lds_u4ptr;
+          const gq_u4 t = *reinterpret_cast<lds_u4ptr>(wp);
+          fr[kl][i].v = make_uint4(t[0], t[1], t[2], t[3]);
+        }
+      }
+    }
+    const bool last_of_group = sig + 1u == stages_per_group;
+    step(sig == 0u, false, fa[0][0], fa[0][1], fr[0][0], fr[0][1], slot + kSOff);
+    step(false, last_of_group, fa[1][0], fa[1][1], fr[1][0], fr[1][1], slot + kSOff);
+    sig = last_of_group ? 0u : sig + 1u;
+  }
+  // ---- epilogue: LoRA term per adapter present in the tile, store (the ring is free: its last reads are done)
+  lds_barrier();
+  float (*zs)[64] = reinterpret_cast<float (*)[64]>(gq_lds + wave * 32u * 64u * 4u);
+  const bool two_cols = cbase + 2u * wc + 1u < a.n_col_blocks;
+  if (rbase + 2u * wr < n_rb && cbase + 2u * wc < a.n_col_blocks) {
+    gq_store_row_block(a, outv[0], rbs[0], col, two_cols, zs, lane);
+    if (rbase + 2u * wr + 1u < n_rb) gq_store_row_block(a, outv[1], rbs[1], col, two_cols, zs, lane);
+  }
 }
 
 // ---------------------------------------------------------------------------------------

@@ -77,10 +77,11 @@ def prepare_group_weight(weight) -> PackedGroupWeight:
 
 
 def forward(x: torch.Tensor, weight, lora_a=None, lora_b=None, lora_scaling=None, *, activation_bits: int = 8,
-            adapter_indices: torch.Tensor | None = None, return_aux: bool = False):
+            adapter_indices: torch.Tensor | None = None, return_aux: bool = False, flags: int = 0):
     """bf16(base + s[idx] * ((x @ A[idx]) @ B[idx])) with the grouped-scale base of
     quantized_lora.py:215-254.  ``lora_a`` / ``lora_b`` are [K, r] / [r, N] with a scalar scaling, or
-    stacked [n, K, r] / [n, r, N] with ``lora_scaling`` [n] and one adapter index per row."""
+    stacked [n, K, r] / [n, r, N] with ``lora_scaling`` [n] and one adapter index per row.
+    ``flags``: 0, or ``_native.FLAG_GQ_DIRECT`` for the kernel without LDS staging (same bits)."""
     if activation_bits not in (4, 8):
         raise ValueError(f"bits must be 4 or 8, got {activation_bits}")
     if x.dtype != torch.bfloat16:
@@ -132,6 +133,7 @@ def forward(x: torch.Tensor, weight, lora_a=None, lora_b=None, lora_scaling=None
         aux["base"] = torch.empty((m, n), dtype=torch.float32, device=dev)
     p = _native.GqProblem()
     p.struct_size = ctypes.sizeof(_native.GqProblem)
+    p.flags = int(flags)
     p.m, p.k, p.k_pad, p.n = m, k, pw.padded_in_features, n
     p.group_size, p.weight_bits, p.activation_bits = pw.group_size, pw.bits, activation_bits
     p.n_adapters, p.rank = n_ad, r

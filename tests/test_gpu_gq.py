@@ -129,6 +129,35 @@ def test_gq_linear_matches_oracle(dev, pkg, m, k, n, wb, ab, group, rank, n_ad):
     assert rep["violations"] == 0, rep
 
 
+@pytest.mark.parametrize("m,k,n,wb,ab,group,rank,n_ad", [
+    (70, 512, 264, 8, 8, 128, 16, 3),
+    (2050, 200, 2056, 4, 8, 64, 8, 3),     # ragged edges in both directions
+    (333, 1024, 1100, 4, 4, 256, 0, 0),
+])
+def test_gq_lds_staged_and_direct_kernels_agree_bitwise(dev, pkg, m, k, n, wb, ab, group, rank, n_ad):
+    """Groups of whole 64-wide k steps run on the LDS-staged 128 x 128 tiles; the kernel that feeds its wave
+    tiles from the L2 (FLAG_GQ_DIRECT) gives the same float32 base and the same output, bit for bit."""
+    import torch
+
+    rng = np.random.default_rng(m + 3 * k + 5 * n)
+    x = o.bf16_round(rng.standard_t(4, (m, k)).astype(F32))
+    w = o.quantize_frozen_weight((rng.standard_normal((k, n)) * 0.05).astype(F32), bits=wb, group_size=group,
+                                 scale_dtype="f32")
+    args = [_bf(dev, x), _to_dev(pkg, dev, w)]
+    kw = dict(activation_bits=ab, return_aux=True)
+    if n_ad:
+        a = o.bf16_round((rng.standard_normal((n_ad, k, rank)) * 0.05).astype(F32))
+        b = o.bf16_round((rng.standard_normal((n_ad, rank, n)) * 0.05).astype(F32))
+        args += [_bf(dev, a), _bf(dev, b), torch.from_numpy(rng.uniform(0.5, 2.0, n_ad).astype(F32)).to(dev)]
+        kw["adapter_indices"] = torch.from_numpy(rng.integers(0, n_ad, m).astype(np.int32)).to(dev)
+    print(f"[case] gq kernels m={m} k={k} n={n} W{wb}A{ab} group={group}", flush=True)
+    staged, aux_s = pkg.gq_linear.forward(*args, **kw)
+    direct, aux_d = pkg.gq_linear.forward(*args, flags=pkg._native.FLAG_GQ_DIRECT, **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(aux_s["base"].view(torch.int32), aux_d["base"].view(torch.int32))
+    assert torch.equal(staged.view(torch.int16), direct.view(torch.int16))
+
+
 def test_gq_single_adapter_through_the_reference_entry_point(dev, pkg):
     import torch
 
