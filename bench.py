@@ -1213,7 +1213,7 @@ def measure_linear(args, cfg, pkg, dev, steps, warmup, rotate, workload=None, fl
     # the training-style step: the adapters changed since the last call (every optimizer step does that),
     # so the launch that lays out the LoRA operands runs again -- timed over at least 20 steps
     repack = None
-    if cfg.get("n_adapters", 0) and not getattr(args, "repack_lora", False):
+    if cfg.get("n_adapters", 0) and not getattr(args, "repack_lora", False) and not getattr(args, "no_repack", False):
         n_rep = max(steps, 20)
         for pl in plans:
             pl.keep_lora_pack = False
@@ -1328,6 +1328,9 @@ def main() -> int:
     ap.add_argument("--repack-lora", action="store_true",
                     help="transpose / pack the LoRA factors on every step (a training step's forward) instead of "
                          "keeping them in the plan's workspace while the adapters are unchanged")
+    ap.add_argument("--no-repack", action="store_true",
+                    help="skip the block that times the step with the LoRA operands packed again every step "
+                         "(counter runs: the steady call then has the most dispatches of its kernel)")
     ap.add_argument("--no-decode", action="store_true", help="default workload: skip the decode block")
     ap.add_argument("--no-ceilings", action="store_true", help="default workload: skip the measured ceilings")
     args = ap.parse_args()
