@@ -275,14 +275,53 @@ __device__ inline v4i gq_weight_fragment(const unsigned char* p) {
   return *reinterpret_cast<const v4i*>(p);
 }
 
+// The end of one 32-row block of a wave's tile: a row's low-rank sum scaled by its adapter's factor, the add,
+// the cast, the store.  outv[j][v] is the float32 base of column block j, row 8 (v / 4) + 4 (lane / 32) + v % 4;
+// lacc[j][v] the unscaled low-rank sum of the same place.
+__device__ inline void gq_finish_row_block(const GqGemmArgs& a, const float (&outv)[2][16], const v16f (&lacc)[2], bool lora,
+                                           uint32_t rb, const uint32_t (&col)[2], bool two_cols, uint32_t lane) {
+  const uint32_t h = lane >> 5;
+  float sg[16];
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    sg[v] = 0.0f;
+    if (lora) {
+      const uint32_t row = rb * 32u + 8u * (v >> 2) + 4u * h + (v & 3);
+      int ad = (a.idx && row < a.M) ? a.idx[row] : 0;
+      ad = ad < 0 ? 0 : (ad >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad);
+      sg[v] = a.lora_scaling[ad];
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    if (j == 1 && !two_cols) break;
+    if (col[j] >= a.N) continue;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const uint32_t row = rb * 32u + 8u * (v >> 2) + 4u * h + (v & 3);
+      if (row >= a.M) continue;
+      float y = outv[j][v];
+      if (a.aux_base) a.aux_base[(size_t)row * a.N + col[j]] = y;
+      if (lora) {
+        const float low = lacc[j][v] * sg[v];
+        y = y + low;
+      }
+      a.out[(size_t)row * a.N + col[j]] = (uint16_t)f32_to_bf16_bits(y);
+    }
+  }
+}
+
 // Epilogue of one 32-row block of a wave's tile: the LoRA term per adapter present among the block's
 // rows (their z rows staged in the wave's LDS buffer), the add, the cast, the store.  outv[j][v] is the
 // float32 base of column block j, row 8 (v / 4) + 4 (lane / 32) + v % 4.
 __device__ inline void gq_store_row_block(const GqGemmArgs& a, const float (&outv)[2][16], uint32_t rb,
                                           const uint32_t (&col)[2], bool two_cols, float (*zbuf)[64], uint32_t lane) {
-  const uint32_t h = lane >> 5;
   const bool lora = a.z != nullptr;
-  float low[2][16];
+  v16f lacc[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) lacc[j][v] = 0.0f;
   if (lora) {
     __builtin_amdgcn_wave_barrier();  // the buffer's previous use by this wave is over
     for (uint32_t t = lane; t < 32u * 64u; t += 64u) {
@@ -306,11 +345,6 @@ __device__ inline void gq_store_row_block(const GqGemmArgs& a, const float (&out
       const int ad = a.idx ? a.idx[rowg] : 0;
       my_ad = ad < 0 ? 0 : (ad >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad);
     }
-    v16f lacc[2];
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) lacc[j][v] = 0.0f;
     for (uint32_t r0 = 0; r0 < a.r; r0 += 16u) {
       uint32_t term[3][4];
 #pragma unroll
@@ -363,28 +397,144 @@ __device__ inline void gq_store_row_block(const GqGemmArgs& a, const float (&out
         }
       }
     }
+  }
+  gq_finish_row_block(a, outv, lacc, lora, rb, col, two_cols, lane);
+}
+
+// The low-rank sums of a workgroup's 128 x 128 tile with B staged through the LDS (the stage ring is free by
+// then): per 16 ranks and per batch of up to eight adapters present among the tile's rows, the four waves
+// bring the adapters' B values of the tile's 128 columns in with direct-to-LDS loads (a slot of 16 ranks x
+// 256 bytes per adapter, 1 KiB per instruction), and every wave then takes its passes -- one per adapter
+// present in a row block, the rows of the other adapters zeroed -- with its operands from there.  Per output
+// the passes, their order and their operands are those of gq_store_row_block, which asks memory for the
+// same B values once per pass, row block and lane, one dependent round trip after the other.  z comes
+// straight from memory: a lane's eight values of a 16-rank step are 32 consecutive bytes.
+// Needs N % 8 == 0 and B aligned to 16 bytes (the 16-byte pieces), at most 64 adapters (the mask).
+// LDS: [0, 32 KiB) the batch, [32 KiB, + 32) the waves' adapter masks.  All four waves must call it.
+constexpr uint32_t kGqLoraLdsBytes = 32768u + 64u;
+__device__ inline bool gq_tile_lora_ok(const GqGemmArgs& a) {
+  return a.n_adapters <= 64u && (a.N & 7u) == 0 && (reinterpret_cast<uintptr_t>(a.lora_b) & 15u) == 0;
+}
+__device__ inline void gq_tile_lora_sums(const GqGemmArgs& a, unsigned char* lds, const uint32_t (&rbs)[2],
+                                         const bool (&rb_ok)[2], uint32_t cbase, uint32_t wave, uint32_t wc, uint32_t lane,
+                                         v16f (&lacc)[2][2]) {
+  typedef __attribute__((address_space(3))) const uint16_t* lds_u16ptr;
+  const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)lds;
+  const uint32_t rowl = lane & 31u, kg = lane >> 5, c = lane & 31u;
+  int my_ad[2];
+  uint32_t zrow[2];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const uint32_t row = rb * 32u + 8u * (v >> 2) + 4u * h + (v & 3);
-      int ad = (a.idx && row < a.M) ? a.idx[row] : 0;
-      ad = ad < 0 ? 0 : (ad >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad);
-      const float sg = a.lora_scaling[ad];
-#pragma unroll
-      for (int j = 0; j < 2; ++j) low[j][v] = lacc[j][v] * sg;
+  for (int i = 0; i < 2; ++i) {
+    const uint32_t rowg = rbs[i] * 32u + rowl;
+    my_ad[i] = -1;  // rows beyond M (and row blocks beyond the edge) belong to no adapter
+    zrow[i] = 0;
+    if (rb_ok[i] && rowg < a.M) {
+      const int ad = a.idx ? a.idx[rowg] : 0;
+      my_ad[i] = ad < 0 ? 0 : (ad >= (int)a.n_adapters ? (int)a.n_adapters - 1 : ad);
+      zrow[i] = a.z_slot ? (uint32_t)a.z_slot[rowg] : rowg;
     }
   }
+  unsigned long long pm[2] = {0ull, 0ull};  // adapters present in the wave's row blocks (wave-uniform)
+  for (uint32_t ad = 0; ad < a.n_adapters; ++ad)
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    if (j == 1 && !two_cols) break;
-    if (col[j] >= a.N) continue;
+    for (int i = 0; i < 2; ++i)
+      if (__builtin_amdgcn_ballot_w64(my_ad[i] == (int)ad) != 0) pm[i] |= 1ull << ad;
+  unsigned long long* const masks = reinterpret_cast<unsigned long long*>(lds + 32768u);
+  if (lane == 0) masks[wave] = pm[0] | pm[1];
+  __syncthreads();
+  const unsigned long long wg_mask = masks[0] | masks[1] | masks[2] | masks[3];
+  // what this lane brings in per slot: rank 4 wave + lane / 16 of the step, columns 8 (lane % 16) .. + 7 of the tile
+  const uint32_t ld_rank = 4u * wave + (lane >> 4), ld_col = cbase * 32u + (lane & 15u) * 8u;
+  for (uint32_t r0 = 0; r0 < a.r; r0 += 16u) {
+    uint32_t term[2][3][4];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const uint32_t row = rb * 32u + 8u * (v >> 2) + 4u * h + (v & 3);
-      if (row >= a.M) continue;
-      float y = outv[j][v];
-      if (a.aux_base) a.aux_base[(size_t)row * a.N + col[j]] = y;
-      if (lora) y = y + low[j][v];
-      a.out[(size_t)row * a.N + col[j]] = (uint16_t)f32_to_bf16_bits(y);
+    for (int i = 0; i < 2; ++i) {
+      float z8[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) z8[e] = 0.0f;
+      if (my_ad[i] >= 0) {
+        const float4 lo4 = *reinterpret_cast<const float4*>(a.z + (size_t)zrow[i] * 64u + r0 + 8u * kg);
+        const float4 hi4 = *reinterpret_cast<const float4*>(a.z + (size_t)zrow[i] * 64u + r0 + 8u * kg + 4u);
+        const float t8[8] = {lo4.x, lo4.y, lo4.z, lo4.w, hi4.x, hi4.y, hi4.z, hi4.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) z8[e] = r0 + 8u * kg + (uint32_t)e < a.r ? t8[e] : 0.0f;
+      }
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        float hi[2], mid[2], lo[2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          const float z = z8[2 * d + e];
+          hi[e] = bf16_round_f32(z);
+          const float r1 = z - hi[e];
+          mid[e] = bf16_round_f32(r1);
+          lo[e] = bf16_round_f32(r1 - mid[e]);
+        }
+        term[i][0][d] = pack_bf16x2(hi[0], hi[1]);
+        term[i][1][d] = pack_bf16x2(mid[0], mid[1]);
+        term[i][2][d] = pack_bf16x2(lo[0], lo[1]);
+      }
+    }
+    const bool ld_on = r0 + ld_rank < a.r && ld_col < a.N;
+    const uint32_t ld_off = ((r0 + ld_rank) * a.N + ld_col) * 2u;
+    unsigned long long rem = wg_mask;
+    while (rem) {  // batches of up to eight adapters, smallest first (workgroup-uniform)
+      uint32_t ads[8], nb = 0;
+#pragma unroll
+      for (int sl = 0; sl < 8; ++sl) {
+        ads[sl] = 0;
+        if (rem) {
+          ads[sl] = (uint32_t)__builtin_ctzll(rem);
+          rem &= rem - 1ull;
+          nb = (uint32_t)sl + 1u;
+        }
+      }
+      __syncthreads();  // the batch before has been read
+#pragma unroll
+      for (uint32_t sl = 0; sl < 8; ++sl) {
+        if (sl < nb && ld_on)
+          lds_load_1k(reinterpret_cast<const unsigned char*>(a.lora_b) + (size_t)ads[sl] * a.r * a.N * 2u, ld_off,
+                      lds_addr + sl * 4096u + wave * 1024u);
+      }
+      wait_vmcnt<0>();
+      __syncthreads();
+#pragma unroll
+      for (uint32_t sl = 0; sl < 8; ++sl) {
+        if (sl >= nb) break;
+        const uint32_t ad = ads[sl];
+        if (!(((pm[0] | pm[1]) >> ad) & 1ull)) continue;  // wave-uniform
+        v4i bo[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const uint32_t lcol = (2u * wc + (uint32_t)j) * 32u + c;
+          const bool col_ok = cbase * 32u + lcol < a.N;
+          uint32_t braw[8];
+#pragma unroll
+          for (uint32_t e = 0; e < 8; ++e) {
+            const uint32_t rank = 8u * kg + e;
+            const uint16_t v = reinterpret_cast<lds_u16ptr>((lptr_t)lds)[(sl * 16u + rank) * 128u + lcol];
+            braw[e] = (col_ok && r0 + rank < a.r) ? (uint32_t)v : 0u;
+          }
+#pragma unroll
+          for (int d = 0; d < 4; ++d) bo[j][d] = (int)(braw[2 * d] | (braw[2 * d + 1] << 16));
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          if (!((pm[i] >> ad) & 1ull)) continue;  // wave-uniform
+          const bool mine = my_ad[i] == (int)ad;
+          v4i za[3];
+#pragma unroll
+          for (int t = 0; t < 3; ++t)
+#pragma unroll
+            for (int d = 0; d < 4; ++d) za[t][d] = mine ? (int)term[i][t][d] : 0;
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int t = 2; t >= 0; --t)
+              lacc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, za[t]),
+                                                                    __builtin_bit_cast(v8bf, bo[j]), lacc[i][j], 0, 0, 0);
+        }
+      }
     }
   }
 }
@@ -516,6 +666,7 @@ __global__ __launch_bounds__(256, 2) void gq_gemm_kernel(GqGemmArgs a) {
 constexpr uint32_t kGqLdsStages = 4;
 __host__ __device__ constexpr uint32_t gq_lds_stage_bytes(bool w4) { return 8192u + (w4 ? 4096u : 8192u) + 1024u; }
 __host__ __device__ constexpr uint32_t gq_lds_bytes(bool w4) { return kGqLdsStages * gq_lds_stage_bytes(w4); }
+static_assert(gq_lds_bytes(true) >= kGqLoraLdsBytes && gq_lds_bytes(true) >= 4u * 32u * 64u * 4u, "the epilogue reuses the ring");
 
 template <bool W4>
 __global__ __launch_bounds__(256, 2) void gq_gemm_lds_kernel(GqGemmArgs a) {
@@ -660,11 +811,27 @@ __global__ __launch_bounds__(256, 2) void gq_gemm_lds_kernel(GqGemmArgs a) {
   }
   // ---- epilogue: LoRA term per adapter present in the tile, store (the ring is free: its last reads are done)
   lds_barrier();
-  float (*zs)[64] = reinterpret_cast<float (*)[64]>(gq_lds + wave * 32u * 64u * 4u);
   const bool two_cols = cbase + 2u * wc + 1u < a.n_col_blocks;
-  if (rbase + 2u * wr < n_rb && cbase + 2u * wc < a.n_col_blocks) {
+  const bool rb_ok[2] = {rbase + 2u * wr < n_rb, rbase + 2u * wr + 1u < n_rb};
+  const bool cols_ok = cbase + 2u * wc < a.n_col_blocks;
+  if (a.z && gq_tile_lora_ok(a)) {  // workgroup-uniform
+    v16f lacc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) lacc[i][j][v] = 0.0f;
+    gq_tile_lora_sums(a, gq_lds, rbs, rb_ok, cbase, wave, wc, lane, lacc);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      if (rb_ok[i] && cols_ok) gq_finish_row_block(a, outv[i], lacc[i], true, rbs[i], col, two_cols, lane);
+    return;
+  }
+  float (*zs)[64] = reinterpret_cast<float (*)[64]>(gq_lds + wave * 32u * 64u * 4u);
+  if (rb_ok[0] && cols_ok) {
     gq_store_row_block(a, outv[0], rbs[0], col, two_cols, zs, lane);
-    if (rbase + 2u * wr + 1u < n_rb) gq_store_row_block(a, outv[1], rbs[1], col, two_cols, zs, lane);
+    if (rb_ok[1]) gq_store_row_block(a, outv[1], rbs[1], col, two_cols, zs, lane);
   }
 }
 

@@ -85,6 +85,8 @@ CASES = [
     (2050, 200, 2056, 4, 8, 64, 8, 3),    # many tiles, ragged edges, an odd number of k blocks
     (2048, 384, 2048, 8, 4, 96, 0, 0),    # 8-bit codes, three k blocks a group
     (1024, 2048, 512, 4, 8, 1024, 40, 5),  # long groups
+    (260, 256, 136, 4, 8, 64, 24, 20),    # twenty adapters: three batches of the LDS-staged LoRA epilogue
+    (130, 128, 132, 8, 8, 64, 8, 3),      # N not a multiple of 8: the epilogue that reads B from memory
 ]
 
 
@@ -133,6 +135,8 @@ def test_gq_linear_matches_oracle(dev, pkg, m, k, n, wb, ab, group, rank, n_ad):
     (70, 512, 264, 8, 8, 128, 16, 3),
     (2050, 200, 2056, 4, 8, 64, 8, 3),     # ragged edges in both directions
     (333, 1024, 1100, 4, 4, 256, 0, 0),
+    (260, 256, 136, 4, 8, 64, 24, 20),     # more adapters than one batch of the staged LoRA epilogue holds
+    (130, 128, 132, 8, 8, 64, 8, 3),       # N not a multiple of 8
 ])
 def test_gq_lds_staged_and_direct_kernels_agree_bitwise(dev, pkg, m, k, n, wb, ab, group, rank, n_ad):
     """Groups of whole 64-wide k steps run on the LDS-staged 128 x 128 tiles; the kernel that feeds its wave
