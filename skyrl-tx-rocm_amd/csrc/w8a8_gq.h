@@ -100,6 +100,7 @@ __device__ inline void gq_load_piece(const GqQuantArgs& a, const uint16_t* xr, b
 __global__ __launch_bounds__(256) void gq_quant_kernel(GqQuantArgs a) {
   __shared__ float piece_max[4][kGqMaxPieces];
   __shared__ float group_scale[4][kGqMaxGroups];
+  __shared__ float group_rscale[4][kGqMaxGroups];  // 1 / scale, or -1: divide
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
   const uint32_t row = blockIdx.x * 4u + wave;
   if (row >= a.M_pad) return;
@@ -111,6 +112,98 @@ __global__ __launch_bounds__(256) void gq_quant_kernel(GqQuantArgs a) {
   const uint32_t g_hi = g_lo + a.groups_per_slice < a.G ? g_lo + a.groups_per_slice : a.G;
   if (g_lo >= g_hi) return;
   const uint32_t p_lo = g_lo * pieces_per_group, n_pieces = (g_hi - g_lo) * pieces_per_group;
+  auto scales_from_piece_maxima = [&]() {
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_wave_barrier();
+    for (uint32_t gl = lane; gl < g_hi - g_lo; gl += 64u) {
+      const uint32_t g = g_lo + gl;
+      float amax = 0.0f;
+      for (uint32_t p = 0; p < pieces_per_group; ++p) amax = fmaxf(amax, piece_max[wave][gl * pieces_per_group + p]);
+      const float scale = amax > 0.0f ? amax / a.qmax : 1.0f;
+      group_scale[wave][gl] = scale;
+      group_rscale[wave][gl] = (amax == amax && scale > 1e-30f && scale < 1e30f) ? __builtin_amdgcn_rcpf(scale) : -1.0f;
+      a.scales[(size_t)g * a.M_pad + row] = scale;
+      if (a.scales_rm && live) a.scales_rm[(size_t)row * a.G + g] = scale;
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_wave_barrier();
+  };
+  // codes = clip(rint(v / scale)) with the correctly rounded quotient.  v * (1 / scale) with the hardware
+  // reciprocal is within 3 * 2^-24 * 128 < 2.3e-5 of it (|quotient| <= qmax <= 127), and forming it biased by
+  // 128 in one fused step adds at most 2^-17: both round to the same integer unless the product lies within
+  // 4e-5 of a tie.  Those pieces, and groups whose scale is not an ordinary number (rscale < 0), are redone
+  // with the division.  |v| <= the group's maximum, so the clip only ever acts in the redone cases.  The
+  // biased value lands in its byte with one v_cvt_pk_u8_f32; flipping bit 7 makes it two's complement.
+  auto quantize_piece = [&](uint32_t p, const float (&v)[8]) {
+    const uint32_t k = (p_lo + p) * 8u;
+    const float scale = group_scale[wave][p / pieces_per_group];
+    const float rscale = group_rscale[wave][p / pieces_per_group];
+    float c[8];
+    float off_integer = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float t = __builtin_fmaf(v[j], rscale, 128.0f);
+      c[j] = rintf(t);
+      off_integer = fmaxf(off_integer, fabsf(t - c[j]));
+    }
+    const bool redo = rscale < 0.0f || off_integer > 0.49996f;
+    if (__builtin_amdgcn_ballot_w64(redo) != 0) {  // wave-uniform
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        float q = __builtin_rintf(v[j] / scale);
+        q = fminf(fmaxf(q, -a.qmax), a.qmax);
+        c[j] = q + 128.0f;
+      }
+    }
+    uint32_t w[2] = {0, 0};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      w[0] = __builtin_amdgcn_cvt_pk_u8_f32(c[j], (uint32_t)j, w[0]);
+      w[1] = __builtin_amdgcn_cvt_pk_u8_f32(c[j + 4], (uint32_t)j, w[1]);
+    }
+    w[0] ^= 0x80808080u;
+    w[1] ^= 0x80808080u;
+    *reinterpret_cast<uint2*>(cblk + (size_t)(k >> 5) * 1024u + ((k >> 4) & 1u) * 512u + (k & 15u)) = make_uint2(w[0], w[1]);
+    if (a.codes_rm && live) *reinterpret_cast<uint2*>(a.codes_rm + (size_t)row * a.K_pad + k) = make_uint2(w[0], w[1]);
+  };
+  if ((a.K & 7u) == 0) {
+    // rows of 16-byte pieces: the wave's share of the row (at most 2048 pieces, 32 per lane) stays in registers
+    // between the pass that finds the maxima and the pass that quantizes, so the row is read once
+    constexpr uint32_t kIt = kGqMaxPieces / 64u;
+    uint4 raw[kIt];
+#pragma unroll
+    for (uint32_t it = 0; it < kIt; ++it) {
+      const uint32_t p = it * 64u + lane, k = (p_lo + p) * 8u;
+      raw[it] = make_uint4(0u, 0u, 0u, 0u);
+      if (it * 64u < n_pieces && p < n_pieces && live && k < a.K) raw[it] = *reinterpret_cast<const uint4*>(xr + k);
+    }
+#pragma unroll
+    for (uint32_t it = 0; it < kIt; ++it) {
+      const uint32_t p = it * 64u + lane;
+      if (it * 64u >= n_pieces) break;  // wave-uniform
+      // |bf16| compares like its 15 magnitude bits as an integer (a NaN ends above every number)
+      typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+      us2 mx = __builtin_bit_cast(us2, raw[it].x & 0x7fff7fffu);
+      mx = __builtin_elementwise_max(mx, __builtin_bit_cast(us2, raw[it].y & 0x7fff7fffu));
+      mx = __builtin_elementwise_max(mx, __builtin_bit_cast(us2, raw[it].z & 0x7fff7fffu));
+      mx = __builtin_elementwise_max(mx, __builtin_bit_cast(us2, raw[it].w & 0x7fff7fffu));
+      const uint32_t top = mx[0] > mx[1] ? mx[0] : mx[1];
+      if (p < n_pieces) piece_max[wave][p] = __uint_as_float(top << 16);
+    }
+    scales_from_piece_maxima();
+#pragma unroll
+    for (uint32_t it = 0; it < kIt; ++it) {
+      const uint32_t p = it * 64u + lane;
+      if (it * 64u >= n_pieces) break;  // wave-uniform
+      if (p >= n_pieces) continue;
+      const uint32_t w[4] = {raw[it].x, raw[it].y, raw[it].z, raw[it].w};
+      float v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = (j & 1) ? __uint_as_float(w[j >> 1] & 0xffff0000u) : __uint_as_float(w[j >> 1] << 16);
+      quantize_piece(p, v);
+    }
+    return;
+  }
   for (uint32_t p = lane; p < n_pieces; p += 64u) {
     float v[8];
     gq_load_piece(a, xr, live, (p_lo + p) * 8u, v);
@@ -119,33 +212,11 @@ __global__ __launch_bounds__(256) void gq_quant_kernel(GqQuantArgs a) {
     for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(v[j]));
     piece_max[wave][p] = m;
   }
-  __builtin_amdgcn_s_waitcnt(0xc07f);
-  __builtin_amdgcn_wave_barrier();
-  for (uint32_t gl = lane; gl < g_hi - g_lo; gl += 64u) {
-    const uint32_t g = g_lo + gl;
-    float amax = 0.0f;
-    for (uint32_t p = 0; p < pieces_per_group; ++p) amax = fmaxf(amax, piece_max[wave][gl * pieces_per_group + p]);
-    const float scale = amax > 0.0f ? amax / a.qmax : 1.0f;
-    group_scale[wave][gl] = scale;
-    a.scales[(size_t)g * a.M_pad + row] = scale;
-    if (a.scales_rm && live) a.scales_rm[(size_t)row * a.G + g] = scale;
-  }
-  __builtin_amdgcn_s_waitcnt(0xc07f);
-  __builtin_amdgcn_wave_barrier();
+  scales_from_piece_maxima();
   for (uint32_t p = lane; p < n_pieces; p += 64u) {
-    const uint32_t k = (p_lo + p) * 8u;
     float v[8];
-    gq_load_piece(a, xr, live, k, v);
-    const float scale = group_scale[wave][p / pieces_per_group];
-    uint32_t w[2] = {0, 0};
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      float q = __builtin_rintf(v[j] / scale);
-      q = fminf(fmaxf(q, -a.qmax), a.qmax);
-      w[j >> 2] |= ((uint32_t)(int)q & 0xffu) << (8 * (j & 3));
-    }
-    *reinterpret_cast<uint2*>(cblk + (size_t)(k >> 5) * 1024u + ((k >> 4) & 1u) * 512u + (k & 15u)) = make_uint2(w[0], w[1]);
-    if (a.codes_rm && live) *reinterpret_cast<uint2*>(a.codes_rm + (size_t)row * a.K_pad + k) = make_uint2(w[0], w[1]);
+    gq_load_piece(a, xr, live, (p_lo + p) * 8u, v);
+    quantize_piece(p, v);
   }
 }
 
