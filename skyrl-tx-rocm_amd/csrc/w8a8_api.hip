@@ -650,7 +650,7 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
   const bool skip_gemm = (p->flags & MI355_W8A8_FLAG_SKIP_GEMM) != 0;
   if (skip_prologue && (p->aux_x_codes || p->aux_x_scales)) return MI355_W8A8_ERR_UNSUPPORTED;
 
-  // launch 1: the slot layout of the groups (one block) next to the LoRA operand re-layouts
+  // launch 1: the slot layout of the groups next to the LoRA operand re-layouts
   if (!skip_prologue) {
     LoraPrepArgs pa{};
     pa.src_row = src_row; pa.dst_pos = dst_pos; pa.blk_range = blk_range;
@@ -661,7 +661,8 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
     pa.bp = ws + w.bp;
     pa.M = p->m; pa.K = p->k; pa.N = p->n; pa.n_groups = p->n_groups; pa.r = p->rank; pa.nkk = w.nkk;
     pa.ncb = n_padded(p->n) / 32u; pa.slots = w.slots;
-    pa.route_blocks = 1;
+    // (the layout is filled slot by slot: a few workgroups, each with the prefix sums of its own)
+    pa.route_blocks = (w.slots + 2047u) / 2048u < 16u ? (w.slots + 2047u) / 2048u : 16u;
     uint32_t b_blocks = 0;
     // (a caller that vouches for the operand packs of an earlier call on this workspace keeps them: the
     // launch then only lays out the slots)
@@ -671,7 +672,7 @@ int run_grouped(const mi355_w8a8_grouped_problem* p, hipStream_t s) {
       pa.a_blocks = (uint32_t)((a_items + 1023u) / 1024u);
       b_blocks = (uint32_t)((b_items + 1023u) / 1024u);
     }
-    hipLaunchKernelGGL(lora_prep_kernel, dim3(1u + pa.a_blocks + b_blocks), dim3(1024), 0, s, pa);
+    hipLaunchKernelGGL(lora_prep_kernel, dim3(pa.route_blocks + pa.a_blocks + b_blocks), dim3(1024), 0, s, pa);
     if ((st = launch_status())) return st;
   }
 

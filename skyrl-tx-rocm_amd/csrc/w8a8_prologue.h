@@ -165,47 +165,85 @@ __device__ inline void route_rows_block(const int32_t* __restrict__ idx, uint32_
 //   blk_range[b] = g | g << 16 for the 32-row blocks in use, -1 beyond
 // ---------------------------------------------------------------------------------------
 constexpr int kMaxGroups = 1024;
-// One workgroup of 1024 threads.  Rows beyond sum(group_sizes) get no slot; their output rows
-// (zero_out, bf16 [M, zero_cols], optional) are cleared here.
+// Exclusive prefix sums of one value per thread over a workgroup of 1024 threads, every partial sum capped
+// at `limit` (a capped sum of non-negative terms does not depend on the order they are added in).  Returns
+// the thread's prefix; *total receives the sum of all.
+__device__ inline uint32_t block_prefix_capped(uint32_t v, uint32_t limit, uint32_t* total) {
+  __shared__ uint32_t wave_sum[17];
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  auto add = [&](uint32_t x, uint32_t y) { const uint64_t t = (uint64_t)x + y; return t > limit ? limit : (uint32_t)t; };
+  uint32_t incl = v > limit ? limit : v;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const uint32_t up = (uint32_t)__shfl_up((int)incl, off, 64);
+    if ((int)lane >= off) incl = add(incl, up);
+  }
+  __syncthreads();  // (the table may still be read from a call before)
+  if (lane == 63u) wave_sum[wave] = incl;
+  __syncthreads();
+  if (tid == 0) {
+    uint32_t run = 0;
+    for (int w = 0; w < 16; ++w) {
+      const uint32_t t = wave_sum[w];
+      wave_sum[w] = run;
+      run = add(run, t);
+    }
+    wave_sum[16] = run;
+  }
+  __syncthreads();
+  *total = wave_sum[16];
+  // exclusive: the waves before, then the lanes before (the capped sum up to the lane before)
+  const uint32_t before = (uint32_t)__shfl_up((int)incl, 1, 64);
+  return add(wave_sum[wave], lane ? before : 0u);
+}
+
+// Part `part` of `n_parts` workgroups of 1024 threads: every part forms the prefix sums for itself (at most
+// 1024 groups, one per thread) and fills its share of the tables, slot by slot.  Group g keeps
+// min(size, rows left) rows, as a sequential pass over the sizes would give it.  Rows beyond
+// sum(group_sizes) get no slot; their output rows (zero_out, bf16 [M, zero_cols], optional) are cleared here.
 __device__ inline void route_groups_block(const int32_t* __restrict__ group_sizes, uint32_t M, uint32_t n_groups,
                                           uint32_t slots, int32_t* __restrict__ src_row,
                                           int32_t* __restrict__ dst_pos, int32_t* __restrict__ blk_range,
-                                          uint32_t pad, uint16_t* __restrict__ zero_out, uint32_t zero_cols) {
-  __shared__ int row_start[kMaxGroups + 1];
-  __shared__ int slot_start[kMaxGroups + 1];
+                                          uint32_t pad, uint16_t* __restrict__ zero_out, uint32_t zero_cols,
+                                          uint32_t part, uint32_t n_parts) {
+  __shared__ uint32_t row_start[kMaxGroups + 1];
+  __shared__ uint32_t slot_start[kMaxGroups + 1];
   const uint32_t tid = threadIdx.x;
-  if (tid < n_groups) row_start[tid] = group_sizes[tid];  // sizes first, starts below
+  int32_t sz = tid < n_groups ? group_sizes[tid] : 0;
+  if (sz < 0) sz = 0;
+  uint32_t rows_total, slots_total;
+  const uint32_t r0 = block_prefix_capped((uint32_t)sz, M, &rows_total);
+  // the group's rows after the cap: up to the next group's start
+  const uint32_t r1 = (uint64_t)r0 + (uint32_t)sz > M ? M : r0 + (uint32_t)sz;
+  const uint32_t padded = (r1 - r0 + pad - 1u) & ~(pad - 1u);
+  const uint32_t p0 = block_prefix_capped(padded, 0xffffffffu, &slots_total);
+  if (tid < n_groups) { row_start[tid] = r0; slot_start[tid] = p0; }
+  if (tid == 0) { row_start[n_groups] = rows_total; slot_start[n_groups] = slots_total; }
   __syncthreads();
-  if (tid == 0) {
-    int r = 0, p = 0;
-    for (uint32_t g = 0; g < n_groups; ++g) {
-      int sz = row_start[g];
-      if (sz < 0) sz = 0;
-      if (r + sz > (int)M) sz = (int)M - r;
-      row_start[g] = r;
-      slot_start[g] = p;
-      r += sz;
-      p += (sz + (int)pad - 1) & ~((int)pad - 1);
+  const uint32_t stride = n_parts * 1024u;
+  for (uint32_t p = part * 1024u + tid; p < slots; p += stride) {
+    int src = -1, range = -1;
+    if (p < slots_total) {
+      // the last group whose first slot is not behind p (empty groups share their successor's first slot)
+      uint32_t lo = 0, hi = n_groups;  // slot_start[lo] <= p < slot_start[hi]
+      while (hi - lo > 1u) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (slot_start[mid] <= p) lo = mid; else hi = mid;
+      }
+      const uint32_t i = p - slot_start[lo];
+      if (i < row_start[lo + 1u] - row_start[lo]) {
+        src = (int)(row_start[lo] + i);
+        dst_pos[src] = (int)p;
+      }
+      range = (int)(lo | (lo << 16));
     }
-    row_start[n_groups] = r;
-    slot_start[n_groups] = p;
+    src_row[p] = src;
+    if ((p & 31u) == 0) blk_range[p >> 5] = range;
   }
-  for (uint32_t p = tid; p < slots; p += 1024) src_row[p] = -1;
-  for (uint32_t i = tid; i < M; i += 1024) dst_pos[i] = -1;
-  for (uint32_t b = tid; b < slots / 32u; b += 1024) blk_range[b] = -1;
-  __syncthreads();
-  const uint32_t wave = tid >> 6, lane = tid & 63;
-  for (uint32_t g = wave; g < n_groups; g += 16) {
-    const int r0 = row_start[g], r1 = row_start[g + 1], p0 = slot_start[g], p1 = slot_start[g + 1];
-    for (int i = (int)lane; i < r1 - r0; i += 64) {
-      src_row[p0 + i] = r0 + i;
-      dst_pos[r0 + i] = p0 + i;
-    }
-    for (int b = p0 / 32 + (int)lane; b < p1 / 32; b += 64) blk_range[b] = (int)(g | (g << 16));
-  }
+  for (uint32_t i = rows_total + part * 1024u + tid; i < M; i += stride) dst_pos[i] = -1;
   if (zero_out) {
-    const size_t begin = (size_t)row_start[n_groups] * zero_cols, end = (size_t)M * zero_cols;
-    for (size_t i = begin + tid; i < end; i += 1024) zero_out[i] = 0;
+    const size_t begin = (size_t)rows_total * zero_cols, end = (size_t)M * zero_cols;
+    for (size_t i = begin + part * 1024u + tid; i < end; i += stride) zero_out[i] = 0;
   }
 }
 
@@ -502,7 +540,7 @@ __global__ __launch_bounds__(1024) void lora_prep_kernel(LoraPrepArgs p) {
   if (b < p.route_blocks) {
     if (p.group_sizes)
       route_groups_block(p.group_sizes, p.M, p.n_groups, p.slots, p.src_row, p.dst_pos, p.blk_range, p.group_pad,
-                         p.zero_out, p.zero_cols);
+                         p.zero_out, p.zero_cols, b, p.route_blocks);
     else
       route_rows_block(p.idx, p.M, p.n_groups, p.slots, p.src_row, p.dst_pos, p.slot_group, p.blk_range, nullptr, false,
                        p.route_pad > 1u ? p.route_pad : 1u);

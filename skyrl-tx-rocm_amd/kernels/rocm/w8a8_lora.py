@@ -755,9 +755,10 @@ def rms_gate_up_lora_swiglu(x: torch.Tensor, gamma: torch.Tensor, weight, lora_a
 # ---------------------------------------------------------------------------------------
 # grouped (ragged, per-expert) variant
 # ---------------------------------------------------------------------------------------
-@dataclass(frozen=True)
+@dataclass(frozen=True, eq=False)
 class PackedGroupedW8Weight:
-    """E stacked [K, N] int8 weights in MFMA fragment order plus float32 scales [E, N]."""
+    """E stacked [K, N] int8 weights in MFMA fragment order plus float32 scales [E, N].  Compared and hashed
+    by identity (it keys the expert layer's plan cache)."""
 
     packed: torch.Tensor
     scales: torch.Tensor
@@ -891,6 +892,13 @@ class GroupedForwardPlan:
         self._lora = (a3, b3) if r else None
         self._packed_lora_key = None  # versions of A and B the workspace holds in operand order
         self.keep_lora_pack = True    # False: pack on every run
+
+    def bind_x(self, x: torch.Tensor) -> None:
+        """Read the rows from another tensor of the same shape from the next run on (the plan keeps it alive)."""
+        if x.dtype != torch.bfloat16 or tuple(x.shape) != tuple(self.x_flat.shape) or x.device != self.device:
+            raise ValueError(f"bind_x needs a BF16 tensor of shape {tuple(self.x_flat.shape)} on {self.device}")
+        self.x_flat = x.contiguous()
+        self.problem.x = self.x_flat.data_ptr()
 
     def run(self, extra_flags: int = 0) -> torch.Tensor:
         """Enqueue the call on torch's current stream; returns the (reused) output tensor.  ``extra_flags``
@@ -1188,10 +1196,12 @@ class _MoeRouteFunction(torch.autograd.Function):
 
 
 def moe_dispatch(tokens: torch.Tensor | None, indices: torch.Tensor, num_groups: int, *, repeat: int = 1,
-                 adapter_indices: torch.Tensor | None = None):
+                 adapter_indices: torch.Tensor | None = None, out=None):
     """Stable sort of rows by group with the gather of their token rows, on the device and without a
     host round trip.  Pair ``p`` reads token ``p // repeat`` (and its adapter index).  Returns
-    ``(sorted_tokens, group_sizes, sort_indices, unsort_indices, sorted_adapters)``."""
+    ``(sorted_tokens, group_sizes, sort_indices, unsort_indices, sorted_adapters)``.  ``out`` names
+    ``(group_sizes, sort_indices, unsort_indices, workspace)`` of an earlier call with the same sizes to write
+    into instead of new tensors."""
     _require_cuda(indices, "indices")
     dev = indices.device
     idx = indices.reshape(-1).to(torch.int32).contiguous()
@@ -1224,10 +1234,17 @@ def moe_dispatch(tokens: torch.Tensor | None, indices: torch.Tensor, num_groups:
         if ad.numel() * repeat != n_pairs:
             raise ValueError(f"adapter_indices must have {n_pairs // repeat} entries, got {ad.numel()}")
         sorted_adapters = torch.empty(n_pairs, dtype=torch.int32, device=dev)
-    group_sizes = torch.empty(num_groups, dtype=torch.int32, device=dev)
-    sort_indices = torch.empty(n_pairs, dtype=torch.int32, device=dev)
-    unsort_indices = torch.empty(n_pairs, dtype=torch.int32, device=dev)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    if out is not None:
+        group_sizes, sort_indices, unsort_indices, ws = out
+        if (group_sizes.numel() != num_groups or sort_indices.numel() != n_pairs or unsort_indices.numel() != n_pairs
+                or ws.numel() < ws_bytes or any(t.device != dev for t in out)
+                or any(t.dtype != torch.int32 for t in out[:3])):
+            raise ValueError("out does not fit this dispatch")
+    else:
+        group_sizes = torch.empty(num_groups, dtype=torch.int32, device=dev)
+        sort_indices = torch.empty(n_pairs, dtype=torch.int32, device=dev)
+        unsort_indices = torch.empty(n_pairs, dtype=torch.int32, device=dev)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     p = _native.MoeDispatchProblem()
     p.struct_size = ctypes.sizeof(_native.MoeDispatchProblem)
     p.n_pairs, p.repeat, p.width, p.n_groups = n_pairs, repeat, width, num_groups
@@ -1366,6 +1383,61 @@ class _MoeExpertMlpFunction(torch.autograd.Function):
         return d_hidden, d_w, d_ga, d_gb, d_da, d_db, d_s, None, None, None, None
 
 
+class _MoeInferencePlan:
+    """The two grouped plans of an expert layer's forward without gradients, their workspaces and the
+    dispatch's buffers, kept between calls with the same token count, weights and adapter tensors: the
+    adapters' operand packs then survive in the workspaces (``FLAG_LORA_PACK_VALID`` while the tensors'
+    ``_version`` stands), and no call allocates the intermediates anew."""
+
+    def __init__(self, h2, top_k, gate_up_weight, down_weight, gate_up_a, gate_up_b, down_a, down_b, lora_scaling):
+        dev = h2.device
+        n_experts = gate_up_weight.n_weights
+        n_pairs = h2.shape[0] * top_k
+        lib = _native.load()
+        ws_bytes = int(lib.mi355_w8a8_moe_dispatch_workspace_bytes(n_pairs, n_experts))
+        if ws_bytes == 0:
+            raise ValueError(f"{n_pairs} rows in {n_experts} groups are outside the native dispatch")
+        self.dispatch_out = (torch.zeros(n_experts, dtype=torch.int32, device=dev),
+                             torch.zeros(n_pairs, dtype=torch.int32, device=dev),
+                             torch.zeros(n_pairs, dtype=torch.int32, device=dev),
+                             torch.empty(ws_bytes, dtype=torch.uint8, device=dev))
+        sizes, sort_indices, _, _ = self.dispatch_out
+        self.gate_up = GroupedForwardPlan(h2, sizes, gate_up_weight, gate_up_a, gate_up_b, lora_scaling, swiglu=True,
+                                          row_map=sort_indices, row_repeat=top_k)
+        self.down = GroupedForwardPlan(self.gate_up.out, sizes, down_weight, down_a, down_b, lora_scaling)
+        # the plans must read the dispatch's own buffers, not converted copies
+        assert self.gate_up.group_sizes.data_ptr() == sizes.data_ptr() == self.down.group_sizes.data_ptr()
+        assert self.gate_up.row_map.data_ptr() == sort_indices.data_ptr()
+        self.top_k, self.n_experts = top_k, n_experts
+        refs = [t for t in (gate_up_a, gate_up_b, down_a, down_b) if t is not None]
+        self._lora_refs = [weakref.ref(t) for t in refs]
+        self._down_weight = weakref.ref(down_weight)
+        self._scaling = lora_scaling if not isinstance(lora_scaling, torch.Tensor) else (weakref.ref(lora_scaling),
+                                                                                          lora_scaling._version)
+        self._shape = (tuple(h2.shape), h2.device)
+
+    def fits(self, h2, top_k, down_weight, lora, lora_scaling) -> bool:
+        if self._shape != (tuple(h2.shape), h2.device) or self.top_k != top_k or self._down_weight() is not down_weight:
+            return False
+        given = [t for t in lora if t is not None]
+        if len(given) != len(self._lora_refs) or any(r() is not t for r, t in zip(self._lora_refs, given)):
+            return False
+        if isinstance(lora_scaling, torch.Tensor):
+            return (isinstance(self._scaling, tuple) and self._scaling[0]() is lora_scaling
+                    and self._scaling[1] == lora_scaling._version)
+        return not isinstance(self._scaling, tuple) and self._scaling == lora_scaling
+
+    def run(self, h2, selected, weights):
+        _, _, _, unsort, _ = moe_dispatch(None, selected, self.n_experts, repeat=self.top_k, out=self.dispatch_out)
+        self.gate_up.bind_x(h2)
+        self.gate_up.run()
+        down = self.down.run()
+        return moe_combine(down, unsort, weights)
+
+
+_moe_inference_plans = weakref.WeakKeyDictionary()  # gate/up weight -> the layer's plan (one token count at a time)
+
+
 def moe_expert_mlp(hidden, router_logits, top_k: int, gate_up_weight, down_weight, gate_up_a=None, gate_up_b=None,
                    down_a=None, down_b=None, lora_scaling=None, *, norm_topk_prob: bool = True):
     """Expert MLP of ``Qwen3Experts.__call__`` (skyrl/tx/models/qwen3.py:172-210) on W8A8 weights.
@@ -1385,12 +1457,16 @@ def moe_expert_mlp(hidden, router_logits, top_k: int, gate_up_weight, down_weigh
     else:
         weights, selected = moe_route(logits2, top_k, norm_topk_prob)
     if not training:
-        # indices only: the first projection gathers the hidden rows itself through the sort order
-        _, group_sizes, sort_indices, unsort, _ = moe_dispatch(None, selected, n_experts, repeat=top_k)
-        act = grouped_forward(h2, group_sizes, gate_up_weight, gate_up_a, gate_up_b, lora_scaling, swiglu=True,
-                              row_map=sort_indices, row_repeat=top_k)
-        down = grouped_forward(act, group_sizes, down_weight, down_a, down_b, lora_scaling)
-        return moe_combine(down, unsort, weights).reshape(hidden.shape)
+        # indices only: the first projection gathers the hidden rows itself through the sort order.  The
+        # layer's plans are kept with its gate/up weight: calls that share a weight object must be ordered on
+        # one stream (they share the intermediates), and not captured into different graphs.
+        h2 = h2.contiguous()
+        plan = _moe_inference_plans.get(gate_up_weight)
+        if plan is None or not plan.fits(h2, top_k, down_weight, (gate_up_a, gate_up_b, down_a, down_b), lora_scaling):
+            plan = _MoeInferencePlan(h2, top_k, gate_up_weight, down_weight, gate_up_a, gate_up_b, down_a, down_b,
+                                     lora_scaling)
+            _moe_inference_plans[gate_up_weight] = plan
+        return plan.run(h2, selected, weights).reshape(hidden.shape)
     scaling = lora_scaling
     if gate_up_a is not None and not isinstance(scaling, torch.Tensor):
         scaling = _scaling_scalar(scaling, hidden.device)

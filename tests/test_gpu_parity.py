@@ -535,6 +535,47 @@ def test_moe_expert_mlp_reduced(dev, pkg):
     assert rep["violations"] < 1e-3 * rep["size"], rep
 
 
+def test_moe_expert_mlp_keeps_its_plans_between_calls(dev, pkg):
+    """Without gradients the expert layer keeps its two grouped plans with the gate/up weight.  A second call
+    (packs kept), a call with other hidden rows and logits (same buffers, another routing), a call after an
+    adapter tensor was written in place (packs redone) and a call with another token count (new plans) all
+    give what a layer with fresh weight objects -- so fresh plans -- gives, bit for bit."""
+    import torch
+
+    rng = np.random.default_rng(77)
+    t, h, inter, e, topk, r = 96, 256, 128, 8, 2, 16
+    gu_codes = torch.from_numpy(rng.integers(-127, 128, (e, h, 2 * inter), dtype=np.int8)).to(dev)
+    gu_scales = torch.from_numpy(rng.uniform(0.001, 0.01, (e, 2 * inter)).astype(F32)).to(dev)
+    dn_codes = torch.from_numpy(rng.integers(-127, 128, (e, inter, h), dtype=np.int8)).to(dev)
+    dn_scales = torch.from_numpy(rng.uniform(0.001, 0.01, (e, h)).astype(F32)).to(dev)
+    w8 = pkg.w8a8_lora
+    bf = lambda shape, s=0.02: torch.from_numpy((rng.standard_normal(shape) * s).astype(F32)).to(dev).to(torch.bfloat16)
+    lora = [bf((e, h, r)), bf((e, r, 2 * inter)), bf((e, inter, r)), bf((e, r, h))]
+    guw, dnw = w8.prepare_grouped_weight(gu_codes, gu_scales), w8.prepare_grouped_weight(dn_codes, dn_scales)
+
+    def kept(hidden, logits):
+        return w8.w8a8_moe_expert_mlp(hidden, logits, topk, guw, dnw, *lora, 1.0, enabled=True).clone()
+
+    def fresh(hidden, logits):
+        a, b = w8.prepare_grouped_weight(gu_codes, gu_scales), w8.prepare_grouped_weight(dn_codes, dn_scales)
+        return w8.w8a8_moe_expert_mlp(hidden, logits, topk, a, b, *[x.clone() for x in lora], 1.0, enabled=True).clone()
+
+    same = lambda x, y: torch.equal(x.view(torch.int16), y.view(torch.int16))
+    h1, l1 = bf((t, h), 1.0), torch.from_numpy(rng.standard_normal((t, e)).astype(F32)).to(dev)
+    h2, l2 = bf((t, h), 1.0), torch.from_numpy(rng.standard_normal((t, e)).astype(F32)).to(dev)
+    first, second = kept(h1, l1), kept(h1, l1)
+    assert same(first, fresh(h1, l1)) and same(second, first)
+    plan = w8._moe_inference_plans[guw]
+    other = kept(h2, l2)
+    assert w8._moe_inference_plans[guw] is plan and same(other, fresh(h2, l2)) and not same(other, first)
+    lora[1].mul_(-1.0)                    # in place: the version counter moves, the next call packs again
+    flipped = kept(h2, l2)
+    assert w8._moe_inference_plans[guw] is plan and same(flipped, fresh(h2, l2)) and not same(flipped, other)
+    h3, l3 = bf((40, h), 1.0), torch.from_numpy(rng.standard_normal((40, e)).astype(F32)).to(dev)
+    fewer = kept(h3, l3)
+    assert w8._moe_inference_plans[guw] is not plan and same(fewer, fresh(h3, l3))
+
+
 @pytest.mark.parametrize("what", ["x_row", "x_elem", "w_col", "w_scale", "a_rank", "b_col", "scaling", "residual",
                                   "gamma", "index"])
 def test_every_operand_matters(dev, what):
