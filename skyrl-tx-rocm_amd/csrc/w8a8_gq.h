@@ -824,23 +824,32 @@ __global__ __launch_bounds__(256, 2) void gq_gemm_lds_kernel(GqGemmArgs a) {
         swl[j] = reinterpret_cast<lds_fptr>(sc)[(2u * wc + (uint32_t)j) * 32u + c];
         if (W4) swl[j] = swl[j] * 0.0625f;
       }
+      // a fragment's sixteen sums at a time, each of the four steps for all sixteen before the next step (the
+      // same operations per output; measured 3 % faster than output by output, where every instruction
+      // needs the result of the one in front of it)
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < 2; ++i) {
+        gq_f4 s4[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const gq_f4 s4 = *reinterpret_cast<lds_f4ptr>(sc + 512u + ((2u * wr + (uint32_t)i) * 32u + 8u * q + 4u * h) * 4u);
-          const float sxq[4] = {s4[0], s4[1], s4[2], s4[3]};
+        for (int q = 0; q < 4; ++q)
+          s4[q] = *reinterpret_cast<lds_f4ptr>(sc + 512u + ((2u * wr + (uint32_t)i) * 32u + 8u * q + 4u * h) * 4u);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int v = 4 * q + e;
+        for (int j = 0; j < 2; ++j) {
+          float t[16];
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-              float t = (float)acc[i][j][v] * sxq[e];
-              t = t * swl[j];
-              outv[i][j][v] = outv[i][j][v] + t;
-            }
-          }
+          for (int v = 0; v < 16; ++v) t[v] = (float)acc[i][j][v];
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int v = 0; v < 16; ++v) t[v] = t[v] * s4[v >> 2][v & 3];
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int v = 0; v < 16; ++v) t[v] = t[v] * swl[j];
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int v = 0; v < 16; ++v) outv[i][j][v] = outv[i][j][v] + t[v];
+          __builtin_amdgcn_sched_barrier(0);
         }
+      }
     }
   };
 
