@@ -18,7 +18,7 @@ import torch
 
 from ... import _native
 from .. import quantized_lora as ql
-from .w8a8_lora import MAX_LORA_RANK, _require_cuda, _stream_ptr
+from .w8a8_lora import MAX_LORA_RANK, _require_cuda, _stream_ptr, _version_of
 
 
 @dataclass(frozen=True)
@@ -46,7 +46,7 @@ def prepare_group_weight(weight) -> PackedGroupWeight:
     codes = weight.codes
     _require_cuda(codes, "weight codes")
     key = (codes.data_ptr(), weight.scales.data_ptr(), weight.padded_in_features, codes.shape[1], weight.bits,
-           weight.group_size, codes._version, weight.scales._version)
+           weight.group_size, _version_of(codes), _version_of(weight.scales))
     with _pack_lock:
         hit = _pack_cache.get(key)
         if hit is not None and hit[0]() is codes:

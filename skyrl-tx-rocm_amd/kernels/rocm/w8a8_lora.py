@@ -79,6 +79,15 @@ def _stream_ptr(device) -> int:
     return int(torch.cuda.current_stream(device).cuda_stream)
 
 
+def _version_of(t: torch.Tensor):
+    """The tensor's version counter, or None where torch keeps none (tensors made under
+    ``torch.inference_mode()``): in-place writes to such a tensor cannot be seen."""
+    try:
+        return t._version
+    except RuntimeError:
+        return None
+
+
 def _require_cuda(t: torch.Tensor, name: str) -> None:
     if not t.is_cuda:
         raise RuntimeError(f"{name} must live on the GPU (there is no CPU path); got device {t.device}")
@@ -116,7 +125,8 @@ def prepare_weight(weight) -> PackedW8Weight:
     if n > MAX_OUT_FEATURES:
         raise ValueError(f"N must not exceed {MAX_OUT_FEATURES}")
     _require_cuda(weight.codes, "weight codes")
-    key = (weight.codes.data_ptr(), weight.scales.data_ptr(), k, n, weight.codes._version, weight.scales._version)
+    # (inference tensors have no version counter: they are keyed by identity and storage alone)
+    key = (weight.codes.data_ptr(), weight.scales.data_ptr(), k, n, _version_of(weight.codes), _version_of(weight.scales))
     with _pack_lock:
         hit = _pack_cache.get(key)
         if hit is not None and hit[0]() is weight.codes:
@@ -363,10 +373,12 @@ class ForwardPlan:
         if self._lora is not None and not capturing and self.keep_lora_pack:
             # (what the workspace holds also depends on the path the flags choose: decode kernels keep B
             # regrouped per row, the tiled kernels A and B in operand order)
-            key = (self._lora[0]._version, self._lora[1]._version,
-                   None if self.adapter_indices is None else self.adapter_indices._version,
-                   flags & ~(_native.FLAG_SKIP_PROLOGUE | _native.FLAG_SKIP_GEMM | _native.FLAG_LORA_PACK_VALID))
-            if key == self._packed_lora_key:
+            versions = (_version_of(self._lora[0]), _version_of(self._lora[1]),
+                        0 if self.adapter_indices is None else _version_of(self.adapter_indices))
+            if None not in versions:  # (a tensor torch keeps no version of may have been written: pack)
+                key = versions + (flags & ~(_native.FLAG_SKIP_PROLOGUE | _native.FLAG_SKIP_GEMM |
+                                            _native.FLAG_LORA_PACK_VALID),)
+            if key is not None and key == self._packed_lora_key:
                 flags |= _native.FLAG_LORA_PACK_VALID
         self.problem.flags = flags
         with torch.cuda.device(self.device):
@@ -911,9 +923,11 @@ class GroupedForwardPlan:
         key = None
         capturing = torch.cuda.is_current_stream_capturing()
         if self._lora is not None and not capturing and self.keep_lora_pack:
-            key = (self._lora[0]._version, self._lora[1]._version,
-                   flags & ~(_native.FLAG_SKIP_PROLOGUE | _native.FLAG_SKIP_GEMM | _native.FLAG_LORA_PACK_VALID))
-            if key == self._packed_lora_key:
+            versions = (_version_of(self._lora[0]), _version_of(self._lora[1]))
+            if None not in versions:  # (a tensor torch keeps no version of may have been written: pack)
+                key = versions + (flags & ~(_native.FLAG_SKIP_PROLOGUE | _native.FLAG_SKIP_GEMM |
+                                            _native.FLAG_LORA_PACK_VALID),)
+            if key is not None and key == self._packed_lora_key:
                 flags |= _native.FLAG_LORA_PACK_VALID
         self.problem.flags = flags
         with torch.cuda.device(self.device):
@@ -1413,7 +1427,7 @@ class _MoeInferencePlan:
         self._lora_refs = [weakref.ref(t) for t in refs]
         self._down_weight = weakref.ref(down_weight)
         self._scaling = lora_scaling if not isinstance(lora_scaling, torch.Tensor) else (weakref.ref(lora_scaling),
-                                                                                          lora_scaling._version)
+                                                                                          _version_of(lora_scaling))
         self._shape = (tuple(h2.shape), h2.device)
 
     def fits(self, h2, top_k, down_weight, lora, lora_scaling) -> bool:
@@ -1424,7 +1438,7 @@ class _MoeInferencePlan:
             return False
         if isinstance(lora_scaling, torch.Tensor):
             return (isinstance(self._scaling, tuple) and self._scaling[0]() is lora_scaling
-                    and self._scaling[1] == lora_scaling._version)
+                    and self._scaling[1] is not None and self._scaling[1] == _version_of(lora_scaling))
         return not isinstance(self._scaling, tuple) and self._scaling == lora_scaling
 
     def run(self, h2, selected, weights):

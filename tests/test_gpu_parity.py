@@ -463,6 +463,35 @@ def test_grouped_ragged_linear(dev, pkg, sizes, k, n, rank, swiglu, extra, tile_
     _assert_close(got, want, f" grouped {sizes} {k}x{n}")
 
 
+def test_forward_under_inference_mode(dev, pkg):
+    """Tensors made under ``torch.inference_mode()`` carry no version counter: the dense and the grouped plan
+    and the group-scaled call take them all the same, pack the adapters on every run (a write to them could
+    not be seen), and give the bits of the same calls on ordinary tensors."""
+    import torch
+
+    case = wc.make_case(70, 256, 192, n_adapters=3, rank=16, seed=5, rms=True)
+    w8 = pkg.w8a8_lora
+
+    def run(t):
+        plan = w8.ForwardPlan(t["x"], t["weight"], t["a"], t["b"], t["s"], adapter_indices=t["idx"],
+                              rms_gamma=t["gamma"], eps=1e-6)
+        first = plan.run().clone()
+        t["b"].mul_(-1.0)                 # no counter moves for an inference tensor: the next run must pack anyway
+        second = plan.run().clone()
+        sizes = torch.tensor([30, 0, 40], dtype=torch.int32, device=dev)
+        gw = w8.prepare_grouped_weight(t["weight"].codes.unsqueeze(0).repeat(3, 1, 1).contiguous(),
+                                       t["weight"].scales.reshape(1, -1).repeat(3, 1).contiguous())
+        grouped = w8.grouped_forward(t["x"], sizes, gw, t["a"], t["b"], 1.0).clone()
+        return first, second, grouped
+
+    plain = run(wc.to_torch(case, dev))
+    with torch.inference_mode():
+        got = run(wc.to_torch(case, dev))
+    for a, b in zip(plain, got):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    assert not torch.equal(plain[0].view(torch.int16), plain[1].view(torch.int16))
+
+
 def test_grouped_plan_keeps_the_lora_packs_until_an_adapter_tensor_is_written(dev, pkg):
     """A grouped plan packs A and B on its first run, keeps the packs while neither tensor is written
     (the second run is told so and gives the same bits), and packs again after an in-place update."""
