@@ -462,3 +462,18 @@ def test_fused_checkpoint_loading(pkg):
         layer.load_split_adapter(0, [a, a + 1, a], bs)
     with pytest.raises(ValueError):
         layer.load_components([torch.from_numpy(q)])
+
+
+def test_version_counter_is_optional(pkg):
+    """``_version_of`` reads a tensor's version counter and answers None for tensors torch keeps none for
+    (made under ``torch.inference_mode()``), which the plans then treat as written at every run."""
+    import torch
+
+    w8 = pkg.w8a8_lora
+    t = torch.ones(3)
+    v0 = w8._version_of(t)
+    t.add_(1.0)
+    assert isinstance(v0, int) and w8._version_of(t) == v0 + 1
+    with torch.inference_mode():
+        u = torch.ones(3)
+    assert w8._version_of(u) is None
