@@ -1602,6 +1602,15 @@ int run_moe_combine_bwd(const void* d_out, const void* expert_out, const int32_t
 }
 
 constexpr uint32_t kGqZSlices = 32;
+// K slices of the routed LoRA-A projection: one workgroup per 32-row block and slice, so that calls with
+// fewer row blocks than the chip has CUs still fill it (the consumer adds the slices in order)
+inline uint32_t gq_z_ksplit(uint32_t m_pad, uint32_t k) {
+  const uint32_t n_blocks = m_pad / 32u, n_steps = (k + 63u) / 64u;
+  uint32_t ks = n_blocks >= 192u ? 1u : (256u + n_blocks - 1u) / n_blocks;
+  if (ks > 4u) ks = 4u;
+  while (ks > 1u && n_steps / ks < 16u) --ks;  // every wave of a slice keeps at least one step
+  return ks;
+}
 struct GqLayout { uint64_t codes, scales, z, src_row, dst_pos, slot_group, blk_range, at, total; uint32_t m_pad, G; };
 
 GqLayout make_gq_layout(uint32_t m, uint32_t k_pad, uint32_t group, uint32_t n_adapters, uint32_t rank) {
@@ -1612,7 +1621,7 @@ GqLayout make_gq_layout(uint32_t m, uint32_t k_pad, uint32_t group, uint32_t n_a
   L.codes = off; off += align256((uint64_t)L.m_pad * k_pad);
   L.scales = off; off += align256((uint64_t)L.m_pad * L.G * 4u);
   // decode (one row block): LoRA-A arrives as up to kGqZSlices slices over K
-  L.z = off; off += rank ? align256((uint64_t)L.m_pad * 64u * 4u * (L.m_pad == 32u ? kGqZSlices : 1u)) : 0u;
+  L.z = off; off += rank ? align256((uint64_t)L.m_pad * 64u * 4u * (L.m_pad == 32u ? kGqZSlices : 4u)) : 0u;
   L.src_row = off; off += rank ? align256((uint64_t)L.m_pad * 4u) : 0u;
   L.dst_pos = off; off += rank ? align256((uint64_t)L.m_pad * 4u) : 0u;
   L.slot_group = off; off += rank ? align256((uint64_t)L.m_pad * 4u) : 0u;
@@ -1702,7 +1711,7 @@ int run_gq_linear(const mi355_w8a8_gq_problem* p, hipStream_t s) {
                       aligned16(p->x) && aligned16(p->lora_a);
   const bool routed = fast_z && p->adapter_indices && p->n_adapters > 1u;
   int32_t* dst_pos = reinterpret_cast<int32_t*>(ws + L.dst_pos);
-  uint32_t z_slices = 1u;
+  uint32_t z_slices = 1u, z_slice_stride = p->m * 64u;
   if (fast_z) {
     int32_t* src_row = reinterpret_cast<int32_t*>(ws + L.src_row);
     int32_t* slot_group = reinterpret_cast<int32_t*>(ws + L.slot_group);
@@ -1732,10 +1741,13 @@ int run_gq_linear(const mi355_w8a8_gq_problem* p, hipStream_t s) {
     la.zf = reinterpret_cast<float*>(ws + L.z);
     la.zf_stride = 64u;
     la.M = p->m; la.K = p->k; la.r = p->rank; la.nkk = rank_chunks(p->rank);
-    la.n_steps = (p->k + 63u) / 64u; la.steps_per_wave = (la.n_steps + 15u) / 16u;
+    const uint32_t nks = gq_z_ksplit(L.m_pad, p->k);
+    la.n_steps = (p->k + 63u) / 64u; la.steps_per_wave = ((la.n_steps + nks - 1u) / nks + 15u) / 16u;
+    la.n_ksplit = nks; la.zf_slice = L.m_pad * 64u;
+    z_slices = nks; z_slice_stride = L.m_pad * 64u;
     la.nterms = 3u;
     la.n_blocks = L.m_pad / 32u;
-    const dim3 zgrid(L.m_pad / 32u), zblock(1024);
+    const dim3 zgrid(L.m_pad / 32u * nks), zblock(1024);
     (void)zblock;
     if ((st = launch_lora_a(la, la.nkk, zgrid, s))) return st;
   } else if (lora) {
@@ -1763,7 +1775,7 @@ int run_gq_linear(const mi355_w8a8_gq_problem* p, hipStream_t s) {
   g.ws = p->w_scales;
   g.z = lora ? reinterpret_cast<const float*>(ws + L.z) : nullptr;
   g.z_slot = routed ? dst_pos : nullptr;
-  g.z_slices = z_slices; g.z_slice_stride = p->m * 64u;
+  g.z_slices = z_slices; g.z_slice_stride = z_slice_stride;
   g.lora_b = static_cast<const uint16_t*>(p->lora_b);
   g.lora_scaling = p->lora_scaling;
   g.idx = p->adapter_indices;

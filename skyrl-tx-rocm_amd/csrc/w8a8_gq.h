@@ -288,7 +288,7 @@ struct GqGemmArgs {
   const float* ws;             // f32 [G, N]
   const float* z;              // f32 [rows or slots, 64] or null
   const int32_t* z_slot;       // int32 [M]: where row m's z lives (rows routed by adapter), or null: row m
-  uint32_t z_slices;           // decode kernel: z arrives as this many slices to add, z_slice_stride floats apart
+  uint32_t z_slices;           // z arrives as this many K slices to add in order, z_slice_stride floats apart
   uint32_t z_slice_stride;
   const uint16_t* lora_b;      // bf16 [n_adapters, r, N]
   const float* lora_scaling;   // f32 [n_adapters]
@@ -400,7 +400,13 @@ __device__ inline void gq_store_row_block(const GqGemmArgs& a, const float (&out
       const uint32_t row = rb * 32u + rr;
       const bool ok = row < a.M && r < a.r;
       const uint32_t zrow = (ok && a.z_slot) ? (uint32_t)a.z_slot[row] : row;
-      zbuf[rr][r] = ok ? a.z[(size_t)zrow * 64u + r] : 0.0f;
+      float zv = 0.0f;
+      if (ok) {  // the K slices of the projection, added in order
+        const float* zp = a.z + (size_t)zrow * 64u + r;
+        zv = zp[0];
+        for (uint32_t sl = 1; sl < a.z_slices; ++sl) zv = zv + zp[(size_t)sl * a.z_slice_stride];
+      }
+      zbuf[rr][r] = zv;
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);
     __builtin_amdgcn_wave_barrier();
@@ -524,8 +530,14 @@ __device__ inline void gq_tile_lora_sums(const GqGemmArgs& a, unsigned char* lds
 #pragma unroll
       for (int e = 0; e < 8; ++e) z8[e] = 0.0f;
       if (my_ad[i] >= 0) {
-        const float4 lo4 = *reinterpret_cast<const float4*>(a.z + (size_t)zrow[i] * 64u + r0 + 8u * kg);
-        const float4 hi4 = *reinterpret_cast<const float4*>(a.z + (size_t)zrow[i] * 64u + r0 + 8u * kg + 4u);
+        const float* zp = a.z + (size_t)zrow[i] * 64u + r0 + 8u * kg;
+        float4 lo4 = *reinterpret_cast<const float4*>(zp), hi4 = *reinterpret_cast<const float4*>(zp + 4);
+        for (uint32_t sl = 1; sl < a.z_slices; ++sl) {  // the K slices of the projection, added in order
+          const float4 l2 = *reinterpret_cast<const float4*>(zp + (size_t)sl * a.z_slice_stride);
+          const float4 h2 = *reinterpret_cast<const float4*>(zp + (size_t)sl * a.z_slice_stride + 4);
+          lo4.x = lo4.x + l2.x; lo4.y = lo4.y + l2.y; lo4.z = lo4.z + l2.z; lo4.w = lo4.w + l2.w;
+          hi4.x = hi4.x + h2.x; hi4.y = hi4.y + h2.y; hi4.z = hi4.z + h2.z; hi4.w = hi4.w + h2.w;
+        }
         const float t8[8] = {lo4.x, lo4.y, lo4.z, lo4.w, hi4.x, hi4.y, hi4.z, hi4.w};
 #pragma unroll
         for (int e = 0; e < 8; ++e) z8[e] = r0 + 8u * kg + (uint32_t)e < a.r ? t8[e] : 0.0f;
