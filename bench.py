@@ -537,7 +537,9 @@ def bench_moe_routing(args, cfg, pkg, dev):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    out = None
     for _ in range(args.steps):
+        out = None  # (the last step's 128 MiB of sorted rows go back to torch's allocator before the next asks for them)
         out = step()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
