@@ -132,8 +132,9 @@ def _is_per_channel_w8a8(weight: GroupQuantizedWeight, activation_bits: int) -> 
     """True for the geometry of the fast W8A8 kernels; validates the arguments either way."""
     _validate_bits(activation_bits)
     validate_quantized_weight(weight)
+    # (K not a multiple of 8 goes the group-scaled way, embedded as one group of the next multiple of 32)
     return (weight.bits == 8 and activation_bits == 8 and weight.group_size == weight.padded_in_features
-            and weight.padded_in_features == weight.original_in_features)
+            and weight.padded_in_features == weight.original_in_features and weight.original_in_features % 8 == 0)
 
 
 def quantized_frozen_linear(x: torch.Tensor, weight: GroupQuantizedWeight, *, activation_bits: int = 8):

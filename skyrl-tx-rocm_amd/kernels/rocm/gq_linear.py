@@ -32,6 +32,11 @@ class PackedGroupWeight:
     out_features: int
     bits: int
     group_size: int
+    # The reference's own group size and padded K where they differ from the packed ones: a group size that is
+    # not a multiple of 32 is embedded, every group followed by zero codes up to the next multiple of 32 (and x
+    # by zeros at the same places), which changes no maximum, no code of a real element and no integer sum.
+    source_group_size: int = 0
+    source_padded_in_features: int = 0
 
 
 _pack_cache: dict = {}
@@ -51,12 +56,22 @@ def prepare_group_weight(weight) -> PackedGroupWeight:
         hit = _pack_cache.get(key)
         if hit is not None and hit[0]() is codes:
             return hit[1]
-    if weight.group_size % 32:
-        raise ValueError(f"the native path needs group_size % 32 == 0, got {weight.group_size}")
     want = torch.uint8 if weight.bits == 4 else torch.int8
     if codes.dtype != want:
         raise TypeError(f"W{weight.bits} codes must have dtype {want}, got {codes.dtype}")
     k_pad, n = weight.padded_in_features, codes.shape[1]
+    group, src_group, src_k_pad = weight.group_size, 0, 0
+    if group % 32:
+        # embed: [G, group, N] -> [G, group32, N] with zero codes behind every group
+        src_group, src_k_pad = group, k_pad
+        group32 = (group + 31) // 32 * 32
+        n_groups = k_pad // group
+        plain = (codes if weight.bits == 8 else ql.unpack_signed_int4(codes))[:k_pad]
+        wide = torch.zeros((n_groups, group32, n), dtype=torch.int8, device=codes.device)
+        wide[:, :group] = plain.reshape(n_groups, group, n)
+        wide = wide.reshape(n_groups * group32, n)
+        codes = wide if weight.bits == 8 else ql.pack_signed_int4(wide)
+        group, k_pad = group32, n_groups * group32
     lib = _native.load()
     nbytes = int(lib.mi355_w8a8_gq_packed_weight_bytes(k_pad, n, weight.bits))
     if nbytes == 0:
@@ -68,11 +83,11 @@ def prepare_group_weight(weight) -> PackedGroupWeight:
                                                   _stream_ptr(codes.device))
     _native.check("mi355_w8a8_gq_pack_weight_v1", status)
     out = PackedGroupWeight(packed, weight.scales.to(torch.float32).contiguous(), weight.original_in_features, k_pad,
-                            n, weight.bits, weight.group_size)
+                            n, weight.bits, group, src_group, src_k_pad)
     with _pack_lock:
         if len(_pack_cache) > 4096:
             _pack_cache.clear()
-        _pack_cache[key] = (weakref.ref(codes), out)
+        _pack_cache[key] = (weakref.ref(weight.codes), out)
     return out
 
 
@@ -94,6 +109,19 @@ def forward(x: torch.Tensor, weight, lora_a=None, lora_b=None, lora_scaling=None
     dev = x.device
     flat = x.reshape(-1, k).contiguous()
     m = flat.shape[0]
+
+    def embed(t, axis):  # the K axis of x (or of LoRA A) with zeros behind every source group
+        src_g, dst_g, n_groups = pw.source_group_size, pw.group_size, pw.padded_in_features // pw.group_size
+        shape = list(t.shape)
+        padded = torch.zeros(shape[:axis] + [pw.source_padded_in_features] + shape[axis + 1:], dtype=t.dtype, device=dev)
+        padded.narrow(axis, 0, k).copy_(t)
+        wide = torch.zeros(shape[:axis] + [n_groups, dst_g] + shape[axis + 1:], dtype=t.dtype, device=dev)
+        wide.narrow(axis + 1, 0, src_g).copy_(padded.reshape(shape[:axis] + [n_groups, src_g] + shape[axis + 1:]))
+        return wide.reshape(shape[:axis] + [n_groups * dst_g] + shape[axis + 1:])
+
+    embedded = pw.source_group_size != 0
+    if embedded:
+        flat = embed(flat, 1)
     a3 = b3 = s1 = idx = None
     n_ad = r = 0
     if lora_a is not None:
@@ -107,7 +135,7 @@ def forward(x: torch.Tensor, weight, lora_a=None, lora_b=None, lora_scaling=None
                              f"K={k}, N={n}")
         if r < 1 or r > MAX_LORA_RANK:
             raise ValueError(f"LoRA rank must be in [1, {MAX_LORA_RANK}], got {r}")
-        a3, b3 = a3.contiguous(), b3.contiguous()
+        a3, b3 = (embed(a3, 1) if embedded else a3).contiguous(), b3.contiguous()
         s1 = torch.as_tensor(lora_scaling, dtype=torch.float32, device=dev).reshape(-1)
         s1 = (s1.expand(n_ad) if s1.numel() == 1 else s1).contiguous()
         if s1.numel() != n_ad:
@@ -134,7 +162,7 @@ def forward(x: torch.Tensor, weight, lora_a=None, lora_b=None, lora_scaling=None
     p = _native.GqProblem()
     p.struct_size = ctypes.sizeof(_native.GqProblem)
     p.flags = int(flags)
-    p.m, p.k, p.k_pad, p.n = m, k, pw.padded_in_features, n
+    p.m, p.k, p.k_pad, p.n = m, (pw.padded_in_features if embedded else k), pw.padded_in_features, n
     p.group_size, p.weight_bits, p.activation_bits = pw.group_size, pw.bits, activation_bits
     p.n_adapters, p.rank = n_ad, r
     p.x = flat.data_ptr()
@@ -154,6 +182,10 @@ def forward(x: torch.Tensor, weight, lora_a=None, lora_b=None, lora_scaling=None
         status = lib.mi355_w8a8_gq_linear_v1(ctypes.byref(p), _stream_ptr(dev))
     _native.check("mi355_w8a8_gq_linear_v1", status)
     result = out.reshape(*x.shape[:-1], n)
+    if return_aux and embedded:  # the codes in the reference's own layout, without the zeros of the embedding
+        n_groups = pw.padded_in_features // pw.group_size
+        aux["x_codes"] = aux["x_codes"].reshape(m, n_groups, pw.group_size)[:, :, :pw.source_group_size].reshape(
+            m, pw.source_padded_in_features).contiguous()
     return (result, aux) if return_aux else result
 
 

@@ -70,6 +70,32 @@ def test_reference_hand_coded_w4a4_case(dev, pkg):
     np.testing.assert_array_equal(got.to(torch.float32).cpu().numpy(), expected)
     via_api = pkg.quantized_lora.quantized_frozen_linear(_bf(dev, x), _to_dev(pkg, dev, big), activation_bits=4)
     assert torch.equal(via_api, got)
+    # and the reference's own weight (groups of 2, K = 3 padded to 4) straight through the entry point, which
+    # embeds it the same way by itself
+    direct = pkg.quantized_lora.quantized_frozen_linear(_bf(dev, x_small), _to_dev(pkg, dev, small), activation_bits=4)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(direct.to(torch.float32).cpu().numpy(), expected)
+
+
+def test_per_channel_w8a8_with_k_not_a_multiple_of_8(dev, pkg):
+    """quantized_lora_linear (quantized_lora.py:257-304) takes any K: a per-channel W8A8 weight with K = 100
+    runs as one group of 128 on the group-scaled kernels, codes, scales and float32 base bit-equal to the oracle."""
+    import torch
+
+    rng = np.random.default_rng(100)
+    m, k, n, r = 40, 100, 72, 8
+    x = o.bf16_round(rng.standard_t(4, (m, k)).astype(F32))
+    w = o.quantize_frozen_weight((rng.standard_normal((k, n)) * 0.05).astype(F32), bits=8, group_size=k, scale_dtype="f32")
+    a = o.bf16_round((rng.standard_normal((k, r)) * 0.05).astype(F32))
+    b = o.bf16_round((rng.standard_normal((r, n)) * 0.05).astype(F32))
+    base = o.quantized_frozen_linear_f32(x, w, activation_bits=8)
+    want = o.bf16_round((base + o.lora_delta_multi(x, a[None], b[None], np.asarray([1.5], F32), np.zeros(m, np.int32))).astype(F32))
+    got = pkg.quantized_lora.quantized_lora_linear(_bf(dev, x), _to_dev(pkg, dev, w), _bf(dev, a), _bf(dev, b), 1.5)
+    frozen = pkg.quantized_lora.quantized_frozen_linear(_bf(dev, x), _to_dev(pkg, dev, w))
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(o.bf16_bits(frozen.to(torch.float32).cpu().numpy()), o.bf16_bits(o.bf16_round(base)))
+    rep = wc.compare(got.to(torch.float32).cpu().numpy(), want)
+    assert rep["violations"] == 0, rep
 
 
 CASES = [
@@ -87,6 +113,10 @@ CASES = [
     (1024, 2048, 512, 4, 8, 1024, 40, 5),  # long groups
     (260, 256, 136, 4, 8, 64, 24, 20),    # twenty adapters: three batches of the LDS-staged LoRA epilogue
     (130, 128, 132, 8, 8, 64, 8, 3),      # N not a multiple of 8: the epilogue that reads B from memory
+    (33, 200, 96, 4, 8, 50, 8, 2),        # groups of 50: embedded in groups of 64 with zero codes behind every group
+    (20, 36, 40, 4, 4, 2, 0, 0),          # the reference test's group size: groups of 2 in groups of 32
+    (64, 100, 48, 8, 8, 100, 6, 1),       # per-channel W8A8 with K = 100: one group of 128
+    (70, 90, 56, 8, 4, 30, 12, 3),        # K padded to the group (90 -> 3 x 30), groups of 30
 ]
 
 
@@ -192,8 +222,11 @@ def test_gq_pack_keeps_four_bits_and_rejects_bad_geometry(dev, pkg):
     assert lib.mi355_w8a8_gq_workspace_bytes(4, 64, 10, 0, 0) == 0
     assert lib.mi355_w8a8_gq_workspace_bytes(4, 64, 32, 2, 8) > lib.mi355_w8a8_gq_workspace_bytes(4, 64, 32, 0, 0) > 0
     w = o.quantize_frozen_weight(np.ones((70, 8), F32), bits=4, group_size=14, scale_dtype="f32")
-    with pytest.raises(ValueError, match="group_size % 32"):
-        pkg.gq_linear.forward(torch.zeros(2, 70, dtype=torch.bfloat16, device=dev), _to_dev(pkg, dev, w))
+    # (the C entry points take groups of whole 32-wide k blocks only -- the workspace query above says so; the
+    # host mirror embeds other group sizes, here 14 in 32)
+    ones = pkg.gq_linear.forward(torch.ones(2, 70, dtype=torch.bfloat16, device=dev), _to_dev(pkg, dev, w))
+    want = o.bf16_round(o.quantized_frozen_linear_f32(np.ones((2, 70), F32), w, activation_bits=8))
+    np.testing.assert_array_equal(ones.to(torch.float32).cpu().numpy(), want)
     w = o.quantize_frozen_weight(np.ones((64, 8), F32), bits=4, group_size=32, scale_dtype="f32")
     wt = _to_dev(pkg, dev, w)
     with pytest.raises(ValueError):
