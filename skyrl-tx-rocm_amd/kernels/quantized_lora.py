@@ -6,8 +6,9 @@ Mirrors the interface of the reference's ``skyrl/tx/kernels/quantized_lora.py``
 ``quantized_lora_linear`` :400-453) on torch tensors.  The forward functions run the
 gfx950 HIP kernels: the per-token / per-channel geometry (``bits == 8``,
 ``group_size == K``, ``activation_bits == 8``) takes the tiled / streaming W8A8
-kernels, every other geometry of the format with ``group_size % 32 == 0`` (W4 codes,
-scales per K group, A4 activations) the group-scaled kernels of ``rocm/gq_linear.py``.
+kernels, every other geometry of the format (W4 codes, scales per K group, A4
+activations, any group size) the group-scaled kernels of ``rocm/gq_linear.py``; under
+autograd that path carries the reference's pullback on float32 library GEMMs.
 The weight quantizer is an offline, one-time torch computation.
 """
 
@@ -137,6 +138,60 @@ def _is_per_channel_w8a8(weight: GroupQuantizedWeight, activation_bits: int) -> 
             and weight.padded_in_features == weight.original_in_features and weight.original_in_features % 8 == 0)
 
 
+def _group_scaled_input_pullback(dy: torch.Tensor, weight: GroupQuantizedWeight) -> torch.Tensor:
+    """``dy @ (codes * scales).T`` in float32, a slab of K groups at a time (quantized_lora.py:355-378: the
+    dequantized K x N matrix is never held as a whole), cut to the original K."""
+    codes = weight.codes if weight.bits == 8 else unpack_signed_int4(weight.codes)
+    codes = codes[: weight.padded_in_features]
+    n = codes.shape[1]
+    g = weight.group_size
+    n_groups = weight.padded_in_features // g
+    scales = weight.scales.to(torch.float32)
+    per_slab = max(1, (1 << 24) // max(1, g * n))  # about 64 MiB of float32 weight at a time
+    parts = []
+    for g0 in range(0, n_groups, per_slab):
+        g1 = min(n_groups, g0 + per_slab)
+        slab = codes[g0 * g: g1 * g].reshape(g1 - g0, g, n).to(torch.float32) * scales[g0:g1, None, :]
+        parts.append(dy @ slab.reshape((g1 - g0) * g, n).T)
+    return torch.cat(parts, dim=1)[:, : weight.original_in_features]
+
+
+class _GroupScaledLoraFunction(torch.autograd.Function):
+    """The group-scaled forward with the reference's pullback (quantized_lora.py:337-394): straight through
+    the quantizers, ``dx = dy @ deq(W).T + r @ A.T`` with ``r = (dy @ B.T) * s``, ``dA = x.T @ r``,
+    ``dB = ((x @ A).T @ dy) * s``, ``ds = sum(dy * ((x @ A) @ B))``, all in float32 on the library GEMMs and
+    cast once.  The frozen weight gets no gradient."""
+
+    @staticmethod
+    def forward(ctx, x, lora_a, lora_b, scaling, weight, activation_bits):
+        from .rocm import gq_linear
+
+        ctx.save_for_backward(x, lora_a, lora_b, scaling)
+        ctx.weight = weight
+        return gq_linear.forward(x, weight, lora_a, lora_b, scaling, activation_bits=activation_bits)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, lora_a, lora_b, scaling = ctx.saved_tensors
+        weight = ctx.weight
+        xf = x.reshape(-1, x.shape[-1]).to(torch.float32)
+        dyf = dy.reshape(-1, dy.shape[-1]).to(torch.float32)
+        a, b = lora_a.to(torch.float32), lora_b.to(torch.float32)
+        s = scaling.to(device=dyf.device, dtype=torch.float32)
+        z = xf @ a
+        r = (dyf @ b.T) * s
+        dx = da = db = ds = None
+        if ctx.needs_input_grad[0]:
+            dx = (_group_scaled_input_pullback(dyf, weight) + r @ a.T).reshape(x.shape).to(x.dtype)
+        if ctx.needs_input_grad[1]:
+            da = (xf.T @ r).to(lora_a.dtype)
+        if ctx.needs_input_grad[2]:
+            db = ((z.T @ dyf) * s).to(lora_b.dtype)
+        if ctx.needs_input_grad[3]:
+            ds = (dyf * (z @ b)).sum().reshape(scaling.shape).to(scaling.dtype)
+        return dx, da, db, ds, None, None
+
+
 def quantized_frozen_linear(x: torch.Tensor, weight: GroupQuantizedWeight, *, activation_bits: int = 8):
     from .rocm import gq_linear, w8a8_lora
 
@@ -173,4 +228,8 @@ def quantized_lora_linear(x: torch.Tensor, weight: GroupQuantizedWeight, lora_a:
         raise ValueError(f"lora_scaling must be scalar, got {tuple(scaling.shape)}")
     if per_channel:
         return w8a8_lora.w8a8_lora_linear(x, weight, lora_a, lora_b, scaling, enabled=True)
+    if torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad
+                                       for t in (x, lora_a, lora_b, lora_scaling)):
+        s_arg = lora_scaling if isinstance(lora_scaling, torch.Tensor) and lora_scaling.requires_grad else scaling
+        return _GroupScaledLoraFunction.apply(x, lora_a, lora_b, s_arg, weight, activation_bits)
     return gq_linear.forward(x, weight, lora_a, lora_b, scaling, activation_bits=activation_bits)
